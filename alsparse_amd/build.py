@@ -1,0 +1,39 @@
+"""Build recipe: compiles the HIP kernels for gfx950 and the C host library into
+``alsparse_amd/lib/libalpha_spblas.so`` and the workload generators into
+``alsparse_amd/lib/libasamd_workloads.so``.  hipcc cross-compiles without a GPU."""
+import os
+import subprocess
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB_DIR = os.path.join(ROOT, "alsparse_amd", "lib")
+LIB_PATH = os.path.join(LIB_DIR, "libalpha_spblas.so")
+WORKLOADS_PATH = os.path.join(LIB_DIR, "libasamd_workloads.so")
+
+
+def _run(cmd, cwd=None):
+    proc = subprocess.run(cmd, cwd=cwd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("build step failed: %s\n%s" % (" ".join(cmd), proc.stdout))
+    return proc.stdout
+
+
+def build_library(force=True, jobs=8):
+    """Compile every HIP extension (always recompiles when ``force``)."""
+    csrc = os.path.join(ROOT, "alsparse_amd", "csrc")
+    if force:
+        _run(["make", "-C", csrc, "clean"])
+    _run(["make", "-C", csrc, "-j%d" % jobs])
+    return LIB_PATH
+
+
+def build_workloads():
+    os.makedirs(LIB_DIR, exist_ok=True)
+    src = os.path.join(ROOT, "alsparse_amd", "workloads", "workloads.c")
+    _run(["gcc", "-std=c11", "-O2", "-fopenmp", "-fPIC", "-shared", "-Wall", "-o", WORKLOADS_PATH, src, "-lm"])
+    return WORKLOADS_PATH
+
+
+def build_oracle():
+    """Compile the CPU oracle (test infrastructure) and, when the reference tree
+    is present, the reference's own CPU kernels into oracle/_ref/."""
+    _run(["make", "-C", os.path.join(ROOT, "oracle")])

@@ -1,0 +1,245 @@
+"""ctypes bindings of ``libalpha_spblas.so``: the same names, argument order and
+status codes as the reference's C API (``include/alphasparse.h`` and
+``include/alpha_spblas_dcu.h`` of this repository list each entry with the
+reference declaration it replaces).
+
+There is no fallback: if the library has not been built, :func:`load` raises.
+"""
+import ctypes
+import os
+from ctypes import POINTER, Structure, byref, c_bool, c_double, c_float, c_int, c_int32, c_size_t, c_void_p
+
+from .build import LIB_PATH
+
+# ---- enums (values are ABI) -------------------------------------------------
+ALPHA_SPARSE_STATUS_SUCCESS = 0
+ALPHA_SPARSE_STATUS_NOT_INITIALIZED = 1
+ALPHA_SPARSE_STATUS_ALLOC_FAILED = 2
+ALPHA_SPARSE_STATUS_INVALID_VALUE = 3
+ALPHA_SPARSE_STATUS_EXECUTION_FAILED = 4
+ALPHA_SPARSE_STATUS_INTERNAL_ERROR = 5
+ALPHA_SPARSE_STATUS_NOT_SUPPORTED = 6
+ALPHA_SPARSE_STATUS_INVALID_POINTER = 7
+ALPHA_SPARSE_STATUS_INVALID_HANDLE = 8
+
+ALPHA_SPARSE_OPERATION_NON_TRANSPOSE = 0
+ALPHA_SPARSE_OPERATION_TRANSPOSE = 1
+ALPHA_SPARSE_OPERATION_CONJUGATE_TRANSPOSE = 2
+
+ALPHA_SPARSE_MATRIX_TYPE_GENERAL = 0
+ALPHA_SPARSE_MATRIX_TYPE_SYMMETRIC = 1
+
+ALPHA_SPARSE_INDEX_BASE_ZERO = 0
+ALPHA_SPARSE_INDEX_BASE_ONE = 1
+
+ALPHA_SPARSE_LAYOUT_ROW_MAJOR = 0
+ALPHA_SPARSE_LAYOUT_COLUMN_MAJOR = 1
+
+ALPHA_SPARSE_FORMAT_CSR = 1
+ALPHA_SPARSE_DATATYPE_FLOAT = 0
+ALPHA_SPARSE_DATATYPE_DOUBLE = 1
+
+# kernel families of the thin kernel ABI (include/alsparse_amd_kernels.h)
+ASAMD_SPMV_AUTO, ASAMD_SPMV_VECTOR, ASAMD_SPMV_ROWCONST, ASAMD_SPMV_MERGE, ASAMD_SPMV_SCALAR = range(5)
+ASAMD_HIST_BINS = 33
+
+
+# ---- structs ------------------------------------------------------------------
+class alphasparse_matrix(Structure):
+    _fields_ = [("mat", c_void_p), ("format", c_int), ("datatype", c_int),
+                ("inspector", c_void_p), ("dcu_info", c_void_p)]
+
+
+alphasparse_matrix_t = POINTER(alphasparse_matrix)
+
+
+class alpha_matrix_descr(Structure):
+    _fields_ = [("type", c_int), ("mode", c_int), ("diag", c_int)]
+
+
+class alpha_dcu_matrix_descr(Structure):
+    _fields_ = [("type", c_int), ("mode", c_int), ("diag", c_int), ("base", c_int)]
+
+
+alpha_dcu_matrix_descr_t = POINTER(alpha_dcu_matrix_descr)
+
+
+def _csr_struct(ctype):
+    class _S(Structure):
+        _fields_ = [("values", POINTER(ctype)), ("rows_start", POINTER(c_int32)),
+                    ("rows_end", POINTER(c_int32)), ("col_indx", POINTER(c_int32)),
+                    ("rows", c_int32), ("cols", c_int32), ("ordered", c_bool),
+                    ("d_values", c_void_p), ("d_row_ptr", c_void_p), ("d_col_indx", c_void_p)]
+    return _S
+
+
+spmat_csr_s_t = _csr_struct(c_float)
+spmat_csr_d_t = _csr_struct(c_double)
+
+
+class _alphasparse_dcu_csrmv_info(Structure):
+    _fields_ = [("algo_tuning", c_bool), ("algo", c_int), ("iter", c_int32), ("size", c_size_t),
+                ("row_blocks", c_void_p), ("csr_adaptive_has_tuned", c_bool), ("trans", c_int),
+                ("m", c_int32), ("n", c_int32), ("nnz", c_int32), ("descr", c_void_p),
+                ("csr_row_ptr", c_void_p), ("csr_col_ind", c_void_p)]
+
+
+class _alphasparse_dcu_mat_info(Structure):
+    _fields_ = ([(n, c_void_p) for n in (
+        "bsrsv_upper_info", "bsrsv_lower_info", "bsrsvt_upper_info", "bsrsvt_lower_info",
+        "bsric0_info", "bsrilu0_info")] +
+        [("csrmv_info", POINTER(_alphasparse_dcu_csrmv_info))] +
+        [(n, c_void_p) for n in (
+            "csric0_info", "csrilu0_info", "csrsv_upper_info", "csrsv_lower_info",
+            "csrsvt_upper_info", "csrsvt_lower_info", "csrsm_upper_info", "csrsm_lower_info",
+            "csrsmt_upper_info", "csrsmt_lower_info", "csrgemm_info", "zero_pivot")] +
+        [("boost_enable", c_int), ("use_double_prec_tol", c_int),
+         ("boost_tol", c_void_p), ("boost_val", c_void_p)])
+
+
+alphasparse_dcu_mat_info_t = POINTER(_alphasparse_dcu_mat_info)
+alphasparse_dcu_handle_t = c_void_p  # opaque from Python: holds a hipDeviceProp_t
+
+
+class asamd_csr_stats(Structure):
+    _fields_ = [("m", c_int32), ("n", c_int32), ("nnz", c_int32), ("base", c_int32),
+                ("min_len", c_int32), ("max_len", c_int32), ("const_len", c_int32),
+                ("first_offset", c_int32), ("algo", c_int32), ("vector_width", c_int32),
+                ("merge_blocks", c_int32), ("trusted", c_int32),
+                ("hist", ctypes.c_int64 * ASAMD_HIST_BINS)]
+
+
+class asamd_dense_strides(Structure):
+    _fields_ = [("b_row_stride", ctypes.c_int64), ("b_col_stride", ctypes.c_int64),
+                ("c_row_stride", ctypes.c_int64), ("c_col_stride", ctypes.c_int64)]
+
+
+_I, _P = c_int32, c_void_p
+
+
+def _per_type(ctype):
+    """Prototypes that exist once per value type; {T} is the scalar ctype."""
+    T, PT = ctype, POINTER(ctype)
+    return {
+        "alphasparse_{s}_create_csr": [POINTER(alphasparse_matrix_t), c_int, _I, _I, _P, _P, _P, _P],
+        "alphasparse_{s}_export_csr": [alphasparse_matrix_t, POINTER(c_int), POINTER(_I), POINTER(_I),
+                                       POINTER(_P), POINTER(_P), POINTER(_P), POINTER(_P)],
+        "alphasparse_{s}_mv": [c_int, T, alphasparse_matrix_t, alpha_matrix_descr, _P, T, _P],
+        "alphasparse_{s}_mm": [c_int, T, alphasparse_matrix_t, alpha_matrix_descr, c_int, _P, _I, _I, T, _P, _I],
+        "host2device_{s}_csr": [alphasparse_matrix_t],
+        "alphasparse_{s}_mv_dcu": [alphasparse_dcu_handle_t, c_int, PT, alphasparse_matrix_t,
+                                   alpha_dcu_matrix_descr_t, _P, PT, _P],
+        "alphasparse_dcu_{s}_csrmv_analysis": [alphasparse_dcu_handle_t, c_int, _I, _I, _I,
+                                               alpha_dcu_matrix_descr_t, _P, _P, _P, _P],
+        "alphasparse_dcu_{s}_csrmv": [alphasparse_dcu_handle_t, c_int, _I, _I, _I, PT,
+                                      alpha_dcu_matrix_descr_t, _P, _P, _P, _P, _P, PT, _P],
+        "alphasparse_dcu_{s}_csrmm": [alphasparse_dcu_handle_t, c_int, c_int, c_int, _I, _I, _I, _I, PT,
+                                      alpha_dcu_matrix_descr_t, _P, _P, _P, _P, _I, PT, _P, _I],
+        "alphasparse_dcu_{s}csr2ell": [alphasparse_dcu_handle_t, _I, alpha_dcu_matrix_descr_t, _P, _P, _P,
+                                       alpha_dcu_matrix_descr_t, _I, _P, _P],
+        # thin kernel ABI
+        "asamd_{s}_csrmv": [_P, _P, T, _P, _P, _P, _P, T, _P],
+        "asamd_{s}_csrmm": [_P, _I, _I, _I, _I, T, _P, _P, _P, _I, _P, T, _P, POINTER(asamd_dense_strides)],
+        "asamd_{s}_csr2ell": [_P, _I, _P, _P, _P, _I, _I, _I, _P, _P],
+    }
+
+
+_COMMON = {
+    "alphasparse_destroy": [alphasparse_matrix_t],
+    "init_handle": [POINTER(alphasparse_dcu_handle_t)],
+    "alphasparse_dcu_get_handle": [POINTER(alphasparse_dcu_handle_t)],
+    "alphasparse_dcu_destory_handle": [alphasparse_dcu_handle_t],
+    "alphasparse_dcu_create_mat_descr": [POINTER(alpha_dcu_matrix_descr_t)],
+    "alphasparse_dcu_destroy_mat_descr": [alpha_dcu_matrix_descr_t],
+    "alphasparse_dcu_create_mat_info": [POINTER(alphasparse_dcu_mat_info_t)],
+    "alphasparse_dcu_destroy_mat_info": [alphasparse_dcu_mat_info_t],
+    "alphasparse_dcu_create_csrmv_info": [POINTER(POINTER(_alphasparse_dcu_csrmv_info)), c_bool],
+    "alphasparse_dcu_destroy_csrmv_info": [POINTER(_alphasparse_dcu_csrmv_info)],
+    "get_alphasparse_dcu_status_for_hip_status": [c_int],
+    "alphasparse_dcu_csrmv_clear": [alphasparse_dcu_handle_t, _P],
+    "alphasparse_dcu_csr2coo": [alphasparse_dcu_handle_t, _P, _I, _I, _P, c_int],
+    "alphasparse_dcu_csr2ell_width": [alphasparse_dcu_handle_t, _I, alpha_dcu_matrix_descr_t, _P,
+                                      alpha_dcu_matrix_descr_t, POINTER(_I)],
+    # thin kernel ABI
+    "asamd_csr_plan_create": [_P, _I, _I, _I, _P, _I, _I, _I, POINTER(_P)],
+    "asamd_csr_plan_destroy": [_P],
+    "asamd_csr_plan_stats": [_P],
+    "asamd_csr_plan_set_algo": [_P, _I],
+    "asamd_csr2coo": [_P, _P, _I, _I, _P, _I],
+    "asamd_csr2ell_width": [_P, _I, _P, POINTER(_I)],
+    "asamd_warmup": [_P],
+}
+
+
+def prototypes():
+    """name -> argtypes for every symbol the public headers declare."""
+    out = dict(_COMMON)
+    for s, ct in (("s", c_float), ("d", c_double)):
+        for k, v in _per_type(ct).items():
+            out[k.format(s=s)] = v
+    return out
+
+
+_RESTYPE = {"asamd_csr_plan_destroy": None, "asamd_csr_plan_stats": POINTER(asamd_csr_stats)}
+
+_lib = None
+
+
+def load():
+    """Load libalpha_spblas.so and attach prototypes.  Raises if it is not built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "%s is missing: build it first (python -c 'import __graft_entry__ as g; g.build()' "
+                "or make -C alsparse_amd/csrc). There is no CPU fallback." % LIB_PATH)
+        lib = ctypes.CDLL(LIB_PATH, mode=ctypes.RTLD_GLOBAL)
+        for name, args in prototypes().items():
+            fn = getattr(lib, name)  # AttributeError if a declared symbol is not exported
+            fn.argtypes = args
+            fn.restype = _RESTYPE.get(name, c_int)
+        _lib = lib
+    return _lib
+
+
+# ---- small conveniences used by tests and the benchmark -----------------------
+def ptr(x):
+    """Device pointer / numpy array / None -> c_void_p."""
+    if x is None:
+        return c_void_p(None)
+    if hasattr(x, "ptr"):
+        return c_void_p(x.ptr)
+    if hasattr(x, "ctypes"):
+        return x.ctypes.data_as(c_void_p)
+    return c_void_p(x)
+
+
+def scalar_type(dtype):
+    import numpy as np
+    return c_float if np.dtype(dtype) == np.float32 else c_double
+
+
+def prefix(dtype):
+    import numpy as np
+    return "s" if np.dtype(dtype) == np.float32 else "d"
+
+
+class Handle:
+    """alphasparse_dcu_get_handle / alphasparse_dcu_destory_handle."""
+
+    def __init__(self):
+        self.lib = load()
+        self.h = alphasparse_dcu_handle_t(None)
+        st = self.lib.alphasparse_dcu_get_handle(byref(self.h))
+        if st != ALPHA_SPARSE_STATUS_SUCCESS:
+            raise RuntimeError("alphasparse_dcu_get_handle -> %d" % st)
+
+    def close(self):
+        if self.h:
+            self.lib.alphasparse_dcu_destory_handle(self.h)
+            self.h = alphasparse_dcu_handle_t(None)
+
+
+def make_descr(base=ALPHA_SPARSE_INDEX_BASE_ZERO, mtype=ALPHA_SPARSE_MATRIX_TYPE_GENERAL):
+    d = alpha_dcu_matrix_descr(mtype, 0, 0, base)
+    return d

@@ -1,0 +1,73 @@
+// Device-side helpers shared by the gfx950 kernels: wave64 lane-group
+// reductions through DPP, XCD-aware workgroup remapping, fused multiply-add
+// wrappers.  Stands in for the reference's wave reductions
+// (include/alphasparse/common_dcu.h:33-164), written for CDNA4's 64-lane waves.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace asamd {
+
+constexpr int kWave = 64;
+constexpr int kXcds = 8;  // MI355X: 8 accelerator complex dies, one L2 each
+
+// Workgroups are handed to the XCDs round-robin (workgroup i runs on XCD
+// i % 8).  Kernels whose neighbouring workgroups share gathered operands want
+// neighbours on the SAME XCD so the shared lines sit in one L2: this maps the
+// hardware workgroup id to a logical id such that every XCD walks one
+// contiguous slab of logical ids.
+__device__ __forceinline__ unsigned xcd_contiguous_id(unsigned hw_id, unsigned nblocks) {
+  const unsigned per = nblocks / kXcds;
+  const unsigned rem = nblocks % kXcds;
+  const unsigned xcd = hw_id % kXcds;
+  const unsigned local = hw_id / kXcds;
+  const unsigned start = xcd * per + (xcd < rem ? xcd : rem);
+  return start + local;
+}
+
+__device__ __forceinline__ float fma_t(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+__device__ __forceinline__ double fma_t(double a, double b, double c) { return __builtin_fma(a, b, c); }
+
+// ---- DPP moves ------------------------------------------------------------
+// dpp_ctrl encodings (GCN3+/CDNA ISA): quad_perm = 0x00..0xFF, row_shr:n =
+// 0x110+n, row_ror:n = 0x120+n, row_mirror = 0x140, row_half_mirror = 0x141.
+template <int Ctrl>
+__device__ __forceinline__ float dpp_mov(float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), Ctrl, 0xF, 0xF, true));
+}
+template <int Ctrl>
+__device__ __forceinline__ double dpp_mov(double v) {
+  // a 64-bit value travels as two 32-bit halves
+  const uint64_t bits = __builtin_bit_cast(uint64_t, v);
+  const int lo = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)bits, Ctrl, 0xF, 0xF, true);
+  const int hi = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)(bits >> 32), Ctrl, 0xF, 0xF, true);
+  return __builtin_bit_cast(double, ((uint64_t)(uint32_t)hi << 32) | (uint64_t)(uint32_t)lo);
+}
+
+// Sum over aligned groups of W consecutive lanes (W a power of two, 1..64).
+// Every lane of the group ends up holding the group's total.  Up to 16 lanes
+// the exchange is pure DPP (quad permutes, then the half-row and row mirrors:
+// after the quad steps all four lanes of a quad hold the quad's total, so a
+// mirror hands each lane the total of the opposite half); the 32- and
+// 64-lane steps cross DPP rows and use the LDS crossbar (ds_bpermute through
+// __shfl_xor), which touches no LDS memory.
+template <int W, typename T>
+__device__ __forceinline__ T group_sum(T v) {
+  static_assert(W >= 1 && W <= 64 && (W & (W - 1)) == 0, "group width");
+  if constexpr (W >= 2) v += dpp_mov<0xB1>(v);   // quad_perm [1,0,3,2]
+  if constexpr (W >= 4) v += dpp_mov<0x4E>(v);   // quad_perm [2,3,0,1]
+  if constexpr (W >= 8) v += dpp_mov<0x141>(v);  // row_half_mirror: lane l <-> 7-l in each 8
+  if constexpr (W >= 16) v += dpp_mov<0x140>(v); // row_mirror: lane l <-> 15-l in each 16
+  if constexpr (W >= 32) v += __shfl_xor(v, 16, kWave);
+  if constexpr (W >= 64) v += __shfl_xor(v, 32, kWave);
+  return v;
+}
+
+// ---- 128-bit streaming loads ------------------------------------------------
+struct alignas(16) Int4 { int x, y, z, w; };
+struct alignas(16) Float4 { float x, y, z, w; };
+struct alignas(16) Double2 { double x, y; };
+
+}  // namespace asamd

@@ -1,0 +1,210 @@
+// CSR SpMM  C = alpha*A*B + beta*C  for gfx950 (wave64).
+//
+//   spmm_rowmajor_kernel<T, V>  unit stride along the dense columns (row-major
+//       B and C, or column-major with op(B) = B^T read as row-major): one wave
+//       per row of A and per chunk of 64*V dense columns; the row's
+//       (col, alpha*val) pairs are read coalesced 64 at a time and broadcast
+//       with v_readlane, so every B row is fetched with one wave-wide load of
+//       64*V contiguous elements; C is read-modified-written once.
+//       This is the layout the reference cannot run on the GPU at all
+//       (dcu_gemm_?_csr_row returns NOT_SUPPORTED,
+//       src/kernel/dcu/level3/mm/csrmm/dcu_gemm_x_csr_row.cpp:15-36).
+//   spmm_strided_kernel<T>      any strides: one lane per (row, dense column),
+//       lanes of a wave on consecutive rows, so column-major C is written
+//       coalesced and B(:, c) is gathered like an SpMV x.  Stands in for
+//       csr_gemm_plain_device (dcu_gemm_csr_col_plain.h:9-39).
+//
+// Arithmetic follows the row-major plain kernel
+// (src/plain/kernel/level3/mm/gemm/gemm_x_csr_row_plain.c:11-19): alpha is
+// folded into each value, products are accumulated with fma in entry order,
+// then C = beta*C + acc.  beta == 0 never reads C.
+
+#include <hip/hip_runtime.h>
+
+#include "alsparse_amd_kernels.h"
+#include "device_utils.hpp"
+
+using namespace asamd;
+
+constexpr int kSpmmBlock = 256;
+constexpr int kSpmmWaves = kSpmmBlock / kWave;
+
+template <typename T, int V>
+struct alignas(sizeof(T) * V) Vec {
+  T e[V];
+};
+
+template <typename T, int V>
+__device__ __forceinline__ Vec<T, V> load_vec(const T* p, bool vector_ok, int valid) {
+  Vec<T, V> r;
+  if (vector_ok && valid == V) {
+    r = *reinterpret_cast<const Vec<T, V>*>(p);
+  } else {
+#pragma unroll
+    for (int i = 0; i < V; ++i) r.e[i] = i < valid ? p[i] : T(0);
+  }
+  return r;
+}
+
+__device__ __forceinline__ float readlane_t(float v, int l) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l));
+}
+__device__ __forceinline__ double readlane_t(double v, int l) {
+  const uint64_t b = __builtin_bit_cast(uint64_t, v);
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)b, l);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(b >> 32), l);
+  return __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);
+}
+
+// grid.x covers rows (one wave each), grid.y covers chunks of 64*V columns.
+template <typename T, int V>
+__global__ __launch_bounds__(kSpmmBlock) void spmm_rowmajor_kernel(
+    int m, int n, T alpha, const T* __restrict__ val, const int* __restrict__ row_ptr,
+    const int* __restrict__ col_ind, int base, const T* __restrict__ B, int64_t ldb, T beta,
+    T* __restrict__ C, int64_t ldc, bool vector_ok) {
+  const int lane = threadIdx.x % kWave;
+  const int wave = threadIdx.x / kWave;
+  const unsigned bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  const int64_t row = (int64_t)bid * kSpmmWaves + wave;
+  if (row >= m) return;  // wave-uniform
+  const int c0 = (blockIdx.y * kWave + lane) * V;  // first dense column of this lane
+  int valid = n - c0;
+  valid = valid > V ? V : (valid < 0 ? 0 : valid);
+
+  const int64_t start = (int64_t)row_ptr[row] - base;
+  const int64_t end = (int64_t)row_ptr[row + 1] - base;
+  T acc[V];
+#pragma unroll
+  for (int i = 0; i < V; ++i) acc[i] = T(0);
+
+  for (int64_t j0 = start; j0 < end; j0 += kWave) {
+    const int64_t j = j0 + lane;
+    int my_col = 0;
+    T my_val = T(0);
+    if (j < end) {
+      my_col = col_ind[j] - base;
+      my_val = alpha * val[j];
+    }
+    const int cnt = (int)(end - j0 < kWave ? end - j0 : kWave);
+    int t = 0;
+    for (; t + 4 <= cnt; t += 4) {
+      Vec<T, V> b[4];
+      T a[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int col = __builtin_amdgcn_readlane(my_col, t + u);
+        a[u] = readlane_t(my_val, t + u);
+        b[u] = load_vec<T, V>(B + (int64_t)col * ldb + c0, vector_ok, valid);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+#pragma unroll
+        for (int i = 0; i < V; ++i) acc[i] = fma_t(a[u], b[u].e[i], acc[i]);
+      }
+    }
+    for (; t < cnt; ++t) {
+      const int col = __builtin_amdgcn_readlane(my_col, t);
+      const T a = readlane_t(my_val, t);
+      const Vec<T, V> b = load_vec<T, V>(B + (int64_t)col * ldb + c0, vector_ok, valid);
+#pragma unroll
+      for (int i = 0; i < V; ++i) acc[i] = fma_t(a, b.e[i], acc[i]);
+    }
+  }
+
+  T* crow = C + row * ldc + c0;
+  if (vector_ok && valid == V) {
+    Vec<T, V> out;
+    if (beta == T(0)) {
+#pragma unroll
+      for (int i = 0; i < V; ++i) out.e[i] = acc[i];
+    } else {
+      const Vec<T, V> old = *reinterpret_cast<const Vec<T, V>*>(crow);
+#pragma unroll
+      for (int i = 0; i < V; ++i) out.e[i] = fma_t(beta, old.e[i], acc[i]);
+    }
+    *reinterpret_cast<Vec<T, V>*>(crow) = out;
+  } else {
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      if (i < valid) crow[i] = beta == T(0) ? acc[i] : fma_t(beta, crow[i], acc[i]);
+    }
+  }
+}
+
+// One lane per (row, dense column); blockDim = (64 rows, 4 columns).
+template <typename T>
+__global__ __launch_bounds__(kSpmmBlock) void spmm_strided_kernel(
+    int m, int n, T alpha, const T* __restrict__ val, const int* __restrict__ row_ptr,
+    const int* __restrict__ col_ind, int base, const T* __restrict__ B, int64_t sbr, int64_t sbc,
+    T beta, T* __restrict__ C, int64_t scr, int64_t scc) {
+  const int64_t row = (int64_t)blockIdx.x * kWave + threadIdx.x;
+  if (row >= m) return;
+  const int64_t start = (int64_t)row_ptr[row] - base;
+  const int64_t end = (int64_t)row_ptr[row + 1] - base;
+  for (int64_t c = (int64_t)blockIdx.y * blockDim.y + threadIdx.y; c < n;
+       c += (int64_t)gridDim.y * blockDim.y) {
+    T acc = T(0);
+    for (int64_t j = start; j < end; ++j) {
+      const int64_t col = (int64_t)col_ind[j] - base;
+      acc = fma_t(alpha * val[j], B[col * sbr + c * sbc], acc);
+    }
+    T* out = C + row * scr + c * scc;
+    *out = beta == T(0) ? acc : fma_t(beta, *out, acc);
+  }
+}
+
+template <typename T>
+static int csrmm_impl(hipStream_t s, int m, int n, int k, int nnz, T alpha, const T* val,
+                      const int* rp, const int* ci, int base, const T* B, T beta, T* C,
+                      const asamd_dense_strides* st) {
+  (void)k;
+  (void)nnz;
+  if (!val || !rp || !ci || !B || !C || !st || m <= 0 || n <= 0) return hipErrorInvalidValue;
+  if (st->b_col_stride == 1 && st->c_col_stride == 1) {
+    const int64_t ldb = st->b_row_stride, ldc = st->c_row_stride;
+    const unsigned gx = (unsigned)(((int64_t)m + kSpmmWaves - 1) / kSpmmWaves);
+    // widest per-lane vector that still gives every lane of a wave work
+    int V = 1;
+    if (n >= 4 * kWave) V = 4;
+    else if (n >= 2 * kWave) V = 2;
+    const size_t vbytes = (size_t)V * sizeof(T);
+    const bool vector_ok = V > 1 && ((uintptr_t)B % vbytes == 0) && ((uintptr_t)C % vbytes == 0) &&
+                           (ldb % V == 0) && (ldc % V == 0);
+    const unsigned gy = (unsigned)((n + kWave * V - 1) / (kWave * V));
+    const dim3 grid(gx, gy);
+    if (V == 4)
+      spmm_rowmajor_kernel<T, 4><<<grid, kSpmmBlock, 0, s>>>(m, n, alpha, val, rp, ci, base, B, ldb,
+                                                             beta, C, ldc, vector_ok);
+    else if (V == 2)
+      spmm_rowmajor_kernel<T, 2><<<grid, kSpmmBlock, 0, s>>>(m, n, alpha, val, rp, ci, base, B, ldb,
+                                                             beta, C, ldc, vector_ok);
+    else
+      spmm_rowmajor_kernel<T, 1><<<grid, kSpmmBlock, 0, s>>>(m, n, alpha, val, rp, ci, base, B, ldb,
+                                                             beta, C, ldc, false);
+  } else {
+    const dim3 block(kWave, kSpmmBlock / kWave);
+    unsigned gy = (unsigned)((n + block.y - 1) / block.y);
+    if (gy > 65535u) gy = 65535u;
+    const dim3 grid((unsigned)(((int64_t)m + kWave - 1) / kWave), gy);
+    spmm_strided_kernel<T><<<grid, block, 0, s>>>(m, n, alpha, val, rp, ci, base, B,
+                                                  st->b_row_stride, st->b_col_stride, beta, C,
+                                                  st->c_row_stride, st->c_col_stride);
+  }
+  return hipGetLastError();
+}
+
+extern "C" int asamd_s_csrmm(hipStream_t stream, int32_t m, int32_t n, int32_t k, int32_t nnz,
+                             float alpha, const float* val, const int32_t* row_ptr,
+                             const int32_t* col_ind, int32_t base, const float* B, float beta,
+                             float* C, const asamd_dense_strides* strides) {
+  return csrmm_impl<float>(stream, m, n, k, nnz, alpha, val, row_ptr, col_ind, base, B, beta, C,
+                           strides);
+}
+
+extern "C" int asamd_d_csrmm(hipStream_t stream, int32_t m, int32_t n, int32_t k, int32_t nnz,
+                             double alpha, const double* val, const int32_t* row_ptr,
+                             const int32_t* col_ind, int32_t base, const double* B, double beta,
+                             double* C, const asamd_dense_strides* strides) {
+  return csrmm_impl<double>(stream, m, n, k, nnz, alpha, val, row_ptr, col_ind, base, B, beta, C,
+                            strides);
+}

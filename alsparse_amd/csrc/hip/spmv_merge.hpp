@@ -1,0 +1,236 @@
+// Merge-path CSR SpMV for gfx950 (wave64).
+//
+// The work list is the merge of the m row-end offsets with the nnz entry
+// indices (m + nnz items).  Every workgroup owns kMergeItems consecutive items
+// of that list, every thread kMergeIpt consecutive items of its workgroup's
+// share, so the load is balanced whatever the row-length distribution is: a
+// 200 000-entry row simply spans ~100 workgroups, a run of empty rows costs
+// one item each.
+//
+//   1. merge_partition_kernel   one binary search per workgroup boundary over
+//                               row_ptr: first row not finished before the
+//                               boundary (cached by the analysis when the
+//                               structure is promised fixed).
+//   2. spmv_merge_kernel        coalesced col/val streaming, x gathers,
+//                               products and row ends staged in LDS; each
+//                               thread walks its items, finished rows go to an
+//                               LDS row buffer, the unfinished tail of each
+//                               thread is combined by a segmented scan (wave
+//                               shuffles, then across the four waves in order);
+//                               rows finished inside the workgroup are written
+//                               coalesced as y = beta*y + alpha*sum; the
+//                               workgroup's unfinished tail goes to a carry slot.
+//   3. merge_fixup_kernel       adds the carries of all workgroups that a row
+//                               crossed, in workgroup order.
+//
+// No floating-point atomics anywhere: results are identical from run to run.
+// The reference has no counterpart (its CSR-adaptive row blocks,
+// src/util_cpp/alphasparse_dcu_x_csrmv_analysis.cpp:58-267, are never read by
+// a kernel); the arithmetic per entry is that of
+// src/kernel/dcu/level2/mv/csrmv/dcu_gemv_vector.h:43-54.
+#pragma once
+
+#include "device_utils.hpp"
+
+namespace asamd {
+
+constexpr int kMergeThreads = 256;
+constexpr int kMergeIpt = 8;
+constexpr int kMergeItems = kMergeThreads * kMergeIpt;  // 2048 items per workgroup
+constexpr int kMergeWaves = kMergeThreads / kWave;
+
+// LDS index with one pad word per 32 so that lanes reading at a stride of
+// kMergeIpt words fall into distinct banks.
+__device__ __forceinline__ int lds_pad(int i) { return i + (i >> 5); }
+
+// block_row[b] = number of rows whose end offset is consumed before merge
+// diagonal b*kMergeItems, for b in [0, nblocks].
+__global__ __launch_bounds__(256) void merge_partition_kernel(int m, int nnz,
+                                                              const int* __restrict__ row_ptr,
+                                                              int base, int nblocks,
+                                                              int* __restrict__ block_row) {
+  const int b = blockIdx.x * blockDim.x + threadIdx.x;
+  if (b > nblocks) return;
+  const int64_t total = (int64_t)m + nnz;
+  int64_t d = (int64_t)b * kMergeItems;
+  if (d > total) d = total;
+  int64_t lo = d > nnz ? d - nnz : 0;
+  int64_t hi = d < m ? d : m;
+  while (lo < hi) {
+    const int64_t mid = (lo + hi) >> 1;
+    // row `mid` is finished before the diagonal iff its end offset does not
+    // exceed the number of entries consumed alongside mid+1 rows
+    if ((int64_t)row_ptr[mid + 1] - base <= d - mid - 1) {
+      lo = mid + 1;
+    } else {
+      hi = mid;
+    }
+  }
+  block_row[b] = (int)lo;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kMergeThreads) void spmv_merge_kernel(
+    int m, int nnz, T alpha, const T* __restrict__ val, const int* __restrict__ row_ptr,
+    const int* __restrict__ col_ind, const T* __restrict__ x, T beta, T* __restrict__ y, int base,
+    const int* __restrict__ block_row, int* __restrict__ carry_row, T* __restrict__ carry_val) {
+  __shared__ int s_rend[kMergeItems + 1];           // row ends, local to this workgroup's entry range
+  __shared__ T s_prod[kMergeItems + kMergeItems / 32 + 1];
+  __shared__ T s_rsum[kMergeItems];                 // totals of rows finished here
+  __shared__ int s_crow[kMergeThreads];             // per-thread unfinished row
+  __shared__ T s_cval[kMergeThreads];               // ... and its scanned partial sum
+  __shared__ int s_wrow[kMergeWaves];
+  __shared__ T s_wval[kMergeWaves];
+
+  const int tid = threadIdx.x;
+  const unsigned b = blockIdx.x;
+  const int64_t total = (int64_t)m + nnz;
+  const int64_t d0 = (int64_t)b * kMergeItems;
+  const int64_t d1 = d0 + kMergeItems < total ? d0 + kMergeItems : total;
+  const int row_b = block_row[b];
+  const int row_e = block_row[b + 1];
+  const int64_t nnz_b = d0 - row_b;
+  const int64_t nnz_e = d1 - row_e;
+  int rows_cnt = row_e - row_b;
+  int nnz_cnt = (int)(nnz_e - nnz_b);
+  // coordinates that do not describe this row_ptr (a stale cache) must not
+  // drive any access out of bounds: clamp to what the LDS arrays and the
+  // global arrays hold, results are then wrong but the launch is safe
+  if (rows_cnt < 0 || rows_cnt > kMergeItems || row_b < 0 || row_e > m) rows_cnt = 0;
+  if (nnz_cnt < 0 || nnz_cnt > kMergeItems || nnz_b < 0 || nnz_e > nnz) nnz_cnt = 0;
+  const int items = rows_cnt + nnz_cnt;
+
+  // ---- stage row ends (one extra: the row still open at the end) ----------
+  for (int i = tid; i <= rows_cnt; i += kMergeThreads) {
+    const int64_t r = (int64_t)row_b + i;
+    const int64_t e = r < m ? (int64_t)row_ptr[r + 1] - base - nnz_b : (int64_t)kMergeItems + 1;
+    s_rend[i] = e > kMergeItems ? kMergeItems + 1 : (e < 0 ? 0 : (int)e);
+  }
+  // ---- stream entries, gather x, stage products ----------------------------
+  {
+    const T* __restrict__ xb = x - base;
+    T v[kMergeIpt];
+    int c[kMergeIpt];
+#pragma unroll
+    for (int s = 0; s < kMergeIpt; ++s) {
+      const int k = tid + s * kMergeThreads;
+      if (k < nnz_cnt) {
+        v[s] = val[nnz_b + k];
+        c[s] = col_ind[nnz_b + k];
+      }
+    }
+    T xv[kMergeIpt];
+#pragma unroll
+    for (int s = 0; s < kMergeIpt; ++s) {
+      const int k = tid + s * kMergeThreads;
+      if (k < nnz_cnt) xv[s] = xb[c[s]];
+    }
+#pragma unroll
+    for (int s = 0; s < kMergeIpt; ++s) {
+      const int k = tid + s * kMergeThreads;
+      if (k < nnz_cnt) s_prod[lds_pad(k)] = v[s] * xv[s];
+    }
+  }
+  __syncthreads();
+
+  // ---- this thread's start on the workgroup-local merge path ---------------
+  int dt = tid * kMergeIpt;
+  if (dt > items) dt = items;
+  int dt_end = dt + kMergeIpt;
+  if (dt_end > items) dt_end = items;
+  int lo = dt > nnz_cnt ? dt - nnz_cnt : 0;
+  int hi = dt < rows_cnt ? dt : rows_cnt;
+  while (lo < hi) {
+    const int mid = (lo + hi) >> 1;
+    if (s_rend[mid] <= dt - mid - 1) {
+      lo = mid + 1;
+    } else {
+      hi = mid;
+    }
+  }
+  int i = lo;       // local row
+  int j = dt - lo;  // local entry
+  const int first_row = i;
+  bool finished_any = false;
+  T acc = T(0);
+#pragma unroll
+  for (int step = 0; step < kMergeIpt; ++step) {
+    if (dt + step < dt_end) {
+      const bool take_entry = j < nnz_cnt && (i >= rows_cnt || j < s_rend[i]);
+      if (take_entry) {
+        acc += s_prod[lds_pad(j)];
+        ++j;
+      } else if (i < rows_cnt) {
+        s_rsum[i] = acc;  // exactly one thread finishes a given row
+        acc = T(0);
+        finished_any = true;
+        ++i;
+      }
+    }
+  }
+
+  // ---- segmented inclusive scan of the unfinished tails, key = row --------
+  // keys are non-decreasing in thread order, so "same key d lanes below"
+  // implies every lane in between has that key too
+  const int lane = tid % kWave;
+  const int wave = tid / kWave;
+  const int key = i;
+  T tail = acc;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const T up = __shfl_up(tail, d, kWave);
+    const int kup = __shfl_up(key, d, kWave);
+    if (lane >= d && kup == key) tail += up;
+  }
+  if (lane == kWave - 1) {
+    s_wrow[wave] = key;
+    s_wval[wave] = tail;
+  }
+  __syncthreads();
+  for (int w = wave - 1; w >= 0; --w) {
+    if (s_wrow[w] != key) break;
+    tail += s_wval[w];
+  }
+  s_crow[tid] = key;
+  s_cval[tid] = tail;
+  __syncthreads();
+
+  // the first row a thread finished may have been started by the threads below
+  if (finished_any && tid > 0 && s_crow[tid - 1] == first_row) s_rsum[first_row] += s_cval[tid - 1];
+  if (tid == kMergeThreads - 1) {
+    carry_row[b] = row_b + key;  // == row_e: the row still open, or m
+    carry_val[b] = tail;
+  }
+  __syncthreads();
+
+  // ---- rows finished here: y = beta*y + alpha*sum, coalesced ----------------
+  for (int r = tid; r < rows_cnt; r += kMergeThreads) {
+    const int64_t row = (int64_t)row_b + r;
+    const T sum = s_rsum[r];
+    if (beta == T(0)) {
+      y[row] = alpha * sum;
+    } else {
+      y[row] = fma_t(beta, y[row], alpha * sum);
+    }
+  }
+}
+
+// Row r may have been open across several consecutive workgroups; their
+// carries are summed in workgroup order by the thread of the first of them and
+// added to the value written by the workgroup that finished the row.
+template <typename T>
+__global__ __launch_bounds__(256) void merge_fixup_kernel(int nblocks, int m, T alpha,
+                                                          const int* __restrict__ carry_row,
+                                                          const T* __restrict__ carry_val,
+                                                          T* __restrict__ y) {
+  const int b = blockIdx.x * blockDim.x + threadIdx.x;
+  if (b >= nblocks) return;
+  const int r = carry_row[b];
+  if (r < 0 || r >= m) return;
+  if (b > 0 && carry_row[b - 1] == r) return;
+  T s = T(0);
+  for (int bb = b; bb < nblocks && carry_row[bb] == r; ++bb) s += carry_val[bb];
+  if (s != T(0)) y[r] += alpha * s;
+}
+
+}  // namespace asamd

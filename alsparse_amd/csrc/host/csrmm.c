@@ -1,0 +1,18 @@
+/* Device SpMM entry points (raw device arrays). */
+#include "internal.h"
+
+#define ASAMD_T float
+#define ASAMD_S s
+#define ASAMD_KERNEL_CSRMM asamd_s_csrmm
+#include "csrmm.inc"
+#undef ASAMD_T
+#undef ASAMD_S
+#undef ASAMD_KERNEL_CSRMM
+
+#define ASAMD_T double
+#define ASAMD_S d
+#define ASAMD_KERNEL_CSRMM asamd_d_csrmm
+#include "csrmm.inc"
+#undef ASAMD_T
+#undef ASAMD_S
+#undef ASAMD_KERNEL_CSRMM

@@ -1,0 +1,67 @@
+/* alphasparse_?_mv / alphasparse_?_mm: the reference's host-pointer entry
+ * points (include/alphasparse/spapi.h:685-699, :899-923).  In the reference
+ * they run OpenMP CPU kernels; here the multiplication runs on the GPU: the
+ * matrix is mirrored to the device on first use, x / X is staged in, y / Y
+ * staged out on the default handle's stream, and the call returns after the
+ * result has landed in host memory (these entry points are synchronous in the
+ * reference too).  There is no CPU compute path: without a usable device the
+ * status is the mapped HIP error. */
+#include <stdlib.h>
+
+#include "internal.h"
+
+/* Make sure A has a device mirror built by this library and return its record. */
+static alphasparse_status_t asamd_host_prepare(const alphasparse_matrix_t A, size_t val_size,
+                                               alphasparse_dcu_handle_t *h, asamd_record **rec) {
+  alphasparse_status_t st = asamd_default_handle(h);
+  if (st != ALPHA_SPARSE_STATUS_SUCCESS) return st;
+  spmat_csr_s_t *m = (spmat_csr_s_t *)A->mat; /* s and d payloads share the layout */
+  asamd_record *r = m->d_row_ptr ? asamd_registry_find(ASAMD_KEY_MATRIX, m->d_row_ptr) : NULL;
+  if (!r) {
+    st = val_size == sizeof(float) ? host2device_s_csr(A) : host2device_d_csr(A);
+    if (st != ALPHA_SPARSE_STATUS_SUCCESS) return st;
+    r = asamd_registry_find(ASAMD_KEY_MATRIX, m->d_row_ptr);
+    if (!r) return ALPHA_SPARSE_STATUS_INTERNAL_ERROR;
+  }
+  *rec = r;
+  return ALPHA_SPARSE_STATUS_SUCCESS;
+}
+
+/* Grow the record's device staging buffers to at least the given sizes. */
+static alphasparse_status_t asamd_host_stage(asamd_record *rec, size_t in_bytes, size_t out_bytes) {
+  if (rec->d_in_bytes < in_bytes) {
+    if (rec->d_in) (void)hipFree(rec->d_in);
+    rec->d_in = NULL;
+    rec->d_in_bytes = 0;
+    ASAMD_HIP_STATUS(hipMalloc(&rec->d_in, in_bytes));
+    rec->d_in_bytes = in_bytes;
+  }
+  if (rec->d_out_bytes < out_bytes) {
+    if (rec->d_out) (void)hipFree(rec->d_out);
+    rec->d_out = NULL;
+    rec->d_out_bytes = 0;
+    ASAMD_HIP_STATUS(hipMalloc(&rec->d_out, out_bytes));
+    rec->d_out_bytes = out_bytes;
+  }
+  return ALPHA_SPARSE_STATUS_SUCCESS;
+}
+
+#define ASAMD_T float
+#define ASAMD_S s
+#define ASAMD_CSR spmat_csr_s_t
+#define ASAMD_DT ALPHA_SPARSE_DATATYPE_FLOAT
+#include "host_api.inc"
+#undef ASAMD_T
+#undef ASAMD_S
+#undef ASAMD_CSR
+#undef ASAMD_DT
+
+#define ASAMD_T double
+#define ASAMD_S d
+#define ASAMD_CSR spmat_csr_d_t
+#define ASAMD_DT ALPHA_SPARSE_DATATYPE_DOUBLE
+#include "host_api.inc"
+#undef ASAMD_T
+#undef ASAMD_S
+#undef ASAMD_CSR
+#undef ASAMD_DT

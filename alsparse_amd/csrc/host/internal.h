@@ -1,0 +1,62 @@
+/* Internals of the C host library: the analysis registry, the process-wide
+ * default handle used by the host-pointer entry points, and small helpers.
+ * Nothing here is part of the drop-in ABI. */
+#ifndef ALSPARSE_AMD_HOST_INTERNAL_H
+#define ALSPARSE_AMD_HOST_INTERNAL_H
+
+#include "alpha_spblas_dcu.h"
+#include "alsparse_amd_kernels.h"
+
+/* How an analysis record is looked up. */
+typedef enum {
+  ASAMD_KEY_MATRIX = 0, /* by alphasparse_matrix_t: device mirror owned by the library      */
+  ASAMD_KEY_INFO = 1,   /* by alphasparse_dcu_mat_info_t: explicit *_csrmv_analysis call      */
+  ASAMD_KEY_LAZY = 2    /* by csr_row_ptr: first multiply without analysis, structure unknown */
+} asamd_key_kind;
+
+typedef struct asamd_record {
+  asamd_key_kind kind;
+  const void *key;
+  /* what the plan was built for; a lookup must match all of these */
+  const void *row_ptr;
+  const void *col_ind;
+  int32_t m, n, nnz, base, val_size;
+  asamd_csr_plan *plan;
+  /* host-pointer entry points: device staging for x / y (ASAMD_KEY_MATRIX only) */
+  void *d_in;
+  size_t d_in_bytes;
+  void *d_out;
+  size_t d_out_bytes;
+  struct asamd_record *next;
+} asamd_record;
+
+/* All registry calls are serialised by one mutex; records are returned
+ * unlocked, which is safe as long as a matrix / info is not destroyed while
+ * another thread multiplies with it (the reference gives no such guarantee
+ * either). */
+asamd_record *asamd_registry_find(asamd_key_kind kind, const void *key);
+asamd_record *asamd_registry_insert(asamd_key_kind kind, const void *key);
+void asamd_registry_erase(asamd_key_kind kind, const void *key);
+void asamd_record_release_device(asamd_record *rec);
+
+/* Plan for a multiply through the raw-pointer API: explicit analysis if `info`
+ * is known and matches, else the lazy cache (created on first use). */
+alphasparse_status_t asamd_plan_for_call(alphasparse_dcu_handle_t handle, const void *info,
+                                         const void *row_ptr, const void *col_ind, int32_t m,
+                                         int32_t n, int32_t nnz, int32_t base, int32_t val_size,
+                                         asamd_csr_plan **plan);
+
+/* Process-wide handle for alphasparse_?_mv / _mm (host pointers). */
+alphasparse_status_t asamd_default_handle(alphasparse_dcu_handle_t *handle);
+
+/* ALSPARSE_AMD_SPMV_ALGO = auto | vector | rowconst | merge | scalar */
+int asamd_env_algo(void);
+
+#define ASAMD_HIP_STATUS(expr)                                           \
+  do {                                                                   \
+    hipError_t asamd_e_ = (hipError_t)(expr);                            \
+    if (asamd_e_ != hipSuccess)                                          \
+      return get_alphasparse_dcu_status_for_hip_status(asamd_e_);        \
+  } while (0)
+
+#endif

@@ -1,0 +1,229 @@
+/*
+ * alphasparse.h -- host-facing C API of the CSR SpMV / SpMM path.
+ *
+ * This header re-declares, with identical enum values, struct field order and
+ * prototypes, the part of AlphaSparse's public C API that the CSR
+ * matrix-vector / matrix-matrix path needs, so that a program written against
+ * the reference headers links against libalpha_spblas.so from this repository
+ * without source changes.  Only the s/d (fp32/fp64) CSR entry points exist.
+ *
+ * Every declaration cites the reference declaration it replaces
+ * (paths relative to the AlphaSparse source tree).
+ *
+ * Behavioural difference to know about: alphasparse_?_mv / alphasparse_?_mm
+ * take HOST pointers exactly as in the reference, but the multiplication runs
+ * on the GPU (device mirror of the matrix, x/B staged in, y/C staged out).
+ * There is no CPU compute path in this library: without a usable HIP device
+ * these entry points return ALPHA_SPARSE_STATUS_EXECUTION_FAILED.
+ */
+#ifndef ALSPARSE_AMD_ALPHASPARSE_H
+#define ALSPARSE_AMD_ALPHASPARSE_H
+
+#include <stdbool.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- scalar / index types: include/alphasparse/types.h:59-61 ------------ */
+#ifndef ALPHA_INT
+#define ALPHA_INT int32_t
+#endif
+
+/* ---- status codes: include/alphasparse/spdef.h:8-19 ---------------------- */
+typedef enum {
+  ALPHA_SPARSE_STATUS_SUCCESS = 0,
+  ALPHA_SPARSE_STATUS_NOT_INITIALIZED = 1,
+  ALPHA_SPARSE_STATUS_ALLOC_FAILED = 2,
+  ALPHA_SPARSE_STATUS_INVALID_VALUE = 3,
+  ALPHA_SPARSE_STATUS_EXECUTION_FAILED = 4,
+  ALPHA_SPARSE_STATUS_INTERNAL_ERROR = 5,
+  ALPHA_SPARSE_STATUS_NOT_SUPPORTED = 6,
+  ALPHA_SPARSE_STATUS_INVALID_POINTER = 7,
+  ALPHA_SPARSE_STATUS_INVALID_HANDLE = 8
+} alphasparse_status_t;
+
+/* ---- op(A): include/alphasparse/spdef.h:22-27 ---------------------------- */
+typedef enum {
+  ALPHA_SPARSE_OPERATION_NON_TRANSPOSE = 0,
+  ALPHA_SPARSE_OPERATION_TRANSPOSE = 1,
+  ALPHA_SPARSE_OPERATION_CONJUGATE_TRANSPOSE = 2
+} alphasparse_operation_t;
+
+/* ---- matrix type: include/alphasparse/spdef.h:32-41 ---------------------- */
+typedef enum {
+  ALPHA_SPARSE_MATRIX_TYPE_GENERAL = 0,
+  ALPHA_SPARSE_MATRIX_TYPE_SYMMETRIC = 1,
+  ALPHA_SPARSE_MATRIX_TYPE_HERMITIAN = 2,
+  ALPHA_SPARSE_MATRIX_TYPE_TRIANGULAR = 3,
+  ALPHA_SPARSE_MATRIX_TYPE_DIAGONAL = 4,
+  ALPHA_SPARSE_MATRIX_TYPE_BLOCK_TRIANGULAR = 5,
+  ALPHA_SPARSE_MATRIX_TYPE_BLOCK_DIAGONAL = 6
+} alphasparse_matrix_type_t;
+
+/* ---- index base: include/alphasparse/spdef.h:46-50 ----------------------- */
+typedef enum {
+  ALPHA_SPARSE_INDEX_BASE_ZERO = 0,
+  ALPHA_SPARSE_INDEX_BASE_ONE = 1
+} alphasparse_index_base_t;
+
+/* ---- fill / diag: include/alphasparse/spdef.h:55-69 ---------------------- */
+typedef enum {
+  ALPHA_SPARSE_FILL_MODE_LOWER = 0,
+  ALPHA_SPARSE_FILL_MODE_UPPER = 1
+} alphasparse_fill_mode_t;
+
+typedef enum {
+  ALPHA_SPARSE_DIAG_NON_UNIT = 0,
+  ALPHA_SPARSE_DIAG_UNIT = 1
+} alphasparse_diag_type_t;
+
+/* ---- dense layout: include/alphasparse/spdef.h:73-77 --------------------- */
+typedef enum {
+  ALPHA_SPARSE_LAYOUT_ROW_MAJOR = 0,
+  ALPHA_SPARSE_LAYOUT_COLUMN_MAJOR = 1
+} alphasparse_layout_t;
+
+/* ---- storage format tags: include/alphasparse/spdef.h:120-133 ------------ */
+typedef enum {
+  ALPHA_SPARSE_FORMAT_COO = 0,
+  ALPHA_SPARSE_FORMAT_CSR = 1,
+  ALPHA_SPARSE_FORMAT_CSC = 2,
+  ALPHA_SPARSE_FORMAT_BSR = 3,
+  ALPHA_SPARSE_FORMAT_SKY = 4,
+  ALPHA_SPARSE_FORMAT_DIA = 5,
+  ALPHA_SPARSE_FORMAT_ELL = 6,
+  ALPHA_SPARSE_FORMAT_GEBSR = 7,
+  ALPHA_SPARSE_FORMAT_HYB = 8,
+  ALPHA_SPARSE_FORMAT_COO_AOS = 9,
+  ALPHA_SPARSE_FORMAT_CSR5 = 10
+} alphasparse_format_t;
+
+/* ---- value type tags: include/alphasparse/spdef.h:137-143 ---------------- */
+typedef enum {
+  ALPHA_SPARSE_DATATYPE_FLOAT = 0,
+  ALPHA_SPARSE_DATATYPE_DOUBLE = 1,
+  ALPHA_SPARSE_DATATYPE_FLOAT_COMPLEX = 2,
+  ALPHA_SPARSE_DATATYPE_DOUBLE_COMPLEX = 3
+} alphasparse_datatype_t;
+
+/* ---- type-erased matrix handle: include/alphasparse/spdef.h:160-172 ------
+ * `inspector` and `dcu_info` are never dereferenced by this library unless it
+ * wrote them itself: handles built by other code leave them uninitialised. */
+typedef void *alpha_internal_spmat;
+
+typedef struct {
+  alpha_internal_spmat mat;
+  alphasparse_format_t format;
+  alphasparse_datatype_t datatype;
+  void *inspector;
+  void *dcu_info;
+} alphasparse_matrix;
+
+typedef alphasparse_matrix *alphasparse_matrix_t;
+
+/* ---- host-side descriptor (passed by value): spdef.h:178-183 ------------- */
+struct alpha_matrix_descr {
+  alphasparse_matrix_type_t type;
+  alphasparse_fill_mode_t mode;
+  alphasparse_diag_type_t diag;
+};
+
+/* ---- CSR payloads: include/alphasparse/spmat.h:174-188 and :203-216 ------
+ * rows_end always aliases rows_start + 1 (three-array CSR inside a four-array
+ * API, src/core/format/alphasparse_x_create_csr.c:25-29).  d_* is the device
+ * mirror filled by host2device_?_csr. */
+typedef struct {
+  float *values;
+  ALPHA_INT *rows_start;
+  ALPHA_INT *rows_end;
+  ALPHA_INT *col_indx;
+  ALPHA_INT rows;
+  ALPHA_INT cols;
+  bool ordered;
+  float *d_values;
+  ALPHA_INT *d_row_ptr;
+  ALPHA_INT *d_col_indx;
+} spmat_csr_s_t;
+
+typedef struct {
+  double *values;
+  ALPHA_INT *rows_start;
+  ALPHA_INT *rows_end;
+  ALPHA_INT *col_indx;
+  ALPHA_INT rows;
+  ALPHA_INT cols;
+  bool ordered;
+  double *d_values;
+  ALPHA_INT *d_row_ptr;
+  ALPHA_INT *d_col_indx;
+} spmat_csr_d_t;
+
+/* ---- handle construction -------------------------------------------------
+ * include/alphasparse/spapi.h:140-156; behaviour from
+ * src/core/format/alphasparse_x_create_csr.c:7-57: deep copy, indices shifted
+ * to base zero, nnz = rows_end[rows-1] - rows_start[0].  Unlike the reference
+ * the device-side fields are zero-initialised. */
+alphasparse_status_t alphasparse_s_create_csr(alphasparse_matrix_t *A,
+                                              const alphasparse_index_base_t indexing,
+                                              const ALPHA_INT rows, const ALPHA_INT cols,
+                                              ALPHA_INT *rows_start, ALPHA_INT *rows_end,
+                                              ALPHA_INT *col_indx, float *values);
+alphasparse_status_t alphasparse_d_create_csr(alphasparse_matrix_t *A,
+                                              const alphasparse_index_base_t indexing,
+                                              const ALPHA_INT rows, const ALPHA_INT cols,
+                                              ALPHA_INT *rows_start, ALPHA_INT *rows_end,
+                                              ALPHA_INT *col_indx, double *values);
+
+/* include/alphasparse/spapi.h:352-368; src/core/format/alphasparse_x_export_csr.c:5-26.
+ * Returns borrowed internal pointers; always reports base zero. */
+alphasparse_status_t alphasparse_s_export_csr(const alphasparse_matrix_t source,
+                                              alphasparse_index_base_t *indexing,
+                                              ALPHA_INT *rows, ALPHA_INT *cols,
+                                              ALPHA_INT **rows_start, ALPHA_INT **rows_end,
+                                              ALPHA_INT **col_indx, float **values);
+alphasparse_status_t alphasparse_d_export_csr(const alphasparse_matrix_t source,
+                                              alphasparse_index_base_t *indexing,
+                                              ALPHA_INT *rows, ALPHA_INT *cols,
+                                              ALPHA_INT **rows_start, ALPHA_INT **rows_end,
+                                              ALPHA_INT **col_indx, double **values);
+
+/* include/alphasparse/spapi.h:288; src/core/op_/alphasparse_destroy.c:186-195.
+ * Also releases the device mirror and any cached analysis of the handle. */
+alphasparse_status_t alphasparse_destroy(alphasparse_matrix_t A);
+
+/* ---- y = alpha*op(A)*x + beta*y ------------------------------------------
+ * include/alphasparse/spapi.h:685-699; validation order from
+ * src/core/op/level2/alphasparse_x_mv.c:1662-1691.  x and y are host arrays. */
+alphasparse_status_t alphasparse_s_mv(const alphasparse_operation_t operation, const float alpha,
+                                      const alphasparse_matrix_t A,
+                                      const struct alpha_matrix_descr descr, const float *x,
+                                      const float beta, float *y);
+alphasparse_status_t alphasparse_d_mv(const alphasparse_operation_t operation, const double alpha,
+                                      const alphasparse_matrix_t A,
+                                      const struct alpha_matrix_descr descr, const double *x,
+                                      const double beta, double *y);
+
+/* ---- Y = alpha*op(A)*X + beta*Y ------------------------------------------
+ * include/alphasparse/spapi.h:899-923; validation order from
+ * src/core/op/level3/alphasparse_x_mm.c:2305-2338.  x and y are host arrays. */
+alphasparse_status_t alphasparse_s_mm(const alphasparse_operation_t operation, const float alpha,
+                                      const alphasparse_matrix_t A,
+                                      const struct alpha_matrix_descr descr,
+                                      const alphasparse_layout_t layout, const float *x,
+                                      const ALPHA_INT columns, const ALPHA_INT ldx,
+                                      const float beta, float *y, const ALPHA_INT ldy);
+alphasparse_status_t alphasparse_d_mm(const alphasparse_operation_t operation, const double alpha,
+                                      const alphasparse_matrix_t A,
+                                      const struct alpha_matrix_descr descr,
+                                      const alphasparse_layout_t layout, const double *x,
+                                      const ALPHA_INT columns, const ALPHA_INT ldx,
+                                      const double beta, double *y, const ALPHA_INT ldy);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* ALSPARSE_AMD_ALPHASPARSE_H */

@@ -1,0 +1,126 @@
+/*
+ * alsparse_amd_kernels.h -- the thin C-ABI layer between the C host library
+ * and the hand-written HIP kernels (gfx950, wave64).
+ *
+ * Everything here takes plain device pointers, sizes and a stream; no C++
+ * types cross the boundary.  Return value is a hipError_t cast to int
+ * (0 == hipSuccess).  The functions enqueue work on `stream` and return
+ * without synchronising unless stated otherwise.
+ *
+ * Each entry names the reference kernel or launch it stands in for
+ * (paths relative to the AlphaSparse source tree).
+ */
+#ifndef ALSPARSE_AMD_KERNELS_H
+#define ALSPARSE_AMD_KERNELS_H
+
+#ifndef __HIP_PLATFORM_AMD__
+#define __HIP_PLATFORM_AMD__ 1
+#endif
+#include <hip/hip_runtime_api.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* SpMV kernel families.  The reference has exactly one: a sub-wavefront per
+ * row (src/kernel/dcu/level2/mv/csrmv/dcu_gemv_vector.h:14-57), chosen
+ * unconditionally (src/kernel/dcu/level2/mv/csrmv/dcu_gemv_x_csr.cpp:21-31). */
+enum asamd_spmv_algo {
+  ASAMD_SPMV_AUTO = 0,     /* pick from the analysis                                */
+  ASAMD_SPMV_VECTOR = 1,   /* W lanes per row, W in {2..64} from the mean row length */
+  ASAMD_SPMV_ROWCONST = 2, /* every row has the same length L = 4*G: no row_ptr read */
+  ASAMD_SPMV_MERGE = 3,    /* merge-path split of (rows + nnz), LDS-staged products  */
+  ASAMD_SPMV_SCALAR = 4    /* one lane per row; diagnostic baseline                  */
+};
+
+#define ASAMD_HIST_BINS 33
+
+/* Row-length statistics gathered on the GPU.  hist[0] counts empty rows,
+ * hist[b] rows whose length lies in [2^(b-1), 2^b). */
+typedef struct {
+  int32_t m, n, nnz, base;
+  int32_t min_len, max_len;
+  int32_t const_len;    /* common row length, or -1                          */
+  int32_t first_offset; /* row_ptr[0] - base                                 */
+  int32_t algo;         /* enum asamd_spmv_algo chosen for this structure     */
+  int32_t vector_width; /* lanes per row when algo == VECTOR                  */
+  int32_t merge_blocks; /* workgroups of the merge-path kernel                */
+  int32_t trusted;      /* 1: structure promised fixed, coordinates cached    */
+  int64_t hist[ASAMD_HIST_BINS];
+} asamd_csr_stats;
+
+typedef struct asamd_csr_plan asamd_csr_plan;
+
+/* Row-length histogram, kernel choice and (trusted != 0) cached merge-path
+ * block coordinates.  Synchronises `stream` once to read the statistics.
+ * Replaces the host-side row-block builder
+ * src/util_cpp/alphasparse_dcu_x_csrmv_analysis.cpp:58-267, :348-379.
+ * val_size is sizeof(value type): 4 or 8. */
+int asamd_csr_plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t nnz,
+                          const int32_t *row_ptr, int32_t base, int32_t val_size, int32_t trusted,
+                          asamd_csr_plan **plan);
+void asamd_csr_plan_destroy(asamd_csr_plan *plan);
+const asamd_csr_stats *asamd_csr_plan_stats(const asamd_csr_plan *plan);
+/* Force a kernel family for later multiplies (AUTO restores the analysis'
+ * own choice).  Returns hipErrorInvalidValue if the structure cannot run it. */
+int asamd_csr_plan_set_algo(asamd_csr_plan *plan, int32_t algo);
+
+/* y = alpha*A*x + beta*y.  Stands in for csr_gemv_vector_dispatch,
+ * src/kernel/dcu/level2/mv/csrmv/dcu_gemv_vector.h:59-182.  `plan` must
+ * describe (m, n, nnz, base); beta == 0 skips the read of y. */
+int asamd_s_csrmv(hipStream_t stream, asamd_csr_plan *plan, float alpha, const float *val,
+                  const int32_t *row_ptr, const int32_t *col_ind, const float *x, float beta,
+                  float *y);
+int asamd_d_csrmv(hipStream_t stream, asamd_csr_plan *plan, double alpha, const double *val,
+                  const int32_t *row_ptr, const int32_t *col_ind, const double *x, double beta,
+                  double *y);
+
+/* Dense operand addressing for SpMM: element (r, c) of B is
+ * B[r*b_row_stride + c*b_col_stride], of C is C[r*c_row_stride + c*c_col_stride]. */
+typedef struct {
+  int64_t b_row_stride, b_col_stride;
+  int64_t c_row_stride, c_col_stride;
+} asamd_dense_strides;
+
+/* C = alpha*A*B + beta*C, A m x k CSR, B k x n, C m x n.  Stands in for
+ * dcu_gemm_?_csr_row (stub, src/kernel/dcu/level3/mm/csrmm/dcu_gemm_x_csr_row.cpp:15-36),
+ * gemm_col_plain_dispatch (dcu_gemm_csr_col_plain.h:42-61) and
+ * csrmmnt_general_device (dcu_gemm_x_csr_col_transB.cpp:39-108, :199-226). */
+int asamd_s_csrmm(hipStream_t stream, int32_t m, int32_t n, int32_t k, int32_t nnz, float alpha,
+                  const float *val, const int32_t *row_ptr, const int32_t *col_ind, int32_t base,
+                  const float *B, float beta, float *C,
+                  const asamd_dense_strides *strides);
+int asamd_d_csrmm(hipStream_t stream, int32_t m, int32_t n, int32_t k, int32_t nnz, double alpha,
+                  const double *val, const int32_t *row_ptr, const int32_t *col_ind, int32_t base,
+                  const double *B, double beta, double *C,
+                  const asamd_dense_strides *strides);
+
+/* coo_row[k] = r + base for k in [row_ptr[r]-base, row_ptr[r+1]-base).
+ * Defines on the GPU what src/core/format/convert_coo_x_csr.c:30-37 does on the host. */
+int asamd_csr2coo(hipStream_t stream, const int32_t *row_ptr, int32_t nnz, int32_t m,
+                  int32_t *coo_row, int32_t base);
+
+/* Longest row.  Synchronises `stream`; *width_host is a host int.
+ * src/core/format/convert_ell_x_coo.c:46-52. */
+int asamd_csr2ell_width(hipStream_t stream, int32_t m, const int32_t *row_ptr,
+                        int32_t *width_host);
+
+/* Column-major ELL, padding (value 0, index ell_base).
+ * src/core/format/convert_ell_x_coo.c:59-79. */
+int asamd_s_csr2ell(hipStream_t stream, int32_t m, const float *val, const int32_t *row_ptr,
+                    const int32_t *col_ind, int32_t csr_base, int32_t ell_base, int32_t width,
+                    float *ell_val, int32_t *ell_col);
+int asamd_d_csr2ell(hipStream_t stream, int32_t m, const double *val, const int32_t *row_ptr,
+                    const int32_t *col_ind, int32_t csr_base, int32_t ell_base, int32_t width,
+                    double *ell_val, int32_t *ell_col);
+
+/* Empty kernel; forces code-object load (src/util_cpp/handle.cpp:19, :113). */
+int asamd_warmup(hipStream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* ALSPARSE_AMD_KERNELS_H */

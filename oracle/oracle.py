@@ -1,0 +1,220 @@
+"""TEST INFRASTRUCTURE -- not part of the product.
+
+ctypes bindings of the CPU oracle (``liboracle.so``: reproducible rounding;
+``liboracle_fast.so``: the reference's build flags, for the timed baseline) and,
+where it was built, of the reference's own CPU kernels (``oracle/_ref``).
+Only tests/, ``__graft_entry__.smoke()`` and bench.py's ``cpu_baseline`` leg may
+import this module.
+"""
+import ctypes
+import os
+from ctypes import POINTER, Structure, byref, c_bool, c_double, c_float, c_int32, c_int64, c_void_p
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+_libs = {}
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(c_void_p)
+
+
+def _ct(dtype):
+    return c_float if np.dtype(dtype) == np.float32 else c_double
+
+
+def _pre(dtype):
+    return "s" if np.dtype(dtype) == np.float32 else "d"
+
+
+def lib(fast=False):
+    key = "fast" if fast else "o2"
+    if key not in _libs:
+        path = os.path.join(HERE, "liboracle_fast.so" if fast else "liboracle.so")
+        if not os.path.exists(path):
+            raise RuntimeError("%s missing: make -C oracle" % path)
+        L = ctypes.CDLL(path)
+        I, P = c_int32, c_void_p
+        for s, T in (("s", c_float), ("d", c_double)):
+            f = getattr(L, "oracle_%s_csrmv_plain" % s)
+            f.restype, f.argtypes = None, [I, P, P, P, P, T, P, T, P]
+            f = getattr(L, "oracle_%s_csrmv_omp" % s)
+            f.restype, f.argtypes = None, [I, P, P, P, P, T, P, T, P, I]
+            f = getattr(L, "oracle_%s_csrmv_f64acc" % s)
+            f.restype, f.argtypes = None, [I, P, P, P, P, c_double, P, c_double, P, P]
+            for n in ("row_plain", "row_omp", "col_plain"):
+                f = getattr(L, "oracle_%s_csrmm_%s" % (s, n))
+                f.restype, f.argtypes = None, [I, P, P, P, P, T, P, I, I, T, P, I]
+            f = getattr(L, "oracle_%s_csr2ell" % s)
+            f.restype, f.argtypes = I, [I, P, P, P, I, I, I, P, P]
+            f = getattr(L, "oracle_%s_csrmv_err" % s)
+            f.restype, f.argtypes = c_double, [I, P, P, P, P, c_double, P, P, P, POINTER(c_int64), POINTER(c_int64), POINTER(c_double)]
+            f = getattr(L, "oracle_%s_csrmm_err" % s)
+            f.restype, f.argtypes = c_double, [I, I, P, P, P, P, c_double, P, c_int64, c_int64, P, P, c_int64, c_int64, POINTER(c_int64)]
+        L.oracle_partition_rows_by_nnz.restype = None
+        L.oracle_partition_rows_by_nnz.argtypes = [P, I, I, P]
+        L.oracle_csr2coo.restype = None
+        L.oracle_csr2coo.argtypes = [I, P, I, P]
+        L.oracle_csr2ell_width.restype = I
+        L.oracle_csr2ell_width.argtypes = [I, P]
+        L.oracle_num_procs.restype = I
+        _libs[key] = L
+    return _libs[key]
+
+
+def _zero_based(a):
+    """(rows_start, rows_end, col_indx) zero-based views of a workloads.Csr."""
+    if a.base == 0:
+        return a.row_ptr[:-1], a.row_ptr[1:], a.col_ind
+    rp = (a.row_ptr - a.base).astype(np.int32)
+    return rp[:-1], rp[1:], (a.col_ind - a.base).astype(np.int32)
+
+
+def csrmv_plain(a, alpha, x, beta, y0, fast=False):
+    """y = alpha*A*x + beta*y0 with the serial plain kernel's rounding order."""
+    rs, re, ci = (np.ascontiguousarray(v) for v in _zero_based(a))
+    y = np.array(y0, dtype=a.dtype, copy=True)
+    T = _ct(a.dtype)
+    getattr(lib(fast), "oracle_%s_csrmv_plain" % _pre(a.dtype))(
+        a.rows, _p(rs), _p(re), _p(ci), _p(a.values), T(alpha), _p(x), T(beta), _p(y))
+    return y
+
+
+def csrmv_omp(a, alpha, x, beta, y0, threads=0, fast=True):
+    rs, re, ci = (np.ascontiguousarray(v) for v in _zero_based(a))
+    y = np.array(y0, dtype=a.dtype, copy=True)
+    T = _ct(a.dtype)
+    getattr(lib(fast), "oracle_%s_csrmv_omp" % _pre(a.dtype))(
+        a.rows, _p(rs), _p(re), _p(ci), _p(a.values), T(alpha), _p(x), T(beta), _p(y), threads)
+    return y
+
+
+def csrmv_f64acc(a, alpha, x, beta, y0):
+    rs, re, ci = (np.ascontiguousarray(v) for v in _zero_based(a))
+    out = np.empty(a.rows, dtype=np.float64)
+    y0 = np.ascontiguousarray(y0, dtype=a.dtype)
+    getattr(lib(), "oracle_%s_csrmv_f64acc" % _pre(a.dtype))(
+        a.rows, _p(rs), _p(re), _p(ci), _p(a.values), float(alpha), _p(x), float(beta), _p(y0), _p(out))
+    return out
+
+
+def csrmv_err(a, alpha, x, y_test, y_ref):
+    """(worst per-row normalised error, its row, #zero-denominator mismatches,
+    the reference's own max-norm ratio)."""
+    rs, re, ci = (np.ascontiguousarray(v) for v in _zero_based(a))
+    wr, zb, rr = c_int64(-1), c_int64(0), c_double(0)
+    y_test = np.ascontiguousarray(y_test, dtype=a.dtype)
+    y_ref = np.ascontiguousarray(y_ref, dtype=a.dtype)
+    e = getattr(lib(), "oracle_%s_csrmv_err" % _pre(a.dtype))(
+        a.rows, _p(rs), _p(re), _p(ci), _p(a.values), float(alpha), _p(x), _p(y_test), _p(y_ref),
+        byref(wr), byref(zb), byref(rr))
+    return e, wr.value, zb.value, rr.value
+
+
+def csrmm_plain(a, alpha, B, beta, C0, layout="row", omp=False, fast=False):
+    """C = alpha*A*B + beta*C0.  Row-major: B is (k, n) C-contiguous with ld = its
+    row length.  Column-major: pass B and C0 as Fortran-ordered 2-D arrays."""
+    rs, re, ci = (np.ascontiguousarray(v) for v in _zero_based(a))
+    T = _ct(a.dtype)
+    if layout == "row":
+        C = np.array(C0, dtype=a.dtype, order="C", copy=True)
+        B = np.ascontiguousarray(B, dtype=a.dtype)
+        n, ldb, ldc = C.shape[1], B.shape[1], C.shape[1]
+        fn = getattr(lib(fast), "oracle_%s_csrmm_%s" % (_pre(a.dtype), "row_omp" if omp else "row_plain"))
+    else:
+        C = np.array(C0, dtype=a.dtype, order="F", copy=True)
+        B = np.asfortranarray(B, dtype=a.dtype)
+        n, ldb, ldc = C.shape[1], B.shape[0], C.shape[0]
+        fn = getattr(lib(fast), "oracle_%s_csrmm_col_plain" % _pre(a.dtype))
+    fn(a.rows, _p(rs), _p(re), _p(ci), _p(a.values), T(alpha), _p(B), n, ldb, T(beta), _p(C), ldc)
+    return C
+
+
+def csrmm_err(a, alpha, B, C_test, C_ref):
+    """Worst per-element normalised error and #zero-denominator mismatches; B, C
+    are 2-D arrays of any (C or Fortran) contiguity with matching strides for C."""
+    rs, re, ci = (np.ascontiguousarray(v) for v in _zero_based(a))
+    it = a.dtype.itemsize
+    assert C_test.strides == C_ref.strides
+    zb = c_int64(0)
+    e = getattr(lib(), "oracle_%s_csrmm_err" % _pre(a.dtype))(
+        a.rows, C_test.shape[1], _p(rs), _p(re), _p(ci), _p(a.values), float(alpha), _p(B),
+        B.strides[0] // it, B.strides[1] // it, _p(C_test), _p(C_ref),
+        C_test.strides[0] // it, C_test.strides[1] // it, byref(zb))
+    return e, zb.value
+
+
+def csr2coo(a):
+    out = np.empty(a.nnz, dtype=np.int32)
+    lib().oracle_csr2coo(a.rows, _p(a.row_ptr), a.base, _p(out))
+    return out
+
+
+def csr2ell_width(a):
+    return int(lib().oracle_csr2ell_width(a.rows, _p(a.row_ptr)))
+
+
+def csr2ell(a, width=None, ell_base=0):
+    width = csr2ell_width(a) if width is None else width
+    ev = np.empty(width * a.rows, dtype=a.dtype)
+    ec = np.empty(width * a.rows, dtype=np.int32)
+    rc = getattr(lib(), "oracle_%s_csr2ell" % _pre(a.dtype))(
+        a.rows, _p(a.row_ptr), _p(a.col_ind), _p(a.values), a.base, ell_base, width, _p(ev), _p(ec))
+    if rc != 0:
+        raise OverflowError("width*m >= 2^31")
+    return ev, ec
+
+
+def partition_rows_by_nnz(rows_end, threads):
+    rows_end = np.ascontiguousarray(rows_end, dtype=np.int32)
+    out = np.empty(threads + 1, dtype=np.int32)
+    lib().oracle_partition_rows_by_nnz(_p(rows_end), rows_end.size, threads, _p(out))
+    return out
+
+
+def num_procs():
+    return int(lib().oracle_num_procs())
+
+
+# ---- the reference's own CPU kernels, compiled from its sources ---------------
+def _ref_csr_struct(T):
+    class S(Structure):
+        _fields_ = [("values", c_void_p), ("rows_start", c_void_p), ("rows_end", c_void_p),
+                    ("col_indx", c_void_p), ("rows", c_int32), ("cols", c_int32), ("ordered", c_bool),
+                    ("d_values", c_void_p), ("d_row_ptr", c_void_p), ("d_col_indx", c_void_p)]
+    return S
+
+
+def ref_available(fast=False):
+    return os.path.exists(os.path.join(HERE, "_ref", "libalphasparse_ref_%s.so" % ("fast" if fast else "o2")))
+
+
+def ref_lib(fast=False):
+    key = "ref_fast" if fast else "ref_o2"
+    if key not in _libs:
+        _libs[key] = ctypes.CDLL(os.path.join(HERE, "_ref", "libalphasparse_ref_%s.so" % ("fast" if fast else "o2")))
+        _libs[key].alpha_set_thread_num.argtypes = [ctypes.c_int]
+    return _libs[key]
+
+
+class RefCsr:
+    """A spmat_csr_?_t (include/alphasparse/spmat.h:174-216 of the reference) whose
+    arrays are numpy-owned; passed by pointer to the reference's kernels."""
+
+    def __init__(self, a):
+        self.keep = [np.ascontiguousarray(v) for v in _zero_based(a)] + [a.values]
+        rs, re, ci, v = self.keep
+        self.s = _ref_csr_struct(_ct(a.dtype))(_p(v), _p(rs), _p(re), _p(ci), a.rows, a.cols, False, None, None, None)
+        self.dtype = a.dtype
+
+
+def ref_call(name, a, *args, fast=False, threads=None):
+    """Call a reference kernel ``<name>`` with {t} replaced by s/d, e.g.
+    ``gemv_{t}_csr_plain(alpha, mat, x, beta, y)``."""
+    L = ref_lib(fast)
+    if threads is not None:
+        L.alpha_set_thread_num(threads)
+    fn = getattr(L, name.format(t=_pre(a.dtype)))
+    fn.restype = c_int32
+    return fn, RefCsr(a)
