@@ -168,6 +168,8 @@ _COMMON = {
     "asamd_csr2coo": [_P, _P, _I, _I, _P, _I],
     "asamd_csr2ell_width": [_P, _I, _P, POINTER(_I)],
     "asamd_warmup": [_P],
+    "asamd_analysis_stats": [_P],
+    "asamd_analysis_set_algo": [_P, _I],
 }
 
 
@@ -180,7 +182,11 @@ def prototypes():
     return out
 
 
-_RESTYPE = {"asamd_csr_plan_destroy": None, "asamd_csr_plan_stats": POINTER(asamd_csr_stats)}
+_RESTYPE = {"asamd_csr_plan_destroy": None, "asamd_csr_plan_stats": POINTER(asamd_csr_stats),
+            "asamd_analysis_stats": POINTER(asamd_csr_stats)}
+
+ALGO_NAMES = {ASAMD_SPMV_AUTO: "auto", ASAMD_SPMV_VECTOR: "vector", ASAMD_SPMV_ROWCONST: "rowconst",
+              ASAMD_SPMV_MERGE: "merge-path", ASAMD_SPMV_SCALAR: "scalar"}
 
 _lib = None
 

@@ -73,6 +73,7 @@ struct asamd_csr_plan {
   int* d_block_row;   // merge-path coordinates, merge_blocks + 1 ints
   int* d_carry_row;   // merge_blocks ints
   void* d_carry_val;  // merge_blocks values
+  void* d_head_val;   // merge_blocks values: partial sum of each workgroup's first row
   bool coords_valid;  // d_block_row filled for a structure promised fixed
 };
 
@@ -158,6 +159,7 @@ extern "C" int asamd_csr_plan_create(hipStream_t stream, int32_t m, int32_t n, i
   e = hipMalloc(&p->d_block_row, (nb + 1) * sizeof(int));
   if (e == hipSuccess) e = hipMalloc(&p->d_carry_row, nb * sizeof(int));
   if (e == hipSuccess) e = hipMalloc(&p->d_carry_val, nb * (size_t)val_size);
+  if (e == hipSuccess) e = hipMalloc(&p->d_head_val, nb * (size_t)val_size);
   if (e != hipSuccess) {
     asamd_csr_plan_destroy(p);
     return e;
@@ -181,6 +183,7 @@ extern "C" void asamd_csr_plan_destroy(asamd_csr_plan* p) {
   if (p->d_block_row) (void)hipFree(p->d_block_row);
   if (p->d_carry_row) (void)hipFree(p->d_carry_row);
   if (p->d_carry_val) (void)hipFree(p->d_carry_val);
+  if (p->d_head_val) (void)hipFree(p->d_head_val);
   delete p;
 }
 
@@ -263,9 +266,11 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
       }
       spmv_merge_kernel<T><<<nb, kMergeThreads, 0, s>>>(st.m, st.nnz, alpha, val, rp, ci, x, beta, y,
                                                         st.base, p->d_block_row, p->d_carry_row,
-                                                        (T*)p->d_carry_val);
-      merge_fixup_kernel<T><<<(nb + 255) / 256, 256, 0, s>>>(nb, st.m, alpha, p->d_carry_row,
-                                                             (const T*)p->d_carry_val, y);
+                                                        (T*)p->d_carry_val, (T*)p->d_head_val);
+      if (nb > 1)
+        merge_fixup_kernel<T><<<(nb + 255) / 256, 256, 0, s>>>(nb, st.m, alpha, beta, p->d_carry_row,
+                                                               (const T*)p->d_carry_val,
+                                                               (const T*)p->d_head_val, y);
       break;
     }
     case ASAMD_SPMV_VECTOR:

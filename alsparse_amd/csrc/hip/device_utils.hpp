@@ -29,6 +29,26 @@ __device__ __forceinline__ unsigned xcd_contiguous_id(unsigned hw_id, unsigned n
 __device__ __forceinline__ float fma_t(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
 __device__ __forceinline__ double fma_t(double a, double b, double c) { return __builtin_fma(a, b, c); }
 
+// y <- beta*y + alpha*sum with the reference's rounding points: both products
+// are rounded separately and then added, never contracted into an fma
+// (src/kernel/dcu/level2/mv/csrmv/dcu_gemv_vector.h:50-54 and
+// src/plain/kernel/level2/mv/gemv/gemv_x_csr_plain.c:14,21 agree on this).
+// beta == 0 does not read y at all.
+__device__ __forceinline__ float axpby_rn(float alpha, float sum, float beta, float yold) {
+  return __fadd_rn(__fmul_rn(yold, beta), __fmul_rn(alpha, sum));
+}
+__device__ __forceinline__ double axpby_rn(double alpha, double sum, double beta, double yold) {
+  return __dadd_rn(__dmul_rn(yold, beta), __dmul_rn(alpha, sum));
+}
+template <typename T>
+__device__ __forceinline__ void store_axpby(T* __restrict__ y, int64_t row, T alpha, T sum, T beta) {
+  if (beta == T(0)) {
+    y[row] = alpha * sum;
+  } else {
+    y[row] = axpby_rn(alpha, sum, beta, y[row]);
+  }
+}
+
 // ---- DPP moves ------------------------------------------------------------
 // dpp_ctrl encodings (GCN3+/CDNA ISA): quad_perm = 0x00..0xFF, row_shr:n =
 // 0x110+n, row_ror:n = 0x120+n, row_mirror = 0x140, row_half_mirror = 0x141.

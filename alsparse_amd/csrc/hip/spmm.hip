@@ -120,13 +120,13 @@ __global__ __launch_bounds__(kSpmmBlock) void spmm_rowmajor_kernel(
     } else {
       const Vec<T, V> old = *reinterpret_cast<const Vec<T, V>*>(crow);
 #pragma unroll
-      for (int i = 0; i < V; ++i) out.e[i] = fma_t(beta, old.e[i], acc[i]);
+      for (int i = 0; i < V; ++i) out.e[i] = old.e[i] * beta + acc[i];
     }
     *reinterpret_cast<Vec<T, V>*>(crow) = out;
   } else {
 #pragma unroll
     for (int i = 0; i < V; ++i) {
-      if (i < valid) crow[i] = beta == T(0) ? acc[i] : fma_t(beta, crow[i], acc[i]);
+      if (i < valid) crow[i] = beta == T(0) ? acc[i] : crow[i] * beta + acc[i];
     }
   }
 }
@@ -149,7 +149,7 @@ __global__ __launch_bounds__(kSpmmBlock) void spmm_strided_kernel(
       acc = fma_t(alpha * val[j], B[col * sbr + c * sbc], acc);
     }
     T* out = C + row * scr + c * scc;
-    *out = beta == T(0) ? acc : fma_t(beta, *out, acc);
+    *out = beta == T(0) ? acc : *out * beta + acc;
   }
 }
 

@@ -18,10 +18,14 @@
 //                               thread is combined by a segmented scan (wave
 //                               shuffles, then across the four waves in order);
 //                               rows finished inside the workgroup are written
-//                               coalesced as y = beta*y + alpha*sum; the
-//                               workgroup's unfinished tail goes to a carry slot.
-//   3. merge_fixup_kernel       adds the carries of all workgroups that a row
-//                               crossed, in workgroup order.
+//                               coalesced as y = beta*y + alpha*sum, except the
+//                               workgroup's first row, which may have begun in
+//                               earlier workgroups: its partial sum goes to a
+//                               head slot, the unfinished tail to a carry slot.
+//   3. merge_fixup_kernel       one thread per workgroup that finished a row:
+//                               sums the carries of the workgroups its first row
+//                               crossed, in workgroup order, adds the head slot
+//                               and writes that row's y once.
 //
 // No floating-point atomics anywhere: results are identical from run to run.
 // The reference has no counterpart (its CSR-adaptive row blocks,
@@ -73,7 +77,8 @@ template <typename T>
 __global__ __launch_bounds__(kMergeThreads) void spmv_merge_kernel(
     int m, int nnz, T alpha, const T* __restrict__ val, const int* __restrict__ row_ptr,
     const int* __restrict__ col_ind, const T* __restrict__ x, T beta, T* __restrict__ y, int base,
-    const int* __restrict__ block_row, int* __restrict__ carry_row, T* __restrict__ carry_val) {
+    const int* __restrict__ block_row, int* __restrict__ carry_row, T* __restrict__ carry_val,
+    T* __restrict__ head_val) {
   __shared__ int s_rend[kMergeItems + 1];           // row ends, local to this workgroup's entry range
   __shared__ T s_prod[kMergeItems + kMergeItems / 32 + 1];
   __shared__ T s_rsum[kMergeItems];                 // totals of rows finished here
@@ -204,33 +209,36 @@ __global__ __launch_bounds__(kMergeThreads) void spmv_merge_kernel(
   __syncthreads();
 
   // ---- rows finished here: y = beta*y + alpha*sum, coalesced ----------------
-  for (int r = tid; r < rows_cnt; r += kMergeThreads) {
-    const int64_t row = (int64_t)row_b + r;
-    const T sum = s_rsum[r];
-    if (beta == T(0)) {
-      y[row] = alpha * sum;
-    } else {
-      y[row] = fma_t(beta, y[row], alpha * sum);
-    }
-  }
+  // Local row 0 of every workgroup but the first may have begun earlier: the
+  // fix-up kernel completes it from head_val and the carries.
+  const int first_direct = b > 0 ? 1 : 0;
+  if (tid == 0 && b > 0) head_val[b] = rows_cnt > 0 ? s_rsum[0] : T(0);
+  for (int r = tid + first_direct; r < rows_cnt; r += kMergeThreads)
+    store_axpby(y, (int64_t)row_b + r, alpha, s_rsum[r], beta);
 }
 
-// Row r may have been open across several consecutive workgroups; their
-// carries are summed in workgroup order by the thread of the first of them and
-// added to the value written by the workgroup that finished the row.
+// Thread bb completes the first row of workgroup bb (bb >= 1) if that
+// workgroup finished it: the row is carry_row[bb-1]; every earlier workgroup
+// whose carry names the same row contributed a partial sum.  They are added in
+// workgroup order, then the finishing workgroup's own part, then y is written
+// once with the same rounding points as everywhere else.
 template <typename T>
-__global__ __launch_bounds__(256) void merge_fixup_kernel(int nblocks, int m, T alpha,
+__global__ __launch_bounds__(256) void merge_fixup_kernel(int nblocks, int m, T alpha, T beta,
                                                           const int* __restrict__ carry_row,
                                                           const T* __restrict__ carry_val,
+                                                          const T* __restrict__ head_val,
                                                           T* __restrict__ y) {
-  const int b = blockIdx.x * blockDim.x + threadIdx.x;
-  if (b >= nblocks) return;
-  const int r = carry_row[b];
+  const int bb = blockIdx.x * blockDim.x + threadIdx.x;
+  if (bb < 1 || bb >= nblocks) return;
+  const int r = carry_row[bb - 1];
   if (r < 0 || r >= m) return;
-  if (b > 0 && carry_row[b - 1] == r) return;
+  if (carry_row[bb] == r) return;  // workgroup bb finished no row
+  int first = bb - 1;
+  while (first > 0 && carry_row[first - 1] == r) --first;
   T s = T(0);
-  for (int bb = b; bb < nblocks && carry_row[bb] == r; ++bb) s += carry_val[bb];
-  if (s != T(0)) y[r] += alpha * s;
+  for (int k = first; k < bb; ++k) s += carry_val[k];
+  s += head_val[bb];
+  store_axpby(y, (int64_t)r, alpha, s, beta);
 }
 
 }  // namespace asamd

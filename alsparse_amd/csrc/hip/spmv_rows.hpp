@@ -20,15 +20,6 @@ namespace asamd {
 
 constexpr int kRowsBlock = 256;  // threads per workgroup of the row kernels
 
-template <typename T>
-__device__ __forceinline__ void store_axpby(T* __restrict__ y, int64_t row, T alpha, T sum, T beta) {
-  if (beta == T(0)) {
-    y[row] = alpha * sum;
-  } else {
-    y[row] = fma_t(beta, y[row], alpha * sum);
-  }
-}
-
 template <typename T, int W>
 __global__ __launch_bounds__(kRowsBlock) void spmv_vector_kernel(
     int m, T alpha, const T* __restrict__ val, const int* __restrict__ row_ptr,

@@ -135,3 +135,21 @@ alphasparse_status_t asamd_default_handle(alphasparse_dcu_handle_t *handle) {
   pthread_mutex_unlock(&g_lock);
   return st;
 }
+
+static asamd_record *find_any(const void *key) {
+  asamd_record *r = asamd_registry_find(ASAMD_KEY_INFO, key);
+  if (!r) r = asamd_registry_find(ASAMD_KEY_MATRIX, key);
+  if (!r) r = asamd_registry_find(ASAMD_KEY_LAZY, key);
+  return r;
+}
+
+const asamd_csr_stats *asamd_analysis_stats(const void *key) {
+  asamd_record *r = find_any(key);
+  return r && r->plan ? asamd_csr_plan_stats(r->plan) : NULL;
+}
+
+int asamd_analysis_set_algo(const void *key, int32_t algo) {
+  asamd_record *r = find_any(key);
+  if (!r || !r->plan) return (int)hipErrorInvalidValue;
+  return asamd_csr_plan_set_algo(r->plan, algo);
+}

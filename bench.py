@@ -1,0 +1,263 @@
+#!/usr/bin/env python3
+"""Benchmark of the CSR SpMV hot path on one MI355X.
+
+A "step" is one y <- alpha*A*x + beta*y through the C API
+(alphasparse_dcu_?_csrmv after alphasparse_dcu_?_csrmv_analysis) on a synthetic
+matrix that is resident in HBM before the timed region starts.  The default
+workload is benchmark configuration 3 (fp32, 16 777 216 rows x 16 entries per
+row, beta = 0.5), the one the bandwidth target is stated on; --config selects
+2 (fp64 Laplacian), 4 (fp32 power-law) or 5 (fp32 SpMM, n = 64) instead and
+--all appends their figures under "others".
+
+Prints ONE JSON line: metric/value (effective GB/s under the algorithmic bytes
+model), roofline (against 8 TB/s HBM3E) and cpu_baseline (the reference's
+OpenMP kernel, or its restatement, on the host cores -- reported, not a target).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+from ctypes import byref, c_void_p
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+WORKLOAD_NAMES = {
+    2: "C2: CSR SpMV fp64, 5-point Laplacian 2048x2048 (4194304 rows, 20963328 nnz), alpha=1 beta=0",
+    3: "C3: CSR SpMV fp32, 16777216 rows x 16 nnz/row uniform random sorted columns (268435456 nnz), alpha=1 beta=0.5",
+    4: "C4: CSR SpMV fp32, power-law rows (Zipf 2, <=200000) x R-MAT columns, 8388608 rows, alpha=1 beta=0",
+    5: "C5: CSR SpMM fp32, 1048576 rows x 32 nnz/row, B/C 1048576x64 row-major, alpha=1.5 beta=0.5",
+}
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def time_steps(fn, steps, warmup, hiprt):
+    """Per-launch HIP-event timing on the stream the library launches on (the
+    handle's stream is the null stream), bracketed by device synchronisation."""
+    for _ in range(warmup):
+        fn()
+    hiprt.synchronize()
+    evs = [hiprt.Event() for _ in range(steps + 1)]
+    t0 = time.perf_counter()
+    evs[0].record()
+    for i in range(steps):
+        fn()
+        evs[i + 1].record()
+    evs[-1].synchronize()
+    hiprt.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    per = [evs[i].elapsed_ms(evs[i + 1]) for i in range(steps)]
+    return {"avg_ms": float(np.mean(per)), "min_ms": float(np.min(per)), "median_ms": float(np.median(per)),
+            "wall_ms_per_step": wall_ms / steps}
+
+
+def run_spmv(cfg, steps, warmup, cpu_baseline, check):
+    from alsparse_amd import capi, hiprt, workloads as wl
+    lib = capi.load()
+    t0 = time.time()
+    a, x, y0, alpha, beta, _ = wl.config(cfg)
+    log("[bench] generated %s: %d rows, %d nnz in %.1f s" % (a.name, a.rows, a.nnz, time.time() - t0))
+    T, p = capi.scalar_type(a.dtype), capi.prefix(a.dtype)
+    h = capi.Handle()
+    descr = capi.make_descr()
+    d_val, d_rp, d_ci = (hiprt.DeviceArray.from_numpy(v) for v in (a.values, a.row_ptr, a.col_ind))
+    d_x, d_y = hiprt.DeviceArray.from_numpy(x), hiprt.DeviceArray.from_numpy(y0)
+
+    info = capi.alphasparse_dcu_mat_info_t()
+    assert lib.alphasparse_dcu_create_mat_info(byref(info)) == 0
+    hiprt.synchronize()
+    t0 = time.perf_counter()
+    st = getattr(lib, "alphasparse_dcu_%s_csrmv_analysis" % p)(
+        h.h, 0, a.rows, a.cols, a.nnz, byref(descr), d_val.c_ptr(), d_rp.c_ptr(), d_ci.c_ptr(), info)
+    hiprt.synchronize()
+    analysis_ms = (time.perf_counter() - t0) * 1e3
+    assert st == 0, "analysis status %d" % st
+    stats = lib.asamd_analysis_stats(info).contents
+    algo = capi.ALGO_NAMES.get(stats.algo, "?")
+    if stats.algo == capi.ASAMD_SPMV_VECTOR:
+        algo += "(W=%d)" % stats.vector_width
+
+    al, be = T(alpha), T(beta)
+    csrmv = getattr(lib, "alphasparse_dcu_%s_csrmv" % p)
+
+    def step():
+        s = csrmv(h.h, 0, a.rows, a.cols, a.nnz, byref(al), byref(descr), d_val.c_ptr(), d_rp.c_ptr(),
+                  d_ci.c_ptr(), info, d_x.c_ptr(), byref(be), d_y.c_ptr())
+        if s != 0:
+            raise RuntimeError("csrmv status %d" % s)
+
+    parity = None
+    if check:
+        from oracle import oracle as orc
+        d_y.copy_from(y0)
+        step()
+        hiprt.synchronize()
+        y = d_y.to_numpy()
+        t0 = time.time()
+        ref = orc.csrmv_plain(a, alpha, x, beta, y0)
+        err = orc.csrmv_err(a, alpha, x, beta, y0, y, ref)
+        tol = 1e-4 if a.dtype == np.float32 else 1e-12
+        parity = {"max_row_err": err.strict, "max_row_err_with_beta_y": err.full, "tol": tol,
+                  "zero_den_mismatch": err.zero_den_mismatch, "reference_check_ratio": err.ref_ratio,
+                  "ok": bool(err.strict <= tol and err.zero_den_mismatch == 0)}
+        log("[bench] parity vs plain-kernel oracle: %s (oracle %.1f s)" % (parity, time.time() - t0))
+        d_y.copy_from(y0)
+
+    t = time_steps(step, steps, warmup, hiprt)
+    nbytes = wl.spmv_bytes(a.rows, a.cols, a.nnz, a.dtype.itemsize, beta)
+    res = {"workload": WORKLOAD_NAMES[cfg], "rows": a.rows, "nnz": a.nnz, "algorithmic_bytes": int(nbytes),
+           "flops": 2 * a.nnz, "kernel": algo, "analysis_ms": analysis_ms, "timing": t,
+           "gbs": nbytes / t["avg_ms"] / 1e6, "gflops": 2 * a.nnz / t["avg_ms"] / 1e6,
+           "dtype": "f32" if a.dtype == np.float32 else "f64", "parity": parity}
+    res["hbm_frac"] = res["gbs"] / HBM_PEAK_GBS
+
+    if cpu_baseline:
+        res["cpu_baseline"] = cpu_spmv(a, x, y0, alpha, beta, nbytes)
+    lib.alphasparse_dcu_destroy_mat_info(info)
+    for d in (d_val, d_rp, d_ci, d_x, d_y):
+        d.free()
+    h.close()
+    return res
+
+
+def cpu_spmv(a, x, y0, alpha, beta, nbytes):
+    """The reference's OpenMP CSR kernel (gemv_?_csr compiled from its own sources
+    into oracle/_ref with its -Ofast flags) on all host cores; falls back to this
+    repository's restatement when that library is absent."""
+    from oracle import oracle as orc
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or orc.num_procs()
+    iters = 5
+    times = []
+    if orc.ref_available(fast=True):
+        kind = "reference"
+        fn, mat = orc.ref_call("gemv_{t}_csr", a, fast=True, threads=threads)
+        from ctypes import c_double, c_float
+        T = c_float if a.dtype == np.float32 else c_double
+        fn.argtypes = [T, c_void_p, c_void_p, T, c_void_p]
+        y = y0.copy()
+        for i in range(iters + 1):
+            t0 = time.perf_counter()
+            fn(T(alpha), byref(mat.s), x.ctypes.data_as(c_void_p), T(beta), y.ctypes.data_as(c_void_p))
+            if i:
+                times.append(time.perf_counter() - t0)
+    else:
+        kind = "port"
+        for i in range(iters + 1):
+            t0 = time.perf_counter()
+            orc.csrmv_omp(a, alpha, x, beta, y0, threads=threads, fast=True)
+            if i:
+                times.append(time.perf_counter() - t0)
+    best = min(times)
+    return {"value": nbytes / best / 1e9, "unit": "GB/s", "cores": threads, "kind": kind,
+            "gflops": 2 * a.nnz / best / 1e9, "ms": best * 1e3, "median_ms": float(np.median(times)) * 1e3,
+            "sample": "the full workload (%d rows, %d nnz), 1 warm-up + %d timed multiplies, best of %d"
+                      % (a.rows, a.nnz, iters, iters)}
+
+
+def run_spmm(steps, warmup, check):
+    from alsparse_amd import capi, hiprt, workloads as wl
+    lib = capi.load()
+    a, B, C0, alpha, beta, extra = wl.config(5)
+    n = extra["n"]
+    h = capi.Handle()
+    descr = capi.make_descr()
+    from ctypes import c_float
+    d_val, d_rp, d_ci = (hiprt.DeviceArray.from_numpy(v) for v in (a.values, a.row_ptr, a.col_ind))
+    d_B, d_C = hiprt.DeviceArray.from_numpy(B), hiprt.DeviceArray.from_numpy(C0)
+    al, be = c_float(alpha), c_float(beta)
+
+    def step():
+        s = lib.alphasparse_dcu_s_csrmm(h.h, 0, 0, capi.ALPHA_SPARSE_LAYOUT_ROW_MAJOR, a.rows, n, a.cols, a.nnz,
+                                        byref(al), byref(descr), d_val.c_ptr(), d_rp.c_ptr(), d_ci.c_ptr(),
+                                        d_B.c_ptr(), n, byref(be), d_C.c_ptr(), n)
+        if s != 0:
+            raise RuntimeError("csrmm status %d" % s)
+
+    parity = None
+    if check:
+        from oracle import oracle as orc
+        step()
+        hiprt.synchronize()
+        C = d_C.to_numpy()
+        ref = orc.csrmm_plain(a, alpha, B, beta, C0, omp=True)
+        err = orc.csrmm_err(a, alpha, B, beta, C0, C, ref)
+        parity = {"max_elem_err": err.strict, "max_elem_err_with_beta_c": err.full, "tol": 1e-4,
+                  "zero_den_mismatch": err.zero_den_mismatch, "ok": bool(err.strict <= 1e-4 and err.zero_den_mismatch == 0)}
+        d_C.copy_from(C0)
+    t = time_steps(step, steps, warmup, hiprt)
+    nbytes = wl.spmm_bytes(a.rows, a.cols, n, a.nnz, 4, beta)
+    res = {"workload": WORKLOAD_NAMES[5], "rows": a.rows, "nnz": a.nnz, "algorithmic_bytes": int(nbytes),
+           "gather_upper_bound_bytes": int(a.nnz) * n * 4, "flops": 2 * a.nnz * n, "timing": t,
+           "gbs": nbytes / t["avg_ms"] / 1e6, "gflops": 2 * a.nnz * n / t["avg_ms"] / 1e6, "dtype": "f32",
+           "parity": parity}
+    res["hbm_frac"] = res["gbs"] / HBM_PEAK_GBS
+    for d in (d_val, d_rp, d_ci, d_B, d_C):
+        d.free()
+    h.close()
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", type=int, default=3, choices=[2, 3, 4, 5])
+    ap.add_argument("--all", action="store_true", help="also measure the other configurations")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-check", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on exactly one GPU (rows would shard across GPUs with an "
+                 "all-gather of x; that path is a design note only). Re-run with --gpus 1.")
+
+    from alsparse_amd import hiprt
+    if hiprt.device_count() < 1:
+        sys.exit("bench.py: no GPU visible")
+    hiprt.set_device(0)
+
+    check = not args.no_check
+    if args.config == 5:
+        main_res = run_spmm(args.steps, args.warmup, check)
+    else:
+        main_res = run_spmv(args.config, args.steps, args.warmup, not args.no_cpu_baseline, check)
+    others = {}
+    if args.all:
+        for c in (2, 3, 4, 5):
+            if c == args.config:
+                continue
+            r = run_spmm(args.steps, args.warmup, check) if c == 5 else run_spmv(c, args.steps, args.warmup, False, check)
+            others["C%d" % c] = {k: r[k] for k in ("workload", "gbs", "gflops", "hbm_frac", "timing", "parity", "kernel") if k in r}
+
+    t = main_res["timing"]
+    out = {
+        "metric": "CSR SpMV effective GB/s (algorithmic bytes / time), 1 GPU" if args.config != 5
+                  else "CSR SpMM effective GB/s (algorithmic bytes / time), 1 GPU",
+        "value": main_res["gbs"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": t["avg_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": main_res["dtype"], "data": "synthetic",
+        "config": {"workload": main_res["workload"], "rows": main_res["rows"], "nnz": main_res["nnz"],
+                   "kernel": main_res.get("kernel", "spmm row-major"), "analysis_ms": main_res.get("analysis_ms")},
+        "gflops": main_res["gflops"], "pct_of_hbm_peak": 100.0 * main_res["hbm_frac"],
+        "min_ms": t["min_ms"], "median_ms": t["median_ms"], "wall_ms_per_step": t["wall_ms_per_step"],
+        "parity": main_res["parity"],
+        "roofline": {"bound": "hbm", "achieved": main_res["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": main_res["hbm_frac"], "traffic": None,
+                     "algorithmic_bytes_per_launch": main_res["algorithmic_bytes"]},
+        "cpu_baseline": main_res.get("cpu_baseline"),
+    }
+    if others:
+        out["others"] = others
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

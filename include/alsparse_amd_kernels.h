@@ -116,6 +116,16 @@ int asamd_d_csr2ell(hipStream_t stream, int32_t m, const double *val, const int3
                     const int32_t *col_ind, int32_t csr_base, int32_t ell_base, int32_t width,
                     double *ell_val, int32_t *ell_col);
 
+/* Introspection for benchmarks and tests: statistics of the analysis that a
+ * multiply would use for `key`, where key is the alphasparse_dcu_mat_info_t of an
+ * explicit analysis, or a device csr_row_ptr (library-built mirror or lazily
+ * analysed array).  NULL if nothing is recorded.  Implemented by the host
+ * library's registry; no reference counterpart. */
+const asamd_csr_stats *asamd_analysis_stats(const void *key);
+/* Force a kernel family (enum asamd_spmv_algo) on the analysis recorded for
+ * `key`; returns 0 on success, a hipError_t otherwise. */
+int asamd_analysis_set_algo(const void *key, int32_t algo);
+
 /* Empty kernel; forces code-object load (src/util_cpp/handle.cpp:19, :113). */
 int asamd_warmup(hipStream_t stream);
 

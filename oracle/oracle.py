@@ -49,9 +49,11 @@ def lib(fast=False):
             f = getattr(L, "oracle_%s_csr2ell" % s)
             f.restype, f.argtypes = I, [I, P, P, P, I, I, I, P, P]
             f = getattr(L, "oracle_%s_csrmv_err" % s)
-            f.restype, f.argtypes = c_double, [I, P, P, P, P, c_double, P, P, P, POINTER(c_int64), POINTER(c_int64), POINTER(c_double)]
+            f.restype, f.argtypes = c_double, [I, P, P, P, P, c_double, P, c_double, P, P, P, POINTER(c_int64),
+                                               POINTER(c_int64), POINTER(c_double), POINTER(c_double)]
             f = getattr(L, "oracle_%s_csrmm_err" % s)
-            f.restype, f.argtypes = c_double, [I, I, P, P, P, P, c_double, P, c_int64, c_int64, P, P, c_int64, c_int64, POINTER(c_int64)]
+            f.restype, f.argtypes = c_double, [I, I, P, P, P, P, c_double, P, c_int64, c_int64, c_double, P, P, P,
+                                               c_int64, c_int64, POINTER(c_int64), POINTER(c_double)]
         L.oracle_partition_rows_by_nnz.restype = None
         L.oracle_partition_rows_by_nnz.argtypes = [P, I, I, P]
         L.oracle_csr2coo.restype = None
@@ -99,17 +101,30 @@ def csrmv_f64acc(a, alpha, x, beta, y0):
     return out
 
 
-def csrmv_err(a, alpha, x, y_test, y_ref):
-    """(worst per-row normalised error, its row, #zero-denominator mismatches,
-    the reference's own max-norm ratio)."""
+class SpmvError:
+    """full: worst |dy| / (|alpha| sum|a x| + |beta y0|); strict: worst |dy| / (|alpha| sum|a x|);
+    zero_den_mismatch: rows with no non-zero product that differ from the reference;
+    ref_ratio: the reference's own max-norm statistic (check_s / check_d)."""
+
+    def __init__(self, full, strict, row, zero_den_mismatch, ref_ratio=None):
+        self.full, self.strict, self.row = full, strict, row
+        self.zero_den_mismatch, self.ref_ratio = zero_den_mismatch, ref_ratio
+
+    def __repr__(self):
+        return "SpmvError(full=%.3e, strict=%.3e, row=%d, zero_den_mismatch=%d)" % (
+            self.full, self.strict, self.row, self.zero_den_mismatch)
+
+
+def csrmv_err(a, alpha, x, beta, y0, y_test, y_ref):
     rs, re, ci = (np.ascontiguousarray(v) for v in _zero_based(a))
-    wr, zb, rr = c_int64(-1), c_int64(0), c_double(0)
+    wr, zb, rr, ws = c_int64(-1), c_int64(0), c_double(0), c_double(0)
     y_test = np.ascontiguousarray(y_test, dtype=a.dtype)
     y_ref = np.ascontiguousarray(y_ref, dtype=a.dtype)
+    y0 = None if (y0 is None or beta == 0) else np.ascontiguousarray(y0, dtype=a.dtype)
     e = getattr(lib(), "oracle_%s_csrmv_err" % _pre(a.dtype))(
-        a.rows, _p(rs), _p(re), _p(ci), _p(a.values), float(alpha), _p(x), _p(y_test), _p(y_ref),
-        byref(wr), byref(zb), byref(rr))
-    return e, wr.value, zb.value, rr.value
+        a.rows, _p(rs), _p(re), _p(ci), _p(a.values), float(alpha), _p(x), float(beta), _p(y0),
+        _p(y_test), _p(y_ref), byref(wr), byref(zb), byref(rr), byref(ws))
+    return SpmvError(e, ws.value, wr.value, zb.value, rr.value)
 
 
 def csrmm_plain(a, alpha, B, beta, C0, layout="row", omp=False, fast=False):
@@ -131,18 +146,22 @@ def csrmm_plain(a, alpha, B, beta, C0, layout="row", omp=False, fast=False):
     return C
 
 
-def csrmm_err(a, alpha, B, C_test, C_ref):
-    """Worst per-element normalised error and #zero-denominator mismatches; B, C
-    are 2-D arrays of any (C or Fortran) contiguity with matching strides for C."""
+def csrmm_err(a, alpha, B, beta, C0, C_test, C_ref):
+    """Per-element errors of C; B and the three C arrays are 2-D arrays of any (C or
+    Fortran) contiguity, the C arrays sharing one layout."""
     rs, re, ci = (np.ascontiguousarray(v) for v in _zero_based(a))
     it = a.dtype.itemsize
     assert C_test.strides == C_ref.strides
-    zb = c_int64(0)
+    if C0 is not None and beta != 0:
+        assert C0.strides == C_ref.strides
+    else:
+        C0 = None
+    zb, ws = c_int64(0), c_double(0)
     e = getattr(lib(), "oracle_%s_csrmm_err" % _pre(a.dtype))(
         a.rows, C_test.shape[1], _p(rs), _p(re), _p(ci), _p(a.values), float(alpha), _p(B),
-        B.strides[0] // it, B.strides[1] // it, _p(C_test), _p(C_ref),
-        C_test.strides[0] // it, C_test.strides[1] // it, byref(zb))
-    return e, zb.value
+        B.strides[0] // it, B.strides[1] // it, float(beta), _p(C0), _p(C_test), _p(C_ref),
+        C_test.strides[0] // it, C_test.strides[1] // it, byref(zb), byref(ws))
+    return SpmvError(e, ws.value, -1, zb.value)
 
 
 def csr2coo(a):

@@ -1,0 +1,130 @@
+"""Shared helpers of the GPU parity tests: run the C-ABI entry points on device
+buffers and compare with the CPU oracle on the same seeded inputs."""
+import sys
+from ctypes import byref
+
+import numpy as np
+
+from alsparse_amd import capi, hiprt, workloads as wl
+from oracle import oracle as orc
+
+TOL = {np.dtype(np.float32): 1e-4, np.dtype(np.float64): 1e-12}
+
+ALGOS = {"auto": capi.ASAMD_SPMV_AUTO, "vector": capi.ASAMD_SPMV_VECTOR, "rowconst": capi.ASAMD_SPMV_ROWCONST,
+         "merge": capi.ASAMD_SPMV_MERGE, "scalar": capi.ASAMD_SPMV_SCALAR}
+
+
+def announce(*what):
+    """Name the case before touching the GPU, flushed, so a fault can be attributed."""
+    print("[gpu-case]", *what, flush=True)
+
+
+def csr_from_lengths(lengths, cols, dtype, seed=7, base=0):
+    """CSR with the given row lengths, sorted distinct random columns, values in [-1, 1)."""
+    rng = np.random.default_rng(seed)
+    lengths = np.minimum(np.asarray(lengths, dtype=np.int64), cols)
+    row_ptr = np.zeros(len(lengths) + 1, dtype=np.int64)
+    np.cumsum(lengths, out=row_ptr[1:])
+    col = np.empty(int(row_ptr[-1]), dtype=np.int32)
+    for r, n in enumerate(lengths):
+        if n:
+            if n * 4 < cols:
+                c = np.unique(rng.integers(0, cols, size=int(n * 1.3) + 8))
+                while c.size < n:
+                    c = np.unique(np.concatenate([c, rng.integers(0, cols, size=int(n))]))
+                c = np.sort(rng.choice(c, size=int(n), replace=False))
+            else:
+                c = np.sort(rng.choice(cols, size=int(n), replace=False))
+            col[row_ptr[r]:row_ptr[r + 1]] = c
+    vals = rng.uniform(-1, 1, size=col.size).astype(dtype)
+    return wl.Csr(len(lengths), cols, (row_ptr + base).astype(np.int32), col + np.int32(base), vals, base,
+                  "lengths(m=%d,nnz=%d)" % (len(lengths), col.size))
+
+
+class DeviceCsr:
+    def __init__(self, a):
+        self.a = a
+        self.val = hiprt.DeviceArray.from_numpy(a.values)
+        self.row_ptr = hiprt.DeviceArray.from_numpy(a.row_ptr)
+        self.col = hiprt.DeviceArray.from_numpy(a.col_ind)
+
+    def free(self):
+        for d in (self.val, self.row_ptr, self.col):
+            d.free()
+
+
+def run_csrmv(h, da, alpha, x, beta, y0, info=None):
+    """alphasparse_dcu_?_csrmv on device copies of x, y0; returns y as numpy."""
+    a = da.a
+    lib = capi.load()
+    T = capi.scalar_type(a.dtype)
+    descr = capi.make_descr(base=a.base)
+    dx = hiprt.DeviceArray.from_numpy(np.ascontiguousarray(x, dtype=a.dtype))
+    dy = hiprt.DeviceArray.from_numpy(np.ascontiguousarray(y0, dtype=a.dtype))
+    al, be = T(alpha), T(beta)
+    st = getattr(lib, "alphasparse_dcu_%s_csrmv" % capi.prefix(a.dtype))(
+        h.h, 0, a.rows, a.cols, a.nnz, byref(al), byref(descr), da.val.c_ptr(), da.row_ptr.c_ptr(),
+        da.col.c_ptr(), info, dx.c_ptr(), byref(be), dy.c_ptr())
+    assert st == 0, "csrmv status %d" % st
+    hiprt.synchronize()
+    y = dy.to_numpy()
+    dx.free()
+    dy.free()
+    return y
+
+
+def run_plan_csrmv(da, algo, alpha, x, beta, y0, trusted=1):
+    """The thin kernel ABI directly, with a forced kernel family."""
+    a = da.a
+    lib = capi.load()
+    from ctypes import c_void_p
+    plan = c_void_p()
+    e = lib.asamd_csr_plan_create(None, a.rows, a.cols, a.nnz, da.row_ptr.c_ptr(), a.base,
+                                  a.dtype.itemsize, trusted, byref(plan))
+    assert e == 0, "plan_create hip error %d" % e
+    try:
+        e = lib.asamd_csr_plan_set_algo(plan, ALGOS[algo])
+        if e != 0:
+            return None  # this structure cannot run that family
+        T = capi.scalar_type(a.dtype)
+        dx = hiprt.DeviceArray.from_numpy(np.ascontiguousarray(x, dtype=a.dtype))
+        dy = hiprt.DeviceArray.from_numpy(np.ascontiguousarray(y0, dtype=a.dtype))
+        e = getattr(lib, "asamd_%s_csrmv" % capi.prefix(a.dtype))(
+            None, plan, T(alpha), da.val.c_ptr(), da.row_ptr.c_ptr(), da.col.c_ptr(), dx.c_ptr(), T(beta), dy.c_ptr())
+        assert e == 0, "asamd csrmv hip error %d" % e
+        hiprt.synchronize()
+        y = dy.to_numpy()
+        dx.free()
+        dy.free()
+        return y
+    finally:
+        lib.asamd_csr_plan_destroy(plan)
+
+
+def plan_stats(da, trusted=1):
+    a = da.a
+    lib = capi.load()
+    from ctypes import c_void_p
+    plan = c_void_p()
+    e = lib.asamd_csr_plan_create(None, a.rows, a.cols, a.nnz, da.row_ptr.c_ptr(), a.base,
+                                  a.dtype.itemsize, trusted, byref(plan))
+    assert e == 0
+    st = lib.asamd_csr_plan_stats(plan).contents
+    out = {k: getattr(st, k) for k, _ in st._fields_ if k != "hist"}
+    out["hist"] = list(st.hist)
+    lib.asamd_csr_plan_destroy(plan)
+    return out
+
+
+def check_spmv(a, alpha, x, beta, y0, y, what="", strict=False):
+    """Compare y with the plain-kernel oracle.  Always: zero-denominator rows exact and
+    the error relative to |alpha| sum|a x| + |beta y0| within tolerance; strict=True
+    also demands the criterion normalised by the products alone."""
+    ref = orc.csrmv_plain(a, alpha, x, beta, y0)
+    err = orc.csrmv_err(a, alpha, x, beta, y0, y, ref)
+    tol = TOL[a.dtype]
+    assert err.zero_den_mismatch == 0, "%s: %d rows with zero denominator differ" % (what, err.zero_den_mismatch)
+    assert err.full <= tol, "%s: per-row error %.3e at row %d exceeds %g" % (what, err.full, err.row, tol)
+    if strict or beta == 0:
+        assert err.strict <= tol, "%s: strict per-row error %.3e exceeds %g" % (what, err.strict, tol)
+    return err

@@ -1,0 +1,222 @@
+"""GPU parity of CSR SpMV against the CPU oracle, through the C-ABI.
+
+Tolerance (north star): per row |y - y_ref| / (|alpha| * sum_j |a_ij x_j|)
+<= 1e-4 for fp32 and <= 1e-12 for fp64; rows with a zero denominator must match
+exactly."""
+from ctypes import byref, c_void_p
+
+import numpy as np
+import pytest
+
+from alsparse_amd import capi, hiprt, workloads as wl
+from oracle import oracle as orc
+from helpers import (ALGOS, DeviceCsr, announce, check_spmv, csr_from_lengths, plan_stats, run_csrmv,
+                     run_plan_csrmv)
+
+pytestmark = pytest.mark.gpu
+
+
+def _vectors(a, seed=3):
+    return wl.uniform(a.cols, a.dtype, 3, seed), wl.uniform(a.rows, a.dtype, 4, seed)
+
+
+SHAPES = {
+    "points_1000": lambda dt: wl.random_points(1000, 1000, 5000, dt),
+    "laplace_64x48": lambda dt: wl.laplace2d(64, 48, dt),
+    "uniform16_5000": lambda dt: wl.uniform_rows(5000, 7000, 16, dt),
+    "uniform32_3000": lambda dt: wl.uniform_rows(3000, 3000, 32, dt),
+    "uniform5_4099": lambda dt: wl.uniform_rows(4099, 999, 5, dt),
+    "powerlaw_2^13": lambda dt: wl.powerlaw_rmat(13, 3000, dt),
+    "powerlaw_2^15_long": lambda dt: wl.powerlaw_rmat(15, 200000, dt),
+    "one_row_70000": lambda dt: csr_from_lengths([70000], 100000, dt),
+    "empty_rows_mixed": lambda dt: csr_from_lengths([0, 0, 5, 0, 3000, 0, 0, 1, 1, 0, 64, 65, 0], 5000, dt),
+    "all_rows_length_1": lambda dt: csr_from_lengths([1] * 10000, 10000, dt),
+    "many_empty_then_long": lambda dt: csr_from_lengths([0] * 5000 + [9000] + [0] * 3000 + [2, 2049, 2047], 20000, dt),
+    "single_entry": lambda dt: csr_from_lengths([1], 1, dt),
+    "ragged_tail": lambda dt: csr_from_lengths(list(range(0, 300)), 4000, dt),
+    "wide_few_rows": lambda dt: csr_from_lengths([4096, 4095, 4097, 1, 0, 8192], 10000, dt),
+}
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
+@pytest.mark.parametrize("shape", sorted(SHAPES))
+def test_every_kernel_family_matches_oracle(gpu, shape, dtype):
+    a = SHAPES[shape](dtype)
+    x, y0 = _vectors(a)
+    da = DeviceCsr(a)
+    try:
+        for algo in ("vector", "merge", "scalar", "rowconst", "auto"):
+            for alpha, beta in ((1.0, 0.0), (2.0, 3.0), (-0.75, 1.0)):
+                announce("spmv", shape, np.dtype(dtype).name, algo, alpha, beta)
+                y = run_plan_csrmv(da, algo, alpha, x, beta, y0)
+                if y is None:
+                    assert algo == "rowconst"
+                    continue
+                check_spmv(a, alpha, x, beta, y0, y, "%s/%s/%s" % (shape, algo, (alpha, beta)))
+    finally:
+        da.free()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
+def test_index_base_one(gpu, dtype):
+    for maker in (lambda: wl.uniform_rows(3000, 2500, 16, dtype, base=1),
+                  lambda: wl.powerlaw_rmat(12, 2000, dtype, base=1),
+                  lambda: wl.laplace2d(40, 30, dtype, base=1)):
+        a = maker()
+        x, y0 = _vectors(a)
+        da = DeviceCsr(a)
+        try:
+            for algo in ("vector", "merge", "scalar", "auto"):
+                announce("spmv base1", a.name, algo)
+                y = run_plan_csrmv(da, algo, 1.5, x, 0.25, y0)
+                check_spmv(a, 1.5, x, 0.25, y0, y, a.name + "/" + algo)
+            y = run_csrmv(gpu, da, 1.5, x, 0.25, y0)
+            check_spmv(a, 1.5, x, 0.25, y0, y, a.name + "/api")
+        finally:
+            da.free()
+
+
+def test_beta_zero_ignores_nan_in_y(gpu):
+    """beta == 0 must not read y: NaN / Inf in the output buffer may not leak
+    (the bytes model counts y once in that case)."""
+    a = wl.powerlaw_rmat(12, 2000, np.float32)
+    x, _ = _vectors(a)
+    y0 = np.full(a.rows, np.nan, dtype=np.float32)
+    da = DeviceCsr(a)
+    try:
+        for algo in ("vector", "merge", "scalar"):
+            announce("spmv beta0 nan", algo)
+            y = run_plan_csrmv(da, algo, 1.0, x, 0.0, y0)
+            assert np.isfinite(y).all()
+            check_spmv(a, 1.0, x, 0.0, np.zeros_like(y0), y, algo)
+    finally:
+        da.free()
+
+
+def test_deterministic_across_runs(gpu):
+    a = wl.powerlaw_rmat(15, 200000, np.float32)
+    x, y0 = _vectors(a)
+    da = DeviceCsr(a)
+    try:
+        announce("spmv determinism merge")
+        runs = [run_plan_csrmv(da, "merge", 1.0, x, 0.5, y0) for _ in range(3)]
+        assert np.array_equal(runs[0], runs[1]) and np.array_equal(runs[0], runs[2])
+    finally:
+        da.free()
+
+
+def test_analysis_statistics(gpu):
+    lengths = [0, 1, 2, 3, 4, 7, 8, 100, 1024, 0, 5]
+    a = csr_from_lengths(lengths, 5000, np.float32)
+    da = DeviceCsr(a)
+    try:
+        announce("analysis stats")
+        st = plan_stats(da)
+        assert st["min_len"] == 0 and st["max_len"] == 1024 and st["const_len"] == -1
+        want = [0] * capi.ASAMD_HIST_BINS
+        for n in lengths:
+            want[0 if n == 0 else int(n).bit_length()] += 1
+        assert st["hist"] == want
+        assert sum(st["hist"]) == a.rows
+    finally:
+        da.free()
+    a = wl.uniform_rows(2048, 2048, 16, np.float32)
+    da = DeviceCsr(a)
+    try:
+        st = plan_stats(da)
+        assert st["const_len"] == 16 and st["algo"] == capi.ASAMD_SPMV_ROWCONST
+        st = plan_stats(da, trusted=0)
+        assert st["algo"] != capi.ASAMD_SPMV_ROWCONST  # untrusted structure never skips row_ptr
+    finally:
+        da.free()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
+def test_explicit_analysis_and_garbage_info(gpu, dtype):
+    """csrmv with (a) info == NULL, (b) an analysed info, (c) a hand-allocated info
+    full of garbage (as the reference's own fp64 test passes), (d) after clear."""
+    lib = capi.load()
+    a = wl.powerlaw_rmat(13, 4000, dtype)
+    x, y0 = _vectors(a)
+    da = DeviceCsr(a)
+    descr = capi.make_descr()
+    p = capi.prefix(dtype)
+    try:
+        announce("csrmv info NULL")
+        check_spmv(a, 2.0, x, 3.0, y0, run_csrmv(gpu, da, 2.0, x, 3.0, y0), "null info")
+        info = capi.alphasparse_dcu_mat_info_t()
+        assert lib.alphasparse_dcu_create_mat_info(byref(info)) == 0
+        st = getattr(lib, "alphasparse_dcu_%s_csrmv_analysis" % p)(
+            gpu.h, 0, a.rows, a.cols, a.nnz, byref(descr), da.val.c_ptr(), da.row_ptr.c_ptr(), da.col.c_ptr(), info)
+        assert st == 0
+        assert info.contents.csrmv_info.contents.m == a.rows and info.contents.csrmv_info.contents.nnz == a.nnz
+        announce("csrmv analysed info")
+        check_spmv(a, 2.0, x, 3.0, y0, run_csrmv(gpu, da, 2.0, x, 3.0, y0, info), "analysed info")
+        assert lib.alphasparse_dcu_csrmv_clear(gpu.h, info) == 0
+        announce("csrmv cleared info")
+        check_spmv(a, 2.0, x, 3.0, y0, run_csrmv(gpu, da, 2.0, x, 3.0, y0, info), "cleared info")
+        assert lib.alphasparse_dcu_destroy_mat_info(info) == 0
+        garbage = (capi._alphasparse_dcu_mat_info * 1)()
+        np.frombuffer(garbage, dtype=np.uint8)[:] = 0xA5
+        announce("csrmv garbage info")
+        check_spmv(a, 2.0, x, 3.0, y0, run_csrmv(gpu, da, 2.0, x, 3.0, y0, garbage), "garbage info")
+    finally:
+        da.free()
+
+
+def test_lazy_cache_survives_structure_change_at_same_address(gpu):
+    """Two different structures with equal (m, nnz) living at the same device
+    address one after the other: the cached lazy plan may be stale, results may not."""
+    lens1 = [1] * 4000 + [4000]
+    lens2 = [4000] + [1] * 4000
+    a1 = csr_from_lengths(lens1, 9000, np.float32, seed=1)
+    a2 = csr_from_lengths(lens2, 9000, np.float32, seed=2)
+    assert a1.nnz == a2.nnz and a1.rows == a2.rows
+    da = DeviceCsr(a1)
+    try:
+        x, y0 = _vectors(a1)
+        announce("lazy plan structure 1")
+        check_spmv(a1, 1.0, x, 0.5, y0, run_csrmv(gpu, da, 1.0, x, 0.5, y0), "structure 1")
+        da.row_ptr.copy_from(a2.row_ptr)
+        da.col.copy_from(a2.col_ind)
+        da.val.copy_from(a2.values)
+        da.a = a2
+        announce("lazy plan structure 2 at the same address")
+        check_spmv(a2, 1.0, x, 0.5, y0, run_csrmv(gpu, da, 1.0, x, 0.5, y0), "structure 2")
+    finally:
+        da.free()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
+def test_handle_api_host_and_device(gpu, dtype):
+    """create_csr -> host2device -> mv_dcu (device vectors) and alphasparse_?_mv
+    (host vectors, computed on the GPU) -> export -> destroy."""
+    lib = capi.load()
+    p = capi.prefix(dtype)
+    T = capi.scalar_type(dtype)
+    for base, maker in ((0, lambda: wl.powerlaw_rmat(12, 3000, dtype)), (1, lambda: wl.uniform_rows(2000, 1500, 16, dtype, base=1))):
+        a = maker()
+        x, y0 = _vectors(a)
+        A = capi.alphasparse_matrix_t()
+        rs = np.ascontiguousarray(a.row_ptr[:-1])
+        re = np.ascontiguousarray(a.row_ptr[1:])
+        st = getattr(lib, "alphasparse_%s_create_csr" % p)(byref(A), base, a.rows, a.cols, capi.ptr(rs), capi.ptr(re),
+                                                           capi.ptr(a.col_ind), capi.ptr(a.values))
+        assert st == 0
+        a0 = wl.Csr(a.rows, a.cols, (a.row_ptr - base).astype(np.int32), (a.col_ind - base).astype(np.int32), a.values, 0, a.name)
+        announce("host api mv", a.name)
+        y = y0.copy()
+        st = getattr(lib, "alphasparse_%s_mv" % p)(0, T(1.5), A, capi.alpha_matrix_descr(0, 0, 0), capi.ptr(x), T(0.5), capi.ptr(y))
+        assert st == 0
+        check_spmv(a0, 1.5, x, 0.5, y0, y, "alphasparse_mv host")
+        announce("mv_dcu", a.name)
+        dx, dy = hiprt.DeviceArray.from_numpy(x), hiprt.DeviceArray.from_numpy(y0)
+        al, be = T(-2.0), T(1.0)
+        descr = capi.make_descr()
+        st = getattr(lib, "alphasparse_%s_mv_dcu" % p)(gpu.h, 0, byref(al), A, byref(descr), dx.c_ptr(), byref(be), dy.c_ptr())
+        assert st == 0
+        hiprt.synchronize()
+        check_spmv(a0, -2.0, x, 1.0, y0, dy.to_numpy(), "mv_dcu")
+        assert lib.alphasparse_destroy(A) == 0
+        dx.free()
+        dy.free()
