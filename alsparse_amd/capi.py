@@ -168,6 +168,7 @@ _COMMON = {
     "asamd_csr2coo": [_P, _P, _I, _I, _P, _I],
     "asamd_csr2ell_width": [_P, _I, _P, POINTER(_I)],
     "asamd_warmup": [_P],
+    "asamd_copy_bytes": [_P, _P, _P, c_size_t],
     "asamd_analysis_stats": [_P],
     "asamd_analysis_set_algo": [_P, _I],
 }

@@ -64,6 +64,13 @@ __global__ void stats_init_kernel(int* out) {
 
 __global__ void warmup_kernel() {}
 
+__global__ __launch_bounds__(256) void copy_bytes_kernel(Int4* __restrict__ dst,
+                                                         const Int4* __restrict__ src, size_t n16) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16;
+       i += (size_t)gridDim.x * blockDim.x)
+    dst[i] = src[i];
+}
+
 // ---------------------------------------------------------------------------
 struct asamd_csr_plan {
   asamd_csr_stats st;
@@ -298,6 +305,17 @@ extern "C" int asamd_d_csrmv(hipStream_t stream, asamd_csr_plan* plan, double al
                              const double* val, const int32_t* row_ptr, const int32_t* col_ind,
                              const double* x, double beta, double* y) {
   return csrmv_impl<double>(stream, plan, alpha, val, row_ptr, col_ind, x, beta, y);
+}
+
+extern "C" int asamd_copy_bytes(hipStream_t stream, void* dst, const void* src, size_t nbytes) {
+  if (!dst || !src || (nbytes & 15u) || (((uintptr_t)dst | (uintptr_t)src) & 15u))
+    return hipErrorInvalidValue;
+  const size_t n16 = nbytes / 16;
+  if (n16 == 0) return hipSuccess;
+  size_t grid = (n16 + 255) / 256;
+  if (grid > 256 * 64) grid = 256 * 64;
+  copy_bytes_kernel<<<(unsigned)grid, 256, 0, stream>>>((Int4*)dst, (const Int4*)src, n16);
+  return hipGetLastError();
 }
 
 extern "C" int asamd_warmup(hipStream_t stream) {

@@ -214,6 +214,9 @@ def main():
     ap.add_argument("--all", action="store_true", help="also measure the other configurations")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
+                    help="also launch one plain copy kernel of this many MiB (reads and writes that many "
+                         "bytes each) so that a counter run can be scaled against a known transfer")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (rows would shard across GPUs with an "
@@ -223,6 +226,17 @@ def main():
     if hiprt.device_count() < 1:
         sys.exit("bench.py: no GPU visible")
     hiprt.set_device(0)
+
+    if args.calibrate_copy:
+        from alsparse_amd import capi
+        nb = args.calibrate_copy << 20
+        src, dst = hiprt.DeviceArray((nb,), np.uint8), hiprt.DeviceArray((nb,), np.uint8)
+        src.fill_bytes(1)
+        for _ in range(2):
+            assert capi.load().asamd_copy_bytes(None, dst.c_ptr(), src.c_ptr(), nb) == 0
+        hiprt.synchronize()
+        src.free()
+        dst.free()
 
     check = not args.no_check
     if args.config == 5:

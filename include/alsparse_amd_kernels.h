@@ -126,6 +126,11 @@ const asamd_csr_stats *asamd_analysis_stats(const void *key);
  * `key`; returns 0 on success, a hipError_t otherwise. */
 int asamd_analysis_set_algo(const void *key, int32_t algo);
 
+/* Plain 16-byte-per-lane copy of nbytes (a multiple of 16, both pointers 16-byte
+ * aligned).  Exists to calibrate hardware byte counters against a transfer of
+ * known size; no reference counterpart. */
+int asamd_copy_bytes(hipStream_t stream, void *dst, const void *src, size_t nbytes);
+
 /* Empty kernel; forces code-object load (src/util_cpp/handle.cpp:19, :113). */
 int asamd_warmup(hipStream_t stream);
 

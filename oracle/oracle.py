@@ -147,20 +147,19 @@ def csrmm_plain(a, alpha, B, beta, C0, layout="row", omp=False, fast=False):
 
 
 def csrmm_err(a, alpha, B, beta, C0, C_test, C_ref):
-    """Per-element errors of C; B and the three C arrays are 2-D arrays of any (C or
-    Fortran) contiguity, the C arrays sharing one layout."""
+    """Per-element errors of C; B (k, n) and the C arrays (m, n) are 2-D arrays in any
+    memory layout (the metric does not depend on it)."""
     rs, re, ci = (np.ascontiguousarray(v) for v in _zero_based(a))
-    it = a.dtype.itemsize
-    assert C_test.strides == C_ref.strides
-    if C0 is not None and beta != 0:
-        assert C0.strides == C_ref.strides
-    else:
-        C0 = None
+    B = np.ascontiguousarray(B, dtype=a.dtype)
+    C_test = np.ascontiguousarray(C_test, dtype=a.dtype)
+    C_ref = np.ascontiguousarray(C_ref, dtype=a.dtype)
+    C0 = None if (C0 is None or beta == 0) else np.ascontiguousarray(C0, dtype=a.dtype)
+    assert C_test.shape == C_ref.shape and B.shape[1] == C_ref.shape[1]
+    n = C_ref.shape[1]
     zb, ws = c_int64(0), c_double(0)
     e = getattr(lib(), "oracle_%s_csrmm_err" % _pre(a.dtype))(
-        a.rows, C_test.shape[1], _p(rs), _p(re), _p(ci), _p(a.values), float(alpha), _p(B),
-        B.strides[0] // it, B.strides[1] // it, float(beta), _p(C0), _p(C_test), _p(C_ref),
-        C_test.strides[0] // it, C_test.strides[1] // it, byref(zb), byref(ws))
+        a.rows, n, _p(rs), _p(re), _p(ci), _p(a.values), float(alpha), _p(B), n, 1, float(beta), _p(C0),
+        _p(C_test), _p(C_ref), n, 1, byref(zb), byref(ws))
     return SpmvError(e, ws.value, -1, zb.value)
 
 

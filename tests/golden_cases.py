@@ -1,0 +1,34 @@
+"""The seeded inputs whose reference outputs are frozen under tests/golden/."""
+import numpy as np
+
+from alsparse_amd import workloads as wl
+from helpers_shapes import csr_from_lengths
+
+
+def golden_matrices():
+    out = {}
+    for dt, t in ((np.float32, "s"), (np.float64, "d")):
+        out[t + ".points"] = wl.random_points(1000, 1000, 5000, dt)                     # benchmark configuration 1
+        out[t + ".laplace"] = wl.laplace2d(24, 16, dt)
+        out[t + ".uniform16"] = wl.uniform_rows(512, 2048, 16, dt)
+        out[t + ".powerlaw"] = wl.powerlaw_rmat(10, 600, dt)
+        out[t + ".empty_rows"] = csr_from_lengths([0, 3, 0, 0, 7, 1, 0, 2, 0, 0], 16, dt, seed=5)
+    return out
+
+
+def checksum_cases():
+    out = {}
+    a, x, y0, _, _, _ = wl.config(1)
+    out["config1"] = {"nnz": a.nnz, "row_ptr": a.row_ptr, "col_ind": a.col_ind, "values": a.values, "x": x}
+    a = wl.laplace2d(2048, 2048, np.float64)
+    out["config2"] = {"nnz": a.nnz, "row_ptr": a.row_ptr, "col_ind": a.col_ind, "values": a.values}
+    a = wl.uniform_rows(1 << 16, 1 << 24, 16, np.float32)
+    out["config3_first_65536_rows"] = {"nnz": a.nnz, "row_ptr": a.row_ptr, "col_ind": a.col_ind, "values": a.values}
+    a = wl.powerlaw_rmat(16, 200000, np.float32)
+    out["config4_2^16_rows"] = {"nnz": a.nnz, "row_ptr": a.row_ptr, "col_ind": a.col_ind, "values": a.values,
+                                "max_len": int(np.diff(a.row_ptr).max())}
+    a = wl.uniform_rows(1 << 14, 1 << 20, 32, np.float32)
+    out["config5_first_16384_rows"] = {"nnz": a.nnz, "row_ptr": a.row_ptr, "col_ind": a.col_ind, "values": a.values}
+    out["vectors"] = {"x_f32": wl.uniform(4096, np.float32, 3), "y_f64": wl.uniform(4096, np.float64, 4),
+                      "B_f32": wl.uniform(4096, np.float32, 5)}
+    return out

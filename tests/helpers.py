@@ -7,6 +7,7 @@ import numpy as np
 
 from alsparse_amd import capi, hiprt, workloads as wl
 from oracle import oracle as orc
+from helpers_shapes import csr_from_lengths  # noqa: F401
 
 TOL = {np.dtype(np.float32): 1e-4, np.dtype(np.float64): 1e-12}
 
@@ -17,28 +18,6 @@ ALGOS = {"auto": capi.ASAMD_SPMV_AUTO, "vector": capi.ASAMD_SPMV_VECTOR, "rowcon
 def announce(*what):
     """Name the case before touching the GPU, flushed, so a fault can be attributed."""
     print("[gpu-case]", *what, flush=True)
-
-
-def csr_from_lengths(lengths, cols, dtype, seed=7, base=0):
-    """CSR with the given row lengths, sorted distinct random columns, values in [-1, 1)."""
-    rng = np.random.default_rng(seed)
-    lengths = np.minimum(np.asarray(lengths, dtype=np.int64), cols)
-    row_ptr = np.zeros(len(lengths) + 1, dtype=np.int64)
-    np.cumsum(lengths, out=row_ptr[1:])
-    col = np.empty(int(row_ptr[-1]), dtype=np.int32)
-    for r, n in enumerate(lengths):
-        if n:
-            if n * 4 < cols:
-                c = np.unique(rng.integers(0, cols, size=int(n * 1.3) + 8))
-                while c.size < n:
-                    c = np.unique(np.concatenate([c, rng.integers(0, cols, size=int(n))]))
-                c = np.sort(rng.choice(c, size=int(n), replace=False))
-            else:
-                c = np.sort(rng.choice(cols, size=int(n), replace=False))
-            col[row_ptr[r]:row_ptr[r + 1]] = c
-    vals = rng.uniform(-1, 1, size=col.size).astype(dtype)
-    return wl.Csr(len(lengths), cols, (row_ptr + base).astype(np.int32), col + np.int32(base), vals, base,
-                  "lengths(m=%d,nnz=%d)" % (len(lengths), col.size))
 
 
 class DeviceCsr:

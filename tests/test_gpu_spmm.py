@@ -1,0 +1,127 @@
+"""GPU parity of CSR SpMM against the CPU oracle, through alphasparse_dcu_?_csrmm.
+Tolerance per element as for SpMV (1e-4 fp32 / 1e-12 fp64)."""
+from ctypes import byref
+
+import numpy as np
+import pytest
+
+from alsparse_amd import capi, hiprt, workloads as wl
+from oracle import oracle as orc
+from helpers import TOL, DeviceCsr, announce
+from helpers_shapes import csr_from_lengths
+
+pytestmark = pytest.mark.gpu
+
+
+def run_csrmm(h, da, layout, trans_b, alpha, B, ldb, beta, C0, ldc, n, k):
+    a = da.a
+    lib = capi.load()
+    T = capi.scalar_type(a.dtype)
+    descr = capi.make_descr(base=a.base)
+    dB, dC = hiprt.DeviceArray.from_numpy(B), hiprt.DeviceArray.from_numpy(C0)
+    al, be = T(alpha), T(beta)
+    st = getattr(lib, "alphasparse_dcu_%s_csrmm" % capi.prefix(a.dtype))(
+        h.h, 0, trans_b, layout, a.rows, n, k, a.nnz, byref(al), byref(descr), da.val.c_ptr(), da.row_ptr.c_ptr(),
+        da.col.c_ptr(), dB.c_ptr(), ldb, byref(be), dC.c_ptr(), ldc)
+    assert st == 0, "csrmm status %d" % st
+    hiprt.synchronize()
+    out = dC.to_numpy()
+    dB.free()
+    dC.free()
+    return out
+
+
+def check(a, alpha, B2, beta, C02, C2, what):
+    ref = orc.csrmm_plain(a, alpha, np.ascontiguousarray(B2), beta, np.ascontiguousarray(C02))
+    err = orc.csrmm_err(a, alpha, np.ascontiguousarray(B2), beta, np.ascontiguousarray(C02), np.ascontiguousarray(C2), ref)
+    assert err.zero_den_mismatch == 0, what
+    assert err.full <= TOL[a.dtype], "%s: %r" % (what, err)
+    if beta == 0:
+        assert err.strict <= TOL[a.dtype], "%s: %r" % (what, err)
+
+
+MATS = {
+    "uniform32": lambda dt, base: wl.uniform_rows(3000, 2500, 32, dt, base=base),
+    "powerlaw": lambda dt, base: wl.powerlaw_rmat(11, 1500, dt, base=base),
+    "ragged": lambda dt, base: csr_from_lengths([0, 1, 0, 130, 64, 65, 63, 2, 0, 300, 1, 1], 400, dt, base=base),
+}
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
+@pytest.mark.parametrize("mat", sorted(MATS))
+@pytest.mark.parametrize("n", [1, 7, 64, 100, 128, 300])
+def test_row_major(gpu, mat, n, dtype):
+    for base in (0, 1):
+        a = MATS[mat](dtype, base)
+        da = DeviceCsr(a)
+        try:
+            for pad_b, pad_c in ((0, 0), (3, 5)):
+                ldb, ldc = n + pad_b, n + pad_c
+                Bfull = wl.uniform(a.cols * ldb, dtype, 5).reshape(a.cols, ldb)
+                Cfull = wl.uniform(a.rows * ldc, dtype, 4).reshape(a.rows, ldc)
+                for alpha, beta in ((1.5, 0.5), (1.0, 0.0)):
+                    announce("spmm row-major", mat, n, np.dtype(dtype).name, base, ldb, ldc, alpha, beta)
+                    out = run_csrmm(gpu, da, capi.ALPHA_SPARSE_LAYOUT_ROW_MAJOR, 0, alpha, Bfull, ldb, beta, Cfull, ldc, n, a.cols)
+                    check(a, alpha, Bfull[:, :n], beta, Cfull[:, :n], out[:, :n], "%s n=%d" % (mat, n))
+                    assert np.array_equal(out[:, n:], Cfull[:, n:]), "padding columns of C were touched"
+        finally:
+            da.free()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
+@pytest.mark.parametrize("n", [1, 5, 64, 70])
+def test_column_major_and_transposed_b(gpu, n, dtype):
+    a = wl.uniform_rows(1500, 1200, 16, dtype)
+    da = DeviceCsr(a)
+    try:
+        ldc = a.rows + 3
+        C0 = np.asfortranarray(wl.uniform(ldc * n, dtype, 4).reshape(n, ldc).T)          # (ldc, n) column-major
+        # op(B) = B: B is k x n column-major with ldb >= k
+        ldb = a.cols + 2
+        B = np.asfortranarray(wl.uniform(ldb * n, dtype, 5).reshape(n, ldb).T)            # (ldb, n) column-major
+        announce("spmm col-major N/N", n, np.dtype(dtype).name)
+        out = run_csrmm(gpu, da, capi.ALPHA_SPARSE_LAYOUT_COLUMN_MAJOR, 0, 1.5, B.T.reshape(-1), ldb, 0.5,
+                        C0.T.reshape(-1), ldc, n, a.cols)
+        out = out.reshape(n, ldc).T
+        check(a, 1.5, B[:a.cols, :], 0.5, C0[:a.rows, :], out[:a.rows, :], "col-major n=%d" % n)
+        ref_col = orc.csrmm_plain(a, 1.5, np.asfortranarray(B[:a.cols, :]), 0.5, np.asfortranarray(C0[:a.rows, :]), layout="col")
+        e = orc.csrmm_err(a, 1.5, np.asfortranarray(B[:a.cols, :]), 0.5, np.asfortranarray(C0[:a.rows, :]),
+                          np.asfortranarray(out[:a.rows, :]), ref_col)
+        assert e.full <= TOL[a.dtype]
+        assert np.array_equal(out[a.rows:, :], C0[a.rows:, :])
+        # op(B) = B^T: B is stored n x k column-major (ldb >= n), i.e. the memory of a row-major k x n matrix
+        ldb = n + 1
+        Bt = wl.uniform(a.cols * ldb, dtype, 5).reshape(a.cols, ldb)                       # row r of op(B) at Bt[r, :n]
+        announce("spmm col-major N/T", n, np.dtype(dtype).name)
+        out = run_csrmm(gpu, da, capi.ALPHA_SPARSE_LAYOUT_COLUMN_MAJOR, 1, 1.5, Bt.reshape(-1), ldb, 0.5,
+                        C0.T.reshape(-1), ldc, n, a.cols)
+        out = out.reshape(n, ldc).T
+        check(a, 1.5, Bt[:, :n], 0.5, C0[:a.rows, :], out[:a.rows, :], "col-major transB n=%d" % n)
+    finally:
+        da.free()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
+def test_host_pointer_mm(gpu, dtype):
+    lib = capi.load()
+    p, T = capi.prefix(dtype), capi.scalar_type(dtype)
+    a = wl.uniform_rows(1000, 800, 16, dtype)
+    A = capi.alphasparse_matrix_t()
+    rs, re = np.ascontiguousarray(a.row_ptr[:-1]), np.ascontiguousarray(a.row_ptr[1:])
+    assert getattr(lib, "alphasparse_%s_create_csr" % p)(byref(A), 0, a.rows, a.cols, capi.ptr(rs), capi.ptr(re),
+                                                         capi.ptr(a.col_ind), capi.ptr(a.values)) == 0
+    n = 10
+    B = wl.uniform(a.cols * n, dtype, 5).reshape(a.cols, n)
+    C0 = wl.uniform(a.rows * n, dtype, 4).reshape(a.rows, n)
+    C = C0.copy()
+    announce("host api mm row-major")
+    st = getattr(lib, "alphasparse_%s_mm" % p)(0, T(1.5), A, capi.alpha_matrix_descr(0, 0, 0), 0, capi.ptr(B), n, n, T(0.5), capi.ptr(C), n)
+    assert st == 0
+    check(a, 1.5, B, 0.5, C0, C, "alphasparse_mm row-major")
+    Bf, Cf0 = np.asfortranarray(B), np.asfortranarray(C0)
+    Cf = Cf0.copy(order="F")
+    announce("host api mm col-major")
+    st = getattr(lib, "alphasparse_%s_mm" % p)(0, T(1.5), A, capi.alpha_matrix_descr(0, 0, 0), 1, capi.ptr(Bf), n, a.cols, T(0.5), capi.ptr(Cf), a.rows)
+    assert st == 0
+    check(a, 1.5, B, 0.5, C0, np.ascontiguousarray(Cf), "alphasparse_mm col-major")
+    assert lib.alphasparse_destroy(A) == 0
