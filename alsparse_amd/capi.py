@@ -40,7 +40,7 @@ ALPHA_SPARSE_DATATYPE_FLOAT = 0
 ALPHA_SPARSE_DATATYPE_DOUBLE = 1
 
 # kernel families of the thin kernel ABI (include/alsparse_amd_kernels.h)
-ASAMD_SPMV_AUTO, ASAMD_SPMV_VECTOR, ASAMD_SPMV_ROWCONST, ASAMD_SPMV_MERGE, ASAMD_SPMV_SCALAR = range(5)
+ASAMD_SPMV_AUTO, ASAMD_SPMV_VECTOR, ASAMD_SPMV_ROWCONST, ASAMD_SPMV_MERGE, ASAMD_SPMV_SCALAR, ASAMD_SPMV_TILED = range(6)
 ASAMD_HIST_BINS = 33
 
 
@@ -105,7 +105,9 @@ class asamd_csr_stats(Structure):
     _fields_ = [("m", c_int32), ("n", c_int32), ("nnz", c_int32), ("base", c_int32),
                 ("min_len", c_int32), ("max_len", c_int32), ("const_len", c_int32),
                 ("first_offset", c_int32), ("algo", c_int32), ("vector_width", c_int32),
-                ("merge_blocks", c_int32), ("trusted", c_int32),
+                ("merge_blocks", c_int32), ("trusted", c_int32), ("tiled_built", c_int32),
+                ("tile_col_blocks", c_int32), ("tile_row_blocks", c_int32),
+                ("tune_ms_base", c_float), ("tune_ms_tiled", c_float),
                 ("hist", ctypes.c_int64 * ASAMD_HIST_BINS)]
 
 
@@ -161,7 +163,7 @@ _COMMON = {
     "alphasparse_dcu_csr2ell_width": [alphasparse_dcu_handle_t, _I, alpha_dcu_matrix_descr_t, _P,
                                       alpha_dcu_matrix_descr_t, POINTER(_I)],
     # thin kernel ABI
-    "asamd_csr_plan_create": [_P, _I, _I, _I, _P, _I, _I, _I, POINTER(_P)],
+    "asamd_csr_plan_create": [_P, _I, _I, _I, _P, _P, _P, _I, _I, _I, POINTER(_P)],
     "asamd_csr_plan_destroy": [_P],
     "asamd_csr_plan_stats": [_P],
     "asamd_csr_plan_set_algo": [_P, _I],
@@ -187,7 +189,7 @@ _RESTYPE = {"asamd_csr_plan_destroy": None, "asamd_csr_plan_stats": POINTER(asam
             "asamd_analysis_stats": POINTER(asamd_csr_stats)}
 
 ALGO_NAMES = {ASAMD_SPMV_AUTO: "auto", ASAMD_SPMV_VECTOR: "vector", ASAMD_SPMV_ROWCONST: "rowconst",
-              ASAMD_SPMV_MERGE: "merge-path", ASAMD_SPMV_SCALAR: "scalar"}
+              ASAMD_SPMV_MERGE: "merge-path", ASAMD_SPMV_SCALAR: "scalar", ASAMD_SPMV_TILED: "tiled two-phase"}
 
 _lib = None
 

@@ -10,11 +10,14 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <new>
 
 #include "alsparse_amd_kernels.h"
 #include "spmv_merge.hpp"
 #include "spmv_rows.hpp"
+#include "spmv_tiled.hpp"
+#include "tile_sort.hpp"
 
 using namespace asamd;
 
@@ -82,6 +85,16 @@ struct asamd_csr_plan {
   void* d_carry_val;  // merge_blocks values
   void* d_head_val;   // merge_blocks values: partial sum of each workgroup's first row
   bool coords_valid;  // d_block_row filled for a structure promised fixed
+  // tiled two-phase copy (trusted plans only)
+  int tile_cols_log2, n_chunks;
+  TileRange* d_ranges;        // row_blocks * col_blocks tile ranges, row block major
+  LongTile* d_long;           // tiles summed by a whole workgroup, grouped by workgroup
+  int* d_long_ptr;            // reduce workgroups + 1
+  void* d_tval;               // nnz values in tile order
+  unsigned short* d_tcol;     // nnz local columns
+  unsigned short* d_trow;     // nnz local rows
+  void* d_tprod;              // nnz products (phase 1 -> phase 2)
+  TiledChunk* d_chunks;       // phase-1 work list
 };
 
 static int width_for_mean(double mean) {
@@ -118,8 +131,217 @@ static void choose_algo(asamd_csr_plan* p) {
   st.vector_width = p->auto_width;
 }
 
+template <typename T>
+static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, const int* rp,
+                      const int* ci, const T* x, T beta, T* y);
+
+static void free_tiled(asamd_csr_plan* p) {
+  if (p->d_ranges) (void)hipFree(p->d_ranges);
+  if (p->d_long) (void)hipFree(p->d_long);
+  if (p->d_long_ptr) (void)hipFree(p->d_long_ptr);
+  p->d_long = nullptr;
+  p->d_long_ptr = nullptr;
+  if (p->d_tval) (void)hipFree(p->d_tval);
+  if (p->d_tcol) (void)hipFree(p->d_tcol);
+  if (p->d_trow) (void)hipFree(p->d_trow);
+  if (p->d_tprod) (void)hipFree(p->d_tprod);
+  if (p->d_chunks) (void)hipFree(p->d_chunks);
+  p->d_ranges = nullptr;
+  p->d_tval = p->d_tprod = nullptr;
+  p->d_tcol = p->d_trow = nullptr;
+  p->d_chunks = nullptr;
+  p->st.tiled_built = 0;
+}
+
+static int ilog2(int v) {
+  int l = 0;
+  while ((1 << l) < v) ++l;
+  return l;
+}
+
+template <typename T>
+static bool tiled_eligible(const asamd_csr_stats& st, bool force) {
+  const int64_t cb = ((int64_t)st.n + TileDims<T>::cols - 1) / TileDims<T>::cols;
+  const int64_t rb = ((int64_t)st.m + TileDims<T>::rows - 1) / TileDims<T>::rows;
+  if (!st.trusted || cb > kTiledMaxColBlocks || cb * rb > kTiledMaxTiles) return false;
+  // worth a try only when x cannot live in an XCD's 4 MiB L2 and the matrix is large
+  return force || ((int64_t)st.n * (int64_t)sizeof(T) >= ((int64_t)8 << 20) && st.nnz >= (1 << 22));
+}
+
+// Stable sort of the entries by (column block, row block), then the arrays of
+// both phases in that order and the two tile tables.
+template <typename T>
+static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* row_ptr,
+                              const int* col_ind, const T* val) {
+  asamd_csr_stats& st = p->st;
+  const int cb = (int)(((int64_t)st.n + TileDims<T>::cols - 1) / TileDims<T>::cols);
+  const int rb = (int)(((int64_t)st.m + TileDims<T>::rows - 1) / TileDims<T>::rows);
+  const int64_t tiles = (int64_t)cb * rb;
+  p->tile_cols_log2 = ilog2(TileDims<T>::cols);
+  st.tile_col_blocks = cb;
+  st.tile_row_blocks = rb;
+  const size_t nnz = (size_t)st.nnz;
+  unsigned key_bits = 1;
+  while (((int64_t)1 << key_bits) < tiles) ++key_bits;
+
+  int *d_coo = nullptr, *d_tile_ptr = nullptr, *d_long_count = nullptr;
+  LongTile* d_long_raw = nullptr;
+  unsigned *d_key = nullptr, *d_key2 = nullptr, *d_idx = nullptr, *d_perm = nullptr;
+  int* h_colptr = nullptr;
+  TiledChunk* h_chunks = nullptr;
+  hipError_t e = hipMalloc(&d_coo, nnz * sizeof(int));
+  if (e == hipSuccess) e = hipMalloc(&d_key, nnz * sizeof(unsigned));
+  if (e == hipSuccess) e = hipMalloc(&d_key2, nnz * sizeof(unsigned));
+  if (e == hipSuccess) e = hipMalloc(&d_idx, nnz * sizeof(unsigned));
+  if (e == hipSuccess) e = hipMalloc(&d_perm, nnz * sizeof(unsigned));
+  if (e == hipSuccess) e = hipMalloc(&d_tile_ptr, (size_t)(tiles + 1) * sizeof(int));
+  if (e == hipSuccess) e = hipMalloc(&p->d_ranges, (size_t)tiles * sizeof(TileRange));
+  const size_t long_cap = nnz / kLongTile + 1;  // a long tile holds more than kLongTile entries
+  if (e == hipSuccess) e = hipMalloc(&d_long_raw, long_cap * sizeof(LongTile));
+  if (e == hipSuccess) e = hipMalloc(&d_long_count, sizeof(int));
+  if (e == hipSuccess) e = hipMalloc(&p->d_tval, nnz * sizeof(T));
+  if (e == hipSuccess) e = hipMalloc(&p->d_tcol, nnz * sizeof(unsigned short));
+  if (e == hipSuccess) e = hipMalloc(&p->d_trow, nnz * sizeof(unsigned short));
+  if (e == hipSuccess) e = hipMalloc(&p->d_tprod, nnz * sizeof(T));
+  if (e == hipSuccess) e = (hipError_t)asamd_csr2coo(stream, row_ptr, st.nnz, st.m, d_coo, st.base);
+  if (e == hipSuccess) {
+    tile_keys_kernel<<<256 * 32, 256, 0, stream>>>(st.nnz, d_coo, col_ind, st.base, p->tile_cols_log2,
+                                                   TileDims<T>::rows_log2, rb, d_key, d_idx);
+    e = sort_pairs_u32(stream, d_key, d_key2, d_idx, d_perm, nnz, key_bits);
+  }
+  if (e == hipSuccess) {
+    tile_gather_kernel<T><<<256 * 32, 256, 0, stream>>>(st.nnz, d_perm, d_coo, col_ind, val, st.base,
+                                                        p->tile_cols_log2, TileDims<T>::rows_log2,
+                                                        (T*)p->d_tval, p->d_tcol, p->d_trow);
+    tile_bounds_kernel<<<(unsigned)((tiles + 1 + 255) / 256), 256, 0, stream>>>(st.nnz, d_key2, tiles,
+                                                                                d_tile_ptr);
+    e = hipMemsetAsync(d_long_count, 0, sizeof(int), stream);
+    tile_ranges_kernel<<<(unsigned)((tiles + 255) / 256), 256, 0, stream>>>(rb, cb, d_tile_ptr, p->d_ranges,
+                                                                            d_long_raw, d_long_count);
+    // phase-1 work list: every column block cut into chunks of at most kChunk entries
+    h_colptr = (int*)malloc((size_t)(cb + 1) * sizeof(int));
+    if (!h_colptr) e = hipErrorOutOfMemory;
+  }
+  if (e == hipSuccess)  // column block c starts at tile_ptr[c * rb]
+    e = hipMemcpy2DAsync(h_colptr, sizeof(int), d_tile_ptr, (size_t)rb * sizeof(int), sizeof(int),
+                         (size_t)cb + 1, hipMemcpyDeviceToHost, stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(stream);
+  if (e == hipSuccess) {
+    // long tiles, grouped by the reduce workgroup that owns their row block
+    const int n_wg = (rb + kRedWaves - 1) / kRedWaves;
+    int n_long = 0;
+    e = hipMemcpy(&n_long, d_long_count, sizeof(int), hipMemcpyDeviceToHost);
+    LongTile* h_long = (LongTile*)malloc((size_t)(n_long > 0 ? n_long : 1) * sizeof(LongTile));
+    int* h_lptr = (int*)calloc((size_t)n_wg + 1, sizeof(int));
+    if (!h_long || !h_lptr) e = hipErrorOutOfMemory;
+    if (e == hipSuccess && n_long > 0)
+      e = hipMemcpy(h_long, d_long_raw, (size_t)n_long * sizeof(LongTile), hipMemcpyDeviceToHost);
+    if (e == hipSuccess) {
+      std::sort(h_long, h_long + n_long, [](const LongTile& a, const LongTile& b) {
+        return a.row_block != b.row_block ? a.row_block < b.row_block : a.begin < b.begin;
+      });
+      for (int i = 0; i < n_long; ++i) h_lptr[h_long[i].row_block / kRedWaves + 1]++;
+      for (int g = 0; g < n_wg; ++g) h_lptr[g + 1] += h_lptr[g];
+      e = hipMalloc(&p->d_long, (size_t)(n_long > 0 ? n_long : 1) * sizeof(LongTile));
+      if (e == hipSuccess) e = hipMalloc(&p->d_long_ptr, ((size_t)n_wg + 1) * sizeof(int));
+      if (e == hipSuccess && n_long > 0)
+        e = hipMemcpy(p->d_long, h_long, (size_t)n_long * sizeof(LongTile), hipMemcpyHostToDevice);
+      if (e == hipSuccess)
+        e = hipMemcpy(p->d_long_ptr, h_lptr, ((size_t)n_wg + 1) * sizeof(int), hipMemcpyHostToDevice);
+    }
+    free(h_long);
+    free(h_lptr);
+  }
+  if (e == hipSuccess) {
+    const int kChunk = 128 * 1024;
+    int64_t n_chunks = 0;
+    for (int c = 0; c < cb; ++c) n_chunks += ((int64_t)h_colptr[c + 1] - h_colptr[c] + kChunk - 1) / kChunk;
+    h_chunks = (TiledChunk*)malloc((size_t)(n_chunks > 0 ? n_chunks : 1) * sizeof(TiledChunk));
+    if (!h_chunks) {
+      e = hipErrorOutOfMemory;
+    } else {
+      int64_t q = 0;
+      for (int c = 0; c < cb; ++c) {
+        for (int64_t b = h_colptr[c]; b < h_colptr[c + 1]; b += kChunk) {
+          h_chunks[q].col_block = c;
+          h_chunks[q].begin = (int)b;
+          h_chunks[q].end = (int)(b + kChunk < h_colptr[c + 1] ? b + kChunk : h_colptr[c + 1]);
+          ++q;
+        }
+      }
+      p->n_chunks = (int)n_chunks;
+      e = hipMalloc(&p->d_chunks, (size_t)(n_chunks > 0 ? n_chunks : 1) * sizeof(TiledChunk));
+      if (e == hipSuccess && n_chunks > 0)
+        e = hipMemcpy(p->d_chunks, h_chunks, (size_t)n_chunks * sizeof(TiledChunk), hipMemcpyHostToDevice);
+    }
+  }
+  if (e == hipSuccess)  // both phases use more than the default 64 KiB of dynamic LDS
+    e = hipFuncSetAttribute((const void*)tiled_products_kernel<T>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kTileBytes);
+  if (e == hipSuccess)
+    e = hipFuncSetAttribute((const void*)tiled_reduce_kernel<T>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kRedBytes);
+  free(h_colptr);
+  free(h_chunks);
+  for (void* d : {(void*)d_coo, (void*)d_key, (void*)d_key2, (void*)d_idx, (void*)d_perm, (void*)d_tile_ptr,
+                  (void*)d_long_raw, (void*)d_long_count})
+    if (d) (void)hipFree(d);
+  if (e != hipSuccess) {
+    free_tiled(p);
+    return e;
+  }
+  st.tiled_built = 1;
+  return hipSuccess;
+}
+
+// Time the current choice against the tiled kernel pair on scratch vectors and
+// keep the faster one.
+template <typename T>
+static hipError_t tune_tiled(hipStream_t stream, asamd_csr_plan* p, const int* row_ptr,
+                             const int* col_ind, const T* val) {
+  asamd_csr_stats& st = p->st;
+  T *x = nullptr, *y = nullptr;
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  hipError_t e = hipMalloc(&x, (size_t)st.n * sizeof(T));
+  if (e == hipSuccess) e = hipMalloc(&y, (size_t)st.m * sizeof(T));
+  if (e == hipSuccess) e = hipMemsetAsync(x, 0, (size_t)st.n * sizeof(T), stream);
+  if (e == hipSuccess) e = hipEventCreate(&e0);
+  if (e == hipSuccess) e = hipEventCreate(&e1);
+  float best[2] = {0.f, 0.f};
+  const int algos[2] = {p->auto_algo, ASAMD_SPMV_TILED};
+  for (int a = 0; a < 2 && e == hipSuccess; ++a) {
+    st.algo = algos[a];
+    for (int rep = 0; rep < 3 && e == hipSuccess; ++rep) {
+      e = hipEventRecord(e0, stream);
+      if (e == hipSuccess)
+        e = (hipError_t)csrmv_impl<T>(stream, p, T(1), val, row_ptr, col_ind, x, T(0), y);
+      if (e == hipSuccess) e = hipEventRecord(e1, stream);
+      if (e == hipSuccess) e = hipEventSynchronize(e1);
+      float ms = 0.f;
+      if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+      if (rep > 0 && (best[a] == 0.f || ms < best[a])) best[a] = ms;  // first run warms up
+    }
+  }
+  if (e0) (void)hipEventDestroy(e0);
+  if (e1) (void)hipEventDestroy(e1);
+  if (x) (void)hipFree(x);
+  if (y) (void)hipFree(y);
+  st.algo = p->auto_algo;
+  if (e != hipSuccess) return e;
+  st.tune_ms_base = best[0];
+  st.tune_ms_tiled = best[1];
+  if (best[1] > 0.f && best[1] < 0.9f * best[0]) {
+    p->auto_algo = ASAMD_SPMV_TILED;
+    st.algo = ASAMD_SPMV_TILED;
+  } else {
+    free_tiled(p);  // not worth its memory
+  }
+  return hipSuccess;
+}
+
 extern "C" int asamd_csr_plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t nnz,
-                                     const int32_t* row_ptr, int32_t base, int32_t val_size,
+                                     const int32_t* row_ptr, const int32_t* col_ind,
+                                     const void* val, int32_t base, int32_t val_size,
                                      int32_t trusted, asamd_csr_plan** out) {
   if (!out || !row_ptr || m <= 0 || nnz < 0 || (val_size != 4 && val_size != 8))
     return hipErrorInvalidValue;
@@ -181,6 +403,28 @@ extern "C" int asamd_csr_plan_create(hipStream_t stream, int32_t m, int32_t n, i
     }
     p->coords_valid = true;
   }
+  if (col_ind && val && nnz > 0) {
+    // trusted == 2: build the tiled copy whatever the size and skip the timing
+    // (lets small matrices exercise the tiled kernels)
+    const bool force = trusted == 2;
+    const bool ok = val_size == 4 ? tiled_eligible<float>(p->st, force) : tiled_eligible<double>(p->st, force);
+    if (ok) {
+      e = val_size == 4 ? build_tiled<float>(stream, p, row_ptr, col_ind, (const float*)val)
+                        : build_tiled<double>(stream, p, row_ptr, col_ind, (const double*)val);
+      if (e == hipSuccess && !force)
+        e = val_size == 4 ? tune_tiled<float>(stream, p, row_ptr, col_ind, (const float*)val)
+                          : tune_tiled<double>(stream, p, row_ptr, col_ind, (const double*)val);
+      if (e == hipErrorOutOfMemory) {
+        (void)hipGetLastError();  // the tiled copy is optional: carry on without it
+        free_tiled(p);
+        e = hipSuccess;
+      }
+      if (e != hipSuccess) {
+        asamd_csr_plan_destroy(p);
+        return e;
+      }
+    }
+  }
   *out = p;
   return hipSuccess;
 }
@@ -191,6 +435,7 @@ extern "C" void asamd_csr_plan_destroy(asamd_csr_plan* p) {
   if (p->d_carry_row) (void)hipFree(p->d_carry_row);
   if (p->d_carry_val) (void)hipFree(p->d_carry_val);
   if (p->d_head_val) (void)hipFree(p->d_head_val);
+  free_tiled(p);
   delete p;
 }
 
@@ -206,6 +451,10 @@ extern "C" int asamd_csr_plan_set_algo(asamd_csr_plan* p, int32_t algo) {
       return hipSuccess;
     case ASAMD_SPMV_ROWCONST:
       if (!rowconst_ok(p->st)) return hipErrorInvalidValue;
+      p->st.algo = algo;
+      return hipSuccess;
+    case ASAMD_SPMV_TILED:
+      if (!p->st.tiled_built) return hipErrorInvalidValue;
       p->st.algo = algo;
       return hipSuccess;
     case ASAMD_SPMV_VECTOR:
@@ -248,7 +497,18 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
     const bool aligned = (((uintptr_t)val | (uintptr_t)ci) & 15u) == 0;
     if (!aligned || !rowconst_ok(st)) algo = ASAMD_SPMV_VECTOR;
   }
+  if (algo == ASAMD_SPMV_TILED && !st.tiled_built) algo = p->auto_algo == ASAMD_SPMV_TILED ? ASAMD_SPMV_MERGE : p->auto_algo;
   switch (algo) {
+    case ASAMD_SPMV_TILED: {
+      // the tiled copy holds zero-based local indices and its own values
+      if (p->n_chunks > 0)
+        tiled_products_kernel<T><<<p->n_chunks, kProdThreads, kTileBytes, s>>>(
+            st.n, p->d_chunks, (const T*)p->d_tval, p->d_tcol, x, (T*)p->d_tprod);
+      tiled_reduce_kernel<T><<<(st.tile_row_blocks + kRedWaves - 1) / kRedWaves, kRedThreads, kRedBytes, s>>>(
+          st.m, st.tile_row_blocks, st.tile_col_blocks, p->d_ranges, p->d_long_ptr, p->d_long, p->d_trow,
+          (const T*)p->d_tprod, alpha, beta, y);
+      break;
+    }
     case ASAMD_SPMV_ROWCONST:
       switch (st.const_len / 4) {
         case 1: launch_rowconst<T, 1>(s, st, alpha, val, ci, x, beta, y); break;

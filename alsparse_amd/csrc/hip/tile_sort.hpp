@@ -1,0 +1,10 @@
+// Internal: stable device sort of (key, value) pairs of 32-bit unsigned integers
+// on the low `end_bit` bits of the key; synchronises the stream.
+#pragma once
+#include <hip/hip_runtime_api.h>
+#include <stddef.h>
+
+namespace asamd {
+hipError_t sort_pairs_u32(hipStream_t stream, unsigned* keys_in, unsigned* keys_out, unsigned* vals_in,
+                          unsigned* vals_out, size_t n, unsigned end_bit);
+}

@@ -161,5 +161,6 @@ int asamd_env_algo(void) {
   if (!strcmp(e, "rowconst")) return ASAMD_SPMV_ROWCONST;
   if (!strcmp(e, "merge")) return ASAMD_SPMV_MERGE;
   if (!strcmp(e, "scalar")) return ASAMD_SPMV_SCALAR;
+  if (!strcmp(e, "tiled")) return ASAMD_SPMV_TILED;
   return ASAMD_SPMV_AUTO;
 }

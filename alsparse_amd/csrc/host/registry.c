@@ -96,7 +96,7 @@ alphasparse_status_t asamd_plan_for_call(alphasparse_dcu_handle_t handle, const 
   if (!r) {
     asamd_csr_plan *p = NULL;
     ASAMD_HIP_STATUS(asamd_csr_plan_create(handle->stream, m, n, nnz, (const int32_t *)row_ptr,
-                                           base, val_size, /*trusted=*/0, &p));
+                                           NULL, NULL, base, val_size, /*trusted=*/0, &p));
     r = asamd_registry_insert(ASAMD_KEY_LAZY, row_ptr);
     if (!r) {
       asamd_csr_plan_destroy(p);

@@ -32,7 +32,9 @@ enum asamd_spmv_algo {
   ASAMD_SPMV_VECTOR = 1,   /* W lanes per row, W in {2..64} from the mean row length */
   ASAMD_SPMV_ROWCONST = 2, /* every row has the same length L = 4*G: no row_ptr read */
   ASAMD_SPMV_MERGE = 3,    /* merge-path split of (rows + nnz), LDS-staged products  */
-  ASAMD_SPMV_SCALAR = 4    /* one lane per row; diagnostic baseline                  */
+  ASAMD_SPMV_SCALAR = 4,   /* one lane per row; diagnostic baseline                  */
+  ASAMD_SPMV_TILED = 5     /* two-phase, (column block x row block) tiles: every x
+                              gather and y update in LDS, HBM sees only streams     */
 };
 
 #define ASAMD_HIST_BINS 33
@@ -48,19 +50,31 @@ typedef struct {
   int32_t vector_width; /* lanes per row when algo == VECTOR                  */
   int32_t merge_blocks; /* workgroups of the merge-path kernel                */
   int32_t trusted;      /* 1: structure promised fixed, coordinates cached    */
+  int32_t tiled_built;  /* 1: a tiled copy exists (TILED can be selected)     */
+  int32_t tile_col_blocks, tile_row_blocks;
+  float tune_ms_base;   /* analysis-time timing of the non-tiled choice, or 0 */
+  float tune_ms_tiled;  /* ... and of the tiled kernel pair, or 0             */
   int64_t hist[ASAMD_HIST_BINS];
 } asamd_csr_stats;
 
 typedef struct asamd_csr_plan asamd_csr_plan;
 
 /* Row-length histogram, kernel choice and (trusted != 0) cached merge-path
- * block coordinates.  Synchronises `stream` once to read the statistics.
+ * block coordinates.  Synchronises `stream` to read the statistics.
  * Replaces the host-side row-block builder
  * src/util_cpp/alphasparse_dcu_x_csrmv_analysis.cpp:58-267, :348-379.
- * val_size is sizeof(value type): 4 or 8. */
+ * val_size is sizeof(value type): 4 or 8.
+ * trusted != 0 promises that the structure behind row_ptr / col_ind and the
+ * values behind val stay as they are for the life of the plan.  If in addition
+ * col_ind and val are given (they may be NULL) and x is much larger than the L2,
+ * a tiled copy of the matrix is built and the tiled two-phase kernel is timed
+ * against the row / merge-path choice on scratch vectors; the faster one wins
+ * (the reference's analysis record carries an `algo_tuning` flag for exactly
+ * this, include/alphasparse/handle.h:120-123).  trusted == 2 builds the tiled
+ * copy whatever the size and skips the timing (for tests of the tiled kernels). */
 int asamd_csr_plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t nnz,
-                          const int32_t *row_ptr, int32_t base, int32_t val_size, int32_t trusted,
-                          asamd_csr_plan **plan);
+                          const int32_t *row_ptr, const int32_t *col_ind, const void *val,
+                          int32_t base, int32_t val_size, int32_t trusted, asamd_csr_plan **plan);
 void asamd_csr_plan_destroy(asamd_csr_plan *plan);
 const asamd_csr_stats *asamd_csr_plan_stats(const asamd_csr_plan *plan);
 /* Force a kernel family for later multiplies (AUTO restores the analysis'

@@ -12,7 +12,7 @@ from helpers_shapes import csr_from_lengths  # noqa: F401
 TOL = {np.dtype(np.float32): 1e-4, np.dtype(np.float64): 1e-12}
 
 ALGOS = {"auto": capi.ASAMD_SPMV_AUTO, "vector": capi.ASAMD_SPMV_VECTOR, "rowconst": capi.ASAMD_SPMV_ROWCONST,
-         "merge": capi.ASAMD_SPMV_MERGE, "scalar": capi.ASAMD_SPMV_SCALAR}
+         "merge": capi.ASAMD_SPMV_MERGE, "scalar": capi.ASAMD_SPMV_SCALAR, "tiled": capi.ASAMD_SPMV_TILED}
 
 
 def announce(*what):
@@ -58,8 +58,10 @@ def run_plan_csrmv(da, algo, alpha, x, beta, y0, trusted=1):
     lib = capi.load()
     from ctypes import c_void_p
     plan = c_void_p()
-    e = lib.asamd_csr_plan_create(None, a.rows, a.cols, a.nnz, da.row_ptr.c_ptr(), a.base,
-                                  a.dtype.itemsize, trusted, byref(plan))
+    if algo == "tiled":
+        trusted = 2  # build the tiled copy whatever the size
+    e = lib.asamd_csr_plan_create(None, a.rows, a.cols, a.nnz, da.row_ptr.c_ptr(), da.col.c_ptr(), da.val.c_ptr(),
+                                  a.base, a.dtype.itemsize, trusted, byref(plan))
     assert e == 0, "plan_create hip error %d" % e
     try:
         e = lib.asamd_csr_plan_set_algo(plan, ALGOS[algo])
@@ -85,7 +87,7 @@ def plan_stats(da, trusted=1):
     lib = capi.load()
     from ctypes import c_void_p
     plan = c_void_p()
-    e = lib.asamd_csr_plan_create(None, a.rows, a.cols, a.nnz, da.row_ptr.c_ptr(), a.base,
+    e = lib.asamd_csr_plan_create(None, a.rows, a.cols, a.nnz, da.row_ptr.c_ptr(), None, None, a.base,
                                   a.dtype.itemsize, trusted, byref(plan))
     assert e == 0
     st = lib.asamd_csr_plan_stats(plan).contents

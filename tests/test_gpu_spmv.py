@@ -45,7 +45,7 @@ def test_every_kernel_family_matches_oracle(gpu, shape, dtype):
     x, y0 = _vectors(a)
     da = DeviceCsr(a)
     try:
-        for algo in ("vector", "merge", "scalar", "rowconst", "auto"):
+        for algo in ("vector", "merge", "scalar", "rowconst", "tiled", "auto"):
             for alpha, beta in ((1.0, 0.0), (2.0, 3.0), (-0.75, 1.0)):
                 announce("spmv", shape, np.dtype(dtype).name, algo, alpha, beta)
                 y = run_plan_csrmv(da, algo, alpha, x, beta, y0)
@@ -66,7 +66,7 @@ def test_index_base_one(gpu, dtype):
         x, y0 = _vectors(a)
         da = DeviceCsr(a)
         try:
-            for algo in ("vector", "merge", "scalar", "auto"):
+            for algo in ("vector", "merge", "scalar", "tiled", "auto"):
                 announce("spmv base1", a.name, algo)
                 y = run_plan_csrmv(da, algo, 1.5, x, 0.25, y0)
                 check_spmv(a, 1.5, x, 0.25, y0, y, a.name + "/" + algo)
@@ -84,7 +84,7 @@ def test_beta_zero_ignores_nan_in_y(gpu):
     y0 = np.full(a.rows, np.nan, dtype=np.float32)
     da = DeviceCsr(a)
     try:
-        for algo in ("vector", "merge", "scalar"):
+        for algo in ("vector", "merge", "scalar", "tiled"):
             announce("spmv beta0 nan", algo)
             y = run_plan_csrmv(da, algo, 1.0, x, 0.0, y0)
             assert np.isfinite(y).all()
