@@ -40,7 +40,8 @@ ALPHA_SPARSE_DATATYPE_FLOAT = 0
 ALPHA_SPARSE_DATATYPE_DOUBLE = 1
 
 # kernel families of the thin kernel ABI (include/alsparse_amd_kernels.h)
-ASAMD_SPMV_AUTO, ASAMD_SPMV_VECTOR, ASAMD_SPMV_ROWCONST, ASAMD_SPMV_MERGE, ASAMD_SPMV_SCALAR, ASAMD_SPMV_TILED = range(6)
+(ASAMD_SPMV_AUTO, ASAMD_SPMV_VECTOR, ASAMD_SPMV_ROWCONST, ASAMD_SPMV_MERGE, ASAMD_SPMV_SCALAR, ASAMD_SPMV_TILED,
+ ASAMD_SPMV_STREAM) = range(7)
 ASAMD_HIST_BINS = 33
 
 
@@ -189,7 +190,8 @@ _RESTYPE = {"asamd_csr_plan_destroy": None, "asamd_csr_plan_stats": POINTER(asam
             "asamd_analysis_stats": POINTER(asamd_csr_stats)}
 
 ALGO_NAMES = {ASAMD_SPMV_AUTO: "auto", ASAMD_SPMV_VECTOR: "vector", ASAMD_SPMV_ROWCONST: "rowconst",
-              ASAMD_SPMV_MERGE: "merge-path", ASAMD_SPMV_SCALAR: "scalar", ASAMD_SPMV_TILED: "tiled two-phase"}
+              ASAMD_SPMV_MERGE: "merge-path", ASAMD_SPMV_SCALAR: "scalar", ASAMD_SPMV_TILED: "tiled two-phase",
+              ASAMD_SPMV_STREAM: "row-block stream"}
 
 _lib = None
 

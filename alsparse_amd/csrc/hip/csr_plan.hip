@@ -11,6 +11,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cstdlib>
 #include <new>
 
 #include "alsparse_amd_kernels.h"
@@ -80,6 +81,7 @@ struct asamd_csr_plan {
   int auto_algo;
   int auto_width;
   int val_size;
+  int merge_ipt;      // items per thread of the merge-path kernel (4, 8 or 16)
   int* d_block_row;   // merge-path coordinates, merge_blocks + 1 ints
   int* d_carry_row;   // merge_blocks ints
   void* d_carry_val;  // merge_blocks values
@@ -114,6 +116,13 @@ static bool rowconst_ok(const asamd_csr_stats& st) {
          (L == 4 || L == 8 || L == 16 || L == 32 || L == 64 || L == 128 || L == 256);
 }
 
+// The LDS-staged row-block kernel sizes its staging area for rows of at most
+// kStreamMaxLen entries; the bound comes from the analysis, so the structure
+// must be promised fixed.
+static bool stream_ok(const asamd_csr_stats& st) {
+  return st.trusted && st.max_len <= kStreamMaxLen && st.max_len >= 1;
+}
+
 static void choose_algo(asamd_csr_plan* p) {
   asamd_csr_stats& st = p->st;
   const double mean = st.m > 0 ? (double)st.nnz / st.m : 0.0;
@@ -121,6 +130,8 @@ static void choose_algo(asamd_csr_plan* p) {
   p->auto_width = w;
   if (rowconst_ok(st)) {
     p->auto_algo = ASAMD_SPMV_ROWCONST;
+  } else if (stream_ok(st)) {
+    p->auto_algo = ASAMD_SPMV_STREAM;
   } else if ((int64_t)st.max_len <= (int64_t)w * 16 && mean >= 6.0) {
     // regular rows: a lane group per row wastes little and needs no LDS
     p->auto_algo = ASAMD_SPMV_VECTOR;
@@ -379,7 +390,14 @@ extern "C" int asamd_csr_plan_create(hipStream_t stream, int32_t m, int32_t n, i
   for (int b = 0; b < ASAMD_HIST_BINS; ++b) p->st.hist[b] = h[3 + b];
 
   const int64_t total = (int64_t)m + nnz;
-  const int64_t nb = (total + kMergeItems - 1) / kMergeItems;
+  // fp64 doubles the LDS per item: fewer items keep more workgroups resident
+  p->merge_ipt = val_size == 8 ? 4 : 8;
+  if (const char* ev = getenv("ALSPARSE_AMD_MERGE_IPT")) {
+    const int v = atoi(ev);
+    if (v == 4 || v == 8 || v == 16) p->merge_ipt = v;
+  }
+  const int merge_items = kMergeThreads * p->merge_ipt;
+  const int64_t nb = (total + merge_items - 1) / merge_items;
   p->st.merge_blocks = (int)nb;
   choose_algo(p);
 
@@ -395,7 +413,7 @@ extern "C" int asamd_csr_plan_create(hipStream_t stream, int32_t m, int32_t n, i
   }
   if (p->st.trusted) {
     merge_partition_kernel<<<(int)((nb + 1 + 255) / 256), 256, 0, stream>>>(
-        m, nnz, row_ptr, base, (int)nb, p->d_block_row);
+        m, nnz, row_ptr, base, (int)nb, merge_items, p->d_block_row);
     e = hipStreamSynchronize(stream);
     if (e != hipSuccess) {
       asamd_csr_plan_destroy(p);
@@ -457,6 +475,10 @@ extern "C" int asamd_csr_plan_set_algo(asamd_csr_plan* p, int32_t algo) {
       if (!p->st.tiled_built) return hipErrorInvalidValue;
       p->st.algo = algo;
       return hipSuccess;
+    case ASAMD_SPMV_STREAM:
+      if (!stream_ok(p->st)) return hipErrorInvalidValue;
+      p->st.algo = algo;
+      return hipSuccess;
     case ASAMD_SPMV_VECTOR:
     case ASAMD_SPMV_MERGE:
     case ASAMD_SPMV_SCALAR:
@@ -497,6 +519,7 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
     const bool aligned = (((uintptr_t)val | (uintptr_t)ci) & 15u) == 0;
     if (!aligned || !rowconst_ok(st)) algo = ASAMD_SPMV_VECTOR;
   }
+  if (algo == ASAMD_SPMV_STREAM && !stream_ok(st)) algo = ASAMD_SPMV_MERGE;
   if (algo == ASAMD_SPMV_TILED && !st.tiled_built) algo = p->auto_algo == ASAMD_SPMV_TILED ? ASAMD_SPMV_MERGE : p->auto_algo;
   switch (algo) {
     case ASAMD_SPMV_TILED: {
@@ -520,6 +543,11 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
         default: launch_rowconst<T, 64>(s, st, alpha, val, ci, x, beta, y); break;
       }
       break;
+    case ASAMD_SPMV_STREAM: {
+      const unsigned grid = (unsigned)(((int64_t)st.m + kStreamRows - 1) / kStreamRows);
+      spmv_stream_kernel<T><<<grid, kStreamRows, 0, s>>>(st.m, alpha, val, rp, ci, x, beta, y, st.base);
+      break;
+    }
     case ASAMD_SPMV_SCALAR: {
       const unsigned grid = (unsigned)(((int64_t)st.m + kRowsBlock - 1) / kRowsBlock);
       spmv_scalar_kernel<T><<<grid, kRowsBlock, 0, s>>>(st.m, alpha, val, rp, ci, x, beta, y, st.base);
@@ -528,12 +556,17 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
     case ASAMD_SPMV_MERGE: {
       const int nb = st.merge_blocks;
       if (!p->coords_valid) {
-        merge_partition_kernel<<<(nb + 1 + 255) / 256, 256, 0, s>>>(st.m, st.nnz, rp, st.base, nb,
-                                                                    p->d_block_row);
+        merge_partition_kernel<<<(nb + 1 + 255) / 256, 256, 0, s>>>(
+            st.m, st.nnz, rp, st.base, nb, kMergeThreads * p->merge_ipt, p->d_block_row);
       }
-      spmv_merge_kernel<T><<<nb, kMergeThreads, 0, s>>>(st.m, st.nnz, alpha, val, rp, ci, x, beta, y,
-                                                        st.base, p->d_block_row, p->d_carry_row,
-                                                        (T*)p->d_carry_val, (T*)p->d_head_val);
+#define ASAMD_LAUNCH_MERGE(IPT)                                                                       \
+  spmv_merge_kernel<T, IPT><<<nb, kMergeThreads, 0, s>>>(st.m, st.nnz, alpha, val, rp, ci, x, beta, y, \
+                                                         st.base, p->d_block_row, p->d_carry_row,      \
+                                                         (T*)p->d_carry_val, (T*)p->d_head_val)
+      if (p->merge_ipt == 4) ASAMD_LAUNCH_MERGE(4);
+      else if (p->merge_ipt == 16) ASAMD_LAUNCH_MERGE(16);
+      else ASAMD_LAUNCH_MERGE(8);
+#undef ASAMD_LAUNCH_MERGE
       if (nb > 1)
         merge_fixup_kernel<T><<<(nb + 255) / 256, 256, 0, s>>>(nb, st.m, alpha, beta, p->d_carry_row,
                                                                (const T*)p->d_carry_val,

@@ -1,8 +1,8 @@
 // Merge-path CSR SpMV for gfx950 (wave64).
 //
 // The work list is the merge of the m row-end offsets with the nnz entry
-// indices (m + nnz items).  Every workgroup owns kMergeItems consecutive items
-// of that list, every thread kMergeIpt consecutive items of its workgroup's
+// indices (m + nnz items).  Every workgroup owns 256*IPT consecutive items
+// of that list, every thread IPT consecutive items of its workgroup's
 // share, so the load is balanced whatever the row-length distribution is: a
 // 200 000-entry row simply spans ~100 workgroups, a run of empty rows costs
 // one item each.
@@ -13,15 +13,17 @@
 //                               structure is promised fixed).
 //   2. spmv_merge_kernel        coalesced col/val streaming, x gathers,
 //                               products and row ends staged in LDS; each
-//                               thread walks its items, finished rows go to an
-//                               LDS row buffer, the unfinished tail of each
-//                               thread is combined by a segmented scan (wave
-//                               shuffles, then across the four waves in order);
-//                               rows finished inside the workgroup are written
-//                               coalesced as y = beta*y + alpha*sum, except the
-//                               workgroup's first row, which may have begun in
-//                               earlier workgroups: its partial sum goes to a
-//                               head slot, the unfinished tail to a carry slot.
+//                               thread walks its items, sums of finished rows go
+//                               to an LDS row buffer; the unfinished tail of
+//                               each thread is combined by a segmented scan
+//                               (wave shuffles, then across the four waves in
+//                               order) and completes the first row the next
+//                               thread finishes; rows finished inside the
+//                               workgroup are written unit stride as y = beta*y
+//                               + alpha*sum.  The workgroup's first row may have
+//                               begun in earlier workgroups: its partial sum
+//                               goes to a head slot, the unfinished tail of the
+//                               workgroup to a carry slot.
 //   3. merge_fixup_kernel       one thread per workgroup that finished a row:
 //                               sums the carries of the workgroups its first row
 //                               crossed, in workgroup order, adds the head slot
@@ -39,24 +41,23 @@
 namespace asamd {
 
 constexpr int kMergeThreads = 256;
-constexpr int kMergeIpt = 8;
-constexpr int kMergeItems = kMergeThreads * kMergeIpt;  // 2048 items per workgroup
 constexpr int kMergeWaves = kMergeThreads / kWave;
 
 // LDS index with one pad word per 32 so that lanes reading at a stride of
-// kMergeIpt words fall into distinct banks.
+// IPT words fall into distinct banks.
 __device__ __forceinline__ int lds_pad(int i) { return i + (i >> 5); }
 
 // block_row[b] = number of rows whose end offset is consumed before merge
-// diagonal b*kMergeItems, for b in [0, nblocks].
+// diagonal b*items_per_block, for b in [0, nblocks].
 __global__ __launch_bounds__(256) void merge_partition_kernel(int m, int nnz,
                                                               const int* __restrict__ row_ptr,
                                                               int base, int nblocks,
+                                                              int items_per_block,
                                                               int* __restrict__ block_row) {
   const int b = blockIdx.x * blockDim.x + threadIdx.x;
   if (b > nblocks) return;
   const int64_t total = (int64_t)m + nnz;
-  int64_t d = (int64_t)b * kMergeItems;
+  int64_t d = (int64_t)b * items_per_block;
   if (d > total) d = total;
   int64_t lo = d > nnz ? d - nnz : 0;
   int64_t hi = d < m ? d : m;
@@ -73,25 +74,28 @@ __global__ __launch_bounds__(256) void merge_partition_kernel(int m, int nnz,
   block_row[b] = (int)lo;
 }
 
-template <typename T>
+// IPT items per thread, kMergeThreads * IPT items per workgroup.
+template <typename T, int IPT>
 __global__ __launch_bounds__(kMergeThreads) void spmv_merge_kernel(
     int m, int nnz, T alpha, const T* __restrict__ val, const int* __restrict__ row_ptr,
     const int* __restrict__ col_ind, const T* __restrict__ x, T beta, T* __restrict__ y, int base,
     const int* __restrict__ block_row, int* __restrict__ carry_row, T* __restrict__ carry_val,
     T* __restrict__ head_val) {
-  __shared__ int s_rend[kMergeItems + 1];           // row ends, local to this workgroup's entry range
-  __shared__ T s_prod[kMergeItems + kMergeItems / 32 + 1];
-  __shared__ T s_rsum[kMergeItems];                 // totals of rows finished here
-  __shared__ int s_crow[kMergeThreads];             // per-thread unfinished row
-  __shared__ T s_cval[kMergeThreads];               // ... and its scanned partial sum
+  constexpr int kItems = kMergeThreads * IPT;
+  __shared__ int s_rend[kItems + 1];  // row ends, local to this workgroup's entry range
+  __shared__ T s_prod[kItems + kItems / 32 + 1];
+  __shared__ T s_rsum[kItems];           // totals of rows finished here, for unit-stride writes of y
+  __shared__ int s_crow[kMergeThreads];  // per-thread unfinished row
+  __shared__ T s_cval[kMergeThreads];    // ... and its scanned partial sum
   __shared__ int s_wrow[kMergeWaves];
   __shared__ T s_wval[kMergeWaves];
 
   const int tid = threadIdx.x;
-  const unsigned b = blockIdx.x;
+  // neighbouring workgroups gather neighbouring x: keep them on one XCD's L2
+  const unsigned b = xcd_contiguous_id(blockIdx.x, gridDim.x);
   const int64_t total = (int64_t)m + nnz;
-  const int64_t d0 = (int64_t)b * kMergeItems;
-  const int64_t d1 = d0 + kMergeItems < total ? d0 + kMergeItems : total;
+  const int64_t d0 = (int64_t)b * kItems;
+  const int64_t d1 = d0 + kItems < total ? d0 + kItems : total;
   const int row_b = block_row[b];
   const int row_e = block_row[b + 1];
   const int64_t nnz_b = d0 - row_b;
@@ -101,37 +105,37 @@ __global__ __launch_bounds__(kMergeThreads) void spmv_merge_kernel(
   // coordinates that do not describe this row_ptr (a stale cache) must not
   // drive any access out of bounds: clamp to what the LDS arrays and the
   // global arrays hold, results are then wrong but the launch is safe
-  if (rows_cnt < 0 || rows_cnt > kMergeItems || row_b < 0 || row_e > m) rows_cnt = 0;
-  if (nnz_cnt < 0 || nnz_cnt > kMergeItems || nnz_b < 0 || nnz_e > nnz) nnz_cnt = 0;
+  if (rows_cnt < 0 || rows_cnt > kItems || row_b < 0 || row_e > m) rows_cnt = 0;
+  if (nnz_cnt < 0 || nnz_cnt > kItems || nnz_b < 0 || nnz_e > nnz) nnz_cnt = 0;
   const int items = rows_cnt + nnz_cnt;
 
   // ---- stage row ends (one extra: the row still open at the end) ----------
   for (int i = tid; i <= rows_cnt; i += kMergeThreads) {
     const int64_t r = (int64_t)row_b + i;
-    const int64_t e = r < m ? (int64_t)row_ptr[r + 1] - base - nnz_b : (int64_t)kMergeItems + 1;
-    s_rend[i] = e > kMergeItems ? kMergeItems + 1 : (e < 0 ? 0 : (int)e);
+    const int64_t e = r < m ? (int64_t)row_ptr[r + 1] - base - nnz_b : (int64_t)kItems + 1;
+    s_rend[i] = e > kItems ? kItems + 1 : (e < 0 ? 0 : (int)e);
   }
   // ---- stream entries, gather x, stage products ----------------------------
   {
     const T* __restrict__ xb = x - base;
-    T v[kMergeIpt];
-    int c[kMergeIpt];
+    T v[IPT];
+    int c[IPT];
 #pragma unroll
-    for (int s = 0; s < kMergeIpt; ++s) {
+    for (int s = 0; s < IPT; ++s) {
       const int k = tid + s * kMergeThreads;
       if (k < nnz_cnt) {
         v[s] = val[nnz_b + k];
         c[s] = col_ind[nnz_b + k];
       }
     }
-    T xv[kMergeIpt];
+    T xv[IPT];
 #pragma unroll
-    for (int s = 0; s < kMergeIpt; ++s) {
+    for (int s = 0; s < IPT; ++s) {
       const int k = tid + s * kMergeThreads;
       if (k < nnz_cnt) xv[s] = xb[c[s]];
     }
 #pragma unroll
-    for (int s = 0; s < kMergeIpt; ++s) {
+    for (int s = 0; s < IPT; ++s) {
       const int k = tid + s * kMergeThreads;
       if (k < nnz_cnt) s_prod[lds_pad(k)] = v[s] * xv[s];
     }
@@ -139,9 +143,9 @@ __global__ __launch_bounds__(kMergeThreads) void spmv_merge_kernel(
   __syncthreads();
 
   // ---- this thread's start on the workgroup-local merge path ---------------
-  int dt = tid * kMergeIpt;
+  int dt = tid * IPT;
   if (dt > items) dt = items;
-  int dt_end = dt + kMergeIpt;
+  int dt_end = dt + IPT;
   if (dt_end > items) dt_end = items;
   int lo = dt > nnz_cnt ? dt - nnz_cnt : 0;
   int hi = dt < rows_cnt ? dt : rows_cnt;
@@ -157,18 +161,26 @@ __global__ __launch_bounds__(kMergeThreads) void spmv_merge_kernel(
   int j = dt - lo;  // local entry
   const int first_row = i;
   bool finished_any = false;
+  T first_sum = T(0);  // this thread's part of the first row it finishes
   T acc = T(0);
 #pragma unroll
-  for (int step = 0; step < kMergeIpt; ++step) {
+  for (int step = 0; step < IPT; ++step) {
     if (dt + step < dt_end) {
       const bool take_entry = j < nnz_cnt && (i >= rows_cnt || j < s_rend[i]);
       if (take_entry) {
         acc += s_prod[lds_pad(j)];
         ++j;
       } else if (i < rows_cnt) {
-        s_rsum[i] = acc;  // exactly one thread finishes a given row
+        // exactly one thread finishes a given row.  The first row it finishes
+        // may have been begun by the threads below and waits for their tails;
+        // any further row lies entirely inside this thread's items.
+        if (!finished_any) {
+          first_sum = acc;
+          finished_any = true;
+        } else {
+          s_rsum[i] = acc;
+        }
         acc = T(0);
-        finished_any = true;
         ++i;
       }
     }
@@ -200,17 +212,20 @@ __global__ __launch_bounds__(kMergeThreads) void spmv_merge_kernel(
   s_cval[tid] = tail;
   __syncthreads();
 
-  // the first row a thread finished may have been started by the threads below
-  if (finished_any && tid > 0 && s_crow[tid - 1] == first_row) s_rsum[first_row] += s_cval[tid - 1];
+  if (finished_any) {
+    // add what the threads below contributed to this thread's first finished row
+    if (tid > 0 && s_crow[tid - 1] == first_row) first_sum += s_cval[tid - 1];
+    s_rsum[first_row] = first_sum;
+  }
   if (tid == kMergeThreads - 1) {
     carry_row[b] = row_b + key;  // == row_e: the row still open, or m
     carry_val[b] = tail;
   }
   __syncthreads();
 
-  // ---- rows finished here: y = beta*y + alpha*sum, coalesced ----------------
-  // Local row 0 of every workgroup but the first may have begun earlier: the
-  // fix-up kernel completes it from head_val and the carries.
+  // ---- rows finished here: y = beta*y + alpha*sum, unit stride -----------------
+  // Local row 0 of every workgroup but the first may have begun in earlier
+  // workgroups: the fix-up kernel completes it from head_val and the carries.
   const int first_direct = b > 0 ? 1 : 0;
   if (tid == 0 && b > 0) head_val[b] = rows_cnt > 0 ? s_rsum[0] : T(0);
   for (int r = tid + first_direct; r < rows_cnt; r += kMergeThreads)

@@ -7,6 +7,9 @@
 //                               row*4*G: no row_ptr traffic, one 128-bit load of
 //                               values and one of indices per lane.
 //   spmv_scalar_kernel<T>       one lane per row (diagnostic baseline).
+//   spmv_stream_kernel<T>       rows of at most 16 entries: a workgroup stages the
+//                               products of 256 consecutive rows in LDS, one lane
+//                               per row sums them.
 //
 // They stand in for the reference's only CSR SpMV kernel, csr_gemv_vector
 // (src/kernel/dcu/level2/mv/csrmv/dcu_gemv_vector.h:14-57): same arithmetic
@@ -61,6 +64,58 @@ __global__ __launch_bounds__(kRowsBlock) void spmv_scalar_kernel(
   const T* __restrict__ xb = x - base;
   T sum = T(0);
   for (int64_t j = start; j < end; ++j) sum = fma_t(val[j], xb[col_ind[j]], sum);
+  store_axpby(y, row, alpha, sum, beta);
+}
+
+// ---- short rows: LDS-staged row blocks ---------------------------------------
+// A workgroup owns kStreamRows consecutive rows, none longer than
+// kStreamMaxLen.  Their entries are one contiguous range of the CSR streams: it
+// is read fully coalesced (lane k takes entries k, k + 256, ...), multiplied
+// with the gathered x and staged in LDS; after one barrier every lane sums the
+// few products of its own row from LDS (a lane's run is contiguous and runs of
+// neighbouring lanes are adjacent, so the reads spread over the banks) and
+// writes y unit stride.  No searches, no scans: this is what rows of 3-5
+// entries (stencils) want.
+constexpr int kStreamRows = 256;
+constexpr int kStreamMaxLen = 16;
+
+template <typename T>
+__global__ __launch_bounds__(kStreamRows) void spmv_stream_kernel(
+    int m, T alpha, const T* __restrict__ val, const int* __restrict__ row_ptr,
+    const int* __restrict__ col_ind, const T* __restrict__ x, T beta, T* __restrict__ y, int base) {
+  __shared__ T s_prod[kStreamRows * kStreamMaxLen];
+  const unsigned bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  const int64_t row0 = (int64_t)bid * kStreamRows;
+  const int64_t row = row0 + threadIdx.x;
+  int64_t row_last = row0 + kStreamRows;
+  if (row_last > m) row_last = m;
+  const int64_t e0 = (int64_t)row_ptr[row0] - base;
+  const int n = (int)((int64_t)row_ptr[row_last] - base - e0);  // <= kStreamRows * kStreamMaxLen by contract
+  int my_begin = 0, my_end = 0;
+  if (row < m) {
+    my_begin = (int)((int64_t)row_ptr[row] - base - e0);
+    my_end = (int)((int64_t)row_ptr[row + 1] - base - e0);
+  }
+  const T* __restrict__ xb = x - base;
+  T v[kStreamMaxLen];
+  int c[kStreamMaxLen];
+#pragma unroll
+  for (int s = 0; s < kStreamMaxLen; ++s) {
+    const int k = threadIdx.x + s * kStreamRows;
+    if (k < n) {
+      v[s] = val[e0 + k];
+      c[s] = col_ind[e0 + k];
+    }
+  }
+#pragma unroll
+  for (int s = 0; s < kStreamMaxLen; ++s) {
+    const int k = threadIdx.x + s * kStreamRows;
+    if (k < n) s_prod[k] = v[s] * xb[c[s]];
+  }
+  __syncthreads();
+  if (row >= m) return;
+  T sum = T(0);
+  for (int k = my_begin; k < my_end; ++k) sum += s_prod[k];
   store_axpby(y, row, alpha, sum, beta);
 }
 

@@ -162,5 +162,6 @@ int asamd_env_algo(void) {
   if (!strcmp(e, "merge")) return ASAMD_SPMV_MERGE;
   if (!strcmp(e, "scalar")) return ASAMD_SPMV_SCALAR;
   if (!strcmp(e, "tiled")) return ASAMD_SPMV_TILED;
+  if (!strcmp(e, "stream")) return ASAMD_SPMV_STREAM;
   return ASAMD_SPMV_AUTO;
 }

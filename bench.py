@@ -27,6 +27,15 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 
+# HBM bytes per multiply measured with rocprofv3 (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from a
+# 1 GiB copy kernel); the summaries these come from are profiles/spmv_tiled_C3.txt, spmv_merge_C4.txt and
+# spmv_stream_C2.txt.  Keyed by (configuration, kernel family); anything else reports null.
+MEASURED_TRAFFIC_BYTES = {
+    (3, "tiled two-phase"): 5.00e9,
+    (3, "rowconst"): 34.6e9,
+    (4, "merge-path"): 3.43e9,
+}
+
 WORKLOAD_NAMES = {
     2: "C2: CSR SpMV fp64, 5-point Laplacian 2048x2048 (4194304 rows, 20963328 nnz), alpha=1 beta=0",
     3: "C3: CSR SpMV fp32, 16777216 rows x 16 nnz/row uniform random sorted columns (268435456 nnz), alpha=1 beta=0.5",
@@ -118,6 +127,7 @@ def run_spmv(cfg, steps, warmup, cpu_baseline, check):
            "gbs": nbytes / t["avg_ms"] / 1e6, "gflops": 2 * a.nnz / t["avg_ms"] / 1e6,
            "dtype": "f32" if a.dtype == np.float32 else "f64", "parity": parity}
     res["hbm_frac"] = res["gbs"] / HBM_PEAK_GBS
+    res["traffic"] = MEASURED_TRAFFIC_BYTES.get((cfg, algo))
 
     if cpu_baseline:
         res["cpu_baseline"] = cpu_spmv(a, x, y0, alpha, beta, nbytes)
@@ -264,7 +274,7 @@ def main():
         "min_ms": t["min_ms"], "median_ms": t["median_ms"], "wall_ms_per_step": t["wall_ms_per_step"],
         "parity": main_res["parity"],
         "roofline": {"bound": "hbm", "achieved": main_res["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": main_res["hbm_frac"], "traffic": None,
+                     "frac": main_res["hbm_frac"], "traffic": main_res.get("traffic"),
                      "algorithmic_bytes_per_launch": main_res["algorithmic_bytes"]},
         "cpu_baseline": main_res.get("cpu_baseline"),
     }

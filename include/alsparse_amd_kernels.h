@@ -33,8 +33,9 @@ enum asamd_spmv_algo {
   ASAMD_SPMV_ROWCONST = 2, /* every row has the same length L = 4*G: no row_ptr read */
   ASAMD_SPMV_MERGE = 3,    /* merge-path split of (rows + nnz), LDS-staged products  */
   ASAMD_SPMV_SCALAR = 4,   /* one lane per row; diagnostic baseline                  */
-  ASAMD_SPMV_TILED = 5     /* two-phase, (column block x row block) tiles: every x
+  ASAMD_SPMV_TILED = 5,    /* two-phase, (column block x row block) tiles: every x
                               gather and y update in LDS, HBM sees only streams     */
+  ASAMD_SPMV_STREAM = 6    /* rows of <= 16 entries: 256 rows' products staged in LDS */
 };
 
 #define ASAMD_HIST_BINS 33
