@@ -13,6 +13,7 @@
 #include <algorithm>
 #include <cstdlib>
 #include <new>
+#include <vector>
 
 #include "alsparse_amd_kernels.h"
 #include "spmv_merge.hpp"
@@ -88,10 +89,11 @@ struct asamd_csr_plan {
   void* d_head_val;   // merge_blocks values: partial sum of each workgroup's first row
   bool coords_valid;  // d_block_row filled for a structure promised fixed
   // tiled two-phase copy (trusted plans only)
-  int tile_cols_log2, n_chunks;
+  int n_chunks;
+  int* d_row_block_start;     // row_blocks + 1 first rows
   TileRange* d_ranges;        // row_blocks * col_blocks tile ranges, row block major
-  LongTile* d_long;           // tiles summed by a whole workgroup, grouped by workgroup
-  int* d_long_ptr;            // reduce workgroups + 1
+  LongChunk* d_long;          // phase-3 work list: chunks of the tiles too long for phase 2
+  int n_long_chunks;
   void* d_tval;               // nnz values in tile order
   unsigned short* d_tcol;     // nnz local columns
   unsigned short* d_trow;     // nnz local rows
@@ -148,10 +150,11 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
 
 static void free_tiled(asamd_csr_plan* p) {
   if (p->d_ranges) (void)hipFree(p->d_ranges);
+  if (p->d_row_block_start) (void)hipFree(p->d_row_block_start);
+  p->d_row_block_start = nullptr;
   if (p->d_long) (void)hipFree(p->d_long);
-  if (p->d_long_ptr) (void)hipFree(p->d_long_ptr);
   p->d_long = nullptr;
-  p->d_long_ptr = nullptr;
+  p->n_long_chunks = 0;
   if (p->d_tval) (void)hipFree(p->d_tval);
   if (p->d_tcol) (void)hipFree(p->d_tcol);
   if (p->d_trow) (void)hipFree(p->d_trow);
@@ -164,43 +167,115 @@ static void free_tiled(asamd_csr_plan* p) {
   p->st.tiled_built = 0;
 }
 
-static int ilog2(int v) {
-  int l = 0;
-  while ((1 << l) < v) ++l;
-  return l;
-}
-
 template <typename T>
 static bool tiled_eligible(const asamd_csr_stats& st, bool force) {
+  // full-width block counts; the equal-entry cut (at most twice as many blocks
+  // per dimension) is checked again once it is known
   const int64_t cb = ((int64_t)st.n + TileDims<T>::cols - 1) / TileDims<T>::cols;
   const int64_t rb = ((int64_t)st.m + TileDims<T>::rows - 1) / TileDims<T>::rows;
-  if (!st.trusted || cb > kTiledMaxColBlocks || cb * rb > kTiledMaxTiles) return false;
+  if (!st.trusted || 2 * cb > kTiledMaxColBlocks || cb * rb > kTiledMaxTiles / 2) return false;
   // worth a try only when x cannot live in an XCD's 4 MiB L2 and the matrix is large
   return force || ((int64_t)st.n * (int64_t)sizeof(T) >= ((int64_t)8 << 20) && st.nnz >= (1 << 22));
 }
 
-// Stable sort of the entries by (column block, row block), then the arrays of
-// both phases in that order and the two tile tables.
+// Cuts groups [0, groups) with cumulative entry counts off[0..groups] into
+// consecutive blocks of at most max_groups groups holding about `target`
+// entries each.  group_block[g] = block of group g; returns the block starts
+// (in groups), the last element being `groups`.
+static std::vector<int> cut_blocks(const int* off, int groups, int max_groups, int64_t target,
+                                   std::vector<int>& group_block) {
+  std::vector<int> start;
+  group_block.resize((size_t)groups);
+  int g = 0;
+  while (g < groups) {
+    start.push_back(g);
+    int e = g + 1;  // a block holds at least one group
+    while (e < groups && e - g < max_groups && (int64_t)off[e + 1] - off[g] <= target) ++e;
+    for (int i = g; i < e; ++i) group_block[(size_t)i] = (int)start.size() - 1;
+    g = e;
+  }
+  start.push_back(groups);
+  return start;
+}
+
+// Equal-entry column / row blocks, stable sort of the entries by (column block,
+// row block), then the arrays of both phases in that order and the tile tables.
 template <typename T>
 static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* row_ptr,
                               const int* col_ind, const T* val) {
   asamd_csr_stats& st = p->st;
-  const int cb = (int)(((int64_t)st.n + TileDims<T>::cols - 1) / TileDims<T>::cols);
-  const int rb = (int)(((int64_t)st.m + TileDims<T>::rows - 1) / TileDims<T>::rows);
-  const int64_t tiles = (int64_t)cb * rb;
-  p->tile_cols_log2 = ilog2(TileDims<T>::cols);
+  const size_t nnz = (size_t)st.nnz;
+  const int col_groups = (int)(((int64_t)st.n + (1 << kColGroupLog2) - 1) >> kColGroupLog2);
+  const int row_groups = (int)(((int64_t)st.m + (1 << kRowGroupLog2) - 1) >> kRowGroupLog2);
+
+  int *d_coo = nullptr, *d_tile_ptr = nullptr, *d_long_count = nullptr, *d_cnt = nullptr;
+  int *d_cgb = nullptr, *d_rgb = nullptr, *d_cbs = nullptr;
+  LongTile* d_long_raw = nullptr;
+  unsigned *d_key = nullptr, *d_key2 = nullptr, *d_idx = nullptr, *d_perm = nullptr;
+  std::vector<int> h_off, cgb, rgb, cstart, rstart, h_colptr;
+  std::vector<TiledChunk> h_chunks;
+  int cb = 0, rb = 0;
+  int64_t tiles = 0;
+
+  // ---- 1. entry counts per column group and per row group -> block cuts ----------
+  const size_t cnt_n = (size_t)(col_groups > row_groups ? col_groups : row_groups) + 1;
+  hipError_t e = hipMalloc(&d_cnt, cnt_n * sizeof(int));
+  if (e == hipSuccess) e = hipMemsetAsync(d_cnt, 0, cnt_n * sizeof(int), stream);
+  if (e == hipSuccess) {
+    col_group_count_kernel<<<256 * 32, 256, 0, stream>>>(st.nnz, col_ind, st.base, d_cnt);
+    h_off.resize(cnt_n + 1);
+    e = hipMemcpyAsync(h_off.data() + 1, d_cnt, (size_t)col_groups * sizeof(int), hipMemcpyDeviceToHost, stream);
+  }
+  if (e == hipSuccess) e = hipStreamSynchronize(stream);
+  if (e == hipSuccess) {
+    h_off[0] = 0;
+    for (int g = 0; g < col_groups; ++g) h_off[(size_t)g + 1] += h_off[(size_t)g];
+    const int64_t full = ((int64_t)st.n + TileDims<T>::cols - 1) / TileDims<T>::cols;
+    cstart = cut_blocks(h_off.data(), col_groups, TileDims<T>::cols >> kColGroupLog2,
+                        (int64_t)st.nnz / full + 1, cgb);
+    cb = (int)cstart.size() - 1;
+    row_group_offsets_kernel<<<(row_groups + 1 + 255) / 256, 256, 0, stream>>>(st.m, row_ptr, row_groups, d_cnt);
+    e = hipMemcpyAsync(h_off.data(), d_cnt, ((size_t)row_groups + 1) * sizeof(int), hipMemcpyDeviceToHost, stream);
+  }
+  if (e == hipSuccess) e = hipStreamSynchronize(stream);
+  if (e == hipSuccess) {
+    for (int g = 0; g <= row_groups; ++g) h_off[(size_t)g] -= st.base;
+    const int64_t full = ((int64_t)st.m + TileDims<T>::rows - 1) / TileDims<T>::rows;
+    rstart = cut_blocks(h_off.data(), row_groups, TileDims<T>::rows >> kRowGroupLog2,
+                        (int64_t)st.nnz / full + 1, rgb);
+    rb = (int)rstart.size() - 1;
+    tiles = (int64_t)cb * rb;
+    if (cb > kTiledMaxColBlocks || tiles > kTiledMaxTiles) e = hipErrorOutOfMemory;  // treated as "no tiled copy"
+  }
   st.tile_col_blocks = cb;
   st.tile_row_blocks = rb;
-  const size_t nnz = (size_t)st.nnz;
   unsigned key_bits = 1;
   while (((int64_t)1 << key_bits) < tiles) ++key_bits;
 
-  int *d_coo = nullptr, *d_tile_ptr = nullptr, *d_long_count = nullptr;
-  LongTile* d_long_raw = nullptr;
-  unsigned *d_key = nullptr, *d_key2 = nullptr, *d_idx = nullptr, *d_perm = nullptr;
-  int* h_colptr = nullptr;
-  TiledChunk* h_chunks = nullptr;
-  hipError_t e = hipMalloc(&d_coo, nnz * sizeof(int));
+  // block starts in columns / rows
+  std::vector<int> h_cbs((size_t)cb + 1), h_rbs((size_t)rb + 1);
+  if (e == hipSuccess) {
+    for (int c = 0; c <= cb; ++c) {
+      const int64_t v = (int64_t)cstart[(size_t)c] << kColGroupLog2;
+      h_cbs[(size_t)c] = (int)(v < st.n ? v : st.n);
+    }
+    for (int r = 0; r <= rb; ++r) {
+      const int64_t v = (int64_t)rstart[(size_t)r] << kRowGroupLog2;
+      h_rbs[(size_t)r] = (int)(v < st.m ? v : st.m);
+    }
+  }
+  if (e == hipSuccess) e = hipMalloc(&d_cgb, (size_t)col_groups * sizeof(int));
+  if (e == hipSuccess) e = hipMalloc(&d_rgb, (size_t)row_groups * sizeof(int));
+  if (e == hipSuccess) e = hipMalloc(&d_cbs, ((size_t)cb + 1) * sizeof(int));
+  if (e == hipSuccess) e = hipMalloc(&p->d_row_block_start, ((size_t)rb + 1) * sizeof(int));
+  if (e == hipSuccess) e = hipMemcpy(d_cgb, cgb.data(), (size_t)col_groups * sizeof(int), hipMemcpyHostToDevice);
+  if (e == hipSuccess) e = hipMemcpy(d_rgb, rgb.data(), (size_t)row_groups * sizeof(int), hipMemcpyHostToDevice);
+  if (e == hipSuccess) e = hipMemcpy(d_cbs, h_cbs.data(), ((size_t)cb + 1) * sizeof(int), hipMemcpyHostToDevice);
+  if (e == hipSuccess)
+    e = hipMemcpy(p->d_row_block_start, h_rbs.data(), ((size_t)rb + 1) * sizeof(int), hipMemcpyHostToDevice);
+
+  // ---- 2. sort the entries by tile, gather the tile-ordered arrays ---------------
+  if (e == hipSuccess) e = hipMalloc(&d_coo, nnz * sizeof(int));
   if (e == hipSuccess) e = hipMalloc(&d_key, nnz * sizeof(unsigned));
   if (e == hipSuccess) e = hipMalloc(&d_key2, nnz * sizeof(unsigned));
   if (e == hipSuccess) e = hipMalloc(&d_idx, nnz * sizeof(unsigned));
@@ -216,75 +291,68 @@ static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* 
   if (e == hipSuccess) e = hipMalloc(&p->d_tprod, nnz * sizeof(T));
   if (e == hipSuccess) e = (hipError_t)asamd_csr2coo(stream, row_ptr, st.nnz, st.m, d_coo, st.base);
   if (e == hipSuccess) {
-    tile_keys_kernel<<<256 * 32, 256, 0, stream>>>(st.nnz, d_coo, col_ind, st.base, p->tile_cols_log2,
-                                                   TileDims<T>::rows_log2, rb, d_key, d_idx);
+    tile_keys_kernel<<<256 * 32, 256, 0, stream>>>(st.nnz, d_coo, col_ind, st.base, d_cgb, d_rgb, rb, d_key, d_idx);
     e = sort_pairs_u32(stream, d_key, d_key2, d_idx, d_perm, nnz, key_bits);
   }
   if (e == hipSuccess) {
-    tile_gather_kernel<T><<<256 * 32, 256, 0, stream>>>(st.nnz, d_perm, d_coo, col_ind, val, st.base,
-                                                        p->tile_cols_log2, TileDims<T>::rows_log2,
-                                                        (T*)p->d_tval, p->d_tcol, p->d_trow);
+    tile_gather_kernel<T><<<256 * 32, 256, 0, stream>>>(st.nnz, d_perm, d_coo, col_ind, val, st.base, d_cgb, d_cbs,
+                                                        d_rgb, p->d_row_block_start, (T*)p->d_tval,
+                                                        p->d_tcol, p->d_trow);
     tile_bounds_kernel<<<(unsigned)((tiles + 1 + 255) / 256), 256, 0, stream>>>(st.nnz, d_key2, tiles,
                                                                                 d_tile_ptr);
     e = hipMemsetAsync(d_long_count, 0, sizeof(int), stream);
     tile_ranges_kernel<<<(unsigned)((tiles + 255) / 256), 256, 0, stream>>>(rb, cb, d_tile_ptr, p->d_ranges,
                                                                             d_long_raw, d_long_count);
-    // phase-1 work list: every column block cut into chunks of at most kChunk entries
-    h_colptr = (int*)malloc((size_t)(cb + 1) * sizeof(int));
-    if (!h_colptr) e = hipErrorOutOfMemory;
+    h_colptr.resize((size_t)cb + 1);
   }
   if (e == hipSuccess)  // column block c starts at tile_ptr[c * rb]
-    e = hipMemcpy2DAsync(h_colptr, sizeof(int), d_tile_ptr, (size_t)rb * sizeof(int), sizeof(int),
+    e = hipMemcpy2DAsync(h_colptr.data(), sizeof(int), d_tile_ptr, (size_t)rb * sizeof(int), sizeof(int),
                          (size_t)cb + 1, hipMemcpyDeviceToHost, stream);
   if (e == hipSuccess) e = hipStreamSynchronize(stream);
+
+  // ---- 3. tiles too long for phase 2: cut into phase-3 chunks ----------------------
   if (e == hipSuccess) {
-    // long tiles, grouped by the reduce workgroup that owns their row block
-    const int n_wg = (rb + kRedWaves - 1) / kRedWaves;
     int n_long = 0;
     e = hipMemcpy(&n_long, d_long_count, sizeof(int), hipMemcpyDeviceToHost);
-    LongTile* h_long = (LongTile*)malloc((size_t)(n_long > 0 ? n_long : 1) * sizeof(LongTile));
-    int* h_lptr = (int*)calloc((size_t)n_wg + 1, sizeof(int));
-    if (!h_long || !h_lptr) e = hipErrorOutOfMemory;
+    std::vector<LongTile> h_long((size_t)(n_long > 0 ? n_long : 1));
     if (e == hipSuccess && n_long > 0)
-      e = hipMemcpy(h_long, d_long_raw, (size_t)n_long * sizeof(LongTile), hipMemcpyDeviceToHost);
-    if (e == hipSuccess) {
-      std::sort(h_long, h_long + n_long, [](const LongTile& a, const LongTile& b) {
-        return a.row_block != b.row_block ? a.row_block < b.row_block : a.begin < b.begin;
-      });
-      for (int i = 0; i < n_long; ++i) h_lptr[h_long[i].row_block / kRedWaves + 1]++;
-      for (int g = 0; g < n_wg; ++g) h_lptr[g + 1] += h_lptr[g];
-      e = hipMalloc(&p->d_long, (size_t)(n_long > 0 ? n_long : 1) * sizeof(LongTile));
-      if (e == hipSuccess) e = hipMalloc(&p->d_long_ptr, ((size_t)n_wg + 1) * sizeof(int));
-      if (e == hipSuccess && n_long > 0)
-        e = hipMemcpy(p->d_long, h_long, (size_t)n_long * sizeof(LongTile), hipMemcpyHostToDevice);
-      if (e == hipSuccess)
-        e = hipMemcpy(p->d_long_ptr, h_lptr, ((size_t)n_wg + 1) * sizeof(int), hipMemcpyHostToDevice);
-    }
-    free(h_long);
-    free(h_lptr);
-  }
-  if (e == hipSuccess) {
-    const int kChunk = 128 * 1024;
-    int64_t n_chunks = 0;
-    for (int c = 0; c < cb; ++c) n_chunks += ((int64_t)h_colptr[c + 1] - h_colptr[c] + kChunk - 1) / kChunk;
-    h_chunks = (TiledChunk*)malloc((size_t)(n_chunks > 0 ? n_chunks : 1) * sizeof(TiledChunk));
-    if (!h_chunks) {
-      e = hipErrorOutOfMemory;
-    } else {
-      int64_t q = 0;
-      for (int c = 0; c < cb; ++c) {
-        for (int64_t b = h_colptr[c]; b < h_colptr[c + 1]; b += kChunk) {
-          h_chunks[q].col_block = c;
-          h_chunks[q].begin = (int)b;
-          h_chunks[q].end = (int)(b + kChunk < h_colptr[c + 1] ? b + kChunk : h_colptr[c + 1]);
-          ++q;
+      e = hipMemcpy(h_long.data(), d_long_raw, (size_t)n_long * sizeof(LongTile), hipMemcpyDeviceToHost);
+    if (e == hipSuccess && n_long > 0) {
+      std::sort(h_long.begin(), h_long.begin() + n_long,
+                [](const LongTile& a, const LongTile& b) { return a.begin < b.begin; });
+      std::vector<LongChunk> h_lc;
+      for (int i = 0; i < n_long; ++i) {
+        for (int64_t b = h_long[(size_t)i].begin; b < h_long[(size_t)i].end; b += kLongChunk) {
+          LongChunk c;
+          c.begin = (int)b;
+          c.end = (int)(b + kLongChunk < h_long[(size_t)i].end ? b + kLongChunk : h_long[(size_t)i].end);
+          c.row0 = h_rbs[(size_t)h_long[(size_t)i].row_block];
+          h_lc.push_back(c);
         }
       }
-      p->n_chunks = (int)n_chunks;
-      e = hipMalloc(&p->d_chunks, (size_t)(n_chunks > 0 ? n_chunks : 1) * sizeof(TiledChunk));
-      if (e == hipSuccess && n_chunks > 0)
-        e = hipMemcpy(p->d_chunks, h_chunks, (size_t)n_chunks * sizeof(TiledChunk), hipMemcpyHostToDevice);
+      p->n_long_chunks = (int)h_lc.size();
+      e = hipMalloc(&p->d_long, h_lc.size() * sizeof(LongChunk));
+      if (e == hipSuccess)
+        e = hipMemcpy(p->d_long, h_lc.data(), h_lc.size() * sizeof(LongChunk), hipMemcpyHostToDevice);
     }
+  }
+  // ---- 4. phase-1 work list: every column block cut into chunks of at most kChunk entries
+  if (e == hipSuccess) {
+    const int kChunk = 128 * 1024;
+    for (int c = 0; c < cb; ++c) {
+      for (int64_t b = h_colptr[(size_t)c]; b < h_colptr[(size_t)c + 1]; b += kChunk) {
+        TiledChunk ch;
+        ch.col0 = h_cbs[(size_t)c];
+        ch.ncols = h_cbs[(size_t)c + 1] - h_cbs[(size_t)c];
+        ch.begin = (int)b;
+        ch.end = (int)(b + kChunk < h_colptr[(size_t)c + 1] ? b + kChunk : h_colptr[(size_t)c + 1]);
+        h_chunks.push_back(ch);
+      }
+    }
+    p->n_chunks = (int)h_chunks.size();
+    e = hipMalloc(&p->d_chunks, (h_chunks.size() ? h_chunks.size() : 1) * sizeof(TiledChunk));
+    if (e == hipSuccess && !h_chunks.empty())
+      e = hipMemcpy(p->d_chunks, h_chunks.data(), h_chunks.size() * sizeof(TiledChunk), hipMemcpyHostToDevice);
   }
   if (e == hipSuccess)  // both phases use more than the default 64 KiB of dynamic LDS
     e = hipFuncSetAttribute((const void*)tiled_products_kernel<T>,
@@ -292,10 +360,8 @@ static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* 
   if (e == hipSuccess)
     e = hipFuncSetAttribute((const void*)tiled_reduce_kernel<T>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, kRedBytes);
-  free(h_colptr);
-  free(h_chunks);
   for (void* d : {(void*)d_coo, (void*)d_key, (void*)d_key2, (void*)d_idx, (void*)d_perm, (void*)d_tile_ptr,
-                  (void*)d_long_raw, (void*)d_long_count})
+                  (void*)d_long_raw, (void*)d_long_count, (void*)d_cnt, (void*)d_cgb, (void*)d_rgb, (void*)d_cbs})
     if (d) (void)hipFree(d);
   if (e != hipSuccess) {
     free_tiled(p);
@@ -526,10 +592,13 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
       // the tiled copy holds zero-based local indices and its own values
       if (p->n_chunks > 0)
         tiled_products_kernel<T><<<p->n_chunks, kProdThreads, kTileBytes, s>>>(
-            st.n, p->d_chunks, (const T*)p->d_tval, p->d_tcol, x, (T*)p->d_tprod);
+            p->d_chunks, (const T*)p->d_tval, p->d_tcol, x, (T*)p->d_tprod);
       tiled_reduce_kernel<T><<<(st.tile_row_blocks + kRedWaves - 1) / kRedWaves, kRedThreads, kRedBytes, s>>>(
-          st.m, st.tile_row_blocks, st.tile_col_blocks, p->d_ranges, p->d_long_ptr, p->d_long, p->d_trow,
+          st.m, st.tile_row_blocks, st.tile_col_blocks, p->d_row_block_start, p->d_ranges, p->d_trow,
           (const T*)p->d_tprod, alpha, beta, y);
+      if (p->n_long_chunks > 0)
+        tiled_long_kernel<T><<<p->n_long_chunks, kLongThreads, 0, s>>>(p->d_long, p->d_trow,
+                                                                       (const T*)p->d_tprod, alpha, y);
       break;
     }
     case ASAMD_SPMV_ROWCONST:
@@ -545,7 +614,12 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
       break;
     case ASAMD_SPMV_STREAM: {
       const unsigned grid = (unsigned)(((int64_t)st.m + kStreamRows - 1) / kStreamRows);
-      spmv_stream_kernel<T><<<grid, kStreamRows, 0, s>>>(st.m, alpha, val, rp, ci, x, beta, y, st.base);
+      if (st.max_len <= 4)
+        spmv_stream_kernel<T, 4><<<grid, kStreamRows, 0, s>>>(st.m, alpha, val, rp, ci, x, beta, y, st.base);
+      else if (st.max_len <= 8)
+        spmv_stream_kernel<T, 8><<<grid, kStreamRows, 0, s>>>(st.m, alpha, val, rp, ci, x, beta, y, st.base);
+      else
+        spmv_stream_kernel<T, 16><<<grid, kStreamRows, 0, s>>>(st.m, alpha, val, rp, ci, x, beta, y, st.base);
       break;
     }
     case ASAMD_SPMV_SCALAR: {

@@ -79,28 +79,30 @@ __global__ __launch_bounds__(kRowsBlock) void spmv_scalar_kernel(
 constexpr int kStreamRows = 256;
 constexpr int kStreamMaxLen = 16;
 
-template <typename T>
+// CAP: compile-time bound on the row length (4, 8 or 16): sizes the LDS staging
+// area, so shorter rows leave room for more resident workgroups.
+template <typename T, int CAP>
 __global__ __launch_bounds__(kStreamRows) void spmv_stream_kernel(
     int m, T alpha, const T* __restrict__ val, const int* __restrict__ row_ptr,
     const int* __restrict__ col_ind, const T* __restrict__ x, T beta, T* __restrict__ y, int base) {
-  __shared__ T s_prod[kStreamRows * kStreamMaxLen];
+  __shared__ T s_prod[kStreamRows * CAP];
   const unsigned bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
   const int64_t row0 = (int64_t)bid * kStreamRows;
   const int64_t row = row0 + threadIdx.x;
   int64_t row_last = row0 + kStreamRows;
   if (row_last > m) row_last = m;
   const int64_t e0 = (int64_t)row_ptr[row0] - base;
-  const int n = (int)((int64_t)row_ptr[row_last] - base - e0);  // <= kStreamRows * kStreamMaxLen by contract
+  const int n = (int)((int64_t)row_ptr[row_last] - base - e0);  // <= kStreamRows * CAP by contract
   int my_begin = 0, my_end = 0;
   if (row < m) {
     my_begin = (int)((int64_t)row_ptr[row] - base - e0);
     my_end = (int)((int64_t)row_ptr[row + 1] - base - e0);
   }
   const T* __restrict__ xb = x - base;
-  T v[kStreamMaxLen];
-  int c[kStreamMaxLen];
+  T v[CAP];
+  int c[CAP];
 #pragma unroll
-  for (int s = 0; s < kStreamMaxLen; ++s) {
+  for (int s = 0; s < CAP; ++s) {
     const int k = threadIdx.x + s * kStreamRows;
     if (k < n) {
       v[s] = val[e0 + k];
@@ -108,7 +110,7 @@ __global__ __launch_bounds__(kStreamRows) void spmv_stream_kernel(
     }
   }
 #pragma unroll
-  for (int s = 0; s < kStreamMaxLen; ++s) {
+  for (int s = 0; s < CAP; ++s) {
     const int k = threadIdx.x + s * kStreamRows;
     if (k < n) s_prod[k] = v[s] * xb[c[s]];
   }

@@ -5,9 +5,12 @@
 // L2 of an XCD, each x gather of the row-parallel kernels misses L2 and moves a
 // whole 128-byte line for 4 useful bytes; measured on the 16 M-row uniform
 // matrix that is 34.6 GB of fabric traffic for 2.4 GB of algorithmic bytes.
-// Here the matrix is re-laid-out once (analysis) into tiles of
-// TileDims::cols columns x kTileRows rows, tiles ordered by (column block, row
-// block), entries inside a tile in CSR order (stable sort):
+// Here the matrix is re-laid-out once (analysis) into tiles: column blocks of at
+// most TileDims::cols columns and row blocks of at most TileDims::rows rows, both
+// cut so that every block holds about the same number of entries (hot columns
+// and long rows get narrower blocks, so tiles stay even on skewed matrices);
+// tiles are ordered by (column block, row block), entries inside a tile in CSR
+// order (stable sort):
 //
 //   phase 1  tiled_products_kernel   one workgroup per chunk of a column block:
 //            the block's x slice (128 KiB) is copied to LDS, then the chunk's
@@ -26,13 +29,17 @@
 //            consecutive row blocks, whose tiles are adjacent in memory, and a
 //            barrier per batch of column blocks keeps them in step, so DRAM sees
 //            one multi-KiB burst per column block instead of scattered 256-byte
-//            reads.  Tiles longer than kLongTile entries (long rows) are summed
-//            by the whole workgroup beforehand, one LDS atomic per wave and row.
-//            Finally y = beta*y + alpha*acc, unit stride.
+//            reads.  Finally y = beta*y + alpha*acc, unit stride.
+//   phase 3  tiled_long_kernel       only if some tile holds more than kLongTile
+//            entries (long rows, hot columns): those tiles are left out of phase
+//            2 and streamed by as many workgroups as their size needs; rows are
+//            pre-combined inside each wave and added to y with global atomics
+//            (a 200 000-entry row costs a few thousand of them).
 //
 // HBM traffic is 2*sizeof(T) + 4 bytes per entry more than plain CSR (the
 // product round trip and the second index), all of it streamed.  The order of
-// every addition is fixed by the layout, so results are bit-reproducible.
+// every addition in phases 1 and 2 is fixed by the layout, so results are
+// bit-reproducible; only rows that reach phase 3 see atomics in arbitrary order.
 // The reference has no counterpart; per-entry arithmetic is that of
 // src/kernel/dcu/level2/mv/csrmv/dcu_gemv_vector.h:43-54.
 #pragma once
@@ -48,20 +55,24 @@ constexpr int kRedWaves = 8;            // phase-2 workgroup: 8 waves = 8 consec
 constexpr int kRedThreads = kRedWaves * kWave;  // whose tiles are adjacent in memory for every column block
 constexpr int kRedUnroll = 8;
 constexpr int kRedBytes = kTileBytes / 2;  // LDS bytes of a phase-2 workgroup's accumulators
-constexpr int kLongTile = 1024;         // tiles with more entries are summed by the whole workgroup
+constexpr int kLongTile = 2 * kWave;     // phase 2 takes two entries per lane and tile; longer tiles go to phase 3
+constexpr int kLongThreads = 256;
+constexpr int kLongChunk = kLongThreads * 16;  // entries per phase-3 workgroup
 constexpr int kTiledMaxColBlocks = 2048;       // keeps the tile table small
-constexpr int64_t kTiledMaxTiles = (int64_t)1 << 24;
+constexpr int64_t kTiledMaxTiles = (int64_t)1 << 25;  // 12 bytes of tables per tile
+
+constexpr int kColGroupLog2 = 8;        // column blocks are cut at multiples of 256 columns,
+constexpr int kRowGroupLog2 = 6;        // row blocks at multiples of 64 rows
 
 template <typename T>
 struct TileDims {
-  static constexpr int cols = kTileBytes / (int)sizeof(T);            // 32768 fp32, 16384 fp64
-  static constexpr int rows = kRedBytes / kRedWaves / (int)sizeof(T);  // rows per wave: 2048 fp32, 1024 fp64
-  static constexpr int rows_log2 = sizeof(T) == 4 ? 11 : 10;
+  static constexpr int cols = kTileBytes / (int)sizeof(T);            // widest column block: 32768 fp32, 16384 fp64
+  static constexpr int rows = kRedBytes / kRedWaves / (int)sizeof(T);  // tallest row block: 2048 fp32, 1024 fp64
 };
 
 struct TiledChunk {
-  int col_block;
-  int begin;  // entry range [begin, end) in tile order
+  int col0, ncols;  // the chunk's column block
+  int begin;        // entry range [begin, end) in tile order
   int end;
 };
 
@@ -74,35 +85,63 @@ struct LongTile {
   int row_block;
 };
 
+struct LongChunk {
+  int begin, end;  // entry range inside one long tile
+  int row0;        // first row of the tile's row block
+};
+
 // ---- analysis ----------------------------------------------------------------
+// Entries per group of 256 columns (for cutting equal-entry column blocks).
+__global__ __launch_bounds__(256) void col_group_count_kernel(int nnz, const int* __restrict__ col_ind,
+                                                              int base, int* __restrict__ count) {
+  for (int64_t k = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; k < nnz;
+       k += (int64_t)gridDim.x * blockDim.x)
+    atomicAdd(&count[(col_ind[k] - base) >> kColGroupLog2], 1);
+}
+
+// out[g] = row_ptr[g * 64] for g in [0, groups], the last one clamped to row_ptr[m].
+__global__ __launch_bounds__(256) void row_group_offsets_kernel(int m, const int* __restrict__ row_ptr,
+                                                                int groups, int* __restrict__ out) {
+  const int g = blockIdx.x * blockDim.x + threadIdx.x;
+  if (g > groups) return;
+  int64_t r = (int64_t)g << kRowGroupLog2;
+  if (r > m) r = m;
+  out[g] = row_ptr[r];
+}
+
 // key[k] = col_block * row_blocks + row_block of entry k; idx[k] = k.
-// coo_row holds the row of every entry in the matrix's index base.
+// coo_row holds the row of every entry in the matrix's index base; the block of
+// a column / row is looked up through its group.
 __global__ __launch_bounds__(256) void tile_keys_kernel(int nnz, const int* __restrict__ coo_row,
                                                         const int* __restrict__ col_ind, int base,
-                                                        int tile_cols_log2, int tile_rows_log2,
+                                                        const int* __restrict__ col_group_block,
+                                                        const int* __restrict__ row_group_block,
                                                         int row_blocks, unsigned* __restrict__ key,
                                                         unsigned* __restrict__ idx) {
   for (int64_t k = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; k < nnz;
        k += (int64_t)gridDim.x * blockDim.x) {
-    const unsigned cb = (unsigned)(col_ind[k] - base) >> tile_cols_log2;
-    const unsigned rb = (unsigned)(coo_row[k] - base) >> tile_rows_log2;
+    const unsigned cb = (unsigned)col_group_block[(col_ind[k] - base) >> kColGroupLog2];
+    const unsigned rb = (unsigned)row_group_block[(coo_row[k] - base) >> kRowGroupLog2];
     key[k] = cb * (unsigned)row_blocks + rb;
     idx[k] = (unsigned)k;
   }
 }
 
-// Entries in sorted order: values, local columns, local rows.
+// Entries in sorted order: values, columns and rows local to their blocks.
 template <typename T>
 __global__ __launch_bounds__(256) void tile_gather_kernel(
     int nnz, const unsigned* __restrict__ perm, const int* __restrict__ coo_row,
-    const int* __restrict__ col_ind, const T* __restrict__ val, int base, int tile_cols_log2,
-    int tile_rows_log2, T* __restrict__ t_val, unsigned short* __restrict__ t_col, unsigned short* __restrict__ t_row) {
+    const int* __restrict__ col_ind, const T* __restrict__ val, int base,
+    const int* __restrict__ col_group_block, const int* __restrict__ col_block_start,
+    const int* __restrict__ row_group_block, const int* __restrict__ row_block_start,
+    T* __restrict__ t_val, unsigned short* __restrict__ t_col, unsigned short* __restrict__ t_row) {
   for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < nnz;
        q += (int64_t)gridDim.x * blockDim.x) {
     const unsigned k = perm[q];
+    const int col = col_ind[k] - base, row = coo_row[k] - base;
     t_val[q] = val[k];
-    t_col[q] = (unsigned short)((col_ind[k] - base) & ((1 << tile_cols_log2) - 1));
-    t_row[q] = (unsigned short)((coo_row[k] - base) & ((1 << tile_rows_log2) - 1));
+    t_col[q] = (unsigned short)(col - col_block_start[col_group_block[col >> kColGroupLog2]]);
+    t_row[q] = (unsigned short)(row - row_block_start[row_group_block[row >> kRowGroupLog2]]);
   }
 }
 
@@ -148,15 +187,12 @@ __global__ __launch_bounds__(256) void tile_ranges_kernel(int row_blocks, int co
 // ---- phase 1 -------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(kProdThreads) void tiled_products_kernel(
-    int n, const TiledChunk* __restrict__ chunks, const T* __restrict__ t_val,
+    const TiledChunk* __restrict__ chunks, const T* __restrict__ t_val,
     const unsigned short* __restrict__ t_col, const T* __restrict__ x, T* __restrict__ prod) {
   extern __shared__ __align__(16) unsigned char smem[];
   T* xs = reinterpret_cast<T*>(smem);
   const TiledChunk ch = chunks[blockIdx.x];
-  const int64_t col0 = (int64_t)ch.col_block * TileDims<T>::cols;
-  int64_t ncols = (int64_t)n - col0;
-  if (ncols > TileDims<T>::cols) ncols = TileDims<T>::cols;
-  for (int i = threadIdx.x; i < ncols; i += kProdThreads) xs[i] = x[col0 + i];
+  for (int i = threadIdx.x; i < ch.ncols; i += kProdThreads) xs[i] = x[(int64_t)ch.col0 + i];
   __syncthreads();
   constexpr int kStep = kProdThreads * kProdUnroll;
   int k = ch.begin + threadIdx.x;
@@ -176,16 +212,23 @@ __global__ __launch_bounds__(kProdThreads) void tiled_products_kernel(
 
 // ---- phase 2 -------------------------------------------------------------------
 // acc[r] += v for the valid lanes of one wave instruction.  acc is private to
-// the wave.  Entries of one row are adjacent (a tile is stored in CSR order), so
-// lanes that share a row with their neighbour are combined inside the wave
-// first and the read-modify-writes of one instruction never collide.  Isolated
-// pairs (the usual case on short rows) cost three DPP wave shifts; longer runs
-// take a segmented suffix sum.
+// the wave (or updated atomically).  Entries of one row are adjacent (a tile is
+// stored in CSR order), so the lanes of a run of equal rows must not all do
+// their read-modify-write at once.  From the ballot of "same row as the lane
+// below" every lane knows its position in its run:
+//   * only isolated pairs: the first lane of a pair takes its neighbour's value
+//     through a DPP wave shift;
+//   * runs of at most kMaxPasses lanes: pass p lets the p-th lane of every run
+//     add, so the lanes of one pass always hold distinct rows;
+//   * longer runs (long rows): a segmented suffix sum inside the wave leaves the
+//     run's total in its first lane, which adds alone.
 template <bool Atomic, typename T>
 __device__ __forceinline__ void rmw(T* p, T v) {
   if constexpr (Atomic) atomicAdd(p, v);
   else *p += v;
 }
+
+constexpr int kMaxPasses = 4;
 
 template <bool Atomic = false, typename T>
 __device__ __forceinline__ void add_rows(T* acc, int r, T v, bool valid) {
@@ -195,28 +238,49 @@ __device__ __forceinline__ void add_rows(T* acc, int r, T v, bool valid) {
   const uint64_t dup = __builtin_amdgcn_ballot_w64(same_as_prev);
   if (dup == 0) {
     if (valid) rmw<Atomic>(&acc[r], v);
-  } else if ((dup & (dup << 1)) == 0) {
-    // runs of exactly two: the first lane takes its neighbour's value
+    return;
+  }
+  if ((dup & (dup << 1)) == 0) {
+    // runs of exactly two (the usual case on short rows): the first lane takes
+    // its neighbour's value, three DPP wave shifts in all
     const T v_next = dpp_mov<0x130>(v);  // wave_shl:1: value of lane + 1 (0 past the end)
     if ((dup >> 1 >> lane) & 1) v += v_next;
     if (valid && !same_as_prev) rmw<Atomic>(&acc[r], v);
-  } else {
-#pragma unroll
-    for (int d = 1; d < kWave; d <<= 1) {
-      const T vd = __shfl_down(v, d, kWave);
-      const int rd = __shfl_down(r, d, kWave);
-      if (lane + d < kWave && rd == r) v += vd;
-    }
-    if (valid && !same_as_prev) rmw<Atomic>(&acc[r], v);
+    return;
   }
+  // first lane of my run: highest lane <= me whose dup bit is clear
+  const uint64_t heads_below = ~dup & (((uint64_t)2 << lane) - 1);
+  const int pos = lane - (63 - __builtin_clzll(heads_below));
+  // a run longer than kMaxPasses shows as kMaxPasses consecutive dup bits
+  uint64_t longrun = dup;
+#pragma unroll
+  for (int p = 1; p < kMaxPasses; ++p) longrun &= dup >> p;
+  if (longrun == 0) {
+    if (!Atomic) {
+#pragma unroll
+      for (int p = 0; p < kMaxPasses; ++p) {
+        if (p > 0 && __builtin_amdgcn_ballot_w64(valid && pos == p) == 0) break;
+        if (valid && pos == p) acc[r] += v;
+      }
+      return;
+    }
+  }
+  // suffix sums inside every run; lane + d belongs to my run iff the d dup bits above me are all set
+  const uint64_t above = dup >> 1 >> lane;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const T vd = __shfl_down(v, d, kWave);
+    const uint64_t need = ((uint64_t)1 << d) - 1;
+    if ((above & need) == need) v += vd;
+  }
+  if (valid && !same_as_prev) rmw<Atomic>(&acc[r], v);
 }
 
 template <typename T>
 __global__ __launch_bounds__(kRedThreads) void tiled_reduce_kernel(
-    int m, int row_blocks, int col_blocks, const TileRange* __restrict__ ranges,
-    const int* __restrict__ long_ptr, const LongTile* __restrict__ long_tiles,
-    const unsigned short* __restrict__ t_row, const T* __restrict__ prod, T alpha, T beta,
-    T* __restrict__ y) {
+    int m, int row_blocks, int col_blocks, const int* __restrict__ row_block_start,
+    const TileRange* __restrict__ ranges, const unsigned short* __restrict__ t_row,
+    const T* __restrict__ prod, T alpha, T beta, T* __restrict__ y) {
   extern __shared__ __align__(16) unsigned char smem[];
   T* s_acc = reinterpret_cast<T*>(smem);
   constexpr int kTileRows = TileDims<T>::rows;
@@ -226,66 +290,108 @@ __global__ __launch_bounds__(kRedThreads) void tiled_reduce_kernel(
   const bool active = rb < row_blocks;  // wave-uniform; idle waves still meet the barriers
   T* acc = s_acc + wave * kTileRows;
   for (int i = lane; i < kTileRows; i += kWave) acc[i] = T(0);
-  __syncthreads();
 
-  // ---- long tiles of this workgroup: all waves, one LDS atomic per wave and row
-  const int lt0 = long_ptr[blockIdx.x], lt1 = long_ptr[blockIdx.x + 1];
-  for (int lt = lt0; lt < lt1; ++lt) {
-    const LongTile t = long_tiles[lt];
-    T* tacc = s_acc + (t.row_block - blockIdx.x * kRedWaves) * kTileRows;
-    for (int k0 = t.begin; k0 < t.end; k0 += kRedThreads) {  // workgroup-uniform trip count
-      const int k = k0 + threadIdx.x;
-      const bool ok = k < t.end;
-      const T v = ok ? prod[k] : T(0);
-      const int r = ok ? (int)t_row[k] : -1 - lane;
-      add_rows<true>(tacc, r, v, ok);
-    }
-  }
-  if (lt1 > lt0) __syncthreads();
-
-  // ---- short tiles: wave-private accumulators, batches of kRedUnroll column blocks
+  // Wave-private accumulators; the tiles of kRedUnroll column blocks form a batch
+  // (every tile listed in `ranges` has at most kLongTile = 128 entries: two per
+  // lane).  The loads of batch q + 1 are issued before batch q is added, so the
+  // LDS read-modify-write chain of one batch hides the memory latency of the next.
+  struct Batch {
+    T v[kRedUnroll][2];
+    int r[kRedUnroll][2];
+    int len[kRedUnroll];
+  };
   const TileRange* my = ranges + (int64_t)(active ? rb : 0) * col_blocks;
-  for (int cb0 = 0; cb0 < col_blocks; cb0 += kWave) {
-    TileRange tr = {0, 0};
-    if (active && cb0 + lane < col_blocks) tr = my[cb0 + lane];  // 64 tile ranges, one coalesced load
-    const int ncb = col_blocks - cb0 < kWave ? col_blocks - cb0 : kWave;
-    for (int j = 0; j < ncb; j += kRedUnroll) {
-      // every lane takes up to two entries of each of kRedUnroll tiles, all loads in flight together
-      T v[kRedUnroll][2];
-      int r[kRedUnroll][2];
-      int b[kRedUnroll], e[kRedUnroll];
+  constexpr int kPerGroup = kWave / kRedUnroll;  // batches per group of 64 tile ranges
+  const int nq = (col_blocks + kRedUnroll - 1) / kRedUnroll;
+  auto load_ranges = [&](int group) {  // 64 tile ranges, one coalesced load
+    TileRange t = {0, 0};
+    const int cb = group * kWave + lane;
+    if (active && cb < col_blocks) t = my[cb];
+    return t;
+  };
+  auto fetch = [&](const TileRange& tr, int q, Batch& bt) {
+    const int j = (q % kPerGroup) * kRedUnroll;
+    const int left = col_blocks - (q / kPerGroup) * kWave;
+    const int ncb = left < kWave ? left : kWave;
 #pragma unroll
-      for (int u = 0; u < kRedUnroll; ++u) {
-        const int src = j + u < ncb ? j + u : j;
-        b[u] = __builtin_amdgcn_readlane(tr.begin, src);
-        e[u] = j + u < ncb ? __builtin_amdgcn_readlane(tr.end, src) : b[u];
+    for (int u = 0; u < kRedUnroll; ++u) {
+      const int src = j + u < ncb ? j + u : j;
+      const int b = __builtin_amdgcn_readlane(tr.begin, src);
+      const int e = j + u < ncb ? __builtin_amdgcn_readlane(tr.end, src) : b;
+      bt.len[u] = e - b;
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          const int k = b[u] + h * kWave + lane;
-          const bool ok = k < e[u];
-          v[u][h] = ok ? prod[k] : T(0);
-          r[u][h] = ok ? (int)t_row[k] : -1 - lane;
-        }
+      for (int h = 0; h < 2; ++h) {
+        const int k = b + h * kWave + lane;
+        const bool ok = k < e;
+        bt.v[u][h] = ok ? prod[k] : T(0);
+        bt.r[u][h] = ok ? (int)t_row[k] : -1 - lane;
       }
-#pragma unroll
-      for (int u = 0; u < kRedUnroll; ++u) {
-        add_rows(acc, r[u][0], v[u][0], r[u][0] >= 0);
-        if (e[u] - b[u] > kWave) add_rows(acc, r[u][1], v[u][1], r[u][1] >= 0);  // wave-uniform
-        for (int k = b[u] + 2 * kWave + lane; k - lane < e[u]; k += kWave) {  // tiles of 129 .. kLongTile entries
-          const bool ok = k < e[u];
-          const T v2 = ok ? prod[k] : T(0);
-          const int r2 = ok ? (int)t_row[k] : -1 - lane;
-          add_rows(acc, r2, v2, ok);
-        }
-      }
-      __syncthreads();  // keeps the waves on neighbouring tiles: their reads form one burst
     }
+  };
+  auto add = [&](const Batch& bt) {
+#pragma unroll
+    for (int u = 0; u < kRedUnroll; ++u) {
+      add_rows(acc, bt.r[u][0], bt.v[u][0], bt.r[u][0] >= 0);
+      if (bt.len[u] > kWave) add_rows(acc, bt.r[u][1], bt.v[u][1], bt.r[u][1] >= 0);  // wave-uniform
+    }
+  };
+  Batch A, B;
+  TileRange tr = load_ranges(0);
+  if (nq > 0) fetch(tr, 0, A);
+  for (int q = 0; q < nq; q += 2) {
+    // A holds batch q
+    if (q + 1 < nq) {
+      if ((q + 1) % kPerGroup == 0) tr = load_ranges((q + 1) / kPerGroup);
+      fetch(tr, q + 1, B);
+    }
+    add(A);
+    __syncthreads();  // keeps the waves on neighbouring tiles: their reads form one burst
+    if (q + 1 >= nq) break;
+    if (q + 2 < nq) {
+      if ((q + 2) % kPerGroup == 0) tr = load_ranges((q + 2) / kPerGroup);
+      fetch(tr, q + 2, A);
+    }
+    add(B);
+    __syncthreads();
   }
   if (!active) return;
-  const int64_t row0 = (int64_t)rb * kTileRows;
-  int64_t nrows = (int64_t)m - row0;
-  if (nrows > kTileRows) nrows = kTileRows;
+  const int64_t row0 = row_block_start[rb];
+  const int nrows = row_block_start[rb + 1] - (int)row0;  // <= kTileRows
   for (int i = lane; i < nrows; i += kWave) store_axpby(y, row0 + i, alpha, acc[i], beta);
+}
+
+// ---- phase 3 -------------------------------------------------------------------
+// y[row0 + r] += alpha * v for the entries of one chunk of a long tile; rows are
+// pre-combined inside every wave instruction (add_rows), what is left goes to y
+// with global atomics.  Runs after phase 2 has written y = beta*y + alpha*acc.
+template <typename T>
+__global__ __launch_bounds__(kLongThreads) void tiled_long_kernel(
+    const LongChunk* __restrict__ chunks, const unsigned short* __restrict__ t_row,
+    const T* __restrict__ prod, T alpha, T* __restrict__ y) {
+  const LongChunk ch = chunks[blockIdx.x];
+  const int lane = threadIdx.x % kWave;
+  T* yb = y + ch.row0;
+  constexpr int kU = 4;
+  int k0 = ch.begin;
+  for (; k0 + kLongThreads * kU <= ch.end; k0 += kLongThreads * kU) {
+    T v[kU];
+    int r[kU];
+#pragma unroll
+    for (int u = 0; u < kU; ++u) {  // wave w takes 64 * kU consecutive entries: runs of one row stay together
+      const int k = k0 + (threadIdx.x / kWave) * (kWave * kU) + u * kWave + lane;
+      v[u] = alpha * prod[k];
+      r[u] = t_row[k];
+    }
+#pragma unroll
+    for (int u = 0; u < kU; ++u) add_rows<true>(yb, r[u], v[u], true);
+  }
+  for (; k0 < ch.end; k0 += kLongThreads) {  // workgroup-uniform trip count
+    const int k = k0 + threadIdx.x;
+    const bool ok = k < ch.end;
+    const T v = ok ? alpha * prod[k] : T(0);
+    const int r = ok ? (int)t_row[k] : -1 - lane;
+    add_rows<true>(yb, r, v, ok);
+  }
 }
 
 }  // namespace asamd
