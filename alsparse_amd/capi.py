@@ -7,7 +7,7 @@ There is no fallback: if the library has not been built, :func:`load` raises.
 """
 import ctypes
 import os
-from ctypes import POINTER, Structure, byref, c_bool, c_double, c_float, c_int, c_int32, c_size_t, c_void_p
+from ctypes import POINTER, Structure, byref, c_bool, c_double, c_float, c_int, c_int32, c_int64, c_size_t, c_void_p
 
 from .build import LIB_PATH
 
@@ -140,8 +140,14 @@ def _per_type(ctype):
                                       alpha_dcu_matrix_descr_t, _P, _P, _P, _P, _I, PT, _P, _I],
         "alphasparse_dcu_{s}csr2ell": [alphasparse_dcu_handle_t, _I, alpha_dcu_matrix_descr_t, _P, _P, _P,
                                        alpha_dcu_matrix_descr_t, _I, _P, _P],
+        "alphasparse_dcu_{s}_coomv": [alphasparse_dcu_handle_t, c_int, _I, _I, _I, PT, alpha_dcu_matrix_descr_t,
+                                      _P, _P, _P, _P, PT, _P],
+        "alphasparse_dcu_{s}_ellmv": [alphasparse_dcu_handle_t, c_int, _I, _I, PT, alpha_dcu_matrix_descr_t,
+                                      _P, _P, _I, _P, PT, _P],
         # thin kernel ABI
         "asamd_{s}_csrmv": [_P, _P, T, _P, _P, _P, _P, T, _P],
+        "asamd_{s}_ellmv": [_P, _I, _I, T, _P, _P, _I, _I, _P, T, _P],
+        "asamd_{s}_coomv": [_P, _I, _I, c_int64, T, _P, _P, _P, _I, _P, T, _P],
         "asamd_{s}_csrmm": [_P, _I, _I, _I, _I, T, _P, _P, _P, _I, _P, T, _P, POINTER(asamd_dense_strides)],
         "asamd_{s}_csr2ell": [_P, _I, _P, _P, _P, _I, _I, _I, _P, _P],
     }

@@ -1,0 +1,187 @@
+// SpMV for the two formats the CSR converters produce, y = alpha*A*x + beta*y:
+//
+//   ELL (column-major slots, slot s of row r at [s*m + r]): one lane per row,
+//   so the lanes of a wave read consecutive addresses in every slot.  Replaces
+//   src/kernel/dcu/level2/mv/dcu_gemv_x_ell.cpp:10-43 (same traversal; the
+//   slot loop is unrolled so that four independent gathers are in flight, and
+//   the index base of the descriptor is honoured).
+//
+//   COO (entries grouped by row, as csr2coo leaves them): every wave owns one
+//   contiguous run of entries and reduces it 64 at a time with a segmented
+//   scan across its lanes; the last lane of every row segment adds the
+//   segment's sum to y, the open segment at the end of a step is carried into
+//   the next one in registers.  Replaces
+//   src/kernel/dcu/level2/mv/dcu_gemv_x_coo.cpp:10-195, which stages the same
+//   scan through LDS with a barrier per step, writes y without atomics (a row
+//   shared by two waves races there) and finishes with a one-workgroup pass.
+//   Here segment sums reach y through hardware float atomics, so rows split
+//   between waves, and even entries that are not grouped by row at all, are
+//   summed correctly; only the order of the additions to such a shared row is
+//   not fixed.  y is scaled by beta beforehand, as in the reference (:161-169).
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "alsparse_amd_kernels.h"
+#include "device_utils.hpp"
+
+namespace asamd {
+namespace {
+
+constexpr int kEllThreads = 256;
+constexpr int kEllUnroll = 4;
+
+template <typename T>
+__global__ __launch_bounds__(kEllThreads) void ellmv_kernel(int m, int n, T alpha,
+                                                            const T* __restrict__ ell_val,
+                                                            const int* __restrict__ ell_col, int width,
+                                                            int base, const T* __restrict__ x, T beta,
+                                                            T* __restrict__ y) {
+  const int row = blockIdx.x * kEllThreads + threadIdx.x;
+  if (row >= m) return;
+  T sum = T(0);
+  int s = 0;
+  for (; s + kEllUnroll <= width; s += kEllUnroll) {
+    int c[kEllUnroll];
+    T v[kEllUnroll], xv[kEllUnroll];
+#pragma unroll
+    for (int u = 0; u < kEllUnroll; ++u) {
+      const int64_t idx = (int64_t)(s + u) * m + row;
+      c[u] = __builtin_nontemporal_load(&ell_col[idx]) - base;
+      v[u] = __builtin_nontemporal_load(&ell_val[idx]);
+    }
+#pragma unroll
+    for (int u = 0; u < kEllUnroll; ++u) xv[u] = (unsigned)c[u] < (unsigned)n ? x[c[u]] : T(0);
+#pragma unroll
+    for (int u = 0; u < kEllUnroll; ++u)
+      if ((unsigned)c[u] < (unsigned)n) sum = fma_t(v[u], xv[u], sum);
+  }
+  for (; s < width; ++s) {
+    const int64_t idx = (int64_t)s * m + row;
+    const int c = ell_col[idx] - base;
+    if ((unsigned)c < (unsigned)n) sum = fma_t(ell_val[idx], x[c], sum);
+  }
+  store_axpby(y, row, alpha, sum, beta);
+}
+
+// y <- beta * y ahead of an accumulating kernel (beta == 0 stores zeros without reading)
+template <typename T>
+__global__ __launch_bounds__(256) void scale_y_kernel(int m, T beta, T* __restrict__ y) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= m) return;
+  y[i] = beta == T(0) ? T(0) : y[i] * beta;
+}
+
+constexpr int kCooThreads = 256;
+constexpr int kCooSteps = 16;                        // 64-entry steps per wave
+constexpr int kCooPerWave = kWave * kCooSteps;       // entries per wave
+constexpr int kCooPerBlock = kCooPerWave * (kCooThreads / kWave);
+
+template <typename T>
+__global__ __launch_bounds__(kCooThreads) void coomv_kernel(int64_t nnz, int m, int n, T alpha,
+                                                            const T* __restrict__ coo_val,
+                                                            const int* __restrict__ coo_row,
+                                                            const int* __restrict__ coo_col, int base,
+                                                            const T* __restrict__ x, T* __restrict__ y) {
+  const int lane = threadIdx.x % kWave;
+  const int64_t wave = (int64_t)blockIdx.x * (kCooThreads / kWave) + threadIdx.x / kWave;
+  const int64_t begin = wave * kCooPerWave;
+  const int64_t end = begin + kCooPerWave < nnz ? begin + kCooPerWave : nnz;
+  int carry_row = -1;  // open segment handed from one step to the next (same in all lanes)
+  T carry_val = T(0);
+  for (int64_t k0 = begin; k0 < end; k0 += kWave) {
+    const int64_t k = k0 + lane;
+    int r = -1;
+    T v = T(0);
+    if (k < end) {
+      const int rr = __builtin_nontemporal_load(&coo_row[k]) - base;
+      const int c = __builtin_nontemporal_load(&coo_col[k]) - base;
+      if ((unsigned)rr < (unsigned)m && (unsigned)c < (unsigned)n) {
+        r = rr;
+        v = __builtin_nontemporal_load(&coo_val[k]) * x[c];
+      }
+    }
+    if (lane == 0) {
+      if (carry_row == r) v += carry_val;
+      else if (carry_row >= 0) atomicAdd(&y[carry_row], alpha * carry_val);
+    }
+    const int r_prev = __shfl_up(r, 1, kWave);
+    const bool head = lane == 0 || r_prev != r;
+    // inclusive segmented scan: after the step of distance d, v holds the sum of
+    // the lane's segment over the last 2d lanes, f says whether a head lies among them
+    int f = head;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+      const T vd = __shfl_up(v, d, kWave);
+      const int fd = __shfl_up(f, d, kWave);
+      if (lane >= d && !f) {
+        v += vd;
+        f = fd;
+      }
+    }
+    const int head_next = __shfl_down((int)head, 1, kWave);
+    if (lane < kWave - 1 && head_next && r >= 0) atomicAdd(&y[r], alpha * v);
+    carry_row = __shfl(r, kWave - 1, kWave);
+    carry_val = __shfl(v, kWave - 1, kWave);
+  }
+  if (lane == 0 && carry_row >= 0) atomicAdd(&y[carry_row], alpha * carry_val);
+}
+
+template <typename T>
+int ellmv_impl(hipStream_t stream, int32_t m, int32_t n, T alpha, const T* ell_val, const int32_t* ell_col,
+               int32_t width, int32_t base, const T* x, T beta, T* y) {
+  if (m < 0 || n < 0 || width < 0) return (int)hipErrorInvalidValue;
+  if (m == 0) return (int)hipSuccess;
+  const unsigned grid = (unsigned)(((int64_t)m + kEllThreads - 1) / kEllThreads);
+  ellmv_kernel<T><<<grid, kEllThreads, 0, stream>>>(m, n, alpha, ell_val, ell_col, width, base, x, beta, y);
+  return (int)hipGetLastError();
+}
+
+template <typename T>
+int coomv_impl(hipStream_t stream, int32_t m, int32_t n, int64_t nnz, T alpha, const T* coo_val,
+               const int32_t* coo_row, const int32_t* coo_col, int32_t base, const T* x, T beta, T* y) {
+  if (m < 0 || n < 0 || nnz < 0) return (int)hipErrorInvalidValue;
+  if (m == 0) return (int)hipSuccess;
+  if (beta != T(1)) {
+    scale_y_kernel<T><<<(unsigned)(((int64_t)m + 255) / 256), 256, 0, stream>>>(m, beta, y);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return (int)e;
+  }
+  if (nnz == 0) return (int)hipSuccess;
+  const int64_t grid = (nnz + kCooPerBlock - 1) / kCooPerBlock;
+  if (grid > 0x7fffffff) return (int)hipErrorInvalidValue;
+  coomv_kernel<T><<<(unsigned)grid, kCooThreads, 0, stream>>>(nnz, m, n, alpha, coo_val, coo_row, coo_col, base, x,
+                                                              y);
+  return (int)hipGetLastError();
+}
+
+}  // namespace
+}  // namespace asamd
+
+extern "C" {
+
+int asamd_s_ellmv(hipStream_t stream, int32_t m, int32_t n, float alpha, const float* ell_val,
+                  const int32_t* ell_col_ind, int32_t ell_width, int32_t base, const float* x, float beta,
+                  float* y) {
+  return asamd::ellmv_impl<float>(stream, m, n, alpha, ell_val, ell_col_ind, ell_width, base, x, beta, y);
+}
+
+int asamd_d_ellmv(hipStream_t stream, int32_t m, int32_t n, double alpha, const double* ell_val,
+                  const int32_t* ell_col_ind, int32_t ell_width, int32_t base, const double* x, double beta,
+                  double* y) {
+  return asamd::ellmv_impl<double>(stream, m, n, alpha, ell_val, ell_col_ind, ell_width, base, x, beta, y);
+}
+
+int asamd_s_coomv(hipStream_t stream, int32_t m, int32_t n, int64_t nnz, float alpha, const float* coo_val,
+                  const int32_t* coo_row_ind, const int32_t* coo_col_ind, int32_t base, const float* x,
+                  float beta, float* y) {
+  return asamd::coomv_impl<float>(stream, m, n, nnz, alpha, coo_val, coo_row_ind, coo_col_ind, base, x, beta, y);
+}
+
+int asamd_d_coomv(hipStream_t stream, int32_t m, int32_t n, int64_t nnz, double alpha, const double* coo_val,
+                  const int32_t* coo_row_ind, const int32_t* coo_col_ind, int32_t base, const double* x,
+                  double beta, double* y) {
+  return asamd::coomv_impl<double>(stream, m, n, nnz, alpha, coo_val, coo_row_ind, coo_col_ind, base, x, beta,
+                                   y);
+}
+
+}  // extern "C"

@@ -82,22 +82,24 @@ __global__ __launch_bounds__(kSpmmBlock) void spmm_rowmajor_kernel(
     int my_col = 0;
     T my_val = T(0);
     if (j < end) {
-      my_col = col_ind[j] - base;
-      my_val = alpha * val[j];
+      // A and C are touched once: non-temporal, so that they do not push rows of B out of the caches
+      my_col = __builtin_nontemporal_load(col_ind + j) - base;
+      my_val = alpha * __builtin_nontemporal_load(val + j);
     }
     const int cnt = (int)(end - j0 < kWave ? end - j0 : kWave);
     int t = 0;
-    for (; t + 4 <= cnt; t += 4) {
-      Vec<T, V> b[4];
-      T a[4];
+    constexpr int kU = 4;  // B rows in flight per wave (8 and 16 measured no faster)
+    for (; t + kU <= cnt; t += kU) {
+      Vec<T, V> b[kU];
+      T a[kU];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
+      for (int u = 0; u < kU; ++u) {
         const int col = __builtin_amdgcn_readlane(my_col, t + u);
         a[u] = readlane_t(my_val, t + u);
         b[u] = load_vec<T, V>(B + (int64_t)col * ldb + c0, vector_ok, valid);
       }
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
+      for (int u = 0; u < kU; ++u) {
 #pragma unroll
         for (int i = 0; i < V; ++i) acc[i] = fma_t(a[u], b[u].e[i], acc[i]);
       }
@@ -126,7 +128,10 @@ __global__ __launch_bounds__(kSpmmBlock) void spmm_rowmajor_kernel(
   } else {
 #pragma unroll
     for (int i = 0; i < V; ++i) {
-      if (i < valid) crow[i] = beta == T(0) ? acc[i] : crow[i] * beta + acc[i];
+      if (i < valid) {
+        const T res = beta == T(0) ? acc[i] : __builtin_nontemporal_load(crow + i) * beta + acc[i];
+        __builtin_nontemporal_store(res, crow + i);
+      }
     }
   }
 }

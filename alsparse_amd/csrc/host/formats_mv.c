@@ -1,0 +1,22 @@
+/* Device SpMV entry points for COO and ELL operands (raw device arrays). */
+#include "internal.h"
+
+#define ASAMD_T float
+#define ASAMD_S s
+#define ASAMD_KERNEL_COOMV asamd_s_coomv
+#define ASAMD_KERNEL_ELLMV asamd_s_ellmv
+#include "formats_mv.inc"
+#undef ASAMD_T
+#undef ASAMD_S
+#undef ASAMD_KERNEL_COOMV
+#undef ASAMD_KERNEL_ELLMV
+
+#define ASAMD_T double
+#define ASAMD_S d
+#define ASAMD_KERNEL_COOMV asamd_d_coomv
+#define ASAMD_KERNEL_ELLMV asamd_d_ellmv
+#include "formats_mv.inc"
+#undef ASAMD_T
+#undef ASAMD_S
+#undef ASAMD_KERNEL_COOMV
+#undef ASAMD_KERNEL_ELLMV

@@ -172,6 +172,75 @@ def cpu_spmv(a, x, y0, alpha, beta, nbytes):
                       % (a.rows, a.nnz, iters, iters)}
 
 
+def run_format_spmv(cfg, fmt, steps, warmup, check):
+    """SpMV on the ELL or COO form of configuration `cfg`, converted on the GPU
+    (alphasparse_dcu_csr2coo / _csr2ell) and multiplied by alphasparse_dcu_?_coomv / _ellmv."""
+    from ctypes import c_int32
+    from alsparse_amd import capi, hiprt, workloads as wl
+    lib = capi.load()
+    a, x, y0, alpha, beta, _ = wl.config(cfg)
+    T, p, sz = capi.scalar_type(a.dtype), capi.prefix(a.dtype), a.dtype.itemsize
+    h = capi.Handle()
+    descr = capi.make_descr()
+    d_val, d_rp, d_ci = (hiprt.DeviceArray.from_numpy(v) for v in (a.values, a.row_ptr, a.col_ind))
+    d_x, d_y = hiprt.DeviceArray.from_numpy(x), hiprt.DeviceArray.from_numpy(y0)
+    al, be = T(alpha), T(beta)
+    extra = []
+    if fmt == "coo":
+        d_rows = hiprt.DeviceArray((a.nnz,), np.int32)
+        extra.append(d_rows)
+        assert lib.alphasparse_dcu_csr2coo(h.h, d_rp.c_ptr(), a.nnz, a.rows, d_rows.c_ptr(), 0) == 0
+        fn = getattr(lib, "alphasparse_dcu_%s_coomv" % p)
+
+        def step():
+            s = fn(h.h, 0, a.rows, a.cols, a.nnz, byref(al), byref(descr), d_val.c_ptr(), d_rows.c_ptr(), d_ci.c_ptr(),
+                   d_x.c_ptr(), byref(be), d_y.c_ptr())
+            if s != 0:
+                raise RuntimeError("coomv status %d" % s)
+        nbytes = a.nnz * (8 + sz) + a.cols * sz + a.rows * sz * (2 if beta != 0 else 1)
+        kernel = "coo segmented scan"
+    else:
+        w = c_int32(-1)
+        assert lib.alphasparse_dcu_csr2ell_width(h.h, a.rows, byref(descr), d_rp.c_ptr(), byref(descr), byref(w)) == 0
+        ev, ec = hiprt.DeviceArray((w.value * a.rows,), a.dtype), hiprt.DeviceArray((w.value * a.rows,), np.int32)
+        extra += [ev, ec]
+        conv = lib.alphasparse_dcu_scsr2ell if a.dtype == np.float32 else lib.alphasparse_dcu_dcsr2ell
+        assert conv(h.h, a.rows, byref(descr), d_val.c_ptr(), d_rp.c_ptr(), d_ci.c_ptr(), byref(descr), w.value,
+                    ev.c_ptr(), ec.c_ptr()) == 0
+        fn = getattr(lib, "alphasparse_dcu_%s_ellmv" % p)
+
+        def step():
+            s = fn(h.h, 0, a.rows, a.cols, byref(al), byref(descr), ev.c_ptr(), ec.c_ptr(), w.value, d_x.c_ptr(),
+                   byref(be), d_y.c_ptr())
+            if s != 0:
+                raise RuntimeError("ellmv status %d" % s)
+        nbytes = a.rows * w.value * (4 + sz) + a.cols * sz + a.rows * sz * (2 if beta != 0 else 1)
+        kernel = "ell row-per-lane (width %d)" % w.value
+    hiprt.synchronize()
+    parity = None
+    if check:
+        from oracle import oracle as orc
+        step()
+        hiprt.synchronize()
+        y = d_y.to_numpy()
+        err = orc.csrmv_err(a, alpha, x, beta, y0, y, orc.csrmv_plain(a, alpha, x, beta, y0))
+        tol = 1e-4 if a.dtype == np.float32 else 1e-12
+        parity = {"max_row_err": err.strict, "max_row_err_with_beta_y": err.full, "tol": tol,
+                  "zero_den_mismatch": err.zero_den_mismatch,
+                  "ok": bool(err.strict <= tol and err.zero_den_mismatch == 0)}
+        d_y.copy_from(y0)
+    t = time_steps(step, steps, warmup, hiprt)
+    res = {"workload": WORKLOAD_NAMES[cfg].replace("CSR", fmt.upper() + " (from CSR on the GPU)"), "rows": a.rows,
+           "nnz": a.nnz, "algorithmic_bytes": int(nbytes), "flops": 2 * a.nnz, "kernel": kernel, "timing": t,
+           "gbs": nbytes / t["avg_ms"] / 1e6, "gflops": 2 * a.nnz / t["avg_ms"] / 1e6,
+           "dtype": "f32" if a.dtype == np.float32 else "f64", "parity": parity}
+    res["hbm_frac"] = res["gbs"] / HBM_PEAK_GBS
+    for d in [d_val, d_rp, d_ci, d_x, d_y] + extra:
+        d.free()
+    h.close()
+    return res
+
+
 def run_spmm(steps, warmup, check):
     from alsparse_amd import capi, hiprt, workloads as wl
     lib = capi.load()
@@ -221,6 +290,8 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--config", type=int, default=3, choices=[2, 3, 4, 5])
+    ap.add_argument("--format", default="csr", choices=["csr", "ell", "coo"],
+                    help="multiply the ELL / COO form of configuration 2 or 3 (converted on the GPU) instead")
     ap.add_argument("--all", action="store_true", help="also measure the other configurations")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
@@ -249,7 +320,11 @@ def main():
         dst.free()
 
     check = not args.no_check
-    if args.config == 5:
+    if args.format != "csr":
+        if args.config not in (2, 3):
+            sys.exit("bench.py: --format ell|coo is measured on configuration 2 or 3")
+        main_res = run_format_spmv(args.config, args.format, args.steps, args.warmup, check)
+    elif args.config == 5:
         main_res = run_spmm(args.steps, args.warmup, check)
     else:
         main_res = run_spmv(args.config, args.steps, args.warmup, not args.no_cpu_baseline, check)
@@ -260,11 +335,17 @@ def main():
                 continue
             r = run_spmm(args.steps, args.warmup, check) if c == 5 else run_spmv(c, args.steps, args.warmup, False, check)
             others["C%d" % c] = {k: r[k] for k in ("workload", "gbs", "gflops", "hbm_frac", "timing", "parity", "kernel") if k in r}
+        for c, fmt in ((2, "ell"), (2, "coo"), (3, "ell"), (3, "coo")):
+            if args.format == fmt and args.config == c:
+                continue
+            r = run_format_spmv(c, fmt, args.steps, args.warmup, check)
+            others["C%d_%s" % (c, fmt)] = {k: r[k] for k in ("workload", "gbs", "gflops", "hbm_frac", "timing", "parity", "kernel")}
 
     t = main_res["timing"]
     out = {
-        "metric": "CSR SpMV effective GB/s (algorithmic bytes / time), 1 GPU" if args.config != 5
-                  else "CSR SpMM effective GB/s (algorithmic bytes / time), 1 GPU",
+        "metric": ("CSR SpMV effective GB/s (algorithmic bytes / time), 1 GPU" if args.format == "csr"
+                   else "%s SpMV effective GB/s (algorithmic bytes / time), 1 GPU" % args.format.upper())
+                  if args.config != 5 else "CSR SpMM effective GB/s (algorithmic bytes / time), 1 GPU",
         "value": main_res["gbs"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": t["avg_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": main_res["dtype"], "data": "synthetic",

@@ -266,6 +266,37 @@ alphasparse_status_t alphasparse_dcu_dcsr2ell(
     const alpha_dcu_matrix_descr_t ell_descr, ALPHA_INT ell_width, double *ell_val,
     ALPHA_INT *ell_col_ind);
 
+/* ---- SpMV on the converters' output formats ------------------------------------
+ * include/alphasparse/spapi_dcu.h:469-481, :483-495 (coomv) and :858-869, :871-882
+ * (ellmv); validation order of src/core/op_dcu/level2/alphasparse_dcu_x_coomv.cpp:50-95
+ * and alphasparse_dcu_x_ellmv.cpp:48-93: only NON_TRANSPOSE and GENERAL are
+ * supported, as there.  Unlike the reference's kernels, which read indices as
+ * zero-based whatever the descriptor says, descr->base is honoured. */
+alphasparse_status_t alphasparse_dcu_s_coomv(alphasparse_dcu_handle_t handle,
+                                             alphasparse_operation_t trans, ALPHA_INT m, ALPHA_INT n,
+                                             ALPHA_INT nnz, const float *alpha,
+                                             const alpha_dcu_matrix_descr_t descr, const float *coo_val,
+                                             const ALPHA_INT *coo_row_ind, const ALPHA_INT *coo_col_ind,
+                                             const float *x, const float *beta, float *y);
+alphasparse_status_t alphasparse_dcu_d_coomv(alphasparse_dcu_handle_t handle,
+                                             alphasparse_operation_t trans, ALPHA_INT m, ALPHA_INT n,
+                                             ALPHA_INT nnz, const double *alpha,
+                                             const alpha_dcu_matrix_descr_t descr, const double *coo_val,
+                                             const ALPHA_INT *coo_row_ind, const ALPHA_INT *coo_col_ind,
+                                             const double *x, const double *beta, double *y);
+alphasparse_status_t alphasparse_dcu_s_ellmv(alphasparse_dcu_handle_t handle,
+                                             alphasparse_operation_t trans, ALPHA_INT m, ALPHA_INT n,
+                                             const float *alpha, const alpha_dcu_matrix_descr_t descr,
+                                             const float *ell_val, const ALPHA_INT *ell_col_ind,
+                                             ALPHA_INT ell_width, const float *x, const float *beta,
+                                             float *y);
+alphasparse_status_t alphasparse_dcu_d_ellmv(alphasparse_dcu_handle_t handle,
+                                             alphasparse_operation_t trans, ALPHA_INT m, ALPHA_INT n,
+                                             const double *alpha, const alpha_dcu_matrix_descr_t descr,
+                                             const double *ell_val, const ALPHA_INT *ell_col_ind,
+                                             ALPHA_INT ell_width, const double *x, const double *beta,
+                                             double *y);
+
 #ifdef __cplusplus
 }
 #endif

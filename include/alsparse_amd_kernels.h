@@ -131,6 +131,28 @@ int asamd_d_csr2ell(hipStream_t stream, int32_t m, const double *val, const int3
                     const int32_t *col_ind, int32_t csr_base, int32_t ell_base, int32_t width,
                     double *ell_val, int32_t *ell_col);
 
+/* y = alpha*A*x + beta*y, A in column-major ELL (slot s of row r at [s*m + r]);
+ * slots whose index (minus base) is outside [0, n) are skipped.  Stands in for
+ * dcu_gemv_?_ell, src/kernel/dcu/level2/mv/dcu_gemv_x_ell.cpp:10-43, :48-69. */
+int asamd_s_ellmv(hipStream_t stream, int32_t m, int32_t n, float alpha, const float *ell_val,
+                  const int32_t *ell_col_ind, int32_t ell_width, int32_t base, const float *x,
+                  float beta, float *y);
+int asamd_d_ellmv(hipStream_t stream, int32_t m, int32_t n, double alpha, const double *ell_val,
+                  const int32_t *ell_col_ind, int32_t ell_width, int32_t base, const double *x,
+                  double beta, double *y);
+
+/* y = alpha*A*x + beta*y, A in COO.  Fastest when entries are grouped by row
+ * (as asamd_csr2coo leaves them) but correct for any order; entries whose row or
+ * column (minus base) is out of range are skipped.  y must be ordinary device
+ * memory (hardware float atomics).  Stands in for dcu_gemv_?_coo,
+ * src/kernel/dcu/level2/mv/dcu_gemv_x_coo.cpp:10-195. */
+int asamd_s_coomv(hipStream_t stream, int32_t m, int32_t n, int64_t nnz, float alpha,
+                  const float *coo_val, const int32_t *coo_row_ind, const int32_t *coo_col_ind,
+                  int32_t base, const float *x, float beta, float *y);
+int asamd_d_coomv(hipStream_t stream, int32_t m, int32_t n, int64_t nnz, double alpha,
+                  const double *coo_val, const int32_t *coo_row_ind, const int32_t *coo_col_ind,
+                  int32_t base, const double *x, double beta, double *y);
+
 /* Introspection for benchmarks and tests: statistics of the analysis that a
  * multiply would use for `key`, where key is the alphasparse_dcu_mat_info_t of an
  * explicit analysis, or a device csr_row_ptr (library-built mirror or lazily

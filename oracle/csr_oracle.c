@@ -237,6 +237,49 @@ ORACLE_CSR2ELL(oracle_s_csr2ell, float)
 ORACLE_CSR2ELL(oracle_d_csr2ell, double)
 
 /* ------------------------------------------------------------------------- *
+ * COO SpMV: src/plain/kernel/level2/mv/gemv/gemv_x_coo_plain.c:11-24
+ *   y[i] *= beta for all i; then per entry, in storage order,
+ *   v = val*x[col]; y[row] += alpha*v.   Indices zero-based.
+ * ------------------------------------------------------------------------- */
+#define ORACLE_COOMV(NAME, T)                                                                 \
+  void NAME(int32_t m, int32_t nnz, const int32_t *row_indx, const int32_t *col_indx,        \
+            const T *values, T alpha, const T *x, T beta, T *y) {                            \
+    for (int32_t i = 0; i < m; i++) y[i] *= beta;                                             \
+    for (int32_t i = 0; i < nnz; i++) {                                                       \
+      T v = values[i] * x[col_indx[i]];                                                       \
+      y[row_indx[i]] += alpha * v;                                                            \
+    }                                                                                         \
+  }
+ORACLE_COOMV(oracle_s_coomv_plain, float)
+ORACLE_COOMV(oracle_d_coomv_plain, double)
+
+/* ------------------------------------------------------------------------- *
+ * ELL SpMV: src/kernel/dcu/level2/mv/dcu_gemv_x_ell.cpp:22-42 (the reference has
+ * no CPU kernel for this format; this follows its device kernel).  Per row ar:
+ *   sum = 0; for slot i: idx = m*i + ar, col = ell_col[idx]; if (col < n)
+ *   sum = fma(ell_val[idx], x[col], sum)   (device madde is an fma,
+ *   include/alphasparse/real_compute.h:37-39); y[ar] = beta*y[ar] + alpha*sum.
+ * Indices zero-based; a negative index is not guarded in the reference and is
+ * skipped here.
+ * ------------------------------------------------------------------------- */
+#define ORACLE_ELLMV(NAME, T, FMA)                                                            \
+  void NAME(int32_t m, int32_t n, T alpha, const T *ell_val, const int32_t *ell_col,         \
+            int32_t width, const T *x, T beta, T *y) {                                        \
+    for (int32_t ar = 0; ar < m; ar++) {                                                      \
+      T sum = 0;                                                                              \
+      for (int32_t i = 0; i < width; i++) {                                                   \
+        size_t idx = (size_t)m * i + ar;                                                      \
+        int32_t col = ell_col[idx];                                                           \
+        if (col >= 0 && col < n) sum = FMA(ell_val[idx], x[col], sum);                        \
+      }                                                                                       \
+      T left = beta * y[ar], right = alpha * sum;                                             \
+      y[ar] = left + right;                                                                   \
+    }                                                                                         \
+  }
+ORACLE_ELLMV(oracle_s_ellmv, float, fmaf)
+ORACLE_ELLMV(oracle_d_ellmv, double, fma)
+
+/* ------------------------------------------------------------------------- *
  * Parity metric.  For every row i, with all sums accumulated in fp64,
  *     strict_i = |y_test[i] - y_ref[i]| / (|alpha| * sum_j |a_ij * x_j|)
  *     full_i   = |y_test[i] - y_ref[i]| / (|alpha| * sum_j |a_ij * x_j| + |beta * y0[i]|)

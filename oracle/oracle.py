@@ -48,6 +48,10 @@ def lib(fast=False):
                 f.restype, f.argtypes = None, [I, P, P, P, P, T, P, I, I, T, P, I]
             f = getattr(L, "oracle_%s_csr2ell" % s)
             f.restype, f.argtypes = I, [I, P, P, P, I, I, I, P, P]
+            f = getattr(L, "oracle_%s_coomv_plain" % s)
+            f.restype, f.argtypes = None, [I, I, P, P, P, T, P, T, P]
+            f = getattr(L, "oracle_%s_ellmv" % s)
+            f.restype, f.argtypes = None, [I, I, T, P, P, I, P, T, P]
             f = getattr(L, "oracle_%s_csrmv_err" % s)
             f.restype, f.argtypes = c_double, [I, P, P, P, P, c_double, P, c_double, P, P, P, POINTER(c_int64),
                                                POINTER(c_int64), POINTER(c_double), POINTER(c_double)]
@@ -182,6 +186,27 @@ def csr2ell(a, width=None, ell_base=0):
     if rc != 0:
         raise OverflowError("width*m >= 2^31")
     return ev, ec
+
+
+def coomv_plain(a, coo_row, alpha, x, beta, y0):
+    """COO SpMV over the entries of ``a`` with zero-based row indices ``coo_row``."""
+    y = np.array(y0, dtype=a.dtype, copy=True)
+    T = _ct(a.dtype)
+    ci = np.ascontiguousarray(a.col_ind - a.base, dtype=np.int32)
+    rows = np.ascontiguousarray(coo_row, dtype=np.int32)
+    getattr(lib(), "oracle_%s_coomv_plain" % _pre(a.dtype))(
+        a.rows, rows.size, _p(rows), _p(ci), _p(a.values), T(alpha), _p(x), T(beta), _p(y))
+    return y
+
+
+def ellmv(m, n, ell_val, ell_col, width, alpha, x, beta, y0):
+    """ELL SpMV, zero-based column-major ELL arrays."""
+    y = np.array(y0, dtype=ell_val.dtype, copy=True)
+    T = _ct(ell_val.dtype)
+    ec = np.ascontiguousarray(ell_col, dtype=np.int32)
+    getattr(lib(), "oracle_%s_ellmv" % _pre(ell_val.dtype))(
+        m, n, T(alpha), _p(ell_val), _p(ec), width, _p(x), T(beta), _p(y))
+    return y
 
 
 def partition_rows_by_nnz(rows_end, threads):

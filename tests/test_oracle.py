@@ -10,7 +10,7 @@ runs on time-seeded random matrices), so the oracle is pinned by
     (skipped where that library is absent) and with the committed fixtures it produced.
 A dropped term, a wrong sign, a transposed operand or a shifted index fails at least one."""
 import os
-from ctypes import byref, c_double, c_float, c_int32, c_void_p
+from ctypes import Structure, byref, c_bool, c_double, c_float, c_int32, c_void_p
 
 import numpy as np
 import pytest
@@ -206,6 +206,54 @@ def test_csr2coo_and_csr2ell_definitions():
         orc.csr2ell(big, width=256)             # 2^31 entries: the reference aborts here
 
 
+@pytest.mark.parametrize("dtype", DT)
+def test_coomv_and_ellmv_against_brute_force_and_csr(dtype):
+    """COO and ELL products: fp64 brute force straight from the format's arrays (so a
+    row-major / column-major mix-up or a shifted slot fails), any entry order for COO,
+    out-of-range ELL slots skipped, and bit-equality with the CSR oracle on integer data
+    (where every partial sum is exact, so the order and fma contraction cannot matter)."""
+    rng = np.random.default_rng(11)
+    for a in (csr_from_lengths([0, 3, 0, 0, 5, 1, 0, 2, 0, 70], 90, dtype, seed=2), wl.laplace2d(9, 7, dtype),
+              wl.powerlaw_rmat(7, 300, dtype)):
+        x, y0 = wl.uniform(a.cols, dtype, 3), wl.uniform(a.rows, dtype, 4)
+        rows = orc.csr2coo(a)
+        alpha, beta = 2.0, 3.0
+        want = beta * y0.astype(np.float64)
+        for k in range(a.nnz):
+            want[rows[k]] += alpha * float(a.values[k]) * float(x[a.col_ind[k]])
+        bound = gamma_bound(a, alpha, x, beta, y0)
+        assert np.all(np.abs(orc.coomv_plain(a, rows, alpha, x, beta, y0) - want) <= bound)
+        # any storage order gives the same product
+        perm = rng.permutation(a.nnz)
+        shuffled = wl.Csr(a.rows, a.cols, a.row_ptr, a.col_ind[perm], a.values[perm], 0)
+        assert np.all(np.abs(orc.coomv_plain(shuffled, rows[perm], alpha, x, beta, y0) - want) <= bound)
+        # ELL: brute force from the column-major arrays themselves
+        w = orc.csr2ell_width(a)
+        ev, ec = orc.csr2ell(a)
+        ec = ec.copy()
+        want = beta * y0.astype(np.float64)
+        for r in range(a.rows):
+            for s_ in range(w):
+                want[r] += alpha * float(ev[s_ * a.rows + r]) * float(x[ec[s_ * a.rows + r]])
+        assert np.all(np.abs(orc.ellmv(a.rows, a.cols, ev, ec, w, alpha, x, beta, y0) - want) <= bound)
+        # a slot whose index is >= n is skipped (dcu_gemv_x_ell.cpp:33), whatever its value
+        pad = np.flatnonzero(ev == 0)
+        if pad.size:
+            ev2, ec2 = ev.copy(), ec.copy()
+            ev2[pad[0]], ec2[pad[0]] = 1e6, a.cols
+            assert np.array_equal(orc.ellmv(a.rows, a.cols, ev2, ec2, w, alpha, x, beta, y0),
+                                  orc.ellmv(a.rows, a.cols, ev, ec, w, alpha, x, beta, y0))
+        # integer data: exact in every order
+        ai = wl.Csr(a.rows, a.cols, a.row_ptr, a.col_ind, rng.integers(-4, 5, a.nnz).astype(dtype), 0)
+        xi, yi = rng.integers(-4, 5, a.cols).astype(dtype), rng.integers(-4, 5, a.rows).astype(dtype)
+        ref = orc.csrmv_plain(ai, 2.0, xi, 3.0, yi)
+        assert np.array_equal(orc.coomv_plain(ai, rows, 2.0, xi, 3.0, yi), ref)
+        evi, eci = orc.csr2ell(ai)
+        assert np.array_equal(orc.ellmv(a.rows, a.cols, evi, eci, w, 2.0, xi, 3.0, yi), ref)
+        # beta = 0 still multiplies: y0 = 0 stays 0 on empty rows
+        assert orc.coomv_plain(a, rows, 1.0, x, 0.0, y0)[0] == 0 or np.diff(a.row_ptr)[0] > 0
+
+
 def test_error_metric_detects_planted_errors():
     a = wl.uniform_rows(400, 300, 16, np.float32)
     x, y0 = wl.uniform(a.cols, np.float32, 3), wl.uniform(a.rows, np.float32, 4)
@@ -246,6 +294,35 @@ def _ref_mm(name, a, alpha, B, ldb, beta, C0, ldc, n):
     C = C0.copy(order="K")
     assert fn(T(alpha), byref(mat.s), B.ctypes.data_as(c_void_p), n, ldb, T(beta), C.ctypes.data_as(c_void_p), ldc) == 0
     return C
+
+
+class _RefCoo(Structure):  # spmat_coo_?_t, include/alphasparse/spmat.h:73-86 of the reference
+    _fields_ = [("values", c_void_p), ("row_indx", c_void_p), ("col_indx", c_void_p), ("rows", c_int32),
+                ("cols", c_int32), ("nnz", c_int32), ("ordered", c_bool), ("d_rows_indx", c_void_p),
+                ("d_cols_indx", c_void_p), ("d_values", c_void_p)]
+
+
+@needs_ref
+@pytest.mark.parametrize("dtype", DT)
+def test_coomv_oracle_is_bit_identical_to_reference_kernel(dtype):
+    T = c_float if dtype == np.float32 else c_double
+    fn = getattr(orc.ref_lib(), "gemv_%s_coo_plain" % ("s" if dtype == np.float32 else "d"))
+    fn.argtypes, fn.restype = [T, c_void_p, c_void_p, T, c_void_p], c_int32
+    rng = np.random.default_rng(5)
+    for a in (wl.random_points(1000, 1000, 5000, dtype), wl.powerlaw_rmat(12, 3000, dtype),
+              csr_from_lengths([0, 1, 0, 70, 3, 0], 100, dtype)):
+        x, y0 = wl.uniform(a.cols, dtype, 3), wl.uniform(a.rows, dtype, 4)
+        rows, cols, vals = orc.csr2coo(a), a.col_ind.copy(), a.values.copy()
+        for shuffle in (False, True):
+            if shuffle:
+                perm = rng.permutation(a.nnz)
+                rows, cols, vals = rows[perm].copy(), cols[perm].copy(), vals[perm].copy()
+            coo = _RefCoo(vals.ctypes.data, rows.ctypes.data, cols.ctypes.data, a.rows, a.cols, a.nnz, False, None, None, None)
+            for alpha, beta in ((1.0, 0.0), (2.0, 3.0)):
+                y = y0.copy()
+                assert fn(T(alpha), byref(coo), x.ctypes.data_as(c_void_p), T(beta), y.ctypes.data_as(c_void_p)) == 0
+                mine = orc.coomv_plain(wl.Csr(a.rows, a.cols, a.row_ptr, cols, vals, 0), rows, alpha, x, beta, y0)
+                assert np.array_equal(mine, y), (a.name, shuffle, alpha, beta)
 
 
 @needs_ref

@@ -112,6 +112,38 @@ def test_csrmm_status_precedence(lib, p, T):
     assert call(layout=0, tb=1) == S.ALPHA_SPARSE_STATUS_NOT_SUPPORTED   # row-major with op(B) = B^T
 
 
+@pytest.mark.parametrize("p,T", [("s", c_float), ("d", c_double)])
+def test_coomv_and_ellmv_status_precedence(lib, p, T):
+    """alphasparse_dcu_x_coomv.cpp:50-95 and alphasparse_dcu_x_ellmv.cpp:48-93."""
+    a, b, d = T(1), T(0), descr()
+    coomv, ellmv = getattr(lib, "alphasparse_dcu_%s_coomv" % p), getattr(lib, "alphasparse_dcu_%s_ellmv" % p)
+
+    def coo(h=H, trans=0, m=4, n=4, nnz=8, alpha=byref(a), de=byref(d), val=P, ri=P, ci=P, x=P, beta=byref(b), y=P):
+        return coomv(h, trans, m, n, nnz, alpha, de, val, ri, ci, x, beta, y)
+
+    def ell(h=H, trans=0, m=4, n=4, alpha=byref(a), de=byref(d), val=P, ci=P, width=2, x=P, beta=byref(b), y=P):
+        return ellmv(h, trans, m, n, alpha, de, val, ci, width, x, beta, y)
+
+    bad, sym = descr(base=7), descr(mtype=S.ALPHA_SPARSE_MATRIX_TYPE_SYMMETRIC)
+    for call, sizes, zero, ptrs in ((coo, ("m", "n", "nnz"), ("m", "n", "nnz"), ("val", "ri", "ci", "x", "y")),
+                                    (ell, ("m", "n"), ("m", "n", "width"), ("val", "ci", "x", "y"))):
+        assert call(h=NULL, de=None) == S.ALPHA_SPARSE_STATUS_INVALID_HANDLE
+        assert call(de=None) == S.ALPHA_SPARSE_STATUS_INVALID_POINTER
+        assert call(de=byref(bad), m=-1) == S.ALPHA_SPARSE_STATUS_INVALID_VALUE
+        for k in sizes:
+            assert call(**{k: -1}) == S.ALPHA_SPARSE_STATUS_INVALID_VALUE
+        for k in zero:  # quick return beats the pointer checks
+            assert call(alpha=None, val=NULL, y=NULL, **{k: 0}) == S.ALPHA_SPARSE_STATUS_SUCCESS
+        assert call(alpha=None) == S.ALPHA_SPARSE_STATUS_INVALID_POINTER
+        assert call(beta=None) == S.ALPHA_SPARSE_STATUS_INVALID_POINTER
+        for k in ptrs:
+            assert call(**{k: NULL}) == S.ALPHA_SPARSE_STATUS_INVALID_POINTER
+        assert call(de=byref(sym)) == S.ALPHA_SPARSE_STATUS_NOT_SUPPORTED
+        assert call(de=byref(sym), val=NULL) == S.ALPHA_SPARSE_STATUS_INVALID_POINTER
+        assert call(trans=S.ALPHA_SPARSE_OPERATION_TRANSPOSE) == S.ALPHA_SPARSE_STATUS_NOT_SUPPORTED
+    assert ell(width=-3) == S.ALPHA_SPARSE_STATUS_INVALID_VALUE
+
+
 def test_conversion_status_codes(lib):
     d = descr()
     w = c_int32(-5)
