@@ -41,7 +41,7 @@ ALPHA_SPARSE_DATATYPE_DOUBLE = 1
 
 # kernel families of the thin kernel ABI (include/alsparse_amd_kernels.h)
 (ASAMD_SPMV_AUTO, ASAMD_SPMV_VECTOR, ASAMD_SPMV_ROWCONST, ASAMD_SPMV_MERGE, ASAMD_SPMV_SCALAR, ASAMD_SPMV_TILED,
- ASAMD_SPMV_STREAM) = range(7)
+ ASAMD_SPMV_STREAM, ASAMD_SPMV_ELL) = range(8)
 ASAMD_HIST_BINS = 33
 
 
@@ -108,7 +108,8 @@ class asamd_csr_stats(Structure):
                 ("first_offset", c_int32), ("algo", c_int32), ("vector_width", c_int32),
                 ("merge_blocks", c_int32), ("trusted", c_int32), ("tiled_built", c_int32),
                 ("tile_col_blocks", c_int32), ("tile_row_blocks", c_int32),
-                ("tune_ms_base", c_float), ("tune_ms_tiled", c_float),
+                ("tune_ms_base", c_float), ("tune_ms_tiled", c_float), ("tune_ms_ell", c_float),
+                ("ell_built", c_int32), ("ell_width", c_int32),
                 ("hist", ctypes.c_int64 * ASAMD_HIST_BINS)]
 
 
@@ -197,7 +198,7 @@ _RESTYPE = {"asamd_csr_plan_destroy": None, "asamd_csr_plan_stats": POINTER(asam
 
 ALGO_NAMES = {ASAMD_SPMV_AUTO: "auto", ASAMD_SPMV_VECTOR: "vector", ASAMD_SPMV_ROWCONST: "rowconst",
               ASAMD_SPMV_MERGE: "merge-path", ASAMD_SPMV_SCALAR: "scalar", ASAMD_SPMV_TILED: "tiled two-phase",
-              ASAMD_SPMV_STREAM: "row-block stream"}
+              ASAMD_SPMV_STREAM: "row-block stream", ASAMD_SPMV_ELL: "ell copy"}
 
 _lib = None
 

@@ -16,6 +16,7 @@
 #include <vector>
 
 #include "alsparse_amd_kernels.h"
+#include "spmv_ell.hpp"
 #include "spmv_merge.hpp"
 #include "spmv_rows.hpp"
 #include "spmv_tiled.hpp"
@@ -99,6 +100,9 @@ struct asamd_csr_plan {
   unsigned short* d_trow;     // nnz local rows
   void* d_tprod;              // nnz products (phase 1 -> phase 2)
   TiledChunk* d_chunks;       // phase-1 work list
+  // ELL copy (trusted plans of short, nearly equal rows)
+  void* d_eval;               // ell_width * m values, column-major
+  int* d_ecol;                // ... and zero-based columns
 };
 
 static int width_for_mean(double mean) {
@@ -165,6 +169,49 @@ static void free_tiled(asamd_csr_plan* p) {
   p->d_tcol = p->d_trow = nullptr;
   p->d_chunks = nullptr;
   p->st.tiled_built = 0;
+}
+
+static void free_ell(asamd_csr_plan* p) {
+  if (p->d_eval) (void)hipFree(p->d_eval);
+  if (p->d_ecol) (void)hipFree(p->d_ecol);
+  p->d_eval = nullptr;
+  p->d_ecol = nullptr;
+  p->st.ell_built = 0;
+}
+
+// An ELL copy pays when rows are short and padding them to the longest costs
+// little: the kernel then streams 4 + sizeof(T) bytes per entry at full width
+// with neither row_ptr nor LDS staging.
+static bool ell_eligible(const asamd_csr_stats& st, bool force) {
+  if (!st.trusted || st.max_len < 1 || st.max_len > 32) return false;
+  const int64_t slots = (int64_t)st.m * st.max_len;
+  if (slots >= ((int64_t)1 << 31) || slots > (int64_t)st.nnz + st.nnz / 8) return false;
+  return force || st.nnz >= (1 << 18);
+}
+
+template <typename T>
+static hipError_t build_ell(hipStream_t stream, asamd_csr_plan* p, const int* row_ptr, const int* col_ind,
+                            const T* val) {
+  asamd_csr_stats& st = p->st;
+  const size_t slots = (size_t)st.m * (size_t)st.max_len;
+  hipError_t e = hipMalloc(&p->d_eval, slots * sizeof(T));
+  if (e == hipSuccess) e = hipMalloc(&p->d_ecol, slots * sizeof(int));
+  if (e == hipSuccess) {
+    if constexpr (sizeof(T) == 4)
+      e = (hipError_t)asamd_s_csr2ell(stream, st.m, val, row_ptr, col_ind, st.base, 0, st.max_len, (float*)p->d_eval,
+                                      p->d_ecol);
+    else
+      e = (hipError_t)asamd_d_csr2ell(stream, st.m, val, row_ptr, col_ind, st.base, 0, st.max_len, (double*)p->d_eval,
+                                      p->d_ecol);
+  }
+  if (e == hipSuccess) e = hipStreamSynchronize(stream);
+  if (e != hipSuccess) {
+    free_ell(p);
+    return e;
+  }
+  st.ell_built = 1;
+  st.ell_width = st.max_len;
+  return hipSuccess;
 }
 
 template <typename T>
@@ -371,11 +418,12 @@ static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* 
   return hipSuccess;
 }
 
-// Time the current choice against the tiled kernel pair on scratch vectors and
-// keep the faster one.
+// Time the structural choice against the copies that were built (tiled, ELL) on
+// scratch vectors, keep the fastest and free the copies that lost.  A copy has
+// to win by a margin to be worth its memory.
 template <typename T>
-static hipError_t tune_tiled(hipStream_t stream, asamd_csr_plan* p, const int* row_ptr,
-                             const int* col_ind, const T* val) {
+static hipError_t tune_copies(hipStream_t stream, asamd_csr_plan* p, const int* row_ptr,
+                              const int* col_ind, const T* val) {
   asamd_csr_stats& st = p->st;
   T *x = nullptr, *y = nullptr;
   hipEvent_t e0 = nullptr, e1 = nullptr;
@@ -384,9 +432,11 @@ static hipError_t tune_tiled(hipStream_t stream, asamd_csr_plan* p, const int* r
   if (e == hipSuccess) e = hipMemsetAsync(x, 0, (size_t)st.n * sizeof(T), stream);
   if (e == hipSuccess) e = hipEventCreate(&e0);
   if (e == hipSuccess) e = hipEventCreate(&e1);
-  float best[2] = {0.f, 0.f};
-  const int algos[2] = {p->auto_algo, ASAMD_SPMV_TILED};
-  for (int a = 0; a < 2 && e == hipSuccess; ++a) {
+  float best[3] = {0.f, 0.f, 0.f};
+  const int algos[3] = {p->auto_algo, ASAMD_SPMV_TILED, ASAMD_SPMV_ELL};
+  const bool have[3] = {true, st.tiled_built != 0, st.ell_built != 0};
+  for (int a = 0; a < 3 && e == hipSuccess; ++a) {
+    if (!have[a]) continue;
     st.algo = algos[a];
     for (int rep = 0; rep < 3 && e == hipSuccess; ++rep) {
       e = hipEventRecord(e0, stream);
@@ -407,11 +457,18 @@ static hipError_t tune_tiled(hipStream_t stream, asamd_csr_plan* p, const int* r
   if (e != hipSuccess) return e;
   st.tune_ms_base = best[0];
   st.tune_ms_tiled = best[1];
-  if (best[1] > 0.f && best[1] < 0.9f * best[0]) {
-    p->auto_algo = ASAMD_SPMV_TILED;
-    st.algo = ASAMD_SPMV_TILED;
-  } else {
-    free_tiled(p);  // not worth its memory
+  st.tune_ms_ell = best[2];
+  const bool tiled_wins = best[1] > 0.f && best[1] < 0.9f * best[0];
+  const bool ell_wins = best[2] > 0.f && best[2] < 0.95f * best[0];
+  int pick = 0;
+  if (tiled_wins && ell_wins) pick = best[1] < best[2] ? 1 : 2;
+  else if (tiled_wins) pick = 1;
+  else if (ell_wins) pick = 2;
+  if (pick != 1) free_tiled(p);
+  if (pick != 2) free_ell(p);
+  if (pick != 0) {
+    p->auto_algo = algos[pick];
+    st.algo = algos[pick];
   }
   return hipSuccess;
 }
@@ -491,22 +548,27 @@ extern "C" int asamd_csr_plan_create(hipStream_t stream, int32_t m, int32_t n, i
     // trusted == 2: build the tiled copy whatever the size and skip the timing
     // (lets small matrices exercise the tiled kernels)
     const bool force = trusted == 2;
-    const bool ok = val_size == 4 ? tiled_eligible<float>(p->st, force) : tiled_eligible<double>(p->st, force);
-    if (ok) {
+    const bool tiled_ok = val_size == 4 ? tiled_eligible<float>(p->st, force) : tiled_eligible<double>(p->st, force);
+    const bool ell_ok = ell_eligible(p->st, force);
+    if (tiled_ok)
       e = val_size == 4 ? build_tiled<float>(stream, p, row_ptr, col_ind, (const float*)val)
                         : build_tiled<double>(stream, p, row_ptr, col_ind, (const double*)val);
-      if (e == hipSuccess && !force)
-        e = val_size == 4 ? tune_tiled<float>(stream, p, row_ptr, col_ind, (const float*)val)
-                          : tune_tiled<double>(stream, p, row_ptr, col_ind, (const double*)val);
-      if (e == hipErrorOutOfMemory) {
-        (void)hipGetLastError();  // the tiled copy is optional: carry on without it
-        free_tiled(p);
-        e = hipSuccess;
-      }
-      if (e != hipSuccess) {
-        asamd_csr_plan_destroy(p);
-        return e;
-      }
+    if (e == hipSuccess && ell_ok)
+      e = val_size == 4 ? build_ell<float>(stream, p, row_ptr, col_ind, (const float*)val)
+                        : build_ell<double>(stream, p, row_ptr, col_ind, (const double*)val);
+    if (e == hipSuccess && !force && (p->st.tiled_built || p->st.ell_built))
+      e = val_size == 4 ? tune_copies<float>(stream, p, row_ptr, col_ind, (const float*)val)
+                        : tune_copies<double>(stream, p, row_ptr, col_ind, (const double*)val);
+    if (e == hipErrorOutOfMemory) {
+      (void)hipGetLastError();  // the copies are optional: carry on without them
+      free_tiled(p);
+      free_ell(p);
+      p->st.algo = p->auto_algo;
+      e = hipSuccess;
+    }
+    if (e != hipSuccess) {
+      asamd_csr_plan_destroy(p);
+      return e;
     }
   }
   *out = p;
@@ -520,6 +582,7 @@ extern "C" void asamd_csr_plan_destroy(asamd_csr_plan* p) {
   if (p->d_carry_val) (void)hipFree(p->d_carry_val);
   if (p->d_head_val) (void)hipFree(p->d_head_val);
   free_tiled(p);
+  free_ell(p);
   delete p;
 }
 
@@ -543,6 +606,10 @@ extern "C" int asamd_csr_plan_set_algo(asamd_csr_plan* p, int32_t algo) {
       return hipSuccess;
     case ASAMD_SPMV_STREAM:
       if (!stream_ok(p->st)) return hipErrorInvalidValue;
+      p->st.algo = algo;
+      return hipSuccess;
+    case ASAMD_SPMV_ELL:
+      if (!p->st.ell_built) return hipErrorInvalidValue;
       p->st.algo = algo;
       return hipSuccess;
     case ASAMD_SPMV_VECTOR:
@@ -587,7 +654,15 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
   }
   if (algo == ASAMD_SPMV_STREAM && !stream_ok(st)) algo = ASAMD_SPMV_MERGE;
   if (algo == ASAMD_SPMV_TILED && !st.tiled_built) algo = p->auto_algo == ASAMD_SPMV_TILED ? ASAMD_SPMV_MERGE : p->auto_algo;
+  if (algo == ASAMD_SPMV_ELL && !st.ell_built) algo = p->auto_algo == ASAMD_SPMV_ELL ? ASAMD_SPMV_MERGE : p->auto_algo;
   switch (algo) {
+    case ASAMD_SPMV_ELL: {
+      // the ELL copy holds zero-based columns and its own values
+      const unsigned grid = (unsigned)(((int64_t)st.m + kEllThreads - 1) / kEllThreads);
+      ellmv_kernel<T><<<grid, kEllThreads, 0, s>>>(st.m, st.n, alpha, (const T*)p->d_eval, p->d_ecol, st.ell_width, 0,
+                                                   x, beta, y);
+      break;
+    }
     case ASAMD_SPMV_TILED: {
       // the tiled copy holds zero-based local indices and its own values
       if (p->n_chunks > 0)

@@ -163,5 +163,6 @@ int asamd_env_algo(void) {
   if (!strcmp(e, "scalar")) return ASAMD_SPMV_SCALAR;
   if (!strcmp(e, "tiled")) return ASAMD_SPMV_TILED;
   if (!strcmp(e, "stream")) return ASAMD_SPMV_STREAM;
+  if (!strcmp(e, "ell")) return ASAMD_SPMV_ELL;
   return ASAMD_SPMV_AUTO;
 }

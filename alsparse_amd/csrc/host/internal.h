@@ -49,7 +49,7 @@ alphasparse_status_t asamd_plan_for_call(alphasparse_dcu_handle_t handle, const 
 /* Process-wide handle for alphasparse_?_mv / _mm (host pointers). */
 alphasparse_status_t asamd_default_handle(alphasparse_dcu_handle_t *handle);
 
-/* ALSPARSE_AMD_SPMV_ALGO = auto | vector | rowconst | merge | scalar | tiled | stream */
+/* ALSPARSE_AMD_SPMV_ALGO = auto | vector | rowconst | merge | scalar | tiled | stream | ell */
 int asamd_env_algo(void);
 
 #define ASAMD_HIP_STATUS(expr)                                           \

@@ -35,7 +35,9 @@ enum asamd_spmv_algo {
   ASAMD_SPMV_SCALAR = 4,   /* one lane per row; diagnostic baseline                  */
   ASAMD_SPMV_TILED = 5,    /* two-phase, (column block x row block) tiles: every x
                               gather and y update in LDS, HBM sees only streams     */
-  ASAMD_SPMV_STREAM = 6    /* rows of <= 16 entries: 256 rows' products staged in LDS */
+  ASAMD_SPMV_STREAM = 6,   /* rows of <= 16 entries: 256 rows' products staged in LDS */
+  ASAMD_SPMV_ELL = 7       /* short, nearly equal rows: a column-major ELL copy, one
+                              lane per row                                          */
 };
 
 #define ASAMD_HIST_BINS 33
@@ -55,6 +57,9 @@ typedef struct {
   int32_t tile_col_blocks, tile_row_blocks;
   float tune_ms_base;   /* analysis-time timing of the non-tiled choice, or 0 */
   float tune_ms_tiled;  /* ... and of the tiled kernel pair, or 0             */
+  float tune_ms_ell;    /* ... and of the ELL copy's kernel, or 0             */
+  int32_t ell_built;    /* 1: an ELL copy exists (ELL can be selected)        */
+  int32_t ell_width;    /* its slots per row                                  */
   int64_t hist[ASAMD_HIST_BINS];
 } asamd_csr_stats;
 
@@ -71,8 +76,11 @@ typedef struct asamd_csr_plan asamd_csr_plan;
  * a tiled copy of the matrix is built and the tiled two-phase kernel is timed
  * against the row / merge-path choice on scratch vectors; the faster one wins
  * (the reference's analysis record carries an `algo_tuning` flag for exactly
- * this, include/alphasparse/handle.h:120-123).  trusted == 2 builds the tiled
- * copy whatever the size and skips the timing (for tests of the tiled kernels). */
+ * this, include/alphasparse/handle.h:120-123).  Likewise, when rows are short
+ * (<= 32) and padding them to the longest adds at most 1/8 to the entry count,
+ * a column-major ELL copy is built and timed.  Copies that lose are freed.
+ * trusted == 2 builds both copies whatever the size and skips the timing (for
+ * tests of those kernels); the kernel choice then stays the structural one. */
 int asamd_csr_plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t nnz,
                           const int32_t *row_ptr, const int32_t *col_ind, const void *val,
                           int32_t base, int32_t val_size, int32_t trusted, asamd_csr_plan **plan);

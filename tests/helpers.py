@@ -13,7 +13,7 @@ TOL = {np.dtype(np.float32): 1e-4, np.dtype(np.float64): 1e-12}
 
 ALGOS = {"auto": capi.ASAMD_SPMV_AUTO, "vector": capi.ASAMD_SPMV_VECTOR, "rowconst": capi.ASAMD_SPMV_ROWCONST,
          "merge": capi.ASAMD_SPMV_MERGE, "scalar": capi.ASAMD_SPMV_SCALAR, "tiled": capi.ASAMD_SPMV_TILED,
-         "stream": capi.ASAMD_SPMV_STREAM}
+         "stream": capi.ASAMD_SPMV_STREAM, "ell": capi.ASAMD_SPMV_ELL}
 
 
 def announce(*what):
@@ -59,15 +59,15 @@ def run_plan_csrmv(da, algo, alpha, x, beta, y0, trusted=1):
     lib = capi.load()
     from ctypes import c_void_p
     plan = c_void_p()
-    if algo == "tiled":
-        trusted = 2  # build the tiled copy whatever the size
+    if algo in ("tiled", "ell"):
+        trusted = 2  # build the copies whatever the size
     e = lib.asamd_csr_plan_create(None, a.rows, a.cols, a.nnz, da.row_ptr.c_ptr(), da.col.c_ptr(), da.val.c_ptr(),
                                   a.base, a.dtype.itemsize, trusted, byref(plan))
     assert e == 0, "plan_create hip error %d" % e
     try:
         e = lib.asamd_csr_plan_set_algo(plan, ALGOS[algo])
         if e != 0:
-            assert algo in ("rowconst", "stream"), algo
+            assert algo in ("rowconst", "stream", "ell"), algo
             return None  # this structure cannot run that family
         T = capi.scalar_type(a.dtype)
         dx = hiprt.DeviceArray.from_numpy(np.ascontiguousarray(x, dtype=a.dtype))

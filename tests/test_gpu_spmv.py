@@ -45,7 +45,7 @@ def test_every_kernel_family_matches_oracle(gpu, shape, dtype):
     x, y0 = _vectors(a)
     da = DeviceCsr(a)
     try:
-        for algo in ("vector", "merge", "scalar", "rowconst", "stream", "tiled", "auto"):
+        for algo in ("vector", "merge", "scalar", "rowconst", "stream", "tiled", "ell", "auto"):
             for alpha, beta in ((1.0, 0.0), (2.0, 3.0), (-0.75, 1.0)):
                 announce("spmv", shape, np.dtype(dtype).name, algo, alpha, beta)
                 y = run_plan_csrmv(da, algo, alpha, x, beta, y0)
@@ -65,7 +65,7 @@ def test_index_base_one(gpu, dtype):
         x, y0 = _vectors(a)
         da = DeviceCsr(a)
         try:
-            for algo in ("vector", "merge", "scalar", "stream", "tiled", "auto"):
+            for algo in ("vector", "merge", "scalar", "stream", "tiled", "ell", "auto"):
                 announce("spmv base1", a.name, algo)
                 y = run_plan_csrmv(da, algo, 1.5, x, 0.25, y0)
                 if y is None:
@@ -92,6 +92,27 @@ def test_beta_zero_ignores_nan_in_y(gpu):
             check_spmv(a, 1.0, x, 0.0, np.zeros_like(y0), y, algo)
     finally:
         da.free()
+
+
+def test_ell_copy_is_built_only_for_short_even_rows(gpu):
+    lib = capi.load()
+    from ctypes import byref, c_void_p
+    for a, want in ((wl.laplace2d(64, 48, np.float64), 1), (wl.uniform_rows(3000, 3000, 32, np.float32), 1),
+                    (wl.powerlaw_rmat(13, 3000, np.float32), 0), (csr_from_lengths([1] * 900 + [30] * 100, 500, np.float32), 0)):
+        da = DeviceCsr(a)
+        plan = c_void_p()
+        try:
+            announce("ell eligibility", a.name)
+            assert lib.asamd_csr_plan_create(None, a.rows, a.cols, a.nnz, da.row_ptr.c_ptr(), da.col.c_ptr(), da.val.c_ptr(),
+                                             a.base, a.dtype.itemsize, 2, byref(plan)) == 0
+            st = lib.asamd_csr_plan_stats(plan).contents
+            assert st.ell_built == want, a.name
+            if want:
+                assert st.ell_width == int(np.diff(a.row_ptr).max())
+            assert (lib.asamd_csr_plan_set_algo(plan, capi.ASAMD_SPMV_ELL) == 0) == bool(want)
+        finally:
+            lib.asamd_csr_plan_destroy(plan)
+            da.free()
 
 
 def test_deterministic_across_runs(gpu):
