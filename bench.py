@@ -28,12 +28,14 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per multiply measured with rocprofv3 (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from a
-# 1 GiB copy kernel); the summaries these come from are profiles/spmv_tiled_C3.txt, spmv_merge_C4.txt and
-# spmv_stream_C2.txt.  Keyed by (configuration, kernel family); anything else reports null.
+# 1 GiB copy kernel); the summaries these come from are profiles/spmv_tiled_C3.txt, spmv_merge_C4.txt,
+# spmv_ell_copy_C2.txt and spmm_rowmajor_C5.txt.  Keyed by (configuration, kernel family); anything else reports null.
 MEASURED_TRAFFIC_BYTES = {
     (3, "tiled two-phase"): 5.00e9,
     (3, "rowconst"): 34.6e9,
     (4, "merge-path"): 3.43e9,
+    (2, "ell copy"): 322.5e6,
+    (5, "spmm row-major"): 9.27e9,
 }
 
 WORKLOAD_NAMES = {
@@ -278,6 +280,7 @@ def run_spmm(steps, warmup, check):
            "gbs": nbytes / t["avg_ms"] / 1e6, "gflops": 2 * a.nnz * n / t["avg_ms"] / 1e6, "dtype": "f32",
            "parity": parity}
     res["hbm_frac"] = res["gbs"] / HBM_PEAK_GBS
+    res["traffic"] = MEASURED_TRAFFIC_BYTES.get((5, "spmm row-major"))
     for d in (d_val, d_rp, d_ci, d_B, d_C):
         d.free()
     h.close()
