@@ -109,7 +109,7 @@ class asamd_csr_stats(Structure):
                 ("merge_blocks", c_int32), ("trusted", c_int32), ("tiled_built", c_int32),
                 ("tile_col_blocks", c_int32), ("tile_row_blocks", c_int32),
                 ("tune_ms_base", c_float), ("tune_ms_tiled", c_float), ("tune_ms_ell", c_float),
-                ("ell_built", c_int32), ("ell_width", c_int32),
+                ("ell_built", c_int32), ("ell_width", c_int32), ("transpose_built", c_int32),
                 ("hist", ctypes.c_int64 * ASAMD_HIST_BINS)]
 
 
@@ -147,6 +147,7 @@ def _per_type(ctype):
                                       _P, _P, _I, _P, PT, _P],
         # thin kernel ABI
         "asamd_{s}_csrmv": [_P, _P, T, _P, _P, _P, _P, T, _P],
+        "asamd_{s}_csrmv_trans": [_P, _P, T, _P, _P, _P, _P, T, _P],
         "asamd_{s}_ellmv": [_P, _I, _I, T, _P, _P, _I, _I, _P, T, _P],
         "asamd_{s}_coomv": [_P, _I, _I, c_int64, T, _P, _P, _P, _I, _P, T, _P],
         "asamd_{s}_csrmm": [_P, _I, _I, _I, _I, T, _P, _P, _P, _I, _P, T, _P, POINTER(asamd_dense_strides)],
@@ -175,11 +176,15 @@ _COMMON = {
     "asamd_csr_plan_destroy": [_P],
     "asamd_csr_plan_stats": [_P],
     "asamd_csr_plan_set_algo": [_P, _I],
+    "asamd_csr_plan_build_transpose": [_P, _P, _P, _P, _P],
+    "asamd_csr_plan_set_lazy_transpose": [_P, _I],
+    "asamd_csr_plan_transpose_stats": [_P],
     "asamd_csr2coo": [_P, _P, _I, _I, _P, _I],
     "asamd_csr2ell_width": [_P, _I, _P, POINTER(_I)],
     "asamd_warmup": [_P],
     "asamd_copy_bytes": [_P, _P, _P, c_size_t],
     "asamd_analysis_stats": [_P],
+    "asamd_analysis_transpose_stats": [_P],
     "asamd_analysis_set_algo": [_P, _I],
 }
 
@@ -194,6 +199,8 @@ def prototypes():
 
 
 _RESTYPE = {"asamd_csr_plan_destroy": None, "asamd_csr_plan_stats": POINTER(asamd_csr_stats),
+            "asamd_csr_plan_transpose_stats": POINTER(asamd_csr_stats),
+            "asamd_analysis_transpose_stats": POINTER(asamd_csr_stats),
             "asamd_analysis_stats": POINTER(asamd_csr_stats)}
 
 ALGO_NAMES = {ASAMD_SPMV_AUTO: "auto", ASAMD_SPMV_VECTOR: "vector", ASAMD_SPMV_ROWCONST: "rowconst",

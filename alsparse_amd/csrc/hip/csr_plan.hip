@@ -20,6 +20,7 @@
 #include "spmv_merge.hpp"
 #include "spmv_rows.hpp"
 #include "spmv_tiled.hpp"
+#include "spmv_trans.hpp"
 #include "tile_sort.hpp"
 
 using namespace asamd;
@@ -103,6 +104,12 @@ struct asamd_csr_plan {
   // ELL copy (trusted plans of short, nearly equal rows)
   void* d_eval;               // ell_width * m values, column-major
   int* d_ecol;                // ... and zero-based columns
+  // CSR copy of the transpose (trusted plans, on request) and its own plan
+  asamd_csr_plan* tr_plan;
+  int* d_tr_row_ptr;          // n + 1
+  int* d_tr_col;              // nnz zero-based rows of A
+  void* d_tr_val;             // nnz values
+  bool lazy_transpose;        // build the copy on the first transposed multiply
 };
 
 static int width_for_mean(double mean) {
@@ -177,6 +184,18 @@ static void free_ell(asamd_csr_plan* p) {
   p->d_eval = nullptr;
   p->d_ecol = nullptr;
   p->st.ell_built = 0;
+}
+
+static void free_transpose(asamd_csr_plan* p) {
+  if (p->tr_plan) asamd_csr_plan_destroy(p->tr_plan);
+  p->tr_plan = nullptr;
+  if (p->d_tr_row_ptr) (void)hipFree(p->d_tr_row_ptr);
+  if (p->d_tr_col) (void)hipFree(p->d_tr_col);
+  if (p->d_tr_val) (void)hipFree(p->d_tr_val);
+  p->d_tr_row_ptr = nullptr;
+  p->d_tr_col = nullptr;
+  p->d_tr_val = nullptr;
+  p->st.transpose_built = 0;
 }
 
 // An ELL copy pays when rows are short and padding them to the longest costs
@@ -583,7 +602,75 @@ extern "C" void asamd_csr_plan_destroy(asamd_csr_plan* p) {
   if (p->d_head_val) (void)hipFree(p->d_head_val);
   free_tiled(p);
   free_ell(p);
+  free_transpose(p);
   delete p;
+}
+
+// CSR of A^T: sort (column, entry) pairs by column (stable: rows ascending inside
+// a column), read the column offsets off the sorted keys, gather rows and values.
+template <typename T>
+static hipError_t build_transpose(hipStream_t stream, asamd_csr_plan* p, const int* row_ptr, const int* col_ind,
+                                  const T* val) {
+  asamd_csr_stats& st = p->st;
+  const int nnz = st.nnz, n = st.n;
+  int* d_coo = nullptr;
+  unsigned *d_key = nullptr, *d_key2 = nullptr, *d_idx = nullptr, *d_perm = nullptr;
+  hipError_t e = hipMalloc(&d_coo, (size_t)nnz * sizeof(int));
+  if (e == hipSuccess) e = hipMalloc(&d_key, (size_t)nnz * sizeof(unsigned));
+  if (e == hipSuccess) e = hipMalloc(&d_key2, (size_t)nnz * sizeof(unsigned));
+  if (e == hipSuccess) e = hipMalloc(&d_idx, (size_t)nnz * sizeof(unsigned));
+  if (e == hipSuccess) e = hipMalloc(&d_perm, (size_t)nnz * sizeof(unsigned));
+  if (e == hipSuccess) e = hipMalloc(&p->d_tr_row_ptr, ((size_t)n + 1) * sizeof(int));
+  if (e == hipSuccess) e = hipMalloc(&p->d_tr_col, (size_t)nnz * sizeof(int));
+  if (e == hipSuccess) e = hipMalloc(&p->d_tr_val, (size_t)nnz * sizeof(T));
+  if (e == hipSuccess) e = (hipError_t)asamd_csr2coo(stream, row_ptr, nnz, st.m, d_coo, st.base);
+  if (e == hipSuccess) {
+    int grid = (nnz + 255) / 256;
+    if (grid > 256 * 32) grid = 256 * 32;
+    transpose_keys_kernel<<<grid, 256, 0, stream>>>(nnz, col_ind, st.base, d_key, d_idx);
+    e = hipGetLastError();
+    unsigned bits = 1;
+    while (bits < 32 && ((int64_t)1 << bits) < (int64_t)n) ++bits;
+    if (e == hipSuccess) e = sort_pairs_u32(stream, d_key, d_key2, d_idx, d_perm, (size_t)nnz, bits);
+    if (e == hipSuccess) {
+      tile_bounds_kernel<<<(unsigned)(((int64_t)n + 1 + 255) / 256), 256, 0, stream>>>(nnz, d_key2, (int64_t)n,
+                                                                                      p->d_tr_row_ptr);
+      transpose_gather_kernel<T><<<grid, 256, 0, stream>>>(nnz, d_perm, d_coo, val, st.base, p->d_tr_col,
+                                                           (T*)p->d_tr_val);
+      e = hipGetLastError();
+    }
+    if (e == hipSuccess) e = hipStreamSynchronize(stream);
+  }
+  for (void* d : {(void*)d_coo, (void*)d_key, (void*)d_key2, (void*)d_idx, (void*)d_perm})
+    if (d) (void)hipFree(d);
+  if (e == hipSuccess)
+    e = (hipError_t)asamd_csr_plan_create(stream, n, st.m, nnz, p->d_tr_row_ptr, p->d_tr_col, p->d_tr_val, 0,
+                                          (int32_t)sizeof(T), /*trusted=*/1, &p->tr_plan);
+  if (e != hipSuccess) {
+    free_transpose(p);
+    return e;
+  }
+  st.transpose_built = 1;
+  return hipSuccess;
+}
+
+extern "C" int asamd_csr_plan_build_transpose(hipStream_t stream, asamd_csr_plan* p, const int32_t* row_ptr,
+                                              const int32_t* col_ind, const void* val) {
+  if (!p || !row_ptr || !col_ind || !val || !p->st.trusted || p->st.n <= 0) return hipErrorInvalidValue;
+  if (p->st.transpose_built) return hipSuccess;
+  if (p->st.nnz == 0) return hipSuccess;  // the scatter route has nothing to add
+  return p->val_size == 4 ? build_transpose<float>(stream, p, row_ptr, col_ind, (const float*)val)
+                          : build_transpose<double>(stream, p, row_ptr, col_ind, (const double*)val);
+}
+
+extern "C" int asamd_csr_plan_set_lazy_transpose(asamd_csr_plan* p, int32_t on) {
+  if (!p || !p->st.trusted) return hipErrorInvalidValue;
+  p->lazy_transpose = on != 0;
+  return hipSuccess;
+}
+
+extern "C" const asamd_csr_stats* asamd_csr_plan_transpose_stats(const asamd_csr_plan* p) {
+  return p && p->tr_plan ? &p->tr_plan->st : nullptr;
 }
 
 extern "C" const asamd_csr_stats* asamd_csr_plan_stats(const asamd_csr_plan* p) {
@@ -735,6 +822,55 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
       break;
   }
   return hipGetLastError();
+}
+
+template <typename T, int W>
+static void launch_trans_scatter(hipStream_t s, const asamd_csr_stats& st, T alpha, const T* val, const int* rp,
+                                 const int* ci, const T* x, T* y) {
+  constexpr int rows_per_block = kTransThreads / W;
+  const unsigned grid = (unsigned)(((int64_t)st.m + rows_per_block - 1) / rows_per_block);
+  csrmv_trans_scatter_kernel<T, W><<<grid, kTransThreads, 0, s>>>(st.m, st.n, alpha, val, rp, ci, x, y, st.base);
+}
+
+template <typename T>
+static int csrmv_trans_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, const int* rp, const int* ci,
+                            const T* x, T beta, T* y) {
+  if (!p || !val || !rp || !ci || !x || !y) return hipErrorInvalidValue;
+  if (p->val_size != (int)sizeof(T)) return hipErrorInvalidValue;
+  const asamd_csr_stats& st = p->st;
+  if (!p->tr_plan && p->lazy_transpose && st.trusted && st.nnz > 0) {
+    const hipError_t e = build_transpose<T>(s, p, rp, ci, val);
+    if (e == hipErrorOutOfMemory) {
+      (void)hipGetLastError();  // no room for the copy: scatter instead, and do not try again
+      p->lazy_transpose = false;
+    } else if (e != hipSuccess) {
+      return e;
+    }
+  }
+  if (p->tr_plan)
+    return csrmv_impl<T>(s, p->tr_plan, alpha, (const T*)p->d_tr_val, p->d_tr_row_ptr, p->d_tr_col, x, beta, y);
+  if (beta != T(1)) scale_vec_kernel<T><<<(unsigned)(((int64_t)st.n + 255) / 256), 256, 0, s>>>(st.n, beta, y);
+  switch (p->auto_width) {
+    case 2: launch_trans_scatter<T, 2>(s, st, alpha, val, rp, ci, x, y); break;
+    case 4: launch_trans_scatter<T, 4>(s, st, alpha, val, rp, ci, x, y); break;
+    case 8: launch_trans_scatter<T, 8>(s, st, alpha, val, rp, ci, x, y); break;
+    case 16: launch_trans_scatter<T, 16>(s, st, alpha, val, rp, ci, x, y); break;
+    case 32: launch_trans_scatter<T, 32>(s, st, alpha, val, rp, ci, x, y); break;
+    default: launch_trans_scatter<T, 64>(s, st, alpha, val, rp, ci, x, y); break;
+  }
+  return hipGetLastError();
+}
+
+extern "C" int asamd_s_csrmv_trans(hipStream_t stream, asamd_csr_plan* plan, float alpha, const float* val,
+                                   const int32_t* row_ptr, const int32_t* col_ind, const float* x, float beta,
+                                   float* y) {
+  return csrmv_trans_impl<float>(stream, plan, alpha, val, row_ptr, col_ind, x, beta, y);
+}
+
+extern "C" int asamd_d_csrmv_trans(hipStream_t stream, asamd_csr_plan* plan, double alpha, const double* val,
+                                   const int32_t* row_ptr, const int32_t* col_ind, const double* x, double beta,
+                                   double* y) {
+  return csrmv_trans_impl<double>(stream, plan, alpha, val, row_ptr, col_ind, x, beta, y);
 }
 
 extern "C" int asamd_s_csrmv(hipStream_t stream, asamd_csr_plan* plan, float alpha,

@@ -10,24 +10,28 @@
 #define ASAMD_CSR spmat_csr_s_t
 #define ASAMD_DT ALPHA_SPARSE_DATATYPE_FLOAT
 #define ASAMD_KERNEL_CSRMV asamd_s_csrmv
+#define ASAMD_KERNEL_CSRMV_TRANS asamd_s_csrmv_trans
 #include "csrmv.inc"
 #undef ASAMD_T
 #undef ASAMD_S
 #undef ASAMD_CSR
 #undef ASAMD_DT
 #undef ASAMD_KERNEL_CSRMV
+#undef ASAMD_KERNEL_CSRMV_TRANS
 
 #define ASAMD_T double
 #define ASAMD_S d
 #define ASAMD_CSR spmat_csr_d_t
 #define ASAMD_DT ALPHA_SPARSE_DATATYPE_DOUBLE
 #define ASAMD_KERNEL_CSRMV asamd_d_csrmv
+#define ASAMD_KERNEL_CSRMV_TRANS asamd_d_csrmv_trans
 #include "csrmv.inc"
 #undef ASAMD_T
 #undef ASAMD_S
 #undef ASAMD_CSR
 #undef ASAMD_DT
 #undef ASAMD_KERNEL_CSRMV
+#undef ASAMD_KERNEL_CSRMV_TRANS
 
 /* Declared at include/alphasparse/spapi_dcu.h:573 and never defined in the
  * reference; semantics taken from the declaration's rocSPARSE namesake:

@@ -148,6 +148,11 @@ const asamd_csr_stats *asamd_analysis_stats(const void *key) {
   return r && r->plan ? asamd_csr_plan_stats(r->plan) : NULL;
 }
 
+const asamd_csr_stats *asamd_analysis_transpose_stats(const void *key) {
+  asamd_record *r = find_any(key);
+  return r && r->plan ? asamd_csr_plan_transpose_stats(r->plan) : NULL;
+}
+
 int asamd_analysis_set_algo(const void *key, int32_t algo) {
   asamd_record *r = find_any(key);
   if (!r || !r->plan) return (int)hipErrorInvalidValue;

@@ -70,7 +70,7 @@ def time_steps(fn, steps, warmup, hiprt):
             "wall_ms_per_step": wall_ms / steps}
 
 
-def run_spmv(cfg, steps, warmup, cpu_baseline, check):
+def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False):
     from alsparse_amd import capi, hiprt, workloads as wl
     lib = capi.load()
     t0 = time.time()
@@ -80,6 +80,9 @@ def run_spmv(cfg, steps, warmup, cpu_baseline, check):
     h = capi.Handle()
     descr = capi.make_descr()
     d_val, d_rp, d_ci = (hiprt.DeviceArray.from_numpy(v) for v in (a.values, a.row_ptr, a.col_ind))
+    op = capi.ALPHA_SPARSE_OPERATION_TRANSPOSE if transpose else capi.ALPHA_SPARSE_OPERATION_NON_TRANSPOSE
+    if transpose:  # y = alpha*A^T*x + beta*y: x has `rows` entries, y has `cols`
+        x, y0 = wl.uniform(a.rows, a.dtype, 3), wl.uniform(a.cols, a.dtype, 4)
     d_x, d_y = hiprt.DeviceArray.from_numpy(x), hiprt.DeviceArray.from_numpy(y0)
 
     info = capi.alphasparse_dcu_mat_info_t()
@@ -87,11 +90,14 @@ def run_spmv(cfg, steps, warmup, cpu_baseline, check):
     hiprt.synchronize()
     t0 = time.perf_counter()
     st = getattr(lib, "alphasparse_dcu_%s_csrmv_analysis" % p)(
-        h.h, 0, a.rows, a.cols, a.nnz, byref(descr), d_val.c_ptr(), d_rp.c_ptr(), d_ci.c_ptr(), info)
+        h.h, op, a.rows, a.cols, a.nnz, byref(descr), d_val.c_ptr(), d_rp.c_ptr(), d_ci.c_ptr(), info)
     hiprt.synchronize()
     analysis_ms = (time.perf_counter() - t0) * 1e3
     assert st == 0, "analysis status %d" % st
     stats = lib.asamd_analysis_stats(info).contents
+    if transpose:
+        assert stats.transpose_built == 1, "no room for the transposed copy"
+        stats = lib.asamd_analysis_transpose_stats(info).contents
     algo = capi.ALGO_NAMES.get(stats.algo, "?")
     if stats.algo == capi.ASAMD_SPMV_VECTOR:
         algo += "(W=%d)" % stats.vector_width
@@ -100,7 +106,7 @@ def run_spmv(cfg, steps, warmup, cpu_baseline, check):
     csrmv = getattr(lib, "alphasparse_dcu_%s_csrmv" % p)
 
     def step():
-        s = csrmv(h.h, 0, a.rows, a.cols, a.nnz, byref(al), byref(descr), d_val.c_ptr(), d_rp.c_ptr(),
+        s = csrmv(h.h, op, a.rows, a.cols, a.nnz, byref(al), byref(descr), d_val.c_ptr(), d_rp.c_ptr(),
                   d_ci.c_ptr(), info, d_x.c_ptr(), byref(be), d_y.c_ptr())
         if s != 0:
             raise RuntimeError("csrmv status %d" % s)
@@ -113,25 +119,35 @@ def run_spmv(cfg, steps, warmup, cpu_baseline, check):
         hiprt.synchronize()
         y = d_y.to_numpy()
         t0 = time.time()
-        ref = orc.csrmv_plain(a, alpha, x, beta, y0)
-        err = orc.csrmv_err(a, alpha, x, beta, y0, y, ref)
         tol = 1e-4 if a.dtype == np.float32 else 1e-12
-        parity = {"max_row_err": err.strict, "max_row_err_with_beta_y": err.full, "tol": tol,
-                  "zero_den_mismatch": err.zero_den_mismatch, "reference_check_ratio": err.ref_ratio,
-                  "ok": bool(err.strict <= tol and err.zero_den_mismatch == 0)}
+        if transpose:
+            ref = orc.csrmv_trans_plain(a, alpha, x, beta, y0)
+            absa = wl.Csr(a.rows, a.cols, a.row_ptr, a.col_ind, np.abs(a.values), a.base)
+            den = abs(alpha) * orc.csrmv_trans_plain(absa, 1.0, np.abs(x), 0.0, np.zeros(a.cols, a.dtype)).astype(np.float64)
+            diff = np.abs(y.astype(np.float64) - ref.astype(np.float64))
+            zbad = int(np.count_nonzero(diff[den == 0]))
+            strict = float(np.max(diff[den > 0] / den[den > 0])) if np.any(den > 0) else 0.0
+            parity = {"max_row_err": strict, "tol": tol, "zero_den_mismatch": zbad, "ok": bool(strict <= tol and zbad == 0)}
+        else:
+            ref = orc.csrmv_plain(a, alpha, x, beta, y0)
+            err = orc.csrmv_err(a, alpha, x, beta, y0, y, ref)
+            parity = {"max_row_err": err.strict, "max_row_err_with_beta_y": err.full, "tol": tol,
+                      "zero_den_mismatch": err.zero_den_mismatch, "reference_check_ratio": err.ref_ratio,
+                      "ok": bool(err.strict <= tol and err.zero_den_mismatch == 0)}
         log("[bench] parity vs plain-kernel oracle: %s (oracle %.1f s)" % (parity, time.time() - t0))
         d_y.copy_from(y0)
 
     t = time_steps(step, steps, warmup, hiprt)
-    nbytes = wl.spmv_bytes(a.rows, a.cols, a.nnz, a.dtype.itemsize, beta)
-    res = {"workload": WORKLOAD_NAMES[cfg], "rows": a.rows, "nnz": a.nnz, "algorithmic_bytes": int(nbytes),
+    nbytes = (wl.spmv_bytes(a.cols, a.rows, a.nnz, a.dtype.itemsize, beta) if transpose
+              else wl.spmv_bytes(a.rows, a.cols, a.nnz, a.dtype.itemsize, beta))
+    res = {"workload": WORKLOAD_NAMES[cfg] + (" -- TRANSPOSED operation" if transpose else ""), "rows": a.rows, "nnz": a.nnz, "algorithmic_bytes": int(nbytes),
            "flops": 2 * a.nnz, "kernel": algo, "analysis_ms": analysis_ms, "timing": t,
            "gbs": nbytes / t["avg_ms"] / 1e6, "gflops": 2 * a.nnz / t["avg_ms"] / 1e6,
            "dtype": "f32" if a.dtype == np.float32 else "f64", "parity": parity}
     res["hbm_frac"] = res["gbs"] / HBM_PEAK_GBS
-    res["traffic"] = MEASURED_TRAFFIC_BYTES.get((cfg, algo))
+    res["traffic"] = None if transpose else MEASURED_TRAFFIC_BYTES.get((cfg, algo))
 
-    if cpu_baseline:
+    if cpu_baseline and not transpose:
         res["cpu_baseline"] = cpu_spmv(a, x, y0, alpha, beta, nbytes)
     lib.alphasparse_dcu_destroy_mat_info(info)
     for d in (d_val, d_rp, d_ci, d_x, d_y):
@@ -295,6 +311,8 @@ def main():
     ap.add_argument("--config", type=int, default=3, choices=[2, 3, 4, 5])
     ap.add_argument("--format", default="csr", choices=["csr", "ell", "coo"],
                     help="multiply the ELL / COO form of configuration 2 or 3 (converted on the GPU) instead")
+    ap.add_argument("--transpose", action="store_true",
+                    help="y = alpha*A^T*x + beta*y of configuration 2, 3 or 4 (analysis asked for the transposed operation)")
     ap.add_argument("--all", action="store_true", help="also measure the other configurations")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
@@ -330,14 +348,19 @@ def main():
     elif args.config == 5:
         main_res = run_spmm(args.steps, args.warmup, check)
     else:
-        main_res = run_spmv(args.config, args.steps, args.warmup, not args.no_cpu_baseline, check)
+        main_res = run_spmv(args.config, args.steps, args.warmup, not args.no_cpu_baseline, check, args.transpose)
     others = {}
     if args.all:
         for c in (2, 3, 4, 5):
-            if c == args.config:
+            if c == args.config and not args.transpose and args.format == "csr":
                 continue
             r = run_spmm(args.steps, args.warmup, check) if c == 5 else run_spmv(c, args.steps, args.warmup, False, check)
             others["C%d" % c] = {k: r[k] for k in ("workload", "gbs", "gflops", "hbm_frac", "timing", "parity", "kernel") if k in r}
+        for c in (3, 4):
+            if args.transpose and c == args.config:
+                continue
+            r = run_spmv(c, args.steps, args.warmup, False, check, True)
+            others["C%d_transposed" % c] = {k: r[k] for k in ("workload", "gbs", "gflops", "hbm_frac", "timing", "parity", "kernel")}
         for c, fmt in ((2, "ell"), (2, "coo"), (3, "ell"), (3, "coo")):
             if args.format == fmt and args.config == c:
                 continue

@@ -60,6 +60,7 @@ typedef struct {
   float tune_ms_ell;    /* ... and of the ELL copy's kernel, or 0             */
   int32_t ell_built;    /* 1: an ELL copy exists (ELL can be selected)        */
   int32_t ell_width;    /* its slots per row                                  */
+  int32_t transpose_built; /* 1: a CSR copy of the transpose exists           */
   int64_t hist[ASAMD_HIST_BINS];
 } asamd_csr_stats;
 
@@ -99,6 +100,29 @@ int asamd_s_csrmv(hipStream_t stream, asamd_csr_plan *plan, float alpha, const f
 int asamd_d_csrmv(hipStream_t stream, asamd_csr_plan *plan, double alpha, const double *val,
                   const int32_t *row_ptr, const int32_t *col_ind, const double *x, double beta,
                   double *y);
+
+/* CSR copy of the transpose, owned by the plan (trusted plans only; row_ptr,
+ * col_ind, val are the arrays the plan was created for).  Later transposed
+ * multiplies run the ordinary kernels on that copy (with an analysis of its
+ * own: asamd_csr_plan_transpose_stats).  No reference counterpart: the
+ * reference always scatters with atomics. */
+int asamd_csr_plan_build_transpose(hipStream_t stream, asamd_csr_plan *plan, const int32_t *row_ptr,
+                                   const int32_t *col_ind, const void *val);
+/* on != 0: the first transposed multiply builds that copy from the arrays it
+ * is given (for matrices whose device arrays the library owns). */
+int asamd_csr_plan_set_lazy_transpose(asamd_csr_plan *plan, int32_t on);
+const asamd_csr_stats *asamd_csr_plan_transpose_stats(const asamd_csr_plan *plan);
+
+/* y = alpha*A^T*x + beta*y: x has m entries, y has n.  Uses the transposed copy
+ * when the plan has one; otherwise scales y and scatters with hardware float
+ * atomics (y must be ordinary device memory), as
+ * src/kernel/dcu/level2/mv/csrmv/dcu_gemv_x_csr_trans.cpp:11-45, :49-68 does. */
+int asamd_s_csrmv_trans(hipStream_t stream, asamd_csr_plan *plan, float alpha, const float *val,
+                        const int32_t *row_ptr, const int32_t *col_ind, const float *x, float beta,
+                        float *y);
+int asamd_d_csrmv_trans(hipStream_t stream, asamd_csr_plan *plan, double alpha, const double *val,
+                        const int32_t *row_ptr, const int32_t *col_ind, const double *x, double beta,
+                        double *y);
 
 /* Dense operand addressing for SpMM: element (r, c) of B is
  * B[r*b_row_stride + c*b_col_stride], of C is C[r*c_row_stride + c*c_col_stride]. */
@@ -167,6 +191,8 @@ int asamd_d_coomv(hipStream_t stream, int32_t m, int32_t n, int64_t nnz, double 
  * analysed array).  NULL if nothing is recorded.  Implemented by the host
  * library's registry; no reference counterpart. */
 const asamd_csr_stats *asamd_analysis_stats(const void *key);
+/* ... and of the analysis of the transposed copy, or NULL if there is none. */
+const asamd_csr_stats *asamd_analysis_transpose_stats(const void *key);
 /* Force a kernel family (enum asamd_spmv_algo) on the analysis recorded for
  * `key`; returns 0 on success, a hipError_t otherwise. */
 int asamd_analysis_set_algo(const void *key, int32_t algo);

@@ -43,6 +43,26 @@
 ORACLE_MV_PLAIN(oracle_s_csrmv_plain, float)
 ORACLE_MV_PLAIN(oracle_d_csrmv_plain, double)
 
+/* ------------------------------------------------------------------------- *
+ * Plain transposed SpMV, y = alpha*A^T*x + beta*y (x has m entries, y has n):
+ * src/plain/kernel/level2/mv/gemv/gemv_x_csr_trans_plain.c:10-24
+ *   y[j] *= beta for j < n; per entry, row by row: val = alpha*values[ai];
+ *   y[col] += val*x[row].
+ * ------------------------------------------------------------------------- */
+#define ORACLE_MV_TRANS_PLAIN(NAME, T)                                                        \
+  void NAME(int32_t m, int32_t n, const int32_t *rows_start, const int32_t *rows_end,        \
+            const int32_t *col_indx, const T *values, T alpha, const T *x, T beta, T *y) {   \
+    for (int32_t j = 0; j < n; ++j) y[j] *= beta;                                             \
+    for (int32_t i = 0; i < m; i++) {                                                         \
+      for (int32_t ai = rows_start[i]; ai < rows_end[i]; ai++) {                              \
+        T val = alpha * values[ai];                                                           \
+        y[col_indx[ai]] += val * x[i];                                                        \
+      }                                                                                       \
+    }                                                                                         \
+  }
+ORACLE_MV_TRANS_PLAIN(oracle_s_csrmv_trans_plain, float)
+ORACLE_MV_TRANS_PLAIN(oracle_d_csrmv_trans_plain, double)
+
 /* Same product with every row accumulated in fp64 whatever T is: separates the
  * oracle's own rounding noise from a real error on long rows.  Not a
  * restatement of reference code. */

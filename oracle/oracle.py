@@ -48,6 +48,8 @@ def lib(fast=False):
                 f.restype, f.argtypes = None, [I, P, P, P, P, T, P, I, I, T, P, I]
             f = getattr(L, "oracle_%s_csr2ell" % s)
             f.restype, f.argtypes = I, [I, P, P, P, I, I, I, P, P]
+            f = getattr(L, "oracle_%s_csrmv_trans_plain" % s)
+            f.restype, f.argtypes = None, [I, I, P, P, P, P, T, P, T, P]
             f = getattr(L, "oracle_%s_coomv_plain" % s)
             f.restype, f.argtypes = None, [I, I, P, P, P, T, P, T, P]
             f = getattr(L, "oracle_%s_ellmv" % s)
@@ -85,6 +87,28 @@ def csrmv_plain(a, alpha, x, beta, y0, fast=False):
     getattr(lib(fast), "oracle_%s_csrmv_plain" % _pre(a.dtype))(
         a.rows, _p(rs), _p(re), _p(ci), _p(a.values), T(alpha), _p(x), T(beta), _p(y))
     return y
+
+
+def csrmv_trans_plain(a, alpha, x, beta, y0):
+    """y = alpha*A^T*x + beta*y0: x has a.rows entries, y0 has a.cols."""
+    rs, re, ci = (np.ascontiguousarray(v) for v in _zero_based(a))
+    y = np.array(y0, dtype=a.dtype, copy=True)
+    T = _ct(a.dtype)
+    getattr(lib(), "oracle_%s_csrmv_trans_plain" % _pre(a.dtype))(
+        a.rows, a.cols, _p(rs), _p(re), _p(ci), _p(a.values), T(alpha), _p(x), T(beta), _p(y))
+    return y
+
+
+def transpose(a):
+    """CSR of A^T, zero-based; rows of A stay ascending inside every column (stable sort)."""
+    from alsparse_amd import workloads as wl
+    rp = a.row_ptr.astype(np.int64) - a.base
+    ci = a.col_ind.astype(np.int64) - a.base
+    rows = np.repeat(np.arange(a.rows, dtype=np.int32), np.diff(rp))
+    order = np.argsort(ci, kind="stable")
+    trp = np.concatenate([[0], np.cumsum(np.bincount(ci, minlength=a.cols))]).astype(np.int32)
+    return wl.Csr(a.cols, a.rows, trp, np.ascontiguousarray(rows[order]), np.ascontiguousarray(a.values[order]), 0,
+                  "transpose(%s)" % a.name)
 
 
 def csrmv_omp(a, alpha, x, beta, y0, threads=0, fast=True):

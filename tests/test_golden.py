@@ -31,6 +31,8 @@ def test_oracle_reproduces_reference_outputs_bit_for_bit(key):
     assert np.array_equal(np.ascontiguousarray(col), GOLD[key + ".mm_col_plain"])
     assert np.array_equal(orc.csr2coo(a), GOLD[key + ".coo_rows"])
     assert np.array_equal(orc.coomv_plain(a, orc.csr2coo(a), 2.0, x, 3.0, y0), GOLD[key + ".coomv_plain"])
+    xt, yt = wl.uniform(a.rows, a.dtype, 3), wl.uniform(a.cols, a.dtype, 4)
+    assert np.array_equal(orc.csrmv_trans_plain(a, 2.0, xt, 3.0, yt), GOLD[key + ".mv_trans_plain"])
     assert orc.csr2ell_width(a) == int(GOLD[key + ".ell_ld"][0])
     ev, ec = orc.csr2ell(a)
     assert np.array_equal(ev, GOLD[key + ".ell_val"]) and np.array_equal(ec, GOLD[key + ".ell_col"])

@@ -254,6 +254,33 @@ def test_coomv_and_ellmv_against_brute_force_and_csr(dtype):
         assert orc.coomv_plain(a, rows, 1.0, x, 0.0, y0)[0] == 0 or np.diff(a.row_ptr)[0] > 0
 
 
+@pytest.mark.parametrize("dtype", DT)
+def test_transposed_spmv_against_dense_scipy_and_the_untransposed_oracle(dtype):
+    """y = alpha A^T x + beta y: dense fp64 brute force on rectangular matrices (a swapped
+    m / n or a forgotten transpose cannot pass), scipy, and the plain oracle applied to an
+    explicitly transposed matrix (same sums in another order: within the rounding bound;
+    bit-equal on integer data)."""
+    rng = np.random.default_rng(13)
+    for a in (csr_from_lengths([0, 3, 0, 0, 5, 1, 0, 2, 0, 70], 90, dtype, seed=2), wl.laplace2d(9, 7, dtype),
+              wl.powerlaw_rmat(7, 300, dtype), wl.uniform_rows(50, 400, 8, dtype, base=1)):
+        x, y0 = wl.uniform(a.rows, dtype, 3), wl.uniform(a.cols, dtype, 4)
+        at = orc.transpose(a)
+        assert (at.rows, at.cols, at.nnz) == (a.cols, a.rows, a.nnz)
+        D = dense(a)
+        assert np.array_equal(dense(at), D.T)
+        for alpha, beta in ((1.0, 0.0), (2.0, 3.0), (-0.5, 1.0)):
+            got = orc.csrmv_trans_plain(a, alpha, x, beta, y0)
+            want = alpha * (D.T @ x.astype(np.float64)) + beta * y0.astype(np.float64)
+            bound = gamma_bound(at, alpha, x, beta, y0)
+            assert np.all(np.abs(got - want) <= bound)
+            sp_want = alpha * (sp.csr_matrix(D).T @ x.astype(np.float64)) + beta * y0.astype(np.float64)
+            assert np.all(np.abs(got - sp_want) <= bound)
+            assert np.all(np.abs(got - orc.csrmv_plain(at, alpha, x, beta, y0)) <= 2 * bound)
+        ai = wl.Csr(a.rows, a.cols, a.row_ptr, a.col_ind, rng.integers(-4, 5, a.nnz).astype(dtype), a.base)
+        xi, yi = rng.integers(-4, 5, a.rows).astype(dtype), rng.integers(-4, 5, a.cols).astype(dtype)
+        assert np.array_equal(orc.csrmv_trans_plain(ai, 2.0, xi, 3.0, yi), orc.csrmv_plain(orc.transpose(ai), 2.0, xi, 3.0, yi))
+
+
 def test_error_metric_detects_planted_errors():
     a = wl.uniform_rows(400, 300, 16, np.float32)
     x, y0 = wl.uniform(a.cols, np.float32, 3), wl.uniform(a.rows, np.float32, 4)
@@ -334,6 +361,9 @@ def test_oracle_is_bit_identical_to_reference_kernels(dtype):
         x, y0 = wl.uniform(a.cols, dtype, 3), wl.uniform(a.rows, dtype, 4)
         for alpha, beta in ((1.0, 0.0), (2.0, 3.0), (1.0, 0.5)):
             assert np.array_equal(orc.csrmv_plain(a, alpha, x, beta, y0), _ref_mv("gemv_{t}_csr_plain", a, alpha, x, beta, y0)), a.name
+            xt, yt = wl.uniform(a.rows, dtype, 3), wl.uniform(a.cols, dtype, 4)
+            assert np.array_equal(orc.csrmv_trans_plain(a, alpha, xt, beta, yt),
+                                  _ref_mv("gemv_{t}_csr_trans_plain", a, alpha, xt, beta, yt)), a.name
             for th in (1, 3, 8):
                 assert np.array_equal(orc.csrmv_omp(a, alpha, x, beta, y0, threads=th, fast=False),
                                       _ref_mv("gemv_{t}_csr", a, alpha, x, beta, y0, threads=th)), (a.name, th)
