@@ -151,6 +151,8 @@ def _per_type(ctype):
         "asamd_{s}_ellmv": [_P, _I, _I, T, _P, _P, _I, _I, _P, T, _P],
         "asamd_{s}_coomv": [_P, _I, _I, c_int64, T, _P, _P, _P, _I, _P, T, _P],
         "asamd_{s}_csrmm": [_P, _I, _I, _I, _I, T, _P, _P, _P, _I, _P, T, _P, POINTER(asamd_dense_strides)],
+        "asamd_{s}_csrmm_ws": [_P, _I, _I, _I, _I, T, _P, _P, _P, _I, _P, T, _P, POINTER(asamd_dense_strides), _P,
+                               c_size_t],
         "asamd_{s}_csr2ell": [_P, _I, _P, _P, _P, _I, _I, _I, _P, _P],
     }
 
@@ -179,6 +181,7 @@ _COMMON = {
     "asamd_csr_plan_build_transpose": [_P, _P, _P, _P, _P],
     "asamd_csr_plan_set_lazy_transpose": [_P, _I],
     "asamd_csr_plan_transpose_stats": [_P],
+    "asamd_csrmm_workspace_bytes": [_I, _I, _I, _I, POINTER(asamd_dense_strides)],
     "asamd_csr2coo": [_P, _P, _I, _I, _P, _I],
     "asamd_csr2ell_width": [_P, _I, _P, POINTER(_I)],
     "asamd_warmup": [_P],
@@ -198,7 +201,7 @@ def prototypes():
     return out
 
 
-_RESTYPE = {"asamd_csr_plan_destroy": None, "asamd_csr_plan_stats": POINTER(asamd_csr_stats),
+_RESTYPE = {"asamd_csr_plan_destroy": None, "asamd_csrmm_workspace_bytes": c_size_t, "asamd_csr_plan_stats": POINTER(asamd_csr_stats),
             "asamd_csr_plan_transpose_stats": POINTER(asamd_csr_stats),
             "asamd_analysis_transpose_stats": POINTER(asamd_csr_stats),
             "asamd_analysis_stats": POINTER(asamd_csr_stats)}

@@ -3,7 +3,7 @@
 
 #define ASAMD_T float
 #define ASAMD_S s
-#define ASAMD_KERNEL_CSRMM asamd_s_csrmm
+#define ASAMD_KERNEL_CSRMM asamd_s_csrmm_ws
 #include "csrmm.inc"
 #undef ASAMD_T
 #undef ASAMD_S
@@ -11,7 +11,7 @@
 
 #define ASAMD_T double
 #define ASAMD_S d
-#define ASAMD_KERNEL_CSRMM asamd_d_csrmm
+#define ASAMD_KERNEL_CSRMM asamd_d_csrmm_ws
 #include "csrmm.inc"
 #undef ASAMD_T
 #undef ASAMD_S

@@ -259,7 +259,7 @@ def run_format_spmv(cfg, fmt, steps, warmup, check):
     return res
 
 
-def run_spmm(steps, warmup, check):
+def run_spmm(steps, warmup, check, col_major=False):
     from alsparse_amd import capi, hiprt, workloads as wl
     lib = capi.load()
     a, B, C0, alpha, beta, extra = wl.config(5)
@@ -268,13 +268,18 @@ def run_spmm(steps, warmup, check):
     descr = capi.make_descr()
     from ctypes import c_float
     d_val, d_rp, d_ci = (hiprt.DeviceArray.from_numpy(v) for v in (a.values, a.row_ptr, a.col_ind))
-    d_B, d_C = hiprt.DeviceArray.from_numpy(B), hiprt.DeviceArray.from_numpy(C0)
+    # column-major: the same B and C stored column by column (ldb = k, ldc = m)
+    B_dev = np.ascontiguousarray(B.T) if col_major else B
+    C_dev = np.ascontiguousarray(C0.T) if col_major else C0
+    d_B, d_C = hiprt.DeviceArray.from_numpy(B_dev), hiprt.DeviceArray.from_numpy(C_dev)
     al, be = c_float(alpha), c_float(beta)
+    layout = capi.ALPHA_SPARSE_LAYOUT_COLUMN_MAJOR if col_major else capi.ALPHA_SPARSE_LAYOUT_ROW_MAJOR
+    ldb, ldc = (a.cols, a.rows) if col_major else (n, n)
 
     def step():
-        s = lib.alphasparse_dcu_s_csrmm(h.h, 0, 0, capi.ALPHA_SPARSE_LAYOUT_ROW_MAJOR, a.rows, n, a.cols, a.nnz,
+        s = lib.alphasparse_dcu_s_csrmm(h.h, 0, 0, layout, a.rows, n, a.cols, a.nnz,
                                         byref(al), byref(descr), d_val.c_ptr(), d_rp.c_ptr(), d_ci.c_ptr(),
-                                        d_B.c_ptr(), n, byref(be), d_C.c_ptr(), n)
+                                        d_B.c_ptr(), ldb, byref(be), d_C.c_ptr(), ldc)
         if s != 0:
             raise RuntimeError("csrmm status %d" % s)
 
@@ -284,19 +289,22 @@ def run_spmm(steps, warmup, check):
         step()
         hiprt.synchronize()
         C = d_C.to_numpy()
+        if col_major:
+            C = np.ascontiguousarray(C.reshape(n, a.rows).T)
         ref = orc.csrmm_plain(a, alpha, B, beta, C0, omp=True)
         err = orc.csrmm_err(a, alpha, B, beta, C0, C, ref)
         parity = {"max_elem_err": err.strict, "max_elem_err_with_beta_c": err.full, "tol": 1e-4,
                   "zero_den_mismatch": err.zero_den_mismatch, "ok": bool(err.strict <= 1e-4 and err.zero_den_mismatch == 0)}
-        d_C.copy_from(C0)
+        d_C.copy_from(C_dev)
     t = time_steps(step, steps, warmup, hiprt)
     nbytes = wl.spmm_bytes(a.rows, a.cols, n, a.nnz, 4, beta)
-    res = {"workload": WORKLOAD_NAMES[5], "rows": a.rows, "nnz": a.nnz, "algorithmic_bytes": int(nbytes),
+    res = {"workload": WORKLOAD_NAMES[5].replace("row-major", "column-major") if col_major else WORKLOAD_NAMES[5],
+           "kernel": "spmm column-major (B transposed into scratch)" if col_major else "spmm row-major", "rows": a.rows, "nnz": a.nnz, "algorithmic_bytes": int(nbytes),
            "gather_upper_bound_bytes": int(a.nnz) * n * 4, "flops": 2 * a.nnz * n, "timing": t,
            "gbs": nbytes / t["avg_ms"] / 1e6, "gflops": 2 * a.nnz * n / t["avg_ms"] / 1e6, "dtype": "f32",
            "parity": parity}
     res["hbm_frac"] = res["gbs"] / HBM_PEAK_GBS
-    res["traffic"] = MEASURED_TRAFFIC_BYTES.get((5, "spmm row-major"))
+    res["traffic"] = None if col_major else MEASURED_TRAFFIC_BYTES.get((5, "spmm row-major"))
     for d in (d_val, d_rp, d_ci, d_B, d_C):
         d.free()
     h.close()
@@ -311,6 +319,7 @@ def main():
     ap.add_argument("--config", type=int, default=3, choices=[2, 3, 4, 5])
     ap.add_argument("--format", default="csr", choices=["csr", "ell", "coo"],
                     help="multiply the ELL / COO form of configuration 2 or 3 (converted on the GPU) instead")
+    ap.add_argument("--col-major", action="store_true", help="configuration 5 with column-major B and C")
     ap.add_argument("--transpose", action="store_true",
                     help="y = alpha*A^T*x + beta*y of configuration 2, 3 or 4 (analysis asked for the transposed operation)")
     ap.add_argument("--all", action="store_true", help="also measure the other configurations")
@@ -346,16 +355,19 @@ def main():
             sys.exit("bench.py: --format ell|coo is measured on configuration 2 or 3")
         main_res = run_format_spmv(args.config, args.format, args.steps, args.warmup, check)
     elif args.config == 5:
-        main_res = run_spmm(args.steps, args.warmup, check)
+        main_res = run_spmm(args.steps, args.warmup, check, args.col_major)
     else:
         main_res = run_spmv(args.config, args.steps, args.warmup, not args.no_cpu_baseline, check, args.transpose)
     others = {}
     if args.all:
         for c in (2, 3, 4, 5):
-            if c == args.config and not args.transpose and args.format == "csr":
+            if c == args.config and not args.transpose and args.format == "csr" and not args.col_major:
                 continue
             r = run_spmm(args.steps, args.warmup, check) if c == 5 else run_spmv(c, args.steps, args.warmup, False, check)
             others["C%d" % c] = {k: r[k] for k in ("workload", "gbs", "gflops", "hbm_frac", "timing", "parity", "kernel") if k in r}
+        if not (args.config == 5 and args.col_major):
+            r = run_spmm(args.steps, args.warmup, check, True)
+            others["C5_column_major"] = {k: r[k] for k in ("workload", "gbs", "gflops", "hbm_frac", "timing", "parity", "kernel")}
         for c in (3, 4):
             if args.transpose and c == args.config:
                 continue

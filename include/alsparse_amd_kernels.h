@@ -144,6 +144,23 @@ int asamd_d_csrmm(hipStream_t stream, int32_t m, int32_t n, int32_t k, int32_t n
                   const double *B, double beta, double *C,
                   const asamd_dense_strides *strides);
 
+/* Column-major B next to column-major C is multiplied from a row-major copy of B
+ * (k*n elements) in a caller-provided device workspace; without one, or with too
+ * small a one, the multiply falls back to gathering B element by element, which
+ * is tens of times slower.  asamd_csrmm_workspace_bytes returns what those strides
+ * need (0 for every other layout).  The workspace only has to live until the
+ * call's kernels have run on `stream`. */
+size_t asamd_csrmm_workspace_bytes(int32_t val_size, int32_t m, int32_t n, int32_t k,
+                                   const asamd_dense_strides *strides);
+int asamd_s_csrmm_ws(hipStream_t stream, int32_t m, int32_t n, int32_t k, int32_t nnz, float alpha,
+                     const float *val, const int32_t *row_ptr, const int32_t *col_ind, int32_t base,
+                     const float *B, float beta, float *C, const asamd_dense_strides *strides,
+                     void *workspace, size_t workspace_bytes);
+int asamd_d_csrmm_ws(hipStream_t stream, int32_t m, int32_t n, int32_t k, int32_t nnz, double alpha,
+                     const double *val, const int32_t *row_ptr, const int32_t *col_ind, int32_t base,
+                     const double *B, double beta, double *C, const asamd_dense_strides *strides,
+                     void *workspace, size_t workspace_bytes);
+
 /* coo_row[k] = r + base for k in [row_ptr[r]-base, row_ptr[r+1]-base).
  * Defines on the GPU what src/core/format/convert_coo_x_csr.c:30-37 does on the host. */
 int asamd_csr2coo(hipStream_t stream, const int32_t *row_ptr, int32_t nnz, int32_t m,

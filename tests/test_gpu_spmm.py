@@ -125,3 +125,68 @@ def test_host_pointer_mm(gpu, dtype):
     assert st == 0
     check(a, 1.5, B, 0.5, C0, np.ascontiguousarray(Cf), "alphasparse_mm col-major")
     assert lib.alphasparse_destroy(A) == 0
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
+@pytest.mark.parametrize("mat", sorted(MATS))
+def test_column_major_every_matrix_shape_and_scratch_growth(gpu, mat, dtype):
+    """Column-major B and C on ragged / skewed / one-based matrices, with the dense width going up and
+    down between calls on one handle (its scratch buffer grows, then is reused for smaller products),
+    and beta = 0 over a C full of NaN."""
+    for base in (0, 1):
+        a = MATS[mat](dtype, base)
+        da = DeviceCsr(a)
+        try:
+            for n in (2, 130, 3, 64, 65):
+                ldb, ldc = a.cols + 1, a.rows + 2
+                B = np.asfortranarray(wl.uniform(ldb * n, dtype, 5).reshape(n, ldb).T)
+                C0 = np.asfortranarray(wl.uniform(ldc * n, dtype, 4).reshape(n, ldc).T)
+                for alpha, beta in ((1.5, 0.5), (1.0, 0.0)):
+                    Cin = C0 if beta != 0 else np.full_like(C0, np.nan)
+                    announce("spmm col-major", mat, n, np.dtype(dtype).name, base, alpha, beta)
+                    out = run_csrmm(gpu, da, capi.ALPHA_SPARSE_LAYOUT_COLUMN_MAJOR, 0, alpha, B.T.reshape(-1), ldb, beta,
+                                    Cin.T.reshape(-1), ldc, n, a.cols).reshape(n, ldc).T
+                    check(a, alpha, B[:a.cols, :], beta, np.zeros_like(C0[:a.rows, :]) if beta == 0 else C0[:a.rows, :],
+                          out[:a.rows, :], "col-major %s n=%d" % (mat, n))
+                    if beta != 0:
+                        assert np.array_equal(out[a.rows:, :], C0[a.rows:, :]), "padding rows of C were touched"
+        finally:
+            da.free()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
+def test_kernel_abi_with_and_without_workspace(gpu, dtype):
+    """asamd_?_csrmm (no workspace: element-wise gathers of column-major B) and asamd_?_csrmm_ws
+    (row-major copy of B in the workspace) agree with the oracle; a workspace that is too small is ignored."""
+    lib = capi.load()
+    a = wl.powerlaw_rmat(11, 1500, dtype)
+    n = 37
+    p, T = capi.prefix(dtype), capi.scalar_type(dtype)
+    B = np.asfortranarray(wl.uniform(a.cols * n, dtype, 5).reshape(n, a.cols).T)
+    C0 = np.asfortranarray(wl.uniform(a.rows * n, dtype, 4).reshape(n, a.rows).T)
+    st = capi.asamd_dense_strides(1, a.cols, 1, a.rows)
+    need = lib.asamd_csrmm_workspace_bytes(a.dtype.itemsize, a.rows, n, a.cols, byref(st))
+    assert need >= a.cols * n * a.dtype.itemsize
+    row_major = capi.asamd_dense_strides(n, 1, n, 1)
+    assert lib.asamd_csrmm_workspace_bytes(a.dtype.itemsize, a.rows, n, a.cols, byref(row_major)) == 0
+    da = DeviceCsr(a)
+    dB = hiprt.DeviceArray.from_numpy(B.T.reshape(-1))
+    ws = hiprt.DeviceArray((need,), np.uint8)
+    try:
+        outs = []
+        for what, w, wb in (("none", None, 0), ("full", ws.c_ptr(), need), ("too small", ws.c_ptr(), need // 2)):
+            announce("csrmm_ws workspace", what, np.dtype(dtype).name)
+            dC = hiprt.DeviceArray.from_numpy(C0.T.reshape(-1))
+            e = getattr(lib, "asamd_%s_csrmm_ws" % p)(None, a.rows, n, a.cols, a.nnz, T(1.5), da.val.c_ptr(), da.row_ptr.c_ptr(),
+                                                     da.col.c_ptr(), 0, dB.c_ptr(), T(0.5), dC.c_ptr(), byref(st), w, wb)
+            assert e == 0
+            hiprt.synchronize()
+            out = dC.to_numpy().reshape(n, a.rows).T
+            dC.free()
+            check(a, 1.5, B, 0.5, C0, out, "csrmm_ws %s" % what)
+            outs.append(out)
+        assert np.array_equal(outs[0], outs[2])   # both took the fallback
+    finally:
+        ws.free()
+        dB.free()
+        da.free()
