@@ -35,9 +35,11 @@ ALPHA_SPARSE_INDEX_BASE_ONE = 1
 ALPHA_SPARSE_LAYOUT_ROW_MAJOR = 0
 ALPHA_SPARSE_LAYOUT_COLUMN_MAJOR = 1
 
-ALPHA_SPARSE_FORMAT_CSR = 1
+ALPHA_SPARSE_FORMAT_COO, ALPHA_SPARSE_FORMAT_CSR, ALPHA_SPARSE_FORMAT_BSR = 0, 1, 3
+ALPHA_SPARSE_FORMAT_ELL, ALPHA_SPARSE_FORMAT_COO_AOS = 6, 9
 ALPHA_SPARSE_DATATYPE_FLOAT = 0
 ALPHA_SPARSE_DATATYPE_DOUBLE = 1
+ALPHA_SPARSE_DATATYPE_FLOAT_COMPLEX, ALPHA_SPARSE_DATATYPE_DOUBLE_COMPLEX = 2, 3
 
 # kernel families of the thin kernel ABI (include/alsparse_amd_kernels.h)
 (ASAMD_SPMV_AUTO, ASAMD_SPMV_VECTOR, ASAMD_SPMV_ROWCONST, ASAMD_SPMV_MERGE, ASAMD_SPMV_SCALAR, ASAMD_SPMV_TILED,
@@ -100,6 +102,22 @@ class _alphasparse_dcu_mat_info(Structure):
 
 alphasparse_dcu_mat_info_t = POINTER(_alphasparse_dcu_mat_info)
 alphasparse_dcu_handle_t = c_void_p  # opaque from Python: holds a hipDeviceProp_t
+
+
+class alphasparse_dcu_spmat_descr(Structure):  # include/alphasparse/handle.h:272-295 of the reference
+    _fields_ = [("init", c_bool), ("analysed", c_bool), ("rows", c_int64), ("cols", c_int64), ("nnz", c_int64),
+                ("row_data", c_void_p), ("col_data", c_void_p), ("ind_data", c_void_p), ("val_data", c_void_p),
+                ("row_type", c_int), ("col_type", c_int), ("data_type", c_int), ("idx_base", c_int), ("format", c_int),
+                ("descr", POINTER(alpha_dcu_matrix_descr)), ("info", alphasparse_dcu_mat_info_t)]
+
+
+class alphasparse_dcu_dnvec_descr(Structure):  # include/alphasparse/handle.h:297-304
+    _fields_ = [("init", c_bool), ("size", c_int64), ("values", c_void_p), ("data_type", c_int)]
+
+
+ALPHA_SPARSE_DCU_INDEXTYPE_U16, ALPHA_SPARSE_DCU_INDEXTYPE_I32, ALPHA_SPARSE_DCU_INDEXTYPE_I64 = 1, 2, 3
+(ALPHA_SPARSE_DCU_SPMV_ALG_DEFAULT, ALPHA_SPARSE_DCU_SPMV_ALG_COO, ALPHA_SPARSE_DCU_SPMV_ALG_CSR_ADAPTIVE,
+ ALPHA_SPARSE_DCU_SPMV_ALG_CSR_STREAM, ALPHA_SPARSE_DCU_SPMV_ALG_ELL) = range(5)
 
 
 class asamd_csr_stats(Structure):
@@ -170,6 +188,9 @@ _COMMON = {
     "alphasparse_dcu_destroy_csrmv_info": [POINTER(_alphasparse_dcu_csrmv_info)],
     "get_alphasparse_dcu_status_for_hip_status": [c_int],
     "alphasparse_dcu_csrmv_clear": [alphasparse_dcu_handle_t, _P],
+    "alphasparse_dcu_spmv": [alphasparse_dcu_handle_t, c_int, _P, POINTER(alphasparse_dcu_spmat_descr),
+                             POINTER(alphasparse_dcu_dnvec_descr), _P, POINTER(alphasparse_dcu_dnvec_descr), c_int, c_int,
+                             POINTER(c_size_t), _P],
     "alphasparse_dcu_csr2coo": [alphasparse_dcu_handle_t, _P, _I, _I, _P, c_int],
     "alphasparse_dcu_csr2ell_width": [alphasparse_dcu_handle_t, _I, alpha_dcu_matrix_descr_t, _P,
                                       alpha_dcu_matrix_descr_t, POINTER(_I)],

@@ -297,6 +297,70 @@ alphasparse_status_t alphasparse_dcu_d_ellmv(alphasparse_dcu_handle_t handle,
                                              ALPHA_INT ell_width, const double *x, const double *beta,
                                              double *y);
 
+/* ---- generic (descriptor) SpMV -------------------------------------------------
+ * Enums: include/alphasparse/spdef.h:209-213 (index types), :244-251 (algorithms).
+ * Descriptors: include/alphasparse/handle.h:272-304.  The reference has no
+ * constructors for them: callers fill the structs themselves (init = true).
+ * For an ELL matrix `nnz` holds the ELL width and col_data / val_data the
+ * column-major arrays (src/core/op_dcu/generic/alphasparse_dcu_spmv.cpp:215-229). */
+typedef enum {
+  ALPHA_SPARSE_DCU_INDEXTYPE_U16 = 1,
+  ALPHA_SPARSE_DCU_INDEXTYPE_I32 = 2,
+  ALPHA_SPARSE_DCU_INDEXTYPE_I64 = 3
+} alphasparse_dcu_indextype_t;
+
+typedef enum {
+  ALPHA_SPARSE_DCU_SPMV_ALG_DEFAULT = 0,
+  ALPHA_SPARSE_DCU_SPMV_ALG_COO = 1,
+  ALPHA_SPARSE_DCU_SPMV_ALG_CSR_ADAPTIVE = 2,
+  ALPHA_SPARSE_DCU_SPMV_ALG_CSR_STREAM = 3,
+  ALPHA_SPARSE_DCU_SPMV_ALG_ELL = 4
+} alphasparse_dcu_spmv_alg_t;
+
+struct _alphasparse_dcu_spmat_descr {
+  bool init;
+  bool analysed;
+  int64_t rows;
+  int64_t cols;
+  int64_t nnz;
+  void *row_data;
+  void *col_data;
+  void *ind_data;
+  void *val_data;
+  alphasparse_dcu_indextype_t row_type;
+  alphasparse_dcu_indextype_t col_type;
+  alphasparse_datatype_t data_type;
+  alphasparse_index_base_t idx_base;
+  alphasparse_format_t format;
+  struct alpha_dcu_matrix_descr *descr;
+  alphasparse_dcu_mat_info_t info;
+};
+struct _alphasparse_dcu_dnvec_descr {
+  bool init;
+  int64_t size;
+  void *values;
+  alphasparse_datatype_t data_type;
+};
+typedef struct _alphasparse_dcu_spmat_descr *alphasparse_dcu_spmat_descr_t;
+typedef struct _alphasparse_dcu_dnvec_descr *alphasparse_dcu_dnvec_descr_t;
+
+/* include/alphasparse/spapi_dcu.h:4371-4381; behaviour of
+ * src/core/op_dcu/generic/alphasparse_dcu_spmv.cpp:17-275: a call with
+ * temp_buffer == NULL reports *buffer_size = 4 and, for a CSR matrix under the
+ * DEFAULT / CSR_ADAPTIVE algorithm, runs the csrmv analysis once; a call with a
+ * buffer multiplies (COO, CSR or ELL; fp32 / fp64).  Differences: the analysis
+ * is run in the matrix's own precision (the reference always calls the fp32
+ * one, :68-71), and a successful CSR / ELL multiply returns its status
+ * (SUCCESS) where the reference falls through to NOT_SUPPORTED (:274).
+ * Complex data types return NOT_SUPPORTED. */
+alphasparse_status_t alphasparse_dcu_spmv(alphasparse_dcu_handle_t handle, alphasparse_operation_t trans,
+                                          const void *alpha, const alphasparse_dcu_spmat_descr_t mat,
+                                          const alphasparse_dcu_dnvec_descr_t x, const void *beta,
+                                          const alphasparse_dcu_dnvec_descr_t y,
+                                          alphasparse_datatype_t compute_type,
+                                          alphasparse_dcu_spmv_alg_t alg, size_t *buffer_size,
+                                          void *temp_buffer);
+
 #ifdef __cplusplus
 }
 #endif

@@ -84,6 +84,11 @@ int main(void) {
          offsetof(struct _alphasparse_dcu_mat_info, boost_enable));
   printf("%zu %zu\n", sizeof(asamd_csr_stats), offsetof(asamd_csr_stats, hist));
   printf("%zu %zu\n", sizeof(struct alpha_dcu_matrix_descr), sizeof(struct alpha_matrix_descr));
+  printf("%zu %zu %zu %zu %zu\n", sizeof(struct _alphasparse_dcu_spmat_descr), offsetof(struct _alphasparse_dcu_spmat_descr, rows),
+         offsetof(struct _alphasparse_dcu_spmat_descr, val_data), offsetof(struct _alphasparse_dcu_spmat_descr, format),
+         offsetof(struct _alphasparse_dcu_spmat_descr, info));
+  printf("%zu %zu %zu\n", sizeof(struct _alphasparse_dcu_dnvec_descr), offsetof(struct _alphasparse_dcu_dnvec_descr, values),
+         offsetof(struct _alphasparse_dcu_dnvec_descr, data_type));
   return 0;
 }''')
     exe = tmp_path / "layout"
@@ -98,6 +103,9 @@ int main(void) {
     assert nums[3] == [ctypes.sizeof(MI), MI.csrmv_info.offset, MI.boost_enable.offset]
     assert nums[4] == [ctypes.sizeof(ST), ST.hist.offset]
     assert nums[5] == [ctypes.sizeof(capi.alpha_dcu_matrix_descr), ctypes.sizeof(capi.alpha_matrix_descr)]
+    SM, DV = capi.alphasparse_dcu_spmat_descr, capi.alphasparse_dcu_dnvec_descr
+    assert nums[6] == [ctypes.sizeof(SM), SM.rows.offset, SM.val_data.offset, SM.format.offset, SM.info.offset]
+    assert nums[7] == [ctypes.sizeof(DV), DV.values.offset, DV.data_type.offset]
 
 
 def test_no_product_code_touches_the_oracle():

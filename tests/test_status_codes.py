@@ -145,6 +145,50 @@ def test_coomv_and_ellmv_status_precedence(lib, p, T):
     assert ell(width=-3) == S.ALPHA_SPARSE_STATUS_INVALID_VALUE
 
 
+def test_generic_spmv_status_codes(lib):
+    """src/core/op_dcu/generic/alphasparse_dcu_spmv.cpp:30-76: check order, size query."""
+    from ctypes import c_size_t
+    SM, DV = capi.alphasparse_dcu_spmat_descr, capi.alphasparse_dcu_dnvec_descr
+    d = descr()
+    a, b = c_float(1), c_float(0)
+
+    def mat(**kw):
+        m = SM(True, True, 4, 4, 8, P, P, None, P, S.ALPHA_SPARSE_DCU_INDEXTYPE_I32, S.ALPHA_SPARSE_DCU_INDEXTYPE_I32,
+               S.ALPHA_SPARSE_DATATYPE_FLOAT, 0, S.ALPHA_SPARSE_FORMAT_CSR, ctypes.pointer(d), None)
+        for k, v in kw.items():
+            setattr(m, k, v)
+        return m
+
+    x, y = DV(True, 4, P, S.ALPHA_SPARSE_DATATYPE_FLOAT), DV(True, 4, P, S.ALPHA_SPARSE_DATATYPE_FLOAT)
+    size = c_size_t(0)
+    buf = P
+
+    def call(h=H, m=None, xx=x, yy=y, al=byref(a), be=byref(b), ct=S.ALPHA_SPARSE_DATATYPE_FLOAT, alg=0, bs=byref(size), tb=None):
+        m = mat() if m is None else m
+        return lib.alphasparse_dcu_spmv(h, 0, al, byref(m) if m is not False else None, byref(xx) if xx is not None else None, be,
+                                        byref(yy) if yy is not None else None, ct, alg, bs, tb)
+
+    assert call(h=NULL) == S.ALPHA_SPARSE_STATUS_INVALID_HANDLE
+    for kw in ({"m": False}, {"xx": None}, {"yy": None}, {"al": None}, {"be": None}):
+        assert call(**kw) == S.ALPHA_SPARSE_STATUS_INVALID_POINTER
+    assert call(m=mat(init=False)) == S.ALPHA_SPARSE_STATUS_INVALID_VALUE
+    assert call(xx=DV(False, 4, P, 0)) == S.ALPHA_SPARSE_STATUS_INVALID_VALUE
+    assert call(ct=S.ALPHA_SPARSE_DATATYPE_DOUBLE) == S.ALPHA_SPARSE_STATUS_NOT_SUPPORTED       # mixed precision
+    assert call(m=mat(row_type=S.ALPHA_SPARSE_DCU_INDEXTYPE_I64)) == S.ALPHA_SPARSE_STATUS_NOT_SUPPORTED
+    assert call(m=mat(col_type=S.ALPHA_SPARSE_DCU_INDEXTYPE_U16)) == S.ALPHA_SPARSE_STATUS_NOT_SUPPORTED
+    # size query on an already analysed matrix: no device work, 4 bytes
+    assert call() == S.ALPHA_SPARSE_STATUS_SUCCESS and size.value == 4
+    # complex data and formats other than COO / CSR / ELL are refused at the multiply
+    cx = S.ALPHA_SPARSE_DATATYPE_FLOAT_COMPLEX
+    assert call(m=mat(data_type=cx), xx=DV(True, 4, P, cx), yy=DV(True, 4, P, cx), ct=cx, tb=buf) == S.ALPHA_SPARSE_STATUS_NOT_SUPPORTED
+    assert call(m=mat(format=S.ALPHA_SPARSE_FORMAT_COO_AOS), tb=buf) == S.ALPHA_SPARSE_STATUS_NOT_SUPPORTED
+    assert call(m=mat(format=S.ALPHA_SPARSE_FORMAT_BSR), tb=buf) == S.ALPHA_SPARSE_STATUS_NOT_SUPPORTED
+    # the typed entry points' own validation shows through
+    assert call(m=mat(val_data=None), tb=buf) == S.ALPHA_SPARSE_STATUS_INVALID_POINTER
+    assert call(m=mat(rows=0), tb=buf) == S.ALPHA_SPARSE_STATUS_SUCCESS
+    assert call(m=mat(rows=1 << 40), tb=buf) == S.ALPHA_SPARSE_STATUS_INVALID_VALUE
+
+
 def test_conversion_status_codes(lib):
     d = descr()
     w = c_int32(-5)
