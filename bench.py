@@ -51,26 +51,86 @@ def log(*a):
 
 
 def time_steps(fn, steps, warmup, hiprt):
-    """Per-launch HIP-event timing on the stream the library launches on (the
-    handle's stream is the null stream), bracketed by device synchronisation."""
+    """HIP-event timing on the stream the library launches on (the handle's stream is the
+    null stream), bracketed by device synchronisation.  The K steps are timed once
+    back to back between two events (avg_ms: what a caller's loop sees) and once
+    more with an event after every step (min / median; each event costs a few
+    microseconds of gap, which shows on the 60 us kernels)."""
     for _ in range(warmup):
         fn()
     hiprt.synchronize()
-    evs = [hiprt.Event() for _ in range(steps + 1)]
+    e0, e1 = hiprt.Event(), hiprt.Event()
     t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    e1.synchronize()
+    hiprt.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    avg = e0.elapsed_ms(e1) / steps
+    evs = [hiprt.Event() for _ in range(steps + 1)]
     evs[0].record()
     for i in range(steps):
         fn()
         evs[i + 1].record()
     evs[-1].synchronize()
     hiprt.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3
     per = [evs[i].elapsed_ms(evs[i + 1]) for i in range(steps)]
-    return {"avg_ms": float(np.mean(per)), "min_ms": float(np.min(per)), "median_ms": float(np.median(per)),
-            "wall_ms_per_step": wall_ms / steps}
+    return {"avg_ms": float(avg), "min_ms": float(np.min(per)), "median_ms": float(np.median(per)),
+            "per_step_events_avg_ms": float(np.mean(per)), "wall_ms_per_step": wall_ms / steps}
 
 
-def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False):
+ROCSPARSE = "/opt/rocm/lib/librocsparse.so"
+
+
+def vendor_spmv(a, x, y0, alpha, beta, nbytes, steps, warmup, transpose=False):
+    """rocSPARSE's csrmv (with its analysis) on the same device arrays' contents, timed the same
+    way: the vendor library that the reference's own tests compare against
+    (test/dcu/level2/mv_csr_s_dcu_test.cpp:41-147).  A reported comparison, never part of the
+    product; None when the library is not installed."""
+    if not os.path.exists(ROCSPARSE):
+        return None
+    import ctypes
+    from ctypes import c_double, c_float, c_int
+    from alsparse_amd import hiprt
+    R = ctypes.CDLL(ROCSPARSE)
+    f32 = a.dtype == np.float32
+    T, p = (c_float, "s") if f32 else (c_double, "d")
+    h, descr, info = c_void_p(), c_void_p(), c_void_p()
+    if R.rocsparse_create_handle(byref(h)) or R.rocsparse_create_mat_descr(byref(descr)) or R.rocsparse_create_mat_info(byref(info)):
+        return None
+    a0 = a
+    d = [hiprt.DeviceArray.from_numpy(np.ascontiguousarray(v)) for v in (a0.values, a0.row_ptr - a0.base, a0.col_ind - a0.base, x, y0)]
+    mv, an = getattr(R, "rocsparse_%scsrmv" % p), getattr(R, "rocsparse_%scsrmv_analysis" % p)
+    P = c_void_p
+    mv.argtypes = [P, c_int, c_int, c_int, c_int, P, P, P, P, P, P, P, P, P]
+    an.argtypes = [P, c_int, c_int, c_int, c_int, P, P, P, P, P]
+    op = 112 if transpose else 111  # rocsparse_operation_transpose / _none
+    al, be = T(alpha), T(beta)
+    t0 = time.perf_counter()
+    st = an(h, op, a.rows, a.cols, a.nnz, descr, d[0].c_ptr(), d[1].c_ptr(), d[2].c_ptr(), info)
+    hiprt.synchronize()
+    analysis_ms = (time.perf_counter() - t0) * 1e3
+    if st != 0:
+        return None
+
+    def step():
+        s_ = mv(h, op, a.rows, a.cols, a.nnz, byref(al), descr, d[0].c_ptr(), d[1].c_ptr(), d[2].c_ptr(), info,
+                d[3].c_ptr(), byref(be), d[4].c_ptr())
+        if s_ != 0:
+            raise RuntimeError("rocsparse csrmv status %d" % s_)
+    t = time_steps(step, steps, warmup, hiprt)
+    for v in d:
+        v.free()
+    R.rocsparse_destroy_mat_info(info)
+    R.rocsparse_destroy_mat_descr(descr)
+    R.rocsparse_destroy_handle(h)
+    return {"library": "rocSPARSE csrmv after csrmv_analysis", "value": nbytes / t["avg_ms"] / 1e6, "unit": "GB/s",
+            "ms": t["avg_ms"], "analysis_ms": analysis_ms}
+
+
+def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False, vendor=False):
     from alsparse_amd import capi, hiprt, workloads as wl
     lib = capi.load()
     t0 = time.time()
@@ -149,6 +209,8 @@ def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False):
 
     if cpu_baseline and not transpose:
         res["cpu_baseline"] = cpu_spmv(a, x, y0, alpha, beta, nbytes)
+    if vendor:
+        res["vendor_baseline"] = vendor_spmv(a, x, y0, alpha, beta, nbytes, steps, warmup, transpose)
     lib.alphasparse_dcu_destroy_mat_info(info)
     for d in (d_val, d_rp, d_ci, d_x, d_y):
         d.free()
@@ -259,7 +321,7 @@ def run_format_spmv(cfg, fmt, steps, warmup, check):
     return res
 
 
-def run_spmm(steps, warmup, check, col_major=False):
+def run_spmm(steps, warmup, check, col_major=False, vendor=False):
     from alsparse_amd import capi, hiprt, workloads as wl
     lib = capi.load()
     a, B, C0, alpha, beta, extra = wl.config(5)
@@ -305,6 +367,26 @@ def run_spmm(steps, warmup, check, col_major=False):
            "parity": parity}
     res["hbm_frac"] = res["gbs"] / HBM_PEAK_GBS
     res["traffic"] = None if col_major else MEASURED_TRAFFIC_BYTES.get((5, "spmm row-major"))
+    if col_major and vendor and os.path.exists(ROCSPARSE):
+        # rocSPARSE's legacy csrmm takes column-major operands only: compared on this layout
+        import ctypes
+        from ctypes import c_int
+        R = ctypes.CDLL(ROCSPARSE)
+        rh, rd = c_void_p(), c_void_p()
+        if R.rocsparse_create_handle(byref(rh)) == 0 and R.rocsparse_create_mat_descr(byref(rd)) == 0:
+            P = c_void_p
+            R.rocsparse_scsrmm.argtypes = [P, c_int, c_int, c_int, c_int, c_int, c_int, P, P, P, P, P, P, c_int, P, P, c_int]
+
+            def vstep():
+                s_ = R.rocsparse_scsrmm(rh, 111, 111, a.rows, n, a.cols, a.nnz, byref(al), rd, d_val.c_ptr(), d_rp.c_ptr(),
+                                        d_ci.c_ptr(), d_B.c_ptr(), ldb, byref(be), d_C.c_ptr(), ldc)
+                if s_ != 0:
+                    raise RuntimeError("rocsparse csrmm status %d" % s_)
+            vt = time_steps(vstep, max(2, steps // 4), 1, hiprt)
+            res["vendor_baseline"] = {"library": "rocSPARSE csrmm (column-major)", "value": nbytes / vt["avg_ms"] / 1e6,
+                                      "unit": "GB/s", "ms": vt["avg_ms"]}
+            R.rocsparse_destroy_mat_descr(rd)
+            R.rocsparse_destroy_handle(rh)
     for d in (d_val, d_rp, d_ci, d_B, d_C):
         d.free()
     h.close()
@@ -324,6 +406,8 @@ def main():
                     help="y = alpha*A^T*x + beta*y of configuration 2, 3 or 4 (analysis asked for the transposed operation)")
     ap.add_argument("--all", action="store_true", help="also measure the other configurations")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-vendor-baseline", action="store_true",
+                    help="skip timing rocSPARSE's csrmv on the same workload (reported as vendor_baseline)")
     ap.add_argument("--no-check", action="store_true")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
                     help="also launch one plain copy kernel of this many MiB (reads and writes that many "
@@ -355,19 +439,23 @@ def main():
             sys.exit("bench.py: --format ell|coo is measured on configuration 2 or 3")
         main_res = run_format_spmv(args.config, args.format, args.steps, args.warmup, check)
     elif args.config == 5:
-        main_res = run_spmm(args.steps, args.warmup, check, args.col_major)
+        main_res = run_spmm(args.steps, args.warmup, check, args.col_major, not args.no_vendor_baseline)
     else:
-        main_res = run_spmv(args.config, args.steps, args.warmup, not args.no_cpu_baseline, check, args.transpose)
+        main_res = run_spmv(args.config, args.steps, args.warmup, not args.no_cpu_baseline, check, args.transpose,
+                            not args.no_vendor_baseline)
     others = {}
     if args.all:
         for c in (2, 3, 4, 5):
             if c == args.config and not args.transpose and args.format == "csr" and not args.col_major:
                 continue
-            r = run_spmm(args.steps, args.warmup, check) if c == 5 else run_spmv(c, args.steps, args.warmup, False, check)
-            others["C%d" % c] = {k: r[k] for k in ("workload", "gbs", "gflops", "hbm_frac", "timing", "parity", "kernel") if k in r}
+            r = (run_spmm(args.steps, args.warmup, check) if c == 5
+                 else run_spmv(c, args.steps, args.warmup, False, check, False, not args.no_vendor_baseline))
+            others["C%d" % c] = {k: r[k] for k in ("workload", "gbs", "gflops", "hbm_frac", "timing", "parity", "kernel",
+                                                    "vendor_baseline") if k in r}
         if not (args.config == 5 and args.col_major):
-            r = run_spmm(args.steps, args.warmup, check, True)
-            others["C5_column_major"] = {k: r[k] for k in ("workload", "gbs", "gflops", "hbm_frac", "timing", "parity", "kernel")}
+            r = run_spmm(args.steps, args.warmup, check, True, not args.no_vendor_baseline)
+            others["C5_column_major"] = {k: r[k] for k in ("workload", "gbs", "gflops", "hbm_frac", "timing", "parity", "kernel",
+                                                            "vendor_baseline") if k in r}
         for c in (3, 4):
             if args.transpose and c == args.config:
                 continue
@@ -396,6 +484,7 @@ def main():
                      "frac": main_res["hbm_frac"], "traffic": main_res.get("traffic"),
                      "algorithmic_bytes_per_launch": main_res["algorithmic_bytes"]},
         "cpu_baseline": main_res.get("cpu_baseline"),
+        "vendor_baseline": main_res.get("vendor_baseline"),
     }
     if others:
         out["others"] = others
