@@ -144,6 +144,7 @@ def _per_type(ctype):
     T, PT = ctype, POINTER(ctype)
     return {
         "alphasparse_{s}_create_csr": [POINTER(alphasparse_matrix_t), c_int, _I, _I, _P, _P, _P, _P],
+        "alphasparse_{s}_create_coo": [POINTER(alphasparse_matrix_t), c_int, _I, _I, _I, _P, _P, _P],
         "alphasparse_{s}_export_csr": [alphasparse_matrix_t, POINTER(c_int), POINTER(_I), POINTER(_I),
                                        POINTER(_P), POINTER(_P), POINTER(_P), POINTER(_P)],
         "alphasparse_{s}_mv": [c_int, T, alphasparse_matrix_t, alpha_matrix_descr, _P, T, _P],
@@ -177,6 +178,33 @@ def _per_type(ctype):
 
 _COMMON = {
     "alphasparse_destroy": [alphasparse_matrix_t],
+    "alphasparse_convert_csr": [alphasparse_matrix_t, c_int, POINTER(alphasparse_matrix_t)],
+    # driver helpers (include/alphasparse_util.h)
+    "alpha_malloc": [c_size_t],
+    "alpha_memalign": [c_size_t, c_size_t],
+    "alpha_free": [_P],
+    "alpha_fill_random_s": [_P, ctypes.c_uint, c_size_t],
+    "alpha_fill_random_d": [_P, ctypes.c_uint, c_size_t],
+    "alpha_read_coo": [ctypes.c_char_p, POINTER(_I), POINTER(_I), POINTER(_I), POINTER(_P), POINTER(_P), POINTER(_P)],
+    "alpha_read_coo_d": [ctypes.c_char_p, POINTER(_I), POINTER(_I), POINTER(_I), POINTER(_P), POINTER(_P), POINTER(_P)],
+    "check_s": [_P, c_size_t, _P, c_size_t],
+    "check_d": [_P, c_size_t, _P, c_size_t],
+    "args_help": [c_int, POINTER(ctypes.c_char_p)],
+    "args_get_if_check": [c_int, POINTER(ctypes.c_char_p)],
+    "args_get_thread_num": [c_int, POINTER(ctypes.c_char_p)],
+    "args_get_columns": [c_int, POINTER(ctypes.c_char_p), c_int],
+    "args_get_iter": [c_int, POINTER(ctypes.c_char_p)],
+    "args_get_data_file": [c_int, POINTER(ctypes.c_char_p)],
+    "args_get_data_fileA": [c_int, POINTER(ctypes.c_char_p)],
+    "args_get_data_fileB": [c_int, POINTER(ctypes.c_char_p)],
+    "alpha_args_get_layout": [c_int, POINTER(ctypes.c_char_p)],
+    "alpha_args_get_layoutB": [c_int, POINTER(ctypes.c_char_p)],
+    "alpha_args_get_layoutC": [c_int, POINTER(ctypes.c_char_p)],
+    "alpha_args_get_matrix_descrA": [c_int, POINTER(ctypes.c_char_p)],
+    "alpha_args_get_matrix_descrB": [c_int, POINTER(ctypes.c_char_p)],
+    "alpha_args_get_transA": [c_int, POINTER(ctypes.c_char_p)],
+    "alpha_args_get_transB": [c_int, POINTER(ctypes.c_char_p)],
+    "get_time_us": [],
     "init_handle": [POINTER(alphasparse_dcu_handle_t)],
     "alphasparse_dcu_get_handle": [POINTER(alphasparse_dcu_handle_t)],
     "alphasparse_dcu_destory_handle": [alphasparse_dcu_handle_t],
@@ -222,7 +250,12 @@ def prototypes():
     return out
 
 
-_RESTYPE = {"asamd_csr_plan_destroy": None, "asamd_csrmm_workspace_bytes": c_size_t, "asamd_csr_plan_stats": POINTER(asamd_csr_stats),
+_RESTYPE = {"asamd_csr_plan_destroy": None, "alpha_malloc": c_void_p, "alpha_memalign": c_void_p, "alpha_free": None,
+            "alpha_fill_random_s": None, "alpha_fill_random_d": None, "alpha_read_coo": None, "alpha_read_coo_d": None,
+            "args_help": None, "args_get_if_check": c_bool, "args_get_data_file": ctypes.c_char_p,
+            "args_get_data_fileA": ctypes.c_char_p, "args_get_data_fileB": ctypes.c_char_p,
+            "alpha_args_get_matrix_descrA": alpha_matrix_descr, "alpha_args_get_matrix_descrB": alpha_matrix_descr,
+            "get_time_us": c_double, "asamd_csrmm_workspace_bytes": c_size_t, "asamd_csr_plan_stats": POINTER(asamd_csr_stats),
             "asamd_csr_plan_transpose_stats": POINTER(asamd_csr_stats),
             "asamd_analysis_transpose_stats": POINTER(asamd_csr_stats),
             "asamd_analysis_stats": POINTER(asamd_csr_stats)}

@@ -1,0 +1,126 @@
+/* COO matrix handles and COO -> CSR conversion: what the reference's drivers
+ * call between reading a coordinate file and exporting CSR arrays.
+ * Reference behaviour: src/core/format/alphasparse_x_create_coo.c:7-48,
+ * src/core/format/convert_csr_x_coo.c:14-81,
+ * src/core/op_/alphasparse_convert_csr.c:125-141. */
+#include <stdlib.h>
+#include <string.h>
+
+#include "internal.h"
+
+#define ASAMD_CREATE_COO(NAME, T, COO, DT)                                                          \
+  alphasparse_status_t NAME(alphasparse_matrix_t *A, const alphasparse_index_base_t indexing,       \
+                            const ALPHA_INT rows, const ALPHA_INT cols, const ALPHA_INT nnz,        \
+                            ALPHA_INT *row_indx, ALPHA_INT *col_indx, T *values) {                  \
+    if (!A) return ALPHA_SPARSE_STATUS_INVALID_POINTER;                                             \
+    *A = NULL;                                                                                      \
+    if (rows <= 0 || cols <= 0 || nnz < 0) return ALPHA_SPARSE_STATUS_INVALID_VALUE;                \
+    if (indexing != ALPHA_SPARSE_INDEX_BASE_ZERO && indexing != ALPHA_SPARSE_INDEX_BASE_ONE)        \
+      return ALPHA_SPARSE_STATUS_INVALID_VALUE;                                                     \
+    if (nnz > 0 && (!row_indx || !col_indx || !values)) return ALPHA_SPARSE_STATUS_INVALID_POINTER; \
+    const ALPHA_INT shift = indexing == ALPHA_SPARSE_INDEX_BASE_ONE ? 1 : 0;                        \
+    alphasparse_matrix *AA = (alphasparse_matrix *)calloc(1, sizeof(*AA));                          \
+    COO *mat = (COO *)calloc(1, sizeof(*mat));                                                      \
+    const size_t cnt = (size_t)(nnz ? nnz : 1);                                                     \
+    ALPHA_INT *r = (ALPHA_INT *)malloc(cnt * sizeof(ALPHA_INT));                                    \
+    ALPHA_INT *c = (ALPHA_INT *)malloc(cnt * sizeof(ALPHA_INT));                                    \
+    T *v = (T *)malloc(cnt * sizeof(T));                                                            \
+    if (!AA || !mat || !r || !c || !v) {                                                            \
+      free(AA); free(mat); free(r); free(c); free(v);                                               \
+      return ALPHA_SPARSE_STATUS_ALLOC_FAILED;                                                      \
+    }                                                                                               \
+    for (ALPHA_INT i = 0; i < nnz; ++i) {                                                           \
+      r[i] = row_indx[i] - shift;                                                                   \
+      c[i] = col_indx[i] - shift;                                                                   \
+      v[i] = values[i];                                                                             \
+    }                                                                                               \
+    mat->values = v;                                                                                \
+    mat->row_indx = r;                                                                              \
+    mat->col_indx = c;                                                                              \
+    mat->rows = rows;                                                                               \
+    mat->cols = cols;                                                                               \
+    mat->nnz = nnz;                                                                                 \
+    AA->mat = mat;                                                                                  \
+    AA->format = ALPHA_SPARSE_FORMAT_COO;                                                           \
+    AA->datatype = DT;                                                                              \
+    *A = AA;                                                                                        \
+    return ALPHA_SPARSE_STATUS_SUCCESS;                                                             \
+  }
+ASAMD_CREATE_COO(alphasparse_s_create_coo, float, spmat_coo_s_t, ALPHA_SPARSE_DATATYPE_FLOAT)
+ASAMD_CREATE_COO(alphasparse_d_create_coo, double, spmat_coo_d_t, ALPHA_SPARSE_DATATYPE_DOUBLE)
+
+/* Position of every entry in (row, column) order, ties in source order: a
+ * counting sort by row, then each row's slice ordered by (column, position). */
+typedef struct {
+  ALPHA_INT col;
+  ALPHA_INT pos;
+} col_pos;
+
+static int col_pos_cmp(const void *a, const void *b) {
+  const col_pos *x = (const col_pos *)a, *y = (const col_pos *)b;
+  if (x->col != y->col) return x->col < y->col ? -1 : 1;
+  return x->pos < y->pos ? -1 : (x->pos > y->pos);
+}
+
+alphasparse_status_t alphasparse_convert_csr(const alphasparse_matrix_t source,
+                                             const alphasparse_operation_t operation,
+                                             alphasparse_matrix_t *dest) {
+  if (!source || !source->mat) return ALPHA_SPARSE_STATUS_NOT_INITIALIZED;
+  if (!dest) return ALPHA_SPARSE_STATUS_INVALID_POINTER;
+  *dest = NULL;
+  if (source->format != ALPHA_SPARSE_FORMAT_COO) return ALPHA_SPARSE_STATUS_INVALID_VALUE;
+  if (source->datatype != ALPHA_SPARSE_DATATYPE_FLOAT && source->datatype != ALPHA_SPARSE_DATATYPE_DOUBLE)
+    return ALPHA_SPARSE_STATUS_INVALID_VALUE;
+  if (operation != ALPHA_SPARSE_OPERATION_NON_TRANSPOSE) return ALPHA_SPARSE_STATUS_NOT_SUPPORTED;
+  /* both COO payloads share one layout up to the value pointer type */
+  const spmat_coo_s_t *coo = (const spmat_coo_s_t *)source->mat;
+  const ALPHA_INT m = coo->rows, nnz = coo->nnz;
+  for (ALPHA_INT i = 0; i < nnz; ++i)
+    if (coo->row_indx[i] < 0 || coo->row_indx[i] >= m || coo->col_indx[i] < 0 || coo->col_indx[i] >= coo->cols)
+      return ALPHA_SPARSE_STATUS_INVALID_VALUE;
+  ALPHA_INT *offsets = (ALPHA_INT *)calloc((size_t)m + 1, sizeof(ALPHA_INT));
+  ALPHA_INT *fill = (ALPHA_INT *)malloc(((size_t)m + 1) * sizeof(ALPHA_INT));
+  col_pos *order = (col_pos *)malloc((size_t)(nnz ? nnz : 1) * sizeof(col_pos));
+  ALPHA_INT *cols = (ALPHA_INT *)malloc((size_t)(nnz ? nnz : 1) * sizeof(ALPHA_INT));
+  if (!offsets || !fill || !order || !cols) {
+    free(offsets); free(fill); free(order); free(cols);
+    return ALPHA_SPARSE_STATUS_ALLOC_FAILED;
+  }
+  for (ALPHA_INT i = 0; i < nnz; ++i) offsets[coo->row_indx[i] + 1]++;
+  for (ALPHA_INT r = 0; r < m; ++r) offsets[r + 1] += offsets[r];
+  memcpy(fill, offsets, ((size_t)m + 1) * sizeof(ALPHA_INT));
+  for (ALPHA_INT i = 0; i < nnz; ++i) {
+    const ALPHA_INT at = fill[coo->row_indx[i]]++;
+    order[at].col = coo->col_indx[i];
+    order[at].pos = i;
+  }
+  for (ALPHA_INT r = 0; r < m; ++r)
+    qsort(order + offsets[r], (size_t)(offsets[r + 1] - offsets[r]), sizeof(col_pos), col_pos_cmp);
+  for (ALPHA_INT i = 0; i < nnz; ++i) cols[i] = order[i].col;
+  alphasparse_status_t st;
+  if (source->datatype == ALPHA_SPARSE_DATATYPE_FLOAT) {
+    float *vals = (float *)malloc((size_t)(nnz ? nnz : 1) * sizeof(float));
+    if (!vals) {
+      st = ALPHA_SPARSE_STATUS_ALLOC_FAILED;
+    } else {
+      for (ALPHA_INT i = 0; i < nnz; ++i) vals[i] = coo->values[order[i].pos];
+      st = alphasparse_s_create_csr(dest, ALPHA_SPARSE_INDEX_BASE_ZERO, m, coo->cols, offsets, offsets + 1, cols, vals);
+      free(vals);
+    }
+  } else {
+    const double *src = ((const spmat_coo_d_t *)source->mat)->values;
+    double *vals = (double *)malloc((size_t)(nnz ? nnz : 1) * sizeof(double));
+    if (!vals) {
+      st = ALPHA_SPARSE_STATUS_ALLOC_FAILED;
+    } else {
+      for (ALPHA_INT i = 0; i < nnz; ++i) vals[i] = src[order[i].pos];
+      st = alphasparse_d_create_csr(dest, ALPHA_SPARSE_INDEX_BASE_ZERO, m, coo->cols, offsets, offsets + 1, cols, vals);
+      free(vals);
+    }
+  }
+  free(offsets);
+  free(fill);
+  free(order);
+  free(cols);
+  return st;
+}

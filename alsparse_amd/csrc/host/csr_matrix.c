@@ -38,9 +38,19 @@ static void asamd_release_mirror(void *d_row_ptr, void *d_col, void *d_val) {
 alphasparse_status_t alphasparse_destroy(alphasparse_matrix_t A) {
   if (!A) return ALPHA_SPARSE_STATUS_SUCCESS;
   if (A->mat) {
-    if (A->format != ALPHA_SPARSE_FORMAT_CSR) return ALPHA_SPARSE_STATUS_INVALID_VALUE;
+    if (A->format != ALPHA_SPARSE_FORMAT_CSR && A->format != ALPHA_SPARSE_FORMAT_COO)
+      return ALPHA_SPARSE_STATUS_INVALID_VALUE;
     if (A->datatype != ALPHA_SPARSE_DATATYPE_FLOAT && A->datatype != ALPHA_SPARSE_DATATYPE_DOUBLE)
       return ALPHA_SPARSE_STATUS_INVALID_VALUE;
+    if (A->format == ALPHA_SPARSE_FORMAT_COO) { /* src/core/format/destroy_x_coo.c */
+      spmat_coo_s_t *c = (spmat_coo_s_t *)A->mat;
+      free(c->values);
+      free(c->row_indx);
+      free(c->col_indx);
+      free(c);
+      free(A);
+      return ALPHA_SPARSE_STATUS_SUCCESS;
+    }
     /* both payload structs share one layout up to the value pointer types */
     spmat_csr_s_t *m = (spmat_csr_s_t *)A->mat;
     if (m->d_row_ptr && asamd_registry_find(ASAMD_KEY_MATRIX, m->d_row_ptr))

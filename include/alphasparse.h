@@ -161,6 +161,56 @@ typedef struct {
   ALPHA_INT *d_col_indx;
 } spmat_csr_d_t;
 
+/* ---- COO payloads: include/alphasparse/spmat.h:73-86 and :96-110 ----------- */
+typedef struct {
+  float *values;
+  ALPHA_INT *row_indx;
+  ALPHA_INT *col_indx;
+  ALPHA_INT rows;
+  ALPHA_INT cols;
+  ALPHA_INT nnz;
+  bool ordered;
+  ALPHA_INT *d_rows_indx;
+  ALPHA_INT *d_cols_indx;
+  float *d_values;
+} spmat_coo_s_t;
+
+typedef struct {
+  double *values;
+  ALPHA_INT *row_indx;
+  ALPHA_INT *col_indx;
+  ALPHA_INT rows;
+  ALPHA_INT cols;
+  ALPHA_INT nnz;
+  bool ordered;
+  ALPHA_INT *d_rows_indx;
+  ALPHA_INT *d_cols_indx;
+  double *d_values;
+} spmat_coo_d_t;
+
+/* include/alphasparse/spapi.h (create_coo); src/core/format/alphasparse_x_create_coo.c:7-48:
+ * deep copy of nnz entries in the order given, indices shifted to base zero.
+ * This is how the reference's drivers get from a coordinate file to a handle. */
+alphasparse_status_t alphasparse_s_create_coo(alphasparse_matrix_t *A,
+                                              const alphasparse_index_base_t indexing,
+                                              const ALPHA_INT rows, const ALPHA_INT cols,
+                                              const ALPHA_INT nnz, ALPHA_INT *row_indx,
+                                              ALPHA_INT *col_indx, float *values);
+alphasparse_status_t alphasparse_d_create_coo(alphasparse_matrix_t *A,
+                                              const alphasparse_index_base_t indexing,
+                                              const ALPHA_INT rows, const ALPHA_INT cols,
+                                              const ALPHA_INT nnz, ALPHA_INT *row_indx,
+                                              ALPHA_INT *col_indx, double *values);
+
+/* src/core/op_/alphasparse_convert_csr.c:125-141 over
+ * src/core/format/convert_csr_x_coo.c:14-81: entries sorted by (row, column),
+ * duplicates kept.  Only a COO source and NON_TRANSPOSE are supported here.
+ * The reference's qsort leaves the order of duplicate coordinates unspecified;
+ * here they keep the order they had in the source. */
+alphasparse_status_t alphasparse_convert_csr(const alphasparse_matrix_t source,
+                                             const alphasparse_operation_t operation,
+                                             alphasparse_matrix_t *dest);
+
 /* ---- handle construction -------------------------------------------------
  * include/alphasparse/spapi.h:140-156; behaviour from
  * src/core/format/alphasparse_x_create_csr.c:7-57: deep copy, indices shifted
@@ -221,6 +271,8 @@ alphasparse_status_t alphasparse_d_mm(const alphasparse_operation_t operation, c
                                       const alphasparse_layout_t layout, const double *x,
                                       const ALPHA_INT columns, const ALPHA_INT ldx,
                                       const double beta, double *y, const ALPHA_INT ldy);
+
+#include "alphasparse_util.h"
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,90 @@
+/* Helpers that the reference's test drivers call next to the sparse API: matrix
+ * files, command-line flags, allocation, random fill, result comparison, timing.
+ * Own text; each declaration cites the reference declaration it stands in for
+ * (paths relative to the AlphaSparse tree).  Included by alphasparse.h inside
+ * its extern "C" block. */
+#ifndef ALSPARSE_AMD_ALPHASPARSE_UTIL_H
+#define ALSPARSE_AMD_ALPHASPARSE_UTIL_H
+
+#include <stdbool.h>
+#include <stddef.h>
+#include <stdio.h>
+#include <stdlib.h>
+
+/* include/alphasparse/util/malloc.h:13-17, :37-38.  alpha_free releases the
+ * block (the reference's frees only NULL pointers, src/util/malloc.c:45-48). */
+void *alpha_malloc(size_t bytes);
+void *alpha_memalign(size_t bytes, size_t alignment);
+void alpha_free(void *point);
+/* uniform values from rand() after srand(seed); seed 0 takes the clock */
+void alpha_fill_random_s(float *arr, unsigned int seed, const size_t size);
+void alpha_fill_random_d(double *arr, unsigned int seed, const size_t size);
+
+/* include/alphasparse/util/io.h:19-20; src/util/io.c:39-114: Matrix Market
+ * coordinate text ("%%MatrixMarket matrix coordinate <field> <symmetry>"):
+ * one-based "row col [value]" lines become zero-based triplets, a missing value
+ * reads as 1, a "symmetric" header mirrors every off-diagonal entry.  The
+ * arrays are allocated with alpha_malloc. */
+void alpha_read_coo(const char *file, ALPHA_INT *m_p, ALPHA_INT *n_p, ALPHA_INT *nnz_p,
+                    ALPHA_INT **row_index, ALPHA_INT **col_index, float **values);
+void alpha_read_coo_d(const char *file, ALPHA_INT *m_p, ALPHA_INT *n_p, ALPHA_INT *nnz_p,
+                      ALPHA_INT **row_index, ALPHA_INT **col_index, double **values);
+
+/* include/alphasparse/util/check.h:45-46; src/util/check.c:701-776:
+ * max|answer - result| / max|result|, printed as "correct,<ratio>" (return 0)
+ * or "error,<ratio>" (return -1) against 2e-5 (fp32) / 1e-10 (fp64). */
+int check_s(const float *answer_data, size_t answer_size, const float *result_data, size_t result_size);
+int check_d(const double *answer_data, size_t answer_size, const double *result_data, size_t result_size);
+
+/* include/alphasparse/util/args.h:16-44; src/util/args.c: GNU long options
+ * --help --check --thread-num= --transA= --transB= --typeA= --fillA= --diagA=
+ * --typeB= --fillB= --diagB= --data-file= --data-fileA= --data-fileB= --layout=
+ * --layoutB= --layoutC= --columns= --iter= --formatA= --formatB= --data-type= */
+void args_help(const int argc, const char *argv[]);
+bool args_get_if_check(const int argc, const char *argv[]);
+int args_get_thread_num(const int argc, const char *argv[]);
+int args_get_columns(const int argc, const char *argv[], int k);
+int args_get_iter(const int argc, const char *argv[]);
+const char *args_get_data_file(const int argc, const char *argv[]);
+const char *args_get_data_fileA(const int argc, const char *argv[]);
+const char *args_get_data_fileB(const int argc, const char *argv[]);
+alphasparse_layout_t alpha_args_get_layout(const int argc, const char *argv[]);
+alphasparse_layout_t alpha_args_get_layoutB(const int argc, const char *argv[]);
+alphasparse_layout_t alpha_args_get_layoutC(const int argc, const char *argv[]);
+struct alpha_matrix_descr alpha_args_get_matrix_descrA(const int argc, const char *argv[]);
+struct alpha_matrix_descr alpha_args_get_matrix_descrB(const int argc, const char *argv[]);
+alphasparse_operation_t alpha_args_get_transA(const int argc, const char *argv[]);
+alphasparse_operation_t alpha_args_get_transB(const int argc, const char *argv[]);
+
+/* include/alphasparse/handle.h:334; src/util_cpp/handle.cpp:487-493:
+ * wall clock in microseconds after a device synchronisation. */
+double get_time_us(void);
+
+/* include/alphasparse/util/error.h:9-45 and :139-150 */
+#define alpha_call_exit(func, message)                                      \
+  do {                                                                      \
+    alphasparse_status_t alpha_status_ = (func);                            \
+    if (alpha_status_ != ALPHA_SPARSE_STATUS_SUCCESS) {                     \
+      printf("%s\nstatus : %d\n", (message), (int)alpha_status_);           \
+      exit(-1);                                                             \
+    }                                                                       \
+  } while (0)
+
+#define roc_call_exit(func, message)                                        \
+  do {                                                                      \
+    int roc_status_ = (int)(func);                                          \
+    if (roc_status_ != 0) {                                                 \
+      printf("%s\nstatus : %d\n", (message), roc_status_);                  \
+      exit(-1);                                                             \
+    }                                                                       \
+  } while (0)
+
+#define PRINT_IF_HIP_ERROR(INPUT_STATUS_FOR_CHECK)                                            \
+  {                                                                                           \
+    int TMP_STATUS_FOR_CHECK = (int)(INPUT_STATUS_FOR_CHECK);                                 \
+    if (TMP_STATUS_FOR_CHECK != 0) {                                                          \
+      fprintf(stderr, "hip error code: %d at %s:%d\n", TMP_STATUS_FOR_CHECK, __FILE__, __LINE__); \
+    }                                                                                         \
+  }
+
+#endif /* ALSPARSE_AMD_ALPHASPARSE_UTIL_H */

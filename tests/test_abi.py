@@ -10,7 +10,7 @@ import pytest
 from alsparse_amd import capi
 from alsparse_amd.build import LIB_PATH, ROOT
 
-HEADERS = ["alphasparse.h", "alpha_spblas_dcu.h", "alsparse_amd_kernels.h"]
+HEADERS = ["alphasparse.h", "alphasparse_util.h", "alpha_spblas_dcu.h", "alsparse_amd_kernels.h"]
 
 
 def declared_functions():
@@ -20,7 +20,9 @@ def declared_functions():
         text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
         for m in re.finditer(r"\b([A-Za-z_][A-Za-z0-9_]*)\s*\(", text):
             n = m.group(1)
-            if n.startswith(("alphasparse_", "asamd_", "host2device_", "init_handle", "get_alphasparse")):
+            if n.startswith(("alphasparse_", "asamd_", "host2device_", "init_handle", "get_alphasparse", "alpha_malloc",
+                             "alpha_memalign", "alpha_free", "alpha_fill_", "alpha_read_", "alpha_args_", "args_", "check_",
+                             "get_time_us")):
                 names.add(n)
     return names
 
