@@ -145,6 +145,8 @@ def _per_type(ctype):
     return {
         "alphasparse_{s}_create_csr": [POINTER(alphasparse_matrix_t), c_int, _I, _I, _P, _P, _P, _P],
         "alphasparse_{s}_create_coo": [POINTER(alphasparse_matrix_t), c_int, _I, _I, _I, _P, _P, _P],
+        "alphasparse_{s}_export_ell": [alphasparse_matrix_t, POINTER(c_int), POINTER(_I), POINTER(_I), POINTER(_I),
+                                       POINTER(_P), POINTER(_P)],
         "alphasparse_{s}_export_csr": [alphasparse_matrix_t, POINTER(c_int), POINTER(_I), POINTER(_I),
                                        POINTER(_P), POINTER(_P), POINTER(_P), POINTER(_P)],
         "alphasparse_{s}_mv": [c_int, T, alphasparse_matrix_t, alpha_matrix_descr, _P, T, _P],
@@ -179,6 +181,7 @@ def _per_type(ctype):
 _COMMON = {
     "alphasparse_destroy": [alphasparse_matrix_t],
     "alphasparse_convert_csr": [alphasparse_matrix_t, c_int, POINTER(alphasparse_matrix_t)],
+    "alphasparse_convert_ell": [alphasparse_matrix_t, c_int, POINTER(alphasparse_matrix_t)],
     # driver helpers (include/alphasparse_util.h)
     "alpha_malloc": [c_size_t],
     "alpha_memalign": [c_size_t, c_size_t],

@@ -900,3 +900,20 @@ extern "C" int asamd_warmup(hipStream_t stream) {
   warmup_kernel<<<1, 1, 0, stream>>>();
   return hipGetLastError();
 }
+
+// Mean of the samples below twice the plain mean: src/util_cpp/handle.cpp:495-510.
+#include <vector>
+extern "C" double get_avg_time(std::vector<double> times) {
+  if (times.empty()) return 0.0;
+  double avg = 0.0;
+  for (double t : times) avg += t;
+  avg /= (double)times.size();
+  double kept = 0.0;
+  int cnt = 0;
+  for (double t : times)
+    if (t < 2 * avg) {
+      kept += t;
+      ++cnt;
+    }
+  return cnt ? kept / cnt : avg;
+}

@@ -124,3 +124,84 @@ alphasparse_status_t alphasparse_convert_csr(const alphasparse_matrix_t source,
   free(cols);
   return st;
 }
+
+/* ---- COO -> ELL ------------------------------------------------------------- */
+alphasparse_status_t alphasparse_convert_ell(const alphasparse_matrix_t source,
+                                             const alphasparse_operation_t operation,
+                                             alphasparse_matrix_t *dest) {
+  if (!source || !source->mat) return ALPHA_SPARSE_STATUS_NOT_INITIALIZED;
+  if (!dest) return ALPHA_SPARSE_STATUS_INVALID_POINTER;
+  *dest = NULL;
+  if (source->format != ALPHA_SPARSE_FORMAT_COO) return ALPHA_SPARSE_STATUS_INVALID_VALUE;
+  if (operation != ALPHA_SPARSE_OPERATION_NON_TRANSPOSE) return ALPHA_SPARSE_STATUS_NOT_SUPPORTED;
+  /* the reference goes COO -> CSR -> ELL as well (convert_ell_x_coo.c:11-14) */
+  alphasparse_matrix_t csr = NULL;
+  alphasparse_status_t st = alphasparse_convert_csr(source, operation, &csr);
+  if (st != ALPHA_SPARSE_STATUS_SUCCESS) return st;
+  const spmat_csr_s_t *c = (const spmat_csr_s_t *)csr->mat; /* layouts agree up to the value type */
+  const ALPHA_INT m = c->rows;
+  ALPHA_INT ld = 0;
+  for (ALPHA_INT r = 0; r < m; ++r) {
+    const ALPHA_INT len = c->rows_end[r] - c->rows_start[r];
+    if (len > ld) ld = len;
+  }
+  const int is_s = source->datatype == ALPHA_SPARSE_DATATYPE_FLOAT;
+  const size_t vsize = is_s ? sizeof(float) : sizeof(double);
+  const uint64_t slots = (uint64_t)ld * (uint64_t)m;
+  alphasparse_matrix *AA = NULL;
+  spmat_ell_s_t *ell = NULL;
+  void *vals = NULL;
+  ALPHA_INT *idx = NULL;
+  if (slots >= ((uint64_t)1 << 31)) {
+    st = ALPHA_SPARSE_STATUS_INVALID_VALUE;
+  } else {
+    AA = (alphasparse_matrix *)calloc(1, sizeof(*AA));
+    ell = (spmat_ell_s_t *)calloc(1, sizeof(*ell));
+    vals = calloc(slots ? slots : 1, vsize);
+    idx = (ALPHA_INT *)calloc(slots ? slots : 1, sizeof(ALPHA_INT));
+    if (!AA || !ell || !vals || !idx) st = ALPHA_SPARSE_STATUS_ALLOC_FAILED;
+  }
+  if (st == ALPHA_SPARSE_STATUS_SUCCESS) {
+    for (ALPHA_INT r = 0; r < m; ++r) {
+      const ALPHA_INT b = c->rows_start[r], e = c->rows_end[r];
+      for (ALPHA_INT k = b; k < e; ++k) {
+        const size_t at = (size_t)(k - b) * (size_t)m + (size_t)r;
+        idx[at] = c->col_indx[k];
+        if (is_s) ((float *)vals)[at] = c->values[k];
+        else ((double *)vals)[at] = ((const spmat_csr_d_t *)csr->mat)->values[k];
+      }
+    }
+    ell->values = (float *)vals;
+    ell->indices = idx;
+    ell->rows = m;
+    ell->cols = c->cols;
+    ell->ld = ld;
+    AA->mat = ell;
+    AA->format = ALPHA_SPARSE_FORMAT_ELL;
+    AA->datatype = source->datatype;
+    *dest = AA;
+  } else {
+    free(AA); free(ell); free(vals); free(idx);
+  }
+  (void)alphasparse_destroy(csr);
+  return st;
+}
+
+#define ASAMD_EXPORT_ELL(NAME, T, ELL, DT)                                                        \
+  alphasparse_status_t NAME(const alphasparse_matrix_t source, alphasparse_index_base_t *indexing, \
+                            ALPHA_INT *rows, ALPHA_INT *cols, ALPHA_INT *width,                   \
+                            ALPHA_INT **col_indx, T **values) {                                   \
+    if (!source || !source->mat) return ALPHA_SPARSE_STATUS_NOT_SUPPORTED;                        \
+    if (source->datatype != DT) return ALPHA_SPARSE_STATUS_INVALID_VALUE;                         \
+    if (source->format != ALPHA_SPARSE_FORMAT_ELL) return ALPHA_SPARSE_STATUS_INVALID_VALUE;      \
+    ELL *mat = (ELL *)source->mat;                                                                \
+    *indexing = ALPHA_SPARSE_INDEX_BASE_ZERO;                                                     \
+    *rows = mat->rows;                                                                            \
+    *cols = mat->cols;                                                                            \
+    *width = mat->ld;                                                                             \
+    *col_indx = mat->indices;                                                                     \
+    *values = mat->values;                                                                        \
+    return ALPHA_SPARSE_STATUS_SUCCESS;                                                           \
+  }
+ASAMD_EXPORT_ELL(alphasparse_s_export_ell, float, spmat_ell_s_t, ALPHA_SPARSE_DATATYPE_FLOAT)
+ASAMD_EXPORT_ELL(alphasparse_d_export_ell, double, spmat_ell_d_t, ALPHA_SPARSE_DATATYPE_DOUBLE)

@@ -38,10 +38,19 @@ static void asamd_release_mirror(void *d_row_ptr, void *d_col, void *d_val) {
 alphasparse_status_t alphasparse_destroy(alphasparse_matrix_t A) {
   if (!A) return ALPHA_SPARSE_STATUS_SUCCESS;
   if (A->mat) {
-    if (A->format != ALPHA_SPARSE_FORMAT_CSR && A->format != ALPHA_SPARSE_FORMAT_COO)
+    if (A->format != ALPHA_SPARSE_FORMAT_CSR && A->format != ALPHA_SPARSE_FORMAT_COO &&
+        A->format != ALPHA_SPARSE_FORMAT_ELL)
       return ALPHA_SPARSE_STATUS_INVALID_VALUE;
     if (A->datatype != ALPHA_SPARSE_DATATYPE_FLOAT && A->datatype != ALPHA_SPARSE_DATATYPE_DOUBLE)
       return ALPHA_SPARSE_STATUS_INVALID_VALUE;
+    if (A->format == ALPHA_SPARSE_FORMAT_ELL) { /* src/core/format/destroy_x_ell.c */
+      spmat_ell_s_t *e = (spmat_ell_s_t *)A->mat;
+      free(e->values);
+      free(e->indices);
+      free(e);
+      free(A);
+      return ALPHA_SPARSE_STATUS_SUCCESS;
+    }
     if (A->format == ALPHA_SPARSE_FORMAT_COO) { /* src/core/format/destroy_x_coo.c */
       spmat_coo_s_t *c = (spmat_coo_s_t *)A->mat;
       free(c->values);

@@ -211,6 +211,44 @@ alphasparse_status_t alphasparse_convert_csr(const alphasparse_matrix_t source,
                                              const alphasparse_operation_t operation,
                                              alphasparse_matrix_t *dest);
 
+/* ---- ELL payloads: include/alphasparse/spmat.h:617-636 (column-major, ld slots per row) */
+typedef struct {
+  float *values;
+  ALPHA_INT *indices;
+  ALPHA_INT rows;
+  ALPHA_INT cols;
+  ALPHA_INT ld;
+  float *d_values;
+  ALPHA_INT *d_indices;
+} spmat_ell_s_t;
+
+typedef struct {
+  double *values;
+  ALPHA_INT *indices;
+  ALPHA_INT rows;
+  ALPHA_INT cols;
+  ALPHA_INT ld;
+  double *d_values;
+  ALPHA_INT *d_indices;
+} spmat_ell_d_t;
+
+/* src/core/op_/alphasparse_convert_ell.c:122-143 over src/core/format/convert_ell_x_coo.c:9-84:
+ * COO -> (row, column)-sorted -> ELL with ld = longest row, slot i of row j at [i*rows + j],
+ * padding (value 0, index 0); ld*rows >= 2^31 is refused (INVALID_VALUE; the reference exits).
+ * Only a COO source and NON_TRANSPOSE are supported. */
+alphasparse_status_t alphasparse_convert_ell(const alphasparse_matrix_t source,
+                                             const alphasparse_operation_t operation,
+                                             alphasparse_matrix_t *dest);
+/* include/alphasparse/spapi.h:424-438; src/core/format/alphasparse_x_export_ell.c:5-24 */
+alphasparse_status_t alphasparse_s_export_ell(const alphasparse_matrix_t source,
+                                              alphasparse_index_base_t *indexing, ALPHA_INT *rows,
+                                              ALPHA_INT *cols, ALPHA_INT *width,
+                                              ALPHA_INT **col_indx, float **values);
+alphasparse_status_t alphasparse_d_export_ell(const alphasparse_matrix_t source,
+                                              alphasparse_index_base_t *indexing, ALPHA_INT *rows,
+                                              ALPHA_INT *cols, ALPHA_INT *width,
+                                              ALPHA_INT **col_indx, double **values);
+
 /* ---- handle construction -------------------------------------------------
  * include/alphasparse/spapi.h:140-156; behaviour from
  * src/core/format/alphasparse_x_create_csr.c:7-57: deep copy, indices shifted

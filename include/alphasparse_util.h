@@ -60,6 +60,15 @@ alphasparse_operation_t alpha_args_get_transB(const int argc, const char *argv[]
  * wall clock in microseconds after a device synchronisation. */
 double get_time_us(void);
 
+#ifdef __cplusplus
+/* include/alphasparse/handle.h:336; src/util_cpp/handle.cpp:495-510: mean of the
+ * samples below twice the plain mean (drops warm-up outliers).  C++ callers only. */
+extern "C++" {
+#include <vector>
+}
+double get_avg_time(std::vector<double> times);
+#endif
+
 /* include/alphasparse/util/error.h:9-45 and :139-150 */
 #define alpha_call_exit(func, message)                                      \
   do {                                                                      \

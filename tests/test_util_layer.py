@@ -189,3 +189,31 @@ def test_result_check_and_fill(lib, capfd):
     p = lib.alpha_memalign(100, 64)
     assert p % 64 == 0
     lib.alpha_free(p)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
+def test_coo_to_ell_conversion(lib, dtype):
+    """alphasparse_convert_ell + alphasparse_?_export_ell against the oracle's csr2ell (itself pinned
+    bit for bit against the reference's converter) on shuffled entries."""
+    p = "s" if dtype == np.float32 else "d"
+    T = c_float if p == "s" else c_double
+    a = wl.powerlaw_rmat(9, 60, dtype)
+    perm = np.random.default_rng(6).permutation(a.nnz)
+    rows, cols, vals = orc.csr2coo(a)[perm].copy(), a.col_ind[perm].copy(), a.values[perm].copy()
+    coo, ell = capi.alphasparse_matrix_t(), capi.alphasparse_matrix_t()
+    assert getattr(lib, "alphasparse_%s_create_coo" % p)(byref(coo), 0, a.rows, a.cols, a.nnz, capi.ptr(rows), capi.ptr(cols), capi.ptr(vals)) == 0
+    assert lib.alphasparse_convert_ell(coo, 0, byref(ell)) == 0
+    idx, rr, cc, w = ctypes.c_int(), c_int32(), c_int32(), c_int32()
+    ci, va = c_void_p(), c_void_p()
+    assert getattr(lib, "alphasparse_%s_export_ell" % p)(ell, byref(idx), byref(rr), byref(cc), byref(w), byref(ci), byref(va)) == 0
+    assert (idx.value, rr.value, cc.value, w.value) == (0, a.rows, a.cols, orc.csr2ell_width(a))
+    n = w.value * a.rows
+    got_c = np.ctypeslib.as_array(ctypes.cast(ci, POINTER(c_int32)), (n,)).copy()
+    got_v = np.ctypeslib.as_array(ctypes.cast(va, POINTER(T)), (n,)).copy()
+    ev, ec = orc.csr2ell(a)
+    assert np.array_equal(got_c, ec) and np.array_equal(got_v, ev)
+    other = "d" if p == "s" else "s"
+    assert getattr(lib, "alphasparse_%s_export_ell" % other)(ell, byref(idx), byref(rr), byref(cc), byref(w), byref(ci), byref(va)) == S.ALPHA_SPARSE_STATUS_INVALID_VALUE
+    assert getattr(lib, "alphasparse_%s_export_ell" % p)(coo, byref(idx), byref(rr), byref(cc), byref(w), byref(ci), byref(va)) == S.ALPHA_SPARSE_STATUS_INVALID_VALUE
+    assert lib.alphasparse_convert_ell(ell, 0, byref(capi.alphasparse_matrix_t())) == S.ALPHA_SPARSE_STATUS_INVALID_VALUE
+    assert lib.alphasparse_destroy(coo) == 0 and lib.alphasparse_destroy(ell) == 0
