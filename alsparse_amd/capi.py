@@ -152,6 +152,8 @@ def _per_type(ctype):
         "alphasparse_{s}_mv": [c_int, T, alphasparse_matrix_t, alpha_matrix_descr, _P, T, _P],
         "alphasparse_{s}_mm": [c_int, T, alphasparse_matrix_t, alpha_matrix_descr, c_int, _P, _I, _I, T, _P, _I],
         "host2device_{s}_csr": [alphasparse_matrix_t],
+        "host2device_{s}_coo": [alphasparse_matrix_t],
+        "host2device_{s}_ell": [alphasparse_matrix_t],
         "alphasparse_{s}_mv_dcu": [alphasparse_dcu_handle_t, c_int, PT, alphasparse_matrix_t,
                                    alpha_dcu_matrix_descr_t, _P, PT, _P],
         "alphasparse_dcu_{s}_csrmv_analysis": [alphasparse_dcu_handle_t, c_int, _I, _I, _I,

@@ -205,3 +205,63 @@ alphasparse_status_t alphasparse_convert_ell(const alphasparse_matrix_t source,
   }
 ASAMD_EXPORT_ELL(alphasparse_s_export_ell, float, spmat_ell_s_t, ALPHA_SPARSE_DATATYPE_FLOAT)
 ASAMD_EXPORT_ELL(alphasparse_d_export_ell, double, spmat_ell_d_t, ALPHA_SPARSE_DATATYPE_DOUBLE)
+
+/* ---- device mirrors of COO / ELL handles ------------------------------------
+ * src/core/format/host2device_x_coo.cpp:14-40, host2device_x_ell.cpp:14-33.  The
+ * reference refuses a COO handle whose `ordered` flag is clear (and never sets
+ * it); coomv here takes entries in any order, so the flag is not consulted.  A
+ * second call replaces the mirror. */
+static alphasparse_status_t upload(void **dst, const void *src, size_t bytes) {
+  *dst = NULL;
+  hipError_t e = hipMalloc(dst, bytes ? bytes : 1);
+  if (e == hipSuccess && bytes) e = hipMemcpy(*dst, src, bytes, hipMemcpyHostToDevice);
+  if (e != hipSuccess) {
+    if (*dst) (void)hipFree(*dst);
+    *dst = NULL;
+  }
+  return get_alphasparse_dcu_status_for_hip_status(e);
+}
+
+static alphasparse_status_t host2device_coo(alphasparse_matrix_t mtx, alphasparse_datatype_t dt, size_t vsize) {
+  if (!mtx) return ALPHA_SPARSE_STATUS_INVALID_POINTER;
+  if (mtx->format != ALPHA_SPARSE_FORMAT_COO || mtx->datatype != dt) return ALPHA_SPARSE_STATUS_INVALID_VALUE;
+  spmat_coo_s_t *A = (spmat_coo_s_t *)mtx->mat;
+  if (!A || !A->row_indx || !A->col_indx || !A->values) return ALPHA_SPARSE_STATUS_INVALID_POINTER;
+  (void)hipFree(A->d_rows_indx);
+  (void)hipFree(A->d_cols_indx);
+  (void)hipFree(A->d_values);
+  A->d_rows_indx = A->d_cols_indx = NULL;
+  A->d_values = NULL;
+  const size_t nnz = (size_t)A->nnz;
+  alphasparse_status_t st = upload((void **)&A->d_rows_indx, A->row_indx, nnz * sizeof(ALPHA_INT));
+  if (st == ALPHA_SPARSE_STATUS_SUCCESS) st = upload((void **)&A->d_cols_indx, A->col_indx, nnz * sizeof(ALPHA_INT));
+  if (st == ALPHA_SPARSE_STATUS_SUCCESS) st = upload((void **)&A->d_values, A->values, nnz * vsize);
+  return st;
+}
+alphasparse_status_t host2device_s_coo(alphasparse_matrix_t mtx) {
+  return host2device_coo(mtx, ALPHA_SPARSE_DATATYPE_FLOAT, sizeof(float));
+}
+alphasparse_status_t host2device_d_coo(alphasparse_matrix_t mtx) {
+  return host2device_coo(mtx, ALPHA_SPARSE_DATATYPE_DOUBLE, sizeof(double));
+}
+
+static alphasparse_status_t host2device_ell(alphasparse_matrix_t mtx, alphasparse_datatype_t dt, size_t vsize) {
+  if (!mtx) return ALPHA_SPARSE_STATUS_INVALID_POINTER;
+  if (mtx->format != ALPHA_SPARSE_FORMAT_ELL || mtx->datatype != dt) return ALPHA_SPARSE_STATUS_INVALID_VALUE;
+  spmat_ell_s_t *A = (spmat_ell_s_t *)mtx->mat;
+  if (!A || !A->indices || !A->values) return ALPHA_SPARSE_STATUS_INVALID_POINTER;
+  (void)hipFree(A->d_indices);
+  (void)hipFree(A->d_values);
+  A->d_indices = NULL;
+  A->d_values = NULL;
+  const size_t slots = (size_t)A->ld * (size_t)A->rows;
+  alphasparse_status_t st = upload((void **)&A->d_indices, A->indices, slots * sizeof(ALPHA_INT));
+  if (st == ALPHA_SPARSE_STATUS_SUCCESS) st = upload((void **)&A->d_values, A->values, slots * vsize);
+  return st;
+}
+alphasparse_status_t host2device_s_ell(alphasparse_matrix_t mtx) {
+  return host2device_ell(mtx, ALPHA_SPARSE_DATATYPE_FLOAT, sizeof(float));
+}
+alphasparse_status_t host2device_d_ell(alphasparse_matrix_t mtx) {
+  return host2device_ell(mtx, ALPHA_SPARSE_DATATYPE_DOUBLE, sizeof(double));
+}

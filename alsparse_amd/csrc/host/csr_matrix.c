@@ -45,6 +45,8 @@ alphasparse_status_t alphasparse_destroy(alphasparse_matrix_t A) {
       return ALPHA_SPARSE_STATUS_INVALID_VALUE;
     if (A->format == ALPHA_SPARSE_FORMAT_ELL) { /* src/core/format/destroy_x_ell.c */
       spmat_ell_s_t *e = (spmat_ell_s_t *)A->mat;
+      (void)hipFree(e->d_values);
+      (void)hipFree(e->d_indices);
       free(e->values);
       free(e->indices);
       free(e);
@@ -53,6 +55,9 @@ alphasparse_status_t alphasparse_destroy(alphasparse_matrix_t A) {
     }
     if (A->format == ALPHA_SPARSE_FORMAT_COO) { /* src/core/format/destroy_x_coo.c */
       spmat_coo_s_t *c = (spmat_coo_s_t *)A->mat;
+      (void)hipFree(c->d_values);
+      (void)hipFree(c->d_rows_indx);
+      (void)hipFree(c->d_cols_indx);
       free(c->values);
       free(c->row_indx);
       free(c->col_indx);

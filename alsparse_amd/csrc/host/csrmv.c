@@ -8,6 +8,8 @@
 #define ASAMD_T float
 #define ASAMD_S s
 #define ASAMD_CSR spmat_csr_s_t
+#define ASAMD_COO spmat_coo_s_t
+#define ASAMD_ELL spmat_ell_s_t
 #define ASAMD_DT ALPHA_SPARSE_DATATYPE_FLOAT
 #define ASAMD_KERNEL_CSRMV asamd_s_csrmv
 #define ASAMD_KERNEL_CSRMV_TRANS asamd_s_csrmv_trans
@@ -15,6 +17,8 @@
 #undef ASAMD_T
 #undef ASAMD_S
 #undef ASAMD_CSR
+#undef ASAMD_COO
+#undef ASAMD_ELL
 #undef ASAMD_DT
 #undef ASAMD_KERNEL_CSRMV
 #undef ASAMD_KERNEL_CSRMV_TRANS
@@ -22,6 +26,8 @@
 #define ASAMD_T double
 #define ASAMD_S d
 #define ASAMD_CSR spmat_csr_d_t
+#define ASAMD_COO spmat_coo_d_t
+#define ASAMD_ELL spmat_ell_d_t
 #define ASAMD_DT ALPHA_SPARSE_DATATYPE_DOUBLE
 #define ASAMD_KERNEL_CSRMV asamd_d_csrmv
 #define ASAMD_KERNEL_CSRMV_TRANS asamd_d_csrmv_trans
@@ -29,6 +35,8 @@
 #undef ASAMD_T
 #undef ASAMD_S
 #undef ASAMD_CSR
+#undef ASAMD_COO
+#undef ASAMD_ELL
 #undef ASAMD_DT
 #undef ASAMD_KERNEL_CSRMV
 #undef ASAMD_KERNEL_CSRMV_TRANS

@@ -159,6 +159,13 @@ alphasparse_status_t get_alphasparse_dcu_status_for_hip_status(hipError_t status
  * for it inside a timed loop. */
 alphasparse_status_t host2device_s_csr(alphasparse_matrix_t A);
 alphasparse_status_t host2device_d_csr(alphasparse_matrix_t A);
+/* src/core/format/host2device_x_coo.cpp:14-40, host2device_x_ell.cpp:14-33: device
+ * mirrors of COO / ELL handles, which alphasparse_?_mv_dcu then multiplies with
+ * the coomv / ellmv kernels.  The COO `ordered` flag is not required. */
+alphasparse_status_t host2device_s_coo(alphasparse_matrix_t mtx);
+alphasparse_status_t host2device_d_coo(alphasparse_matrix_t mtx);
+alphasparse_status_t host2device_s_ell(alphasparse_matrix_t mtx);
+alphasparse_status_t host2device_d_ell(alphasparse_matrix_t mtx);
 
 /* ---- handle-based SpMV on device vectors ----------------------------------
  * include/alphasparse/spapi_dcu.h:4441-4457;

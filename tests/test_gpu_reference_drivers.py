@@ -1,5 +1,5 @@
 """The reference's OWN GPU test programs (test/dcu/level2/mv_csr_?_dcu_test.cpp, mv_coo_?, mv_ell_?,
-spmv_csr_s, test/dcu/level3/mm_csr_?_dcu_test.cpp, mm_csr_s_dcu_row_test.cpp), compiled unchanged
+spmv_{csr,coo,ell}_s, test/dcu/level3/mm_csr_?_dcu_test.cpp, mm_csr_s_dcu_row_test.cpp), compiled unchanged
 against this repository's headers and library by `make -C oracle ref_drivers` (into oracle/_ref/,
 where the reference tree is present) and run here on a coordinate file: they read the file, take
 the COO -> CSR / ELL route, call alphasparse_dcu_?_csrmv / _csrmm / _coomv / _ellmv and compare with
@@ -27,6 +27,8 @@ PROGRAMS = {
     "mv_ell_s_dcu_test": [[]],
     "mv_ell_d_dcu_test": [[]],
     "spmv_csr_s_dcu_test": [[]],
+    "spmv_coo_s_dcu_test": [[]],
+    "spmv_ell_s_dcu_test": [[]],
     "mm_csr_s_dcu_test": [["--columns=8", "--layout=C"], ["--columns=70", "--layout=C"]],
     "mm_csr_d_dcu_test": [["--columns=8", "--layout=C"]],
     "mm_csr_s_dcu_row_test": [["--columns=64"]],
