@@ -205,3 +205,40 @@ def test_conversion_pipelines_agree_with_csrmv(gpu, shape, dtype):
             b.free()
     finally:
         da.free()
+
+
+@pytest.mark.parametrize("dtype", DT, ids=IDS)
+def test_handle_api_coo_and_ell(gpu, dtype):
+    """create_coo -> host2device_?_coo -> alphasparse_?_mv_dcu, and convert_ell -> host2device_?_ell ->
+    alphasparse_?_mv_dcu: the route of the reference's spmv_coo / spmv_ell programs."""
+    lib = capi.load()
+    p, T = capi.prefix(dtype), capi.scalar_type(dtype)
+    a = wl.powerlaw_rmat(12, 150, dtype)
+    x, y0 = wl.uniform(a.cols, dtype, 3), wl.uniform(a.rows, dtype, 4)
+    perm = np.random.default_rng(1).permutation(a.nnz)
+    rows, cols, vals = orc.csr2coo(a)[perm].copy(), a.col_ind[perm].copy(), a.values[perm].copy()
+    coo, ell = capi.alphasparse_matrix_t(), capi.alphasparse_matrix_t()
+    assert getattr(lib, "alphasparse_%s_create_coo" % p)(byref(coo), 0, a.rows, a.cols, a.nnz, capi.ptr(rows), capi.ptr(cols), capi.ptr(vals)) == 0
+    assert lib.alphasparse_convert_ell(coo, 0, byref(ell)) == 0
+    al, be = T(2.0), T(3.0)
+    descr = capi.make_descr()
+    mv_dcu = getattr(lib, "alphasparse_%s_mv_dcu" % p)
+    dx = dev(x)
+    ref = orc.csrmv_plain(a, 2.0, x, 3.0, y0)
+    try:
+        for name, h, upload in (("coo", coo, "host2device_%s_coo" % p), ("ell", ell, "host2device_%s_ell" % p)):
+            dy = dev(y0)
+            announce("mv_dcu on a %s handle" % name, np.dtype(dtype).name)
+            assert mv_dcu(gpu.h, 0, byref(al), h, byref(descr), dx.c_ptr(), byref(be), dy.c_ptr()) == capi.ALPHA_SPARSE_STATUS_NOT_INITIALIZED
+            assert getattr(lib, upload)(h) == 0
+            assert getattr(lib, upload)(h) == 0   # a second upload replaces the mirror
+            assert mv_dcu(gpu.h, 0, byref(al), h, byref(descr), dx.c_ptr(), byref(be), dy.c_ptr()) == 0
+            hiprt.synchronize()
+            check(a, 2.0, x, 3.0, y0, dy.to_numpy(), ref, "mv_dcu %s" % name)
+            dy.free()
+        other = "d" if p == "s" else "s"
+        assert getattr(lib, "host2device_%s_coo" % other)(coo) == capi.ALPHA_SPARSE_STATUS_INVALID_VALUE
+        assert getattr(lib, "host2device_%s_ell" % p)(coo) == capi.ALPHA_SPARSE_STATUS_INVALID_VALUE
+    finally:
+        dx.free()
+        assert lib.alphasparse_destroy(coo) == 0 and lib.alphasparse_destroy(ell) == 0
