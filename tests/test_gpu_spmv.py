@@ -242,3 +242,43 @@ def test_handle_api_host_and_device(gpu, dtype):
         assert lib.alphasparse_destroy(A) == 0
         dx.free()
         dy.free()
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_random_structures_every_family(gpu, seed):
+    """Seeded sweep over odd shapes: tiny and lopsided dimensions, mixtures of empty, short and very
+    long rows, both index bases and precisions, through every kernel family (the tiled and ELL copies
+    are forced so that they see shapes their size thresholds would never give them)."""
+    rng = np.random.default_rng(1000 + seed)
+    dtype = [np.float32, np.float64][seed % 2]
+    base = (seed // 2) % 2
+    m = int(rng.choice([1, 2, 63, 64, 65, 257, 1000, 4097]))
+    n = int(rng.choice([1, 2, 255, 256, 257, 1000, 33000, 70001]))
+    kind = seed % 4
+    if kind == 0:
+        lens = rng.integers(0, min(n, 6) + 1, m)
+    elif kind == 1:
+        lens = np.minimum(rng.geometric(0.08, m) - 1, n)
+    elif kind == 2:
+        lens = np.where(rng.random(m) < 0.7, 0, rng.integers(1, min(n, 40) + 1, m))
+    else:
+        lens = np.minimum(rng.zipf(1.5, m), n)
+    if m > 2:
+        lens[rng.integers(0, m)] = min(n, 9000)       # one long row
+    a = csr_from_lengths([int(v) for v in lens], n, dtype, seed=seed + 1, base=base)
+    if a.nnz == 0:
+        a = csr_from_lengths([min(n, 3)] + [0] * (m - 1), n, dtype, seed=seed + 1, base=base)
+    x, y0 = _vectors(a, seed)
+    da = DeviceCsr(a)
+    try:
+        for algo in ("vector", "merge", "scalar", "rowconst", "stream", "tiled", "ell", "auto"):
+            for alpha, beta in ((1.5, 0.0), (-2.0, 0.5)):
+                announce("spmv random", seed, m, n, a.nnz, np.dtype(dtype).name, base, algo, alpha, beta)
+                y = run_plan_csrmv(da, algo, alpha, x, beta, y0)
+                if y is None:
+                    continue
+                check_spmv(a, alpha, x, beta, y0, y, "seed %d %dx%d %s" % (seed, m, n, algo))
+        announce("spmv random api", seed)
+        check_spmv(a, 1.0, x, 1.0, y0, run_csrmv(gpu, da, 1.0, x, 1.0, y0), "seed %d api" % seed)
+    finally:
+        da.free()
