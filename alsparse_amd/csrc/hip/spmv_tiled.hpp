@@ -234,7 +234,9 @@ template <bool Atomic = false, typename T>
 __device__ __forceinline__ void add_rows(T* acc, int r, T v, bool valid) {
   const int lane = threadIdx.x % kWave;
   const int r_up = __builtin_amdgcn_update_dpp(-1, r, 0x138, 0xF, 0xF, false);  // wave_shr:1, lane 0 keeps -1
-  const bool same_as_prev = valid && lane > 0 && r_up == r;
+  // lanes without an entry carry r = -2 - lane: negative, distinct from each other and from the
+  // -1 that lane 0 sees below it, so the comparison alone tells a continued run
+  const bool same_as_prev = r_up == r;
   const uint64_t dup = __builtin_amdgcn_ballot_w64(same_as_prev);
   if (dup == 0) {
     if (valid) rmw<Atomic>(&acc[r], v);
@@ -309,6 +311,7 @@ __global__ __launch_bounds__(kRedThreads) void tiled_reduce_kernel(
     if (active && cb < col_blocks) t = my[cb];
     return t;
   };
+  const int r_none = -2 - lane;  // "no entry": negative and different in every lane
   auto fetch = [&](const TileRange& tr, int q, Batch& bt) {
     const int j = (q % kPerGroup) * kRedUnroll;
     const int left = col_blocks - (q / kPerGroup) * kWave;
@@ -319,12 +322,17 @@ __global__ __launch_bounds__(kRedThreads) void tiled_reduce_kernel(
       const int b = __builtin_amdgcn_readlane(tr.begin, src);
       const int e = j + u < ncb ? __builtin_amdgcn_readlane(tr.end, src) : b;
       bt.len[u] = e - b;
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const int k = b + h * kWave + lane;
+      {
+        const int k = b + lane;
         const bool ok = k < e;
-        bt.v[u][h] = ok ? prod[k] : T(0);
-        bt.r[u][h] = ok ? (int)t_row[k] : -1 - lane;
+        bt.v[u][0] = ok ? prod[k] : T(0);
+        bt.r[u][0] = ok ? (int)t_row[k] : -2 - lane;
+      }
+      if (e - b > kWave) {  // wave-uniform: half of the tiles never need the second load pair
+        const int k = b + kWave + lane;
+        const bool ok = k < e;
+        bt.v[u][1] = ok ? prod[k] : T(0);
+        bt.r[u][1] = ok ? (int)t_row[k] : -2 - lane;
       }
     }
   };
@@ -389,7 +397,7 @@ __global__ __launch_bounds__(kLongThreads) void tiled_long_kernel(
     const int k = k0 + threadIdx.x;
     const bool ok = k < ch.end;
     const T v = ok ? alpha * prod[k] : T(0);
-    const int r = ok ? (int)t_row[k] : -1 - lane;
+    const int r = ok ? (int)t_row[k] : -2 - lane;
     add_rows<true>(yb, r, v, ok);
   }
 }
