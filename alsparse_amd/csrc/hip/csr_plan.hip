@@ -240,6 +240,9 @@ static bool tiled_eligible(const asamd_csr_stats& st, bool force) {
   const int64_t cb = ((int64_t)st.n + TileDims<T>::cols - 1) / TileDims<T>::cols;
   const int64_t rb = ((int64_t)st.m + TileDims<T>::rows - 1) / TileDims<T>::rows;
   if (!st.trusted || 2 * cb > kTiledMaxColBlocks || cb * rb > kTiledMaxTiles / 2) return false;
+  // entry positions of the tiled copy are 32-bit and the kernels step past a range's end by up to
+  // a workgroup's stride before they test it
+  if ((int64_t)st.nnz > (int64_t)0x7fffffff - (1 << 16)) return false;
   // worth a try only when x cannot live in an XCD's 4 MiB L2 and the matrix is large
   return force || ((int64_t)st.n * (int64_t)sizeof(T) >= ((int64_t)8 << 20) && st.nnz >= (1 << 22));
 }
