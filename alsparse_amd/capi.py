@@ -239,6 +239,8 @@ _COMMON = {
     "asamd_csr2coo": [_P, _P, _I, _I, _P, _I],
     "asamd_csr2ell_width": [_P, _I, _P, POINTER(_I)],
     "asamd_warmup": [_P],
+    "asamd_handle_set_stream": [_P, _P],
+    "asamd_handle_get_stream": [_P],
     "asamd_copy_bytes": [_P, _P, _P, c_size_t],
     "asamd_analysis_stats": [_P],
     "asamd_analysis_transpose_stats": [_P],
@@ -255,7 +257,7 @@ def prototypes():
     return out
 
 
-_RESTYPE = {"asamd_csr_plan_destroy": None, "alpha_malloc": c_void_p, "alpha_memalign": c_void_p, "alpha_free": None,
+_RESTYPE = {"asamd_csr_plan_destroy": None, "asamd_handle_get_stream": c_void_p, "alpha_malloc": c_void_p, "alpha_memalign": c_void_p, "alpha_free": None,
             "alpha_fill_random_s": None, "alpha_fill_random_d": None, "alpha_read_coo": None, "alpha_read_coo_d": None,
             "args_help": None, "args_get_if_check": c_bool, "args_get_data_file": ctypes.c_char_p,
             "args_get_data_fileA": ctypes.c_char_p, "args_get_data_fileB": ctypes.c_char_p,

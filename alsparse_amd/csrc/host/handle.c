@@ -154,6 +154,18 @@ alphasparse_status_t alphasparse_dcu_destroy_mat_info(alphasparse_dcu_mat_info_t
   return ALPHA_SPARSE_STATUS_SUCCESS;
 }
 
+/* The stream lives in a public struct field (handle->stream), which C callers set themselves as
+ * with the reference; these two are for bindings that cannot see the struct layout. */
+int asamd_handle_set_stream(void *handle, hipStream_t stream) {
+  if (!handle) return (int)hipErrorInvalidValue;
+  ((alphasparse_dcu_handle_t)handle)->stream = stream;
+  return (int)hipSuccess;
+}
+
+hipStream_t asamd_handle_get_stream(void *handle) {
+  return handle ? ((alphasparse_dcu_handle_t)handle)->stream : NULL;
+}
+
 int asamd_env_algo(void) {
   const char *e = getenv("ALSPARSE_AMD_SPMV_ALGO");
   if (!e || !*e) return ASAMD_SPMV_AUTO;

@@ -219,6 +219,13 @@ int asamd_analysis_set_algo(const void *key, int32_t algo);
  * known size; no reference counterpart. */
 int asamd_copy_bytes(hipStream_t stream, void *dst, const void *src, size_t nbytes);
 
+/* handle->stream for callers that cannot see the handle struct (language bindings); C callers assign
+ * the field, as with the reference.  `handle` is an alphasparse_dcu_handle_t.  Every multiply that
+ * runs from an explicit analysis only launches kernels on that stream, so it can be captured into
+ * a HIP graph. */
+int asamd_handle_set_stream(void *handle, hipStream_t stream);
+hipStream_t asamd_handle_get_stream(void *handle);
+
 /* Empty kernel; forces code-object load (src/util_cpp/handle.cpp:19, :113). */
 int asamd_warmup(hipStream_t stream);
 

@@ -1,0 +1,140 @@
+"""An analysed csrmv only launches kernels on the handle's stream (no allocation, no memset, no
+synchronisation), so it can be recorded into a HIP graph and replayed.  Every replay is checked
+against the eager result, with eager work and synchronisations between replays."""
+import ctypes
+from ctypes import byref, c_void_p
+
+import numpy as np
+import pytest
+
+from alsparse_amd import capi, hiprt, workloads as wl
+from helpers import ALGOS, TOL, DeviceCsr, announce, check_spmv
+from oracle import oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("shape", ["powerlaw_merge", "laplace_ell", "uniform_tiled", "transposed"])
+def test_analysed_csrmv_replays_from_a_hip_graph(gpu, shape):
+    lib, hip = capi.load(), hiprt.lib()
+    dtype = np.float64 if shape == "laplace_ell" else np.float32
+    if shape == "powerlaw_merge":
+        a = wl.powerlaw_rmat(15, 200000, dtype)
+    elif shape == "laplace_ell":
+        a = wl.laplace2d(700, 600, dtype)
+    else:
+        a = wl.uniform_rows(1 << 19, 1 << 22, 12, dtype)   # x = 16 MiB: the tiled copy is built and timed
+    trans = capi.ALPHA_SPARSE_OPERATION_TRANSPOSE if shape == "transposed" else 0
+    xlen, ylen = (a.rows, a.cols) if trans else (a.cols, a.rows)
+    x, y0 = wl.uniform(xlen, dtype, 3), wl.uniform(ylen, dtype, 4)
+    T, p = capi.scalar_type(dtype), capi.prefix(dtype)
+    da = DeviceCsr(a)
+    dx, dy = hiprt.DeviceArray.from_numpy(x), hiprt.DeviceArray.from_numpy(y0)
+    stream, graph, gexec = c_void_p(), c_void_p(), c_void_p()
+    hiprt.check(hip.hipStreamCreate(byref(stream)), "hipStreamCreate")
+    h = capi.Handle()
+    info = capi.alphasparse_dcu_mat_info_t()
+    assert lib.alphasparse_dcu_create_mat_info(byref(info)) == 0
+    descr = capi.make_descr()
+    al, be = T(1.25), T(0.5)
+    csrmv = getattr(lib, "alphasparse_dcu_%s_csrmv" % p)
+
+    def multiply():
+        return csrmv(h.h, trans, a.rows, a.cols, a.nnz, byref(al), byref(descr), da.val.c_ptr(), da.row_ptr.c_ptr(),
+                     da.col.c_ptr(), info, dx.c_ptr(), byref(be), dy.c_ptr())
+    try:
+        assert lib.asamd_handle_set_stream(h.h, stream) == 0
+        announce("graph capture: analysis", shape)
+        assert getattr(lib, "alphasparse_dcu_%s_csrmv_analysis" % p)(
+            h.h, trans, a.rows, a.cols, a.nnz, byref(descr), da.val.c_ptr(), da.row_ptr.c_ptr(), da.col.c_ptr(), info) == 0
+        stats = lib.asamd_analysis_stats(info).contents
+        announce("graph capture: analysis chose", capi.ALGO_NAMES[stats.algo])
+        assert multiply() == 0                                   # eager, on the stream
+        hiprt.check(hip.hipStreamSynchronize(stream), "sync")
+        eager = dy.to_numpy()
+        if trans:
+            ref = orc.csrmv_trans_plain(a, 1.25, x, 0.5, y0)
+            err = orc.csrmv_err(orc.transpose(a), 1.25, x, 0.5, y0, eager, ref)
+            assert err.zero_den_mismatch == 0 and err.full <= TOL[a.dtype], err
+        else:
+            check_spmv(a, 1.25, x, 0.5, y0, eager, "eager " + shape)
+        announce("graph capture: record", shape)
+        hiprt.check(hip.hipStreamBeginCapture(stream, 0), "hipStreamBeginCapture")
+        st = multiply()
+        hiprt.check(hip.hipStreamEndCapture(stream, byref(graph)), "hipStreamEndCapture")
+        assert st == 0
+        hiprt.check(hip.hipGraphInstantiate(byref(gexec), graph, None, None, ctypes.c_size_t(0)), "hipGraphInstantiate")
+        for replay in range(3):
+            dy.copy_from(y0)                                     # eager work between the replays
+            hiprt.synchronize()
+            announce("graph capture: replay", shape, replay)
+            hiprt.check(hip.hipGraphLaunch(gexec, stream), "hipGraphLaunch")
+            hiprt.check(hip.hipStreamSynchronize(stream), "sync")
+            got = dy.to_numpy()
+            if stats.tiled_built:  # long tiles reach y through atomics: order-dependent in the last bits
+                check_spmv(a, 1.25, x, 0.5, y0, got, "replay %d" % replay)
+            else:
+                assert np.array_equal(got, eager), "replay %d differs from the eager result" % replay
+    finally:
+        if gexec:
+            hip.hipGraphExecDestroy(gexec)
+        if graph:
+            hip.hipGraphDestroy(graph)
+        lib.alphasparse_dcu_destroy_mat_info(info)
+        h.close()
+        hip.hipStreamDestroy(stream)
+        for d in (dx, dy):
+            d.free()
+        da.free()
+
+
+@pytest.mark.parametrize("algo", ["vector", "rowconst", "merge", "scalar", "tiled", "stream", "ell"])
+def test_every_kernel_family_replays_from_a_hip_graph(gpu, algo):
+    """The thin kernel ABI with a forced family, recorded on a caller's stream."""
+    lib, hip = capi.load(), hiprt.lib()
+    a = wl.uniform_rows(60000, 50000, 16, np.float32)
+    x, y0 = wl.uniform(a.cols, a.dtype, 5), wl.uniform(a.rows, a.dtype, 6)
+    da = DeviceCsr(a)
+    dx, dy = hiprt.DeviceArray.from_numpy(x), hiprt.DeviceArray.from_numpy(y0)
+    stream, graph, gexec, plan = c_void_p(), c_void_p(), c_void_p(), c_void_p()
+    hiprt.check(hip.hipStreamCreate(byref(stream)), "hipStreamCreate")
+    try:
+        announce("graph capture: plan", algo)
+        assert lib.asamd_csr_plan_create(stream, a.rows, a.cols, a.nnz, da.row_ptr.c_ptr(), da.col.c_ptr(),
+                                         da.val.c_ptr(), a.base, a.dtype.itemsize, 2, byref(plan)) == 0
+        assert lib.asamd_csr_plan_set_algo(plan, ALGOS[algo]) == 0, "this matrix can run every family"
+
+        def multiply():
+            return lib.asamd_s_csrmv(stream, plan, ctypes.c_float(-0.75), da.val.c_ptr(), da.row_ptr.c_ptr(),
+                                     da.col.c_ptr(), dx.c_ptr(), ctypes.c_float(2.0), dy.c_ptr())
+        assert multiply() == 0
+        hiprt.check(hip.hipStreamSynchronize(stream), "sync")
+        eager = dy.to_numpy()
+        check_spmv(a, -0.75, x, 2.0, y0, eager, "eager " + algo)
+        hiprt.check(hip.hipStreamBeginCapture(stream, 0), "hipStreamBeginCapture")
+        st = multiply()
+        hiprt.check(hip.hipStreamEndCapture(stream, byref(graph)), "hipStreamEndCapture")
+        assert st == 0
+        hiprt.check(hip.hipGraphInstantiate(byref(gexec), graph, None, None, ctypes.c_size_t(0)), "hipGraphInstantiate")
+        for replay in range(3):
+            dy.copy_from(y0)
+            hiprt.synchronize()
+            announce("graph capture: replay", algo, replay)
+            hiprt.check(hip.hipGraphLaunch(gexec, stream), "hipGraphLaunch")
+            hiprt.check(hip.hipStreamSynchronize(stream), "sync")
+            got = dy.to_numpy()
+            if algo == "tiled":   # long tiles reach y through atomics: order-dependent in the last bits
+                check_spmv(a, -0.75, x, 2.0, y0, got, "replay %d" % replay)
+            else:
+                assert np.array_equal(got, eager), "replay %d differs from the eager result" % replay
+    finally:
+        if gexec:
+            hip.hipGraphExecDestroy(gexec)
+        if graph:
+            hip.hipGraphDestroy(graph)
+        if plan:
+            lib.asamd_csr_plan_destroy(plan)
+        hip.hipStreamDestroy(stream)
+        for d in (dx, dy):
+            d.free()
+        da.free()
