@@ -139,8 +139,27 @@ class asamd_dense_strides(Structure):
 _I, _P = c_int32, c_void_p
 
 
+class ALPHA_Complex8(Structure):  # include/alphasparse/types.h:42-47 of the reference
+    _fields_ = [("real", c_float), ("imag", c_float)]
+
+    def __init__(self, v=0):
+        v = complex(v)
+        super().__init__(v.real, v.imag)
+
+
+class ALPHA_Complex16(Structure):  # include/alphasparse/types.h:50-55
+    _fields_ = [("real", c_double), ("imag", c_double)]
+
+    def __init__(self, v=0):
+        v = complex(v)
+        super().__init__(v.real, v.imag)
+
+
+ASAMD_DTYPE_FLOAT, ASAMD_DTYPE_DOUBLE, ASAMD_DTYPE_FLOAT_COMPLEX, ASAMD_DTYPE_DOUBLE_COMPLEX = range(4)
+
+
 def _per_type(ctype):
-    """Prototypes that exist once per value type; {T} is the scalar ctype."""
+    """Public entry points that exist once per value type (s, d, c, z); T is the scalar ctype."""
     T, PT = ctype, POINTER(ctype)
     return {
         "alphasparse_{s}_create_csr": [POINTER(alphasparse_matrix_t), c_int, _I, _I, _P, _P, _P, _P],
@@ -168,12 +187,32 @@ def _per_type(ctype):
                                       _P, _P, _P, _P, PT, _P],
         "alphasparse_dcu_{s}_ellmv": [alphasparse_dcu_handle_t, c_int, _I, _I, PT, alpha_dcu_matrix_descr_t,
                                       _P, _P, _I, _P, PT, _P],
-        # thin kernel ABI
+    }
+
+
+def _per_real_type(ctype):
+    """Thin kernel ABI of the real value types."""
+    T = ctype
+    return {
         "asamd_{s}_csrmv": [_P, _P, T, _P, _P, _P, _P, T, _P],
         "asamd_{s}_csrmv_trans": [_P, _P, T, _P, _P, _P, _P, T, _P],
         "asamd_{s}_ellmv": [_P, _I, _I, T, _P, _P, _I, _I, _P, T, _P],
         "asamd_{s}_coomv": [_P, _I, _I, c_int64, T, _P, _P, _P, _I, _P, T, _P],
         "asamd_{s}_csrmm": [_P, _I, _I, _I, _I, T, _P, _P, _P, _I, _P, T, _P, POINTER(asamd_dense_strides)],
+        "asamd_{s}_csrmm_ws": [_P, _I, _I, _I, _I, T, _P, _P, _P, _I, _P, T, _P, POINTER(asamd_dense_strides), _P,
+                               c_size_t],
+        "asamd_{s}_csr2ell": [_P, _I, _P, _P, _P, _I, _I, _I, _P, _P],
+    }
+
+
+def _per_complex_type(ctype):
+    """Prototypes that exist for the complex value types only; T is passed by value."""
+    T = ctype
+    return {
+        # thin kernel ABI
+        "asamd_{s}_csrmv_op": [_P, _P, _I, T, _P, _P, _P, _P, T, _P],
+        "asamd_{s}_ellmv": [_P, _I, _I, T, _P, _P, _I, _I, _P, T, _P],
+        "asamd_{s}_coomv": [_P, _I, _I, c_int64, T, _P, _P, _P, _I, _P, T, _P],
         "asamd_{s}_csrmm_ws": [_P, _I, _I, _I, _I, T, _P, _P, _P, _I, _P, T, _P, POINTER(asamd_dense_strides), _P,
                                c_size_t],
         "asamd_{s}_csr2ell": [_P, _I, _P, _P, _P, _I, _I, _I, _P, _P],
@@ -190,6 +229,12 @@ _COMMON = {
     "alpha_free": [_P],
     "alpha_fill_random_s": [_P, ctypes.c_uint, c_size_t],
     "alpha_fill_random_d": [_P, ctypes.c_uint, c_size_t],
+    "alpha_fill_random_c": [_P, ctypes.c_uint, c_size_t],
+    "alpha_fill_random_z": [_P, ctypes.c_uint, c_size_t],
+    "alpha_read_coo_c": [ctypes.c_char_p, POINTER(_I), POINTER(_I), POINTER(_I), POINTER(_P), POINTER(_P), POINTER(_P)],
+    "alpha_read_coo_z": [ctypes.c_char_p, POINTER(_I), POINTER(_I), POINTER(_I), POINTER(_P), POINTER(_P), POINTER(_P)],
+    "check_c": [_P, c_size_t, _P, c_size_t],
+    "check_z": [_P, c_size_t, _P, c_size_t],
     "alpha_read_coo": [ctypes.c_char_p, POINTER(_I), POINTER(_I), POINTER(_I), POINTER(_P), POINTER(_P), POINTER(_P)],
     "alpha_read_coo_d": [ctypes.c_char_p, POINTER(_I), POINTER(_I), POINTER(_I), POINTER(_P), POINTER(_P), POINTER(_P)],
     "check_s": [_P, c_size_t, _P, c_size_t],
@@ -229,6 +274,8 @@ _COMMON = {
                                       alpha_dcu_matrix_descr_t, POINTER(_I)],
     # thin kernel ABI
     "asamd_csr_plan_create": [_P, _I, _I, _I, _P, _P, _P, _I, _I, _I, POINTER(_P)],
+    "asamd_csr_plan_create_dtype": [_P, _I, _I, _I, _P, _P, _P, _I, _I, _I, POINTER(_P)],
+    "asamd_csr_plan_build_conj_transpose": [_P, _P, _P, _P, _P],
     "asamd_csr_plan_destroy": [_P],
     "asamd_csr_plan_stats": [_P],
     "asamd_csr_plan_set_algo": [_P, _I],
@@ -251,14 +298,17 @@ _COMMON = {
 def prototypes():
     """name -> argtypes for every symbol the public headers declare."""
     out = dict(_COMMON)
-    for s, ct in (("s", c_float), ("d", c_double)):
+    for s, ct in (("s", c_float), ("d", c_double), ("c", ALPHA_Complex8), ("z", ALPHA_Complex16)):
         for k, v in _per_type(ct).items():
+            out[k.format(s=s)] = v
+        for k, v in (_per_real_type(ct) if s in "sd" else _per_complex_type(ct)).items():
             out[k.format(s=s)] = v
     return out
 
 
 _RESTYPE = {"asamd_csr_plan_destroy": None, "asamd_handle_get_stream": c_void_p, "alpha_malloc": c_void_p, "alpha_memalign": c_void_p, "alpha_free": None,
             "alpha_fill_random_s": None, "alpha_fill_random_d": None, "alpha_read_coo": None, "alpha_read_coo_d": None,
+            "alpha_fill_random_c": None, "alpha_fill_random_z": None, "alpha_read_coo_c": None, "alpha_read_coo_z": None,
             "args_help": None, "args_get_if_check": c_bool, "args_get_data_file": ctypes.c_char_p,
             "args_get_data_fileA": ctypes.c_char_p, "args_get_data_fileB": ctypes.c_char_p,
             "alpha_args_get_matrix_descrA": alpha_matrix_descr, "alpha_args_get_matrix_descrB": alpha_matrix_descr,
@@ -305,12 +355,19 @@ def ptr(x):
 
 def scalar_type(dtype):
     import numpy as np
-    return c_float if np.dtype(dtype) == np.float32 else c_double
+    return {np.dtype(np.float32): c_float, np.dtype(np.float64): c_double, np.dtype(np.complex64): ALPHA_Complex8,
+            np.dtype(np.complex128): ALPHA_Complex16}[np.dtype(dtype)]
 
 
 def prefix(dtype):
     import numpy as np
-    return "s" if np.dtype(dtype) == np.float32 else "d"
+    return {np.dtype(np.float32): "s", np.dtype(np.float64): "d", np.dtype(np.complex64): "c",
+            np.dtype(np.complex128): "z"}[np.dtype(dtype)]
+
+
+def dtype_tag(dtype):
+    """enum asamd_dtype / alphasparse_datatype_t of a numpy dtype."""
+    return "sdcz".index(prefix(dtype))
 
 
 class Handle:

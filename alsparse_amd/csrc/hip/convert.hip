@@ -131,15 +131,16 @@ extern "C" int asamd_csr2ell_width(hipStream_t stream, int32_t m, const int32_t*
 // than the LDS window are read from global memory directly.
 // ---------------------------------------------------------------------------
 constexpr int kEllRows = 256;
-constexpr int kEllWindow = 4096;  // staged entries per workgroup pass
+constexpr int kEllWindow = 4096;  // staged entries per workgroup pass (half of it for 16-byte values)
 
 template <typename T>
 __global__ __launch_bounds__(kEllRows) void csr2ell_kernel(
     int m, const T* __restrict__ val, const int* __restrict__ row_ptr,
     const int* __restrict__ col_ind, int csr_base, int ell_base, int width,
     T* __restrict__ ell_val, int* __restrict__ ell_col) {
-  __shared__ T s_val[kEllWindow];
-  __shared__ int s_col[kEllWindow];
+  constexpr int kWindow = sizeof(T) > 8 ? kEllWindow / 2 : kEllWindow;  // at most 32 KiB of staged values
+  __shared__ T s_val[kWindow];
+  __shared__ int s_col[kWindow];
   const int64_t row_first = (int64_t)blockIdx.x * kEllRows;
   const int64_t row = row_first + threadIdx.x;
   int64_t row_last = row_first + kEllRows;
@@ -151,7 +152,7 @@ __global__ __launch_bounds__(kEllRows) void csr2ell_kernel(
     my_begin = (int64_t)row_ptr[row] - csr_base;
     my_end = (int64_t)row_ptr[row + 1] - csr_base;
   }
-  const bool staged = blk_end - blk_begin <= kEllWindow;  // workgroup-uniform
+  const bool staged = blk_end - blk_begin <= kWindow;  // workgroup-uniform
   if (staged) {
     for (int64_t k = blk_begin + threadIdx.x; k < blk_end; k += kEllRows) {
       s_val[k - blk_begin] = val[k];
@@ -183,6 +184,7 @@ template <typename T>
 static int csr2ell_impl(hipStream_t stream, int m, const T* val, const int* rp, const int* ci,
                         int csr_base, int ell_base, int width, T* ell_val, int* ell_col) {
   if (!val || !rp || !ci || !ell_val || !ell_col || m <= 0 || width < 0) return hipErrorInvalidValue;
+  if (((uintptr_t)val | (uintptr_t)ell_val) % alignof(T)) return hipErrorInvalidValue;
   if (width == 0) return hipSuccess;
   const unsigned grid = (unsigned)(((int64_t)m + kEllRows - 1) / kEllRows);
   csr2ell_kernel<T><<<grid, kEllRows, 0, stream>>>(m, val, rp, ci, csr_base, ell_base, width, ell_val,
@@ -202,4 +204,21 @@ extern "C" int asamd_d_csr2ell(hipStream_t stream, int32_t m, const double* val,
                                int32_t ell_base, int32_t width, double* ell_val, int32_t* ell_col) {
   return csr2ell_impl<double>(stream, m, val, row_ptr, col_ind, csr_base, ell_base, width, ell_val,
                               ell_col);
+}
+
+// Complex values are copied bit for bit and the padding is all-zero bits, so the 8-byte
+// complex type runs the fp64 instantiation; the 16-byte one has its own.
+extern "C" int asamd_c_csr2ell(hipStream_t stream, int32_t m, const asamd_complex8* val,
+                               const int32_t* row_ptr, const int32_t* col_ind, int32_t csr_base,
+                               int32_t ell_base, int32_t width, asamd_complex8* ell_val, int32_t* ell_col) {
+  return csr2ell_impl<double>(stream, m, (const double*)val, row_ptr, col_ind, csr_base, ell_base, width,
+                              (double*)ell_val, ell_col);
+}
+
+extern "C" int asamd_z_csr2ell(hipStream_t stream, int32_t m, const asamd_complex16* val,
+                               const int32_t* row_ptr, const int32_t* col_ind, int32_t csr_base,
+                               int32_t ell_base, int32_t width, asamd_complex16* ell_val, int32_t* ell_col) {
+  using T = asamd::Cx<double>;
+  return csr2ell_impl<T>(stream, m, (const T*)val, row_ptr, col_ind, csr_base, ell_base, width, (T*)ell_val,
+                         ell_col);
 }

@@ -13,6 +13,7 @@
 #include <algorithm>
 #include <cstdlib>
 #include <new>
+#include <type_traits>
 #include <vector>
 
 #include "alsparse_amd_kernels.h"
@@ -83,7 +84,8 @@ struct asamd_csr_plan {
   asamd_csr_stats st;
   int auto_algo;
   int auto_width;
-  int val_size;
+  int dtype;          // ASAMD_DTYPE_*: element type of the values
+  int val_size;       // bytes per value
   int merge_ipt;      // items per thread of the merge-path kernel (4, 8 or 16)
   int* d_block_row;   // merge-path coordinates, merge_blocks + 1 ints
   int* d_carry_row;   // merge_blocks ints
@@ -104,13 +106,39 @@ struct asamd_csr_plan {
   // ELL copy (trusted plans of short, nearly equal rows)
   void* d_eval;               // ell_width * m values, column-major
   int* d_ecol;                // ... and zero-based columns
-  // CSR copy of the transpose (trusted plans, on request) and its own plan
-  asamd_csr_plan* tr_plan;
-  int* d_tr_row_ptr;          // n + 1
-  int* d_tr_col;              // nnz zero-based rows of A
-  void* d_tr_val;             // nnz values
-  bool lazy_transpose;        // build the copy on the first transposed multiply
+  // CSR copies of the transpose [0] and of the conjugate transpose [1] (trusted plans, on
+  // request), each with a plan of its own
+  struct TransCopy {
+    asamd_csr_plan* plan;
+    int* d_row_ptr;           // n + 1
+    int* d_col;               // nnz zero-based rows of A
+    void* d_val;              // nnz values (conjugated in copy [1])
+  } tr[2];
+  bool lazy_transpose;        // build a copy on the first transposed multiply
 };
+
+// element type <-> tag
+template <typename T> struct DtypeOf;
+template <> struct DtypeOf<float> { static constexpr int value = ASAMD_DTYPE_FLOAT; };
+template <> struct DtypeOf<double> { static constexpr int value = ASAMD_DTYPE_DOUBLE; };
+template <> struct DtypeOf<Cx<float>> { static constexpr int value = ASAMD_DTYPE_FLOAT_COMPLEX; };
+template <> struct DtypeOf<Cx<double>> { static constexpr int value = ASAMD_DTYPE_DOUBLE_COMPLEX; };
+template <typename T>
+constexpr bool kIsReal = std::is_floating_point<T>::value;
+
+// calls f with a null pointer of the plan's element type: f's parameter type names T
+template <typename F>
+static hipError_t by_dtype(int dtype, F&& f) {
+  switch (dtype) {
+    case ASAMD_DTYPE_FLOAT: return f((float*)nullptr);
+    case ASAMD_DTYPE_DOUBLE: return f((double*)nullptr);
+    case ASAMD_DTYPE_FLOAT_COMPLEX: return f((Cx<float>*)nullptr);
+    case ASAMD_DTYPE_DOUBLE_COMPLEX: return f((Cx<double>*)nullptr);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+static bool is_complex(const asamd_csr_plan* p) { return p->dtype >= ASAMD_DTYPE_FLOAT_COMPLEX; }
 
 static int width_for_mean(double mean) {
   // lanes per row from the mean row length; same break points as the
@@ -123,16 +151,19 @@ static int width_for_mean(double mean) {
   return 64;
 }
 
-static bool rowconst_ok(const asamd_csr_stats& st) {
+static bool rowconst_ok(const asamd_csr_plan* p) {
+  const asamd_csr_stats& st = p->st;
   const int L = st.const_len;
-  return st.trusted && st.first_offset == 0 &&
+  // the kernel loads four values as 128-bit pieces: real element types only
+  return !is_complex(p) && st.trusted && st.first_offset == 0 &&
          (L == 4 || L == 8 || L == 16 || L == 32 || L == 64 || L == 128 || L == 256);
 }
 
 // The LDS-staged row-block kernel sizes its staging area for rows of at most
 // kStreamMaxLen entries; the bound comes from the analysis, so the structure
 // must be promised fixed.
-static bool stream_ok(const asamd_csr_stats& st) {
+static bool stream_ok(const asamd_csr_plan* p) {
+  const asamd_csr_stats& st = p->st;
   return st.trusted && st.max_len <= kStreamMaxLen && st.max_len >= 1;
 }
 
@@ -141,9 +172,9 @@ static void choose_algo(asamd_csr_plan* p) {
   const double mean = st.m > 0 ? (double)st.nnz / st.m : 0.0;
   const int w = width_for_mean(mean);
   p->auto_width = w;
-  if (rowconst_ok(st)) {
+  if (rowconst_ok(p)) {
     p->auto_algo = ASAMD_SPMV_ROWCONST;
-  } else if (stream_ok(st)) {
+  } else if (stream_ok(p)) {
     p->auto_algo = ASAMD_SPMV_STREAM;
   } else if ((int64_t)st.max_len <= (int64_t)w * 16 && mean >= 6.0) {
     // regular rows: a lane group per row wastes little and needs no LDS
@@ -186,16 +217,14 @@ static void free_ell(asamd_csr_plan* p) {
   p->st.ell_built = 0;
 }
 
-static void free_transpose(asamd_csr_plan* p) {
-  if (p->tr_plan) asamd_csr_plan_destroy(p->tr_plan);
-  p->tr_plan = nullptr;
-  if (p->d_tr_row_ptr) (void)hipFree(p->d_tr_row_ptr);
-  if (p->d_tr_col) (void)hipFree(p->d_tr_col);
-  if (p->d_tr_val) (void)hipFree(p->d_tr_val);
-  p->d_tr_row_ptr = nullptr;
-  p->d_tr_col = nullptr;
-  p->d_tr_val = nullptr;
-  p->st.transpose_built = 0;
+static void free_transpose(asamd_csr_plan* p, int which) {
+  asamd_csr_plan::TransCopy& t = p->tr[which];
+  if (t.plan) asamd_csr_plan_destroy(t.plan);
+  if (t.d_row_ptr) (void)hipFree(t.d_row_ptr);
+  if (t.d_col) (void)hipFree(t.d_col);
+  if (t.d_val) (void)hipFree(t.d_val);
+  t = asamd_csr_plan::TransCopy{nullptr, nullptr, nullptr, nullptr};
+  p->st.transpose_built &= ~(1 << which);
 }
 
 // An ELL copy pays when rows are short and padding them to the longest costs
@@ -216,12 +245,16 @@ static hipError_t build_ell(hipStream_t stream, asamd_csr_plan* p, const int* ro
   hipError_t e = hipMalloc(&p->d_eval, slots * sizeof(T));
   if (e == hipSuccess) e = hipMalloc(&p->d_ecol, slots * sizeof(int));
   if (e == hipSuccess) {
+    // the conversion copies values bit for bit and pads with zero bits: only the element size matters
     if constexpr (sizeof(T) == 4)
-      e = (hipError_t)asamd_s_csr2ell(stream, st.m, val, row_ptr, col_ind, st.base, 0, st.max_len, (float*)p->d_eval,
-                                      p->d_ecol);
+      e = (hipError_t)asamd_s_csr2ell(stream, st.m, (const float*)val, row_ptr, col_ind, st.base, 0, st.max_len,
+                                      (float*)p->d_eval, p->d_ecol);
+    else if constexpr (sizeof(T) == 8)
+      e = (hipError_t)asamd_d_csr2ell(stream, st.m, (const double*)val, row_ptr, col_ind, st.base, 0, st.max_len,
+                                      (double*)p->d_eval, p->d_ecol);
     else
-      e = (hipError_t)asamd_d_csr2ell(stream, st.m, val, row_ptr, col_ind, st.base, 0, st.max_len, (double*)p->d_eval,
-                                      p->d_ecol);
+      e = (hipError_t)asamd_z_csr2ell(stream, st.m, (const asamd_complex16*)val, row_ptr, col_ind, st.base, 0,
+                                      st.max_len, (asamd_complex16*)p->d_eval, p->d_ecol);
   }
   if (e == hipSuccess) e = hipStreamSynchronize(stream);
   if (e != hipSuccess) {
@@ -235,6 +268,9 @@ static hipError_t build_ell(hipStream_t stream, asamd_csr_plan* p, const int* ro
 
 template <typename T>
 static bool tiled_eligible(const asamd_csr_stats& st, bool force) {
+  if constexpr (!kIsReal<T>) {
+    return false;  // the tiled kernels are written for real element types
+  } else {
   // full-width block counts; the equal-entry cut (at most twice as many blocks
   // per dimension) is checked again once it is known
   const int64_t cb = ((int64_t)st.n + TileDims<T>::cols - 1) / TileDims<T>::cols;
@@ -245,6 +281,7 @@ static bool tiled_eligible(const asamd_csr_stats& st, bool force) {
   if ((int64_t)st.nnz > (int64_t)0x7fffffff - (1 << 16)) return false;
   // worth a try only when x cannot live in an XCD's 4 MiB L2 and the matrix is large
   return force || ((int64_t)st.n * (int64_t)sizeof(T) >= ((int64_t)8 << 20) && st.nnz >= (1 << 22));
+  }
 }
 
 // Cuts groups [0, groups) with cumulative entry counts off[0..groups] into
@@ -495,12 +532,14 @@ static hipError_t tune_copies(hipStream_t stream, asamd_csr_plan* p, const int* 
   return hipSuccess;
 }
 
-extern "C" int asamd_csr_plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t nnz,
-                                     const int32_t* row_ptr, const int32_t* col_ind,
-                                     const void* val, int32_t base, int32_t val_size,
-                                     int32_t trusted, asamd_csr_plan** out) {
-  if (!out || !row_ptr || m <= 0 || nnz < 0 || (val_size != 4 && val_size != 8))
+static hipError_t plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t nnz, const int32_t* row_ptr,
+                              const int32_t* col_ind, const void* val, int32_t base, int32_t dtype,
+                              int32_t trusted, asamd_csr_plan** out) {
+  if (!out || !row_ptr || m <= 0 || nnz < 0 || dtype < ASAMD_DTYPE_FLOAT || dtype > ASAMD_DTYPE_DOUBLE_COMPLEX)
     return hipErrorInvalidValue;
+  static const int kValSize[4] = {4, 8, 8, 16};
+  const int val_size = kValSize[dtype];
+  if (val && (uintptr_t)val % (size_t)val_size) return hipErrorInvalidValue;
   asamd_csr_plan* p = new (std::nothrow) asamd_csr_plan();
   if (!p) return hipErrorOutOfMemory;
   p->st.m = m;
@@ -508,6 +547,7 @@ extern "C" int asamd_csr_plan_create(hipStream_t stream, int32_t m, int32_t n, i
   p->st.nnz = nnz;
   p->st.base = base;
   p->st.trusted = trusted ? 1 : 0;
+  p->dtype = dtype;
   p->val_size = val_size;
 
   int* d_stats = nullptr;
@@ -535,12 +575,13 @@ extern "C" int asamd_csr_plan_create(hipStream_t stream, int32_t m, int32_t n, i
   for (int b = 0; b < ASAMD_HIST_BINS; ++b) p->st.hist[b] = h[3 + b];
 
   const int64_t total = (int64_t)m + nnz;
-  // fp64 doubles the LDS per item: fewer items keep more workgroups resident
-  p->merge_ipt = val_size == 8 ? 4 : 8;
+  // wider values take more LDS per item: fewer items keep more workgroups resident
+  p->merge_ipt = val_size >= 8 ? 4 : 8;
   if (const char* ev = getenv("ALSPARSE_AMD_MERGE_IPT")) {
     const int v = atoi(ev);
-    if (v == 4 || v == 8 || v == 16) p->merge_ipt = v;
+    if (v == 4 || v == 8 || (v == 16 && dtype <= ASAMD_DTYPE_DOUBLE)) p->merge_ipt = v;
   }
+  if (val_size == 16) p->merge_ipt = 4;  // the only instantiation for 16-byte values
   const int merge_items = kMergeThreads * p->merge_ipt;
   const int64_t nb = (total + merge_items - 1) / merge_items;
   p->st.merge_blocks = (int)nb;
@@ -570,17 +611,18 @@ extern "C" int asamd_csr_plan_create(hipStream_t stream, int32_t m, int32_t n, i
     // trusted == 2: build the tiled copy whatever the size and skip the timing
     // (lets small matrices exercise the tiled kernels)
     const bool force = trusted == 2;
-    const bool tiled_ok = val_size == 4 ? tiled_eligible<float>(p->st, force) : tiled_eligible<double>(p->st, force);
-    const bool ell_ok = ell_eligible(p->st, force);
-    if (tiled_ok)
-      e = val_size == 4 ? build_tiled<float>(stream, p, row_ptr, col_ind, (const float*)val)
-                        : build_tiled<double>(stream, p, row_ptr, col_ind, (const double*)val);
-    if (e == hipSuccess && ell_ok)
-      e = val_size == 4 ? build_ell<float>(stream, p, row_ptr, col_ind, (const float*)val)
-                        : build_ell<double>(stream, p, row_ptr, col_ind, (const double*)val);
-    if (e == hipSuccess && !force && (p->st.tiled_built || p->st.ell_built))
-      e = val_size == 4 ? tune_copies<float>(stream, p, row_ptr, col_ind, (const float*)val)
-                        : tune_copies<double>(stream, p, row_ptr, col_ind, (const double*)val);
+    e = by_dtype(dtype, [&](auto* tag) -> hipError_t {
+      using T = std::remove_pointer_t<decltype(tag)>;
+      hipError_t err = hipSuccess;
+      if constexpr (kIsReal<T>) {
+        if (tiled_eligible<T>(p->st, force)) err = build_tiled<T>(stream, p, row_ptr, col_ind, (const T*)val);
+      }
+      if (err == hipSuccess && ell_eligible(p->st, force))
+        err = build_ell<T>(stream, p, row_ptr, col_ind, (const T*)val);
+      if (err == hipSuccess && !force && (p->st.tiled_built || p->st.ell_built))
+        err = tune_copies<T>(stream, p, row_ptr, col_ind, (const T*)val);
+      return err;
+    });
     if (e == hipErrorOutOfMemory) {
       (void)hipGetLastError();  // the copies are optional: carry on without them
       free_tiled(p);
@@ -597,6 +639,21 @@ extern "C" int asamd_csr_plan_create(hipStream_t stream, int32_t m, int32_t n, i
   return hipSuccess;
 }
 
+extern "C" int asamd_csr_plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t nnz,
+                                     const int32_t* row_ptr, const int32_t* col_ind,
+                                     const void* val, int32_t base, int32_t val_size,
+                                     int32_t trusted, asamd_csr_plan** out) {
+  if (val_size != 4 && val_size != 8) return hipErrorInvalidValue;
+  return plan_create(stream, m, n, nnz, row_ptr, col_ind, val, base,
+                     val_size == 4 ? ASAMD_DTYPE_FLOAT : ASAMD_DTYPE_DOUBLE, trusted, out);
+}
+
+extern "C" int asamd_csr_plan_create_dtype(hipStream_t stream, int32_t m, int32_t n, int32_t nnz,
+                                           const int32_t* row_ptr, const int32_t* col_ind, const void* val,
+                                           int32_t base, int32_t dtype, int32_t trusted, asamd_csr_plan** out) {
+  return plan_create(stream, m, n, nnz, row_ptr, col_ind, val, base, dtype, trusted, out);
+}
+
 extern "C" void asamd_csr_plan_destroy(asamd_csr_plan* p) {
   if (!p) return;
   if (p->d_block_row) (void)hipFree(p->d_block_row);
@@ -605,7 +662,8 @@ extern "C" void asamd_csr_plan_destroy(asamd_csr_plan* p) {
   if (p->d_head_val) (void)hipFree(p->d_head_val);
   free_tiled(p);
   free_ell(p);
-  free_transpose(p);
+  free_transpose(p, 0);
+  free_transpose(p, 1);
   delete p;
 }
 
@@ -613,8 +671,9 @@ extern "C" void asamd_csr_plan_destroy(asamd_csr_plan* p) {
 // a column), read the column offsets off the sorted keys, gather rows and values.
 template <typename T>
 static hipError_t build_transpose(hipStream_t stream, asamd_csr_plan* p, const int* row_ptr, const int* col_ind,
-                                  const T* val) {
+                                  const T* val, int which) {
   asamd_csr_stats& st = p->st;
+  asamd_csr_plan::TransCopy& t = p->tr[which];
   const int nnz = st.nnz, n = st.n;
   int* d_coo = nullptr;
   unsigned *d_key = nullptr, *d_key2 = nullptr, *d_idx = nullptr, *d_perm = nullptr;
@@ -623,9 +682,9 @@ static hipError_t build_transpose(hipStream_t stream, asamd_csr_plan* p, const i
   if (e == hipSuccess) e = hipMalloc(&d_key2, (size_t)nnz * sizeof(unsigned));
   if (e == hipSuccess) e = hipMalloc(&d_idx, (size_t)nnz * sizeof(unsigned));
   if (e == hipSuccess) e = hipMalloc(&d_perm, (size_t)nnz * sizeof(unsigned));
-  if (e == hipSuccess) e = hipMalloc(&p->d_tr_row_ptr, ((size_t)n + 1) * sizeof(int));
-  if (e == hipSuccess) e = hipMalloc(&p->d_tr_col, (size_t)nnz * sizeof(int));
-  if (e == hipSuccess) e = hipMalloc(&p->d_tr_val, (size_t)nnz * sizeof(T));
+  if (e == hipSuccess) e = hipMalloc(&t.d_row_ptr, ((size_t)n + 1) * sizeof(int));
+  if (e == hipSuccess) e = hipMalloc(&t.d_col, (size_t)nnz * sizeof(int));
+  if (e == hipSuccess) e = hipMalloc(&t.d_val, (size_t)nnz * sizeof(T));
   if (e == hipSuccess) e = (hipError_t)asamd_csr2coo(stream, row_ptr, nnz, st.m, d_coo, st.base);
   if (e == hipSuccess) {
     int grid = (nnz + 255) / 256;
@@ -637,9 +696,13 @@ static hipError_t build_transpose(hipStream_t stream, asamd_csr_plan* p, const i
     if (e == hipSuccess) e = sort_pairs_u32(stream, d_key, d_key2, d_idx, d_perm, (size_t)nnz, bits);
     if (e == hipSuccess) {
       tile_bounds_kernel<<<(unsigned)(((int64_t)n + 1 + 255) / 256), 256, 0, stream>>>(nnz, d_key2, (int64_t)n,
-                                                                                      p->d_tr_row_ptr);
-      transpose_gather_kernel<T><<<grid, 256, 0, stream>>>(nnz, d_perm, d_coo, val, st.base, p->d_tr_col,
-                                                           (T*)p->d_tr_val);
+                                                                                      t.d_row_ptr);
+      if (which == 1)
+        transpose_gather_kernel<T, true><<<grid, 256, 0, stream>>>(nnz, d_perm, d_coo, val, st.base, t.d_col,
+                                                                   (T*)t.d_val);
+      else
+        transpose_gather_kernel<T, false><<<grid, 256, 0, stream>>>(nnz, d_perm, d_coo, val, st.base, t.d_col,
+                                                                    (T*)t.d_val);
       e = hipGetLastError();
     }
     if (e == hipSuccess) e = hipStreamSynchronize(stream);
@@ -647,23 +710,36 @@ static hipError_t build_transpose(hipStream_t stream, asamd_csr_plan* p, const i
   for (void* d : {(void*)d_coo, (void*)d_key, (void*)d_key2, (void*)d_idx, (void*)d_perm})
     if (d) (void)hipFree(d);
   if (e == hipSuccess)
-    e = (hipError_t)asamd_csr_plan_create(stream, n, st.m, nnz, p->d_tr_row_ptr, p->d_tr_col, p->d_tr_val, 0,
-                                          (int32_t)sizeof(T), /*trusted=*/1, &p->tr_plan);
+    e = plan_create(stream, n, st.m, nnz, t.d_row_ptr, t.d_col, t.d_val, 0, DtypeOf<T>::value, /*trusted=*/1,
+                    &t.plan);
   if (e != hipSuccess) {
-    free_transpose(p);
+    free_transpose(p, which);
     return e;
   }
-  st.transpose_built = 1;
+  st.transpose_built |= 1 << which;
   return hipSuccess;
+}
+
+static int build_transpose_any(hipStream_t stream, asamd_csr_plan* p, const int32_t* row_ptr,
+                               const int32_t* col_ind, const void* val, int which) {
+  if (!p || !row_ptr || !col_ind || !val || !p->st.trusted || p->st.n <= 0) return hipErrorInvalidValue;
+  if (which == 1 && !is_complex(p)) return hipErrorInvalidValue;
+  if (p->st.transpose_built & (1 << which)) return hipSuccess;
+  if (p->st.nnz == 0) return hipSuccess;  // the scatter route has nothing to add
+  return by_dtype(p->dtype, [&](auto* tag) -> hipError_t {
+    using T = std::remove_pointer_t<decltype(tag)>;
+    return build_transpose<T>(stream, p, row_ptr, col_ind, (const T*)val, which);
+  });
 }
 
 extern "C" int asamd_csr_plan_build_transpose(hipStream_t stream, asamd_csr_plan* p, const int32_t* row_ptr,
                                               const int32_t* col_ind, const void* val) {
-  if (!p || !row_ptr || !col_ind || !val || !p->st.trusted || p->st.n <= 0) return hipErrorInvalidValue;
-  if (p->st.transpose_built) return hipSuccess;
-  if (p->st.nnz == 0) return hipSuccess;  // the scatter route has nothing to add
-  return p->val_size == 4 ? build_transpose<float>(stream, p, row_ptr, col_ind, (const float*)val)
-                          : build_transpose<double>(stream, p, row_ptr, col_ind, (const double*)val);
+  return build_transpose_any(stream, p, row_ptr, col_ind, val, 0);
+}
+
+extern "C" int asamd_csr_plan_build_conj_transpose(hipStream_t stream, asamd_csr_plan* p, const int32_t* row_ptr,
+                                                   const int32_t* col_ind, const void* val) {
+  return build_transpose_any(stream, p, row_ptr, col_ind, val, 1);
 }
 
 extern "C" int asamd_csr_plan_set_lazy_transpose(asamd_csr_plan* p, int32_t on) {
@@ -673,7 +749,9 @@ extern "C" int asamd_csr_plan_set_lazy_transpose(asamd_csr_plan* p, int32_t on) 
 }
 
 extern "C" const asamd_csr_stats* asamd_csr_plan_transpose_stats(const asamd_csr_plan* p) {
-  return p && p->tr_plan ? &p->tr_plan->st : nullptr;
+  if (!p) return nullptr;
+  if (p->tr[0].plan) return &p->tr[0].plan->st;
+  return p->tr[1].plan ? &p->tr[1].plan->st : nullptr;
 }
 
 extern "C" const asamd_csr_stats* asamd_csr_plan_stats(const asamd_csr_plan* p) {
@@ -687,7 +765,7 @@ extern "C" int asamd_csr_plan_set_algo(asamd_csr_plan* p, int32_t algo) {
       p->st.algo = p->auto_algo;
       return hipSuccess;
     case ASAMD_SPMV_ROWCONST:
-      if (!rowconst_ok(p->st)) return hipErrorInvalidValue;
+      if (!rowconst_ok(p)) return hipErrorInvalidValue;
       p->st.algo = algo;
       return hipSuccess;
     case ASAMD_SPMV_TILED:
@@ -695,7 +773,7 @@ extern "C" int asamd_csr_plan_set_algo(asamd_csr_plan* p, int32_t algo) {
       p->st.algo = algo;
       return hipSuccess;
     case ASAMD_SPMV_STREAM:
-      if (!stream_ok(p->st)) return hipErrorInvalidValue;
+      if (!stream_ok(p)) return hipErrorInvalidValue;
       p->st.algo = algo;
       return hipSuccess;
     case ASAMD_SPMV_ELL:
@@ -734,15 +812,17 @@ template <typename T>
 static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, const int* rp,
                       const int* ci, const T* x, T beta, T* y) {
   if (!p || !val || !rp || !ci || !x || !y) return hipErrorInvalidValue;
-  if (p->val_size != (int)sizeof(T)) return hipErrorInvalidValue;
+  if (p->dtype != DtypeOf<T>::value) return hipErrorInvalidValue;
+  if (((uintptr_t)val | (uintptr_t)x | (uintptr_t)y) % alignof(T)) return hipErrorInvalidValue;
   const asamd_csr_stats& st = p->st;
   int algo = st.algo;
+  if (!kIsReal<T> && (algo == ASAMD_SPMV_ROWCONST || algo == ASAMD_SPMV_TILED)) algo = ASAMD_SPMV_VECTOR;
   if (algo == ASAMD_SPMV_ROWCONST) {
     // 128-bit loads need 16-byte aligned streams; fall back otherwise
     const bool aligned = (((uintptr_t)val | (uintptr_t)ci) & 15u) == 0;
-    if (!aligned || !rowconst_ok(st)) algo = ASAMD_SPMV_VECTOR;
+    if (!aligned || !rowconst_ok(p)) algo = ASAMD_SPMV_VECTOR;
   }
-  if (algo == ASAMD_SPMV_STREAM && !stream_ok(st)) algo = ASAMD_SPMV_MERGE;
+  if (algo == ASAMD_SPMV_STREAM && !stream_ok(p)) algo = ASAMD_SPMV_MERGE;
   if (algo == ASAMD_SPMV_TILED && !st.tiled_built) algo = p->auto_algo == ASAMD_SPMV_TILED ? ASAMD_SPMV_MERGE : p->auto_algo;
   if (algo == ASAMD_SPMV_ELL && !st.ell_built) algo = p->auto_algo == ASAMD_SPMV_ELL ? ASAMD_SPMV_MERGE : p->auto_algo;
   switch (algo) {
@@ -753,7 +833,7 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
                                                    x, beta, y);
       break;
     }
-    case ASAMD_SPMV_TILED: {
+    case ASAMD_SPMV_TILED: if constexpr (kIsReal<T>) {
       // the tiled copy holds zero-based local indices and its own values
       if (p->n_chunks > 0)
         tiled_products_kernel<T><<<p->n_chunks, kProdThreads, kTileBytes, s>>>(
@@ -766,7 +846,7 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
                                                                        (const T*)p->d_tprod, alpha, y);
       break;
     }
-    case ASAMD_SPMV_ROWCONST:
+    case ASAMD_SPMV_ROWCONST: if constexpr (kIsReal<T>) {
       switch (st.const_len / 4) {
         case 1: launch_rowconst<T, 1>(s, st, alpha, val, ci, x, beta, y); break;
         case 2: launch_rowconst<T, 2>(s, st, alpha, val, ci, x, beta, y); break;
@@ -777,6 +857,7 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
         default: launch_rowconst<T, 64>(s, st, alpha, val, ci, x, beta, y); break;
       }
       break;
+    }
     case ASAMD_SPMV_STREAM: {
       const unsigned grid = (unsigned)(((int64_t)st.m + kStreamRows - 1) / kStreamRows);
       if (st.max_len <= 4)
@@ -802,9 +883,14 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
   spmv_merge_kernel<T, IPT><<<nb, kMergeThreads, 0, s>>>(st.m, st.nnz, alpha, val, rp, ci, x, beta, y, \
                                                          st.base, p->d_block_row, p->d_carry_row,      \
                                                          (T*)p->d_carry_val, (T*)p->d_head_val)
-      if (p->merge_ipt == 4) ASAMD_LAUNCH_MERGE(4);
-      else if (p->merge_ipt == 16) ASAMD_LAUNCH_MERGE(16);
-      else ASAMD_LAUNCH_MERGE(8);
+      // LDS per workgroup grows with IPT * sizeof(T): 16-byte values run 4 items only, 8-byte ones up to 16
+      if constexpr (sizeof(T) <= 8) {
+        if (p->merge_ipt == 16 && kIsReal<T>) ASAMD_LAUNCH_MERGE(16);
+        else if (p->merge_ipt == 8) ASAMD_LAUNCH_MERGE(8);
+        else ASAMD_LAUNCH_MERGE(4);
+      } else {
+        ASAMD_LAUNCH_MERGE(4);
+      }
 #undef ASAMD_LAUNCH_MERGE
       if (nb > 1)
         merge_fixup_kernel<T><<<(nb + 255) / 256, 256, 0, s>>>(nb, st.m, alpha, beta, p->d_carry_row,
@@ -827,22 +913,40 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
   return hipGetLastError();
 }
 
-template <typename T, int W>
+template <typename T, int W, bool CONJ>
 static void launch_trans_scatter(hipStream_t s, const asamd_csr_stats& st, T alpha, const T* val, const int* rp,
                                  const int* ci, const T* x, T* y) {
   constexpr int rows_per_block = kTransThreads / W;
   const unsigned grid = (unsigned)(((int64_t)st.m + rows_per_block - 1) / rows_per_block);
-  csrmv_trans_scatter_kernel<T, W><<<grid, kTransThreads, 0, s>>>(st.m, st.n, alpha, val, rp, ci, x, y, st.base);
+  csrmv_trans_scatter_kernel<T, W, CONJ><<<grid, kTransThreads, 0, s>>>(st.m, st.n, alpha, val, rp, ci, x, y,
+                                                                         st.base);
 }
 
+template <typename T, bool CONJ>
+static void trans_scatter(hipStream_t s, const asamd_csr_plan* p, T alpha, const T* val, const int* rp,
+                          const int* ci, const T* x, T* y) {
+  const asamd_csr_stats& st = p->st;
+  switch (p->auto_width) {
+    case 2: launch_trans_scatter<T, 2, CONJ>(s, st, alpha, val, rp, ci, x, y); break;
+    case 4: launch_trans_scatter<T, 4, CONJ>(s, st, alpha, val, rp, ci, x, y); break;
+    case 8: launch_trans_scatter<T, 8, CONJ>(s, st, alpha, val, rp, ci, x, y); break;
+    case 16: launch_trans_scatter<T, 16, CONJ>(s, st, alpha, val, rp, ci, x, y); break;
+    case 32: launch_trans_scatter<T, 32, CONJ>(s, st, alpha, val, rp, ci, x, y); break;
+    default: launch_trans_scatter<T, 64, CONJ>(s, st, alpha, val, rp, ci, x, y); break;
+  }
+}
+
+// which = 0: y = alpha*A^T*x + beta*y; which = 1 (complex element types): A^H in place of A^T
 template <typename T>
 static int csrmv_trans_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, const int* rp, const int* ci,
-                            const T* x, T beta, T* y) {
+                            const T* x, T beta, T* y, int which) {
   if (!p || !val || !rp || !ci || !x || !y) return hipErrorInvalidValue;
-  if (p->val_size != (int)sizeof(T)) return hipErrorInvalidValue;
+  if (p->dtype != DtypeOf<T>::value || (which == 1 && kIsReal<T>)) return hipErrorInvalidValue;
+  if (((uintptr_t)val | (uintptr_t)x | (uintptr_t)y) % alignof(T)) return hipErrorInvalidValue;
   const asamd_csr_stats& st = p->st;
-  if (!p->tr_plan && p->lazy_transpose && st.trusted && st.nnz > 0) {
-    const hipError_t e = build_transpose<T>(s, p, rp, ci, val);
+  asamd_csr_plan::TransCopy& t = p->tr[which];
+  if (!t.plan && p->lazy_transpose && st.trusted && st.nnz > 0) {
+    const hipError_t e = build_transpose<T>(s, p, rp, ci, val, which);
     if (e == hipErrorOutOfMemory) {
       (void)hipGetLastError();  // no room for the copy: scatter instead, and do not try again
       p->lazy_transpose = false;
@@ -850,30 +954,28 @@ static int csrmv_trans_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* 
       return e;
     }
   }
-  if (p->tr_plan)
-    return csrmv_impl<T>(s, p->tr_plan, alpha, (const T*)p->d_tr_val, p->d_tr_row_ptr, p->d_tr_col, x, beta, y);
+  if (t.plan) return csrmv_impl<T>(s, t.plan, alpha, (const T*)t.d_val, t.d_row_ptr, t.d_col, x, beta, y);
   if (beta != T(1)) scale_vec_kernel<T><<<(unsigned)(((int64_t)st.n + 255) / 256), 256, 0, s>>>(st.n, beta, y);
-  switch (p->auto_width) {
-    case 2: launch_trans_scatter<T, 2>(s, st, alpha, val, rp, ci, x, y); break;
-    case 4: launch_trans_scatter<T, 4>(s, st, alpha, val, rp, ci, x, y); break;
-    case 8: launch_trans_scatter<T, 8>(s, st, alpha, val, rp, ci, x, y); break;
-    case 16: launch_trans_scatter<T, 16>(s, st, alpha, val, rp, ci, x, y); break;
-    case 32: launch_trans_scatter<T, 32>(s, st, alpha, val, rp, ci, x, y); break;
-    default: launch_trans_scatter<T, 64>(s, st, alpha, val, rp, ci, x, y); break;
+  if constexpr (!kIsReal<T>) {
+    if (which == 1) {
+      trans_scatter<T, true>(s, p, alpha, val, rp, ci, x, y);
+      return hipGetLastError();
+    }
   }
+  trans_scatter<T, false>(s, p, alpha, val, rp, ci, x, y);
   return hipGetLastError();
 }
 
 extern "C" int asamd_s_csrmv_trans(hipStream_t stream, asamd_csr_plan* plan, float alpha, const float* val,
                                    const int32_t* row_ptr, const int32_t* col_ind, const float* x, float beta,
                                    float* y) {
-  return csrmv_trans_impl<float>(stream, plan, alpha, val, row_ptr, col_ind, x, beta, y);
+  return csrmv_trans_impl<float>(stream, plan, alpha, val, row_ptr, col_ind, x, beta, y, 0);
 }
 
 extern "C" int asamd_d_csrmv_trans(hipStream_t stream, asamd_csr_plan* plan, double alpha, const double* val,
                                    const int32_t* row_ptr, const int32_t* col_ind, const double* x, double beta,
                                    double* y) {
-  return csrmv_trans_impl<double>(stream, plan, alpha, val, row_ptr, col_ind, x, beta, y);
+  return csrmv_trans_impl<double>(stream, plan, alpha, val, row_ptr, col_ind, x, beta, y, 0);
 }
 
 extern "C" int asamd_s_csrmv(hipStream_t stream, asamd_csr_plan* plan, float alpha,
@@ -886,6 +988,32 @@ extern "C" int asamd_d_csrmv(hipStream_t stream, asamd_csr_plan* plan, double al
                              const double* val, const int32_t* row_ptr, const int32_t* col_ind,
                              const double* x, double beta, double* y) {
   return csrmv_impl<double>(stream, plan, alpha, val, row_ptr, col_ind, x, beta, y);
+}
+
+// complex element types: op = 0 (A), 1 (A^T), 2 (A^H), the values of alphasparse_operation_t
+static_assert(sizeof(asamd_complex8) == sizeof(Cx<float>) && sizeof(asamd_complex16) == sizeof(Cx<double>),
+              "complex layouts");
+
+template <typename T, typename C>
+static int csrmv_complex(hipStream_t stream, asamd_csr_plan* plan, int32_t op, C alpha, const C* val,
+                         const int32_t* row_ptr, const int32_t* col_ind, const C* x, C beta, C* y) {
+  const T a(alpha.real, alpha.imag), b(beta.real, beta.imag);
+  if (op == 0) return csrmv_impl<T>(stream, plan, a, (const T*)val, row_ptr, col_ind, (const T*)x, b, (T*)y);
+  if (op == 1 || op == 2)
+    return csrmv_trans_impl<T>(stream, plan, a, (const T*)val, row_ptr, col_ind, (const T*)x, b, (T*)y, op - 1);
+  return hipErrorInvalidValue;
+}
+
+extern "C" int asamd_c_csrmv_op(hipStream_t stream, asamd_csr_plan* plan, int32_t op, asamd_complex8 alpha,
+                                const asamd_complex8* val, const int32_t* row_ptr, const int32_t* col_ind,
+                                const asamd_complex8* x, asamd_complex8 beta, asamd_complex8* y) {
+  return csrmv_complex<Cx<float>>(stream, plan, op, alpha, val, row_ptr, col_ind, x, beta, y);
+}
+
+extern "C" int asamd_z_csrmv_op(hipStream_t stream, asamd_csr_plan* plan, int32_t op, asamd_complex16 alpha,
+                                const asamd_complex16* val, const int32_t* row_ptr, const int32_t* col_ind,
+                                const asamd_complex16* x, asamd_complex16 beta, asamd_complex16* y) {
+  return csrmv_complex<Cx<double>>(stream, plan, op, alpha, val, row_ptr, col_ind, x, beta, y);
 }
 
 extern "C" int asamd_copy_bytes(hipStream_t stream, void* dst, const void* src, size_t nbytes) {

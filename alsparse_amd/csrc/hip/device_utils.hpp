@@ -29,16 +29,119 @@ __device__ __forceinline__ unsigned xcd_contiguous_id(unsigned hw_id, unsigned n
 __device__ __forceinline__ float fma_t(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
 __device__ __forceinline__ double fma_t(double a, double b, double c) { return __builtin_fma(a, b, c); }
 
+// single operations that the compiler may not contract into fused multiply-adds
+// (the pragma takes the `contract` flag off the operation itself, so it stays
+// unfused wherever the function is inlined)
+template <typename R>
+__device__ __forceinline__ R mul_rn(R a, R b) {
+#pragma clang fp contract(off)
+  return a * b;
+}
+template <typename R>
+__device__ __forceinline__ R add_rn(R a, R b) {
+#pragma clang fp contract(off)
+  return a + b;
+}
+
+// ---- complex scalars ---------------------------------------------------------
+// Cx<float> / Cx<double> have the memory layout of the reference's
+// ALPHA_Complex8 / ALPHA_Complex16 ({real, imag}, include/alphasparse/types.h:42-56).
+// Device arrays of them are assumed aligned to the element size (the entry
+// points check), so one element is one 64- or 128-bit load.
+//   a * b      the four-multiplication form, every operation rounded on its own,
+//              as the reference's cmp_mul (include/alphasparse/complex_compute.h:76-82)
+//   fma_t      c + a*b with the fused chain of the reference's device cmp_madde
+//              (complex_compute.h:139-146)
+template <typename R>
+struct alignas(2 * sizeof(R)) Cx {
+  R re, im;
+  Cx() = default;
+  __host__ __device__ constexpr Cx(R r, R i = R(0)) : re(r), im(i) {}
+  __device__ __forceinline__ Cx& operator+=(const Cx& o) {
+    re += o.re;
+    im += o.im;
+    return *this;
+  }
+};
+template <typename R>
+__device__ __forceinline__ Cx<R> operator+(Cx<R> a, Cx<R> b) { return Cx<R>(add_rn(a.re, b.re), add_rn(a.im, b.im)); }
+template <typename R>
+__device__ __forceinline__ Cx<R> operator*(Cx<R> a, Cx<R> b) {
+  return Cx<R>(add_rn(mul_rn(a.re, b.re), -mul_rn(a.im, b.im)), add_rn(mul_rn(a.im, b.re), mul_rn(a.re, b.im)));
+}
+template <typename R>
+__host__ __device__ __forceinline__ bool operator==(Cx<R> a, Cx<R> b) { return a.re == b.re && a.im == b.im; }
+template <typename R>
+__host__ __device__ __forceinline__ bool operator!=(Cx<R> a, Cx<R> b) { return !(a == b); }
+template <typename R>
+__device__ __forceinline__ Cx<R> fma_t(Cx<R> a, Cx<R> b, Cx<R> c) {
+  return Cx<R>(fma_t(-a.im, b.im, fma_t(a.re, b.re, c.re)), fma_t(a.re, b.im, fma_t(a.im, b.re, c.im)));
+}
+__device__ __forceinline__ float conj_t(float a) { return a; }
+__device__ __forceinline__ double conj_t(double a) { return a; }
+template <typename R>
+__device__ __forceinline__ Cx<R> conj_t(Cx<R> a) { return Cx<R>(a.re, -a.im); }
+
+// ---- wave shuffles, streaming loads / stores and atomic adds for every scalar type
+template <typename T>
+__device__ __forceinline__ T lane_up(T v, unsigned d) { return __shfl_up(v, d, kWave); }
+template <typename T>
+__device__ __forceinline__ T lane_down(T v, unsigned d) { return __shfl_down(v, d, kWave); }
+template <typename T>
+__device__ __forceinline__ T lane_xor(T v, int mask) { return __shfl_xor(v, mask, kWave); }
+template <typename T>
+__device__ __forceinline__ T lane_get(T v, int src) { return __shfl(v, src, kWave); }
+template <typename R>
+__device__ __forceinline__ Cx<R> lane_up(Cx<R> v, unsigned d) { return Cx<R>(lane_up(v.re, d), lane_up(v.im, d)); }
+template <typename R>
+__device__ __forceinline__ Cx<R> lane_down(Cx<R> v, unsigned d) { return Cx<R>(lane_down(v.re, d), lane_down(v.im, d)); }
+template <typename R>
+__device__ __forceinline__ Cx<R> lane_xor(Cx<R> v, int mask) { return Cx<R>(lane_xor(v.re, mask), lane_xor(v.im, mask)); }
+template <typename R>
+__device__ __forceinline__ Cx<R> lane_get(Cx<R> v, int src) { return Cx<R>(lane_get(v.re, src), lane_get(v.im, src)); }
+
+template <typename T>
+__device__ __forceinline__ T nt_load(const T* p) { return __builtin_nontemporal_load(p); }
+template <typename T>
+__device__ __forceinline__ void nt_store(T v, T* p) { __builtin_nontemporal_store(v, p); }
+template <typename R>
+__device__ __forceinline__ Cx<R> nt_load(const Cx<R>* p) {
+  typedef R Pair __attribute__((ext_vector_type(2)));
+  const Pair v = __builtin_nontemporal_load(reinterpret_cast<const Pair*>(p));
+  return Cx<R>(v.x, v.y);
+}
+template <typename R>
+__device__ __forceinline__ void nt_store(Cx<R> v, Cx<R>* p) {
+  typedef R Pair __attribute__((ext_vector_type(2)));
+  Pair q;
+  q.x = v.re;
+  q.y = v.im;
+  __builtin_nontemporal_store(q, reinterpret_cast<Pair*>(p));
+}
+
+template <typename T>
+__device__ __forceinline__ void atomic_add(T* p, T v) { atomicAdd(p, v); }
+// the two halves of a complex sum are independent additions
+template <typename R>
+__device__ __forceinline__ void atomic_add(Cx<R>* p, Cx<R> v) {
+  atomicAdd(&p->re, v.re);
+  atomicAdd(&p->im, v.im);
+}
+
 // y <- beta*y + alpha*sum with the reference's rounding points: both products
 // are rounded separately and then added, never contracted into an fma
 // (src/kernel/dcu/level2/mv/csrmv/dcu_gemv_vector.h:50-54 and
 // src/plain/kernel/level2/mv/gemv/gemv_x_csr_plain.c:14,21 agree on this).
 // beta == 0 does not read y at all.
 __device__ __forceinline__ float axpby_rn(float alpha, float sum, float beta, float yold) {
-  return __fadd_rn(__fmul_rn(yold, beta), __fmul_rn(alpha, sum));
+  return add_rn(mul_rn(yold, beta), mul_rn(alpha, sum));
 }
 __device__ __forceinline__ double axpby_rn(double alpha, double sum, double beta, double yold) {
-  return __dadd_rn(__dmul_rn(yold, beta), __dmul_rn(alpha, sum));
+  return add_rn(mul_rn(yold, beta), mul_rn(alpha, sum));
+}
+template <typename R>
+__device__ __forceinline__ Cx<R> axpby_rn(Cx<R> alpha, Cx<R> sum, Cx<R> beta, Cx<R> yold) {
+  return yold * beta + alpha * sum;  // operator* rounds every operation on its own
 }
 template <typename T>
 __device__ __forceinline__ void store_axpby(T* __restrict__ y, int64_t row, T alpha, T sum, T beta) {
@@ -73,6 +176,11 @@ __device__ __forceinline__ double dpp_mov(double v) {
 // mirror hands each lane the total of the opposite half); the 32- and
 // 64-lane steps cross DPP rows and use the LDS crossbar (ds_bpermute through
 // __shfl_xor), which touches no LDS memory.
+template <int Ctrl, typename R>
+__device__ __forceinline__ Cx<R> dpp_mov(Cx<R> v) {
+  return Cx<R>(dpp_mov<Ctrl>(v.re), dpp_mov<Ctrl>(v.im));
+}
+
 template <int W, typename T>
 __device__ __forceinline__ T group_sum(T v) {
   static_assert(W >= 1 && W <= 64 && (W & (W - 1)) == 0, "group width");
@@ -80,8 +188,8 @@ __device__ __forceinline__ T group_sum(T v) {
   if constexpr (W >= 4) v += dpp_mov<0x4E>(v);   // quad_perm [2,3,0,1]
   if constexpr (W >= 8) v += dpp_mov<0x141>(v);  // row_half_mirror: lane l <-> 7-l in each 8
   if constexpr (W >= 16) v += dpp_mov<0x140>(v); // row_mirror: lane l <-> 15-l in each 16
-  if constexpr (W >= 32) v += __shfl_xor(v, 16, kWave);
-  if constexpr (W >= 64) v += __shfl_xor(v, 32, kWave);
+  if constexpr (W >= 32) v += lane_xor(v, 16);
+  if constexpr (W >= 64) v += lane_xor(v, 32);
   return v;
 }
 

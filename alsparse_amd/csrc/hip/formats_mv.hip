@@ -62,12 +62,12 @@ __global__ __launch_bounds__(kCooThreads) void coomv_kernel(int64_t nnz, int m, 
       const int c = __builtin_nontemporal_load(&coo_col[k]) - base;
       if ((unsigned)rr < (unsigned)m && (unsigned)c < (unsigned)n) {
         r = rr;
-        v = __builtin_nontemporal_load(&coo_val[k]) * x[c];
+        v = nt_load(&coo_val[k]) * x[c];
       }
     }
     if (lane == 0) {
       if (carry_row == r) v += carry_val;
-      else if (carry_row >= 0) atomicAdd(&y[carry_row], alpha * carry_val);
+      else if (carry_row >= 0) atomic_add(&y[carry_row], alpha * carry_val);
     }
     const int r_prev = __shfl_up(r, 1, kWave);
     const bool head = lane == 0 || r_prev != r;
@@ -76,7 +76,7 @@ __global__ __launch_bounds__(kCooThreads) void coomv_kernel(int64_t nnz, int m, 
     int f = head;
 #pragma unroll
     for (int d = 1; d < kWave; d <<= 1) {
-      const T vd = __shfl_up(v, d, kWave);
+      const T vd = lane_up(v, d);
       const int fd = __shfl_up(f, d, kWave);
       if (lane >= d && !f) {
         v += vd;
@@ -84,17 +84,18 @@ __global__ __launch_bounds__(kCooThreads) void coomv_kernel(int64_t nnz, int m, 
       }
     }
     const int head_next = __shfl_down((int)head, 1, kWave);
-    if (lane < kWave - 1 && head_next && r >= 0) atomicAdd(&y[r], alpha * v);
+    if (lane < kWave - 1 && head_next && r >= 0) atomic_add(&y[r], alpha * v);
     carry_row = __shfl(r, kWave - 1, kWave);
-    carry_val = __shfl(v, kWave - 1, kWave);
+    carry_val = lane_get(v, kWave - 1);
   }
-  if (lane == 0 && carry_row >= 0) atomicAdd(&y[carry_row], alpha * carry_val);
+  if (lane == 0 && carry_row >= 0) atomic_add(&y[carry_row], alpha * carry_val);
 }
 
 template <typename T>
 int ellmv_impl(hipStream_t stream, int32_t m, int32_t n, T alpha, const T* ell_val, const int32_t* ell_col,
                int32_t width, int32_t base, const T* x, T beta, T* y) {
   if (m < 0 || n < 0 || width < 0) return (int)hipErrorInvalidValue;
+  if (((uintptr_t)ell_val | (uintptr_t)x | (uintptr_t)y) % alignof(T)) return (int)hipErrorInvalidValue;
   if (m == 0) return (int)hipSuccess;
   const unsigned grid = (unsigned)(((int64_t)m + kEllThreads - 1) / kEllThreads);
   ellmv_kernel<T><<<grid, kEllThreads, 0, stream>>>(m, n, alpha, ell_val, ell_col, width, base, x, beta, y);
@@ -105,6 +106,7 @@ template <typename T>
 int coomv_impl(hipStream_t stream, int32_t m, int32_t n, int64_t nnz, T alpha, const T* coo_val,
                const int32_t* coo_row, const int32_t* coo_col, int32_t base, const T* x, T beta, T* y) {
   if (m < 0 || n < 0 || nnz < 0) return (int)hipErrorInvalidValue;
+  if (((uintptr_t)coo_val | (uintptr_t)x | (uintptr_t)y) % alignof(T)) return (int)hipErrorInvalidValue;
   if (m == 0) return (int)hipSuccess;
   if (beta != T(1)) {
     scale_y_kernel<T><<<(unsigned)(((int64_t)m + 255) / 256), 256, 0, stream>>>(m, beta, y);
@@ -147,6 +149,39 @@ int asamd_d_coomv(hipStream_t stream, int32_t m, int32_t n, int64_t nnz, double 
                   double beta, double* y) {
   return asamd::coomv_impl<double>(stream, m, n, nnz, alpha, coo_val, coo_row_ind, coo_col_ind, base, x, beta,
                                    y);
+}
+
+// complex element types: the same kernels over Cx<float> / Cx<double>
+int asamd_c_ellmv(hipStream_t stream, int32_t m, int32_t n, asamd_complex8 alpha, const asamd_complex8* ell_val,
+                  const int32_t* ell_col_ind, int32_t ell_width, int32_t base, const asamd_complex8* x,
+                  asamd_complex8 beta, asamd_complex8* y) {
+  using T = asamd::Cx<float>;
+  return asamd::ellmv_impl<T>(stream, m, n, T(alpha.real, alpha.imag), (const T*)ell_val, ell_col_ind, ell_width,
+                              base, (const T*)x, T(beta.real, beta.imag), (T*)y);
+}
+
+int asamd_z_ellmv(hipStream_t stream, int32_t m, int32_t n, asamd_complex16 alpha, const asamd_complex16* ell_val,
+                  const int32_t* ell_col_ind, int32_t ell_width, int32_t base, const asamd_complex16* x,
+                  asamd_complex16 beta, asamd_complex16* y) {
+  using T = asamd::Cx<double>;
+  return asamd::ellmv_impl<T>(stream, m, n, T(alpha.real, alpha.imag), (const T*)ell_val, ell_col_ind, ell_width,
+                              base, (const T*)x, T(beta.real, beta.imag), (T*)y);
+}
+
+int asamd_c_coomv(hipStream_t stream, int32_t m, int32_t n, int64_t nnz, asamd_complex8 alpha,
+                  const asamd_complex8* coo_val, const int32_t* coo_row_ind, const int32_t* coo_col_ind,
+                  int32_t base, const asamd_complex8* x, asamd_complex8 beta, asamd_complex8* y) {
+  using T = asamd::Cx<float>;
+  return asamd::coomv_impl<T>(stream, m, n, nnz, T(alpha.real, alpha.imag), (const T*)coo_val, coo_row_ind,
+                              coo_col_ind, base, (const T*)x, T(beta.real, beta.imag), (T*)y);
+}
+
+int asamd_z_coomv(hipStream_t stream, int32_t m, int32_t n, int64_t nnz, asamd_complex16 alpha,
+                  const asamd_complex16* coo_val, const int32_t* coo_row_ind, const int32_t* coo_col_ind,
+                  int32_t base, const asamd_complex16* x, asamd_complex16 beta, asamd_complex16* y) {
+  using T = asamd::Cx<double>;
+  return asamd::coomv_impl<T>(stream, m, n, nnz, T(alpha.real, alpha.imag), (const T*)coo_val, coo_row_ind,
+                              coo_col_ind, base, (const T*)x, T(beta.real, beta.imag), (T*)y);
 }
 
 }  // extern "C"

@@ -66,6 +66,11 @@ __device__ __forceinline__ double readlane_t(double v, int l) {
   return __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);
 }
 
+template <typename R>
+__device__ __forceinline__ Cx<R> readlane_t(Cx<R> v, int l) {
+  return Cx<R>(readlane_t(v.re, l), readlane_t(v.im, l));
+}
+
 // grid.x covers rows (one wave each), grid.y covers chunks of 64*V columns.
 template <typename T, int V>
 __global__ __launch_bounds__(kSpmmBlock) void spmm_rowmajor_kernel(
@@ -93,8 +98,8 @@ __global__ __launch_bounds__(kSpmmBlock) void spmm_rowmajor_kernel(
     T my_val = T(0);
     if (j < end) {
       // A and C are touched once: non-temporal, so that they do not push rows of B out of the caches
-      my_col = __builtin_nontemporal_load(col_ind + j) - base;
-      my_val = alpha * __builtin_nontemporal_load(val + j);
+      my_col = nt_load(col_ind + j) - base;
+      my_val = alpha * nt_load(val + j);
     }
     const int cnt = (int)(end - j0 < kWave ? end - j0 : kWave);
     int t = 0;
@@ -139,8 +144,8 @@ __global__ __launch_bounds__(kSpmmBlock) void spmm_rowmajor_kernel(
 #pragma unroll
     for (int i = 0; i < V; ++i) {
       if (i < valid) {
-        const T res = beta == T(0) ? acc[i] : __builtin_nontemporal_load(crow + i) * beta + acc[i];
-        __builtin_nontemporal_store(res, crow + i);
+        const T res = beta == T(0) ? acc[i] : nt_load(crow + i) * beta + acc[i];
+        nt_store(res, crow + i);
       }
     }
   }
@@ -212,7 +217,7 @@ __global__ __launch_bounds__(kSpmmBlock) void dense_transpose_kernel(int rows, i
   for (int i = ty; i < kWave; i += kSpmmWaves) {
     const int64_t r = r0 + tx;
     const int c = c0 + i;
-    tile[i][tx] = (r < rows && c < cols) ? __builtin_nontemporal_load(in + r + (int64_t)c * in_ld) : T(0);
+    tile[i][tx] = (r < rows && c < cols) ? nt_load(in + r + (int64_t)c * in_ld) : T(0);
   }
   __syncthreads();
 #pragma unroll 4
@@ -249,8 +254,8 @@ __global__ __launch_bounds__(kSpmmBlock) void spmm_colmajor_kernel(
         int my_col = 0;
         T my_val = T(0);
         if (j < end) {
-          my_col = __builtin_nontemporal_load(col_ind + j) - base;
-          my_val = alpha * __builtin_nontemporal_load(val + j);
+          my_col = nt_load(col_ind + j) - base;
+          my_val = alpha * nt_load(val + j);
         }
         const int cnt = (int)(end - j0 < kWave ? end - j0 : kWave);
         int t = 0;
@@ -283,8 +288,8 @@ __global__ __launch_bounds__(kSpmmBlock) void spmm_colmajor_kernel(
     if (c >= n) break;
     T* out = C + row + (int64_t)c * ldc;
     const T acc = tile[lane][cc];
-    const T res = beta == T(0) ? acc : __builtin_nontemporal_load(out) * beta + acc;
-    __builtin_nontemporal_store(res, out);
+    const T res = beta == T(0) ? acc : nt_load(out) * beta + acc;
+    nt_store(res, out);
   }
 }
 
@@ -327,6 +332,7 @@ static int csrmm_impl(hipStream_t s, int m, int n, int k, int nnz, T alpha, cons
                       const asamd_dense_strides* st, void* ws, size_t ws_bytes) {
   (void)nnz;
   if (!val || !rp || !ci || !B || !C || !st || m <= 0 || n <= 0) return hipErrorInvalidValue;
+  if (((uintptr_t)val | (uintptr_t)B | (uintptr_t)C) % alignof(T)) return hipErrorInvalidValue;
   if (n > 1 && st->c_row_stride == 1 && st->c_col_stride != 1) {
     // column-major C: rows of op(B) must be contiguous for the wave-wide loads
     const T* Bt = nullptr;
@@ -360,18 +366,23 @@ static int csrmm_impl(hipStream_t s, int m, int n, int k, int nnz, T alpha, cons
     }
     const unsigned gx = (unsigned)(((int64_t)m + kSpmmWaves - 1) / kSpmmWaves);
     // widest per-lane vector that still gives every lane of a wave work
+    constexpr int kMaxV = 32 / (int)sizeof(T) >= 4 ? 4 : 32 / (int)sizeof(T);  // at most 32 bytes per lane and load
     int V = 1;
-    if (n >= 4 * kWave) V = 4;
-    else if (n >= 2 * kWave) V = 2;
+    if (n >= 4 * kWave && kMaxV >= 4) V = 4;
+    else if (n >= 2 * kWave && kMaxV >= 2) V = 2;
     const size_t vbytes = (size_t)V * sizeof(T);
     const bool vector_ok = V > 1 && ((uintptr_t)B % vbytes == 0) && ((uintptr_t)C % vbytes == 0) &&
                            (ldb % V == 0) && (ldc % V == 0);
     const unsigned gy = (unsigned)((n + kWave * V - 1) / (kWave * V));
     const dim3 grid(gx, gy);
-    if (V == 4)
-      spmm_rowmajor_kernel<T, 4><<<grid, kSpmmBlock, 0, s>>>(m, n, alpha, val, rp, ci, base, B, ldb,
-                                                             beta, C, ldc, vector_ok);
-    else if (V == 2)
+    if constexpr (kMaxV >= 4) {
+      if (V == 4) {
+        spmm_rowmajor_kernel<T, 4><<<grid, kSpmmBlock, 0, s>>>(m, n, alpha, val, rp, ci, base, B, ldb,
+                                                               beta, C, ldc, vector_ok);
+        return hipGetLastError();
+      }
+    }
+    if (V == 2)
       spmm_rowmajor_kernel<T, 2><<<grid, kSpmmBlock, 0, s>>>(m, n, alpha, val, rp, ci, base, B, ldb,
                                                              beta, C, ldc, vector_ok);
     else
@@ -400,7 +411,7 @@ extern "C" int asamd_s_csrmm(hipStream_t stream, int32_t m, int32_t n, int32_t k
 extern "C" size_t asamd_csrmm_workspace_bytes(int32_t val_size, int32_t m, int32_t n, int32_t k,
                                               const asamd_dense_strides* strides) {
   (void)m;
-  return (val_size == 4 || val_size == 8) ? workspace_bytes((size_t)val_size, n, k, strides) : 0;
+  return (val_size == 4 || val_size == 8 || val_size == 16) ? workspace_bytes((size_t)val_size, n, k, strides) : 0;
 }
 
 extern "C" int asamd_s_csrmm_ws(hipStream_t stream, int32_t m, int32_t n, int32_t k, int32_t nnz, float alpha,
@@ -425,4 +436,28 @@ extern "C" int asamd_d_csrmm(hipStream_t stream, int32_t m, int32_t n, int32_t k
                              double* C, const asamd_dense_strides* strides) {
   return csrmm_impl<double>(stream, m, n, k, nnz, alpha, val, row_ptr, col_ind, base, B, beta, C,
                             strides, nullptr, 0);
+}
+
+// ---- complex element types: the same kernels over Cx<float> / Cx<double> -------------------
+static_assert(sizeof(asamd_complex8) == sizeof(Cx<float>) && sizeof(asamd_complex16) == sizeof(Cx<double>),
+              "complex layouts");
+
+extern "C" int asamd_c_csrmm_ws(hipStream_t stream, int32_t m, int32_t n, int32_t k, int32_t nnz,
+                                asamd_complex8 alpha, const asamd_complex8* val, const int32_t* row_ptr,
+                                const int32_t* col_ind, int32_t base, const asamd_complex8* B, asamd_complex8 beta,
+                                asamd_complex8* C, const asamd_dense_strides* strides, void* workspace,
+                                size_t workspace_bytes) {
+  using T = Cx<float>;
+  return csrmm_impl<T>(stream, m, n, k, nnz, T(alpha.real, alpha.imag), (const T*)val, row_ptr, col_ind, base,
+                       (const T*)B, T(beta.real, beta.imag), (T*)C, strides, workspace, workspace_bytes);
+}
+
+extern "C" int asamd_z_csrmm_ws(hipStream_t stream, int32_t m, int32_t n, int32_t k, int32_t nnz,
+                                asamd_complex16 alpha, const asamd_complex16* val, const int32_t* row_ptr,
+                                const int32_t* col_ind, int32_t base, const asamd_complex16* B,
+                                asamd_complex16 beta, asamd_complex16* C, const asamd_dense_strides* strides,
+                                void* workspace, size_t workspace_bytes) {
+  using T = Cx<double>;
+  return csrmm_impl<T>(stream, m, n, k, nnz, T(alpha.real, alpha.imag), (const T*)val, row_ptr, col_ind, base,
+                       (const T*)B, T(beta.real, beta.imag), (T*)C, strides, workspace, workspace_bytes);
 }

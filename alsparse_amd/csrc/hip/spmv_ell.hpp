@@ -33,7 +33,7 @@ __global__ __launch_bounds__(kEllThreads) void ellmv_kernel(int m, int n, T alph
     for (int u = 0; u < kEllUnroll; ++u) {
       const int64_t idx = (int64_t)(s + u) * m + row;
       c[u] = __builtin_nontemporal_load(&ell_col[idx]) - base;
-      v[u] = __builtin_nontemporal_load(&ell_val[idx]);
+      v[u] = nt_load(&ell_val[idx]);
     }
 #pragma unroll
     for (int u = 0; u < kEllUnroll; ++u) xv[u] = (unsigned)c[u] < (unsigned)n ? x[c[u]] : T(0);

@@ -195,7 +195,7 @@ __global__ __launch_bounds__(kMergeThreads) void spmv_merge_kernel(
   T tail = acc;
 #pragma unroll
   for (int d = 1; d < kWave; d <<= 1) {
-    const T up = __shfl_up(tail, d, kWave);
+    const T up = lane_up(tail, d);
     const int kup = __shfl_up(key, d, kWave);
     if (lane >= d && kup == key) tail += up;
   }

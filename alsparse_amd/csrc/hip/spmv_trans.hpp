@@ -10,7 +10,9 @@
 //     is what the reference always does, one lane per row
 //     (src/kernel/dcu/level2/mv/csrmv/dcu_gemv_x_csr_trans.cpp:11-45; its beta
 //     pass covers m elements of y where n are meant, :61-64); here W lanes share
-//     a row so that the entry loads coalesce.
+//     a row so that the entry loads coalesce.  CONJ conjugates the values on
+//     the way: y = alpha*A^H*x + beta*y, the reference's
+//     csr_gemv_conj_scalar_atomicadd (dcu_gemv_c_csr_conj.cpp:22-48).
 #pragma once
 
 #include "device_utils.hpp"
@@ -29,7 +31,8 @@ __global__ __launch_bounds__(256) void transpose_keys_kernel(int nnz, const int*
 }
 
 // entries of A^T in column-sorted order: zero-based row of A as the new column index
-template <typename T>
+// (CONJ: values conjugated, which makes the copy A^H)
+template <typename T, bool CONJ>
 __global__ __launch_bounds__(256) void transpose_gather_kernel(int nnz, const unsigned* __restrict__ perm,
                                                                const int* __restrict__ coo_row,
                                                                const T* __restrict__ val, int base,
@@ -38,7 +41,7 @@ __global__ __launch_bounds__(256) void transpose_gather_kernel(int nnz, const un
        q += (int64_t)gridDim.x * blockDim.x) {
     const unsigned k = perm[q];
     t_col[q] = coo_row[k] - base;
-    t_val[q] = val[k];
+    t_val[q] = CONJ ? conj_t(val[k]) : val[k];
   }
 }
 
@@ -52,7 +55,7 @@ __global__ __launch_bounds__(256) void scale_vec_kernel(int n, T beta, T* __rest
 
 constexpr int kTransThreads = 256;
 
-template <typename T, int W>
+template <typename T, int W, bool CONJ>
 __global__ __launch_bounds__(kTransThreads) void csrmv_trans_scatter_kernel(
     int m, int n, T alpha, const T* __restrict__ val, const int* __restrict__ row_ptr,
     const int* __restrict__ col_ind, const T* __restrict__ x, T* __restrict__ y, int base) {
@@ -63,7 +66,7 @@ __global__ __launch_bounds__(kTransThreads) void csrmv_trans_scatter_kernel(
   const int64_t b = (int64_t)row_ptr[row] - base, e = (int64_t)row_ptr[row + 1] - base;
   for (int64_t k = b + sub; k < e; k += W) {
     const int c = col_ind[k] - base;
-    if ((unsigned)c < (unsigned)n) atomicAdd(&y[c], val[k] * t);
+    if ((unsigned)c < (unsigned)n) atomic_add(&y[c], (CONJ ? conj_t(val[k]) : val[k]) * t);
   }
 }
 

@@ -66,6 +66,8 @@ alphasparse_status_t alphasparse_dcu_csr2ell_width(alphasparse_dcu_handle_t hand
     if (csr_val == NULL || csr_row_ptr == NULL || csr_col_ind == NULL || ell_val == NULL ||        \
         ell_col_ind == NULL)                                                                       \
       return ALPHA_SPARSE_STATUS_INVALID_POINTER;                                                  \
+    if (ASAMD_MISALIGNED(T, csr_val) || ASAMD_MISALIGNED(T, ell_val))                              \
+      return ALPHA_SPARSE_STATUS_INVALID_VALUE;                                                    \
     ASAMD_HIP_STATUS(KERNEL(handle->stream, m, csr_val, csr_row_ptr, csr_col_ind,                  \
                             (int32_t)csr_descr->base, (int32_t)ell_descr->base, ell_width,         \
                             ell_val, ell_col_ind));                                                \
@@ -74,3 +76,5 @@ alphasparse_status_t alphasparse_dcu_csr2ell_width(alphasparse_dcu_handle_t hand
 
 ASAMD_CSR2ELL(alphasparse_dcu_scsr2ell, float, asamd_s_csr2ell)
 ASAMD_CSR2ELL(alphasparse_dcu_dcsr2ell, double, asamd_d_csr2ell)
+ASAMD_CSR2ELL(alphasparse_dcu_ccsr2ell, ALPHA_Complex8, asamd_c_csr2ell)
+ASAMD_CSR2ELL(alphasparse_dcu_zcsr2ell, ALPHA_Complex16, asamd_z_csr2ell)

@@ -48,6 +48,19 @@
   }
 ASAMD_CREATE_COO(alphasparse_s_create_coo, float, spmat_coo_s_t, ALPHA_SPARSE_DATATYPE_FLOAT)
 ASAMD_CREATE_COO(alphasparse_d_create_coo, double, spmat_coo_d_t, ALPHA_SPARSE_DATATYPE_DOUBLE)
+ASAMD_CREATE_COO(alphasparse_c_create_coo, ALPHA_Complex8, spmat_coo_c_t, ALPHA_SPARSE_DATATYPE_FLOAT_COMPLEX)
+ASAMD_CREATE_COO(alphasparse_z_create_coo, ALPHA_Complex16, spmat_coo_z_t, ALPHA_SPARSE_DATATYPE_DOUBLE_COMPLEX)
+
+/* bytes per value of a datatype tag, 0 for an unknown tag */
+static size_t value_size(alphasparse_datatype_t dt) {
+  switch (dt) {
+    case ALPHA_SPARSE_DATATYPE_FLOAT: return sizeof(float);
+    case ALPHA_SPARSE_DATATYPE_DOUBLE: return sizeof(double);
+    case ALPHA_SPARSE_DATATYPE_FLOAT_COMPLEX: return sizeof(ALPHA_Complex8);
+    case ALPHA_SPARSE_DATATYPE_DOUBLE_COMPLEX: return sizeof(ALPHA_Complex16);
+    default: return 0;
+  }
+}
 
 /* Position of every entry in (row, column) order, ties in source order: a
  * counting sort by row, then each row's slice ordered by (column, position). */
@@ -69,10 +82,10 @@ alphasparse_status_t alphasparse_convert_csr(const alphasparse_matrix_t source,
   if (!dest) return ALPHA_SPARSE_STATUS_INVALID_POINTER;
   *dest = NULL;
   if (source->format != ALPHA_SPARSE_FORMAT_COO) return ALPHA_SPARSE_STATUS_INVALID_VALUE;
-  if (source->datatype != ALPHA_SPARSE_DATATYPE_FLOAT && source->datatype != ALPHA_SPARSE_DATATYPE_DOUBLE)
-    return ALPHA_SPARSE_STATUS_INVALID_VALUE;
+  const size_t vsize = value_size(source->datatype);
+  if (vsize == 0) return ALPHA_SPARSE_STATUS_INVALID_VALUE;
   if (operation != ALPHA_SPARSE_OPERATION_NON_TRANSPOSE) return ALPHA_SPARSE_STATUS_NOT_SUPPORTED;
-  /* both COO payloads share one layout up to the value pointer type */
+  /* the COO payloads of all value types share one layout up to the value pointer type */
   const spmat_coo_s_t *coo = (const spmat_coo_s_t *)source->mat;
   const ALPHA_INT m = coo->rows, nnz = coo->nnz;
   for (ALPHA_INT i = 0; i < nnz; ++i)
@@ -98,25 +111,29 @@ alphasparse_status_t alphasparse_convert_csr(const alphasparse_matrix_t source,
     qsort(order + offsets[r], (size_t)(offsets[r + 1] - offsets[r]), sizeof(col_pos), col_pos_cmp);
   for (ALPHA_INT i = 0; i < nnz; ++i) cols[i] = order[i].col;
   alphasparse_status_t st;
-  if (source->datatype == ALPHA_SPARSE_DATATYPE_FLOAT) {
-    float *vals = (float *)malloc((size_t)(nnz ? nnz : 1) * sizeof(float));
-    if (!vals) {
-      st = ALPHA_SPARSE_STATUS_ALLOC_FAILED;
-    } else {
-      for (ALPHA_INT i = 0; i < nnz; ++i) vals[i] = coo->values[order[i].pos];
-      st = alphasparse_s_create_csr(dest, ALPHA_SPARSE_INDEX_BASE_ZERO, m, coo->cols, offsets, offsets + 1, cols, vals);
-      free(vals);
-    }
+  /* values are moved as opaque vsize-byte items */
+  char *vals = (char *)malloc((size_t)(nnz ? nnz : 1) * vsize);
+  if (!vals) {
+    st = ALPHA_SPARSE_STATUS_ALLOC_FAILED;
   } else {
-    const double *src = ((const spmat_coo_d_t *)source->mat)->values;
-    double *vals = (double *)malloc((size_t)(nnz ? nnz : 1) * sizeof(double));
-    if (!vals) {
-      st = ALPHA_SPARSE_STATUS_ALLOC_FAILED;
-    } else {
-      for (ALPHA_INT i = 0; i < nnz; ++i) vals[i] = src[order[i].pos];
-      st = alphasparse_d_create_csr(dest, ALPHA_SPARSE_INDEX_BASE_ZERO, m, coo->cols, offsets, offsets + 1, cols, vals);
-      free(vals);
+    const char *src = (const char *)coo->values;
+    for (ALPHA_INT i = 0; i < nnz; ++i) memcpy(vals + (size_t)i * vsize, src + (size_t)order[i].pos * vsize, vsize);
+    const alphasparse_index_base_t b0 = ALPHA_SPARSE_INDEX_BASE_ZERO;
+    switch (source->datatype) {
+      case ALPHA_SPARSE_DATATYPE_FLOAT:
+        st = alphasparse_s_create_csr(dest, b0, m, coo->cols, offsets, offsets + 1, cols, (float *)vals);
+        break;
+      case ALPHA_SPARSE_DATATYPE_DOUBLE:
+        st = alphasparse_d_create_csr(dest, b0, m, coo->cols, offsets, offsets + 1, cols, (double *)vals);
+        break;
+      case ALPHA_SPARSE_DATATYPE_FLOAT_COMPLEX:
+        st = alphasparse_c_create_csr(dest, b0, m, coo->cols, offsets, offsets + 1, cols, (ALPHA_Complex8 *)vals);
+        break;
+      default:
+        st = alphasparse_z_create_csr(dest, b0, m, coo->cols, offsets, offsets + 1, cols, (ALPHA_Complex16 *)vals);
+        break;
     }
+    free(vals);
   }
   free(offsets);
   free(fill);
@@ -145,8 +162,7 @@ alphasparse_status_t alphasparse_convert_ell(const alphasparse_matrix_t source,
     const ALPHA_INT len = c->rows_end[r] - c->rows_start[r];
     if (len > ld) ld = len;
   }
-  const int is_s = source->datatype == ALPHA_SPARSE_DATATYPE_FLOAT;
-  const size_t vsize = is_s ? sizeof(float) : sizeof(double);
+  const size_t vsize = value_size(source->datatype);
   const uint64_t slots = (uint64_t)ld * (uint64_t)m;
   alphasparse_matrix *AA = NULL;
   spmat_ell_s_t *ell = NULL;
@@ -167,8 +183,7 @@ alphasparse_status_t alphasparse_convert_ell(const alphasparse_matrix_t source,
       for (ALPHA_INT k = b; k < e; ++k) {
         const size_t at = (size_t)(k - b) * (size_t)m + (size_t)r;
         idx[at] = c->col_indx[k];
-        if (is_s) ((float *)vals)[at] = c->values[k];
-        else ((double *)vals)[at] = ((const spmat_csr_d_t *)csr->mat)->values[k];
+        memcpy((char *)vals + at * vsize, (const char *)c->values + (size_t)k * vsize, vsize);
       }
     }
     ell->values = (float *)vals;
@@ -205,6 +220,8 @@ alphasparse_status_t alphasparse_convert_ell(const alphasparse_matrix_t source,
   }
 ASAMD_EXPORT_ELL(alphasparse_s_export_ell, float, spmat_ell_s_t, ALPHA_SPARSE_DATATYPE_FLOAT)
 ASAMD_EXPORT_ELL(alphasparse_d_export_ell, double, spmat_ell_d_t, ALPHA_SPARSE_DATATYPE_DOUBLE)
+ASAMD_EXPORT_ELL(alphasparse_c_export_ell, ALPHA_Complex8, spmat_ell_c_t, ALPHA_SPARSE_DATATYPE_FLOAT_COMPLEX)
+ASAMD_EXPORT_ELL(alphasparse_z_export_ell, ALPHA_Complex16, spmat_ell_z_t, ALPHA_SPARSE_DATATYPE_DOUBLE_COMPLEX)
 
 /* ---- device mirrors of COO / ELL handles ------------------------------------
  * src/core/format/host2device_x_coo.cpp:14-40, host2device_x_ell.cpp:14-33.  The
@@ -244,6 +261,12 @@ alphasparse_status_t host2device_s_coo(alphasparse_matrix_t mtx) {
 alphasparse_status_t host2device_d_coo(alphasparse_matrix_t mtx) {
   return host2device_coo(mtx, ALPHA_SPARSE_DATATYPE_DOUBLE, sizeof(double));
 }
+alphasparse_status_t host2device_c_coo(alphasparse_matrix_t mtx) {
+  return host2device_coo(mtx, ALPHA_SPARSE_DATATYPE_FLOAT_COMPLEX, sizeof(ALPHA_Complex8));
+}
+alphasparse_status_t host2device_z_coo(alphasparse_matrix_t mtx) {
+  return host2device_coo(mtx, ALPHA_SPARSE_DATATYPE_DOUBLE_COMPLEX, sizeof(ALPHA_Complex16));
+}
 
 static alphasparse_status_t host2device_ell(alphasparse_matrix_t mtx, alphasparse_datatype_t dt, size_t vsize) {
   if (!mtx) return ALPHA_SPARSE_STATUS_INVALID_POINTER;
@@ -264,4 +287,10 @@ alphasparse_status_t host2device_s_ell(alphasparse_matrix_t mtx) {
 }
 alphasparse_status_t host2device_d_ell(alphasparse_matrix_t mtx) {
   return host2device_ell(mtx, ALPHA_SPARSE_DATATYPE_DOUBLE, sizeof(double));
+}
+alphasparse_status_t host2device_c_ell(alphasparse_matrix_t mtx) {
+  return host2device_ell(mtx, ALPHA_SPARSE_DATATYPE_FLOAT_COMPLEX, sizeof(ALPHA_Complex8));
+}
+alphasparse_status_t host2device_z_ell(alphasparse_matrix_t mtx) {
+  return host2device_ell(mtx, ALPHA_SPARSE_DATATYPE_DOUBLE_COMPLEX, sizeof(ALPHA_Complex16));
 }

@@ -35,13 +35,33 @@ static void asamd_release_mirror(void *d_row_ptr, void *d_col, void *d_val) {
 #undef ASAMD_CSR
 #undef ASAMD_DT
 
+#define ASAMD_T ALPHA_Complex8
+#define ASAMD_S c
+#define ASAMD_CSR spmat_csr_c_t
+#define ASAMD_DT ALPHA_SPARSE_DATATYPE_FLOAT_COMPLEX
+#include "csr_matrix.inc"
+#undef ASAMD_T
+#undef ASAMD_S
+#undef ASAMD_CSR
+#undef ASAMD_DT
+
+#define ASAMD_T ALPHA_Complex16
+#define ASAMD_S z
+#define ASAMD_CSR spmat_csr_z_t
+#define ASAMD_DT ALPHA_SPARSE_DATATYPE_DOUBLE_COMPLEX
+#include "csr_matrix.inc"
+#undef ASAMD_T
+#undef ASAMD_S
+#undef ASAMD_CSR
+#undef ASAMD_DT
+
 alphasparse_status_t alphasparse_destroy(alphasparse_matrix_t A) {
   if (!A) return ALPHA_SPARSE_STATUS_SUCCESS;
   if (A->mat) {
     if (A->format != ALPHA_SPARSE_FORMAT_CSR && A->format != ALPHA_SPARSE_FORMAT_COO &&
         A->format != ALPHA_SPARSE_FORMAT_ELL)
       return ALPHA_SPARSE_STATUS_INVALID_VALUE;
-    if (A->datatype != ALPHA_SPARSE_DATATYPE_FLOAT && A->datatype != ALPHA_SPARSE_DATATYPE_DOUBLE)
+    if (A->datatype < ALPHA_SPARSE_DATATYPE_FLOAT || A->datatype > ALPHA_SPARSE_DATATYPE_DOUBLE_COMPLEX)
       return ALPHA_SPARSE_STATUS_INVALID_VALUE;
     if (A->format == ALPHA_SPARSE_FORMAT_ELL) { /* src/core/format/destroy_x_ell.c */
       spmat_ell_s_t *e = (spmat_ell_s_t *)A->mat;
@@ -65,7 +85,7 @@ alphasparse_status_t alphasparse_destroy(alphasparse_matrix_t A) {
       free(A);
       return ALPHA_SPARSE_STATUS_SUCCESS;
     }
-    /* both payload structs share one layout up to the value pointer types */
+    /* the payload structs of all value types share one layout up to the value pointer types */
     spmat_csr_s_t *m = (spmat_csr_s_t *)A->mat;
     if (m->d_row_ptr && asamd_registry_find(ASAMD_KEY_MATRIX, m->d_row_ptr))
       asamd_release_mirror(m->d_row_ptr, m->d_col_indx, m->d_values);

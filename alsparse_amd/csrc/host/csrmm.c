@@ -16,3 +16,19 @@
 #undef ASAMD_T
 #undef ASAMD_S
 #undef ASAMD_KERNEL_CSRMM
+
+#define ASAMD_T ALPHA_Complex8
+#define ASAMD_S c
+#define ASAMD_KERNEL_CSRMM asamd_c_csrmm_ws
+#include "csrmm.inc"
+#undef ASAMD_T
+#undef ASAMD_S
+#undef ASAMD_KERNEL_CSRMM
+
+#define ASAMD_T ALPHA_Complex16
+#define ASAMD_S z
+#define ASAMD_KERNEL_CSRMM asamd_z_csrmm_ws
+#include "csrmm.inc"
+#undef ASAMD_T
+#undef ASAMD_S
+#undef ASAMD_KERNEL_CSRMM

@@ -11,14 +11,19 @@
 #include "internal.h"
 
 /* Make sure A has a device mirror built by this library and return its record. */
-static alphasparse_status_t asamd_host_prepare(const alphasparse_matrix_t A, size_t val_size,
-                                               alphasparse_dcu_handle_t *h, asamd_record **rec) {
+static alphasparse_status_t asamd_host_prepare(const alphasparse_matrix_t A, alphasparse_dcu_handle_t *h,
+                                               asamd_record **rec) {
   alphasparse_status_t st = asamd_default_handle(h);
   if (st != ALPHA_SPARSE_STATUS_SUCCESS) return st;
-  spmat_csr_s_t *m = (spmat_csr_s_t *)A->mat; /* s and d payloads share the layout */
+  spmat_csr_s_t *m = (spmat_csr_s_t *)A->mat; /* the payloads of all value types share the layout */
   asamd_record *r = m->d_row_ptr ? asamd_registry_find(ASAMD_KEY_MATRIX, m->d_row_ptr) : NULL;
   if (!r) {
-    st = val_size == sizeof(float) ? host2device_s_csr(A) : host2device_d_csr(A);
+    switch (A->datatype) {
+      case ALPHA_SPARSE_DATATYPE_FLOAT: st = host2device_s_csr(A); break;
+      case ALPHA_SPARSE_DATATYPE_DOUBLE: st = host2device_d_csr(A); break;
+      case ALPHA_SPARSE_DATATYPE_FLOAT_COMPLEX: st = host2device_c_csr(A); break;
+      default: st = host2device_z_csr(A); break;
+    }
     if (st != ALPHA_SPARSE_STATUS_SUCCESS) return st;
     r = asamd_registry_find(ASAMD_KEY_MATRIX, m->d_row_ptr);
     if (!r) return ALPHA_SPARSE_STATUS_INTERNAL_ERROR;
@@ -46,22 +51,76 @@ static alphasparse_status_t asamd_host_stage(asamd_record *rec, size_t in_bytes,
   return ALPHA_SPARSE_STATUS_SUCCESS;
 }
 
+/* beta*y with the operation order of the reference's cmp_mule
+ * (include/alphasparse/complex_compute.h:76-82, :103) */
+#define ASAMD_CX_SCALE(R, y, b)                            \
+  do {                                                     \
+    const R re_ = (b).real * (y).real - (b).imag * (y).imag; \
+    const R im_ = (b).imag * (y).real + (b).real * (y).imag; \
+    (y).real = re_;                                        \
+    (y).imag = im_;                                        \
+  } while (0)
+
 #define ASAMD_T float
 #define ASAMD_S s
 #define ASAMD_CSR spmat_csr_s_t
 #define ASAMD_DT ALPHA_SPARSE_DATATYPE_FLOAT
+#define ASAMD_IS_COMPLEX 0
+#define ASAMD_IS_ZERO(v) ((v) == 0)
+#define ASAMD_SCALE(y, b) ((y) *= (b))
 #include "host_api.inc"
 #undef ASAMD_T
 #undef ASAMD_S
 #undef ASAMD_CSR
 #undef ASAMD_DT
+#undef ASAMD_IS_COMPLEX
+#undef ASAMD_IS_ZERO
+#undef ASAMD_SCALE
 
 #define ASAMD_T double
 #define ASAMD_S d
 #define ASAMD_CSR spmat_csr_d_t
 #define ASAMD_DT ALPHA_SPARSE_DATATYPE_DOUBLE
+#define ASAMD_IS_COMPLEX 0
+#define ASAMD_IS_ZERO(v) ((v) == 0)
+#define ASAMD_SCALE(y, b) ((y) *= (b))
 #include "host_api.inc"
 #undef ASAMD_T
 #undef ASAMD_S
 #undef ASAMD_CSR
 #undef ASAMD_DT
+#undef ASAMD_IS_COMPLEX
+#undef ASAMD_IS_ZERO
+#undef ASAMD_SCALE
+
+#define ASAMD_T ALPHA_Complex8
+#define ASAMD_S c
+#define ASAMD_CSR spmat_csr_c_t
+#define ASAMD_DT ALPHA_SPARSE_DATATYPE_FLOAT_COMPLEX
+#define ASAMD_IS_COMPLEX 1
+#define ASAMD_IS_ZERO(v) ((v).real == 0 && (v).imag == 0)
+#define ASAMD_SCALE(y, b) ASAMD_CX_SCALE(float, y, b)
+#include "host_api.inc"
+#undef ASAMD_T
+#undef ASAMD_S
+#undef ASAMD_CSR
+#undef ASAMD_DT
+#undef ASAMD_IS_COMPLEX
+#undef ASAMD_IS_ZERO
+#undef ASAMD_SCALE
+
+#define ASAMD_T ALPHA_Complex16
+#define ASAMD_S z
+#define ASAMD_CSR spmat_csr_z_t
+#define ASAMD_DT ALPHA_SPARSE_DATATYPE_DOUBLE_COMPLEX
+#define ASAMD_IS_COMPLEX 1
+#define ASAMD_IS_ZERO(v) ((v).real == 0 && (v).imag == 0)
+#define ASAMD_SCALE(y, b) ASAMD_CX_SCALE(double, y, b)
+#include "host_api.inc"
+#undef ASAMD_T
+#undef ASAMD_S
+#undef ASAMD_CSR
+#undef ASAMD_DT
+#undef ASAMD_IS_COMPLEX
+#undef ASAMD_IS_ZERO
+#undef ASAMD_SCALE

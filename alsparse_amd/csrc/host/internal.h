@@ -4,6 +4,8 @@
 #ifndef ALSPARSE_AMD_HOST_INTERNAL_H
 #define ALSPARSE_AMD_HOST_INTERNAL_H
 
+#include <stdint.h>
+
 #include "alpha_spblas_dcu.h"
 #include "alsparse_amd_kernels.h"
 
@@ -20,7 +22,7 @@ typedef struct asamd_record {
   /* what the plan was built for; a lookup must match all of these */
   const void *row_ptr;
   const void *col_ind;
-  int32_t m, n, nnz, base, val_size;
+  int32_t m, n, nnz, base, dtype; /* dtype: enum asamd_dtype == alphasparse_datatype_t */
   asamd_csr_plan *plan;
   /* host-pointer entry points: device staging for x / y (ASAMD_KEY_MATRIX only) */
   void *d_in;
@@ -43,7 +45,7 @@ void asamd_record_release_device(asamd_record *rec);
  * is known and matches, else the lazy cache (created on first use). */
 alphasparse_status_t asamd_plan_for_call(alphasparse_dcu_handle_t handle, const void *info,
                                          const void *row_ptr, const void *col_ind, int32_t m,
-                                         int32_t n, int32_t nnz, int32_t base, int32_t val_size,
+                                         int32_t n, int32_t nnz, int32_t base, int32_t dtype,
                                          asamd_csr_plan **plan);
 
 /* Process-wide handle for alphasparse_?_mv / _mm (host pointers). */
@@ -51,6 +53,9 @@ alphasparse_status_t asamd_default_handle(alphasparse_dcu_handle_t *handle);
 
 /* ALSPARSE_AMD_SPMV_ALGO = auto | vector | rowconst | merge | scalar | tiled | stream | ell */
 int asamd_env_algo(void);
+
+/* device arrays of values must be aligned to their element size (one element = one load) */
+#define ASAMD_MISALIGNED(T, p) (((uintptr_t)(p)) % sizeof(T) != 0)
 
 #define ASAMD_HIP_STATUS(expr)                                           \
   do {                                                                   \

@@ -58,20 +58,20 @@ void asamd_registry_erase(asamd_key_kind kind, const void *key) {
 }
 
 static int record_matches(const asamd_record *r, const void *row_ptr, const void *col_ind,
-                          int32_t m, int32_t n, int32_t nnz, int32_t base, int32_t val_size) {
+                          int32_t m, int32_t n, int32_t nnz, int32_t base, int32_t dtype) {
   return r->plan && r->row_ptr == row_ptr && (col_ind == NULL || r->col_ind == col_ind) &&
-         r->m == m && r->n == n && r->nnz == nnz && r->base == base && r->val_size == val_size;
+         r->m == m && r->n == n && r->nnz == nnz && r->base == base && r->dtype == dtype;
 }
 
 alphasparse_status_t asamd_plan_for_call(alphasparse_dcu_handle_t handle, const void *info,
                                          const void *row_ptr, const void *col_ind, int32_t m,
-                                         int32_t n, int32_t nnz, int32_t base, int32_t val_size,
+                                         int32_t n, int32_t nnz, int32_t base, int32_t dtype,
                                          asamd_csr_plan **plan) {
   /* 1. an explicit analysis of exactly these arrays (info may be garbage: it is
    *    only ever compared by address, never dereferenced) */
   if (info) {
     asamd_record *r = asamd_registry_find(ASAMD_KEY_INFO, info);
-    if (r && record_matches(r, row_ptr, col_ind, m, n, nnz, base, val_size)) {
+    if (r && record_matches(r, row_ptr, col_ind, m, n, nnz, base, dtype)) {
       *plan = r->plan;
       return ALPHA_SPARSE_STATUS_SUCCESS;
     }
@@ -79,7 +79,7 @@ alphasparse_status_t asamd_plan_for_call(alphasparse_dcu_handle_t handle, const 
   /* 2. a device mirror that this library built (alphasparse_?_mv_dcu path) */
   {
     asamd_record *r = asamd_registry_find(ASAMD_KEY_MATRIX, row_ptr);
-    if (r && record_matches(r, row_ptr, col_ind, m, n, nnz, base, val_size)) {
+    if (r && record_matches(r, row_ptr, col_ind, m, n, nnz, base, dtype)) {
       *plan = r->plan;
       return ALPHA_SPARSE_STATUS_SUCCESS;
     }
@@ -89,14 +89,14 @@ alphasparse_status_t asamd_plan_for_call(alphasparse_dcu_handle_t handle, const 
    *    steers the kernel choice, and every kernel it can pick reads row_ptr
    *    afresh on each call. */
   asamd_record *r = asamd_registry_find(ASAMD_KEY_LAZY, row_ptr);
-  if (r && !record_matches(r, row_ptr, NULL, m, n, nnz, base, val_size)) {
+  if (r && !record_matches(r, row_ptr, NULL, m, n, nnz, base, dtype)) {
     asamd_registry_erase(ASAMD_KEY_LAZY, row_ptr);
     r = NULL;
   }
   if (!r) {
     asamd_csr_plan *p = NULL;
-    ASAMD_HIP_STATUS(asamd_csr_plan_create(handle->stream, m, n, nnz, (const int32_t *)row_ptr,
-                                           NULL, NULL, base, val_size, /*trusted=*/0, &p));
+    ASAMD_HIP_STATUS(asamd_csr_plan_create_dtype(handle->stream, m, n, nnz, (const int32_t *)row_ptr,
+                                           NULL, NULL, base, dtype, /*trusted=*/0, &p));
     r = asamd_registry_insert(ASAMD_KEY_LAZY, row_ptr);
     if (!r) {
       asamd_csr_plan_destroy(p);
@@ -108,7 +108,7 @@ alphasparse_status_t asamd_plan_for_call(alphasparse_dcu_handle_t handle, const 
     r->n = n;
     r->nnz = nnz;
     r->base = base;
-    r->val_size = val_size;
+    r->dtype = dtype;
     r->plan = p;
     const int forced = asamd_env_algo();
     if (forced != ASAMD_SPMV_AUTO) (void)asamd_csr_plan_set_algo(p, forced);

@@ -44,6 +44,15 @@ void alpha_fill_random_d(double *arr, unsigned int seed, const size_t size) {
   for (size_t i = 0; i < size; ++i) arr[i] = (double)rand() / (double)RAND_MAX;
 }
 
+/* src/util/malloc.c:104-112: a complex array is filled as twice as many reals */
+void alpha_fill_random_c(ALPHA_Complex8 *arr, unsigned int seed, const size_t size) {
+  alpha_fill_random_s((float *)arr, seed, size * 2);
+}
+
+void alpha_fill_random_z(ALPHA_Complex16 *arr, unsigned int seed, const size_t size) {
+  alpha_fill_random_d((double *)arr, seed, size * 2);
+}
+
 /* ---- Matrix Market coordinate reader ------------------------------------- */
 typedef struct {
   ALPHA_INT m, n, nnz;
@@ -138,6 +147,38 @@ void alpha_read_coo_d(const char *file, ALPHA_INT *m_p, ALPHA_INT *n_p, ALPHA_IN
   *values = t.val;
 }
 
+/* src/util/io.c:193-268, :270-345: the one value of a line becomes both the real and the
+ * imaginary part (a line without a value reads as 1 + 1i) */
+void alpha_read_coo_c(const char *file, ALPHA_INT *m_p, ALPHA_INT *n_p, ALPHA_INT *nnz_p,
+                      ALPHA_INT **row_index, ALPHA_INT **col_index, ALPHA_Complex8 **values) {
+  coo_triplets t;
+  read_coo_triplets(file, &t);
+  ALPHA_Complex8 *v = (ALPHA_Complex8 *)alpha_malloc((size_t)t.nnz * sizeof(ALPHA_Complex8));
+  for (ALPHA_INT i = 0; i < t.nnz; ++i) v[i].real = v[i].imag = (float)t.val[i];
+  alpha_free(t.val);
+  *m_p = t.m;
+  *n_p = t.n;
+  *nnz_p = t.nnz;
+  *row_index = t.row;
+  *col_index = t.col;
+  *values = v;
+}
+
+void alpha_read_coo_z(const char *file, ALPHA_INT *m_p, ALPHA_INT *n_p, ALPHA_INT *nnz_p,
+                      ALPHA_INT **row_index, ALPHA_INT **col_index, ALPHA_Complex16 **values) {
+  coo_triplets t;
+  read_coo_triplets(file, &t);
+  ALPHA_Complex16 *v = (ALPHA_Complex16 *)alpha_malloc((size_t)t.nnz * sizeof(ALPHA_Complex16));
+  for (ALPHA_INT i = 0; i < t.nnz; ++i) v[i].real = v[i].imag = t.val[i];
+  alpha_free(t.val);
+  *m_p = t.m;
+  *n_p = t.n;
+  *nnz_p = t.nnz;
+  *row_index = t.row;
+  *col_index = t.col;
+  *values = v;
+}
+
 /* ---- result check ---------------------------------------------------------- */
 #define ASAMD_CHECK(NAME, T, FABS, TOL)                                                          \
   int NAME(const T *answer_data, size_t answer_size, const T *result_data, size_t result_size) { \
@@ -165,6 +206,17 @@ void alpha_read_coo_d(const char *file, ALPHA_INT *m_p, ALPHA_INT *n_p, ALPHA_IN
   }
 ASAMD_CHECK(check_s, float, fabsf, 2e-5)
 ASAMD_CHECK(check_d, double, fabs, 1e-10)
+
+/* src/util/check.c:778-786: complex arrays are compared as twice as many reals */
+int check_c(const ALPHA_Complex8 *answer_data, size_t answer_size, const ALPHA_Complex8 *result_data,
+            size_t result_size) {
+  return check_s((const float *)answer_data, answer_size * 2, (const float *)result_data, result_size * 2);
+}
+
+int check_z(const ALPHA_Complex16 *answer_data, size_t answer_size, const ALPHA_Complex16 *result_data,
+            size_t result_size) {
+  return check_d((const double *)answer_data, answer_size * 2, (const double *)result_data, result_size * 2);
+}
 
 /* ---- command line ---------------------------------------------------------- */
 enum {

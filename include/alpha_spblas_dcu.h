@@ -48,11 +48,6 @@ typedef enum {
   ALPHA_SPARSE_DCU_LAYER_MODE_LOG_BENCH = 2
 } alphasparse_dcu_layer_mode_t;
 
-/* complex scalars only appear as pointer members of the handle:
- * include/alphasparse/types.h:43-57 */
-typedef struct { float real, imag; } ALPHA_Complex8;
-typedef struct { double real, imag; } ALPHA_Complex16;
-
 /* ---- library handle: include/alphasparse/handle.h:18-46 -------------------
  * Field order is ABI.  `buffer` is device scratch owned by the handle; this
  * library uses it for merge-path carries and reduction partials. */
@@ -304,6 +299,100 @@ alphasparse_status_t alphasparse_dcu_d_ellmv(alphasparse_dcu_handle_t handle,
                                              ALPHA_INT ell_width, const double *x, const double *beta,
                                              double *y);
 
+/* ---- complex element types ---------------------------------------------------
+ * The same entry points for ALPHA_Complex8 (c) and ALPHA_Complex16 (z), with the
+ * semantics, validation order and extensions described at their fp32 / fp64
+ * namesakes above: include/alphasparse/spapi_dcu.h:4404-4405, :4414-4415, :4419-4420
+ * (host2device), :4459-4476 (mv_dcu), :549-570 (csrmv_analysis), :607-636 (csrmv),
+ * :1228-1265 (csrmm), :3334-3355 (csr2ell), :497-524 (coomv), :884-909 (ellmv).
+ * csrmv additionally accepts trans == CONJUGATE_TRANSPOSE, the third entry of the
+ * reference's dispatch table for complex types
+ * (src/core/op_dcu/level2/alphasparse_dcu_x_csrmv.cpp:17-35 over
+ * src/kernel/dcu/level2/mv/csrmv/dcu_gemv_c_csr_conj.cpp:22-75); an analysis asked
+ * for that operation keeps a CSR copy of A^H.  Device arrays of complex values must
+ * be aligned to the element size (INVALID_VALUE otherwise). */
+alphasparse_status_t host2device_c_csr(alphasparse_matrix_t A);
+alphasparse_status_t host2device_c_coo(alphasparse_matrix_t mtx);
+alphasparse_status_t host2device_c_ell(alphasparse_matrix_t mtx);
+alphasparse_status_t alphasparse_c_mv_dcu(alphasparse_dcu_handle_t handle,
+                                          const alphasparse_operation_t operation,
+                                          const ALPHA_Complex8 *alpha, const alphasparse_matrix_t A,
+                                          const alpha_dcu_matrix_descr_t descr, const ALPHA_Complex8 *x,
+                                          const ALPHA_Complex8 *beta, ALPHA_Complex8 *y);
+alphasparse_status_t alphasparse_dcu_c_csrmv_analysis(
+    alphasparse_dcu_handle_t handle, alphasparse_operation_t trans, ALPHA_INT m, ALPHA_INT n,
+    ALPHA_INT nnz, const alpha_dcu_matrix_descr_t descr, const ALPHA_Complex8 *csr_val,
+    const ALPHA_INT *csr_row_ptr, const ALPHA_INT *csr_col_ind, alphasparse_dcu_mat_info_t info);
+alphasparse_status_t alphasparse_dcu_c_csrmv(
+    alphasparse_dcu_handle_t handle, alphasparse_operation_t trans, ALPHA_INT m, ALPHA_INT n,
+    ALPHA_INT nnz, const ALPHA_Complex8 *alpha, const alpha_dcu_matrix_descr_t descr, const ALPHA_Complex8 *csr_val,
+    const ALPHA_INT *csr_row_ptr, const ALPHA_INT *csr_col_ind, alphasparse_dcu_mat_info_t info,
+    const ALPHA_Complex8 *x, const ALPHA_Complex8 *beta, ALPHA_Complex8 *y);
+alphasparse_status_t alphasparse_dcu_c_csrmm(
+    alphasparse_dcu_handle_t handle, alphasparse_operation_t trans_A,
+    alphasparse_operation_t trans_B, alphasparse_layout_t layout, ALPHA_INT m, ALPHA_INT n,
+    ALPHA_INT k, ALPHA_INT nnz, const ALPHA_Complex8 *alpha, const alpha_dcu_matrix_descr_t descr,
+    const ALPHA_Complex8 *csr_val, const ALPHA_INT *csr_row_ptr, const ALPHA_INT *csr_col_ind,
+    const ALPHA_Complex8 *B, ALPHA_INT ldb, const ALPHA_Complex8 *beta, ALPHA_Complex8 *C, ALPHA_INT ldc);
+alphasparse_status_t alphasparse_dcu_ccsr2ell(
+    alphasparse_dcu_handle_t handle, ALPHA_INT m, const alpha_dcu_matrix_descr_t csr_descr,
+    const ALPHA_Complex8 *csr_val, const ALPHA_INT *csr_row_ptr, const ALPHA_INT *csr_col_ind,
+    const alpha_dcu_matrix_descr_t ell_descr, ALPHA_INT ell_width, ALPHA_Complex8 *ell_val,
+    ALPHA_INT *ell_col_ind);
+alphasparse_status_t alphasparse_dcu_c_coomv(alphasparse_dcu_handle_t handle,
+                                             alphasparse_operation_t trans, ALPHA_INT m, ALPHA_INT n,
+                                             ALPHA_INT nnz, const ALPHA_Complex8 *alpha,
+                                             const alpha_dcu_matrix_descr_t descr, const ALPHA_Complex8 *coo_val,
+                                             const ALPHA_INT *coo_row_ind, const ALPHA_INT *coo_col_ind,
+                                             const ALPHA_Complex8 *x, const ALPHA_Complex8 *beta, ALPHA_Complex8 *y);
+alphasparse_status_t alphasparse_dcu_c_ellmv(alphasparse_dcu_handle_t handle,
+                                             alphasparse_operation_t trans, ALPHA_INT m, ALPHA_INT n,
+                                             const ALPHA_Complex8 *alpha, const alpha_dcu_matrix_descr_t descr,
+                                             const ALPHA_Complex8 *ell_val, const ALPHA_INT *ell_col_ind,
+                                             ALPHA_INT ell_width, const ALPHA_Complex8 *x, const ALPHA_Complex8 *beta,
+                                             ALPHA_Complex8 *y);
+
+alphasparse_status_t host2device_z_csr(alphasparse_matrix_t A);
+alphasparse_status_t host2device_z_coo(alphasparse_matrix_t mtx);
+alphasparse_status_t host2device_z_ell(alphasparse_matrix_t mtx);
+alphasparse_status_t alphasparse_z_mv_dcu(alphasparse_dcu_handle_t handle,
+                                          const alphasparse_operation_t operation,
+                                          const ALPHA_Complex16 *alpha, const alphasparse_matrix_t A,
+                                          const alpha_dcu_matrix_descr_t descr, const ALPHA_Complex16 *x,
+                                          const ALPHA_Complex16 *beta, ALPHA_Complex16 *y);
+alphasparse_status_t alphasparse_dcu_z_csrmv_analysis(
+    alphasparse_dcu_handle_t handle, alphasparse_operation_t trans, ALPHA_INT m, ALPHA_INT n,
+    ALPHA_INT nnz, const alpha_dcu_matrix_descr_t descr, const ALPHA_Complex16 *csr_val,
+    const ALPHA_INT *csr_row_ptr, const ALPHA_INT *csr_col_ind, alphasparse_dcu_mat_info_t info);
+alphasparse_status_t alphasparse_dcu_z_csrmv(
+    alphasparse_dcu_handle_t handle, alphasparse_operation_t trans, ALPHA_INT m, ALPHA_INT n,
+    ALPHA_INT nnz, const ALPHA_Complex16 *alpha, const alpha_dcu_matrix_descr_t descr, const ALPHA_Complex16 *csr_val,
+    const ALPHA_INT *csr_row_ptr, const ALPHA_INT *csr_col_ind, alphasparse_dcu_mat_info_t info,
+    const ALPHA_Complex16 *x, const ALPHA_Complex16 *beta, ALPHA_Complex16 *y);
+alphasparse_status_t alphasparse_dcu_z_csrmm(
+    alphasparse_dcu_handle_t handle, alphasparse_operation_t trans_A,
+    alphasparse_operation_t trans_B, alphasparse_layout_t layout, ALPHA_INT m, ALPHA_INT n,
+    ALPHA_INT k, ALPHA_INT nnz, const ALPHA_Complex16 *alpha, const alpha_dcu_matrix_descr_t descr,
+    const ALPHA_Complex16 *csr_val, const ALPHA_INT *csr_row_ptr, const ALPHA_INT *csr_col_ind,
+    const ALPHA_Complex16 *B, ALPHA_INT ldb, const ALPHA_Complex16 *beta, ALPHA_Complex16 *C, ALPHA_INT ldc);
+alphasparse_status_t alphasparse_dcu_zcsr2ell(
+    alphasparse_dcu_handle_t handle, ALPHA_INT m, const alpha_dcu_matrix_descr_t csr_descr,
+    const ALPHA_Complex16 *csr_val, const ALPHA_INT *csr_row_ptr, const ALPHA_INT *csr_col_ind,
+    const alpha_dcu_matrix_descr_t ell_descr, ALPHA_INT ell_width, ALPHA_Complex16 *ell_val,
+    ALPHA_INT *ell_col_ind);
+alphasparse_status_t alphasparse_dcu_z_coomv(alphasparse_dcu_handle_t handle,
+                                             alphasparse_operation_t trans, ALPHA_INT m, ALPHA_INT n,
+                                             ALPHA_INT nnz, const ALPHA_Complex16 *alpha,
+                                             const alpha_dcu_matrix_descr_t descr, const ALPHA_Complex16 *coo_val,
+                                             const ALPHA_INT *coo_row_ind, const ALPHA_INT *coo_col_ind,
+                                             const ALPHA_Complex16 *x, const ALPHA_Complex16 *beta, ALPHA_Complex16 *y);
+alphasparse_status_t alphasparse_dcu_z_ellmv(alphasparse_dcu_handle_t handle,
+                                             alphasparse_operation_t trans, ALPHA_INT m, ALPHA_INT n,
+                                             const ALPHA_Complex16 *alpha, const alpha_dcu_matrix_descr_t descr,
+                                             const ALPHA_Complex16 *ell_val, const ALPHA_INT *ell_col_ind,
+                                             ALPHA_INT ell_width, const ALPHA_Complex16 *x, const ALPHA_Complex16 *beta,
+                                             ALPHA_Complex16 *y);
+
 /* ---- generic (descriptor) SpMV -------------------------------------------------
  * Enums: include/alphasparse/spdef.h:209-213 (index types), :244-251 (algorithms).
  * Descriptors: include/alphasparse/handle.h:272-304.  The reference has no
@@ -359,7 +448,7 @@ typedef struct _alphasparse_dcu_dnvec_descr *alphasparse_dcu_dnvec_descr_t;
  * is run in the matrix's own precision (the reference always calls the fp32
  * one, :68-71), and a successful CSR / ELL multiply returns its status
  * (SUCCESS) where the reference falls through to NOT_SUPPORTED (:274).
- * Complex data types return NOT_SUPPORTED. */
+ * All four data types are served. */
 alphasparse_status_t alphasparse_dcu_spmv(alphasparse_dcu_handle_t handle, alphasparse_operation_t trans,
                                           const void *alpha, const alphasparse_dcu_spmat_descr_t mat,
                                           const alphasparse_dcu_dnvec_descr_t x, const void *beta,

@@ -32,6 +32,13 @@ extern "C" {
 #define ALPHA_INT int32_t
 #endif
 
+/* complex scalars: include/alphasparse/types.h:42-56 */
+#ifndef ALPHA_COMPLEX_TYPES_DEFINED
+#define ALPHA_COMPLEX_TYPES_DEFINED
+typedef struct { float real, imag; } ALPHA_Complex8;
+typedef struct { double real, imag; } ALPHA_Complex16;
+#endif
+
 /* ---- status codes: include/alphasparse/spdef.h:8-19 ---------------------- */
 typedef enum {
   ALPHA_SPARSE_STATUS_SUCCESS = 0,
@@ -309,6 +316,139 @@ alphasparse_status_t alphasparse_d_mm(const alphasparse_operation_t operation, c
                                       const alphasparse_layout_t layout, const double *x,
                                       const ALPHA_INT columns, const ALPHA_INT ldx,
                                       const double beta, double *y, const ALPHA_INT ldy);
+
+/* ---- complex element types ---------------------------------------------------
+ * Payloads and entry points for ALPHA_Complex8 (c) and ALPHA_Complex16 (z), as their
+ * fp32 / fp64 namesakes above: include/alphasparse/spmat.h:120-158 (COO), :231-273
+ * (CSR), :638-659 (ELL); include/alphasparse/spapi.h:111-128 (create_coo), :158-174
+ * (create_csr), :370-386 (export_csr), :440-454 (export_ell), :701-715 (mv), :923-945
+ * (mm).  mv additionally accepts CONJUGATE_TRANSPOSE
+ * (src/plain/kernel/level2/mv/gemv/gemv_c_csr_conj_plain.c:10-27). */
+typedef struct {
+  ALPHA_Complex8 *values;
+  ALPHA_INT *rows_start;
+  ALPHA_INT *rows_end;
+  ALPHA_INT *col_indx;
+  ALPHA_INT rows;
+  ALPHA_INT cols;
+  bool ordered;
+  ALPHA_Complex8 *d_values;
+  ALPHA_INT *d_row_ptr;
+  ALPHA_INT *d_col_indx;
+} spmat_csr_c_t;
+typedef struct {
+  ALPHA_Complex8 *values;
+  ALPHA_INT *row_indx;
+  ALPHA_INT *col_indx;
+  ALPHA_INT rows;
+  ALPHA_INT cols;
+  ALPHA_INT nnz;
+  bool ordered;
+  ALPHA_INT *d_rows_indx;
+  ALPHA_INT *d_cols_indx;
+  ALPHA_Complex8 *d_values;
+} spmat_coo_c_t;
+alphasparse_status_t alphasparse_c_create_coo(alphasparse_matrix_t *A,
+                                              const alphasparse_index_base_t indexing,
+                                              const ALPHA_INT rows, const ALPHA_INT cols,
+                                              const ALPHA_INT nnz, ALPHA_INT *row_indx,
+                                              ALPHA_INT *col_indx, ALPHA_Complex8 *values);
+typedef struct {
+  ALPHA_Complex8 *values;
+  ALPHA_INT *indices;
+  ALPHA_INT rows;
+  ALPHA_INT cols;
+  ALPHA_INT ld;
+  ALPHA_Complex8 *d_values;
+  ALPHA_INT *d_indices;
+} spmat_ell_c_t;
+alphasparse_status_t alphasparse_c_export_ell(const alphasparse_matrix_t source,
+                                              alphasparse_index_base_t *indexing, ALPHA_INT *rows,
+                                              ALPHA_INT *cols, ALPHA_INT *width,
+                                              ALPHA_INT **col_indx, ALPHA_Complex8 **values);
+alphasparse_status_t alphasparse_c_create_csr(alphasparse_matrix_t *A,
+                                              const alphasparse_index_base_t indexing,
+                                              const ALPHA_INT rows, const ALPHA_INT cols,
+                                              ALPHA_INT *rows_start, ALPHA_INT *rows_end,
+                                              ALPHA_INT *col_indx, ALPHA_Complex8 *values);
+alphasparse_status_t alphasparse_c_export_csr(const alphasparse_matrix_t source,
+                                              alphasparse_index_base_t *indexing,
+                                              ALPHA_INT *rows, ALPHA_INT *cols,
+                                              ALPHA_INT **rows_start, ALPHA_INT **rows_end,
+                                              ALPHA_INT **col_indx, ALPHA_Complex8 **values);
+alphasparse_status_t alphasparse_c_mv(const alphasparse_operation_t operation, const ALPHA_Complex8 alpha,
+                                      const alphasparse_matrix_t A,
+                                      const struct alpha_matrix_descr descr, const ALPHA_Complex8 *x,
+                                      const ALPHA_Complex8 beta, ALPHA_Complex8 *y);
+alphasparse_status_t alphasparse_c_mm(const alphasparse_operation_t operation, const ALPHA_Complex8 alpha,
+                                      const alphasparse_matrix_t A,
+                                      const struct alpha_matrix_descr descr,
+                                      const alphasparse_layout_t layout, const ALPHA_Complex8 *x,
+                                      const ALPHA_INT columns, const ALPHA_INT ldx,
+                                      const ALPHA_Complex8 beta, ALPHA_Complex8 *y, const ALPHA_INT ldy);
+
+typedef struct {
+  ALPHA_Complex16 *values;
+  ALPHA_INT *rows_start;
+  ALPHA_INT *rows_end;
+  ALPHA_INT *col_indx;
+  ALPHA_INT rows;
+  ALPHA_INT cols;
+  bool ordered;
+  ALPHA_Complex16 *d_values;
+  ALPHA_INT *d_row_ptr;
+  ALPHA_INT *d_col_indx;
+} spmat_csr_z_t;
+typedef struct {
+  ALPHA_Complex16 *values;
+  ALPHA_INT *row_indx;
+  ALPHA_INT *col_indx;
+  ALPHA_INT rows;
+  ALPHA_INT cols;
+  ALPHA_INT nnz;
+  bool ordered;
+  ALPHA_INT *d_rows_indx;
+  ALPHA_INT *d_cols_indx;
+  ALPHA_Complex16 *d_values;
+} spmat_coo_z_t;
+alphasparse_status_t alphasparse_z_create_coo(alphasparse_matrix_t *A,
+                                              const alphasparse_index_base_t indexing,
+                                              const ALPHA_INT rows, const ALPHA_INT cols,
+                                              const ALPHA_INT nnz, ALPHA_INT *row_indx,
+                                              ALPHA_INT *col_indx, ALPHA_Complex16 *values);
+typedef struct {
+  ALPHA_Complex16 *values;
+  ALPHA_INT *indices;
+  ALPHA_INT rows;
+  ALPHA_INT cols;
+  ALPHA_INT ld;
+  ALPHA_Complex16 *d_values;
+  ALPHA_INT *d_indices;
+} spmat_ell_z_t;
+alphasparse_status_t alphasparse_z_export_ell(const alphasparse_matrix_t source,
+                                              alphasparse_index_base_t *indexing, ALPHA_INT *rows,
+                                              ALPHA_INT *cols, ALPHA_INT *width,
+                                              ALPHA_INT **col_indx, ALPHA_Complex16 **values);
+alphasparse_status_t alphasparse_z_create_csr(alphasparse_matrix_t *A,
+                                              const alphasparse_index_base_t indexing,
+                                              const ALPHA_INT rows, const ALPHA_INT cols,
+                                              ALPHA_INT *rows_start, ALPHA_INT *rows_end,
+                                              ALPHA_INT *col_indx, ALPHA_Complex16 *values);
+alphasparse_status_t alphasparse_z_export_csr(const alphasparse_matrix_t source,
+                                              alphasparse_index_base_t *indexing,
+                                              ALPHA_INT *rows, ALPHA_INT *cols,
+                                              ALPHA_INT **rows_start, ALPHA_INT **rows_end,
+                                              ALPHA_INT **col_indx, ALPHA_Complex16 **values);
+alphasparse_status_t alphasparse_z_mv(const alphasparse_operation_t operation, const ALPHA_Complex16 alpha,
+                                      const alphasparse_matrix_t A,
+                                      const struct alpha_matrix_descr descr, const ALPHA_Complex16 *x,
+                                      const ALPHA_Complex16 beta, ALPHA_Complex16 *y);
+alphasparse_status_t alphasparse_z_mm(const alphasparse_operation_t operation, const ALPHA_Complex16 alpha,
+                                      const alphasparse_matrix_t A,
+                                      const struct alpha_matrix_descr descr,
+                                      const alphasparse_layout_t layout, const ALPHA_Complex16 *x,
+                                      const ALPHA_INT columns, const ALPHA_INT ldx,
+                                      const ALPHA_Complex16 beta, ALPHA_Complex16 *y, const ALPHA_INT ldy);
 
 #include "alphasparse_util.h"
 

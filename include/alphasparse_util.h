@@ -19,6 +19,9 @@ void alpha_free(void *point);
 /* uniform values from rand() after srand(seed); seed 0 takes the clock */
 void alpha_fill_random_s(float *arr, unsigned int seed, const size_t size);
 void alpha_fill_random_d(double *arr, unsigned int seed, const size_t size);
+/* include/alphasparse/util/malloc.h:39-41; src/util/malloc.c:104-112: 2*size reals */
+void alpha_fill_random_c(ALPHA_Complex8 *arr, unsigned int seed, const size_t size);
+void alpha_fill_random_z(ALPHA_Complex16 *arr, unsigned int seed, const size_t size);
 
 /* include/alphasparse/util/io.h:19-20; src/util/io.c:39-114: Matrix Market
  * coordinate text ("%%MatrixMarket matrix coordinate <field> <symmetry>"):
@@ -29,12 +32,23 @@ void alpha_read_coo(const char *file, ALPHA_INT *m_p, ALPHA_INT *n_p, ALPHA_INT 
                     ALPHA_INT **row_index, ALPHA_INT **col_index, float **values);
 void alpha_read_coo_d(const char *file, ALPHA_INT *m_p, ALPHA_INT *n_p, ALPHA_INT *nnz_p,
                       ALPHA_INT **row_index, ALPHA_INT **col_index, double **values);
+/* include/alphasparse/util/io.h:21-22; src/util/io.c:193-345: the value of a line is
+ * taken as both the real and the imaginary part */
+void alpha_read_coo_c(const char *file, ALPHA_INT *m_p, ALPHA_INT *n_p, ALPHA_INT *nnz_p,
+                      ALPHA_INT **row_index, ALPHA_INT **col_index, ALPHA_Complex8 **values);
+void alpha_read_coo_z(const char *file, ALPHA_INT *m_p, ALPHA_INT *n_p, ALPHA_INT *nnz_p,
+                      ALPHA_INT **row_index, ALPHA_INT **col_index, ALPHA_Complex16 **values);
 
 /* include/alphasparse/util/check.h:45-46; src/util/check.c:701-776:
  * max|answer - result| / max|result|, printed as "correct,<ratio>" (return 0)
  * or "error,<ratio>" (return -1) against 2e-5 (fp32) / 1e-10 (fp64). */
 int check_s(const float *answer_data, size_t answer_size, const float *result_data, size_t result_size);
 int check_d(const double *answer_data, size_t answer_size, const double *result_data, size_t result_size);
+/* include/alphasparse/util/check.h:47-48; src/util/check.c:778-786: as 2*size reals */
+int check_c(const ALPHA_Complex8 *answer_data, size_t answer_size, const ALPHA_Complex8 *result_data,
+            size_t result_size);
+int check_z(const ALPHA_Complex16 *answer_data, size_t answer_size, const ALPHA_Complex16 *result_data,
+            size_t result_size);
 
 /* include/alphasparse/util/args.h:16-44; src/util/args.c: GNU long options
  * --help --check --thread-num= --transA= --transB= --typeA= --fillA= --diagA=

@@ -42,6 +42,27 @@ enum asamd_spmv_algo {
 
 #define ASAMD_HIST_BINS 33
 
+/* Element types; the values are those of the reference's alphasparse_datatype_t
+ * (include/alphasparse/spdef.h:137-143). */
+enum asamd_dtype {
+  ASAMD_DTYPE_FLOAT = 0,
+  ASAMD_DTYPE_DOUBLE = 1,
+  ASAMD_DTYPE_FLOAT_COMPLEX = 2,
+  ASAMD_DTYPE_DOUBLE_COMPLEX = 3
+};
+
+/* Complex scalars with the memory layout of the reference's ALPHA_Complex8 /
+ * ALPHA_Complex16 (include/alphasparse/types.h:42-56).  Device arrays of them
+ * must be aligned to the element size (8 / 16 bytes), as hipMalloc'ed arrays are;
+ * entry points return hipErrorInvalidValue otherwise. */
+#ifndef ALPHA_COMPLEX_TYPES_DEFINED
+#define ALPHA_COMPLEX_TYPES_DEFINED
+typedef struct { float real, imag; } ALPHA_Complex8;
+typedef struct { double real, imag; } ALPHA_Complex16;
+#endif
+typedef ALPHA_Complex8 asamd_complex8;
+typedef ALPHA_Complex16 asamd_complex16;
+
 /* Row-length statistics gathered on the GPU.  hist[0] counts empty rows,
  * hist[b] rows whose length lies in [2^(b-1), 2^b). */
 typedef struct {
@@ -60,7 +81,8 @@ typedef struct {
   float tune_ms_ell;    /* ... and of the ELL copy's kernel, or 0             */
   int32_t ell_built;    /* 1: an ELL copy exists (ELL can be selected)        */
   int32_t ell_width;    /* its slots per row                                  */
-  int32_t transpose_built; /* 1: a CSR copy of the transpose exists           */
+  int32_t transpose_built; /* bit 0: a CSR copy of the transpose exists, bit 1: of the
+                              conjugate transpose                              */
   int64_t hist[ASAMD_HIST_BINS];
 } asamd_csr_stats;
 
@@ -70,7 +92,7 @@ typedef struct asamd_csr_plan asamd_csr_plan;
  * block coordinates.  Synchronises `stream` to read the statistics.
  * Replaces the host-side row-block builder
  * src/util_cpp/alphasparse_dcu_x_csrmv_analysis.cpp:58-267, :348-379.
- * val_size is sizeof(value type): 4 or 8.
+ * val_size is sizeof(value type): 4 (fp32) or 8 (fp64).
  * trusted != 0 promises that the structure behind row_ptr / col_ind and the
  * values behind val stay as they are for the life of the plan.  If in addition
  * col_ind and val are given (they may be NULL) and x is much larger than the L2,
@@ -85,6 +107,13 @@ typedef struct asamd_csr_plan asamd_csr_plan;
 int asamd_csr_plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t nnz,
                           const int32_t *row_ptr, const int32_t *col_ind, const void *val,
                           int32_t base, int32_t val_size, int32_t trusted, asamd_csr_plan **plan);
+/* The same for any element type (dtype: enum asamd_dtype).  Complex plans run the
+ * lane-group, merge-path, row-block and ELL-copy kernels (src/kernel/dcu/level2/mv/csrmv/
+ * dcu_gemv_vector.h:14-57 is type-generic through ALPHA_Number); the tiled and the
+ * constant-row-length kernels are for real types. */
+int asamd_csr_plan_create_dtype(hipStream_t stream, int32_t m, int32_t n, int32_t nnz,
+                                const int32_t *row_ptr, const int32_t *col_ind, const void *val,
+                                int32_t base, int32_t dtype, int32_t trusted, asamd_csr_plan **plan);
 void asamd_csr_plan_destroy(asamd_csr_plan *plan);
 const asamd_csr_stats *asamd_csr_plan_stats(const asamd_csr_plan *plan);
 /* Force a kernel family for later multiplies (AUTO restores the analysis'
@@ -108,6 +137,9 @@ int asamd_d_csrmv(hipStream_t stream, asamd_csr_plan *plan, double alpha, const 
  * reference always scatters with atomics. */
 int asamd_csr_plan_build_transpose(hipStream_t stream, asamd_csr_plan *plan, const int32_t *row_ptr,
                                    const int32_t *col_ind, const void *val);
+/* The same with conjugated values: a CSR copy of A^H (complex plans only). */
+int asamd_csr_plan_build_conj_transpose(hipStream_t stream, asamd_csr_plan *plan, const int32_t *row_ptr,
+                                        const int32_t *col_ind, const void *val);
 /* on != 0: the first transposed multiply builds that copy from the arrays it
  * is given (for matrices whose device arrays the library owns). */
 int asamd_csr_plan_set_lazy_transpose(asamd_csr_plan *plan, int32_t on);
@@ -123,6 +155,18 @@ int asamd_s_csrmv_trans(hipStream_t stream, asamd_csr_plan *plan, float alpha, c
 int asamd_d_csrmv_trans(hipStream_t stream, asamd_csr_plan *plan, double alpha, const double *val,
                         const int32_t *row_ptr, const int32_t *col_ind, const double *x, double beta,
                         double *y);
+
+/* Complex element types: y = alpha*op(A)*x + beta*y with op = 0 (A), 1 (A^T), 2 (A^H), the
+ * values of alphasparse_operation_t.  op = 0 stands in for csr_gemv_vector_dispatch as above,
+ * op = 1 for dcu_gemv_x_csr_trans.cpp:11-68, op = 2 for csr_gemv_conj_scalar_atomicadd
+ * (src/kernel/dcu/level2/mv/csrmv/dcu_gemv_c_csr_conj.cpp:22-75); 1 and 2 use the plan's copy
+ * of A^T / A^H when it has one and scatter with atomics otherwise. */
+int asamd_c_csrmv_op(hipStream_t stream, asamd_csr_plan *plan, int32_t op, asamd_complex8 alpha,
+                     const asamd_complex8 *val, const int32_t *row_ptr, const int32_t *col_ind,
+                     const asamd_complex8 *x, asamd_complex8 beta, asamd_complex8 *y);
+int asamd_z_csrmv_op(hipStream_t stream, asamd_csr_plan *plan, int32_t op, asamd_complex16 alpha,
+                     const asamd_complex16 *val, const int32_t *row_ptr, const int32_t *col_ind,
+                     const asamd_complex16 *x, asamd_complex16 beta, asamd_complex16 *y);
 
 /* Dense operand addressing for SpMM: element (r, c) of B is
  * B[r*b_row_stride + c*b_col_stride], of C is C[r*c_row_stride + c*c_col_stride]. */
@@ -161,6 +205,15 @@ int asamd_d_csrmm_ws(hipStream_t stream, int32_t m, int32_t n, int32_t k, int32_
                      const double *B, double beta, double *C, const asamd_dense_strides *strides,
                      void *workspace, size_t workspace_bytes);
 
+int asamd_c_csrmm_ws(hipStream_t stream, int32_t m, int32_t n, int32_t k, int32_t nnz, asamd_complex8 alpha,
+                     const asamd_complex8 *val, const int32_t *row_ptr, const int32_t *col_ind, int32_t base,
+                     const asamd_complex8 *B, asamd_complex8 beta, asamd_complex8 *C,
+                     const asamd_dense_strides *strides, void *workspace, size_t workspace_bytes);
+int asamd_z_csrmm_ws(hipStream_t stream, int32_t m, int32_t n, int32_t k, int32_t nnz, asamd_complex16 alpha,
+                     const asamd_complex16 *val, const int32_t *row_ptr, const int32_t *col_ind, int32_t base,
+                     const asamd_complex16 *B, asamd_complex16 beta, asamd_complex16 *C,
+                     const asamd_dense_strides *strides, void *workspace, size_t workspace_bytes);
+
 /* coo_row[k] = r + base for k in [row_ptr[r]-base, row_ptr[r+1]-base).
  * Defines on the GPU what src/core/format/convert_coo_x_csr.c:30-37 does on the host. */
 int asamd_csr2coo(hipStream_t stream, const int32_t *row_ptr, int32_t nnz, int32_t m,
@@ -179,6 +232,12 @@ int asamd_s_csr2ell(hipStream_t stream, int32_t m, const float *val, const int32
 int asamd_d_csr2ell(hipStream_t stream, int32_t m, const double *val, const int32_t *row_ptr,
                     const int32_t *col_ind, int32_t csr_base, int32_t ell_base, int32_t width,
                     double *ell_val, int32_t *ell_col);
+int asamd_c_csr2ell(hipStream_t stream, int32_t m, const asamd_complex8 *val, const int32_t *row_ptr,
+                    const int32_t *col_ind, int32_t csr_base, int32_t ell_base, int32_t width,
+                    asamd_complex8 *ell_val, int32_t *ell_col);
+int asamd_z_csr2ell(hipStream_t stream, int32_t m, const asamd_complex16 *val, const int32_t *row_ptr,
+                    const int32_t *col_ind, int32_t csr_base, int32_t ell_base, int32_t width,
+                    asamd_complex16 *ell_val, int32_t *ell_col);
 
 /* y = alpha*A*x + beta*y, A in column-major ELL (slot s of row r at [s*m + r]);
  * slots whose index (minus base) is outside [0, n) are skipped.  Stands in for
@@ -189,6 +248,12 @@ int asamd_s_ellmv(hipStream_t stream, int32_t m, int32_t n, float alpha, const f
 int asamd_d_ellmv(hipStream_t stream, int32_t m, int32_t n, double alpha, const double *ell_val,
                   const int32_t *ell_col_ind, int32_t ell_width, int32_t base, const double *x,
                   double beta, double *y);
+int asamd_c_ellmv(hipStream_t stream, int32_t m, int32_t n, asamd_complex8 alpha, const asamd_complex8 *ell_val,
+                  const int32_t *ell_col_ind, int32_t ell_width, int32_t base, const asamd_complex8 *x,
+                  asamd_complex8 beta, asamd_complex8 *y);
+int asamd_z_ellmv(hipStream_t stream, int32_t m, int32_t n, asamd_complex16 alpha, const asamd_complex16 *ell_val,
+                  const int32_t *ell_col_ind, int32_t ell_width, int32_t base, const asamd_complex16 *x,
+                  asamd_complex16 beta, asamd_complex16 *y);
 
 /* y = alpha*A*x + beta*y, A in COO.  Fastest when entries are grouped by row
  * (as asamd_csr2coo leaves them) but correct for any order; entries whose row or
@@ -201,6 +266,12 @@ int asamd_s_coomv(hipStream_t stream, int32_t m, int32_t n, int64_t nnz, float a
 int asamd_d_coomv(hipStream_t stream, int32_t m, int32_t n, int64_t nnz, double alpha,
                   const double *coo_val, const int32_t *coo_row_ind, const int32_t *coo_col_ind,
                   int32_t base, const double *x, double beta, double *y);
+int asamd_c_coomv(hipStream_t stream, int32_t m, int32_t n, int64_t nnz, asamd_complex8 alpha,
+                  const asamd_complex8 *coo_val, const int32_t *coo_row_ind, const int32_t *coo_col_ind,
+                  int32_t base, const asamd_complex8 *x, asamd_complex8 beta, asamd_complex8 *y);
+int asamd_z_coomv(hipStream_t stream, int32_t m, int32_t n, int64_t nnz, asamd_complex16 alpha,
+                  const asamd_complex16 *coo_val, const int32_t *coo_row_ind, const int32_t *coo_col_ind,
+                  int32_t base, const asamd_complex16 *x, asamd_complex16 beta, asamd_complex16 *y);
 
 /* Introspection for benchmarks and tests: statistics of the analysis that a
  * multiply would use for `key`, where key is the alphasparse_dcu_mat_info_t of an

@@ -20,12 +20,40 @@ def _p(a):
     return None if a is None else a.ctypes.data_as(c_void_p)
 
 
+class C8(Structure):
+    """ALPHA_Complex8 by value."""
+    _fields_ = [("real", c_float), ("imag", c_float)]
+
+    def __init__(self, v=0):
+        v = complex(v)
+        super().__init__(v.real, v.imag)
+
+
+class C16(Structure):
+    """ALPHA_Complex16 by value."""
+    _fields_ = [("real", c_double), ("imag", c_double)]
+
+    def __init__(self, v=0):
+        v = complex(v)
+        super().__init__(v.real, v.imag)
+
+
+_CT = {np.dtype(np.float32): c_float, np.dtype(np.float64): c_double, np.dtype(np.complex64): C8,
+       np.dtype(np.complex128): C16}
+_PRE = {np.dtype(np.float32): "s", np.dtype(np.float64): "d", np.dtype(np.complex64): "c",
+        np.dtype(np.complex128): "z"}
+
+
 def _ct(dtype):
-    return c_float if np.dtype(dtype) == np.float32 else c_double
+    return _CT[np.dtype(dtype)]
 
 
 def _pre(dtype):
-    return "s" if np.dtype(dtype) == np.float32 else "d"
+    return _PRE[np.dtype(dtype)]
+
+
+def is_complex(dtype):
+    return np.dtype(dtype).kind == "c"
 
 
 def lib(fast=False):
@@ -60,6 +88,21 @@ def lib(fast=False):
             f = getattr(L, "oracle_%s_csrmm_err" % s)
             f.restype, f.argtypes = c_double, [I, I, P, P, P, P, c_double, P, c_int64, c_int64, c_double, P, P, P,
                                                c_int64, c_int64, POINTER(c_int64), POINTER(c_double)]
+        for s, T in (("c", C8), ("z", C16)):
+            f = getattr(L, "oracle_%s_csrmv_plain" % s)
+            f.restype, f.argtypes = None, [I, P, P, P, P, T, P, T, P]
+            for n in ("trans_plain", "conj_plain"):
+                f = getattr(L, "oracle_%s_csrmv_%s" % (s, n))
+                f.restype, f.argtypes = None, [I, I, P, P, P, P, T, P, T, P]
+            for n in ("row_plain", "col_plain"):
+                f = getattr(L, "oracle_%s_csrmm_%s" % (s, n))
+                f.restype, f.argtypes = None, [I, P, P, P, P, T, P, I, I, T, P, I]
+            f = getattr(L, "oracle_%s_csr2ell" % s)
+            f.restype, f.argtypes = I, [I, P, P, P, I, I, I, P, P]
+            f = getattr(L, "oracle_%s_coomv_plain" % s)
+            f.restype, f.argtypes = None, [I, I, P, P, P, T, P, T, P]
+            f = getattr(L, "oracle_%s_ellmv" % s)
+            f.restype, f.argtypes = None, [I, I, T, P, P, I, P, T, P]
         L.oracle_partition_rows_by_nnz.restype = None
         L.oracle_partition_rows_by_nnz.argtypes = [P, I, I, P]
         L.oracle_csr2coo.restype = None
@@ -89,26 +132,30 @@ def csrmv_plain(a, alpha, x, beta, y0, fast=False):
     return y
 
 
-def csrmv_trans_plain(a, alpha, x, beta, y0):
-    """y = alpha*A^T*x + beta*y0: x has a.rows entries, y0 has a.cols."""
+def csrmv_trans_plain(a, alpha, x, beta, y0, conj=False):
+    """y = alpha*A^T*x + beta*y0 (conj: A^H, complex types only): x has a.rows entries, y0 has a.cols."""
     rs, re, ci = (np.ascontiguousarray(v) for v in _zero_based(a))
     y = np.array(y0, dtype=a.dtype, copy=True)
     T = _ct(a.dtype)
-    getattr(lib(), "oracle_%s_csrmv_trans_plain" % _pre(a.dtype))(
+    assert not conj or is_complex(a.dtype)
+    getattr(lib(), "oracle_%s_csrmv_%s_plain" % (_pre(a.dtype), "conj" if conj else "trans"))(
         a.rows, a.cols, _p(rs), _p(re), _p(ci), _p(a.values), T(alpha), _p(x), T(beta), _p(y))
     return y
 
 
-def transpose(a):
-    """CSR of A^T, zero-based; rows of A stay ascending inside every column (stable sort)."""
+def transpose(a, conj=False):
+    """CSR of A^T (conj: of A^H), zero-based; rows of A stay ascending inside every column
+    (stable sort)."""
     from alsparse_amd import workloads as wl
     rp = a.row_ptr.astype(np.int64) - a.base
     ci = a.col_ind.astype(np.int64) - a.base
     rows = np.repeat(np.arange(a.rows, dtype=np.int32), np.diff(rp))
     order = np.argsort(ci, kind="stable")
     trp = np.concatenate([[0], np.cumsum(np.bincount(ci, minlength=a.cols))]).astype(np.int32)
-    return wl.Csr(a.cols, a.rows, trp, np.ascontiguousarray(rows[order]), np.ascontiguousarray(a.values[order]), 0,
-                  "transpose(%s)" % a.name)
+    vals = np.ascontiguousarray(a.values[order])
+    if conj:
+        vals = np.conj(vals)
+    return wl.Csr(a.cols, a.rows, trp, np.ascontiguousarray(rows[order]), vals, 0, "transpose(%s)" % a.name)
 
 
 def csrmv_omp(a, alpha, x, beta, y0, threads=0, fast=True):
@@ -143,7 +190,38 @@ class SpmvError:
             self.full, self.strict, self.row, self.zero_den_mismatch)
 
 
+def _complex_err(den, diff, beta_y0):
+    """The two per-element metrics from |alpha| sum|a||x| (den), |test - ref| (diff) and
+    |beta y0| (or None); complex moduli throughout, everything in fp64."""
+    zero = den == 0
+    zbad = int(np.count_nonzero(zero & (diff != 0)))
+    nz = ~zero
+    if not nz.any():
+        return SpmvError(0.0, 0.0, -1, zbad)
+    with np.errstate(invalid="ignore", divide="ignore"):
+        strict = np.where(nz, diff / np.where(nz, den, 1.0), 0.0)
+        full_den = den + (beta_y0 if beta_y0 is not None else 0.0)
+        full = np.where(nz, diff / np.where(nz, full_den, 1.0), 0.0)
+    strict = np.where(np.isnan(strict), np.inf, strict)
+    full = np.where(np.isnan(full), np.inf, full)
+    return SpmvError(float(full.max()), float(strict.max()), int(np.argmax(full)), zbad)
+
+
+def _row_abs_sums(a, w):
+    """sum over the entries of each row of |a_ij| * w[col] (w real, fp64)."""
+    rp = a.row_ptr.astype(np.int64) - a.base
+    prod = np.abs(a.values.astype(np.complex128)) * w[a.col_ind.astype(np.int64) - a.base]
+    csum = np.concatenate([[0.0], np.cumsum(prod)])
+    return csum[rp[1:]] - csum[rp[:-1]]
+
+
 def csrmv_err(a, alpha, x, beta, y0, y_test, y_ref):
+    if is_complex(a.dtype):
+        # the same two metrics with complex moduli: |dy| / (|alpha| sum |a_ij| |x_j| [+ |beta y0|])
+        den = abs(complex(alpha)) * _row_abs_sums(a, np.abs(np.asarray(x, dtype=np.complex128)))
+        diff = np.abs(np.asarray(y_test, dtype=np.complex128) - np.asarray(y_ref, dtype=np.complex128))
+        by = None if (y0 is None or beta == 0) else np.abs(complex(beta) * np.asarray(y0, dtype=np.complex128))
+        return _complex_err(den, diff, by)
     rs, re, ci = (np.ascontiguousarray(v) for v in _zero_based(a))
     wr, zb, rr, ws = c_int64(-1), c_int64(0), c_double(0), c_double(0)
     y_test = np.ascontiguousarray(y_test, dtype=a.dtype)
@@ -177,6 +255,17 @@ def csrmm_plain(a, alpha, B, beta, C0, layout="row", omp=False, fast=False):
 def csrmm_err(a, alpha, B, beta, C0, C_test, C_ref):
     """Per-element errors of C; B (k, n) and the C arrays (m, n) are 2-D arrays in any
     memory layout (the metric does not depend on it)."""
+    if is_complex(a.dtype):
+        import scipy.sparse as sp
+        rp = a.row_ptr.astype(np.int64) - a.base
+        absA = sp.csr_matrix((np.abs(a.values.astype(np.complex128)), a.col_ind.astype(np.int64) - a.base, rp),
+                             shape=(a.rows, a.cols))
+        den = abs(complex(alpha)) * (absA @ np.abs(np.asarray(B, dtype=np.complex128)))
+        diff = np.abs(np.asarray(C_test, dtype=np.complex128) - np.asarray(C_ref, dtype=np.complex128))
+        by = None if (C0 is None or beta == 0) else np.abs(complex(beta) * np.asarray(C0, dtype=np.complex128))
+        e = _complex_err(den.ravel(), diff.ravel(), None if by is None else by.ravel())
+        e.row = -1
+        return e
     rs, re, ci = (np.ascontiguousarray(v) for v in _zero_based(a))
     B = np.ascontiguousarray(B, dtype=a.dtype)
     C_test = np.ascontiguousarray(C_test, dtype=a.dtype)

@@ -24,3 +24,20 @@ def csr_from_lengths(lengths, cols, dtype, seed=7, base=0):
     vals = rng.uniform(-1, 1, size=col.size).astype(dtype)
     return wl.Csr(len(lengths), cols, (row_ptr + base).astype(np.int32), col + np.int32(base), vals, base,
                   "lengths(m=%d,nnz=%d)" % (len(lengths), col.size))
+
+
+def real_dtype(dtype):
+    """float32 for complex64, float64 for complex128, the dtype itself for real types."""
+    return np.empty(0, dtype=dtype).real.dtype
+
+
+def complex_vector(n, dtype, stream):
+    """Seeded complex vector: real parts from generator stream `stream`, imaginary from stream + 100."""
+    rd = real_dtype(dtype)
+    return (wl.uniform(n, rd, stream) + 1j * wl.uniform(n, rd, stream + 100)).astype(dtype)
+
+
+def complexify(a, dtype, stream=200):
+    """The structure of a real workload with seeded complex values of the given complex dtype."""
+    return wl.Csr(a.rows, a.cols, a.row_ptr, a.col_ind, complex_vector(a.nnz, dtype, stream), a.base,
+                  a.name + ":" + np.dtype(dtype).name)

@@ -1,5 +1,6 @@
-"""The reference's OWN GPU test programs (test/dcu/level2/mv_csr_?_dcu_test.cpp, mv_coo_?, mv_ell_?,
-spmv_{csr,coo,ell}_s, test/dcu/level3/mm_csr_?_dcu_test.cpp, mm_csr_s_dcu_row_test.cpp), compiled unchanged
+"""The reference's OWN GPU test programs (test/dcu/level2/mv_csr_?_dcu_test.cpp, mv_coo_?, mv_ell_?
+for ? in s, d, c, z; spmv_{csr,coo,ell}_s; test/dcu/level3/mm_csr_?_dcu_test.cpp,
+mm_csr_s_dcu_row_test.cpp), compiled unchanged
 against this repository's headers and library by `make -C oracle ref_drivers` (into oracle/_ref/,
 where the reference tree is present) and run here on a coordinate file: they read the file, take
 the COO -> CSR / ELL route, call alphasparse_dcu_?_csrmv / _csrmm / _coomv / _ellmv and compare with
@@ -32,6 +33,14 @@ PROGRAMS = {
     "mm_csr_s_dcu_test": [["--columns=8", "--layout=C"], ["--columns=70", "--layout=C"]],
     "mm_csr_d_dcu_test": [["--columns=8", "--layout=C"]],
     "mm_csr_s_dcu_row_test": [["--columns=64"]],
+    # complex element types (the coordinate reader gives every entry equal real and imaginary parts);
+    # mv_csr_c / mv_csr_z pass rocSPARSE a half-initialised beta and are left out
+    "mv_coo_c_dcu_test": [[]],
+    "mv_coo_z_dcu_test": [[]],
+    "mv_ell_c_dcu_test": [[]],
+    "mv_ell_z_dcu_test": [[]],
+    "mm_csr_c_dcu_test": [["--columns=8", "--layout=C"]],
+    "mm_csr_z_dcu_test": [["--columns=8", "--layout=C"]],
 }
 
 

@@ -178,9 +178,14 @@ def test_generic_spmv_status_codes(lib):
     assert call(m=mat(col_type=S.ALPHA_SPARSE_DCU_INDEXTYPE_U16)) == S.ALPHA_SPARSE_STATUS_NOT_SUPPORTED
     # size query on an already analysed matrix: no device work, 4 bytes
     assert call() == S.ALPHA_SPARSE_STATUS_SUCCESS and size.value == 4
-    # complex data and formats other than COO / CSR / ELL are refused at the multiply
+    # complex data reaches the typed entry points' validation; unknown data types and formats other
+    # than COO / CSR / ELL are refused
     cx = S.ALPHA_SPARSE_DATATYPE_FLOAT_COMPLEX
-    assert call(m=mat(data_type=cx), xx=DV(True, 4, P, cx), yy=DV(True, 4, P, cx), ct=cx, tb=buf) == S.ALPHA_SPARSE_STATUS_NOT_SUPPORTED
+    assert call(m=mat(data_type=cx, val_data=None), xx=DV(True, 4, P, cx), yy=DV(True, 4, P, cx), ct=cx,
+                tb=buf) == S.ALPHA_SPARSE_STATUS_INVALID_POINTER
+    assert call(m=mat(data_type=cx, rows=0), xx=DV(True, 4, P, cx), yy=DV(True, 4, P, cx), ct=cx,
+                tb=buf) == S.ALPHA_SPARSE_STATUS_SUCCESS
+    assert call(m=mat(data_type=7), xx=DV(True, 4, P, 7), yy=DV(True, 4, P, 7), ct=7, tb=buf) == S.ALPHA_SPARSE_STATUS_NOT_SUPPORTED
     assert call(m=mat(format=S.ALPHA_SPARSE_FORMAT_COO_AOS), tb=buf) == S.ALPHA_SPARSE_STATUS_NOT_SUPPORTED
     assert call(m=mat(format=S.ALPHA_SPARSE_FORMAT_BSR), tb=buf) == S.ALPHA_SPARSE_STATUS_NOT_SUPPORTED
     # the typed entry points' own validation shows through
