@@ -2,7 +2,7 @@
 import numpy as np
 
 from alsparse_amd import workloads as wl
-from helpers_shapes import csr_from_lengths
+from helpers_shapes import complexify, csr_from_lengths
 
 
 def golden_matrices():
@@ -13,6 +13,17 @@ def golden_matrices():
         out[t + ".uniform16"] = wl.uniform_rows(512, 2048, 16, dt)
         out[t + ".powerlaw"] = wl.powerlaw_rmat(10, 600, dt)
         out[t + ".empty_rows"] = csr_from_lengths([0, 3, 0, 0, 7, 1, 0, 2, 0, 0], 16, dt, seed=5)
+    return out
+
+
+def golden_complex_matrices():
+    """Complex-valued cases (values seeded as in helpers_shapes.complexify)."""
+    out = {}
+    for dt, rd, t in ((np.complex64, np.float32, "c"), (np.complex128, np.float64, "z")):
+        out[t + ".points"] = complexify(wl.random_points(1000, 1000, 5000, rd), dt)
+        out[t + ".laplace"] = complexify(wl.laplace2d(24, 16, rd), dt)
+        out[t + ".powerlaw"] = complexify(wl.powerlaw_rmat(10, 600, rd), dt)
+        out[t + ".empty_rows"] = complexify(csr_from_lengths([0, 3, 0, 0, 7, 1, 0, 2, 0, 0], 16, rd, seed=5), dt)
     return out
 
 
