@@ -268,9 +268,6 @@ static hipError_t build_ell(hipStream_t stream, asamd_csr_plan* p, const int* ro
 
 template <typename T>
 static bool tiled_eligible(const asamd_csr_stats& st, bool force) {
-  if constexpr (!kIsReal<T>) {
-    return false;  // the tiled kernels are written for real element types
-  } else {
   // full-width block counts; the equal-entry cut (at most twice as many blocks
   // per dimension) is checked again once it is known
   const int64_t cb = ((int64_t)st.n + TileDims<T>::cols - 1) / TileDims<T>::cols;
@@ -281,7 +278,6 @@ static bool tiled_eligible(const asamd_csr_stats& st, bool force) {
   if ((int64_t)st.nnz > (int64_t)0x7fffffff - (1 << 16)) return false;
   // worth a try only when x cannot live in an XCD's 4 MiB L2 and the matrix is large
   return force || ((int64_t)st.n * (int64_t)sizeof(T) >= ((int64_t)8 << 20) && st.nnz >= (1 << 22));
-  }
 }
 
 // Cuts groups [0, groups) with cumulative entry counts off[0..groups] into
@@ -465,7 +461,7 @@ static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* 
                             hipFuncAttributeMaxDynamicSharedMemorySize, kTileBytes);
   if (e == hipSuccess)
     e = hipFuncSetAttribute((const void*)tiled_reduce_kernel<T>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, kRedBytes);
+                            hipFuncAttributeMaxDynamicSharedMemorySize, TileDims<T>::red_bytes);
   for (void* d : {(void*)d_coo, (void*)d_key, (void*)d_key2, (void*)d_idx, (void*)d_perm, (void*)d_tile_ptr,
                   (void*)d_long_raw, (void*)d_long_count, (void*)d_cnt, (void*)d_cgb, (void*)d_rgb, (void*)d_cbs})
     if (d) (void)hipFree(d);
@@ -614,9 +610,7 @@ static hipError_t plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t 
     e = by_dtype(dtype, [&](auto* tag) -> hipError_t {
       using T = std::remove_pointer_t<decltype(tag)>;
       hipError_t err = hipSuccess;
-      if constexpr (kIsReal<T>) {
-        if (tiled_eligible<T>(p->st, force)) err = build_tiled<T>(stream, p, row_ptr, col_ind, (const T*)val);
-      }
+      if (tiled_eligible<T>(p->st, force)) err = build_tiled<T>(stream, p, row_ptr, col_ind, (const T*)val);
       if (err == hipSuccess && ell_eligible(p->st, force))
         err = build_ell<T>(stream, p, row_ptr, col_ind, (const T*)val);
       if (err == hipSuccess && !force && (p->st.tiled_built || p->st.ell_built))
@@ -816,7 +810,7 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
   if (((uintptr_t)val | (uintptr_t)x | (uintptr_t)y) % alignof(T)) return hipErrorInvalidValue;
   const asamd_csr_stats& st = p->st;
   int algo = st.algo;
-  if (!kIsReal<T> && (algo == ASAMD_SPMV_ROWCONST || algo == ASAMD_SPMV_TILED)) algo = ASAMD_SPMV_VECTOR;
+  if (!kIsReal<T> && algo == ASAMD_SPMV_ROWCONST) algo = ASAMD_SPMV_VECTOR;
   if (algo == ASAMD_SPMV_ROWCONST) {
     // 128-bit loads need 16-byte aligned streams; fall back otherwise
     const bool aligned = (((uintptr_t)val | (uintptr_t)ci) & 15u) == 0;
@@ -833,12 +827,12 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
                                                    x, beta, y);
       break;
     }
-    case ASAMD_SPMV_TILED: if constexpr (kIsReal<T>) {
+    case ASAMD_SPMV_TILED: {
       // the tiled copy holds zero-based local indices and its own values
       if (p->n_chunks > 0)
         tiled_products_kernel<T><<<p->n_chunks, kProdThreads, kTileBytes, s>>>(
             p->d_chunks, (const T*)p->d_tval, p->d_tcol, x, (T*)p->d_tprod);
-      tiled_reduce_kernel<T><<<(st.tile_row_blocks + kRedWaves - 1) / kRedWaves, kRedThreads, kRedBytes, s>>>(
+      tiled_reduce_kernel<T><<<(st.tile_row_blocks + kRedWaves - 1) / kRedWaves, kRedThreads, TileDims<T>::red_bytes, s>>>(
           st.m, st.tile_row_blocks, st.tile_col_blocks, p->d_row_block_start, p->d_ranges, p->d_trow,
           (const T*)p->d_tprod, alpha, beta, y);
       if (p->n_long_chunks > 0)

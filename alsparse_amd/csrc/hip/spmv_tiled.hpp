@@ -67,7 +67,10 @@ constexpr int kRowGroupLog2 = 6;        // row blocks at multiples of 64 rows
 template <typename T>
 struct TileDims {
   static constexpr int cols = kTileBytes / (int)sizeof(T);            // widest column block: 32768 fp32, 16384 fp64
-  static constexpr int rows = kRedBytes / kRedWaves / (int)sizeof(T);  // tallest row block: 2048 fp32, 1024 fp64
+  // LDS bytes of a phase-2 workgroup's accumulators: wider values get the larger share, so that a row
+  // block keeps 2048 rows (tiles per matrix, which is what phase 2 pays for, do not double)
+  static constexpr int red_bytes = sizeof(T) >= 8 ? kTileBytes : kRedBytes;
+  static constexpr int rows = red_bytes / kRedWaves / (int)sizeof(T);  // tallest row block: 2048 (1024 for 16-byte values)
 };
 
 struct TiledChunk {
@@ -224,7 +227,7 @@ __global__ __launch_bounds__(kProdThreads) void tiled_products_kernel(
 //     run's total in its first lane, which adds alone.
 template <bool Atomic, typename T>
 __device__ __forceinline__ void rmw(T* p, T v) {
-  if constexpr (Atomic) atomicAdd(p, v);
+  if constexpr (Atomic) atomic_add(p, v);
   else *p += v;
 }
 
@@ -271,7 +274,7 @@ __device__ __forceinline__ void add_rows(T* acc, int r, T v, bool valid) {
   const uint64_t above = dup >> 1 >> lane;
 #pragma unroll
   for (int d = 1; d < kWave; d <<= 1) {
-    const T vd = __shfl_down(v, d, kWave);
+    const T vd = lane_down(v, d);
     const uint64_t need = ((uint64_t)1 << d) - 1;
     if ((above & need) == need) v += vd;
   }

@@ -72,6 +72,26 @@ class Csr:
         return self.values.dtype
 
 
+def real_dtype(dtype):
+    """float32 for complex64, float64 for complex128, the dtype itself for real types."""
+    return np.empty(0, dtype=dtype).real.dtype
+
+
+def complex_vector(n, dtype, stream, seed=SEED):
+    """Seeded complex vector: real parts from generator stream `stream`, imaginary parts from stream + 100."""
+    rd = real_dtype(dtype)
+    out = np.empty(int(n), dtype=dtype)
+    out.real = uniform(n, rd, stream, seed)
+    out.imag = uniform(n, rd, stream + 100, seed)
+    return out
+
+
+def complexify(a, dtype, stream=200):
+    """The structure of a real workload with seeded complex values of the given complex dtype."""
+    return Csr(a.rows, a.cols, a.row_ptr, a.col_ind, complex_vector(a.nnz, dtype, stream), a.base,
+               a.name + ":" + np.dtype(dtype).name)
+
+
 def uniform_rows(rows, cols, k, dtype=np.float32, seed=SEED, base=0, lo=-1.0, hi=1.0):
     lib = _load()
     k = min(k, cols)

@@ -130,19 +130,30 @@ def vendor_spmv(a, x, y0, alpha, beta, nbytes, steps, warmup, transpose=False):
             "ms": t["avg_ms"], "analysis_ms": analysis_ms}
 
 
-def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False, vendor=False):
+def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False, vendor=False, cx=False, conjugate=False):
+    """cx: the configuration's structure with complex values (complex64 for the fp32 configurations,
+    complex128 for the fp64 one), complex x, y, alpha and beta; conjugate: A^H instead of A^T."""
     from alsparse_amd import capi, hiprt, workloads as wl
     lib = capi.load()
     t0 = time.time()
     a, x, y0, alpha, beta, _ = wl.config(cfg)
+    if cx:
+        cdt = np.complex64 if a.dtype == np.float32 else np.complex128
+        a = wl.complexify(a, cdt)
+        x, y0 = wl.complex_vector(a.cols, cdt, 3), wl.complex_vector(a.rows, cdt, 4)
+        alpha, beta = complex(alpha, -0.5), complex(beta, 0.25)
+        cpu_baseline = vendor = False
     log("[bench] generated %s: %d rows, %d nnz in %.1f s" % (a.name, a.rows, a.nnz, time.time() - t0))
     T, p = capi.scalar_type(a.dtype), capi.prefix(a.dtype)
     h = capi.Handle()
     descr = capi.make_descr()
     d_val, d_rp, d_ci = (hiprt.DeviceArray.from_numpy(v) for v in (a.values, a.row_ptr, a.col_ind))
     op = capi.ALPHA_SPARSE_OPERATION_TRANSPOSE if transpose else capi.ALPHA_SPARSE_OPERATION_NON_TRANSPOSE
+    if transpose and conjugate and cx:
+        op = capi.ALPHA_SPARSE_OPERATION_CONJUGATE_TRANSPOSE
     if transpose:  # y = alpha*A^T*x + beta*y: x has `rows` entries, y has `cols`
-        x, y0 = wl.uniform(a.rows, a.dtype, 3), wl.uniform(a.cols, a.dtype, 4)
+        x, y0 = ((wl.complex_vector(a.rows, a.dtype, 3), wl.complex_vector(a.cols, a.dtype, 4)) if cx else
+                 (wl.uniform(a.rows, a.dtype, 3), wl.uniform(a.cols, a.dtype, 4)))
     d_x, d_y = hiprt.DeviceArray.from_numpy(x), hiprt.DeviceArray.from_numpy(y0)
 
     info = capi.alphasparse_dcu_mat_info_t()
@@ -156,7 +167,7 @@ def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False, vendor=Fa
     assert st == 0, "analysis status %d" % st
     stats = lib.asamd_analysis_stats(info).contents
     if transpose:
-        assert stats.transpose_built == 1, "no room for the transposed copy"
+        assert stats.transpose_built != 0, "no room for the transposed copy"
         stats = lib.asamd_analysis_transpose_stats(info).contents
     algo = capi.ALGO_NAMES.get(stats.algo, "?")
     if stats.algo == capi.ASAMD_SPMV_VECTOR:
@@ -172,14 +183,16 @@ def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False, vendor=Fa
             raise RuntimeError("csrmv status %d" % s)
 
     parity = None
-    if check:
+    if check and cx and transpose:
+        log("[bench] parity of the complex transposed operations is covered by tests/test_gpu_complex.py, not here")
+    elif check:
         from oracle import oracle as orc
         d_y.copy_from(y0)
         step()
         hiprt.synchronize()
         y = d_y.to_numpy()
         t0 = time.time()
-        tol = 1e-4 if a.dtype == np.float32 else 1e-12
+        tol = 1e-4 if a.dtype.itemsize // (2 if cx else 1) == 4 else 1e-12
         if transpose:
             ref = orc.csrmv_trans_plain(a, alpha, x, beta, y0)
             absa = wl.Csr(a.rows, a.cols, a.row_ptr, a.col_ind, np.abs(a.values), a.base)
@@ -200,12 +213,16 @@ def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False, vendor=Fa
     t = time_steps(step, steps, warmup, hiprt)
     nbytes = (wl.spmv_bytes(a.cols, a.rows, a.nnz, a.dtype.itemsize, beta) if transpose
               else wl.spmv_bytes(a.rows, a.cols, a.nnz, a.dtype.itemsize, beta))
-    res = {"workload": WORKLOAD_NAMES[cfg] + (" -- TRANSPOSED operation" if transpose else ""), "rows": a.rows, "nnz": a.nnz, "algorithmic_bytes": int(nbytes),
+    opname = "" if not transpose else (" -- CONJUGATE-TRANSPOSED operation" if op == 2 else " -- TRANSPOSED operation")
+    res = {"workload": WORKLOAD_NAMES[cfg] + (" -- COMPLEX values (%s)" % a.dtype.name if cx else "") + opname, "rows": a.rows, "nnz": a.nnz, "algorithmic_bytes": int(nbytes),
            "flops": 2 * a.nnz, "kernel": algo, "analysis_ms": analysis_ms, "timing": t,
            "gbs": nbytes / t["avg_ms"] / 1e6, "gflops": 2 * a.nnz / t["avg_ms"] / 1e6,
-           "dtype": "f32" if a.dtype == np.float32 else "f64", "parity": parity}
+           "dtype": {"float32": "f32", "float64": "f64", "complex64": "c64", "complex128": "c128"}[a.dtype.name],
+           "parity": parity}
+    if cx:  # a complex multiply-add is 8 real flops
+        res["flops"], res["gflops"] = 8 * a.nnz, 8 * a.nnz / t["avg_ms"] / 1e6
     res["hbm_frac"] = res["gbs"] / HBM_PEAK_GBS
-    res["traffic"] = None if transpose else MEASURED_TRAFFIC_BYTES.get((cfg, algo))
+    res["traffic"] = None if (transpose or cx) else MEASURED_TRAFFIC_BYTES.get((cfg, algo))
 
     if cpu_baseline and not transpose:
         res["cpu_baseline"] = cpu_spmv(a, x, y0, alpha, beta, nbytes)
@@ -408,6 +425,9 @@ def main():
     ap.add_argument("--col-major", action="store_true", help="configuration 5 with column-major B and C")
     ap.add_argument("--transpose", action="store_true",
                     help="y = alpha*A^T*x + beta*y of configuration 2, 3 or 4 (analysis asked for the transposed operation)")
+    ap.add_argument("--complex", action="store_true", dest="cx",
+                    help="configuration 2, 3 or 4 with complex values (complex64 / complex128), complex x, y, alpha, beta")
+    ap.add_argument("--conjugate", action="store_true", help="with --complex --transpose: A^H instead of A^T")
     ap.add_argument("--all", action="store_true", help="also measure the other configurations")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-vendor-baseline", action="store_true",
@@ -446,7 +466,7 @@ def main():
         main_res = run_spmm(args.steps, args.warmup, check, args.col_major, not args.no_vendor_baseline)
     else:
         main_res = run_spmv(args.config, args.steps, args.warmup, not args.no_cpu_baseline, check, args.transpose,
-                            not args.no_vendor_baseline)
+                            not args.no_vendor_baseline, args.cx, args.conjugate)
     others = {}
     if args.all:
         for c in (2, 3, 4, 5):
@@ -465,6 +485,11 @@ def main():
                 continue
             r = run_spmv(c, args.steps, args.warmup, False, check, True)
             others["C%d_transposed" % c] = {k: r[k] for k in ("workload", "gbs", "gflops", "hbm_frac", "timing", "parity", "kernel")}
+        for c in (2, 3, 4):
+            if args.cx and c == args.config and not args.transpose:
+                continue
+            r = run_spmv(c, args.steps, args.warmup, False, check, False, False, True)
+            others["C%d_complex" % c] = {k: r[k] for k in ("workload", "gbs", "gflops", "hbm_frac", "timing", "parity", "kernel", "dtype")}
         for c, fmt in ((2, "ell"), (2, "coo"), (3, "ell"), (3, "coo")):
             if args.format == fmt and args.config == c:
                 continue

@@ -107,10 +107,10 @@ typedef struct asamd_csr_plan asamd_csr_plan;
 int asamd_csr_plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t nnz,
                           const int32_t *row_ptr, const int32_t *col_ind, const void *val,
                           int32_t base, int32_t val_size, int32_t trusted, asamd_csr_plan **plan);
-/* The same for any element type (dtype: enum asamd_dtype).  Complex plans run the
- * lane-group, merge-path, row-block and ELL-copy kernels (src/kernel/dcu/level2/mv/csrmv/
- * dcu_gemv_vector.h:14-57 is type-generic through ALPHA_Number); the tiled and the
- * constant-row-length kernels are for real types. */
+/* The same for any element type (dtype: enum asamd_dtype).  Complex plans run every
+ * kernel family (src/kernel/dcu/level2/mv/csrmv/dcu_gemv_vector.h:14-57 is type-generic
+ * through ALPHA_Number) except the constant-row-length one, whose 128-bit quads are
+ * for real types. */
 int asamd_csr_plan_create_dtype(hipStream_t stream, int32_t m, int32_t n, int32_t nnz,
                                 const int32_t *row_ptr, const int32_t *col_ind, const void *val,
                                 int32_t base, int32_t dtype, int32_t trusted, asamd_csr_plan **plan);

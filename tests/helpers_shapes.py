@@ -26,18 +26,5 @@ def csr_from_lengths(lengths, cols, dtype, seed=7, base=0):
                   "lengths(m=%d,nnz=%d)" % (len(lengths), col.size))
 
 
-def real_dtype(dtype):
-    """float32 for complex64, float64 for complex128, the dtype itself for real types."""
-    return np.empty(0, dtype=dtype).real.dtype
-
-
-def complex_vector(n, dtype, stream):
-    """Seeded complex vector: real parts from generator stream `stream`, imaginary from stream + 100."""
-    rd = real_dtype(dtype)
-    return (wl.uniform(n, rd, stream) + 1j * wl.uniform(n, rd, stream + 100)).astype(dtype)
-
-
-def complexify(a, dtype, stream=200):
-    """The structure of a real workload with seeded complex values of the given complex dtype."""
-    return wl.Csr(a.rows, a.cols, a.row_ptr, a.col_ind, complex_vector(a.nnz, dtype, stream), a.base,
-                  a.name + ":" + np.dtype(dtype).name)
+# complex-valued variants of the seeded workloads
+real_dtype, complex_vector, complexify = wl.real_dtype, wl.complex_vector, wl.complexify
