@@ -316,7 +316,7 @@ static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* 
   unsigned *d_key = nullptr, *d_key2 = nullptr, *d_idx = nullptr, *d_perm = nullptr;
   std::vector<int> h_off, cgb, rgb, cstart, rstart, h_colptr;
   std::vector<TiledChunk> h_chunks;
-  int cb = 0, rb = 0;
+  int cb = 0, rb = 0, count_stride = 1;
   int64_t tiles = 0;
 
   // ---- 1. entry counts per column group and per row group -> block cuts ----------
@@ -324,7 +324,9 @@ static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* 
   hipError_t e = hipMalloc(&d_cnt, cnt_n * sizeof(int));
   if (e == hipSuccess) e = hipMemsetAsync(d_cnt, 0, cnt_n * sizeof(int), stream);
   if (e == hipSuccess) {
-    col_group_count_kernel<<<256 * 32, 256, 0, stream>>>(st.nnz, col_ind, st.base, d_cnt);
+    // at least ~4 M sampled entries
+    while (((int64_t)st.nnz >> 23) >= (int64_t)2 * count_stride) count_stride *= 2;
+    col_group_count_kernel<<<256 * 32, 256, 0, stream>>>(st.nnz, col_ind, st.base, count_stride, d_cnt);
     h_off.resize(cnt_n + 1);
     e = hipMemcpyAsync(h_off.data() + 1, d_cnt, (size_t)col_groups * sizeof(int), hipMemcpyDeviceToHost, stream);
   }
@@ -334,7 +336,7 @@ static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* 
     for (int g = 0; g < col_groups; ++g) h_off[(size_t)g + 1] += h_off[(size_t)g];
     const int64_t full = ((int64_t)st.n + TileDims<T>::cols - 1) / TileDims<T>::cols;
     cstart = cut_blocks(h_off.data(), col_groups, TileDims<T>::cols >> kColGroupLog2,
-                        (int64_t)st.nnz / full + 1, cgb);
+                        (int64_t)h_off[(size_t)col_groups] / full + 1, cgb);  // h_off: sampled entries
     cb = (int)cstart.size() - 1;
     row_group_offsets_kernel<<<(row_groups + 1 + 255) / 256, 256, 0, stream>>>(st.m, row_ptr, row_groups, d_cnt);
     e = hipMemcpyAsync(h_off.data(), d_cnt, ((size_t)row_groups + 1) * sizeof(int), hipMemcpyDeviceToHost, stream);
@@ -493,7 +495,8 @@ static hipError_t tune_copies(hipStream_t stream, asamd_csr_plan* p, const int* 
   for (int a = 0; a < 3 && e == hipSuccess; ++a) {
     if (!have[a]) continue;
     st.algo = algos[a];
-    for (int rep = 0; rep < 3 && e == hipSuccess; ++rep) {
+    int reps = 3;  // first run warms up; multiplies of a millisecond and more are timed once, shorter ones twice
+    for (int rep = 0; rep < reps && e == hipSuccess; ++rep) {
       e = hipEventRecord(e0, stream);
       if (e == hipSuccess)
         e = (hipError_t)csrmv_impl<T>(stream, p, T(1), val, row_ptr, col_ind, x, T(0), y);
@@ -501,7 +504,8 @@ static hipError_t tune_copies(hipStream_t stream, asamd_csr_plan* p, const int* 
       if (e == hipSuccess) e = hipEventSynchronize(e1);
       float ms = 0.f;
       if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
-      if (rep > 0 && (best[a] == 0.f || ms < best[a])) best[a] = ms;  // first run warms up
+      if (rep == 0 && ms > 1.0f) reps = 2;
+      if (rep > 0 && (best[a] == 0.f || ms < best[a])) best[a] = ms;
     }
   }
   if (e0) (void)hipEventDestroy(e0);

@@ -94,12 +94,22 @@ struct LongChunk {
 };
 
 // ---- analysis ----------------------------------------------------------------
-// Entries per group of 256 columns (for cutting equal-entry column blocks).
+// Entries per group of 256 columns (for cutting equal-entry column blocks), counted on a sample:
+// every stride-th run of kCountRun consecutive entries.  The counts only steer where the blocks are
+// cut, so a few million samples are as good as all entries, and the atomics (which collide on hot
+// columns) stay few.  Runs of consecutive entries hold whole rows, so the sample is not biased
+// towards any position inside a row.
+constexpr int kCountRun = 1024;
 __global__ __launch_bounds__(256) void col_group_count_kernel(int nnz, const int* __restrict__ col_ind,
-                                                              int base, int* __restrict__ count) {
-  for (int64_t k = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; k < nnz;
-       k += (int64_t)gridDim.x * blockDim.x)
-    atomicAdd(&count[(col_ind[k] - base) >> kColGroupLog2], 1);
+                                                              int base, int stride, int* __restrict__ count) {
+  const int64_t runs = ((int64_t)nnz + kCountRun - 1) / kCountRun;
+  for (int64_t run = (int64_t)blockIdx.x * stride; run < runs; run += (int64_t)gridDim.x * stride) {
+    const int64_t k0 = run * kCountRun;
+    for (int i = threadIdx.x; i < kCountRun; i += 256) {
+      const int64_t k = k0 + i;
+      if (k < nnz) atomicAdd(&count[(col_ind[k] - base) >> kColGroupLog2], 1);
+    }
+  }
 }
 
 // out[g] = row_ptr[g * 64] for g in [0, groups], the last one clamped to row_ptr[m].

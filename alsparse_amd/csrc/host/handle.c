@@ -59,23 +59,25 @@ alphasparse_status_t alphasparse_dcu_get_handle(alphasparse_dcu_handle_t *handle
 
   /* scratch: at least 1 MiB, as the reference sizes it (handle.cpp:94-105) */
   h->buffer_size = (size_t)1 << 20;
-  ASAMD_HIP_STATUS(hipMalloc(&h->buffer, h->buffer_size));
-  ASAMD_HIP_STATUS(hipMalloc((void **)&h->sone, sizeof(float)));
-  ASAMD_HIP_STATUS(hipMalloc((void **)&h->done, sizeof(double)));
-  ASAMD_HIP_STATUS(hipMalloc((void **)&h->cone, sizeof(ALPHA_Complex8)));
-  ASAMD_HIP_STATUS(hipMalloc((void **)&h->zone, sizeof(ALPHA_Complex16)));
-
-  ASAMD_HIP_STATUS(asamd_warmup(h->stream));
-
   const float s1 = 1.0f;
   const double d1 = 1.0;
   const ALPHA_Complex8 c1 = {1.0f, 0.0f};
   const ALPHA_Complex16 z1 = {1.0, 0.0};
-  ASAMD_HIP_STATUS(hipMemcpyAsync(h->sone, &s1, sizeof s1, hipMemcpyHostToDevice, h->stream));
-  ASAMD_HIP_STATUS(hipMemcpyAsync(h->done, &d1, sizeof d1, hipMemcpyHostToDevice, h->stream));
-  ASAMD_HIP_STATUS(hipMemcpyAsync(h->cone, &c1, sizeof c1, hipMemcpyHostToDevice, h->stream));
-  ASAMD_HIP_STATUS(hipMemcpyAsync(h->zone, &z1, sizeof z1, hipMemcpyHostToDevice, h->stream));
-  ASAMD_HIP_STATUS(hipStreamSynchronize(h->stream));
+  hipError_t e = hipMalloc(&h->buffer, h->buffer_size);
+  if (e == hipSuccess) e = hipMalloc((void **)&h->sone, sizeof(float));
+  if (e == hipSuccess) e = hipMalloc((void **)&h->done, sizeof(double));
+  if (e == hipSuccess) e = hipMalloc((void **)&h->cone, sizeof(ALPHA_Complex8));
+  if (e == hipSuccess) e = hipMalloc((void **)&h->zone, sizeof(ALPHA_Complex16));
+  if (e == hipSuccess) e = (hipError_t)asamd_warmup(h->stream);
+  if (e == hipSuccess) e = hipMemcpyAsync(h->sone, &s1, sizeof s1, hipMemcpyHostToDevice, h->stream);
+  if (e == hipSuccess) e = hipMemcpyAsync(h->done, &d1, sizeof d1, hipMemcpyHostToDevice, h->stream);
+  if (e == hipSuccess) e = hipMemcpyAsync(h->cone, &c1, sizeof c1, hipMemcpyHostToDevice, h->stream);
+  if (e == hipSuccess) e = hipMemcpyAsync(h->zone, &z1, sizeof z1, hipMemcpyHostToDevice, h->stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(h->stream); /* the constants above live on this stack frame */
+  if (e != hipSuccess) {
+    (void)alphasparse_dcu_destory_handle(h); /* releases whatever was allocated; the struct stays the caller's */
+    return get_alphasparse_dcu_status_for_hip_status(e);
+  }
   return ALPHA_SPARSE_STATUS_SUCCESS;
 }
 
