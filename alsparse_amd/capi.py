@@ -170,6 +170,10 @@ def _per_type(ctype):
                                        POINTER(_P), POINTER(_P), POINTER(_P), POINTER(_P)],
         "alphasparse_{s}_mv": [c_int, T, alphasparse_matrix_t, alpha_matrix_descr, _P, T, _P],
         "alphasparse_{s}_mm": [c_int, T, alphasparse_matrix_t, alpha_matrix_descr, c_int, _P, _I, _I, T, _P, _I],
+        "alphasparse_{s}_mv_plain": [c_int, T, alphasparse_matrix_t, alpha_matrix_descr, _P, T, _P],
+        "alphasparse_{s}_mm_plain": [c_int, T, alphasparse_matrix_t, alpha_matrix_descr, c_int, _P, _I, _I, T, _P, _I],
+        "asamd_{s}_csrmv_plain": [_P, _I, _I, _I, _I, T, _P, _P, _P, _P, T, _P],
+        "asamd_{s}_csrmm_plain": [_P, _I, _I, T, _P, _P, _P, _I, _P, T, _P, POINTER(asamd_dense_strides)],
         "host2device_{s}_csr": [alphasparse_matrix_t],
         "host2device_{s}_coo": [alphasparse_matrix_t],
         "host2device_{s}_ell": [alphasparse_matrix_t],
@@ -255,6 +259,9 @@ _COMMON = {
     "alpha_args_get_transA": [c_int, POINTER(ctypes.c_char_p)],
     "alpha_args_get_transB": [c_int, POINTER(ctypes.c_char_p)],
     "get_time_us": [],
+    "alpha_get_core_num": [],
+    "alpha_set_thread_num": [c_int],
+    "alpha_get_thread_num": [],
     "init_handle": [POINTER(alphasparse_dcu_handle_t)],
     "alphasparse_dcu_get_handle": [POINTER(alphasparse_dcu_handle_t)],
     "alphasparse_dcu_destory_handle": [alphasparse_dcu_handle_t],
@@ -282,6 +289,7 @@ _COMMON = {
     "asamd_csr_plan_build_transpose": [_P, _P, _P, _P, _P],
     "asamd_csr_plan_set_lazy_transpose": [_P, _I],
     "asamd_csr_plan_transpose_stats": [_P],
+    "asamd_csr_plan_transpose_arrays": [_P, _I, POINTER(_P), POINTER(_P), POINTER(_P)],
     "asamd_csrmm_workspace_bytes": [_I, _I, _I, _I, POINTER(asamd_dense_strides)],
     "asamd_csr2coo": [_P, _P, _I, _I, _P, _I],
     "asamd_csr2ell_width": [_P, _I, _P, POINTER(_I)],
@@ -306,7 +314,7 @@ def prototypes():
     return out
 
 
-_RESTYPE = {"asamd_csr_plan_destroy": None, "asamd_handle_get_stream": c_void_p, "alpha_malloc": c_void_p, "alpha_memalign": c_void_p, "alpha_free": None,
+_RESTYPE = {"alpha_set_thread_num": None, "asamd_csr_plan_destroy": None, "asamd_handle_get_stream": c_void_p, "alpha_malloc": c_void_p, "alpha_memalign": c_void_p, "alpha_free": None,
             "alpha_fill_random_s": None, "alpha_fill_random_d": None, "alpha_read_coo": None, "alpha_read_coo_d": None,
             "alpha_fill_random_c": None, "alpha_fill_random_z": None, "alpha_read_coo_c": None, "alpha_read_coo_z": None,
             "args_help": None, "args_get_if_check": c_bool, "args_get_data_file": ctypes.c_char_p,

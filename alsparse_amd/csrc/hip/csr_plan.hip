@@ -752,6 +752,17 @@ extern "C" const asamd_csr_stats* asamd_csr_plan_transpose_stats(const asamd_csr
   return p->tr[1].plan ? &p->tr[1].plan->st : nullptr;
 }
 
+extern "C" int asamd_csr_plan_transpose_arrays(const asamd_csr_plan* p, int32_t conj, const int32_t** row_ptr,
+                                               const int32_t** col_ind, const void** val) {
+  if (!p || !row_ptr || !col_ind || !val) return hipErrorInvalidValue;
+  const asamd_csr_plan::TransCopy& t = p->tr[conj ? 1 : 0];
+  if (!t.plan) return hipErrorInvalidValue;
+  *row_ptr = t.d_row_ptr;
+  *col_ind = t.d_col;
+  *val = t.d_val;
+  return hipSuccess;
+}
+
 extern "C" const asamd_csr_stats* asamd_csr_plan_stats(const asamd_csr_plan* p) {
   return p ? &p->st : nullptr;
 }
@@ -1012,6 +1023,62 @@ extern "C" int asamd_z_csrmv_op(hipStream_t stream, asamd_csr_plan* plan, int32_
                                 const asamd_complex16* val, const int32_t* row_ptr, const int32_t* col_ind,
                                 const asamd_complex16* x, asamd_complex16 beta, asamd_complex16* y) {
   return csrmv_complex<Cx<double>>(stream, plan, op, alpha, val, row_ptr, col_ind, x, beta, y);
+}
+
+// ---- the unanalysed, one-lane-per-row path ("plain") ---------------------------------------------
+// op 0: every row summed by one lane in storage order; op 1 / 2: y scaled by beta, then one lane per
+// row scatters alpha*op(a)*x[row] with atomics, the traversal of the reference's own transposed kernels.
+template <typename T>
+static int csrmv_plain_impl(hipStream_t s, int32_t op, int32_t m, int32_t n, int32_t base, T alpha, const T* val,
+                            const int* rp, const int* ci, const T* x, T beta, T* y) {
+  if (!val || !rp || !ci || !x || !y || m <= 0 || n <= 0 || op < 0 || op > 2 || (op == 2 && kIsReal<T>))
+    return hipErrorInvalidValue;
+  if (((uintptr_t)val | (uintptr_t)x | (uintptr_t)y) % alignof(T)) return hipErrorInvalidValue;
+  if (op == 0) {
+    const unsigned grid = (unsigned)(((int64_t)m + kRowsBlock - 1) / kRowsBlock);
+    spmv_scalar_kernel<T><<<grid, kRowsBlock, 0, s>>>(m, alpha, val, rp, ci, x, beta, y, base);
+    return hipGetLastError();
+  }
+  if (beta != T(1)) scale_vec_kernel<T><<<(unsigned)(((int64_t)n + 255) / 256), 256, 0, s>>>(n, beta, y);
+  const unsigned grid = (unsigned)(((int64_t)m + kTransThreads - 1) / kTransThreads);
+  if constexpr (!kIsReal<T>) {
+    if (op == 2) {
+      csrmv_trans_scatter_kernel<T, 1, true><<<grid, kTransThreads, 0, s>>>(m, n, alpha, val, rp, ci, x, y, base);
+      return hipGetLastError();
+    }
+  }
+  csrmv_trans_scatter_kernel<T, 1, false><<<grid, kTransThreads, 0, s>>>(m, n, alpha, val, rp, ci, x, y, base);
+  return hipGetLastError();
+}
+
+extern "C" int asamd_s_csrmv_plain(hipStream_t stream, int32_t op, int32_t m, int32_t n, int32_t base, float alpha,
+                                   const float* val, const int32_t* row_ptr, const int32_t* col_ind, const float* x,
+                                   float beta, float* y) {
+  return csrmv_plain_impl<float>(stream, op, m, n, base, alpha, val, row_ptr, col_ind, x, beta, y);
+}
+
+extern "C" int asamd_d_csrmv_plain(hipStream_t stream, int32_t op, int32_t m, int32_t n, int32_t base, double alpha,
+                                   const double* val, const int32_t* row_ptr, const int32_t* col_ind, const double* x,
+                                   double beta, double* y) {
+  return csrmv_plain_impl<double>(stream, op, m, n, base, alpha, val, row_ptr, col_ind, x, beta, y);
+}
+
+extern "C" int asamd_c_csrmv_plain(hipStream_t stream, int32_t op, int32_t m, int32_t n, int32_t base,
+                                   asamd_complex8 alpha, const asamd_complex8* val, const int32_t* row_ptr,
+                                   const int32_t* col_ind, const asamd_complex8* x, asamd_complex8 beta,
+                                   asamd_complex8* y) {
+  using T = Cx<float>;
+  return csrmv_plain_impl<T>(stream, op, m, n, base, T(alpha.real, alpha.imag), (const T*)val, row_ptr, col_ind,
+                             (const T*)x, T(beta.real, beta.imag), (T*)y);
+}
+
+extern "C" int asamd_z_csrmv_plain(hipStream_t stream, int32_t op, int32_t m, int32_t n, int32_t base,
+                                   asamd_complex16 alpha, const asamd_complex16* val, const int32_t* row_ptr,
+                                   const int32_t* col_ind, const asamd_complex16* x, asamd_complex16 beta,
+                                   asamd_complex16* y) {
+  using T = Cx<double>;
+  return csrmv_plain_impl<T>(stream, op, m, n, base, T(alpha.real, alpha.imag), (const T*)val, row_ptr, col_ind,
+                             (const T*)x, T(beta.real, beta.imag), (T*)y);
 }
 
 extern "C" int asamd_copy_bytes(hipStream_t stream, void* dst, const void* src, size_t nbytes) {

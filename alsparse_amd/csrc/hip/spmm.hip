@@ -438,6 +438,51 @@ extern "C" int asamd_d_csrmm(hipStream_t stream, int32_t m, int32_t n, int32_t k
                             strides, nullptr, 0);
 }
 
+// ---- the unanalysed, one-lane-per-element path ("plain"): entries of a row in storage order ---
+template <typename T>
+static int csrmm_plain_impl(hipStream_t s, int m, int n, T alpha, const T* val, const int* rp, const int* ci,
+                            int base, const T* B, T beta, T* C, const asamd_dense_strides* st) {
+  if (!val || !rp || !ci || !B || !C || !st || m <= 0 || n <= 0) return hipErrorInvalidValue;
+  if (((uintptr_t)val | (uintptr_t)B | (uintptr_t)C) % alignof(T)) return hipErrorInvalidValue;
+  const dim3 block(kWave, kSpmmBlock / kWave);
+  unsigned gy = (unsigned)((n + block.y - 1) / block.y);
+  if (gy > 65535u) gy = 65535u;
+  const dim3 grid((unsigned)(((int64_t)m + kWave - 1) / kWave), gy);
+  spmm_strided_kernel<T><<<grid, block, 0, s>>>(m, n, alpha, val, rp, ci, base, B, st->b_row_stride,
+                                                st->b_col_stride, beta, C, st->c_row_stride, st->c_col_stride);
+  return hipGetLastError();
+}
+
+extern "C" int asamd_s_csrmm_plain(hipStream_t stream, int32_t m, int32_t n, float alpha, const float* val,
+                                   const int32_t* row_ptr, const int32_t* col_ind, int32_t base, const float* B,
+                                   float beta, float* C, const asamd_dense_strides* strides) {
+  return csrmm_plain_impl<float>(stream, m, n, alpha, val, row_ptr, col_ind, base, B, beta, C, strides);
+}
+
+extern "C" int asamd_d_csrmm_plain(hipStream_t stream, int32_t m, int32_t n, double alpha, const double* val,
+                                   const int32_t* row_ptr, const int32_t* col_ind, int32_t base, const double* B,
+                                   double beta, double* C, const asamd_dense_strides* strides) {
+  return csrmm_plain_impl<double>(stream, m, n, alpha, val, row_ptr, col_ind, base, B, beta, C, strides);
+}
+
+extern "C" int asamd_c_csrmm_plain(hipStream_t stream, int32_t m, int32_t n, asamd_complex8 alpha,
+                                   const asamd_complex8* val, const int32_t* row_ptr, const int32_t* col_ind,
+                                   int32_t base, const asamd_complex8* B, asamd_complex8 beta, asamd_complex8* C,
+                                   const asamd_dense_strides* strides) {
+  using T = Cx<float>;
+  return csrmm_plain_impl<T>(stream, m, n, T(alpha.real, alpha.imag), (const T*)val, row_ptr, col_ind, base,
+                             (const T*)B, T(beta.real, beta.imag), (T*)C, strides);
+}
+
+extern "C" int asamd_z_csrmm_plain(hipStream_t stream, int32_t m, int32_t n, asamd_complex16 alpha,
+                                   const asamd_complex16* val, const int32_t* row_ptr, const int32_t* col_ind,
+                                   int32_t base, const asamd_complex16* B, asamd_complex16 beta, asamd_complex16* C,
+                                   const asamd_dense_strides* strides) {
+  using T = Cx<double>;
+  return csrmm_plain_impl<T>(stream, m, n, T(alpha.real, alpha.imag), (const T*)val, row_ptr, col_ind, base,
+                             (const T*)B, T(beta.real, beta.imag), (T*)C, strides);
+}
+
 // ---- complex element types: the same kernels over Cx<float> / Cx<double> -------------------
 static_assert(sizeof(asamd_complex8) == sizeof(Cx<float>) && sizeof(asamd_complex16) == sizeof(Cx<double>),
               "complex layouts");

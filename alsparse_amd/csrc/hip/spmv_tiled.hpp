@@ -71,6 +71,9 @@ struct TileDims {
   // block keeps 2048 rows (tiles per matrix, which is what phase 2 pays for, do not double)
   static constexpr int red_bytes = sizeof(T) >= 8 ? kTileBytes : kRedBytes;
   static constexpr int rows = red_bytes / kRedWaves / (int)sizeof(T);  // tallest row block: 2048 (1024 for 16-byte values)
+  // tiles per batch of phase 2 (16 per batch were measured no faster for 8-byte values and spill
+  // registers for 16-byte ones)
+  static constexpr int red_unroll = kRedUnroll;
 };
 
 struct TiledChunk {
@@ -299,6 +302,7 @@ __global__ __launch_bounds__(kRedThreads) void tiled_reduce_kernel(
   extern __shared__ __align__(16) unsigned char smem[];
   T* s_acc = reinterpret_cast<T*>(smem);
   constexpr int kTileRows = TileDims<T>::rows;
+  constexpr int kUnroll = TileDims<T>::red_unroll;
   const int lane = threadIdx.x % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int rb = blockIdx.x * kRedWaves + wave;
@@ -306,18 +310,18 @@ __global__ __launch_bounds__(kRedThreads) void tiled_reduce_kernel(
   T* acc = s_acc + wave * kTileRows;
   for (int i = lane; i < kTileRows; i += kWave) acc[i] = T(0);
 
-  // Wave-private accumulators; the tiles of kRedUnroll column blocks form a batch
+  // Wave-private accumulators; the tiles of kUnroll column blocks form a batch
   // (every tile listed in `ranges` has at most kLongTile = 128 entries: two per
   // lane).  The loads of batch q + 1 are issued before batch q is added, so the
   // LDS read-modify-write chain of one batch hides the memory latency of the next.
   struct Batch {
-    T v[kRedUnroll][2];
-    int r[kRedUnroll][2];
-    int len[kRedUnroll];
+    T v[kUnroll][2];
+    int r[kUnroll][2];
+    int len[kUnroll];
   };
   const TileRange* my = ranges + (int64_t)(active ? rb : 0) * col_blocks;
-  constexpr int kPerGroup = kWave / kRedUnroll;  // batches per group of 64 tile ranges
-  const int nq = (col_blocks + kRedUnroll - 1) / kRedUnroll;
+  constexpr int kPerGroup = kWave / kUnroll;  // batches per group of 64 tile ranges
+  const int nq = (col_blocks + kUnroll - 1) / kUnroll;
   auto load_ranges = [&](int group) {  // 64 tile ranges, one coalesced load
     TileRange t = {0, 0};
     const int cb = group * kWave + lane;
@@ -326,11 +330,11 @@ __global__ __launch_bounds__(kRedThreads) void tiled_reduce_kernel(
   };
   const int r_none = -2 - lane;  // "no entry": negative and different in every lane
   auto fetch = [&](const TileRange& tr, int q, Batch& bt) {
-    const int j = (q % kPerGroup) * kRedUnroll;
+    const int j = (q % kPerGroup) * kUnroll;
     const int left = col_blocks - (q / kPerGroup) * kWave;
     const int ncb = left < kWave ? left : kWave;
 #pragma unroll
-    for (int u = 0; u < kRedUnroll; ++u) {
+    for (int u = 0; u < kUnroll; ++u) {
       const int src = j + u < ncb ? j + u : j;
       const int b = __builtin_amdgcn_readlane(tr.begin, src);
       const int e = j + u < ncb ? __builtin_amdgcn_readlane(tr.end, src) : b;
@@ -351,7 +355,7 @@ __global__ __launch_bounds__(kRedThreads) void tiled_reduce_kernel(
   };
   auto add = [&](const Batch& bt) {
 #pragma unroll
-    for (int u = 0; u < kRedUnroll; ++u) {
+    for (int u = 0; u < kUnroll; ++u) {
       add_rows(acc, bt.r[u][0], bt.v[u][0], bt.r[u][0] >= 0);
       if (bt.len[u] > kWave) add_rows(acc, bt.r[u][1], bt.v[u][1], bt.r[u][1] >= 0);  // wave-uniform
     }

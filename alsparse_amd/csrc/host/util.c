@@ -6,6 +6,7 @@
 #include <getopt.h>
 #include <math.h>
 #include <string.h>
+#include <unistd.h>
 #include <sys/time.h>
 #include <time.h>
 
@@ -43,6 +44,18 @@ void alpha_fill_random_d(double *arr, unsigned int seed, const size_t size) {
   srand(seed_or_clock(seed));
   for (size_t i = 0; i < size; ++i) arr[i] = (double)rand() / (double)RAND_MAX;
 }
+
+/* ---- thread count of the reference's CPU kernels (kept, not used: the GPU multiplies) ---------- */
+static int g_thread_num;
+
+int alpha_get_core_num(void) {
+  const long n = sysconf(_SC_NPROCESSORS_ONLN);
+  return n > 0 ? (int)n : 1;
+}
+
+void alpha_set_thread_num(const int thread_num) { g_thread_num = thread_num; }
+
+int alpha_get_thread_num(void) { return g_thread_num == 0 ? alpha_get_core_num() : g_thread_num; }
 
 /* src/util/malloc.c:104-112: a complex array is filled as twice as many reals */
 void alpha_fill_random_c(ALPHA_Complex8 *arr, unsigned int seed, const size_t size) {

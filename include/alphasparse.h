@@ -303,7 +303,9 @@ alphasparse_status_t alphasparse_d_mv(const alphasparse_operation_t operation, c
 
 /* ---- Y = alpha*op(A)*X + beta*Y ------------------------------------------
  * include/alphasparse/spapi.h:899-923; validation order from
- * src/core/op/level3/alphasparse_x_mm.c:2305-2338.  x and y are host arrays. */
+ * src/core/op/level3/alphasparse_x_mm.c:2305-2338.  x and y are host arrays.  op(A) = A^T (A^H for
+ * complex types) multiplies with a CSR copy of the transpose kept with the handle's device mirror,
+ * as src/kernel/x86_64/level3/mm/gemm/gemm_x_csr_row_trans.c does per call. */
 alphasparse_status_t alphasparse_s_mm(const alphasparse_operation_t operation, const float alpha,
                                       const alphasparse_matrix_t A,
                                       const struct alpha_matrix_descr descr,
@@ -316,6 +318,54 @@ alphasparse_status_t alphasparse_d_mm(const alphasparse_operation_t operation, c
                                       const alphasparse_layout_t layout, const double *x,
                                       const ALPHA_INT columns, const ALPHA_INT ldx,
                                       const double beta, double *y, const ALPHA_INT ldy);
+
+/* ---- the reference's "plain" entry points ---------------------------------------
+ * include/alphasparse/spapi_plain.h:13-43 (mv), :227-275 (mm); validation of
+ * src/plain/op/alphasparse_x_mv_plain.c:537-564 and alphasparse_x_mm_plain.c:912-945.  In the
+ * reference they run its serial, unoptimised CPU kernels and serve as the yardstick of its own tests.
+ * Here they run on the GPU as well, through the unanalysed kernels that keep the plain kernels'
+ * traversal: one lane per row (per element of Y) walking the entries in storage order, transposed
+ * operations as a scatter.  Same arguments and status codes as alphasparse_?_mv / _mm. */
+alphasparse_status_t alphasparse_s_mv_plain(const alphasparse_operation_t operation, const float alpha,
+                                      const alphasparse_matrix_t A,
+                                      const struct alpha_matrix_descr descr, const float *x,
+                                      const float beta, float *y);
+alphasparse_status_t alphasparse_s_mm_plain(const alphasparse_operation_t operation, const float alpha,
+                                      const alphasparse_matrix_t A,
+                                      const struct alpha_matrix_descr descr,
+                                      const alphasparse_layout_t layout, const float *x,
+                                      const ALPHA_INT columns, const ALPHA_INT ldx,
+                                      const float beta, float *y, const ALPHA_INT ldy);
+alphasparse_status_t alphasparse_d_mv_plain(const alphasparse_operation_t operation, const double alpha,
+                                      const alphasparse_matrix_t A,
+                                      const struct alpha_matrix_descr descr, const double *x,
+                                      const double beta, double *y);
+alphasparse_status_t alphasparse_d_mm_plain(const alphasparse_operation_t operation, const double alpha,
+                                      const alphasparse_matrix_t A,
+                                      const struct alpha_matrix_descr descr,
+                                      const alphasparse_layout_t layout, const double *x,
+                                      const ALPHA_INT columns, const ALPHA_INT ldx,
+                                      const double beta, double *y, const ALPHA_INT ldy);
+alphasparse_status_t alphasparse_c_mv_plain(const alphasparse_operation_t operation, const ALPHA_Complex8 alpha,
+                                      const alphasparse_matrix_t A,
+                                      const struct alpha_matrix_descr descr, const ALPHA_Complex8 *x,
+                                      const ALPHA_Complex8 beta, ALPHA_Complex8 *y);
+alphasparse_status_t alphasparse_c_mm_plain(const alphasparse_operation_t operation, const ALPHA_Complex8 alpha,
+                                      const alphasparse_matrix_t A,
+                                      const struct alpha_matrix_descr descr,
+                                      const alphasparse_layout_t layout, const ALPHA_Complex8 *x,
+                                      const ALPHA_INT columns, const ALPHA_INT ldx,
+                                      const ALPHA_Complex8 beta, ALPHA_Complex8 *y, const ALPHA_INT ldy);
+alphasparse_status_t alphasparse_z_mv_plain(const alphasparse_operation_t operation, const ALPHA_Complex16 alpha,
+                                      const alphasparse_matrix_t A,
+                                      const struct alpha_matrix_descr descr, const ALPHA_Complex16 *x,
+                                      const ALPHA_Complex16 beta, ALPHA_Complex16 *y);
+alphasparse_status_t alphasparse_z_mm_plain(const alphasparse_operation_t operation, const ALPHA_Complex16 alpha,
+                                      const alphasparse_matrix_t A,
+                                      const struct alpha_matrix_descr descr,
+                                      const alphasparse_layout_t layout, const ALPHA_Complex16 *x,
+                                      const ALPHA_INT columns, const ALPHA_INT ldx,
+                                      const ALPHA_Complex16 beta, ALPHA_Complex16 *y, const ALPHA_INT ldy);
 
 /* ---- complex element types ---------------------------------------------------
  * Payloads and entry points for ALPHA_Complex8 (c) and ALPHA_Complex16 (z), as their

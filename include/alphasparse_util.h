@@ -23,6 +23,13 @@ void alpha_fill_random_d(double *arr, unsigned int seed, const size_t size);
 void alpha_fill_random_c(ALPHA_Complex8 *arr, unsigned int seed, const size_t size);
 void alpha_fill_random_z(ALPHA_Complex16 *arr, unsigned int seed, const size_t size);
 
+/* include/alphasparse/util/thread.h:10-14; src/util/thread.c:11-38.  The reference's CPU kernels take
+ * their OpenMP thread count from here; this library multiplies on the GPU, so the number is only kept
+ * (0 means "all cores", as there) for programs that set it before alphasparse_?_mv / _mm. */
+int alpha_get_core_num(void);
+void alpha_set_thread_num(const int thread_num);
+int alpha_get_thread_num(void);
+
 /* include/alphasparse/util/io.h:19-20; src/util/io.c:39-114: Matrix Market
  * coordinate text ("%%MatrixMarket matrix coordinate <field> <symmetry>"):
  * one-based "row col [value]" lines become zero-based triplets, a missing value

@@ -168,6 +168,30 @@ int asamd_z_csrmv_op(hipStream_t stream, asamd_csr_plan *plan, int32_t op, asamd
                      const asamd_complex16 *val, const int32_t *row_ptr, const int32_t *col_ind,
                      const asamd_complex16 *x, asamd_complex16 beta, asamd_complex16 *y);
 
+/* Arrays of the plan's CSR copy of A^T (conj == 0) or A^H (conj != 0): n + 1 row offsets, nnz
+ * zero-based column indices (rows of A) and nnz values, owned by the plan.  hipErrorInvalidValue
+ * if that copy has not been built. */
+int asamd_csr_plan_transpose_arrays(const asamd_csr_plan *plan, int32_t conj, const int32_t **row_ptr,
+                                    const int32_t **col_ind, const void **val);
+
+/* y = alpha*op(A)*x + beta*y without any analysis, in the traversal of the reference's plain
+ * kernels: op = 0 one lane per row summing its entries in storage order
+ * (src/plain/kernel/level2/mv/gemv/gemv_x_csr_plain.c:11-22), op = 1 / 2 (2: complex types) one lane
+ * per row scattering into y (gemv_x_csr_trans_plain.c:10-24, gemv_c_csr_conj_plain.c:10-27; atomics
+ * make the order of those additions free).  Backs alphasparse_?_mv_plain. */
+int asamd_s_csrmv_plain(hipStream_t stream, int32_t op, int32_t m, int32_t n, int32_t base, float alpha,
+                        const float *val, const int32_t *row_ptr, const int32_t *col_ind, const float *x,
+                        float beta, float *y);
+int asamd_d_csrmv_plain(hipStream_t stream, int32_t op, int32_t m, int32_t n, int32_t base, double alpha,
+                        const double *val, const int32_t *row_ptr, const int32_t *col_ind, const double *x,
+                        double beta, double *y);
+int asamd_c_csrmv_plain(hipStream_t stream, int32_t op, int32_t m, int32_t n, int32_t base, asamd_complex8 alpha,
+                        const asamd_complex8 *val, const int32_t *row_ptr, const int32_t *col_ind,
+                        const asamd_complex8 *x, asamd_complex8 beta, asamd_complex8 *y);
+int asamd_z_csrmv_plain(hipStream_t stream, int32_t op, int32_t m, int32_t n, int32_t base, asamd_complex16 alpha,
+                        const asamd_complex16 *val, const int32_t *row_ptr, const int32_t *col_ind,
+                        const asamd_complex16 *x, asamd_complex16 beta, asamd_complex16 *y);
+
 /* Dense operand addressing for SpMM: element (r, c) of B is
  * B[r*b_row_stride + c*b_col_stride], of C is C[r*c_row_stride + c*c_col_stride]. */
 typedef struct {
@@ -187,6 +211,22 @@ int asamd_d_csrmm(hipStream_t stream, int32_t m, int32_t n, int32_t k, int32_t n
                   const double *val, const int32_t *row_ptr, const int32_t *col_ind, int32_t base,
                   const double *B, double beta, double *C,
                   const asamd_dense_strides *strides);
+
+/* C = alpha*A*B + beta*C, one lane per element of C walking its row of A in storage order, any
+ * strides (src/plain/kernel/level3/mm/gemm/gemm_x_csr_row_plain.c:6-21, gemm_x_csr_col_plain.c:6-19).
+ * Backs alphasparse_?_mm_plain. */
+int asamd_s_csrmm_plain(hipStream_t stream, int32_t m, int32_t n, float alpha, const float *val,
+                        const int32_t *row_ptr, const int32_t *col_ind, int32_t base, const float *B, float beta,
+                        float *C, const asamd_dense_strides *strides);
+int asamd_d_csrmm_plain(hipStream_t stream, int32_t m, int32_t n, double alpha, const double *val,
+                        const int32_t *row_ptr, const int32_t *col_ind, int32_t base, const double *B, double beta,
+                        double *C, const asamd_dense_strides *strides);
+int asamd_c_csrmm_plain(hipStream_t stream, int32_t m, int32_t n, asamd_complex8 alpha, const asamd_complex8 *val,
+                        const int32_t *row_ptr, const int32_t *col_ind, int32_t base, const asamd_complex8 *B,
+                        asamd_complex8 beta, asamd_complex8 *C, const asamd_dense_strides *strides);
+int asamd_z_csrmm_plain(hipStream_t stream, int32_t m, int32_t n, asamd_complex16 alpha, const asamd_complex16 *val,
+                        const int32_t *row_ptr, const int32_t *col_ind, int32_t base, const asamd_complex16 *B,
+                        asamd_complex16 beta, asamd_complex16 *C, const asamd_dense_strides *strides);
 
 /* Column-major B next to column-major C is multiplied from a row-major copy of B
  * (k*n elements) in a caller-provided device workspace; without one, or with too

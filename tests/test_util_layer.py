@@ -217,3 +217,13 @@ def test_coo_to_ell_conversion(lib, dtype):
     assert getattr(lib, "alphasparse_%s_export_ell" % p)(coo, byref(idx), byref(rr), byref(cc), byref(w), byref(ci), byref(va)) == S.ALPHA_SPARSE_STATUS_INVALID_VALUE
     assert lib.alphasparse_convert_ell(ell, 0, byref(capi.alphasparse_matrix_t())) == S.ALPHA_SPARSE_STATUS_INVALID_VALUE
     assert lib.alphasparse_destroy(coo) == 0 and lib.alphasparse_destroy(ell) == 0
+
+
+def test_thread_count_is_kept_as_in_the_reference():
+    """src/util/thread.c:22-38: 0 means every core, anything else is returned as set."""
+    lib = capi.load()
+    lib.alpha_set_thread_num(0)
+    assert lib.alpha_get_thread_num() == lib.alpha_get_core_num() >= 1
+    lib.alpha_set_thread_num(3)
+    assert lib.alpha_get_thread_num() == 3
+    lib.alpha_set_thread_num(0)
