@@ -172,6 +172,8 @@ def _per_type(ctype):
         "alphasparse_{s}_mm": [c_int, T, alphasparse_matrix_t, alpha_matrix_descr, c_int, _P, _I, _I, T, _P, _I],
         "alphasparse_{s}_mv_plain": [c_int, T, alphasparse_matrix_t, alpha_matrix_descr, _P, T, _P],
         "alphasparse_{s}_mm_plain": [c_int, T, alphasparse_matrix_t, alpha_matrix_descr, c_int, _P, _I, _I, T, _P, _I],
+        "check_{s}_l2": [_P, c_size_t, _P, c_size_t, _P, _P, T, T, c_int, POINTER(ctypes.c_char_p)],
+        "check_{s}_l3": [_P, _I, c_size_t, _P, _I, c_size_t, _P, _P, _I, _P, _I, T, T, c_int, POINTER(ctypes.c_char_p)],
         "asamd_{s}_csrmv_plain": [_P, _I, _I, _I, _I, T, _P, _P, _P, _P, T, _P],
         "asamd_{s}_csrmm_plain": [_P, _I, _I, T, _P, _P, _P, _I, _P, T, _P, POINTER(asamd_dense_strides)],
         "host2device_{s}_csr": [alphasparse_matrix_t],
@@ -259,6 +261,17 @@ _COMMON = {
     "alpha_args_get_transA": [c_int, POINTER(ctypes.c_char_p)],
     "alpha_args_get_transB": [c_int, POINTER(ctypes.c_char_p)],
     "get_time_us": [],
+    "alpha_timing_wtime": [],
+    "alpha_timing_start": [_P],
+    "alpha_timing_end": [_P],
+    "alpha_timing_elapsed_time": [_P],
+    "alpha_timing_gflops": [_P, c_int64],
+    "alpha_timing_elaped_time_print": [_P, ctypes.c_char_p],
+    "alpha_timing_gflops_print": [_P, c_int64, ctypes.c_char_p],
+    "alpha_clear_cache": [],
+    "alphasparse_nnz_counter_coo": [_P, _P, _I, POINTER(_I), POINTER(_I), POINTER(_I)],
+    "alphasparse_operations_mm": [_I, _I, _I, _I, _I, c_int, alpha_matrix_descr, _I, c_int],
+    "alphasparse_operations_mv": [_I, _I, _I, _I, _I, c_int, alpha_matrix_descr, c_int],
     "alpha_get_core_num": [],
     "alpha_set_thread_num": [c_int],
     "alpha_get_thread_num": [],
@@ -314,7 +327,10 @@ def prototypes():
     return out
 
 
-_RESTYPE = {"alpha_set_thread_num": None, "asamd_csr_plan_destroy": None, "asamd_handle_get_stream": c_void_p, "alpha_malloc": c_void_p, "alpha_memalign": c_void_p, "alpha_free": None,
+_RESTYPE = {"alpha_set_thread_num": None, "alpha_timing_wtime": c_double, "alpha_timing_start": None,
+            "alpha_timing_end": None, "alpha_timing_elapsed_time": c_double, "alpha_timing_gflops": c_double,
+            "alpha_timing_elaped_time_print": None, "alpha_timing_gflops_print": None, "alpha_clear_cache": None,
+            "alphasparse_nnz_counter_coo": None, "alphasparse_operations_mm": c_int64, "alphasparse_operations_mv": c_int64, "asamd_csr_plan_destroy": None, "asamd_handle_get_stream": c_void_p, "alpha_malloc": c_void_p, "alpha_memalign": c_void_p, "alpha_free": None,
             "alpha_fill_random_s": None, "alpha_fill_random_d": None, "alpha_read_coo": None, "alpha_read_coo_d": None,
             "alpha_fill_random_c": None, "alpha_fill_random_z": None, "alpha_read_coo_c": None, "alpha_read_coo_z": None,
             "args_help": None, "args_get_if_check": c_bool, "args_get_data_file": ctypes.c_char_p,

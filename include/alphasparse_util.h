@@ -13,6 +13,9 @@
 
 /* include/alphasparse/util/malloc.h:13-17, :37-38.  alpha_free releases the
  * block (the reference's frees only NULL pointers, src/util/malloc.c:45-48). */
+#ifndef DEFAULT_ALIGNMENT
+#define DEFAULT_ALIGNMENT 32 /* include/alphasparse/util/malloc.h:11 */
+#endif
 void *alpha_malloc(size_t bytes);
 void *alpha_memalign(size_t bytes, size_t alignment);
 void alpha_free(void *point);
@@ -56,6 +59,75 @@ int check_c(const ALPHA_Complex8 *answer_data, size_t answer_size, const ALPHA_C
             size_t result_size);
 int check_z(const ALPHA_Complex16 *answer_data, size_t answer_size, const ALPHA_Complex16 *result_data,
             size_t result_size);
+
+/* include/alphasparse/types.h:67-69 */
+#ifndef ALPHA_INT64
+#define ALPHA_INT64 int64_t
+#endif
+
+/* include/alphasparse/util/timing.h:7-20; src/util/timer.c: wall-clock timers of the CPU test programs */
+typedef struct {
+  double start;
+  double end;
+} alpha_timer_t;
+double alpha_timing_wtime(void);
+void alpha_timing_start(alpha_timer_t *timer);
+void alpha_timing_end(alpha_timer_t *timer);
+double alpha_timing_elapsed_time(const alpha_timer_t *timer);
+double alpha_timing_gflops(const alpha_timer_t *timer, int64_t operations);
+void alpha_timing_elaped_time_print(const alpha_timer_t *timer, const char *name);
+void alpha_timing_gflops_print(const alpha_timer_t *timer, int64_t operations, const char *name);
+/* include/alphasparse/util/malloc.h:23: flushes the CPU caches in the reference; no effect here */
+void alpha_clear_cache(void);
+
+/* include/alphasparse/util/analysis.h:6-8; src/util/analysis.c: entries below / on / above the
+ * diagonal, and the operation count the reference's programs divide their times by */
+void alphasparse_nnz_counter_coo(const ALPHA_INT *row_indx, const ALPHA_INT *col_indx, const ALPHA_INT nnz,
+                                 ALPHA_INT *lo_p, ALPHA_INT *diag_p, ALPHA_INT *hi_p);
+ALPHA_INT64 alphasparse_operations_mm(const ALPHA_INT rows, const ALPHA_INT cols, const ALPHA_INT lo,
+                                      const ALPHA_INT diag, const ALPHA_INT hi,
+                                      const alphasparse_operation_t operation,
+                                      const struct alpha_matrix_descr descr, const ALPHA_INT columns,
+                                      const alphasparse_datatype_t datatype);
+ALPHA_INT64 alphasparse_operations_mv(const ALPHA_INT rows, const ALPHA_INT cols, const ALPHA_INT lo,
+                                      const ALPHA_INT diag, const ALPHA_INT hi,
+                                      const alphasparse_operation_t operation,
+                                      const struct alpha_matrix_descr descr,
+                                      const alphasparse_datatype_t datatype);
+
+/* include/alphasparse/util/check.h:50-57; src/util/check.c:7-57 (level 2), :218-345 (level 3): the
+ * residual ||answer - result|| / (max(||A||_1,1) max(||x||,1) max(||result||,1) 10 eps max(m,k[,columns]))
+ * against 50, with A read again from --data-file; prints "correct,<resid>" (0) or "error,<resid>" (-1).
+ * Level 3 is served in its --data-file form (sparse times dense). */
+int check_s_l2(const float *answer_data, size_t answer_size, const float *result_data, size_t result_size,
+               const float *x, const float *y, const float alpha, const float beta, int argc, const char *argv[]);
+int check_d_l2(const double *answer_data, size_t answer_size, const double *result_data, size_t result_size,
+               const double *x, const double *y, const double alpha, const double beta, int argc,
+               const char *argv[]);
+int check_c_l2(const ALPHA_Complex8 *answer_data, size_t answer_size, const ALPHA_Complex8 *result_data,
+               size_t result_size, const ALPHA_Complex8 *x, const ALPHA_Complex8 *y, const ALPHA_Complex8 alpha,
+               const ALPHA_Complex8 beta, int argc, const char *argv[]);
+int check_z_l2(const ALPHA_Complex16 *answer_data, size_t answer_size, const ALPHA_Complex16 *result_data,
+               size_t result_size, const ALPHA_Complex16 *x, const ALPHA_Complex16 *y, const ALPHA_Complex16 alpha,
+               const ALPHA_Complex16 beta, int argc, const char *argv[]);
+int check_s_l3(const float *answer_data, const ALPHA_INT ldans, size_t answer_size, const float *result_data,
+               const ALPHA_INT ldres, size_t result_size, const ALPHA_INT *res_col_indx, const float *x,
+               const ALPHA_INT ldx, const float *y, const ALPHA_INT ldy, const float alpha, const float beta,
+               int argc, const char *argv[]);
+int check_d_l3(const double *answer_data, const ALPHA_INT ldans, size_t answer_size, const double *result_data,
+               const ALPHA_INT ldres, size_t result_size, const ALPHA_INT *res_col_indx, const double *x,
+               const ALPHA_INT ldx, const double *y, const ALPHA_INT ldy, const double alpha, const double beta,
+               int argc, const char *argv[]);
+int check_c_l3(const ALPHA_Complex8 *answer_data, const ALPHA_INT ldans, size_t answer_size,
+               const ALPHA_Complex8 *result_data, const ALPHA_INT ldres, size_t result_size,
+               const ALPHA_INT *res_col_indx, const ALPHA_Complex8 *x, const ALPHA_INT ldx, const ALPHA_Complex8 *y,
+               const ALPHA_INT ldy, const ALPHA_Complex8 alpha, const ALPHA_Complex8 beta, int argc,
+               const char *argv[]);
+int check_z_l3(const ALPHA_Complex16 *answer_data, const ALPHA_INT ldans, size_t answer_size,
+               const ALPHA_Complex16 *result_data, const ALPHA_INT ldres, size_t result_size,
+               const ALPHA_INT *res_col_indx, const ALPHA_Complex16 *x, const ALPHA_INT ldx,
+               const ALPHA_Complex16 *y, const ALPHA_INT ldy, const ALPHA_Complex16 alpha,
+               const ALPHA_Complex16 beta, int argc, const char *argv[]);
 
 /* include/alphasparse/util/args.h:16-44; src/util/args.c: GNU long options
  * --help --check --thread-num= --transA= --transB= --typeA= --fillA= --diagA=

@@ -22,7 +22,8 @@ def declared_functions():
             n = m.group(1)
             if n.startswith(("alphasparse_", "asamd_", "host2device_", "init_handle", "get_alphasparse", "alpha_malloc",
                              "alpha_memalign", "alpha_free", "alpha_fill_", "alpha_read_", "alpha_args_", "args_", "check_",
-                             "alpha_get_core_num", "alpha_set_thread_num", "alpha_get_thread_num",
+                             "alpha_get_core_num", "alpha_set_thread_num", "alpha_get_thread_num", "alpha_timing_",
+                             "alpha_clear_cache",
                              "get_time_us")):
                 names.add(n)
     return names

@@ -1,6 +1,6 @@
 """The reference's OWN GPU test programs (test/dcu/level2/mv_csr_?_dcu_test.cpp, mv_coo_?, mv_ell_?
 for ? in s, d, c, z; spmv_{csr,coo,ell}_s; test/dcu/level3/mm_csr_?_dcu_test.cpp,
-mm_csr_s_dcu_row_test.cpp), compiled unchanged
+mm_csr_s_dcu_row_test.cpp; and the CPU programs test/arm/mv_?_csr_arm_test.c, mm_?_csr_arm_test.c), compiled unchanged
 against this repository's headers and library by `make -C oracle ref_drivers` (into oracle/_ref/,
 where the reference tree is present) and run here on a coordinate file: they read the file, take
 the COO -> CSR / ELL route, call alphasparse_dcu_?_csrmv / _csrmm / _coomv / _ellmv and compare with
@@ -41,6 +41,16 @@ PROGRAMS = {
     "mv_ell_z_dcu_test": [[]],
     "mm_csr_c_dcu_test": [["--columns=8", "--layout=C"]],
     "mm_csr_z_dcu_test": [["--columns=8", "--layout=C"]],
+    # the CPU test programs (test/arm/*.c): alphasparse_?_mv / _mm against the _plain variants through
+    # check_?_l2 / _l3; both run on the GPU here, through different kernels
+    "mv_s_csr_arm_test": [[], ["--transA=T"]],
+    "mv_d_csr_arm_test": [[], ["--transA=T"]],
+    "mv_c_csr_arm_test": [[], ["--transA=T"], ["--transA=H"]],
+    "mv_z_csr_arm_test": [[], ["--transA=T"], ["--transA=H"]],
+    "mm_s_csr_arm_test": [["--columns=8"], ["--columns=8", "--layout=C"], ["--columns=8", "--transA=T"]],
+    "mm_d_csr_arm_test": [["--columns=8"], ["--columns=8", "--layout=C", "--transA=T"]],
+    "mm_c_csr_arm_test": [["--columns=8"], ["--columns=8", "--layout=C", "--transA=H"]],
+    "mm_z_csr_arm_test": [["--columns=8"], ["--columns=8", "--transA=H"]],
 }
 
 

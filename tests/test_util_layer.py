@@ -227,3 +227,50 @@ def test_thread_count_is_kept_as_in_the_reference():
     lib.alpha_set_thread_num(3)
     assert lib.alpha_get_thread_num() == 3
     lib.alpha_set_thread_num(0)
+
+
+def test_operation_counts_and_timers():
+    """src/util/analysis.c:8-56, :126-153 and src/util/timer.c of the reference."""
+    import ctypes
+    from ctypes import byref, c_int32
+    lib = capi.load()
+    rows = np.array([0, 1, 1, 2, 2, 2], dtype=np.int32)
+    cols = np.array([0, 0, 1, 0, 2, 3], dtype=np.int32)
+    lo, di, hi = c_int32(), c_int32(), c_int32()
+    lib.alphasparse_nnz_counter_coo(capi.ptr(rows), capi.ptr(cols), 6, byref(lo), byref(di), byref(hi))
+    assert (lo.value, di.value, hi.value) == (2, 3, 1)
+    general = capi.alpha_matrix_descr(0, 0, 0)
+    # real: 2 flops per entry + 3 per row; complex: 9 per entry + 16 per row; times the dense columns
+    assert lib.alphasparse_operations_mv(3, 4, 2, 3, 1, 0, general, 0) == 6 * 2 + 3 * 3
+    assert lib.alphasparse_operations_mm(3, 4, 2, 3, 1, 0, general, 5, 3) == (6 * 9 + 3 * 16) * 5
+    lower_unit = capi.alpha_matrix_descr(capi.ALPHA_SPARSE_MATRIX_TYPE_SYMMETRIC, 0, 1)
+    assert lib.alphasparse_operations_mv(3, 4, 2, 3, 1, 0, lower_unit, 0) == (2 + 3) * 2 + 3 * 3
+
+    class Timer(ctypes.Structure):
+        _fields_ = [("start", ctypes.c_double), ("end", ctypes.c_double)]
+    t = Timer()
+    lib.alpha_timing_start(byref(t))
+    lib.alpha_timing_end(byref(t))
+    assert 0 <= lib.alpha_timing_elapsed_time(byref(t)) < 1.0
+    t.start, t.end = 1.0, 3.0
+    assert lib.alpha_timing_gflops(byref(t), 4_000_000_000) == 2.0
+    lib.alpha_clear_cache()
+
+
+def test_level2_residual_check_accepts_rounding_and_rejects_errors(tmp_path, capfd):
+    """check_s_l2 (src/util/check.c:7-57): resid = |d| / (|A|_1 |x| |y| 10 eps max(m, k)) against 50."""
+    import ctypes
+    lib = capi.load()
+    path = tmp_path / "m.mtx"
+    path.write_text("%%MatrixMarket matrix coordinate real general\n3 3 4\n1 1 2.0\n2 2 -3.0\n3 1 1.0\n3 3 0.5\n")
+    argv = (ctypes.c_char_p * 2)(b"prog", ("--data-file=%s" % path).encode())
+    x = np.array([1.0, 2.0, 3.0], dtype=np.float32)
+    y = np.array([2.0, -6.0, 2.5], dtype=np.float32)
+    near = y + np.float32(1e-6)
+    far = y + np.float32(1e-2)
+    assert lib.check_s_l2(capi.ptr(near), 3, capi.ptr(y), 3, capi.ptr(x), None, 1.0, 0.0, 2, argv) == 0
+    assert lib.check_s_l2(capi.ptr(far), 3, capi.ptr(y), 3, capi.ptr(x), None, 1.0, 0.0, 2, argv) == -1
+    assert lib.check_s_l2(capi.ptr(y), 3, capi.ptr(y), 2, capi.ptr(x), None, 1.0, 0.0, 2, argv) == -1   # size mismatch
+    ctypes.CDLL(None).fflush(None)
+    out = capfd.readouterr().out
+    assert "correct," in out and "error," in out and "normA : 3.0" in out
