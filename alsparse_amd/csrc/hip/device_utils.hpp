@@ -181,6 +181,71 @@ __device__ __forceinline__ Cx<R> dpp_mov(Cx<R> v) {
   return Cx<R>(dpp_mov<Ctrl>(v.re), dpp_mov<Ctrl>(v.im));
 }
 
+// The same move restricted to the 16-lane rows named in RowMask (bit r = row r); lanes of the
+// other rows, and lanes whose source does not exist, receive zero.
+template <int Ctrl, int RowMask>
+__device__ __forceinline__ int dpp_mov_rows(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, Ctrl, RowMask, 0xF, true);
+}
+template <int Ctrl, int RowMask>
+__device__ __forceinline__ float dpp_mov_rows(float v) {
+  return __builtin_bit_cast(float, dpp_mov_rows<Ctrl, RowMask>(__builtin_bit_cast(int, v)));
+}
+template <int Ctrl, int RowMask>
+__device__ __forceinline__ double dpp_mov_rows(double v) {
+  const uint64_t bits = __builtin_bit_cast(uint64_t, v);
+  const int lo = dpp_mov_rows<Ctrl, RowMask>((int)(uint32_t)bits);
+  const int hi = dpp_mov_rows<Ctrl, RowMask>((int)(uint32_t)(bits >> 32));
+  return __builtin_bit_cast(double, ((uint64_t)(uint32_t)hi << 32) | (uint64_t)(uint32_t)lo);
+}
+template <int Ctrl, int RowMask, typename R>
+__device__ __forceinline__ Cx<R> dpp_mov_rows(Cx<R> v) {
+  return Cx<R>(dpp_mov_rows<Ctrl, RowMask>(v.re), dpp_mov_rows<Ctrl, RowMask>(v.im));
+}
+
+// value of the given lane, the same in every lane (v_readlane: no LDS crossbar)
+__device__ __forceinline__ int lane_bcast(int v, int src) { return __builtin_amdgcn_readlane(v, src); }
+__device__ __forceinline__ float lane_bcast(float v, int src) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), src));
+}
+__device__ __forceinline__ double lane_bcast(double v, int src) {
+  const uint64_t b = __builtin_bit_cast(uint64_t, v);
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)b, src);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(b >> 32), src);
+  return __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);
+}
+template <typename R>
+__device__ __forceinline__ Cx<R> lane_bcast(Cx<R> v, int src) {
+  return Cx<R>(lane_bcast(v.re, src), lane_bcast(v.im, src));
+}
+
+// Inclusive segmented sum over the 64 lanes of a wave: on return v holds the sum of the lane's
+// segment up to and including the lane; `head` marks the first lane of every segment (lane 0 is
+// one).  Pure DPP: shifts by 1, 2, 4, 8 inside the 16-lane rows, then lane 15 of rows 0 / 2
+// broadcast into rows 1 / 3 and lane 31 into rows 2 and 3 -- the steps of a wave prefix sum, each
+// taken only by lanes that have not yet seen the head of their segment.
+template <typename T>
+__device__ __forceinline__ T segmented_scan(T v, bool head) {
+  int f = head;
+#define ASAMD_SCAN_STEP(CTRL, ROWS)                      \
+  {                                                      \
+    const T vd = dpp_mov_rows<CTRL, ROWS>(v);            \
+    const int fd = dpp_mov_rows<CTRL, ROWS>(f);          \
+    if (!f) {                                            \
+      v += vd;                                           \
+      f = fd;                                            \
+    }                                                    \
+  }
+  ASAMD_SCAN_STEP(0x111, 0xF)  // row_shr:1
+  ASAMD_SCAN_STEP(0x112, 0xF)  // row_shr:2
+  ASAMD_SCAN_STEP(0x114, 0xF)  // row_shr:4
+  ASAMD_SCAN_STEP(0x118, 0xF)  // row_shr:8
+  ASAMD_SCAN_STEP(0x142, 0xA)  // row_bcast:15 into rows 1 and 3
+  ASAMD_SCAN_STEP(0x143, 0xC)  // row_bcast:31 into rows 2 and 3
+#undef ASAMD_SCAN_STEP
+  return v;
+}
+
 template <int W, typename T>
 __device__ __forceinline__ T group_sum(T v) {
   static_assert(W >= 1 && W <= 64 && (W & (W - 1)) == 0, "group width");

@@ -8,7 +8,7 @@
 //
 //   COO (entries grouped by row, as csr2coo leaves them): every wave owns one
 //   contiguous run of entries and reduces it 64 at a time with a segmented
-//   scan across its lanes; the last lane of every row segment adds the
+//   scan across its lanes (DPP only); the last lane of every row segment adds the
 //   segment's sum to y, the open segment at the end of a step is carried into
 //   the next one in registers.  Replaces
 //   src/kernel/dcu/level2/mv/dcu_gemv_x_coo.cpp:10-195, which stages the same
@@ -69,24 +69,15 @@ __global__ __launch_bounds__(kCooThreads) void coomv_kernel(int64_t nnz, int m, 
       if (carry_row == r) v += carry_val;
       else if (carry_row >= 0) atomic_add(&y[carry_row], alpha * carry_val);
     }
-    const int r_prev = __shfl_up(r, 1, kWave);
+    // rows of the neighbouring lanes through DPP wave shifts (lane 0 sees -2, lane 63 sees -2: never a row)
+    const int r_prev = __builtin_amdgcn_update_dpp(-2, r, 0x138, 0xF, 0xF, false);  // wave_shr:1
+    const int r_next = __builtin_amdgcn_update_dpp(-2, r, 0x130, 0xF, 0xF, false);  // wave_shl:1
     const bool head = lane == 0 || r_prev != r;
-    // inclusive segmented scan: after the step of distance d, v holds the sum of
-    // the lane's segment over the last 2d lanes, f says whether a head lies among them
-    int f = head;
-#pragma unroll
-    for (int d = 1; d < kWave; d <<= 1) {
-      const T vd = lane_up(v, d);
-      const int fd = __shfl_up(f, d, kWave);
-      if (lane >= d && !f) {
-        v += vd;
-        f = fd;
-      }
-    }
-    const int head_next = __shfl_down((int)head, 1, kWave);
-    if (lane < kWave - 1 && head_next && r >= 0) atomic_add(&y[r], alpha * v);
-    carry_row = __shfl(r, kWave - 1, kWave);
-    carry_val = lane_get(v, kWave - 1);
+    v = segmented_scan(v, head);
+    // the last lane of every row segment adds the segment's sum; lane 63's segment stays open
+    if (lane < kWave - 1 && r_next != r && r >= 0) atomic_add(&y[r], alpha * v);
+    carry_row = lane_bcast(r, kWave - 1);
+    carry_val = lane_bcast(v, kWave - 1);
   }
   if (lane == 0 && carry_row >= 0) atomic_add(&y[carry_row], alpha * carry_val);
 }
