@@ -282,3 +282,51 @@ def test_random_structures_every_family(gpu, seed):
         check_spmv(a, 1.0, x, 1.0, y0, run_csrmv(gpu, da, 1.0, x, 1.0, y0), "seed %d api" % seed)
     finally:
         da.free()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
+def test_unsorted_and_duplicate_columns_and_non_finite_values(gpu, dtype):
+    """CSR does not promise sorted or distinct columns inside a row (alphasparse_convert_csr keeps
+    duplicates): every family must sum such rows like the plain kernel does.  Infinities and NaNs
+    travel to exactly the rows whose entries hold or meet them."""
+    rng = np.random.default_rng(77)
+    m, n = 3000, 2000
+    lens = np.minimum(rng.geometric(0.1, m), 60)
+    lens[5] = 5000
+    rp = np.zeros(m + 1, dtype=np.int32)
+    np.cumsum(lens, out=rp[1:])
+    col = rng.integers(0, n, int(rp[-1])).astype(np.int32)          # unsorted, with repeats
+    val = rng.uniform(-1, 1, col.size).astype(dtype)
+    a = wl.Csr(m, n, rp, col, val, 0, "unsorted-duplicates")
+    x, y0 = _vectors(a, 5)
+    da = DeviceCsr(a)
+    try:
+        for algo in ("vector", "merge", "scalar", "stream", "tiled", "ell", "auto"):
+            announce("spmv unsorted", np.dtype(dtype).name, algo)
+            y = run_plan_csrmv(da, algo, 1.5, x, 0.5, y0)
+            if y is not None:
+                check_spmv(a, 1.5, x, 0.5, y0, y, "unsorted %s" % algo)
+    finally:
+        da.free()
+    # non-finite values: row 7 holds +inf, row 9 meets a NaN in x, row 11 has inf - inf
+    val2 = val.copy()
+    x2 = x.copy()
+    val2[rp[7]] = np.inf
+    x2[col[rp[7]]] = 1.0
+    x2[col[rp[9]]] = np.nan
+    val2[rp[11]], val2[rp[11] + 1] = np.inf, -np.inf
+    x2[col[rp[11]]], x2[col[rp[11] + 1]] = 1.0, 1.0
+    b = wl.Csr(m, n, rp, col, val2, 0, "non-finite")
+    with np.errstate(invalid="ignore", over="ignore"):
+        ref = orc.csrmv_plain(b, 1.0, x2, 0.0, y0)
+    db = DeviceCsr(b)
+    try:
+        for algo in ("vector", "merge", "scalar", "tiled", "auto"):
+            announce("spmv non-finite", np.dtype(dtype).name, algo)
+            y = run_plan_csrmv(db, algo, 1.0, x2, 0.0, y0)
+            assert np.array_equal(np.isnan(y), np.isnan(ref)), algo
+            assert np.array_equal(np.isinf(y), np.isinf(ref)) and np.array_equal(np.sign(y[np.isinf(y)]), np.sign(ref[np.isinf(ref)])), algo
+            finite = np.isfinite(ref)
+            assert np.isnan(ref[9]) and np.isnan(ref[11]) and np.isinf(ref[7]) and finite.sum() >= m - 300
+    finally:
+        db.free()
