@@ -44,6 +44,31 @@ struct alignas(sizeof(T) * V) Vec {
   T e[V];
 };
 
+// Four consecutive elements that are only known to be aligned like a single one: the compiler may
+// still fetch them with one wide load (global memory takes unaligned wide accesses).
+template <typename T>
+struct __attribute__((packed, aligned(alignof(T)))) Quad4 {
+  T e[4];
+};
+
+// The first `valid` (<= V) elements at p, zeros behind them: whole groups of four through one load each.
+template <typename T, int V>
+__device__ __forceinline__ Vec<T, V> load_short_row(const T* p, int valid) {
+  Vec<T, V> r;
+#pragma unroll
+  for (int i = 0; i < V; i += 4) {
+    if (V - i >= 4 && i + 4 <= valid) {
+      const Quad4<T> q = *reinterpret_cast<const Quad4<T>*>(p + i);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) r.e[i + u] = q.e[u];
+    } else {
+#pragma unroll
+      for (int u = 0; u < 4 && i + u < V; ++u) r.e[i + u] = i + u < valid ? p[i + u] : T(0);
+    }
+  }
+  return r;
+}
+
 template <typename T, int V>
 __device__ __forceinline__ Vec<T, V> load_vec(const T* p, bool vector_ok, int valid) {
   Vec<T, V> r;
@@ -151,8 +176,8 @@ __global__ __launch_bounds__(kSpmmBlock) void spmm_rowmajor_kernel(
   }
 }
 
-// Narrow dense operands (n <= 16): G = 2..16 lanes per row of A, 64 / G rows per wave, lane
-// c of a group owns dense column c.  The group walks its row four entries at a time; the
+// Narrow dense operands, lane-per-column form (used for 9..16 columns that are not a multiple of
+// four): G = 16 lanes per row of A, 64 / G rows per wave, lane c of a group owns dense column c.  The group walks its row four entries at a time; the
 // entry loads are the same address for all lanes of a group (one request), each B row is
 // one load of G contiguous elements.  A wave per row would leave 64 - n lanes idle.
 template <typename T, int G>
@@ -201,6 +226,82 @@ static void launch_narrow(hipStream_t s, int m, int n, T alpha, const T* val, co
   constexpr int rows_per_block = kSpmmBlock / G;
   const unsigned grid = (unsigned)(((int64_t)m + rows_per_block - 1) / rows_per_block);
   spmm_rowmajor_narrow_kernel<T, G><<<grid, kSpmmBlock, 0, s>>>(m, n, alpha, val, rp, ci, base, B, ldb, beta, C, ldc);
+}
+
+// Narrow dense operands (n <= NV <= 16): W lanes share a row of A and read its entries coalesced, as
+// in the lane-group SpMV kernel; every lane multiplies its entries with the whole (short) row of B
+// -- one vector load of NV elements when B allows it -- and keeps NV partial sums; the group's sums
+// meet through DPP and lane 0 writes the row of C.  Measured on a 2^20 x 2^20 matrix with 32 entries
+// per row against the lane-per-column kernel above (n: ms -> ms): 1: 0.50 -> 0.21, 2: 0.68 -> 0.37,
+// 4: 0.78 -> 0.48, 6: 0.82 -> 0.64, 8: 0.77 -> 0.55, 12: 0.73 -> 0.72, 16: 0.61 -> 0.60; 13: 0.75 -> 0.89,
+// which is why widths above 8 that are not multiples of four stay with the kernel above.
+template <typename T, int NV>
+__device__ __forceinline__ Vec<T, NV> short_row(const T* p, bool vector_ok, int n) {
+  if (vector_ok) return *reinterpret_cast<const Vec<T, NV>*>(p);  // n == NV and the row is aligned to its size
+  return load_short_row<T, NV>(p, n);
+}
+
+template <typename T, int NV, int W>
+__global__ __launch_bounds__(kSpmmBlock) void spmm_rowmajor_short_kernel(
+    int m, int n, T alpha, const T* __restrict__ val, const int* __restrict__ row_ptr,
+    const int* __restrict__ col_ind, int base, const T* __restrict__ B, int64_t ldb, T beta,
+    T* __restrict__ C, int64_t ldc, bool vector_ok) {
+  constexpr int kRowsPerBlock = kSpmmBlock / W;
+  const unsigned bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  const int lane = threadIdx.x % W;
+  const int64_t row = (int64_t)bid * kRowsPerBlock + threadIdx.x / W;
+  if (row >= m) return;  // whole lane groups leave together
+  const int64_t start = (int64_t)row_ptr[row] - base;
+  const int64_t end = (int64_t)row_ptr[row + 1] - base;
+  T acc[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) acc[i] = T(0);
+  int64_t j = start + lane;
+  // two entries per lane and trip keep two B rows in flight
+  for (; j + W < end; j += 2 * W) {
+    const T a0 = alpha * val[j], a1 = alpha * val[j + W];
+    const int c0 = col_ind[j] - base, c1 = col_ind[j + W] - base;
+    const Vec<T, NV> b0 = short_row<T, NV>(B + (int64_t)c0 * ldb, vector_ok, n);
+    const Vec<T, NV> b1 = short_row<T, NV>(B + (int64_t)c1 * ldb, vector_ok, n);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) acc[i] = fma_t(a0, b0.e[i], acc[i]);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) acc[i] = fma_t(a1, b1.e[i], acc[i]);
+  }
+  if (j < end) {
+    const T a0 = alpha * val[j];
+    const Vec<T, NV> b0 = short_row<T, NV>(B + (int64_t)(col_ind[j] - base) * ldb, vector_ok, n);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) acc[i] = fma_t(a0, b0.e[i], acc[i]);
+  }
+#pragma unroll
+  for (int i = 0; i < NV; ++i) acc[i] = group_sum<W>(acc[i]);
+  if (lane == 0) {
+    T* crow = C + row * ldc;
+#pragma unroll
+    for (int i = 0; i < NV; ++i)
+      if (i < n) crow[i] = beta == T(0) ? acc[i] : crow[i] * beta + acc[i];
+  }
+}
+
+template <typename T, int NV, int W>
+static void launch_short(hipStream_t s, int m, int n, T alpha, const T* val, const int* rp, const int* ci, int base,
+                         const T* B, int64_t ldb, T beta, T* C, int64_t ldc) {
+  constexpr int rows_per_block = kSpmmBlock / W;
+  const unsigned grid = (unsigned)(((int64_t)m + rows_per_block - 1) / rows_per_block);
+  const bool vector_ok = n == NV && ldb % NV == 0 && (uintptr_t)B % (NV * sizeof(T)) == 0;
+  spmm_rowmajor_short_kernel<T, NV, W><<<grid, kSpmmBlock, 0, s>>>(m, n, alpha, val, rp, ci, base, B, ldb, beta, C,
+                                                                     ldc, vector_ok);
+}
+
+// lanes per row from the mean row length
+template <typename T, int NV>
+static void launch_short_w(hipStream_t s, int m, int n, int64_t nnz, T alpha, const T* val, const int* rp,
+                           const int* ci, int base, const T* B, int64_t ldb, T beta, T* C, int64_t ldc) {
+  const double mean = (double)nnz / (double)m;
+  if (mean < 8) launch_short<T, NV, 4>(s, m, n, alpha, val, rp, ci, base, B, ldb, beta, C, ldc);
+  else if (mean < 48) launch_short<T, NV, 16>(s, m, n, alpha, val, rp, ci, base, B, ldb, beta, C, ldc);
+  else launch_short<T, NV, 64>(s, m, n, alpha, val, rp, ci, base, B, ldb, beta, C, ldc);
 }
 
 // out[r * out_ld + c] = in[r + c * in_ld] for r < rows, c < cols: 64 x 64 tiles, reads
@@ -330,7 +431,6 @@ template <typename T>
 static int csrmm_impl(hipStream_t s, int m, int n, int k, int nnz, T alpha, const T* val,
                       const int* rp, const int* ci, int base, const T* B, T beta, T* C,
                       const asamd_dense_strides* st, void* ws, size_t ws_bytes) {
-  (void)nnz;
   if (!val || !rp || !ci || !B || !C || !st || m <= 0 || n <= 0) return hipErrorInvalidValue;
   if (((uintptr_t)val | (uintptr_t)B | (uintptr_t)C) % alignof(T)) return hipErrorInvalidValue;
   if (n > 1 && st->c_row_stride == 1 && st->c_col_stride != 1) {
@@ -357,11 +457,13 @@ static int csrmm_impl(hipStream_t s, int m, int n, int k, int nnz, T alpha, cons
   const bool unit_cols = (st->b_col_stride == 1 && st->c_col_stride == 1) || n == 1;
   if (unit_cols) {
     const int64_t ldb = st->b_row_stride, ldc = st->c_row_stride;
-    if (n <= 16) {  // measured on a 2^20 x 2^20 matrix, 32 entries per row: 0.51-0.78 ms against 0.93 ms; no gain at n = 32
-      if (n <= 2) launch_narrow<T, 2>(s, m, n, alpha, val, rp, ci, base, B, ldb, beta, C, ldc);
-      else if (n <= 4) launch_narrow<T, 4>(s, m, n, alpha, val, rp, ci, base, B, ldb, beta, C, ldc);
-      else if (n <= 8) launch_narrow<T, 8>(s, m, n, alpha, val, rp, ci, base, B, ldb, beta, C, ldc);
-      else launch_narrow<T, 16>(s, m, n, alpha, val, rp, ci, base, B, ldb, beta, C, ldc);
+    if (n <= 16) {  // a wave per row would leave 64 - n lanes idle (0.93 ms whatever n is on the matrix below)
+      // 9..16 columns that are not whole groups of four: the lane-per-column kernel loads less padding
+      if (n > 8 && n % 4 != 0) launch_narrow<T, 16>(s, m, n, alpha, val, rp, ci, base, B, ldb, beta, C, ldc);
+      else if (n <= 2) launch_short_w<T, 2>(s, m, n, nnz, alpha, val, rp, ci, base, B, ldb, beta, C, ldc);
+      else if (n <= 4) launch_short_w<T, 4>(s, m, n, nnz, alpha, val, rp, ci, base, B, ldb, beta, C, ldc);
+      else if (n <= 8) launch_short_w<T, 8>(s, m, n, nnz, alpha, val, rp, ci, base, B, ldb, beta, C, ldc);
+      else launch_short_w<T, 16>(s, m, n, nnz, alpha, val, rp, ci, base, B, ldb, beta, C, ldc);
       return hipGetLastError();
     }
     const unsigned gx = (unsigned)(((int64_t)m + kSpmmWaves - 1) / kSpmmWaves);
@@ -370,6 +472,10 @@ static int csrmm_impl(hipStream_t s, int m, int n, int k, int nnz, T alpha, cons
     int V = 1;
     if (n >= 4 * kWave && kMaxV >= 4) V = 4;
     else if (n >= 2 * kWave && kMaxV >= 2) V = 2;
+    // A B too large for the 256 MiB memory-side cache is better taken 64 dense columns at a time
+    // (grid.y runs slowest, so one slice of B is live at a time and stays cached): measured on a
+    // 2^20 x 2^20 matrix with 32 entries per row, n = 128: 3.10 ms with V = 2, against 2 x 1.23 ms.
+    if (k > 0 && (size_t)k * (size_t)n * sizeof(T) > ((size_t)192 << 20)) V = 1;
     const size_t vbytes = (size_t)V * sizeof(T);
     const bool vector_ok = V > 1 && ((uintptr_t)B % vbytes == 0) && ((uintptr_t)C % vbytes == 0) &&
                            (ldb % V == 0) && (ldc % V == 0);
