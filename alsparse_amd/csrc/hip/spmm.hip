@@ -245,7 +245,7 @@ template <typename T, int NV, int W>
 __global__ __launch_bounds__(kSpmmBlock) void spmm_rowmajor_short_kernel(
     int m, int n, T alpha, const T* __restrict__ val, const int* __restrict__ row_ptr,
     const int* __restrict__ col_ind, int base, const T* __restrict__ B, int64_t ldb, T beta,
-    T* __restrict__ C, int64_t ldc, bool vector_ok) {
+    T* __restrict__ C, int64_t c_row_stride, int64_t c_col_stride, bool vector_ok) {
   constexpr int kRowsPerBlock = kSpmmBlock / W;
   const unsigned bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
   const int lane = threadIdx.x % W;
@@ -277,31 +277,45 @@ __global__ __launch_bounds__(kSpmmBlock) void spmm_rowmajor_short_kernel(
 #pragma unroll
   for (int i = 0; i < NV; ++i) acc[i] = group_sum<W>(acc[i]);
   if (lane == 0) {
-    T* crow = C + row * ldc;
+    // row-major C: n consecutive elements; column-major C: the lanes 0 of a wave's groups hold
+    // consecutive rows, so every dense column is written as one contiguous run
+    T* crow = C + row * c_row_stride;
 #pragma unroll
     for (int i = 0; i < NV; ++i)
-      if (i < n) crow[i] = beta == T(0) ? acc[i] : crow[i] * beta + acc[i];
+      if (i < n) crow[i * c_col_stride] = beta == T(0) ? acc[i] : crow[i * c_col_stride] * beta + acc[i];
   }
 }
 
 template <typename T, int NV, int W>
 static void launch_short(hipStream_t s, int m, int n, T alpha, const T* val, const int* rp, const int* ci, int base,
-                         const T* B, int64_t ldb, T beta, T* C, int64_t ldc) {
+                         const T* B, int64_t ldb, T beta, T* C, int64_t scr, int64_t scc) {
   constexpr int rows_per_block = kSpmmBlock / W;
   const unsigned grid = (unsigned)(((int64_t)m + rows_per_block - 1) / rows_per_block);
   const bool vector_ok = n == NV && ldb % NV == 0 && (uintptr_t)B % (NV * sizeof(T)) == 0;
   spmm_rowmajor_short_kernel<T, NV, W><<<grid, kSpmmBlock, 0, s>>>(m, n, alpha, val, rp, ci, base, B, ldb, beta, C,
-                                                                     ldc, vector_ok);
+                                                                     scr, scc, vector_ok);
 }
 
 // lanes per row from the mean row length
 template <typename T, int NV>
 static void launch_short_w(hipStream_t s, int m, int n, int64_t nnz, T alpha, const T* val, const int* rp,
-                           const int* ci, int base, const T* B, int64_t ldb, T beta, T* C, int64_t ldc) {
+                           const int* ci, int base, const T* B, int64_t ldb, T beta, T* C, int64_t scr,
+                           int64_t scc) {
   const double mean = (double)nnz / (double)m;
-  if (mean < 8) launch_short<T, NV, 4>(s, m, n, alpha, val, rp, ci, base, B, ldb, beta, C, ldc);
-  else if (mean < 48) launch_short<T, NV, 16>(s, m, n, alpha, val, rp, ci, base, B, ldb, beta, C, ldc);
-  else launch_short<T, NV, 64>(s, m, n, alpha, val, rp, ci, base, B, ldb, beta, C, ldc);
+  if (mean < 8) launch_short<T, NV, 4>(s, m, n, alpha, val, rp, ci, base, B, ldb, beta, C, scr, scc);
+  else if (mean < 48) launch_short<T, NV, 16>(s, m, n, alpha, val, rp, ci, base, B, ldb, beta, C, scr, scc);
+  else launch_short<T, NV, 64>(s, m, n, alpha, val, rp, ci, base, B, ldb, beta, C, scr, scc);
+}
+
+// B rows of n <= 16 contiguous elements, C with any two strides
+template <typename T>
+static void launch_short_n(hipStream_t s, int m, int n, int64_t nnz, T alpha, const T* val, const int* rp,
+                           const int* ci, int base, const T* B, int64_t ldb, T beta, T* C, int64_t scr,
+                           int64_t scc) {
+  if (n <= 2) launch_short_w<T, 2>(s, m, n, nnz, alpha, val, rp, ci, base, B, ldb, beta, C, scr, scc);
+  else if (n <= 4) launch_short_w<T, 4>(s, m, n, nnz, alpha, val, rp, ci, base, B, ldb, beta, C, scr, scc);
+  else if (n <= 8) launch_short_w<T, 8>(s, m, n, nnz, alpha, val, rp, ci, base, B, ldb, beta, C, scr, scc);
+  else launch_short_w<T, 16>(s, m, n, nnz, alpha, val, rp, ci, base, B, ldb, beta, C, scr, scc);
 }
 
 // out[r * out_ld + c] = in[r + c * in_ld] for r < rows, c < cols: 64 x 64 tiles, reads
@@ -446,6 +460,11 @@ static int csrmm_impl(hipStream_t s, int m, int n, int k, int nnz, T alpha, cons
       Bt = (const T*)ws;
       ldbt = n;
     }
+    if (Bt && n <= 16 && (n <= 8 || n % 4 == 0)) {
+      // few dense columns: the entry-parallel kernel on the row-major B, C written through its strides
+      launch_short_n<T>(s, m, n, nnz, alpha, val, rp, ci, base, Bt, ldbt, beta, C, 1, st->c_col_stride);
+      return hipGetLastError();
+    }
     if (Bt) {
       const dim3 grid((unsigned)(((int64_t)m + kWave - 1) / kWave), (unsigned)((n + kWave - 1) / kWave));
       spmm_colmajor_kernel<T><<<grid, kSpmmBlock, 0, s>>>(m, n, alpha, val, rp, ci, base, Bt, ldbt, beta, C,
@@ -460,10 +479,7 @@ static int csrmm_impl(hipStream_t s, int m, int n, int k, int nnz, T alpha, cons
     if (n <= 16) {  // a wave per row would leave 64 - n lanes idle (0.93 ms whatever n is on the matrix below)
       // 9..16 columns that are not whole groups of four: the lane-per-column kernel loads less padding
       if (n > 8 && n % 4 != 0) launch_narrow<T, 16>(s, m, n, alpha, val, rp, ci, base, B, ldb, beta, C, ldc);
-      else if (n <= 2) launch_short_w<T, 2>(s, m, n, nnz, alpha, val, rp, ci, base, B, ldb, beta, C, ldc);
-      else if (n <= 4) launch_short_w<T, 4>(s, m, n, nnz, alpha, val, rp, ci, base, B, ldb, beta, C, ldc);
-      else if (n <= 8) launch_short_w<T, 8>(s, m, n, nnz, alpha, val, rp, ci, base, B, ldb, beta, C, ldc);
-      else launch_short_w<T, 16>(s, m, n, nnz, alpha, val, rp, ci, base, B, ldb, beta, C, ldc);
+      else launch_short_n<T>(s, m, n, nnz, alpha, val, rp, ci, base, B, ldb, beta, C, ldc, 1);
       return hipGetLastError();
     }
     const unsigned gx = (unsigned)(((int64_t)m + kSpmmWaves - 1) / kSpmmWaves);
