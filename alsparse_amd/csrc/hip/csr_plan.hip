@@ -151,6 +151,9 @@ static int width_for_mean(double mean) {
   return 64;
 }
 
+// rows plus entries below which one launch's latency outweighs the work
+constexpr int64_t kSmallWork = 1 << 17;
+
 static bool rowconst_ok(const asamd_csr_plan* p) {
   const asamd_csr_stats& st = p->st;
   const int L = st.const_len;
@@ -178,6 +181,10 @@ static void choose_algo(asamd_csr_plan* p) {
     p->auto_algo = ASAMD_SPMV_STREAM;
   } else if ((int64_t)st.max_len <= (int64_t)w * 16 && mean >= 6.0) {
     // regular rows: a lane group per row wastes little and needs no LDS
+    p->auto_algo = ASAMD_SPMV_VECTOR;
+  } else if ((int64_t)st.m + st.nnz <= kSmallWork && (int64_t)st.max_len <= (int64_t)w * 64) {
+    // a matrix this small is over in the time of one launch: the single
+    // kernel beats the balanced path's two or three
     p->auto_algo = ASAMD_SPMV_VECTOR;
   } else {
     p->auto_algo = ASAMD_SPMV_MERGE;
