@@ -9,6 +9,9 @@
 //       This is the layout the reference cannot run on the GPU at all
 //       (dcu_gemm_?_csr_row returns NOT_SUPPORTED,
 //       src/kernel/dcu/level3/mm/csrmm/dcu_gemm_x_csr_row.cpp:15-36).
+//   spmm_rowmajor_group_kernel<T, G, V> / spmm_rowmajor_short_kernel<T, NV, W>
+//       the same layout with at most 32 / at most 16 dense columns: several
+//       rows of A per wave (described at the kernels).
 //   dense_transpose_kernel<T> + spmm_colmajor_kernel<T>   column-major B and C
 //       (the layout the reference's GPU path does run): B is first transposed
 //       into a row-major workspace, 64 x 64 tiles through LDS, both sides
@@ -44,12 +47,14 @@ struct alignas(sizeof(T) * V) Vec {
   T e[V];
 };
 
-// Four consecutive elements that are only known to be aligned like a single one: the compiler may
+// N consecutive elements that are only known to be aligned like a single one: the compiler may
 // still fetch them with one wide load (global memory takes unaligned wide accesses).
-template <typename T>
-struct __attribute__((packed, aligned(alignof(T)))) Quad4 {
-  T e[4];
+template <typename T, int N>
+struct __attribute__((packed, aligned(alignof(T)))) Packed {
+  T e[N];
 };
+template <typename T>
+using Quad4 = Packed<T, 4>;
 
 // The first `valid` (<= V) elements at p, zeros behind them: whole groups of four through one load each.
 template <typename T, int V>
@@ -74,6 +79,10 @@ __device__ __forceinline__ Vec<T, V> load_vec(const T* p, bool vector_ok, int va
   Vec<T, V> r;
   if (vector_ok && valid == V) {
     r = *reinterpret_cast<const Vec<T, V>*>(p);
+  } else if (valid == V) {
+    const Packed<T, V> q = *reinterpret_cast<const Packed<T, V>*>(p);
+#pragma unroll
+    for (int i = 0; i < V; ++i) r.e[i] = q.e[i];
   } else {
 #pragma unroll
     for (int i = 0; i < V; ++i) r.e[i] = i < valid ? p[i] : T(0);
@@ -176,63 +185,110 @@ __global__ __launch_bounds__(kSpmmBlock) void spmm_rowmajor_kernel(
   }
 }
 
-// Narrow dense operands, lane-per-column form (used for 9..16 columns that are not a multiple of
-// four): G = 16 lanes per row of A, 64 / G rows per wave, lane c of a group owns dense column c.  The group walks its row four entries at a time; the
-// entry loads are the same address for all lanes of a group (one request), each B row is
-// one load of G contiguous elements.  A wave per row would leave 64 - n lanes idle.
-template <typename T, int G>
-__global__ __launch_bounds__(kSpmmBlock) void spmm_rowmajor_narrow_kernel(
+// Dense operands narrower than a wave, lane-group form: G lanes per row of A, 64 / G rows per wave,
+// lane c of a group owns V consecutive dense columns.  The group walks its row four entries at a
+// time; the entry loads are the same address for all lanes of a group (one request), each B row is
+// one load of G*V contiguous elements, so one wave instruction fetches 64 / G rows of B.  A wave per
+// row would leave 64 - n lanes idle and issue 64 / G times as many loads.
+template <typename T, int G, int V>
+__global__ __launch_bounds__(kSpmmBlock) void spmm_rowmajor_group_kernel(
     int m, int n, T alpha, const T* __restrict__ val, const int* __restrict__ row_ptr,
     const int* __restrict__ col_ind, int base, const T* __restrict__ B, int64_t ldb, T beta,
-    T* __restrict__ C, int64_t ldc) {
+    T* __restrict__ C, int64_t ldc, bool vector_ok) {
   constexpr int kRowsPerBlock = kSpmmBlock / G;
   const unsigned bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
   const int64_t row = (int64_t)bid * kRowsPerBlock + threadIdx.x / G;
-  const int c = threadIdx.x % G;
   if (row >= m) return;
-  const bool col_ok = c < n;
+  const int c0 = (blockIdx.y * G + threadIdx.x % G) * V;  // first dense column of this lane
+  int valid = n - c0;
+  valid = valid > V ? V : (valid < 0 ? 0 : valid);
   const int64_t start = (int64_t)row_ptr[row] - base;
   const int64_t end = (int64_t)row_ptr[row + 1] - base;
-  const T* bcol = B + c;
-  T acc = T(0);
-  int64_t j = start;
-  constexpr int kU = 4;
-  for (; j + kU <= end; j += kU) {
-    int col[kU];
-    T a[kU], b[kU];
+  const T* bcol = B + c0;
+  T acc[V];
 #pragma unroll
-    for (int u = 0; u < kU; ++u) {
-      col[u] = col_ind[j + u] - base;
-      a[u] = alpha * val[j + u];
+  for (int i = 0; i < V; ++i) acc[i] = T(0);
+  if constexpr (V == 1) {
+    // four entries at a time, every lane of the group loading the same entry (one request per group):
+    // measured faster than handing entries round when a lane has a single column (13 columns: 0.75 ms
+    // against 0.81 ms on a 2^20 x 2^20 matrix with 32 entries per row)
+    int64_t j = start;
+    constexpr int kU = 4;
+    for (; j + kU <= end; j += kU) {
+      int col[kU];
+      T a[kU], b[kU];
+#pragma unroll
+      for (int u = 0; u < kU; ++u) {
+        col[u] = col_ind[j + u] - base;
+        a[u] = alpha * val[j + u];
+      }
+#pragma unroll
+      for (int u = 0; u < kU; ++u) b[u] = valid ? bcol[(int64_t)col[u] * ldb] : T(0);
+#pragma unroll
+      for (int u = 0; u < kU; ++u) acc[0] = fma_t(a[u], b[u], acc[0]);
     }
+    for (; j < end; ++j)
+      acc[0] = fma_t(alpha * val[j], valid ? bcol[(int64_t)(col_ind[j] - base) * ldb] : T(0), acc[0]);
+  } else {
+    const int gl = threadIdx.x % G;                  // lane inside the group
+    const int g0 = (threadIdx.x % kWave) - gl;       // the group's first lane in the wave
+    for (int64_t j0 = start; j0 < end; j0 += G) {
+      // the group reads G entries of its row with one coalesced load, then hands them round
+      const int64_t j = j0 + gl;
+      int my_col = 0;
+      T my_val = T(0);
+      if (j < end) {
+        my_col = nt_load(col_ind + j) - base;
+        my_val = alpha * nt_load(val + j);
+      }
+      const int cnt = (int)(end - j0 < G ? end - j0 : G);
+      int t = 0;
+      constexpr int kU = 4;
+      for (; t + kU <= cnt; t += kU) {
+        T a[kU];
+        Vec<T, V> b[kU];
 #pragma unroll
-    for (int u = 0; u < kU; ++u) b[u] = col_ok ? bcol[(int64_t)col[u] * ldb] : T(0);
+        for (int u = 0; u < kU; ++u) {
+          const int col = lane_get(my_col, g0 + t + u);
+          a[u] = lane_get(my_val, g0 + t + u);
+          b[u] = load_vec<T, V>(bcol + (int64_t)col * ldb, vector_ok, valid);
+        }
 #pragma unroll
-    for (int u = 0; u < kU; ++u) acc = fma_t(a[u], b[u], acc);
+        for (int u = 0; u < kU; ++u) {
+#pragma unroll
+          for (int i = 0; i < V; ++i) acc[i] = fma_t(a[u], b[u].e[i], acc[i]);
+        }
+      }
+      for (; t < cnt; ++t) {
+        const int col = lane_get(my_col, g0 + t);
+        const T a = lane_get(my_val, g0 + t);
+        const Vec<T, V> b = load_vec<T, V>(bcol + (int64_t)col * ldb, vector_ok, valid);
+#pragma unroll
+        for (int i = 0; i < V; ++i) acc[i] = fma_t(a, b.e[i], acc[i]);
+      }
+    }
   }
-  for (; j < end; ++j) {
-    const int col = col_ind[j] - base;
-    acc = fma_t(alpha * val[j], col_ok ? bcol[(int64_t)col * ldb] : T(0), acc);
-  }
-  if (col_ok) {
-    T* out = C + row * ldc + c;
-    *out = beta == T(0) ? acc : *out * beta + acc;
-  }
+  T* out = C + row * ldc + c0;
+#pragma unroll
+  for (int i = 0; i < V; ++i)
+    if (i < valid) out[i] = beta == T(0) ? acc[i] : out[i] * beta + acc[i];
 }
 
-template <typename T, int G>
-static void launch_narrow(hipStream_t s, int m, int n, T alpha, const T* val, const int* rp, const int* ci, int base,
-                          const T* B, int64_t ldb, T beta, T* C, int64_t ldc) {
+template <typename T, int G, int V>
+static void launch_group(hipStream_t s, int m, int n, T alpha, const T* val, const int* rp, const int* ci, int base,
+                         const T* B, int64_t ldb, T beta, T* C, int64_t ldc) {
   constexpr int rows_per_block = kSpmmBlock / G;
-  const unsigned grid = (unsigned)(((int64_t)m + rows_per_block - 1) / rows_per_block);
-  spmm_rowmajor_narrow_kernel<T, G><<<grid, kSpmmBlock, 0, s>>>(m, n, alpha, val, rp, ci, base, B, ldb, beta, C, ldc);
+  const dim3 grid((unsigned)(((int64_t)m + rows_per_block - 1) / rows_per_block), (unsigned)((n + G * V - 1) / (G * V)));
+  const bool vector_ok = V > 1 && (uintptr_t)B % (V * sizeof(T)) == 0 && ldb % V == 0;
+  spmm_rowmajor_group_kernel<T, G, V><<<grid, kSpmmBlock, 0, s>>>(m, n, alpha, val, rp, ci, base, B, ldb, beta, C, ldc,
+                                                                  vector_ok);
 }
 
 // Narrow dense operands (n <= NV <= 16): W lanes share a row of A and read its entries coalesced, as
 // in the lane-group SpMV kernel; every lane multiplies its entries with the whole (short) row of B
 // -- one vector load of NV elements when B allows it -- and keeps NV partial sums; the group's sums
 // meet through DPP and lane 0 writes the row of C.  Measured on a 2^20 x 2^20 matrix with 32 entries
-// per row against the lane-per-column kernel above (n: ms -> ms): 1: 0.50 -> 0.21, 2: 0.68 -> 0.37,
+// per row against the lane-group kernel above with a lane per column (n: ms -> ms): 1: 0.50 -> 0.21, 2: 0.68 -> 0.37,
 // 4: 0.78 -> 0.48, 6: 0.82 -> 0.64, 8: 0.77 -> 0.55, 12: 0.73 -> 0.72, 16: 0.61 -> 0.60; 13: 0.75 -> 0.89,
 // which is why widths above 8 that are not multiples of four stay with the kernel above.
 template <typename T, int NV>
@@ -477,9 +533,17 @@ static int csrmm_impl(hipStream_t s, int m, int n, int k, int nnz, T alpha, cons
   if (unit_cols) {
     const int64_t ldb = st->b_row_stride, ldc = st->c_row_stride;
     if (n <= 16) {  // a wave per row would leave 64 - n lanes idle (0.93 ms whatever n is on the matrix below)
-      // 9..16 columns that are not whole groups of four: the lane-per-column kernel loads less padding
-      if (n > 8 && n % 4 != 0) launch_narrow<T, 16>(s, m, n, alpha, val, rp, ci, base, B, ldb, beta, C, ldc);
+      // 9..16 columns that are not whole groups of four: a lane per column loads less padding
+      if (n > 8 && n % 4 != 0) launch_group<T, 16, 1>(s, m, n, alpha, val, rp, ci, base, B, ldb, beta, C, ldc);
       else launch_short_n<T>(s, m, n, nnz, alpha, val, rp, ci, base, B, ldb, beta, C, ldc, 1);
+      return hipGetLastError();
+    }
+    if (n <= 32 && (uintptr_t)B % (2 * sizeof(T)) == 0 && ldb % 2 == 0) {
+      // 17..32 columns in rows of B that pairs of elements can be loaded from: 16 lanes x 2 columns per row,
+      // four rows of B per wave-wide load (n = 32: 0.95 ms with a wave per row -> 0.68 ms, n = 24: 1.00 -> 0.90).
+      // Odd row strides were slower this way (n = 31: 1.23 ms against 1.13 ms), and wider groups or vectors
+      // were no faster than a wave per row above 32 columns.
+      launch_group<T, 16, 2>(s, m, n, alpha, val, rp, ci, base, B, ldb, beta, C, ldc);
       return hipGetLastError();
     }
     const unsigned gx = (unsigned)(((int64_t)m + kSpmmWaves - 1) / kSpmmWaves);

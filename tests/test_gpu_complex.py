@@ -159,7 +159,7 @@ def test_complex_csrmm(gpu, dtype, layout):
         da = DeviceCsr(a)
         descr = capi.make_descr(base=a.base)
         try:
-            for n in (1, 3, 16, 17, 64, 130, 300):
+            for n in (1, 3, 16, 17, 32, 64, 130, 300):
                 if a.rows * n > 6_000_000:
                     continue
                 B = complex_vector(a.cols * n, dtype, 5).reshape(a.cols, n)

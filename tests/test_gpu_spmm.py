@@ -49,7 +49,7 @@ MATS = {
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
 @pytest.mark.parametrize("mat", sorted(MATS))
-@pytest.mark.parametrize("n", [1, 2, 3, 7, 16, 17, 64, 100, 128, 300])
+@pytest.mark.parametrize("n", [1, 2, 3, 7, 16, 17, 24, 31, 32, 64, 100, 128, 300])
 def test_row_major(gpu, mat, n, dtype):
     for base in (0, 1):
         a = MATS[mat](dtype, base)
