@@ -37,3 +37,8 @@ def build_oracle():
     """Compile the CPU oracle (test infrastructure) and, when the reference tree
     is present, the reference's own CPU kernels into oracle/_ref/."""
     _run(["make", "-C", os.path.join(ROOT, "oracle")])
+
+
+def build_c_api_program():
+    """Compile the C lifecycle program of the test suite against the freshly built library."""
+    _run(["make", "-C", os.path.join(ROOT, "tests", "c_api")])
