@@ -273,6 +273,38 @@ def cpu_spmv(a, x, y0, alpha, beta, nbytes):
                       % (a.rows, a.nnz, iters, iters)}
 
 
+def run_host_pointer_spmv(cfg, steps):
+    """alphasparse_?_mv with HOST x and y (the reference's CPU entry point): every call stages x and y
+    to the device, multiplies there and copies y back, so this rate includes PCIe.  Reported beside
+    the device-resident figure, never as `value`."""
+    from alsparse_amd import capi, workloads as wl
+    lib = capi.load()
+    a, x, y0, alpha, beta, _ = wl.config(cfg)
+    T, p = capi.scalar_type(a.dtype), capi.prefix(a.dtype)
+    A = capi.alphasparse_matrix_t()
+    rs, re = np.ascontiguousarray(a.row_ptr[:-1]), np.ascontiguousarray(a.row_ptr[1:])
+    st = getattr(lib, "alphasparse_%s_create_csr" % p)(byref(A), a.base, a.rows, a.cols, capi.ptr(rs), capi.ptr(re),
+                                                      capi.ptr(a.col_ind), capi.ptr(a.values))
+    assert st == 0, "create_csr status %d" % st
+    descr = capi.alpha_matrix_descr(0, 0, 0)
+    mv = getattr(lib, "alphasparse_%s_mv" % p)
+    y = y0.copy()
+    t0 = time.perf_counter()
+    assert mv(0, T(alpha), A, descr, capi.ptr(x), T(beta), capi.ptr(y)) == 0  # mirrors and analyses on first use
+    first_ms = (time.perf_counter() - t0) * 1e3
+    times = []
+    for _ in range(steps):
+        t0 = time.perf_counter()
+        assert mv(0, T(alpha), A, descr, capi.ptr(x), T(beta), capi.ptr(y)) == 0
+        times.append((time.perf_counter() - t0) * 1e3)
+    lib.alphasparse_destroy(A)
+    nbytes = wl.spmv_bytes(a.rows, a.cols, a.nnz, a.dtype.itemsize, beta)
+    avg = sum(times) / len(times)
+    return {"workload": WORKLOAD_NAMES[cfg] + " -- HOST x and y through alphasparse_%s_mv (PCIe-inclusive)" % p,
+            "first_call_ms": first_ms, "avg_ms": avg, "min_ms": min(times), "gbs": nbytes / avg / 1e6,
+            "staged_bytes_per_call": int(x.nbytes + y.nbytes * (2 if beta != 0 else 1))}
+
+
 def run_format_spmv(cfg, fmt, steps, warmup, check):
     """SpMV on the ELL or COO form of configuration `cfg`, converted on the GPU
     (alphasparse_dcu_csr2coo / _csr2ell) and multiplied by alphasparse_dcu_?_coomv / _ellmv."""
@@ -495,6 +527,8 @@ def main():
                 continue
             r = run_format_spmv(c, fmt, args.steps, args.warmup, check)
             others["C%d_%s" % (c, fmt)] = {k: r[k] for k in ("workload", "gbs", "gflops", "hbm_frac", "timing", "parity", "kernel")}
+
+        others["C3_host_pointers"] = run_host_pointer_spmv(3, min(args.steps, 10))
 
     t = main_res["timing"]
     out = {
