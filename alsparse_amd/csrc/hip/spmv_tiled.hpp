@@ -50,7 +50,6 @@ namespace asamd {
 
 constexpr int kTileBytes = 128 * 1024;  // LDS bytes of an x slice (phase 1) / of a workgroup's accumulators (phase 2)
 constexpr int kProdThreads = 1024;      // phase-1 workgroup
-constexpr int kProdUnroll = 8;
 constexpr int kRedWaves = 8;            // phase-2 workgroup: 8 waves = 8 consecutive row blocks,
 constexpr int kRedThreads = kRedWaves * kWave;  // whose tiles are adjacent in memory for every column block
 constexpr int kRedUnroll = 8;
@@ -201,6 +200,22 @@ __global__ __launch_bounds__(256) void tile_ranges_kernel(int row_blocks, int co
 }
 
 // ---- phase 1 -------------------------------------------------------------------
+// kPiece elements of T make one 128-bit access.
+template <typename T>
+struct alignas(16) Piece {
+  static constexpr int n = 16 / (int)sizeof(T);
+  T e[n];
+};
+// the same elements when only T's own alignment is known (x comes from the caller): the hardware takes
+// unaligned wide global loads
+template <typename T>
+struct __attribute__((packed, aligned(alignof(T)))) LoosePiece {
+  T e[Piece<T>::n];
+};
+struct alignas(16) Cols8 {
+  unsigned short c[8];
+};
+
 template <typename T>
 __global__ __launch_bounds__(kProdThreads) void tiled_products_kernel(
     const TiledChunk* __restrict__ chunks, const T* __restrict__ t_val,
@@ -208,22 +223,57 @@ __global__ __launch_bounds__(kProdThreads) void tiled_products_kernel(
   extern __shared__ __align__(16) unsigned char smem[];
   T* xs = reinterpret_cast<T*>(smem);
   const TiledChunk ch = chunks[blockIdx.x];
-  for (int i = threadIdx.x; i < ch.ncols; i += kProdThreads) xs[i] = x[(int64_t)ch.col0 + i];
-  __syncthreads();
-  constexpr int kStep = kProdThreads * kProdUnroll;
-  int k = ch.begin + threadIdx.x;
-  for (; k + kStep - kProdThreads < ch.end; k += kStep) {
-    T v[kProdUnroll];
-    int c[kProdUnroll];  // widened at once: packing two 16-bit loads into one register would serialise them
+  {
+    // x slice -> LDS: 128-bit pieces, all of a thread's loads issued before the first LDS write
+    // (a load-wait-write loop pays the memory latency once per trip: 32 trips of it were a quarter
+    // of this kernel's time)
+    constexpr int kPer = Piece<T>::n;
+    constexpr int kSlicePieces = TileDims<T>::cols / kPer / kProdThreads;  // pieces per thread in a full slice
+    static_assert(kSlicePieces >= 1 && TileDims<T>::cols % (kPer * kProdThreads) == 0, "slice layout");
+    const T* xsrc = x + (int64_t)ch.col0;
+    const int whole = ch.ncols / kPer;
+    LoosePiece<T> tmp[kSlicePieces];
 #pragma unroll
-    for (int u = 0; u < kProdUnroll; ++u) {
-      v[u] = t_val[k + u * kProdThreads];
-      c[u] = t_col[k + u * kProdThreads];
+    for (int u = 0; u < kSlicePieces; ++u) {
+      const int q = threadIdx.x + u * kProdThreads;
+      if (q < whole) tmp[u] = *reinterpret_cast<const LoosePiece<T>*>(xsrc + q * kPer);
     }
 #pragma unroll
-    for (int u = 0; u < kProdUnroll; ++u) prod[k + u * kProdThreads] = v[u] * xs[c[u]];
+    for (int u = 0; u < kSlicePieces; ++u) {
+      const int q = threadIdx.x + u * kProdThreads;
+      if (q < whole) {
+#pragma unroll
+        for (int i = 0; i < kPer; ++i) xs[q * kPer + i] = tmp[u].e[i];
+      }
+    }
+    const int rest = whole * kPer + threadIdx.x;  // fewer than kPer columns at the end of the last block
+    if (rest < ch.ncols) xs[rest] = xsrc[rest];
   }
-  for (; k < ch.end; k += kProdThreads) prod[k] = t_val[k] * xs[t_col[k]];
+  __syncthreads();
+  // Entries: a thread takes 8 consecutive ones -- one 128-bit load of columns, 8*sizeof(T)/16 of values,
+  // as many stores of products -- so a wave instruction moves 1 KiB instead of 128 or 256 bytes.
+  // The arrays are the library's own (256-byte aligned); the chunk's first entries up to a multiple
+  // of 8 and its last few are taken one by one.
+  constexpr int kPer = Piece<T>::n;
+  constexpr int kPieces = 8 / kPer;
+  int head = (ch.begin + 7) & ~7;
+  if (head > ch.end) head = ch.end;
+  for (int k = ch.begin + threadIdx.x; k < head; k += kProdThreads) prod[k] = t_val[k] * xs[t_col[k]];
+  const int groups = (ch.end - head) >> 3;
+  for (int g = threadIdx.x; g < groups; g += kProdThreads) {
+    const int k = head + (g << 3);
+    const Cols8 c = *reinterpret_cast<const Cols8*>(t_col + k);
+    Piece<T> v[kPieces];
+#pragma unroll
+    for (int i = 0; i < kPieces; ++i) v[i] = *reinterpret_cast<const Piece<T>*>(t_val + k + i * kPer);
+#pragma unroll
+    for (int i = 0; i < kPieces; ++i) {
+#pragma unroll
+      for (int j = 0; j < kPer; ++j) v[i].e[j] = v[i].e[j] * xs[c.c[i * kPer + j]];
+      *reinterpret_cast<Piece<T>*>(prod + k + i * kPer) = v[i];
+    }
+  }
+  for (int k = head + (groups << 3) + threadIdx.x; k < ch.end; k += kProdThreads) prod[k] = t_val[k] * xs[t_col[k]];
 }
 
 // ---- phase 2 -------------------------------------------------------------------
