@@ -212,10 +212,6 @@ template <typename T>
 struct __attribute__((packed, aligned(alignof(T)))) LoosePiece {
   T e[Piece<T>::n];
 };
-struct alignas(16) Cols8 {
-  unsigned short c[8];
-};
-
 template <typename T>
 __global__ __launch_bounds__(kProdThreads) void tiled_products_kernel(
     const TiledChunk* __restrict__ chunks, const T* __restrict__ t_val,
@@ -250,30 +246,41 @@ __global__ __launch_bounds__(kProdThreads) void tiled_products_kernel(
     if (rest < ch.ncols) xs[rest] = xsrc[rest];
   }
   __syncthreads();
-  // Entries: a thread takes 8 consecutive ones -- one 128-bit load of columns, 8*sizeof(T)/16 of values,
-  // as many stores of products -- so a wave instruction moves 1 KiB instead of 128 or 256 bytes.
-  // The arrays are the library's own (256-byte aligned); the chunk's first entries up to a multiple
-  // of 8 and its last few are taken one by one.
+  // Entries: a wave takes 512 consecutive ones per trip as 128-bit pieces of values, piece i*64 + lane in
+  // instruction i, so every instruction moves 1 KiB of consecutive bytes; the lane's columns are the
+  // matching Piece<T>::n 16-bit indices, its products go back the same way.  (A 2- or 4-byte access per
+  // lane and entry issues four to eight times as many instructions; consecutive pieces per LANE instead of
+  // per instruction touch every 128-byte line from several instructions.)  The arrays are the library's
+  // own, 256-byte aligned; the chunk's first entries up to a multiple of 8 and what is left after the
+  // last whole 512 are taken one by one.
   constexpr int kPer = Piece<T>::n;
   constexpr int kPieces = 8 / kPer;
+  constexpr int kSpan = 8 * kWave;  // entries per wave and trip
+  struct alignas(2 * kPer) ColPiece {
+    unsigned short c[kPer];
+  };
+  const int lane = threadIdx.x % kWave;
   int head = (ch.begin + 7) & ~7;
   if (head > ch.end) head = ch.end;
   for (int k = ch.begin + threadIdx.x; k < head; k += kProdThreads) prod[k] = t_val[k] * xs[t_col[k]];
-  const int groups = (ch.end - head) >> 3;
-  for (int g = threadIdx.x; g < groups; g += kProdThreads) {
-    const int k = head + (g << 3);
-    const Cols8 c = *reinterpret_cast<const Cols8*>(t_col + k);
+  const int spans = (ch.end - head) / kSpan;
+  for (int g = threadIdx.x / kWave; g < spans; g += kProdThreads / kWave) {
+    const int kb = head + g * kSpan + lane * kPer;
     Piece<T> v[kPieces];
+    ColPiece c[kPieces];
 #pragma unroll
-    for (int i = 0; i < kPieces; ++i) v[i] = *reinterpret_cast<const Piece<T>*>(t_val + k + i * kPer);
+    for (int i = 0; i < kPieces; ++i) {
+      v[i] = *reinterpret_cast<const Piece<T>*>(t_val + kb + i * kWave * kPer);
+      c[i] = *reinterpret_cast<const ColPiece*>(t_col + kb + i * kWave * kPer);
+    }
 #pragma unroll
     for (int i = 0; i < kPieces; ++i) {
 #pragma unroll
-      for (int j = 0; j < kPer; ++j) v[i].e[j] = v[i].e[j] * xs[c.c[i * kPer + j]];
-      *reinterpret_cast<Piece<T>*>(prod + k + i * kPer) = v[i];
+      for (int j = 0; j < kPer; ++j) v[i].e[j] = v[i].e[j] * xs[c[i].c[j]];
+      *reinterpret_cast<Piece<T>*>(prod + kb + i * kWave * kPer) = v[i];
     }
   }
-  for (int k = head + (groups << 3) + threadIdx.x; k < ch.end; k += kProdThreads) prod[k] = t_val[k] * xs[t_col[k]];
+  for (int k = head + spans * kSpan + threadIdx.x; k < ch.end; k += kProdThreads) prod[k] = t_val[k] * xs[t_col[k]];
 }
 
 // ---- phase 2 -------------------------------------------------------------------
