@@ -470,7 +470,7 @@ static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* 
                             hipFuncAttributeMaxDynamicSharedMemorySize, kTileBytes);
   if (e == hipSuccess)
     e = hipFuncSetAttribute((const void*)tiled_reduce_kernel<T>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, TileDims<T>::red_bytes);
+                            hipFuncAttributeMaxDynamicSharedMemorySize, TileDims<T>::red_lds_bytes);
   for (void* d : {(void*)d_coo, (void*)d_key, (void*)d_key2, (void*)d_idx, (void*)d_perm, (void*)d_tile_ptr,
                   (void*)d_long_raw, (void*)d_long_count, (void*)d_cnt, (void*)d_cgb, (void*)d_rgb, (void*)d_cbs})
     if (d) (void)hipFree(d);
@@ -854,7 +854,8 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
       if (p->n_chunks > 0)
         tiled_products_kernel<T><<<p->n_chunks, kProdThreads, kTileBytes, s>>>(
             p->d_chunks, (const T*)p->d_tval, p->d_tcol, x, (T*)p->d_tprod);
-      tiled_reduce_kernel<T><<<(st.tile_row_blocks + kRedWaves - 1) / kRedWaves, kRedThreads, TileDims<T>::red_bytes, s>>>(
+      tiled_reduce_kernel<T><<<(st.tile_row_blocks + TileDims<T>::red_waves - 1) / TileDims<T>::red_waves, TileDims<T>::red_threads,
+                               TileDims<T>::red_lds_bytes, s>>>(
           st.m, st.tile_row_blocks, st.tile_col_blocks, p->d_row_block_start, p->d_ranges, p->d_trow,
           (const T*)p->d_tprod, alpha, beta, y);
       if (p->n_long_chunks > 0)

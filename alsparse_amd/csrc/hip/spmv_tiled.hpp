@@ -50,10 +50,8 @@ namespace asamd {
 
 constexpr int kTileBytes = 128 * 1024;  // LDS bytes of an x slice (phase 1) / of a workgroup's accumulators (phase 2)
 constexpr int kProdThreads = 1024;      // phase-1 workgroup
-constexpr int kRedWaves = 8;            // phase-2 workgroup: 8 waves = 8 consecutive row blocks,
-constexpr int kRedThreads = kRedWaves * kWave;  // whose tiles are adjacent in memory for every column block
+constexpr int kRedWaves = 8;            // phase-2 workgroup: 8 waves = 8 consecutive row blocks, whose tiles are adjacent in memory
 constexpr int kRedUnroll = 8;
-constexpr int kRedBytes = kTileBytes / 2;  // LDS bytes of a phase-2 workgroup's accumulators
 constexpr int kLongTile = 2 * kWave;     // phase 2 takes two entries per lane and tile; longer tiles go to phase 3
 constexpr int kLongThreads = 256;
 constexpr int kLongChunk = kLongThreads * 16;  // entries per phase-3 workgroup
@@ -66,12 +64,17 @@ constexpr int kRowGroupLog2 = 6;        // row blocks at multiples of 64 rows
 template <typename T>
 struct TileDims {
   static constexpr int cols = kTileBytes / (int)sizeof(T);            // widest column block: 32768 fp32, 16384 fp64
-  // LDS bytes of a phase-2 workgroup's accumulators: wider values get the larger share, so that a row
-  // block keeps 2048 rows (tiles per matrix, which is what phase 2 pays for, do not double)
-  static constexpr int red_bytes = sizeof(T) >= 8 ? kTileBytes : kRedBytes;
-  static constexpr int rows = red_bytes / kRedWaves / (int)sizeof(T);  // tallest row block: 2048 (1024 for 16-byte values)
-  // tiles per batch of phase 2 (16 per batch were measured no faster for 8-byte values and spill
-  // registers for 16-byte ones)
+  // Phase 2 pays per TILE, so a row block keeps 2048 rows whatever the value size (1024 for 16-byte
+  // values): 8 waves with 64 KiB of accumulators for 4-byte values, 128 KiB for wider ones.  (16 waves
+  // with 128 KiB for 4-byte values -- runs of 16 adjacent tiles instead of 8 per column block -- were
+  // measured no faster.)
+  static constexpr int red_waves = kRedWaves;
+  static constexpr int red_threads = red_waves * kWave;
+  static constexpr int red_bytes = sizeof(T) >= 8 ? kTileBytes : kTileBytes / 2;
+  static constexpr int rows = red_bytes / red_waves / (int)sizeof(T);  // tallest row block
+  // every wave's accumulators are followed by one dummy row per lane, where lanes without an entry add their zero
+  static constexpr int red_lds_bytes = red_bytes + red_waves * kWave * (int)sizeof(T);
+  // tiles per barrier interval of phase 2
   static constexpr int red_unroll = kRedUnroll;
 };
 
@@ -210,7 +213,7 @@ struct alignas(16) Piece {
 // unaligned wide global loads
 template <typename T>
 struct __attribute__((packed, aligned(alignof(T)))) LoosePiece {
-  T e[Piece<T>::n];
+  unsigned w[4];  // plain words: the piece is only moved, never computed with
 };
 template <typename T>
 __global__ __launch_bounds__(kProdThreads) void tiled_products_kernel(
@@ -238,8 +241,9 @@ __global__ __launch_bounds__(kProdThreads) void tiled_products_kernel(
     for (int u = 0; u < kSlicePieces; ++u) {
       const int q = threadIdx.x + u * kProdThreads;
       if (q < whole) {
+        unsigned* dst = reinterpret_cast<unsigned*>(xs + q * kPer);
 #pragma unroll
-        for (int i = 0; i < kPer; ++i) xs[q * kPer + i] = tmp[u].e[i];
+        for (int i = 0; i < 4; ++i) dst[i] = tmp[u].w[i];
       }
     }
     const int rest = whole * kPer + threadIdx.x;  // fewer than kPer columns at the end of the last block
@@ -265,19 +269,24 @@ __global__ __launch_bounds__(kProdThreads) void tiled_products_kernel(
   for (int k = ch.begin + threadIdx.x; k < head; k += kProdThreads) prod[k] = t_val[k] * xs[t_col[k]];
   const int spans = (ch.end - head) / kSpan;
   for (int g = threadIdx.x / kWave; g < spans; g += kProdThreads / kWave) {
-    const int kb = head + g * kSpan + lane * kPer;
-    Piece<T> v[kPieces];
-    ColPiece c[kPieces];
+    // at most four pieces (64 bytes per lane) in flight at a time: eight 16-byte values would spill
+    constexpr int kFlight = kPieces < 4 ? kPieces : 4;
 #pragma unroll
-    for (int i = 0; i < kPieces; ++i) {
-      v[i] = *reinterpret_cast<const Piece<T>*>(t_val + kb + i * kWave * kPer);
-      c[i] = *reinterpret_cast<const ColPiece*>(t_col + kb + i * kWave * kPer);
-    }
+    for (int i0 = 0; i0 < kPieces; i0 += kFlight) {
+      const int kb = head + g * kSpan + (i0 * kWave + lane) * kPer;
+      Piece<T> v[kFlight];
+      ColPiece c[kFlight];
 #pragma unroll
-    for (int i = 0; i < kPieces; ++i) {
+      for (int i = 0; i < kFlight; ++i) {
+        v[i] = *reinterpret_cast<const Piece<T>*>(t_val + kb + i * kWave * kPer);
+        c[i] = *reinterpret_cast<const ColPiece*>(t_col + kb + i * kWave * kPer);
+      }
 #pragma unroll
-      for (int j = 0; j < kPer; ++j) v[i].e[j] = v[i].e[j] * xs[c[i].c[j]];
-      *reinterpret_cast<Piece<T>*>(prod + kb + i * kWave * kPer) = v[i];
+      for (int i = 0; i < kFlight; ++i) {
+#pragma unroll
+        for (int j = 0; j < kPer; ++j) v[i].e[j] = v[i].e[j] * xs[c[i].c[j]];
+        *reinterpret_cast<Piece<T>*>(prod + kb + i * kWave * kPer) = v[i];
+      }
     }
   }
   for (int k = head + spans * kSpan + threadIdx.x; k < ch.end; k += kProdThreads) prod[k] = t_val[k] * xs[t_col[k]];
@@ -303,12 +312,16 @@ __device__ __forceinline__ void rmw(T* p, T v) {
 
 constexpr int kMaxPasses = 4;
 
-template <bool Atomic = false, typename T>
-__device__ __forceinline__ void add_rows(T* acc, int r, T v, bool valid) {
+// AllValid: every lane holds an entry or a private dummy row of acc (distinct per lane, so it never
+// continues a run), and `valid` is not looked at: no masks around the read-modify-writes.
+template <bool Atomic = false, bool AllValid = false, typename T>
+__device__ __forceinline__ void add_rows(T* acc, int r, T v, bool valid_arg) {
+  const bool valid = AllValid ? true : valid_arg;
   const int lane = threadIdx.x % kWave;
   const int r_up = __builtin_amdgcn_update_dpp(-1, r, 0x138, 0xF, 0xF, false);  // wave_shr:1, lane 0 keeps -1
-  // lanes without an entry carry r = -2 - lane: negative, distinct from each other and from the
-  // -1 that lane 0 sees below it, so the comparison alone tells a continued run
+  // lanes without an entry carry a row of their own (a dummy row, or -2 - lane where acc has none):
+  // distinct from each other and from the -1 that lane 0 sees below it, so the comparison alone
+  // tells a continued run
   const bool same_as_prev = r_up == r;
   const uint64_t dup = __builtin_amdgcn_ballot_w64(same_as_prev);
   if (dup == 0) {
@@ -352,7 +365,7 @@ __device__ __forceinline__ void add_rows(T* acc, int r, T v, bool valid) {
 }
 
 template <typename T>
-__global__ __launch_bounds__(kRedThreads) void tiled_reduce_kernel(
+__global__ __launch_bounds__(TileDims<T>::red_threads) void tiled_reduce_kernel(
     int m, int row_blocks, int col_blocks, const int* __restrict__ row_block_start,
     const TileRange* __restrict__ ranges, const unsigned short* __restrict__ t_row,
     const T* __restrict__ prod, T alpha, T beta, T* __restrict__ y) {
@@ -362,79 +375,79 @@ __global__ __launch_bounds__(kRedThreads) void tiled_reduce_kernel(
   constexpr int kUnroll = TileDims<T>::red_unroll;
   const int lane = threadIdx.x % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-  const int rb = blockIdx.x * kRedWaves + wave;
+  const int rb = blockIdx.x * TileDims<T>::red_waves + wave;
   const bool active = rb < row_blocks;  // wave-uniform; idle waves still meet the barriers
-  T* acc = s_acc + wave * kTileRows;
-  for (int i = lane; i < kTileRows; i += kWave) acc[i] = T(0);
+  T* acc = s_acc + wave * (kTileRows + kWave);
+  for (int i = lane; i < kTileRows + kWave; i += kWave) acc[i] = T(0);
 
-  // Wave-private accumulators; the tiles of kUnroll column blocks form a batch
-  // (every tile listed in `ranges` has at most kLongTile = 128 entries: two per
-  // lane).  The loads of batch q + 1 are issued before batch q is added, so the
-  // LDS read-modify-write chain of one batch hides the memory latency of the next.
-  struct Batch {
-    T v[kUnroll][2];
-    int r[kUnroll][2];
-    int len[kUnroll];
-  };
+  // Wave-private accumulators.  Every tile listed in `ranges` has at most kLongTile = 128 entries: two
+  // per lane.  The wave keeps kSlots tiles in flight in a ring of registers: step s adds the tile in slot s
+  // and at once loads the tile kSlots further on into it, so the loads of the next kSlots - 1 tiles are
+  // outstanding while one tile goes through its LDS read-modify-writes.  For the hardware counter of
+  // outstanding loads to allow that, every load is issued unconditionally (lanes past the end of a
+  // tile re-read its first entry and are masked when the slot is used), and the waves are kept in
+  // step with a bare barrier instruction: they share no data, and the fence of __syncthreads() would
+  // drain all loads at every barrier.
+  constexpr int kSlots = sizeof(T) >= 16 ? kUnroll : 2 * kUnroll;
+  static_assert(kWave % kSlots == 0, "a group of tile ranges is a whole number of rings");
+  T sv[kSlots][2];
+  int sr[kSlots][2];
+  int slen[kSlots];
   const TileRange* my = ranges + (int64_t)(active ? rb : 0) * col_blocks;
-  constexpr int kPerGroup = kWave / kUnroll;  // batches per group of 64 tile ranges
-  const int nq = (col_blocks + kUnroll - 1) / kUnroll;
   auto load_ranges = [&](int group) {  // 64 tile ranges, one coalesced load
-    TileRange t = {0, 0};
     const int cb = group * kWave + lane;
-    if (active && cb < col_blocks) t = my[cb];
+    const bool ok = active && cb < col_blocks;
+    TileRange t = my[ok ? cb : 0];
+    if (!ok) t.begin = t.end = 0;
     return t;
   };
-  const int r_none = -2 - lane;  // "no entry": negative and different in every lane
-  auto fetch = [&](const TileRange& tr, int q, Batch& bt) {
-    const int j = (q % kPerGroup) * kUnroll;
-    const int left = col_blocks - (q / kPerGroup) * kWave;
-    const int ncb = left < kWave ? left : kWave;
-#pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-      const int src = j + u < ncb ? j + u : j;
-      const int b = __builtin_amdgcn_readlane(tr.begin, src);
-      const int e = j + u < ncb ? __builtin_amdgcn_readlane(tr.end, src) : b;
-      bt.len[u] = e - b;
-      {
-        const int k = b + lane;
-        const bool ok = k < e;
-        bt.v[u][0] = ok ? prod[k] : T(0);
-        bt.r[u][0] = ok ? (int)t_row[k] : -2 - lane;
-      }
-      if (e - b > kWave) {  // wave-uniform: half of the tiles never need the second load pair
-        const int k = b + kWave + lane;
-        const bool ok = k < e;
-        bt.v[u][1] = ok ? prod[k] : T(0);
-        bt.r[u][1] = ok ? (int)t_row[k] : -2 - lane;
-      }
-    }
-  };
-  auto add = [&](const Batch& bt) {
-#pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-      add_rows(acc, bt.r[u][0], bt.v[u][0], bt.r[u][0] >= 0);
-      if (bt.len[u] > kWave) add_rows(acc, bt.r[u][1], bt.v[u][1], bt.r[u][1] >= 0);  // wave-uniform
-    }
-  };
-  Batch A, B;
+  const int r_none = kTileRows + lane;  // "no entry": the lane's dummy row behind the accumulators
+  // the tile ranges of a group are loaded while the group before it is worked on
   TileRange tr = load_ranges(0);
-  if (nq > 0) fetch(tr, 0, A);
-  for (int q = 0; q < nq; q += 2) {
-    // A holds batch q
-    if (q + 1 < nq) {
-      if ((q + 1) % kPerGroup == 0) tr = load_ranges((q + 1) / kPerGroup);
-      fetch(tr, q + 1, B);
+  TileRange tr_next = load_ranges(1);
+  auto issue = [&](int s, int ti) {  // tile ti (wave-uniform) -> slot s
+    const int src = ti & (kWave - 1);
+    int b0 = __builtin_amdgcn_readlane(tr.begin, src);
+    const int e0 = __builtin_amdgcn_readlane(tr.end, src);
+    const int len = ti < col_blocks ? e0 - b0 : 0;
+    if (len == 0) b0 = 0;  // keeps the addresses below inside the arrays
+    slen[s] = len;
+    // scalar base per tile, the lane as the only vector part of the address
+    const T* pv = prod + b0;
+    const unsigned short* pr = t_row + b0;
+    const int i0 = lane < len ? lane : 0;
+    const int i1 = lane + kWave < len ? lane + kWave : 0;
+    sv[s][0] = pv[i0];
+    sr[s][0] = pr[i0];
+    sv[s][1] = pv[i1];
+    sr[s][1] = pr[i1];
+  };
+  auto consume = [&](int s) {
+    const int len = slen[s];
+    {
+      const bool ok = lane < len;
+      add_rows<false, true>(acc, ok ? sr[s][0] : r_none, ok ? sv[s][0] : T(0), true);
     }
-    add(A);
-    __syncthreads();  // keeps the waves on neighbouring tiles: their reads form one burst
-    if (q + 1 >= nq) break;
-    if (q + 2 < nq) {
-      if ((q + 2) % kPerGroup == 0) tr = load_ranges((q + 2) / kPerGroup);
-      fetch(tr, q + 2, A);
+    if (len > kWave) {  // wave-uniform
+      const bool ok = lane + kWave < len;
+      add_rows<false, true>(acc, ok ? sr[s][1] : r_none, ok ? sv[s][1] : T(0), true);
     }
-    add(B);
-    __syncthreads();
+  };
+#pragma unroll
+  for (int s = 0; s < kSlots; ++s) issue(s, s);
+  for (int t0 = 0; t0 < col_blocks; t0 += kSlots) {
+#pragma unroll
+    for (int s = 0; s < kSlots; ++s) {
+      consume(s);
+      const int ti = t0 + s + kSlots;
+      if (s == 0 && (ti & (kWave - 1)) == 0) {  // ti is a multiple of kSlots here: groups change at s == 0 only
+        tr = tr_next;
+        tr_next = load_ranges(ti / kWave + 1);
+      }
+      issue(s, ti);
+      // keeps the waves on neighbouring tiles: their reads form one burst
+      if (s % kUnroll == kUnroll - 1) __builtin_amdgcn_s_barrier();
+    }
   }
   if (!active) return;
   const int64_t row0 = row_block_start[rb];
