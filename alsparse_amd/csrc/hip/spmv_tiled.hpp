@@ -395,11 +395,11 @@ __global__ __launch_bounds__(TileDims<T>::red_threads) void tiled_reduce_kernel(
   int slen[kSlots];
   const TileRange* my = ranges + (int64_t)(active ? rb : 0) * col_blocks;
   auto load_ranges = [&](int group) {  // 64 tile ranges, one coalesced load
+    // no select on the loaded value (it would wait for the load at once): tiles past col_blocks are
+    // cut off in issue(), and a wave without a row block of its own re-adds row block 0 into
+    // accumulators that it never writes out
     const int cb = group * kWave + lane;
-    const bool ok = active && cb < col_blocks;
-    TileRange t = my[ok ? cb : 0];
-    if (!ok) t.begin = t.end = 0;
-    return t;
+    return my[cb < col_blocks ? cb : 0];
   };
   const int r_none = kTileRows + lane;  // "no entry": the lane's dummy row behind the accumulators
   // the tile ranges of a group are loaded while the group before it is worked on
@@ -434,7 +434,12 @@ __global__ __launch_bounds__(TileDims<T>::red_threads) void tiled_reduce_kernel(
     }
   };
 #pragma unroll
-  for (int s = 0; s < kSlots; ++s) issue(s, s);
+  for (int s = 0; s < kSlots; ++s) {
+    issue(s, s);
+    // in slot order: the loop's first wait is for slot 0, and the count of loads that may stay
+    // outstanding at that wait is the smaller of what the two ways into the loop guarantee
+    __builtin_amdgcn_sched_barrier(0);
+  }
   for (int t0 = 0; t0 < col_blocks; t0 += kSlots) {
 #pragma unroll
     for (int s = 0; s < kSlots; ++s) {
