@@ -25,11 +25,12 @@
 //            (they are adjacent, the tile being in CSR order) are first combined
 //            inside the wave, so no atomics are needed: LDS float atomics were
 //            measured at ~0.45 lanes per clock, four times slower than the whole
-//            phase takes without them.  The kRedWaves waves of a workgroup own
-//            consecutive row blocks, whose tiles are adjacent in memory, and a
-//            barrier per batch of column blocks keeps them in step, so DRAM sees
-//            one multi-KiB burst per column block instead of scattered 256-byte
-//            reads.  Finally y = beta*y + alpha*acc, unit stride.
+//            phase takes without them.  A wave keeps 16 tiles in flight in a
+//            ring of registers (loads issued unconditionally, so the counter of
+//            outstanding loads lets it wait for the oldest tile only).  The
+//            kRedWaves waves of a workgroup own consecutive row blocks, whose
+//            tiles are adjacent in memory.  Finally y = beta*y + alpha*acc, unit
+//            stride.
 //   phase 3  tiled_long_kernel       only if some tile holds more than kLongTile
 //            entries (long rows, hot columns): those tiles are left out of phase
 //            2 and streamed by as many workgroups as their size needs; rows are
@@ -51,7 +52,7 @@ namespace asamd {
 constexpr int kTileBytes = 128 * 1024;  // LDS bytes of an x slice (phase 1) / of a workgroup's accumulators (phase 2)
 constexpr int kProdThreads = 1024;      // phase-1 workgroup
 constexpr int kRedWaves = 8;            // phase-2 workgroup: 8 waves = 8 consecutive row blocks, whose tiles are adjacent in memory
-constexpr int kRedUnroll = 8;
+constexpr int kRedSlots = 16;
 constexpr int kLongTile = 2 * kWave;     // phase 2 takes two entries per lane and tile; longer tiles go to phase 3
 constexpr int kLongThreads = 256;
 constexpr int kLongChunk = kLongThreads * 16;  // entries per phase-3 workgroup
@@ -74,8 +75,8 @@ struct TileDims {
   static constexpr int rows = red_bytes / red_waves / (int)sizeof(T);  // tallest row block
   // every wave's accumulators are followed by one dummy row per lane, where lanes without an entry add their zero
   static constexpr int red_lds_bytes = red_bytes + red_waves * kWave * (int)sizeof(T);
-  // tiles per barrier interval of phase 2
-  static constexpr int red_unroll = kRedUnroll;
+  // tiles a wave keeps in flight in phase 2 (16 four-register slots would not fit for 16-byte values)
+  static constexpr int red_slots = sizeof(T) >= 16 ? kRedSlots / 2 : kRedSlots;
 };
 
 struct TiledChunk {
@@ -372,11 +373,10 @@ __global__ __launch_bounds__(TileDims<T>::red_threads) void tiled_reduce_kernel(
   extern __shared__ __align__(16) unsigned char smem[];
   T* s_acc = reinterpret_cast<T*>(smem);
   constexpr int kTileRows = TileDims<T>::rows;
-  constexpr int kUnroll = TileDims<T>::red_unroll;
   const int lane = threadIdx.x % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int rb = blockIdx.x * TileDims<T>::red_waves + wave;
-  const bool active = rb < row_blocks;  // wave-uniform; idle waves still meet the barriers
+  if (rb >= row_blocks) return;  // wave-uniform
   T* acc = s_acc + wave * (kTileRows + kWave);
   for (int i = lane; i < kTileRows + kWave; i += kWave) acc[i] = T(0);
 
@@ -385,19 +385,18 @@ __global__ __launch_bounds__(TileDims<T>::red_threads) void tiled_reduce_kernel(
   // and at once loads the tile kSlots further on into it, so the loads of the next kSlots - 1 tiles are
   // outstanding while one tile goes through its LDS read-modify-writes.  For the hardware counter of
   // outstanding loads to allow that, every load is issued unconditionally (lanes past the end of a
-  // tile re-read its first entry and are masked when the slot is used), and the waves are kept in
-  // step with a bare barrier instruction: they share no data, and the fence of __syncthreads() would
-  // drain all loads at every barrier.
-  constexpr int kSlots = sizeof(T) >= 16 ? kUnroll : 2 * kUnroll;
+  // tile re-read its first entry and are masked when the slot is used).  The waves of a workgroup
+  // share no data and meet at no barrier: with one batch of 8 tiles in flight a barrier per batch kept
+  // their reads on neighbouring tiles and doubled the speed, with the ring it measured no different.
+  constexpr int kSlots = TileDims<T>::red_slots;
   static_assert(kWave % kSlots == 0, "a group of tile ranges is a whole number of rings");
   T sv[kSlots][2];
   int sr[kSlots][2];
   int slen[kSlots];
-  const TileRange* my = ranges + (int64_t)(active ? rb : 0) * col_blocks;
+  const TileRange* my = ranges + (int64_t)rb * col_blocks;
   auto load_ranges = [&](int group) {  // 64 tile ranges, one coalesced load
     // no select on the loaded value (it would wait for the load at once): tiles past col_blocks are
-    // cut off in issue(), and a wave without a row block of its own re-adds row block 0 into
-    // accumulators that it never writes out
+    // cut off in issue()
     const int cb = group * kWave + lane;
     return my[cb < col_blocks ? cb : 0];
   };
@@ -450,11 +449,8 @@ __global__ __launch_bounds__(TileDims<T>::red_threads) void tiled_reduce_kernel(
         tr_next = load_ranges(ti / kWave + 1);
       }
       issue(s, ti);
-      // keeps the waves on neighbouring tiles: their reads form one burst
-      if (s % kUnroll == kUnroll - 1) __builtin_amdgcn_s_barrier();
     }
   }
-  if (!active) return;
   const int64_t row0 = row_block_start[rb];
   const int nrows = row_block_start[rb + 1] - (int)row0;  // <= kTileRows
   for (int i = lane; i < nrows; i += kWave) store_axpby(y, row0 + i, alpha, acc[i], beta);
