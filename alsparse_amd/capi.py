@@ -304,7 +304,9 @@ _COMMON = {
     "asamd_csr_plan_transpose_stats": [_P],
     "asamd_csr_plan_transpose_arrays": [_P, _I, POINTER(_P), POINTER(_P), POINTER(_P)],
     "asamd_csrmm_workspace_bytes": [_I, _I, _I, _I, POINTER(asamd_dense_strides)],
+    "asamd_csr2coo_workspace_bytes": [_I],
     "asamd_csr2coo": [_P, _P, _I, _I, _P, _I],
+    "asamd_csr2coo_ws": [_P, _P, _I, _I, _P, _I, _P, c_size_t],
     "asamd_csr2ell_width": [_P, _I, _P, POINTER(_I)],
     "asamd_warmup": [_P],
     "asamd_handle_set_stream": [_P, _P],
@@ -336,7 +338,7 @@ _RESTYPE = {"alpha_set_thread_num": None, "alpha_timing_wtime": c_double, "alpha
             "args_help": None, "args_get_if_check": c_bool, "args_get_data_file": ctypes.c_char_p,
             "args_get_data_fileA": ctypes.c_char_p, "args_get_data_fileB": ctypes.c_char_p,
             "alpha_args_get_matrix_descrA": alpha_matrix_descr, "alpha_args_get_matrix_descrB": alpha_matrix_descr,
-            "get_time_us": c_double, "asamd_csrmm_workspace_bytes": c_size_t, "asamd_csr_plan_stats": POINTER(asamd_csr_stats),
+            "get_time_us": c_double, "asamd_csrmm_workspace_bytes": c_size_t, "asamd_csr2coo_workspace_bytes": c_size_t, "asamd_csr_plan_stats": POINTER(asamd_csr_stats),
             "asamd_csr_plan_transpose_stats": POINTER(asamd_csr_stats),
             "asamd_analysis_transpose_stats": POINTER(asamd_csr_stats),
             "asamd_analysis_stats": POINTER(asamd_csr_stats)}

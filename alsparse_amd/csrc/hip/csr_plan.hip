@@ -400,7 +400,9 @@ static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* 
   if (e == hipSuccess) e = hipMalloc(&p->d_tcol, nnz * sizeof(unsigned short));
   if (e == hipSuccess) e = hipMalloc(&p->d_trow, nnz * sizeof(unsigned short));
   if (e == hipSuccess) e = hipMalloc(&p->d_tprod, nnz * sizeof(T));
-  if (e == hipSuccess) e = (hipError_t)asamd_csr2coo(stream, row_ptr, st.nnz, st.m, d_coo, st.base);
+  // d_key2 is free until the sort: it serves csr2coo as its table of chunk rows
+  if (e == hipSuccess)
+    e = (hipError_t)asamd_csr2coo_ws(stream, row_ptr, st.nnz, st.m, d_coo, st.base, d_key2, (size_t)nnz * sizeof(unsigned));
   if (e == hipSuccess) {
     tile_keys_kernel<<<256 * 32, 256, 0, stream>>>(st.nnz, d_coo, col_ind, st.base, d_cgb, d_rgb, rb, d_key, d_idx);
     e = sort_pairs_u32(stream, d_key, d_key2, d_idx, d_perm, nnz, key_bits);
@@ -690,7 +692,8 @@ static hipError_t build_transpose(hipStream_t stream, asamd_csr_plan* p, const i
   if (e == hipSuccess) e = hipMalloc(&t.d_row_ptr, ((size_t)n + 1) * sizeof(int));
   if (e == hipSuccess) e = hipMalloc(&t.d_col, (size_t)nnz * sizeof(int));
   if (e == hipSuccess) e = hipMalloc(&t.d_val, (size_t)nnz * sizeof(T));
-  if (e == hipSuccess) e = (hipError_t)asamd_csr2coo(stream, row_ptr, nnz, st.m, d_coo, st.base);
+  if (e == hipSuccess)  // d_key2 is free until the sort
+    e = (hipError_t)asamd_csr2coo_ws(stream, row_ptr, nnz, st.m, d_coo, st.base, d_key2, (size_t)nnz * sizeof(unsigned));
   if (e == hipSuccess) {
     int grid = (nnz + 255) / 256;
     if (grid > 256 * 32) grid = 256 * 32;

@@ -16,7 +16,9 @@ alphasparse_status_t alphasparse_dcu_csr2coo(alphasparse_dcu_handle_t handle,
   if (nnz < 0 || m < 0) return ALPHA_SPARSE_STATUS_INVALID_VALUE;
   if (nnz == 0 || m == 0) return ALPHA_SPARSE_STATUS_SUCCESS;
   if (csr_row_ptr == NULL || coo_row_ind == NULL) return ALPHA_SPARSE_STATUS_INVALID_POINTER;
-  ASAMD_HIP_STATUS(asamd_csr2coo(handle->stream, csr_row_ptr, nnz, m, coo_row_ind, (int32_t)idx_base));
+  /* the handle's scratch holds the table of chunk rows whenever it is large enough (1 MiB: up to 2^31 entries) */
+  ASAMD_HIP_STATUS(asamd_csr2coo_ws(handle->stream, csr_row_ptr, nnz, m, coo_row_ind, (int32_t)idx_base,
+                                    handle->buffer, handle->buffer_size));
   return ALPHA_SPARSE_STATUS_SUCCESS;
 }
 

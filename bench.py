@@ -305,6 +305,45 @@ def run_host_pointer_spmv(cfg, steps):
             "staged_bytes_per_call": int(x.nbytes + y.nbytes * (2 if beta != 0 else 1))}
 
 
+def run_conversions(cfg, steps, warmup):
+    """alphasparse_dcu_csr2coo and alphasparse_dcu_?csr2ell on configuration `cfg`, device-resident:
+    ms per conversion and GB/s of compulsory traffic (csr2coo reads row_ptr and writes nnz row
+    indices; csr2ell reads the CSR arrays and writes m * width slots of value and index)."""
+    from ctypes import c_int32
+    from alsparse_amd import capi, hiprt, workloads as wl
+    lib = capi.load()
+    a, _, _, _, _, _ = wl.config(cfg)
+    sz = a.dtype.itemsize
+    h = capi.Handle()
+    descr = capi.make_descr()
+    d_val, d_rp, d_ci = (hiprt.DeviceArray.from_numpy(v) for v in (a.values, a.row_ptr, a.col_ind))
+    d_rows = hiprt.DeviceArray((a.nnz,), np.int32)
+
+    def coo_step():
+        if lib.alphasparse_dcu_csr2coo(h.h, d_rp.c_ptr(), a.nnz, a.rows, d_rows.c_ptr(), 0) != 0:
+            raise RuntimeError("csr2coo failed")
+    t_coo = time_steps(coo_step, steps, warmup, hiprt)
+    w = c_int32(-1)
+    assert lib.alphasparse_dcu_csr2ell_width(h.h, a.rows, byref(descr), d_rp.c_ptr(), byref(descr), byref(w)) == 0
+    ev, ec = hiprt.DeviceArray((w.value * a.rows,), a.dtype), hiprt.DeviceArray((w.value * a.rows,), np.int32)
+    conv = lib.alphasparse_dcu_scsr2ell if a.dtype == np.float32 else lib.alphasparse_dcu_dcsr2ell
+
+    def ell_step():
+        if conv(h.h, a.rows, byref(descr), d_val.c_ptr(), d_rp.c_ptr(), d_ci.c_ptr(), byref(descr), w.value,
+                ev.c_ptr(), ec.c_ptr()) != 0:
+            raise RuntimeError("csr2ell failed")
+    t_ell = time_steps(ell_step, steps, warmup, hiprt)
+    coo_bytes = (a.rows + 1) * 4 + a.nnz * 4
+    ell_bytes = a.nnz * (4 + sz) + (a.rows + 1) * 4 + a.rows * w.value * (4 + sz)
+    for d in (d_val, d_rp, d_ci, d_rows, ev, ec):
+        d.free()
+    h.close()
+    return {"workload": WORKLOAD_NAMES[cfg] + " -- conversions on the GPU",
+            "csr2coo": {"avg_ms": t_coo["avg_ms"], "bytes": int(coo_bytes), "gbs": coo_bytes / t_coo["avg_ms"] / 1e6},
+            "csr2ell": {"avg_ms": t_ell["avg_ms"], "width": w.value, "bytes": int(ell_bytes),
+                        "gbs": ell_bytes / t_ell["avg_ms"] / 1e6}}
+
+
 def run_format_spmv(cfg, fmt, steps, warmup, check):
     """SpMV on the ELL or COO form of configuration `cfg`, converted on the GPU
     (alphasparse_dcu_csr2coo / _csr2ell) and multiplied by alphasparse_dcu_?_coomv / _ellmv."""
@@ -529,6 +568,8 @@ def main():
             others["C%d_%s" % (c, fmt)] = {k: r[k] for k in ("workload", "gbs", "gflops", "hbm_frac", "timing", "parity", "kernel")}
 
         others["C3_host_pointers"] = run_host_pointer_spmv(3, min(args.steps, 10))
+        for c in (2, 3):
+            others["C%d_conversions" % c] = run_conversions(c, min(args.steps, 10), 2)
 
     t = main_res["timing"]
     out = {

@@ -66,6 +66,54 @@ def test_csr2coo_bit_exact(gpu, shape):
             da.free()
 
 
+BOUNDARY_SHAPES = {
+    # entries per workgroup chunk: 8192.  Rows that start exactly on chunk boundaries, a chunk that is one
+    # row, empty rows around the boundaries, an entry count that is a whole number of chunks and one off it
+    "rows_of_8192": [8192] * 3,
+    "rows_of_4096": [4096] * 5,
+    "empties_at_boundaries": [8192, 0, 0, 8191, 1, 0, 8192, 0],
+    "one_short": [8192, 8191],
+    "one_over": [8192, 8193],
+    "long_row_over_chunks": [3, 30000, 0, 5],
+    "many_empty_rows": [1] + [0] * 20000 + [1] + [0] * 20000 + [8190],
+}
+
+
+@pytest.mark.parametrize("shape", sorted(BOUNDARY_SHAPES))
+def test_csr2coo_entry_points_and_chunk_boundaries(gpu, shape):
+    """asamd_csr2coo (every workgroup searches its rows), asamd_csr2coo_ws (table of chunk rows), an output
+    array that is not 16-byte aligned (no 128-bit stores), both index bases."""
+    lib = capi.load()
+    lens = BOUNDARY_SHAPES[shape]
+    for base in (0, 1):
+        a = csr_from_lengths(lens, max(max(lens), 8), np.float32, base=base)
+        want = orc.csr2coo(a)
+        d_rp = hiprt.DeviceArray.from_numpy(a.row_ptr)
+        ws_bytes = lib.asamd_csr2coo_workspace_bytes(a.nnz)
+        assert ws_bytes == 4 * ((a.nnz + 8191) // 8192 + 1)
+        ws = hiprt.DeviceArray((ws_bytes,), np.uint8)
+        out = hiprt.DeviceArray((a.nnz + 8,), np.int32)
+        try:
+            for shift in (0, 1, 3):                     # elements: 0 = aligned, 1 and 3 = misaligned for 128-bit stores
+                for with_ws in (False, True):
+                    announce("csr2coo raw", shape, base, shift, with_ws)
+                    out.fill_bytes(0xEE)
+                    ptr = out.c_ptr().value + 4 * shift
+                    if with_ws:
+                        st = lib.asamd_csr2coo_ws(None, d_rp.c_ptr(), a.nnz, a.rows, ptr, a.base, ws.c_ptr(), ws_bytes)
+                    else:
+                        st = lib.asamd_csr2coo(None, d_rp.c_ptr(), a.nnz, a.rows, ptr, a.base)
+                    assert st == 0
+                    hiprt.synchronize()
+                    got = out.to_numpy()
+                    assert np.array_equal(got[shift:shift + a.nnz], want)
+                    guard = np.int32(-286331154)        # 0xEEEEEEEE: nothing outside [shift, shift + nnz) is written
+                    assert np.all(got[:shift] == guard) and np.all(got[shift + a.nnz:] == guard)
+        finally:
+            for d in (d_rp, ws, out):
+                d.free()
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
 @pytest.mark.parametrize("shape", ["uniform16", "laplace", "empty_runs", "single_row", "ones"])
 def test_csr2ell_bit_exact(gpu, shape, dtype):
