@@ -231,8 +231,11 @@ __global__ __launch_bounds__(kEllRows) void csr2ell_kernel(
     const int* __restrict__ col_ind, int csr_base, int ell_base, int width,
     T* __restrict__ ell_val, int* __restrict__ ell_col) {
   constexpr int kWindow = sizeof(T) > 8 ? kEllWindow / 2 : kEllWindow;  // at most 32 KiB of staged values
-  __shared__ T s_val[kWindow];
-  __shared__ int s_col[kWindow];
+  // staged entry p lives at p + p / 32: lanes read slot s of consecutive rows, i.e. positions a row
+  // length apart, and without the skew rows of 16 or 32 entries would all fall into a few LDS banks
+  auto at = [](int p) { return p + (p >> 5); };
+  __shared__ T s_val[kWindow + kWindow / 32];
+  __shared__ int s_col[kWindow + kWindow / 32];
   const int64_t row_first = (int64_t)blockIdx.x * kEllRows;
   const int64_t row = row_first + threadIdx.x;
   int64_t row_last = row_first + kEllRows;
@@ -246,9 +249,28 @@ __global__ __launch_bounds__(kEllRows) void csr2ell_kernel(
   }
   const bool staged = blk_end - blk_begin <= kWindow;  // workgroup-uniform
   if (staged) {
-    for (int64_t k = blk_begin + threadIdx.x; k < blk_end; k += kEllRows) {
-      s_val[k - blk_begin] = val[k];
-      s_col[k - blk_begin] = col_ind[k];
+    // eight loads of each stream in flight per thread before the first LDS write: a load-wait-write
+    // loop pays the memory latency once per trip
+    constexpr int kU = 8;
+    const int count = (int)(blk_end - blk_begin);
+    for (int p0 = threadIdx.x; p0 < count; p0 += kU * kEllRows) {
+      T v[kU];
+      int c[kU];
+#pragma unroll
+      for (int u = 0; u < kU; ++u) {
+        const int p = p0 + u * kEllRows;
+        const int q = p < count ? p : p0;  // unconditional loads: the tail re-reads a staged entry
+        v[u] = val[blk_begin + q];
+        c[u] = col_ind[blk_begin + q];
+      }
+#pragma unroll
+      for (int u = 0; u < kU; ++u) {
+        const int p = p0 + u * kEllRows;
+        if (p < count) {
+          s_val[at(p)] = v[u];
+          s_col[at(p)] = c[u];
+        }
+      }
     }
     __syncthreads();
   }
@@ -259,8 +281,9 @@ __global__ __launch_bounds__(kEllRows) void csr2ell_kernel(
     int c = ell_base;
     if (s < len) {
       if (staged) {
-        v = s_val[my_begin - blk_begin + s];
-        c = s_col[my_begin - blk_begin + s] - csr_base + ell_base;
+        const int p = (int)(my_begin - blk_begin) + s;
+        v = s_val[at(p)];
+        c = s_col[at(p)] - csr_base + ell_base;
       } else {
         v = val[my_begin + s];
         c = col_ind[my_begin + s] - csr_base + ell_base;
