@@ -187,10 +187,20 @@ __global__ __launch_bounds__(256) void max_row_len_kernel(int m, const int* __re
   if (threadIdx.x == 0) s_max = 0;
   __syncthreads();
   int lmax = 0;
-  for (int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; r < m;
-       r += (int64_t)gridDim.x * blockDim.x) {
-    const int len = row_ptr[r + 1] - row_ptr[r];
-    lmax = len > lmax ? len : lmax;
+  // eight rows per thread and trip, all sixteen loads issued before the first is used
+  constexpr int kU = 8;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t r0 = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; r0 < m; r0 += kU * stride) {
+    int lo[kU], hi[kU];
+#pragma unroll
+    for (int u = 0; u < kU; ++u) {
+      const int64_t r = r0 + u * stride;
+      const int64_t q = r < m ? r : r0;  // unconditional loads
+      lo[u] = row_ptr[q];
+      hi[u] = row_ptr[q + 1];
+    }
+#pragma unroll
+    for (int u = 0; u < kU; ++u) lmax = max(lmax, hi[u] - lo[u]);
   }
   atomicMax(&s_max, lmax);
   __syncthreads();
@@ -206,8 +216,9 @@ extern "C" int asamd_csr2ell_width(hipStream_t stream, int32_t m, const int32_t*
   hipError_t e = hipMalloc(&d, sizeof(int));
   if (e != hipSuccess) return e;
   zero_int_kernel<<<1, 1, 0, stream>>>(d);
-  int grid = (m + 255) / 256;
-  if (grid > 4096) grid = 4096;
+  // every workgroup ends with one atomic on the same word: few, long-running workgroups
+  int grid = (m + 256 * 8 - 1) / (256 * 8);
+  if (grid > 1024) grid = 1024;
   max_row_len_kernel<<<grid, 256, 0, stream>>>(m, row_ptr, d);
   e = hipMemcpyAsync(width_host, d, sizeof(int), hipMemcpyDeviceToHost, stream);
   if (e == hipSuccess) e = hipStreamSynchronize(stream);

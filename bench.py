@@ -339,9 +339,11 @@ def run_conversions(cfg, steps, warmup):
         d.free()
     h.close()
     return {"workload": WORKLOAD_NAMES[cfg] + " -- conversions on the GPU",
-            "csr2coo": {"avg_ms": t_coo["avg_ms"], "bytes": int(coo_bytes), "gbs": coo_bytes / t_coo["avg_ms"] / 1e6},
+            "rows": a.rows, "nnz": a.nnz, "dtype": "f32" if a.dtype == np.float32 else "f64",
+            "csr2coo": {"avg_ms": t_coo["avg_ms"], "bytes": int(coo_bytes), "gbs": coo_bytes / t_coo["avg_ms"] / 1e6,
+                        "timing": t_coo},
             "csr2ell": {"avg_ms": t_ell["avg_ms"], "width": w.value, "bytes": int(ell_bytes),
-                        "gbs": ell_bytes / t_ell["avg_ms"] / 1e6}}
+                        "gbs": ell_bytes / t_ell["avg_ms"] / 1e6, "timing": t_ell}}
 
 
 def run_format_spmv(cfg, fmt, steps, warmup, check):
@@ -499,6 +501,8 @@ def main():
     ap.add_argument("--complex", action="store_true", dest="cx",
                     help="configuration 2, 3 or 4 with complex values (complex64 / complex128), complex x, y, alpha, beta")
     ap.add_argument("--conjugate", action="store_true", help="with --complex --transpose: A^H instead of A^T")
+    ap.add_argument("--conversions", action="store_true",
+                    help="measure alphasparse_dcu_csr2coo (the main line) and ?csr2ell on configuration 2 or 3")
     ap.add_argument("--all", action="store_true", help="also measure the other configurations")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-vendor-baseline", action="store_true",
@@ -529,7 +533,16 @@ def main():
         dst.free()
 
     check = not args.no_check
-    if args.format != "csr":
+    conv = None
+    if args.conversions:
+        if args.config not in (2, 3):
+            sys.exit("bench.py: --conversions is measured on configuration 2 or 3")
+        conv = run_conversions(args.config, args.steps, args.warmup)
+        main_res = {"workload": conv["workload"], "rows": conv["rows"], "nnz": conv["nnz"], "dtype": "int32",
+                    "algorithmic_bytes": conv["csr2coo"]["bytes"], "gbs": conv["csr2coo"]["gbs"], "gflops": 0.0,
+                    "hbm_frac": conv["csr2coo"]["gbs"] / HBM_PEAK_GBS, "timing": conv["csr2coo"]["timing"],
+                    "kernel": "csr2coo", "parity": None}
+    elif args.format != "csr":
         if args.config not in (2, 3):
             sys.exit("bench.py: --format ell|coo is measured on configuration 2 or 3")
         main_res = run_format_spmv(args.config, args.format, args.steps, args.warmup, check)
@@ -573,7 +586,8 @@ def main():
 
     t = main_res["timing"]
     out = {
-        "metric": ("CSR SpMV effective GB/s (algorithmic bytes / time), 1 GPU" if args.format == "csr"
+        "metric": "CSR -> COO conversion GB/s (row_ptr read + row indices written / time), 1 GPU" if conv else
+                  ("CSR SpMV effective GB/s (algorithmic bytes / time), 1 GPU" if args.format == "csr"
                    else "%s SpMV effective GB/s (algorithmic bytes / time), 1 GPU" % args.format.upper())
                   if args.config != 5 else "CSR SpMM effective GB/s (algorithmic bytes / time), 1 GPU",
         "value": main_res["gbs"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -590,6 +604,8 @@ def main():
         "cpu_baseline": main_res.get("cpu_baseline"),
         "vendor_baseline": main_res.get("vendor_baseline"),
     }
+    if conv:
+        others["csr2ell"] = {k: v for k, v in conv["csr2ell"].items() if k != "timing"}
     if others:
         out["others"] = others
     print(json.dumps(out), flush=True)
