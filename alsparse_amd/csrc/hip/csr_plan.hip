@@ -484,12 +484,13 @@ static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* 
   return hipSuccess;
 }
 
-// Time the structural choice against the copies that were built (tiled, ELL) on
-// scratch vectors, keep the fastest and free the copies that lost.  A copy has
-// to win by a margin to be worth its memory.
+// Time the structural choice on scratch vectors, then the copies that the matrix is eligible for:
+// the ELL copy (cheap to build), and the tiled copy only if the fastest so far is slower than the
+// tiled pair could possibly be.  Keep the fastest and free the copies that lost.  A copy has to win
+// by a margin to be worth its memory.
 template <typename T>
 static hipError_t tune_copies(hipStream_t stream, asamd_csr_plan* p, const int* row_ptr,
-                              const int* col_ind, const T* val) {
+                              const int* col_ind, const T* val, bool tiled_ok, bool ell_ok) {
   asamd_csr_stats& st = p->st;
   T *x = nullptr, *y = nullptr;
   hipEvent_t e0 = nullptr, e1 = nullptr;
@@ -500,9 +501,7 @@ static hipError_t tune_copies(hipStream_t stream, asamd_csr_plan* p, const int* 
   if (e == hipSuccess) e = hipEventCreate(&e1);
   float best[3] = {0.f, 0.f, 0.f};
   const int algos[3] = {p->auto_algo, ASAMD_SPMV_TILED, ASAMD_SPMV_ELL};
-  const bool have[3] = {true, st.tiled_built != 0, st.ell_built != 0};
-  for (int a = 0; a < 3 && e == hipSuccess; ++a) {
-    if (!have[a]) continue;
+  auto time_algo = [&](int a) {
     st.algo = algos[a];
     int reps = 3;  // first run warms up; multiplies of a millisecond and more are timed once, shorter ones twice
     for (int rep = 0; rep < reps && e == hipSuccess; ++rep) {
@@ -515,6 +514,26 @@ static hipError_t tune_copies(hipStream_t stream, asamd_csr_plan* p, const int* 
       if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
       if (rep == 0 && ms > 1.0f) reps = 2;
       if (rep > 0 && (best[a] == 0.f || ms < best[a])) best[a] = ms;
+    }
+  };
+  if (e == hipSuccess) time_algo(0);
+  if (e == hipSuccess && ell_ok) {
+    e = build_ell<T>(stream, p, row_ptr, col_ind, val);
+    if (e == hipSuccess) time_algo(2);
+  }
+  if (e == hipSuccess && tiled_ok) {
+    // The tiled pair streams about twice the algorithmic bytes (16 instead of 8 bytes per fp32 entry), so
+    // it cannot finish before 2 * bytes / (the ~5 TB/s that streams reach).  A row kernel that is
+    // already that fast (banded matrices, whose gathers stay in the caches) makes the copy pointless:
+    // its layout pass (a sort of all entries) and its memory are saved.
+    const double bytes = (double)st.nnz * (4.0 + sizeof(T)) + ((double)st.m + 1) * 4.0 +
+                         ((double)st.n + (double)st.m) * sizeof(T);
+    const float tiled_floor_ms = (float)(2.0 * bytes / 5.0e9);
+    float fastest = best[0];
+    if (best[2] > 0.f && best[2] < fastest) fastest = best[2];
+    if (fastest > 1.1f * tiled_floor_ms) {
+      e = build_tiled<T>(stream, p, row_ptr, col_ind, val);
+      if (e == hipSuccess && st.tiled_built) time_algo(1);
     }
   }
   if (e0) (void)hipEventDestroy(e0);
@@ -623,11 +642,13 @@ static hipError_t plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t 
     e = by_dtype(dtype, [&](auto* tag) -> hipError_t {
       using T = std::remove_pointer_t<decltype(tag)>;
       hipError_t err = hipSuccess;
-      if (tiled_eligible<T>(p->st, force)) err = build_tiled<T>(stream, p, row_ptr, col_ind, (const T*)val);
-      if (err == hipSuccess && ell_eligible(p->st, force))
-        err = build_ell<T>(stream, p, row_ptr, col_ind, (const T*)val);
-      if (err == hipSuccess && !force && (p->st.tiled_built || p->st.ell_built))
-        err = tune_copies<T>(stream, p, row_ptr, col_ind, (const T*)val);
+      const bool tiled_ok = tiled_eligible<T>(p->st, force), ell_ok = ell_eligible(p->st, force);
+      if (force) {
+        if (tiled_ok) err = build_tiled<T>(stream, p, row_ptr, col_ind, (const T*)val);
+        if (err == hipSuccess && ell_ok) err = build_ell<T>(stream, p, row_ptr, col_ind, (const T*)val);
+      } else if (tiled_ok || ell_ok) {
+        err = tune_copies<T>(stream, p, row_ptr, col_ind, (const T*)val, tiled_ok, ell_ok);
+      }
       return err;
     });
     if (e == hipErrorOutOfMemory) {
