@@ -117,23 +117,23 @@ __global__ __launch_bounds__(kMergeThreads) void spmv_merge_kernel(
   }
   // ---- stream entries, gather x, stage products ----------------------------
   {
+    // Every load is issued unconditionally (a thread past the end of the range re-reads the range's
+    // first entry): loads under a branch make the compiler wait for ALL outstanding loads before
+    // each use, which turned the IPT gathers of a thread into a chain of IPT memory latencies.
     const T* __restrict__ xb = x - base;
+    const int64_t safe = nnz_cnt > 0 ? nnz_b : 0;
     T v[IPT];
     int c[IPT];
 #pragma unroll
     for (int s = 0; s < IPT; ++s) {
       const int k = tid + s * kMergeThreads;
-      if (k < nnz_cnt) {
-        v[s] = val[nnz_b + k];
-        c[s] = col_ind[nnz_b + k];
-      }
+      const int64_t kk = k < nnz_cnt ? nnz_b + k : safe;
+      v[s] = val[kk];
+      c[s] = col_ind[kk];
     }
     T xv[IPT];
 #pragma unroll
-    for (int s = 0; s < IPT; ++s) {
-      const int k = tid + s * kMergeThreads;
-      if (k < nnz_cnt) xv[s] = xb[c[s]];
-    }
+    for (int s = 0; s < IPT; ++s) xv[s] = xb[c[s]];
 #pragma unroll
     for (int s = 0; s < IPT; ++s) {
       const int k = tid + s * kMergeThreads;
