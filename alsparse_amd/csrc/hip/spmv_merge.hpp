@@ -128,8 +128,9 @@ __global__ __launch_bounds__(kMergeThreads) void spmv_merge_kernel(
     for (int s = 0; s < IPT; ++s) {
       const int k = tid + s * kMergeThreads;
       const int64_t kk = k < nnz_cnt ? nnz_b + k : safe;
-      v[s] = val[kk];
-      c[s] = col_ind[kk];
+      // the streams are touched once: non-temporal, so that they do not push x out of the caches
+      v[s] = nt_load(val + kk);
+      c[s] = nt_load(col_ind + kk);
     }
     T xv[IPT];
 #pragma unroll
