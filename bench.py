@@ -33,7 +33,7 @@ HBM_PEAK_GBS = 8000.0
 MEASURED_TRAFFIC_BYTES = {
     (3, "tiled two-phase"): 4.99e9,
     (3, "rowconst"): 34.6e9,
-    (4, "merge-path"): 3.43e9,
+    (4, "merge-path"): 3.32e9,
     (2, "ell copy"): 322.5e6,
     (5, "spmm row-major"): 9.27e9,
 }
