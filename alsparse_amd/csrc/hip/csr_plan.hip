@@ -503,7 +503,9 @@ static hipError_t tune_copies(hipStream_t stream, asamd_csr_plan* p, const int* 
   const int algos[3] = {p->auto_algo, ASAMD_SPMV_TILED, ASAMD_SPMV_ELL};
   auto time_algo = [&](int a) {
     st.algo = algos[a];
-    int reps = 3;  // first run warms up; multiplies of a millisecond and more are timed once, shorter ones twice
+    // first run warms up; multiplies of a millisecond and more are timed once, shorter ones twice; a
+    // first run of more than two milliseconds is its own measurement (cold caches are noise at that length)
+    int reps = 3;
     for (int rep = 0; rep < reps && e == hipSuccess; ++rep) {
       e = hipEventRecord(e0, stream);
       if (e == hipSuccess)
@@ -512,23 +514,31 @@ static hipError_t tune_copies(hipStream_t stream, asamd_csr_plan* p, const int* 
       if (e == hipSuccess) e = hipEventSynchronize(e1);
       float ms = 0.f;
       if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
-      if (rep == 0 && ms > 1.0f) reps = 2;
-      if (rep > 0 && (best[a] == 0.f || ms < best[a])) best[a] = ms;
+      if (rep == 0 && ms > 1.0f) reps = ms > 2.0f ? 1 : 2;
+      if ((rep > 0 || reps == 1) && (best[a] == 0.f || ms < best[a])) best[a] = ms;
     }
   };
+  // The tiled pair streams about twice the algorithmic bytes (16 instead of 8 bytes per fp32 entry), so
+  // it cannot finish before 2 * bytes / (the ~5 TB/s that streams reach).
+  const double bytes = (double)st.nnz * (4.0 + sizeof(T)) + ((double)st.m + 1) * 4.0 +
+                       ((double)st.n + (double)st.m) * sizeof(T);
+  const float tiled_floor_ms = (float)(2.0 * bytes / 5.0e9);
   if (e == hipSuccess) time_algo(0);
-  if (e == hipSuccess && ell_ok) {
-    e = build_ell<T>(stream, p, row_ptr, col_ind, val);
-    if (e == hipSuccess) time_algo(2);
-  }
+  // An ELL copy gathers x row by row like the kernel just timed; when that one is several times slower
+  // than the tiled floor the gathers are the problem and the ELL copy (as large as the matrix) is not
+  // worth building: the tiled copy is tried first, the ELL copy only if that does not win.
+  const bool ell_first = !(tiled_ok && best[0] > 2.5f * tiled_floor_ms);
+  auto try_ell = [&]() {
+    if (e == hipSuccess && ell_ok) {
+      e = build_ell<T>(stream, p, row_ptr, col_ind, val);
+      if (e == hipSuccess) time_algo(2);
+    }
+  };
+  if (ell_first) try_ell();
   if (e == hipSuccess && tiled_ok) {
-    // The tiled pair streams about twice the algorithmic bytes (16 instead of 8 bytes per fp32 entry), so
-    // it cannot finish before 2 * bytes / (the ~5 TB/s that streams reach).  A row kernel that is
-    // already that fast (banded matrices, whose gathers stay in the caches) makes the copy pointless:
-    // its layout pass (a sort of all entries) and its memory are saved.
-    const double bytes = (double)st.nnz * (4.0 + sizeof(T)) + ((double)st.m + 1) * 4.0 +
-                         ((double)st.n + (double)st.m) * sizeof(T);
-    const float tiled_floor_ms = (float)(2.0 * bytes / 5.0e9);
+    // A row kernel that is already as fast as the tiled floor (banded matrices, whose gathers stay in
+    // the caches) makes the tiled copy pointless: its layout pass (a sort of all entries) and its
+    // memory are saved.
     float fastest = best[0];
     if (best[2] > 0.f && best[2] < fastest) fastest = best[2];
     if (fastest > 1.1f * tiled_floor_ms) {
@@ -536,6 +546,7 @@ static hipError_t tune_copies(hipStream_t stream, asamd_csr_plan* p, const int* 
       if (e == hipSuccess && st.tiled_built) time_algo(1);
     }
   }
+  if (!ell_first && !(best[1] > 0.f && best[1] < 0.9f * best[0])) try_ell();
   if (e0) (void)hipEventDestroy(e0);
   if (e1) (void)hipEventDestroy(e1);
   if (x) (void)hipFree(x);
