@@ -83,6 +83,8 @@ __global__ __launch_bounds__(256) void copy_bytes_kernel(Int4* __restrict__ dst,
 struct asamd_csr_plan {
   asamd_csr_stats st;
   int auto_algo;
+  int struct_algo = ASAMD_SPMV_MERGE;   // the choice from the row statistics alone (no copy involved)
+  const void* copy_val_src = nullptr;   // the value array that the tiled / ELL copy was taken from
   int auto_width;
   int dtype;          // ASAMD_DTYPE_*: element type of the values
   int val_size;       // bytes per value
@@ -113,6 +115,7 @@ struct asamd_csr_plan {
     int* d_row_ptr;           // n + 1
     int* d_col;               // nnz zero-based rows of A
     void* d_val;              // nnz values (conjugated in copy [1])
+    const void* val_src;      // the value array that d_val was gathered from
   } tr[2];
   bool lazy_transpose;        // build a copy on the first transposed multiply
 };
@@ -189,6 +192,7 @@ static void choose_algo(asamd_csr_plan* p) {
   } else {
     p->auto_algo = ASAMD_SPMV_MERGE;
   }
+  p->struct_algo = p->auto_algo;
   st.algo = p->auto_algo;
   st.vector_width = p->auto_width;
 }
@@ -230,7 +234,7 @@ static void free_transpose(asamd_csr_plan* p, int which) {
   if (t.d_row_ptr) (void)hipFree(t.d_row_ptr);
   if (t.d_col) (void)hipFree(t.d_col);
   if (t.d_val) (void)hipFree(t.d_val);
-  t = asamd_csr_plan::TransCopy{nullptr, nullptr, nullptr, nullptr};
+  t = asamd_csr_plan::TransCopy{nullptr, nullptr, nullptr, nullptr, nullptr};
   p->st.transpose_built &= ~(1 << which);
 }
 
@@ -567,6 +571,7 @@ static hipError_t tune_copies(hipStream_t stream, asamd_csr_plan* p, const int* 
   if (pick != 0) {
     p->auto_algo = algos[pick];
     st.algo = algos[pick];
+    p->copy_val_src = val;
   }
   return hipSuccess;
 }
@@ -657,6 +662,7 @@ static hipError_t plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t 
       if (force) {
         if (tiled_ok) err = build_tiled<T>(stream, p, row_ptr, col_ind, (const T*)val);
         if (err == hipSuccess && ell_ok) err = build_ell<T>(stream, p, row_ptr, col_ind, (const T*)val);
+        p->copy_val_src = val;
       } else if (tiled_ok || ell_ok) {
         err = tune_copies<T>(stream, p, row_ptr, col_ind, (const T*)val, tiled_ok, ell_ok);
       }
@@ -756,6 +762,7 @@ static hipError_t build_transpose(hipStream_t stream, asamd_csr_plan* p, const i
     free_transpose(p, which);
     return e;
   }
+  t.val_src = val;
   st.transpose_built |= 1 << which;
   return hipSuccess;
 }
@@ -867,6 +874,12 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
   if (((uintptr_t)val | (uintptr_t)x | (uintptr_t)y) % alignof(T)) return hipErrorInvalidValue;
   const asamd_csr_stats& st = p->st;
   int algo = st.algo;
+  // The tiled and ELL copies hold the values of the array they were built from.  A multiply that
+  // brings another value array (same structure, new numbers) must not see the old ones: it runs
+  // the kernel that the row statistics alone would pick.  (Values changed IN PLACE cannot be seen
+  // from here: that needs a new analysis.)
+  if ((algo == ASAMD_SPMV_TILED || algo == ASAMD_SPMV_ELL) && p->copy_val_src && val != p->copy_val_src)
+    algo = p->struct_algo;
   if (!kIsReal<T> && algo == ASAMD_SPMV_ROWCONST) algo = ASAMD_SPMV_VECTOR;
   if (algo == ASAMD_SPMV_ROWCONST) {
     // 128-bit loads need 16-byte aligned streams; fall back otherwise
@@ -1006,7 +1019,9 @@ static int csrmv_trans_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* 
       return e;
     }
   }
-  if (t.plan) return csrmv_impl<T>(s, t.plan, alpha, (const T*)t.d_val, t.d_row_ptr, t.d_col, x, beta, y);
+  // the copy holds the values it was gathered from: another value array takes the scatter route below
+  if (t.plan && val == t.val_src)
+    return csrmv_impl<T>(s, t.plan, alpha, (const T*)t.d_val, t.d_row_ptr, t.d_col, x, beta, y);
   if (beta != T(1)) scale_vec_kernel<T><<<(unsigned)(((int64_t)st.n + 255) / 256), 256, 0, s>>>(st.n, beta, y);
   if constexpr (!kIsReal<T>) {
     if (which == 1) {

@@ -3,14 +3,14 @@
 Tolerance (north star): per row |y - y_ref| / (|alpha| * sum_j |a_ij x_j|)
 <= 1e-4 for fp32 and <= 1e-12 for fp64; rows with a zero denominator must match
 exactly."""
-from ctypes import byref, c_void_p
+from ctypes import byref, c_float, c_void_p
 
 import numpy as np
 import pytest
 
 from alsparse_amd import capi, hiprt, workloads as wl
 from oracle import oracle as orc
-from helpers import (ALGOS, DeviceCsr, announce, check_spmv, csr_from_lengths, plan_stats, run_csrmv,
+from helpers import (ALGOS, TOL, DeviceCsr, announce, check_spmv, csr_from_lengths, plan_stats, run_csrmv,
                      run_plan_csrmv)
 
 pytestmark = pytest.mark.gpu
@@ -330,3 +330,37 @@ def test_unsorted_and_duplicate_columns_and_non_finite_values(gpu, dtype):
             assert np.isnan(ref[9]) and np.isnan(ref[11]) and np.isinf(ref[7]) and finite.sum() >= m - 300
     finally:
         db.free()
+
+
+@pytest.mark.parametrize("algo", ["tiled", "ell"])
+def test_copy_is_not_used_for_another_value_array(gpu, algo):
+    """The tiled and ELL copies hold the values they were built from.  A multiply that passes a different
+    value array (same structure, new numbers) must be computed from the new numbers."""
+    from ctypes import c_void_p
+    lib = capi.load()
+    a = wl.uniform_rows(6000, 5000, 8, np.float32)
+    x, y0 = wl.uniform(a.cols, a.dtype, 3), wl.uniform(a.rows, a.dtype, 4)
+    da = DeviceCsr(a)
+    new_vals = (a.values * np.float32(-3.0) + np.float32(0.25)).astype(np.float32)
+    b = wl.Csr(a.rows, a.cols, a.row_ptr, a.col_ind, new_vals, a.base, "new values")
+    d_new = hiprt.DeviceArray.from_numpy(new_vals)
+    plan = c_void_p()
+    try:
+        assert lib.asamd_csr_plan_create(None, a.rows, a.cols, a.nnz, da.row_ptr.c_ptr(), da.col.c_ptr(), da.val.c_ptr(),
+                                         a.base, 4, 2, byref(plan)) == 0
+        assert lib.asamd_csr_plan_set_algo(plan, ALGOS[algo]) == 0
+        for vals, mat in ((da.val, a), (d_new, b), (da.val, a)):
+            announce("value array", algo, mat.name)
+            dx, dy = hiprt.DeviceArray.from_numpy(x), hiprt.DeviceArray.from_numpy(y0)
+            assert lib.asamd_s_csrmv(None, plan, c_float(1.5), vals.c_ptr(), da.row_ptr.c_ptr(), da.col.c_ptr(),
+                                     dx.c_ptr(), c_float(0.5), dy.c_ptr()) == 0
+            hiprt.synchronize()
+            y = dy.to_numpy()
+            dx.free()
+            dy.free()
+            err = orc.csrmv_err(mat, 1.5, x, 0.5, y0, y, orc.csrmv_plain(mat, 1.5, x, 0.5, y0))
+            assert err.full <= TOL[a.dtype] and err.zero_den_mismatch == 0, (mat.name, err)
+    finally:
+        lib.asamd_csr_plan_destroy(plan)
+        da.free()
+        d_new.free()

@@ -88,6 +88,17 @@ def test_transposed_csrmv_scatter_and_analysed(gpu, shape, dtype):
             runs.append(y)
         # the copy of A^T is multiplied by the ordinary kernels: reproducible
         assert np.array_equal(runs[1], run_csrmv_trans(gpu, da, 2.0, x, 3.0, y0, info))
+        # another value array on the analysed structure: the copy holds the old values and must not be used
+        b = wl.Csr(a.rows, a.cols, a.row_ptr, a.col_ind, (a.values * dtype(-2.0)).astype(dtype), a.base, "new values")
+        old_val = da.val
+        da.a, da.val = b, hiprt.DeviceArray.from_numpy(b.values)
+        try:
+            announce("csrmv trans analysed, other value array", shape, np.dtype(dtype).name)
+            y = run_csrmv_trans(gpu, da, 2.0, x, 3.0, y0, info)
+            check_trans(b, 2.0, x, 3.0, y0, y, "%s other values" % shape)
+        finally:
+            da.val.free()
+            da.a, da.val = a, old_val
     finally:
         lib.alphasparse_dcu_destroy_mat_info(info)
         da.free()
