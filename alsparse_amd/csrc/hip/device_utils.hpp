@@ -258,6 +258,28 @@ __device__ __forceinline__ T group_sum(T v) {
   return v;
 }
 
+// ---- buffer loads with the hardware's range check ------------------------------
+// A raw buffer resource over [p, p + bytes): loads at byte offsets >= bytes return zero and touch
+// no memory.  0x00020000 is the 32-bit data format word of gfx9 resources.
+using BufferRsrc = __amdgpu_buffer_rsrc_t;
+__device__ __forceinline__ BufferRsrc make_rsrc(const void* p, int bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
+}
+__device__ __forceinline__ int buffer_load_u16(BufferRsrc r, int byte_offset) {
+  return (int)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(r, byte_offset, 0, 0);
+}
+template <typename T>
+__device__ __forceinline__ T buffer_load(BufferRsrc r, int byte_offset) {
+  if constexpr (sizeof(T) == 4) {
+    return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b32(r, byte_offset, 0, 0));
+  } else if constexpr (sizeof(T) == 8) {
+    return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b64(r, byte_offset, 0, 0));
+  } else {
+    static_assert(sizeof(T) == 16, "element size");
+    return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b128(r, byte_offset, 0, 0));
+  }
+}
+
 // ---- 128-bit streaming loads ------------------------------------------------
 struct alignas(16) Int4 { int x, y, z, w; };
 struct alignas(16) Float4 { float x, y, z, w; };

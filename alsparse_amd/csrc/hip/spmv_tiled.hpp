@@ -404,33 +404,30 @@ __global__ __launch_bounds__(TileDims<T>::red_threads) void tiled_reduce_kernel(
   // the tile ranges of a group are loaded while the group before it is worked on
   TileRange tr = load_ranges(0);
   TileRange tr_next = load_ranges(1);
+  // Buffer loads: the tile's two streams are described by resource words in scalar registers (base =
+  // the tile's first entry, extent = the tile), the lane supplies a constant byte offset, and a
+  // lane past the end of the tile gets zero from the hardware's range check without touching
+  // memory: no address arithmetic and no masks in vector instructions.
+  const int off_v = lane * (int)sizeof(T), off_r = lane * 2;
   auto issue = [&](int s, int ti) {  // tile ti (wave-uniform) -> slot s
     const int src = ti & (kWave - 1);
-    int b0 = __builtin_amdgcn_readlane(tr.begin, src);
+    const int b0 = __builtin_amdgcn_readlane(tr.begin, src);
     const int e0 = __builtin_amdgcn_readlane(tr.end, src);
     const int len = ti < col_blocks ? e0 - b0 : 0;
-    if (len == 0) b0 = 0;  // keeps the addresses below inside the arrays
     slen[s] = len;
-    // scalar base per tile, the lane as the only vector part of the address
-    const T* pv = prod + b0;
-    const unsigned short* pr = t_row + b0;
-    const int i0 = lane < len ? lane : 0;
-    const int i1 = lane + kWave < len ? lane + kWave : 0;
-    sv[s][0] = pv[i0];
-    sr[s][0] = pr[i0];
-    sv[s][1] = pv[i1];
-    sr[s][1] = pr[i1];
+    const BufferRsrc rv = make_rsrc(prod + b0, len * (int)sizeof(T));
+    const BufferRsrc rr = make_rsrc(t_row + b0, len * 2);
+    sv[s][0] = buffer_load<T>(rv, off_v);
+    sr[s][0] = buffer_load_u16(rr, off_r);
+    sv[s][1] = buffer_load<T>(rv, off_v + kWave * (int)sizeof(T));
+    sr[s][1] = buffer_load_u16(rr, off_r + kWave * 2);
   };
   auto consume = [&](int s) {
     const int len = slen[s];
-    {
-      const bool ok = lane < len;
-      add_rows<false, true>(acc, ok ? sr[s][0] : r_none, ok ? sv[s][0] : T(0), true);
-    }
-    if (len > kWave) {  // wave-uniform
-      const bool ok = lane + kWave < len;
-      add_rows<false, true>(acc, ok ? sr[s][1] : r_none, ok ? sv[s][1] : T(0), true);
-    }
+    // a lane without an entry holds value zero already; its row becomes the lane's dummy row
+    add_rows<false, true>(acc, lane < len ? sr[s][0] : r_none, sv[s][0], true);
+    if (len > kWave)  // wave-uniform
+      add_rows<false, true>(acc, lane + kWave < len ? sr[s][1] : r_none, sv[s][1], true);
   };
 #pragma unroll
   for (int s = 0; s < kSlots; ++s) {
