@@ -31,7 +31,7 @@ HBM_PEAK_GBS = 8000.0
 # 1 GiB copy kernel); the summaries these come from are profiles/spmv_tiled_C3.txt, spmv_merge_C4.txt,
 # spmv_ell_copy_C2.txt and spmm_rowmajor_C5.txt.  Keyed by (configuration, kernel family); anything else reports null.
 MEASURED_TRAFFIC_BYTES = {
-    (3, "tiled two-phase"): 4.99e9,
+    (3, "tiled two-phase"): 5.00e9,
     (3, "rowconst"): 34.6e9,
     (4, "merge-path"): 3.32e9,
     (2, "ell copy"): 322.5e6,
