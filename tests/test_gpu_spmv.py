@@ -364,3 +364,36 @@ def test_copy_is_not_used_for_another_value_array(gpu, algo):
         lib.asamd_csr_plan_destroy(plan)
         da.free()
         d_new.free()
+
+
+def test_analysis_choices(gpu):
+    """What the analysis decides and what it skips: a banded matrix keeps the ELL copy and never lays out
+    the tiled one (its floor is slower than the ELL kernel measured); a matrix small enough to be
+    launch-bound takes the single-kernel path however skewed its rows are."""
+    lib = capi.load()
+    a, x, y0, alpha, beta, _ = wl.config(2)
+    da = DeviceCsr(a)
+    info = capi.alphasparse_dcu_mat_info_t()
+    assert lib.alphasparse_dcu_create_mat_info(byref(info)) == 0
+    descr = capi.make_descr(base=a.base)
+    try:
+        announce("analysis choices", a.name)
+        assert lib.alphasparse_dcu_d_csrmv_analysis(gpu.h, 0, a.rows, a.cols, a.nnz, byref(descr), da.val.c_ptr(),
+                                                    da.row_ptr.c_ptr(), da.col.c_ptr(), info) == 0
+        st = lib.asamd_analysis_stats(info).contents
+        assert st.algo == capi.ASAMD_SPMV_ELL and st.ell_built == 1 and st.tiled_built == 0
+        assert st.tune_ms_ell > 0 and st.tune_ms_base > 0 and st.tune_ms_tiled == 0
+        check_spmv(a, alpha, x, beta, y0, run_csrmv(gpu, da, alpha, x, beta, y0, info), "config 2 analysed")
+    finally:
+        lib.alphasparse_dcu_destroy_mat_info(info)
+        da.free()
+    b = csr_from_lengths([0, 1, 700, 3, 0, 2, 2, 9] * 40, 5000, np.float32)
+    db = DeviceCsr(b)
+    try:
+        xb, yb = wl.uniform(b.cols, b.dtype, 3), wl.uniform(b.rows, b.dtype, 4)
+        announce("analysis choices", b.name)
+        check_spmv(b, 1.0, xb, 0.0, yb, run_csrmv(gpu, db, 1.0, xb, 0.0, yb), "small skewed, lazy")
+        st = lib.asamd_analysis_stats(db.row_ptr.c_ptr()).contents
+        assert st.algo == capi.ASAMD_SPMV_VECTOR, capi.ALGO_NAMES[st.algo]
+    finally:
+        db.free()
