@@ -393,8 +393,11 @@ static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* 
   if (e == hipSuccess) e = hipMalloc(&d_coo, nnz * sizeof(int));
   if (e == hipSuccess) e = hipMalloc(&d_key, nnz * sizeof(unsigned));
   if (e == hipSuccess) e = hipMalloc(&d_key2, nnz * sizeof(unsigned));
-  if (e == hipSuccess) e = hipMalloc(&d_idx, nnz * sizeof(unsigned));
-  if (e == hipSuccess) e = hipMalloc(&d_perm, nnz * sizeof(unsigned));
+  // 4-byte values are sorted together with their keys (64-bit payloads); wider ones through a permutation
+  constexpr bool kPayloadSort = sizeof(T) == 4;
+  constexpr size_t kSortValBytes = kPayloadSort ? sizeof(unsigned long long) : sizeof(unsigned);
+  if (e == hipSuccess) e = hipMalloc(&d_idx, nnz * kSortValBytes);
+  if (e == hipSuccess) e = hipMalloc(&d_perm, nnz * kSortValBytes);
   if (e == hipSuccess) e = hipMalloc(&d_tile_ptr, (size_t)(tiles + 1) * sizeof(int));
   if (e == hipSuccess) e = hipMalloc(&p->d_ranges, (size_t)tiles * sizeof(TileRange));
   const size_t long_cap = nnz / kLongTile + 1;  // a long tile holds more than kLongTile entries
@@ -408,13 +411,24 @@ static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* 
   if (e == hipSuccess)
     e = (hipError_t)asamd_csr2coo_ws(stream, row_ptr, st.nnz, st.m, d_coo, st.base, d_key2, (size_t)nnz * sizeof(unsigned));
   if (e == hipSuccess) {
-    tile_keys_kernel<<<256 * 32, 256, 0, stream>>>(st.nnz, d_coo, col_ind, st.base, d_cgb, d_rgb, rb, d_key, d_idx);
-    e = sort_pairs_u32(stream, d_key, d_key2, d_idx, d_perm, nnz, key_bits);
+    if constexpr (kPayloadSort) {
+      tile_keys_payload_kernel<<<256 * 32, 256, 0, stream>>>(st.nnz, d_coo, col_ind, (const unsigned*)val, st.base, d_cgb,
+                                                             d_cbs, d_rgb, p->d_row_block_start, rb, d_key,
+                                                             (unsigned long long*)d_idx);
+      e = sort_pairs_u32_u64(stream, d_key, d_key2, (unsigned long long*)d_idx, (unsigned long long*)d_perm, nnz, key_bits);
+    } else {
+      tile_keys_kernel<<<256 * 32, 256, 0, stream>>>(st.nnz, d_coo, col_ind, st.base, d_cgb, d_rgb, rb, d_key, d_idx);
+      e = sort_pairs_u32(stream, d_key, d_key2, d_idx, d_perm, nnz, key_bits);
+    }
   }
   if (e == hipSuccess) {
-    tile_gather_kernel<T><<<256 * 32, 256, 0, stream>>>(st.nnz, d_perm, d_coo, col_ind, val, st.base, d_cgb, d_cbs,
-                                                        d_rgb, p->d_row_block_start, (T*)p->d_tval,
-                                                        p->d_tcol, p->d_trow);
+    if constexpr (kPayloadSort)
+      tile_unpack_kernel<<<256 * 32, 256, 0, stream>>>(st.nnz, (const unsigned long long*)d_perm, (unsigned*)p->d_tval,
+                                                       p->d_tcol, p->d_trow);
+    else
+      tile_gather_kernel<T><<<256 * 32, 256, 0, stream>>>(st.nnz, d_perm, d_coo, col_ind, val, st.base, d_cgb, d_cbs,
+                                                          d_rgb, p->d_row_block_start, (T*)p->d_tval,
+                                                          p->d_tcol, p->d_trow);
     tile_bounds_kernel<<<(unsigned)((tiles + 1 + 255) / 256), 256, 0, stream>>>(st.nnz, d_key2, tiles,
                                                                                 d_tile_ptr);
     e = hipMemsetAsync(d_long_count, 0, sizeof(int), stream);

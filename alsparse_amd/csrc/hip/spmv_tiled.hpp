@@ -146,6 +146,39 @@ __global__ __launch_bounds__(256) void tile_keys_kernel(int nnz, const int* __re
   }
 }
 
+// For 4-byte values the entry itself travels with its key through the sort: payload = value bits
+// (high word) | column local to its block << 16 | row local to its block.  Gathering the three CSR
+// streams through the sorted permutation afterwards moves a 128-byte line per entry and stream
+// (18 ms for 2^28 entries, against 3 ms more in the sort and a streaming unpack).
+__global__ __launch_bounds__(256) void tile_keys_payload_kernel(
+    int nnz, const int* __restrict__ coo_row, const int* __restrict__ col_ind, const unsigned* __restrict__ val_bits,
+    int base, const int* __restrict__ col_group_block, const int* __restrict__ col_block_start,
+    const int* __restrict__ row_group_block, const int* __restrict__ row_block_start, int row_blocks,
+    unsigned* __restrict__ key, unsigned long long* __restrict__ payload) {
+  for (int64_t k = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; k < nnz;
+       k += (int64_t)gridDim.x * blockDim.x) {
+    const int col = col_ind[k] - base, row = coo_row[k] - base;
+    const unsigned cb = (unsigned)col_group_block[col >> kColGroupLog2];
+    const unsigned rb = (unsigned)row_group_block[row >> kRowGroupLog2];
+    key[k] = cb * (unsigned)row_blocks + rb;
+    const unsigned lc = (unsigned)(col - col_block_start[cb]), lr = (unsigned)(row - row_block_start[rb]);
+    payload[k] = ((unsigned long long)val_bits[k] << 32) | (lc << 16) | lr;
+  }
+}
+
+__global__ __launch_bounds__(256) void tile_unpack_kernel(int nnz, const unsigned long long* __restrict__ payload,
+                                                          unsigned* __restrict__ t_val_bits,
+                                                          unsigned short* __restrict__ t_col,
+                                                          unsigned short* __restrict__ t_row) {
+  for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < nnz;
+       q += (int64_t)gridDim.x * blockDim.x) {
+    const unsigned long long w = payload[q];
+    t_val_bits[q] = (unsigned)(w >> 32);
+    t_col[q] = (unsigned short)(w >> 16);
+    t_row[q] = (unsigned short)w;
+  }
+}
+
 // Entries in sorted order: values, columns and rows local to their blocks.
 template <typename T>
 __global__ __launch_bounds__(256) void tile_gather_kernel(
