@@ -540,7 +540,11 @@ static hipError_t tune_copies(hipStream_t stream, asamd_csr_plan* p, const int* 
   // it cannot finish before 2 * bytes / (the ~5 TB/s that streams reach).
   const double bytes = (double)st.nnz * (4.0 + sizeof(T)) + ((double)st.m + 1) * 4.0 +
                        ((double)st.n + (double)st.m) * sizeof(T);
-  const float tiled_floor_ms = (float)(2.0 * bytes / 5.0e9);
+  float tiled_floor_ms = (float)(2.0 * bytes / 5.0e9);
+  // Heavy-tailed rows (power-law graphs) make uneven tiles: the in-wave combining of equal rows and the
+  // long-tile phase then cost the tiled pair about 2.5 times its floor (measured 0.8-0.9 ms against 0.34 ms
+  // on an 8 M-row R-MAT matrix whose longest row has 200 000 entries).
+  if ((double)st.max_len > 32.0 * ((double)st.nnz / (double)st.m) + 256.0) tiled_floor_ms *= 2.5f;
   if (e == hipSuccess) time_algo(0);
   // An ELL copy gathers x row by row like the kernel just timed; when that one is several times slower
   // than the tiled floor the gathers are the problem and the ELL copy (as large as the matrix) is not
