@@ -417,8 +417,9 @@ __global__ __launch_bounds__(TileDims<T>::red_threads) void tiled_reduce_kernel(
   // per lane.  The wave keeps kSlots tiles in flight in a ring of registers: step s adds the tile in slot s
   // and at once loads the tile kSlots further on into it, so the loads of the next kSlots - 1 tiles are
   // outstanding while one tile goes through its LDS read-modify-writes.  For the hardware counter of
-  // outstanding loads to allow that, every load is issued unconditionally (lanes past the end of a
-  // tile re-read its first entry and are masked when the slot is used).  The waves of a workgroup
+  // outstanding loads to allow that, every load is issued unconditionally (the compiler can only
+  // wait for "all but the N newest" when N is certain; lanes past the end of a tile are cut off by
+  // the buffer range check and masked when the slot is used).  The waves of a workgroup
   // share no data and meet at no barrier: with one batch of 8 tiles in flight a barrier per batch kept
   // their reads on neighbouring tiles and doubled the speed, with the ring it measured no different.
   constexpr int kSlots = TileDims<T>::red_slots;
