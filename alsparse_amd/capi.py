@@ -128,6 +128,7 @@ class asamd_csr_stats(Structure):
                 ("tile_col_blocks", c_int32), ("tile_row_blocks", c_int32),
                 ("tune_ms_base", c_float), ("tune_ms_tiled", c_float), ("tune_ms_ell", c_float),
                 ("ell_built", c_int32), ("ell_width", c_int32), ("transpose_built", c_int32),
+                ("tile_entries_per_lane", c_int32),
                 ("hist", ctypes.c_int64 * ASAMD_HIST_BINS)]
 
 

@@ -217,7 +217,7 @@ extern "C" int asamd_csr2ell_width(hipStream_t stream, int32_t m, const int32_t*
   if (e != hipSuccess) return e;
   zero_int_kernel<<<1, 1, 0, stream>>>(d);
   // every workgroup ends with one atomic on the same word: few, long-running workgroups
-  int grid = (m + 256 * 8 - 1) / (256 * 8);
+  int grid = (int)(((int64_t)m + 256 * 8 - 1) / (256 * 8));
   if (grid > 1024) grid = 1024;
   max_row_len_kernel<<<grid, 256, 0, stream>>>(m, row_ptr, d);
   e = hipMemcpyAsync(width_host, d, sizeof(int), hipMemcpyDeviceToHost, stream);

@@ -100,6 +100,7 @@ struct asamd_csr_plan {
   TileRange* d_ranges;        // row_blocks * col_blocks tile ranges, row block major
   LongChunk* d_long;          // phase-3 work list: chunks of the tiles too long for phase 2
   int n_long_chunks;
+  int tiled_halves;           // entries per lane and tile in phase 2: 2, or 1 where (nearly) all tiles are short
   void* d_tval;               // nnz values in tile order
   unsigned short* d_tcol;     // nnz local columns
   unsigned short* d_trow;     // nnz local rows
@@ -208,6 +209,7 @@ static void free_tiled(asamd_csr_plan* p) {
   if (p->d_long) (void)hipFree(p->d_long);
   p->d_long = nullptr;
   p->n_long_chunks = 0;
+  p->tiled_halves = 2;
   if (p->d_tval) (void)hipFree(p->d_tval);
   if (p->d_tcol) (void)hipFree(p->d_tcol);
   if (p->d_trow) (void)hipFree(p->d_trow);
@@ -218,6 +220,7 @@ static void free_tiled(asamd_csr_plan* p) {
   p->d_tcol = p->d_trow = nullptr;
   p->d_chunks = nullptr;
   p->st.tiled_built = 0;
+  p->st.tile_entries_per_lane = 0;
 }
 
 static void free_ell(asamd_csr_plan* p) {
@@ -322,6 +325,10 @@ static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* 
   const int row_groups = (int)(((int64_t)st.m + (1 << kRowGroupLog2) - 1) >> kRowGroupLog2);
 
   int *d_coo = nullptr, *d_tile_ptr = nullptr, *d_long_count = nullptr, *d_cnt = nullptr;
+  unsigned long long* d_mid = nullptr;
+  // share of the entries that may sit in tiles of 65..128 entries for phase 2 to run one entry per lane
+  // (every such tile then costs a phase-3 workgroup of its own)
+  constexpr double kMidShare = 0.01;
   int *d_cgb = nullptr, *d_rgb = nullptr, *d_cbs = nullptr;
   LongTile* d_long_raw = nullptr;
   unsigned *d_key = nullptr, *d_key2 = nullptr, *d_idx = nullptr, *d_perm = nullptr;
@@ -400,9 +407,10 @@ static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* 
   if (e == hipSuccess) e = hipMalloc(&d_perm, nnz * kSortValBytes);
   if (e == hipSuccess) e = hipMalloc(&d_tile_ptr, (size_t)(tiles + 1) * sizeof(int));
   if (e == hipSuccess) e = hipMalloc(&p->d_ranges, (size_t)tiles * sizeof(TileRange));
-  const size_t long_cap = nnz / kLongTile + 1;  // a long tile holds more than kLongTile entries
+  const size_t long_cap = nnz / kWave + 1;  // a long tile holds more than kWave entries, at the least
   if (e == hipSuccess) e = hipMalloc(&d_long_raw, long_cap * sizeof(LongTile));
   if (e == hipSuccess) e = hipMalloc(&d_long_count, sizeof(int));
+  if (e == hipSuccess) e = hipMalloc(&d_mid, sizeof(unsigned long long));
   if (e == hipSuccess) e = hipMalloc(&p->d_tval, nnz * sizeof(T));
   if (e == hipSuccess) e = hipMalloc(&p->d_tcol, nnz * sizeof(unsigned short));
   if (e == hipSuccess) e = hipMalloc(&p->d_trow, nnz * sizeof(unsigned short));
@@ -431,9 +439,22 @@ static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* 
                                                           p->d_tcol, p->d_trow);
     tile_bounds_kernel<<<(unsigned)((tiles + 1 + 255) / 256), 256, 0, stream>>>(st.nnz, d_key2, tiles,
                                                                                 d_tile_ptr);
-    e = hipMemsetAsync(d_long_count, 0, sizeof(int), stream);
-    tile_ranges_kernel<<<(unsigned)((tiles + 255) / 256), 256, 0, stream>>>(rb, cb, d_tile_ptr, p->d_ranges,
-                                                                            d_long_raw, d_long_count);
+    // Entries in tiles of 65..128 entries: if they are few, phase 2 runs in its one-entry-per-lane form
+    // (twice the tiles in flight) and leaves those tiles to phase 3.
+    e = hipMemsetAsync(d_mid, 0, sizeof(unsigned long long), stream);
+    tile_mid_entries_kernel<<<1024, 256, 0, stream>>>(tiles, d_tile_ptr, d_mid);
+    unsigned long long h_mid = 0;
+    if (e == hipSuccess) e = hipMemcpyAsync(&h_mid, d_mid, sizeof(h_mid), hipMemcpyDeviceToHost, stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(stream);
+    p->tiled_halves = (double)h_mid <= kMidShare * (double)st.nnz ? 1 : 2;
+    if (const char* ev = getenv("ALSPARSE_AMD_TILED_HALVES")) {
+      const int v = atoi(ev);
+      if (v == 1 || v == 2) p->tiled_halves = v;
+    }
+    p->st.tile_entries_per_lane = p->tiled_halves;
+    if (e == hipSuccess) e = hipMemsetAsync(d_long_count, 0, sizeof(int), stream);
+    tile_ranges_kernel<<<(unsigned)((tiles + 255) / 256), 256, 0, stream>>>(
+        rb, cb, p->tiled_halves * kWave, d_tile_ptr, p->d_ranges, d_long_raw, d_long_count);
     h_colptr.resize((size_t)cb + 1);
   }
   if (e == hipSuccess)  // column block c starts at tile_ptr[c * rb]
@@ -489,10 +510,13 @@ static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* 
     e = hipFuncSetAttribute((const void*)tiled_products_kernel<T>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, kTileBytes);
   if (e == hipSuccess)
-    e = hipFuncSetAttribute((const void*)tiled_reduce_kernel<T>,
+    e = hipFuncSetAttribute((const void*)tiled_reduce_kernel<T, 1>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, TileDims<T>::red_lds_bytes);
+  if (e == hipSuccess)
+    e = hipFuncSetAttribute((const void*)tiled_reduce_kernel<T, 2>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, TileDims<T>::red_lds_bytes);
   for (void* d : {(void*)d_coo, (void*)d_key, (void*)d_key2, (void*)d_idx, (void*)d_perm, (void*)d_tile_ptr,
-                  (void*)d_long_raw, (void*)d_long_count, (void*)d_cnt, (void*)d_cgb, (void*)d_rgb, (void*)d_cbs})
+                  (void*)d_long_raw, (void*)d_long_count, (void*)d_mid, (void*)d_cnt, (void*)d_cgb, (void*)d_rgb, (void*)d_cbs})
     if (d) (void)hipFree(d);
   if (e != hipSuccess) {
     free_tiled(p);
@@ -619,9 +643,9 @@ static hipError_t plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t 
     return e;
   }
   stats_init_kernel<<<1, 64, 0, stream>>>(d_stats);
-  int grid = (m + 255) / 256;
+  int64_t grid = ((int64_t)m + 255) / 256;
   if (grid > 256 * 16) grid = 256 * 16;
-  row_stats_kernel<<<grid, 256, 0, stream>>>(m, row_ptr, d_stats);
+  row_stats_kernel<<<(unsigned)grid, 256, 0, stream>>>(m, row_ptr, d_stats);
   int h[kStatWords];
   e = hipMemcpyAsync(h, d_stats, sizeof(h), hipMemcpyDeviceToHost, stream);
   if (e == hipSuccess) e = hipStreamSynchronize(stream);
@@ -751,9 +775,9 @@ static hipError_t build_transpose(hipStream_t stream, asamd_csr_plan* p, const i
   if (e == hipSuccess)  // d_key2 is free until the sort
     e = (hipError_t)asamd_csr2coo_ws(stream, row_ptr, nnz, st.m, d_coo, st.base, d_key2, (size_t)nnz * sizeof(unsigned));
   if (e == hipSuccess) {
-    int grid = (nnz + 255) / 256;
+    int64_t grid = ((int64_t)nnz + 255) / 256;
     if (grid > 256 * 32) grid = 256 * 32;
-    transpose_keys_kernel<<<grid, 256, 0, stream>>>(nnz, col_ind, st.base, d_key, d_idx);
+    transpose_keys_kernel<<<(unsigned)grid, 256, 0, stream>>>(nnz, col_ind, st.base, d_key, d_idx);
     e = hipGetLastError();
     unsigned bits = 1;
     while (bits < 32 && ((int64_t)1 << bits) < (int64_t)n) ++bits;
@@ -920,10 +944,15 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
       if (p->n_chunks > 0)
         tiled_products_kernel<T><<<p->n_chunks, kProdThreads, kTileBytes, s>>>(
             p->d_chunks, (const T*)p->d_tval, p->d_tcol, x, (T*)p->d_tprod);
-      tiled_reduce_kernel<T><<<(st.tile_row_blocks + TileDims<T>::red_waves - 1) / TileDims<T>::red_waves, TileDims<T>::red_threads,
-                               TileDims<T>::red_lds_bytes, s>>>(
-          st.m, st.tile_row_blocks, st.tile_col_blocks, p->d_row_block_start, p->d_ranges, p->d_trow,
-          (const T*)p->d_tprod, alpha, beta, y);
+      const unsigned red_grid = (unsigned)((st.tile_row_blocks + TileDims<T>::red_waves - 1) / TileDims<T>::red_waves);
+      if (p->tiled_halves == 1)
+        tiled_reduce_kernel<T, 1><<<red_grid, TileDims<T>::red_threads, TileDims<T>::red_lds_bytes, s>>>(
+            st.m, st.tile_row_blocks, st.tile_col_blocks, p->d_row_block_start, p->d_ranges, p->d_trow,
+            (const T*)p->d_tprod, alpha, beta, y);
+      else
+        tiled_reduce_kernel<T, 2><<<red_grid, TileDims<T>::red_threads, TileDims<T>::red_lds_bytes, s>>>(
+            st.m, st.tile_row_blocks, st.tile_col_blocks, p->d_row_block_start, p->d_ranges, p->d_trow,
+            (const T*)p->d_tprod, alpha, beta, y);
       if (p->n_long_chunks > 0)
         tiled_long_kernel<T><<<p->n_long_chunks, kLongThreads, 0, s>>>(p->d_long, p->d_trow,
                                                                        (const T*)p->d_tprod, alpha, y);

@@ -31,7 +31,7 @@ namespace {
 // y <- beta * y ahead of an accumulating kernel (beta == 0 stores zeros without reading)
 template <typename T>
 __global__ __launch_bounds__(256) void scale_y_kernel(int m, T beta, T* __restrict__ y) {
-  const int i = blockIdx.x * 256 + threadIdx.x;
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= m) return;
   y[i] = beta == T(0) ? T(0) : y[i] * beta;
 }

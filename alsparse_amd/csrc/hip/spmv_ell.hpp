@@ -22,7 +22,7 @@ __global__ __launch_bounds__(kEllThreads) void ellmv_kernel(int m, int n, T alph
                                                             const int* __restrict__ ell_col, int width,
                                                             int base, const T* __restrict__ x, T beta,
                                                             T* __restrict__ y) {
-  const int row = blockIdx.x * kEllThreads + threadIdx.x;
+  const int64_t row = (int64_t)blockIdx.x * kEllThreads + threadIdx.x;
   if (row >= m) return;
   T sum = T(0);
   int s = 0;

@@ -27,7 +27,8 @@
 //            measured at ~0.45 lanes per clock, four times slower than the whole
 //            phase takes without them.  A wave keeps 16 tiles in flight in a
 //            ring of registers (loads issued unconditionally, so the counter of
-//            outstanding loads lets it wait for the oldest tile only).  The
+//            outstanding loads lets it wait for the oldest tile only), 32 where
+//            no tile holds more than one entry per lane.  The
 //            kRedWaves waves of a workgroup own consecutive row blocks, whose
 //            tiles are adjacent in memory.  Finally y = beta*y + alpha*acc, unit
 //            stride.
@@ -53,7 +54,7 @@ constexpr int kTileBytes = 128 * 1024;  // LDS bytes of an x slice (phase 1) / o
 constexpr int kProdThreads = 1024;      // phase-1 workgroup
 constexpr int kRedWaves = 8;            // phase-2 workgroup: 8 waves = 8 consecutive row blocks, whose tiles are adjacent in memory
 constexpr int kRedSlots = 16;
-constexpr int kLongTile = 2 * kWave;     // phase 2 takes two entries per lane and tile; longer tiles go to phase 3
+constexpr int kLongTile = 2 * kWave;     // phase 2 takes at most two entries per lane and tile; longer tiles go to phase 3
 constexpr int kLongThreads = 256;
 constexpr int kLongChunk = kLongThreads * 16;  // entries per phase-3 workgroup
 constexpr int kTiledMaxColBlocks = 2048;       // keeps the tile table small
@@ -75,7 +76,8 @@ struct TileDims {
   static constexpr int rows = red_bytes / red_waves / (int)sizeof(T);  // tallest row block
   // every wave's accumulators are followed by one dummy row per lane, where lanes without an entry add their zero
   static constexpr int red_lds_bytes = red_bytes + red_waves * kWave * (int)sizeof(T);
-  // tiles a wave keeps in flight in phase 2 (16 four-register slots would not fit for 16-byte values)
+  // tiles a wave keeps in flight in phase 2 when a tile may take two entries per lane (16 four-register
+  // slots would not fit for 16-byte values); twice as many when every tile fits one entry per lane
   static constexpr int red_slots = sizeof(T) >= 16 ? kRedSlots / 2 : kRedSlots;
 };
 
@@ -211,10 +213,30 @@ __global__ __launch_bounds__(256) void tile_bounds_kernel(int nnz, const unsigne
   tile_ptr[t] = lo;
 }
 
+// out[0] += entries held by tiles of more than kWave and at most kLongTile entries (one atomic per
+// workgroup): phase 2 handles those only in its two-entries-per-lane form.
+__global__ __launch_bounds__(256) void tile_mid_entries_kernel(int64_t tiles, const int* __restrict__ tile_ptr,
+                                                               unsigned long long* __restrict__ out) {
+  __shared__ unsigned long long s_sum[256 / kWave];
+  unsigned long long mine = 0;
+  for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < tiles; t += (int64_t)gridDim.x * blockDim.x) {
+    const int len = tile_ptr[t + 1] - tile_ptr[t];
+    if (len > kWave && len <= kLongTile) mine += (unsigned long long)len;
+  }
+  for (int d = kWave / 2; d > 0; d >>= 1) mine += __shfl_down(mine, d, kWave);
+  if (threadIdx.x % kWave == 0) s_sum[threadIdx.x / kWave] = mine;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    unsigned long long total = 0;
+    for (int w = 0; w < 256 / kWave; ++w) total += s_sum[w];
+    if (total) atomicAdd(out, total);
+  }
+}
+
 // Phase 2 reads the tile table row block by row block:
 // ranges[rb * col_blocks + cb] = {tile_ptr[cb*row_blocks + rb], tile_ptr[cb*row_blocks + rb + 1]}.
-// Tiles longer than kLongTile go to long_list instead (their range is left empty).
-__global__ __launch_bounds__(256) void tile_ranges_kernel(int row_blocks, int col_blocks,
+// Tiles longer than long_tile go to long_list instead (their range is left empty).
+__global__ __launch_bounds__(256) void tile_ranges_kernel(int row_blocks, int col_blocks, int long_tile,
                                                           const int* __restrict__ tile_ptr,
                                                           TileRange* __restrict__ ranges,
                                                           LongTile* __restrict__ long_list,
@@ -225,7 +247,7 @@ __global__ __launch_bounds__(256) void tile_ranges_kernel(int row_blocks, int co
   const int64_t t = (int64_t)cb * row_blocks + rb;
   int b = tile_ptr[t];
   const int e = tile_ptr[t + 1];
-  if (e - b > kLongTile) {
+  if (e - b > long_tile) {
     const int slot = atomicAdd(long_count, 1);
     long_list[slot].begin = b;
     long_list[slot].end = e;
@@ -398,7 +420,11 @@ __device__ __forceinline__ void add_rows(T* acc, int r, T v, bool valid_arg) {
   if (valid && !same_as_prev) rmw<Atomic>(&acc[r], v);
 }
 
-template <typename T>
+// H = entries per lane and tile: 2 takes tiles of up to kLongTile entries with red_slots tiles in flight,
+// 1 takes tiles of up to kWave entries with twice as many in flight (for the same number of outstanding
+// loads: where tiles are short -- wide values make narrow column blocks -- the loads of the second half
+// would all come back empty, and the bytes in flight, which bound the speed, would halve).
+template <typename T, int H>
 __global__ __launch_bounds__(TileDims<T>::red_threads) void tiled_reduce_kernel(
     int m, int row_blocks, int col_blocks, const int* __restrict__ row_block_start,
     const TileRange* __restrict__ ranges, const unsigned short* __restrict__ t_row,
@@ -413,8 +439,8 @@ __global__ __launch_bounds__(TileDims<T>::red_threads) void tiled_reduce_kernel(
   T* acc = s_acc + wave * (kTileRows + kWave);
   for (int i = lane; i < kTileRows + kWave; i += kWave) acc[i] = T(0);
 
-  // Wave-private accumulators.  Every tile listed in `ranges` has at most kLongTile = 128 entries: two
-  // per lane.  The wave keeps kSlots tiles in flight in a ring of registers: step s adds the tile in slot s
+  // Wave-private accumulators.  Every tile listed in `ranges` has at most H * 64 entries: H per lane.
+  // The wave keeps kSlots tiles in flight in a ring of registers: step s adds the tile in slot s
   // and at once loads the tile kSlots further on into it, so the loads of the next kSlots - 1 tiles are
   // outstanding while one tile goes through its LDS read-modify-writes.  For the hardware counter of
   // outstanding loads to allow that, every load is issued unconditionally (the compiler can only
@@ -422,10 +448,11 @@ __global__ __launch_bounds__(TileDims<T>::red_threads) void tiled_reduce_kernel(
   // the buffer range check and masked when the slot is used).  The waves of a workgroup
   // share no data and meet at no barrier: with one batch of 8 tiles in flight a barrier per batch kept
   // their reads on neighbouring tiles and doubled the speed, with the ring it measured no different.
-  constexpr int kSlots = TileDims<T>::red_slots;
+  constexpr int kSlots = TileDims<T>::red_slots * (H == 1 ? 2 : 1);
+  static_assert(H == 1 || H == 2, "one or two entries per lane");
   static_assert(kWave % kSlots == 0, "a group of tile ranges is a whole number of rings");
-  T sv[kSlots][2];
-  int sr[kSlots][2];
+  T sv[kSlots][H];
+  int sr[kSlots][H];
   int slen[kSlots];
   const TileRange* my = ranges + (int64_t)rb * col_blocks;
   auto load_ranges = [&](int group) {  // 64 tile ranges, one coalesced load
@@ -453,15 +480,19 @@ __global__ __launch_bounds__(TileDims<T>::red_threads) void tiled_reduce_kernel(
     const BufferRsrc rr = make_rsrc(t_row + b0, len * 2);
     sv[s][0] = buffer_load<T>(rv, off_v);
     sr[s][0] = buffer_load_u16(rr, off_r);
-    sv[s][1] = buffer_load<T>(rv, off_v + kWave * (int)sizeof(T));
-    sr[s][1] = buffer_load_u16(rr, off_r + kWave * 2);
+    if constexpr (H == 2) {
+      sv[s][1] = buffer_load<T>(rv, off_v + kWave * (int)sizeof(T));
+      sr[s][1] = buffer_load_u16(rr, off_r + kWave * 2);
+    }
   };
   auto consume = [&](int s) {
     const int len = slen[s];
     // a lane without an entry holds value zero already; its row becomes the lane's dummy row
     add_rows<false, true>(acc, lane < len ? sr[s][0] : r_none, sv[s][0], true);
-    if (len > kWave)  // wave-uniform
-      add_rows<false, true>(acc, lane + kWave < len ? sr[s][1] : r_none, sv[s][1], true);
+    if constexpr (H == 2) {
+      if (len > kWave)  // wave-uniform
+        add_rows<false, true>(acc, lane + kWave < len ? sr[s][1] : r_none, sv[s][1], true);
+    }
   };
 #pragma unroll
   for (int s = 0; s < kSlots; ++s) {

@@ -48,7 +48,7 @@ __global__ __launch_bounds__(256) void transpose_gather_kernel(int nnz, const un
 // y <- beta*y over n elements (beta == 0 stores zeros without reading)
 template <typename T>
 __global__ __launch_bounds__(256) void scale_vec_kernel(int n, T beta, T* __restrict__ y) {
-  const int i = blockIdx.x * 256 + threadIdx.x;
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= n) return;
   y[i] = beta == T(0) ? T(0) : y[i] * beta;
 }

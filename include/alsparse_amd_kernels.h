@@ -83,6 +83,9 @@ typedef struct {
   int32_t ell_width;    /* its slots per row                                  */
   int32_t transpose_built; /* bit 0: a CSR copy of the transpose exists, bit 1: of the
                               conjugate transpose                              */
+  int32_t tile_entries_per_lane; /* tiled copy: entries per lane and tile in its second
+                                    phase (1: twice the tiles in flight; tiles of more
+                                    than 64 entries go to the long-tile kernel), or 0  */
   int64_t hist[ASAMD_HIST_BINS];
 } asamd_csr_stats;
 

@@ -397,3 +397,54 @@ def test_analysis_choices(gpu):
         assert st.algo == capi.ASAMD_SPMV_VECTOR, capi.ALGO_NAMES[st.algo]
     finally:
         db.free()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
+@pytest.mark.parametrize("per_row", [1, 2, 5])
+def test_tiled_second_phase_in_both_forms(gpu, dtype, per_row, monkeypatch):
+    """The tiled copy's second phase takes one or two entries per lane and tile.  Both forms, forced and as
+    the analysis picks them, on structures whose tiles hold around 32, 64 and 128+ entries (2048 rows x one
+    column block each): tiles too long for the form in use must reach the long-tile kernel instead."""
+    from ctypes import c_void_p
+    lib = capi.load()
+    a = wl.uniform_rows(3 * 2048 + 77, 1 << 20, per_row, dtype)
+    x, y0 = _vectors(a)
+    da = DeviceCsr(a)
+    T = capi.scalar_type(a.dtype)
+    # what the analysis must pick where the tile sizes leave no doubt (blocks are cut to even entry counts,
+    # so tiles hold somewhat under 2048 rows x per_row x block width / columns: mean about 25: hardly a tile
+    # above 64; about 100: most entries in tiles of 65..128)
+    clear = {("float64", 1): 1, ("float32", 2): 2}
+    try:
+        for forced in (None, "1", "2"):
+            if forced is None:
+                monkeypatch.delenv("ALSPARSE_AMD_TILED_HALVES", raising=False)
+            else:
+                monkeypatch.setenv("ALSPARSE_AMD_TILED_HALVES", forced)
+            plan = c_void_p()
+            announce("tiled forms", np.dtype(dtype).name, per_row, forced)
+            assert lib.asamd_csr_plan_create(None, a.rows, a.cols, a.nnz, da.row_ptr.c_ptr(), da.col.c_ptr(),
+                                             da.val.c_ptr(), a.base, a.dtype.itemsize, 2, byref(plan)) == 0
+            try:
+                st = lib.asamd_csr_plan_stats(plan).contents
+                assert st.tiled_built == 1
+                if forced is None:  # few entries in tiles of 65..128 entries <=> one entry per lane
+                    want = clear.get((np.dtype(dtype).name, per_row))
+                    assert st.tile_entries_per_lane in ((1, 2) if want is None else (want,)), st.tile_entries_per_lane
+                else:
+                    assert st.tile_entries_per_lane == int(forced)
+                assert lib.asamd_csr_plan_set_algo(plan, ALGOS["tiled"]) == 0
+                for alpha, beta in ((1.0, 0.0), (-1.5, 0.5)):
+                    dx, dy = hiprt.DeviceArray.from_numpy(x), hiprt.DeviceArray.from_numpy(y0)
+                    assert getattr(lib, "asamd_%s_csrmv" % capi.prefix(a.dtype))(
+                        None, plan, T(alpha), da.val.c_ptr(), da.row_ptr.c_ptr(), da.col.c_ptr(), dx.c_ptr(), T(beta),
+                        dy.c_ptr()) == 0
+                    hiprt.synchronize()
+                    y = dy.to_numpy()
+                    dx.free()
+                    dy.free()
+                    check_spmv(a, alpha, x, beta, y0, y, "tiled form %s, %d per row" % (forced, per_row))
+            finally:
+                lib.asamd_csr_plan_destroy(plan)
+    finally:
+        da.free()
