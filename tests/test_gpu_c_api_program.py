@@ -3,6 +3,8 @@ info bundles through their whole lifecycle, stale analysis records under freed a
 device arrays, all four element types, results checked on the CPU inside the program.  Built by
 `make -C tests/c_api` (the package's build step runs it).  When `make -C tests/c_api asan` was run
 as well, the same program is run against the library built with ASan + UBSan on its host code."""
+import glob
+import hashlib
 import os
 import subprocess
 
@@ -33,9 +35,20 @@ def test_c_lifecycle_program_with_host_sanitizers(gpu):
     exe = os.path.join(BIN, "asan", "lifecycle")
     if not os.path.exists(exe):
         pytest.skip("the sanitized build is optional (make -C tests/c_api asan)")
-    product = os.path.join(os.path.dirname(BIN), "..", "..", "alsparse_amd", "lib", "libalpha_spblas.so")
-    if os.path.exists(product) and os.path.getmtime(os.path.join(BIN, "asan", "libalpha_spblas.so")) < os.path.getmtime(product):
-        pytest.skip("the sanitized build is older than the library (make -C tests/c_api asan)")
+    # the build keeps the digest of the sources it was made from (the Makefile's SAN_SOURCES, in byte order)
+    root = os.path.abspath(os.path.join(os.path.dirname(BIN), "..", ".."))
+    csrc = os.path.join(root, "alsparse_amd", "csrc")
+    files = []
+    for pattern in ("host/*.c", "host/*.h", "hip/*.hip", "hip/*.hpp"):
+        files += glob.glob(os.path.join(csrc, pattern))
+    files += glob.glob(os.path.join(root, "include", "*.h")) + [os.path.join(os.path.dirname(BIN), "lifecycle.c")]
+    digest = hashlib.sha256()
+    for f in sorted(files):
+        with open(f, "rb") as fh:
+            digest.update(fh.read())
+    stamp = os.path.join(BIN, "asan", "sources.sha256")
+    if not os.path.exists(stamp) or open(stamp).read().strip() != digest.hexdigest():
+        pytest.skip("the sanitized build was made from other sources than the present ones (make -C tests/c_api asan)")
     env = dict(os.environ)
     # the GPU runtime maps memory where the sanitizer would put its shadow gap; leaks of the GPU
     # runtime's own start-up allocations are not this library's
