@@ -290,8 +290,10 @@ static bool tiled_eligible(const asamd_csr_stats& st, bool force) {
   // entry positions of the tiled copy are 32-bit and the kernels step past a range's end by up to
   // a workgroup's stride before they test it
   if ((int64_t)st.nnz > (int64_t)0x7fffffff - (1 << 16)) return false;
-  // worth a try only when x cannot live in an XCD's 4 MiB L2 and the matrix is large
-  return force || ((int64_t)st.n * (int64_t)sizeof(T) >= ((int64_t)8 << 20) && st.nnz >= (1 << 22));
+  // worth a try only when x fills an XCD's 4 MiB L2 (the matrix streams through the same cache; with
+  // 2 MiB of x the tiled pair measured 0.43 ms against 0.34 ms, with 4 MiB 0.084 against 0.095) and the
+  // matrix is large; the timing run of the analysis has the last word
+  return force || ((int64_t)st.n * (int64_t)sizeof(T) >= ((int64_t)4 << 20) && st.nnz >= (1 << 22));
 }
 
 // Cuts groups [0, groups) with cumulative entry counts off[0..groups] into
@@ -362,9 +364,26 @@ static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* 
   if (e == hipSuccess) e = hipStreamSynchronize(stream);
   if (e == hipSuccess) {
     for (int g = 0; g <= row_groups; ++g) h_off[(size_t)g] -= st.base;
-    const int64_t full = ((int64_t)st.m + TileDims<T>::rows - 1) / TileDims<T>::rows;
-    rstart = cut_blocks(h_off.data(), row_groups, TileDims<T>::rows >> kRowGroupLog2,
-                        (int64_t)st.nnz / full + 1, rgb);
+    // Height of a row block: at most TileDims<T>::rows (the accumulators of a wave).  Phase 2 takes tiles
+    // of up to 128 entries and longer ones go to the slow long-tile kernel: where the column blocks are
+    // few (a narrow matrix) or the rows long, a full-height block would put more than that into most
+    // tiles, so the height is cut to leave a tile about 64 entries on average (only if that takes a
+    // quarter off or more: up to 85 entries on average still fit).  (Shortening the blocks
+    // further so that their number fills whole rounds of the waves the chip holds -- 1.2 rounds cost two
+    // -- gained 4-6 % on even rows and lost 20 % on skewed ones, whose waves are bound by the number of
+    // tiles they walk, not by their entries.)
+    const int group_rows = 1 << kRowGroupLog2;
+    int max_groups = TileDims<T>::rows >> kRowGroupLog2;
+    const double per_row = (double)st.nnz / (double)(st.m > 0 ? st.m : 1);
+    const double fit_rows = 64.0 * (double)cb / (per_row > 1e-9 ? per_row : 1e-9);
+    if (fit_rows < 0.75 * max_groups * group_rows) max_groups = fit_rows < group_rows ? 1 : (int)(fit_rows / group_rows);
+    const int64_t full = ((int64_t)st.m + (int64_t)max_groups * group_rows - 1) / ((int64_t)max_groups * group_rows);
+    // the entry limit is for skewed rows; with even rows the height decides: the mean content of a block
+    // of full height plus 6 % always fits (random row lengths of mean 16 vary by 0.6 % per block, and every
+    // block that the entry limit cuts short adds one to a count that otherwise fills whole rounds of waves)
+    const int64_t even = (int64_t)((double)max_groups * group_rows * per_row * 1.0625) + 1;
+    const int64_t row_target = std::max<int64_t>((int64_t)st.nnz / full + 1, even);
+    rstart = cut_blocks(h_off.data(), row_groups, max_groups, row_target, rgb);
     rb = (int)rstart.size() - 1;
     tiles = (int64_t)cb * rb;
     if (cb > kTiledMaxColBlocks || tiles > kTiledMaxTiles) e = hipErrorOutOfMemory;  // treated as "no tiled copy"

@@ -52,12 +52,17 @@ def test_analysed_csrmv_replays_from_a_hip_graph(gpu, shape):
         assert multiply() == 0                                   # eager, on the stream
         hiprt.check(hip.hipStreamSynchronize(stream), "sync")
         eager = dy.to_numpy()
-        if trans:
-            ref = orc.csrmv_trans_plain(a, 1.25, x, 0.5, y0)
-            err = orc.csrmv_err(orc.transpose(a), 1.25, x, 0.5, y0, eager, ref)
-            assert err.zero_den_mismatch == 0 and err.full <= TOL[a.dtype], err
-        else:
-            check_spmv(a, 1.25, x, 0.5, y0, eager, "eager " + shape)
+
+        def verify(y, what):
+            if trans:
+                ref = orc.csrmv_trans_plain(a, 1.25, x, 0.5, y0)
+                err = orc.csrmv_err(orc.transpose(a), 1.25, x, 0.5, y0, y, ref)
+                assert err.zero_den_mismatch == 0 and err.full <= TOL[a.dtype], (what, err)
+            else:
+                check_spmv(a, 1.25, x, 0.5, y0, y, what)
+        verify(eager, "eager " + shape)
+        # the plan that runs the multiply: the transposed copy has an analysis of its own
+        running = lib.asamd_analysis_transpose_stats(info).contents if trans else stats
         announce("graph capture: record", shape)
         hiprt.check(hip.hipStreamBeginCapture(stream, 0), "hipStreamBeginCapture")
         st = multiply()
@@ -71,8 +76,8 @@ def test_analysed_csrmv_replays_from_a_hip_graph(gpu, shape):
             hiprt.check(hip.hipGraphLaunch(gexec, stream), "hipGraphLaunch")
             hiprt.check(hip.hipStreamSynchronize(stream), "sync")
             got = dy.to_numpy()
-            if stats.tiled_built:  # long tiles reach y through atomics: order-dependent in the last bits
-                check_spmv(a, 1.25, x, 0.5, y0, got, "replay %d" % replay)
+            if running.tiled_built:  # long tiles reach y through atomics: order-dependent in the last bits
+                verify(got, "replay %d" % replay)
             else:
                 assert np.array_equal(got, eager), "replay %d differs from the eager result" % replay
     finally:

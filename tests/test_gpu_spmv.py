@@ -448,3 +448,30 @@ def test_tiled_second_phase_in_both_forms(gpu, dtype, per_row, monkeypatch):
                 lib.asamd_csr_plan_destroy(plan)
     finally:
         da.free()
+
+
+def test_tiled_row_blocks_follow_the_tile_population(gpu):
+    """2 M x 2 M with 16 entries per row: 64 column blocks, so a 2 048-row block would put 512 entries into
+    every tile and leave them all to the long-tile kernel.  The analysis cuts the blocks to about 256 rows
+    (64 entries per tile), and the tiled pair then wins its timing run against the row kernels."""
+    lib = capi.load()
+    a = wl.uniform_rows(1 << 21, 1 << 21, 16, np.float32)
+    x, y0 = _vectors(a)
+    da = DeviceCsr(a)
+    info = capi.alphasparse_dcu_mat_info_t()
+    assert lib.alphasparse_dcu_create_mat_info(byref(info)) == 0
+    descr = capi.make_descr(base=a.base)
+    try:
+        announce("tile population", a.name)
+        assert lib.alphasparse_dcu_s_csrmv_analysis(gpu.h, 0, a.rows, a.cols, a.nnz, byref(descr), da.val.c_ptr(),
+                                                    da.row_ptr.c_ptr(), da.col.c_ptr(), info) == 0
+        st = lib.asamd_analysis_stats(info).contents
+        assert st.tiled_built == 1 and st.algo == capi.ASAMD_SPMV_TILED, capi.ALGO_NAMES[st.algo]
+        assert 6000 <= st.tile_row_blocks <= 9000, st.tile_row_blocks
+        mean_tile = a.nnz / (st.tile_row_blocks * st.tile_col_blocks)
+        assert 40 <= mean_tile <= 80, mean_tile
+        assert 0 < st.tune_ms_tiled < st.tune_ms_base
+        check_spmv(a, 1.5, x, 0.5, y0, run_csrmv(gpu, da, 1.5, x, 0.5, y0, info), "2M x 2M analysed")
+    finally:
+        lib.alphasparse_dcu_destroy_mat_info(info)
+        da.free()
