@@ -368,16 +368,30 @@ static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* 
     // of up to 128 entries and longer ones go to the slow long-tile kernel: where the column blocks are
     // few (a narrow matrix) or the rows long, a full-height block would put more than that into most
     // tiles, so the height is cut to leave a tile about 64 entries on average (only if that takes a
-    // quarter off or more: up to 85 entries on average still fit).  (Shortening the blocks
-    // further so that their number fills whole rounds of the waves the chip holds -- 1.2 rounds cost two
-    // -- gained 4-6 % on even rows and lost 20 % on skewed ones, whose waves are bound by the number of
-    // tiles they walk, not by their entries.)
+    // quarter off or more: up to 85 entries on average still fit).
+    // Phase 2 runs one row block per wave and the chip holds a fixed number of its waves at a time (the
+    // accumulators fill the LDS): N blocks take ceil(N / slots) rounds, so 2.01 rounds of blocks cost three.
+    // With even rows (the height decides every block, and a wave's time follows its entries) the blocks
+    // are made just short enough to fill a whole number of rounds: 4-9 % on 5-10 M rows.  Not with skewed
+    // rows: their waves are bound by the number of tiles they walk, and shorter blocks lost 20 % there.
     const int group_rows = 1 << kRowGroupLog2;
     int max_groups = TileDims<T>::rows >> kRowGroupLog2;
     const double per_row = (double)st.nnz / (double)(st.m > 0 ? st.m : 1);
     const double fit_rows = 64.0 * (double)cb / (per_row > 1e-9 ? per_row : 1e-9);
     if (fit_rows < 0.75 * max_groups * group_rows) max_groups = fit_rows < group_rows ? 1 : (int)(fit_rows / group_rows);
-    const int64_t full = ((int64_t)st.m + (int64_t)max_groups * group_rows - 1) / ((int64_t)max_groups * group_rows);
+    int64_t full = ((int64_t)st.m + (int64_t)max_groups * group_rows - 1) / ((int64_t)max_groups * group_rows);
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      cus = 256;
+    const int64_t slots = (int64_t)cus * TileDims<T>::red_waves * (kLdsPerCu / TileDims<T>::red_lds_bytes);
+    const bool even_rows = (double)st.max_len <= 3.0 * per_row + 16.0;
+    if (even_rows && full > slots && full % slots != 0) {
+      const int64_t want = (full + slots - 1) / slots * slots;
+      const int64_t rows_each = ((int64_t)st.m + want - 1) / want;
+      max_groups = (int)((rows_each + group_rows - 1) / group_rows);
+      full = ((int64_t)st.m + (int64_t)max_groups * group_rows - 1) / ((int64_t)max_groups * group_rows);
+    }
     // the entry limit is for skewed rows; with even rows the height decides: the mean content of a block
     // of full height plus 6 % always fits (random row lengths of mean 16 vary by 0.6 % per block, and every
     // block that the entry limit cuts short adds one to a count that otherwise fills whole rounds of waves)

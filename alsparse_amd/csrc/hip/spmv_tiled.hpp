@@ -50,6 +50,7 @@
 
 namespace asamd {
 
+constexpr int kLdsPerCu = 160 * 1024;   // LDS of one compute unit
 constexpr int kTileBytes = 128 * 1024;  // LDS bytes of an x slice (phase 1) / of a workgroup's accumulators (phase 2)
 constexpr int kProdThreads = 1024;      // phase-1 workgroup
 constexpr int kRedWaves = 8;            // phase-2 workgroup: 8 waves = 8 consecutive row blocks, whose tiles are adjacent in memory
