@@ -354,8 +354,19 @@ static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* 
   if (e == hipSuccess) {
     h_off[0] = 0;
     for (int g = 0; g < col_groups; ++g) h_off[(size_t)g + 1] += h_off[(size_t)g];
-    const int64_t full = ((int64_t)st.n + TileDims<T>::cols - 1) / TileDims<T>::cols;
-    cstart = cut_blocks(h_off.data(), col_groups, TileDims<T>::cols >> kColGroupLog2,
+    // Width of a column block: at most TileDims<T>::cols (the x slice of phase 1).  A row block cannot be
+    // shorter than one group of 64 rows, whose tiles hold 64 * entries per row / column blocks entries on
+    // average: where the rows are so long that this exceeds 64 the column blocks are made narrower
+    // (2 M x 2 M with 128 entries per row: 65 blocks -> 128).
+    int col_max_groups = TileDims<T>::cols >> kColGroupLog2;
+    int64_t full = ((int64_t)st.n + TileDims<T>::cols - 1) / TileDims<T>::cols;
+    const double mean_len = (double)st.nnz / (double)(st.m > 0 ? st.m : 1);
+    if (mean_len > (double)full) {
+      const int64_t width = (int64_t)((double)st.n / mean_len);
+      col_max_groups = width < (2 << kColGroupLog2) ? 1 : (int)(width >> kColGroupLog2);
+      full = ((int64_t)st.n + ((int64_t)col_max_groups << kColGroupLog2) - 1) / ((int64_t)col_max_groups << kColGroupLog2);
+    }
+    cstart = cut_blocks(h_off.data(), col_groups, col_max_groups,
                         (int64_t)h_off[(size_t)col_groups] / full + 1, cgb);  // h_off: sampled entries
     cb = (int)cstart.size() - 1;
     row_group_offsets_kernel<<<(row_groups + 1 + 255) / 256, 256, 0, stream>>>(st.m, row_ptr, row_groups, d_cnt);
