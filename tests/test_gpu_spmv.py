@@ -450,12 +450,15 @@ def test_tiled_second_phase_in_both_forms(gpu, dtype, per_row, monkeypatch):
         da.free()
 
 
-def test_tiled_row_blocks_follow_the_tile_population(gpu):
+@pytest.mark.parametrize("m,n,per_row", [(1 << 21, 1 << 21, 16), (1 << 19, 1 << 21, 128)], ids=["16_per_row", "128_per_row"])
+def test_tiled_row_blocks_follow_the_tile_population(gpu, m, n, per_row):
     """2 M x 2 M with 16 entries per row: 64 column blocks, so a 2 048-row block would put 512 entries into
     every tile and leave them all to the long-tile kernel.  The analysis cuts the blocks to about 256 rows
-    (64 entries per tile), and the tiled pair then wins its timing run against the row kernels."""
+    (64 entries per tile), and the tiled pair then wins its timing run against the row kernels.  With 128
+    entries per row even the shortest row block (64 rows) would overfill its tiles: the column blocks are
+    made narrower as well (about 128 of them instead of 64)."""
     lib = capi.load()
-    a = wl.uniform_rows(1 << 21, 1 << 21, 16, np.float32)
+    a = wl.uniform_rows(m, n, per_row, np.float32)
     x, y0 = _vectors(a)
     da = DeviceCsr(a)
     info = capi.alphasparse_dcu_mat_info_t()
@@ -471,7 +474,8 @@ def test_tiled_row_blocks_follow_the_tile_population(gpu):
         mean_tile = a.nnz / (st.tile_row_blocks * st.tile_col_blocks)
         assert 40 <= mean_tile <= 80, mean_tile
         assert 0 < st.tune_ms_tiled < st.tune_ms_base
-        check_spmv(a, 1.5, x, 0.5, y0, run_csrmv(gpu, da, 1.5, x, 0.5, y0, info), "2M x 2M analysed")
+        assert (st.tile_col_blocks > 100) == (per_row == 128), st.tile_col_blocks
+        check_spmv(a, 1.5, x, 0.5, y0, run_csrmv(gpu, da, 1.5, x, 0.5, y0, info), "%d per row analysed" % per_row)
     finally:
         lib.alphasparse_dcu_destroy_mat_info(info)
         da.free()
