@@ -136,7 +136,15 @@ def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False, vendor=Fa
     from alsparse_amd import capi, hiprt, workloads as wl
     lib = capi.load()
     t0 = time.time()
-    a, x, y0, alpha, beta, _ = wl.config(cfg)
+    if isinstance(cfg, tuple):  # ("uniform", rows, cols, entries per row, dtype): not a benchmark configuration
+        _, um, un, uk, udt = cfg
+        a = wl.uniform_rows(um, un, uk, udt)
+        x, y0, alpha, beta = wl.uniform(a.cols, udt, 3), wl.uniform(a.rows, udt, 4), 1.0, 0.5
+        workload_name = "uniform rows: CSR SpMV %s, %d rows x %d columns, %d nnz/row uniform random sorted columns, alpha=1 beta=0.5" % (
+            np.dtype(udt).name, um, un, uk)
+    else:
+        a, x, y0, alpha, beta, _ = wl.config(cfg)
+        workload_name = WORKLOAD_NAMES[cfg]
     if cx:
         cdt = np.complex64 if a.dtype == np.float32 else np.complex128
         a = wl.complexify(a, cdt)
@@ -214,7 +222,7 @@ def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False, vendor=Fa
     nbytes = (wl.spmv_bytes(a.cols, a.rows, a.nnz, a.dtype.itemsize, beta) if transpose
               else wl.spmv_bytes(a.rows, a.cols, a.nnz, a.dtype.itemsize, beta))
     opname = "" if not transpose else (" -- CONJUGATE-TRANSPOSED operation" if op == 2 else " -- TRANSPOSED operation")
-    res = {"workload": WORKLOAD_NAMES[cfg] + (" -- COMPLEX values (%s)" % a.dtype.name if cx else "") + opname, "rows": a.rows, "nnz": a.nnz, "algorithmic_bytes": int(nbytes),
+    res = {"workload": workload_name + (" -- COMPLEX values (%s)" % a.dtype.name if cx else "") + opname, "rows": a.rows, "nnz": a.nnz, "algorithmic_bytes": int(nbytes),
            "flops": 2 * a.nnz, "kernel": algo, "analysis_ms": analysis_ms, "timing": t,
            "gbs": nbytes / t["avg_ms"] / 1e6, "gflops": 2 * a.nnz / t["avg_ms"] / 1e6,
            "dtype": {"float32": "f32", "float64": "f64", "complex64": "c64", "complex128": "c128"}[a.dtype.name],
@@ -503,6 +511,10 @@ def main():
     ap.add_argument("--conjugate", action="store_true", help="with --complex --transpose: A^H instead of A^T")
     ap.add_argument("--conversions", action="store_true",
                     help="measure alphasparse_dcu_csr2coo (the main line) and ?csr2ell on configuration 2 or 3")
+    ap.add_argument("--uniform", nargs=3, type=int, metavar=("ROWS", "COLS", "PER_ROW"),
+                    help="instead of a configuration: CSR SpMV on a matrix of that shape with PER_ROW uniform random "
+                         "columns per row (fp32, --fp64 for fp64); same analysis, timing and parity check")
+    ap.add_argument("--fp64", action="store_true", help="with --uniform: fp64 values")
     ap.add_argument("--all", action="store_true", help="also measure the other configurations")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-vendor-baseline", action="store_true",
@@ -549,7 +561,10 @@ def main():
     elif args.config == 5:
         main_res = run_spmm(args.steps, args.warmup, check, args.col_major, not args.no_vendor_baseline)
     else:
-        main_res = run_spmv(args.config, args.steps, args.warmup, not args.no_cpu_baseline, check, args.transpose,
+        cfg = args.config
+        if args.uniform:
+            cfg = ("uniform", args.uniform[0], args.uniform[1], args.uniform[2], np.float64 if args.fp64 else np.float32)
+        main_res = run_spmv(cfg, args.steps, args.warmup, not args.no_cpu_baseline, check, args.transpose,
                             not args.no_vendor_baseline, args.cx, args.conjugate)
     others = {}
     if args.all:
