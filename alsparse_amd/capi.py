@@ -310,6 +310,7 @@ _COMMON = {
     "asamd_csr2coo_ws": [_P, _P, _I, _I, _P, _I, _P, c_size_t],
     "asamd_csr2ell_width": [_P, _I, _P, POINTER(_I)],
     "asamd_warmup": [_P],
+    "asamd_s_csrmv_noalloc": [_P, _I, _I, _I, _I, c_float, _P, _P, _P, _P, c_float, _P],
     "asamd_handle_set_stream": [_P, _P],
     "asamd_handle_get_stream": [_P],
     "asamd_copy_bytes": [_P, _P, _P, c_size_t],

@@ -133,6 +133,23 @@ int asamd_d_csrmv(hipStream_t stream, asamd_csr_plan *plan, double alpha, const 
                   const int32_t *row_ptr, const int32_t *col_ind, const double *x, double beta,
                   double *y);
 
+/* asamd_s_csrmv without a plan and without any allocation: for callers that cannot call hipMalloc
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid it).  No counterpart in
+ * the reference.  Runs the merge-path kernels (any row-length distribution, no float atomics); their
+ * workgroup coordinates, carries and head sums live in a fixed device array of
+ * ASAMD_CSRMV_NOALLOC_SCRATCH_BYTES that the library holds per GPU until the process ends.
+ * m + nnz above ASAMD_CSRMV_NOALLOC_MAX_ITEMS returns hipErrorOutOfMemory (2) before anything is
+ * launched; other bad arguments return hipErrorInvalidValue.  base is 0 or 1; nnz == 0 gives
+ * y = beta*y.  Calls hipMalloc, hipFree or an allocating library routine never; asamd_warmup (run by
+ * alphasparse_dcu_get_handle) resolves the array's address for the current device, and the first
+ * call on a device does so itself otherwise.  All calls on one GPU share the array: calls that
+ * overlap there (two streams, two threads) race; calls on one stream are ordered and safe. */
+#define ASAMD_CSRMV_NOALLOC_SCRATCH_BYTES (4 << 20)
+#define ASAMD_CSRMV_NOALLOC_MAX_ITEMS 536868864LL /* (SCRATCH_BYTES / 16 - 1) workgroups x 2048 items */
+int asamd_s_csrmv_noalloc(hipStream_t stream, int32_t m, int32_t n, int32_t nnz, int32_t base, float alpha,
+                          const float *val, const int32_t *row_ptr, const int32_t *col_ind, const float *x,
+                          float beta, float *y);
+
 /* CSR copy of the transpose, owned by the plan (trusted plans only; row_ptr,
  * col_ind, val are the arrays the plan was created for).  Later transposed
  * multiplies run the ordinary kernels on that copy (with an analysis of its
@@ -347,7 +364,8 @@ int asamd_copy_bytes(hipStream_t stream, void *dst, const void *src, size_t nbyt
 int asamd_handle_set_stream(void *handle, hipStream_t stream);
 hipStream_t asamd_handle_get_stream(void *handle);
 
-/* Empty kernel; forces code-object load (src/util_cpp/handle.cpp:19, :113). */
+/* Empty kernel; forces code-object load (src/util_cpp/handle.cpp:19, :113).  Also looks up, for the
+ * current device, the address of the fixed array that asamd_s_csrmv_noalloc works in. */
 int asamd_warmup(hipStream_t stream);
 
 #ifdef __cplusplus
