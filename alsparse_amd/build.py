@@ -6,7 +6,8 @@ import subprocess
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB_DIR = os.path.join(ROOT, "alsparse_amd", "lib")
-LIB_PATH = os.path.join(LIB_DIR, "libalpha_spblas.so")
+# ALSPARSE_AMD_LIB names another build of the same library (kernel experiments); there is no other fallback
+LIB_PATH = os.environ.get("ALSPARSE_AMD_LIB") or os.path.join(LIB_DIR, "libalpha_spblas.so")
 WORKLOADS_PATH = os.path.join(LIB_DIR, "libasamd_workloads.so")
 
 

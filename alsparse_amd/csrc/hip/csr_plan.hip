@@ -553,7 +553,7 @@ static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* 
   }
   if (e == hipSuccess)  // both phases use more than the default 64 KiB of dynamic LDS
     e = hipFuncSetAttribute((const void*)tiled_products_kernel<T>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, kTileBytes);
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kSliceBytes);
   if (e == hipSuccess)
     e = hipFuncSetAttribute((const void*)tiled_reduce_kernel<T, 1>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, TileDims<T>::red_lds_bytes);
@@ -987,7 +987,7 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
     case ASAMD_SPMV_TILED: {
       // the tiled copy holds zero-based local indices and its own values
       if (p->n_chunks > 0)
-        tiled_products_kernel<T><<<p->n_chunks, kProdThreads, kTileBytes, s>>>(
+        tiled_products_kernel<T><<<p->n_chunks, kProdThreads, kSliceBytes, s>>>(
             p->d_chunks, (const T*)p->d_tval, p->d_tcol, x, (T*)p->d_tprod);
       const unsigned red_grid = (unsigned)((st.tile_row_blocks + TileDims<T>::red_waves - 1) / TileDims<T>::red_waves);
       if (p->tiled_halves == 1)

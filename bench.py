@@ -27,16 +27,22 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes per multiply measured with rocprofv3 (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from a
-# 1 GiB copy kernel); the summaries these come from are profiles/spmv_tiled_C3.txt, spmv_merge_C4.txt,
-# spmv_ell_copy_C2.txt and spmm_rowmajor_C5.txt.  Keyed by (configuration, kernel family); anything else reports null.
+# HBM bytes per multiply measured with rocprofv3 in separate counter runs (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000,
+# factors from a 1 GiB copy kernel) -- a table of earlier measurements, not an in-run reading; each entry names the
+# summary under profiles/ it comes from.  Keyed by (configuration, kernel family); anything else reports null.
 MEASURED_TRAFFIC_BYTES = {
-    (3, "tiled two-phase"): 5.00e9,
-    (3, "rowconst"): 34.6e9,
-    (4, "merge-path"): 3.32e9,
-    (2, "ell copy"): 322.5e6,
-    (5, "spmm row-major"): 9.27e9,
+    (3, "tiled two-phase"): (5.00e9, "profiles/spmv_tiled_C3.txt"),
+    (3, "rowconst"): (34.6e9, "profiles/spmv_tiled_C3.txt"),
+    (4, "merge-path"): (3.32e9, "profiles/spmv_merge_C4.txt"),
+    (2, "ell copy"): (322.5e6, "profiles/spmv_ell_copy_C2.txt"),
+    (5, "spmm row-major"): (9.27e9, "profiles/spmm_rowmajor_C5.txt"),
 }
+
+
+def measured_traffic(cfg, kernel):
+    """(bytes, source file) of the counter measurement recorded for this configuration and kernel, or (None, None)."""
+    return MEASURED_TRAFFIC_BYTES.get((cfg, kernel), (None, None))
+
 
 WORKLOAD_NAMES = {
     2: "C2: CSR SpMV fp64, 5-point Laplacian 2048x2048 (4194304 rows, 20963328 nnz), alpha=1 beta=0",
@@ -230,7 +236,7 @@ def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False, vendor=Fa
     if cx:  # a complex multiply-add is 8 real flops
         res["flops"], res["gflops"] = 8 * a.nnz, 8 * a.nnz / t["avg_ms"] / 1e6
     res["hbm_frac"] = res["gbs"] / HBM_PEAK_GBS
-    res["traffic"] = None if (transpose or cx) else MEASURED_TRAFFIC_BYTES.get((cfg, algo))
+    res["traffic"], res["traffic_source"] = (None, None) if (transpose or cx or isinstance(cfg, tuple)) else measured_traffic(cfg, algo)
 
     if cpu_baseline and not transpose:
         res["cpu_baseline"] = cpu_spmv(a, x, y0, alpha, beta, nbytes)
@@ -468,7 +474,7 @@ def run_spmm(steps, warmup, check, col_major=False, vendor=False):
            "gbs": nbytes / t["avg_ms"] / 1e6, "gflops": 2 * a.nnz * n / t["avg_ms"] / 1e6, "dtype": "f32",
            "parity": parity}
     res["hbm_frac"] = res["gbs"] / HBM_PEAK_GBS
-    res["traffic"] = None if col_major else MEASURED_TRAFFIC_BYTES.get((5, "spmm row-major"))
+    res["traffic"], res["traffic_source"] = (None, None) if col_major else measured_traffic(5, "spmm row-major")
     if col_major and vendor and os.path.exists(ROCSPARSE):
         # rocSPARSE's legacy csrmm takes column-major operands only: compared on this layout
         import ctypes
@@ -495,6 +501,57 @@ def run_spmm(steps, warmup, check, col_major=False, vendor=False):
     return res
 
 
+def run_ceilings(steps, warmup):
+    """What this GPU sustains with plain kernels (alsparse_amd/csrc/hip/ceilings.hip): 2 GiB read-only, write-only
+    and copy streams, whole 256-byte rows gathered at random from 256 MiB (the B operand of configuration 5) and
+    single floats gathered at random from 64 MiB / 4 MiB / 16 KiB (the x of configuration 3; an L2-sized x; an
+    L1-sized x).  TB/s of useful bytes, and gathers per second."""
+    from ctypes import c_int64
+    from alsparse_amd import capi, hiprt
+    lib = capi.load()
+    big = 2 << 30
+    a, b = hiprt.DeviceArray((big,), np.uint8), hiprt.DeviceArray((big,), np.uint8)
+    sink = hiprt.DeviceArray((4,), np.uint8)
+    a.fill_bytes(1)
+    b.fill_bytes(2)
+    moved = c_int64(0)
+    out = {}
+
+    def measure(name, kind, dst, src, nbytes, count):
+        def step():
+            e = lib.asamd_ceiling_kernel(None, kind, dst, src, nbytes, count, sink.c_ptr(), byref(moved))
+            if e != 0:
+                raise RuntimeError("asamd_ceiling_kernel(%s) hip error %d" % (name, e))
+        t = time_steps(step, steps, warmup, hiprt)
+        out[name] = {"avg_ms": t["avg_ms"], "min_ms": t["min_ms"], "useful_bytes": moved.value,
+                     "tb_per_s": moved.value / t["avg_ms"] / 1e9}
+        return out[name]
+    measure("read_2GiB", 0, None, a.c_ptr(), big, 0)
+    measure("read_2GiB_nontemporal", 5, None, a.c_ptr(), big, 0)
+    measure("write_2GiB", 1, b.c_ptr(), None, big, 0)
+    measure("copy_2GiB", 2, b.c_ptr(), a.c_ptr(), big, 0)
+    measure("copy_2GiB_nontemporal", 6, b.c_ptr(), a.c_ptr(), big, 0)
+    r = measure("row_gather_256B_from_256MiB", 3, None, a.c_ptr(), 256 << 20, 1 << 25)
+    r["rows_per_s"] = r["useful_bytes"] / 256 / r["avg_ms"] * 1e3
+    r = measure("row_gather_256B_from_2GiB", 3, None, a.c_ptr(), big, 1 << 25)
+    r["rows_per_s"] = r["useful_bytes"] / 256 / r["avg_ms"] * 1e3
+    for label, nb in (("64MiB", 64 << 20), ("32MiB", 32 << 20), ("4MiB", 4 << 20), ("2MiB", 2 << 20), ("16KiB", 16 << 10)):
+        r = measure("elem_gather_4B_from_" + label, 4, None, a.c_ptr(), nb, 1 << 28)
+        r["gathers_per_s"] = r["useful_bytes"] / 4 / r["avg_ms"] * 1e3
+    for d in (a, b, sink):
+        d.free()
+    return out
+
+
+def brief(r):
+    """The figures of one configuration that the default line carries under `others`."""
+    t = r["timing"]
+    return {"workload": r["workload"], "kernel": r.get("kernel"), "dtype": r["dtype"], "ms": t["avg_ms"], "min_ms": t["min_ms"],
+            "gbs": r["gbs"], "gflops": r["gflops"], "hbm_frac": r["hbm_frac"], "algorithmic_bytes": r["algorithmic_bytes"],
+            "analysis_ms": r.get("analysis_ms"), "parity": r["parity"], "traffic": r.get("traffic"),
+            "traffic_source": r.get("traffic_source")}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -516,6 +573,11 @@ def main():
                          "columns per row (fp32, --fp64 for fp64); same analysis, timing and parity check")
     ap.add_argument("--fp64", action="store_true", help="with --uniform: fp64 values")
     ap.add_argument("--all", action="store_true", help="also measure the other configurations")
+    ap.add_argument("--only", action="store_true",
+                    help="measure the selected configuration alone (by default the line also carries brief figures of "
+                         "configurations 2, 4 and 5 under `others`)")
+    ap.add_argument("--stream-ceiling", action="store_true",
+                    help="instead of a workload: time plain read / write / copy / gather kernels and print their TB/s")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-vendor-baseline", action="store_true",
                     help="skip timing rocSPARSE's csrmv on the same workload (reported as vendor_baseline)")
@@ -544,6 +606,12 @@ def main():
         src.free()
         dst.free()
 
+    if args.stream_ceiling:
+        print(json.dumps({"metric": "practical memory ceilings of this GPU (plain kernels, useful bytes / time)",
+                          "unit": "TB/s", "steps": args.steps, "warmup": args.warmup, "hbm_peak_tb_per_s": HBM_PEAK_GBS / 1e3,
+                          "ceilings": run_ceilings(args.steps, args.warmup)}), flush=True)
+        return
+
     check = not args.no_check
     conv = None
     if args.conversions:
@@ -567,6 +635,14 @@ def main():
         main_res = run_spmv(cfg, args.steps, args.warmup, not args.no_cpu_baseline, check, args.transpose,
                             not args.no_vendor_baseline, args.cx, args.conjugate)
     others = {}
+    plain_default = (args.config == 3 and not (args.all or args.only or args.uniform or args.transpose or args.cx or
+                                               args.conversions or args.col_major) and args.format == "csr")
+    if plain_default:
+        # the default line is configuration 3; the other device configurations ride along, briefly
+        for c in (2, 4, 5):
+            r = (run_spmm(args.steps, args.warmup, check) if c == 5
+                 else run_spmv(c, args.steps, args.warmup, False, check, False, False))
+            others["C%d" % c] = brief(r)
     if args.all:
         for c in (2, 3, 4, 5):
             if c == args.config and not args.transpose and args.format == "csr" and not args.col_major:
@@ -615,6 +691,7 @@ def main():
         "parity": main_res["parity"],
         "roofline": {"bound": "hbm", "achieved": main_res["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": main_res["hbm_frac"], "traffic": main_res.get("traffic"),
+                     "traffic_source": main_res.get("traffic_source"),
                      "algorithmic_bytes_per_launch": main_res["algorithmic_bytes"]},
         "cpu_baseline": main_res.get("cpu_baseline"),
         "vendor_baseline": main_res.get("vendor_baseline"),

@@ -357,6 +357,25 @@ int asamd_analysis_set_algo(const void *key, int32_t algo);
  * known size; no reference counterpart. */
 int asamd_copy_bytes(hipStream_t stream, void *dst, const void *src, size_t nbytes);
 
+/* Plain memory kernels that measure what the GPU sustains (the practical ceilings that the kernels'
+ * roofline figures are read against); no reference counterpart.  kind: READ / WRITE / COPY stream nbytes
+ * (a multiple of 16; 16 bytes per lane and access) from src / into dst; ROW_GATHER fetches `count`
+ * 256-byte rows at random positions of the nbytes at src, one wave per row (what the row-major SpMM does
+ * per entry of A with 64 dense columns); ELEM_GATHER fetches `count` single floats at random positions
+ * (what a row SpMV kernel does per entry).  sink: 4 device bytes that are practically never written.
+ * *bytes_moved receives the useful bytes of the launch (copy: read + written). */
+enum asamd_ceiling_kind {
+  ASAMD_CEILING_READ = 0,
+  ASAMD_CEILING_WRITE = 1,
+  ASAMD_CEILING_COPY = 2,
+  ASAMD_CEILING_ROW_GATHER = 3,
+  ASAMD_CEILING_ELEM_GATHER = 4,
+  ASAMD_CEILING_READ_NT = 5, /* the same streams with non-temporal accesses */
+  ASAMD_CEILING_COPY_NT = 6
+};
+int asamd_ceiling_kernel(hipStream_t stream, int32_t kind, void *dst, const void *src, size_t nbytes,
+                         int64_t count, void *sink, int64_t *bytes_moved);
+
 /* handle->stream for callers that cannot see the handle struct (language bindings); C callers assign
  * the field, as with the reference.  `handle` is an alphasparse_dcu_handle_t.  Every multiply that
  * runs from an explicit analysis only launches kernels on that stream, so it can be captured into
