@@ -300,6 +300,8 @@ _COMMON = {
     "asamd_csr_plan_destroy": [_P],
     "asamd_csr_plan_stats": [_P],
     "asamd_csr_plan_set_algo": [_P, _I],
+    "asamd_csr_plan_refresh_values": [_P, _P, _P, _P, _P],
+    "asamd_csr_structure_hash": [_P, _I, _I, _P, _P, POINTER(ctypes.c_uint64)],
     "asamd_csr_plan_build_transpose": [_P, _P, _P, _P, _P],
     "asamd_csr_plan_set_lazy_transpose": [_P, _I],
     "asamd_csr_plan_transpose_stats": [_P],

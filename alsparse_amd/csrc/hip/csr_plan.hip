@@ -103,6 +103,7 @@ struct asamd_csr_plan {
   int n_long_chunks;
   int tiled_halves;           // entries per lane and tile in phase 2: 2, or 1 where (nearly) all tiles are short
   void* d_tval;               // nnz values in tile order
+  unsigned* d_tperm;          // nnz: CSR position of the entry in every tile-order slot (for refreshing d_tval)
   unsigned short* d_tcol;     // nnz local columns
   unsigned short* d_trow;     // nnz local rows
   void* d_tprod;              // nnz products (phase 1 -> phase 2)
@@ -117,6 +118,7 @@ struct asamd_csr_plan {
     int* d_row_ptr;           // n + 1
     int* d_col;               // nnz zero-based rows of A
     void* d_val;              // nnz values (conjugated in copy [1])
+    unsigned* d_perm;         // nnz: CSR position of every entry of the copy (for refreshing d_val)
     const void* val_src;      // the value array that d_val was gathered from
   } tr[2];
   bool lazy_transpose;        // build a copy on the first transposed multiply
@@ -180,7 +182,12 @@ static void choose_algo(asamd_csr_plan* p) {
   const double mean = st.m > 0 ? (double)st.nnz / st.m : 0.0;
   const int w = width_for_mean(mean);
   p->auto_width = w;
-  if (rowconst_ok(p)) {
+  if (st.first_offset != 0) {
+    // row_ptr points into the middle of a larger array: only the kernels that index with the absolute
+    // offsets (as the reference's csr_gemv_vector does) see the right entries; merge-path and csr2coo,
+    // the source of every re-ordered copy, count entries from position 0
+    p->auto_algo = stream_ok(p) ? ASAMD_SPMV_STREAM : ASAMD_SPMV_VECTOR;
+  } else if (rowconst_ok(p)) {
     p->auto_algo = ASAMD_SPMV_ROWCONST;
   } else if (stream_ok(p)) {
     p->auto_algo = ASAMD_SPMV_STREAM;
@@ -212,6 +219,8 @@ static void free_tiled(asamd_csr_plan* p) {
   p->n_long_chunks = 0;
   p->tiled_halves = 2;
   if (p->d_tval) (void)hipFree(p->d_tval);
+  if (p->d_tperm) (void)hipFree(p->d_tperm);
+  p->d_tperm = nullptr;
   if (p->d_tcol) (void)hipFree(p->d_tcol);
   if (p->d_trow) (void)hipFree(p->d_trow);
   if (p->d_tprod) (void)hipFree(p->d_tprod);
@@ -238,7 +247,8 @@ static void free_transpose(asamd_csr_plan* p, int which) {
   if (t.d_row_ptr) (void)hipFree(t.d_row_ptr);
   if (t.d_col) (void)hipFree(t.d_col);
   if (t.d_val) (void)hipFree(t.d_val);
-  t = asamd_csr_plan::TransCopy{nullptr, nullptr, nullptr, nullptr, nullptr};
+  if (t.d_perm) (void)hipFree(t.d_perm);
+  t = asamd_csr_plan::TransCopy{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
   p->st.transpose_built &= ~(1 << which);
 }
 
@@ -246,7 +256,7 @@ static void free_transpose(asamd_csr_plan* p, int which) {
 // little: the kernel then streams 4 + sizeof(T) bytes per entry at full width
 // with neither row_ptr nor LDS staging.
 static bool ell_eligible(const asamd_csr_stats& st, bool force) {
-  if (!st.trusted || st.max_len < 1 || st.max_len > 32) return false;
+  if (!st.trusted || st.first_offset != 0 || st.max_len < 1 || st.max_len > 32) return false;
   const int64_t slots = (int64_t)st.m * st.max_len;
   if (slots >= ((int64_t)1 << 31) || slots > (int64_t)st.nnz + st.nnz / 8) return false;
   return force || st.nnz >= (1 << 18);
@@ -287,7 +297,7 @@ static bool tiled_eligible(const asamd_csr_stats& st, bool force) {
   // per dimension) is checked again once it is known
   const int64_t cb = ((int64_t)st.n + TileDims<T>::cols - 1) / TileDims<T>::cols;
   const int64_t rb = ((int64_t)st.m + TileDims<T>::rows - 1) / TileDims<T>::rows;
-  if (!st.trusted || 2 * cb > kTiledMaxColBlocks || cb * rb > kTiledMaxTiles / 2) return false;
+  if (!st.trusted || st.first_offset != 0 || 2 * cb > kTiledMaxColBlocks || cb * rb > kTiledMaxTiles / 2) return false;
   // entry positions of the tiled copy are 32-bit and the kernels step past a range's end by up to
   // a workgroup's stride before they test it
   if ((int64_t)st.nnz > (int64_t)0x7fffffff - (1 << 16)) return false;
@@ -412,7 +422,7 @@ static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* 
     rstart = cut_blocks(h_off.data(), row_groups, max_groups, row_target, rgb);
     rb = (int)rstart.size() - 1;
     tiles = (int64_t)cb * rb;
-    if (cb > kTiledMaxColBlocks || tiles > kTiledMaxTiles) e = hipErrorOutOfMemory;  // treated as "no tiled copy"
+    if (cb > kTiledMaxColBlocks || tiles > kTiledMaxTiles) e = hipErrorNotSupported;  // "no tiled copy": not an error
   }
   st.tile_col_blocks = cb;
   st.tile_row_blocks = rb;
@@ -445,7 +455,8 @@ static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* 
   if (e == hipSuccess) e = hipMalloc(&d_coo, nnz * sizeof(int));
   if (e == hipSuccess) e = hipMalloc(&d_key, nnz * sizeof(unsigned));
   if (e == hipSuccess) e = hipMalloc(&d_key2, nnz * sizeof(unsigned));
-  // 4-byte values are sorted together with their keys (64-bit payloads); wider ones through a permutation
+  // 4-byte values: the local indices are sorted together with the keys (64-bit payloads that also carry
+  // the entry's position); wider ones through a permutation alone
   constexpr bool kPayloadSort = sizeof(T) == 4;
   constexpr size_t kSortValBytes = kPayloadSort ? sizeof(unsigned long long) : sizeof(unsigned);
   if (e == hipSuccess) e = hipMalloc(&d_idx, nnz * kSortValBytes);
@@ -465,7 +476,7 @@ static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* 
     e = (hipError_t)asamd_csr2coo_ws(stream, row_ptr, st.nnz, st.m, d_coo, st.base, d_key2, (size_t)nnz * sizeof(unsigned));
   if (e == hipSuccess) {
     if constexpr (kPayloadSort) {
-      tile_keys_payload_kernel<<<256 * 32, 256, 0, stream>>>(st.nnz, d_coo, col_ind, (const unsigned*)val, st.base, d_cgb,
+      tile_keys_payload_kernel<<<256 * 32, 256, 0, stream>>>(st.nnz, d_coo, col_ind, st.base, d_cgb,
                                                              d_cbs, d_rgb, p->d_row_block_start, rb, d_key,
                                                              (unsigned long long*)d_idx);
       e = sort_pairs_u32_u64(stream, d_key, d_key2, (unsigned long long*)d_idx, (unsigned long long*)d_perm, nnz, key_bits);
@@ -474,14 +485,19 @@ static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* 
       e = sort_pairs_u32(stream, d_key, d_key2, d_idx, d_perm, nnz, key_bits);
     }
   }
+  if (e == hipSuccess && kPayloadSort) e = hipMalloc(&p->d_tperm, nnz * sizeof(unsigned));
   if (e == hipSuccess) {
-    if constexpr (kPayloadSort)
-      tile_unpack_kernel<<<256 * 32, 256, 0, stream>>>(st.nnz, (const unsigned long long*)d_perm, (unsigned*)p->d_tval,
+    if constexpr (kPayloadSort) {
+      tile_unpack_kernel<<<256 * 32, 256, 0, stream>>>(st.nnz, (const unsigned long long*)d_perm, p->d_tperm,
                                                        p->d_tcol, p->d_trow);
-    else
+      gather_values_kernel<T, false><<<256 * 32, 256, 0, stream>>>(st.nnz, p->d_tperm, val, (T*)p->d_tval);
+    } else {
       tile_gather_kernel<T><<<256 * 32, 256, 0, stream>>>(st.nnz, d_perm, d_coo, col_ind, val, st.base, d_cgb, d_cbs,
                                                           d_rgb, p->d_row_block_start, (T*)p->d_tval,
                                                           p->d_tcol, p->d_trow);
+      p->d_tperm = d_perm;  // the sorted permutation stays with the plan
+      d_perm = nullptr;
+    }
     tile_bounds_kernel<<<(unsigned)((tiles + 1 + 255) / 256), 256, 0, stream>>>(st.nnz, d_key2, tiles,
                                                                                 d_tile_ptr);
     // Entries in tiles of 65..128 entries: if they are few, phase 2 runs in its one-entry-per-lane form
@@ -565,7 +581,8 @@ static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* 
     if (d) (void)hipFree(d);
   if (e != hipSuccess) {
     free_tiled(p);
-    return e;
+    // too many blocks for the tile tables: the matrix simply gets no tiled copy (tiled_built stays 0)
+    return e == hipErrorNotSupported ? hipSuccess : e;
   }
   st.tiled_built = 1;
   return hipSuccess;
@@ -840,8 +857,9 @@ static hipError_t build_transpose(hipStream_t stream, asamd_csr_plan* p, const i
     }
     if (e == hipSuccess) e = hipStreamSynchronize(stream);
   }
-  for (void* d : {(void*)d_coo, (void*)d_key, (void*)d_key2, (void*)d_idx, (void*)d_perm})
+  for (void* d : {(void*)d_coo, (void*)d_key, (void*)d_key2, (void*)d_idx})
     if (d) (void)hipFree(d);
+  t.d_perm = d_perm;  // kept: the values of the copy can be gathered again through it
   if (e == hipSuccess)
     e = plan_create(stream, n, st.m, nnz, t.d_row_ptr, t.d_col, t.d_val, 0, DtypeOf<T>::value, /*trusted=*/1,
                     &t.plan);
@@ -860,6 +878,7 @@ static int build_transpose_any(hipStream_t stream, asamd_csr_plan* p, const int3
   if (which == 1 && !is_complex(p)) return hipErrorInvalidValue;
   if (p->st.transpose_built & (1 << which)) return hipSuccess;
   if (p->st.nnz == 0) return hipSuccess;  // the scatter route has nothing to add
+  if (p->st.first_offset != 0) return hipSuccess;  // no copy (csr2coo counts from position 0): the scatter route serves
   return by_dtype(p->dtype, [&](auto* tag) -> hipError_t {
     using T = std::remove_pointer_t<decltype(tag)>;
     return build_transpose<T>(stream, p, row_ptr, col_ind, (const T*)val, which);
@@ -899,6 +918,76 @@ extern "C" int asamd_csr_plan_transpose_arrays(const asamd_csr_plan* p, int32_t 
   return hipSuccess;
 }
 
+// The copies of a plan hold values: gather them again from `val` (the array the copies were laid out
+// from, or one with the same structure).  Only kernels, on `stream`; nothing is allocated or waited for.
+template <typename T>
+static hipError_t refresh_values(hipStream_t stream, asamd_csr_plan* p, const int* row_ptr, const int* col_ind,
+                                 const T* val) {
+  const asamd_csr_stats& st = p->st;
+  hipError_t e = hipSuccess;
+  if (st.tiled_built) {
+    if (!p->d_tperm) return hipErrorInvalidValue;
+    gather_values_kernel<T, false><<<256 * 32, 256, 0, stream>>>(st.nnz, p->d_tperm, val, (T*)p->d_tval);
+    e = hipGetLastError();
+  }
+  if (e == hipSuccess && st.ell_built) {
+    if constexpr (sizeof(T) == 4)
+      e = (hipError_t)asamd_s_csr2ell(stream, st.m, (const float*)val, row_ptr, col_ind, st.base, 0, st.ell_width,
+                                      (float*)p->d_eval, p->d_ecol);
+    else if constexpr (sizeof(T) == 8)
+      e = (hipError_t)asamd_d_csr2ell(stream, st.m, (const double*)val, row_ptr, col_ind, st.base, 0, st.ell_width,
+                                      (double*)p->d_eval, p->d_ecol);
+    else
+      e = (hipError_t)asamd_z_csr2ell(stream, st.m, (const asamd_complex16*)val, row_ptr, col_ind, st.base, 0,
+                                      st.ell_width, (asamd_complex16*)p->d_eval, p->d_ecol);
+  }
+  if (e == hipSuccess && (st.tiled_built || st.ell_built)) p->copy_val_src = val;
+  for (int which = 0; which < 2 && e == hipSuccess; ++which) {
+    asamd_csr_plan::TransCopy& t = p->tr[which];
+    if (!t.plan) continue;
+    if (!t.d_perm) return hipErrorInvalidValue;
+    if (which == 1)
+      gather_values_kernel<T, true><<<256 * 32, 256, 0, stream>>>(st.nnz, t.d_perm, val, (T*)t.d_val);
+    else
+      gather_values_kernel<T, false><<<256 * 32, 256, 0, stream>>>(st.nnz, t.d_perm, val, (T*)t.d_val);
+    e = hipGetLastError();
+    t.val_src = val;
+    // the transposed copy has a plan of its own, which may hold copies of the copy's values
+    if (e == hipSuccess) e = refresh_values<T>(stream, t.plan, t.d_row_ptr, t.d_col, (const T*)t.d_val);
+  }
+  return e;
+}
+
+extern "C" int asamd_csr_plan_refresh_values(hipStream_t stream, asamd_csr_plan* p, const int32_t* row_ptr,
+                                             const int32_t* col_ind, const void* val) {
+  if (!p || !row_ptr || !col_ind || !val || !p->st.trusted) return hipErrorInvalidValue;
+  if ((uintptr_t)val % (size_t)p->val_size) return hipErrorInvalidValue;
+  return by_dtype(p->dtype, [&](auto* tag) -> hipError_t {
+    using T = std::remove_pointer_t<decltype(tag)>;
+    return refresh_values<T>(stream, p, row_ptr, col_ind, (const T*)val);
+  });
+}
+
+extern "C" int asamd_csr_structure_hash(hipStream_t stream, int32_t m, int32_t nnz, const int32_t* row_ptr,
+                                        const int32_t* col_ind, uint64_t* hash_host) {
+  if (!row_ptr || !hash_host || m < 0 || nnz < 0 || (nnz > 0 && !col_ind)) return hipErrorInvalidValue;
+  unsigned long long* d_hash = nullptr;
+  hipError_t e = hipMalloc(&d_hash, sizeof(unsigned long long));
+  if (e != hipSuccess) return e;
+  e = hipMemsetAsync(d_hash, 0, sizeof(unsigned long long), stream);
+  if (e == hipSuccess) {
+    index_hash_kernel<<<256 * 8, 256, 0, stream>>>((int64_t)m + 1, row_ptr, 0x1234567ull, d_hash);
+    if (nnz > 0) index_hash_kernel<<<256 * 16, 256, 0, stream>>>((int64_t)nnz, col_ind, 0xABCDEF01ull << 8, d_hash);
+    e = hipGetLastError();
+  }
+  unsigned long long h = 0;
+  if (e == hipSuccess) e = hipMemcpyAsync(&h, d_hash, sizeof(h), hipMemcpyDeviceToHost, stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(stream);
+  (void)hipFree(d_hash);
+  *hash_host = (uint64_t)h;
+  return e;
+}
+
 extern "C" const asamd_csr_stats* asamd_csr_plan_stats(const asamd_csr_plan* p) {
   return p ? &p->st : nullptr;
 }
@@ -925,8 +1014,11 @@ extern "C" int asamd_csr_plan_set_algo(asamd_csr_plan* p, int32_t algo) {
       if (!p->st.ell_built) return hipErrorInvalidValue;
       p->st.algo = algo;
       return hipSuccess;
-    case ASAMD_SPMV_VECTOR:
     case ASAMD_SPMV_MERGE:
+      if (p->st.first_offset != 0) return hipErrorInvalidValue;
+      p->st.algo = algo;
+      return hipSuccess;
+    case ASAMD_SPMV_VECTOR:
     case ASAMD_SPMV_SCALAR:
       p->st.algo = algo;
       return hipSuccess;
@@ -974,6 +1066,7 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
     if (!aligned || !rowconst_ok(p)) algo = ASAMD_SPMV_VECTOR;
   }
   if (algo == ASAMD_SPMV_STREAM && !stream_ok(p)) algo = ASAMD_SPMV_MERGE;
+  if (algo == ASAMD_SPMV_MERGE && st.first_offset != 0) algo = ASAMD_SPMV_VECTOR;
   if (algo == ASAMD_SPMV_TILED && !st.tiled_built) algo = p->auto_algo == ASAMD_SPMV_TILED ? ASAMD_SPMV_MERGE : p->auto_algo;
   if (algo == ASAMD_SPMV_ELL && !st.ell_built) algo = p->auto_algo == ASAMD_SPMV_ELL ? ASAMD_SPMV_MERGE : p->auto_algo;
   switch (algo) {
@@ -1102,7 +1195,16 @@ static int csrmv_trans_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* 
   if (((uintptr_t)val | (uintptr_t)x | (uintptr_t)y) % alignof(T)) return hipErrorInvalidValue;
   const asamd_csr_stats& st = p->st;
   asamd_csr_plan::TransCopy& t = p->tr[which];
-  if (!t.plan && p->lazy_transpose && st.trusted && st.nnz > 0) {
+  // A library-owned mirror lays out its copy of the transpose on the first transposed multiply: that
+  // allocates and waits, which a stream under capture must not do -- such a call scatters instead, and
+  // the copy is laid out by the first call outside a capture.
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (!t.plan && p->lazy_transpose && hipStreamIsCapturing(s, &capturing) != hipSuccess) {
+    (void)hipGetLastError();
+    capturing = hipStreamCaptureStatusActive;  // unknown: do not risk it
+  }
+  if (!t.plan && p->lazy_transpose && st.trusted && st.nnz > 0 && st.first_offset == 0 &&
+      capturing == hipStreamCaptureStatusNone) {
     const hipError_t e = build_transpose<T>(s, p, rp, ci, val, which);
     if (e == hipErrorOutOfMemory) {
       (void)hipGetLastError();  // no room for the copy: scatter instead, and do not try again

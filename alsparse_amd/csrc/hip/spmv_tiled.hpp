@@ -152,12 +152,14 @@ __global__ __launch_bounds__(256) void tile_keys_kernel(int nnz, const int* __re
   }
 }
 
-// For 4-byte values the entry itself travels with its key through the sort: payload = value bits
-// (high word) | column local to its block << 16 | row local to its block.  Gathering the three CSR
-// streams through the sorted permutation afterwards moves a 128-byte line per entry and stream
-// (18 ms for 2^28 entries, against 3 ms more in the sort and a streaming unpack).
+// For 4-byte values the entry's position and local indices travel with its key through the sort:
+// payload = entry index (high word) | column local to its block << 16 | row local to its block.
+// Gathering all three CSR streams through the sorted permutation afterwards moves a 128-byte line per
+// entry and stream (18 ms for 2^28 entries, against 3 ms more in the sort and a streaming unpack); only
+// the values are gathered that way (gather_values_kernel), and the permutation is kept so that they can
+// be gathered again when the caller has changed them.
 __global__ __launch_bounds__(256) void tile_keys_payload_kernel(
-    int nnz, const int* __restrict__ coo_row, const int* __restrict__ col_ind, const unsigned* __restrict__ val_bits,
+    int nnz, const int* __restrict__ coo_row, const int* __restrict__ col_ind,
     int base, const int* __restrict__ col_group_block, const int* __restrict__ col_block_start,
     const int* __restrict__ row_group_block, const int* __restrict__ row_block_start, int row_blocks,
     unsigned* __restrict__ key, unsigned long long* __restrict__ payload) {
@@ -168,20 +170,64 @@ __global__ __launch_bounds__(256) void tile_keys_payload_kernel(
     const unsigned rb = (unsigned)row_group_block[row >> kRowGroupLog2];
     key[k] = cb * (unsigned)row_blocks + rb;
     const unsigned lc = (unsigned)(col - col_block_start[cb]), lr = (unsigned)(row - row_block_start[rb]);
-    payload[k] = ((unsigned long long)val_bits[k] << 32) | (lc << 16) | lr;
+    payload[k] = ((unsigned long long)(unsigned)k << 32) | (lc << 16) | lr;
   }
 }
 
 __global__ __launch_bounds__(256) void tile_unpack_kernel(int nnz, const unsigned long long* __restrict__ payload,
-                                                          unsigned* __restrict__ t_val_bits,
+                                                          unsigned* __restrict__ t_perm,
                                                           unsigned short* __restrict__ t_col,
                                                           unsigned short* __restrict__ t_row) {
   for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < nnz;
        q += (int64_t)gridDim.x * blockDim.x) {
     const unsigned long long w = payload[q];
-    t_val_bits[q] = (unsigned)(w >> 32);
+    t_perm[q] = (unsigned)(w >> 32);
     t_col[q] = (unsigned short)(w >> 16);
     t_row[q] = (unsigned short)w;
+  }
+}
+
+// out[q] = val[perm[q]] (CONJ: conjugated): the values of a re-ordered copy, taken afresh from the
+// caller's array.  Eight gathers in flight per lane.
+template <typename T, bool CONJ>
+__global__ __launch_bounds__(256) void gather_values_kernel(int nnz, const unsigned* __restrict__ perm,
+                                                            const T* __restrict__ val, T* __restrict__ out) {
+  constexpr int kU = 8;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  for (; q + (kU - 1) * stride < nnz; q += kU * stride) {
+    unsigned k[kU];
+    T v[kU];
+#pragma unroll
+    for (int u = 0; u < kU; ++u) k[u] = nt_load(perm + q + u * stride);
+#pragma unroll
+    for (int u = 0; u < kU; ++u) v[u] = val[k[u]];
+#pragma unroll
+    for (int u = 0; u < kU; ++u) out[q + u * stride] = CONJ ? conj_t(v[u]) : v[u];
+  }
+  for (; q < nnz; q += stride) out[q] = CONJ ? conj_t(val[perm[q]]) : val[perm[q]];
+}
+
+// hash[0] += sum over i of mix(a[i], i + salt): a fingerprint of an index array that does not depend on
+// the order of the (integer, wrapping) additions.
+__device__ __forceinline__ unsigned long long mix_index(unsigned long long v, unsigned long long i) {
+  unsigned long long z = (v + 0x9E3779B97F4A7C15ull) * 0xBF58476D1CE4E5B9ull ^ (i * 0x94D049BB133111EBull);
+  z = (z ^ (z >> 29)) * 0xD6E8FEB86659FD93ull;
+  return z ^ (z >> 32);
+}
+__global__ __launch_bounds__(256) void index_hash_kernel(int64_t n, const int* __restrict__ a, unsigned long long salt,
+                                                         unsigned long long* __restrict__ hash) {
+  __shared__ unsigned long long s_sum[256 / kWave];
+  unsigned long long mine = 0;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
+    mine += mix_index((unsigned long long)(unsigned)nt_load(a + i), (unsigned long long)i + salt);
+  for (int d = kWave / 2; d > 0; d >>= 1) mine += __shfl_down(mine, d, kWave);
+  if (threadIdx.x % kWave == 0) s_sum[threadIdx.x / kWave] = mine;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    unsigned long long total = 0;
+    for (int w = 0; w < 256 / kWave; ++w) total += s_sum[w];
+    atomicAdd(hash, total);
   }
 }
 

@@ -180,3 +180,8 @@ int asamd_env_algo(void) {
   if (!strcmp(e, "ell")) return ASAMD_SPMV_ELL;
   return ASAMD_SPMV_AUTO;
 }
+
+int asamd_env_structure_only(void) {
+  const char *e = getenv("ALSPARSE_AMD_ANALYSIS");
+  return e && !strcmp(e, "structure");
+}

@@ -28,6 +28,23 @@ static alphasparse_status_t asamd_host_prepare(const alphasparse_matrix_t A, alp
     r = asamd_registry_find(ASAMD_KEY_MATRIX, m->d_row_ptr);
     if (!r) return ALPHA_SPARSE_STATUS_INTERNAL_ERROR;
   }
+  /* The host arrays stay the caller's to change (alphasparse_?_export_csr hands out pointers into them, and
+   * the reference's CPU kernels read them on every call).  A cheap fingerprint of a sample of the values tells
+   * when they have been rewritten: the mirror's values are copied again and the copies that its analysis
+   * keeps are refreshed.  (A change of a few single values can slip through the sample: host2device_?_csr
+   * mirrors afresh.) */
+  static const size_t kElem[4] = {4, 8, 8, 16};
+  const size_t elem = kElem[A->datatype & 3];
+  const size_t nnz = (size_t)(m->rows > 0 && m->rows_end[m->rows - 1] > 0 ? m->rows_end[m->rows - 1] : 0);
+  if (nnz > 0 && r->plan) {
+    const uint64_t fp = asamd_host_fingerprint(m->values, nnz, elem);
+    if (fp != r->host_val_fingerprint) {
+      ASAMD_HIP_STATUS(hipStreamSynchronize((*h)->stream));
+      ASAMD_HIP_STATUS(hipMemcpy(m->d_values, m->values, nnz * elem, hipMemcpyHostToDevice));
+      ASAMD_HIP_STATUS(asamd_csr_plan_refresh_values((*h)->stream, r->plan, m->d_row_ptr, m->d_col_indx, m->d_values));
+      r->host_val_fingerprint = fp;
+    }
+  }
   *rec = r;
   return ALPHA_SPARSE_STATUS_SUCCESS;
 }

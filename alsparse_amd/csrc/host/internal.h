@@ -24,6 +24,11 @@ typedef struct asamd_record {
   const void *col_ind;
   int32_t m, n, nnz, base, dtype; /* dtype: enum asamd_dtype == alphasparse_datatype_t */
   asamd_csr_plan *plan;
+  /* explicit analyses: fingerprint of the structure arrays at analysis time (asamd_csr_structure_hash) */
+  uint64_t structure_hash;
+  int has_structure_hash;
+  /* library-built mirrors: fingerprint of a sample of the HOST values at the time they were copied */
+  uint64_t host_val_fingerprint;
   /* host-pointer entry points: device staging for x / y (ASAMD_KEY_MATRIX only) */
   void *d_in;
   size_t d_in_bytes;
@@ -48,11 +53,18 @@ alphasparse_status_t asamd_plan_for_call(alphasparse_dcu_handle_t handle, const 
                                          int32_t n, int32_t nnz, int32_t base, int32_t dtype,
                                          asamd_csr_plan **plan);
 
+/* Fingerprint of up to 1024 evenly spread elements (elem bytes each) of a host array: cheap enough to
+ * take on every host-pointer multiply, and changes whenever a caller has rewritten the array as a whole. */
+uint64_t asamd_host_fingerprint(const void *values, size_t count, size_t elem);
+
 /* Process-wide handle for alphasparse_?_mv / _mm (host pointers). */
 alphasparse_status_t asamd_default_handle(alphasparse_dcu_handle_t *handle);
 
 /* ALSPARSE_AMD_SPMV_ALGO = auto | vector | rowconst | merge | scalar | tiled | stream | ell */
 int asamd_env_algo(void);
+/* ALSPARSE_AMD_ANALYSIS = structure: analyses keep no copies of the matrix values (as the reference's),
+ * so values may change in place at any time; the default lets an analysis keep re-ordered copies. */
+int asamd_env_structure_only(void);
 
 /* device arrays of values must be aligned to their element size (one element = one load) */
 #define ASAMD_MISALIGNED(T, p) (((uintptr_t)(p)) % sizeof(T) != 0)

@@ -117,6 +117,19 @@ alphasparse_status_t asamd_plan_for_call(alphasparse_dcu_handle_t handle, const 
   return ALPHA_SPARSE_STATUS_SUCCESS;
 }
 
+uint64_t asamd_host_fingerprint(const void *values, size_t count, size_t elem) {
+  const unsigned char *p = (const unsigned char *)values;
+  const size_t samples = count < 1024 ? count : 1024;
+  uint64_t h = 0x9E3779B97F4A7C15ull ^ (uint64_t)count;
+  for (size_t s = 0; s < samples; ++s) {
+    /* sample s sits at a fixed position of its 1/samples share of the array */
+    const size_t i = (size_t)(((unsigned __int128)s * count) / samples) + (s * 2654435761u) % (count / samples ? count / samples : 1);
+    const unsigned char *q = p + (i < count ? i : count - 1) * elem;
+    for (size_t b = 0; b < elem; ++b) h = (h ^ q[b]) * 0x100000001B3ull;
+  }
+  return h;
+}
+
 static alphasparse_dcu_handle_t g_default_handle;
 
 alphasparse_status_t asamd_default_handle(alphasparse_dcu_handle_t *handle) {

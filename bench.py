@@ -225,11 +225,20 @@ def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False, vendor=Fa
         d_y.copy_from(y0)
 
     t = time_steps(step, steps, warmup, hiprt)
+    # the analysis repeated on the same arrays, as a caller does after rewriting csr_val in place: the structure
+    # is fingerprinted, found unchanged, and only the values of the plan's copies are gathered again
+    hiprt.synchronize()
+    t0 = time.perf_counter()
+    st = getattr(lib, "alphasparse_dcu_%s_csrmv_analysis" % p)(
+        h.h, op, a.rows, a.cols, a.nnz, byref(descr), d_val.c_ptr(), d_rp.c_ptr(), d_ci.c_ptr(), info)
+    hiprt.synchronize()
+    reanalysis_ms = (time.perf_counter() - t0) * 1e3
+    assert st == 0, "repeated analysis status %d" % st
     nbytes = (wl.spmv_bytes(a.cols, a.rows, a.nnz, a.dtype.itemsize, beta) if transpose
               else wl.spmv_bytes(a.rows, a.cols, a.nnz, a.dtype.itemsize, beta))
     opname = "" if not transpose else (" -- CONJUGATE-TRANSPOSED operation" if op == 2 else " -- TRANSPOSED operation")
     res = {"workload": workload_name + (" -- COMPLEX values (%s)" % a.dtype.name if cx else "") + opname, "rows": a.rows, "nnz": a.nnz, "algorithmic_bytes": int(nbytes),
-           "flops": 2 * a.nnz, "kernel": algo, "analysis_ms": analysis_ms, "timing": t,
+           "flops": 2 * a.nnz, "kernel": algo, "analysis_ms": analysis_ms, "reanalysis_ms": reanalysis_ms, "timing": t,
            "gbs": nbytes / t["avg_ms"] / 1e6, "gflops": 2 * a.nnz / t["avg_ms"] / 1e6,
            "dtype": {"float32": "f32", "float64": "f64", "complex64": "c64", "complex128": "c128"}[a.dtype.name],
            "parity": parity}
@@ -548,7 +557,7 @@ def brief(r):
     t = r["timing"]
     return {"workload": r["workload"], "kernel": r.get("kernel"), "dtype": r["dtype"], "ms": t["avg_ms"], "min_ms": t["min_ms"],
             "gbs": r["gbs"], "gflops": r["gflops"], "hbm_frac": r["hbm_frac"], "algorithmic_bytes": r["algorithmic_bytes"],
-            "analysis_ms": r.get("analysis_ms"), "parity": r["parity"], "traffic": r.get("traffic"),
+            "analysis_ms": r.get("analysis_ms"), "reanalysis_ms": r.get("reanalysis_ms"), "parity": r["parity"], "traffic": r.get("traffic"),
             "traffic_source": r.get("traffic_source")}
 
 
@@ -685,7 +694,8 @@ def main():
         "ms_per_step": t["avg_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": main_res["dtype"], "data": "synthetic",
         "config": {"workload": main_res["workload"], "rows": main_res["rows"], "nnz": main_res["nnz"],
-                   "kernel": main_res.get("kernel", "spmm row-major"), "analysis_ms": main_res.get("analysis_ms")},
+                   "kernel": main_res.get("kernel", "spmm row-major"), "analysis_ms": main_res.get("analysis_ms"),
+                   "reanalysis_ms": main_res.get("reanalysis_ms")},
         "gflops": main_res["gflops"], "pct_of_hbm_peak": 100.0 * main_res["hbm_frac"],
         "min_ms": t["min_ms"], "median_ms": t["median_ms"], "wall_ms_per_step": t["wall_ms_per_step"],
         "parity": main_res["parity"],

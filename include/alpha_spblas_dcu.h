@@ -180,8 +180,17 @@ alphasparse_status_t alphasparse_d_mv_dcu(alphasparse_dcu_handle_t handle,
  * include/alphasparse/spapi_dcu.h:527-547; validation order from
  * src/util_cpp/alphasparse_dcu_x_csrmv_analysis.cpp:269-333.  Runs on the GPU:
  * row-length statistics and histogram, kernel selection, merge-path block
- * coordinates.  Results stay valid while the sparsity structure behind
- * csr_row_ptr is unchanged; call alphasparse_dcu_csrmv_clear before changing it. */
+ * coordinates, and -- where a timing run inside the analysis shows that it pays --
+ * a re-ordered copy of the matrix (tiled, ELL, transposed) that later multiplies
+ * read INSTEAD of csr_val.  The reference's analysis keeps structure only
+ * (:382-388), so the rule for callers is one the reference does not have:
+ *   after writing new values into csr_val, call the analysis again
+ * with the same arguments.  It notices that the structure arrays are unchanged
+ * (a fingerprint of csr_row_ptr / csr_col_ind: one streaming pass) and only
+ * gathers the values again; a changed structure is laid out afresh.  With the
+ * environment variable ALSPARSE_AMD_ANALYSIS=structure no analysis keeps values
+ * at all: multiplies then always read csr_val, at the speed of the row kernels.
+ * Call alphasparse_dcu_csrmv_clear to forget an analysis. */
 alphasparse_status_t alphasparse_dcu_s_csrmv_analysis(
     alphasparse_dcu_handle_t handle, alphasparse_operation_t trans, ALPHA_INT m, ALPHA_INT n,
     ALPHA_INT nnz, const alpha_dcu_matrix_descr_t descr, const float *csr_val,

@@ -150,6 +150,19 @@ int asamd_s_csrmv_noalloc(hipStream_t stream, int32_t m, int32_t n, int32_t nnz,
                           const float *val, const int32_t *row_ptr, const int32_t *col_ind, const float *x,
                           float beta, float *y);
 
+/* A trusted plan may hold re-ordered copies of the matrix VALUES (tiled, ELL, transposed); the
+ * reference's analysis keeps structure only (src/util_cpp/alphasparse_dcu_x_csrmv_analysis.cpp:382-388).
+ * When the caller has changed the values behind `val` in place (same structure), this gathers every
+ * copy again through the permutations that the plan kept: streaming kernels on `stream` only, no sort,
+ * no allocation, no wait.  row_ptr / col_ind are the arrays the plan was created for. */
+int asamd_csr_plan_refresh_values(hipStream_t stream, asamd_csr_plan *plan, const int32_t *row_ptr,
+                                  const int32_t *col_ind, const void *val);
+/* 64-bit fingerprint of the structure arrays (m + 1 offsets, nnz column indices): equal arrays give equal
+ * values; used to tell a changed structure from changed values when an analysis is repeated.
+ * Synchronises `stream`; *hash_host is a host word. */
+int asamd_csr_structure_hash(hipStream_t stream, int32_t m, int32_t nnz, const int32_t *row_ptr,
+                             const int32_t *col_ind, uint64_t *hash_host);
+
 /* CSR copy of the transpose, owned by the plan (trusted plans only; row_ptr,
  * col_ind, val are the arrays the plan was created for).  Later transposed
  * multiplies run the ordinary kernels on that copy (with an analysis of its

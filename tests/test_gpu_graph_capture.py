@@ -143,3 +143,64 @@ def test_every_kernel_family_replays_from_a_hip_graph(gpu, algo):
         for d in (dx, dy):
             d.free()
         da.free()
+
+
+def test_first_transposed_multiply_of_a_mirror_can_be_captured(gpu):
+    """A library-built mirror lays out its copy of the transpose on the first transposed multiply -- which
+    allocates and waits, so a call under stream capture scatters with atomics instead (kernels only); the
+    copy is laid out by the first transposed multiply outside a capture."""
+    from ctypes import POINTER, cast, c_float
+    lib, hip = capi.load(), hiprt.lib()
+    a = wl.powerlaw_rmat(13, 3000, np.float32)
+    x, y0 = wl.uniform(a.rows, a.dtype, 3), wl.uniform(a.cols, a.dtype, 4)
+    A = capi.alphasparse_matrix_t()
+    rs, re = np.ascontiguousarray(a.row_ptr[:-1]), np.ascontiguousarray(a.row_ptr[1:])
+    assert lib.alphasparse_s_create_csr(byref(A), a.base, a.rows, a.cols, capi.ptr(rs), capi.ptr(re), capi.ptr(a.col_ind),
+                                        capi.ptr(a.values)) == 0
+    dx, dy = hiprt.DeviceArray.from_numpy(x), hiprt.DeviceArray.from_numpy(y0)
+    stream, graph, gexec = c_void_p(), c_void_p(), c_void_p()
+    hiprt.check(hip.hipStreamCreate(byref(stream)), "hipStreamCreate")
+    h = capi.Handle()
+    descr = capi.make_descr()
+    al, be = c_float(1.25), c_float(0.5)
+    T = capi.ALPHA_SPARSE_OPERATION_TRANSPOSE
+
+    def multiply():
+        return lib.alphasparse_s_mv_dcu(h.h, T, byref(al), A, byref(descr), dx.c_ptr(), byref(be), dy.c_ptr())
+
+    def verify(y, what):
+        ref = orc.csrmv_trans_plain(a, 1.25, x, 0.5, y0)
+        err = orc.csrmv_err(orc.transpose(a), 1.25, x, 0.5, y0, y, ref)
+        assert err.zero_den_mismatch == 0 and err.full <= TOL[a.dtype], (what, err)
+    try:
+        assert lib.host2device_s_csr(A) == 0
+        key = cast(A.contents.mat, POINTER(capi.spmat_csr_s_t)).contents.d_row_ptr
+        assert lib.asamd_handle_set_stream(h.h, stream) == 0
+        announce("graph capture: first transposed multiply of a mirror")
+        hiprt.check(hip.hipStreamBeginCapture(stream, 0), "hipStreamBeginCapture")
+        st = multiply()
+        hiprt.check(hip.hipStreamEndCapture(stream, byref(graph)), "hipStreamEndCapture")
+        assert st == 0
+        assert not lib.asamd_analysis_transpose_stats(key), "no copy may be laid out under capture"
+        hiprt.check(hip.hipGraphInstantiate(byref(gexec), graph, None, None, ctypes.c_size_t(0)), "hipGraphInstantiate")
+        for replay in range(3):
+            dy.copy_from(y0)
+            hiprt.synchronize()
+            hiprt.check(hip.hipGraphLaunch(gexec, stream), "hipGraphLaunch")
+            hiprt.check(hip.hipStreamSynchronize(stream), "sync")
+            verify(dy.to_numpy(), "replay %d" % replay)
+        dy.copy_from(y0)
+        assert multiply() == 0                                   # eager: lays out the copy and uses it
+        hiprt.check(hip.hipStreamSynchronize(stream), "sync")
+        verify(dy.to_numpy(), "eager after the capture")
+        assert lib.asamd_analysis_transpose_stats(key), "the eager call lays out the copy of the transpose"
+    finally:
+        if gexec:
+            hip.hipGraphExecDestroy(gexec)
+        if graph:
+            hip.hipGraphDestroy(graph)
+        h.close()
+        hip.hipStreamDestroy(stream)
+        lib.alphasparse_destroy(A)
+        for d in (dx, dy):
+            d.free()

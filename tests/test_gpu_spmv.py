@@ -479,3 +479,52 @@ def test_tiled_row_blocks_follow_the_tile_population(gpu, m, n, per_row):
     finally:
         lib.alphasparse_dcu_destroy_mat_info(info)
         da.free()
+
+
+@pytest.mark.parametrize("maker", [lambda: wl.powerlaw_rmat(13, 3000, np.float32), lambda: wl.uniform_rows(5000, 7000, 16, np.float32),
+                                   lambda: wl.laplace2d(64, 48, np.float32)], ids=["powerlaw", "uniform16", "laplace"])
+def test_row_ptr_into_the_middle_of_larger_arrays(gpu, maker):
+    """row_ptr[0] > base: the matrix is a row slice of a larger one whose col / val arrays are passed whole.
+    The reference's kernel indexes with the absolute offsets (dcu_gemv_vector.h:38-45); every path here must
+    see the same entries: un-analysed, analysed (no merge-path, no re-ordered copy) and transposed."""
+    lib = capi.load()
+    a = maker()
+    lead = 777
+    rng = np.random.default_rng(5)
+    big = wl.Csr(a.rows, a.cols, (a.row_ptr + lead).astype(np.int32),
+                 np.concatenate([rng.integers(0, a.cols, lead).astype(np.int32), a.col_ind]),
+                 np.concatenate([rng.uniform(-9, 9, lead).astype(a.dtype), a.values]), a.base, a.name + "+lead")
+    assert big.nnz == a.nnz + lead
+    x, y0 = _vectors(a)
+    xt, yt0 = wl.uniform(a.rows, a.dtype, 5), wl.uniform(a.cols, a.dtype, 6)
+    da = DeviceCsr(big)
+    da.a = wl.Csr(a.rows, a.cols, big.row_ptr, big.col_ind, big.values, a.base, big.name)
+    da.a.nnz = a.nnz  # what the caller passes as nnz: the entries of these rows
+    info = capi.alphasparse_dcu_mat_info_t()
+    assert lib.alphasparse_dcu_create_mat_info(byref(info)) == 0
+    descr = capi.make_descr(base=a.base)
+    try:
+        announce("row_ptr[0] > base", a.name)
+        check_spmv(a, 1.5, x, 0.5, y0, run_csrmv(gpu, da, 1.5, x, 0.5, y0), "un-analysed")
+        assert lib.alphasparse_dcu_s_csrmv_analysis(gpu.h, 1, a.rows, a.cols, a.nnz, byref(descr), da.val.c_ptr(),
+                                                    da.row_ptr.c_ptr(), da.col.c_ptr(), info) == 0
+        st = lib.asamd_analysis_stats(info).contents
+        assert st.first_offset == lead
+        assert st.algo in (capi.ASAMD_SPMV_VECTOR, capi.ASAMD_SPMV_STREAM), capi.ALGO_NAMES[st.algo]
+        assert st.tiled_built == 0 and st.ell_built == 0 and st.transpose_built == 0
+        check_spmv(a, 1.5, x, 0.5, y0, run_csrmv(gpu, da, 1.5, x, 0.5, y0, info), "analysed")
+        # transposed: the scatter route
+        dx, dy = hiprt.DeviceArray.from_numpy(xt), hiprt.DeviceArray.from_numpy(yt0)
+        al, be = c_float(1.5), c_float(0.5)
+        assert lib.alphasparse_dcu_s_csrmv(gpu.h, 1, a.rows, a.cols, a.nnz, byref(al), byref(descr), da.val.c_ptr(),
+                                           da.row_ptr.c_ptr(), da.col.c_ptr(), info, dx.c_ptr(), byref(be), dy.c_ptr()) == 0
+        hiprt.synchronize()
+        got = dy.to_numpy()
+        ref = orc.csrmv_trans_plain(a, 1.5, xt, 0.5, yt0)
+        err = orc.csrmv_err(orc.transpose(a), 1.5, xt, 0.5, yt0, got, ref)
+        assert err.zero_den_mismatch == 0 and err.full <= TOL[a.dtype], err
+        dx.free()
+        dy.free()
+    finally:
+        lib.alphasparse_dcu_destroy_mat_info(info)
+        da.free()
