@@ -317,6 +317,7 @@ _COMMON = {
     "asamd_handle_get_stream": [_P],
     "asamd_copy_bytes": [_P, _P, _P, c_size_t],
     "asamd_ceiling_kernel": [_P, _I, _P, _P, c_size_t, c_int64, _P, POINTER(c_int64)],
+    "asamd_registry_lazy_count": [],
     "asamd_analysis_stats": [_P],
     "asamd_analysis_transpose_stats": [_P],
     "asamd_analysis_set_algo": [_P, _I],

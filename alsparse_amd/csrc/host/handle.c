@@ -83,6 +83,7 @@ alphasparse_status_t alphasparse_dcu_get_handle(alphasparse_dcu_handle_t *handle
 
 alphasparse_status_t alphasparse_dcu_destory_handle(alphasparse_dcu_handle_t handle) {
   if (!handle) return ALPHA_SPARSE_STATUS_INVALID_HANDLE;
+  asamd_registry_drop_handle(handle); /* the analyses this handle made on its own for un-analysed matrices */
   (void)hipFree(handle->buffer);
   (void)hipFree(handle->sone);
   (void)hipFree(handle->done);

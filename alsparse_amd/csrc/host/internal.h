@@ -19,6 +19,12 @@ typedef enum {
 typedef struct asamd_record {
   asamd_key_kind kind;
   const void *key;
+  /* lazy records only: the handle the record belongs to, the multiplies that hold it at the moment, its
+   * last use (for evicting the oldest) and whether it has been taken out of the registry */
+  const void *owner;
+  int leases;
+  int dead;
+  uint64_t last_use;
   /* what the plan was built for; a lookup must match all of these */
   const void *row_ptr;
   const void *col_ind;
@@ -37,21 +43,28 @@ typedef struct asamd_record {
   struct asamd_record *next;
 } asamd_record;
 
-/* All registry calls are serialised by one mutex; records are returned
- * unlocked, which is safe as long as a matrix / info is not destroyed while
- * another thread multiplies with it (the reference gives no such guarantee
- * either). */
+/* All registry calls are serialised by one mutex.  Records of explicit analyses and of mirrors belong to
+ * an object of the caller's (an info bundle, a matrix handle) and are returned unlocked, which is safe as
+ * long as that object is not destroyed while another thread multiplies with it (the reference gives no such
+ * guarantee either).  Lazy records come and go on their own: see asamd_plan_for_call. */
 asamd_record *asamd_registry_find(asamd_key_kind kind, const void *key);
 asamd_record *asamd_registry_insert(asamd_key_kind kind, const void *key);
 void asamd_registry_erase(asamd_key_kind kind, const void *key);
 void asamd_record_release_device(asamd_record *rec);
 
 /* Plan for a multiply through the raw-pointer API: explicit analysis if `info`
- * is known and matches, else the lazy cache (created on first use). */
+ * is known and matches, else the mirror's, else the handle's lazy record for this row_ptr (created on
+ * first use; at most 64 are kept, the least recently used one makes room).  *lease is non-NULL when the plan
+ * belongs to a lazy record: pass it to asamd_plan_release once the multiply's kernels are enqueued. */
 alphasparse_status_t asamd_plan_for_call(alphasparse_dcu_handle_t handle, const void *info,
                                          const void *row_ptr, const void *col_ind, int32_t m,
                                          int32_t n, int32_t nnz, int32_t base, int32_t dtype,
-                                         asamd_csr_plan **plan);
+                                         asamd_csr_plan **plan, asamd_record **lease);
+void asamd_plan_release(asamd_record *lease);
+/* forgets the lazy records of a handle that is being destroyed */
+void asamd_registry_drop_handle(const void *handle);
+/* number of lazy records alive (tests) */
+int asamd_registry_lazy_count(void);
 
 /* Fingerprint of up to 1024 evenly spread elements (elem bytes each) of a host array: cheap enough to
  * take on every host-pointer multiply, and changes whenever a caller has rewritten the array as a whole. */

@@ -13,6 +13,13 @@
 
 static pthread_mutex_t g_lock = PTHREAD_MUTEX_INITIALIZER;
 static asamd_record *g_head[3];
+static int g_lazy_count;       /* live ASAMD_KEY_LAZY records */
+static uint64_t g_tick;        /* use counter: the lazy record with the smallest stamp is the oldest */
+
+/* At most this many lazily analysed matrices are remembered (each holds a few small device buffers); the
+ * least recently used one makes room.  A process that streams many un-analysed matrices through csrmv
+ * therefore holds a bounded amount of device memory. */
+#define ASAMD_LAZY_CAP 64
 
 asamd_record *asamd_registry_find(asamd_key_kind kind, const void *key) {
   pthread_mutex_lock(&g_lock);
@@ -63,10 +70,51 @@ static int record_matches(const asamd_record *r, const void *row_ptr, const void
          r->m == m && r->n == n && r->nnz == nnz && r->base == base && r->dtype == dtype;
 }
 
+/* ---- lazy records ------------------------------------------------------------------------------
+ * Keyed by (csr_row_ptr, handle): each handle analyses an un-analysed matrix for itself, so the
+ * scratch of such a plan (merge-path carries, rewritten by every multiply) is only ever used on one
+ * handle's stream.  A record is found, unlinked and freed under the lock; a multiply holds a lease
+ * (`leases`) from lookup until its kernels are enqueued, and a record that is replaced or evicted
+ * meanwhile (`dead`) is freed by the last lease that lets go.  hipFree waits for work in flight. */
+static asamd_record *lazy_unlink_locked(asamd_record *victim) {
+  asamd_record **pp = &g_head[ASAMD_KEY_LAZY];
+  while (*pp && *pp != victim) pp = &(*pp)->next;
+  if (*pp) {
+    *pp = victim->next;
+    victim->next = NULL;
+    victim->dead = 1;
+    --g_lazy_count;
+  }
+  return victim->leases == 0 ? victim : NULL; /* the caller frees it outside the lock */
+}
+
+static void lazy_free(asamd_record *r) {
+  if (!r) return;
+  asamd_record_release_device(r);
+  free(r);
+}
+
+void asamd_plan_release(asamd_record *lease) {
+  if (!lease) return;
+  asamd_record *to_free = NULL;
+  pthread_mutex_lock(&g_lock);
+  if (--lease->leases == 0 && lease->dead) to_free = lease;
+  pthread_mutex_unlock(&g_lock);
+  lazy_free(to_free);
+}
+
+int asamd_registry_lazy_count(void) {
+  pthread_mutex_lock(&g_lock);
+  const int n = g_lazy_count;
+  pthread_mutex_unlock(&g_lock);
+  return n;
+}
+
 alphasparse_status_t asamd_plan_for_call(alphasparse_dcu_handle_t handle, const void *info,
                                          const void *row_ptr, const void *col_ind, int32_t m,
                                          int32_t n, int32_t nnz, int32_t base, int32_t dtype,
-                                         asamd_csr_plan **plan) {
+                                         asamd_csr_plan **plan, asamd_record **lease) {
+  *lease = NULL;
   /* 1. an explicit analysis of exactly these arrays (info may be garbage: it is
    *    only ever compared by address, never dereferenced) */
   if (info) {
@@ -84,24 +132,37 @@ alphasparse_status_t asamd_plan_for_call(alphasparse_dcu_handle_t handle, const 
       return ALPHA_SPARSE_STATUS_SUCCESS;
     }
   }
-  /* 3. lazy: statistics cached per row_ptr address.  The structure behind the
+  /* 3. lazy: statistics cached per (row_ptr address, handle).  The structure behind the
    *    address may change without notice, so the plan is untrusted: it only
    *    steers the kernel choice, and every kernel it can pick reads row_ptr
    *    afresh on each call. */
-  asamd_record *r = asamd_registry_find(ASAMD_KEY_LAZY, row_ptr);
-  if (r && !record_matches(r, row_ptr, NULL, m, n, nnz, base, dtype)) {
-    asamd_registry_erase(ASAMD_KEY_LAZY, row_ptr);
-    r = NULL;
+  asamd_record *stale = NULL, *found = NULL;
+  pthread_mutex_lock(&g_lock);
+  for (asamd_record *r = g_head[ASAMD_KEY_LAZY]; r; r = r->next) {
+    if (r->key != row_ptr || r->owner != (const void *)handle) continue;
+    if (record_matches(r, row_ptr, NULL, m, n, nnz, base, dtype)) {
+      found = r;
+      ++r->leases;
+      r->last_use = ++g_tick;
+    } else {
+      stale = lazy_unlink_locked(r); /* another matrix lives at this address now */
+    }
+    break;
   }
-  if (!r) {
+  pthread_mutex_unlock(&g_lock);
+  lazy_free(stale);
+  if (!found) {
     asamd_csr_plan *p = NULL;
     ASAMD_HIP_STATUS(asamd_csr_plan_create_dtype(handle->stream, m, n, nnz, (const int32_t *)row_ptr,
-                                           NULL, NULL, base, dtype, /*trusted=*/0, &p));
-    r = asamd_registry_insert(ASAMD_KEY_LAZY, row_ptr);
+                                                 NULL, NULL, base, dtype, /*trusted=*/0, &p));
+    asamd_record *r = (asamd_record *)calloc(1, sizeof(*r));
     if (!r) {
       asamd_csr_plan_destroy(p);
       return ALPHA_SPARSE_STATUS_ALLOC_FAILED;
     }
+    r->kind = ASAMD_KEY_LAZY;
+    r->key = row_ptr;
+    r->owner = (const void *)handle;
     r->row_ptr = row_ptr;
     r->col_ind = col_ind;
     r->m = m;
@@ -110,11 +171,44 @@ alphasparse_status_t asamd_plan_for_call(alphasparse_dcu_handle_t handle, const 
     r->base = base;
     r->dtype = dtype;
     r->plan = p;
+    r->leases = 1;
     const int forced = asamd_env_algo();
     if (forced != ASAMD_SPMV_AUTO) (void)asamd_csr_plan_set_algo(p, forced);
+    asamd_record *evicted = NULL;
+    pthread_mutex_lock(&g_lock);
+    r->last_use = ++g_tick;
+    r->next = g_head[ASAMD_KEY_LAZY];
+    g_head[ASAMD_KEY_LAZY] = r;
+    if (++g_lazy_count > ASAMD_LAZY_CAP) {
+      asamd_record *oldest = NULL;
+      for (asamd_record *q = g_head[ASAMD_KEY_LAZY]; q; q = q->next)
+        if (q != r && (!oldest || q->last_use < oldest->last_use)) oldest = q;
+      if (oldest) evicted = lazy_unlink_locked(oldest);
+    }
+    pthread_mutex_unlock(&g_lock);
+    lazy_free(evicted);
+    found = r;
   }
-  *plan = r->plan;
+  *plan = found->plan;
+  *lease = found;
   return ALPHA_SPARSE_STATUS_SUCCESS;
+}
+
+/* every lazy record of a handle goes with the handle */
+void asamd_registry_drop_handle(const void *handle) {
+  for (;;) {
+    asamd_record *victim = NULL, *to_free = NULL;
+    pthread_mutex_lock(&g_lock);
+    for (asamd_record *r = g_head[ASAMD_KEY_LAZY]; r; r = r->next)
+      if (r->owner == handle) {
+        victim = r;
+        break;
+      }
+    if (victim) to_free = lazy_unlink_locked(victim);
+    pthread_mutex_unlock(&g_lock);
+    if (!victim) break;
+    lazy_free(to_free);
+  }
 }
 
 uint64_t asamd_host_fingerprint(const void *values, size_t count, size_t elem) {

@@ -353,6 +353,11 @@ int asamd_z_coomv(hipStream_t stream, int32_t m, int32_t n, int64_t nnz, asamd_c
                   const asamd_complex16 *coo_val, const int32_t *coo_row_ind, const int32_t *coo_col_ind,
                   int32_t base, const asamd_complex16 *x, asamd_complex16 beta, asamd_complex16 *y);
 
+/* Number of lazily made analyses (multiplies with info == NULL on arrays that no analysis or mirror
+ * covers) that the library remembers at the moment: at most 64, the least recently used one makes room,
+ * and a handle's own go with the handle.  For tests. */
+int asamd_registry_lazy_count(void);
+
 /* Introspection for benchmarks and tests: statistics of the analysis that a
  * multiply would use for `key`, where key is the alphasparse_dcu_mat_info_t of an
  * explicit analysis, or a device csr_row_ptr (library-built mirror or lazily

@@ -528,3 +528,51 @@ def test_row_ptr_into_the_middle_of_larger_arrays(gpu, maker):
     finally:
         lib.alphasparse_dcu_destroy_mat_info(info)
         da.free()
+
+
+def test_lazy_analyses_are_bounded(gpu):
+    """10 000 un-analysed matrices at distinct row_ptr addresses multiplied one after the other: the library
+    remembers at most 64 lazy analyses (least recently used goes), device memory stays put, a matrix whose
+    record was evicted still multiplies correctly, and a handle's records go with the handle."""
+    lib = capi.load()
+    a = csr_from_lengths([3, 0, 5, 1, 7, 2, 0, 4], 40, np.float32)
+    x, y0 = _vectors(a)
+    count = 10000
+    stride = 16  # ints per copy of row_ptr: 64 bytes apart
+    pool = np.zeros(count * stride, dtype=np.int32)
+    for k in range(count):
+        pool[k * stride:k * stride + a.rows + 1] = a.row_ptr
+    d_pool = hiprt.DeviceArray.from_numpy(pool)
+    d_col, d_val = hiprt.DeviceArray.from_numpy(a.col_ind), hiprt.DeviceArray.from_numpy(a.values)
+    dx, dy = hiprt.DeviceArray.from_numpy(x), hiprt.DeviceArray.from_numpy(y0)
+    h = capi.Handle()
+    descr = capi.make_descr()
+    al, be = c_float(1.0), c_float(0.0)
+
+    def multiply(k):
+        rp = c_void_p(d_pool.ptr + 4 * stride * k)
+        assert lib.alphasparse_dcu_s_csrmv(h.h, 0, a.rows, a.cols, a.nnz, byref(al), byref(descr), d_val.c_ptr(), rp,
+                                           d_col.c_ptr(), None, dx.c_ptr(), byref(be), dy.c_ptr()) == 0
+    try:
+        announce("lazy analyses bounded")
+        before = lib.asamd_registry_lazy_count()
+        for k in range(200):
+            multiply(k)
+        hiprt.synchronize()
+        free_mid, _ = hiprt.mem_info()
+        assert lib.asamd_registry_lazy_count() <= 64
+        for k in range(200, count):
+            multiply(k)
+        hiprt.synchronize()
+        free_end, _ = hiprt.mem_info()
+        assert lib.asamd_registry_lazy_count() <= 64
+        assert free_mid - free_end <= 8 << 20, "device memory grew by %d bytes over 9 800 more matrices" % (free_mid - free_end)
+        multiply(0)  # evicted long ago
+        hiprt.synchronize()
+        check_spmv(a, 1.0, x, 0.0, y0, dy.to_numpy(), "evicted matrix")
+        h.close()
+        assert lib.asamd_registry_lazy_count() <= before, "a handle's lazy analyses go with the handle"
+    finally:
+        h.close()
+        for d in (d_pool, d_col, d_val, dx, dy):
+            d.free()
