@@ -43,7 +43,7 @@ ALPHA_SPARSE_DATATYPE_FLOAT_COMPLEX, ALPHA_SPARSE_DATATYPE_DOUBLE_COMPLEX = 2, 3
 
 # kernel families of the thin kernel ABI (include/alsparse_amd_kernels.h)
 (ASAMD_SPMV_AUTO, ASAMD_SPMV_VECTOR, ASAMD_SPMV_ROWCONST, ASAMD_SPMV_MERGE, ASAMD_SPMV_SCALAR, ASAMD_SPMV_TILED,
- ASAMD_SPMV_STREAM, ASAMD_SPMV_ELL) = range(8)
+ ASAMD_SPMV_STREAM, ASAMD_SPMV_ELL, ASAMD_SPMV_MERGE_HOT) = range(9)
 ASAMD_HIST_BINS = 33
 
 
@@ -129,7 +129,9 @@ class asamd_csr_stats(Structure):
                 ("tune_ms_base", c_float), ("tune_ms_tiled", c_float), ("tune_ms_ell", c_float),
                 ("ell_built", c_int32), ("ell_width", c_int32), ("transpose_built", c_int32),
                 ("tile_entries_per_lane", c_int32),
-                ("hist", ctypes.c_int64 * ASAMD_HIST_BINS)]
+                ("hist", ctypes.c_int64 * ASAMD_HIST_BINS),
+                ("hot_built", c_int32), ("hot_cols_lds", c_int32), ("hot_cols", c_int32),
+                ("hot_share_lds", c_float), ("tune_ms_hot", c_float)]
 
 
 class asamd_dense_strides(Structure):
@@ -351,7 +353,8 @@ _RESTYPE = {"alpha_set_thread_num": None, "alpha_timing_wtime": c_double, "alpha
 
 ALGO_NAMES = {ASAMD_SPMV_AUTO: "auto", ASAMD_SPMV_VECTOR: "vector", ASAMD_SPMV_ROWCONST: "rowconst",
               ASAMD_SPMV_MERGE: "merge-path", ASAMD_SPMV_SCALAR: "scalar", ASAMD_SPMV_TILED: "tiled two-phase",
-              ASAMD_SPMV_STREAM: "row-block stream", ASAMD_SPMV_ELL: "ell copy"}
+              ASAMD_SPMV_STREAM: "row-block stream", ASAMD_SPMV_ELL: "ell copy",
+              ASAMD_SPMV_MERGE_HOT: "merge-path, hot columns in LDS"}
 
 _lib = None
 

@@ -13,12 +13,14 @@
 #include <algorithm>
 #include <atomic>
 #include <cstdlib>
+#include <cstring>
 #include <new>
 #include <type_traits>
 #include <vector>
 
 #include "alsparse_amd_kernels.h"
 #include "spmv_ell.hpp"
+#include "spmv_hot.hpp"
 #include "spmv_merge.hpp"
 #include "spmv_rows.hpp"
 #include "spmv_tiled.hpp"
@@ -108,6 +110,15 @@ struct asamd_csr_plan {
   unsigned short* d_trow;     // nnz local rows
   void* d_tprod;              // nnz products (phase 1 -> phase 2)
   TiledChunk* d_chunks;       // phase-1 work list
+  // hot-column copy (trusted plans of matrices whose entries crowd into few columns): structure only
+  unsigned* d_pcol;           // nnz positions: rank of a hot column, or hot_cols + column
+  int* d_hot_cols;            // hot_cols zero-based columns, most popular first
+  void* d_xhot;               // their x, gathered by every multiply
+  int hot_blocks;             // wave-sized merge blocks of the hot-column kernel, with their coordinates
+  int* d_hot_block_row;       // hot_blocks + 1
+  int* d_hot_carry_row;       // hot_blocks
+  void* d_hot_carry_val;      // hot_blocks values
+  void* d_hot_head_val;       // hot_blocks values
   // ELL copy (trusted plans of short, nearly equal rows)
   void* d_eval;               // ell_width * m values, column-major
   int* d_ecol;                // ... and zero-based columns
@@ -239,6 +250,21 @@ static void free_ell(asamd_csr_plan* p) {
   p->d_eval = nullptr;
   p->d_ecol = nullptr;
   p->st.ell_built = 0;
+}
+
+static void free_hot(asamd_csr_plan* p) {
+  for (void* d : {(void*)p->d_pcol, (void*)p->d_hot_cols, p->d_xhot, (void*)p->d_hot_block_row,
+                  (void*)p->d_hot_carry_row, p->d_hot_carry_val, p->d_hot_head_val})
+    if (d) (void)hipFree(d);
+  p->d_pcol = nullptr;
+  p->d_hot_cols = nullptr;
+  p->d_xhot = nullptr;
+  p->d_hot_block_row = nullptr;
+  p->d_hot_carry_row = nullptr;
+  p->d_hot_carry_val = nullptr;
+  p->d_hot_head_val = nullptr;
+  p->hot_blocks = 0;
+  p->st.hot_built = 0;
 }
 
 static void free_transpose(asamd_csr_plan* p, int which) {
@@ -588,13 +614,123 @@ static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* 
   return hipSuccess;
 }
 
+// The hot-column kernel pays when x is far larger than an XCD's L2 and yet most entries fall into a few
+// columns (power-law graphs).  Whether they do is only known after counting (build_hot).
+constexpr int kHotFrontBytes = 1 << 20;  // of every XCD's 4 MiB L2, beside the streams passing through
+template <typename T>
+struct HotKernel {
+  // 4-byte values: 8 items per lane and 16 waves; 8-byte values: 4 items per lane (the staging areas of
+  // 16 waves must leave room for the table)
+  static constexpr int ipt = sizeof(T) == 4 ? 8 : 4;
+  static constexpr int nw = 16;
+  using Dims = HotDims<T, ipt, nw>;
+};
+template <typename T>
+static bool hot_eligible(const asamd_csr_plan* p, bool force) {
+  const asamd_csr_stats& st = p->st;
+  if (sizeof(T) > 8 || !st.trusted || st.first_offset != 0 || st.nnz < 1 || st.n < 1) return false;
+  // positions are 32-bit words, x is addressed through a buffer resource with 32-bit byte offsets
+  if (((int64_t)st.n + (int64_t)kHotFrontBytes) >= (int64_t)UINT32_MAX) return false;
+  if ((int64_t)st.m + st.nnz >= (int64_t)INT32_MAX / 2) return false;
+  if (force) return true;
+  // Not tried unless asked for (ALSPARSE_AMD_TUNE_HOT=1): counting and ranking the columns costs several
+  // multiplies, and on the power-law matrices it is meant for the kernel gained 4 % where a copy has to
+  // gain 5 % to be kept.
+  static const bool asked = [] {
+    const char* a = getenv("ALSPARSE_AMD_TUNE_HOT");
+    const char* b = getenv("ALSPARSE_AMD_TUNE_PICK");
+    return (a && atoi(a) > 0) || (b && !strcmp(b, "hot"));
+  }();
+  return asked && (int64_t)st.n * (int64_t)sizeof(T) >= ((int64_t)8 << 20) && st.nnz >= (1 << 22);
+}
+
+// Counts the entries of every column, ranks the columns, rewrites the column stream as positions (LDS
+// slot or column) and caches the merge coordinates of the wave-sized blocks.  Leaves hot_built = 0 (and
+// no error) when the popular columns hold too few entries.
+template <typename T>
+static hipError_t build_hot(hipStream_t stream, asamd_csr_plan* p, const int* row_ptr, const int* col_ind, bool force) {
+  using HK = HotKernel<T>;
+  asamd_csr_stats& st = p->st;
+  const int n = st.n;
+  const size_t nnz = (size_t)st.nnz;
+  int h1 = HK::Dims::lds_cols;
+  if (const char* ev = getenv("ALSPARSE_AMD_HOT_COLS")) {
+    const int v = atoi(ev);
+    if (v > 0 && v < h1) h1 = v;
+  }
+  if (h1 > n) h1 = n;
+  // the compact front: the columns that share an XCD's L2 with the streams passing through
+  int hc = (int)(((int64_t)kHotFrontBytes) / (int64_t)sizeof(T));
+  if (const char* ev = getenv("ALSPARSE_AMD_HOT_FRONT")) {
+    const int v = atoi(ev);
+    if (v > 0) hc = v;
+  }
+  if (hc > n) hc = n;
+  if (hc < h1) hc = h1;
+  const int64_t nb = ((int64_t)st.m + st.nnz + HK::Dims::items - 1) / HK::Dims::items;
+  unsigned *d_cnt = nullptr, *d_key = nullptr, *d_key2 = nullptr, *d_idx = nullptr, *d_sorted = nullptr, *d_rank = nullptr;
+  hipError_t e = hipMalloc(&d_cnt, (size_t)n * sizeof(unsigned));
+  if (e == hipSuccess) e = hipMalloc(&d_key, (size_t)n * sizeof(unsigned));
+  if (e == hipSuccess) e = hipMalloc(&d_key2, (size_t)n * sizeof(unsigned));
+  if (e == hipSuccess) e = hipMalloc(&d_idx, (size_t)n * sizeof(unsigned));
+  if (e == hipSuccess) e = hipMalloc(&d_sorted, (size_t)n * sizeof(unsigned));
+  if (e == hipSuccess) e = hipMemsetAsync(d_cnt, 0, (size_t)n * sizeof(unsigned), stream);
+  std::vector<unsigned> h_key((size_t)h1);
+  if (e == hipSuccess) {
+    col_count_kernel<<<256 * 32, 256, 0, stream>>>(st.nnz, col_ind, st.base, d_cnt);
+    col_rank_keys_kernel<<<(unsigned)(((int64_t)n + 255) / 256), 256, 0, stream>>>(n, d_cnt, d_key, d_idx);
+    e = hipGetLastError();
+  }
+  if (e == hipSuccess) e = sort_pairs_u32(stream, d_key, d_key2, d_idx, d_sorted, (size_t)n, 32);
+  if (e == hipSuccess) e = hipMemcpy(h_key.data(), d_key2, (size_t)h1 * sizeof(unsigned), hipMemcpyDeviceToHost);
+  if (e == hipSuccess) {
+    double in_lds = 0.0;
+    for (int i = 0; i < h1; ++i) in_lds += (double)(~h_key[(size_t)i]);
+    st.hot_cols_lds = h1;
+    st.hot_cols = hc;
+    st.hot_share_lds = (float)(in_lds / (double)nnz);
+    // worth laying out only if the LDS serves a good part of the gathers
+    if (!force && st.hot_share_lds < 0.2f) e = hipErrorNotSupported;
+  }
+  if (e == hipSuccess) e = hipMalloc(&d_rank, (size_t)n * sizeof(unsigned));
+  if (e == hipSuccess) e = hipMalloc(&p->d_pcol, nnz * sizeof(unsigned));
+  if (e == hipSuccess) e = hipMalloc(&p->d_hot_cols, (size_t)hc * sizeof(int));
+  if (e == hipSuccess) e = hipMalloc(&p->d_xhot, (size_t)hc * sizeof(T));
+  if (e == hipSuccess) e = hipMalloc(&p->d_hot_block_row, ((size_t)nb + 1) * sizeof(int));
+  if (e == hipSuccess) e = hipMalloc(&p->d_hot_carry_row, (size_t)nb * sizeof(int));
+  if (e == hipSuccess) e = hipMalloc(&p->d_hot_carry_val, (size_t)nb * sizeof(T));
+  if (e == hipSuccess) e = hipMalloc(&p->d_hot_head_val, (size_t)nb * sizeof(T));
+  if (e == hipSuccess) e = hipMemsetAsync(d_rank, 0xFF, (size_t)n * sizeof(unsigned), stream);
+  if (e == hipSuccess) e = hipMemsetAsync(p->d_hot_head_val, 0, (size_t)nb * sizeof(T), stream);
+  if (e == hipSuccess) {
+    col_rank_scatter_kernel<<<(unsigned)((hc + 255) / 256), 256, 0, stream>>>(hc, d_sorted, d_rank, p->d_hot_cols);
+    hot_pcol_kernel<<<256 * 32, 256, 0, stream>>>(st.nnz, col_ind, st.base, hc, d_rank, p->d_pcol);
+    merge_partition_kernel<<<(unsigned)((nb + 1 + 255) / 256), 256, 0, stream>>>(st.m, st.nnz, row_ptr, st.base, (int)nb,
+                                                                                HK::Dims::items, p->d_hot_block_row);
+    e = hipGetLastError();
+  }
+  if (e == hipSuccess)
+    e = hipFuncSetAttribute((const void*)spmv_merge_hot_kernel<T, HK::ipt, HK::nw>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, HK::Dims::table_bytes + HK::Dims::stage_bytes);
+  if (e == hipSuccess) e = hipStreamSynchronize(stream);
+  for (void* d : {(void*)d_cnt, (void*)d_key, (void*)d_key2, (void*)d_idx, (void*)d_sorted, (void*)d_rank})
+    if (d) (void)hipFree(d);
+  if (e != hipSuccess) {
+    free_hot(p);
+    return e == hipErrorNotSupported ? hipSuccess : e;
+  }
+  p->hot_blocks = (int)nb;
+  st.hot_built = 1;
+  return hipSuccess;
+}
+
 // Time the structural choice on scratch vectors, then the copies that the matrix is eligible for:
 // the ELL copy (cheap to build), and the tiled copy only if the fastest so far is slower than the
 // tiled pair could possibly be.  Keep the fastest and free the copies that lost.  A copy has to win
 // by a margin to be worth its memory.
 template <typename T>
 static hipError_t tune_copies(hipStream_t stream, asamd_csr_plan* p, const int* row_ptr,
-                              const int* col_ind, const T* val, bool tiled_ok, bool ell_ok) {
+                              const int* col_ind, const T* val, bool tiled_ok, bool ell_ok, bool hot_ok) {
   asamd_csr_stats& st = p->st;
   T *x = nullptr, *y = nullptr;
   hipEvent_t e0 = nullptr, e1 = nullptr;
@@ -603,8 +739,8 @@ static hipError_t tune_copies(hipStream_t stream, asamd_csr_plan* p, const int* 
   if (e == hipSuccess) e = hipMemsetAsync(x, 0, (size_t)st.n * sizeof(T), stream);
   if (e == hipSuccess) e = hipEventCreate(&e0);
   if (e == hipSuccess) e = hipEventCreate(&e1);
-  float best[3] = {0.f, 0.f, 0.f};
-  const int algos[3] = {p->auto_algo, ASAMD_SPMV_TILED, ASAMD_SPMV_ELL};
+  float best[4] = {0.f, 0.f, 0.f, 0.f};
+  const int algos[4] = {p->auto_algo, ASAMD_SPMV_TILED, ASAMD_SPMV_ELL, ASAMD_SPMV_MERGE_HOT};
   auto time_algo = [&](int a) {
     st.algo = algos[a];
     // first run warms up; multiplies of a millisecond and more are timed once, shorter ones twice; a
@@ -655,6 +791,12 @@ static hipError_t tune_copies(hipStream_t stream, asamd_csr_plan* p, const int* 
     }
   }
   if (!ell_first && !(best[1] > 0.f && best[1] < 0.9f * best[0])) try_ell();
+  // Skewed matrices on merge-path: count the entries per column and, if few columns hold most of them,
+  // time the kernel that keeps those columns' x in LDS.
+  if (e == hipSuccess && hot_ok && p->auto_algo == ASAMD_SPMV_MERGE) {
+    e = build_hot<T>(stream, p, row_ptr, col_ind, false);
+    if (e == hipSuccess && st.hot_built) time_algo(3);
+  }
   if (e0) (void)hipEventDestroy(e0);
   if (e1) (void)hipEventDestroy(e1);
   if (x) (void)hipFree(x);
@@ -664,18 +806,26 @@ static hipError_t tune_copies(hipStream_t stream, asamd_csr_plan* p, const int* 
   st.tune_ms_base = best[0];
   st.tune_ms_tiled = best[1];
   st.tune_ms_ell = best[2];
-  const bool tiled_wins = best[1] > 0.f && best[1] < 0.9f * best[0];
-  const bool ell_wins = best[2] > 0.f && best[2] < 0.95f * best[0];
+  st.tune_ms_hot = best[3];
+  // a copy has to win by a margin to be worth its memory; among the winners the fastest is kept
+  const float margin[4] = {1.f, 0.9f, 0.95f, 0.95f};
   int pick = 0;
-  if (tiled_wins && ell_wins) pick = best[1] < best[2] ? 1 : 2;
-  else if (tiled_wins) pick = 1;
-  else if (ell_wins) pick = 2;
+  for (int a = 1; a < 4; ++a)
+    if (best[a] > 0.f && best[a] < margin[a] * best[0] && (pick == 0 || best[a] < best[pick])) pick = a;
+  // ALSPARSE_AMD_TUNE_PICK = base | tiled | ell | hot overrides the timing's verdict among the candidates
+  // that were built (for profiling a kernel that lost)
+  if (const char* ev = getenv("ALSPARSE_AMD_TUNE_PICK")) {
+    const char* names[4] = {"base", "tiled", "ell", "hot"};
+    for (int a = 0; a < 4; ++a)
+      if (!strcmp(ev, names[a]) && (a == 0 || best[a] > 0.f)) pick = a;
+  }
   if (pick != 1) free_tiled(p);
   if (pick != 2) free_ell(p);
+  if (pick != 3) free_hot(p);
   if (pick != 0) {
     p->auto_algo = algos[pick];
     st.algo = algos[pick];
-    p->copy_val_src = val;
+    if (pick != 3) p->copy_val_src = val;  // the hot-column copy holds no values
   }
   return hipSuccess;
 }
@@ -763,12 +913,14 @@ static hipError_t plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t 
       using T = std::remove_pointer_t<decltype(tag)>;
       hipError_t err = hipSuccess;
       const bool tiled_ok = tiled_eligible<T>(p->st, force), ell_ok = ell_eligible(p->st, force);
+      const bool hot_ok = hot_eligible<T>(p, force);
       if (force) {
         if (tiled_ok) err = build_tiled<T>(stream, p, row_ptr, col_ind, (const T*)val);
         if (err == hipSuccess && ell_ok) err = build_ell<T>(stream, p, row_ptr, col_ind, (const T*)val);
+        if (err == hipSuccess && hot_ok) err = build_hot<T>(stream, p, row_ptr, col_ind, true);
         p->copy_val_src = val;
-      } else if (tiled_ok || ell_ok) {
-        err = tune_copies<T>(stream, p, row_ptr, col_ind, (const T*)val, tiled_ok, ell_ok);
+      } else if (tiled_ok || ell_ok || hot_ok) {
+        err = tune_copies<T>(stream, p, row_ptr, col_ind, (const T*)val, tiled_ok, ell_ok, hot_ok);
       }
       return err;
     });
@@ -776,6 +928,9 @@ static hipError_t plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t 
       (void)hipGetLastError();  // the copies are optional: carry on without them
       free_tiled(p);
       free_ell(p);
+      free_hot(p);
+      if (p->auto_algo == ASAMD_SPMV_TILED || p->auto_algo == ASAMD_SPMV_ELL || p->auto_algo == ASAMD_SPMV_MERGE_HOT)
+        p->auto_algo = p->struct_algo;
       p->st.algo = p->auto_algo;
       e = hipSuccess;
     }
@@ -811,6 +966,7 @@ extern "C" void asamd_csr_plan_destroy(asamd_csr_plan* p) {
   if (p->d_head_val) (void)hipFree(p->d_head_val);
   free_tiled(p);
   free_ell(p);
+  free_hot(p);
   free_transpose(p, 0);
   free_transpose(p, 1);
   delete p;
@@ -1014,6 +1170,10 @@ extern "C" int asamd_csr_plan_set_algo(asamd_csr_plan* p, int32_t algo) {
       if (!p->st.ell_built) return hipErrorInvalidValue;
       p->st.algo = algo;
       return hipSuccess;
+    case ASAMD_SPMV_MERGE_HOT:
+      if (!p->st.hot_built) return hipErrorInvalidValue;
+      p->st.algo = algo;
+      return hipSuccess;
     case ASAMD_SPMV_MERGE:
       if (p->st.first_offset != 0) return hipErrorInvalidValue;
       p->st.algo = algo;
@@ -1069,6 +1229,7 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
   if (algo == ASAMD_SPMV_MERGE && st.first_offset != 0) algo = ASAMD_SPMV_VECTOR;
   if (algo == ASAMD_SPMV_TILED && !st.tiled_built) algo = p->auto_algo == ASAMD_SPMV_TILED ? ASAMD_SPMV_MERGE : p->auto_algo;
   if (algo == ASAMD_SPMV_ELL && !st.ell_built) algo = p->auto_algo == ASAMD_SPMV_ELL ? ASAMD_SPMV_MERGE : p->auto_algo;
+  if (algo == ASAMD_SPMV_MERGE_HOT && !st.hot_built) algo = ASAMD_SPMV_MERGE;
   switch (algo) {
     case ASAMD_SPMV_ELL: {
       // the ELL copy holds zero-based columns and its own values
@@ -1121,6 +1282,33 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
     case ASAMD_SPMV_SCALAR: {
       const unsigned grid = (unsigned)(((int64_t)st.m + kRowsBlock - 1) / kRowsBlock);
       spmv_scalar_kernel<T><<<grid, kRowsBlock, 0, s>>>(st.m, alpha, val, rp, ci, x, beta, y, st.base);
+      break;
+    }
+    case ASAMD_SPMV_MERGE_HOT: {
+      // x of the hot columns, then persistent workgroups, one per compute unit
+      if constexpr (sizeof(T) <= 8) {
+        using HK = HotKernel<T>;
+        const int nb = p->hot_blocks;
+        const int h1 = st.hot_cols_lds, hc = st.hot_cols;
+        hot_prepare_kernel<T><<<(unsigned)((hc + 255) / 256), 256, 0, s>>>(hc, p->d_hot_cols, x, (T*)p->d_xhot);
+        static const int cus = [] {
+          int dev = 0, n_cu = 0;
+          if (hipGetDevice(&dev) != hipSuccess ||
+              hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n_cu <= 0)
+            n_cu = 256;
+          return n_cu;
+        }();
+        const int per_wg = (nb + HK::nw - 1) / HK::nw;
+        const int grid = per_wg < cus ? per_wg : cus;
+        spmv_merge_hot_kernel<T, HK::ipt, HK::nw>
+            <<<grid, HK::Dims::threads, HK::Dims::table_bytes + HK::Dims::stage_bytes, s>>>(
+                st.m, st.nnz, alpha, val, rp, p->d_pcol, x, (const T*)p->d_xhot, h1, hc, beta, y, st.base, p->d_hot_block_row, p->d_hot_carry_row,
+                (T*)p->d_hot_carry_val, (T*)p->d_hot_head_val, nb);
+        if (nb > 1)
+          merge_fixup_kernel<T><<<(nb + 255) / 256, 256, 0, s>>>(nb, st.m, alpha, beta, p->d_hot_carry_row,
+                                                                 (const T*)p->d_hot_carry_val,
+                                                                 (const T*)p->d_hot_head_val, y);
+      }
       break;
     }
     case ASAMD_SPMV_MERGE: {

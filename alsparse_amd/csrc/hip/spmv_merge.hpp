@@ -249,10 +249,31 @@ __global__ __launch_bounds__(256) void merge_fixup_kernel(int nblocks, int m, T 
   const int r = carry_row[bb - 1];
   if (r < 0 || r >= m) return;
   if (carry_row[bb] == r) return;  // workgroup bb finished no row
+  // the carries name rows in ascending order: the run of blocks that the row crossed starts at the first
+  // carry that names it
   int first = bb - 1;
-  while (first > 0 && carry_row[first - 1] == r) --first;
+  if (first > 0 && carry_row[first - 1] == r) {
+    int lo = 0, hi = first - 1;  // carry_row[hi] == r
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (carry_row[mid] < r) {
+        lo = mid + 1;
+      } else {
+        hi = mid;
+      }
+    }
+    first = lo;
+  }
   T s = T(0);
-  for (int k = first; k < bb; ++k) s += carry_val[k];
+  int k = first;
+  for (; k + 4 <= bb; k += 4) {
+    const T c0 = carry_val[k], c1 = carry_val[k + 1], c2 = carry_val[k + 2], c3 = carry_val[k + 3];
+    s += c0;
+    s += c1;
+    s += c2;
+    s += c3;
+  }
+  for (; k < bb; ++k) s += carry_val[k];
   s += head_val[bb];
   store_axpby(y, (int64_t)r, alpha, s, beta);
 }

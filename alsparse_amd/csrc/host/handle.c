@@ -179,6 +179,7 @@ int asamd_env_algo(void) {
   if (!strcmp(e, "tiled")) return ASAMD_SPMV_TILED;
   if (!strcmp(e, "stream")) return ASAMD_SPMV_STREAM;
   if (!strcmp(e, "ell")) return ASAMD_SPMV_ELL;
+  if (!strcmp(e, "hot")) return ASAMD_SPMV_MERGE_HOT;
   return ASAMD_SPMV_AUTO;
 }
 

@@ -36,8 +36,11 @@ enum asamd_spmv_algo {
   ASAMD_SPMV_TILED = 5,    /* two-phase, (column block x row block) tiles: every x
                               gather and y update in LDS, HBM sees only streams     */
   ASAMD_SPMV_STREAM = 6,   /* rows of <= 16 entries: 256 rows' products staged in LDS */
-  ASAMD_SPMV_ELL = 7       /* short, nearly equal rows: a column-major ELL copy, one
+  ASAMD_SPMV_ELL = 7,      /* short, nearly equal rows: a column-major ELL copy, one
                               lane per row                                          */
+  ASAMD_SPMV_MERGE_HOT = 8 /* merge-path whose persistent workgroups keep x of the most
+                              popular columns in LDS (power-law graphs); the copy it
+                              needs is structure only: values come from the caller  */
 };
 
 #define ASAMD_HIST_BINS 33
@@ -87,6 +90,11 @@ typedef struct {
                                     phase (1: twice the tiles in flight; tiles of more
                                     than 64 entries go to the long-tile kernel), or 0  */
   int64_t hist[ASAMD_HIST_BINS];
+  int32_t hot_built;     /* 1: the hot-column copy exists (MERGE_HOT can be selected)        */
+  int32_t hot_cols_lds;  /* columns whose x the kernel keeps in LDS                            */
+  int32_t hot_cols;      /* most popular columns whose x every multiply gathers into a compact front */
+  float hot_share_lds;   /* share of the entries that fall into the LDS columns               */
+  float tune_ms_hot;     /* analysis-time timing of the hot-column kernel, or 0               */
 } asamd_csr_stats;
 
 typedef struct asamd_csr_plan asamd_csr_plan;

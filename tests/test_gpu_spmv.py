@@ -45,7 +45,7 @@ def test_every_kernel_family_matches_oracle(gpu, shape, dtype):
     x, y0 = _vectors(a)
     da = DeviceCsr(a)
     try:
-        for algo in ("vector", "merge", "scalar", "rowconst", "stream", "tiled", "ell", "auto"):
+        for algo in ("vector", "merge", "scalar", "rowconst", "stream", "tiled", "ell", "hot", "auto"):
             for alpha, beta in ((1.0, 0.0), (2.0, 3.0), (-0.75, 1.0)):
                 announce("spmv", shape, np.dtype(dtype).name, algo, alpha, beta)
                 y = run_plan_csrmv(da, algo, alpha, x, beta, y0)
@@ -65,7 +65,7 @@ def test_index_base_one(gpu, dtype):
         x, y0 = _vectors(a)
         da = DeviceCsr(a)
         try:
-            for algo in ("vector", "merge", "scalar", "stream", "tiled", "ell", "auto"):
+            for algo in ("vector", "merge", "scalar", "stream", "tiled", "ell", "hot", "auto"):
                 announce("spmv base1", a.name, algo)
                 y = run_plan_csrmv(da, algo, 1.5, x, 0.25, y0)
                 if y is None:
@@ -85,7 +85,7 @@ def test_beta_zero_ignores_nan_in_y(gpu):
     y0 = np.full(a.rows, np.nan, dtype=np.float32)
     da = DeviceCsr(a)
     try:
-        for algo in ("vector", "merge", "scalar", "tiled"):
+        for algo in ("vector", "merge", "scalar", "tiled", "hot"):
             announce("spmv beta0 nan", algo)
             y = run_plan_csrmv(da, algo, 1.0, x, 0.0, y0)
             assert np.isfinite(y).all()
@@ -271,7 +271,7 @@ def test_random_structures_every_family(gpu, seed):
     x, y0 = _vectors(a, seed)
     da = DeviceCsr(a)
     try:
-        for algo in ("vector", "merge", "scalar", "rowconst", "stream", "tiled", "ell", "auto"):
+        for algo in ("vector", "merge", "scalar", "rowconst", "stream", "tiled", "ell", "hot", "auto"):
             for alpha, beta in ((1.5, 0.0), (-2.0, 0.5)):
                 announce("spmv random", seed, m, n, a.nnz, np.dtype(dtype).name, base, algo, alpha, beta)
                 y = run_plan_csrmv(da, algo, alpha, x, beta, y0)
@@ -301,7 +301,7 @@ def test_unsorted_and_duplicate_columns_and_non_finite_values(gpu, dtype):
     x, y0 = _vectors(a, 5)
     da = DeviceCsr(a)
     try:
-        for algo in ("vector", "merge", "scalar", "stream", "tiled", "ell", "auto"):
+        for algo in ("vector", "merge", "scalar", "stream", "tiled", "ell", "hot", "auto"):
             announce("spmv unsorted", np.dtype(dtype).name, algo)
             y = run_plan_csrmv(da, algo, 1.5, x, 0.5, y0)
             if y is not None:
@@ -321,7 +321,7 @@ def test_unsorted_and_duplicate_columns_and_non_finite_values(gpu, dtype):
         ref = orc.csrmv_plain(b, 1.0, x2, 0.0, y0)
     db = DeviceCsr(b)
     try:
-        for algo in ("vector", "merge", "scalar", "tiled", "auto"):
+        for algo in ("vector", "merge", "scalar", "tiled", "hot", "auto"):
             announce("spmv non-finite", np.dtype(dtype).name, algo)
             y = run_plan_csrmv(db, algo, 1.0, x2, 0.0, y0)
             assert np.array_equal(np.isnan(y), np.isnan(ref)), algo
