@@ -34,6 +34,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
 #include "alsparse_amd_kernels.h"
 #include "device_utils.hpp"
 
@@ -182,6 +184,83 @@ __global__ __launch_bounds__(kSpmmBlock) void spmm_rowmajor_kernel(
         nt_store(res, crow + i);
       }
     }
+  }
+}
+
+// Four entries of a row per wave instruction: the wave's lanes form four groups of 16, lane l of a group owns
+// the E = 16 / sizeof(T) dense columns from (blockIdx.y * 16 + l) * E on and loads them with one 128-bit load,
+// so one instruction fetches 16 * E contiguous elements of FOUR rows of B (group g takes the row's entries
+// 4i + g), and all the loads of up to 32 entries are in flight at once: a 32-entry row waits for B once, not
+// eight times in turn.  The four partial sums meet at the end (two exchanges across the groups).  Needs B and C
+// rows that 128-bit loads can address: pointers and row strides multiples of 16 bytes, n a multiple of E.
+template <typename T>
+__global__ __launch_bounds__(kSpmmBlock) void spmm_rowmajor_quad_kernel(
+    int m, int n, T alpha, const T* __restrict__ val, const int* __restrict__ row_ptr,
+    const int* __restrict__ col_ind, int base, const T* __restrict__ B, int64_t ldb, T beta,
+    T* __restrict__ C, int64_t ldc) {
+  constexpr int E = 16 / (int)sizeof(T);
+  constexpr int kU = 8;  // loads in flight per lane
+  const int lane = threadIdx.x % kWave;
+  const int wave = threadIdx.x / kWave;
+  const unsigned bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  const int64_t row = (int64_t)bid * kSpmmWaves + wave;
+  if (row >= m) return;  // wave-uniform
+  const int g = lane / 16;
+  const int c0 = (blockIdx.y * 16 + lane % 16) * E;
+  const bool owns = c0 < n;
+  const T* bcol = B + (owns ? c0 : 0);
+
+  const int64_t start = (int64_t)row_ptr[row] - base;
+  const int64_t end = (int64_t)row_ptr[row + 1] - base;
+  T acc[E];
+#pragma unroll
+  for (int i = 0; i < E; ++i) acc[i] = T(0);
+
+  for (int64_t j0 = start; j0 < end; j0 += kWave) {
+    const int64_t j = j0 + lane < end ? j0 + lane : j0;  // lanes past the end repeat the chunk's first entry
+    // A and C are touched once: non-temporal, so that they do not push rows of B out of the caches
+    const int my_col = nt_load(col_ind + j) - base;
+    const T my_val = alpha * nt_load(val + j);
+    const int cnt = (int)(end - j0 < kWave ? end - j0 : kWave);
+    for (int t0 = 0; t0 < cnt; t0 += 4 * kU) {
+      Vec<T, E> b[kU];
+      T a[kU];
+      // every load is issued whatever the group needs (a group past the end loads the chunk's first row of
+      // B again and adds nothing): loads under branches would wait for one another
+#pragma unroll
+      for (int u = 0; u < kU; ++u) {
+        const int t = t0 + 4 * u + g;
+        const int src = t < cnt ? t : 0;
+        const int col = lane_get(my_col, src);
+        a[u] = lane_get(my_val, src);
+        b[u] = *reinterpret_cast<const Vec<T, E>*>(bcol + (int64_t)col * ldb);
+      }
+#pragma unroll
+      for (int u = 0; u < kU; ++u) {
+        if (t0 + 4 * u + g < cnt) {
+#pragma unroll
+          for (int i = 0; i < E; ++i) acc[i] = fma_t(a[u], b[u].e[i], acc[i]);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < E; ++i) {
+    acc[i] += lane_xor(acc[i], 16);
+    acc[i] += lane_xor(acc[i], 32);
+  }
+  if (g == 0 && owns) {
+    T* crow = C + row * ldc + c0;
+    Vec<T, E> out;
+    if (beta == T(0)) {
+#pragma unroll
+      for (int i = 0; i < E; ++i) out.e[i] = acc[i];
+    } else {
+      const Vec<T, E> old = *reinterpret_cast<const Vec<T, E>*>(crow);
+#pragma unroll
+      for (int i = 0; i < E; ++i) out.e[i] = old.e[i] * beta + acc[i];
+    }
+    *reinterpret_cast<Vec<T, E>*>(crow) = out;
   }
 }
 
@@ -547,6 +626,16 @@ static int csrmm_impl(hipStream_t s, int m, int n, int k, int nnz, T alpha, cons
       return hipGetLastError();
     }
     const unsigned gx = (unsigned)(((int64_t)m + kSpmmWaves - 1) / kSpmmWaves);
+    {
+      // rows of B and C that 128-bit loads can address: four rows of B per wave instruction
+      constexpr int E = 16 / (int)sizeof(T);
+      static const bool quad_off = getenv("ALSPARSE_AMD_SPMM_QUAD") && atoi(getenv("ALSPARSE_AMD_SPMM_QUAD")) == 0;
+      if (!quad_off && n % E == 0 && ldb % E == 0 && ldc % E == 0 && (uintptr_t)B % 16 == 0 && (uintptr_t)C % 16 == 0) {
+        const dim3 grid(gx, (unsigned)((n + 16 * E - 1) / (16 * E)));
+        spmm_rowmajor_quad_kernel<T><<<grid, kSpmmBlock, 0, s>>>(m, n, alpha, val, rp, ci, base, B, ldb, beta, C, ldc);
+        return hipGetLastError();
+      }
+    }
     // widest per-lane vector that still gives every lane of a wave work
     constexpr int kMaxV = 32 / (int)sizeof(T) >= 4 ? 4 : 32 / (int)sizeof(T);  // at most 32 bytes per lane and load
     int V = 1;
