@@ -113,6 +113,24 @@ __global__ __launch_bounds__(kCeilThreads) void ceiling_elem_gather_kernel(const
   if (acc == 1.2345e-30f) sink[0] = acc;
 }
 
+// A copy in runs of R floats (R a multiple of 4, 16 bytes per lane): run r of the one side is run
+// (r * mult) mod nruns of the other (mult and nruns coprime), so one side streams and the other jumps
+// from run to run.  A workgroup takes 128 consecutive runs at a time.
+__global__ __launch_bounds__(1024) void ceiling_run_copy_kernel(const float* __restrict__ in, float* __restrict__ out,
+                                                                long nruns, int R, bool scatter, long mult) {
+  const long per_wg = 128;
+  const int q = R / 4;
+  for (long r0 = (long)blockIdx.x * per_wg; r0 < nruns; r0 += (long)gridDim.x * per_wg) {
+    for (int i = threadIdx.x; i < per_wg * q; i += 1024) {
+      const long r = r0 + i / q;
+      if (r >= nruns) break;
+      const int o = (i % q) * 4;
+      const long pr = (r * mult) % nruns;
+      const long src = (scatter ? r : pr) * R + o, dst = (scatter ? pr : r) * R + o;
+      *reinterpret_cast<Int4v*>(out + dst) = *reinterpret_cast<const Int4v*>(in + src);
+    }
+  }
+}
 }  // namespace
 
 extern "C" int asamd_ceiling_kernel(hipStream_t stream, int32_t kind, void* dst, const void* src, size_t nbytes,
@@ -169,6 +187,20 @@ extern "C" int asamd_ceiling_kernel(hipStream_t stream, int32_t kind, void* dst,
       ceiling_elem_gather_kernel<<<256 * 32, kCeilThreads, 0, stream>>>((const float*)src, (uint32_t)elems, per_lane,
                                                                          (float*)sink);
       *bytes_moved = lanes * per_lane * 4;  // useful bytes; every gather moves a whole cache line behind them
+      break;
+    }
+    case ASAMD_CEILING_RUN_GATHER:
+    case ASAMD_CEILING_RUN_SCATTER: {
+      if (!src || !dst || count < 4 || count % 4 != 0 || count > (1 << 20)) return hipErrorInvalidValue;
+      const long nruns = (long)(nbytes / 4 / (size_t)count);
+      if (nruns < 2) return hipErrorInvalidValue;
+      long mult = 2654435761L % nruns;  // a multiplier that shares no factor with the number of runs
+      if (mult < 2) mult = 1;
+      auto gcd = [](long a, long b) { while (b) { const long t = a % b; a = b; b = t; } return a; };
+      while (gcd(mult, nruns) != 1) ++mult;
+      ceiling_run_copy_kernel<<<512, 1024, 0, stream>>>((const float*)src, (float*)dst, nruns, (int)count,
+                                                        kind == ASAMD_CEILING_RUN_SCATTER, mult);
+      *bytes_moved = 2 * nruns * count * 4;
       break;
     }
     default:

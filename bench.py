@@ -512,7 +512,8 @@ def run_spmm(steps, warmup, check, col_major=False, vendor=False):
 
 def run_ceilings(steps, warmup):
     """What this GPU sustains with plain kernels (alsparse_amd/csrc/hip/ceilings.hip): 2 GiB read-only, write-only
-    and copy streams, whole 256-byte rows gathered at random from 256 MiB (the B operand of configuration 5) and
+    and copy streams, copies in short runs that one side reads or writes out of order (the product runs of the
+    tiled SpMV's second phase), whole 256-byte rows gathered at random from 256 MiB (the B operand of configuration 5) and
     single floats gathered at random from 64 MiB / 4 MiB / 16 KiB (the x of configuration 3; an L2-sized x; an
     L1-sized x).  TB/s of useful bytes, and gathers per second."""
     from ctypes import c_int64
@@ -540,6 +541,9 @@ def run_ceilings(steps, warmup):
     measure("write_2GiB", 1, b.c_ptr(), None, big, 0)
     measure("copy_2GiB", 2, b.c_ptr(), a.c_ptr(), big, 0)
     measure("copy_2GiB_nontemporal", 6, b.c_ptr(), a.c_ptr(), big, 0)
+    for runlen in (64, 80, 160):
+        measure("copy_1GiB_in_runs_of_%d_floats_gathered" % runlen, 7, b.c_ptr(), a.c_ptr(), 1 << 30, runlen)
+        measure("copy_1GiB_in_runs_of_%d_floats_scattered" % runlen, 8, b.c_ptr(), a.c_ptr(), 1 << 30, runlen)
     r = measure("row_gather_256B_from_256MiB", 3, None, a.c_ptr(), 256 << 20, 1 << 25)
     r["rows_per_s"] = r["useful_bytes"] / 256 / r["avg_ms"] * 1e3
     r = measure("row_gather_256B_from_2GiB", 3, None, a.c_ptr(), big, 1 << 25)

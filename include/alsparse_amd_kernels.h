@@ -388,7 +388,10 @@ int asamd_copy_bytes(hipStream_t stream, void *dst, const void *src, size_t nbyt
  * (a multiple of 16; 16 bytes per lane and access) from src / into dst; ROW_GATHER fetches `count`
  * 256-byte rows at random positions of the nbytes at src, one wave per row (what the row-major SpMM does
  * per entry of A with 64 dense columns); ELEM_GATHER fetches `count` single floats at random positions
- * (what a row SpMV kernel does per entry).  sink: 4 device bytes that are practically never written.
+ * (what a row SpMV kernel does per entry); RUN_GATHER / RUN_SCATTER copy nbytes in runs of `count` floats
+ * (a multiple of 4) whose order differs between source and destination: the runs are contiguous on the
+ * write side and scattered on the read side (what the second phase of the tiled SpMV reads), or the other
+ * way round.  sink: 4 device bytes that are practically never written.
  * *bytes_moved receives the useful bytes of the launch (copy: read + written). */
 enum asamd_ceiling_kind {
   ASAMD_CEILING_READ = 0,
@@ -397,7 +400,9 @@ enum asamd_ceiling_kind {
   ASAMD_CEILING_ROW_GATHER = 3,
   ASAMD_CEILING_ELEM_GATHER = 4,
   ASAMD_CEILING_READ_NT = 5, /* the same streams with non-temporal accesses */
-  ASAMD_CEILING_COPY_NT = 6
+  ASAMD_CEILING_COPY_NT = 6,
+  ASAMD_CEILING_RUN_GATHER = 7,
+  ASAMD_CEILING_RUN_SCATTER = 8
 };
 int asamd_ceiling_kernel(hipStream_t stream, int32_t kind, void *dst, const void *src, size_t nbytes,
                          int64_t count, void *sink, int64_t *bytes_moved);
