@@ -43,7 +43,7 @@ ALPHA_SPARSE_DATATYPE_FLOAT_COMPLEX, ALPHA_SPARSE_DATATYPE_DOUBLE_COMPLEX = 2, 3
 
 # kernel families of the thin kernel ABI (include/alsparse_amd_kernels.h)
 (ASAMD_SPMV_AUTO, ASAMD_SPMV_VECTOR, ASAMD_SPMV_ROWCONST, ASAMD_SPMV_MERGE, ASAMD_SPMV_SCALAR, ASAMD_SPMV_TILED,
- ASAMD_SPMV_STREAM, ASAMD_SPMV_ELL, ASAMD_SPMV_MERGE_HOT) = range(9)
+ ASAMD_SPMV_STREAM, ASAMD_SPMV_ELL, ASAMD_SPMV_MERGE_HOT, ASAMD_SPMV_BINNED) = range(10)
 ASAMD_HIST_BINS = 33
 
 
@@ -131,7 +131,8 @@ class asamd_csr_stats(Structure):
                 ("tile_entries_per_lane", c_int32),
                 ("hist", ctypes.c_int64 * ASAMD_HIST_BINS),
                 ("hot_built", c_int32), ("hot_cols_lds", c_int32), ("hot_cols", c_int32),
-                ("hot_share_lds", c_float), ("tune_ms_hot", c_float)]
+                ("hot_share_lds", c_float), ("tune_ms_hot", c_float),
+                ("binned_built", c_int32), ("bin_rows", c_int32 * 4), ("tune_ms_binned", c_float)]
 
 
 class asamd_dense_strides(Structure):
@@ -354,7 +355,7 @@ _RESTYPE = {"alpha_set_thread_num": None, "alpha_timing_wtime": c_double, "alpha
 ALGO_NAMES = {ASAMD_SPMV_AUTO: "auto", ASAMD_SPMV_VECTOR: "vector", ASAMD_SPMV_ROWCONST: "rowconst",
               ASAMD_SPMV_MERGE: "merge-path", ASAMD_SPMV_SCALAR: "scalar", ASAMD_SPMV_TILED: "tiled two-phase",
               ASAMD_SPMV_STREAM: "row-block stream", ASAMD_SPMV_ELL: "ell copy",
-              ASAMD_SPMV_MERGE_HOT: "merge-path, hot columns in LDS"}
+              ASAMD_SPMV_MERGE_HOT: "merge-path, hot columns in LDS", ASAMD_SPMV_BINNED: "row-length bins"}
 
 _lib = None
 

@@ -20,6 +20,7 @@
 
 #include "alsparse_amd_kernels.h"
 #include "spmv_ell.hpp"
+#include "spmv_binned.hpp"
 #include "spmv_hot.hpp"
 #include "spmv_merge.hpp"
 #include "spmv_rows.hpp"
@@ -119,6 +120,13 @@ struct asamd_csr_plan {
   int* d_hot_carry_row;       // hot_blocks
   void* d_hot_carry_val;      // hot_blocks values
   void* d_hot_head_val;       // hot_blocks values
+  // row-length bins (trusted plans of very uneven rows): structure only
+  int* d_bin_rows;            // m row numbers sorted by length class, ascending inside a class
+  int bin_count[kBinClasses]; // rows per class
+  int bin_chunks;             // chunks that the rows of the last class are cut into
+  BinChunk* d_bin_chunk;      // bin_chunks
+  int* d_bin_first;           // bin_count[3] + 1: first chunk of every long row
+  void* d_bin_partial;        // bin_chunks values
   // ELL copy (trusted plans of short, nearly equal rows)
   void* d_eval;               // ell_width * m values, column-major
   int* d_ecol;                // ... and zero-based columns
@@ -265,6 +273,17 @@ static void free_hot(asamd_csr_plan* p) {
   p->d_hot_head_val = nullptr;
   p->hot_blocks = 0;
   p->st.hot_built = 0;
+}
+
+static void free_binned(asamd_csr_plan* p) {
+  for (void* d : {(void*)p->d_bin_rows, (void*)p->d_bin_chunk, (void*)p->d_bin_first, p->d_bin_partial})
+    if (d) (void)hipFree(d);
+  p->d_bin_rows = nullptr;
+  p->d_bin_chunk = nullptr;
+  p->d_bin_first = nullptr;
+  p->d_bin_partial = nullptr;
+  p->bin_chunks = 0;
+  p->st.binned_built = 0;
 }
 
 static void free_transpose(asamd_csr_plan* p, int which) {
@@ -724,13 +743,97 @@ static hipError_t build_hot(hipStream_t stream, asamd_csr_plan* p, const int* ro
   return hipSuccess;
 }
 
+// Row numbers sorted by length class and the chunk table of the longest rows.
+template <typename T>
+static bool binned_eligible(const asamd_csr_plan* p, bool force) {
+  const asamd_csr_stats& st = p->st;
+  if (!st.trusted || st.m < 1 || st.nnz < 1) return false;
+  if (force) return true;
+  if (st.nnz < (1 << 20) || st.max_len <= kBinShort) return false;
+  // rows that differ enough in length for one mapping not to fit: the structural choice was merge-path, or
+  // a lane group per row whose width (from the MEAN length) leaves three quarters of the lanes idle on a
+  // quarter of the rows (row-length histogram: bin b holds the rows of 2^(b-1) .. 2^b - 1 entries)
+  if (p->auto_algo == ASAMD_SPMV_MERGE) return st.max_len > kBinMid;
+  if (p->auto_algo != ASAMD_SPMV_VECTOR) return false;
+  int64_t short_rows = 0;
+  for (int b = 0; b < ASAMD_HIST_BINS && ((int64_t)1 << b) <= p->auto_width / 4; ++b) short_rows += st.hist[b];
+  return short_rows * 4 >= (int64_t)st.m;
+}
+
+template <typename T>
+static hipError_t build_binned(hipStream_t stream, asamd_csr_plan* p, const int* row_ptr) {
+  asamd_csr_stats& st = p->st;
+  const int m = st.m;
+  unsigned *d_key = nullptr, *d_key2 = nullptr, *d_idx = nullptr;
+  int *d_count = nullptr, *d_bounds = nullptr;
+  int h_count[kBinClasses] = {0, 0, 0, 0};
+  hipError_t e = hipMalloc(&d_key, (size_t)m * sizeof(unsigned));
+  if (e == hipSuccess) e = hipMalloc(&d_key2, (size_t)m * sizeof(unsigned));
+  if (e == hipSuccess) e = hipMalloc(&d_idx, (size_t)m * sizeof(unsigned));
+  if (e == hipSuccess) e = hipMalloc(&p->d_bin_rows, (size_t)m * sizeof(int));
+  if (e == hipSuccess) e = hipMalloc(&d_count, sizeof(h_count));
+  if (e == hipSuccess) e = hipMemsetAsync(d_count, 0, sizeof(h_count), stream);
+  if (e == hipSuccess) {
+    bin_keys_kernel<<<(unsigned)(((int64_t)m + 255) / 256), 256, 0, stream>>>(m, row_ptr, d_key, d_idx, d_count);
+    e = hipGetLastError();
+  }
+  if (e == hipSuccess) e = sort_pairs_u32(stream, d_key, d_key2, d_idx, (unsigned*)p->d_bin_rows, (size_t)m, 2);
+  if (e == hipSuccess) e = hipMemcpyAsync(h_count, d_count, sizeof(h_count), hipMemcpyDeviceToHost, stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(stream);
+  const int nlong = h_count[kBinClasses - 1];
+  std::vector<int> bounds, first;
+  std::vector<BinChunk> chunks;
+  if (e == hipSuccess && nlong > 0) {
+    // the long rows' offsets come to the host, which cuts them into chunks
+    bounds.resize((size_t)nlong * 2);
+    e = hipMalloc(&d_bounds, bounds.size() * sizeof(int));
+    if (e == hipSuccess) {
+      bin_row_bounds_kernel<<<(unsigned)((nlong + 255) / 256), 256, 0, stream>>>(nlong, p->d_bin_rows + (m - nlong), row_ptr,
+                                                                               d_bounds);
+      e = hipGetLastError();
+    }
+    if (e == hipSuccess) e = hipMemcpy(bounds.data(), d_bounds, bounds.size() * sizeof(int), hipMemcpyDeviceToHost);
+    if (e == hipSuccess) {
+      std::vector<int> rows((size_t)nlong);
+      e = hipMemcpy(rows.data(), p->d_bin_rows + (m - nlong), rows.size() * sizeof(int), hipMemcpyDeviceToHost);
+      first.resize((size_t)nlong + 1);
+      for (int i = 0; i < nlong && e == hipSuccess; ++i) {
+        first[(size_t)i] = (int)chunks.size();
+        const int64_t b = (int64_t)bounds[2 * (size_t)i] - st.base, en = (int64_t)bounds[2 * (size_t)i + 1] - st.base;
+        for (int64_t c = b; c < en; c += kBinChunk)
+          chunks.push_back(BinChunk{rows[(size_t)i], (int)c, (int)(c + kBinChunk < en ? c + kBinChunk : en)});
+      }
+      first[(size_t)nlong] = (int)chunks.size();
+    }
+    if (e == hipSuccess) e = hipMalloc(&p->d_bin_chunk, chunks.size() * sizeof(BinChunk));
+    if (e == hipSuccess) e = hipMalloc(&p->d_bin_first, first.size() * sizeof(int));
+    if (e == hipSuccess) e = hipMalloc(&p->d_bin_partial, chunks.size() * sizeof(T));
+    if (e == hipSuccess) e = hipMemcpy(p->d_bin_chunk, chunks.data(), chunks.size() * sizeof(BinChunk), hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemcpy(p->d_bin_first, first.data(), first.size() * sizeof(int), hipMemcpyHostToDevice);
+  }
+  for (void* d : {(void*)d_key, (void*)d_key2, (void*)d_idx, (void*)d_count, (void*)d_bounds})
+    if (d) (void)hipFree(d);
+  if (e != hipSuccess) {
+    free_binned(p);
+    return e;
+  }
+  for (int c = 0; c < kBinClasses; ++c) {
+    p->bin_count[c] = h_count[c];
+    st.bin_rows[c] = h_count[c];
+  }
+  p->bin_chunks = (int)chunks.size();
+  st.binned_built = 1;
+  return hipSuccess;
+}
+
 // Time the structural choice on scratch vectors, then the copies that the matrix is eligible for:
 // the ELL copy (cheap to build), and the tiled copy only if the fastest so far is slower than the
 // tiled pair could possibly be.  Keep the fastest and free the copies that lost.  A copy has to win
 // by a margin to be worth its memory.
 template <typename T>
 static hipError_t tune_copies(hipStream_t stream, asamd_csr_plan* p, const int* row_ptr,
-                              const int* col_ind, const T* val, bool tiled_ok, bool ell_ok, bool hot_ok) {
+                              const int* col_ind, const T* val, bool tiled_ok, bool ell_ok, bool hot_ok,
+                              bool binned_ok) {
   asamd_csr_stats& st = p->st;
   T *x = nullptr, *y = nullptr;
   hipEvent_t e0 = nullptr, e1 = nullptr;
@@ -739,8 +842,9 @@ static hipError_t tune_copies(hipStream_t stream, asamd_csr_plan* p, const int* 
   if (e == hipSuccess) e = hipMemsetAsync(x, 0, (size_t)st.n * sizeof(T), stream);
   if (e == hipSuccess) e = hipEventCreate(&e0);
   if (e == hipSuccess) e = hipEventCreate(&e1);
-  float best[4] = {0.f, 0.f, 0.f, 0.f};
-  const int algos[4] = {p->auto_algo, ASAMD_SPMV_TILED, ASAMD_SPMV_ELL, ASAMD_SPMV_MERGE_HOT};
+  constexpr int kCand = 5;
+  float best[kCand] = {0.f, 0.f, 0.f, 0.f, 0.f};
+  const int algos[kCand] = {p->auto_algo, ASAMD_SPMV_TILED, ASAMD_SPMV_ELL, ASAMD_SPMV_MERGE_HOT, ASAMD_SPMV_BINNED};
   auto time_algo = [&](int a) {
     st.algo = algos[a];
     // first run warms up; multiplies of a millisecond and more are timed once, shorter ones twice; a
@@ -797,35 +901,42 @@ static hipError_t tune_copies(hipStream_t stream, asamd_csr_plan* p, const int* 
     e = build_hot<T>(stream, p, row_ptr, col_ind, false);
     if (e == hipSuccess && st.hot_built) time_algo(3);
   }
+  // Very uneven rows: one launch per row-length class (cheap to lay out: a sort of the row numbers)
+  if (e == hipSuccess && binned_ok) {
+    e = build_binned<T>(stream, p, row_ptr);
+    if (e == hipSuccess && st.binned_built) time_algo(4);
+  }
   if (e0) (void)hipEventDestroy(e0);
   if (e1) (void)hipEventDestroy(e1);
   if (x) (void)hipFree(x);
   if (y) (void)hipFree(y);
   st.algo = p->auto_algo;
   if (e != hipSuccess) return e;
+  st.tune_ms_binned = best[4];
   st.tune_ms_base = best[0];
   st.tune_ms_tiled = best[1];
   st.tune_ms_ell = best[2];
   st.tune_ms_hot = best[3];
   // a copy has to win by a margin to be worth its memory; among the winners the fastest is kept
-  const float margin[4] = {1.f, 0.9f, 0.95f, 0.95f};
+  const float margin[kCand] = {1.f, 0.9f, 0.95f, 0.95f, 0.95f};
   int pick = 0;
-  for (int a = 1; a < 4; ++a)
+  for (int a = 1; a < kCand; ++a)
     if (best[a] > 0.f && best[a] < margin[a] * best[0] && (pick == 0 || best[a] < best[pick])) pick = a;
-  // ALSPARSE_AMD_TUNE_PICK = base | tiled | ell | hot overrides the timing's verdict among the candidates
+  // ALSPARSE_AMD_TUNE_PICK = base | tiled | ell | hot | binned overrides the timing's verdict among the candidates
   // that were built (for profiling a kernel that lost)
   if (const char* ev = getenv("ALSPARSE_AMD_TUNE_PICK")) {
-    const char* names[4] = {"base", "tiled", "ell", "hot"};
-    for (int a = 0; a < 4; ++a)
+    const char* names[kCand] = {"base", "tiled", "ell", "hot", "binned"};
+    for (int a = 0; a < kCand; ++a)
       if (!strcmp(ev, names[a]) && (a == 0 || best[a] > 0.f)) pick = a;
   }
   if (pick != 1) free_tiled(p);
   if (pick != 2) free_ell(p);
   if (pick != 3) free_hot(p);
+  if (pick != 4) free_binned(p);
   if (pick != 0) {
     p->auto_algo = algos[pick];
     st.algo = algos[pick];
-    if (pick != 3) p->copy_val_src = val;  // the hot-column copy holds no values
+    if (pick != 3 && pick != 4) p->copy_val_src = val;  // the hot-column copy and the row bins hold no values
   }
   return hipSuccess;
 }
@@ -914,13 +1025,16 @@ static hipError_t plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t 
       hipError_t err = hipSuccess;
       const bool tiled_ok = tiled_eligible<T>(p->st, force), ell_ok = ell_eligible(p->st, force);
       const bool hot_ok = hot_eligible<T>(p, force);
+      const bool binned_ok = binned_eligible<T>(p, force);
       if (force) {
+        if (binned_ok) err = build_binned<T>(stream, p, row_ptr);
+        if (err != hipSuccess) return err;
         if (tiled_ok) err = build_tiled<T>(stream, p, row_ptr, col_ind, (const T*)val);
         if (err == hipSuccess && ell_ok) err = build_ell<T>(stream, p, row_ptr, col_ind, (const T*)val);
         if (err == hipSuccess && hot_ok) err = build_hot<T>(stream, p, row_ptr, col_ind, true);
         p->copy_val_src = val;
-      } else if (tiled_ok || ell_ok || hot_ok) {
-        err = tune_copies<T>(stream, p, row_ptr, col_ind, (const T*)val, tiled_ok, ell_ok, hot_ok);
+      } else if (tiled_ok || ell_ok || hot_ok || binned_ok) {
+        err = tune_copies<T>(stream, p, row_ptr, col_ind, (const T*)val, tiled_ok, ell_ok, hot_ok, binned_ok);
       }
       return err;
     });
@@ -929,7 +1043,9 @@ static hipError_t plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t 
       free_tiled(p);
       free_ell(p);
       free_hot(p);
-      if (p->auto_algo == ASAMD_SPMV_TILED || p->auto_algo == ASAMD_SPMV_ELL || p->auto_algo == ASAMD_SPMV_MERGE_HOT)
+      free_binned(p);
+      if (p->auto_algo == ASAMD_SPMV_TILED || p->auto_algo == ASAMD_SPMV_ELL || p->auto_algo == ASAMD_SPMV_MERGE_HOT ||
+          p->auto_algo == ASAMD_SPMV_BINNED)
         p->auto_algo = p->struct_algo;
       p->st.algo = p->auto_algo;
       e = hipSuccess;
@@ -967,6 +1083,7 @@ extern "C" void asamd_csr_plan_destroy(asamd_csr_plan* p) {
   free_tiled(p);
   free_ell(p);
   free_hot(p);
+  free_binned(p);
   free_transpose(p, 0);
   free_transpose(p, 1);
   delete p;
@@ -1174,6 +1291,10 @@ extern "C" int asamd_csr_plan_set_algo(asamd_csr_plan* p, int32_t algo) {
       if (!p->st.hot_built) return hipErrorInvalidValue;
       p->st.algo = algo;
       return hipSuccess;
+    case ASAMD_SPMV_BINNED:
+      if (!p->st.binned_built) return hipErrorInvalidValue;
+      p->st.algo = algo;
+      return hipSuccess;
     case ASAMD_SPMV_MERGE:
       if (p->st.first_offset != 0) return hipErrorInvalidValue;
       p->st.algo = algo;
@@ -1230,6 +1351,7 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
   if (algo == ASAMD_SPMV_TILED && !st.tiled_built) algo = p->auto_algo == ASAMD_SPMV_TILED ? ASAMD_SPMV_MERGE : p->auto_algo;
   if (algo == ASAMD_SPMV_ELL && !st.ell_built) algo = p->auto_algo == ASAMD_SPMV_ELL ? ASAMD_SPMV_MERGE : p->auto_algo;
   if (algo == ASAMD_SPMV_MERGE_HOT && !st.hot_built) algo = ASAMD_SPMV_MERGE;
+  if (algo == ASAMD_SPMV_BINNED && !st.binned_built) algo = st.first_offset != 0 ? ASAMD_SPMV_VECTOR : ASAMD_SPMV_MERGE;
   switch (algo) {
     case ASAMD_SPMV_ELL: {
       // the ELL copy holds zero-based columns and its own values
@@ -1282,6 +1404,27 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
     case ASAMD_SPMV_SCALAR: {
       const unsigned grid = (unsigned)(((int64_t)st.m + kRowsBlock - 1) / kRowsBlock);
       spmv_scalar_kernel<T><<<grid, kRowsBlock, 0, s>>>(st.m, alpha, val, rp, ci, x, beta, y, st.base);
+      break;
+    }
+    case ASAMD_SPMV_BINNED: {
+      // one launch per row-length class; the classes own disjoint rows, so the launches are independent
+      const int* rows = p->d_bin_rows;
+      const int n0 = p->bin_count[0], n1 = p->bin_count[1], n2 = p->bin_count[2], n3 = p->bin_count[3];
+      auto blocks = [](int count, int w) { return (unsigned)(((int64_t)count * w + kRowsBlock - 1) / kRowsBlock); };
+      if (n0 > 0)
+        spmv_bin_rows_kernel<T, 4><<<blocks(n0, 4), kRowsBlock, 0, s>>>(n0, rows, alpha, val, rp, ci, x, beta, y, st.base);
+      if (n1 > 0)
+        spmv_bin_rows_kernel<T, 16><<<blocks(n1, 16), kRowsBlock, 0, s>>>(n1, rows + n0, alpha, val, rp, ci, x, beta, y,
+                                                                        st.base);
+      if (n2 > 0)
+        spmv_bin_rows_kernel<T, 64><<<blocks(n2, 64), kRowsBlock, 0, s>>>(n2, rows + n0 + n1, alpha, val, rp, ci, x, beta,
+                                                                        y, st.base);
+      if (n3 > 0) {
+        spmv_bin_chunk_kernel<T><<<(unsigned)p->bin_chunks, kRowsBlock, 0, s>>>(p->bin_chunks, p->d_bin_chunk, val, ci, x,
+                                                                               st.base, (T*)p->d_bin_partial);
+        spmv_bin_finish_kernel<T><<<(unsigned)((n3 + 255) / 256), 256, 0, s>>>(n3, rows + n0 + n1 + n2, p->d_bin_first,
+                                                                              (const T*)p->d_bin_partial, alpha, beta, y);
+      }
       break;
     }
     case ASAMD_SPMV_MERGE_HOT: {

@@ -180,6 +180,7 @@ int asamd_env_algo(void) {
   if (!strcmp(e, "stream")) return ASAMD_SPMV_STREAM;
   if (!strcmp(e, "ell")) return ASAMD_SPMV_ELL;
   if (!strcmp(e, "hot")) return ASAMD_SPMV_MERGE_HOT;
+  if (!strcmp(e, "binned")) return ASAMD_SPMV_BINNED;
   return ASAMD_SPMV_AUTO;
 }
 

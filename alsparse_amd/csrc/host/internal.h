@@ -73,7 +73,7 @@ uint64_t asamd_host_fingerprint(const void *values, size_t count, size_t elem);
 /* Process-wide handle for alphasparse_?_mv / _mm (host pointers). */
 alphasparse_status_t asamd_default_handle(alphasparse_dcu_handle_t *handle);
 
-/* ALSPARSE_AMD_SPMV_ALGO = auto | vector | rowconst | merge | scalar | tiled | stream | ell | hot */
+/* ALSPARSE_AMD_SPMV_ALGO = auto | vector | rowconst | merge | scalar | tiled | stream | ell | hot | binned */
 int asamd_env_algo(void);
 /* ALSPARSE_AMD_ANALYSIS = structure: analyses keep no copies of the matrix values (as the reference's),
  * so values may change in place at any time; the default lets an analysis keep re-ordered copies. */

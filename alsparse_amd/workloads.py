@@ -102,6 +102,28 @@ def uniform_rows(rows, cols, k, dtype=np.float32, seed=SEED, base=0, lo=-1.0, hi
     return Csr(rows, cols, row_ptr, col_ind, vals, base, "uniform_rows(%d,%d,%d)" % (rows, cols, k))
 
 
+def bimodal_rows(rows, cols, k_short, k_long, every, dtype=np.float32, seed=SEED, base=0):
+    """Rows of two lengths: every `every`-th row has k_long entries, the others k_short, columns uniform random
+    (sorted, distinct) in both.  Not a benchmark configuration: the workload that the row-length bins are for."""
+    if rows % every:
+        raise ValueError("rows must be a multiple of `every`")
+    periods = rows // every
+    short = uniform_rows(periods * (every - 1), cols, k_short, dtype, seed, base)
+    long_ = uniform_rows(periods, cols, k_long, dtype, seed + 1, base)
+    ks, kl = min(k_short, cols), min(k_long, cols)
+    per = (every - 1) * ks + kl
+    col = np.empty((periods, per), dtype=np.int32)
+    col[:, :(every - 1) * ks] = short.col_ind.reshape(periods, (every - 1) * ks)
+    col[:, (every - 1) * ks:] = long_.col_ind.reshape(periods, kl)
+    lengths = np.full(rows, ks, dtype=np.int64)
+    lengths[every - 1::every] = kl
+    row_ptr = np.zeros(rows + 1, dtype=np.int64)
+    np.cumsum(lengths, out=row_ptr[1:])
+    vals = uniform(periods * per, dtype, 2, seed)
+    return Csr(rows, cols, (row_ptr + base).astype(np.int32), col.reshape(-1), vals, base,
+               "bimodal_rows(%d,%d,%d,%d,%d)" % (rows, cols, k_short, k_long, every))
+
+
 def laplace2d(nx, ny, dtype=np.float64, base=0):
     lib = _load()
     rows = nx * ny

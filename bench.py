@@ -142,7 +142,13 @@ def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False, vendor=Fa
     from alsparse_amd import capi, hiprt, workloads as wl
     lib = capi.load()
     t0 = time.time()
-    if isinstance(cfg, tuple):  # ("uniform", rows, cols, entries per row, dtype): not a benchmark configuration
+    if isinstance(cfg, tuple) and cfg[0] == "bimodal":  # ("bimodal", rows, cols, short, long, every, dtype)
+        _, um, un, ks, kl, every, udt = cfg
+        a = wl.bimodal_rows(um, un, ks, kl, every, udt)
+        x, y0, alpha, beta = wl.uniform(a.cols, udt, 3), wl.uniform(a.rows, udt, 4), 1.0, 0.5
+        workload_name = ("two row lengths: CSR SpMV %s, %d rows x %d columns, every %d-th row %d entries, the others %d, "
+                         "uniform random sorted columns, alpha=1 beta=0.5" % (np.dtype(udt).name, um, un, every, kl, ks))
+    elif isinstance(cfg, tuple):  # ("uniform", rows, cols, entries per row, dtype): not a benchmark configuration
         _, um, un, uk, udt = cfg
         a = wl.uniform_rows(um, un, uk, udt)
         x, y0, alpha, beta = wl.uniform(a.cols, udt, 3), wl.uniform(a.rows, udt, 4), 1.0, 0.5
@@ -242,6 +248,8 @@ def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False, vendor=Fa
            "gbs": nbytes / t["avg_ms"] / 1e6, "gflops": 2 * a.nnz / t["avg_ms"] / 1e6,
            "dtype": {"float32": "f32", "float64": "f64", "complex64": "c64", "complex128": "c128"}[a.dtype.name],
            "parity": parity}
+    # what the analysis measured when it chose the kernel (one multiply each on scratch vectors; 0 = not tried)
+    res["analysis_timings_ms"] = {k: round(float(getattr(stats, "tune_ms_" + k)), 4) for k in ("base", "tiled", "ell", "hot", "binned")}
     if cx:  # a complex multiply-add is 8 real flops
         res["flops"], res["gflops"] = 8 * a.nnz, 8 * a.nnz / t["avg_ms"] / 1e6
     res["hbm_frac"] = res["gbs"] / HBM_PEAK_GBS
@@ -584,7 +592,10 @@ def main():
     ap.add_argument("--uniform", nargs=3, type=int, metavar=("ROWS", "COLS", "PER_ROW"),
                     help="instead of a configuration: CSR SpMV on a matrix of that shape with PER_ROW uniform random "
                          "columns per row (fp32, --fp64 for fp64); same analysis, timing and parity check")
-    ap.add_argument("--fp64", action="store_true", help="with --uniform: fp64 values")
+    ap.add_argument("--bimodal", nargs=5, type=int, metavar=("ROWS", "COLS", "SHORT", "LONG", "EVERY"),
+                    help="instead of a configuration: CSR SpMV on a matrix whose every EVERY-th row has LONG entries "
+                         "and the others SHORT (the workload of the row-length bins)")
+    ap.add_argument("--fp64", action="store_true", help="with --uniform / --bimodal: fp64 values")
     ap.add_argument("--all", action="store_true", help="also measure the other configurations")
     ap.add_argument("--only", action="store_true",
                     help="measure the selected configuration alone (by default the line also carries brief figures of "
@@ -645,10 +656,12 @@ def main():
         cfg = args.config
         if args.uniform:
             cfg = ("uniform", args.uniform[0], args.uniform[1], args.uniform[2], np.float64 if args.fp64 else np.float32)
+        if args.bimodal:
+            cfg = ("bimodal",) + tuple(args.bimodal) + (np.float64 if args.fp64 else np.float32,)
         main_res = run_spmv(cfg, args.steps, args.warmup, not args.no_cpu_baseline, check, args.transpose,
                             not args.no_vendor_baseline, args.cx, args.conjugate)
     others = {}
-    plain_default = (args.config == 3 and not (args.all or args.only or args.uniform or args.transpose or args.cx or
+    plain_default = (args.config == 3 and not (args.all or args.only or args.uniform or args.bimodal or args.transpose or args.cx or
                                                args.conversions or args.col_major) and args.format == "csr")
     if plain_default:
         # the default line is configuration 3; the other device configurations ride along, briefly
@@ -699,7 +712,7 @@ def main():
         "dtype": main_res["dtype"], "data": "synthetic",
         "config": {"workload": main_res["workload"], "rows": main_res["rows"], "nnz": main_res["nnz"],
                    "kernel": main_res.get("kernel", "spmm row-major"), "analysis_ms": main_res.get("analysis_ms"),
-                   "reanalysis_ms": main_res.get("reanalysis_ms")},
+                   "reanalysis_ms": main_res.get("reanalysis_ms"), "analysis_timings_ms": main_res.get("analysis_timings_ms")},
         "gflops": main_res["gflops"], "pct_of_hbm_peak": 100.0 * main_res["hbm_frac"],
         "min_ms": t["min_ms"], "median_ms": t["median_ms"], "wall_ms_per_step": t["wall_ms_per_step"],
         "parity": main_res["parity"],

@@ -38,9 +38,12 @@ enum asamd_spmv_algo {
   ASAMD_SPMV_STREAM = 6,   /* rows of <= 16 entries: 256 rows' products staged in LDS */
   ASAMD_SPMV_ELL = 7,      /* short, nearly equal rows: a column-major ELL copy, one
                               lane per row                                          */
-  ASAMD_SPMV_MERGE_HOT = 8 /* merge-path whose persistent workgroups keep x of the most
+  ASAMD_SPMV_MERGE_HOT = 8, /* merge-path whose persistent workgroups keep x of the most
                               popular columns in LDS (power-law graphs); the copy it
                               needs is structure only: values come from the caller  */
+  ASAMD_SPMV_BINNED = 9    /* one launch per row-length class (4, 16, 64 lanes per row;
+                              the longest rows in chunks, a workgroup each): for very
+                              uneven rows; keeps a list of row numbers, no values   */
 };
 
 #define ASAMD_HIST_BINS 33
@@ -95,6 +98,9 @@ typedef struct {
   int32_t hot_cols;      /* most popular columns whose x every multiply gathers into a compact front */
   float hot_share_lds;   /* share of the entries that fall into the LDS columns               */
   float tune_ms_hot;     /* analysis-time timing of the hot-column kernel, or 0               */
+  int32_t binned_built;  /* 1: the row numbers are sorted by length class (BINNED can be selected) */
+  int32_t bin_rows[4];   /* rows of at most 8 / 64 / 2 048 entries / longer                   */
+  float tune_ms_binned;  /* analysis-time timing of the per-class launches, or 0              */
 } asamd_csr_stats;
 
 typedef struct asamd_csr_plan asamd_csr_plan;

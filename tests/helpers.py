@@ -13,7 +13,7 @@ TOL = {np.dtype(np.float32): 1e-4, np.dtype(np.float64): 1e-12}
 
 ALGOS = {"auto": capi.ASAMD_SPMV_AUTO, "vector": capi.ASAMD_SPMV_VECTOR, "rowconst": capi.ASAMD_SPMV_ROWCONST,
          "merge": capi.ASAMD_SPMV_MERGE, "scalar": capi.ASAMD_SPMV_SCALAR, "tiled": capi.ASAMD_SPMV_TILED,
-         "stream": capi.ASAMD_SPMV_STREAM, "ell": capi.ASAMD_SPMV_ELL, "hot": capi.ASAMD_SPMV_MERGE_HOT}
+         "stream": capi.ASAMD_SPMV_STREAM, "ell": capi.ASAMD_SPMV_ELL, "hot": capi.ASAMD_SPMV_MERGE_HOT, "binned": capi.ASAMD_SPMV_BINNED}
 
 
 def announce(*what):
@@ -59,7 +59,7 @@ def run_plan_csrmv(da, algo, alpha, x, beta, y0, trusted=1):
     lib = capi.load()
     from ctypes import c_void_p
     plan = c_void_p()
-    if algo in ("tiled", "ell", "hot"):
+    if algo in ("tiled", "ell", "hot", "binned"):
         trusted = 2  # build the copies whatever the size
     e = lib.asamd_csr_plan_create(None, a.rows, a.cols, a.nnz, da.row_ptr.c_ptr(), da.col.c_ptr(), da.val.c_ptr(),
                                   a.base, a.dtype.itemsize, trusted, byref(plan))

@@ -112,7 +112,7 @@ def test_complex_csrmv_with_and_without_analysis(gpu, dtype, shape, op):
         da.free()
 
 
-@pytest.mark.parametrize("algo", ["vector", "merge", "scalar", "stream", "ell", "rowconst", "tiled", "hot"])
+@pytest.mark.parametrize("algo", ["vector", "merge", "scalar", "stream", "ell", "rowconst", "tiled", "hot", "binned"])
 @pytest.mark.parametrize("dtype", CX, ids=IDS)
 def test_complex_kernel_families(gpu, dtype, algo):
     """The thin kernel ABI with a forced family; the constant-row-length family (128-bit quads of

@@ -34,6 +34,7 @@ SHAPES = {
     "many_empty_then_long": lambda dt: csr_from_lengths([0] * 5000 + [9000] + [0] * 3000 + [2, 2049, 2047], 20000, dt),
     "single_entry": lambda dt: csr_from_lengths([1], 1, dt),
     "ragged_tail": lambda dt: csr_from_lengths(list(range(0, 300)), 4000, dt),
+    "length_class_edges": lambda dt: csr_from_lengths([8, 9, 0, 64, 65, 2048, 2049, 1, 4096, 4097, 8193, 7, 63], 9000, dt),
     "wide_few_rows": lambda dt: csr_from_lengths([4096, 4095, 4097, 1, 0, 8192], 10000, dt),
 }
 
@@ -45,7 +46,7 @@ def test_every_kernel_family_matches_oracle(gpu, shape, dtype):
     x, y0 = _vectors(a)
     da = DeviceCsr(a)
     try:
-        for algo in ("vector", "merge", "scalar", "rowconst", "stream", "tiled", "ell", "hot", "auto"):
+        for algo in ("vector", "merge", "scalar", "rowconst", "stream", "tiled", "ell", "hot", "binned", "auto"):
             for alpha, beta in ((1.0, 0.0), (2.0, 3.0), (-0.75, 1.0)):
                 announce("spmv", shape, np.dtype(dtype).name, algo, alpha, beta)
                 y = run_plan_csrmv(da, algo, alpha, x, beta, y0)
@@ -65,7 +66,7 @@ def test_index_base_one(gpu, dtype):
         x, y0 = _vectors(a)
         da = DeviceCsr(a)
         try:
-            for algo in ("vector", "merge", "scalar", "stream", "tiled", "ell", "hot", "auto"):
+            for algo in ("vector", "merge", "scalar", "stream", "tiled", "ell", "hot", "binned", "auto"):
                 announce("spmv base1", a.name, algo)
                 y = run_plan_csrmv(da, algo, 1.5, x, 0.25, y0)
                 if y is None:
@@ -85,7 +86,7 @@ def test_beta_zero_ignores_nan_in_y(gpu):
     y0 = np.full(a.rows, np.nan, dtype=np.float32)
     da = DeviceCsr(a)
     try:
-        for algo in ("vector", "merge", "scalar", "tiled", "hot"):
+        for algo in ("vector", "merge", "scalar", "tiled", "hot", "binned"):
             announce("spmv beta0 nan", algo)
             y = run_plan_csrmv(da, algo, 1.0, x, 0.0, y0)
             assert np.isfinite(y).all()
@@ -120,9 +121,11 @@ def test_deterministic_across_runs(gpu):
     x, y0 = _vectors(a)
     da = DeviceCsr(a)
     try:
-        announce("spmv determinism merge")
-        runs = [run_plan_csrmv(da, "merge", 1.0, x, 0.5, y0) for _ in range(3)]
-        assert np.array_equal(runs[0], runs[1]) and np.array_equal(runs[0], runs[2])
+        # the families that sum every row in a fixed order (no floating-point atomics)
+        for algo in ("merge", "hot", "binned", "vector"):
+            announce("spmv determinism", algo)
+            runs = [run_plan_csrmv(da, algo, 1.0, x, 0.5, y0) for _ in range(3)]
+            assert np.array_equal(runs[0], runs[1]) and np.array_equal(runs[0], runs[2]), algo
     finally:
         da.free()
 
@@ -271,7 +274,7 @@ def test_random_structures_every_family(gpu, seed):
     x, y0 = _vectors(a, seed)
     da = DeviceCsr(a)
     try:
-        for algo in ("vector", "merge", "scalar", "rowconst", "stream", "tiled", "ell", "hot", "auto"):
+        for algo in ("vector", "merge", "scalar", "rowconst", "stream", "tiled", "ell", "hot", "binned", "auto"):
             for alpha, beta in ((1.5, 0.0), (-2.0, 0.5)):
                 announce("spmv random", seed, m, n, a.nnz, np.dtype(dtype).name, base, algo, alpha, beta)
                 y = run_plan_csrmv(da, algo, alpha, x, beta, y0)
@@ -301,7 +304,7 @@ def test_unsorted_and_duplicate_columns_and_non_finite_values(gpu, dtype):
     x, y0 = _vectors(a, 5)
     da = DeviceCsr(a)
     try:
-        for algo in ("vector", "merge", "scalar", "stream", "tiled", "ell", "hot", "auto"):
+        for algo in ("vector", "merge", "scalar", "stream", "tiled", "ell", "hot", "binned", "auto"):
             announce("spmv unsorted", np.dtype(dtype).name, algo)
             y = run_plan_csrmv(da, algo, 1.5, x, 0.5, y0)
             if y is not None:
@@ -321,7 +324,7 @@ def test_unsorted_and_duplicate_columns_and_non_finite_values(gpu, dtype):
         ref = orc.csrmv_plain(b, 1.0, x2, 0.0, y0)
     db = DeviceCsr(b)
     try:
-        for algo in ("vector", "merge", "scalar", "tiled", "hot", "auto"):
+        for algo in ("vector", "merge", "scalar", "tiled", "hot", "binned", "auto"):
             announce("spmv non-finite", np.dtype(dtype).name, algo)
             y = run_plan_csrmv(db, algo, 1.0, x2, 0.0, y0)
             assert np.array_equal(np.isnan(y), np.isnan(ref)), algo
