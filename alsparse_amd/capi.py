@@ -132,7 +132,8 @@ class asamd_csr_stats(Structure):
                 ("hist", ctypes.c_int64 * ASAMD_HIST_BINS),
                 ("hot_built", c_int32), ("hot_cols_lds", c_int32), ("hot_cols", c_int32),
                 ("hot_share_lds", c_float), ("tune_ms_hot", c_float),
-                ("binned_built", c_int32), ("bin_rows", c_int32 * 4), ("tune_ms_binned", c_float)]
+                ("binned_built", c_int32), ("bin_rows", c_int32 * 4), ("tune_ms_binned", c_float),
+                ("tile_long_blocks", c_int32)]
 
 
 class asamd_dense_strides(Structure):
@@ -207,7 +208,7 @@ def _per_real_type(ctype):
         "asamd_{s}_csrmv": [_P, _P, T, _P, _P, _P, _P, T, _P],
         "asamd_{s}_csrmv_trans": [_P, _P, T, _P, _P, _P, _P, T, _P],
         "asamd_{s}_ellmv": [_P, _I, _I, T, _P, _P, _I, _I, _P, T, _P],
-        "asamd_{s}_coomv": [_P, _I, _I, c_int64, T, _P, _P, _P, _I, _P, T, _P],
+        "asamd_{s}_coomv": [_P, _I, _I, c_int64, T, _P, _P, _P, _I, _P, T, _P, _P, c_size_t],
         "asamd_{s}_csrmm": [_P, _I, _I, _I, _I, T, _P, _P, _P, _I, _P, T, _P, POINTER(asamd_dense_strides)],
         "asamd_{s}_csrmm_ws": [_P, _I, _I, _I, _I, T, _P, _P, _P, _I, _P, T, _P, POINTER(asamd_dense_strides), _P,
                                c_size_t],
@@ -222,7 +223,7 @@ def _per_complex_type(ctype):
         # thin kernel ABI
         "asamd_{s}_csrmv_op": [_P, _P, _I, T, _P, _P, _P, _P, T, _P],
         "asamd_{s}_ellmv": [_P, _I, _I, T, _P, _P, _I, _I, _P, T, _P],
-        "asamd_{s}_coomv": [_P, _I, _I, c_int64, T, _P, _P, _P, _I, _P, T, _P],
+        "asamd_{s}_coomv": [_P, _I, _I, c_int64, T, _P, _P, _P, _I, _P, T, _P, _P, c_size_t],
         "asamd_{s}_csrmm_ws": [_P, _I, _I, _I, _I, T, _P, _P, _P, _I, _P, T, _P, POINTER(asamd_dense_strides), _P,
                                c_size_t],
         "asamd_{s}_csr2ell": [_P, _I, _P, _P, _P, _I, _I, _I, _P, _P],

@@ -102,8 +102,13 @@ struct asamd_csr_plan {
   int n_chunks;
   int* d_row_block_start;     // row_blocks + 1 first rows
   TileRange* d_ranges;        // row_blocks * col_blocks tile ranges, row block major
-  LongChunk* d_long;          // phase-3 work list: chunks of the tiles too long for phase 2
-  int n_long_chunks;
+  LongBlock* d_long;          // phase-3 work list: the row blocks that have tiles too long for phase 2
+  LongTile* d_long_tiles;     // ... and those tiles, sorted by row block, then by column block
+  int n_long_chunks;          // workgroups of phase 3 (a row block with many long entries has several)
+  int n_long_narrow;          // ... the first so many of them work on row blocks of at most kLongNarrow rows
+  LongFinish* d_long_finish;  // the row blocks that have several, whose sums meet in d_long_scratch
+  int n_long_finish;
+  void* d_long_scratch;
   int tiled_halves;           // entries per lane and tile in phase 2: 2, or 1 where (nearly) all tiles are short
   void* d_tval;               // nnz values in tile order
   unsigned* d_tperm;          // nnz: CSR position of the entry in every tile-order slot (for refreshing d_tval)
@@ -234,7 +239,15 @@ static void free_tiled(asamd_csr_plan* p) {
   if (p->d_row_block_start) (void)hipFree(p->d_row_block_start);
   p->d_row_block_start = nullptr;
   if (p->d_long) (void)hipFree(p->d_long);
+  if (p->d_long_tiles) (void)hipFree(p->d_long_tiles);
+  if (p->d_long_finish) (void)hipFree(p->d_long_finish);
+  if (p->d_long_scratch) (void)hipFree(p->d_long_scratch);
   p->d_long = nullptr;
+  p->d_long_tiles = nullptr;
+  p->d_long_finish = nullptr;
+  p->d_long_scratch = nullptr;
+  p->n_long_finish = 0;
+  p->st.tile_long_blocks = 0;
   p->n_long_chunks = 0;
   p->tiled_halves = 2;
   if (p->d_tval) (void)hipFree(p->d_tval);
@@ -576,22 +589,62 @@ static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* 
     if (e == hipSuccess && n_long > 0)
       e = hipMemcpy(h_long.data(), d_long_raw, (size_t)n_long * sizeof(LongTile), hipMemcpyDeviceToHost);
     if (e == hipSuccess && n_long > 0) {
-      std::sort(h_long.begin(), h_long.begin() + n_long,
-                [](const LongTile& a, const LongTile& b) { return a.begin < b.begin; });
-      std::vector<LongChunk> h_lc;
-      for (int i = 0; i < n_long; ++i) {
-        for (int64_t b = h_long[(size_t)i].begin; b < h_long[(size_t)i].end; b += kLongChunk) {
-          LongChunk c;
-          c.begin = (int)b;
-          c.end = (int)(b + kLongChunk < h_long[(size_t)i].end ? b + kLongChunk : h_long[(size_t)i].end);
-          c.row0 = h_rbs[(size_t)h_long[(size_t)i].row_block];
-          h_lc.push_back(c);
+      // by row block; inside a row block by position, which is column block order
+      std::sort(h_long.begin(), h_long.begin() + n_long, [](const LongTile& a, const LongTile& b) {
+        return a.row_block != b.row_block ? a.row_block < b.row_block : a.begin < b.begin;
+      });
+      std::vector<LongBlock> h_lb;
+      std::vector<LongFinish> h_fin;
+      int64_t scratch_len = 0;
+      int long_blocks = 0;
+      for (int i = 0; i < n_long;) {
+        int j = i;
+        while (j < n_long && h_long[(size_t)j].row_block == h_long[(size_t)i].row_block) ++j;
+        const int rbk = h_long[(size_t)i].row_block;
+        const int row0 = h_rbs[(size_t)rbk], nrows = h_rbs[(size_t)rbk + 1] - h_rbs[(size_t)rbk];
+        // runs of tiles with about kLongPart entries each
+        const size_t first_part = h_lb.size();
+        for (int t = i; t < j;) {
+          int64_t entries = 0;
+          int u = t;
+          while (u < j && (u == t || entries + (h_long[(size_t)u].end - h_long[(size_t)u].begin) <= kLongPart)) {
+            entries += h_long[(size_t)u].end - h_long[(size_t)u].begin;
+            ++u;
+          }
+          h_lb.push_back(LongBlock{t, u - t, row0, nrows, -1});
+          t = u;
         }
+        const int parts = (int)(h_lb.size() - first_part);
+        if (parts > 1) {
+          h_fin.push_back(LongFinish{row0, nrows, (int)scratch_len, parts});
+          for (int q = 0; q < parts; ++q) h_lb[first_part + (size_t)q].out = (int)(scratch_len + (int64_t)q * nrows);
+          scratch_len += (int64_t)parts * nrows;
+        }
+        ++long_blocks;
+        i = j;
       }
-      p->n_long_chunks = (int)h_lc.size();
-      e = hipMalloc(&p->d_long, h_lc.size() * sizeof(LongChunk));
+      // the narrow row blocks first: they are launched with small accumulators, so more of them share a compute unit
+      std::stable_partition(h_lb.begin(), h_lb.end(), [](const LongBlock& b) { return b.nrows <= kLongNarrow; });
+      p->n_long_narrow = 0;
+      for (const LongBlock& b : h_lb) p->n_long_narrow += b.nrows <= kLongNarrow;
+      if (scratch_len >= INT32_MAX) e = hipErrorOutOfMemory;
+      p->n_long_chunks = (int)h_lb.size();
+      p->n_long_finish = (int)h_fin.size();
+      st.tile_long_blocks = long_blocks;
+      if (e == hipSuccess) e = hipMalloc(&p->d_long, h_lb.size() * sizeof(LongBlock));
+      if (e == hipSuccess && !h_fin.empty()) {
+        e = hipMalloc(&p->d_long_finish, h_fin.size() * sizeof(LongFinish));
+        if (e == hipSuccess) e = hipMalloc(&p->d_long_scratch, (size_t)scratch_len * sizeof(T));
+        if (e == hipSuccess)
+          e = hipMemcpy(p->d_long_finish, h_fin.data(), h_fin.size() * sizeof(LongFinish), hipMemcpyHostToDevice);
+      }
+      if (e == hipSuccess) e = hipMalloc(&p->d_long_tiles, (size_t)n_long * sizeof(LongTile));
+      if (e == hipSuccess) e = hipMemcpy(p->d_long, h_lb.data(), h_lb.size() * sizeof(LongBlock), hipMemcpyHostToDevice);
       if (e == hipSuccess)
-        e = hipMemcpy(p->d_long, h_lc.data(), h_lc.size() * sizeof(LongChunk), hipMemcpyHostToDevice);
+        e = hipMemcpy(p->d_long_tiles, h_long.data(), (size_t)n_long * sizeof(LongTile), hipMemcpyHostToDevice);
+      if (e == hipSuccess)
+        e = hipFuncSetAttribute((const void*)tiled_long_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (kLongThreads / kWave) * (TileDims<T>::rows + kWave) * (int)sizeof(T));
     }
   }
   // ---- 4. phase-1 work list: every column block cut into chunks of at most kChunk entries
@@ -868,8 +921,8 @@ static hipError_t tune_copies(hipStream_t stream, asamd_csr_plan* p, const int* 
                        ((double)st.n + (double)st.m) * sizeof(T);
   float tiled_floor_ms = (float)(2.0 * bytes / 5.0e9);
   // Heavy-tailed rows (power-law graphs) make uneven tiles: the in-wave combining of equal rows and the
-  // long-tile phase then cost the tiled pair about 2.5 times its floor (measured 0.8-0.9 ms against 0.34 ms
-  // on an 8 M-row R-MAT matrix whose longest row has 200 000 entries).
+  // long-tile phase then cost the tiled pair about 2.3 times its floor (measured 0.78 ms against 0.34 ms
+  // on an 8 M-row R-MAT matrix whose longest row has 120 000 entries; 0.65 ms on its transpose).
   if ((double)st.max_len > 32.0 * ((double)st.nnz / (double)st.m) + 256.0) tiled_floor_ms *= 2.5f;
   if (e == hipSuccess) time_algo(0);
   // An ELL copy gathers x row by row like the kernel just timed; when that one is several times slower
@@ -1375,8 +1428,18 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
             st.m, st.tile_row_blocks, st.tile_col_blocks, p->d_row_block_start, p->d_ranges, p->d_trow,
             (const T*)p->d_tprod, alpha, beta, y);
       if (p->n_long_chunks > 0)
-        tiled_long_kernel<T><<<p->n_long_chunks, kLongThreads, 0, s>>>(p->d_long, p->d_trow,
-                                                                       (const T*)p->d_tprod, alpha, y);
+        {
+        const int waves = kLongThreads / kWave, narrow = p->n_long_narrow, wide = p->n_long_chunks - narrow;
+        if (narrow > 0)
+          tiled_long_kernel<T><<<narrow, kLongThreads, waves * (kLongNarrow + kWave) * (int)sizeof(T), s>>>(
+              p->d_long, p->d_long_tiles, p->d_trow, (const T*)p->d_tprod, alpha, y, (T*)p->d_long_scratch, kLongNarrow);
+        if (wide > 0)
+          tiled_long_kernel<T><<<wide, kLongThreads, waves * (TileDims<T>::rows + kWave) * (int)sizeof(T), s>>>(
+              p->d_long + narrow, p->d_long_tiles, p->d_trow, (const T*)p->d_tprod, alpha, y, (T*)p->d_long_scratch,
+              TileDims<T>::rows);
+        }
+      if (p->n_long_finish > 0)
+        tiled_long_finish_kernel<T><<<p->n_long_finish, 256, 0, s>>>(p->d_long_finish, (const T*)p->d_long_scratch, alpha, y);
       break;
     }
     case ASAMD_SPMV_ROWCONST: if constexpr (kIsReal<T>) {

@@ -14,10 +14,14 @@
 //   src/kernel/dcu/level2/mv/dcu_gemv_x_coo.cpp:10-195, which stages the same
 //   scan through LDS with a barrier per step, writes y without atomics (a row
 //   shared by two waves races there) and finishes with a one-workgroup pass.
-//   Here segment sums reach y through hardware float atomics, so rows split
-//   between waves, and even entries that are not grouped by row at all, are
-//   summed correctly; only the order of the additions to such a shared row is
-//   not fixed.  y is scaled by beta beforehand, as in the reference (:161-169).
+//   Here the first and the last segment of every wave go to boundary slots and
+//   a second kernel adds the slots of one row up in wave order (the
+//   reference's carry-out and block reduction, :169-255, as one ordered pass);
+//   every sum reaches y through one hardware float atomic.  Entries grouped by
+//   row therefore give the same result from run to run, and entries that are
+//   not grouped by row at all are still summed correctly (then the order of the
+//   additions to a row that turns up in several places is not fixed).  y is
+//   scaled by beta beforehand, as in the reference (:161-169).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -37,22 +41,35 @@ __global__ __launch_bounds__(256) void scale_y_kernel(int m, T beta, T* __restri
 }
 
 constexpr int kCooThreads = 256;
-constexpr int kCooSteps = 16;                        // 64-entry steps per wave
-constexpr int kCooPerWave = kWave * kCooSteps;       // entries per wave
-constexpr int kCooPerBlock = kCooPerWave * (kCooThreads / kWave);
+constexpr int kCooSteps = 16;                        // 64-entry steps per wave (more when the workspace is short)
+constexpr int kCooWaves = kCooThreads / kWave;
 
+// With boundary slots (b_row != nullptr): the wave's first and last row segment -- the ones that may belong
+// to rows shared with the neighbouring waves -- do not go to y but to slots 2w (head) and 2w + 1 (tail) of
+// the wave; coomv_boundary_kernel adds the runs of equal rows up in wave order and adds each run once.
+// Entries that are grouped by row therefore reach every y through a single addition of a sum formed in a
+// fixed order: the result is the same from run to run.
 template <typename T>
 __global__ __launch_bounds__(kCooThreads) void coomv_kernel(int64_t nnz, int m, int n, T alpha,
                                                             const T* __restrict__ coo_val,
                                                             const int* __restrict__ coo_row,
                                                             const int* __restrict__ coo_col, int base,
-                                                            const T* __restrict__ x, T* __restrict__ y) {
+                                                            const T* __restrict__ x, T* __restrict__ y, int per_wave,
+                                                            int* __restrict__ b_row, T* __restrict__ b_val) {
   const int lane = threadIdx.x % kWave;
-  const int64_t wave = (int64_t)blockIdx.x * (kCooThreads / kWave) + threadIdx.x / kWave;
-  const int64_t begin = wave * kCooPerWave;
-  const int64_t end = begin + kCooPerWave < nnz ? begin + kCooPerWave : nnz;
-  int carry_row = -1;  // open segment handed from one step to the next (same in all lanes)
+  const int64_t wave = (int64_t)blockIdx.x * kCooWaves + threadIdx.x / kWave;
+  const int64_t begin = wave * per_wave;
+  const int64_t end = begin + per_wave < nnz ? begin + per_wave : nnz;
+  if (begin >= end) {
+    if (b_row && lane < 2) b_row[2 * wave + lane] = -1;  // a wave past the end: empty slots
+    return;
+  }
+  const bool slots = b_row != nullptr;
+  bool emitted = !slots;  // whether the wave's first segment has gone out (wave-uniform); without slots: nothing special
+  int carry_row = -1;     // open segment handed from one step to the next (same in all lanes)
   T carry_val = T(0);
+  int head_row = -1;
+  T head_val = T(0);
   for (int64_t k0 = begin; k0 < end; k0 += kWave) {
     const int64_t k = k0 + lane;
     int r = -1;
@@ -65,21 +82,73 @@ __global__ __launch_bounds__(kCooThreads) void coomv_kernel(int64_t nnz, int m, 
         v = nt_load(&coo_val[k]) * x[c];
       }
     }
+    const int r0 = lane_bcast(r, 0);
+    const bool flush = carry_row != r0 && carry_row >= 0;  // the carried segment ended with the last step
+    if (flush && !emitted) {
+      head_row = carry_row;
+      head_val = carry_val;
+    }
     if (lane == 0) {
       if (carry_row == r) v += carry_val;
-      else if (carry_row >= 0) atomic_add(&y[carry_row], alpha * carry_val);
+      else if (flush && emitted) atomic_add(&y[carry_row], alpha * carry_val);
     }
+    if (flush) emitted = true;
     // rows of the neighbouring lanes through DPP wave shifts (lane 0 sees -2, lane 63 sees -2: never a row)
     const int r_prev = __builtin_amdgcn_update_dpp(-2, r, 0x138, 0xF, 0xF, false);  // wave_shr:1
     const int r_next = __builtin_amdgcn_update_dpp(-2, r, 0x130, 0xF, 0xF, false);  // wave_shl:1
     const bool head = lane == 0 || r_prev != r;
     v = segmented_scan(v, head);
     // the last lane of every row segment adds the segment's sum; lane 63's segment stays open
-    if (lane < kWave - 1 && r_next != r && r >= 0) atomic_add(&y[r], alpha * v);
+    const bool ends = lane < kWave - 1 && r_next != r && r >= 0;
+    const uint64_t end_mask = __builtin_amdgcn_ballot_w64(ends);
+    const int first_end = end_mask ? __builtin_ctzll(end_mask) : kWave;
+    if (!emitted && end_mask) {  // the wave's first segment ends inside this step
+      head_row = lane_bcast(r, first_end);
+      head_val = lane_bcast(v, first_end);
+    }
+    if (ends && (emitted || lane != first_end)) atomic_add(&y[r], alpha * v);
+    if (end_mask) emitted = true;
     carry_row = lane_bcast(r, kWave - 1);
     carry_val = lane_bcast(v, kWave - 1);
   }
-  if (lane == 0 && carry_row >= 0) atomic_add(&y[carry_row], alpha * carry_val);
+  if (!slots) {
+    if (lane == 0 && carry_row >= 0) atomic_add(&y[carry_row], alpha * carry_val);
+    return;
+  }
+  if (!emitted) {  // one segment (or none) in the whole wave: it is the head, there is no tail
+    head_row = carry_row;
+    head_val = carry_val;
+    carry_row = -1;
+  }
+  if (lane == 0) {
+    b_row[2 * wave] = head_row;
+    b_val[2 * wave] = head_val;
+    b_row[2 * wave + 1] = carry_row;
+    b_val[2 * wave + 1] = carry_val;
+  }
+}
+
+// Slot i starts a run if the nearest filled slot below it names another row; the run's sums are added in
+// slot order and reach y through one addition (atomic: entries that are not grouped by row may have put the
+// same row elsewhere).
+template <typename T>
+__global__ __launch_bounds__(256) void coomv_boundary_kernel(int64_t slots, T alpha, const int* __restrict__ b_row,
+                                                             const T* __restrict__ b_val, T* __restrict__ y) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= slots) return;
+  const int r = b_row[i];
+  if (r < 0) return;
+  int64_t q = i - 1;
+  while (q >= 0 && b_row[q] < 0) --q;
+  if (q >= 0 && b_row[q] == r) return;
+  T sum = b_val[i];
+  for (int64_t j = i + 1; j < slots; ++j) {
+    const int rj = b_row[j];
+    if (rj < 0) continue;
+    if (rj != r) break;
+    sum += b_val[j];
+  }
+  atomic_add(&y[r], alpha * sum);
 }
 
 template <typename T>
@@ -95,7 +164,8 @@ int ellmv_impl(hipStream_t stream, int32_t m, int32_t n, T alpha, const T* ell_v
 
 template <typename T>
 int coomv_impl(hipStream_t stream, int32_t m, int32_t n, int64_t nnz, T alpha, const T* coo_val,
-               const int32_t* coo_row, const int32_t* coo_col, int32_t base, const T* x, T beta, T* y) {
+               const int32_t* coo_row, const int32_t* coo_col, int32_t base, const T* x, T beta, T* y, void* workspace,
+               size_t workspace_bytes) {
   if (m < 0 || n < 0 || nnz < 0) return (int)hipErrorInvalidValue;
   if (((uintptr_t)coo_val | (uintptr_t)x | (uintptr_t)y) % alignof(T)) return (int)hipErrorInvalidValue;
   if (m == 0) return (int)hipSuccess;
@@ -105,10 +175,33 @@ int coomv_impl(hipStream_t stream, int32_t m, int32_t n, int64_t nnz, T alpha, c
     if (e != hipSuccess) return (int)e;
   }
   if (nnz == 0) return (int)hipSuccess;
-  const int64_t grid = (nnz + kCooPerBlock - 1) / kCooPerBlock;
+  // two boundary slots (row, sum) per wave in the workspace; a short workspace means longer waves
+  int per_wave = kWave * kCooSteps;
+  int* b_row = nullptr;
+  T* b_val = nullptr;
+  const size_t slot_bytes = 2 * (sizeof(T) + sizeof(int));
+  if (workspace && (uintptr_t)workspace % 16 == 0 && workspace_bytes >= 64 * slot_bytes) {
+    const int64_t max_waves = (int64_t)(workspace_bytes / slot_bytes) / kCooWaves * kCooWaves;
+    int64_t waves = (nnz + per_wave - 1) / per_wave;
+    if (waves > max_waves) {
+      const int64_t steps = (nnz + max_waves * kWave - 1) / (max_waves * kWave);
+      if (steps * kWave < INT32_MAX / 2) per_wave = (int)(steps * kWave);
+      waves = (nnz + per_wave - 1) / per_wave;
+    }
+    if (waves <= max_waves) {
+      b_val = (T*)workspace;
+      b_row = (int*)((char*)workspace + (size_t)max_waves * 2 * sizeof(T));
+    }
+  }
+  const int64_t per_block = (int64_t)per_wave * kCooWaves;
+  const int64_t grid = (nnz + per_block - 1) / per_block;
   if (grid > 0x7fffffff) return (int)hipErrorInvalidValue;
-  coomv_kernel<T><<<(unsigned)grid, kCooThreads, 0, stream>>>(nnz, m, n, alpha, coo_val, coo_row, coo_col, base, x,
-                                                              y);
+  coomv_kernel<T><<<(unsigned)grid, kCooThreads, 0, stream>>>(nnz, m, n, alpha, coo_val, coo_row, coo_col, base, x, y,
+                                                              per_wave, b_row, b_val);
+  if (b_row) {
+    const int64_t slots = grid * kCooWaves * 2;
+    coomv_boundary_kernel<T><<<(unsigned)((slots + 255) / 256), 256, 0, stream>>>(slots, alpha, b_row, b_val, y);
+  }
   return (int)hipGetLastError();
 }
 
@@ -131,15 +224,16 @@ int asamd_d_ellmv(hipStream_t stream, int32_t m, int32_t n, double alpha, const 
 
 int asamd_s_coomv(hipStream_t stream, int32_t m, int32_t n, int64_t nnz, float alpha, const float* coo_val,
                   const int32_t* coo_row_ind, const int32_t* coo_col_ind, int32_t base, const float* x,
-                  float beta, float* y) {
-  return asamd::coomv_impl<float>(stream, m, n, nnz, alpha, coo_val, coo_row_ind, coo_col_ind, base, x, beta, y);
+                  float beta, float* y, void* workspace, size_t workspace_bytes) {
+  return asamd::coomv_impl<float>(stream, m, n, nnz, alpha, coo_val, coo_row_ind, coo_col_ind, base, x, beta, y, workspace,
+                                  workspace_bytes);
 }
 
 int asamd_d_coomv(hipStream_t stream, int32_t m, int32_t n, int64_t nnz, double alpha, const double* coo_val,
                   const int32_t* coo_row_ind, const int32_t* coo_col_ind, int32_t base, const double* x,
-                  double beta, double* y) {
+                  double beta, double* y, void* workspace, size_t workspace_bytes) {
   return asamd::coomv_impl<double>(stream, m, n, nnz, alpha, coo_val, coo_row_ind, coo_col_ind, base, x, beta,
-                                   y);
+                                   y, workspace, workspace_bytes);
 }
 
 // complex element types: the same kernels over Cx<float> / Cx<double>
@@ -161,18 +255,20 @@ int asamd_z_ellmv(hipStream_t stream, int32_t m, int32_t n, asamd_complex16 alph
 
 int asamd_c_coomv(hipStream_t stream, int32_t m, int32_t n, int64_t nnz, asamd_complex8 alpha,
                   const asamd_complex8* coo_val, const int32_t* coo_row_ind, const int32_t* coo_col_ind,
-                  int32_t base, const asamd_complex8* x, asamd_complex8 beta, asamd_complex8* y) {
+                  int32_t base, const asamd_complex8* x, asamd_complex8 beta, asamd_complex8* y, void* workspace,
+                  size_t workspace_bytes) {
   using T = asamd::Cx<float>;
   return asamd::coomv_impl<T>(stream, m, n, nnz, T(alpha.real, alpha.imag), (const T*)coo_val, coo_row_ind,
-                              coo_col_ind, base, (const T*)x, T(beta.real, beta.imag), (T*)y);
+                              coo_col_ind, base, (const T*)x, T(beta.real, beta.imag), (T*)y, workspace, workspace_bytes);
 }
 
 int asamd_z_coomv(hipStream_t stream, int32_t m, int32_t n, int64_t nnz, asamd_complex16 alpha,
                   const asamd_complex16* coo_val, const int32_t* coo_row_ind, const int32_t* coo_col_ind,
-                  int32_t base, const asamd_complex16* x, asamd_complex16 beta, asamd_complex16* y) {
+                  int32_t base, const asamd_complex16* x, asamd_complex16 beta, asamd_complex16* y, void* workspace,
+                  size_t workspace_bytes) {
   using T = asamd::Cx<double>;
   return asamd::coomv_impl<T>(stream, m, n, nnz, T(alpha.real, alpha.imag), (const T*)coo_val, coo_row_ind,
-                              coo_col_ind, base, (const T*)x, T(beta.real, beta.imag), (T*)y);
+                              coo_col_ind, base, (const T*)x, T(beta.real, beta.imag), (T*)y, workspace, workspace_bytes);
 }
 
 }  // extern "C"

@@ -34,14 +34,14 @@
 //            stride.
 //   phase 3  tiled_long_kernel       only if some tile holds more than kLongTile
 //            entries (long rows, hot columns): those tiles are left out of phase
-//            2 and streamed by as many workgroups as their size needs; rows are
-//            pre-combined inside each wave and added to y with global atomics
-//            (a 200 000-entry row costs a few thousand of them).
+//            2; one workgroup per row block that has any deals them to its waves,
+//            which add them into LDS accumulators of their own; the waves'
+//            accumulators meet in wave order and are added to y.
 //
 // HBM traffic is 2*sizeof(T) + 4 bytes per entry more than plain CSR (the
 // product round trip and the second index), all of it streamed.  The order of
-// every addition in phases 1 and 2 is fixed by the layout, so results are
-// bit-reproducible; only rows that reach phase 3 see atomics in arbitrary order.
+// every addition is fixed by the layout (no floating-point atomics anywhere), so
+// results are bit-reproducible.
 // The reference has no counterpart; per-entry arithmetic is that of
 // src/kernel/dcu/level2/mv/csrmv/dcu_gemv_vector.h:43-54.
 #pragma once
@@ -59,8 +59,9 @@ constexpr int kProdThreads = 1024;      // phase-1 workgroup
 constexpr int kRedWaves = 8;            // phase-2 workgroup: 8 waves = 8 consecutive row blocks, whose tiles are adjacent in memory
 constexpr int kRedSlots = 16;
 constexpr int kLongTile = 2 * kWave;     // phase 2 takes at most two entries per lane and tile; longer tiles go to phase 3
-constexpr int kLongThreads = 256;
-constexpr int kLongChunk = kLongThreads * 16;  // entries per phase-3 workgroup
+constexpr int kLongThreads = 512;  // phase 3: eight waves share the long tiles of one row block
+constexpr int kLongPart = 32768;   // ... up to about this many entries; a row block with more gets several workgroups
+constexpr int kLongNarrow = 256;   // row blocks of at most this many rows (hub rows) run with small accumulators
 constexpr int kTiledMaxColBlocks = 2048;       // keeps the tile table small
 constexpr int64_t kTiledMaxTiles = (int64_t)1 << 25;  // 12 bytes of tables per tile
 
@@ -100,9 +101,15 @@ struct LongTile {
   int row_block;
 };
 
-struct LongChunk {
-  int begin, end;  // entry range inside one long tile
-  int row0;        // first row of the tile's row block
+struct LongBlock {
+  int first, count;  // long tiles of one row block, a run in the sorted list of long tiles
+  int row0, nrows;   // the row block's rows
+  int out;           // -1: the only part of its row block, adds to y itself; else where its sums go in the scratch
+};
+
+struct LongFinish {  // a row block whose long tiles were dealt to several workgroups
+  int row0, nrows;
+  int out0, parts;   // part p left its sums at scratch[out0 + p * nrows ...]
 };
 
 // ---- analysis ----------------------------------------------------------------
@@ -571,36 +578,77 @@ __global__ __launch_bounds__(TileDims<T>::red_threads) void tiled_reduce_kernel(
 }
 
 // ---- phase 3 -------------------------------------------------------------------
-// y[row0 + r] += alpha * v for the entries of one chunk of a long tile; rows are
-// pre-combined inside every wave instruction (add_rows), what is left goes to y
-// with global atomics.  Runs after phase 2 has written y = beta*y + alpha*acc.
+// One workgroup per row block that has tiles too long for phase 2 (several, each with a run of the tiles,
+// where the block has more than kLongPart such entries: a few hub rows can hold a good part of a power-law
+// matrix).  The long tiles (in column block order) are dealt to the workgroup's waves in pieces of 256 entries; every wave
+// streams its pieces and adds them into accumulators of its own in LDS (as phase 2 does: equal rows inside
+// one instruction are combined first), then the waves' accumulators are added in wave order and
+// y[row] += alpha * sum -- or, for a row block with several workgroups, the sums go to a scratch array and
+// tiled_long_finish_kernel adds them up in part order.  Which wave takes which piece and the order of every
+// addition are fixed by the layout: no atomics, results identical from run to run.  Runs after phase 2 has
+// written y = beta*y + alpha*acc.
 template <typename T>
 __global__ __launch_bounds__(kLongThreads) void tiled_long_kernel(
-    const LongChunk* __restrict__ chunks, const unsigned short* __restrict__ t_row,
-    const T* __restrict__ prod, T alpha, T* __restrict__ y) {
-  const LongChunk ch = chunks[blockIdx.x];
+    const LongBlock* __restrict__ blocks, const LongTile* __restrict__ tiles, const unsigned short* __restrict__ t_row,
+    const T* __restrict__ prod, T alpha, T* __restrict__ y, T* __restrict__ scratch, int rows_cap) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  constexpr int kWaves = kLongThreads / kWave;
+  // every wave's accumulators (rows_cap of them: no row block of this launch has more rows), then one dummy
+  // row per lane
+  const int kTileRows = rows_cap;
+  const int kStride = kTileRows + kWave;
+  T* s_acc = reinterpret_cast<T*>(smem);
+  const LongBlock lb = blocks[blockIdx.x];
   const int lane = threadIdx.x % kWave;
-  T* yb = y + ch.row0;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  T* acc = s_acc + wave * kStride;
+  for (int i = lane; i < kStride; i += kWave) acc[i] = T(0);
+  const int r_none = kTileRows + lane;
   constexpr int kU = 4;
-  int k0 = ch.begin;
-  for (; k0 + kLongThreads * kU <= ch.end; k0 += kLongThreads * kU) {
-    T v[kU];
-    int r[kU];
+  for (int t = lb.first; t < lb.first + lb.count; ++t) {
+    const int begin = tiles[t].begin, end = tiles[t].end;
+    // pieces of 64 * kU consecutive entries go to the waves in turn; the turn carries on from tile to tile
+    // (tile t starts with wave t mod kWaves), so that short tiles do not all land on the first waves
+    const int lead = (wave - (t - lb.first) % kWaves + kWaves) % kWaves;
+    for (int k0 = begin + lead * (kWave * kU); k0 < end; k0 += kWaves * kWave * kU) {
+      if (k0 + kWave * kU <= end) {
+        T v[kU];
+        int r[kU];
 #pragma unroll
-    for (int u = 0; u < kU; ++u) {  // wave w takes 64 * kU consecutive entries: runs of one row stay together
-      const int k = k0 + (threadIdx.x / kWave) * (kWave * kU) + u * kWave + lane;
-      v[u] = alpha * prod[k];
-      r[u] = t_row[k];
+        for (int u = 0; u < kU; ++u) {
+          v[u] = prod[k0 + u * kWave + lane];
+          r[u] = t_row[k0 + u * kWave + lane];
+        }
+#pragma unroll
+        for (int u = 0; u < kU; ++u) add_rows<false, true>(acc, r[u], v[u], true);
+      } else {
+        for (int k1 = k0; k1 < end; k1 += kWave) {  // wave-uniform trip count
+          const int k = k1 + lane;
+          const bool ok = k < end;
+          add_rows<false, true>(acc, ok ? (int)t_row[k] : r_none, ok ? prod[k] : T(0), true);
+        }
+      }
     }
-#pragma unroll
-    for (int u = 0; u < kU; ++u) add_rows<true>(yb, r[u], v[u], true);
   }
-  for (; k0 < ch.end; k0 += kLongThreads) {  // workgroup-uniform trip count
-    const int k = k0 + threadIdx.x;
-    const bool ok = k < ch.end;
-    const T v = ok ? alpha * prod[k] : T(0);
-    const int r = ok ? (int)t_row[k] : -2 - lane;
-    add_rows<true>(yb, r, v, ok);
+  __syncthreads();
+  for (int i = threadIdx.x; i < lb.nrows; i += kLongThreads) {
+    T sum = s_acc[i];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) sum += s_acc[w * kStride + i];
+    if (lb.out < 0) y[(int64_t)lb.row0 + i] += alpha * sum;
+    else scratch[(int64_t)lb.out + i] = sum;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void tiled_long_finish_kernel(const LongFinish* __restrict__ fin,
+                                                                const T* __restrict__ scratch, T alpha,
+                                                                T* __restrict__ y) {
+  const LongFinish f = fin[blockIdx.x];
+  for (int i = threadIdx.x; i < f.nrows; i += 256) {
+    T sum = scratch[(int64_t)f.out0 + i];
+    for (int p = 1; p < f.parts; ++p) sum += scratch[(int64_t)f.out0 + (int64_t)p * f.nrows + i];
+    y[(int64_t)f.row0 + i] += alpha * sum;
   }
 }
 

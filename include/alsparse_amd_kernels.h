@@ -101,6 +101,8 @@ typedef struct {
   int32_t binned_built;  /* 1: the row numbers are sorted by length class (BINNED can be selected) */
   int32_t bin_rows[4];   /* rows of at most 8 / 64 / 2 048 entries / longer                   */
   float tune_ms_binned;  /* analysis-time timing of the per-class launches, or 0              */
+  int32_t tile_long_blocks; /* tiled copy: row blocks with tiles too long for its second phase (its third
+                               phase takes them), or 0                                           */
 } asamd_csr_stats;
 
 typedef struct asamd_csr_plan asamd_csr_plan;
@@ -352,20 +354,29 @@ int asamd_z_ellmv(hipStream_t stream, int32_t m, int32_t n, asamd_complex16 alph
 /* y = alpha*A*x + beta*y, A in COO.  Fastest when entries are grouped by row
  * (as asamd_csr2coo leaves them) but correct for any order; entries whose row or
  * column (minus base) is out of range are skipped.  y must be ordinary device
- * memory (hardware float atomics).  Stands in for dcu_gemv_?_coo,
+ * memory (hardware float atomics).  workspace: device memory, 16-byte aligned, for two
+ * (row, sum) slots per wave, where the first and last row segment of every wave meet
+ * their neighbours' in wave order, so that entries grouped by row give the same y from
+ * run to run; a small workspace makes the waves longer (1 MiB serves any size), NULL
+ * sends every segment to y at once (rows shared by waves then add up in any order).
+ * Stands in for dcu_gemv_?_coo,
  * src/kernel/dcu/level2/mv/dcu_gemv_x_coo.cpp:10-195. */
 int asamd_s_coomv(hipStream_t stream, int32_t m, int32_t n, int64_t nnz, float alpha,
                   const float *coo_val, const int32_t *coo_row_ind, const int32_t *coo_col_ind,
-                  int32_t base, const float *x, float beta, float *y);
+                  int32_t base, const float *x, float beta, float *y, void *workspace,
+                  size_t workspace_bytes);
 int asamd_d_coomv(hipStream_t stream, int32_t m, int32_t n, int64_t nnz, double alpha,
                   const double *coo_val, const int32_t *coo_row_ind, const int32_t *coo_col_ind,
-                  int32_t base, const double *x, double beta, double *y);
+                  int32_t base, const double *x, double beta, double *y, void *workspace,
+                  size_t workspace_bytes);
 int asamd_c_coomv(hipStream_t stream, int32_t m, int32_t n, int64_t nnz, asamd_complex8 alpha,
                   const asamd_complex8 *coo_val, const int32_t *coo_row_ind, const int32_t *coo_col_ind,
-                  int32_t base, const asamd_complex8 *x, asamd_complex8 beta, asamd_complex8 *y);
+                  int32_t base, const asamd_complex8 *x, asamd_complex8 beta, asamd_complex8 *y, void *workspace,
+                  size_t workspace_bytes);
 int asamd_z_coomv(hipStream_t stream, int32_t m, int32_t n, int64_t nnz, asamd_complex16 alpha,
                   const asamd_complex16 *coo_val, const int32_t *coo_row_ind, const int32_t *coo_col_ind,
-                  int32_t base, const asamd_complex16 *x, asamd_complex16 beta, asamd_complex16 *y);
+                  int32_t base, const asamd_complex16 *x, asamd_complex16 beta, asamd_complex16 *y, void *workspace,
+                  size_t workspace_bytes);
 
 /* Number of lazily made analyses (multiplies with info == NULL on arrays that no analysis or mirror
  * covers) that the library remembers at the moment: at most 64, the least recently used one makes room,

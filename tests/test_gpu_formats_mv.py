@@ -92,6 +92,19 @@ def test_coomv_matches_oracle(gpu, shape, dtype):
             check(a, alpha, x, beta, y0, y, orc.coomv_plain(a, rows, alpha, x, beta, y0), "coomv %s" % shape)
 
 
+@pytest.mark.parametrize("shape", ["powerlaw", "long_and_empty", "single_row"])
+def test_coomv_grouped_by_row_is_the_same_every_run(gpu, shape):
+    """Rows that several waves share (every row of more than a thousand entries, and any row across a wave
+    boundary) are summed in wave order: entries grouped by row give the same bits from run to run."""
+    a = SHAPES[shape](np.float32)
+    x, y0 = wl.uniform(a.cols, np.float32, 3), wl.uniform(a.rows, np.float32, 4)
+    rows = orc.csr2coo(a)
+    announce("coomv determinism", shape)
+    runs = [run_coomv(gpu, a.rows, a.cols, a.values, rows, a.col_ind, 0, 1.5, x, 0.5, y0) for _ in range(4)]
+    for y in runs[1:]:
+        assert np.array_equal(runs[0], y)
+
+
 @pytest.mark.parametrize("dtype", DT, ids=IDS)
 def test_coomv_any_entry_order_and_out_of_range_entries(gpu, dtype):
     """Entries need not be grouped by row; entries whose row or column is out of range are skipped."""

@@ -122,10 +122,18 @@ def test_deterministic_across_runs(gpu):
     da = DeviceCsr(a)
     try:
         # the families that sum every row in a fixed order (no floating-point atomics)
-        for algo in ("merge", "hot", "binned", "vector"):
+        # (the tiled copy of this matrix has tiles too long for its second phase: the third phase runs)
+        for algo in ("merge", "hot", "binned", "vector", "tiled"):
             announce("spmv determinism", algo)
             runs = [run_plan_csrmv(da, algo, 1.0, x, 0.5, y0) for _ in range(3)]
             assert np.array_equal(runs[0], runs[1]) and np.array_equal(runs[0], runs[2]), algo
+        lib, plan = capi.load(), c_void_p()
+        assert lib.asamd_csr_plan_create(None, a.rows, a.cols, a.nnz, da.row_ptr.c_ptr(), da.col.c_ptr(), da.val.c_ptr(),
+                                         a.base, a.dtype.itemsize, 2, byref(plan)) == 0
+        st = lib.asamd_csr_plan_stats(plan).contents
+        built, long_blocks = st.tiled_built, st.tile_long_blocks
+        lib.asamd_csr_plan_destroy(plan)
+        assert built and long_blocks > 0, "the tiled copy was meant to have long tiles"
     finally:
         da.free()
 
