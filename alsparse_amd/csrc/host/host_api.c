@@ -6,9 +6,110 @@
  * result has landed in host memory (these entry points are synchronous in the
  * reference too).  There is no CPU compute path: without a usable device the
  * status is the mapped HIP error. */
+#include <omp.h>
+#include <pthread.h>
 #include <stdlib.h>
+#include <string.h>
 
 #include "internal.h"
+
+/* ---- host <-> device through pinned bounce buffers -------------------------------------------
+ * The vectors of these entry points live in the caller's pageable memory.  hipMemcpy stages such memory
+ * through a pinned buffer of its own with one thread; here the processor's copy into (out of) a ring of
+ * pinned chunks is spread over the OpenMP threads and overlaps the DMA of the chunk before (after) it.
+ * (Registering the caller's memory would avoid the copy, but costs more than the transfer it saves.)
+ * One ring per process, used under a lock; transfers below one chunk go through hipMemcpyAsync as before. */
+enum { kStageChunks = 4 };
+static const size_t kStageChunk = (size_t)8 << 20;
+static pthread_mutex_t g_stage_lock = PTHREAD_MUTEX_INITIALIZER;
+static void *g_stage_buf[kStageChunks];
+static hipEvent_t g_stage_ev[kStageChunks];
+static int g_stage_state; /* 0: not tried, 1: ready, -1: no pinned memory (plain copies) */
+
+static int asamd_stage_ready(void) {
+  if (g_stage_state) return g_stage_state > 0;
+  for (int i = 0; i < kStageChunks; ++i) {
+    if (hipHostMalloc(&g_stage_buf[i], kStageChunk, hipHostMallocDefault) != hipSuccess ||
+        hipEventCreateWithFlags(&g_stage_ev[i], hipEventDisableTiming) != hipSuccess) {
+      (void)hipGetLastError();
+      g_stage_state = -1;
+      return 0;
+    }
+  }
+  g_stage_state = 1;
+  return 1;
+}
+
+static void asamd_parallel_copy(void *dst, const void *src, size_t bytes) {
+  const size_t piece = (size_t)1 << 20;
+  const long pieces = (long)((bytes + piece - 1) / piece);
+  int threads = omp_get_max_threads();
+  if (threads > 16) threads = 16;
+#pragma omp parallel for num_threads(threads) schedule(static)
+  for (long i = 0; i < pieces; ++i) {
+    const size_t off = (size_t)i * piece;
+    memcpy((char *)dst + off, (const char *)src + off, bytes - off < piece ? bytes - off : piece);
+  }
+}
+
+/* Stream-ordered like hipMemcpyAsync; src may be reused when the call returns. */
+static hipError_t asamd_staged_h2d(hipStream_t s, void *dst, const void *src, size_t bytes) {
+  if (bytes < kStageChunk) return hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, s);
+  pthread_mutex_lock(&g_stage_lock);
+  hipError_t e = hipSuccess;
+  if (!asamd_stage_ready()) {
+    e = hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, s);
+  } else {
+    int slot = 0;
+    for (size_t off = 0; off < bytes && e == hipSuccess; off += kStageChunk, slot = (slot + 1) % kStageChunks) {
+      const size_t n = bytes - off < kStageChunk ? bytes - off : kStageChunk;
+      e = hipEventSynchronize(g_stage_ev[slot]); /* the chunk's earlier transfer has left it */
+      if (e != hipSuccess) break;
+      asamd_parallel_copy(g_stage_buf[slot], (const char *)src + off, n);
+      e = hipMemcpyAsync((char *)dst + off, g_stage_buf[slot], n, hipMemcpyHostToDevice, s);
+      if (e == hipSuccess) e = hipEventRecord(g_stage_ev[slot], s);
+    }
+  }
+  pthread_mutex_unlock(&g_stage_lock);
+  return e;
+}
+
+/* Returns after everything queued on s before it, and the copy, have finished. */
+static hipError_t asamd_staged_d2h_sync(hipStream_t s, void *dst, const void *src, size_t bytes) {
+  hipError_t e;
+  if (bytes < kStageChunk) {
+    e = hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, s);
+    return e == hipSuccess ? hipStreamSynchronize(s) : e;
+  }
+  pthread_mutex_lock(&g_stage_lock);
+  if (!asamd_stage_ready()) {
+    e = hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+  } else {
+    const size_t chunks = (bytes + kStageChunk - 1) / kStageChunk;
+    e = hipSuccess;
+    /* the ring is filled ahead; chunk c is copied out once its transfer has landed, then its slot takes
+     * chunk c + kStageChunks */
+    for (size_t c = 0; c < chunks + kStageChunks && e == hipSuccess; ++c) {
+      if (c >= kStageChunks) {
+        const size_t d = c - kStageChunks, off = d * kStageChunk;
+        const int slot = (int)(d % kStageChunks);
+        e = hipEventSynchronize(g_stage_ev[slot]);
+        if (e != hipSuccess) break;
+        asamd_parallel_copy((char *)dst + off, g_stage_buf[slot], bytes - off < kStageChunk ? bytes - off : kStageChunk);
+      }
+      if (c < chunks) {
+        const size_t off = c * kStageChunk;
+        const int slot = (int)(c % kStageChunks);
+        e = hipMemcpyAsync(g_stage_buf[slot], (const char *)src + off, bytes - off < kStageChunk ? bytes - off : kStageChunk,
+                           hipMemcpyDeviceToHost, s);
+        if (e == hipSuccess) e = hipEventRecord(g_stage_ev[slot], s);
+      }
+    }
+  }
+  pthread_mutex_unlock(&g_stage_lock);
+  return e;
+}
 
 /* Make sure A has a device mirror built by this library and return its record. */
 static alphasparse_status_t asamd_host_prepare(const alphasparse_matrix_t A, alphasparse_dcu_handle_t *h,
