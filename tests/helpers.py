@@ -99,10 +99,29 @@ def plan_stats(da, trusted=1):
     return out
 
 
+def check_beta_rows(a, alpha, x, beta, y0, y, ref, tol, what=""):
+    """beta != 0: the strict criterion plus nothing but the rounding of the last addition.  Both sides form
+    fl(fl(beta*y0) + fl(alpha*sum)): the first term rounds identically, the sum's error is the strict criterion's
+    business (tol * |alpha| sum|a x|), and the addition rounds to within half an ulp of the result on each side
+    (complex: each component, and the four-multiplication beta*y0 identically on both sides).  `a` is the matrix
+    whose rows are the outputs (the transpose for the transposed operations)."""
+    x64 = np.abs(np.asarray(x, dtype=np.complex128 if np.iscomplexobj(x) else np.float64))
+    den = abs(complex(alpha)) * orc._row_abs_sums(a, x64)
+    by = np.abs(complex(beta) * np.asarray(y0, dtype=np.complex128))
+    real = {"f": np.float32, "d": np.float64, "F": np.float32, "D": np.float64}[np.dtype(a.dtype).char]
+    u = float(np.finfo(real).eps) / 2
+    diff = np.abs(np.asarray(y, dtype=np.complex128) - np.asarray(ref, dtype=np.complex128))
+    allow = tol * den + 4 * u * (by + den)
+    bad = np.flatnonzero(diff > allow)
+    assert bad.size == 0, "%s: output %d off by %.3e, allowed %.3e (strict criterion + rounding of beta*y)" % (
+        what, bad[0], diff[bad[0]], allow[bad[0]])
+
+
 def check_spmv(a, alpha, x, beta, y0, y, what="", strict=False):
     """Compare y with the plain-kernel oracle.  Always: zero-denominator rows exact and
-    the error relative to |alpha| sum|a x| + |beta y0| within tolerance; strict=True
-    also demands the criterion normalised by the products alone."""
+    the error relative to |alpha| sum|a x| + |beta y0| within tolerance.  beta == 0 (or strict=True): the
+    north-star criterion, normalised by the products alone.  beta != 0: the same criterion with an allowance
+    of four units of round-off of |beta y0| + |alpha| sum|a x| for the rounding of the final addition."""
     ref = orc.csrmv_plain(a, alpha, x, beta, y0)
     err = orc.csrmv_err(a, alpha, x, beta, y0, y, ref)
     tol = TOL[a.dtype]
@@ -110,4 +129,6 @@ def check_spmv(a, alpha, x, beta, y0, y, what="", strict=False):
     assert err.full <= tol, "%s: per-row error %.3e at row %d exceeds %g" % (what, err.full, err.row, tol)
     if strict or beta == 0:
         assert err.strict <= tol, "%s: strict per-row error %.3e exceeds %g" % (what, err.strict, tol)
+    else:
+        check_beta_rows(a, alpha, x, beta, y0, y, ref, tol, what)
     return err

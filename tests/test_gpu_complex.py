@@ -12,7 +12,7 @@ import pytest
 
 from alsparse_amd import capi, hiprt, workloads as wl
 from oracle import oracle as orc
-from helpers import ALGOS, DeviceCsr, announce
+from helpers import ALGOS, DeviceCsr, announce, check_beta_rows
 from helpers_shapes import complex_vector, complexify, csr_from_lengths, real_dtype
 from test_gpu_formats_mv import dev, run_coomv, run_ellmv
 
@@ -54,6 +54,8 @@ def check(metric_matrix, alpha, x, beta, y0, y, ref, what):
     assert err.full <= tol, "%s: error %.3e at %d exceeds %g" % (what, err.full, err.row, tol)
     if beta == 0:
         assert err.strict <= tol, "%s: strict error %.3e exceeds %g" % (what, err.strict, tol)
+    else:
+        check_beta_rows(metric_matrix, alpha, x, beta, y0, y, ref, tol, what)
 
 
 def run_csrmv(h, da, op, alpha, x, beta, y0, info=None):

@@ -9,7 +9,7 @@ import pytest
 
 from alsparse_amd import capi, hiprt, workloads as wl
 from oracle import oracle as orc
-from helpers import DeviceCsr, TOL, announce, run_csrmv
+from helpers import DeviceCsr, TOL, announce, check_beta_rows, run_csrmv
 from helpers_shapes import csr_from_lengths
 
 pytestmark = pytest.mark.gpu
@@ -63,6 +63,8 @@ def check(a, alpha, x, beta, y0, y, ref, what):
     assert err.full <= tol, "%s: per-row error %.3e at row %d exceeds %g" % (what, err.full, err.row, tol)
     if beta == 0:
         assert err.strict <= tol, "%s: strict per-row error %.3e exceeds %g" % (what, err.strict, tol)
+    else:
+        check_beta_rows(a, alpha, x, beta, y0, y, ref, tol, what)
 
 
 SHAPES = {

@@ -10,7 +10,7 @@ import pytest
 
 from alsparse_amd import capi, hiprt, workloads as wl
 from oracle import oracle as orc
-from helpers import DeviceCsr, TOL, announce
+from helpers import DeviceCsr, TOL, announce, check_beta_rows
 from helpers_shapes import csr_from_lengths
 
 pytestmark = pytest.mark.gpu
@@ -40,6 +40,8 @@ def check_trans(a, alpha, x, beta, y0, y, what):
     assert err.full <= tol, "%s: error %.3e at column %d exceeds %g" % (what, err.full, err.row, tol)
     if beta == 0:
         assert err.strict <= tol, "%s: strict error %.3e exceeds %g" % (what, err.strict, tol)
+    else:
+        check_beta_rows(at, alpha, x, beta, y0, y, ref, tol, what)
 
 
 def run_csrmv_trans(h, da, alpha, x, beta, y0, info=None):
