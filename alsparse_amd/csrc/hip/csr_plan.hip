@@ -1411,6 +1411,14 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
   switch (algo) {
     case ASAMD_SPMV_ELL: {
       // the ELL copy holds zero-based columns and its own values
+      if constexpr (sizeof(T) <= 8) {
+        if (st.m % 2 == 0) {  // the copy is the library's own (256-byte aligned): row pairs are aligned when m is even
+          const unsigned grid2 = (unsigned)(((int64_t)st.m / 2 + kEllThreads - 1) / kEllThreads);
+          ellmv_multi_kernel<T, 2><<<grid2, kEllThreads, 0, s>>>(st.m, st.n, alpha, (const T*)p->d_eval, p->d_ecol,
+                                                                 st.ell_width, 0, x, beta, y);
+          break;
+        }
+      }
       const unsigned grid = (unsigned)(((int64_t)st.m + kEllThreads - 1) / kEllThreads);
       ellmv_kernel<T><<<grid, kEllThreads, 0, s>>>(st.m, st.n, alpha, (const T*)p->d_eval, p->d_ecol, st.ell_width, 0,
                                                    x, beta, y);

@@ -157,6 +157,14 @@ int ellmv_impl(hipStream_t stream, int32_t m, int32_t n, T alpha, const T* ell_v
   if (m < 0 || n < 0 || width < 0) return (int)hipErrorInvalidValue;
   if (((uintptr_t)ell_val | (uintptr_t)x | (uintptr_t)y) % alignof(T)) return (int)hipErrorInvalidValue;
   if (m == 0) return (int)hipSuccess;
+  if constexpr (sizeof(T) <= 8) {
+    // two rows per lane where the caller's arrays allow aligned pairs
+    if (m % 2 == 0 && (uintptr_t)ell_val % (2 * sizeof(T)) == 0 && (uintptr_t)ell_col % 8 == 0) {
+      const unsigned grid2 = (unsigned)(((int64_t)m / 2 + kEllThreads - 1) / kEllThreads);
+      ellmv_multi_kernel<T, 2><<<grid2, kEllThreads, 0, stream>>>(m, n, alpha, ell_val, ell_col, width, base, x, beta, y);
+      return (int)hipGetLastError();
+    }
+  }
   const unsigned grid = (unsigned)(((int64_t)m + kEllThreads - 1) / kEllThreads);
   ellmv_kernel<T><<<grid, kEllThreads, 0, stream>>>(m, n, alpha, ell_val, ell_col, width, base, x, beta, y);
   return (int)hipGetLastError();
