@@ -669,7 +669,10 @@ static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* 
       e = hipMemcpy(p->d_chunks, h_chunks.data(), h_chunks.size() * sizeof(TiledChunk), hipMemcpyHostToDevice);
   }
   if (e == hipSuccess)  // both phases use more than the default 64 KiB of dynamic LDS
-    e = hipFuncSetAttribute((const void*)tiled_products_kernel<T>,
+    e = hipFuncSetAttribute((const void*)tiled_products_kernel<T, false>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kSliceBytes);
+  if (e == hipSuccess)
+    e = hipFuncSetAttribute((const void*)tiled_products_kernel<T, true>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, kSliceBytes);
   if (e == hipSuccess)
     e = hipFuncSetAttribute((const void*)tiled_reduce_kernel<T, 1>,
@@ -1426,9 +1429,15 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
     }
     case ASAMD_SPMV_TILED: {
       // the tiled copy holds zero-based local indices and its own values
-      if (p->n_chunks > 0)
-        tiled_products_kernel<T><<<p->n_chunks, kProdThreads, kSliceBytes, s>>>(
-            p->d_chunks, (const T*)p->d_tval, p->d_tcol, x, (T*)p->d_tprod);
+      if (p->n_chunks > 0) {
+        // products that the memory-side cache cannot hold anyway are stored past it
+        if ((int64_t)st.nnz * (int64_t)sizeof(T) > ((int64_t)512 << 20))
+          tiled_products_kernel<T, true><<<p->n_chunks, kProdThreads, kSliceBytes, s>>>(
+              p->d_chunks, (const T*)p->d_tval, p->d_tcol, x, (T*)p->d_tprod);
+        else
+          tiled_products_kernel<T, false><<<p->n_chunks, kProdThreads, kSliceBytes, s>>>(
+              p->d_chunks, (const T*)p->d_tval, p->d_tcol, x, (T*)p->d_tprod);
+      }
       const unsigned red_grid = (unsigned)((st.tile_row_blocks + TileDims<T>::red_waves - 1) / TileDims<T>::red_waves);
       if (p->tiled_halves == 1)
         tiled_reduce_kernel<T, 1><<<red_grid, TileDims<T>::red_threads, TileDims<T>::red_lds_bytes, s>>>(
