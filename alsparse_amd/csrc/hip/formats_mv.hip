@@ -79,7 +79,7 @@ __global__ __launch_bounds__(kCooThreads) void coomv_kernel(int64_t nnz, int m, 
       const int c = __builtin_nontemporal_load(&coo_col[k]) - base;
       if ((unsigned)rr < (unsigned)m && (unsigned)c < (unsigned)n) {
         r = rr;
-        v = nt_load(&coo_val[k]) * x[c];
+        v = coo_val[k] * x[c];  // indices non-temporal, values not: 107 -> 100 us on a 21 M-entry Laplacian (all three: 107)
       }
     }
     const int r0 = lane_bcast(r, 0);
