@@ -208,7 +208,9 @@ __global__ __launch_bounds__(kSpmmBlock) void spmm_rowmajor_quad_kernel(
   const int g = lane / 16;
   const int c0 = (blockIdx.y * 16 + lane % 16) * E;
   const bool owns = c0 < n;
-  const T* bcol = B + (owns ? c0 : 0);
+  // lanes past the last dense column load what the group's first lane loads (the same cache line: no request
+  // of their own) and add nothing
+  const T* bcol = B + (owns ? c0 : blockIdx.y * 16 * E);
 
   const int64_t start = (int64_t)row_ptr[row] - base;
   const int64_t end = (int64_t)row_ptr[row + 1] - base;
@@ -630,7 +632,13 @@ static int csrmm_impl(hipStream_t s, int m, int n, int k, int nnz, T alpha, cons
       // rows of B and C that 128-bit loads can address: four rows of B per wave instruction
       constexpr int E = 16 / (int)sizeof(T);
       static const bool quad_off = getenv("ALSPARSE_AMD_SPMM_QUAD") && atoi(getenv("ALSPARSE_AMD_SPMM_QUAD")) == 0;
-      if (!quad_off && n % E == 0 && ldb % E == 0 && ldc % E == 0 && (uintptr_t)B % 16 == 0 && (uintptr_t)C % 16 == 0) {
+      // Measured on 2^20 rows x 32 entries, n = 64, against one wave-wide load per row of B: B of 4 / 16 / 32 MiB
+      // 0.64 / 0.95 / 1.10 ms against 0.97 / 1.05 / 1.11; 64-256 MiB 1.18-1.23 against 1.17-1.22 (the L2-miss
+      // path is the limit either way); 512 MiB 1.22 against 1.38; n = 256 (1 GiB) 4.95 against 5.46.
+      const size_t b_bytes = (size_t)(k > 0 ? k : 0) * (size_t)n * sizeof(T);
+      const bool quad_pays = k <= 0 || b_bytes <= ((size_t)48 << 20) || b_bytes > ((size_t)384 << 20);
+      if (!quad_off && quad_pays && n % E == 0 && ldb % E == 0 && ldc % E == 0 && (uintptr_t)B % 16 == 0 &&
+          (uintptr_t)C % 16 == 0) {
         const dim3 grid(gx, (unsigned)((n + 16 * E - 1) / (16 * E)));
         spmm_rowmajor_quad_kernel<T><<<grid, kSpmmBlock, 0, s>>>(m, n, alpha, val, rp, ci, base, B, ldb, beta, C, ldc);
         return hipGetLastError();
