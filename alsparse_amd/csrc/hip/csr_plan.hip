@@ -69,6 +69,13 @@ __global__ __launch_bounds__(256) void row_stats_kernel(int m, const int* __rest
   }
 }
 
+// dst[i] = src[i * stride]
+__global__ __launch_bounds__(256) void strided_gather_kernel(int count, const int* __restrict__ src, int64_t stride,
+                                                             int* __restrict__ dst) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < count) dst[i] = src[(int64_t)i * stride];
+}
+
 __global__ void stats_init_kernel(int* out) {
   const int t = threadIdx.x;
   if (t < kStatWords) out[t] = t == 0 ? 0x7fffffff : 0;
@@ -576,9 +583,12 @@ static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan* p, const int* 
         rb, cb, p->tiled_halves * kWave, d_tile_ptr, p->d_ranges, d_long_raw, d_long_count);
     h_colptr.resize((size_t)cb + 1);
   }
-  if (e == hipSuccess)  // column block c starts at tile_ptr[c * rb]
-    e = hipMemcpy2DAsync(h_colptr.data(), sizeof(int), d_tile_ptr, (size_t)rb * sizeof(int), sizeof(int),
-                         (size_t)cb + 1, hipMemcpyDeviceToHost, stream);
+  if (e == hipSuccess) {
+    // column block c starts at tile_ptr[c * rb]: gathered on the device (d_cnt is free again and holds more
+    // than cb + 1 ints), then one small copy -- a strided 2-D copy of these few hundred words took 22 ms
+    strided_gather_kernel<<<(unsigned)((cb + 1 + 255) / 256), 256, 0, stream>>>(cb + 1, d_tile_ptr, (int64_t)rb, d_cnt);
+    e = hipMemcpyAsync(h_colptr.data(), d_cnt, ((size_t)cb + 1) * sizeof(int), hipMemcpyDeviceToHost, stream);
+  }
   if (e == hipSuccess) e = hipStreamSynchronize(stream);
 
   // ---- 3. tiles too long for phase 2: cut into phase-3 chunks ----------------------
