@@ -417,7 +417,7 @@ __global__ __launch_bounds__(kProdThreads) void tiled_products_kernel(
 
 // ---- phase 2 -------------------------------------------------------------------
 // acc[r] += v for the valid lanes of one wave instruction.  acc is private to
-// the wave (or updated atomically).  Entries of one row are adjacent (a tile is
+// the wave.  Entries of one row are adjacent (a tile is
 // stored in CSR order), so the lanes of a run of equal rows must not all do
 // their read-modify-write at once.  From the ballot of "same row as the lane
 // below" every lane knows its position in its run:
@@ -427,17 +427,11 @@ __global__ __launch_bounds__(kProdThreads) void tiled_products_kernel(
 //     add, so the lanes of one pass always hold distinct rows;
 //   * longer runs (long rows): a segmented suffix sum inside the wave leaves the
 //     run's total in its first lane, which adds alone.
-template <bool Atomic, typename T>
-__device__ __forceinline__ void rmw(T* p, T v) {
-  if constexpr (Atomic) atomic_add(p, v);
-  else *p += v;
-}
-
 constexpr int kMaxPasses = 4;
 
 // AllValid: every lane holds an entry or a private dummy row of acc (distinct per lane, so it never
 // continues a run), and `valid` is not looked at: no masks around the read-modify-writes.
-template <bool Atomic = false, bool AllValid = false, typename T>
+template <bool AllValid = false, typename T>
 __device__ __forceinline__ void add_rows(T* acc, int r, T v, bool valid_arg) {
   const bool valid = AllValid ? true : valid_arg;
   const int lane = threadIdx.x % kWave;
@@ -448,7 +442,7 @@ __device__ __forceinline__ void add_rows(T* acc, int r, T v, bool valid_arg) {
   const bool same_as_prev = r_up == r;
   const uint64_t dup = __builtin_amdgcn_ballot_w64(same_as_prev);
   if (dup == 0) {
-    if (valid) rmw<Atomic>(&acc[r], v);
+    if (valid) acc[r] += v;
     return;
   }
   if ((dup & (dup << 1)) == 0) {
@@ -456,7 +450,7 @@ __device__ __forceinline__ void add_rows(T* acc, int r, T v, bool valid_arg) {
     // its neighbour's value, three DPP wave shifts in all
     const T v_next = dpp_mov<0x130>(v);  // wave_shl:1: value of lane + 1 (0 past the end)
     if ((dup >> 1 >> lane) & 1) v += v_next;
-    if (valid && !same_as_prev) rmw<Atomic>(&acc[r], v);
+    if (valid && !same_as_prev) acc[r] += v;
     return;
   }
   // first lane of my run: highest lane <= me whose dup bit is clear
@@ -467,14 +461,12 @@ __device__ __forceinline__ void add_rows(T* acc, int r, T v, bool valid_arg) {
 #pragma unroll
   for (int p = 1; p < kMaxPasses; ++p) longrun &= dup >> p;
   if (longrun == 0) {
-    if (!Atomic) {
 #pragma unroll
-      for (int p = 0; p < kMaxPasses; ++p) {
-        if (p > 0 && __builtin_amdgcn_ballot_w64(valid && pos == p) == 0) break;
-        if (valid && pos == p) acc[r] += v;
-      }
-      return;
+    for (int p = 0; p < kMaxPasses; ++p) {
+      if (p > 0 && __builtin_amdgcn_ballot_w64(valid && pos == p) == 0) break;
+      if (valid && pos == p) acc[r] += v;
     }
+    return;
   }
   // suffix sums inside every run; lane + d belongs to my run iff the d dup bits above me are all set
   const uint64_t above = dup >> 1 >> lane;
@@ -484,7 +476,7 @@ __device__ __forceinline__ void add_rows(T* acc, int r, T v, bool valid_arg) {
     const uint64_t need = ((uint64_t)1 << d) - 1;
     if ((above & need) == need) v += vd;
   }
-  if (valid && !same_as_prev) rmw<Atomic>(&acc[r], v);
+  if (valid && !same_as_prev) acc[r] += v;
 }
 
 // H = entries per lane and tile: 2 takes tiles of up to kLongTile entries with red_slots tiles in flight,
@@ -555,10 +547,10 @@ __global__ __launch_bounds__(TileDims<T>::red_threads) void tiled_reduce_kernel(
   auto consume = [&](int s) {
     const int len = slen[s];
     // a lane without an entry holds value zero already; its row becomes the lane's dummy row
-    add_rows<false, true>(acc, lane < len ? sr[s][0] : r_none, sv[s][0], true);
+    add_rows<true>(acc, lane < len ? sr[s][0] : r_none, sv[s][0], true);
     if constexpr (H == 2) {
       if (len > kWave)  // wave-uniform
-        add_rows<false, true>(acc, lane + kWave < len ? sr[s][1] : r_none, sv[s][1], true);
+        add_rows<true>(acc, lane + kWave < len ? sr[s][1] : r_none, sv[s][1], true);
     }
   };
 #pragma unroll
@@ -628,12 +620,12 @@ __global__ __launch_bounds__(kLongThreads) void tiled_long_kernel(
           r[u] = t_row[k0 + u * kWave + lane];
         }
 #pragma unroll
-        for (int u = 0; u < kU; ++u) add_rows<false, true>(acc, r[u], v[u], true);
+        for (int u = 0; u < kU; ++u) add_rows<true>(acc, r[u], v[u], true);
       } else {
         for (int k1 = k0; k1 < end; k1 += kWave) {  // wave-uniform trip count
           const int k = k1 + lane;
           const bool ok = k < end;
-          add_rows<false, true>(acc, ok ? (int)t_row[k] : r_none, ok ? prod[k] : T(0), true);
+          add_rows<true>(acc, ok ? (int)t_row[k] : r_none, ok ? prod[k] : T(0), true);
         }
       }
     }
