@@ -31,7 +31,7 @@ HBM_PEAK_GBS = 8000.0
 # factors from a 1 GiB copy kernel) -- a table of earlier measurements, not an in-run reading; each entry names the
 # summary under profiles/ it comes from.  Keyed by (configuration, kernel family); anything else reports null.
 MEASURED_TRAFFIC_BYTES = {
-    (3, "tiled two-phase"): (5.18e9, "profiles/spmv_tiled_C3.txt"),
+    (3, "tiled two-phase"): (5.17e9, "profiles/spmv_tiled_C3.txt"),
     (3, "rowconst"): (34.6e9, "profiles/spmv_tiled_C3.txt"),
     (4, "merge-path"): (3.32e9, "profiles/spmv_merge_C4.txt"),
     (2, "ell copy"): (322.5e6, "profiles/spmv_ell_copy_C2.txt"),
