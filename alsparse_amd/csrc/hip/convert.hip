@@ -30,6 +30,10 @@ using namespace asamd;
 // 0.3 ms).  The row-index stream is written as 128-bit pieces, 1 KiB of
 // consecutive bytes per wave instruction.
 // ---------------------------------------------------------------------------
+// Output that the L2s (8 x 4 MiB) cannot hold is written with non-temporal stores: measured on 84 MB to
+// 2 GiB of output, csr2coo 30 -> 25 us and 0.266 -> 0.198 ms, csr2ell 129 -> 87 us and 0.90 -> 0.86 ms.
+static bool stores_bypass_caches(size_t out_bytes) { return out_bytes > ((size_t)32 << 20); }
+
 constexpr int kCooThreads = 256;
 constexpr int kCooRound = kCooThreads * 4;  // entries per scan round
 constexpr int kCooRounds = 8;
@@ -65,6 +69,7 @@ __global__ __launch_bounds__(256) void csr2coo_chunk_rows_kernel(const int* __re
 }
 
 // chunk_row: the table above, or null (then every workgroup searches for its own rows)
+template <bool NTS>
 __global__ __launch_bounds__(kCooThreads) void csr2coo_kernel(const int* __restrict__ row_ptr,
                                                               int nnz, int m,
                                                               int* __restrict__ coo_row, int base,
@@ -147,7 +152,12 @@ __global__ __launch_bounds__(kCooThreads) void csr2coo_kernel(const int* __restr
     const int64_t k = k0 + (int64_t)j * kCooRound + 4 * threadIdx.x;
     const int o[4] = {rb + max(lead, v[j][0]), rb + max(lead, v[j][1]), rb + max(lead, v[j][2]), rb + max(lead, v[j][3])};
     if (wide && k + 4 <= k1) {
-      *reinterpret_cast<Int4*>(coo_row + k) = Int4{o[0], o[1], o[2], o[3]};
+      if constexpr (NTS) {
+        typedef int V4 __attribute__((ext_vector_type(4)));
+        __builtin_nontemporal_store(V4{o[0], o[1], o[2], o[3]}, reinterpret_cast<V4*>(coo_row + k));
+      } else {
+        *reinterpret_cast<Int4*>(coo_row + k) = Int4{o[0], o[1], o[2], o[3]};
+      }
     } else {
       for (int q = 0; q < 4 && k + q < k1; ++q) coo_row[k + q] = o[q];
     }
@@ -169,7 +179,10 @@ extern "C" int asamd_csr2coo_ws(hipStream_t stream, const int32_t* row_ptr, int3
     csr2coo_chunk_rows_kernel<<<(unsigned)((chunks + 1 + 255) / 256), 256, 0, stream>>>(row_ptr, nnz, m, base, chunks,
                                                                                         chunk_row);
   }
-  csr2coo_kernel<<<(unsigned)chunks, kCooThreads, 0, stream>>>(row_ptr, nnz, m, coo_row, base, chunk_row);
+  if (stores_bypass_caches((size_t)nnz * sizeof(int)))
+    csr2coo_kernel<true><<<(unsigned)chunks, kCooThreads, 0, stream>>>(row_ptr, nnz, m, coo_row, base, chunk_row);
+  else
+    csr2coo_kernel<false><<<(unsigned)chunks, kCooThreads, 0, stream>>>(row_ptr, nnz, m, coo_row, base, chunk_row);
   return hipGetLastError();
 }
 
@@ -236,7 +249,7 @@ extern "C" int asamd_csr2ell_width(hipStream_t stream, int32_t m, const int32_t*
 constexpr int kEllRows = 256;
 constexpr int kEllWindow = 4096;  // staged entries per workgroup pass (half of it for 16-byte values)
 
-template <typename T>
+template <typename T, bool NTS>
 __global__ __launch_bounds__(kEllRows) void csr2ell_kernel(
     int m, const T* __restrict__ val, const int* __restrict__ row_ptr,
     const int* __restrict__ col_ind, int csr_base, int ell_base, int width,
@@ -301,8 +314,13 @@ __global__ __launch_bounds__(kEllRows) void csr2ell_kernel(
       }
     }
     const int64_t o = (int64_t)s * m + row;
-    ell_val[o] = v;
-    ell_col[o] = c;
+    if constexpr (NTS) {
+      nt_store(v, ell_val + o);
+      nt_store(c, ell_col + o);
+    } else {
+      ell_val[o] = v;
+      ell_col[o] = c;
+    }
   }
 }
 
@@ -313,8 +331,10 @@ static int csr2ell_impl(hipStream_t stream, int m, const T* val, const int* rp, 
   if (((uintptr_t)val | (uintptr_t)ell_val) % alignof(T)) return hipErrorInvalidValue;
   if (width == 0) return hipSuccess;
   const unsigned grid = (unsigned)(((int64_t)m + kEllRows - 1) / kEllRows);
-  csr2ell_kernel<T><<<grid, kEllRows, 0, stream>>>(m, val, rp, ci, csr_base, ell_base, width, ell_val,
-                                                   ell_col);
+  if (stores_bypass_caches((size_t)m * (size_t)width * (sizeof(T) + sizeof(int))))
+    csr2ell_kernel<T, true><<<grid, kEllRows, 0, stream>>>(m, val, rp, ci, csr_base, ell_base, width, ell_val, ell_col);
+  else
+    csr2ell_kernel<T, false><<<grid, kEllRows, 0, stream>>>(m, val, rp, ci, csr_base, ell_base, width, ell_val, ell_col);
   return hipGetLastError();
 }
 

@@ -152,6 +152,16 @@ __device__ __forceinline__ void store_axpby(T* __restrict__ y, int64_t row, T al
   }
 }
 
+// The same with non-temporal accesses to y: for kernels whose other streams should keep the caches
+template <typename T>
+__device__ __forceinline__ void store_axpby_nt(T* __restrict__ y, int64_t row, T alpha, T sum, T beta) {
+  if (beta == T(0)) {
+    nt_store(alpha * sum, y + row);
+  } else {
+    nt_store(axpby_rn(alpha, sum, beta, nt_load(y + row)), y + row);
+  }
+}
+
 // ---- DPP moves ------------------------------------------------------------
 // dpp_ctrl encodings (GCN3+/CDNA ISA): quad_perm = 0x00..0xFF, row_shr:n =
 // 0x110+n, row_ror:n = 0x120+n, row_mirror = 0x140, row_half_mirror = 0x141.

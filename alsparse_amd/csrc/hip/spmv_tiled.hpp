@@ -574,7 +574,7 @@ __global__ __launch_bounds__(TileDims<T>::red_threads) void tiled_reduce_kernel(
   }
   const int64_t row0 = row_block_start[rb];
   const int nrows = row_block_start[rb + 1] - (int)row0;  // <= kTileRows
-  for (int i = lane; i < nrows; i += kWave) store_axpby(y, row0 + i, alpha, acc[i], beta);
+  for (int i = lane; i < nrows; i += kWave) store_axpby_nt(y, row0 + i, alpha, acc[i], beta);
 }
 
 // ---- phase 3 -------------------------------------------------------------------
