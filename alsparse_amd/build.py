@@ -36,10 +36,17 @@ def build_workloads():
 
 def build_oracle():
     """Compile the CPU oracle (test infrastructure) and, when the reference tree
-    is present, the reference's own CPU kernels into oracle/_ref/."""
+    is present, the reference's own CPU kernels and its own test programs of this path
+    (unchanged sources, linked against this library) into oracle/_ref/."""
     _run(["make", "-C", os.path.join(ROOT, "oracle")])
+    if os.path.isdir("/root/reference/test") and os.path.exists(LIB_PATH):
+        _run(["make", "-C", os.path.join(ROOT, "oracle"), "ref_drivers"])
 
 
-def build_c_api_program():
-    """Compile the C lifecycle program of the test suite against the freshly built library."""
+def build_c_api_program(sanitized=True, jobs=8):
+    """Compile the C lifecycle program of the test suite against the freshly built library, and (sanitized)
+    the same program with a copy of the library whose host code carries ASan + UBSan: the test that runs it
+    refuses a copy made from other sources than the present ones, so it is made whenever the library is."""
     _run(["make", "-C", os.path.join(ROOT, "tests", "c_api")])
+    if sanitized:
+        _run(["make", "-C", os.path.join(ROOT, "tests", "c_api"), "-j%d" % jobs, "asan"])
