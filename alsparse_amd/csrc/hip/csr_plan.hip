@@ -200,13 +200,26 @@ static bool rowconst_ok(const asamd_csr_plan* p) {
          (L == 4 || L == 8 || L == 16 || L == 32 || L == 64 || L == 128 || L == 256);
 }
 
-// The LDS-staged row-block kernel sizes its staging area for rows of at most
-// kStreamMaxLen entries; the bound comes from the analysis, so the structure
-// must be promised fixed.
-static bool stream_ok(const asamd_csr_plan* p) {
+// The LDS-staged row-block kernel sizes its staging area for rows of at most CAP * G entries (G lanes sum a
+// row); the bound comes from the analysis, so the structure must be promised fixed.  Returns G, or 0 when the
+// kernel cannot take the matrix.  With `regular_only`, also 0 for G > 1 when the rows are so much shorter than
+// the longest that a workgroup's 256 / G rows hold fewer than four entries per thread.
+// 16 KiB of products per workgroup: 16 entries per thread for 4-byte values, 8 for 8-byte, 4 for 16-byte ones
+// (measured on a 27-point stencil, fp64: 32 KiB per workgroup 317 us, 16 KiB 295 us)
+static int stream_cap(const asamd_csr_plan* p) { return 64 / p->val_size; }
+static int stream_group(const asamd_csr_plan* p, bool regular_only) {
   const asamd_csr_stats& st = p->st;
-  return st.trusted && st.max_len <= kStreamMaxLen && st.max_len >= 1;
+  if (!st.trusted || st.max_len < 1) return 0;
+  const int cap = stream_cap(p);
+  if (st.max_len <= cap) return 1;
+  int g = 2;
+  while (g * cap < st.max_len && g <= kStreamMaxGroup) g *= 2;
+  if (g > kStreamMaxGroup) return 0;
+  // regular: the mean row is at least a quarter of the longest row the kernel is sized for
+  if (regular_only && (double)st.nnz / (double)st.m < 0.25 * g * cap) return 0;
+  return g;
 }
+static bool stream_ok(const asamd_csr_plan* p) { return stream_group(p, false) > 0; }
 
 static void choose_algo(asamd_csr_plan* p) {
   asamd_csr_stats& st = p->st;
@@ -217,10 +230,11 @@ static void choose_algo(asamd_csr_plan* p) {
     // row_ptr points into the middle of a larger array: only the kernels that index with the absolute
     // offsets (as the reference's csr_gemv_vector does) see the right entries; merge-path and csr2coo,
     // the source of every re-ordered copy, count entries from position 0
-    p->auto_algo = stream_ok(p) ? ASAMD_SPMV_STREAM : ASAMD_SPMV_VECTOR;
+    p->auto_algo = stream_group(p, true) > 0 ? ASAMD_SPMV_STREAM : ASAMD_SPMV_VECTOR;
   } else if (rowconst_ok(p)) {
     p->auto_algo = ASAMD_SPMV_ROWCONST;
-  } else if (stream_ok(p)) {
+  } else if (stream_group(p, true) > 0) {
+    // short rows, or rows of some tens of entries of similar lengths
     p->auto_algo = ASAMD_SPMV_STREAM;
   } else if ((int64_t)st.max_len <= (int64_t)w * 16 && mean >= 6.0) {
     // regular rows: a lane group per row wastes little and needs no LDS
@@ -913,7 +927,7 @@ static hipError_t tune_copies(hipStream_t stream, asamd_csr_plan* p, const int* 
   if (e == hipSuccess) e = hipEventCreate(&e1);
   constexpr int kCand = 5;
   float best[kCand] = {0.f, 0.f, 0.f, 0.f, 0.f};
-  const int algos[kCand] = {p->auto_algo, ASAMD_SPMV_TILED, ASAMD_SPMV_ELL, ASAMD_SPMV_MERGE_HOT, ASAMD_SPMV_BINNED};
+  int algos[kCand] = {p->auto_algo, ASAMD_SPMV_TILED, ASAMD_SPMV_ELL, ASAMD_SPMV_MERGE_HOT, ASAMD_SPMV_BINNED};
   auto time_algo = [&](int a) {
     st.algo = algos[a];
     // first run warms up; multiplies of a millisecond and more are timed once, shorter ones twice; a
@@ -941,6 +955,21 @@ static hipError_t tune_copies(hipStream_t stream, asamd_csr_plan* p, const int* 
   // on an 8 M-row R-MAT matrix whose longest row has 120 000 entries; 0.65 ms on its transpose).
   if ((double)st.max_len > 32.0 * ((double)st.nnz / (double)st.m) + 256.0) tiled_floor_ms *= 2.5f;
   if (e == hipSuccess) time_algo(0);
+  // A lane group per row, or a staged block of rows with several lanes per row, was chosen from the mean and
+  // the longest row alone; merge-path takes any distribution and needs no copy either: the faster one stays.
+  if (e == hipSuccess && st.first_offset == 0 &&
+      (p->auto_algo == ASAMD_SPMV_VECTOR || (p->auto_algo == ASAMD_SPMV_STREAM && stream_group(p, false) > 1))) {
+    const float first = best[0];
+    best[0] = 0.f;
+    algos[0] = ASAMD_SPMV_MERGE;
+    time_algo(0);
+    if (e == hipSuccess && best[0] < 0.97f * first) {
+      p->auto_algo = p->struct_algo = ASAMD_SPMV_MERGE;
+    } else {
+      algos[0] = p->auto_algo;
+      best[0] = first;
+    }
+  }
   // An ELL copy gathers x row by row like the kernel just timed; when that one is several times slower
   // than the tiled floor the gathers are the problem and the ELL copy (as large as the matrix) is not
   // worth building: the tiled copy is tried first, the ELL copy only if that does not win.
@@ -1485,13 +1514,40 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
       break;
     }
     case ASAMD_SPMV_STREAM: {
-      const unsigned grid = (unsigned)(((int64_t)st.m + kStreamRows - 1) / kStreamRows);
-      if (st.max_len <= 4)
-        spmv_stream_kernel<T, 4><<<grid, kStreamRows, 0, s>>>(st.m, alpha, val, rp, ci, x, beta, y, st.base);
-      else if (st.max_len <= 8)
-        spmv_stream_kernel<T, 8><<<grid, kStreamRows, 0, s>>>(st.m, alpha, val, rp, ci, x, beta, y, st.base);
-      else
-        spmv_stream_kernel<T, 16><<<grid, kStreamRows, 0, s>>>(st.m, alpha, val, rp, ci, x, beta, y, st.base);
+      const int g = stream_group(p, false);
+      const unsigned grid = (unsigned)(((int64_t)st.m * g + kStreamRows - 1) / kStreamRows);
+      constexpr int kCap = 64 / (int)sizeof(T);  // stream_cap(p)
+      // 128-bit loads need 16-byte aligned streams
+      const bool wide = (((uintptr_t)val | (uintptr_t)ci) & 15u) == 0;
+      const int64_t limit = (int64_t)st.first_offset + st.nnz;
+#define ASAMD_STREAM_LAUNCH(CAP, G)                                                                                      \
+  do {                                                                                                                   \
+    if (wide)                                                                                                            \
+      spmv_stream_wide_kernel<T, CAP, G><<<grid, kStreamRows, 0, s>>>(st.m, alpha, val, rp, ci, x, beta, y, st.base,    \
+                                                                      limit);                                           \
+    else                                                                                                                 \
+      spmv_stream_kernel<T, CAP, G><<<grid, kStreamRows, 0, s>>>(st.m, alpha, val, rp, ci, x, beta, y, st.base);        \
+  } while (0)
+      if (g == 1) {
+        if (st.max_len <= 4) {
+          ASAMD_STREAM_LAUNCH(4, 1);
+        } else if constexpr (kCap >= 8) {
+          if (st.max_len <= 8) {
+            ASAMD_STREAM_LAUNCH(8, 1);
+          } else if constexpr (kCap >= 16) {
+            ASAMD_STREAM_LAUNCH(16, 1);
+          }
+        }
+      } else if (g == 2) {
+        ASAMD_STREAM_LAUNCH(kCap, 2);
+      } else if (g == 4) {
+        ASAMD_STREAM_LAUNCH(kCap, 4);
+      } else if (g == 8) {
+        ASAMD_STREAM_LAUNCH(kCap, 8);
+      } else {
+        ASAMD_STREAM_LAUNCH(kCap, 16);
+      }
+#undef ASAMD_STREAM_LAUNCH
       break;
     }
     case ASAMD_SPMV_SCALAR: {

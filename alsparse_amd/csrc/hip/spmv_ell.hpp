@@ -49,29 +49,6 @@ __global__ __launch_bounds__(kEllThreads) void ellmv_kernel(int m, int n, T alph
   store_axpby(y, row, alpha, sum, beta);
 }
 
-// A non-temporal load of an aligned trivially copyable object of 4, 8, 16 or 32 bytes (the streams are touched
-// once: they should not push x out of the caches).
-template <typename P>
-__device__ __forceinline__ P nt_load_object(const P* p) {
-  typedef int V2 __attribute__((ext_vector_type(2)));
-  typedef int V4 __attribute__((ext_vector_type(4)));
-  static_assert(sizeof(P) == 4 || sizeof(P) == 8 || sizeof(P) == 16 || sizeof(P) == 32, "object size");
-  if constexpr (sizeof(P) == 4) {
-    return __builtin_bit_cast(P, __builtin_nontemporal_load(reinterpret_cast<const int*>(p)));
-  } else if constexpr (sizeof(P) == 8) {
-    return __builtin_bit_cast(P, __builtin_nontemporal_load(reinterpret_cast<const V2*>(p)));
-  } else if constexpr (sizeof(P) == 16) {
-    return __builtin_bit_cast(P, __builtin_nontemporal_load(reinterpret_cast<const V4*>(p)));
-  } else {
-    struct Two {
-      V4 a, b;
-    } t;
-    t.a = __builtin_nontemporal_load(reinterpret_cast<const V4*>(p));
-    t.b = __builtin_nontemporal_load(reinterpret_cast<const V4*>(p) + 1);
-    return __builtin_bit_cast(P, t);
-  }
-}
-
 // R consecutive rows per lane: when the number of rows is a multiple of R every slot starts at a multiple of
 // R, so the lane's R values and R indices of a slot are aligned vector loads (for 8-byte values and R = 2:
 // 16 / 8 bytes per lane instead of 8 / 4): 1 / R as many memory instructions for the same bytes.  Measured on

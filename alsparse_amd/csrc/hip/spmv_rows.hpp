@@ -16,7 +16,6 @@
 // (fma accumulation per lane, then y = beta*y + alpha*sum), different mapping.
 // beta == 0 never reads y.  All element offsets are formed in 64 bits.
 #pragma once
-
 #include "device_utils.hpp"
 
 namespace asamd {
@@ -67,29 +66,68 @@ __global__ __launch_bounds__(kRowsBlock) void spmv_scalar_kernel(
   store_axpby(y, row, alpha, sum, beta);
 }
 
-// ---- short rows: LDS-staged row blocks ---------------------------------------
-// A workgroup owns kStreamRows consecutive rows, none longer than
-// kStreamMaxLen.  Their entries are one contiguous range of the CSR streams: it
-// is read fully coalesced (lane k takes entries k, k + 256, ...), multiplied
-// with the gathered x and staged in LDS; after one barrier every lane sums the
-// few products of its own row from LDS (a lane's run is contiguous and runs of
-// neighbouring lanes are adjacent, so the reads spread over the banks) and
-// writes y unit stride.  No searches, no scans: this is what rows of 3-5
-// entries (stencils) want.
-constexpr int kStreamRows = 256;
-constexpr int kStreamMaxLen = 16;
+// ---- four values at a time --------------------------------------------------
+// four consecutive values: 128-bit pieces for the real types, one load per value otherwise
+template <typename T>
+struct Quad {
+  T e[4];
+  __device__ __forceinline__ void load(const T* p) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) e[i] = p[i];
+  }
+  __device__ __forceinline__ T get(int i) const { return e[i]; }
+};
+template <>
+struct Quad<float> {
+  Float4 q;
+  __device__ __forceinline__ void load(const float* p) { q = *reinterpret_cast<const Float4*>(p); }
+  __device__ __forceinline__ void load_nt(const float* p) { q = nt_load_object(reinterpret_cast<const Float4*>(p)); }
+  __device__ __forceinline__ float get(int i) const { return i == 0 ? q.x : i == 1 ? q.y : i == 2 ? q.z : q.w; }
+};
+template <>
+struct Quad<double> {
+  Double2 a, b;
+  __device__ __forceinline__ void load(const double* p) {
+    a = *reinterpret_cast<const Double2*>(p);
+    b = *reinterpret_cast<const Double2*>(p + 2);
+  }
+  __device__ __forceinline__ void load_nt(const double* p) {
+    a = nt_load_object(reinterpret_cast<const Double2*>(p));
+    b = nt_load_object(reinterpret_cast<const Double2*>(p + 2));
+  }
+  __device__ __forceinline__ double get(int i) const { return i == 0 ? a.x : i == 1 ? a.y : i == 2 ? b.x : b.y; }
+};
 
-// CAP: compile-time bound on the row length (4, 8 or 16): sizes the LDS staging
-// area, so shorter rows leave room for more resident workgroups.
-template <typename T, int CAP>
+// ---- regular rows: LDS-staged row blocks ---------------------------------------
+// A workgroup owns kStreamRows / G consecutive rows, none longer than CAP * G
+// entries.  Their entries are one contiguous range of the CSR streams: it
+// is read fully coalesced (lane k takes entries k, k + 256, ...: every load of
+// the workgroup is issued before the first is used), multiplied
+// with the gathered x and staged in LDS; after one barrier G lanes sum the
+// products of a row from LDS (with G = 1 a lane's run is contiguous and runs of
+// neighbouring lanes are adjacent, so the reads spread over the banks), a butterfly
+// joins them and the rows' y are written unit stride.  No searches, no scans: this is
+// what rows of 3-5 entries (stencils, G = 1) want, and with G = 2 .. 16 rows of some tens of
+// entries whose lengths differ too little to need merge-path (a lane group per row straight from
+// global memory has three dependent loads per row and few of them in flight).
+// The indices are loaded non-temporally, the values not: measured on 4 M - 8 M rows of 5 entries,
+// 21 % (fp64 stencil), 17 % (fp32) and 3 % (fp64, random columns) faster than both plain.
+constexpr int kStreamRows = 256;
+constexpr int kStreamMaxLen = 16;        // longest row of the one-lane-per-row form
+constexpr int kStreamMaxGroup = 16;      // most lanes per row
+
+// CAP: entries per thread that the LDS staging area is sized for (256 * CAP products), G: lanes per row
+template <typename T, int CAP, int G = 1>
 __global__ __launch_bounds__(kStreamRows) void spmv_stream_kernel(
     int m, T alpha, const T* __restrict__ val, const int* __restrict__ row_ptr,
     const int* __restrict__ col_ind, const T* __restrict__ x, T beta, T* __restrict__ y, int base) {
+  constexpr int kRows = kStreamRows / G;
   __shared__ T s_prod[kStreamRows * CAP];
   const unsigned bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
-  const int64_t row0 = (int64_t)bid * kStreamRows;
-  const int64_t row = row0 + threadIdx.x;
-  int64_t row_last = row0 + kStreamRows;
+  const int64_t row0 = (int64_t)bid * kRows;
+  const int lane = threadIdx.x % G;
+  const int64_t row = row0 + threadIdx.x / G;
+  int64_t row_last = row0 + kRows;
   if (row_last > m) row_last = m;
   const int64_t e0 = (int64_t)row_ptr[row0] - base;
   const int n = (int)((int64_t)row_ptr[row_last] - base - e0);  // <= kStreamRows * CAP by contract
@@ -106,7 +144,7 @@ __global__ __launch_bounds__(kStreamRows) void spmv_stream_kernel(
     const int k = threadIdx.x + s * kStreamRows;
     if (k < n) {
       v[s] = val[e0 + k];
-      c[s] = col_ind[e0 + k];
+      c[s] = nt_load(col_ind + e0 + k);
     }
   }
 #pragma unroll
@@ -115,31 +153,87 @@ __global__ __launch_bounds__(kStreamRows) void spmv_stream_kernel(
     if (k < n) s_prod[k] = v[s] * xb[c[s]];
   }
   __syncthreads();
-  if (row >= m) return;
+  if (row >= m) return;  // whole lane groups leave together
   T sum = T(0);
-  for (int k = my_begin; k < my_end; ++k) sum += s_prod[k];
-  store_axpby(y, row, alpha, sum, beta);
+  for (int k = my_begin + lane; k < my_end; k += G) sum += s_prod[k];
+  if constexpr (G > 1) sum = group_sum<G>(sum);
+  if (lane == 0) store_axpby(y, row, alpha, sum, beta);
+}
+
+// The same with 128-bit loads: the window of the workgroup's entries starts at the multiple of four entries
+// at or before its first entry, thread t takes pieces t, t + 256, ... of four consecutive entries (values and
+// indices; one more piece than CAP / 4 because of the up to three entries in front), and the entries outside
+// the block are dropped.  A quarter of the memory instructions for the same bytes.  val and col_ind must be
+// 16-byte aligned; `limit` is the number of entries in the arrays (counted like row_ptr - base): pieces that
+// would reach past it -- in the last workgroup only -- are read entry by entry.
+template <typename T, int CAP, int G>
+__global__ __launch_bounds__(kStreamRows) void spmv_stream_wide_kernel(
+    int m, T alpha, const T* __restrict__ val, const int* __restrict__ row_ptr,
+    const int* __restrict__ col_ind, const T* __restrict__ x, T beta, T* __restrict__ y, int base, int64_t limit) {
+  constexpr int kRows = kStreamRows / G;
+  constexpr int kPieces = CAP / 4 + 1;
+  __shared__ T s_prod[kStreamRows * CAP];
+  const unsigned bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  const int64_t row0 = (int64_t)bid * kRows;
+  const int lane = threadIdx.x % G;
+  const int64_t row = row0 + threadIdx.x / G;
+  int64_t row_last = row0 + kRows;
+  if (row_last > m) row_last = m;
+  const int64_t e0 = (int64_t)row_ptr[row0] - base;
+  const int n = (int)((int64_t)row_ptr[row_last] - base - e0);  // <= kStreamRows * CAP by contract
+  int my_begin = 0, my_end = 0;
+  if (row < m) {
+    my_begin = (int)((int64_t)row_ptr[row] - base - e0);
+    my_end = (int)((int64_t)row_ptr[row + 1] - base - e0);
+  }
+  const T* __restrict__ xb = x - base;
+  const int64_t a0 = e0 & ~(int64_t)3;
+  const int head = (int)(e0 - a0);
+  const int span = n + head;  // entries of the window
+  Quad<T> v[kPieces];
+  Int4 c[kPieces];
+#pragma unroll
+  for (int s = 0; s < kPieces; ++s) {
+    const int k = 4 * (threadIdx.x + s * kStreamRows);
+    if (k < span) {
+      if (a0 + k + 4 <= limit) {
+        v[s].load(val + a0 + k);
+        c[s] = nt_load_object(reinterpret_cast<const Int4*>(col_ind + a0 + k));
+      } else {
+        // the arrays end inside this piece
+        alignas(32) T tv[4] = {T(0), T(0), T(0), T(0)};
+        int tc[4] = {base, base, base, base};
+        for (int j = 0; j < 4 && a0 + k + j < limit; ++j) {
+          tv[j] = val[a0 + k + j];
+          tc[j] = col_ind[a0 + k + j];
+        }
+        v[s].load(tv);
+        c[s] = Int4{tc[0], tc[1], tc[2], tc[3]};
+      }
+    }
+  }
+#pragma unroll
+  for (int s = 0; s < kPieces; ++s) {
+    const int k = 4 * (threadIdx.x + s * kStreamRows) - head;  // position of the piece's first entry in the block
+    if (k + head < span) {
+      const int cc[4] = {c[s].x, c[s].y, c[s].z, c[s].w};
+      T xv[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) xv[j] = (k + j >= 0 && k + j < n) ? xb[cc[j]] : T(0);
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (k + j >= 0 && k + j < n) s_prod[k + j] = v[s].get(j) * xv[j];
+    }
+  }
+  __syncthreads();
+  if (row >= m) return;  // whole lane groups leave together
+  T sum = T(0);
+  for (int k = my_begin + lane; k < my_end; k += G) sum += s_prod[k];
+  if constexpr (G > 1) sum = group_sum<G>(sum);
+  if (lane == 0) store_axpby(y, row, alpha, sum, beta);
 }
 
 // ---- constant row length ----------------------------------------------------
-template <typename T>
-struct Quad;  // four consecutive values loaded as 128-bit pieces
-template <>
-struct Quad<float> {
-  Float4 q;
-  __device__ __forceinline__ void load(const float* p) { q = *reinterpret_cast<const Float4*>(p); }
-  __device__ __forceinline__ float get(int i) const { return i == 0 ? q.x : i == 1 ? q.y : i == 2 ? q.z : q.w; }
-};
-template <>
-struct Quad<double> {
-  Double2 a, b;
-  __device__ __forceinline__ void load(const double* p) {
-    a = *reinterpret_cast<const Double2*>(p);
-    b = *reinterpret_cast<const Double2*>(p + 2);
-  }
-  __device__ __forceinline__ double get(int i) const { return i == 0 ? a.x : i == 1 ? a.y : i == 2 ? b.x : b.y; }
-};
-
 // G lanes per row, each owning 4 consecutive entries: L = 4*G.  R rows per
 // lane group and launch keep 4*R gathers per lane in flight.
 template <typename T, int G, int R>
@@ -161,8 +255,11 @@ __global__ __launch_bounds__(kRowsBlock) void spmv_rowconst_kernel(
     const int64_t row = row0 + (int64_t)r * kGroups;
     if (row < m) {
       const int64_t off = row * L + lane * 4;
-      v[r].load(val + off);
-      c[r] = *reinterpret_cast<const Int4*>(col_ind + off);
+      // cache policy as measured (4 M - 8 M rows of 8 or 16 entries, x in the L1, an L2 or beyond): the
+      // indices non-temporal gains up to 6 %; the values too for 4-byte types (5 % more), not for 8-byte ones
+      if constexpr (sizeof(T) == 4) v[r].load_nt(val + off);
+      else v[r].load(val + off);
+      c[r] = nt_load_object(reinterpret_cast<const Int4*>(col_ind + off));
     }
   }
   T xs[R][4];

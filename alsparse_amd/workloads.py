@@ -124,6 +124,34 @@ def bimodal_rows(rows, cols, k_short, k_long, every, dtype=np.float32, seed=SEED
                "bimodal_rows(%d,%d,%d,%d,%d)" % (rows, cols, k_short, k_long, every))
 
 
+def stencil3d(nx, ny, nz, dtype=np.float64, seed=SEED, base=0):
+    """The 27-point stencil on an nx x ny x nz grid (x fastest): every grid point is coupled to itself and to its
+    neighbours within one step in each direction, 8 to 27 entries per row, columns ascending, random values.
+    Not a benchmark configuration: the structure of a trilinear finite-element matrix, rows of similar lengths
+    whose x entries neighbouring rows share."""
+    rows = nx * ny * nz
+    idx = np.arange(rows, dtype=np.int64)
+    ix, iy, iz = idx % nx, (idx // nx) % ny, idx // (nx * ny)
+    offsets = [(dz, dy, dx) for dz in (-1, 0, 1) for dy in (-1, 0, 1) for dx in (-1, 0, 1)]  # ascending columns
+    masks = [((ix + dx >= 0) & (ix + dx < nx) & (iy + dy >= 0) & (iy + dy < ny) & (iz + dz >= 0) & (iz + dz < nz))
+             for dz, dy, dx in offsets]
+    lengths = np.zeros(rows, dtype=np.int64)
+    for mk in masks:
+        lengths += mk
+    row_ptr = np.zeros(rows + 1, dtype=np.int64)
+    np.cumsum(lengths, out=row_ptr[1:])
+    nnz = int(row_ptr[-1])
+    if nnz >= 2 ** 31:
+        raise ValueError("more than 2^31 - 1 entries")
+    col_ind = np.empty(nnz, dtype=np.int32)
+    pos = row_ptr[:-1].copy()
+    for (dz, dy, dx), mk in zip(offsets, masks):
+        col_ind[pos[mk]] = (idx[mk] + (dz * ny + dy) * nx + dx + base).astype(np.int32)
+        pos += mk
+    vals = uniform(nnz, dtype, 2, seed)
+    return Csr(rows, rows, (row_ptr + base).astype(np.int32), col_ind, vals, base, "stencil3d(%d,%d,%d)" % (nx, ny, nz))
+
+
 def laplace2d(nx, ny, dtype=np.float64, base=0):
     lib = _load()
     rows = nx * ny

@@ -34,7 +34,8 @@ MEASURED_TRAFFIC_BYTES = {
     (3, "tiled two-phase"): (5.17e9, "profiles/spmv_tiled_C3.txt"),
     (3, "rowconst"): (34.6e9, "profiles/spmv_tiled_C3.txt"),
     (4, "merge-path"): (3.32e9, "profiles/spmv_merge_C4.txt"),
-    (2, "ell copy"): (322.5e6, "profiles/spmv_ell_copy_C2.txt"),
+    (2, "ell copy"): (356.6e6, "profiles/spmv_ell_copy_C2.txt"),
+    (2, "row-block stream"): (338.8e6, "profiles/spmv_stream_C2.txt"),
     (5, "spmm row-major"): (9.27e9, "profiles/spmm_rowmajor_C5.txt"),
 }
 
@@ -148,6 +149,12 @@ def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False, vendor=Fa
         x, y0, alpha, beta = wl.uniform(a.cols, udt, 3), wl.uniform(a.rows, udt, 4), 1.0, 0.5
         workload_name = ("two row lengths: CSR SpMV %s, %d rows x %d columns, every %d-th row %d entries, the others %d, "
                          "uniform random sorted columns, alpha=1 beta=0.5" % (np.dtype(udt).name, um, un, every, kl, ks))
+    elif isinstance(cfg, tuple) and cfg[0] == "stencil3d":  # ("stencil3d", nx, ny, nz, dtype)
+        _, gx, gy, gz, udt = cfg
+        a = wl.stencil3d(gx, gy, gz, udt)
+        x, y0, alpha, beta = wl.uniform(a.cols, udt, 3), wl.uniform(a.rows, udt, 4), 1.0, 0.5
+        workload_name = "27-point stencil: CSR SpMV %s, %d x %d x %d grid (%d rows, %d nnz), alpha=1 beta=0.5" % (
+            np.dtype(udt).name, gx, gy, gz, a.rows, a.nnz)
     elif isinstance(cfg, tuple):  # ("uniform", rows, cols, entries per row, dtype): not a benchmark configuration
         _, um, un, uk, udt = cfg
         a = wl.uniform_rows(um, un, uk, udt)
@@ -595,7 +602,9 @@ def main():
     ap.add_argument("--bimodal", nargs=5, type=int, metavar=("ROWS", "COLS", "SHORT", "LONG", "EVERY"),
                     help="instead of a configuration: CSR SpMV on a matrix whose every EVERY-th row has LONG entries "
                          "and the others SHORT (the workload of the row-length bins)")
-    ap.add_argument("--fp64", action="store_true", help="with --uniform / --bimodal: fp64 values")
+    ap.add_argument("--stencil3d", nargs=3, type=int, metavar=("NX", "NY", "NZ"),
+                    help="instead of a configuration: the 27-point stencil on an NX x NY x NZ grid (8 to 27 entries per row)")
+    ap.add_argument("--fp64", action="store_true", help="with --uniform / --bimodal / --stencil3d: fp64 values")
     ap.add_argument("--all", action="store_true", help="also measure the other configurations")
     ap.add_argument("--only", action="store_true",
                     help="measure the selected configuration alone (by default the line also carries brief figures of "
@@ -658,10 +667,12 @@ def main():
             cfg = ("uniform", args.uniform[0], args.uniform[1], args.uniform[2], np.float64 if args.fp64 else np.float32)
         if args.bimodal:
             cfg = ("bimodal",) + tuple(args.bimodal) + (np.float64 if args.fp64 else np.float32,)
+        if args.stencil3d:
+            cfg = ("stencil3d",) + tuple(args.stencil3d) + (np.float64 if args.fp64 else np.float32,)
         main_res = run_spmv(cfg, args.steps, args.warmup, not args.no_cpu_baseline, check, args.transpose,
                             not args.no_vendor_baseline, args.cx, args.conjugate)
     others = {}
-    plain_default = (args.config == 3 and not (args.all or args.only or args.uniform or args.bimodal or args.transpose or args.cx or
+    plain_default = (args.config == 3 and not (args.all or args.only or args.uniform or args.bimodal or args.stencil3d or args.transpose or args.cx or
                                                args.conversions or args.col_major) and args.format == "csr")
     if plain_default:
         # the default line is configuration 3; the other device configurations ride along, briefly

@@ -21,12 +21,33 @@ def announce(*what):
     print("[gpu-case]", *what, flush=True)
 
 
+class _ShiftedArray:
+    """A device array that starts `shift` elements into its allocation (so that it is not 16-byte aligned)."""
+
+    def __init__(self, host, shift):
+        import ctypes
+        self._ctypes = ctypes
+        lead = np.zeros(shift, dtype=host.dtype)
+        self.dev = hiprt.DeviceArray.from_numpy(np.concatenate([lead, host]))
+        self.offset = shift * host.dtype.itemsize
+
+    def c_ptr(self):
+        return self._ctypes.c_void_p(self.dev.ptr + self.offset)
+
+    def free(self):
+        self.dev.free()
+
+
 class DeviceCsr:
-    def __init__(self, a):
+    def __init__(self, a, shift=0):
+        """shift: elements by which val and col_ind are moved off their allocations' (256-byte) alignment"""
         self.a = a
-        self.val = hiprt.DeviceArray.from_numpy(a.values)
         self.row_ptr = hiprt.DeviceArray.from_numpy(a.row_ptr)
-        self.col = hiprt.DeviceArray.from_numpy(a.col_ind)
+        if shift:
+            self.val, self.col = _ShiftedArray(a.values, shift), _ShiftedArray(a.col_ind, shift)
+        else:
+            self.val = hiprt.DeviceArray.from_numpy(a.values)
+            self.col = hiprt.DeviceArray.from_numpy(a.col_ind)
 
     def free(self):
         for d in (self.val, self.row_ptr, self.col):

@@ -36,6 +36,11 @@ SHAPES = {
     "ragged_tail": lambda dt: csr_from_lengths(list(range(0, 300)), 4000, dt),
     "length_class_edges": lambda dt: csr_from_lengths([8, 9, 0, 64, 65, 2048, 2049, 1, 4096, 4097, 8193, 7, 63], 9000, dt),
     "wide_few_rows": lambda dt: csr_from_lengths([4096, 4095, 4097, 1, 0, 8192], 10000, dt),
+    # rows of similar lengths: the staged row-block kernel with 2, 4, 8 and 16 lanes per row
+    "stencil3d_12x10x9": lambda dt: wl.stencil3d(12, 10, 9, dt),
+    "regular_40_60": lambda dt: csr_from_lengths(list(40 + (np.arange(1500) * 7) % 21), 3000, dt),
+    "regular_90_128": lambda dt: csr_from_lengths(list(90 + (np.arange(700) * 5) % 39), 3000, dt),
+    "regular_200_256": lambda dt: csr_from_lengths(list(200 + (np.arange(300) * 11) % 57), 3000, dt),
 }
 
 
@@ -58,8 +63,30 @@ def test_every_kernel_family_matches_oracle(gpu, shape, dtype):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
+@pytest.mark.parametrize("shift", [1, 3], ids=["shift1", "shift3"])
+def test_streams_off_16_byte_alignment(gpu, dtype, shift):
+    """val and col_ind that are element-aligned only: the kernels with 128-bit loads (constant row length,
+    staged row blocks, ELL pairs) must take their narrow forms, not fault and not read other bytes."""
+    for maker in (lambda: wl.stencil3d(12, 10, 9, dtype), lambda: wl.uniform_rows(3000, 2500, 16, dtype),
+                  lambda: wl.laplace2d(40, 30, dtype), lambda: csr_from_lengths(list(40 + (np.arange(1500) * 7) % 21), 3000, dtype)):
+        a = maker()
+        x, y0 = _vectors(a)
+        da = DeviceCsr(a, shift=shift)
+        try:
+            for algo in ("vector", "merge", "rowconst", "stream", "binned", "auto"):
+                announce("spmv shifted streams", a.name, np.dtype(dtype).name, algo, shift)
+                y = run_plan_csrmv(da, algo, 1.5, x, 0.25, y0)
+                if y is None:
+                    continue
+                check_spmv(a, 1.5, x, 0.25, y0, y, "%s/%s/shift%d" % (a.name, algo, shift))
+        finally:
+            da.free()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
 def test_index_base_one(gpu, dtype):
     for maker in (lambda: wl.uniform_rows(3000, 2500, 16, dtype, base=1),
+                  lambda: wl.stencil3d(9, 8, 7, dtype, base=1),
                   lambda: wl.powerlaw_rmat(12, 2000, dtype, base=1),
                   lambda: wl.laplace2d(40, 30, dtype, base=1)):
         a = maker()
@@ -378,9 +405,10 @@ def test_copy_is_not_used_for_another_value_array(gpu, algo):
 
 
 def test_analysis_choices(gpu):
-    """What the analysis decides and what it skips: a banded matrix keeps the ELL copy and never lays out
-    the tiled one (its floor is slower than the ELL kernel measured); a matrix small enough to be
-    launch-bound takes the single-kernel path however skewed its rows are."""
+    """What the analysis decides and what it skips: a banded matrix runs the staged row-block kernel on the
+    caller's arrays, or the ELL copy if that measured at least 5 % faster (the two are within a few per cent
+    of each other), and never lays out the tiled copy (its floor is slower than either); a matrix small
+    enough to be launch-bound takes the single-kernel path however skewed its rows are."""
     lib = capi.load()
     a, x, y0, alpha, beta, _ = wl.config(2)
     da = DeviceCsr(a)
@@ -392,8 +420,10 @@ def test_analysis_choices(gpu):
         assert lib.alphasparse_dcu_d_csrmv_analysis(gpu.h, 0, a.rows, a.cols, a.nnz, byref(descr), da.val.c_ptr(),
                                                     da.row_ptr.c_ptr(), da.col.c_ptr(), info) == 0
         st = lib.asamd_analysis_stats(info).contents
-        assert st.algo == capi.ASAMD_SPMV_ELL and st.ell_built == 1 and st.tiled_built == 0
+        assert st.algo in (capi.ASAMD_SPMV_ELL, capi.ASAMD_SPMV_STREAM), capi.ALGO_NAMES[st.algo]
+        assert st.ell_built == (1 if st.algo == capi.ASAMD_SPMV_ELL else 0) and st.tiled_built == 0
         assert st.tune_ms_ell > 0 and st.tune_ms_base > 0 and st.tune_ms_tiled == 0
+        assert (st.algo == capi.ASAMD_SPMV_ELL) == (st.tune_ms_ell < 0.95 * st.tune_ms_base)
         check_spmv(a, alpha, x, beta, y0, run_csrmv(gpu, da, alpha, x, beta, y0, info), "config 2 analysed")
     finally:
         lib.alphasparse_dcu_destroy_mat_info(info)
