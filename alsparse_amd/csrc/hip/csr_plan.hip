@@ -201,7 +201,9 @@ static bool rowconst_ok(const asamd_csr_plan* p) {
 }
 
 // The LDS-staged row-block kernel sizes its staging area for rows of at most CAP * G entries (G lanes sum a
-// row); the bound comes from the analysis, so the structure must be promised fixed.  Returns G, or 0 when the
+// row); the bound comes from the row statistics.  A workgroup whose rows hold more than that (the structure
+// behind row_ptr changed under a plan that was not promised a fixed one) takes them straight from global
+// memory, so the choice is safe for such plans too.  Returns G, or 0 when the
 // kernel cannot take the matrix.  With `regular_only`, also 0 for G > 1 when the rows are so much shorter than
 // the longest that a workgroup's 256 / G rows hold fewer than four entries per thread.
 // 16 KiB of products per workgroup: 16 entries per thread for 4-byte values, 8 for 8-byte, 4 for 16-byte ones
@@ -209,7 +211,7 @@ static bool rowconst_ok(const asamd_csr_plan* p) {
 static int stream_cap(const asamd_csr_plan* p) { return 64 / p->val_size; }
 static int stream_group(const asamd_csr_plan* p, bool regular_only) {
   const asamd_csr_stats& st = p->st;
-  if (!st.trusted || st.max_len < 1) return 0;
+  if (st.max_len < 1) return 0;
   const int cap = stream_cap(p);
   if (st.max_len <= cap) return 1;
   int g = 2;
@@ -1609,10 +1611,19 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
         merge_partition_kernel<<<(nb + 1 + 255) / 256, 256, 0, s>>>(
             st.m, st.nnz, rp, st.base, nb, kMergeThreads * p->merge_ipt, p->d_block_row);
       }
-#define ASAMD_LAUNCH_MERGE(IPT)                                                                       \
-  spmv_merge_kernel<T, IPT><<<nb, kMergeThreads, 0, s>>>(st.m, st.nnz, alpha, val, rp, ci, x, beta, y, \
-                                                         st.base, p->d_block_row, p->d_carry_row,      \
-                                                         (T*)p->d_carry_val, (T*)p->d_head_val)
+      // 128-bit loads of the streams need them 16-byte aligned
+      const bool merge_wide = (((uintptr_t)val | (uintptr_t)ci) & 15u) == 0;
+#define ASAMD_LAUNCH_MERGE(IPT)                                                                                  \
+  do {                                                                                                           \
+    if (merge_wide && (IPT) % 4 == 0)                                                                            \
+      spmv_merge_kernel<T, IPT, true><<<nb, kMergeThreads, 0, s>>>(st.m, st.nnz, alpha, val, rp, ci, x, beta, y, \
+                                                                   st.base, p->d_block_row, p->d_carry_row,      \
+                                                                   (T*)p->d_carry_val, (T*)p->d_head_val);       \
+    else                                                                                                         \
+      spmv_merge_kernel<T, IPT><<<nb, kMergeThreads, 0, s>>>(st.m, st.nnz, alpha, val, rp, ci, x, beta, y,       \
+                                                             st.base, p->d_block_row, p->d_carry_row,            \
+                                                             (T*)p->d_carry_val, (T*)p->d_head_val);             \
+  } while (0)
       // LDS per workgroup grows with IPT * sizeof(T): 16-byte values run 4 items only, 8-byte ones up to 16
       if constexpr (sizeof(T) <= 8) {
         if (p->merge_ipt == 16 && kIsReal<T>) ASAMD_LAUNCH_MERGE(16);

@@ -318,4 +318,41 @@ struct alignas(16) Int4 { int x, y, z, w; };
 struct alignas(16) Float4 { float x, y, z, w; };
 struct alignas(16) Double2 { double x, y; };
 
+// ---- four values at a time --------------------------------------------------
+// four consecutive values: 128-bit pieces for the real types, one load per value otherwise
+template <typename T>
+struct Quad {
+  T e[4];
+  __device__ __forceinline__ void load(const T* p) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) e[i] = p[i];
+  }
+  __device__ __forceinline__ void load_nt(const T* p) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) e[i] = nt_load(p + i);
+  }
+  __device__ __forceinline__ T get(int i) const { return e[i]; }
+};
+template <>
+struct Quad<float> {
+  Float4 q;
+  __device__ __forceinline__ void load(const float* p) { q = *reinterpret_cast<const Float4*>(p); }
+  __device__ __forceinline__ void load_nt(const float* p) { q = nt_load_object(reinterpret_cast<const Float4*>(p)); }
+  __device__ __forceinline__ float get(int i) const { return i == 0 ? q.x : i == 1 ? q.y : i == 2 ? q.z : q.w; }
+};
+template <>
+struct Quad<double> {
+  Double2 a, b;
+  __device__ __forceinline__ void load(const double* p) {
+    a = *reinterpret_cast<const Double2*>(p);
+    b = *reinterpret_cast<const Double2*>(p + 2);
+  }
+  __device__ __forceinline__ void load_nt(const double* p) {
+    a = nt_load_object(reinterpret_cast<const Double2*>(p));
+    b = nt_load_object(reinterpret_cast<const Double2*>(p + 2));
+  }
+  __device__ __forceinline__ double get(int i) const { return i == 0 ? a.x : i == 1 ? a.y : i == 2 ? b.x : b.y; }
+};
+
+
 }  // namespace asamd

@@ -74,8 +74,11 @@ __global__ __launch_bounds__(256) void merge_partition_kernel(int m, int nnz,
   block_row[b] = (int)lo;
 }
 
-// IPT items per thread, kMergeThreads * IPT items per workgroup.
-template <typename T, int IPT>
+// IPT items per thread, kMergeThreads * IPT items per workgroup.  WIDE: val and col_ind are 16-byte aligned
+// and the workgroup's entries are read as pieces of four from the multiple of four at or before its first
+// entry (a quarter of the memory instructions); a workgroup whose last piece would reach past the end of
+// the arrays reads entry by entry.
+template <typename T, int IPT, bool WIDE = false>
 __global__ __launch_bounds__(kMergeThreads) void spmv_merge_kernel(
     int m, int nnz, T alpha, const T* __restrict__ val, const int* __restrict__ row_ptr,
     const int* __restrict__ col_ind, const T* __restrict__ x, T beta, T* __restrict__ y, int base,
@@ -116,7 +119,45 @@ __global__ __launch_bounds__(kMergeThreads) void spmv_merge_kernel(
     s_rend[i] = e > kItems ? kItems + 1 : (e < 0 ? 0 : (int)e);
   }
   // ---- stream entries, gather x, stage products ----------------------------
-  {
+  const int64_t win0 = nnz_b & ~(int64_t)3;  // the window of whole pieces around the workgroup's entries
+  const int head = (int)(nnz_b - win0);
+  const int span = (nnz_cnt + head + 3) & ~3;
+  if (WIDE && IPT % 4 == 0 && nnz_cnt > 0 && win0 + span <= nnz) {  // workgroup-uniform
+    // Every load is issued unconditionally (a thread past the end of the window re-reads its first piece), and
+    // so is every gather: the entries in front of and behind the workgroup's own are entries of the matrix too.
+    const T* __restrict__ xb = x - base;
+    constexpr int kPieces = IPT / 4;
+    Quad<T> v[kPieces];
+    Int4 c[kPieces];
+#pragma unroll
+    for (int s = 0; s < kPieces; ++s) {
+      const int k = 4 * (tid + s * kMergeThreads);
+      const int64_t kk = win0 + (k < span ? k : 0);
+      v[s].load_nt(val + kk);
+      c[s] = nt_load_object(reinterpret_cast<const Int4*>(col_ind + kk));
+    }
+    T xv[kPieces][4];
+#pragma unroll
+    for (int s = 0; s < kPieces; ++s) {
+      xv[s][0] = xb[c[s].x];
+      xv[s][1] = xb[c[s].y];
+      xv[s][2] = xb[c[s].z];
+      xv[s][3] = xb[c[s].w];
+    }
+#pragma unroll
+    for (int s = 0; s < kPieces; ++s) {
+      const int k = 4 * (tid + s * kMergeThreads) - head;  // the piece's first entry, counted from the workgroup's
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (k + j >= 0 && k + j < nnz_cnt) s_prod[lds_pad(k + j)] = v[s].get(j) * xv[s][j];
+    }
+    // a workgroup of nothing but entries that starts off a multiple of four has one piece more: thread 0 takes it
+    if (tid == 0 && span > kItems) {
+      const int k = kItems - head;
+      for (int j = 0; j < 4; ++j)
+        if (k + j < nnz_cnt) s_prod[lds_pad(k + j)] = nt_load(val + nnz_b + k + j) * xb[nt_load(col_ind + nnz_b + k + j)];
+    }
+  } else {
     // Every load is issued unconditionally (a thread past the end of the range re-reads the range's
     // first entry): loads under a branch make the compiler wait for ALL outstanding loads before
     // each use, which turned the IPT gathers of a thread into a chain of IPT memory latencies.

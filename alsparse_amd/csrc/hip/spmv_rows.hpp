@@ -66,38 +66,6 @@ __global__ __launch_bounds__(kRowsBlock) void spmv_scalar_kernel(
   store_axpby(y, row, alpha, sum, beta);
 }
 
-// ---- four values at a time --------------------------------------------------
-// four consecutive values: 128-bit pieces for the real types, one load per value otherwise
-template <typename T>
-struct Quad {
-  T e[4];
-  __device__ __forceinline__ void load(const T* p) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) e[i] = p[i];
-  }
-  __device__ __forceinline__ T get(int i) const { return e[i]; }
-};
-template <>
-struct Quad<float> {
-  Float4 q;
-  __device__ __forceinline__ void load(const float* p) { q = *reinterpret_cast<const Float4*>(p); }
-  __device__ __forceinline__ void load_nt(const float* p) { q = nt_load_object(reinterpret_cast<const Float4*>(p)); }
-  __device__ __forceinline__ float get(int i) const { return i == 0 ? q.x : i == 1 ? q.y : i == 2 ? q.z : q.w; }
-};
-template <>
-struct Quad<double> {
-  Double2 a, b;
-  __device__ __forceinline__ void load(const double* p) {
-    a = *reinterpret_cast<const Double2*>(p);
-    b = *reinterpret_cast<const Double2*>(p + 2);
-  }
-  __device__ __forceinline__ void load_nt(const double* p) {
-    a = nt_load_object(reinterpret_cast<const Double2*>(p));
-    b = nt_load_object(reinterpret_cast<const Double2*>(p + 2));
-  }
-  __device__ __forceinline__ double get(int i) const { return i == 0 ? a.x : i == 1 ? a.y : i == 2 ? b.x : b.y; }
-};
-
 // ---- regular rows: LDS-staged row blocks ---------------------------------------
 // A workgroup owns kStreamRows / G consecutive rows, none longer than CAP * G
 // entries.  Their entries are one contiguous range of the CSR streams: it
@@ -116,6 +84,20 @@ constexpr int kStreamRows = 256;
 constexpr int kStreamMaxLen = 16;        // longest row of the one-lane-per-row form
 constexpr int kStreamMaxGroup = 16;      // most lanes per row
 
+// What a workgroup of the staged kernels does when its rows hold more entries than its staging area: G lanes
+// per row, straight from global memory.
+template <typename T, int G>
+__device__ __forceinline__ void stream_rows_direct(int m, int64_t row, int lane, T alpha, const T* __restrict__ val,
+                                                   const int* __restrict__ row_ptr, const int* __restrict__ col_ind,
+                                                   const T* __restrict__ xb, T beta, T* __restrict__ y, int base) {
+  if (row >= m) return;  // whole lane groups leave together
+  const int64_t end = (int64_t)row_ptr[row + 1] - base;
+  T sum = T(0);
+  for (int64_t k = (int64_t)row_ptr[row] - base + lane; k < end; k += G) sum = fma_t(val[k], xb[col_ind[k]], sum);
+  if constexpr (G > 1) sum = group_sum<G>(sum);
+  if (lane == 0) store_axpby(y, row, alpha, sum, beta);
+}
+
 // CAP: entries per thread that the LDS staging area is sized for (256 * CAP products), G: lanes per row
 template <typename T, int CAP, int G = 1>
 __global__ __launch_bounds__(kStreamRows) void spmv_stream_kernel(
@@ -130,13 +112,20 @@ __global__ __launch_bounds__(kStreamRows) void spmv_stream_kernel(
   int64_t row_last = row0 + kRows;
   if (row_last > m) row_last = m;
   const int64_t e0 = (int64_t)row_ptr[row0] - base;
-  const int n = (int)((int64_t)row_ptr[row_last] - base - e0);  // <= kStreamRows * CAP by contract
+  const int64_t n64 = (int64_t)row_ptr[row_last] - base - e0;  // at most kStreamRows * CAP for the analysed structure
+  const int n = n64 > INT32_MAX || n64 < 0 ? -1 : (int)n64;
   int my_begin = 0, my_end = 0;
   if (row < m) {
     my_begin = (int)((int64_t)row_ptr[row] - base - e0);
     my_end = (int)((int64_t)row_ptr[row + 1] - base - e0);
   }
   const T* __restrict__ xb = x - base;
+  if (n < 0 || n > kStreamRows * CAP) {
+    // The rows do not fit the staging area: row_ptr no longer holds the structure that the launch was sized
+    // for.  (Workgroup-uniform.)  The lane groups take their rows straight from the arrays.
+    stream_rows_direct<T, G>(m, row, lane, alpha, val, row_ptr, col_ind, xb, beta, y, base);
+    return;
+  }
   T v[CAP];
   int c[CAP];
 #pragma unroll
@@ -180,13 +169,20 @@ __global__ __launch_bounds__(kStreamRows) void spmv_stream_wide_kernel(
   int64_t row_last = row0 + kRows;
   if (row_last > m) row_last = m;
   const int64_t e0 = (int64_t)row_ptr[row0] - base;
-  const int n = (int)((int64_t)row_ptr[row_last] - base - e0);  // <= kStreamRows * CAP by contract
+  const int64_t n64 = (int64_t)row_ptr[row_last] - base - e0;  // at most kStreamRows * CAP for the analysed structure
+  const int n = n64 > INT32_MAX || n64 < 0 ? -1 : (int)n64;
   int my_begin = 0, my_end = 0;
   if (row < m) {
     my_begin = (int)((int64_t)row_ptr[row] - base - e0);
     my_end = (int)((int64_t)row_ptr[row + 1] - base - e0);
   }
   const T* __restrict__ xb = x - base;
+  if (n < 0 || n > kStreamRows * CAP) {
+    // The rows do not fit the staging area: row_ptr no longer holds the structure that the launch was sized
+    // for.  (Workgroup-uniform.)  The lane groups take their rows straight from the arrays.
+    stream_rows_direct<T, G>(m, row, lane, alpha, val, row_ptr, col_ind, xb, beta, y, base);
+    return;
+  }
   const int64_t a0 = e0 & ~(int64_t)3;
   const int head = (int)(e0 - a0);
   const int span = n + head;  // entries of the window

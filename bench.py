@@ -26,6 +26,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+NO_ANALYSIS = False  # --no-analysis
 
 # HBM bytes per multiply measured with rocprofv3 in separate counter runs (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000,
 # factors from a 1 GiB copy kernel) -- a table of earlier measurements, not an in-run reading; each entry names the
@@ -185,29 +186,33 @@ def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False, vendor=Fa
 
     info = capi.alphasparse_dcu_mat_info_t()
     assert lib.alphasparse_dcu_create_mat_info(byref(info)) == 0
+    al, be = T(alpha), T(beta)
+    csrmv = getattr(lib, "alphasparse_dcu_%s_csrmv" % p)
+    analysed = not (NO_ANALYSIS and not transpose)
+
+    def step():
+        s = csrmv(h.h, op, a.rows, a.cols, a.nnz, byref(al), byref(descr), d_val.c_ptr(), d_rp.c_ptr(),
+                  d_ci.c_ptr(), info if analysed else None, d_x.c_ptr(), byref(be), d_y.c_ptr())
+        if s != 0:
+            raise RuntimeError("csrmv status %d" % s)
+
     hiprt.synchronize()
     t0 = time.perf_counter()
-    st = getattr(lib, "alphasparse_dcu_%s_csrmv_analysis" % p)(
-        h.h, op, a.rows, a.cols, a.nnz, byref(descr), d_val.c_ptr(), d_rp.c_ptr(), d_ci.c_ptr(), info)
+    if analysed:
+        st = getattr(lib, "alphasparse_dcu_%s_csrmv_analysis" % p)(
+            h.h, op, a.rows, a.cols, a.nnz, byref(descr), d_val.c_ptr(), d_rp.c_ptr(), d_ci.c_ptr(), info)
+        assert st == 0, "analysis status %d" % st
+    else:
+        step()  # the first call without analysis looks at row_ptr once and remembers what it saw
     hiprt.synchronize()
     analysis_ms = (time.perf_counter() - t0) * 1e3
-    assert st == 0, "analysis status %d" % st
-    stats = lib.asamd_analysis_stats(info).contents
+    stats = lib.asamd_analysis_stats(info if analysed else d_rp.c_ptr()).contents
     if transpose:
         assert stats.transpose_built != 0, "no room for the transposed copy"
         stats = lib.asamd_analysis_transpose_stats(info).contents
     algo = capi.ALGO_NAMES.get(stats.algo, "?")
     if stats.algo == capi.ASAMD_SPMV_VECTOR:
         algo += "(W=%d)" % stats.vector_width
-
-    al, be = T(alpha), T(beta)
-    csrmv = getattr(lib, "alphasparse_dcu_%s_csrmv" % p)
-
-    def step():
-        s = csrmv(h.h, op, a.rows, a.cols, a.nnz, byref(al), byref(descr), d_val.c_ptr(), d_rp.c_ptr(),
-                  d_ci.c_ptr(), info, d_x.c_ptr(), byref(be), d_y.c_ptr())
-        if s != 0:
-            raise RuntimeError("csrmv status %d" % s)
 
     parity = None
     if check and cx and transpose:
@@ -242,15 +247,16 @@ def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False, vendor=Fa
     # is fingerprinted, found unchanged, and only the values of the plan's copies are gathered again
     hiprt.synchronize()
     t0 = time.perf_counter()
-    st = getattr(lib, "alphasparse_dcu_%s_csrmv_analysis" % p)(
-        h.h, op, a.rows, a.cols, a.nnz, byref(descr), d_val.c_ptr(), d_rp.c_ptr(), d_ci.c_ptr(), info)
+    if analysed:
+        st = getattr(lib, "alphasparse_dcu_%s_csrmv_analysis" % p)(
+            h.h, op, a.rows, a.cols, a.nnz, byref(descr), d_val.c_ptr(), d_rp.c_ptr(), d_ci.c_ptr(), info)
+        assert st == 0, "repeated analysis status %d" % st
     hiprt.synchronize()
-    reanalysis_ms = (time.perf_counter() - t0) * 1e3
-    assert st == 0, "repeated analysis status %d" % st
+    reanalysis_ms = (time.perf_counter() - t0) * 1e3 if analysed else None
     nbytes = (wl.spmv_bytes(a.cols, a.rows, a.nnz, a.dtype.itemsize, beta) if transpose
               else wl.spmv_bytes(a.rows, a.cols, a.nnz, a.dtype.itemsize, beta))
     opname = "" if not transpose else (" -- CONJUGATE-TRANSPOSED operation" if op == 2 else " -- TRANSPOSED operation")
-    res = {"workload": workload_name + (" -- COMPLEX values (%s)" % a.dtype.name if cx else "") + opname, "rows": a.rows, "nnz": a.nnz, "algorithmic_bytes": int(nbytes),
+    res = {"workload": workload_name + (" -- COMPLEX values (%s)" % a.dtype.name if cx else "") + opname + ("" if analysed else " -- WITHOUT analysis (info = NULL)"), "rows": a.rows, "nnz": a.nnz, "algorithmic_bytes": int(nbytes),
            "flops": 2 * a.nnz, "kernel": algo, "analysis_ms": analysis_ms, "reanalysis_ms": reanalysis_ms, "timing": t,
            "gbs": nbytes / t["avg_ms"] / 1e6, "gflops": 2 * a.nnz / t["avg_ms"] / 1e6,
            "dtype": {"float32": "f32", "float64": "f64", "complex64": "c64", "complex128": "c128"}[a.dtype.name],
@@ -611,6 +617,9 @@ def main():
                          "configurations 2, 4 and 5 under `others`)")
     ap.add_argument("--stream-ceiling", action="store_true",
                     help="instead of a workload: time plain read / write / copy / gather kernels and print their TB/s")
+    ap.add_argument("--no-analysis", action="store_true",
+                    help="CSR SpMV without alphasparse_dcu_?_csrmv_analysis (info = NULL, as the reference's own tests call it): "
+                         "analysis_ms is then the first call, which looks at row_ptr once")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-vendor-baseline", action="store_true",
                     help="skip timing rocSPARSE's csrmv on the same workload (reported as vendor_baseline)")
@@ -645,6 +654,8 @@ def main():
                           "ceilings": run_ceilings(args.steps, args.warmup)}), flush=True)
         return
 
+    global NO_ANALYSIS
+    NO_ANALYSIS = args.no_analysis
     check = not args.no_check
     conv = None
     if args.conversions:
@@ -672,7 +683,7 @@ def main():
         main_res = run_spmv(cfg, args.steps, args.warmup, not args.no_cpu_baseline, check, args.transpose,
                             not args.no_vendor_baseline, args.cx, args.conjugate)
     others = {}
-    plain_default = (args.config == 3 and not (args.all or args.only or args.uniform or args.bimodal or args.stencil3d or args.transpose or args.cx or
+    plain_default = (args.config == 3 and not (args.all or args.only or args.uniform or args.bimodal or args.stencil3d or args.no_analysis or args.transpose or args.cx or
                                                args.conversions or args.col_major) and args.format == "csr")
     if plain_default:
         # the default line is configuration 3; the other device configurations ride along, briefly

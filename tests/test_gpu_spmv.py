@@ -571,6 +571,39 @@ def test_row_ptr_into_the_middle_of_larger_arrays(gpu, maker):
         da.free()
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
+def test_structure_swapped_under_an_unanalysed_plan(gpu, dtype):
+    """Un-analysed calls remember row statistics per row_ptr address and pick the staged row-block kernel for
+    short rows.  Another matrix of the same m, n and nnz written over the arrays in place is multiplied with
+    those stale statistics: workgroups whose rows no longer fit the staging area must take them straight from
+    the arrays (the result is right whatever the statistics said), and nothing may be written out of bounds."""
+    lib = capi.load()
+    m, cols = 4096, 3000
+    a1 = csr_from_lengths([5] * m, cols, dtype)
+    lengths = np.zeros(m, dtype=np.int64)
+    lengths[0:6] = 3000
+    lengths[300:300 + 496] = 5
+    a2 = csr_from_lengths(list(lengths), cols, dtype, seed=11)
+    assert a1.nnz == a2.nnz == 5 * m
+    x, y0 = _vectors(a1)
+    da = DeviceCsr(a1)
+    try:
+        announce("structure swapped under a lazy plan", np.dtype(dtype).name, "first structure")
+        check_spmv(a1, 1.5, x, 0.5, y0, run_csrmv(gpu, da, 1.5, x, 0.5, y0), "first structure")
+        st = lib.asamd_analysis_stats(da.row_ptr.c_ptr()).contents
+        assert st.algo == capi.ASAMD_SPMV_STREAM and st.trusted == 0, capi.ALGO_NAMES[st.algo]
+        da.row_ptr.copy_from(a2.row_ptr)
+        da.col.copy_from(a2.col_ind)
+        da.val.copy_from(a2.values)
+        da.a = a2
+        announce("structure swapped under a lazy plan", np.dtype(dtype).name, "second structure, stale statistics")
+        check_spmv(a2, 1.5, x, 0.5, y0, run_csrmv(gpu, da, 1.5, x, 0.5, y0), "second structure")
+        st = lib.asamd_analysis_stats(da.row_ptr.c_ptr()).contents
+        assert st.algo == capi.ASAMD_SPMV_STREAM and st.max_len == 5, "the statistics were meant to be stale"
+    finally:
+        da.free()
+
+
 def test_lazy_analyses_are_bounded(gpu):
     """10 000 un-analysed matrices at distinct row_ptr addresses multiplied one after the other: the library
     remembers at most 64 lazy analyses (least recently used goes), device memory stays put, a matrix whose
