@@ -92,8 +92,8 @@ __global__ __launch_bounds__(kRowsBlock) void spmv_bin_rows_kernel(
       int c[4];
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        v[u] = nt_load(val + j + u * W);
-        c[u] = nt_load(col_ind + j + u * W);
+        v[u] = val[j + u * W];
+        c[u] = col_ind[j + u * W];
       }
       T xv[4];
 #pragma unroll
@@ -136,8 +136,8 @@ __global__ __launch_bounds__(kRowsBlock) void spmv_bin_chunk_kernel(
     int c[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-      v[u] = nt_load(val + j + u * kRowsBlock);
-      c[u] = nt_load(col_ind + j + u * kRowsBlock);
+      v[u] = val[j + u * kRowsBlock];
+      c[u] = col_ind[j + u * kRowsBlock];
     }
     T xv[4];
 #pragma unroll
