@@ -911,6 +911,15 @@ static hipError_t build_binned(hipStream_t stream, asamd_csr_plan* p, const int*
   return hipSuccess;
 }
 
+// Whether the structural choice has rivals that need no copy either (merge-path, a lane group per row): it has
+// when it is a lane group per row or a staged block with several lanes per row, merge-path can run (row_ptr
+// starts at the base) and the matrix is not so small that one launch's latency is all there is to time.
+static bool structural_alternatives(const asamd_csr_plan* p) {
+  const asamd_csr_stats& st = p->st;
+  if (st.first_offset != 0 || (int64_t)st.m + st.nnz <= kSmallWork) return false;
+  return p->auto_algo == ASAMD_SPMV_VECTOR || (p->auto_algo == ASAMD_SPMV_STREAM && stream_group(p, false) > 1);
+}
+
 // Time the structural choice on scratch vectors, then the copies that the matrix is eligible for:
 // the ELL copy (cheap to build), and the tiled copy only if the fastest so far is slower than the
 // tiled pair could possibly be.  Keep the fastest and free the copies that lost.  A copy has to win
@@ -958,18 +967,23 @@ static hipError_t tune_copies(hipStream_t stream, asamd_csr_plan* p, const int* 
   if ((double)st.max_len > 32.0 * ((double)st.nnz / (double)st.m) + 256.0) tiled_floor_ms *= 2.5f;
   if (e == hipSuccess) time_algo(0);
   // A lane group per row, or a staged block of rows with several lanes per row, was chosen from the mean and
-  // the longest row alone; merge-path takes any distribution and needs no copy either: the faster one stays.
-  if (e == hipSuccess && st.first_offset == 0 &&
-      (p->auto_algo == ASAMD_SPMV_VECTOR || (p->auto_algo == ASAMD_SPMV_STREAM && stream_group(p, false) > 1))) {
-    const float first = best[0];
-    best[0] = 0.f;
-    algos[0] = ASAMD_SPMV_MERGE;
-    time_algo(0);
-    if (e == hipSuccess && best[0] < 0.97f * first) {
-      p->auto_algo = p->struct_algo = ASAMD_SPMV_MERGE;
-    } else {
-      algos[0] = p->auto_algo;
-      best[0] = first;
+  // the longest row alone.  Neither needs a copy, nor does merge-path, which takes any distribution: the
+  // fastest of them stays.
+  if (e == hipSuccess && structural_alternatives(p)) {
+    int alts[2] = {ASAMD_SPMV_MERGE, p->auto_algo == ASAMD_SPMV_STREAM ? ASAMD_SPMV_VECTOR : -1};
+    for (int alt : alts) {
+      if (alt < 0 || e != hipSuccess) continue;
+      const float first = best[0];
+      const int kept = algos[0];
+      best[0] = 0.f;
+      algos[0] = alt;
+      time_algo(0);
+      if (e == hipSuccess && best[0] > 0.f && best[0] < 0.97f * first) {
+        p->auto_algo = p->struct_algo = alt;
+      } else {
+        algos[0] = kept;
+        best[0] = first;
+      }
     }
   }
   // An ELL copy gathers x row by row like the kernel just timed; when that one is several times slower
@@ -1133,7 +1147,7 @@ static hipError_t plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t 
         if (err == hipSuccess && ell_ok) err = build_ell<T>(stream, p, row_ptr, col_ind, (const T*)val);
         if (err == hipSuccess && hot_ok) err = build_hot<T>(stream, p, row_ptr, col_ind, true);
         p->copy_val_src = val;
-      } else if (tiled_ok || ell_ok || hot_ok || binned_ok) {
+      } else if (tiled_ok || ell_ok || hot_ok || binned_ok || structural_alternatives(p)) {
         err = tune_copies<T>(stream, p, row_ptr, col_ind, (const T*)val, tiled_ok, ell_ok, hot_ok, binned_ok);
       }
       return err;
