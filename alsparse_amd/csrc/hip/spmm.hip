@@ -35,6 +35,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdlib>
+#include <mutex>
 
 #include "alsparse_amd_kernels.h"
 #include "device_utils.hpp"
@@ -573,6 +574,85 @@ static bool colmajor_nn(const asamd_dense_strides* st, int n) {
   return n > 1 && st->b_row_stride == 1 && st->b_col_stride != 1 && st->c_row_stride == 1;
 }
 
+// ---- do neighbouring rows of A share columns? --------------------------------------------------
+// Stencils and finite-element matrices do (a row of B fetched for one row of A is wanted again by the next
+// rows), matrices with random columns do not, and which of the two row-major kernels is faster depends on it
+// (27-point stencil, n = 64: four rows of B per wave instruction 0.56 ms, one per instruction 0.88 ms; random
+// columns over a B of 64-256 MiB: 1.23 against 1.22 ms).  csrmm has no analysis call, so the first multiply of a
+// matrix looks: kProbeRows rows scattered over the matrix, the share of their entries (the first 64 of each) whose column is in
+// the next row as well.  One small kernel and one synchronisation, remembered per (row_ptr, col_ind, m, nnz);
+// not done while the stream is being captured.
+constexpr int kProbeRows = 2048;
+__global__ __launch_bounds__(256) void spmm_reuse_probe_kernel(int m, const int* __restrict__ row_ptr,
+                                                               const int* __restrict__ col_ind, int base,
+                                                               unsigned* __restrict__ out) {
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  if (t >= kProbeRows || m < 2) return;
+  // scattered rows: evenly spaced ones fall on the same position of every grid line of a stencil
+  const int64_t r = (int64_t)((((uint64_t)t + 1) * 0x9E3779B97F4A7C15ull >> 20) % (uint64_t)(m - 1));
+  const int64_t b0 = (int64_t)row_ptr[r] - base, e0 = (int64_t)row_ptr[r + 1] - base, e1 = (int64_t)row_ptr[r + 2] - base;
+  unsigned shared = 0, total = 0;
+  for (int64_t j = b0; j < e0 && j < b0 + 64; ++j) {
+    const int c = col_ind[j];
+    int64_t lo = e0, hi = e1;  // rows with unsorted columns simply count as sharing nothing
+    while (lo < hi) {
+      const int64_t mid = (lo + hi) >> 1;
+      if (col_ind[mid] < c) lo = mid + 1;
+      else hi = mid;
+    }
+    shared += (lo < e1 && col_ind[lo] == c) ? 1u : 0u;
+    ++total;
+  }
+  if (total) {
+    atomicAdd(&out[0], shared);
+    atomicAdd(&out[1], total);
+  }
+}
+
+static bool rows_share_columns(hipStream_t s, int m, int nnz, const int* rp, const int* ci, int base) {
+  struct Seen {
+    const int *rp, *ci;
+    int m, nnz;
+    bool shares;
+  };
+  constexpr int kSeen = 16, kMaxDevices = 64;
+  static std::mutex lock;
+  static Seen seen[kSeen];
+  static int next = 0;
+  static unsigned* d_out[kMaxDevices];
+  std::lock_guard<std::mutex> guard(lock);
+  for (const Seen& e : seen)
+    if (e.rp == rp && e.ci == ci && e.m == m && e.nnz == nnz) return e.shares;
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(s, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
+    (void)hipGetLastError();
+    return false;
+  }
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return false;
+  if (!d_out[dev] && hipMalloc(&d_out[dev], 2 * sizeof(unsigned)) != hipSuccess) {
+    (void)hipGetLastError();
+    d_out[dev] = nullptr;
+    return false;
+  }
+  unsigned h_out[2] = {0, 0};
+  bool ok = hipMemsetAsync(d_out[dev], 0, sizeof(h_out), s) == hipSuccess;
+  if (ok) {
+    spmm_reuse_probe_kernel<<<kProbeRows / 256, 256, 0, s>>>(m, rp, ci, base, d_out[dev]);
+    ok = hipGetLastError() == hipSuccess &&
+         hipMemcpyAsync(h_out, d_out[dev], sizeof(h_out), hipMemcpyDeviceToHost, s) == hipSuccess &&
+         hipStreamSynchronize(s) == hipSuccess;
+  }
+  if (!ok) {
+    (void)hipGetLastError();
+    return false;
+  }
+  const bool shares = h_out[1] > 0 && 4ull * h_out[0] >= (unsigned long long)h_out[1];
+  seen[next] = Seen{rp, ci, m, nnz, shares};
+  next = (next + 1) % kSeen;
+  return shares;
+}
+
 static size_t workspace_bytes(size_t val_size, int n, int k, const asamd_dense_strides* st) {
   if (!st || n <= 0 || k <= 0 || !colmajor_nn(st, n)) return 0;
   return (((size_t)k * (size_t)n * val_size) + 255) & ~(size_t)255;
@@ -632,13 +712,16 @@ static int csrmm_impl(hipStream_t s, int m, int n, int k, int nnz, T alpha, cons
       // rows of B and C that 128-bit loads can address: four rows of B per wave instruction
       constexpr int E = 16 / (int)sizeof(T);
       static const bool quad_off = getenv("ALSPARSE_AMD_SPMM_QUAD") && atoi(getenv("ALSPARSE_AMD_SPMM_QUAD")) == 0;
-      // Measured on 2^20 rows x 32 entries, n = 64, against one wave-wide load per row of B: B of 4 / 16 / 32 MiB
-      // 0.64 / 0.95 / 1.10 ms against 0.97 / 1.05 / 1.11; 64-256 MiB 1.18-1.23 against 1.17-1.22 (the L2-miss
-      // path is the limit either way); 512 MiB 1.22 against 1.38; n = 256 (1 GiB) 4.95 against 5.46.
+      // Measured on 2^20 rows x 32 entries with random columns, n = 64, against one wave-wide load per row of B: B of
+      // 4 / 16 / 32 MiB 0.64 / 0.95 / 1.10 ms against 0.97 / 1.05 / 1.11; 64-256 MiB 1.18-1.23 against 1.17-1.22 (the
+      // L2-miss path is the limit either way); 512 MiB 1.22 against 1.38; n = 256 (1 GiB) 4.95 against 5.46.  Where
+      // neighbouring rows of A share their columns the four-row form wins at any footprint (see above).
       const size_t b_bytes = (size_t)(k > 0 ? k : 0) * (size_t)n * sizeof(T);
-      const bool quad_pays = k <= 0 || b_bytes <= ((size_t)48 << 20) || b_bytes > ((size_t)384 << 20);
-      if (!quad_off && quad_pays && n % E == 0 && ldb % E == 0 && ldc % E == 0 && (uintptr_t)B % 16 == 0 &&
-          (uintptr_t)C % 16 == 0) {
+      const bool eligible = !quad_off && n % E == 0 && ldb % E == 0 && ldc % E == 0 && (uintptr_t)B % 16 == 0 &&
+                            (uintptr_t)C % 16 == 0;
+      const bool quad_pays = eligible && (k <= 0 || b_bytes <= ((size_t)48 << 20) || b_bytes > ((size_t)384 << 20) ||
+                                          rows_share_columns(s, m, nnz, rp, ci, base));
+      if (quad_pays) {
         const dim3 grid(gx, (unsigned)((n + 16 * E - 1) / (16 * E)));
         spmm_rowmajor_quad_kernel<T><<<grid, kSpmmBlock, 0, s>>>(m, n, alpha, val, rp, ci, base, B, ldb, beta, C, ldc);
         return hipGetLastError();

@@ -459,11 +459,23 @@ def run_format_spmv(cfg, fmt, steps, warmup, check):
     return res
 
 
-def run_spmm(steps, warmup, check, col_major=False, vendor=False):
+def run_spmm(steps, warmup, check, col_major=False, vendor=False, stencil=None, dense_cols=None):
+    """stencil = (nx, ny, nz): instead of configuration 5's matrix, the 27-point stencil on that grid times a
+    random dense matrix of dense_cols (default 64) columns."""
     from alsparse_amd import capi, hiprt, workloads as wl
     lib = capi.load()
-    a, B, C0, alpha, beta, extra = wl.config(5)
-    n = extra["n"]
+    if stencil:
+        a = wl.stencil3d(stencil[0], stencil[1], stencil[2], np.float32)
+        n = dense_cols or 64
+        B = wl.uniform(a.cols * n, np.float32, 3).reshape(a.cols, n)
+        C0 = wl.uniform(a.rows * n, np.float32, 4).reshape(a.rows, n)
+        alpha, beta = 1.0, 0.0
+    else:
+        a, B, C0, alpha, beta, extra = wl.config(5)
+        n = dense_cols or extra["n"]
+        if n != extra["n"]:
+            B = wl.uniform(a.cols * n, np.float32, 3).reshape(a.cols, n)
+            C0 = wl.uniform(a.rows * n, np.float32, 4).reshape(a.rows, n)
     h = capi.Handle()
     descr = capi.make_descr()
     from ctypes import c_float
@@ -498,7 +510,12 @@ def run_spmm(steps, warmup, check, col_major=False, vendor=False):
         d_C.copy_from(C_dev)
     t = time_steps(step, steps, warmup, hiprt)
     nbytes = wl.spmm_bytes(a.rows, a.cols, n, a.nnz, 4, beta)
-    res = {"workload": WORKLOAD_NAMES[5].replace("row-major", "column-major") if col_major else WORKLOAD_NAMES[5],
+    wname = WORKLOAD_NAMES[5] if not stencil else (
+        "27-point stencil SpMM: CSR fp32 %d x %d x %d grid (%d rows, %d nnz) times dense %d x %d row-major, alpha=1 beta=0"
+        % (stencil[0], stencil[1], stencil[2], a.rows, a.nnz, a.cols, n))
+    if not stencil and n != 64:
+        wname += " -- with %d dense columns" % n
+    res = {"workload": wname.replace("row-major", "column-major") if col_major else wname,
            "kernel": "spmm column-major (B transposed into scratch)" if col_major else "spmm row-major", "rows": a.rows, "nnz": a.nnz, "algorithmic_bytes": int(nbytes),
            "gather_upper_bound_bytes": int(a.nnz) * n * 4, "flops": 2 * a.nnz * n, "timing": t,
            "gbs": nbytes / t["avg_ms"] / 1e6, "gflops": 2 * a.nnz * n / t["avg_ms"] / 1e6, "dtype": "f32",
@@ -610,6 +627,8 @@ def main():
                          "and the others SHORT (the workload of the row-length bins)")
     ap.add_argument("--stencil3d", nargs=3, type=int, metavar=("NX", "NY", "NZ"),
                     help="instead of a configuration: the 27-point stencil on an NX x NY x NZ grid (8 to 27 entries per row)")
+    ap.add_argument("--dense-cols", type=int, default=None, metavar="N",
+                    help="with --config 5: N dense columns instead of 64 (with --stencil3d too: the stencil as the sparse matrix)")
     ap.add_argument("--fp64", action="store_true", help="with --uniform / --bimodal / --stencil3d: fp64 values")
     ap.add_argument("--all", action="store_true", help="also measure the other configurations")
     ap.add_argument("--only", action="store_true",
@@ -671,7 +690,8 @@ def main():
             sys.exit("bench.py: --format ell|coo is measured on configuration 2 or 3")
         main_res = run_format_spmv(args.config, args.format, args.steps, args.warmup, check)
     elif args.config == 5:
-        main_res = run_spmm(args.steps, args.warmup, check, args.col_major, not args.no_vendor_baseline)
+        main_res = run_spmm(args.steps, args.warmup, check, args.col_major, not args.no_vendor_baseline,
+                            args.stencil3d, args.dense_cols)
     else:
         cfg = args.config
         if args.uniform:

@@ -68,6 +68,27 @@ def test_row_major(gpu, mat, n, dtype):
             da.free()
 
 
+@pytest.mark.parametrize("maker", [lambda: wl.stencil3d(64, 60, 56, np.float32), lambda: wl.uniform_rows(215040, 215040, 12, np.float32)],
+                         ids=["stencil", "random_columns"])
+def test_row_major_operand_of_the_middle_sizes(gpu, maker):
+    """A dense operand of 48 to 384 MiB: which row-major kernel runs is decided by a look at the matrix (do
+    neighbouring rows share columns?) on the first multiply.  Both answers, twice each (the second multiply
+    reuses the first one's answer), against the oracle."""
+    a = maker()
+    n = 64
+    assert 48 << 20 < a.cols * n * 4 <= 384 << 20
+    B = wl.uniform(a.cols * n, np.float32, 5).reshape(a.cols, n)
+    C0 = wl.uniform(a.rows * n, np.float32, 6).reshape(a.rows, n)
+    da = DeviceCsr(a)
+    try:
+        for rep in range(2):
+            announce("spmm row-major, operand of the middle sizes", a.name, rep)
+            C = run_csrmm(gpu, da, capi.ALPHA_SPARSE_LAYOUT_ROW_MAJOR, 0, 1.25, B, n, 0.5, C0, n, n, a.cols)
+            check(a, 1.25, B, 0.5, C0, C.reshape(a.rows, n), "%s rep %d" % (a.name, rep))
+    finally:
+        da.free()
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
 @pytest.mark.parametrize("n", [1, 5, 64, 70])
 def test_column_major_and_transposed_b(gpu, n, dtype):
