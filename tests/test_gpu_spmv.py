@@ -62,6 +62,53 @@ def test_every_kernel_family_matches_oracle(gpu, shape, dtype):
         da.free()
 
 
+def _random_structure(rng, dtype):
+    """A seeded random CSR structure: row count, column count, a row-length law (constant, narrow band, wide band,
+    geometric with some empty rows, a few very long rows among short ones), index base and the element offset of
+    val / col_ind inside their allocations."""
+    m = int(rng.integers(1, 3000))
+    cols = int(rng.integers(1, 5000))
+    law = int(rng.integers(0, 5))
+    if law == 0:
+        lengths = np.full(m, int(rng.integers(1, 70)))
+    elif law == 1:
+        lo = int(rng.integers(1, 120))
+        lengths = rng.integers(lo, lo + int(rng.integers(1, 12)) + 1, size=m)
+    elif law == 2:
+        lengths = rng.integers(0, int(rng.integers(2, 300)) + 1, size=m)
+    elif law == 3:
+        lengths = rng.geometric(1.0 / float(rng.integers(2, 30)), size=m) - 1
+    else:
+        lengths = rng.integers(0, 6, size=m)
+        lengths[rng.integers(0, m, size=max(1, m // 200))] = int(rng.integers(300, 4500))
+    base = int(rng.integers(0, 2))
+    a = csr_from_lengths(list(np.minimum(lengths, cols)), cols, dtype, seed=int(rng.integers(1, 1 << 30)), base=base)
+    return a, int(rng.integers(0, 4))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
+@pytest.mark.parametrize("seed", range(24))
+def test_random_structures_every_family(gpu, seed, dtype):
+    rng = np.random.default_rng(1000 + seed)
+    a, shift = _random_structure(rng, dtype)
+    if a.nnz == 0:
+        pytest.skip("drew a matrix without entries")
+    x, y0 = _vectors(a)
+    da = DeviceCsr(a, shift=shift)
+    try:
+        for algo in ("vector", "merge", "scalar", "rowconst", "stream", "tiled", "ell", "binned", "auto"):
+            alpha, beta = ((1.0, 0.0), (2.0, 3.0), (-0.75, 1.0))[int(rng.integers(0, 3))]
+            announce("spmv random structure", seed, a.name, "base", a.base, "shift", shift, np.dtype(dtype).name, algo, alpha, beta)
+            y = run_plan_csrmv(da, algo, alpha, x, beta, y0)
+            if y is None:
+                continue
+            check_spmv(a, alpha, x, beta, y0, y, "seed %d/%s/%s" % (seed, algo, (alpha, beta)))
+        y = run_csrmv(gpu, da, 1.5, x, 0.25, y0)
+        check_spmv(a, 1.5, x, 0.25, y0, y, "seed %d/api without analysis" % seed)
+    finally:
+        da.free()
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
 @pytest.mark.parametrize("shift", [1, 3], ids=["shift1", "shift3"])
 def test_streams_off_16_byte_alignment(gpu, dtype, shift):
