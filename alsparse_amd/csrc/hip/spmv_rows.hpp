@@ -7,9 +7,11 @@
 //                               row*4*G: no row_ptr traffic, one 128-bit load of
 //                               values and one of indices per lane.
 //   spmv_scalar_kernel<T>       one lane per row (diagnostic baseline).
-//   spmv_stream_kernel<T>       rows of at most 16 entries: a workgroup stages the
-//                               products of 256 consecutive rows in LDS, one lane
-//                               per row sums them.
+//   spmv_stream_wide_kernel<T, CAP, G>, spmv_stream_kernel<T, CAP, G>
+//                               rows of similar lengths, at most CAP * G entries: a workgroup
+//                               stages the products of 256 / G consecutive rows in LDS (their
+//                               entries are one contiguous range, read with 128-bit or 4-byte
+//                               loads), G lanes per row sum them.
 //
 // They stand in for the reference's only CSR SpMV kernel, csr_gemv_vector
 // (src/kernel/dcu/level2/mv/csrmv/dcu_gemv_vector.h:14-57): same arithmetic

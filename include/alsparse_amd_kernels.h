@@ -35,7 +35,8 @@ enum asamd_spmv_algo {
   ASAMD_SPMV_SCALAR = 4,   /* one lane per row; diagnostic baseline                  */
   ASAMD_SPMV_TILED = 5,    /* two-phase, (column block x row block) tiles: every x
                               gather and y update in LDS, HBM sees only streams     */
-  ASAMD_SPMV_STREAM = 6,   /* rows of <= 16 entries: 256 rows' products staged in LDS */
+  ASAMD_SPMV_STREAM = 6,   /* rows of similar lengths (<= 256 entries): a row block's
+                              products staged in LDS, 1..16 lanes sum a row          */
   ASAMD_SPMV_ELL = 7,      /* short, nearly equal rows: a column-major ELL copy, one
                               lane per row                                          */
   ASAMD_SPMV_MERGE_HOT = 8, /* merge-path whose persistent workgroups keep x of the most
