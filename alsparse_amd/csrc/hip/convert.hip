@@ -249,7 +249,10 @@ extern "C" int asamd_csr2ell_width(hipStream_t stream, int32_t m, const int32_t*
 constexpr int kEllRows = 256;
 constexpr int kEllWindow = 4096;  // staged entries per workgroup pass (half of it for 16-byte values)
 
-template <typename T, bool NTS>
+// WIDE: val and col_ind are 16-byte aligned; the staged range is then read as pieces of four entries from the
+// multiple of four at or before its start (a quarter of the load instructions); pieces that would reach past
+// the end of the arrays -- in the last workgroup only -- are read entry by entry.
+template <typename T, bool NTS, bool WIDE>
 __global__ __launch_bounds__(kEllRows) void csr2ell_kernel(
     int m, const T* __restrict__ val, const int* __restrict__ row_ptr,
     const int* __restrict__ col_ind, int csr_base, int ell_base, int width,
@@ -272,7 +275,53 @@ __global__ __launch_bounds__(kEllRows) void csr2ell_kernel(
     my_end = (int64_t)row_ptr[row + 1] - csr_base;
   }
   const bool staged = blk_end - blk_begin <= kWindow;  // workgroup-uniform
-  if (staged) {
+  if (staged && WIDE) {
+    const int count = (int)(blk_end - blk_begin);
+    const int64_t limit = (int64_t)row_ptr[m] - csr_base;  // entries in the arrays
+    const int64_t a0 = blk_begin & ~(int64_t)3;
+    const int head = (int)(blk_begin - a0);
+    const int span = count + head;
+    constexpr int kU = 4;  // pieces of each stream in flight per thread before the first LDS write
+    for (int p0 = 4 * threadIdx.x; p0 < span; p0 += 4 * kU * kEllRows) {
+      Quad<T> v[kU];
+      Int4 c[kU];
+#pragma unroll
+      for (int u = 0; u < kU; ++u) {
+        const int k = p0 + u * 4 * kEllRows;
+        if (k < span) {
+          if (a0 + k + 4 <= limit) {
+            v[u].load(val + a0 + k);
+            c[u] = *reinterpret_cast<const Int4*>(col_ind + a0 + k);
+          } else {
+            alignas(32) T tv[4] = {T(0), T(0), T(0), T(0)};
+            int tc[4] = {0, 0, 0, 0};
+            for (int j = 0; j < 4 && a0 + k + j < limit; ++j) {
+              tv[j] = val[a0 + k + j];
+              tc[j] = col_ind[a0 + k + j];
+            }
+            v[u].load(tv);
+            c[u] = Int4{tc[0], tc[1], tc[2], tc[3]};
+          }
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kU; ++u) {
+        const int k = p0 + u * 4 * kEllRows;
+        if (k < span) {
+          const int cc[4] = {c[u].x, c[u].y, c[u].z, c[u].w};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int p = k + j - head;
+            if (p >= 0 && p < count) {
+              s_val[at(p)] = v[u].get(j);
+              s_col[at(p)] = cc[j];
+            }
+          }
+        }
+      }
+    }
+    __syncthreads();
+  } else if (staged) {
     // eight loads of each stream in flight per thread before the first LDS write: a load-wait-write
     // loop pays the memory latency once per trip
     constexpr int kU = 8;
@@ -331,10 +380,15 @@ static int csr2ell_impl(hipStream_t stream, int m, const T* val, const int* rp, 
   if (((uintptr_t)val | (uintptr_t)ell_val) % alignof(T)) return hipErrorInvalidValue;
   if (width == 0) return hipSuccess;
   const unsigned grid = (unsigned)(((int64_t)m + kEllRows - 1) / kEllRows);
-  if (stores_bypass_caches((size_t)m * (size_t)width * (sizeof(T) + sizeof(int))))
-    csr2ell_kernel<T, true><<<grid, kEllRows, 0, stream>>>(m, val, rp, ci, csr_base, ell_base, width, ell_val, ell_col);
-  else
-    csr2ell_kernel<T, false><<<grid, kEllRows, 0, stream>>>(m, val, rp, ci, csr_base, ell_base, width, ell_val, ell_col);
+  const bool nts = stores_bypass_caches((size_t)m * (size_t)width * (sizeof(T) + sizeof(int)));
+  const bool wide = (((uintptr_t)val | (uintptr_t)ci) & 15u) == 0;
+#define ASAMD_CSR2ELL(NTS, WIDE) \
+  csr2ell_kernel<T, NTS, WIDE><<<grid, kEllRows, 0, stream>>>(m, val, rp, ci, csr_base, ell_base, width, ell_val, ell_col)
+  if (nts && wide) ASAMD_CSR2ELL(true, true);
+  else if (nts) ASAMD_CSR2ELL(true, false);
+  else if (wide) ASAMD_CSR2ELL(false, true);
+  else ASAMD_CSR2ELL(false, false);
+#undef ASAMD_CSR2ELL
   return hipGetLastError();
 }
 
