@@ -33,6 +33,9 @@ SHAPES = {
                                                   20000, rd),
     "base_one": lambda rd: wl.uniform_rows(3000, 2500, 7, rd, base=1),
     "tiny": lambda rd: csr_from_lengths([2, 0, 1], 5, rd),
+    # rows of similar lengths: the staged row-block kernel with several lanes per row
+    "stencil27": lambda rd: wl.stencil3d(14, 11, 9, rd),
+    "regular_40_60": lambda rd: csr_from_lengths(list(40 + (np.arange(1200) * 7) % 21), 3000, rd, base=1),
 }
 
 
@@ -122,7 +125,7 @@ def test_complex_kernel_families(gpu, dtype, algo):
     lib = capi.load()
     T, p = capi.scalar_type(dtype), capi.prefix(dtype)
     ran = 0
-    for shape in ("uniform16", "powerlaw", "laplace", "long_and_empty", "base_one", "tiny"):
+    for shape in ("uniform16", "powerlaw", "laplace", "long_and_empty", "base_one", "tiny", "stencil27", "regular_40_60"):
         a = make(shape, dtype)
         x, y0 = complex_vector(a.cols, dtype, 3), complex_vector(a.rows, dtype, 4)
         da = DeviceCsr(a)
