@@ -20,6 +20,7 @@
 
 #include "alsparse_amd_kernels.h"
 #include "spmv_ell.hpp"
+#include "stream_policy.hpp"
 #include "spmv_binned.hpp"
 #include "spmv_hot.hpp"
 #include "spmv_merge.hpp"
@@ -1422,6 +1423,12 @@ extern "C" int asamd_csr_plan_set_algo(asamd_csr_plan* p, int32_t algo) {
   }
 }
 
+// the cache policy of a CSR multiply's streams (stream_policy.hpp) from the plan's statistics
+static int stream_policy(const asamd_csr_stats& st, size_t val_size) {
+  return asamd::stream_policy((double)st.nnz, val_size,
+                              ((double)st.m + 1.0) * 4.0 + ((double)st.m + (double)st.n) * (double)val_size);
+}
+
 // ---------------------------------------------------------------------------
 template <typename T, int W>
 static void launch_vector(hipStream_t s, const asamd_csr_stats& st, T alpha, const T* val,
@@ -1437,7 +1444,8 @@ static void launch_rowconst(hipStream_t s, const asamd_csr_stats& st, T alpha, c
   constexpr int R = G >= 16 ? 1 : 2;
   constexpr int rows_per_block = (kRowsBlock / G) * R;
   const unsigned grid = (unsigned)(((int64_t)st.m + rows_per_block - 1) / rows_per_block);
-  spmv_rowconst_kernel<T, G, R><<<grid, kRowsBlock, 0, s>>>(st.m, alpha, val, ci, x, beta, y, st.base);
+  spmv_rowconst_kernel<T, G, R><<<grid, kRowsBlock, 0, s>>>(st.m, alpha, val, ci, x, beta, y, st.base,
+                                                            stream_policy(st, sizeof(T)));
 }
 
 template <typename T>
@@ -1472,8 +1480,17 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
       if constexpr (sizeof(T) <= 8) {
         if (st.m % 2 == 0) {  // the copy is the library's own (256-byte aligned): row pairs are aligned when m is even
           const unsigned grid2 = (unsigned)(((int64_t)st.m / 2 + kEllThreads - 1) / kEllThreads);
-          ellmv_multi_kernel<T, 2><<<grid2, kEllThreads, 0, s>>>(st.m, st.n, alpha, (const T*)p->d_eval, p->d_ecol,
-                                                                 st.ell_width, 0, x, beta, y);
+          // the ELL copy's streams: m * width slots of values and of indices
+          const int policy = asamd::stream_policy((double)st.m * st.ell_width, sizeof(T),
+                                                  ((double)st.m + (double)st.n) * (double)sizeof(T));
+#define ASAMD_ELL_LAUNCH(NTV, NTC)                                                                                  \
+  ellmv_multi_kernel<T, 2, NTV, NTC><<<grid2, kEllThreads, 0, s>>>(st.m, st.n, alpha, (const T*)p->d_eval, p->d_ecol, \
+                                                                   st.ell_width, 0, x, beta, y)
+          if (policy == 0) ASAMD_ELL_LAUNCH(false, false);
+          else if (policy == kStreamNtValues) ASAMD_ELL_LAUNCH(true, false);
+          else if (policy == kStreamNtIndices) ASAMD_ELL_LAUNCH(false, true);
+          else ASAMD_ELL_LAUNCH(true, true);
+#undef ASAMD_ELL_LAUNCH
           break;
         }
       }
@@ -1540,7 +1557,7 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
   do {                                                                                                                   \
     if (wide)                                                                                                            \
       spmv_stream_wide_kernel<T, CAP, G><<<grid, kStreamRows, 0, s>>>(st.m, alpha, val, rp, ci, x, beta, y, st.base,    \
-                                                                      limit);                                           \
+                                                                      limit, stream_policy(st, sizeof(T)));             \
     else                                                                                                                 \
       spmv_stream_kernel<T, CAP, G><<<grid, kStreamRows, 0, s>>>(st.m, alpha, val, rp, ci, x, beta, y, st.base);        \
   } while (0)
@@ -1632,7 +1649,8 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
     if (merge_wide && (IPT) % 4 == 0)                                                                            \
       spmv_merge_kernel<T, IPT, true><<<nb, kMergeThreads, 0, s>>>(st.m, st.nnz, alpha, val, rp, ci, x, beta, y, \
                                                                    st.base, p->d_block_row, p->d_carry_row,      \
-                                                                   (T*)p->d_carry_val, (T*)p->d_head_val);       \
+                                                                   (T*)p->d_carry_val, (T*)p->d_head_val,        \
+                                                                   stream_policy(st, sizeof(T)));                \
     else                                                                                                         \
       spmv_merge_kernel<T, IPT><<<nb, kMergeThreads, 0, s>>>(st.m, st.nnz, alpha, val, rp, ci, x, beta, y,       \
                                                              st.base, p->d_block_row, p->d_carry_row,            \

@@ -54,7 +54,8 @@ __global__ __launch_bounds__(kEllThreads) void ellmv_kernel(int m, int n, T alph
 // 16 / 8 bytes per lane instead of 8 / 4): 1 / R as many memory instructions for the same bytes.  Measured on
 // the 5-point Laplacian of 4 M rows, fp64 (one row per lane, both streams non-temporal: 56.0 us): R = 2 with
 // the indices non-temporal and the values not 50.0 us, both non-temporal 53.4, values only 51.6, neither
-// 59.3; R = 1 with that mix 54.4; R = 4 65.5 (too few lanes in flight).
+// 59.3; R = 1 with that mix 54.4; R = 4 65.5 (too few lanes in flight).  NTV / NTC: which stream bypasses the
+// caches; the launch picks them from the sizes of the streams (stream_policy.hpp).
 template <typename T, int R, bool NTV = false, bool NTC = true>
 __global__ __launch_bounds__(kEllThreads) void ellmv_multi_kernel(int m, int n, T alpha,
                                                                   const T* __restrict__ ell_val,

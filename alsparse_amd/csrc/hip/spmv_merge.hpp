@@ -83,7 +83,7 @@ __global__ __launch_bounds__(kMergeThreads) void spmv_merge_kernel(
     int m, int nnz, T alpha, const T* __restrict__ val, const int* __restrict__ row_ptr,
     const int* __restrict__ col_ind, const T* __restrict__ x, T beta, T* __restrict__ y, int base,
     const int* __restrict__ block_row, int* __restrict__ carry_row, T* __restrict__ carry_val,
-    T* __restrict__ head_val) {
+    T* __restrict__ head_val, int policy = kStreamNtValues | kStreamNtIndices) {
   constexpr int kItems = kMergeThreads * IPT;
   __shared__ int s_rend[kItems + 1];  // row ends, local to this workgroup's entry range
   __shared__ T s_prod[kItems + kItems / 32 + 1];
@@ -133,8 +133,10 @@ __global__ __launch_bounds__(kMergeThreads) void spmv_merge_kernel(
     for (int s = 0; s < kPieces; ++s) {
       const int k = 4 * (tid + s * kMergeThreads);
       const int64_t kk = win0 + (k < span ? k : 0);
-      v[s].load_nt(val + kk);
-      c[s] = nt_load_object(reinterpret_cast<const Int4*>(col_ind + kk));
+      if (policy & kStreamNtValues) v[s].load_nt(val + kk);
+      else v[s].load(val + kk);
+      if (policy & kStreamNtIndices) c[s] = nt_load_object(reinterpret_cast<const Int4*>(col_ind + kk));
+      else c[s] = *reinterpret_cast<const Int4*>(col_ind + kk);
     }
     T xv[kPieces][4];
 #pragma unroll

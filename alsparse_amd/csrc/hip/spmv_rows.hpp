@@ -98,8 +98,8 @@ __global__ __launch_bounds__(kRowsBlock) void spmv_scalar_kernel(
 // what rows of 3-5 entries (stencils, G = 1) want, and with G = 2 .. 16 rows of some tens of
 // entries whose lengths differ too little to need merge-path (a lane group per row straight from
 // global memory has three dependent loads per row and few of them in flight).
-// The indices are loaded non-temporally, the values not: measured on 4 M - 8 M rows of 5 entries,
-// 21 % (fp64 stencil), 17 % (fp32) and 3 % (fp64, random columns) faster than both plain.
+// Which stream bypasses the caches is the host's choice (the wide form's `policy`, see stream_policy.hpp);
+// the 4-byte form loads its indices non-temporally and its values plainly.
 constexpr int kStreamRows = 256;
 constexpr int kStreamMaxLen = 16;        // longest row of the one-lane-per-row form
 constexpr int kStreamMaxGroup = 16;      // most lanes per row
@@ -178,7 +178,8 @@ __global__ __launch_bounds__(kStreamRows) void spmv_stream_kernel(
 template <typename T, int CAP, int G>
 __global__ __launch_bounds__(kStreamRows) void spmv_stream_wide_kernel(
     int m, T alpha, const T* __restrict__ val, const int* __restrict__ row_ptr,
-    const int* __restrict__ col_ind, const T* __restrict__ x, T beta, T* __restrict__ y, int base, int64_t limit) {
+    const int* __restrict__ col_ind, const T* __restrict__ x, T beta, T* __restrict__ y, int base, int64_t limit,
+    int policy) {
   constexpr int kRows = kStreamRows / G;
   constexpr int kPieces = CAP / 4 + 1;
   __shared__ T s_prod[kStreamRows * CAP];
@@ -213,8 +214,10 @@ __global__ __launch_bounds__(kStreamRows) void spmv_stream_wide_kernel(
     const int k = 4 * (threadIdx.x + s * kStreamRows);
     if (k < span) {
       if (a0 + k + 4 <= limit) {
-        v[s].load(val + a0 + k);
-        c[s] = nt_load_object(reinterpret_cast<const Int4*>(col_ind + a0 + k));
+        if (policy & kStreamNtValues) v[s].load_nt(val + a0 + k);
+        else v[s].load(val + a0 + k);
+        if (policy & kStreamNtIndices) c[s] = nt_load_object(reinterpret_cast<const Int4*>(col_ind + a0 + k));
+        else c[s] = *reinterpret_cast<const Int4*>(col_ind + a0 + k);
       } else {
         // the arrays end inside this piece
         alignas(32) T tv[4] = {T(0), T(0), T(0), T(0)};
@@ -255,7 +258,7 @@ __global__ __launch_bounds__(kStreamRows) void spmv_stream_wide_kernel(
 template <typename T, int G, int R>
 __global__ __launch_bounds__(kRowsBlock) void spmv_rowconst_kernel(
     int m, T alpha, const T* __restrict__ val, const int* __restrict__ col_ind,
-    const T* __restrict__ x, T beta, T* __restrict__ y, int base) {
+    const T* __restrict__ x, T beta, T* __restrict__ y, int base, int policy) {
   constexpr int kGroups = kRowsBlock / G;  // lane groups per workgroup
   constexpr int L = 4 * G;
   const unsigned bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
@@ -271,11 +274,11 @@ __global__ __launch_bounds__(kRowsBlock) void spmv_rowconst_kernel(
     const int64_t row = row0 + (int64_t)r * kGroups;
     if (row < m) {
       const int64_t off = row * L + lane * 4;
-      // cache policy as measured (4 M - 8 M rows of 8 or 16 entries, x in the L1, an L2 or beyond): the
-      // indices non-temporal gains up to 6 %; the values too for 4-byte types (5 % more), not for 8-byte ones
-      if constexpr (sizeof(T) == 4) v[r].load_nt(val + off);
+      // policy (kernel-uniform): which stream bypasses the caches, see kStreamNt*
+      if (policy & kStreamNtValues) v[r].load_nt(val + off);
       else v[r].load(val + off);
-      c[r] = nt_load_object(reinterpret_cast<const Int4*>(col_ind + off));
+      if (policy & kStreamNtIndices) c[r] = nt_load_object(reinterpret_cast<const Int4*>(col_ind + off));
+      else c[r] = *reinterpret_cast<const Int4*>(col_ind + off);
     }
   }
   T xs[R][4];
