@@ -1424,9 +1424,9 @@ extern "C" int asamd_csr_plan_set_algo(asamd_csr_plan* p, int32_t algo) {
 }
 
 // the cache policy of a CSR multiply's streams (stream_policy.hpp) from the plan's statistics
-static int stream_policy(const asamd_csr_stats& st, size_t val_size) {
+static int stream_policy(const asamd_csr_stats& st, size_t val_size, bool wide_both = false) {
   return asamd::stream_policy((double)st.nnz, val_size,
-                              ((double)st.m + 1.0) * 4.0 + ((double)st.m + (double)st.n) * (double)val_size);
+                              ((double)st.m + 1.0) * 4.0 + ((double)st.m + (double)st.n) * (double)val_size, wide_both);
 }
 
 // ---------------------------------------------------------------------------
@@ -1482,7 +1482,7 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
           const unsigned grid2 = (unsigned)(((int64_t)st.m / 2 + kEllThreads - 1) / kEllThreads);
           // the ELL copy's streams: m * width slots of values and of indices
           const int policy = asamd::stream_policy((double)st.m * st.ell_width, sizeof(T),
-                                                  ((double)st.m + (double)st.n) * (double)sizeof(T));
+                                                  ((double)st.m + (double)st.n) * (double)sizeof(T), true);
 #define ASAMD_ELL_LAUNCH(NTV, NTC)                                                                                  \
   ellmv_multi_kernel<T, 2, NTV, NTC><<<grid2, kEllThreads, 0, s>>>(st.m, st.n, alpha, (const T*)p->d_eval, p->d_ecol, \
                                                                    st.ell_width, 0, x, beta, y)
@@ -1650,7 +1650,7 @@ static int csrmv_impl(hipStream_t s, asamd_csr_plan* p, T alpha, const T* val, c
       spmv_merge_kernel<T, IPT, true><<<nb, kMergeThreads, 0, s>>>(st.m, st.nnz, alpha, val, rp, ci, x, beta, y, \
                                                                    st.base, p->d_block_row, p->d_carry_row,      \
                                                                    (T*)p->d_carry_val, (T*)p->d_head_val,        \
-                                                                   stream_policy(st, sizeof(T)));                \
+                                                                   stream_policy(st, sizeof(T), true));          \
     else                                                                                                         \
       spmv_merge_kernel<T, IPT><<<nb, kMergeThreads, 0, s>>>(st.m, st.nnz, alpha, val, rp, ci, x, beta, y,       \
                                                              st.base, p->d_block_row, p->d_carry_row,            \

@@ -162,7 +162,7 @@ int ellmv_impl(hipStream_t stream, int32_t m, int32_t n, T alpha, const T* ell_v
     // two rows per lane where the caller's arrays allow aligned pairs
     if (m % 2 == 0 && (uintptr_t)ell_val % (2 * sizeof(T)) == 0 && (uintptr_t)ell_col % 8 == 0) {
       const unsigned grid2 = (unsigned)(((int64_t)m / 2 + kEllThreads - 1) / kEllThreads);
-      const int policy = stream_policy((double)m * width, sizeof(T), ((double)m + (double)n) * (double)sizeof(T));
+      const int policy = stream_policy((double)m * width, sizeof(T), ((double)m + (double)n) * (double)sizeof(T), true);
 #define ASAMD_ELL_LAUNCH(NTV, NTC) \
   ellmv_multi_kernel<T, 2, NTV, NTC><<<grid2, kEllThreads, 0, stream>>>(m, n, alpha, ell_val, ell_col, width, base, x, beta, y)
       if (policy == 0) ASAMD_ELL_LAUNCH(false, false);

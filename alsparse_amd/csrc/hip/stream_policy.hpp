@@ -14,8 +14,9 @@
 //   27-point stencil 160^3, fp32 (437 + 437 MB)          208.5  206.3  205.8  198.7
 //   27-point stencil 128^3, fp64 (446 + 223 MB)          148.6  149.8  147.4  162.7
 //   power-law, 8 M rows, fp32 (379 + 379 MB)             595.8  583.0  582.6  567.3
-// Both streams non-temporal pays only with 4-byte values.  What is not a matrix stream (row offsets, x, y) is
-// always kept.  ALSPARSE_AMD_STREAM_POLICY = 0..3 forces a combination (bit 0: values, bit 1: indices).
+// Both streams non-temporal pays with 4-byte values, and with wider ones in merge-path (power-law rows,
+// complex64: 954 / 912 / 938 / 892 us) and the ELL kernel (that stencil, fp64: 280 / 279 / 277 / 252 us), not in the
+// staged and the constant-row-length kernels (the stencil line above).  What is not a matrix stream (row offsets, x, y) is always kept.  ALSPARSE_AMD_STREAM_POLICY = 0..3 forces a combination (bit 0: values, bit 1: indices).
 #pragma once
 
 #include <cstddef>
@@ -25,8 +26,9 @@
 
 namespace asamd {
 
-// entries: stored entries (padding included); rest_bytes: everything else the multiply touches
-inline int stream_policy(double entries, size_t val_size, double rest_bytes) {
+// entries: stored entries (padding included); rest_bytes: everything else the multiply touches; wide_both: whether
+// the kernel gains from both streams non-temporal with values of 8 bytes and more
+inline int stream_policy(double entries, size_t val_size, double rest_bytes, bool wide_both = false) {
   static const int forced = getenv("ALSPARSE_AMD_STREAM_POLICY") ? atoi(getenv("ALSPARSE_AMD_STREAM_POLICY")) : -1;
   if (forced >= 0) return forced & (kStreamNtValues | kStreamNtIndices);
   const double cache = 256.0e6;
@@ -39,7 +41,7 @@ inline int stream_policy(double entries, size_t val_size, double rest_bytes) {
     if (rest_bytes + indices <= cache) return kStreamNtValues;
     if (rest_bytes + values <= cache) return kStreamNtIndices;
   }
-  return val_size == 4 ? (kStreamNtValues | kStreamNtIndices) : kStreamNtIndices;
+  return val_size == 4 || wide_both ? (kStreamNtValues | kStreamNtIndices) : kStreamNtIndices;
 }
 
 }  // namespace asamd
