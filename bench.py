@@ -433,7 +433,7 @@ def run_format_spmv(cfg, fmt, steps, warmup, check):
             if s != 0:
                 raise RuntimeError("ellmv status %d" % s)
         nbytes = a.rows * w.value * (4 + sz) + a.cols * sz + a.rows * sz * (2 if beta != 0 else 1)
-        kernel = "ell row-per-lane (width %d)" % w.value
+        kernel = "ell, two rows per lane (width %d)" % w.value
     hiprt.synchronize()
     parity = None
     if check:
