@@ -50,7 +50,8 @@ constexpr int kCooWaves = kCooThreads / kWave;
 // the wave; coomv_boundary_kernel adds the runs of equal rows up in wave order and adds each run once.
 // Entries that are grouped by row therefore reach every y through a single addition of a sum formed in a
 // fixed order: the result is the same from run to run.
-template <typename T>
+// NTI / NTV: the index streams / the values are loaded non-temporally (see stream_policy.hpp)
+template <typename T, bool NTI, bool NTV>
 __global__ __launch_bounds__(kCooThreads) void coomv_kernel(int64_t nnz, int m, int n, T alpha,
                                                             const T* __restrict__ coo_val,
                                                             const int* __restrict__ coo_row,
@@ -76,11 +77,11 @@ __global__ __launch_bounds__(kCooThreads) void coomv_kernel(int64_t nnz, int m, 
     int r = -1;
     T v = T(0);
     if (k < end) {
-      const int rr = __builtin_nontemporal_load(&coo_row[k]) - base;
-      const int c = __builtin_nontemporal_load(&coo_col[k]) - base;
+      const int rr = (NTI ? __builtin_nontemporal_load(&coo_row[k]) : coo_row[k]) - base;
+      const int c = (NTI ? __builtin_nontemporal_load(&coo_col[k]) : coo_col[k]) - base;
       if ((unsigned)rr < (unsigned)m && (unsigned)c < (unsigned)n) {
         r = rr;
-        v = coo_val[k] * x[c];  // indices non-temporal, values not: 107 -> 100 us on a 21 M-entry Laplacian (all three: 107)
+        v = (NTV ? nt_load(coo_val + k) : coo_val[k]) * x[c];
       }
     }
     const int r0 = lane_bcast(r, 0);
@@ -212,8 +213,16 @@ int coomv_impl(hipStream_t stream, int32_t m, int32_t n, int64_t nnz, T alpha, c
   const int64_t per_block = (int64_t)per_wave * kCooWaves;
   const int64_t grid = (nnz + per_block - 1) / per_block;
   if (grid > 0x7fffffff) return (int)hipErrorInvalidValue;
-  coomv_kernel<T><<<(unsigned)grid, kCooThreads, 0, stream>>>(nnz, m, n, alpha, coo_val, coo_row, coo_col, base, x, y,
-                                                              per_wave, b_row, b_val);
+  // (21 M-entry Laplacian, fp64: indices non-temporal and values not 100 us, all three non-temporal 107 us)
+  const int policy = stream_policy((double)nnz, sizeof(T), ((double)m + (double)n) * (double)sizeof(T), false, 8.0);
+#define ASAMD_COO_LAUNCH(NTI, NTV)                                                                                    \
+  coomv_kernel<T, NTI, NTV><<<(unsigned)grid, kCooThreads, 0, stream>>>(nnz, m, n, alpha, coo_val, coo_row, coo_col, base, \
+                                                                        x, y, per_wave, b_row, b_val)
+  if (policy == 0) ASAMD_COO_LAUNCH(false, false);
+  else if (policy == kStreamNtValues) ASAMD_COO_LAUNCH(false, true);
+  else if (policy == kStreamNtIndices) ASAMD_COO_LAUNCH(true, false);
+  else ASAMD_COO_LAUNCH(true, true);
+#undef ASAMD_COO_LAUNCH
   if (b_row) {
     const int64_t slots = grid * kCooWaves * 2;
     coomv_boundary_kernel<T><<<(unsigned)((slots + 255) / 256), 256, 0, stream>>>(slots, alpha, b_row, b_val, y);

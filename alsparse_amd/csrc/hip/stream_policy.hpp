@@ -27,12 +27,14 @@
 namespace asamd {
 
 // entries: stored entries (padding included); rest_bytes: everything else the multiply touches; wide_both: whether
-// the kernel gains from both streams non-temporal with values of 8 bytes and more
-inline int stream_policy(double entries, size_t val_size, double rest_bytes, bool wide_both = false) {
+// the kernel gains from both streams non-temporal with values of 8 bytes and more; index_bytes: per entry (8 for
+// the coordinate format's row and column)
+inline int stream_policy(double entries, size_t val_size, double rest_bytes, bool wide_both = false,
+                         double index_bytes = 4.0) {
   static const int forced = getenv("ALSPARSE_AMD_STREAM_POLICY") ? atoi(getenv("ALSPARSE_AMD_STREAM_POLICY")) : -1;
   if (forced >= 0) return forced & (kStreamNtValues | kStreamNtIndices);
   const double cache = 256.0e6;
-  const double values = entries * (double)val_size, indices = entries * 4.0;
+  const double values = entries * (double)val_size, indices = entries * index_bytes;
   if (rest_bytes + values + indices <= 300.0e6) return 0;  // a little more than the cache holds still gains from it
   if (values >= indices) {
     if (rest_bytes + values <= cache) return kStreamNtIndices;

@@ -396,7 +396,11 @@ def run_format_spmv(cfg, fmt, steps, warmup, check):
     from ctypes import c_int32
     from alsparse_amd import capi, hiprt, workloads as wl
     lib = capi.load()
-    a, x, y0, alpha, beta, _ = wl.config(cfg)
+    if isinstance(cfg, tuple):  # ("stencil3d", nx, ny, nz, dtype): not a benchmark configuration
+        a = wl.stencil3d(cfg[1], cfg[2], cfg[3], cfg[4])
+        x, y0, alpha, beta = wl.uniform(a.cols, a.dtype, 3), wl.uniform(a.rows, a.dtype, 4), 1.0, 0.5
+    else:
+        a, x, y0, alpha, beta, _ = wl.config(cfg)
     T, p, sz = capi.scalar_type(a.dtype), capi.prefix(a.dtype), a.dtype.itemsize
     h = capi.Handle()
     descr = capi.make_descr()
@@ -448,7 +452,10 @@ def run_format_spmv(cfg, fmt, steps, warmup, check):
                   "ok": bool(err.strict <= tol and err.zero_den_mismatch == 0)}
         d_y.copy_from(y0)
     t = time_steps(step, steps, warmup, hiprt)
-    res = {"workload": WORKLOAD_NAMES[cfg].replace("CSR", fmt.upper() + " (from CSR on the GPU)"), "rows": a.rows,
+    wname = WORKLOAD_NAMES[cfg] if not isinstance(cfg, tuple) else (
+        "27-point stencil: CSR SpMV %s, %d x %d x %d grid (%d rows, %d nnz), alpha=1 beta=0.5"
+        % (a.dtype.name, cfg[1], cfg[2], cfg[3], a.rows, a.nnz))
+    res = {"workload": wname.replace("CSR", fmt.upper() + " (from CSR on the GPU)"), "rows": a.rows,
            "nnz": a.nnz, "algorithmic_bytes": int(nbytes), "flops": 2 * a.nnz, "kernel": kernel, "timing": t,
            "gbs": nbytes / t["avg_ms"] / 1e6, "gflops": 2 * a.nnz / t["avg_ms"] / 1e6,
            "dtype": "f32" if a.dtype == np.float32 else "f64", "parity": parity}
@@ -686,9 +693,10 @@ def main():
                     "hbm_frac": conv["csr2coo"]["gbs"] / HBM_PEAK_GBS, "timing": conv["csr2coo"]["timing"],
                     "kernel": "csr2coo", "parity": None}
     elif args.format != "csr":
-        if args.config not in (2, 3):
-            sys.exit("bench.py: --format ell|coo is measured on configuration 2 or 3")
-        main_res = run_format_spmv(args.config, args.format, args.steps, args.warmup, check)
+        if args.config not in (2, 3) and not args.stencil3d:
+            sys.exit("bench.py: --format ell|coo is measured on configuration 2 or 3 (or --stencil3d)")
+        fcfg = (("stencil3d",) + tuple(args.stencil3d) + (np.float64 if args.fp64 else np.float32,)) if args.stencil3d else args.config
+        main_res = run_format_spmv(fcfg, args.format, args.steps, args.warmup, check)
     elif args.config == 5:
         main_res = run_spmm(args.steps, args.warmup, check, args.col_major, not args.no_vendor_baseline,
                             args.stencil3d, args.dense_cols)
