@@ -68,6 +68,51 @@ def test_row_major(gpu, mat, n, dtype):
             da.free()
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
+@pytest.mark.parametrize("seed", range(12))
+def test_random_structures_widths_and_layouts(gpu, seed, dtype):
+    """Seeded random structures (row-length law, base), a random number of dense columns and random padding of the
+    leading dimensions, row-major and column-major."""
+    rng = np.random.default_rng(500 + seed)
+    m, cols = int(rng.integers(1, 1500)), int(rng.integers(1, 2000))
+    law = int(rng.integers(0, 4))
+    if law == 0:
+        lengths = np.full(m, int(rng.integers(1, 40)))
+    elif law == 1:
+        lengths = rng.integers(0, int(rng.integers(2, 120)) + 1, size=m)
+    elif law == 2:
+        lengths = rng.geometric(1.0 / float(rng.integers(2, 20)), size=m) - 1
+    else:
+        lengths = rng.integers(0, 5, size=m)
+        lengths[rng.integers(0, m, size=max(1, m // 100))] = int(rng.integers(200, 1500))
+    base = int(rng.integers(0, 2))
+    a = csr_from_lengths(list(np.minimum(lengths, cols)), cols, dtype, seed=int(rng.integers(1, 1 << 30)), base=base)
+    if a.nnz == 0:
+        pytest.skip("drew a matrix without entries")
+    n = int(rng.choice([1, 2, 3, 4, 5, 8, 12, 16, 17, 20, 31, 32, 33, 48, 64, 65, 96, 128, 130]))
+    da = DeviceCsr(a)
+    try:
+        ldb, ldc = n + int(rng.integers(0, 4)), n + int(rng.integers(0, 4))
+        B = wl.uniform(a.cols * ldb, dtype, 5).reshape(a.cols, ldb)
+        C0 = wl.uniform(a.rows * ldc, dtype, 4).reshape(a.rows, ldc)
+        alpha, beta = ((1.5, 0.5), (1.0, 0.0), (-2.0, 1.0))[int(rng.integers(0, 3))]
+        announce("spmm random structure, row-major", seed, a.name, n, np.dtype(dtype).name, base, ldb, ldc, alpha, beta)
+        out = run_csrmm(gpu, da, capi.ALPHA_SPARSE_LAYOUT_ROW_MAJOR, 0, alpha, B, ldb, beta, C0, ldc, n, a.cols)
+        check(a, alpha, B[:, :n], beta, C0[:, :n], out[:, :n], "seed %d row-major n=%d" % (seed, n))
+        assert np.array_equal(out[:, n:], C0[:, n:]), "padding columns of C were touched"
+        # column-major: B is k x n with leading dimension ldbc >= k, C is m x n with ldcc >= m
+        ldbc, ldcc = a.cols + int(rng.integers(0, 3)), a.rows + int(rng.integers(0, 3))
+        Bc = wl.uniform(ldbc * n, dtype, 7).reshape(n, ldbc)
+        Cc = wl.uniform(ldcc * n, dtype, 8).reshape(n, ldcc)
+        announce("spmm random structure, column-major", seed, a.name, n, ldbc, ldcc)
+        outc = run_csrmm(gpu, da, capi.ALPHA_SPARSE_LAYOUT_COLUMN_MAJOR, 0, alpha, Bc, ldbc, beta, Cc, ldcc, n, a.cols)
+        check(a, alpha, Bc[:, :a.cols].T, beta, Cc[:, :a.rows].T, outc.reshape(n, ldcc)[:, :a.rows].T,
+              "seed %d column-major n=%d" % (seed, n))
+        assert np.array_equal(outc.reshape(n, ldcc)[:, a.rows:], Cc[:, a.rows:]), "padding rows of C were touched"
+    finally:
+        da.free()
+
+
 @pytest.mark.parametrize("maker", [lambda: wl.stencil3d(64, 60, 56, np.float32), lambda: wl.uniform_rows(215040, 215040, 12, np.float32)],
                          ids=["stencil", "random_columns"])
 def test_row_major_operand_of_the_middle_sizes(gpu, maker):
