@@ -138,7 +138,8 @@ def vendor_spmv(a, x, y0, alpha, beta, nbytes, steps, warmup, transpose=False):
             "ms": t["avg_ms"], "analysis_ms": analysis_ms}
 
 
-def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False, vendor=False, cx=False, conjugate=False):
+def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False, vendor=False, cx=False, conjugate=False,
+             analyse=None):
     """cx: the configuration's structure with complex values (complex64 for the fp32 configurations,
     complex128 for the fp64 one), complex x, y, alpha and beta; conjugate: A^H instead of A^T."""
     from alsparse_amd import capi, hiprt, workloads as wl
@@ -188,7 +189,8 @@ def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False, vendor=Fa
     assert lib.alphasparse_dcu_create_mat_info(byref(info)) == 0
     al, be = T(alpha), T(beta)
     csrmv = getattr(lib, "alphasparse_dcu_%s_csrmv" % p)
-    analysed = not (NO_ANALYSIS and not transpose)
+    # analyse=False: without alphasparse_dcu_?_csrmv_analysis (info = NULL); None: as --no-analysis says
+    analysed = not ((NO_ANALYSIS if analyse is None else not analyse) and not transpose)
 
     def step():
         s = csrmv(h.h, op, a.rows, a.cols, a.nnz, byref(al), byref(descr), d_val.c_ptr(), d_rp.c_ptr(),
@@ -719,6 +721,10 @@ def main():
             r = (run_spmm(args.steps, args.warmup, check) if c == 5
                  else run_spmv(c, args.steps, args.warmup, False, check, False, False))
             others["C%d" % c] = brief(r)
+        # and two of them as a caller who never analyses sees them (info = NULL, as the reference's own tests call)
+        for c in (2, 4):
+            others["C%d_without_analysis" % c] = brief(run_spmv(c, args.steps, args.warmup, False, check, False, False,
+                                                               analyse=False))
     if args.all:
         for c in (2, 3, 4, 5):
             if c == args.config and not args.transpose and args.format == "csr" and not args.col_major:
