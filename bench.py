@@ -190,7 +190,7 @@ def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False, vendor=Fa
     al, be = T(alpha), T(beta)
     csrmv = getattr(lib, "alphasparse_dcu_%s_csrmv" % p)
     # analyse=False: without alphasparse_dcu_?_csrmv_analysis (info = NULL); None: as --no-analysis says
-    analysed = not ((NO_ANALYSIS if analyse is None else not analyse) and not transpose)
+    analysed = not (NO_ANALYSIS if analyse is None else not analyse)
 
     def step():
         s = csrmv(h.h, op, a.rows, a.cols, a.nnz, byref(al), byref(descr), d_val.c_ptr(), d_rp.c_ptr(),
@@ -209,12 +209,14 @@ def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False, vendor=Fa
     hiprt.synchronize()
     analysis_ms = (time.perf_counter() - t0) * 1e3
     stats = lib.asamd_analysis_stats(info if analysed else d_rp.c_ptr()).contents
-    if transpose:
+    if transpose and analysed:
         assert stats.transpose_built != 0, "no room for the transposed copy"
         stats = lib.asamd_analysis_transpose_stats(info).contents
     algo = capi.ALGO_NAMES.get(stats.algo, "?")
     if stats.algo == capi.ASAMD_SPMV_VECTOR:
         algo += "(W=%d)" % stats.vector_width
+    if transpose and not analysed:
+        algo = "scatter with atomics (no copy of the transpose)"
 
     parity = None
     if check and cx and transpose:
