@@ -9,6 +9,7 @@ LIB_DIR = os.path.join(ROOT, "alsparse_amd", "lib")
 # ALSPARSE_AMD_LIB names another build of the same library (kernel experiments); there is no other fallback
 LIB_PATH = os.environ.get("ALSPARSE_AMD_LIB") or os.path.join(LIB_DIR, "libalpha_spblas.so")
 WORKLOADS_PATH = os.path.join(LIB_DIR, "libasamd_workloads.so")
+PROBES_PATH = os.path.join(LIB_DIR, "libasamd_probes.so")
 
 
 def _run(cmd, cwd=None):
@@ -32,6 +33,17 @@ def build_workloads():
     src = os.path.join(ROOT, "alsparse_amd", "workloads", "workloads.c")
     _run(["gcc", "-std=c11", "-O2", "-fopenmp", "-fPIC", "-shared", "-Wall", "-o", WORKLOADS_PATH, src, "-lm"])
     return WORKLOADS_PATH
+
+
+def build_probes():
+    """The benchmark's plain memory kernels (stream / gather ceilings, the counter-calibration copy): a
+    library of their own, so that nothing of them ships inside libalpha_spblas.so."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    src = os.path.join(ROOT, "alsparse_amd", "probes", "ceilings.hip")
+    _run(["/opt/rocm/bin/hipcc", "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument",
+          "-I" + os.path.join(ROOT, "alsparse_amd", "probes"), "-o", PROBES_PATH, src])
+    return PROBES_PATH
 
 
 def build_oracle():

@@ -9,7 +9,7 @@ import ctypes
 import os
 from ctypes import POINTER, Structure, byref, c_bool, c_double, c_float, c_int, c_int32, c_int64, c_size_t, c_void_p
 
-from .build import LIB_PATH
+from .build import LIB_PATH, PROBES_PATH
 
 # ---- enums (values are ABI) -------------------------------------------------
 ALPHA_SPARSE_STATUS_SUCCESS = 0
@@ -133,7 +133,14 @@ class asamd_csr_stats(Structure):
                 ("hot_built", c_int32), ("hot_cols_lds", c_int32), ("hot_cols", c_int32),
                 ("hot_share_lds", c_float), ("tune_ms_hot", c_float),
                 ("binned_built", c_int32), ("bin_rows", c_int32 * 4), ("tune_ms_binned", c_float),
-                ("tile_long_blocks", c_int32)]
+                ("tile_long_blocks", c_int32), ("value_check", c_int32), ("tune_mode", c_int32),
+                ("device_bytes", c_int64), ("workspace_bytes", c_int64)]
+
+
+class asamd_spmv_args(Structure):  # include/alsparse_amd_kernels.h
+    _fields_ = [("dtype", c_int32), ("m", c_int32), ("n", c_int32), ("nnz", c_int32), ("base", c_int32),
+                ("alpha", c_void_p), ("beta", c_void_p), ("val", c_void_p), ("row_ptr", c_void_p),
+                ("col_ind", c_void_p), ("x", c_void_p), ("y", c_void_p)]
 
 
 class asamd_dense_strides(Structure):
@@ -205,8 +212,6 @@ def _per_real_type(ctype):
     """Thin kernel ABI of the real value types."""
     T = ctype
     return {
-        "asamd_{s}_csrmv": [_P, _P, T, _P, _P, _P, _P, T, _P],
-        "asamd_{s}_csrmv_trans": [_P, _P, T, _P, _P, _P, _P, T, _P],
         "asamd_{s}_ellmv": [_P, _I, _I, T, _P, _P, _I, _I, _P, T, _P],
         "asamd_{s}_coomv": [_P, _I, _I, c_int64, T, _P, _P, _P, _I, _P, T, _P, _P, c_size_t],
         "asamd_{s}_csrmm": [_P, _I, _I, _I, _I, T, _P, _P, _P, _I, _P, T, _P, POINTER(asamd_dense_strides)],
@@ -221,7 +226,6 @@ def _per_complex_type(ctype):
     T = ctype
     return {
         # thin kernel ABI
-        "asamd_{s}_csrmv_op": [_P, _P, _I, T, _P, _P, _P, _P, T, _P],
         "asamd_{s}_ellmv": [_P, _I, _I, T, _P, _P, _I, _I, _P, T, _P],
         "asamd_{s}_coomv": [_P, _I, _I, c_int64, T, _P, _P, _P, _I, _P, T, _P, _P, c_size_t],
         "asamd_{s}_csrmm_ws": [_P, _I, _I, _I, _I, T, _P, _P, _P, _I, _P, T, _P, POINTER(asamd_dense_strides), _P,
@@ -305,7 +309,36 @@ _COMMON = {
     "asamd_csr_plan_stats": [_P],
     "asamd_csr_plan_set_algo": [_P, _I],
     "asamd_csr_plan_refresh_values": [_P, _P, _P, _P, _P],
-    "asamd_csr_structure_hash": [_P, _I, _I, _P, _P, POINTER(ctypes.c_uint64)],
+    "asamd_csr_structure_hash": [_P, _I, _I, _P, _P, _P, POINTER(ctypes.c_uint64)],
+    "asamd_csr_plan_workspace_bytes": [_P],
+    "asamd_csr_plan_csrmv": [_P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, c_size_t],
+    "asamd_handle_reserve": [_P, c_size_t],
+    # stateless launchers and layout builders (records are passed as opaque pointers here)
+    "asamd_spmv_vector": [_P, POINTER(asamd_spmv_args), _I],
+    "asamd_spmv_scalar": [_P, POINTER(asamd_spmv_args)],
+    "asamd_spmv_rowconst": [_P, POINTER(asamd_spmv_args), _I],
+    "asamd_spmv_stream": [_P, POINTER(asamd_spmv_args), _I, _I, _I],
+    "asamd_merge_partition": [_P, _I, _I, _P, _I, _I, _I, _P],
+    "asamd_spmv_merge": [_P, POINTER(asamd_spmv_args), _I, _P, _P, _P, _P],
+    "asamd_spmv_trans_scatter": [_P, POINTER(asamd_spmv_args), _I, _I],
+    "asamd_tiled_fits": [_I, _I, _I, _I],
+    "asamd_tiled_build": [_P, _I, _I, _I, _I, _I, _P, _P, _P, _I, _I, _P],
+    "asamd_tiled_free": [_P],
+    "asamd_spmv_tiled": [_P, POINTER(asamd_spmv_args), _P, _P, _P],
+    "asamd_hot_build": [_P, _I, _I, _I, _I, _I, _P, _P, _I, _I, _I, _P],
+    "asamd_hot_free": [_P],
+    "asamd_spmv_hot": [_P, POINTER(asamd_spmv_args), _P, _P, _P, _P, _P],
+    "asamd_binned_build": [_P, _I, _I, _P, _P],
+    "asamd_binned_free": [_P],
+    "asamd_spmv_binned": [_P, POINTER(asamd_spmv_args), _P, _P],
+    "asamd_transpose_build": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P],
+    "asamd_transpose_free": [_P],
+    "asamd_csr_row_stats": [_P, _I, _P, _P, _P],
+    "asamd_value_guard_run": [c_size_t],
+    "asamd_value_guard": [_P, _P, c_size_t, _I, _P, _P],
+    "asamd_value_guard_commit": [_P, _P, _P],
+    "asamd_gather_values": [_P, _I, _I, _I, _P, _P, _P, _P],
+    "asamd_csr2ell_gated": [_P, _I, _I, _P, _P, _P, _I, _I, _I, _P, _P, _P],
     "asamd_csr_plan_build_transpose": [_P, _P, _P, _P, _P],
     "asamd_csr_plan_set_lazy_transpose": [_P, _I],
     "asamd_csr_plan_transpose_stats": [_P],
@@ -319,8 +352,6 @@ _COMMON = {
     "asamd_s_csrmv_noalloc": [_P, _I, _I, _I, _I, c_float, _P, _P, _P, _P, c_float, _P],
     "asamd_handle_set_stream": [_P, _P],
     "asamd_handle_get_stream": [_P],
-    "asamd_copy_bytes": [_P, _P, _P, c_size_t],
-    "asamd_ceiling_kernel": [_P, _I, _P, _P, c_size_t, c_int64, _P, POINTER(c_int64)],
     "asamd_registry_lazy_count": [],
     "asamd_analysis_stats": [_P],
     "asamd_analysis_transpose_stats": [_P],
@@ -348,7 +379,7 @@ _RESTYPE = {"alpha_set_thread_num": None, "alpha_timing_wtime": c_double, "alpha
             "args_help": None, "args_get_if_check": c_bool, "args_get_data_file": ctypes.c_char_p,
             "args_get_data_fileA": ctypes.c_char_p, "args_get_data_fileB": ctypes.c_char_p,
             "alpha_args_get_matrix_descrA": alpha_matrix_descr, "alpha_args_get_matrix_descrB": alpha_matrix_descr,
-            "get_time_us": c_double, "asamd_csrmm_workspace_bytes": c_size_t, "asamd_csr2coo_workspace_bytes": c_size_t, "asamd_csr_plan_stats": POINTER(asamd_csr_stats),
+            "get_time_us": c_double, "asamd_csrmm_workspace_bytes": c_size_t, "asamd_csr2coo_workspace_bytes": c_size_t, "asamd_csr_plan_workspace_bytes": c_size_t, "asamd_value_guard_run": c_size_t, "asamd_tiled_free": None, "asamd_hot_free": None, "asamd_binned_free": None, "asamd_transpose_free": None, "asamd_csr_plan_stats": POINTER(asamd_csr_stats),
             "asamd_csr_plan_transpose_stats": POINTER(asamd_csr_stats),
             "asamd_analysis_transpose_stats": POINTER(asamd_csr_stats),
             "asamd_analysis_stats": POINTER(asamd_csr_stats)}
@@ -376,6 +407,26 @@ def load():
             fn.restype = _RESTYPE.get(name, c_int)
         _lib = lib
     return _lib
+
+
+_probes = None
+
+
+def load_probes():
+    """The benchmark's plain memory kernels (libasamd_probes.so): stream / gather ceilings and the copy that
+    calibrates the byte counters.  Not part of the product library."""
+    global _probes
+    if _probes is None:
+        if not os.path.exists(PROBES_PATH):
+            raise RuntimeError("%s is missing: build it first (python -c 'import __graft_entry__ as g; g.build()')"
+                               % PROBES_PATH)
+        lib = ctypes.CDLL(PROBES_PATH)
+        lib.asamd_copy_bytes.argtypes = [_P, _P, _P, c_size_t]
+        lib.asamd_copy_bytes.restype = c_int
+        lib.asamd_ceiling_kernel.argtypes = [_P, _I, _P, _P, c_size_t, c_int64, _P, POINTER(c_int64)]
+        lib.asamd_ceiling_kernel.restype = c_int
+        _probes = lib
+    return _probes
 
 
 # ---- small conveniences used by tests and the benchmark -----------------------
@@ -426,3 +477,22 @@ class Handle:
 def make_descr(base=ALPHA_SPARSE_INDEX_BASE_ZERO, mtype=ALPHA_SPARSE_MATRIX_TYPE_GENERAL):
     d = alpha_dcu_matrix_descr(mtype, 0, 0, base)
     return d
+
+
+class Workspace:
+    """Per-call device scratch for asamd_csr_plan_csrmv, sized for a plan."""
+
+    def __init__(self, lib, plan, extra=0):
+        from . import hiprt
+        self.bytes = int(lib.asamd_csr_plan_workspace_bytes(plan)) + extra
+        self.buf = hiprt.DeviceArray(max(self.bytes, 256), "uint8")
+
+    def c_ptr(self):
+        return self.buf.c_ptr()
+
+
+def plan_csrmv(lib, stream, plan, op, alpha, val, row_ptr, col_ind, x, beta, y, ws=None):
+    """asamd_csr_plan_csrmv with ctypes scalars of the plan's element type (alpha, beta) and a Workspace (or none)."""
+    return lib.asamd_csr_plan_csrmv(stream, plan, op, ctypes.cast(byref(alpha), c_void_p), val, row_ptr, col_ind, x,
+                                    ctypes.cast(byref(beta), c_void_p), y, ws.c_ptr() if ws else None,
+                                    ws.bytes if ws else 0)

@@ -1,0 +1,217 @@
+// Analysis building blocks on the GPU (gfx950): row-length statistics, fingerprints of the structure
+// arrays and of the values.  Each entry point is one self-contained operation on plain device arrays;
+// the host library's plan strings them together.  The row statistics replace the host-side walk over
+// row_ptr of src/util_cpp/alphasparse_dcu_x_csrmv_analysis.cpp:58-267 and its device-to-host round trip
+// at :348-379; the fingerprints have no counterpart (the reference's analysis keeps nothing that a change
+// of values could invalidate, :382-388).
+
+#include <hip/hip_runtime.h>
+
+#include "alsparse_amd_kernels.h"
+#include "launch_utils.hpp"
+
+using namespace asamd;
+
+// ---------------------------------------------------------------------------
+// Row-length statistics.  out[0] = min, out[1] = max, out[2] = row_ptr[0],
+// out[3 .. 3+33) = histogram counters: a bin can hold at most m < 2^31.
+// ---------------------------------------------------------------------------
+constexpr int kStatWords = ASAMD_ROW_STATS_WORDS;
+
+__global__ __launch_bounds__(256) void row_stats_kernel(int m, const int* __restrict__ row_ptr,
+                                                        int* __restrict__ out) {
+  __shared__ int s_hist[ASAMD_HIST_BINS];
+  __shared__ int s_min, s_max;
+  if (threadIdx.x < ASAMD_HIST_BINS) s_hist[threadIdx.x] = 0;
+  if (threadIdx.x == 0) {
+    s_min = 0x7fffffff;
+    s_max = 0;
+  }
+  __syncthreads();
+  int lmin = 0x7fffffff, lmax = 0;
+  for (int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; r < m;
+       r += (int64_t)gridDim.x * blockDim.x) {
+    int len = row_ptr[r + 1] - row_ptr[r];
+    if (len < 0) len = 0;  // malformed offsets: counted as empty, never indexed with
+    lmin = len < lmin ? len : lmin;
+    lmax = len > lmax ? len : lmax;
+    const int bin = len == 0 ? 0 : 32 - __builtin_clz((unsigned)len);
+    atomicAdd(&s_hist[bin], 1);
+  }
+  atomicMin(&s_min, lmin);
+  atomicMax(&s_max, lmax);
+  __syncthreads();
+  if (threadIdx.x < ASAMD_HIST_BINS && s_hist[threadIdx.x] != 0)
+    atomicAdd(&out[3 + threadIdx.x], s_hist[threadIdx.x]);
+  if (threadIdx.x == 0) {
+    atomicMin(&out[0], s_min);
+    atomicMax(&out[1], s_max);
+    if (blockIdx.x == 0) out[2] = row_ptr[0];
+  }
+}
+
+__global__ void stats_init_kernel(int* out) {
+  const int t = threadIdx.x;
+  if (t < kStatWords) out[t] = t == 0 ? 0x7fffffff : 0;
+}
+
+extern "C" int asamd_csr_row_stats(hipStream_t stream, int32_t m, const int32_t* row_ptr, int32_t* d_scratch,
+                                   int32_t* stats_host) {
+  if (!row_ptr || !d_scratch || !stats_host || m <= 0) return hipErrorInvalidValue;
+  stats_init_kernel<<<1, 64, 0, stream>>>(d_scratch);
+  int64_t grid = ((int64_t)m + 255) / 256;
+  if (grid > 256 * 16) grid = 256 * 16;
+  row_stats_kernel<<<(unsigned)grid, 256, 0, stream>>>(m, row_ptr, d_scratch);
+  hipError_t e = hipGetLastError();
+  if (e == hipSuccess)
+    e = hipMemcpyAsync(stats_host, d_scratch, kStatWords * sizeof(int), hipMemcpyDeviceToHost, stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(stream);
+  return e;
+}
+
+// ---------------------------------------------------------------------------
+// hash[0] += sum over i of mix(a[i], i + salt): a fingerprint of an index array that does not depend on
+// the order of the (integer, wrapping) additions.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ unsigned long long mix_index(unsigned long long v, unsigned long long i) {
+  unsigned long long z = (v + 0x9E3779B97F4A7C15ull) * 0xBF58476D1CE4E5B9ull ^ (i * 0x94D049BB133111EBull);
+  z = (z ^ (z >> 29)) * 0xD6E8FEB86659FD93ull;
+  return z ^ (z >> 32);
+}
+
+__device__ __forceinline__ unsigned long long block_sum_u64(unsigned long long mine) {
+  __shared__ unsigned long long s_sum[256 / kWave];
+  for (int d = kWave / 2; d > 0; d >>= 1) mine += __shfl_down(mine, d, kWave);
+  if (threadIdx.x % kWave == 0) s_sum[threadIdx.x / kWave] = mine;
+  __syncthreads();
+  unsigned long long total = 0;
+  if (threadIdx.x == 0)
+    for (int w = 0; w < 256 / kWave; ++w) total += s_sum[w];
+  return total;  // valid in thread 0
+}
+
+__global__ __launch_bounds__(256) void index_hash_kernel(int64_t n, const int* __restrict__ a, unsigned long long salt,
+                                                         unsigned long long* __restrict__ hash) {
+  unsigned long long mine = 0;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
+    mine += mix_index((unsigned long long)(unsigned)nt_load(a + i), (unsigned long long)i + salt);
+  const unsigned long long total = block_sum_u64(mine);
+  if (threadIdx.x == 0) atomicAdd(hash, total);
+}
+
+__global__ void zero_u64_kernel(unsigned long long* p) { *p = 0; }
+
+extern "C" int asamd_csr_structure_hash(hipStream_t stream, int32_t m, int32_t nnz, const int32_t* row_ptr,
+                                        const int32_t* col_ind, void* d_scratch, uint64_t* hash_host) {
+  if (!row_ptr || !hash_host || !d_scratch || ((uintptr_t)d_scratch & 7u) || m < 0 || nnz < 0 || (nnz > 0 && !col_ind))
+    return hipErrorInvalidValue;
+  unsigned long long* d_hash = (unsigned long long*)d_scratch;
+  zero_u64_kernel<<<1, 1, 0, stream>>>(d_hash);
+  index_hash_kernel<<<256 * 8, 256, 0, stream>>>((int64_t)m + 1, row_ptr, 0x1234567ull, d_hash);
+  if (nnz > 0) index_hash_kernel<<<256 * 16, 256, 0, stream>>>((int64_t)nnz, col_ind, 0xABCDEF01ull << 8, d_hash);
+  hipError_t e = hipGetLastError();
+  unsigned long long h = 0;
+  if (e == hipSuccess) e = hipMemcpyAsync(&h, d_hash, sizeof(h), hipMemcpyDeviceToHost, stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(stream);
+  *hash_host = (uint64_t)h;
+  return e;
+}
+
+// ---------------------------------------------------------------------------
+// Value guard.  The array is taken as 4-byte words in runs of run_words words (a multiple of 64); of
+// every run one wave reads 64 consecutive words (256 bytes) at a position that varies from run to run
+// (a fixed stride would sample the same memory channels and the same residues over and over), each
+// word is mixed with its position, and the sums of all lanes add up to the fingerprint -- integer
+// additions, so the order does not matter and equal arrays give equal words.  run_words == 64 reads
+// everything.
+// ---------------------------------------------------------------------------
+constexpr int kGuardBlocks = 2048;
+constexpr int kGuardUnroll = 8;
+static_assert(ASAMD_GUARD_WS_BYTES >= kGuardBlocks * 8 + 16, "guard scratch holds the partial sums, the word and the flag");
+
+struct GuardWs {
+  unsigned long long partial[kGuardBlocks];
+  unsigned long long fp;
+  int flag;
+};
+static_assert(offsetof(GuardWs, flag) == 8 * kGuardBlocks + 8, "ASAMD_GUARD_FLAG points at the flag");
+
+__device__ __forceinline__ unsigned long long mix_word(unsigned w, unsigned long long idx) {
+  const unsigned i = (unsigned)idx ^ ((unsigned)(idx >> 32) * 0x9E3779B1u);
+  unsigned a = ((w + 0x7F4A7C15u) * 0x9E3779B1u) ^ (i * 0x85EBCA6Bu);
+  a = (a ^ (a >> 15)) * 0xC2B2AE35u;
+  a ^= a >> 13;
+  unsigned b = ((w ^ 0xD6E8FEB8u) * 0x27D4EB2Fu) + ((i ^ (i >> 17)) * 0x165667B1u);
+  b = (b ^ (b >> 16)) * 0x94D049BBu;
+  return ((unsigned long long)b << 32) | a;
+}
+
+__global__ __launch_bounds__(256) void value_hash_kernel(const unsigned* __restrict__ words, int64_t total_words,
+                                                         int64_t run_words, unsigned long long* __restrict__ partial) {
+  const int lane = threadIdx.x % kWave;
+  const int64_t waves = (int64_t)gridDim.x * (256 / kWave);
+  const int64_t wave = (int64_t)blockIdx.x * (256 / kWave) + threadIdx.x / kWave;
+  const int64_t runs = (total_words + run_words - 1) / run_words;
+  const unsigned slots = (unsigned)(run_words / kWave);  // positions a sample can take inside its run
+  unsigned long long mine = 0;
+  for (int64_t r0 = wave; r0 < runs; r0 += waves * kGuardUnroll) {
+    unsigned w[kGuardUnroll];
+    int64_t idx[kGuardUnroll];
+#pragma unroll
+    for (int u = 0; u < kGuardUnroll; ++u) {
+      const int64_t r = r0 + (int64_t)u * waves;
+      const int64_t start = r * run_words;
+      int64_t pos = start + (int64_t)((((unsigned)r * 2654435761u) >> 7) % slots) * kWave;
+      if (pos >= total_words) pos = start;  // the last, short run
+      idx[u] = r < runs && pos + lane < total_words ? pos + lane : -1;
+      w[u] = idx[u] >= 0 ? nt_load(words + idx[u]) : 0u;
+    }
+#pragma unroll
+    for (int u = 0; u < kGuardUnroll; ++u)
+      if (idx[u] >= 0) mine += mix_word(w[u], (unsigned long long)idx[u]);
+  }
+  const unsigned long long total = block_sum_u64(mine);
+  if (threadIdx.x == 0) partial[blockIdx.x] = total;
+}
+
+__global__ __launch_bounds__(256) void value_verdict_kernel(GuardWs* __restrict__ ws, int64_t total_words,
+                                                            const unsigned long long* __restrict__ stored) {
+  unsigned long long mine = 0;
+  for (int i = threadIdx.x; i < kGuardBlocks; i += 256) mine += ws->partial[i];
+  unsigned long long fp = block_sum_u64(mine);
+  if (threadIdx.x == 0) {
+    fp ^= (unsigned long long)total_words * 0x9E3779B97F4A7C15ull;
+    ws->fp = fp;
+    ws->flag = (!stored || *stored != fp) ? 1 : 0;
+  }
+}
+
+__global__ void value_commit_kernel(const GuardWs* __restrict__ ws, unsigned long long* __restrict__ stored) {
+  if (ws->flag) *stored = ws->fp;
+}
+
+extern "C" size_t asamd_value_guard_run(size_t nbytes) {
+  // 256 bytes of every run, 32 MiB in all at the most: the run is the smallest power of two (in 256-byte
+  // units) that gets there
+  size_t run = 256;
+  while (nbytes / run * 256 > ASAMD_GUARD_FULL_BYTES) run *= 2;
+  return run;
+}
+
+extern "C" int asamd_value_guard(hipStream_t stream, const void* val, size_t nbytes, int32_t full,
+                                 const uint64_t* stored, void* ws) {
+  if (!val || !ws || ((uintptr_t)ws & 7u) || ((uintptr_t)val & 3u) || (nbytes & 3u) || nbytes == 0)
+    return hipErrorInvalidValue;
+  const int64_t total_words = (int64_t)(nbytes / 4);
+  const int64_t run_words = (int64_t)((full || nbytes <= ASAMD_GUARD_FULL_BYTES ? (size_t)256 : asamd_value_guard_run(nbytes)) / 4);
+  GuardWs* g = (GuardWs*)ws;
+  value_hash_kernel<<<kGuardBlocks, 256, 0, stream>>>((const unsigned*)val, total_words, run_words, g->partial);
+  value_verdict_kernel<<<1, 256, 0, stream>>>(g, total_words, (const unsigned long long*)stored);
+  return hipGetLastError();
+}
+
+extern "C" int asamd_value_guard_commit(hipStream_t stream, const void* ws, uint64_t* stored) {
+  if (!ws || !stored) return hipErrorInvalidValue;
+  value_commit_kernel<<<1, 1, 0, stream>>>((const GuardWs*)ws, (unsigned long long*)stored);
+  return hipGetLastError();
+}

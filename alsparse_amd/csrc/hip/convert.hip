@@ -256,7 +256,8 @@ template <typename T, bool NTS, bool WIDE>
 __global__ __launch_bounds__(kEllRows) void csr2ell_kernel(
     int m, const T* __restrict__ val, const int* __restrict__ row_ptr,
     const int* __restrict__ col_ind, int csr_base, int ell_base, int width,
-    T* __restrict__ ell_val, int* __restrict__ ell_col) {
+    T* __restrict__ ell_val, int* __restrict__ ell_col, const int* __restrict__ gate) {
+  if (gate && *gate == 0) return;  // a refresh behind the value guard: nothing has changed
   constexpr int kWindow = sizeof(T) > 8 ? kEllWindow / 2 : kEllWindow;  // at most 32 KiB of staged values
   // staged entry p lives at p + p / 32: lanes read slot s of consecutive rows, i.e. positions a row
   // length apart, and without the skew rows of 16 or 32 entries would all fall into a few LDS banks
@@ -375,7 +376,8 @@ __global__ __launch_bounds__(kEllRows) void csr2ell_kernel(
 
 template <typename T>
 static int csr2ell_impl(hipStream_t stream, int m, const T* val, const int* rp, const int* ci,
-                        int csr_base, int ell_base, int width, T* ell_val, int* ell_col) {
+                        int csr_base, int ell_base, int width, T* ell_val, int* ell_col,
+                        const int* gate = nullptr) {
   if (!val || !rp || !ci || !ell_val || !ell_col || m <= 0 || width < 0) return hipErrorInvalidValue;
   if (((uintptr_t)val | (uintptr_t)ell_val) % alignof(T)) return hipErrorInvalidValue;
   if (width == 0) return hipSuccess;
@@ -383,7 +385,7 @@ static int csr2ell_impl(hipStream_t stream, int m, const T* val, const int* rp, 
   const bool nts = stores_bypass_caches((size_t)m * (size_t)width * (sizeof(T) + sizeof(int)));
   const bool wide = (((uintptr_t)val | (uintptr_t)ci) & 15u) == 0;
 #define ASAMD_CSR2ELL(NTS, WIDE) \
-  csr2ell_kernel<T, NTS, WIDE><<<grid, kEllRows, 0, stream>>>(m, val, rp, ci, csr_base, ell_base, width, ell_val, ell_col)
+  csr2ell_kernel<T, NTS, WIDE><<<grid, kEllRows, 0, stream>>>(m, val, rp, ci, csr_base, ell_base, width, ell_val, ell_col, gate)
   if (nts && wide) ASAMD_CSR2ELL(true, true);
   else if (nts) ASAMD_CSR2ELL(true, false);
   else if (wide) ASAMD_CSR2ELL(false, true);
@@ -421,4 +423,22 @@ extern "C" int asamd_z_csr2ell(hipStream_t stream, int32_t m, const asamd_comple
   using T = asamd::Cx<double>;
   return csr2ell_impl<T>(stream, m, (const T*)val, row_ptr, col_ind, csr_base, ell_base, width, (T*)ell_val,
                          ell_col);
+}
+
+// Elements copied bit for bit: only their size matters.  gate: see asamd_value_guard.
+extern "C" int asamd_csr2ell_gated(hipStream_t stream, int32_t elem_bytes, int32_t m, const void* val,
+                                   const int32_t* row_ptr, const int32_t* col_ind, int32_t csr_base, int32_t ell_base,
+                                   int32_t width, void* ell_val, int32_t* ell_col, const int32_t* gate) {
+  if (elem_bytes == 4)
+    return csr2ell_impl<float>(stream, m, (const float*)val, row_ptr, col_ind, csr_base, ell_base, width,
+                               (float*)ell_val, ell_col, gate);
+  if (elem_bytes == 8)
+    return csr2ell_impl<double>(stream, m, (const double*)val, row_ptr, col_ind, csr_base, ell_base, width,
+                                (double*)ell_val, ell_col, gate);
+  if (elem_bytes == 16) {
+    using T = asamd::Cx<double>;
+    return csr2ell_impl<T>(stream, m, (const T*)val, row_ptr, col_ind, csr_base, ell_base, width, (T*)ell_val,
+                           ell_col, gate);
+  }
+  return hipErrorInvalidValue;
 }

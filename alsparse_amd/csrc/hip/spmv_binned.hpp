@@ -43,7 +43,7 @@ __device__ __forceinline__ int bin_class(int len) {
 }
 
 // key[r] = length class of row r, idx[r] = r
-__global__ __launch_bounds__(256) void bin_keys_kernel(int m, const int* __restrict__ row_ptr, unsigned* __restrict__ key,
+static __global__ __launch_bounds__(256) void bin_keys_kernel(int m, const int* __restrict__ row_ptr, unsigned* __restrict__ key,
                                                        unsigned* __restrict__ idx, int* __restrict__ count) {
   __shared__ int s_count[kBinClasses];
   if (threadIdx.x < kBinClasses) s_count[threadIdx.x] = 0;
@@ -60,7 +60,7 @@ __global__ __launch_bounds__(256) void bin_keys_kernel(int m, const int* __restr
 }
 
 // (row_ptr[r], row_ptr[r + 1]) of the listed rows, for the host that cuts the long rows into chunks
-__global__ __launch_bounds__(256) void bin_row_bounds_kernel(int count, const int* __restrict__ rows,
+static __global__ __launch_bounds__(256) void bin_row_bounds_kernel(int count, const int* __restrict__ rows,
                                                              const int* __restrict__ row_ptr, int* __restrict__ bounds) {
   const int i = blockIdx.x * 256 + threadIdx.x;
   if (i >= count) return;

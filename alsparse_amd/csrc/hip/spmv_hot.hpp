@@ -280,13 +280,13 @@ __global__ __launch_bounds__(kWave* NW) void spmv_merge_hot_kernel(
 }
 
 // ---- analysis of the hot columns ------------------------------------------------------------------
-__global__ __launch_bounds__(256) void col_count_kernel(int nnz, const int* __restrict__ col_ind, int base,
+static __global__ __launch_bounds__(256) void col_count_kernel(int nnz, const int* __restrict__ col_ind, int base,
                                                         unsigned* __restrict__ count) {
   for (int64_t k = (int64_t)blockIdx.x * 256 + threadIdx.x; k < nnz; k += (int64_t)gridDim.x * 256)
     atomicAdd(&count[nt_load(col_ind + k) - base], 1u);
 }
 // key[c] = ~count[c] (an ascending sort then puts the most popular column first), idx[c] = c
-__global__ __launch_bounds__(256) void col_rank_keys_kernel(int n, const unsigned* __restrict__ count,
+static __global__ __launch_bounds__(256) void col_rank_keys_kernel(int n, const unsigned* __restrict__ count,
                                                             unsigned* __restrict__ key, unsigned* __restrict__ idx) {
   const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (c >= n) return;
@@ -294,7 +294,7 @@ __global__ __launch_bounds__(256) void col_rank_keys_kernel(int n, const unsigne
   idx[c] = (unsigned)c;
 }
 // rank[sorted_col[i]] = i for i < hc (rank was filled with 0xFFFFFFFF)
-__global__ __launch_bounds__(256) void col_rank_scatter_kernel(int hc, const unsigned* __restrict__ sorted_col,
+static __global__ __launch_bounds__(256) void col_rank_scatter_kernel(int hc, const unsigned* __restrict__ sorted_col,
                                                                unsigned* __restrict__ rank, int* __restrict__ hot_cols) {
   const int i = blockIdx.x * 256 + threadIdx.x;
   if (i >= hc) return;
@@ -302,7 +302,7 @@ __global__ __launch_bounds__(256) void col_rank_scatter_kernel(int hc, const uns
   hot_cols[i] = (int)sorted_col[i];
 }
 // pcol[k] = rank of entry k's column if it is one of the hc most popular, else hc + column
-__global__ __launch_bounds__(256) void hot_pcol_kernel(int nnz, const int* __restrict__ col_ind, int base, int hc,
+static __global__ __launch_bounds__(256) void hot_pcol_kernel(int nnz, const int* __restrict__ col_ind, int base, int hc,
                                                        const unsigned* __restrict__ rank, unsigned* __restrict__ pcol) {
   for (int64_t k = (int64_t)blockIdx.x * 256 + threadIdx.x; k < nnz; k += (int64_t)gridDim.x * 256) {
     const unsigned c = (unsigned)(nt_load(col_ind + k) - base);

@@ -1,0 +1,310 @@
+// Stateless launchers of the CSR SpMV kernel families that work on the caller's CSR arrays
+// (gfx950, wave64).  Each stands in for csr_gemv_vector_dispatch,
+// src/kernel/dcu/level2/mv/csrmv/dcu_gemv_vector.h:59-182, for one mapping of rows to lanes; which
+// one runs is decided by the host library's plan.  Nothing here allocates, copies or waits.
+
+#include <hip/hip_runtime.h>
+
+#include "alsparse_amd_kernels.h"
+#include "launch_utils.hpp"
+#include "spmv_merge.hpp"
+#include "spmv_rows.hpp"
+#include "spmv_trans.hpp"
+#include "stream_policy.hpp"
+
+using namespace asamd;
+
+static_assert(kMergeThreads == ASAMD_MERGE_THREADS, "the header documents the merge block size");
+static_assert(kStreamMaxGroup == ASAMD_STREAM_MAX_GROUP, "the header documents the widest lane group");
+
+// the cache policy of a CSR multiply's two matrix streams (stream_policy.hpp) from its sizes
+static int csr_stream_policy(const asamd_spmv_args* a, size_t val_size, bool wide_both = false) {
+  return asamd::stream_policy((double)a->nnz, val_size,
+                              ((double)a->m + 1.0) * 4.0 + ((double)a->m + (double)a->n) * (double)val_size, wide_both);
+}
+
+// ---- W lanes per row ----------------------------------------------------------------------------
+template <typename T, int W>
+static void launch_vector(hipStream_t s, const asamd_spmv_args* a) {
+  constexpr int rows_per_block = kRowsBlock / W;
+  const unsigned grid = (unsigned)(((int64_t)a->m + rows_per_block - 1) / rows_per_block);
+  spmv_vector_kernel<T, W><<<grid, kRowsBlock, 0, s>>>(a->m, scalar_of<T>(a->alpha), (const T*)a->val, a->row_ptr,
+                                                       a->col_ind, (const T*)a->x, scalar_of<T>(a->beta), (T*)a->y,
+                                                       a->base);
+}
+
+extern "C" int asamd_spmv_vector(hipStream_t s, const asamd_spmv_args* a, int32_t width) {
+  if (!a) return hipErrorInvalidValue;
+  return by_dtype(a->dtype, [&](auto* tag) -> int {
+    using T = std::remove_pointer_t<decltype(tag)>;
+    if (!args_ok<T>(a)) return hipErrorInvalidValue;
+    switch (width) {
+      case 2: launch_vector<T, 2>(s, a); break;
+      case 4: launch_vector<T, 4>(s, a); break;
+      case 8: launch_vector<T, 8>(s, a); break;
+      case 16: launch_vector<T, 16>(s, a); break;
+      case 32: launch_vector<T, 32>(s, a); break;
+      case 64: launch_vector<T, 64>(s, a); break;
+      default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+  });
+}
+
+extern "C" int asamd_spmv_scalar(hipStream_t s, const asamd_spmv_args* a) {
+  if (!a) return hipErrorInvalidValue;
+  return by_dtype(a->dtype, [&](auto* tag) -> int {
+    using T = std::remove_pointer_t<decltype(tag)>;
+    if (!args_ok<T>(a)) return hipErrorInvalidValue;
+    const unsigned grid = (unsigned)(((int64_t)a->m + kRowsBlock - 1) / kRowsBlock);
+    spmv_scalar_kernel<T><<<grid, kRowsBlock, 0, s>>>(a->m, scalar_of<T>(a->alpha), (const T*)a->val, a->row_ptr,
+                                                      a->col_ind, (const T*)a->x, scalar_of<T>(a->beta), (T*)a->y,
+                                                      a->base);
+    return hipGetLastError();
+  });
+}
+
+// ---- every row has 4 * G entries ---------------------------------------------------------------
+template <typename T, int G>
+static void launch_rowconst(hipStream_t s, const asamd_spmv_args* a) {
+  constexpr int R = G >= 16 ? 1 : 2;
+  constexpr int rows_per_block = (kRowsBlock / G) * R;
+  const unsigned grid = (unsigned)(((int64_t)a->m + rows_per_block - 1) / rows_per_block);
+  spmv_rowconst_kernel<T, G, R><<<grid, kRowsBlock, 0, s>>>(a->m, scalar_of<T>(a->alpha), (const T*)a->val,
+                                                            a->col_ind, (const T*)a->x, scalar_of<T>(a->beta),
+                                                            (T*)a->y, a->base, csr_stream_policy(a, sizeof(T)));
+}
+
+template <typename T>
+static int rowconst_impl(hipStream_t s, const asamd_spmv_args* a, int row_len) {
+  if (!args_ok<T>(a)) return hipErrorInvalidValue;
+  // 128-bit loads need 16-byte aligned streams
+  if ((((uintptr_t)a->val | (uintptr_t)a->col_ind) & 15u) != 0) return hipErrorInvalidValue;
+  switch (row_len) {
+    case 4: launch_rowconst<T, 1>(s, a); break;
+    case 8: launch_rowconst<T, 2>(s, a); break;
+    case 16: launch_rowconst<T, 4>(s, a); break;
+    case 32: launch_rowconst<T, 8>(s, a); break;
+    case 64: launch_rowconst<T, 16>(s, a); break;
+    case 128: launch_rowconst<T, 32>(s, a); break;
+    case 256: launch_rowconst<T, 64>(s, a); break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
+extern "C" int asamd_spmv_rowconst(hipStream_t s, const asamd_spmv_args* a, int32_t row_len) {
+  if (!a) return hipErrorInvalidValue;
+  // the kernel loads four values as one 128-bit piece: real element types only
+  if (a->dtype == ASAMD_DTYPE_FLOAT) return rowconst_impl<float>(s, a, row_len);
+  if (a->dtype == ASAMD_DTYPE_DOUBLE) return rowconst_impl<double>(s, a, row_len);
+  return hipErrorInvalidValue;
+}
+
+// ---- a block of rows staged in LDS, G lanes per row ----------------------------------------------
+extern "C" int asamd_spmv_stream(hipStream_t s, const asamd_spmv_args* a, int32_t g, int32_t max_len,
+                                 int32_t first_offset) {
+  if (!a) return hipErrorInvalidValue;
+  return by_dtype(a->dtype, [&](auto* tag) -> int {
+    using T = std::remove_pointer_t<decltype(tag)>;
+    if (!args_ok<T>(a)) return hipErrorInvalidValue;
+    constexpr int kCap = 64 / (int)sizeof(T);  // 16 KiB of products per workgroup
+    if (g < 1 || g > kStreamMaxGroup || (g & (g - 1)) != 0) return hipErrorInvalidValue;
+    const unsigned grid = (unsigned)(((int64_t)a->m * g + kStreamRows - 1) / kStreamRows);
+    // 128-bit loads need 16-byte aligned streams
+    const bool wide = (((uintptr_t)a->val | (uintptr_t)a->col_ind) & 15u) == 0;
+    const int64_t limit = (int64_t)first_offset + a->nnz;
+    const T alpha = scalar_of<T>(a->alpha), beta = scalar_of<T>(a->beta);
+    const T* val = (const T*)a->val;
+    const T* x = (const T*)a->x;
+    T* y = (T*)a->y;
+    const int policy = csr_stream_policy(a, sizeof(T));
+#define ASAMD_STREAM_LAUNCH(CAP, G)                                                                                \
+  do {                                                                                                             \
+    if (wide)                                                                                                      \
+      spmv_stream_wide_kernel<T, CAP, G><<<grid, kStreamRows, 0, s>>>(a->m, alpha, val, a->row_ptr, a->col_ind, x, \
+                                                                      beta, y, a->base, limit, policy);            \
+    else                                                                                                           \
+      spmv_stream_kernel<T, CAP, G><<<grid, kStreamRows, 0, s>>>(a->m, alpha, val, a->row_ptr, a->col_ind, x,      \
+                                                                 beta, y, a->base);                                \
+  } while (0)
+    if (g == 1) {
+      // the smallest staging area that holds the longest row
+      if (max_len <= 4) {
+        ASAMD_STREAM_LAUNCH(4, 1);
+      } else if constexpr (kCap >= 8) {
+        if (max_len <= 8) {
+          ASAMD_STREAM_LAUNCH(8, 1);
+        } else if constexpr (kCap >= 16) {
+          ASAMD_STREAM_LAUNCH(16, 1);
+        } else {
+          ASAMD_STREAM_LAUNCH(8, 1);
+        }
+      } else {
+        ASAMD_STREAM_LAUNCH(4, 1);
+      }
+    } else if (g == 2) {
+      ASAMD_STREAM_LAUNCH(kCap, 2);
+    } else if (g == 4) {
+      ASAMD_STREAM_LAUNCH(kCap, 4);
+    } else if (g == 8) {
+      ASAMD_STREAM_LAUNCH(kCap, 8);
+    } else {
+      ASAMD_STREAM_LAUNCH(kCap, 16);
+    }
+#undef ASAMD_STREAM_LAUNCH
+    return hipGetLastError();
+  });
+}
+
+// ---- merge-path ------------------------------------------------------------------------------------
+extern "C" int asamd_merge_partition(hipStream_t s, int32_t m, int32_t nnz, const int32_t* row_ptr, int32_t base,
+                                     int32_t blocks, int32_t items_per_block, int32_t* block_row) {
+  if (!row_ptr || !block_row || m <= 0 || nnz < 0 || blocks < 1 || items_per_block < 1) return hipErrorInvalidValue;
+  merge_partition_kernel<<<(unsigned)(((int64_t)blocks + 1 + 255) / 256), 256, 0, s>>>(m, nnz, row_ptr, base, blocks,
+                                                                                     items_per_block, block_row);
+  return hipGetLastError();
+}
+
+extern "C" int asamd_spmv_merge(hipStream_t s, const asamd_spmv_args* a, int32_t ipt, const int32_t* block_row,
+                                int32_t* carry_row, void* carry_val, void* head_val) {
+  if (!a || !block_row || !carry_row || !carry_val || !head_val) return hipErrorInvalidValue;
+  return by_dtype(a->dtype, [&](auto* tag) -> int {
+    using T = std::remove_pointer_t<decltype(tag)>;
+    if (!args_ok<T>(a)) return hipErrorInvalidValue;
+    if (ipt != 4 && ipt != 8 && ipt != 16) return hipErrorInvalidValue;
+    // LDS per workgroup grows with ipt * sizeof(T): 16-byte values run 4 items only, 8 complex bytes up to 8
+    if ((sizeof(T) == 16 && ipt != 4) || (!kIsReal<T> && ipt == 16)) return hipErrorInvalidValue;
+    const int64_t items = (int64_t)kMergeThreads * ipt;
+    const int nb = (int)(((int64_t)a->m + a->nnz + items - 1) / items);
+    const T alpha = scalar_of<T>(a->alpha), beta = scalar_of<T>(a->beta);
+    const T* val = (const T*)a->val;
+    const T* x = (const T*)a->x;
+    T* y = (T*)a->y;
+    // 128-bit loads of the streams need them 16-byte aligned
+    const bool wide = (((uintptr_t)a->val | (uintptr_t)a->col_ind) & 15u) == 0;
+    const int policy = csr_stream_policy(a, sizeof(T), true);
+#define ASAMD_LAUNCH_MERGE(IPT)                                                                                      \
+  do {                                                                                                               \
+    if (wide)                                                                                                        \
+      spmv_merge_kernel<T, IPT, true><<<nb, kMergeThreads, 0, s>>>(a->m, a->nnz, alpha, val, a->row_ptr, a->col_ind, \
+                                                                   x, beta, y, a->base, block_row, carry_row,        \
+                                                                   (T*)carry_val, (T*)head_val, policy);             \
+    else                                                                                                             \
+      spmv_merge_kernel<T, IPT><<<nb, kMergeThreads, 0, s>>>(a->m, a->nnz, alpha, val, a->row_ptr, a->col_ind, x,    \
+                                                             beta, y, a->base, block_row, carry_row, (T*)carry_val,  \
+                                                             (T*)head_val);                                          \
+  } while (0)
+    if constexpr (sizeof(T) <= 8) {
+      if constexpr (kIsReal<T>) {
+        if (ipt == 16) ASAMD_LAUNCH_MERGE(16);
+        else if (ipt == 8) ASAMD_LAUNCH_MERGE(8);
+        else ASAMD_LAUNCH_MERGE(4);
+      } else {
+        if (ipt == 8) ASAMD_LAUNCH_MERGE(8);
+        else ASAMD_LAUNCH_MERGE(4);
+      }
+    } else {
+      ASAMD_LAUNCH_MERGE(4);
+    }
+#undef ASAMD_LAUNCH_MERGE
+    if (nb > 1)
+      merge_fixup_kernel<T><<<(nb + 255) / 256, 256, 0, s>>>(nb, a->m, alpha, beta, carry_row, (const T*)carry_val,
+                                                             (const T*)head_val, y);
+    return hipGetLastError();
+  });
+}
+
+// ---- transposed product as an atomic scatter ------------------------------------------------------
+template <typename T, int W, bool CONJ>
+static void launch_trans_scatter(hipStream_t s, const asamd_spmv_args* a) {
+  constexpr int rows_per_block = kTransThreads / W;
+  const unsigned grid = (unsigned)(((int64_t)a->m + rows_per_block - 1) / rows_per_block);
+  csrmv_trans_scatter_kernel<T, W, CONJ><<<grid, kTransThreads, 0, s>>>(a->m, a->n, scalar_of<T>(a->alpha),
+                                                                         (const T*)a->val, a->row_ptr, a->col_ind,
+                                                                         (const T*)a->x, (T*)a->y, a->base);
+}
+
+template <typename T, bool CONJ>
+static int trans_scatter(hipStream_t s, const asamd_spmv_args* a, int width) {
+  switch (width) {
+    case 1: launch_trans_scatter<T, 1, CONJ>(s, a); break;
+    case 2: launch_trans_scatter<T, 2, CONJ>(s, a); break;
+    case 4: launch_trans_scatter<T, 4, CONJ>(s, a); break;
+    case 8: launch_trans_scatter<T, 8, CONJ>(s, a); break;
+    case 16: launch_trans_scatter<T, 16, CONJ>(s, a); break;
+    case 32: launch_trans_scatter<T, 32, CONJ>(s, a); break;
+    case 64: launch_trans_scatter<T, 64, CONJ>(s, a); break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
+extern "C" int asamd_spmv_trans_scatter(hipStream_t s, const asamd_spmv_args* a, int32_t width, int32_t conj) {
+  if (!a) return hipErrorInvalidValue;
+  return by_dtype(a->dtype, [&](auto* tag) -> int {
+    using T = std::remove_pointer_t<decltype(tag)>;
+    if (!args_ok<T>(a) || a->n <= 0 || (conj && kIsReal<T>)) return hipErrorInvalidValue;
+    const T beta = scalar_of<T>(a->beta);
+    if (beta != T(1))
+      scale_vec_kernel<T><<<(unsigned)(((int64_t)a->n + 255) / 256), 256, 0, s>>>(a->n, beta, (T*)a->y);
+    if constexpr (!kIsReal<T>) {
+      if (conj) return trans_scatter<T, true>(s, a, width);
+    }
+    return trans_scatter<T, false>(s, a, width);
+  });
+}
+
+// ---- the unanalysed, one-lane-per-row path ("plain") ---------------------------------------------
+// op 0: every row summed by one lane in storage order; op 1 / 2: y scaled by beta, then one lane per
+// row scatters alpha*op(a)*x[row] with atomics, the traversal of the reference's own transposed kernels.
+template <typename T>
+static int csrmv_plain_impl(hipStream_t s, int32_t op, int32_t m, int32_t n, int32_t base, T alpha, const T* val,
+                            const int* rp, const int* ci, const T* x, T beta, T* y) {
+  if (m <= 0 || n <= 0 || op < 0 || op > 2 || (op == 2 && kIsReal<T>)) return hipErrorInvalidValue;
+  asamd_spmv_args a;
+  a.dtype = DtypeOf<T>::value;
+  a.m = m;
+  a.n = n;
+  a.nnz = 0;  // not read by these two kernels
+  a.base = base;
+  a.alpha = &alpha;
+  a.beta = &beta;
+  a.val = val;
+  a.row_ptr = rp;
+  a.col_ind = ci;
+  a.x = x;
+  a.y = y;
+  if (op == 0) return asamd_spmv_scalar(s, &a);
+  return asamd_spmv_trans_scatter(s, &a, 1, op == 2);
+}
+
+extern "C" int asamd_s_csrmv_plain(hipStream_t stream, int32_t op, int32_t m, int32_t n, int32_t base, float alpha,
+                                   const float* val, const int32_t* row_ptr, const int32_t* col_ind, const float* x,
+                                   float beta, float* y) {
+  return csrmv_plain_impl<float>(stream, op, m, n, base, alpha, val, row_ptr, col_ind, x, beta, y);
+}
+
+extern "C" int asamd_d_csrmv_plain(hipStream_t stream, int32_t op, int32_t m, int32_t n, int32_t base, double alpha,
+                                   const double* val, const int32_t* row_ptr, const int32_t* col_ind, const double* x,
+                                   double beta, double* y) {
+  return csrmv_plain_impl<double>(stream, op, m, n, base, alpha, val, row_ptr, col_ind, x, beta, y);
+}
+
+extern "C" int asamd_c_csrmv_plain(hipStream_t stream, int32_t op, int32_t m, int32_t n, int32_t base,
+                                   asamd_complex8 alpha, const asamd_complex8* val, const int32_t* row_ptr,
+                                   const int32_t* col_ind, const asamd_complex8* x, asamd_complex8 beta,
+                                   asamd_complex8* y) {
+  using T = Cx<float>;
+  return csrmv_plain_impl<T>(stream, op, m, n, base, T(alpha.real, alpha.imag), (const T*)val, row_ptr, col_ind,
+                             (const T*)x, T(beta.real, beta.imag), (T*)y);
+}
+
+extern "C" int asamd_z_csrmv_plain(hipStream_t stream, int32_t op, int32_t m, int32_t n, int32_t base,
+                                   asamd_complex16 alpha, const asamd_complex16* val, const int32_t* row_ptr,
+                                   const int32_t* col_ind, const asamd_complex16* x, asamd_complex16 beta,
+                                   asamd_complex16* y) {
+  using T = Cx<double>;
+  return csrmv_plain_impl<T>(stream, op, m, n, base, T(alpha.real, alpha.imag), (const T*)val, row_ptr, col_ind,
+                             (const T*)x, T(beta.real, beta.imag), (T*)y);
+}

@@ -49,7 +49,7 @@ __device__ __forceinline__ int lds_pad(int i) { return i + (i >> 5); }
 
 // block_row[b] = number of rows whose end offset is consumed before merge
 // diagonal b*items_per_block, for b in [0, nblocks].
-__global__ __launch_bounds__(256) void merge_partition_kernel(int m, int nnz,
+static __global__ __launch_bounds__(256) void merge_partition_kernel(int m, int nnz,
                                                               const int* __restrict__ row_ptr,
                                                               int base, int nblocks,
                                                               int items_per_block,

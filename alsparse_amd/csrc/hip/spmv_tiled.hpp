@@ -119,7 +119,7 @@ struct LongFinish {  // a row block whose long tiles were dealt to several workg
 // columns) stay few.  Runs of consecutive entries hold whole rows, so the sample is not biased
 // towards any position inside a row.
 constexpr int kCountRun = 1024;
-__global__ __launch_bounds__(256) void col_group_count_kernel(int nnz, const int* __restrict__ col_ind,
+static __global__ __launch_bounds__(256) void col_group_count_kernel(int nnz, const int* __restrict__ col_ind,
                                                               int base, int stride, int* __restrict__ count) {
   const int64_t runs = ((int64_t)nnz + kCountRun - 1) / kCountRun;
   for (int64_t run = (int64_t)blockIdx.x * stride; run < runs; run += (int64_t)gridDim.x * stride) {
@@ -132,7 +132,7 @@ __global__ __launch_bounds__(256) void col_group_count_kernel(int nnz, const int
 }
 
 // out[g] = row_ptr[g * 64] for g in [0, groups], the last one clamped to row_ptr[m].
-__global__ __launch_bounds__(256) void row_group_offsets_kernel(int m, const int* __restrict__ row_ptr,
+static __global__ __launch_bounds__(256) void row_group_offsets_kernel(int m, const int* __restrict__ row_ptr,
                                                                 int groups, int* __restrict__ out) {
   const int g = blockIdx.x * blockDim.x + threadIdx.x;
   if (g > groups) return;
@@ -144,7 +144,7 @@ __global__ __launch_bounds__(256) void row_group_offsets_kernel(int m, const int
 // key[k] = col_block * row_blocks + row_block of entry k; idx[k] = k.
 // coo_row holds the row of every entry in the matrix's index base; the block of
 // a column / row is looked up through its group.
-__global__ __launch_bounds__(256) void tile_keys_kernel(int nnz, const int* __restrict__ coo_row,
+static __global__ __launch_bounds__(256) void tile_keys_kernel(int nnz, const int* __restrict__ coo_row,
                                                         const int* __restrict__ col_ind, int base,
                                                         const int* __restrict__ col_group_block,
                                                         const int* __restrict__ row_group_block,
@@ -165,7 +165,7 @@ __global__ __launch_bounds__(256) void tile_keys_kernel(int nnz, const int* __re
 // entry and stream (18 ms for 2^28 entries, against 3 ms more in the sort and a streaming unpack); only
 // the values are gathered that way (gather_values_kernel), and the permutation is kept so that they can
 // be gathered again when the caller has changed them.
-__global__ __launch_bounds__(256) void tile_keys_payload_kernel(
+static __global__ __launch_bounds__(256) void tile_keys_payload_kernel(
     int nnz, const int* __restrict__ coo_row, const int* __restrict__ col_ind,
     int base, const int* __restrict__ col_group_block, const int* __restrict__ col_block_start,
     const int* __restrict__ row_group_block, const int* __restrict__ row_block_start, int row_blocks,
@@ -181,7 +181,7 @@ __global__ __launch_bounds__(256) void tile_keys_payload_kernel(
   }
 }
 
-__global__ __launch_bounds__(256) void tile_unpack_kernel(int nnz, const unsigned long long* __restrict__ payload,
+static __global__ __launch_bounds__(256) void tile_unpack_kernel(int nnz, const unsigned long long* __restrict__ payload,
                                                           unsigned* __restrict__ t_perm,
                                                           unsigned short* __restrict__ t_col,
                                                           unsigned short* __restrict__ t_row) {
@@ -195,10 +195,13 @@ __global__ __launch_bounds__(256) void tile_unpack_kernel(int nnz, const unsigne
 }
 
 // out[q] = val[perm[q]] (CONJ: conjugated): the values of a re-ordered copy, taken afresh from the
-// caller's array.  Eight gathers in flight per lane.
+// caller's array.  Eight gathers in flight per lane.  gate: null, or a flag left by the value guard --
+// zero means that the values have not changed, and the kernel returns at once.
 template <typename T, bool CONJ>
 __global__ __launch_bounds__(256) void gather_values_kernel(int nnz, const unsigned* __restrict__ perm,
-                                                            const T* __restrict__ val, T* __restrict__ out) {
+                                                            const T* __restrict__ val, T* __restrict__ out,
+                                                            const int* __restrict__ gate) {
+  if (gate && *gate == 0) return;
   constexpr int kU = 8;
   const int64_t stride = (int64_t)gridDim.x * 256;
   int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -213,29 +216,6 @@ __global__ __launch_bounds__(256) void gather_values_kernel(int nnz, const unsig
     for (int u = 0; u < kU; ++u) out[q + u * stride] = CONJ ? conj_t(v[u]) : v[u];
   }
   for (; q < nnz; q += stride) out[q] = CONJ ? conj_t(val[perm[q]]) : val[perm[q]];
-}
-
-// hash[0] += sum over i of mix(a[i], i + salt): a fingerprint of an index array that does not depend on
-// the order of the (integer, wrapping) additions.
-__device__ __forceinline__ unsigned long long mix_index(unsigned long long v, unsigned long long i) {
-  unsigned long long z = (v + 0x9E3779B97F4A7C15ull) * 0xBF58476D1CE4E5B9ull ^ (i * 0x94D049BB133111EBull);
-  z = (z ^ (z >> 29)) * 0xD6E8FEB86659FD93ull;
-  return z ^ (z >> 32);
-}
-__global__ __launch_bounds__(256) void index_hash_kernel(int64_t n, const int* __restrict__ a, unsigned long long salt,
-                                                         unsigned long long* __restrict__ hash) {
-  __shared__ unsigned long long s_sum[256 / kWave];
-  unsigned long long mine = 0;
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
-    mine += mix_index((unsigned long long)(unsigned)nt_load(a + i), (unsigned long long)i + salt);
-  for (int d = kWave / 2; d > 0; d >>= 1) mine += __shfl_down(mine, d, kWave);
-  if (threadIdx.x % kWave == 0) s_sum[threadIdx.x / kWave] = mine;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    unsigned long long total = 0;
-    for (int w = 0; w < 256 / kWave; ++w) total += s_sum[w];
-    atomicAdd(hash, total);
-  }
 }
 
 // Entries in sorted order: values, columns and rows local to their blocks.
@@ -257,7 +237,7 @@ __global__ __launch_bounds__(256) void tile_gather_kernel(
 }
 
 // tile_ptr[t] = first position whose key is >= t, for t in [0, tiles].
-__global__ __launch_bounds__(256) void tile_bounds_kernel(int nnz, const unsigned* __restrict__ sorted_key,
+static __global__ __launch_bounds__(256) void tile_bounds_kernel(int nnz, const unsigned* __restrict__ sorted_key,
                                                           int64_t tiles, int* __restrict__ tile_ptr) {
   const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (t > tiles) return;
@@ -272,7 +252,7 @@ __global__ __launch_bounds__(256) void tile_bounds_kernel(int nnz, const unsigne
 
 // out[0] += entries held by tiles of more than kWave and at most kLongTile entries (one atomic per
 // workgroup): phase 2 handles those only in its two-entries-per-lane form.
-__global__ __launch_bounds__(256) void tile_mid_entries_kernel(int64_t tiles, const int* __restrict__ tile_ptr,
+static __global__ __launch_bounds__(256) void tile_mid_entries_kernel(int64_t tiles, const int* __restrict__ tile_ptr,
                                                                unsigned long long* __restrict__ out) {
   __shared__ unsigned long long s_sum[256 / kWave];
   unsigned long long mine = 0;
@@ -293,7 +273,7 @@ __global__ __launch_bounds__(256) void tile_mid_entries_kernel(int64_t tiles, co
 // Phase 2 reads the tile table row block by row block:
 // ranges[rb * col_blocks + cb] = {tile_ptr[cb*row_blocks + rb], tile_ptr[cb*row_blocks + rb + 1]}.
 // Tiles longer than long_tile go to long_list instead (their range is left empty).
-__global__ __launch_bounds__(256) void tile_ranges_kernel(int row_blocks, int col_blocks, int long_tile,
+static __global__ __launch_bounds__(256) void tile_ranges_kernel(int row_blocks, int col_blocks, int long_tile,
                                                           const int* __restrict__ tile_ptr,
                                                           TileRange* __restrict__ ranges,
                                                           LongTile* __restrict__ long_list,

@@ -20,7 +20,7 @@
 namespace asamd {
 
 // key[k] = zero-based column of entry k, idx[k] = k
-__global__ __launch_bounds__(256) void transpose_keys_kernel(int nnz, const int* __restrict__ col_ind, int base,
+static __global__ __launch_bounds__(256) void transpose_keys_kernel(int nnz, const int* __restrict__ col_ind, int base,
                                                              unsigned* __restrict__ key,
                                                              unsigned* __restrict__ idx) {
   for (int64_t k = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; k < nnz;

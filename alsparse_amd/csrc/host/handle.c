@@ -157,6 +157,32 @@ alphasparse_status_t alphasparse_dcu_destroy_mat_info(alphasparse_dcu_mat_info_t
   return ALPHA_SPARSE_STATUS_SUCCESS;
 }
 
+/* The handle's scratch buffer serves whatever the current call needs (reference: sized once,
+ * src/util_cpp/handle.cpp:94-105): multiplies carve their per-call scratch from it, column-major csrmm
+ * keeps a row-major copy of B in it.  Calls on one handle are ordered by its stream, so they can share it. */
+int asamd_handle_reserve(void *handle, size_t bytes) {
+  alphasparse_dcu_handle_t h = (alphasparse_dcu_handle_t)handle;
+  if (!h) return (int)ALPHA_SPARSE_STATUS_INVALID_HANDLE;
+  if (bytes <= h->buffer_size) return (int)ALPHA_SPARSE_STATUS_SUCCESS;
+  /* a stream that is being captured can neither be waited for nor may memory be allocated under it:
+   * the buffer stays, and the caller makes do with it */
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(h->stream, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
+    (void)hipGetLastError();
+    return (int)ALPHA_SPARSE_STATUS_SUCCESS;
+  }
+  ASAMD_HIP_STATUS(hipStreamSynchronize(h->stream));
+  void *bigger = NULL;
+  if (hipMalloc(&bigger, bytes) != hipSuccess) {
+    (void)hipGetLastError(); /* no room: the caller makes do with the buffer there is */
+    return (int)ALPHA_SPARSE_STATUS_SUCCESS;
+  }
+  (void)hipFree(h->buffer);
+  h->buffer = bigger;
+  h->buffer_size = bytes;
+  return (int)ALPHA_SPARSE_STATUS_SUCCESS;
+}
+
 /* The stream lives in a public struct field (handle->stream), which C callers set themselves as
  * with the reference; these two are for bindings that cannot see the struct layout. */
 int asamd_handle_set_stream(void *handle, hipStream_t stream) {

@@ -130,20 +130,41 @@ static alphasparse_status_t asamd_host_prepare(const alphasparse_matrix_t A, alp
     if (!r) return ALPHA_SPARSE_STATUS_INTERNAL_ERROR;
   }
   /* The host arrays stay the caller's to change (alphasparse_?_export_csr hands out pointers into them, and
-   * the reference's CPU kernels read them on every call).  A cheap fingerprint of a sample of the values tells
-   * when they have been rewritten: the mirror's values are copied again and the copies that its analysis
-   * keeps are refreshed.  (A change of a few single values can slip through the sample: host2device_?_csr
-   * mirrors afresh.) */
+   * the reference's CPU kernels read them on every call).  Every call therefore fingerprints ALL of the values
+   * and of the structure arrays (one streaming pass over the OpenMP threads): changed values are copied to the
+   * mirror again and the copies that its analysis keeps are refreshed; a changed structure gets a new mirror
+   * and a new analysis.  ALSPARSE_AMD_HOST_CHECK=off promises that the host arrays stay as they were when they
+   * were mirrored and skips the pass. */
+  static int check = -1;
+  if (check < 0) {
+    const char *ev = getenv("ALSPARSE_AMD_HOST_CHECK");
+    check = !(ev && !strcmp(ev, "off"));
+  }
   static const size_t kElem[4] = {4, 8, 8, 16};
   const size_t elem = kElem[A->datatype & 3];
   const size_t nnz = (size_t)(m->rows > 0 && m->rows_end[m->rows - 1] > 0 ? m->rows_end[m->rows - 1] : 0);
-  if (nnz > 0 && r->plan) {
-    const uint64_t fp = asamd_host_fingerprint(m->values, nnz, elem);
-    if (fp != r->host_val_fingerprint) {
+  if (check) {
+    const uint64_t ifp = asamd_host_fingerprint(m->rows_start, sizeof(ALPHA_INT) * (size_t)(m->rows + 1)) ^
+                         (asamd_host_fingerprint(m->col_indx, sizeof(ALPHA_INT) * nnz) * 3);
+    if (ifp != r->host_idx_fingerprint || (int32_t)nnz != r->nnz) {
       ASAMD_HIP_STATUS(hipStreamSynchronize((*h)->stream));
-      ASAMD_HIP_STATUS(hipMemcpy(m->d_values, m->values, nnz * elem, hipMemcpyHostToDevice));
-      ASAMD_HIP_STATUS(asamd_csr_plan_refresh_values((*h)->stream, r->plan, m->d_row_ptr, m->d_col_indx, m->d_values));
-      r->host_val_fingerprint = fp;
+      switch (A->datatype) {
+        case ALPHA_SPARSE_DATATYPE_FLOAT: st = host2device_s_csr(A); break;
+        case ALPHA_SPARSE_DATATYPE_DOUBLE: st = host2device_d_csr(A); break;
+        case ALPHA_SPARSE_DATATYPE_FLOAT_COMPLEX: st = host2device_c_csr(A); break;
+        default: st = host2device_z_csr(A); break;
+      }
+      if (st != ALPHA_SPARSE_STATUS_SUCCESS) return st;
+      r = asamd_registry_find(ASAMD_KEY_MATRIX, m->d_row_ptr);
+      if (!r) return ALPHA_SPARSE_STATUS_INTERNAL_ERROR;
+    } else if (nnz > 0 && r->plan) {
+      const uint64_t fp = asamd_host_fingerprint(m->values, nnz * elem);
+      if (fp != r->host_val_fingerprint) {
+        ASAMD_HIP_STATUS(hipStreamSynchronize((*h)->stream));
+        ASAMD_HIP_STATUS(hipMemcpy(m->d_values, m->values, nnz * elem, hipMemcpyHostToDevice));
+        ASAMD_HIP_STATUS(asamd_csr_plan_refresh_values((*h)->stream, r->plan, m->d_row_ptr, m->d_col_indx, m->d_values));
+        r->host_val_fingerprint = fp;
+      }
     }
   }
   *rec = r;

@@ -8,6 +8,7 @@
 
 #include "alpha_spblas_dcu.h"
 #include "alsparse_amd_kernels.h"
+#include "alsparse_amd_plan.h"
 
 /* How an analysis record is looked up. */
 typedef enum {
@@ -33,8 +34,9 @@ typedef struct asamd_record {
   /* explicit analyses: fingerprint of the structure arrays at analysis time (asamd_csr_structure_hash) */
   uint64_t structure_hash;
   int has_structure_hash;
-  /* library-built mirrors: fingerprint of a sample of the HOST values at the time they were copied */
+  /* library-built mirrors: fingerprints of the HOST values and structure arrays at the time they were copied */
   uint64_t host_val_fingerprint;
+  uint64_t host_idx_fingerprint;
   /* host-pointer entry points: device staging for x / y (ASAMD_KEY_MATRIX only) */
   void *d_in;
   size_t d_in_bytes;
@@ -66,17 +68,18 @@ void asamd_registry_drop_handle(const void *handle);
 /* number of lazy records alive (tests) */
 int asamd_registry_lazy_count(void);
 
-/* Fingerprint of up to 1024 evenly spread elements (elem bytes each) of a host array: cheap enough to
- * take on every host-pointer multiply, and changes whenever a caller has rewritten the array as a whole. */
-uint64_t asamd_host_fingerprint(const void *values, size_t count, size_t elem);
+/* Fingerprint of EVERY byte of a host array (one streaming pass spread over the OpenMP threads): taken on
+ * every host-pointer multiply of the values and of both index arrays, because the reference's CPU kernels
+ * read the caller's arrays on every call and alphasparse_?_export_csr hands out pointers into them. */
+uint64_t asamd_host_fingerprint(const void *data, size_t bytes);
 
 /* Process-wide handle for alphasparse_?_mv / _mm (host pointers). */
 alphasparse_status_t asamd_default_handle(alphasparse_dcu_handle_t *handle);
 
 /* ALSPARSE_AMD_SPMV_ALGO = auto | vector | rowconst | merge | scalar | tiled | stream | ell | hot | binned */
 int asamd_env_algo(void);
-/* ALSPARSE_AMD_ANALYSIS = structure: analyses keep no copies of the matrix values (as the reference's),
- * so values may change in place at any time; the default lets an analysis keep re-ordered copies. */
+/* ALSPARSE_AMD_ANALYSIS = structure: analyses keep no copies of the matrix values (as the reference's);
+ * the default lets an analysis keep re-ordered copies, which every multiply checks against csr_val. */
 int asamd_env_structure_only(void);
 
 /* device arrays of values must be aligned to their element size (one element = one load) */

@@ -1,0 +1,1036 @@
+/* The CSR analysis object: row statistics -> kernel family, the copies that win the analysis, and the
+ * dispatch of a multiply to the launcher of its family (include/alsparse_amd_plan.h).
+ *
+ * Stands in for the reference's host-side analysis (src/util_cpp/alphasparse_dcu_x_csrmv_analysis.cpp:58-391:
+ * a serial walk over row_ptr that builds CSR-adaptive row blocks no kernel reads) and for
+ * csr_gemv_vector_dispatch (src/kernel/dcu/level2/mv/csrmv/dcu_gemv_vector.h:59-182: lanes per row from
+ * the mean row length).  Everything that touches the GPU goes through the launchers and layout builders of
+ * include/alsparse_amd_kernels.h; this file decides, owns memory and carves the per-call workspace. */
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "internal.h"
+
+typedef struct {
+  asamd_transpose_layout t;
+  asamd_csr_plan *plan;    /* the analysis of the copy */
+  const void *val_src;     /* the value array that t.val was gathered from */
+} asamd_trans_copy;
+
+struct asamd_csr_plan {
+  asamd_csr_stats st;
+  int auto_algo;           /* the analysis' choice */
+  int struct_algo;         /* the choice from the row statistics alone (no copy involved) */
+  int auto_width;
+  int dtype;               /* ASAMD_DTYPE_*: element type of the values */
+  int val_size;            /* bytes per value */
+  int merge_ipt;           /* items per thread of the merge-path kernel (4, 8 or 16) */
+  int32_t *d_block_row;    /* merge-path coordinates of a structure promised fixed, merge_blocks + 1 ints */
+  asamd_tiled_layout tiled;
+  asamd_hot_layout hot;
+  asamd_binned_layout binned;
+  void *d_eval;            /* ELL copy: ell_width * m values, column-major */
+  int32_t *d_ecol;         /* ... and zero-based columns */
+  const void *copy_val_src; /* the value array that the tiled / ELL copy was taken from */
+  asamd_trans_copy tr[2];  /* CSR copies of the transpose [0] and of the conjugate transpose [1] */
+  int lazy_transpose;      /* build a copy on the first transposed multiply */
+  uint64_t *d_fp;          /* 3 device words: fingerprints of the values that the copies were taken from
+                              (tiled / ELL, A^T, A^H) */
+  void *d_setup;           /* device scratch of the plan's own set-up work (statistics, first fingerprints) */
+};
+
+#define SETUP_BYTES (ASAMD_GUARD_WS_BYTES + 1024)
+
+static const int kValSize[4] = {4, 8, 8, 16};
+
+/* rows plus entries below which one launch's latency outweighs the work */
+#define SMALL_WORK ((int64_t)1 << 17)
+
+static int is_complex(const asamd_csr_plan *p) { return p->dtype >= ASAMD_DTYPE_FLOAT_COMPLEX; }
+
+/* ---- environment switches (read once) ------------------------------------------------------------ */
+static int env_int(const char *name, int fallback) {
+  const char *e = getenv(name);
+  return e && *e ? atoi(e) : fallback;
+}
+
+static int env_value_check(void) {
+  const char *e = getenv("ALSPARSE_AMD_VALUE_CHECK");
+  if (e && !strcmp(e, "off")) return 0;
+  if (e && !strcmp(e, "full")) return 2;
+  return 1;
+}
+
+static int env_tune_model(void) {
+  const char *e = getenv("ALSPARSE_AMD_TUNE");
+  return e && !strcmp(e, "model");
+}
+
+/* ---- kernel choice from the row statistics --------------------------------------------------------- */
+static int width_for_mean(double mean) {
+  /* lanes per row from the mean row length; same break points as the
+   * reference's dispatch (dcu_gemv_vector.h:77,94,111,128,145,162) */
+  if (mean < 4) return 2;
+  if (mean < 8) return 4;
+  if (mean < 16) return 8;
+  if (mean < 32) return 16;
+  if (mean < 64) return 32;
+  return 64;
+}
+
+static int rowconst_ok(const asamd_csr_plan *p) {
+  const asamd_csr_stats *st = &p->st;
+  const int L = st->const_len;
+  /* the kernel loads four values as 128-bit pieces: real element types only */
+  return !is_complex(p) && st->trusted && st->first_offset == 0 &&
+         (L == 4 || L == 8 || L == 16 || L == 32 || L == 64 || L == 128 || L == 256);
+}
+
+/* The LDS-staged row-block kernel sizes its staging area for rows of at most cap * G entries (G lanes sum a
+ * row); the bound comes from the row statistics.  A workgroup whose rows hold more than that (the structure
+ * behind row_ptr changed under a plan that was not promised a fixed one) takes them straight from global
+ * memory, so the choice is safe for such plans too.  Returns G, or 0 when the kernel cannot take the matrix.
+ * With `regular_only`, also 0 for G > 1 when the rows are so much shorter than the longest that a workgroup's
+ * 256 / G rows hold fewer than four entries per thread.
+ * 16 KiB of products per workgroup: 16 entries per thread for 4-byte values, 8 for 8-byte, 4 for 16-byte ones
+ * (measured on a 27-point stencil, fp64: 32 KiB per workgroup 317 us, 16 KiB 295 us) */
+static int stream_cap(const asamd_csr_plan *p) { return 64 / p->val_size; }
+static int stream_group(const asamd_csr_plan *p, int regular_only) {
+  const asamd_csr_stats *st = &p->st;
+  if (st->max_len < 1) return 0;
+  const int cap = stream_cap(p);
+  if (st->max_len <= cap) return 1;
+  int g = 2;
+  while (g * cap < st->max_len && g <= ASAMD_STREAM_MAX_GROUP) g *= 2;
+  if (g > ASAMD_STREAM_MAX_GROUP) return 0;
+  /* regular: the mean row is at least a quarter of the longest row the kernel is sized for */
+  if (regular_only && (double)st->nnz / (double)st->m < 0.25 * g * cap) return 0;
+  return g;
+}
+static int stream_ok(const asamd_csr_plan *p) { return stream_group(p, 0) > 0; }
+
+static void choose_algo(asamd_csr_plan *p) {
+  asamd_csr_stats *st = &p->st;
+  const double mean = st->m > 0 ? (double)st->nnz / st->m : 0.0;
+  const int w = width_for_mean(mean);
+  p->auto_width = w;
+  if (st->first_offset != 0) {
+    /* row_ptr points into the middle of a larger array: only the kernels that index with the absolute
+     * offsets (as the reference's csr_gemv_vector does) see the right entries; merge-path and csr2coo,
+     * the source of every re-ordered copy, count entries from position 0 */
+    p->auto_algo = stream_group(p, 1) > 0 ? ASAMD_SPMV_STREAM : ASAMD_SPMV_VECTOR;
+  } else if (rowconst_ok(p)) {
+    p->auto_algo = ASAMD_SPMV_ROWCONST;
+  } else if (stream_group(p, 1) > 0) {
+    /* short rows, or rows of some tens of entries of similar lengths */
+    p->auto_algo = ASAMD_SPMV_STREAM;
+  } else if ((int64_t)st->max_len <= (int64_t)w * 16 && mean >= 6.0) {
+    /* regular rows: a lane group per row wastes little and needs no LDS */
+    p->auto_algo = ASAMD_SPMV_VECTOR;
+  } else if ((int64_t)st->m + st->nnz <= SMALL_WORK && (int64_t)st->max_len <= (int64_t)w * 64) {
+    /* a matrix this small is over in the time of one launch: the single kernel beats the balanced
+     * path's two or three */
+    p->auto_algo = ASAMD_SPMV_VECTOR;
+  } else {
+    p->auto_algo = ASAMD_SPMV_MERGE;
+  }
+  p->struct_algo = p->auto_algo;
+  st->algo = p->auto_algo;
+  st->vector_width = p->auto_width;
+}
+
+/* ---- which copies a matrix is eligible for -------------------------------------------------------- */
+/* An ELL copy pays when rows are short and padding them to the longest costs little: the kernel then
+ * streams 4 + sizeof(T) bytes per entry at full width with neither row_ptr nor LDS staging. */
+static int ell_eligible(const asamd_csr_stats *st, int force) {
+  if (!st->trusted || st->first_offset != 0 || st->max_len < 1 || st->max_len > 32) return 0;
+  const int64_t slots = (int64_t)st->m * st->max_len;
+  if (slots >= ((int64_t)1 << 31) || slots > (int64_t)st->nnz + st->nnz / 8) return 0;
+  return force || st->nnz >= (1 << 18);
+}
+
+static int tiled_eligible(const asamd_csr_plan *p, int force) {
+  const asamd_csr_stats *st = &p->st;
+  if (!st->trusted || st->first_offset != 0 || !asamd_tiled_fits(p->dtype, st->m, st->n, st->nnz)) return 0;
+  /* worth a try only when x fills an XCD's 4 MiB L2 (the matrix streams through the same cache; with
+   * 2 MiB of x the tiled pair measured 0.43 ms against 0.34 ms, with 4 MiB 0.084 against 0.095) and the
+   * matrix is large; the comparison inside the analysis has the last word */
+  return force || ((int64_t)st->n * (int64_t)p->val_size >= ((int64_t)4 << 20) && st->nnz >= (1 << 22));
+}
+
+static int hot_eligible(const asamd_csr_plan *p, int force) {
+  const asamd_csr_stats *st = &p->st;
+  if (p->val_size > 8 || !st->trusted || st->first_offset != 0 || st->nnz < 1 || st->n < 1) return 0;
+  /* positions are 32-bit words, x is addressed through a buffer resource with 32-bit byte offsets */
+  if (((int64_t)st->n + ((int64_t)1 << 20)) >= (int64_t)UINT32_MAX) return 0;
+  if ((int64_t)st->m + st->nnz >= (int64_t)INT32_MAX / 2) return 0;
+  if (force) return 1;
+  /* Not tried unless asked for (ALSPARSE_AMD_TUNE_HOT=1): counting and ranking the columns costs several
+   * multiplies, and on the power-law matrices it is meant for the kernel gained 4 % where a copy has to
+   * gain 5 % to be kept. */
+  const char *pick = getenv("ALSPARSE_AMD_TUNE_PICK");
+  const int asked = env_int("ALSPARSE_AMD_TUNE_HOT", 0) > 0 || (pick && !strcmp(pick, "hot"));
+  return asked && (int64_t)st->n * (int64_t)p->val_size >= ((int64_t)8 << 20) && st->nnz >= (1 << 22);
+}
+
+static int binned_eligible(const asamd_csr_plan *p, int force) {
+  const asamd_csr_stats *st = &p->st;
+  if (!st->trusted || st->m < 1 || st->nnz < 1) return 0;
+  if (force) return 1;
+  if (st->nnz < (1 << 20) || st->max_len <= 8) return 0;
+  /* rows that differ enough in length for one mapping not to fit: the structural choice was merge-path, or
+   * a lane group per row whose width (from the MEAN length) leaves three quarters of the lanes idle on a
+   * quarter of the rows (row-length histogram: bin b holds the rows of 2^(b-1) .. 2^b - 1 entries) */
+  if (p->auto_algo == ASAMD_SPMV_MERGE) return st->max_len > 64;
+  if (p->auto_algo != ASAMD_SPMV_VECTOR) return 0;
+  int64_t short_rows = 0;
+  for (int b = 0; b < ASAMD_HIST_BINS && ((int64_t)1 << b) <= p->auto_width / 4; ++b) short_rows += st->hist[b];
+  return short_rows * 4 >= (int64_t)st->m;
+}
+
+/* Whether the structural choice has rivals that need no copy either (merge-path, a lane group per row): it has
+ * when it is a lane group per row or a staged block with several lanes per row, merge-path can run (row_ptr
+ * starts at the base) and the matrix is not so small that one launch's latency is all there is to time. */
+static int structural_alternatives(const asamd_csr_plan *p) {
+  const asamd_csr_stats *st = &p->st;
+  if (st->first_offset != 0 || (int64_t)st->m + st->nnz <= SMALL_WORK) return 0;
+  return p->auto_algo == ASAMD_SPMV_VECTOR || (p->auto_algo == ASAMD_SPMV_STREAM && stream_group(p, 0) > 1);
+}
+
+/* ---- copies: lay out, free, account ------------------------------------------------------------------ */
+static void free_tiled(asamd_csr_plan *p) {
+  asamd_tiled_free(&p->tiled);
+  p->st.tiled_built = 0;
+  p->st.tile_entries_per_lane = 0;
+  p->st.tile_long_blocks = 0;
+}
+
+static void free_ell(asamd_csr_plan *p) {
+  if (p->d_eval) (void)hipFree(p->d_eval);
+  if (p->d_ecol) (void)hipFree(p->d_ecol);
+  p->d_eval = NULL;
+  p->d_ecol = NULL;
+  p->st.ell_built = 0;
+}
+
+static void free_hot(asamd_csr_plan *p) {
+  asamd_hot_free(&p->hot);
+  p->st.hot_built = 0;
+}
+
+static void free_binned(asamd_csr_plan *p) {
+  asamd_binned_free(&p->binned);
+  p->st.binned_built = 0;
+}
+
+static void free_transpose(asamd_csr_plan *p, int which) {
+  asamd_trans_copy *t = &p->tr[which];
+  if (t->plan) asamd_csr_plan_destroy(t->plan);
+  asamd_transpose_free(&t->t);
+  t->plan = NULL;
+  t->val_src = NULL;
+  p->st.transpose_built &= ~(1 << which);
+}
+
+static hipError_t build_tiled(hipStream_t stream, asamd_csr_plan *p, const int32_t *row_ptr, const int32_t *col_ind,
+                              const void *val) {
+  asamd_csr_stats *st = &p->st;
+  /* ALSPARSE_AMD_TILED_HALVES = 1 | 2 forces the form of the second phase */
+  int halves = env_int("ALSPARSE_AMD_TILED_HALVES", 0);
+  if (halves != 1 && halves != 2) halves = 0;
+  hipError_t e = (hipError_t)asamd_tiled_build(stream, p->dtype, st->m, st->n, st->nnz, st->base, row_ptr, col_ind, val,
+                                               st->max_len, halves, &p->tiled);
+  if (e != hipSuccess) return e;
+  st->tile_col_blocks = p->tiled.col_blocks;
+  st->tile_row_blocks = p->tiled.row_blocks;
+  if (!p->tiled.tval) return hipSuccess; /* the matrix simply gets no tiled copy */
+  st->tiled_built = 1;
+  st->tile_entries_per_lane = p->tiled.entries_per_lane;
+  st->tile_long_blocks = p->tiled.long_blocks;
+  return hipSuccess;
+}
+
+static hipError_t build_ell(hipStream_t stream, asamd_csr_plan *p, const int32_t *row_ptr, const int32_t *col_ind,
+                            const void *val) {
+  asamd_csr_stats *st = &p->st;
+  const size_t slots = (size_t)st->m * (size_t)st->max_len;
+  hipError_t e = hipMalloc(&p->d_eval, slots * (size_t)p->val_size);
+  if (e == hipSuccess) e = hipMalloc((void **)&p->d_ecol, slots * sizeof(int32_t));
+  /* the conversion copies values bit for bit and pads with zero bits: only the element size matters */
+  if (e == hipSuccess)
+    e = (hipError_t)asamd_csr2ell_gated(stream, p->val_size, st->m, val, row_ptr, col_ind, st->base, 0, st->max_len,
+                                        p->d_eval, p->d_ecol, NULL);
+  if (e == hipSuccess) e = hipStreamSynchronize(stream);
+  if (e != hipSuccess) {
+    free_ell(p);
+    return e;
+  }
+  st->ell_built = 1;
+  st->ell_width = st->max_len;
+  return hipSuccess;
+}
+
+static hipError_t build_hot(hipStream_t stream, asamd_csr_plan *p, const int32_t *row_ptr, const int32_t *col_ind,
+                            int force) {
+  asamd_csr_stats *st = &p->st;
+  /* ALSPARSE_AMD_HOT_COLS / ALSPARSE_AMD_HOT_FRONT size the LDS table and the compact front (columns) */
+  hipError_t e = (hipError_t)asamd_hot_build(stream, p->dtype, st->m, st->n, st->nnz, st->base, row_ptr, col_ind, force,
+                                             env_int("ALSPARSE_AMD_HOT_COLS", 0), env_int("ALSPARSE_AMD_HOT_FRONT", 0),
+                                             &p->hot);
+  if (e != hipSuccess) return e;
+  st->hot_cols_lds = p->hot.cols_lds;
+  st->hot_cols = p->hot.cols_front;
+  st->hot_share_lds = p->hot.share_lds;
+  st->hot_built = p->hot.pcol != NULL;
+  return hipSuccess;
+}
+
+static hipError_t build_binned(hipStream_t stream, asamd_csr_plan *p, const int32_t *row_ptr) {
+  hipError_t e = (hipError_t)asamd_binned_build(stream, p->st.m, p->st.base, row_ptr, &p->binned);
+  if (e != hipSuccess) return e;
+  for (int c = 0; c < 4; ++c) p->st.bin_rows[c] = p->binned.count[c];
+  p->st.binned_built = p->binned.rows != NULL;
+  return hipSuccess;
+}
+
+static size_t align256(size_t b) { return (b + 255) & ~(size_t)255; }
+
+/* per-call scratch of one kernel family */
+static size_t algo_scratch(const asamd_csr_plan *p, int algo) {
+  const asamd_csr_stats *st = &p->st;
+  const size_t vs = (size_t)p->val_size;
+  switch (algo) {
+    case ASAMD_SPMV_MERGE: {
+      const size_t nb = (size_t)st->merge_blocks;
+      return (p->d_block_row ? 0 : align256((nb + 1) * 4)) + align256(nb * 4) + 2 * align256(nb * vs);
+    }
+    case ASAMD_SPMV_TILED:
+      if (!st->tiled_built) return 0;
+      return align256((size_t)st->nnz * vs) + align256((size_t)p->tiled.long_scratch_elems * vs);
+    case ASAMD_SPMV_MERGE_HOT:
+      if (!st->hot_built) return 0;
+      return align256((size_t)p->hot.cols_front * vs) + align256((size_t)p->hot.blocks * 4) +
+             2 * align256((size_t)p->hot.blocks * vs);
+    case ASAMD_SPMV_BINNED:
+      return st->binned_built ? align256((size_t)p->binned.chunks * vs) : 0;
+    default:
+      return 0;
+  }
+}
+
+static int has_value_copy(const asamd_csr_plan *p) { return p->st.tiled_built || p->st.ell_built; }
+
+size_t asamd_csr_plan_workspace_bytes(const asamd_csr_plan *p) {
+  if (!p) return 0;
+  size_t need = 0;
+  for (int a = ASAMD_SPMV_VECTOR; a <= ASAMD_SPMV_BINNED; ++a) {
+    if (a == ASAMD_SPMV_MERGE && p->st.first_offset != 0) continue;
+    const size_t s = algo_scratch(p, a);
+    if (s > need) need = s;
+  }
+  if (has_value_copy(p)) need += align256(ASAMD_GUARD_WS_BYTES);
+  for (int w = 0; w < 2; ++w)
+    if (p->tr[w].plan) {
+      const size_t s = align256(ASAMD_GUARD_WS_BYTES) + asamd_csr_plan_workspace_bytes(p->tr[w].plan);
+      if (s > need) need = s;
+    }
+  return need + 256; /* room for aligning the base up */
+}
+
+static void account(asamd_csr_plan *p) {
+  asamd_csr_stats *st = &p->st;
+  int64_t b = SETUP_BYTES + 3 * 8;
+  if (p->d_block_row) b += ((int64_t)st->merge_blocks + 1) * 4;
+  b += p->tiled.device_bytes + p->hot.device_bytes + p->binned.device_bytes;
+  if (st->ell_built) b += (int64_t)st->m * st->ell_width * ((int64_t)p->val_size + 4);
+  for (int w = 0; w < 2; ++w)
+    if (p->tr[w].plan) b += p->tr[w].t.device_bytes + p->tr[w].plan->st.device_bytes;
+  st->device_bytes = b;
+  st->workspace_bytes = (int64_t)asamd_csr_plan_workspace_bytes(p);
+}
+
+/* ---- the per-call workspace ----------------------------------------------------------------------- */
+typedef struct {
+  char *p;
+  size_t left;
+} ws_cursor;
+
+static ws_cursor ws_open(void *ws, size_t bytes) {
+  ws_cursor c = {NULL, 0};
+  if (!ws) return c;
+  const uintptr_t a = ((uintptr_t)ws + 255) & ~(uintptr_t)255;
+  const size_t skip = (size_t)(a - (uintptr_t)ws);
+  if (skip >= bytes) return c;
+  c.p = (char *)a;
+  c.left = bytes - skip;
+  return c;
+}
+
+static void *ws_take(ws_cursor *c, size_t bytes) {
+  const size_t need = align256(bytes ? bytes : 1);
+  if (!c->p || c->left < need) return NULL;
+  void *r = c->p;
+  c->p += need;
+  c->left -= need;
+  return r;
+}
+
+/* ---- launching one family --------------------------------------------------------------------------- */
+static int ellmv_any(hipStream_t s, int dtype, int32_t m, int32_t n, const void *alpha, const void *ev, const int32_t *ec,
+                     int32_t width, const void *x, const void *beta, void *y) {
+  switch (dtype) {
+    case ASAMD_DTYPE_FLOAT:
+      return asamd_s_ellmv(s, m, n, *(const float *)alpha, (const float *)ev, ec, width, 0, (const float *)x,
+                           *(const float *)beta, (float *)y);
+    case ASAMD_DTYPE_DOUBLE:
+      return asamd_d_ellmv(s, m, n, *(const double *)alpha, (const double *)ev, ec, width, 0, (const double *)x,
+                           *(const double *)beta, (double *)y);
+    case ASAMD_DTYPE_FLOAT_COMPLEX:
+      return asamd_c_ellmv(s, m, n, *(const asamd_complex8 *)alpha, (const asamd_complex8 *)ev, ec, width, 0,
+                           (const asamd_complex8 *)x, *(const asamd_complex8 *)beta, (asamd_complex8 *)y);
+    default:
+      return asamd_z_ellmv(s, m, n, *(const asamd_complex16 *)alpha, (const asamd_complex16 *)ev, ec, width, 0,
+                           (const asamd_complex16 *)x, *(const asamd_complex16 *)beta, (asamd_complex16 *)y);
+  }
+}
+
+/* The family that actually runs for a wish: every step leads to a family that needs less. */
+static int settle_algo(const asamd_csr_plan *p, int algo, const void *val, const int32_t *ci) {
+  const asamd_csr_stats *st = &p->st;
+  for (int pass = 0; pass < 6; ++pass) {
+    int next = algo;
+    if (algo == ASAMD_SPMV_AUTO) next = p->auto_algo;
+    else if (algo == ASAMD_SPMV_TILED && !st->tiled_built) next = p->auto_algo == ASAMD_SPMV_TILED ? p->struct_algo : p->auto_algo;
+    else if (algo == ASAMD_SPMV_ELL && !st->ell_built) next = p->auto_algo == ASAMD_SPMV_ELL ? p->struct_algo : p->auto_algo;
+    else if (algo == ASAMD_SPMV_MERGE_HOT && !st->hot_built) next = ASAMD_SPMV_MERGE;
+    else if (algo == ASAMD_SPMV_BINNED && !st->binned_built) next = ASAMD_SPMV_MERGE;
+    else if (algo == ASAMD_SPMV_ROWCONST &&
+             (!rowconst_ok(p) || (((uintptr_t)val | (uintptr_t)ci) & 15u) != 0)) /* 128-bit loads */
+      next = ASAMD_SPMV_VECTOR;
+    else if (algo == ASAMD_SPMV_STREAM && !stream_ok(p)) next = ASAMD_SPMV_MERGE;
+    else if (algo == ASAMD_SPMV_MERGE && st->first_offset != 0) next = ASAMD_SPMV_VECTOR;
+    if (next == algo) break;
+    algo = next;
+  }
+  return algo;
+}
+
+static int run_algo(hipStream_t s, const asamd_csr_plan *p, int algo, const asamd_spmv_args *a, ws_cursor ws) {
+  const asamd_csr_stats *st = &p->st;
+  const size_t vs = (size_t)p->val_size;
+  switch (algo) {
+    case ASAMD_SPMV_ELL:
+      /* the ELL copy holds zero-based columns and its own values */
+      return ellmv_any(s, p->dtype, st->m, st->n, a->alpha, p->d_eval, p->d_ecol, st->ell_width, a->x, a->beta, a->y);
+    case ASAMD_SPMV_TILED: {
+      void *prod = ws_take(&ws, (size_t)st->nnz * vs);
+      void *lscr = p->tiled.long_scratch_elems > 0 ? ws_take(&ws, (size_t)p->tiled.long_scratch_elems * vs) : NULL;
+      if (!prod || (p->tiled.long_scratch_elems > 0 && !lscr)) return -1;
+      return asamd_spmv_tiled(s, a, &p->tiled, prod, lscr);
+    }
+    case ASAMD_SPMV_ROWCONST:
+      return asamd_spmv_rowconst(s, a, st->const_len);
+    case ASAMD_SPMV_STREAM:
+      return asamd_spmv_stream(s, a, stream_group(p, 0), st->max_len, st->first_offset);
+    case ASAMD_SPMV_SCALAR:
+      return asamd_spmv_scalar(s, a);
+    case ASAMD_SPMV_BINNED: {
+      void *partial = p->binned.chunks > 0 ? ws_take(&ws, (size_t)p->binned.chunks * vs) : NULL;
+      if (p->binned.chunks > 0 && !partial) return -1;
+      return asamd_spmv_binned(s, a, &p->binned, partial);
+    }
+    case ASAMD_SPMV_MERGE_HOT: {
+      void *front = ws_take(&ws, (size_t)p->hot.cols_front * vs);
+      int32_t *carry_row = (int32_t *)ws_take(&ws, (size_t)p->hot.blocks * 4);
+      void *carry_val = ws_take(&ws, (size_t)p->hot.blocks * vs);
+      void *head_val = ws_take(&ws, (size_t)p->hot.blocks * vs);
+      if (!head_val) return -1;
+      return asamd_spmv_hot(s, a, &p->hot, front, carry_row, carry_val, head_val);
+    }
+    case ASAMD_SPMV_MERGE: {
+      const size_t nb = (size_t)st->merge_blocks;
+      const int32_t *block_row = p->d_block_row;
+      if (!block_row) {
+        /* structure not promised fixed: the coordinates are computed for this call */
+        int32_t *fresh = (int32_t *)ws_take(&ws, (nb + 1) * 4);
+        if (!fresh) return -1;
+        const int e = asamd_merge_partition(s, st->m, st->nnz, a->row_ptr, st->base, st->merge_blocks,
+                                            ASAMD_MERGE_THREADS * p->merge_ipt, fresh);
+        if (e != hipSuccess) return e;
+        block_row = fresh;
+      }
+      int32_t *carry_row = (int32_t *)ws_take(&ws, nb * 4);
+      void *carry_val = ws_take(&ws, nb * vs);
+      void *head_val = ws_take(&ws, nb * vs);
+      if (!head_val) return -1;
+      return asamd_spmv_merge(s, a, p->merge_ipt, block_row, carry_row, carry_val, head_val);
+    }
+    case ASAMD_SPMV_VECTOR:
+    default:
+      return asamd_spmv_vector(s, a, p->auto_width);
+  }
+}
+
+/* Gathers the plan's tiled / ELL copy again from val; gate: NULL, or the value guard's flag. */
+static hipError_t refresh_main(hipStream_t s, asamd_csr_plan *p, const int32_t *rp, const int32_t *ci, const void *val,
+                               const int32_t *gate) {
+  const asamd_csr_stats *st = &p->st;
+  hipError_t e = hipSuccess;
+  if (st->tiled_built)
+    e = (hipError_t)asamd_gather_values(s, p->dtype, 0, st->nnz, p->tiled.tperm, val, p->tiled.tval, gate);
+  if (e == hipSuccess && st->ell_built)
+    e = (hipError_t)asamd_csr2ell_gated(s, p->val_size, st->m, val, rp, ci, st->base, 0, st->ell_width, p->d_eval,
+                                        p->d_ecol, gate);
+  return e;
+}
+
+/* ... and one transposed copy with everything its own analysis keeps */
+static hipError_t refresh_trans(hipStream_t s, asamd_csr_plan *p, int which, const void *val, const int32_t *gate) {
+  asamd_trans_copy *t = &p->tr[which];
+  hipError_t e = (hipError_t)asamd_gather_values(s, p->dtype, which == 1, p->st.nnz, t->t.perm, val, t->t.val, gate);
+  if (e == hipSuccess) e = refresh_main(s, t->plan, t->t.row_ptr, t->t.col_ind, t->t.val, gate);
+  return e;
+}
+
+static int csrmv_inner(hipStream_t s, asamd_csr_plan *p, const asamd_spmv_args *a, ws_cursor ws, int guard) {
+  const asamd_csr_stats *st = &p->st;
+  int algo = st->algo;
+  /* The tiled and ELL copies hold the values of the array they were built from.  A multiply that brings
+   * another value array (same structure, new numbers) must not see the old ones: it runs the kernel that
+   * the row statistics alone would pick. */
+  if ((algo == ASAMD_SPMV_TILED || algo == ASAMD_SPMV_ELL) && p->copy_val_src && a->val != p->copy_val_src)
+    algo = p->struct_algo;
+  algo = settle_algo(p, algo, a->val, a->col_ind);
+  if ((algo == ASAMD_SPMV_TILED || algo == ASAMD_SPMV_ELL) && guard && st->value_check) {
+    /* Values changed IN PLACE under the copy: fingerprint, compare, gather again if need be, and only
+     * then record the new fingerprint -- a multiply on another stream that reads the recorded word
+     * either finds the old one (and gathers the same values again itself) or finds the copy done. */
+    void *g = ws_take(&ws, ASAMD_GUARD_WS_BYTES);
+    if (!g) {
+      algo = settle_algo(p, p->struct_algo, a->val, a->col_ind); /* no room to check the copy: do not use it */
+    } else {
+      int e = asamd_value_guard(s, a->val, (size_t)st->nnz * (size_t)p->val_size, st->value_check == 2, p->d_fp, g);
+      if (e == hipSuccess) e = (int)refresh_main(s, p, a->row_ptr, a->col_ind, a->val, ASAMD_GUARD_FLAG(g));
+      if (e == hipSuccess) e = asamd_value_guard_commit(s, g, p->d_fp);
+      if (e != hipSuccess) return e;
+    }
+  }
+  int e = run_algo(s, p, algo, a, ws);
+  if (e == -1) {
+    /* the workspace does not hold this family's scratch: a lane group per row needs none */
+    e = asamd_spmv_vector(s, a, p->auto_width);
+  }
+  return e;
+}
+
+static void fill_args(asamd_spmv_args *a, const asamd_csr_plan *p, const void *alpha, const void *val,
+                      const int32_t *rp, const int32_t *ci, const void *x, const void *beta, void *y) {
+  a->dtype = p->dtype;
+  a->m = p->st.m;
+  a->n = p->st.n;
+  a->nnz = p->st.nnz;
+  a->base = p->st.base;
+  a->alpha = alpha;
+  a->beta = beta;
+  a->val = val;
+  a->row_ptr = rp;
+  a->col_ind = ci;
+  a->x = x;
+  a->y = y;
+}
+
+static hipError_t build_transpose(hipStream_t stream, asamd_csr_plan *p, const int32_t *rp, const int32_t *ci,
+                                  const void *val, int which);
+
+int asamd_csr_plan_csrmv(hipStream_t s, asamd_csr_plan *p, int32_t op, const void *alpha, const void *val,
+                         const int32_t *rp, const int32_t *ci, const void *x, const void *beta, void *y,
+                         void *workspace, size_t workspace_bytes) {
+  if (!p || !alpha || !beta || !val || !rp || !ci || !x || !y) return hipErrorInvalidValue;
+  if (op < 0 || op > 2 || (op == 2 && !is_complex(p))) return hipErrorInvalidValue;
+  if (((uintptr_t)val | (uintptr_t)x | (uintptr_t)y) % (size_t)p->val_size) return hipErrorInvalidValue;
+  const asamd_csr_stats *st = &p->st;
+  ws_cursor ws = ws_open(workspace, workspace_bytes);
+  asamd_spmv_args a;
+  fill_args(&a, p, alpha, val, rp, ci, x, beta, y);
+  if (op == 0) return csrmv_inner(s, p, &a, ws, 1);
+
+  const int which = op - 1;
+  asamd_trans_copy *t = &p->tr[which];
+  /* A library-owned mirror lays out its copy of the transpose on the first transposed multiply: that
+   * allocates and waits, which a stream under capture must not do -- such a call scatters instead, and
+   * the copy is laid out by the first call outside a capture. */
+  if (!t->plan && p->lazy_transpose && st->trusted && st->nnz > 0 && st->first_offset == 0) {
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &capturing) != hipSuccess) {
+      (void)hipGetLastError();
+      capturing = hipStreamCaptureStatusActive; /* unknown: do not risk it */
+    }
+    if (capturing == hipStreamCaptureStatusNone) {
+      const hipError_t e = build_transpose(s, p, rp, ci, val, which);
+      if (e == hipErrorOutOfMemory) {
+        (void)hipGetLastError(); /* no room for the copy: scatter instead, and do not try again */
+        p->lazy_transpose = 0;
+      } else if (e != hipSuccess) {
+        return e;
+      }
+    }
+  }
+  /* the copy holds the values it was gathered from: another value array takes the scatter route below */
+  if (t->plan && val == t->val_src) {
+    int usable = 1;
+    if (st->value_check) {
+      void *g = ws_take(&ws, ASAMD_GUARD_WS_BYTES);
+      if (!g) {
+        usable = 0; /* no room to check the copy: do not use it */
+      } else {
+        int e = asamd_value_guard(s, val, (size_t)st->nnz * (size_t)p->val_size, st->value_check == 2,
+                                  p->d_fp + 1 + which, g);
+        if (e == hipSuccess) e = (int)refresh_trans(s, p, which, val, ASAMD_GUARD_FLAG(g));
+        if (e == hipSuccess) e = asamd_value_guard_commit(s, g, p->d_fp + 1 + which);
+        if (e != hipSuccess) return e;
+      }
+    }
+    if (usable) {
+      asamd_spmv_args at;
+      fill_args(&at, t->plan, alpha, t->t.val, t->t.row_ptr, t->t.col_ind, x, beta, y);
+      return csrmv_inner(s, t->plan, &at, ws, 0);
+    }
+  }
+  return asamd_spmv_trans_scatter(s, &a, p->auto_width, which == 1);
+}
+
+/* ---- analysis: timing the candidates ----------------------------------------------------------------- */
+enum { CAND_BASE = 0, CAND_TILED, CAND_ELL, CAND_HOT, CAND_BINNED, CAND_COUNT };
+
+typedef struct {
+  hipStream_t stream;
+  asamd_csr_plan *p;
+  const int32_t *row_ptr, *col_ind;
+  const void *val;
+  void *x, *y, *ws;
+  size_t ws_bytes;
+  hipEvent_t e0, e1;
+  float best[CAND_COUNT];
+  int algos[CAND_COUNT];
+  hipError_t err;
+} tune_ctx;
+
+/* the candidates' scratch comes from a buffer of the analysis' own, grown as the candidates ask */
+static void tune_reserve(tune_ctx *t, size_t bytes) {
+  if (t->err != hipSuccess || bytes <= t->ws_bytes) return;
+  if (t->ws) (void)hipFree(t->ws);
+  t->ws = NULL;
+  t->ws_bytes = 0;
+  t->err = hipMalloc(&t->ws, bytes);
+  if (t->err == hipSuccess) t->ws_bytes = bytes;
+}
+
+static void time_algo(tune_ctx *t, int cand) {
+  asamd_csr_plan *p = t->p;
+  p->st.algo = t->algos[cand];
+  tune_reserve(t, algo_scratch(p, t->algos[cand]) + 512);
+  static const double one[2] = {1.0, 0.0}, zero[2] = {0.0, 0.0};
+  static const float onef[2] = {1.0f, 0.0f}, zerof[2] = {0.0f, 0.0f};
+  const int wide = p->dtype == ASAMD_DTYPE_DOUBLE || p->dtype == ASAMD_DTYPE_DOUBLE_COMPLEX;
+  const void *alpha = wide ? (const void *)one : (const void *)onef;
+  const void *beta = wide ? (const void *)zero : (const void *)zerof;
+  asamd_spmv_args a;
+  fill_args(&a, p, alpha, t->val, t->row_ptr, t->col_ind, t->x, beta, t->y);
+  /* first run warms up; multiplies of a millisecond and more are timed once, shorter ones twice; a
+   * first run of more than two milliseconds is its own measurement (cold caches are noise at that length) */
+  int reps = 3;
+  for (int rep = 0; rep < reps && t->err == hipSuccess; ++rep) {
+    t->err = hipEventRecord(t->e0, t->stream);
+    if (t->err == hipSuccess) t->err = (hipError_t)csrmv_inner(t->stream, p, &a, ws_open(t->ws, t->ws_bytes), 0);
+    if (t->err == hipSuccess) t->err = hipEventRecord(t->e1, t->stream);
+    if (t->err == hipSuccess) t->err = hipEventSynchronize(t->e1);
+    float ms = 0.f;
+    if (t->err == hipSuccess) t->err = hipEventElapsedTime(&ms, t->e0, t->e1);
+    if (rep == 0 && ms > 1.0f) reps = ms > 2.0f ? 1 : 2;
+    if ((rep > 0 || reps == 1) && (t->best[cand] == 0.f || ms < t->best[cand])) t->best[cand] = ms;
+  }
+}
+
+/* Time the structural choice on scratch vectors, then the copies that the matrix is eligible for:
+ * the ELL copy (cheap to build), and the tiled copy only if the fastest so far is slower than the
+ * tiled pair could possibly be.  Keep the fastest and free the copies that lost.  A copy has to win
+ * by a margin to be worth its memory. */
+static hipError_t tune_copies(hipStream_t stream, asamd_csr_plan *p, const int32_t *row_ptr, const int32_t *col_ind,
+                              const void *val, int tiled_ok, int ell_ok, int hot_ok, int binned_ok) {
+  asamd_csr_stats *st = &p->st;
+  const size_t vs = (size_t)p->val_size;
+  tune_ctx t;
+  memset(&t, 0, sizeof t);
+  t.stream = stream;
+  t.p = p;
+  t.row_ptr = row_ptr;
+  t.col_ind = col_ind;
+  t.val = val;
+  t.err = hipMalloc(&t.x, (size_t)st->n * vs);
+  if (t.err == hipSuccess) t.err = hipMalloc(&t.y, (size_t)st->m * vs);
+  if (t.err == hipSuccess) t.err = hipMemsetAsync(t.x, 0, (size_t)st->n * vs, stream);
+  if (t.err == hipSuccess) t.err = hipEventCreate(&t.e0);
+  if (t.err == hipSuccess) t.err = hipEventCreate(&t.e1);
+  t.algos[CAND_BASE] = p->auto_algo;
+  t.algos[CAND_TILED] = ASAMD_SPMV_TILED;
+  t.algos[CAND_ELL] = ASAMD_SPMV_ELL;
+  t.algos[CAND_HOT] = ASAMD_SPMV_MERGE_HOT;
+  t.algos[CAND_BINNED] = ASAMD_SPMV_BINNED;
+  /* The tiled pair streams about twice the algorithmic bytes (16 instead of 8 bytes per fp32 entry), so
+   * it cannot finish before 2 * bytes / (the ~5 TB/s that streams reach). */
+  const double bytes = (double)st->nnz * (4.0 + (double)vs) + ((double)st->m + 1) * 4.0 +
+                       ((double)st->n + (double)st->m) * (double)vs;
+  float tiled_floor_ms = (float)(2.0 * bytes / 5.0e9);
+  /* Heavy-tailed rows (power-law graphs) make uneven tiles: the in-wave combining of equal rows and the
+   * long-tile phase then cost the tiled pair about 2.3 times its floor (measured 0.78 ms against 0.34 ms
+   * on an 8 M-row R-MAT matrix whose longest row has 120 000 entries; 0.65 ms on its transpose). */
+  if ((double)st->max_len > 32.0 * ((double)st->nnz / (double)st->m) + 256.0) tiled_floor_ms *= 2.5f;
+  if (t.err == hipSuccess) time_algo(&t, CAND_BASE);
+  /* A lane group per row, or a staged block of rows with several lanes per row, was chosen from the mean and
+   * the longest row alone.  Neither needs a copy, nor does merge-path, which takes any distribution: the
+   * fastest of them stays. */
+  if (t.err == hipSuccess && structural_alternatives(p)) {
+    const int alts[2] = {ASAMD_SPMV_MERGE, p->auto_algo == ASAMD_SPMV_STREAM ? ASAMD_SPMV_VECTOR : -1};
+    for (int i = 0; i < 2; ++i) {
+      const int alt = alts[i];
+      if (alt < 0 || t.err != hipSuccess) continue;
+      const float first = t.best[CAND_BASE];
+      const int kept = t.algos[CAND_BASE];
+      t.best[CAND_BASE] = 0.f;
+      t.algos[CAND_BASE] = alt;
+      time_algo(&t, CAND_BASE);
+      if (t.err == hipSuccess && t.best[CAND_BASE] > 0.f && t.best[CAND_BASE] < 0.97f * first) {
+        p->auto_algo = p->struct_algo = alt;
+      } else {
+        t.algos[CAND_BASE] = kept;
+        t.best[CAND_BASE] = first;
+      }
+    }
+  }
+  /* An ELL copy gathers x row by row like the kernel just timed; when that one is several times slower
+   * than the tiled floor the gathers are the problem and the ELL copy (as large as the matrix) is not
+   * worth building: the tiled copy is tried first, the ELL copy only if that does not win. */
+  const int ell_first = !(tiled_ok && t.best[CAND_BASE] > 2.5f * tiled_floor_ms);
+  if (ell_first && t.err == hipSuccess && ell_ok) {
+    t.err = build_ell(stream, p, row_ptr, col_ind, val);
+    if (t.err == hipSuccess) time_algo(&t, CAND_ELL);
+  }
+  if (t.err == hipSuccess && tiled_ok) {
+    /* A row kernel that is already as fast as the tiled floor (banded matrices, whose gathers stay in
+     * the caches) makes the tiled copy pointless: its layout pass (a sort of all entries) and its
+     * memory are saved. */
+    float fastest = t.best[CAND_BASE];
+    if (t.best[CAND_ELL] > 0.f && t.best[CAND_ELL] < fastest) fastest = t.best[CAND_ELL];
+    if (fastest > 1.1f * tiled_floor_ms) {
+      t.err = build_tiled(stream, p, row_ptr, col_ind, val);
+      if (t.err == hipSuccess && st->tiled_built) time_algo(&t, CAND_TILED);
+    }
+  }
+  if (!ell_first && !(t.best[CAND_TILED] > 0.f && t.best[CAND_TILED] < 0.9f * t.best[CAND_BASE]) &&
+      t.err == hipSuccess && ell_ok) {
+    t.err = build_ell(stream, p, row_ptr, col_ind, val);
+    if (t.err == hipSuccess) time_algo(&t, CAND_ELL);
+  }
+  /* Skewed matrices on merge-path: count the entries per column and, if few columns hold most of them,
+   * time the kernel that keeps those columns' x in LDS. */
+  if (t.err == hipSuccess && hot_ok && p->auto_algo == ASAMD_SPMV_MERGE) {
+    t.err = build_hot(stream, p, row_ptr, col_ind, 0);
+    if (t.err == hipSuccess && st->hot_built) time_algo(&t, CAND_HOT);
+  }
+  /* Very uneven rows: one launch per row-length class (cheap to lay out: a sort of the row numbers) */
+  if (t.err == hipSuccess && binned_ok) {
+    t.err = build_binned(stream, p, row_ptr);
+    if (t.err == hipSuccess && st->binned_built) time_algo(&t, CAND_BINNED);
+  }
+  if (t.e0) (void)hipEventDestroy(t.e0);
+  if (t.e1) (void)hipEventDestroy(t.e1);
+  if (t.x) (void)hipFree(t.x);
+  if (t.y) (void)hipFree(t.y);
+  if (t.ws) (void)hipFree(t.ws);
+  st->algo = p->auto_algo;
+  if (t.err != hipSuccess) return t.err;
+  st->tune_ms_binned = t.best[CAND_BINNED];
+  st->tune_ms_base = t.best[CAND_BASE];
+  st->tune_ms_tiled = t.best[CAND_TILED];
+  st->tune_ms_ell = t.best[CAND_ELL];
+  st->tune_ms_hot = t.best[CAND_HOT];
+  /* a copy has to win by a margin to be worth its memory; among the winners the fastest is kept */
+  const float margin[CAND_COUNT] = {1.f, 0.9f, 0.95f, 0.95f, 0.95f};
+  int pick = 0;
+  for (int c = 1; c < CAND_COUNT; ++c)
+    if (t.best[c] > 0.f && t.best[c] < margin[c] * t.best[CAND_BASE] && (pick == 0 || t.best[c] < t.best[pick])) pick = c;
+  /* ALSPARSE_AMD_TUNE_PICK = base | tiled | ell | hot | binned overrides the timing's verdict among the
+   * candidates that were built (for profiling a kernel that lost) */
+  const char *ev = getenv("ALSPARSE_AMD_TUNE_PICK");
+  if (ev) {
+    static const char *names[CAND_COUNT] = {"base", "tiled", "ell", "hot", "binned"};
+    for (int c = 0; c < CAND_COUNT; ++c)
+      if (!strcmp(ev, names[c]) && (c == 0 || t.best[c] > 0.f)) pick = c;
+  }
+  if (pick != CAND_TILED) free_tiled(p);
+  if (pick != CAND_ELL) free_ell(p);
+  if (pick != CAND_HOT) free_hot(p);
+  if (pick != CAND_BINNED) free_binned(p);
+  if (pick != CAND_BASE) {
+    p->auto_algo = t.algos[pick];
+    st->algo = t.algos[pick];
+  }
+  return hipSuccess;
+}
+
+/* the fingerprint of the values a copy set was taken from (set-up work: plan-owned scratch, not concurrent) */
+static hipError_t first_fingerprint(hipStream_t stream, asamd_csr_plan *p, const void *val, int slot) {
+  if (!p->st.value_check) return hipSuccess;
+  hipError_t e = (hipError_t)asamd_value_guard(stream, val, (size_t)p->st.nnz * (size_t)p->val_size,
+                                               p->st.value_check == 2, NULL, p->d_setup);
+  if (e == hipSuccess) e = (hipError_t)asamd_value_guard_commit(stream, p->d_setup, p->d_fp + slot);
+  return e;
+}
+
+static hipError_t plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t nnz, const int32_t *row_ptr,
+                              const int32_t *col_ind, const void *val, int32_t base, int32_t dtype, int32_t trusted,
+                              asamd_csr_plan **out) {
+  if (!out || !row_ptr || m <= 0 || nnz < 0 || dtype < ASAMD_DTYPE_FLOAT || dtype > ASAMD_DTYPE_DOUBLE_COMPLEX)
+    return hipErrorInvalidValue;
+  const int val_size = kValSize[dtype];
+  if (val && (uintptr_t)val % (size_t)val_size) return hipErrorInvalidValue;
+  asamd_csr_plan *p = (asamd_csr_plan *)calloc(1, sizeof(*p));
+  if (!p) return hipErrorOutOfMemory;
+  asamd_csr_stats *st = &p->st;
+  st->m = m;
+  st->n = n;
+  st->nnz = nnz;
+  st->base = base;
+  st->trusted = trusted ? 1 : 0;
+  st->value_check = env_value_check();
+  st->tune_mode = env_tune_model();
+  p->dtype = dtype;
+  p->val_size = val_size;
+
+  hipError_t e = hipMalloc(&p->d_setup, SETUP_BYTES);
+  if (e == hipSuccess) e = hipMalloc((void **)&p->d_fp, 3 * sizeof(uint64_t));
+  int32_t h[ASAMD_ROW_STATS_WORDS];
+  if (e == hipSuccess) e = (hipError_t)asamd_csr_row_stats(stream, m, row_ptr, (int32_t *)p->d_setup, h);
+  if (e != hipSuccess) {
+    asamd_csr_plan_destroy(p);
+    return e;
+  }
+  st->min_len = h[0];
+  st->max_len = h[1];
+  st->first_offset = h[2] - base;
+  st->const_len = h[0] == h[1] ? h[0] : -1;
+  for (int b = 0; b < ASAMD_HIST_BINS; ++b) st->hist[b] = h[3 + b];
+
+  const int64_t total = (int64_t)m + nnz;
+  /* wider values take more LDS per item: fewer items keep more workgroups resident */
+  p->merge_ipt = val_size >= 8 ? 4 : 8;
+  const int want_ipt = env_int("ALSPARSE_AMD_MERGE_IPT", 0);
+  if (want_ipt == 4 || want_ipt == 8 || (want_ipt == 16 && dtype <= ASAMD_DTYPE_DOUBLE)) p->merge_ipt = want_ipt;
+  if (val_size == 16) p->merge_ipt = 4; /* the only instantiation for 16-byte values */
+  const int merge_items = ASAMD_MERGE_THREADS * p->merge_ipt;
+  const int64_t nb = (total + merge_items - 1) / merge_items;
+  st->merge_blocks = (int)nb;
+  choose_algo(p);
+
+  if (st->trusted && st->first_offset == 0) {
+    /* the structure is promised fixed: the merge-path coordinates are computed once */
+    e = hipMalloc((void **)&p->d_block_row, ((size_t)nb + 1) * sizeof(int32_t));
+    if (e == hipSuccess)
+      e = (hipError_t)asamd_merge_partition(stream, m, nnz, row_ptr, base, (int)nb, merge_items, p->d_block_row);
+    if (e == hipSuccess) e = hipStreamSynchronize(stream);
+    if (e != hipSuccess) {
+      asamd_csr_plan_destroy(p);
+      return e;
+    }
+  }
+  if (col_ind && val && nnz > 0) {
+    /* trusted == 2: build every copy whatever the size and skip the timing
+     * (lets small matrices exercise those kernels) */
+    const int force = trusted == 2;
+    const int tiled_ok = tiled_eligible(p, force), ell_ok = ell_eligible(st, force);
+    const int hot_ok = hot_eligible(p, force), binned_ok = binned_eligible(p, force);
+    if (force) {
+      if (binned_ok) e = build_binned(stream, p, row_ptr);
+      if (e == hipSuccess && tiled_ok) e = build_tiled(stream, p, row_ptr, col_ind, val);
+      if (e == hipSuccess && ell_ok) e = build_ell(stream, p, row_ptr, col_ind, val);
+      if (e == hipSuccess && hot_ok) e = build_hot(stream, p, row_ptr, col_ind, 1);
+    } else if (tiled_ok || ell_ok || hot_ok || binned_ok || structural_alternatives(p)) {
+      e = tune_copies(stream, p, row_ptr, col_ind, val, tiled_ok, ell_ok, hot_ok, binned_ok);
+    }
+    if (e == hipErrorOutOfMemory) {
+      (void)hipGetLastError(); /* the copies are optional: carry on without them */
+      free_tiled(p);
+      free_ell(p);
+      free_hot(p);
+      free_binned(p);
+      if (p->auto_algo == ASAMD_SPMV_TILED || p->auto_algo == ASAMD_SPMV_ELL || p->auto_algo == ASAMD_SPMV_MERGE_HOT ||
+          p->auto_algo == ASAMD_SPMV_BINNED)
+        p->auto_algo = p->struct_algo;
+      st->algo = p->auto_algo;
+      e = hipSuccess;
+    }
+    if (e == hipSuccess && has_value_copy(p)) {
+      p->copy_val_src = val;
+      e = first_fingerprint(stream, p, val, 0);
+      if (e == hipSuccess) e = hipStreamSynchronize(stream);
+    }
+    if (e != hipSuccess) {
+      asamd_csr_plan_destroy(p);
+      return e;
+    }
+  }
+  account(p);
+  *out = p;
+  return hipSuccess;
+}
+
+int asamd_csr_plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t nnz, const int32_t *row_ptr,
+                          const int32_t *col_ind, const void *val, int32_t base, int32_t val_size, int32_t trusted,
+                          asamd_csr_plan **out) {
+  if (val_size != 4 && val_size != 8) return hipErrorInvalidValue;
+  return plan_create(stream, m, n, nnz, row_ptr, col_ind, val, base,
+                     val_size == 4 ? ASAMD_DTYPE_FLOAT : ASAMD_DTYPE_DOUBLE, trusted, out);
+}
+
+int asamd_csr_plan_create_dtype(hipStream_t stream, int32_t m, int32_t n, int32_t nnz, const int32_t *row_ptr,
+                                const int32_t *col_ind, const void *val, int32_t base, int32_t dtype, int32_t trusted,
+                                asamd_csr_plan **out) {
+  return plan_create(stream, m, n, nnz, row_ptr, col_ind, val, base, dtype, trusted, out);
+}
+
+void asamd_csr_plan_destroy(asamd_csr_plan *p) {
+  if (!p) return;
+  if (p->d_block_row) (void)hipFree(p->d_block_row);
+  if (p->d_setup) (void)hipFree(p->d_setup);
+  if (p->d_fp) (void)hipFree(p->d_fp);
+  free_tiled(p);
+  free_ell(p);
+  free_hot(p);
+  free_binned(p);
+  free_transpose(p, 0);
+  free_transpose(p, 1);
+  free(p);
+}
+
+/* CSR of A^T (which = 1: of A^H) with an analysis of its own. */
+static hipError_t build_transpose(hipStream_t stream, asamd_csr_plan *p, const int32_t *rp, const int32_t *ci,
+                                  const void *val, int which) {
+  asamd_csr_stats *st = &p->st;
+  asamd_trans_copy *t = &p->tr[which];
+  hipError_t e = (hipError_t)asamd_transpose_build(stream, p->dtype, which == 1, st->m, st->n, st->nnz, st->base, rp, ci,
+                                                   val, &t->t);
+  if (e == hipSuccess)
+    e = plan_create(stream, st->n, st->m, st->nnz, t->t.row_ptr, t->t.col_ind, t->t.val, 0, p->dtype, /*trusted=*/1,
+                    &t->plan);
+  if (e == hipSuccess) e = first_fingerprint(stream, p, val, 1 + which);
+  if (e == hipSuccess) e = hipStreamSynchronize(stream);
+  if (e != hipSuccess) {
+    free_transpose(p, which);
+    return e;
+  }
+  t->val_src = val;
+  st->transpose_built |= 1 << which;
+  account(p);
+  return hipSuccess;
+}
+
+static int build_transpose_any(hipStream_t stream, asamd_csr_plan *p, const int32_t *row_ptr, const int32_t *col_ind,
+                               const void *val, int which) {
+  if (!p || !row_ptr || !col_ind || !val || !p->st.trusted || p->st.n <= 0) return hipErrorInvalidValue;
+  if (which == 1 && !is_complex(p)) return hipErrorInvalidValue;
+  if (p->st.transpose_built & (1 << which)) return hipSuccess;
+  if (p->st.nnz == 0) return hipSuccess;          /* the scatter route has nothing to add */
+  if (p->st.first_offset != 0) return hipSuccess; /* no copy (csr2coo counts from position 0): the scatter route serves */
+  return build_transpose(stream, p, row_ptr, col_ind, val, which);
+}
+
+int asamd_csr_plan_build_transpose(hipStream_t stream, asamd_csr_plan *p, const int32_t *row_ptr,
+                                   const int32_t *col_ind, const void *val) {
+  return build_transpose_any(stream, p, row_ptr, col_ind, val, 0);
+}
+
+int asamd_csr_plan_build_conj_transpose(hipStream_t stream, asamd_csr_plan *p, const int32_t *row_ptr,
+                                        const int32_t *col_ind, const void *val) {
+  return build_transpose_any(stream, p, row_ptr, col_ind, val, 1);
+}
+
+int asamd_csr_plan_set_lazy_transpose(asamd_csr_plan *p, int32_t on) {
+  if (!p || !p->st.trusted) return hipErrorInvalidValue;
+  p->lazy_transpose = on != 0;
+  return hipSuccess;
+}
+
+const asamd_csr_stats *asamd_csr_plan_transpose_stats(const asamd_csr_plan *p) {
+  if (!p) return NULL;
+  if (p->tr[0].plan) return &p->tr[0].plan->st;
+  return p->tr[1].plan ? &p->tr[1].plan->st : NULL;
+}
+
+int asamd_csr_plan_transpose_arrays(const asamd_csr_plan *p, int32_t conj, const int32_t **row_ptr,
+                                    const int32_t **col_ind, const void **val) {
+  if (!p || !row_ptr || !col_ind || !val) return hipErrorInvalidValue;
+  const asamd_trans_copy *t = &p->tr[conj ? 1 : 0];
+  if (!t->plan) return hipErrorInvalidValue;
+  *row_ptr = t->t.row_ptr;
+  *col_ind = t->t.col_ind;
+  *val = t->t.val;
+  return hipSuccess;
+}
+
+int asamd_csr_plan_refresh_values(hipStream_t stream, asamd_csr_plan *p, const int32_t *row_ptr,
+                                  const int32_t *col_ind, const void *val) {
+  if (!p || !row_ptr || !col_ind || !val || !p->st.trusted) return hipErrorInvalidValue;
+  if ((uintptr_t)val % (size_t)p->val_size) return hipErrorInvalidValue;
+  hipError_t e = refresh_main(stream, p, row_ptr, col_ind, val, NULL);
+  if (e == hipSuccess && has_value_copy(p)) {
+    p->copy_val_src = val;
+    e = first_fingerprint(stream, p, val, 0);
+  }
+  for (int which = 0; which < 2 && e == hipSuccess; ++which) {
+    if (!p->tr[which].plan) continue;
+    e = refresh_trans(stream, p, which, val, NULL);
+    p->tr[which].val_src = val;
+    if (e == hipSuccess) e = first_fingerprint(stream, p, val, 1 + which);
+  }
+  return e;
+}
+
+const asamd_csr_stats *asamd_csr_plan_stats(const asamd_csr_plan *p) { return p ? &p->st : NULL; }
+
+int asamd_csr_plan_set_algo(asamd_csr_plan *p, int32_t algo) {
+  if (!p) return hipErrorInvalidValue;
+  switch (algo) {
+    case ASAMD_SPMV_AUTO:
+      p->st.algo = p->auto_algo;
+      return hipSuccess;
+    case ASAMD_SPMV_ROWCONST:
+      if (!rowconst_ok(p)) return hipErrorInvalidValue;
+      break;
+    case ASAMD_SPMV_TILED:
+      if (!p->st.tiled_built) return hipErrorInvalidValue;
+      break;
+    case ASAMD_SPMV_STREAM:
+      if (!stream_ok(p)) return hipErrorInvalidValue;
+      break;
+    case ASAMD_SPMV_ELL:
+      if (!p->st.ell_built) return hipErrorInvalidValue;
+      break;
+    case ASAMD_SPMV_MERGE_HOT:
+      if (!p->st.hot_built) return hipErrorInvalidValue;
+      break;
+    case ASAMD_SPMV_BINNED:
+      if (!p->st.binned_built) return hipErrorInvalidValue;
+      break;
+    case ASAMD_SPMV_MERGE:
+      if (p->st.first_offset != 0) return hipErrorInvalidValue;
+      break;
+    case ASAMD_SPMV_VECTOR:
+    case ASAMD_SPMV_SCALAR:
+      break;
+    default:
+      return hipErrorInvalidValue;
+  }
+  p->st.algo = algo;
+  return hipSuccess;
+}

@@ -6,8 +6,10 @@
  * (test/dcu/level2/mv_csr_d_dcu_test.cpp:210-213).  Nothing in such a record
  * can therefore be trusted; results live here, keyed by the address of the
  * object they belong to and confirmed against the call's arguments before use. */
+#include <omp.h>
 #include <pthread.h>
 #include <stdlib.h>
+#include <string.h>
 
 #include "internal.h"
 
@@ -211,17 +213,40 @@ void asamd_registry_drop_handle(const void *handle) {
   }
 }
 
-uint64_t asamd_host_fingerprint(const void *values, size_t count, size_t elem) {
-  const unsigned char *p = (const unsigned char *)values;
-  const size_t samples = count < 1024 ? count : 1024;
-  uint64_t h = 0x9E3779B97F4A7C15ull ^ (uint64_t)count;
-  for (size_t s = 0; s < samples; ++s) {
-    /* sample s sits at a fixed position of its 1/samples share of the array */
-    const size_t i = (size_t)(((unsigned __int128)s * count) / samples) + (s * 2654435761u) % (count / samples ? count / samples : 1);
-    const unsigned char *q = p + (i < count ? i : count - 1) * elem;
-    for (size_t b = 0; b < elem; ++b) h = (h ^ q[b]) * 0x100000001B3ull;
+/* Every byte counts: pieces of 1 MiB are hashed by the OpenMP threads (four independent multiply-add
+ * chains over 8-byte words, memory-bound), and the pieces' words are combined with their positions. */
+static uint64_t hash_piece(const unsigned char *p, size_t bytes) {
+  uint64_t h0 = 0x9E3779B97F4A7C15ull, h1 = 0xBF58476D1CE4E5B9ull, h2 = 0x94D049BB133111EBull, h3 = 0xD6E8FEB86659FD93ull;
+  size_t i = 0;
+  for (; i + 32 <= bytes; i += 32) {
+    uint64_t w[4];
+    memcpy(w, p + i, 32);
+    h0 = (h0 ^ w[0]) * 0x100000001B3ull + 0x632BE59BD9B4E019ull;
+    h1 = (h1 ^ w[1]) * 0xFF51AFD7ED558CCDull + 1;
+    h2 = (h2 ^ w[2]) * 0xC4CEB9FE1A85EC53ull + 2;
+    h3 = (h3 ^ w[3]) * 0x2545F4914F6CDD1Dull + 3;
   }
-  return h;
+  for (; i < bytes; ++i) h0 = (h0 ^ p[i]) * 0x100000001B3ull;
+  uint64_t h = h0 ^ (h1 >> 7) ^ (h2 << 11) ^ (h3 >> 17) ^ (h1 << 31) ^ (h3 << 23);
+  h ^= h >> 29;
+  h *= 0xBF58476D1CE4E5B9ull;
+  return h ^ (h >> 32);
+}
+
+uint64_t asamd_host_fingerprint(const void *data, size_t bytes) {
+  const unsigned char *p = (const unsigned char *)data;
+  const size_t piece = (size_t)1 << 20;
+  const long pieces = (long)((bytes + piece - 1) / piece);
+  uint64_t sum = 0x9E3779B97F4A7C15ull ^ (uint64_t)bytes;
+  int threads = omp_get_max_threads();
+  if (threads > 16) threads = 16;
+#pragma omp parallel for num_threads(threads) schedule(static) reduction(+ : sum) if (pieces > 4)
+  for (long i = 0; i < pieces; ++i) {
+    const size_t off = (size_t)i * piece;
+    const uint64_t h = hash_piece(p + off, bytes - off < piece ? bytes - off : piece);
+    sum += (h ^ ((uint64_t)i * 0x9E3779B97F4A7C15ull)) * 0xD6E8FEB86659FD93ull;
+  }
+  return sum;
 }
 
 static alphasparse_dcu_handle_t g_default_handle;

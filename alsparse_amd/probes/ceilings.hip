@@ -6,8 +6,8 @@
 
 #include <hip/hip_runtime.h>
 
-#include "alsparse_amd_kernels.h"
-#include "device_utils.hpp"
+#include "asamd_probes.h"
+#include "../csrc/hip/device_utils.hpp"
 
 using namespace asamd;
 
@@ -206,5 +206,21 @@ extern "C" int asamd_ceiling_kernel(hipStream_t stream, int32_t kind, void* dst,
     default:
       return hipErrorInvalidValue;
   }
+  return hipGetLastError();
+}
+
+// Plain copy of known size, to calibrate hardware byte counters against.
+__global__ __launch_bounds__(256) void copy_bytes_kernel(Int4* __restrict__ dst, const Int4* __restrict__ src, size_t n16) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x)
+    dst[i] = src[i];
+}
+
+extern "C" int asamd_copy_bytes(hipStream_t stream, void* dst, const void* src, size_t nbytes) {
+  if (!dst || !src || (nbytes & 15u) || (((uintptr_t)dst | (uintptr_t)src) & 15u)) return hipErrorInvalidValue;
+  const size_t n16 = nbytes / 16;
+  if (n16 == 0) return hipSuccess;
+  size_t grid = (n16 + 255) / 256;
+  if (grid > 256 * 64) grid = 256 * 64;
+  copy_bytes_kernel<<<(unsigned)grid, 256, 0, stream>>>((Int4*)dst, (const Int4*)src, n16);
   return hipGetLastError();
 }

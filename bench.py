@@ -567,7 +567,7 @@ def run_ceilings(steps, warmup):
     L1-sized x).  TB/s of useful bytes, and gathers per second."""
     from ctypes import c_int64
     from alsparse_amd import capi, hiprt
-    lib = capi.load()
+    lib = capi.load_probes()
     big = 2 << 30
     a, b = hiprt.DeviceArray((big,), np.uint8), hiprt.DeviceArray((big,), np.uint8)
     sink = hiprt.DeviceArray((4,), np.uint8)
@@ -673,7 +673,7 @@ def main():
         src, dst = hiprt.DeviceArray((nb,), np.uint8), hiprt.DeviceArray((nb,), np.uint8)
         src.fill_bytes(1)
         for _ in range(2):
-            assert capi.load().asamd_copy_bytes(None, dst.c_ptr(), src.c_ptr(), nb) == 0
+            assert capi.load_probes().asamd_copy_bytes(None, dst.c_ptr(), src.c_ptr(), nb) == 0
         hiprt.synchronize()
         src.free()
         dst.free()

@@ -70,159 +70,184 @@ typedef struct { double real, imag; } ALPHA_Complex16;
 typedef ALPHA_Complex8 asamd_complex8;
 typedef ALPHA_Complex16 asamd_complex16;
 
-/* Row-length statistics gathered on the GPU.  hist[0] counts empty rows,
- * hist[b] rows whose length lies in [2^(b-1), 2^b). */
+/* ---- CSR SpMV launchers ---------------------------------------------------------------------
+ * Stateless: each call enqueues the kernels of ONE family on `stream` and returns.  Nothing is
+ * allocated, copied or waited for, so every one of them can be recorded into a HIP graph.  Whatever a
+ * family needs beyond the CSR arrays -- coordinates, re-ordered copies, per-call scratch -- is passed in
+ * by the caller (the host library's plan, include/alsparse_amd_plan.h, which decides the family and owns
+ * the memory).  All of them stand in for csr_gemv_vector_dispatch,
+ * src/kernel/dcu/level2/mv/csrmv/dcu_gemv_vector.h:59-182, the reference's only kernel. */
 typedef struct {
+  int32_t dtype;            /* enum asamd_dtype: element type of val, x, y, alpha, beta */
   int32_t m, n, nnz, base;
-  int32_t min_len, max_len;
-  int32_t const_len;    /* common row length, or -1                          */
-  int32_t first_offset; /* row_ptr[0] - base                                 */
-  int32_t algo;         /* enum asamd_spmv_algo chosen for this structure     */
-  int32_t vector_width; /* lanes per row when algo == VECTOR                  */
-  int32_t merge_blocks; /* workgroups of the merge-path kernel                */
-  int32_t trusted;      /* 1: structure promised fixed, coordinates cached    */
-  int32_t tiled_built;  /* 1: a tiled copy exists (TILED can be selected)     */
-  int32_t tile_col_blocks, tile_row_blocks;
-  float tune_ms_base;   /* analysis-time timing of the non-tiled choice, or 0 */
-  float tune_ms_tiled;  /* ... and of the tiled kernel pair, or 0             */
-  float tune_ms_ell;    /* ... and of the ELL copy's kernel, or 0             */
-  int32_t ell_built;    /* 1: an ELL copy exists (ELL can be selected)        */
-  int32_t ell_width;    /* its slots per row                                  */
-  int32_t transpose_built; /* bit 0: a CSR copy of the transpose exists, bit 1: of the
-                              conjugate transpose                              */
-  int32_t tile_entries_per_lane; /* tiled copy: entries per lane and tile in its second
-                                    phase (1: twice the tiles in flight; tiles of more
-                                    than 64 entries go to the long-tile kernel), or 0  */
-  int64_t hist[ASAMD_HIST_BINS];
-  int32_t hot_built;     /* 1: the hot-column copy exists (MERGE_HOT can be selected)        */
-  int32_t hot_cols_lds;  /* columns whose x the kernel keeps in LDS                            */
-  int32_t hot_cols;      /* most popular columns whose x every multiply gathers into a compact front */
-  float hot_share_lds;   /* share of the entries that fall into the LDS columns               */
-  float tune_ms_hot;     /* analysis-time timing of the hot-column kernel, or 0               */
-  int32_t binned_built;  /* 1: the row numbers are sorted by length class (BINNED can be selected) */
-  int32_t bin_rows[4];   /* rows of at most 8 / 64 / 2 048 entries / longer                   */
-  float tune_ms_binned;  /* analysis-time timing of the per-class launches, or 0              */
-  int32_t tile_long_blocks; /* tiled copy: row blocks with tiles too long for its second phase (its third
-                               phase takes them), or 0                                           */
-} asamd_csr_stats;
+  const void *alpha, *beta; /* HOST scalars */
+  const void *val;          /* nnz values                                              */
+  const int32_t *row_ptr;   /* m + 1 offsets                                           */
+  const int32_t *col_ind;   /* nnz columns                                             */
+  const void *x;            /* n elements                                              */
+  void *y;                  /* m elements; beta == 0 never reads it                    */
+} asamd_spmv_args;
 
-typedef struct asamd_csr_plan asamd_csr_plan;
+/* `width` in {2, 4, ..., 64} lanes sum a row (the reference's mapping, dcu_gemv_vector.h:14-57). */
+int asamd_spmv_vector(hipStream_t stream, const asamd_spmv_args *a, int32_t width);
+/* One lane per row, entries in storage order (src/plain/kernel/level2/mv/gemv/gemv_x_csr_plain.c:11-22). */
+int asamd_spmv_scalar(hipStream_t stream, const asamd_spmv_args *a);
+/* Every row has row_len entries (4, 8, ..., 256): no row_ptr traffic.  Real element types, row_ptr[0] ==
+ * base, val and col_ind 16-byte aligned; hipErrorInvalidValue otherwise. */
+int asamd_spmv_rowconst(hipStream_t stream, const asamd_spmv_args *a, int32_t row_len);
+/* Rows of at most max_len <= ASAMD_STREAM_MAX_GROUP * (64 / sizeof element) entries: 256 / group rows per
+ * workgroup, their products staged in LDS, `group` lanes (1, 2, 4, 8, 16) sum a row.  A workgroup whose
+ * rows hold more entries than its staging area takes them from global memory, so a max_len that has
+ * gone stale costs speed, not correctness.  first_offset = row_ptr[0] - base. */
+#define ASAMD_STREAM_MAX_GROUP 16
+int asamd_spmv_stream(hipStream_t stream, const asamd_spmv_args *a, int32_t group, int32_t max_len,
+                      int32_t first_offset);
 
-/* Row-length histogram, kernel choice and (trusted != 0) cached merge-path
- * block coordinates.  Synchronises `stream` to read the statistics.
- * Replaces the host-side row-block builder
- * src/util_cpp/alphasparse_dcu_x_csrmv_analysis.cpp:58-267, :348-379.
- * val_size is sizeof(value type): 4 (fp32) or 8 (fp64).
- * trusted != 0 promises that the structure behind row_ptr / col_ind and the
- * values behind val stay as they are for the life of the plan.  If in addition
- * col_ind and val are given (they may be NULL) and x is much larger than the L2,
- * a tiled copy of the matrix is built and the tiled two-phase kernel is timed
- * against the row / merge-path choice on scratch vectors; the faster one wins
- * (the reference's analysis record carries an `algo_tuning` flag for exactly
- * this, include/alphasparse/handle.h:120-123).  Likewise, when rows are short
- * (<= 32) and padding them to the longest adds at most 1/8 to the entry count,
- * a column-major ELL copy is built and timed.  Copies that lose are freed.
- * trusted == 2 builds both copies whatever the size and skips the timing (for
- * tests of those kernels); the kernel choice then stays the structural one. */
-int asamd_csr_plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t nnz,
-                          const int32_t *row_ptr, const int32_t *col_ind, const void *val,
-                          int32_t base, int32_t val_size, int32_t trusted, asamd_csr_plan **plan);
-/* The same for any element type (dtype: enum asamd_dtype).  Complex plans run every
- * kernel family (src/kernel/dcu/level2/mv/csrmv/dcu_gemv_vector.h:14-57 is type-generic
- * through ALPHA_Number) except the constant-row-length one, whose 128-bit quads are
- * for real types. */
-int asamd_csr_plan_create_dtype(hipStream_t stream, int32_t m, int32_t n, int32_t nnz,
-                                const int32_t *row_ptr, const int32_t *col_ind, const void *val,
-                                int32_t base, int32_t dtype, int32_t trusted, asamd_csr_plan **plan);
-void asamd_csr_plan_destroy(asamd_csr_plan *plan);
-const asamd_csr_stats *asamd_csr_plan_stats(const asamd_csr_plan *plan);
-/* Force a kernel family for later multiplies (AUTO restores the analysis'
- * own choice).  Returns hipErrorInvalidValue if the structure cannot run it. */
-int asamd_csr_plan_set_algo(asamd_csr_plan *plan, int32_t algo);
+/* Merge-path: the (m + nnz) items are cut into blocks of ASAMD_MERGE_THREADS * ipt items (ipt: 4, 8, or
+ * 16 for real types of at most 8 bytes; 4 only for 16-byte values).  block_row: blocks + 1 merge
+ * coordinates from asamd_merge_partition (row_ptr[0] must equal base and nnz must be row_ptr[m] - base).
+ * Per-call scratch: carry_row (blocks ints), carry_val and head_val (blocks elements each); every word
+ * that a call reads it has written before, so the scratch needs no clearing, and two multiplies that
+ * run at the same time need a scratch each.  No float atomics. */
+#define ASAMD_MERGE_THREADS 256
+int asamd_merge_partition(hipStream_t stream, int32_t m, int32_t nnz, const int32_t *row_ptr, int32_t base,
+                          int32_t blocks, int32_t items_per_block, int32_t *block_row);
+int asamd_spmv_merge(hipStream_t stream, const asamd_spmv_args *a, int32_t ipt, const int32_t *block_row,
+                     int32_t *carry_row, void *carry_val, void *head_val);
 
-/* y = alpha*A*x + beta*y.  Stands in for csr_gemv_vector_dispatch,
- * src/kernel/dcu/level2/mv/csrmv/dcu_gemv_vector.h:59-182.  `plan` must
- * describe (m, n, nnz, base); beta == 0 skips the read of y. */
-int asamd_s_csrmv(hipStream_t stream, asamd_csr_plan *plan, float alpha, const float *val,
-                  const int32_t *row_ptr, const int32_t *col_ind, const float *x, float beta,
-                  float *y);
-int asamd_d_csrmv(hipStream_t stream, asamd_csr_plan *plan, double alpha, const double *val,
-                  const int32_t *row_ptr, const int32_t *col_ind, const double *x, double beta,
-                  double *y);
+/* Transposed / conjugate-transposed product without a copy: y (n elements) is scaled by beta, then
+ * `width` lanes per row scatter alpha*op(a)*x[row] with hardware float atomics, the traversal of
+ * src/kernel/dcu/level2/mv/csrmv/dcu_gemv_x_csr_trans.cpp:11-68 and dcu_gemv_c_csr_conj.cpp:22-75.
+ * x has m elements.  conj != 0: complex types only. */
+int asamd_spmv_trans_scatter(hipStream_t stream, const asamd_spmv_args *a, int32_t width, int32_t conj);
 
-/* asamd_s_csrmv without a plan and without any allocation: for callers that cannot call hipMalloc
- * (code under HIP graph capture, tight serving loops, harnesses that forbid it).  No counterpart in
- * the reference.  Runs the merge-path kernels (any row-length distribution, no float atomics); their
- * workgroup coordinates, carries and head sums live in a fixed device array of
- * ASAMD_CSRMV_NOALLOC_SCRATCH_BYTES that the library holds per GPU until the process ends.
- * m + nnz above ASAMD_CSRMV_NOALLOC_MAX_ITEMS returns hipErrorOutOfMemory (2) before anything is
- * launched; other bad arguments return hipErrorInvalidValue.  base is 0 or 1; nnz == 0 gives
- * y = beta*y.  Calls hipMalloc, hipFree or an allocating library routine never; asamd_warmup (run by
- * alphasparse_dcu_get_handle) resolves the array's address for the current device, and the first
- * call on a device does so itself otherwise.  All calls on one GPU share the array: calls that
- * overlap there (two streams, two threads) race; calls on one stream are ordered and safe. */
-#define ASAMD_CSRMV_NOALLOC_SCRATCH_BYTES (4 << 20)
-#define ASAMD_CSRMV_NOALLOC_MAX_ITEMS 536868864LL /* (SCRATCH_BYTES / 16 - 1) workgroups x 2048 items */
-int asamd_s_csrmv_noalloc(hipStream_t stream, int32_t m, int32_t n, int32_t nnz, int32_t base, float alpha,
-                          const float *val, const int32_t *row_ptr, const int32_t *col_ind, const float *x,
-                          float beta, float *y);
+/* ---- re-ordered copies of a CSR matrix ("layouts") and the kernels that multiply with them ------
+ * A layout is a plain record of device pointers and counts, filled by its *_build call (which
+ * allocates, launches the layout kernels on `stream` and synchronises it) and released by *_free.
+ * Builders return hipSuccess with an EMPTY record (first pointer NULL) when the matrix does not suit the
+ * layout; that is not an error.  device_bytes: device memory the record holds. */
 
-/* A trusted plan may hold re-ordered copies of the matrix VALUES (tiled, ELL, transposed); the
- * reference's analysis keeps structure only (src/util_cpp/alphasparse_dcu_x_csrmv_analysis.cpp:382-388).
- * When the caller has changed the values behind `val` in place (same structure), this gathers every
- * copy again through the permutations that the plan kept: streaming kernels on `stream` only, no sort,
- * no allocation, no wait.  row_ptr / col_ind are the arrays the plan was created for. */
-int asamd_csr_plan_refresh_values(hipStream_t stream, asamd_csr_plan *plan, const int32_t *row_ptr,
-                                  const int32_t *col_ind, const void *val);
-/* 64-bit fingerprint of the structure arrays (m + 1 offsets, nnz column indices): equal arrays give equal
- * values; used to tell a changed structure from changed values when an analysis is repeated.
- * Synchronises `stream`; *hash_host is a host word. */
+/* Tiled two-phase SpMV for x far larger than an XCD's L2: entries sorted by (column block, row block);
+ * phase 1 multiplies against an x slice held in LDS and streams the products out, phase 2 adds them
+ * up in per-wave LDS accumulators, phase 3 takes the tiles too long for phase 2.  Holds the VALUES in
+ * tile order (tval) and the CSR position of every slot (tperm), through which asamd_gather_values
+ * refreshes them.  Per-call scratch: nnz elements of products and long_scratch_elems elements. */
+typedef struct {
+  void *tval;                /* nnz values in tile order; NULL: no layout                      */
+  uint32_t *tperm;           /* nnz: CSR position of the entry in every slot                   */
+  uint16_t *tcol, *trow;     /* nnz columns / rows local to their blocks                       */
+  int32_t *row_block_start;  /* row_blocks + 1                                                 */
+  void *ranges, *chunks, *long_list, *long_tiles, *long_finish; /* tile tables and work lists  */
+  int32_t dtype, m, n, nnz;
+  int32_t col_blocks, row_blocks;
+  int32_t entries_per_lane;  /* phase 2 takes 1 or 2 entries per lane and tile                 */
+  int32_t n_chunks, n_long_chunks, n_long_narrow, n_long_finish, long_blocks;
+  int64_t long_scratch_elems;
+  int64_t device_bytes;
+} asamd_tiled_layout;
+/* 1 if the block counts that (dtype, m, n, nnz) give fit the tile tables */
+int asamd_tiled_fits(int32_t dtype, int32_t m, int32_t n, int32_t nnz);
+/* max_len: longest row (steers the block heights); entries_per_lane: 0 = choose from the tile lengths */
+int asamd_tiled_build(hipStream_t stream, int32_t dtype, int32_t m, int32_t n, int32_t nnz, int32_t base,
+                      const int32_t *row_ptr, const int32_t *col_ind, const void *val, int32_t max_len,
+                      int32_t entries_per_lane, asamd_tiled_layout *out);
+void asamd_tiled_free(asamd_tiled_layout *layout);
+/* y = alpha*A*x + beta*y from the layout (a->val, a->row_ptr, a->col_ind are not read) */
+int asamd_spmv_tiled(hipStream_t stream, const asamd_spmv_args *a, const asamd_tiled_layout *layout,
+                     void *products, void *long_scratch);
+
+/* Hot-column merge-path for power-law columns: the column stream rewritten as ranks of the popular
+ * columns (pcol), whose x sits in LDS (the cols_lds most popular) or in a compact front (cols_front).
+ * Structure only: values come from the caller's array.  Per-call scratch: front (cols_front elements),
+ * carry_row (blocks ints), carry_val and head_val (blocks elements each).  Element types of at most 8 bytes. */
+typedef struct {
+  uint32_t *pcol;            /* nnz positions; NULL: no layout */
+  int32_t *hot_cols;         /* cols_front zero-based columns, most popular first */
+  int32_t *block_row;        /* blocks + 1 merge coordinates of the wave-sized blocks */
+  int32_t dtype, blocks, cols_lds, cols_front;
+  float share_lds;           /* share of the entries whose column is one of the cols_lds */
+  int64_t device_bytes;
+} asamd_hot_layout;
+/* force == 0: an empty record when the LDS columns hold less than a fifth of the entries;
+ * cols_lds / cols_front: 0 = the kernel's capacity / what shares an L2 with the streams */
+int asamd_hot_build(hipStream_t stream, int32_t dtype, int32_t m, int32_t n, int32_t nnz, int32_t base,
+                    const int32_t *row_ptr, const int32_t *col_ind, int32_t force, int32_t cols_lds,
+                    int32_t cols_front, asamd_hot_layout *out);
+void asamd_hot_free(asamd_hot_layout *layout);
+int asamd_spmv_hot(hipStream_t stream, const asamd_spmv_args *a, const asamd_hot_layout *layout, void *front,
+                   int32_t *carry_row, void *carry_val, void *head_val);
+
+/* Row-length bins: the row numbers sorted by length class (<= 8, <= 64, <= 2 048 entries, longer), one
+ * launch per class with 4 / 16 / 64 lanes per row, the longest rows in chunks of 4 096 entries whose
+ * sums meet in chunk order.  Structure only.  Per-call scratch: `chunks` elements. */
+typedef struct {
+  int32_t *rows;             /* m row numbers by class, ascending inside a class; NULL: no layout */
+  void *chunk_list;          /* chunks records */
+  int32_t *chunk_first;      /* count[3] + 1: first chunk of every long row */
+  int32_t count[4];          /* rows per class */
+  int32_t chunks;
+  int64_t device_bytes;
+} asamd_binned_layout;
+int asamd_binned_build(hipStream_t stream, int32_t m, int32_t base, const int32_t *row_ptr,
+                       asamd_binned_layout *out);
+void asamd_binned_free(asamd_binned_layout *layout);
+int asamd_spmv_binned(hipStream_t stream, const asamd_spmv_args *a, const asamd_binned_layout *layout,
+                      void *partial);
+
+/* CSR copy of A^T (conj != 0: of A^H, complex types): n + 1 offsets, nnz zero-based columns (rows of
+ * A, ascending inside a row of the copy), nnz values and the CSR position of every entry (perm),
+ * through which asamd_gather_values refreshes the values.  The reference always scatters
+ * (dcu_gemv_x_csr_trans.cpp:11-68); the ordinary kernels run on this copy instead. */
+typedef struct {
+  int32_t *row_ptr;          /* NULL: no copy */
+  int32_t *col_ind;
+  void *val;
+  uint32_t *perm;
+  int64_t device_bytes;
+} asamd_transpose_layout;
+int asamd_transpose_build(hipStream_t stream, int32_t dtype, int32_t conj, int32_t m, int32_t n, int32_t nnz,
+                          int32_t base, const int32_t *row_ptr, const int32_t *col_ind, const void *val,
+                          asamd_transpose_layout *out);
+void asamd_transpose_free(asamd_transpose_layout *layout);
+
+/* ---- analysis building blocks --------------------------------------------------------------- */
+/* One pass over row_ptr: stats_host[0] = shortest row, [1] = longest, [2] = row_ptr[0], [3 + b] = rows
+ * in bin b of the log2 histogram (bin 0: empty rows, bin b: 2^(b-1) .. 2^b - 1 entries).  d_scratch:
+ * ASAMD_ROW_STATS_WORDS device ints.  Synchronises `stream`.  Replaces the host-side row walk of
+ * src/util_cpp/alphasparse_dcu_x_csrmv_analysis.cpp:58-267 and its round trip at :348-379. */
+#define ASAMD_ROW_STATS_WORDS (3 + ASAMD_HIST_BINS)
+int asamd_csr_row_stats(hipStream_t stream, int32_t m, const int32_t *row_ptr, int32_t *d_scratch,
+                        int32_t *stats_host);
+/* 64-bit fingerprint of the structure arrays (m + 1 offsets, nnz columns): equal arrays give equal
+ * values.  d_scratch: 8 device bytes, 8-byte aligned.  Synchronises `stream`; *hash_host is a host word. */
 int asamd_csr_structure_hash(hipStream_t stream, int32_t m, int32_t nnz, const int32_t *row_ptr,
-                             const int32_t *col_ind, uint64_t *hash_host);
-
-/* CSR copy of the transpose, owned by the plan (trusted plans only; row_ptr,
- * col_ind, val are the arrays the plan was created for).  Later transposed
- * multiplies run the ordinary kernels on that copy (with an analysis of its
- * own: asamd_csr_plan_transpose_stats).  No reference counterpart: the
- * reference always scatters with atomics. */
-int asamd_csr_plan_build_transpose(hipStream_t stream, asamd_csr_plan *plan, const int32_t *row_ptr,
-                                   const int32_t *col_ind, const void *val);
-/* The same with conjugated values: a CSR copy of A^H (complex plans only). */
-int asamd_csr_plan_build_conj_transpose(hipStream_t stream, asamd_csr_plan *plan, const int32_t *row_ptr,
-                                        const int32_t *col_ind, const void *val);
-/* on != 0: the first transposed multiply builds that copy from the arrays it
- * is given (for matrices whose device arrays the library owns). */
-int asamd_csr_plan_set_lazy_transpose(asamd_csr_plan *plan, int32_t on);
-const asamd_csr_stats *asamd_csr_plan_transpose_stats(const asamd_csr_plan *plan);
-
-/* y = alpha*A^T*x + beta*y: x has m entries, y has n.  Uses the transposed copy
- * when the plan has one; otherwise scales y and scatters with hardware float
- * atomics (y must be ordinary device memory), as
- * src/kernel/dcu/level2/mv/csrmv/dcu_gemv_x_csr_trans.cpp:11-45, :49-68 does. */
-int asamd_s_csrmv_trans(hipStream_t stream, asamd_csr_plan *plan, float alpha, const float *val,
-                        const int32_t *row_ptr, const int32_t *col_ind, const float *x, float beta,
-                        float *y);
-int asamd_d_csrmv_trans(hipStream_t stream, asamd_csr_plan *plan, double alpha, const double *val,
-                        const int32_t *row_ptr, const int32_t *col_ind, const double *x, double beta,
-                        double *y);
-
-/* Complex element types: y = alpha*op(A)*x + beta*y with op = 0 (A), 1 (A^T), 2 (A^H), the
- * values of alphasparse_operation_t.  op = 0 stands in for csr_gemv_vector_dispatch as above,
- * op = 1 for dcu_gemv_x_csr_trans.cpp:11-68, op = 2 for csr_gemv_conj_scalar_atomicadd
- * (src/kernel/dcu/level2/mv/csrmv/dcu_gemv_c_csr_conj.cpp:22-75); 1 and 2 use the plan's copy
- * of A^T / A^H when it has one and scatter with atomics otherwise. */
-int asamd_c_csrmv_op(hipStream_t stream, asamd_csr_plan *plan, int32_t op, asamd_complex8 alpha,
-                     const asamd_complex8 *val, const int32_t *row_ptr, const int32_t *col_ind,
-                     const asamd_complex8 *x, asamd_complex8 beta, asamd_complex8 *y);
-int asamd_z_csrmv_op(hipStream_t stream, asamd_csr_plan *plan, int32_t op, asamd_complex16 alpha,
-                     const asamd_complex16 *val, const int32_t *row_ptr, const int32_t *col_ind,
-                     const asamd_complex16 *x, asamd_complex16 beta, asamd_complex16 *y);
-
-/* Arrays of the plan's CSR copy of A^T (conj == 0) or A^H (conj != 0): n + 1 row offsets, nnz
- * zero-based column indices (rows of A) and nnz values, owned by the plan.  hipErrorInvalidValue
- * if that copy has not been built. */
-int asamd_csr_plan_transpose_arrays(const asamd_csr_plan *plan, int32_t conj, const int32_t **row_ptr,
-                                    const int32_t **col_ind, const void **val);
+                             const int32_t *col_ind, void *d_scratch, uint64_t *hash_host);
+/* ---- values that change under a copy ---------------------------------------------------------
+ * The reference's analysis keeps structure only (alphasparse_dcu_x_csrmv_analysis.cpp:382-388) and its
+ * kernels read csr_val on every call (dcu_gemv_vector.h:43-46), so callers may rewrite the values in
+ * place between multiplies.  A copy of the values is kept honest on the device, without a host
+ * round trip and inside a HIP graph if need be:
+ *   asamd_value_guard      fingerprints val (nbytes; every byte when nbytes <= ASAMD_GUARD_FULL_BYTES or
+ *                          full != 0, otherwise 256 bytes at a varying position of every run of
+ *                          asamd_value_guard_run(nbytes) bytes, 32 MiB in all), compares with the word
+ *                          at `stored` and leaves the verdict in ws: a flag and the new fingerprint;
+ *   gated kernels          (asamd_gather_values, asamd_csr2ell_gated) take the flag's address and return
+ *                          at once when it is 0;
+ *   asamd_value_guard_commit   stores the new fingerprint at `stored` if the flag is set -- AFTER the
+ *                          gated kernels in stream order, so that another stream that finds the stored
+ *                          word up to date also finds the copies refreshed.
+ * stored == NULL in asamd_value_guard sets the flag whatever the values are (first fingerprint).
+ * ws: ASAMD_GUARD_WS_BYTES of per-call device scratch, 8-byte aligned. */
+#define ASAMD_GUARD_WS_BYTES (16384 + 64)
+#define ASAMD_GUARD_FULL_BYTES ((size_t)32 << 20)
+#define ASAMD_GUARD_FLAG(ws) ((const int32_t *)((const char *)(ws) + 16384 + 8))
+size_t asamd_value_guard_run(size_t nbytes);
+int asamd_value_guard(hipStream_t stream, const void *val, size_t nbytes, int32_t full, const uint64_t *stored,
+                      void *ws);
+int asamd_value_guard_commit(hipStream_t stream, const void *ws, uint64_t *stored);
+/* out[q] = val[perm[q]] (conj != 0: conjugated) for q < nnz; gate: NULL, or a device flag (0 = do nothing) */
+int asamd_gather_values(hipStream_t stream, int32_t dtype, int32_t conj, int32_t nnz, const uint32_t *perm,
+                        const void *val, void *out, const int32_t *gate);
 
 /* y = alpha*op(A)*x + beta*y without any analysis, in the traversal of the reference's plain
  * kernels: op = 0 one lane per row summing its entries in storage order
@@ -335,6 +360,11 @@ int asamd_c_csr2ell(hipStream_t stream, int32_t m, const asamd_complex8 *val, co
 int asamd_z_csr2ell(hipStream_t stream, int32_t m, const asamd_complex16 *val, const int32_t *row_ptr,
                     const int32_t *col_ind, int32_t csr_base, int32_t ell_base, int32_t width,
                     asamd_complex16 *ell_val, int32_t *ell_col);
+/* The same for elements of elem_bytes (4, 8 or 16) bytes, copied bit for bit, behind a gate: a device
+ * flag left by asamd_value_guard (0 = the conversion does nothing), or NULL. */
+int asamd_csr2ell_gated(hipStream_t stream, int32_t elem_bytes, int32_t m, const void *val, const int32_t *row_ptr,
+                        const int32_t *col_ind, int32_t csr_base, int32_t ell_base, int32_t width, void *ell_val,
+                        int32_t *ell_col, const int32_t *gate);
 
 /* y = alpha*A*x + beta*y, A in column-major ELL (slot s of row r at [s*m + r]);
  * slots whose index (minus base) is outside [0, n) are skipped.  Stands in for
@@ -379,52 +409,6 @@ int asamd_z_coomv(hipStream_t stream, int32_t m, int32_t n, int64_t nnz, asamd_c
                   int32_t base, const asamd_complex16 *x, asamd_complex16 beta, asamd_complex16 *y, void *workspace,
                   size_t workspace_bytes);
 
-/* Number of lazily made analyses (multiplies with info == NULL on arrays that no analysis or mirror
- * covers) that the library remembers at the moment: at most 64, the least recently used one makes room,
- * and a handle's own go with the handle.  For tests. */
-int asamd_registry_lazy_count(void);
-
-/* Introspection for benchmarks and tests: statistics of the analysis that a
- * multiply would use for `key`, where key is the alphasparse_dcu_mat_info_t of an
- * explicit analysis, or a device csr_row_ptr (library-built mirror or lazily
- * analysed array).  NULL if nothing is recorded.  Implemented by the host
- * library's registry; no reference counterpart. */
-const asamd_csr_stats *asamd_analysis_stats(const void *key);
-/* ... and of the analysis of the transposed copy, or NULL if there is none. */
-const asamd_csr_stats *asamd_analysis_transpose_stats(const void *key);
-/* Force a kernel family (enum asamd_spmv_algo) on the analysis recorded for
- * `key`; returns 0 on success, a hipError_t otherwise. */
-int asamd_analysis_set_algo(const void *key, int32_t algo);
-
-/* Plain 16-byte-per-lane copy of nbytes (a multiple of 16, both pointers 16-byte
- * aligned).  Exists to calibrate hardware byte counters against a transfer of
- * known size; no reference counterpart. */
-int asamd_copy_bytes(hipStream_t stream, void *dst, const void *src, size_t nbytes);
-
-/* Plain memory kernels that measure what the GPU sustains (the practical ceilings that the kernels'
- * roofline figures are read against); no reference counterpart.  kind: READ / WRITE / COPY stream nbytes
- * (a multiple of 16; 16 bytes per lane and access) from src / into dst; ROW_GATHER fetches `count`
- * 256-byte rows at random positions of the nbytes at src, one wave per row (what the row-major SpMM does
- * per entry of A with 64 dense columns); ELEM_GATHER fetches `count` single floats at random positions
- * (what a row SpMV kernel does per entry); RUN_GATHER / RUN_SCATTER copy nbytes in runs of `count` floats
- * (a multiple of 4) whose order differs between source and destination: the runs are contiguous on the
- * write side and scattered on the read side (what the second phase of the tiled SpMV reads), or the other
- * way round.  sink: 4 device bytes that are practically never written.
- * *bytes_moved receives the useful bytes of the launch (copy: read + written). */
-enum asamd_ceiling_kind {
-  ASAMD_CEILING_READ = 0,
-  ASAMD_CEILING_WRITE = 1,
-  ASAMD_CEILING_COPY = 2,
-  ASAMD_CEILING_ROW_GATHER = 3,
-  ASAMD_CEILING_ELEM_GATHER = 4,
-  ASAMD_CEILING_READ_NT = 5, /* the same streams with non-temporal accesses */
-  ASAMD_CEILING_COPY_NT = 6,
-  ASAMD_CEILING_RUN_GATHER = 7,
-  ASAMD_CEILING_RUN_SCATTER = 8
-};
-int asamd_ceiling_kernel(hipStream_t stream, int32_t kind, void *dst, const void *src, size_t nbytes,
-                         int64_t count, void *sink, int64_t *bytes_moved);
-
 /* handle->stream for callers that cannot see the handle struct (language bindings); C callers assign
  * the field, as with the reference.  `handle` is an alphasparse_dcu_handle_t.  Every multiply that
  * runs from an explicit analysis only launches kernels on that stream, so it can be captured into
@@ -435,6 +419,26 @@ hipStream_t asamd_handle_get_stream(void *handle);
 /* Empty kernel; forces code-object load (src/util_cpp/handle.cpp:19, :113).  Also looks up, for the
  * current device, the address of the fixed array that asamd_s_csrmv_noalloc works in. */
 int asamd_warmup(hipStream_t stream);
+
+/* asamd_s_csrmv without a plan and without any allocation: for callers that cannot call hipMalloc
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid it).  No counterpart in
+ * the reference.  Runs the merge-path kernels (any row-length distribution, no float atomics); their
+ * workgroup coordinates, carries and head sums live in a fixed device array of
+ * ASAMD_CSRMV_NOALLOC_SCRATCH_BYTES that the library holds per GPU until the process ends.
+ * m + nnz above ASAMD_CSRMV_NOALLOC_MAX_ITEMS returns hipErrorOutOfMemory (2) before anything is
+ * launched; other bad arguments return hipErrorInvalidValue.  base is 0 or 1; nnz == 0 gives
+ * y = beta*y.  Required and NOT checked (the check would need a look at device memory): row_ptr[0] ==
+ * base and nnz == row_ptr[m] - base, i.e. row_ptr describes exactly the nnz entries passed -- a slice
+ * of a larger matrix's row_ptr gives wrong results here.  Calls hipMalloc, hipFree or an allocating
+ * library routine never; asamd_warmup (run by alphasparse_dcu_get_handle) resolves the array's address
+ * for the current device; a first call on a device where that has not happened does so itself, which a
+ * stream under capture may not allow: call asamd_warmup first.  All calls on one GPU share the array:
+ * calls that overlap there (two streams, two threads) race; calls on one stream are ordered and safe. */
+#define ASAMD_CSRMV_NOALLOC_SCRATCH_BYTES (4 << 20)
+#define ASAMD_CSRMV_NOALLOC_MAX_ITEMS 536868864LL /* (SCRATCH_BYTES / 16 - 1) workgroups x 2048 items */
+int asamd_s_csrmv_noalloc(hipStream_t stream, int32_t m, int32_t n, int32_t nnz, int32_t base, float alpha,
+                          const float *val, const int32_t *row_ptr, const int32_t *col_ind, const float *x,
+                          float beta, float *y);
 
 #ifdef __cplusplus
 }

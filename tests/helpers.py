@@ -93,13 +93,15 @@ def run_plan_csrmv(da, algo, alpha, x, beta, y0, trusted=1):
         T = capi.scalar_type(a.dtype)
         dx = hiprt.DeviceArray.from_numpy(np.ascontiguousarray(x, dtype=a.dtype))
         dy = hiprt.DeviceArray.from_numpy(np.ascontiguousarray(y0, dtype=a.dtype))
-        e = getattr(lib, "asamd_%s_csrmv" % capi.prefix(a.dtype))(
-            None, plan, T(alpha), da.val.c_ptr(), da.row_ptr.c_ptr(), da.col.c_ptr(), dx.c_ptr(), T(beta), dy.c_ptr())
-        assert e == 0, "asamd csrmv hip error %d" % e
+        ws = capi.Workspace(lib, plan)
+        e = capi.plan_csrmv(lib, None, plan, 0, T(alpha), da.val.c_ptr(), da.row_ptr.c_ptr(), da.col.c_ptr(), dx.c_ptr(),
+                            T(beta), dy.c_ptr(), ws)
+        assert e == 0, "asamd_csr_plan_csrmv hip error %d" % e
         hiprt.synchronize()
         y = dy.to_numpy()
         dx.free()
         dy.free()
+        ws.buf.free()
         return y
     finally:
         lib.asamd_csr_plan_destroy(plan)

@@ -10,7 +10,7 @@ import pytest
 from alsparse_amd import capi
 from alsparse_amd.build import LIB_PATH, ROOT
 
-HEADERS = ["alphasparse.h", "alphasparse_util.h", "alpha_spblas_dcu.h", "alsparse_amd_kernels.h"]
+HEADERS = ["alphasparse.h", "alphasparse_util.h", "alpha_spblas_dcu.h", "alsparse_amd_kernels.h", "alsparse_amd_plan.h"]
 
 
 def declared_functions():
@@ -47,7 +47,7 @@ def test_python_bindings_cover_every_declared_symbol():
 
 def test_headers_compile_as_c_and_cxx(tmp_path):
     src = tmp_path / "t.c"
-    src.write_text('#include "alpha_spblas_dcu.h"\n#include "alsparse_amd_kernels.h"\n'
+    src.write_text('#include "alpha_spblas_dcu.h"\n#include "alsparse_amd_kernels.h"\n#include "alsparse_amd_plan.h"\n'
                    "int main(void){ alphasparse_dcu_handle h; (void)h; return sizeof(struct _alphasparse_dcu_mat_info) == 0; }\n")
     inc = ["-I" + os.path.join(ROOT, "include"), "-I/opt/rocm/include"]
     subprocess.check_call(["gcc", "-std=c11", "-Wall", "-Werror", "-fsyntax-only", str(src)] + inc)
@@ -76,7 +76,7 @@ def test_struct_layouts_match_c(tmp_path):
 #include <stdio.h>
 #include <stddef.h>
 #include "alpha_spblas_dcu.h"
-#include "alsparse_amd_kernels.h"
+#include "alsparse_amd_plan.h"
 int main(void) {
   printf("%zu %zu %zu %zu\n", sizeof(alphasparse_matrix), offsetof(alphasparse_matrix, format),
          offsetof(alphasparse_matrix, inspector), offsetof(alphasparse_matrix, dcu_info));

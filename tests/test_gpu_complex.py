@@ -138,11 +138,12 @@ def test_complex_kernel_families(gpu, dtype, algo):
                 assert algo in ("rowconst", "stream", "ell", "hot"), (algo, shape)
                 continue
             assert algo != "rowconst"
+            ws = capi.Workspace(lib, plan)
             for alpha, beta in SCALARS:
                 dx, dy = dev(x), dev(y0)
                 announce("complex family", np.dtype(dtype).name, shape, algo, alpha, beta)
-                assert getattr(lib, "asamd_%s_csrmv_op" % p)(None, plan, 0, T(alpha), da.val.c_ptr(), da.row_ptr.c_ptr(),
-                                                            da.col.c_ptr(), dx.c_ptr(), T(beta), dy.c_ptr()) == 0
+                assert capi.plan_csrmv(lib, None, plan, 0, T(alpha), da.val.c_ptr(), da.row_ptr.c_ptr(), da.col.c_ptr(),
+                                       dx.c_ptr(), T(beta), dy.c_ptr(), ws) == 0
                 hiprt.synchronize()
                 check(a, alpha, x, beta, y0, dy.to_numpy(), orc.csrmv_plain(a, alpha, x, beta, y0), "%s %s" % (shape, algo))
                 dx.free()

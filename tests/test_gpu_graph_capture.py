@@ -115,9 +115,11 @@ def test_every_kernel_family_replays_from_a_hip_graph(gpu, algo, shape):
                                          da.val.c_ptr(), a.base, a.dtype.itemsize, 2, byref(plan)) == 0
         assert lib.asamd_csr_plan_set_algo(plan, ALGOS[algo]) == 0, "this matrix can run every family"
 
+        ws = capi.Workspace(lib, plan)
+
         def multiply():
-            return lib.asamd_s_csrmv(stream, plan, ctypes.c_float(-0.75), da.val.c_ptr(), da.row_ptr.c_ptr(),
-                                     da.col.c_ptr(), dx.c_ptr(), ctypes.c_float(2.0), dy.c_ptr())
+            return capi.plan_csrmv(lib, stream, plan, 0, ctypes.c_float(-0.75), da.val.c_ptr(), da.row_ptr.c_ptr(),
+                                   da.col.c_ptr(), dx.c_ptr(), ctypes.c_float(2.0), dy.c_ptr(), ws)
         assert multiply() == 0
         hiprt.check(hip.hipStreamSynchronize(stream), "sync")
         eager = dy.to_numpy()

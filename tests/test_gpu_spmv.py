@@ -437,8 +437,9 @@ def test_copy_is_not_used_for_another_value_array(gpu, algo):
         for vals, mat in ((da.val, a), (d_new, b), (da.val, a)):
             announce("value array", algo, mat.name)
             dx, dy = hiprt.DeviceArray.from_numpy(x), hiprt.DeviceArray.from_numpy(y0)
-            assert lib.asamd_s_csrmv(None, plan, c_float(1.5), vals.c_ptr(), da.row_ptr.c_ptr(), da.col.c_ptr(),
-                                     dx.c_ptr(), c_float(0.5), dy.c_ptr()) == 0
+            ws = capi.Workspace(lib, plan)
+            assert capi.plan_csrmv(lib, None, plan, 0, c_float(1.5), vals.c_ptr(), da.row_ptr.c_ptr(), da.col.c_ptr(),
+                                   dx.c_ptr(), c_float(0.5), dy.c_ptr(), ws) == 0
             hiprt.synchronize()
             y = dy.to_numpy()
             dx.free()
@@ -522,11 +523,11 @@ def test_tiled_second_phase_in_both_forms(gpu, dtype, per_row, monkeypatch):
                 else:
                     assert st.tile_entries_per_lane == int(forced)
                 assert lib.asamd_csr_plan_set_algo(plan, ALGOS["tiled"]) == 0
+                ws = capi.Workspace(lib, plan)
                 for alpha, beta in ((1.0, 0.0), (-1.5, 0.5)):
                     dx, dy = hiprt.DeviceArray.from_numpy(x), hiprt.DeviceArray.from_numpy(y0)
-                    assert getattr(lib, "asamd_%s_csrmv" % capi.prefix(a.dtype))(
-                        None, plan, T(alpha), da.val.c_ptr(), da.row_ptr.c_ptr(), da.col.c_ptr(), dx.c_ptr(), T(beta),
-                        dy.c_ptr()) == 0
+                    assert capi.plan_csrmv(lib, None, plan, 0, T(alpha), da.val.c_ptr(), da.row_ptr.c_ptr(), da.col.c_ptr(),
+                                           dx.c_ptr(), T(beta), dy.c_ptr(), ws) == 0
                     hiprt.synchronize()
                     y = dy.to_numpy()
                     dx.free()

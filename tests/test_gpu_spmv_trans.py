@@ -134,8 +134,9 @@ def test_transposed_copy_matches_the_oracle_transpose_bit_for_bit(gpu, dtype):
         assert list(st.hist) == want_hist
         T = capi.scalar_type(dtype)
         dx, dy = hiprt.DeviceArray.from_numpy(x), hiprt.DeviceArray.from_numpy(y0)
-        assert getattr(lib, "asamd_%s_csrmv_trans" % capi.prefix(dtype))(
-            None, plan, T(2.0), da.val.c_ptr(), da.row_ptr.c_ptr(), da.col.c_ptr(), dx.c_ptr(), T(3.0), dy.c_ptr()) == 0
+        ws = capi.Workspace(lib, plan)
+        assert capi.plan_csrmv(lib, None, plan, 1, T(2.0), da.val.c_ptr(), da.row_ptr.c_ptr(), da.col.c_ptr(), dx.c_ptr(),
+                               T(3.0), dy.c_ptr(), ws) == 0
         hiprt.synchronize()
         assert np.array_equal(dy.to_numpy(), orc.csrmv_trans_plain(a, 2.0, x, 3.0, y0))
         dx.free()

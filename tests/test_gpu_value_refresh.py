@@ -50,8 +50,9 @@ def test_plan_refresh_values_brings_every_copy_up_to_date(gpu, algo, dtype):
         def multiply(trans):
             dx = hiprt.DeviceArray.from_numpy(xt if trans else x)
             dy = hiprt.DeviceArray.from_numpy(wl.uniform(a.cols, a.dtype, 6) if trans else y0)
-            fn = getattr(lib, "asamd_%s_csrmv%s" % (p, "_trans" if trans else ""))
-            assert fn(None, plan, T(1.5), da.val.c_ptr(), da.row_ptr.c_ptr(), da.col.c_ptr(), dx.c_ptr(), T(0.0), dy.c_ptr()) == 0
+            ws = capi.Workspace(lib, plan)
+            assert capi.plan_csrmv(lib, None, plan, 1 if trans else 0, T(1.5), da.val.c_ptr(), da.row_ptr.c_ptr(),
+                                   da.col.c_ptr(), dx.c_ptr(), T(0.0), dy.c_ptr(), ws) == 0
             hiprt.synchronize()
             out = dy.to_numpy()
             dx.free()

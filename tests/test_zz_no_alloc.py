@@ -2,7 +2,7 @@
 array) against the existing entry points, through the C-ABI.
 
 Bar: y within 1e-4 per row of the plain-kernel oracle (normalised by |alpha| sum|a x| + |beta y0|; by the products alone when beta == 0),
-and bit-equal to asamd_s_csrmv running the same merge-path kernels from a plan's allocated buffers.
+and bit-equal to asamd_csr_plan_csrmv running the same merge-path kernels in a caller-provided workspace.
 Two calls in a row share the array; the second is smaller, so slots the first call wrote stay behind."""
 from ctypes import byref, c_float, c_void_p
 
