@@ -134,7 +134,8 @@ class asamd_csr_stats(Structure):
                 ("hot_share_lds", c_float), ("tune_ms_hot", c_float),
                 ("binned_built", c_int32), ("bin_rows", c_int32 * 4), ("tune_ms_binned", c_float),
                 ("tile_long_blocks", c_int32), ("value_check", c_int32), ("tune_mode", c_int32),
-                ("device_bytes", c_int64), ("workspace_bytes", c_int64)]
+                ("device_bytes", c_int64), ("workspace_bytes", c_int64),
+                ("lines_per_entry_wave", c_float), ("lines_per_entry_segment", c_float)]
 
 
 class asamd_spmv_args(Structure):  # include/alsparse_amd_kernels.h
@@ -334,6 +335,7 @@ _COMMON = {
     "asamd_transpose_build": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P],
     "asamd_transpose_free": [_P],
     "asamd_csr_row_stats": [_P, _I, _P, _P, _P],
+    "asamd_csr_locality_probe": [_P, _I, _I, _I, _P, _I, _P, POINTER(c_float)],
     "asamd_value_guard_run": [c_size_t],
     "asamd_value_guard": [_P, _P, c_size_t, _I, _P, _P],
     "asamd_value_guard_commit": [_P, _P, _P],

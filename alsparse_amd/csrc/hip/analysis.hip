@@ -215,3 +215,78 @@ extern "C" int asamd_value_guard_commit(hipStream_t stream, const void* ws, uint
   value_commit_kernel<<<1, 1, 0, stream>>>((const GuardWs*)ws, (unsigned long long*)stored);
   return hipGetLastError();
 }
+
+// ---------------------------------------------------------------------------
+// Locality probe: where do the columns of consecutive entries fall?  `segments` runs of kProbeSegment
+// consecutive entries, spread evenly over the entry stream, one workgroup each.  Two counts, both of
+// 128-byte lines of x:
+//   wave scale     distinct lines among every 64 consecutive entries (one gather instruction of a wave in the
+//                  row and merge-path kernels issues that many requests to the L1),
+//   segment scale  distinct lines in the whole run (a bitmap in LDS; what a compute unit's neighbourhood of
+//                  the stream touches, reuse included).
+// Deterministic: the same arrays always give the same counts.
+// ---------------------------------------------------------------------------
+constexpr int kProbeSegment = 1 << 15;
+constexpr int kProbeBits = 1 << 18;  // 32 KiB bitmap
+
+__global__ __launch_bounds__(256) void locality_probe_kernel(int nnz, int base, int elem_shift, int segments,
+                                                             const int* __restrict__ col_ind,
+                                                             unsigned long long* __restrict__ out) {
+  __shared__ unsigned bitmap[kProbeBits / 32];
+  for (int i = threadIdx.x; i < kProbeBits / 32; i += 256) bitmap[i] = 0;
+  __syncthreads();
+  const int lane = threadIdx.x % kWave;
+  const int64_t seg_len = nnz < kProbeSegment ? nnz : kProbeSegment;
+  const int64_t room = (int64_t)nnz - seg_len;
+  const int64_t begin = segments > 1 ? room * blockIdx.x / (segments - 1) : 0;
+  unsigned wave_lines = 0, seg_lines = 0, entries = 0;
+  for (int64_t k0 = begin + (threadIdx.x / kWave) * kWave; k0 < begin + seg_len; k0 += 256) {
+    const int64_t k = k0 + lane;
+    const bool live = k < begin + seg_len;
+    // 128-byte line of x that the entry's gather touches
+    const unsigned line = live ? (unsigned)(((int64_t)(col_ind[k] - base) << elem_shift) >> 7) : 0xFFFFFFFFu;
+    // wave scale: a lane counts if no lower lane of the wave has its line
+    bool first = live;
+    for (int j = 0; j < kWave; ++j) {
+      const unsigned other = __shfl(line, j, kWave);
+      if (j < lane && other == line) first = false;
+    }
+    wave_lines += first ? 1u : 0u;
+    entries += live ? 1u : 0u;
+    if (live) {
+      // lines beyond the bitmap fold onto it (a hash: two lines rarely share a bit within one run)
+      const unsigned bit = (line ^ (line >> 18) * 0x9E3779B1u) & (kProbeBits - 1);
+      const unsigned old = atomicOr(&bitmap[bit >> 5], 1u << (bit & 31));
+      seg_lines += (old >> (bit & 31)) & 1u ? 0u : 1u;
+    }
+  }
+  unsigned long long v[3] = {wave_lines, seg_lines, entries};
+  for (int q = 0; q < 3; ++q) {
+    __syncthreads();  // block_sum_u64 reuses one LDS array
+    const unsigned long long total = block_sum_u64(v[q]);
+    if (threadIdx.x == 0 && total) atomicAdd(&out[q], total);
+  }
+}
+
+__global__ void zero3_u64_kernel(unsigned long long* p) {
+  if (threadIdx.x < 3) p[threadIdx.x] = 0;
+}
+
+extern "C" int asamd_csr_locality_probe(hipStream_t stream, int32_t nnz, int32_t base, int32_t elem_bytes,
+                                        const int32_t* col_ind, int32_t segments, void* d_scratch, float* out_host) {
+  if (!col_ind || !d_scratch || !out_host || ((uintptr_t)d_scratch & 7u) || nnz < 1 || segments < 1)
+    return hipErrorInvalidValue;
+  int shift = 0;
+  while ((1 << shift) < elem_bytes) ++shift;
+  if ((1 << shift) != elem_bytes || elem_bytes > 16) return hipErrorInvalidValue;
+  unsigned long long* d = (unsigned long long*)d_scratch;
+  zero3_u64_kernel<<<1, 64, 0, stream>>>(d);
+  locality_probe_kernel<<<segments, 256, 0, stream>>>(nnz, base, shift, segments, col_ind, d);
+  hipError_t e = hipGetLastError();
+  unsigned long long h[3] = {0, 0, 0};
+  if (e == hipSuccess) e = hipMemcpyAsync(h, d, sizeof(h), hipMemcpyDeviceToHost, stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(stream);
+  out_host[0] = h[2] ? (float)((double)h[0] / (double)h[2]) : 0.f;
+  out_host[1] = h[2] ? (float)((double)h[1] / (double)h[2]) : 0.f;
+  return e;
+}

@@ -62,9 +62,12 @@ static int env_value_check(void) {
   return 1;
 }
 
+/* ALSPARSE_AMD_TUNE = model (default): the analysis decides from the row statistics, the locality probe and fixed
+ * constants; timed: it times the candidates on scratch vectors, which follows the machine at hand more closely but
+ * depends on whatever else the GPU is doing at that moment. */
 static int env_tune_model(void) {
   const char *e = getenv("ALSPARSE_AMD_TUNE");
-  return e && !strcmp(e, "model");
+  return !(e && !strcmp(e, "timed"));
 }
 
 /* ---- kernel choice from the row statistics --------------------------------------------------------- */
@@ -779,6 +782,173 @@ static hipError_t tune_copies(hipStream_t stream, asamd_csr_plan *p, const int32
   return hipSuccess;
 }
 
+/* ---- analysis: deciding from a model ---------------------------------------------------------------
+ * The same decisions without a single timing run, so that one matrix always gets one family whatever else
+ * the GPU is doing while it is analysed.  A multiply is modelled as its matrix streams and its gathers of x,
+ *     t = sqrt(t_stream^2 + t_gather^2),   t_stream = algorithmic bytes / the family's streaming rate,
+ *                                          t_gather = entries * w * T(s),
+ * with the two numbers of the locality probe: w, the distinct 128-byte lines of x per entry among 64
+ * consecutive entries (how many requests a gather instruction sends to the L1), and s, the distinct lines per
+ * entry within 32 768 consecutive entries, which orders matrices by how far their gathers reach (uniform
+ * columns over 2 / 4 / 8 / 16 / 64 MiB of x: s = 0.43 / 0.63 / 0.79 / 0.89 / 0.94; a power-law graph with 32 MiB
+ * of x: 0.45; a stencil: 0.005).  T(s) and the rates are measurements of these kernels on an MI355X:
+ *     s      0     0.25   0.45   0.63   0.68   0.79   0.885   0.94   1      (entries whose line must come from
+ *     T ps   3.6   4.7    5.6    5.9    10.5   10.5   13.5    17.8   19      beyond an XCD's L2 wait 3 x longer)
+ *     TB/s   constant row length 6.0, staged row block 6.6 (one lane per row) / 5.2 (several), lane group per
+ *            row 2.4 x the share of its lanes that hold an entry, merge-path 2.9, ELL copy 6.1 (of its padded
+ *            streams); tiled pair: 0.045 ms + 2 x bytes / 5.6 TB/s, x 1 .. 1.5 with the spread of the row lengths,
+ *            x 2.5 for heavy-tailed rows.
+ * The estimates are within about 10 % of the timings on the shapes they were read from (5-point and 27-point
+ * stencils, uniform rows over 0.25 - 64 MiB of x, two row lengths, power-law rows and columns, fp32 / fp64). */
+static double gather_ps(double s) {
+  static const double xs[9] = {0.0, 0.25, 0.45, 0.63, 0.68, 0.79, 0.885, 0.94, 1.0};
+  static const double ys[9] = {3.6, 4.7, 5.6, 5.9, 10.5, 10.5, 13.5, 17.8, 19.0};
+  if (s <= xs[0]) return ys[0];
+  for (int i = 1; i < 9; ++i)
+    if (s <= xs[i]) return ys[i - 1] + (ys[i] - ys[i - 1]) * (s - xs[i - 1]) / (xs[i] - xs[i - 1]);
+  return ys[8];
+}
+
+static double hypot2(double a, double b) {
+  /* sqrt(a^2 + b^2) without libm: the larger of the two scaled by a few Newton steps */
+  const double big = a > b ? a : b, small = a > b ? b : a;
+  if (big <= 0.0) return 0.0;
+  const double q = small / big, v = 1.0 + q * q;
+  double r = 1.0 + 0.5 * q * q; /* sqrt(v) for v in [1, 2] */
+  for (int i = 0; i < 4; ++i) r = 0.5 * (r + v / r);
+  return big * r;
+}
+
+/* share of the lanes of a W-lane group that hold an entry, over the rows of the log2 histogram */
+static double vector_utilisation(const asamd_csr_stats *st, int w) {
+  double used = 0.0, slots = 0.0;
+  for (int b = 1; b < ASAMD_HIST_BINS; ++b) {
+    if (!st->hist[b]) continue;
+    const double len = b == 1 ? 1.0 : 0.75 * (double)((int64_t)1 << b); /* middle of [2^(b-1), 2^b) */
+    const double trips = (double)(int64_t)((len + w - 1) / w);
+    used += (double)st->hist[b] * len;
+    slots += (double)st->hist[b] * trips * w;
+  }
+  return slots > 0.0 ? used / slots : 1.0;
+}
+
+static double model_ms(const asamd_csr_plan *p, int algo) {
+  const asamd_csr_stats *st = &p->st;
+  const double vs = (double)p->val_size, nnz = (double)st->nnz, m = (double)st->m, n = (double)st->n;
+  const double bytes = nnz * (4.0 + vs) + (m + 1.0) * 4.0 + (n + m) * vs;
+  const double gather = nnz * (double)st->lines_per_entry_wave * gather_ps((double)st->lines_per_entry_segment) * 1e-9;
+  const double mean = nnz / (m > 0 ? m : 1);
+  double rate = 2.9; /* TB/s */
+  switch (algo) {
+    case ASAMD_SPMV_ROWCONST: rate = 6.0; break;
+    case ASAMD_SPMV_STREAM: rate = stream_group(p, 0) > 1 ? 5.2 : 6.6; break;
+    case ASAMD_SPMV_VECTOR: rate = 2.4 * vector_utilisation(st, p->auto_width); break;
+    case ASAMD_SPMV_MERGE: rate = 2.9; break;
+    case ASAMD_SPMV_ELL: {
+      const double ell_bytes = m * (double)st->max_len * (4.0 + vs) + (n + m) * vs;
+      return hypot2(ell_bytes / 6.1e9, gather);
+    }
+    case ASAMD_SPMV_TILED: {
+      double skew = 1.0 + 0.5 * ((double)st->max_len / mean - 1.0) / 8.0;
+      if (skew > 1.5) skew = 1.5;
+      if ((double)st->max_len > 32.0 * mean + 256.0) skew = 2.5; /* heavy tail: long tiles, uneven waves */
+      return (0.045 + 2.0 * bytes / 5.6e9) * skew;
+    }
+    default: break;
+  }
+  return hypot2(bytes / (rate * 1e9), gather);
+}
+
+static hipError_t model_copies(hipStream_t stream, asamd_csr_plan *p, const int32_t *row_ptr, const int32_t *col_ind,
+                               const void *val, int tiled_ok, int ell_ok, int hot_ok, int binned_ok) {
+  asamd_csr_stats *st = &p->st;
+  if (st->lines_per_entry_wave <= 0.f) return hipSuccess; /* not probed (a tiny matrix): the structural choice stays */
+  double base = model_ms(p, p->auto_algo);
+  if (structural_alternatives(p)) {
+    const int alts[2] = {ASAMD_SPMV_MERGE, p->auto_algo == ASAMD_SPMV_STREAM ? ASAMD_SPMV_VECTOR : -1};
+    for (int i = 0; i < 2; ++i) {
+      if (alts[i] < 0) continue;
+      const double alt = model_ms(p, alts[i]);
+      if (alt < 0.97 * base) {
+        p->auto_algo = p->struct_algo = alts[i];
+        base = alt;
+      }
+    }
+  }
+  st->algo = p->auto_algo;
+  st->tune_ms_base = (float)base;
+  /* the copies in the order of their estimates; each is laid out only if it is the best one left */
+  const double est_tiled = tiled_ok ? model_ms(p, ASAMD_SPMV_TILED) : 0.0;
+  const double est_ell = ell_ok ? model_ms(p, ASAMD_SPMV_ELL) : 0.0;
+  st->tune_ms_tiled = (float)est_tiled;
+  st->tune_ms_ell = (float)est_ell;
+  /* The per-class launches read short rows in pieces of a few bytes; they win where the long rows hold nearly
+   * all the entries and the gathers are cheap (x stays in the caches, neighbouring lanes share lines). */
+  int want_binned = 0;
+  if (binned_ok && p->auto_algo == ASAMD_SPMV_MERGE && st->lines_per_entry_wave <= 0.25f) {
+    /* rows of fewer than 128 entries hold at most this many entries (bin b: up to 2^b - 1 each) */
+    double short_entries = 0.0;
+    for (int b = 1; b < 8; ++b) short_entries += (double)st->hist[b] * (double)(((int64_t)1 << b) - 1);
+    want_binned = short_entries <= 0.1 * (double)st->nnz;
+  }
+  const char *ev = getenv("ALSPARSE_AMD_TUNE_PICK");
+  int forced = -1;
+  if (ev) {
+    static const char *names[CAND_COUNT] = {"base", "tiled", "ell", "hot", "binned"};
+    for (int c = 0; c < CAND_COUNT; ++c)
+      if (!strcmp(ev, names[c])) forced = c;
+  }
+  int order[3] = {CAND_BASE, CAND_BASE, CAND_BASE};
+  const int tiled_wins = tiled_ok && est_tiled < 0.9 * base, ell_wins = ell_ok && est_ell < 0.95 * base;
+  int k = 0;
+  if (forced > 0) {
+    order[k++] = forced;
+  } else if (forced < 0) {
+    if (want_binned) order[k++] = CAND_BINNED;
+    if (tiled_wins && ell_wins) {
+      order[k++] = est_tiled < est_ell ? CAND_TILED : CAND_ELL;
+      order[k++] = est_tiled < est_ell ? CAND_ELL : CAND_TILED;
+    } else if (tiled_wins) {
+      order[k++] = CAND_TILED;
+    } else if (ell_wins) {
+      order[k++] = CAND_ELL;
+    }
+  }
+  hipError_t e = hipSuccess;
+  for (int i = 0; i < k && e == hipSuccess; ++i) {
+    int built = 0, algo = p->auto_algo;
+    switch (order[i]) {
+      case CAND_TILED:
+        if (tiled_ok) e = build_tiled(stream, p, row_ptr, col_ind, val);
+        built = st->tiled_built;
+        algo = ASAMD_SPMV_TILED;
+        break;
+      case CAND_ELL:
+        if (ell_ok) e = build_ell(stream, p, row_ptr, col_ind, val);
+        built = st->ell_built;
+        algo = ASAMD_SPMV_ELL;
+        break;
+      case CAND_HOT:
+        if (hot_ok) e = build_hot(stream, p, row_ptr, col_ind, 1);
+        built = st->hot_built;
+        algo = ASAMD_SPMV_MERGE_HOT;
+        break;
+      case CAND_BINNED:
+        if (binned_ok) e = build_binned(stream, p, row_ptr);
+        built = st->binned_built;
+        algo = ASAMD_SPMV_BINNED;
+        break;
+      default: break;
+    }
+    if (e == hipSuccess && built) {
+      p->auto_algo = algo;
+      st->algo = algo;
+      break;
+    }
+  }
+  return e;
+}
+
 /* the fingerprint of the values a copy set was taken from (set-up work: plan-owned scratch, not concurrent) */
 static hipError_t first_fingerprint(hipStream_t stream, asamd_csr_plan *p, const void *val, int slot) {
   if (!p->st.value_check) return hipSuccess;
@@ -844,6 +1014,17 @@ static hipError_t plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t 
       return e;
     }
   }
+  if (col_ind && nnz >= 4096 && st->trusted) {
+    /* where the columns of neighbouring entries fall: two numbers for the record and for the model */
+    float probe[2] = {0.f, 0.f};
+    e = (hipError_t)asamd_csr_locality_probe(stream, nnz, base, val_size, col_ind, 64, p->d_setup, probe);
+    if (e != hipSuccess) {
+      asamd_csr_plan_destroy(p);
+      return e;
+    }
+    st->lines_per_entry_wave = probe[0];
+    st->lines_per_entry_segment = probe[1];
+  }
   if (col_ind && val && nnz > 0) {
     /* trusted == 2: build every copy whatever the size and skip the timing
      * (lets small matrices exercise those kernels) */
@@ -856,7 +1037,8 @@ static hipError_t plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t 
       if (e == hipSuccess && ell_ok) e = build_ell(stream, p, row_ptr, col_ind, val);
       if (e == hipSuccess && hot_ok) e = build_hot(stream, p, row_ptr, col_ind, 1);
     } else if (tiled_ok || ell_ok || hot_ok || binned_ok || structural_alternatives(p)) {
-      e = tune_copies(stream, p, row_ptr, col_ind, val, tiled_ok, ell_ok, hot_ok, binned_ok);
+      e = st->tune_mode ? model_copies(stream, p, row_ptr, col_ind, val, tiled_ok, ell_ok, hot_ok, binned_ok)
+                        : tune_copies(stream, p, row_ptr, col_ind, val, tiled_ok, ell_ok, hot_ok, binned_ok);
     }
     if (e == hipErrorOutOfMemory) {
       (void)hipGetLastError(); /* the copies are optional: carry on without them */

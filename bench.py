@@ -139,9 +139,13 @@ def vendor_spmv(a, x, y0, alpha, beta, nbytes, steps, warmup, transpose=False):
 
 
 def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False, vendor=False, cx=False, conjugate=False,
-             analyse=None):
+             analyse=None, structure_only=False, cold_copies=0, tune=None):
     """cx: the configuration's structure with complex values (complex64 for the fp32 configurations,
-    complex128 for the fp64 one), complex x, y, alpha and beta; conjugate: A^H instead of A^T."""
+    complex128 for the fp64 one), complex x, y, alpha and beta; conjugate: A^H instead of A^T.
+    structure_only: the analysis keeps no copy of the values (ALSPARSE_AMD_ANALYSIS=structure, what the reference's
+    analysis keeps).  cold_copies = K > 1: the multiply is also timed rotating over K copies of the matrix and its
+    vectors, each with an analysis of its own, so that no step finds anything of its operands in the 256 MB
+    memory-side cache ("cold").  tune: "timed" makes the analysis time its candidates instead of deciding from its model (ALSPARSE_AMD_TUNE)."""
     from alsparse_amd import capi, hiprt, workloads as wl
     lib = capi.load()
     t0 = time.time()
@@ -198,6 +202,13 @@ def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False, vendor=Fa
         if s != 0:
             raise RuntimeError("csrmv status %d" % s)
 
+    env_set = {}
+    if structure_only:
+        env_set["ALSPARSE_AMD_ANALYSIS"] = "structure"
+    if tune:
+        env_set["ALSPARSE_AMD_TUNE"] = tune
+    env_old = {k: os.environ.get(k) for k in env_set}
+    os.environ.update(env_set)
     hiprt.synchronize()
     t0 = time.perf_counter()
     if analysed:
@@ -247,6 +258,34 @@ def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False, vendor=Fa
         d_y.copy_from(y0)
 
     t = time_steps(step, steps, warmup, hiprt)
+    cold = None
+    if cold_copies > 1 and analysed and not transpose:
+        # K copies of everything a multiply touches, used in turn: with K * footprint well beyond the 256 MB
+        # memory-side cache every step reads its operands from HBM
+        copies = []
+        for _ in range(cold_copies):
+            arrs = [hiprt.DeviceArray.from_numpy(v) for v in (a.values, a.row_ptr, a.col_ind, x, y0)]
+            inf = capi.alphasparse_dcu_mat_info_t()
+            assert lib.alphasparse_dcu_create_mat_info(byref(inf)) == 0
+            assert getattr(lib, "alphasparse_dcu_%s_csrmv_analysis" % p)(
+                h.h, op, a.rows, a.cols, a.nnz, byref(descr), arrs[0].c_ptr(), arrs[1].c_ptr(), arrs[2].c_ptr(), inf) == 0
+            copies.append((arrs, inf))
+        turn = [0]
+
+        def cold_step():
+            arrs, inf = copies[turn[0] % cold_copies]
+            turn[0] += 1
+            s = csrmv(h.h, op, a.rows, a.cols, a.nnz, byref(al), byref(descr), arrs[0].c_ptr(), arrs[1].c_ptr(),
+                      arrs[2].c_ptr(), inf, arrs[3].c_ptr(), byref(be), arrs[4].c_ptr())
+            if s != 0:
+                raise RuntimeError("csrmv status %d" % s)
+        cold = time_steps(cold_step, steps, warmup, hiprt)
+        cold["copies"] = cold_copies
+        cold["kernel"] = capi.ALGO_NAMES.get(lib.asamd_analysis_stats(copies[0][1]).contents.algo, "?")
+        for arrs, inf in copies:
+            lib.alphasparse_dcu_destroy_mat_info(inf)
+            for d in arrs:
+                d.free()
     # the analysis repeated on the same arrays, as a caller does after rewriting csr_val in place: the structure
     # is fingerprinted, found unchanged, and only the values of the plan's copies are gathered again
     hiprt.synchronize()
@@ -257,10 +296,18 @@ def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False, vendor=Fa
         assert st == 0, "repeated analysis status %d" % st
     hiprt.synchronize()
     reanalysis_ms = (time.perf_counter() - t0) * 1e3 if analysed else None
+    for k, v in env_old.items():
+        if v is None:
+            os.environ.pop(k, None)
+        else:
+            os.environ[k] = v
     nbytes = (wl.spmv_bytes(a.cols, a.rows, a.nnz, a.dtype.itemsize, beta) if transpose
               else wl.spmv_bytes(a.rows, a.cols, a.nnz, a.dtype.itemsize, beta))
     opname = "" if not transpose else (" -- CONJUGATE-TRANSPOSED operation" if op == 2 else " -- TRANSPOSED operation")
-    res = {"workload": workload_name + (" -- COMPLEX values (%s)" % a.dtype.name if cx else "") + opname + ("" if analysed else " -- WITHOUT analysis (info = NULL)"), "rows": a.rows, "nnz": a.nnz, "algorithmic_bytes": int(nbytes),
+    mode = "" if analysed else " -- WITHOUT analysis (info = NULL)"
+    if structure_only:
+        mode = " -- analysis keeps STRUCTURE ONLY (no copy of the values, as the reference's)"
+    res = {"workload": workload_name + (" -- COMPLEX values (%s)" % a.dtype.name if cx else "") + opname + mode, "rows": a.rows, "nnz": a.nnz, "algorithmic_bytes": int(nbytes),
            "flops": 2 * a.nnz, "kernel": algo, "analysis_ms": analysis_ms, "reanalysis_ms": reanalysis_ms, "timing": t,
            "gbs": nbytes / t["avg_ms"] / 1e6, "gflops": 2 * a.nnz / t["avg_ms"] / 1e6,
            "dtype": {"float32": "f32", "float64": "f64", "complex64": "c64", "complex128": "c128"}[a.dtype.name],
@@ -271,6 +318,18 @@ def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False, vendor=Fa
         res["flops"], res["gflops"] = 8 * a.nnz, 8 * a.nnz / t["avg_ms"] / 1e6
     res["hbm_frac"] = res["gbs"] / HBM_PEAK_GBS
     res["traffic"], res["traffic_source"] = (None, None) if (transpose or cx or isinstance(cfg, tuple)) else measured_traffic(cfg, algo)
+    # device memory that the analysis holds beside the caller's CSR arrays, and the per-call scratch in the handle
+    res["analysis_bytes"] = int(stats.device_bytes)
+    res["workspace_bytes"] = int(stats.workspace_bytes)
+    res["value_check"] = {0: "off", 1: "sampled fingerprint of csr_val before every multiply that uses a copy",
+                          2: "full fingerprint"}[int(stats.value_check)]
+    res["tune_mode"] = "model" if stats.tune_mode else "timed"
+    res["locality_probe"] = {"lines_per_entry_wave": float(stats.lines_per_entry_wave),
+                             "lines_per_entry_segment": float(stats.lines_per_entry_segment)}
+    if cold:
+        res["cold"] = {"ms": cold["avg_ms"], "min_ms": cold["min_ms"], "gbs": nbytes / cold["avg_ms"] / 1e6,
+                       "frac_of_8TBps": nbytes / cold["avg_ms"] / 1e6 / HBM_PEAK_GBS, "copies_rotated": cold["copies"],
+                       "kernel": cold["kernel"]}
 
     if cpu_baseline and not transpose:
         res["cpu_baseline"] = cpu_spmv(a, x, y0, alpha, beta, nbytes)
@@ -559,12 +618,13 @@ def run_spmm(steps, warmup, check, col_major=False, vendor=False, stencil=None, 
     return res
 
 
-def run_ceilings(steps, warmup):
-    """What this GPU sustains with plain kernels (alsparse_amd/csrc/hip/ceilings.hip): 2 GiB read-only, write-only
+def run_ceilings(steps, warmup, short=False):
+    """What this GPU sustains with plain kernels (alsparse_amd/probes/ceilings.hip): 2 GiB read-only, write-only
     and copy streams, copies in short runs that one side reads or writes out of order (the product runs of the
     tiled SpMV's second phase), whole 256-byte rows gathered at random from 256 MiB (the B operand of configuration 5) and
     single floats gathered at random from 64 MiB / 4 MiB / 16 KiB (the x of configuration 3; an L2-sized x; an
-    L1-sized x).  TB/s of useful bytes, and gathers per second."""
+    L1-sized x).  TB/s of useful bytes, and gathers per second.  short: only the ones that the configurations' figures
+    are read against (the default line carries them)."""
     from ctypes import c_int64
     from alsparse_amd import capi, hiprt
     lib = capi.load_probes()
@@ -587,17 +647,22 @@ def run_ceilings(steps, warmup):
         return out[name]
     measure("read_2GiB", 0, None, a.c_ptr(), big, 0)
     measure("read_2GiB_nontemporal", 5, None, a.c_ptr(), big, 0)
-    measure("write_2GiB", 1, b.c_ptr(), None, big, 0)
+    if not short:
+        measure("write_2GiB", 1, b.c_ptr(), None, big, 0)
     measure("copy_2GiB", 2, b.c_ptr(), a.c_ptr(), big, 0)
-    measure("copy_2GiB_nontemporal", 6, b.c_ptr(), a.c_ptr(), big, 0)
-    for runlen in (64, 80, 160):
+    if not short:
+        measure("copy_2GiB_nontemporal", 6, b.c_ptr(), a.c_ptr(), big, 0)
+    for runlen in ((80,) if short else (64, 80, 160)):
         measure("copy_1GiB_in_runs_of_%d_floats_gathered" % runlen, 7, b.c_ptr(), a.c_ptr(), 1 << 30, runlen)
-        measure("copy_1GiB_in_runs_of_%d_floats_scattered" % runlen, 8, b.c_ptr(), a.c_ptr(), 1 << 30, runlen)
+        if not short:
+            measure("copy_1GiB_in_runs_of_%d_floats_scattered" % runlen, 8, b.c_ptr(), a.c_ptr(), 1 << 30, runlen)
     r = measure("row_gather_256B_from_256MiB", 3, None, a.c_ptr(), 256 << 20, 1 << 25)
     r["rows_per_s"] = r["useful_bytes"] / 256 / r["avg_ms"] * 1e3
-    r = measure("row_gather_256B_from_2GiB", 3, None, a.c_ptr(), big, 1 << 25)
-    r["rows_per_s"] = r["useful_bytes"] / 256 / r["avg_ms"] * 1e3
-    for label, nb in (("64MiB", 64 << 20), ("32MiB", 32 << 20), ("4MiB", 4 << 20), ("2MiB", 2 << 20), ("16KiB", 16 << 10)):
+    if not short:
+        r = measure("row_gather_256B_from_2GiB", 3, None, a.c_ptr(), big, 1 << 25)
+        r["rows_per_s"] = r["useful_bytes"] / 256 / r["avg_ms"] * 1e3
+    sizes = (("64MiB", 64 << 20), ("32MiB", 32 << 20), ("4MiB", 4 << 20), ("2MiB", 2 << 20), ("16KiB", 16 << 10))
+    for label, nb in (sizes[:3] if short else sizes):
         r = measure("elem_gather_4B_from_" + label, 4, None, a.c_ptr(), nb, 1 << 28)
         r["gathers_per_s"] = r["useful_bytes"] / 4 / r["avg_ms"] * 1e3
     for d in (a, b, sink):
@@ -605,13 +670,60 @@ def run_ceilings(steps, warmup):
     return out
 
 
-def brief(r):
+def against_ceiling(cfg, r, ceilings):
+    """The measured ceiling that bounds the configuration's kernel, named, and how close the kernel runs to it.
+    C2 streams its algorithmic bytes once: the non-temporal read rate.  C3's tiled pair moves its streams twice
+    (products out and in again): its real traffic (counter measurement, `traffic`) against the copy rate.
+    C4 and the row kernels on C3 gather single elements of x that miss the L1: entries per second against the
+    4-byte gather rates from an L2-resident array and from one of x's size.  C5 fetches one 256-byte row of B per
+    entry of A: rows per second against the random 256-byte row rate."""
+    if not ceilings:
+        return None
+    ms = r["timing"]["avg_ms"]
+    kernel = r.get("kernel") or ""
+    if cfg == 5:
+        c = ceilings["row_gather_256B_from_256MiB"]
+        got = r["nnz"] / ms * 1e3
+        return {"ceiling": "random 256-byte rows gathered from 256 MiB (probe kernel)", "ceiling_value": c["rows_per_s"],
+                "achieved": got, "unit": "rows of B per second", "frac_of_ceiling": got / c["rows_per_s"]}
+    if kernel.startswith("tiled") and r.get("traffic"):
+        c = ceilings["copy_2GiB"]
+        got = r["traffic"] / ms / 1e9
+        return {"ceiling": "plain copy of 2 GiB (probe kernel); achieved = measured HBM traffic of the kernel pair / time",
+                "ceiling_value": c["tb_per_s"], "achieved": got, "unit": "TB/s of real traffic",
+                "frac_of_ceiling": got / c["tb_per_s"]}
+    if kernel.startswith("row-block stream") or kernel.startswith("ell"):
+        c = ceilings["read_2GiB_nontemporal"]
+        got = r["algorithmic_bytes"] / ms / 1e9
+        return {"ceiling": "non-temporal read of 2 GiB (probe kernel)", "ceiling_value": c["tb_per_s"], "achieved": got,
+                "unit": "TB/s", "frac_of_ceiling": got / c["tb_per_s"]}
+    # gather-bound row kernels and merge-path
+    foot = "64MiB" if cfg == 3 else "32MiB"
+    c_l2, c_x = ceilings["elem_gather_4B_from_4MiB"], ceilings["elem_gather_4B_from_" + foot]
+    got = r["nnz"] / ms * 1e3
+    return {"ceiling": "random 4-byte gathers from an L2-sized array (4 MiB; probe kernel); also given: from an array "
+                       "of x's size (%s)" % foot,
+            "ceiling_value": c_l2["gathers_per_s"], "ceiling_value_at_x_size": c_x["gathers_per_s"], "achieved": got,
+            "unit": "gathers of x per second", "frac_of_ceiling": got / c_l2["gathers_per_s"],
+            "frac_of_ceiling_at_x_size": got / c_x["gathers_per_s"]}
+
+
+def brief(r, cfg=None, ceilings=None):
     """The figures of one configuration that the default line carries under `others`."""
     t = r["timing"]
-    return {"workload": r["workload"], "kernel": r.get("kernel"), "dtype": r["dtype"], "ms": t["avg_ms"], "min_ms": t["min_ms"],
-            "gbs": r["gbs"], "gflops": r["gflops"], "hbm_frac": r["hbm_frac"], "algorithmic_bytes": r["algorithmic_bytes"],
-            "analysis_ms": r.get("analysis_ms"), "reanalysis_ms": r.get("reanalysis_ms"), "parity": r["parity"], "traffic": r.get("traffic"),
-            "traffic_source": r.get("traffic_source")}
+    out = {"workload": r["workload"], "kernel": r.get("kernel"), "dtype": r["dtype"], "ms": t["avg_ms"], "min_ms": t["min_ms"],
+           "gbs": r["gbs"], "gflops": r["gflops"], "frac_of_8TBps": r["hbm_frac"], "algorithmic_bytes": r["algorithmic_bytes"],
+           "analysis_ms": r.get("analysis_ms"), "reanalysis_ms": r.get("reanalysis_ms"), "parity": r["parity"], "traffic": r.get("traffic"),
+           "traffic_source": r.get("traffic_source"), "analysis_bytes": r.get("analysis_bytes"),
+           "workspace_bytes": r.get("workspace_bytes")}
+    if r.get("cold"):
+        out["cold"] = r["cold"]
+        out["note"] = ("ms / gbs: the same matrix multiplied back to back, as a solver does -- its values, x and y then come "
+                       "from the 256 MB memory-side cache and only part of the bytes from HBM, so frac_of_8TBps is NOT a "
+                       "fraction of HBM bandwidth; cold: rotating over copies so that every operand comes from HBM")
+    if cfg is not None:
+        out["against_ceiling"] = against_ceiling(cfg, r, ceilings)
+    return out
 
 
 def main():
@@ -715,18 +827,26 @@ def main():
         main_res = run_spmv(cfg, args.steps, args.warmup, not args.no_cpu_baseline, check, args.transpose,
                             not args.no_vendor_baseline, args.cx, args.conjugate)
     others = {}
+    ceilings = None
     plain_default = (args.config == 3 and not (args.all or args.only or args.uniform or args.bimodal or args.stencil3d or args.no_analysis or args.transpose or args.cx or
                                                args.conversions or args.col_major) and args.format == "csr")
     if plain_default:
+        # what this GPU sustains with plain kernels, measured in this very run: the figures below are read against it
+        ceilings = run_ceilings(5, 1, short=True)
         # the default line is configuration 3; the other device configurations ride along, briefly
         for c in (2, 4, 5):
             r = (run_spmm(args.steps, args.warmup, check) if c == 5
-                 else run_spmv(c, args.steps, args.warmup, False, check, False, False))
-            others["C%d" % c] = brief(r)
-        # and two of them as a caller who never analyses sees them (info = NULL, as the reference's own tests call)
-        for c in (2, 4):
-            others["C%d_without_analysis" % c] = brief(run_spmv(c, args.steps, args.warmup, False, check, False, False,
-                                                               analyse=False))
+                 else run_spmv(c, args.steps, args.warmup, False, check, False, False, cold_copies=5 if c == 2 else 0))
+            others["C%d" % c] = brief(r, c, ceilings)
+        # as a caller who never analyses sees them (info = NULL, as the reference's own tests call,
+        # test/dcu/level2/mv_csr_s_dcu_test.cpp:220-222), and configuration 3 with an analysis that keeps structure
+        # only, as the reference's does
+        few = max(2, min(args.steps, 10))
+        for c in (2, 3, 4):
+            others["C%d_without_analysis" % c] = brief(run_spmv(c, args.steps if c != 3 else few, args.warmup if c != 3 else 1,
+                                                               False, check, False, False, analyse=False), c, ceilings)
+        others["C3_structure_only"] = brief(run_spmv(3, few, 1, False, check, False, False, structure_only=True), 3, ceilings)
+        others["C3_timed_analysis"] = brief(run_spmv(3, few, 1, False, False, False, False, tune="timed"), 3, ceilings)
     if args.all:
         for c in (2, 3, 4, 5):
             if c == args.config and not args.transpose and args.format == "csr" and not args.col_major:
@@ -781,6 +901,12 @@ def main():
         "cpu_baseline": main_res.get("cpu_baseline"),
         "vendor_baseline": main_res.get("vendor_baseline"),
     }
+    for k in ("analysis_bytes", "workspace_bytes", "value_check", "tune_mode", "locality_probe"):
+        if main_res.get(k) is not None:
+            out["config"][k] = main_res[k]
+    if ceilings:
+        out["ceilings"] = {k: {kk: vv for kk, vv in v.items() if kk != "useful_bytes"} for k, v in ceilings.items()}
+        out["roofline"]["against_ceiling"] = against_ceiling(args.config, main_res, ceilings)
     if conv:
         others["csr2ell"] = {k: v for k, v in conv["csr2ell"].items() if k != "timing"}
     if others:

@@ -222,6 +222,15 @@ int asamd_csr_row_stats(hipStream_t stream, int32_t m, const int32_t *row_ptr, i
  * values.  d_scratch: 8 device bytes, 8-byte aligned.  Synchronises `stream`; *hash_host is a host word. */
 int asamd_csr_structure_hash(hipStream_t stream, int32_t m, int32_t nnz, const int32_t *row_ptr,
                              const int32_t *col_ind, void *d_scratch, uint64_t *hash_host);
+/* A deterministic look at where the columns of consecutive entries fall: `segments` runs of 32 768
+ * consecutive entries spread evenly over the entry stream.  out_host[0] = distinct 128-byte lines of x per
+ * entry among every 64 consecutive entries (1/64 .. 1: the requests that one gather instruction of a wave
+ * sends to the L1), out_host[1] = distinct lines per entry within a whole run (reuse inside a compute unit's
+ * neighbourhood of the stream counted once).  d_scratch: 24 device bytes, 8-byte aligned.  Synchronises
+ * `stream`.  The same arrays always give the same two numbers. */
+int asamd_csr_locality_probe(hipStream_t stream, int32_t nnz, int32_t base, int32_t elem_bytes,
+                             const int32_t *col_ind, int32_t segments, void *d_scratch, float *out_host);
+
 /* ---- values that change under a copy ---------------------------------------------------------
  * The reference's analysis keeps structure only (alphasparse_dcu_x_csrmv_analysis.cpp:382-388) and its
  * kernels read csr_val on every call (dcu_gemv_vector.h:43-46), so callers may rewrite the values in

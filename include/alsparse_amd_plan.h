@@ -63,6 +63,9 @@ typedef struct {
   int32_t tune_mode;     /* 0: candidates were timed inside the analysis, 1: decided by the model alone */
   int64_t device_bytes;  /* device memory that the plan holds (layouts, copies, coordinates)            */
   int64_t workspace_bytes; /* per-call scratch that a multiply with this plan may ask for              */
+  float lines_per_entry_wave;    /* locality probe (asamd_csr_locality_probe): distinct 128-byte lines of x
+                                    per entry among 64 consecutive entries, or 0 if not probed          */
+  float lines_per_entry_segment; /* ... and within runs of 32 768 consecutive entries                     */
 } asamd_csr_stats;
 
 typedef struct asamd_csr_plan asamd_csr_plan;

@@ -452,11 +452,14 @@ def test_copy_is_not_used_for_another_value_array(gpu, algo):
         d_new.free()
 
 
-def test_analysis_choices(gpu):
+@pytest.mark.parametrize("tune", ["model", "timed"])
+def test_analysis_choices(gpu, tune, monkeypatch):
     """What the analysis decides and what it skips: a banded matrix runs the staged row-block kernel on the
-    caller's arrays, or the ELL copy if that measured at least 5 % faster (the two are within a few per cent
-    of each other), and never lays out the tiled copy (its floor is slower than either); a matrix small
-    enough to be launch-bound takes the single-kernel path however skewed its rows are."""
+    caller's arrays, or the ELL copy if that is at least 5 % faster by the analysis' model (or, with
+    ALSPARSE_AMD_TUNE=timed, by its timing run: the two are within a few per cent of each other), and never
+    lays out the tiled copy (slower than either); a matrix small enough to be launch-bound takes the
+    single-kernel path however skewed its rows are."""
+    monkeypatch.setenv("ALSPARSE_AMD_TUNE", tune)
     lib = capi.load()
     a, x, y0, alpha, beta, _ = wl.config(2)
     da = DeviceCsr(a)
@@ -470,7 +473,9 @@ def test_analysis_choices(gpu):
         st = lib.asamd_analysis_stats(info).contents
         assert st.algo in (capi.ASAMD_SPMV_ELL, capi.ASAMD_SPMV_STREAM), capi.ALGO_NAMES[st.algo]
         assert st.ell_built == (1 if st.algo == capi.ASAMD_SPMV_ELL else 0) and st.tiled_built == 0
-        assert st.tune_ms_ell > 0 and st.tune_ms_base > 0 and st.tune_ms_tiled == 0
+        assert st.tune_ms_ell > 0 and st.tune_ms_base > 0
+        # timed: the tiled copy was not even tried; model: its estimate is there, and slower
+        assert st.tune_ms_tiled == 0 if tune == "timed" else st.tune_ms_tiled > st.tune_ms_base
         assert (st.algo == capi.ASAMD_SPMV_ELL) == (st.tune_ms_ell < 0.95 * st.tune_ms_base)
         check_spmv(a, alpha, x, beta, y0, run_csrmv(gpu, da, alpha, x, beta, y0, info), "config 2 analysed")
     finally:
