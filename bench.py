@@ -692,7 +692,7 @@ def against_ceiling(cfg, r, ceilings):
         return {"ceiling": "plain copy of 2 GiB (probe kernel); achieved = measured HBM traffic of the kernel pair / time",
                 "ceiling_value": c["tb_per_s"], "achieved": got, "unit": "TB/s of real traffic",
                 "frac_of_ceiling": got / c["tb_per_s"]}
-    if kernel.startswith("row-block stream") or kernel.startswith("ell"):
+    if cfg == 2 and (kernel.startswith("row-block stream") or kernel.startswith("ell")):
         c = ceilings["read_2GiB_nontemporal"]
         got = r["algorithmic_bytes"] / ms / 1e9
         return {"ceiling": "non-temporal read of 2 GiB (probe kernel)", "ceiling_value": c["tb_per_s"], "achieved": got,
