@@ -321,7 +321,7 @@ struct alignas(16) Double2 { double x, y; };
 // ---- four values at a time --------------------------------------------------
 // Which of a kernel's two matrix streams is loaded non-temporally (a kernel argument, the same for all lanes).
 // The 256 MB memory-side cache keeps what is loaded plainly from one multiply to the next: the host marks as
-// non-temporal what would push the rest out of it (stream_policy in csr_plan.hip).
+// non-temporal what would push the rest out of it (stream_policy in the plan).
 constexpr int kStreamNtValues = 1;
 constexpr int kStreamNtIndices = 2;
 

@@ -256,3 +256,75 @@ def test_kernel_abi_with_and_without_workspace(gpu, dtype):
         ws.free()
         dB.free()
         da.free()
+
+
+def _band(rows, cols, width, dtype, base=0, seed=11):
+    """Row r holds `width` consecutive columns starting near r * cols / rows: neighbouring rows share nearly all
+    their columns."""
+    rng = np.random.default_rng(seed)
+    start = np.minimum((np.arange(rows, dtype=np.int64) * cols) // rows, cols - width)
+    row_ptr = (np.arange(rows + 1, dtype=np.int64) * width + base).astype(np.int32)
+    col = (start[:, None] + np.arange(width)[None, :] + base).astype(np.int32).reshape(-1)
+    val = rng.uniform(-1, 1, size=rows * width).astype(dtype)
+    return wl.Csr(rows, cols, row_ptr, col, val, base, "band(%d,%d,%d)" % (rows, cols, width))
+
+
+SHARED = {
+    # 27-point stencil: nine runs of three consecutive columns per row; 32 rows share their rows of B
+    "stencil27": lambda dt, base: wl.stencil3d(20, 18, 16, dt, base=base),
+    "laplace": lambda dt, base: wl.laplace2d(90, 70, dt, base=base),
+    # 32 rows x 100 entries exceed the staged entries: the run is halved, then fits
+    "band100": lambda dt, base: _band(3000, 2600, 100, dt, base),
+    # rows whose own columns exceed the tile: halved down to one row, which one wave multiplies from global memory
+    "band300": lambda dt, base: _band(700, 900, 300, dt, base),
+    # a matrix with fewer rows than one workgroup takes, and one that ends inside a run
+    "band_short": lambda dt, base: _band(19, 40, 7, dt, base),
+    "band_tail": lambda dt, base: _band(32 * 5 + 3, 400, 9, dt, base),
+}
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.complex64, np.complex128], ids=["f32", "f64", "c64", "c128"])
+@pytest.mark.parametrize("mat", sorted(SHARED))
+@pytest.mark.parametrize("n", [33, 64, 100, 128])
+@pytest.mark.parametrize("kernel", ["chosen", "lds"])
+def test_row_major_rows_that_share_columns(gpu, mat, n, dtype, kernel, monkeypatch):
+    """Matrices whose neighbouring rows share columns.  "chosen": the kernel the library picks by itself (a
+    device-side look at the structure where the size of B does not decide); "lds": the opt-in kernel that stages
+    the distinct rows of B of a run of rows of A in LDS.  Aligned and padded leading dimensions (128-bit and
+    element-wise loads), both bases, beta zero and not."""
+    from helpers_shapes import complex_vector, complexify, real_dtype
+    if kernel == "lds":
+        monkeypatch.setenv("ALSPARSE_AMD_SPMM_LDS", "1")  # read by the library at every call
+    else:
+        monkeypatch.delenv("ALSPARSE_AMD_SPMM_LDS", raising=False)
+    cx = np.iscomplexobj(np.zeros(1, dtype))
+    tol = {4: 1e-4, 8: 1e-12}[np.dtype(real_dtype(dtype) if cx else dtype).itemsize]
+    for base in (0, 1):
+        a = SHARED[mat](real_dtype(dtype) if cx else dtype, base)
+        if cx:
+            a = complexify(a, dtype)
+        da = DeviceCsr(a)
+        try:
+            for pad_b, pad_c in ((0, 0), (3, 5)):
+                ldb, ldc = n + pad_b, n + pad_c
+                if cx:
+                    Bfull = complex_vector(a.cols * ldb, dtype, 5).reshape(a.cols, ldb)
+                    Cfull = complex_vector(a.rows * ldc, dtype, 4).reshape(a.rows, ldc)
+                else:
+                    Bfull = wl.uniform(a.cols * ldb, dtype, 5).reshape(a.cols, ldb)
+                    Cfull = wl.uniform(a.rows * ldc, dtype, 4).reshape(a.rows, ldc)
+                for alpha, beta in ((1.5, 0.5), (1.0, 0.0)):
+                    announce("spmm rows sharing columns", mat, n, np.dtype(dtype).name, base, ldb, ldc, alpha, beta)
+                    out = run_csrmm(gpu, da, capi.ALPHA_SPARSE_LAYOUT_ROW_MAJOR, 0, alpha, Bfull, ldb, beta, Cfull, ldc, n, a.cols)
+                    B2, C02, C2 = (np.ascontiguousarray(v) for v in (Bfull[:, :n], Cfull[:, :n], out[:, :n]))
+                    ref = orc.csrmm_plain(a, alpha, B2, beta, C02)
+                    err = orc.csrmm_err(a, alpha, B2, beta, C02, C2, ref)
+                    assert err.zero_den_mismatch == 0 and err.full <= tol, "%s n=%d: %r" % (mat, n, err)
+                    if beta == 0:
+                        assert err.strict <= tol, "%s n=%d: %r" % (mat, n, err)
+                    assert np.array_equal(out[:, n:], Cfull[:, n:]), "padding columns of C were touched"
+                    # the same bits on a second run: sums are formed in CSR order whatever slot a column got
+                    again = run_csrmm(gpu, da, capi.ALPHA_SPARSE_LAYOUT_ROW_MAJOR, 0, alpha, Bfull, ldb, beta, Cfull, ldc, n, a.cols)
+                    assert np.array_equal(out.view(np.uint8), again.view(np.uint8))
+        finally:
+            da.free()
