@@ -301,15 +301,16 @@ __device__ __forceinline__ BufferRsrc make_rsrc(const void* p, int bytes) {
 __device__ __forceinline__ int buffer_load_u16(BufferRsrc r, int byte_offset) {
   return (int)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(r, byte_offset, 0, 0);
 }
-template <typename T>
+// AUX: the instruction's cache policy bits (0: default, 2: non-temporal)
+template <typename T, int AUX = 0>
 __device__ __forceinline__ T buffer_load(BufferRsrc r, int byte_offset) {
   if constexpr (sizeof(T) == 4) {
-    return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b32(r, byte_offset, 0, 0));
+    return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b32(r, byte_offset, 0, AUX));
   } else if constexpr (sizeof(T) == 8) {
-    return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b64(r, byte_offset, 0, 0));
+    return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b64(r, byte_offset, 0, AUX));
   } else {
     static_assert(sizeof(T) == 16, "element size");
-    return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b128(r, byte_offset, 0, 0));
+    return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b128(r, byte_offset, 0, AUX));
   }
 }
 

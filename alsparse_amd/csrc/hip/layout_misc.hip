@@ -69,7 +69,7 @@ static hipError_t build_hot(hipStream_t stream, asamd_hot_layout* L, int m, int 
     L->cols_front = hc;
     L->share_lds = (float)(in_lds / (double)nnz);
     // worth laying out only if the LDS serves a good part of the gathers
-    if (!force && L->share_lds < 0.2f) e = hipErrorNotSupported;
+    if (!force && L->share_lds < 0.3f) e = hipErrorNotSupported;
   }
   if (e == hipSuccess) e = hipMalloc(&d_rank, (size_t)n * sizeof(unsigned));
   if (e == hipSuccess) e = hipMalloc(&L->pcol, nnz * sizeof(unsigned));

@@ -82,18 +82,49 @@ __device__ __forceinline__ HotCoords hot_coords(int b, bool exists, int m, int n
   if (c.nnz_cnt == 0) c.nnz_b = 0;
   return c;
 }
-// The block's share of the value and position streams: every load is issued unconditionally (a lane past
-// the end of the range re-reads the range's first entry, a block that does not exist entry 0): the compiler
-// can only count outstanding loads that are certain to be issued.
+// Which of the block's entries a lane holds in slot s of its registers.  Four-byte values: four consecutive
+// entries per 128-bit load (slots 4q .. 4q+3 = entries 256q + 4 lane ..); else one entry per load, a wave's
+// lanes side by side.
+template <typename T, int IPT>
+struct HotSlots {
+  static constexpr bool wide = sizeof(T) == 4 && IPT % 4 == 0;
+  static __device__ __forceinline__ int entry(int lane, int s) {
+    return wide ? (s / 4) * (4 * kWave) + lane * 4 + s % 4 : lane + s * kWave;
+  }
+};
+// The block's share of the value and position streams: every load is issued unconditionally: the compiler
+// can only count outstanding loads that are certain to be issued.  Wide: through buffer resources that end
+// with the block's entries, so the words past the end read as zero and ask memory for nothing (position 0 is
+// a hot column: harmless); narrow: a lane past the end re-reads the range's first entry, a block that does
+// not exist entry 0.
 template <typename T, int IPT>
 __device__ __forceinline__ void hot_load_streams(const HotCoords& c, int lane, const T* __restrict__ val,
                                                  const unsigned* __restrict__ pcol, T (&v)[IPT], unsigned (&p)[IPT]) {
+  if constexpr (HotSlots<T, IPT>::wide) {
+    const BufferRsrc rv = make_rsrc(val + c.nnz_b, c.nnz_cnt * (int)sizeof(T));
+    const BufferRsrc rp = make_rsrc(pcol + c.nnz_b, c.nnz_cnt * (int)sizeof(unsigned));
 #pragma unroll
-  for (int s = 0; s < IPT; ++s) {
-    const int k = lane + s * kWave;
-    const int64_t kk = c.nnz_b + (k < c.nnz_cnt ? k : 0);
-    v[s] = nt_load(val + kk);
-    p[s] = nt_load(pcol + kk);
+    for (int q = 0; q < IPT / 4; ++q) {
+      const int off = (q * 4 * kWave + lane * 4) * 4;
+      const Float4 v4 = buffer_load<Float4, 2>(rv, off);
+      const Int4 p4 = buffer_load<Int4, 2>(rp, off);
+      v[4 * q + 0] = __builtin_bit_cast(T, v4.x);
+      v[4 * q + 1] = __builtin_bit_cast(T, v4.y);
+      v[4 * q + 2] = __builtin_bit_cast(T, v4.z);
+      v[4 * q + 3] = __builtin_bit_cast(T, v4.w);
+      p[4 * q + 0] = (unsigned)p4.x;
+      p[4 * q + 1] = (unsigned)p4.y;
+      p[4 * q + 2] = (unsigned)p4.z;
+      p[4 * q + 3] = (unsigned)p4.w;
+    }
+  } else {
+#pragma unroll
+    for (int s = 0; s < IPT; ++s) {
+      const int k = lane + s * kWave;
+      const int64_t kk = c.nnz_b + (k < c.nnz_cnt ? k : 0);
+      v[s] = nt_load(val + kk);
+      p[s] = nt_load(pcol + kk);
+    }
   }
 }
 
@@ -139,7 +170,7 @@ __device__ __forceinline__ void hot_wave_block(HotWaveSmem<T, IPT>& sm, const in
 #pragma unroll
     for (int s = 0; s < IPT; ++s) {
       const T pr = v[s] * (p[s] < h1 ? l[s] : g[s]);
-      if (lane + s * kWave < nnz_cnt) acc += pr;
+      if (HotSlots<T, IPT>::entry(lane, s) < nnz_cnt) acc += pr;
     }
     acc = group_sum<kWave>(acc);
     if (lane == kWave - 1) {
@@ -159,7 +190,7 @@ __device__ __forceinline__ void hot_wave_block(HotWaveSmem<T, IPT>& sm, const in
   }
 #pragma unroll
   for (int s = 0; s < IPT; ++s) {
-    const int k = lane + s * kWave;
+    const int k = HotSlots<T, IPT>::entry(lane, s);
     if (k < nnz_cnt) sm.prod[lds_pad(k)] = v[s] * (p[s] < h1 ? l[s] : g[s]);
   }
   wave_lds_fence();

@@ -169,12 +169,10 @@ static int hot_eligible(const asamd_csr_plan *p, int force) {
   if (((int64_t)st->n + ((int64_t)1 << 20)) >= (int64_t)UINT32_MAX) return 0;
   if ((int64_t)st->m + st->nnz >= (int64_t)INT32_MAX / 2) return 0;
   if (force) return 1;
-  /* Not tried unless asked for (ALSPARSE_AMD_TUNE_HOT=1): counting and ranking the columns costs several
-   * multiplies, and on the power-law matrices it is meant for the kernel gained 4 % where a copy has to
-   * gain 5 % to be kept. */
-  const char *pick = getenv("ALSPARSE_AMD_TUNE_PICK");
-  const int asked = env_int("ALSPARSE_AMD_TUNE_HOT", 0) > 0 || (pick && !strcmp(pick, "hot"));
-  return asked && (int64_t)st->n * (int64_t)p->val_size >= ((int64_t)8 << 20) && st->nnz >= (1 << 22);
+  /* An x that the L2 of one XCD holds is gathered fast enough as it is, and counting and ranking the columns
+   * costs some forty multiplies: large matrices only.  ALSPARSE_AMD_TUNE_HOT=0 leaves the copy out. */
+  if (env_int("ALSPARSE_AMD_TUNE_HOT", 1) <= 0) return 0;
+  return (int64_t)st->n * (int64_t)p->val_size >= ((int64_t)8 << 20) && st->nnz >= (1 << 22);
 }
 
 static int binned_eligible(const asamd_csr_plan *p, int force) {
@@ -891,6 +889,17 @@ static hipError_t model_copies(hipStream_t stream, asamd_csr_plan *p, const int3
     for (int b = 1; b < 8; ++b) short_entries += (double)st->hist[b] * (double)(((int64_t)1 << b) - 1);
     want_binned = short_entries <= 0.1 * (double)st->nnz;
   }
+  /* Popular columns in LDS: where merge-path runs, the gathers weigh as much as the streams and reach beyond
+   * what the L2s hold, and (the count decides, below) the columns that fit the table hold three entries in ten.
+   * Power-law rows x R-MAT columns, fp32, 2.1 / 4.2 / 8.4 M rows (s = 0.30 / 0.38 / 0.45): 0.122 ms against
+   * 0.117 ms for merge-path, 0.247 against 0.254, 0.526 against 0.580 (37.6 % of the entries from LDS). */
+  int want_hot = 0;
+  if (hot_ok && p->auto_algo == ASAMD_SPMV_MERGE) {
+    const double vs = (double)p->val_size, nnz = (double)st->nnz;
+    const double stream_ms = (nnz * (4.0 + vs) + ((double)st->m + 1.0) * 4.0 + ((double)st->n + (double)st->m) * vs) / 2.9e9;
+    const double gather_ms = nnz * (double)st->lines_per_entry_wave * gather_ps((double)st->lines_per_entry_segment) * 1e-9;
+    want_hot = gather_ms >= 0.5 * stream_ms && st->lines_per_entry_segment >= 0.42f;
+  }
   const char *ev = getenv("ALSPARSE_AMD_TUNE_PICK");
   int forced = -1;
   if (ev) {
@@ -898,13 +907,14 @@ static hipError_t model_copies(hipStream_t stream, asamd_csr_plan *p, const int3
     for (int c = 0; c < CAND_COUNT; ++c)
       if (!strcmp(ev, names[c])) forced = c;
   }
-  int order[3] = {CAND_BASE, CAND_BASE, CAND_BASE};
+  int order[4] = {CAND_BASE, CAND_BASE, CAND_BASE, CAND_BASE};
   const int tiled_wins = tiled_ok && est_tiled < 0.9 * base, ell_wins = ell_ok && est_ell < 0.95 * base;
   int k = 0;
   if (forced > 0) {
     order[k++] = forced;
   } else if (forced < 0) {
     if (want_binned) order[k++] = CAND_BINNED;
+    if (want_hot && !tiled_wins && !ell_wins) order[k++] = CAND_HOT;
     if (tiled_wins && ell_wins) {
       order[k++] = est_tiled < est_ell ? CAND_TILED : CAND_ELL;
       order[k++] = est_tiled < est_ell ? CAND_ELL : CAND_TILED;
@@ -929,7 +939,7 @@ static hipError_t model_copies(hipStream_t stream, asamd_csr_plan *p, const int3
         algo = ASAMD_SPMV_ELL;
         break;
       case CAND_HOT:
-        if (hot_ok) e = build_hot(stream, p, row_ptr, col_ind, 1);
+        if (hot_ok) e = build_hot(stream, p, row_ptr, col_ind, forced == CAND_HOT);
         built = st->hot_built;
         algo = ASAMD_SPMV_MERGE_HOT;
         break;

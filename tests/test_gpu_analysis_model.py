@@ -18,8 +18,10 @@ SHAPES = {
     "laplace_c2": (lambda: wl.laplace2d(2048, 2048, np.float64), capi.ASAMD_SPMV_STREAM),
     # configuration 3's kind at an eighth of its size: scattered columns over 8 MiB of x -> the tiled copy
     "uniform_2M_16": (lambda: wl.uniform_rows(1 << 21, 1 << 21, 16, np.float32), capi.ASAMD_SPMV_TILED),
-    # configuration 4's kind: power-law rows, R-MAT columns -> merge-path
+    # configuration 4's kind at half its size: power-law rows, R-MAT columns, 16 MiB of x -> merge-path
     "powerlaw_4M": (lambda: wl.powerlaw_rmat(22, 200000, np.float32), capi.ASAMD_SPMV_MERGE),
+    # configuration 4 itself (32 MiB of x) -> merge-path with the popular columns' x in LDS
+    "powerlaw_8M": (lambda: wl.powerlaw_rmat(23, 200000, np.float32), capi.ASAMD_SPMV_MERGE_HOT),
     # 27-point stencil, fp64: rows of 8..27 entries -> the ELL copy
     "stencil27_128": (lambda: wl.stencil3d(128, 128, 128, np.float64), capi.ASAMD_SPMV_ELL),
 }
