@@ -35,6 +35,7 @@ MEASURED_TRAFFIC_BYTES = {
     (3, "tiled two-phase"): (5.17e9, "profiles/spmv_tiled_C3.txt"),
     (3, "rowconst"): (34.6e9, "profiles/spmv_tiled_C3.txt"),
     (4, "merge-path"): (3.19e9, "profiles/spmv_merge_C4.txt"),
+    (4, "merge-path, hot columns in LDS"): (2.85e9, "profiles/spmv_merge_hot_C4.txt"),
     (2, "ell copy"): (356.6e6, "profiles/spmv_ell_copy_C2.txt"),
     (2, "row-block stream"): (338.8e6, "profiles/spmv_stream_C2.txt"),
     (5, "spmm row-major"): (9.27e9, "profiles/spmm_rowmajor_C5.txt"),
