@@ -118,7 +118,7 @@ extern "C" int asamd_csr_structure_hash(hipStream_t stream, int32_t m, int32_t n
 }
 
 // ---------------------------------------------------------------------------
-// Value guard.  The array is taken as 4-byte words in runs of run_words words (a multiple of 64); of
+// Value guard.  The array is taken as 4-byte words in runs of run_words words (64 times a power of two); of
 // every run one wave reads 64 consecutive words (256 bytes) at a position that varies from run to run
 // (a fixed stride would sample the same memory channels and the same residues over and over), each
 // word is mixed with its position, and the sums of all lanes add up to the fingerprint -- integer
@@ -136,13 +136,16 @@ struct GuardWs {
 };
 static_assert(offsetof(GuardWs, flag) == 8 * kGuardBlocks + 8, "ASAMD_GUARD_FLAG points at the flag");
 
+// Three 32-bit multiplications per word (they run at a quarter of the rate of an addition, and hashing a
+// whole array must stay a memory-bound pass).  For a fixed position the low half is a bijection of the word, so
+// one changed word always changes the sum; the position enters both halves, so words that change places do too.
 __device__ __forceinline__ unsigned long long mix_word(unsigned w, unsigned long long idx) {
-  const unsigned i = (unsigned)idx ^ ((unsigned)(idx >> 32) * 0x9E3779B1u);
-  unsigned a = ((w + 0x7F4A7C15u) * 0x9E3779B1u) ^ (i * 0x85EBCA6Bu);
-  a = (a ^ (a >> 15)) * 0xC2B2AE35u;
-  a ^= a >> 13;
-  unsigned b = ((w ^ 0xD6E8FEB8u) * 0x27D4EB2Fu) + ((i ^ (i >> 17)) * 0x165667B1u);
-  b = (b ^ (b >> 16)) * 0x94D049BBu;
+  const unsigned i = (unsigned)idx ^ ((unsigned)(idx >> 32) * 0x9E3779B1u);  // (the high part is wave-uniform)
+  const unsigned t = i * 0x85EBCA6Bu;
+  unsigned a = (w ^ t) * 0x9E3779B1u;
+  a ^= a >> 15;
+  unsigned b = (w + ((t >> 7) | (t << 25))) * 0x27D4EB2Fu;
+  b ^= b >> 16;
   return ((unsigned long long)b << 32) | a;
 }
 
@@ -150,9 +153,10 @@ __global__ __launch_bounds__(256) void value_hash_kernel(const unsigned* __restr
                                                          int64_t run_words, unsigned long long* __restrict__ partial) {
   const int lane = threadIdx.x % kWave;
   const int64_t waves = (int64_t)gridDim.x * (256 / kWave);
-  const int64_t wave = (int64_t)blockIdx.x * (256 / kWave) + threadIdx.x / kWave;
+  // (wave-uniform values are made so for the compiler: the position arithmetic then runs on the scalar unit)
+  const int64_t wave = (int64_t)blockIdx.x * (256 / kWave) + __builtin_amdgcn_readfirstlane((int)threadIdx.x / kWave);
   const int64_t runs = (total_words + run_words - 1) / run_words;
-  const unsigned slots = (unsigned)(run_words / kWave);  // positions a sample can take inside its run
+  const unsigned slot_mask = (unsigned)(run_words / kWave) - 1u;  // positions inside a run: a power of two
   unsigned long long mine = 0;
   for (int64_t r0 = wave; r0 < runs; r0 += waves * kGuardUnroll) {
     unsigned w[kGuardUnroll];
@@ -161,7 +165,7 @@ __global__ __launch_bounds__(256) void value_hash_kernel(const unsigned* __restr
     for (int u = 0; u < kGuardUnroll; ++u) {
       const int64_t r = r0 + (int64_t)u * waves;
       const int64_t start = r * run_words;
-      int64_t pos = start + (int64_t)((((unsigned)r * 2654435761u) >> 7) % slots) * kWave;
+      int64_t pos = start + (int64_t)((((unsigned)r * 2654435761u) >> 7) & slot_mask) * kWave;
       if (pos >= total_words) pos = start;  // the last, short run
       idx[u] = r < runs && pos + lane < total_words ? pos + lane : -1;
       w[u] = idx[u] >= 0 ? nt_load(words + idx[u]) : 0u;
