@@ -55,8 +55,11 @@ static hipError_t build_hot(hipStream_t stream, asamd_hot_layout* L, int m, int 
   if (e == hipSuccess) e = hipMalloc(&d_sorted, (size_t)n * sizeof(unsigned));
   if (e == hipSuccess) e = hipMemsetAsync(d_cnt, 0, (size_t)n * sizeof(unsigned), stream);
   std::vector<unsigned> h_key((size_t)h1);
+  // large matrices are counted through one chunk of entries in four (the ranking of the popular columns and the
+  // share below are then estimates, good to a per cent or so)
+  const int sample_shift = nnz_i >= (1 << 24) ? 2 : 0;
   if (e == hipSuccess) {
-    col_count_kernel<<<256 * 32, 256, 0, stream>>>(nnz_i, col_ind, base, d_cnt);
+    col_count_kernel<<<256 * 32, 256, 0, stream>>>(nnz_i, col_ind, base, sample_shift, d_cnt);
     col_rank_keys_kernel<<<(unsigned)(((int64_t)n + 255) / 256), 256, 0, stream>>>(n, d_cnt, d_key, d_idx);
     e = hipGetLastError();
   }
@@ -64,7 +67,7 @@ static hipError_t build_hot(hipStream_t stream, asamd_hot_layout* L, int m, int 
   if (e == hipSuccess) e = hipMemcpy(h_key.data(), d_key2, (size_t)h1 * sizeof(unsigned), hipMemcpyDeviceToHost);
   if (e == hipSuccess) {
     double in_lds = 0.0;
-    for (int i = 0; i < h1; ++i) in_lds += (double)(~h_key[(size_t)i]);
+    for (int i = 0; i < h1; ++i) in_lds += (double)(~h_key[(size_t)i]) * (double)(1 << sample_shift);
     L->cols_lds = h1;
     L->cols_front = hc;
     L->share_lds = (float)(in_lds / (double)nnz);
