@@ -170,7 +170,7 @@ static int hot_eligible(const asamd_csr_plan *p, int force) {
   if ((int64_t)st->m + st->nnz >= (int64_t)INT32_MAX / 2) return 0;
   if (force) return 1;
   /* An x that the L2 of one XCD holds is gathered fast enough as it is, and counting and ranking the columns
-   * costs some forty multiplies: large matrices only.  ALSPARSE_AMD_TUNE_HOT=0 leaves the copy out. */
+   * costs some twenty-five multiplies: large matrices only.  ALSPARSE_AMD_TUNE_HOT=0 leaves the copy out. */
   if (env_int("ALSPARSE_AMD_TUNE_HOT", 1) <= 0) return 0;
   return (int64_t)st->n * (int64_t)p->val_size >= ((int64_t)8 << 20) && st->nnz >= (1 << 22);
 }
