@@ -214,6 +214,55 @@ __device__ __forceinline__ T bperm(int byte_addr, T v) {
   }
 }
 
+// One wave's 64 entries of a row: what the entry loop hands round.  The position of an entry's row of B is kept
+// as a byte offset (NARROW: one word, with kNoRow for lanes past the row's end; else two words).
+template <typename T>
+struct QuadChunk {
+  T val;
+  unsigned off;
+  int off_hi;
+};
+constexpr unsigned kNoRow = 0x80000000u;  // an offset the buffer's range check turns away (B spans less than 2 GiB)
+
+// Requests the (up to 64) entries of [j0, end) -- nothing is waited for here.
+template <typename T, bool NARROW>
+__device__ __forceinline__ QuadChunk<T> quad_load_chunk(int64_t j0, int64_t end, int lane, T alpha,
+                                                        const T* __restrict__ val, const int* __restrict__ col_ind,
+                                                        int base, int64_t row_bytes) {
+  QuadChunk<T> c;
+  c.val = T(0);
+  c.off = NARROW ? kNoRow : 0u;
+  c.off_hi = 0;
+  if (j0 < end) {  // wave-uniform
+    const bool live = j0 + lane < end;
+    const int64_t j = live ? j0 + lane : j0;
+    // A and C are touched once: non-temporal, so that they do not push rows of B out of the caches
+    const int col = nt_load(col_ind + j) - base;
+    const T loaded = alpha * nt_load(val + j);
+    const int64_t off64 = (int64_t)col * row_bytes;
+    if constexpr (NARROW) {
+      // lanes past the end hold (0, no row): a group that reads them adds 0 * 0, so nothing in the entry loop
+      // depends on the row's length
+      c.val = live ? loaded : T(0);
+      c.off = live ? (unsigned)off64 : kNoRow;
+    } else {
+      c.val = loaded;  // (lanes past the end repeat the chunk's first entry, and are never summed)
+      c.off = (unsigned)off64;
+      c.off_hi = (int)(off64 >> 32);
+    }
+  }
+  return c;
+}
+
+// PERSISTENT waves, each walking the rows w, w + W, w + 2W, ... (W = waves of the grid) with the loads of three rows
+// in flight: the row offsets of the row after next, the entries of the next row, the rows of B of the current
+// one -- a wave that handles one row and exits waits for those three in turn.
+// What the kernel's time is (27-point stencil 128 x 128 x 64, n = 64, 0.51 ms): every row of A brings one row of B
+// that no cache holds yet (B has as many rows as A), so every row waits for memory at least once; a wave spends
+// 3 us per row all told, and a compute unit has as many rows in flight as it has waves -- 24 here, each holding
+// its row's 8 KB of B in registers.  Taking a third of the loads of B away, or a third of the ds_bpermutes, changed nothing; nor did row
+// offsets through vector loads, or one combined wait per row with the store of C delayed into the next row's
+// (0.52 / 0.57 ms); 7 or 8 waves per SIMD were had only with spills (0.76 ms).
 template <typename T, bool NARROW>
 __global__ __launch_bounds__(kSpmmBlock) void spmm_rowmajor_quad_kernel(
     int m, int n, T alpha, const T* __restrict__ val, const int* __restrict__ row_ptr,
@@ -223,10 +272,10 @@ __global__ __launch_bounds__(kSpmmBlock) void spmm_rowmajor_quad_kernel(
   constexpr int E = 16 / (int)sizeof(T);
   constexpr int kU = 8;  // loads in flight per lane
   const int lane = threadIdx.x % kWave;
-  const int wave = threadIdx.x / kWave;
-  const unsigned bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
-  const int64_t row = (int64_t)bid * kSpmmWaves + wave;
-  if (row >= m) return;  // wave-uniform
+  const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x / kWave);
+  const int64_t stride = (int64_t)gridDim.x * kSpmmWaves;  // rows between a wave's consecutive rows
+  int64_t row = (int64_t)blockIdx.x * kSpmmWaves + wave;   // wave-uniform
+  if (row >= m) return;
   const int g = lane / 16;
   const int c0 = (blockIdx.y * 16 + lane % 16) * E;
   const bool owns = c0 < n;
@@ -235,98 +284,108 @@ __global__ __launch_bounds__(kSpmmBlock) void spmm_rowmajor_quad_kernel(
   const int my_c = owns ? c0 : blockIdx.y * 16 * E;
   const BufferRsrc brsrc = make_rsrc(B, (int)b_bytes);
   const int64_t row_bytes = ldb * (int64_t)sizeof(T);
-
-  const int64_t start = (int64_t)row_ptr[row] - base;
-  const int64_t end = (int64_t)row_ptr[row + 1] - base;
-  T acc[E];
-#pragma unroll
-  for (int i = 0; i < E; ++i) acc[i] = T(0);
-
-  // ds_bpermute addresses of the lanes that hold this group's entries 4u + g: constants of the kernel
-  int from[kU];
-#pragma unroll
-  for (int u = 0; u < kU; ++u) from[u] = (4 * u + g) * 4;
+  // ds_bpermute address of the lane that holds this group's entry g (entry 4u + g: 16 u further); kept as ONE
+  // register and added to where it is used: registers decide how many waves, hence rows, a compute unit has in
+  // flight, and that is what this kernel's speed hangs on
+  const int from0 = g * 4;
   const unsigned my_c_bytes = (unsigned)my_c * (unsigned)sizeof(T);
-  // NARROW: an offset that the buffer's range check turns away (B spans less than 2 GiB): the load returns
-  // zero and asks memory for nothing
-  constexpr unsigned kNoRow = 0x80000000u;
 
-  for (int64_t j0 = start; j0 < end; j0 += kWave) {
-    const bool live = j0 + lane < end;
-    const int64_t j = live ? j0 + lane : j0;
-    // A and C are touched once: non-temporal, so that they do not push rows of B out of the caches
-    const int my_col = nt_load(col_ind + j) - base;
-    const T loaded = alpha * nt_load(val + j);
-    const int64_t my_off64 = (int64_t)my_col * row_bytes;
-    const int cnt = (int)(end - j0 < kWave ? end - j0 : kWave);
-    if constexpr (NARROW) {
-      // lanes past the end hold (0, no row): a group that reads them adds 0 * 0, so nothing in the entry loop
-      // depends on the row's length
-      const T my_val = live ? loaded : T(0);
-      const unsigned my_off = live ? (unsigned)my_off64 : kNoRow;
+  // prologue: this row's offsets and entries, the next row's offsets
+  int64_t start = (int64_t)row_ptr[row] - base, end = (int64_t)row_ptr[row + 1] - base;
+  QuadChunk<T> cur = quad_load_chunk<T, NARROW>(start, end, lane, alpha, val, col_ind, base, row_bytes);
+  int64_t next = row + stride;
+  int64_t n_start = 0, n_end = 0;
+  if (next < m) {
+    n_start = (int64_t)row_ptr[next] - base;
+    n_end = (int64_t)row_ptr[next + 1] - base;
+  }
+  while (true) {
+    // ---- requests for the rows to come ------------------------------------------------------------
+    QuadChunk<T> nxt = quad_load_chunk<T, NARROW>(n_start, next < m ? n_end : n_start, lane, alpha, val, col_ind,
+                                                  base, row_bytes);
+    const int64_t after = next + stride;
+    int64_t a_start = 0, a_end = 0;
+    if (after < m) {
+      a_start = (int64_t)row_ptr[after] - base;
+      a_end = (int64_t)row_ptr[after + 1] - base;
+    }
+    // ---- the current row ----------------------------------------------------------------------------
+    T acc[E];
 #pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        if (half * 4 * kU >= cnt) break;
-        Vec<T, E> b[kU];
-        T a[kU];
+    for (int i = 0; i < E; ++i) acc[i] = T(0);
+    for (int64_t j0 = start; j0 < end; j0 += kWave) {
+      // (rows of more than 64 entries fetch their further chunks here, unprepared)
+      const QuadChunk<T> ch = j0 == start ? cur : quad_load_chunk<T, NARROW>(j0, end, lane, alpha, val, col_ind,
+                                                                              base, row_bytes);
+      const int cnt = (int)(end - j0 < kWave ? end - j0 : kWave);
+      if constexpr (NARROW) {
 #pragma unroll
-        for (int u = 0; u < kU; ++u) {
-          a[u] = bperm(from[u] + half * 16 * kU, my_val);
-          const unsigned off = (unsigned)__builtin_amdgcn_ds_bpermute(from[u] + half * 16 * kU, (int)my_off);
-          b[u] = buffer_load<Vec<T, E>>(brsrc, (int)(off + my_c_bytes));
-        }
+        for (int half = 0; half < 2; ++half) {
+          if (half * 4 * kU >= cnt) break;
+          Vec<T, E> b[kU];
+          T a[kU];
 #pragma unroll
-        for (int u = 0; u < kU; ++u) {
+          for (int u = 0; u < kU; ++u) {
+            a[u] = bperm(from0 + 16 * u + half * 16 * kU, ch.val);
+            const unsigned off = (unsigned)__builtin_amdgcn_ds_bpermute(from0 + 16 * u + half * 16 * kU, (int)ch.off);
+            b[u] = buffer_load<Vec<T, E>>(brsrc, (int)(off + my_c_bytes));
+          }
 #pragma unroll
-          for (int i = 0; i < E; ++i) acc[i] = fma_t(a[u], b[u].e[i], acc[i]);
-        }
-      }
-    } else {
-      const T my_val = loaded;  // (lanes past the end repeat the chunk's first entry, and are never summed)
-      const unsigned my_off = (unsigned)my_off64;
-      const int my_off_hi = (int)(my_off64 >> 32);
-      for (int t0 = 0; t0 < cnt; t0 += 4 * kU) {
-        Vec<T, E> b[kU];
-        T a[kU];
-        // every load is issued whatever the group needs: loads under branches would wait for one another
-#pragma unroll
-        for (int u = 0; u < kU; ++u) {
-          const int at = from[u] + t0 * 4;
-          a[u] = bperm(at, my_val);
-          const unsigned lo = (unsigned)__builtin_amdgcn_ds_bpermute(at, (int)my_off);
-          const int hi = __builtin_amdgcn_ds_bpermute(at, my_off_hi);
-          const int64_t off = ((int64_t)hi << 32) | lo;
-          b[u] = *reinterpret_cast<const Vec<T, E>*>(reinterpret_cast<const char*>(B + my_c) + off);
-        }
-#pragma unroll
-        for (int u = 0; u < kU; ++u) {
-          if (t0 + 4 * u + g < cnt) {
+          for (int u = 0; u < kU; ++u) {
 #pragma unroll
             for (int i = 0; i < E; ++i) acc[i] = fma_t(a[u], b[u].e[i], acc[i]);
           }
         }
+      } else {
+        for (int t0 = 0; t0 < cnt; t0 += 4 * kU) {
+          Vec<T, E> b[kU];
+          T a[kU];
+          // every load is issued whatever the group needs: loads under branches would wait for one another
+#pragma unroll
+          for (int u = 0; u < kU; ++u) {
+            const int at = from0 + 16 * u + t0 * 4;
+            a[u] = bperm(at, ch.val);
+            const unsigned lo = (unsigned)__builtin_amdgcn_ds_bpermute(at, (int)ch.off);
+            const int hi = __builtin_amdgcn_ds_bpermute(at, ch.off_hi);
+            const int64_t off = ((int64_t)hi << 32) | lo;
+            b[u] = *reinterpret_cast<const Vec<T, E>*>(reinterpret_cast<const char*>(B + my_c) + off);
+          }
+#pragma unroll
+          for (int u = 0; u < kU; ++u) {
+            if (t0 + 4 * u + g < cnt) {
+#pragma unroll
+              for (int i = 0; i < E; ++i) acc[i] = fma_t(a[u], b[u].e[i], acc[i]);
+            }
+          }
+        }
       }
     }
-  }
-  {
-    const int across16 = (lane ^ 16) * 4, across32 = (lane ^ 32) * 4;
 #pragma unroll
-    for (int i = 0; i < E; ++i) acc[i] += bperm(across16, acc[i]);
+    for (int i = 0; i < E; ++i) acc[i] += bperm((lane ^ 16) * 4, acc[i]);
 #pragma unroll
-    for (int i = 0; i < E; ++i) acc[i] += bperm(across32, acc[i]);
-  }
-  if (g == 0 && owns) {
-    T* crow = C + row * ldc + c0;
-    Vec<T, E> out;
-    if (beta == T(0)) {
+    for (int i = 0; i < E; ++i) acc[i] += bperm((lane ^ 32) * 4, acc[i]);
+    if (g == 0 && owns) {
+      T* crow = C + row * ldc + c0;
+      Vec<T, E> out;
+      if (beta == T(0)) {
 #pragma unroll
-      for (int i = 0; i < E; ++i) out.e[i] = acc[i];
-    } else {
-      const Vec<T, E> old = *reinterpret_cast<const Vec<T, E>*>(crow);
+        for (int i = 0; i < E; ++i) out.e[i] = acc[i];
+      } else {
+        const Vec<T, E> old = *reinterpret_cast<const Vec<T, E>*>(crow);
 #pragma unroll
-      for (int i = 0; i < E; ++i) out.e[i] = old.e[i] * beta + acc[i];
+        for (int i = 0; i < E; ++i) out.e[i] = old.e[i] * beta + acc[i];
+      }
+      *reinterpret_cast<Vec<T, E>*>(crow) = out;
     }
-    *reinterpret_cast<Vec<T, E>*>(crow) = out;
+    // ---- on to the next row ---------------------------------------------------------------------------
+    if (next >= m) break;
+    row = next;
+    start = n_start;
+    end = n_end;
+    cur = nxt;
+    next = after;
+    n_start = a_start;
+    n_end = a_end;
   }
 }
 
@@ -1228,7 +1287,24 @@ static int csrmm_impl(hipStream_t s, int m, int n, int k, int nnz, T alpha, cons
       }
     }
     if (quad_can && (quad_by_size || shared == 1 || gate)) {
-      const dim3 grid(gx, (unsigned)((n + 16 * E - 1) / (16 * E)));
+      // persistent waves: as many workgroups as the chip holds at once (fewer for matrices with fewer rows)
+      static const int quad_wgs = [] {
+        int dev = 0, cus = 0, per_cu = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+          cus = 256;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, spmm_rowmajor_quad_kernel<T, true>, kSpmmBlock, 0) !=
+                hipSuccess || per_cu < 1) {
+          (void)hipGetLastError();
+          per_cu = 4;
+        }
+        return cus * per_cu;
+      }();
+      const unsigned gyq = (unsigned)((n + 16 * E - 1) / (16 * E));
+      unsigned gxq = (unsigned)quad_wgs / gyq;
+      if (gxq < 1u) gxq = 1u;
+      if (gxq > gx) gxq = gx;
+      const dim3 grid(gxq, gyq);
       // B within 2 GiB (its row count known): 32-bit offsets into a buffer resource
       const unsigned __int128 span = (unsigned __int128)(k > 0 ? k : 0) * (unsigned __int128)ldb * sizeof(T);
       if (k > 0 && span < ((unsigned __int128)1 << 31))

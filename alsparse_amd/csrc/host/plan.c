@@ -794,8 +794,8 @@ static hipError_t tune_copies(hipStream_t stream, asamd_csr_plan *p, const int32
  *     T ps   3.6   4.7    5.6    5.9    10.5   10.5   13.5    17.8   19      beyond an XCD's L2 wait 3 x longer)
  *     TB/s   constant row length 6.0, staged row block 6.6 (one lane per row) / 5.2 (several), lane group per
  *            row 2.4 x the share of its lanes that hold an entry, merge-path 2.9, ELL copy 6.1 (of its padded
- *            streams); tiled pair: 0.045 ms + 2 x bytes / 5.6 TB/s, x 1 .. 1.5 with the spread of the row lengths,
- *            x 2.5 for heavy-tailed rows.
+ *            streams); tiled pair: 0.045 ms + 2 x bytes / 5.6 TB/s (8-byte values and wider: their 28 / 52 bytes per
+ *            entry at 4.6 TB/s), x 1 .. 1.5 with the spread of the row lengths, x 2.5 for heavy-tailed rows.
  * The estimates are within about 10 % of the timings on the shapes they were read from (5-point and 27-point
  * stencils, uniform rows over 0.25 - 64 MiB of x, two row lengths, power-law rows and columns, fp32 / fp64). */
 static double gather_ps(double s) {
@@ -850,7 +850,10 @@ static double model_ms(const asamd_csr_plan *p, int algo) {
       double skew = 1.0 + 0.5 * ((double)st->max_len / mean - 1.0) / 8.0;
       if (skew > 1.5) skew = 1.5;
       if ((double)st->max_len > 32.0 * mean + 256.0) skew = 2.5; /* heavy tail: long tiles, uneven waves */
-      return (0.045 + 2.0 * bytes / 5.6e9) * skew;
+      /* 4-byte values: twice the CSR bytes at 5.6 TB/s; wider ones move 3 values + 4 index bytes per entry
+       * through both phases and their second phase (shorter row blocks) reaches 4.6 TB/s */
+      const double stream = vs >= 8.0 ? (nnz * (3.0 * vs + 4.0) + (n + m) * vs) / 4.6e9 : 2.0 * bytes / 5.6e9;
+      return (0.045 + stream) * skew;
     }
     default: break;
   }

@@ -65,14 +65,17 @@ def test_model_and_timing_choose_the_same_family(gpu, shape):
         assert model[0]["algo"] == want, (shape, capi.ALGO_NAMES[model[0]["algo"]], model[0])
         # (a timing run may also keep the hot-column kernel at half of configuration 4's size, where it is 3 %
         # ahead of merge-path: the model lays it out only where the gain is beyond doubt)
-        timed_ok = {want, capi.ASAMD_SPMV_MERGE_HOT} if shape == "powerlaw_4M" else {want}
+        # and the staged row-block kernel on the stencil, where the ELL copy wins by 8 % and must win by 5 %)
+        near_ties = {"powerlaw_4M": capi.ASAMD_SPMV_MERGE_HOT, "stencil27_128": capi.ASAMD_SPMV_STREAM}
+        timed_ok = {want, near_ties[shape]} if shape in near_ties else {want}
         assert timed["algo"] in timed_ok, (shape, capi.ALGO_NAMES[timed["algo"]], timed)
         # the model's decision and every number behind it are the same on every analysis
         assert model[0] == model[1] == model[2] == default
         assert 0 < model[0]["lines_per_entry_wave"] <= 1 and 0 < model[0]["lines_per_entry_segment"] <= 1
         # its estimate of the kept family is within a third of what the timing run measured
         key = {capi.ASAMD_SPMV_TILED: "tune_ms_tiled", capi.ASAMD_SPMV_ELL: "tune_ms_ell"}.get(want, "tune_ms_base")
-        assert 0.66 * timed[key] <= model[0][key] <= 1.5 * timed[key], (key, model[0][key], timed[key])
+        if timed[key] > 0:  # (a copy that the timing run did not lay out has no measurement)
+            assert 0.66 * timed[key] <= model[0][key] <= 1.5 * timed[key], (key, model[0][key], timed[key])
     finally:
         da.free()
 
