@@ -314,8 +314,13 @@ _COMMON = {
     "asamd_csr_plan_workspace_bytes": [_P],
     "asamd_csr_plan_csrmv": [_P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, c_size_t],
     "asamd_handle_reserve": [_P, c_size_t],
+    "asamd_csr_plan_watched_workspace_bytes": [_P],
+    "asamd_csr_plan_watch_begin": [_P, _P, _P, _P, _P, _P, c_size_t],
+    "asamd_csr_plan_csrmv_watched": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_size_t, _P],
     # stateless launchers and layout builders (records are passed as opaque pointers here)
     "asamd_spmv_vector": [_P, POINTER(asamd_spmv_args), _I],
+    "asamd_spmv_vector_if": [_P, POINTER(asamd_spmv_args), _I, _P],
+    "asamd_value_guard_any": [_P, _P, _P, _P],
     "asamd_spmv_scalar": [_P, POINTER(asamd_spmv_args)],
     "asamd_spmv_rowconst": [_P, POINTER(asamd_spmv_args), _I],
     "asamd_spmv_stream": [_P, POINTER(asamd_spmv_args), _I, _I, _I],
@@ -325,7 +330,7 @@ _COMMON = {
     "asamd_tiled_fits": [_I, _I, _I, _I],
     "asamd_tiled_build": [_P, _I, _I, _I, _I, _I, _P, _P, _P, _I, _I, _P],
     "asamd_tiled_free": [_P],
-    "asamd_spmv_tiled": [_P, POINTER(asamd_spmv_args), _P, _P, _P],
+    "asamd_spmv_tiled": [_P, POINTER(asamd_spmv_args), _P, _P, _P, _P],
     "asamd_hot_build": [_P, _I, _I, _I, _I, _I, _P, _P, _I, _I, _I, _P],
     "asamd_hot_free": [_P],
     "asamd_spmv_hot": [_P, POINTER(asamd_spmv_args), _P, _P, _P, _P, _P],
@@ -355,6 +360,7 @@ _COMMON = {
     "asamd_handle_set_stream": [_P, _P],
     "asamd_handle_get_stream": [_P],
     "asamd_registry_lazy_count": [],
+    "asamd_registry_lazy_promoted": [_P, _P],
     "asamd_analysis_stats": [_P],
     "asamd_analysis_transpose_stats": [_P],
     "asamd_analysis_set_algo": [_P, _I],
@@ -381,7 +387,7 @@ _RESTYPE = {"alpha_set_thread_num": None, "alpha_timing_wtime": c_double, "alpha
             "args_help": None, "args_get_if_check": c_bool, "args_get_data_file": ctypes.c_char_p,
             "args_get_data_fileA": ctypes.c_char_p, "args_get_data_fileB": ctypes.c_char_p,
             "alpha_args_get_matrix_descrA": alpha_matrix_descr, "alpha_args_get_matrix_descrB": alpha_matrix_descr,
-            "get_time_us": c_double, "asamd_csrmm_workspace_bytes": c_size_t, "asamd_csr2coo_workspace_bytes": c_size_t, "asamd_csr_plan_workspace_bytes": c_size_t, "asamd_value_guard_run": c_size_t, "asamd_tiled_free": None, "asamd_hot_free": None, "asamd_binned_free": None, "asamd_transpose_free": None, "asamd_csr_plan_stats": POINTER(asamd_csr_stats),
+            "get_time_us": c_double, "asamd_csrmm_workspace_bytes": c_size_t, "asamd_csr2coo_workspace_bytes": c_size_t, "asamd_csr_plan_workspace_bytes": c_size_t, "asamd_csr_plan_watched_workspace_bytes": c_size_t, "asamd_value_guard_run": c_size_t, "asamd_tiled_free": None, "asamd_hot_free": None, "asamd_binned_free": None, "asamd_transpose_free": None, "asamd_csr_plan_stats": POINTER(asamd_csr_stats),
             "asamd_csr_plan_transpose_stats": POINTER(asamd_csr_stats),
             "asamd_analysis_transpose_stats": POINTER(asamd_csr_stats),
             "asamd_analysis_stats": POINTER(asamd_csr_stats)}

@@ -214,6 +214,16 @@ extern "C" int asamd_value_guard(hipStream_t stream, const void* val, size_t nby
   return hipGetLastError();
 }
 
+__global__ void guard_any_kernel(const GuardWs* __restrict__ a, const GuardWs* __restrict__ b, int* __restrict__ out) {
+  *out = (a->flag | b->flag) ? 1 : 0;
+}
+
+extern "C" int asamd_value_guard_any(hipStream_t stream, const void* ws_a, const void* ws_b, int32_t* out) {
+  if (!ws_a || !ws_b || !out) return hipErrorInvalidValue;
+  guard_any_kernel<<<1, 1, 0, stream>>>((const GuardWs*)ws_a, (const GuardWs*)ws_b, out);
+  return hipGetLastError();
+}
+
 extern "C" int asamd_value_guard_commit(hipStream_t stream, const void* ws, uint64_t* stored) {
   if (!ws || !stored) return hipErrorInvalidValue;
   value_commit_kernel<<<1, 1, 0, stream>>>((const GuardWs*)ws, (unsigned long long*)stored);

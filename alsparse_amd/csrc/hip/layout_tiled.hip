@@ -397,7 +397,7 @@ extern "C" void asamd_tiled_free(asamd_tiled_layout* L) {
 // (the tiles too long for phase 2) and its ordered finish.  The layout holds zero-based local indices and
 // its own values.
 extern "C" int asamd_spmv_tiled(hipStream_t s, const asamd_spmv_args* a, const asamd_tiled_layout* L, void* products,
-                                void* long_scratch) {
+                                void* long_scratch, const int32_t* skip) {
   if (!a || !L || !L->tval || !products || !a->alpha || !a->beta || !a->x || !a->y) return hipErrorInvalidValue;
   if (a->dtype != L->dtype || a->m != L->m || a->n != L->n || a->nnz != L->nnz) return hipErrorInvalidValue;
   if (L->n_long_finish > 0 && !long_scratch) return hipErrorInvalidValue;
@@ -422,25 +422,25 @@ extern "C" int asamd_spmv_tiled(hipStream_t s, const asamd_spmv_args* a, const a
     if (L->entries_per_lane == 1)
       tiled_reduce_kernel<T, 1><<<red_grid, TileDims<T>::red_threads, TileDims<T>::red_lds_bytes, s>>>(
           L->m, L->row_blocks, L->col_blocks, L->row_block_start, (const TileRange*)L->ranges, L->trow, prod, alpha,
-          beta, y);
+          beta, y, skip);
     else
       tiled_reduce_kernel<T, 2><<<red_grid, TileDims<T>::red_threads, TileDims<T>::red_lds_bytes, s>>>(
           L->m, L->row_blocks, L->col_blocks, L->row_block_start, (const TileRange*)L->ranges, L->trow, prod, alpha,
-          beta, y);
+          beta, y, skip);
     if (L->n_long_chunks > 0) {
       const int waves = kLongThreads / kWave, narrow = L->n_long_narrow, wide = L->n_long_chunks - narrow;
       const LongBlock* list = (const LongBlock*)L->long_list;
       const LongTile* tiles = (const LongTile*)L->long_tiles;
       if (narrow > 0)
         tiled_long_kernel<T><<<narrow, kLongThreads, waves * (kLongNarrow + kWave) * (int)sizeof(T), s>>>(
-            list, tiles, L->trow, prod, alpha, y, (T*)long_scratch, kLongNarrow);
+            list, tiles, L->trow, prod, alpha, y, (T*)long_scratch, kLongNarrow, skip);
       if (wide > 0)
         tiled_long_kernel<T><<<wide, kLongThreads, waves * (TileDims<T>::rows + kWave) * (int)sizeof(T), s>>>(
-            list + narrow, tiles, L->trow, prod, alpha, y, (T*)long_scratch, TileDims<T>::rows);
+            list + narrow, tiles, L->trow, prod, alpha, y, (T*)long_scratch, TileDims<T>::rows, skip);
     }
     if (L->n_long_finish > 0)
       tiled_long_finish_kernel<T><<<L->n_long_finish, 256, 0, s>>>((const LongFinish*)L->long_finish,
-                                                                   (const T*)long_scratch, alpha, y);
+                                                                   (const T*)long_scratch, alpha, y, skip);
     return hipGetLastError();
   });
 }

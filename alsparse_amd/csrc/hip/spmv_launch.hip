@@ -25,30 +25,34 @@ static int csr_stream_policy(const asamd_spmv_args* a, size_t val_size, bool wid
 
 // ---- W lanes per row ----------------------------------------------------------------------------
 template <typename T, int W>
-static void launch_vector(hipStream_t s, const asamd_spmv_args* a) {
+static void launch_vector(hipStream_t s, const asamd_spmv_args* a, const int32_t* run_if) {
   constexpr int rows_per_block = kRowsBlock / W;
   const unsigned grid = (unsigned)(((int64_t)a->m + rows_per_block - 1) / rows_per_block);
   spmv_vector_kernel<T, W><<<grid, kRowsBlock, 0, s>>>(a->m, scalar_of<T>(a->alpha), (const T*)a->val, a->row_ptr,
                                                        a->col_ind, (const T*)a->x, scalar_of<T>(a->beta), (T*)a->y,
-                                                       a->base);
+                                                       a->base, run_if);
 }
 
-extern "C" int asamd_spmv_vector(hipStream_t s, const asamd_spmv_args* a, int32_t width) {
+extern "C" int asamd_spmv_vector_if(hipStream_t s, const asamd_spmv_args* a, int32_t width, const int32_t* run_if) {
   if (!a) return hipErrorInvalidValue;
   return by_dtype(a->dtype, [&](auto* tag) -> int {
     using T = std::remove_pointer_t<decltype(tag)>;
     if (!args_ok<T>(a)) return hipErrorInvalidValue;
     switch (width) {
-      case 2: launch_vector<T, 2>(s, a); break;
-      case 4: launch_vector<T, 4>(s, a); break;
-      case 8: launch_vector<T, 8>(s, a); break;
-      case 16: launch_vector<T, 16>(s, a); break;
-      case 32: launch_vector<T, 32>(s, a); break;
-      case 64: launch_vector<T, 64>(s, a); break;
+      case 2: launch_vector<T, 2>(s, a, run_if); break;
+      case 4: launch_vector<T, 4>(s, a, run_if); break;
+      case 8: launch_vector<T, 8>(s, a, run_if); break;
+      case 16: launch_vector<T, 16>(s, a, run_if); break;
+      case 32: launch_vector<T, 32>(s, a, run_if); break;
+      case 64: launch_vector<T, 64>(s, a, run_if); break;
       default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
   });
+}
+
+extern "C" int asamd_spmv_vector(hipStream_t s, const asamd_spmv_args* a, int32_t width) {
+  return asamd_spmv_vector_if(s, a, width, nullptr);
 }
 
 extern "C" int asamd_spmv_scalar(hipStream_t s, const asamd_spmv_args* a) {

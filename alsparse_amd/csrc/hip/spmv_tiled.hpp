@@ -467,7 +467,8 @@ template <typename T, int H>
 __global__ __launch_bounds__(TileDims<T>::red_threads) void tiled_reduce_kernel(
     int m, int row_blocks, int col_blocks, const int* __restrict__ row_block_start,
     const TileRange* __restrict__ ranges, const unsigned short* __restrict__ t_row,
-    const T* __restrict__ prod, T alpha, T beta, T* __restrict__ y) {
+    const T* __restrict__ prod, T alpha, T beta, T* __restrict__ y, const int* __restrict__ skip) {
+  if (skip && *skip) return;  // the caller's guard found that the layout no longer describes the matrix
   extern __shared__ __align__(16) unsigned char smem[];
   T* s_acc = reinterpret_cast<T*>(smem);
   constexpr int kTileRows = TileDims<T>::rows;
@@ -570,7 +571,9 @@ __global__ __launch_bounds__(TileDims<T>::red_threads) void tiled_reduce_kernel(
 template <typename T>
 __global__ __launch_bounds__(kLongThreads) void tiled_long_kernel(
     const LongBlock* __restrict__ blocks, const LongTile* __restrict__ tiles, const unsigned short* __restrict__ t_row,
-    const T* __restrict__ prod, T alpha, T* __restrict__ y, T* __restrict__ scratch, int rows_cap) {
+    const T* __restrict__ prod, T alpha, T* __restrict__ y, T* __restrict__ scratch, int rows_cap,
+    const int* __restrict__ skip) {
+  if (skip && *skip) return;
   extern __shared__ __align__(16) unsigned char smem[];
   constexpr int kWaves = kLongThreads / kWave;
   // every wave's accumulators (rows_cap of them: no row block of this launch has more rows), then one dummy
@@ -623,7 +626,8 @@ __global__ __launch_bounds__(kLongThreads) void tiled_long_kernel(
 template <typename T>
 __global__ __launch_bounds__(256) void tiled_long_finish_kernel(const LongFinish* __restrict__ fin,
                                                                 const T* __restrict__ scratch, T alpha,
-                                                                T* __restrict__ y) {
+                                                                T* __restrict__ y, const int* __restrict__ skip) {
+  if (skip && *skip) return;
   const LongFinish f = fin[blockIdx.x];
   for (int i = threadIdx.x; i < f.nrows; i += 256) {
     T sum = scratch[(int64_t)f.out0 + i];

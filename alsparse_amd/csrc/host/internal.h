@@ -37,6 +37,19 @@ typedef struct asamd_record {
   /* library-built mirrors: fingerprints of the HOST values and structure arrays at the time they were copied */
   uint64_t host_val_fingerprint;
   uint64_t host_idx_fingerprint;
+  /* lazy records only: a caller who never analyses but multiplies the same arrays again and again is given a
+   * tiled copy that is WATCHED (asamd_csr_plan_csrmv_watched) where the analysis' model expects it to pay:
+   * calls seen in a row on the same three arrays, the value array they named, and the state of the promotion
+   * (0 not tried, 1 in use, 2 not again) with what it owns */
+  uint32_t lazy_calls;
+  const void *lazy_val;
+  int promo_state;
+  asamd_csr_plan *promo_plan;
+  uint64_t *d_watch;    /* fingerprints of row_ptr and col_ind at promotion (device) */
+  int32_t *h_changed;   /* pinned: the last watched multiply's verdict, copied behind it */
+  void *promo_event;    /* hipEvent_t recorded behind that copy */
+  int promo_pending;    /* a copy is on its way */
+  int promo_misses;     /* watched multiplies in a row that found the structure changed */
   /* host-pointer entry points: device staging for x / y (ASAMD_KEY_MATRIX only) */
   void *d_in;
   size_t d_in_bytes;
@@ -63,6 +76,15 @@ alphasparse_status_t asamd_plan_for_call(alphasparse_dcu_handle_t handle, const 
                                          int32_t n, int32_t nnz, int32_t base, int32_t dtype,
                                          asamd_csr_plan **plan, asamd_record **lease);
 void asamd_plan_release(asamd_record *lease);
+/* A multiply without analysis (lease: the lazy record asamd_plan_for_call returned).  Counts repeated calls on
+ * the same arrays, promotes the record to a watched tiled copy when that pays, and then multiplies through it:
+ * *done = 1 if y has been enqueued, 0 if the caller is to go on with the record's ordinary plan.
+ * ALSPARSE_AMD_LAZY_COPIES=0 switches the promotion off, ALSPARSE_AMD_LAZY_AFTER=<calls> sets how many calls on
+ * the same arrays it takes (default 4). */
+alphasparse_status_t asamd_lazy_multiply(alphasparse_dcu_handle_t handle, asamd_record *lease, int32_t trans,
+                                         const void *alpha, const void *val, const void *row_ptr,
+                                         const void *col_ind, const void *x, const void *beta, void *y, int *done);
+
 /* forgets the lazy records of a handle that is being destroyed */
 void asamd_registry_drop_handle(const void *handle);
 /* number of lazy records alive (tests) */

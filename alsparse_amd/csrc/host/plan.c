@@ -428,7 +428,7 @@ static int run_algo(hipStream_t s, const asamd_csr_plan *p, int algo, const asam
       void *prod = ws_take(&ws, (size_t)st->nnz * vs);
       void *lscr = p->tiled.long_scratch_elems > 0 ? ws_take(&ws, (size_t)p->tiled.long_scratch_elems * vs) : NULL;
       if (!prod || (p->tiled.long_scratch_elems > 0 && !lscr)) return -1;
-      return asamd_spmv_tiled(s, a, &p->tiled, prod, lscr);
+      return asamd_spmv_tiled(s, a, &p->tiled, prod, lscr, NULL);
     }
     case ASAMD_SPMV_ROWCONST:
       return asamd_spmv_rowconst(s, a, st->const_len);
@@ -599,6 +599,63 @@ int asamd_csr_plan_csrmv(hipStream_t s, asamd_csr_plan *p, int32_t op, const voi
     }
   }
   return asamd_spmv_trans_scatter(s, &a, p->auto_width, which == 1);
+}
+
+/* ---- a matrix that nobody promised to leave alone ------------------------------------------------------ */
+#define WATCH_FLAG_BYTES 256
+
+size_t asamd_csr_plan_watched_workspace_bytes(const asamd_csr_plan *p) {
+  if (!p) return 0;
+  return asamd_csr_plan_workspace_bytes(p) + 3 * align256(ASAMD_GUARD_WS_BYTES) + WATCH_FLAG_BYTES;
+}
+
+int asamd_csr_plan_watch_begin(hipStream_t s, const asamd_csr_plan *p, const int32_t *rp, const int32_t *ci,
+                               uint64_t *watch, void *workspace, size_t workspace_bytes) {
+  if (!p || !rp || !ci || !watch) return hipErrorInvalidValue;
+  ws_cursor ws = ws_open(workspace, workspace_bytes);
+  void *g = ws_take(&ws, ASAMD_GUARD_WS_BYTES);
+  if (!g) return hipErrorInvalidValue;
+  const asamd_csr_stats *st = &p->st;
+  int e = asamd_value_guard(s, rp, ((size_t)st->m + 1) * 4, 1, NULL, g);
+  if (e == hipSuccess) e = asamd_value_guard_commit(s, g, watch);
+  if (e == hipSuccess) e = asamd_value_guard(s, ci, (size_t)st->nnz * 4, 1, NULL, g);
+  if (e == hipSuccess) e = asamd_value_guard_commit(s, g, watch + 1);
+  return e;
+}
+
+int asamd_csr_plan_csrmv_watched(hipStream_t s, asamd_csr_plan *p, const void *alpha, const void *val,
+                                 const int32_t *rp, const int32_t *ci, const void *x, const void *beta, void *y,
+                                 const uint64_t *watch, void *workspace, size_t workspace_bytes,
+                                 const int32_t **changed) {
+  if (!p || !alpha || !beta || !val || !rp || !ci || !x || !y || !watch) return hipErrorInvalidValue;
+  if (((uintptr_t)val | (uintptr_t)x | (uintptr_t)y) % (size_t)p->val_size) return hipErrorInvalidValue;
+  const asamd_csr_stats *st = &p->st;
+  if (st->algo != ASAMD_SPMV_TILED || !st->tiled_built || val != p->copy_val_src) return hipErrorInvalidValue;
+  if (workspace_bytes < asamd_csr_plan_watched_workspace_bytes(p)) return hipErrorInvalidValue;
+  ws_cursor ws = ws_open(workspace, workspace_bytes);
+  void *g_rp = ws_take(&ws, ASAMD_GUARD_WS_BYTES), *g_ci = ws_take(&ws, ASAMD_GUARD_WS_BYTES);
+  void *g_val = ws_take(&ws, ASAMD_GUARD_WS_BYTES);
+  int32_t *skip = (int32_t *)ws_take(&ws, WATCH_FLAG_BYTES);
+  const size_t vs = (size_t)p->val_size;
+  void *prod = ws_take(&ws, (size_t)st->nnz * vs);
+  void *lscr = p->tiled.long_scratch_elems > 0 ? ws_take(&ws, (size_t)p->tiled.long_scratch_elems * vs) : NULL;
+  if (!g_rp || !g_ci || !g_val || !skip || !prod || (p->tiled.long_scratch_elems > 0 && !lscr))
+    return hipErrorInvalidValue;
+  /* every byte of the three arrays is fingerprinted: a caller who made no promise gets no sampling */
+  int e = asamd_value_guard(s, rp, ((size_t)st->m + 1) * 4, 1, watch, g_rp);
+  if (e == hipSuccess) e = asamd_value_guard(s, ci, (size_t)st->nnz * 4, 1, watch + 1, g_ci);
+  if (e == hipSuccess) e = asamd_value_guard_any(s, g_rp, g_ci, skip);
+  if (e == hipSuccess) e = asamd_value_guard(s, val, (size_t)st->nnz * vs, 1, p->d_fp, g_val);
+  if (e == hipSuccess) e = (int)refresh_main(s, p, rp, ci, val, ASAMD_GUARD_FLAG(g_val));
+  if (e == hipSuccess) e = asamd_value_guard_commit(s, g_val, p->d_fp);
+  asamd_spmv_args a;
+  fill_args(&a, p, alpha, val, rp, ci, x, beta, y);
+  /* the layout's kernels, which return at once if the structure has changed, and the stand-in on the caller's
+   * arrays, which returns at once if it has not */
+  if (e == hipSuccess) e = asamd_spmv_tiled(s, &a, &p->tiled, prod, lscr, skip);
+  if (e == hipSuccess) e = asamd_spmv_vector_if(s, &a, p->auto_width, skip);
+  if (changed) *changed = skip;
+  return e;
 }
 
 /* ---- analysis: timing the candidates ----------------------------------------------------------------- */
@@ -1042,8 +1099,11 @@ static hipError_t plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t 
     /* trusted == 2: build every copy whatever the size and skip the timing
      * (lets small matrices exercise those kernels) */
     const int force = trusted == 2;
-    const int tiled_ok = tiled_eligible(p, force), ell_ok = ell_eligible(st, force);
-    const int hot_ok = hot_eligible(p, force), binned_ok = binned_eligible(p, force);
+    /* trusted == 3: for a matrix that is WATCHED rather than promised fixed (asamd_csr_plan_csrmv_watched): the
+     * tiled copy is the only one whose kernels a watcher can turn away */
+    const int only_tiled = trusted == 3;
+    const int tiled_ok = tiled_eligible(p, force), ell_ok = !only_tiled && ell_eligible(st, force);
+    const int hot_ok = !only_tiled && hot_eligible(p, force), binned_ok = !only_tiled && binned_eligible(p, force);
     if (force) {
       if (binned_ok) e = build_binned(stream, p, row_ptr);
       if (e == hipSuccess && tiled_ok) e = build_tiled(stream, p, row_ptr, col_ind, val);

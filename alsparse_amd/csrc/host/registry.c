@@ -90,8 +90,21 @@ static asamd_record *lazy_unlink_locked(asamd_record *victim) {
   return victim->leases == 0 ? victim : NULL; /* the caller frees it outside the lock */
 }
 
+static void promo_release(asamd_record *r) {
+  if (r->promo_plan) asamd_csr_plan_destroy(r->promo_plan);
+  if (r->d_watch) (void)hipFree(r->d_watch);
+  if (r->h_changed) (void)hipHostFree(r->h_changed);
+  if (r->promo_event) (void)hipEventDestroy((hipEvent_t)r->promo_event);
+  r->promo_plan = NULL;
+  r->d_watch = NULL;
+  r->h_changed = NULL;
+  r->promo_event = NULL;
+  r->promo_pending = 0;
+}
+
 static void lazy_free(asamd_record *r) {
   if (!r) return;
+  promo_release(r);
   asamd_record_release_device(r);
   free(r);
 }
@@ -194,6 +207,148 @@ alphasparse_status_t asamd_plan_for_call(alphasparse_dcu_handle_t handle, const 
   *plan = found->plan;
   *lease = found;
   return ALPHA_SPARSE_STATUS_SUCCESS;
+}
+
+/* ---- lazy records that keep coming back --------------------------------------------------------
+ * The reference's own programs multiply with info == NULL (test/dcu/level2/mv_csr_s_dcu_test.cpp:220-222), and
+ * its kernel reads the caller's arrays on every call.  A caller like that promises nothing, so nothing is
+ * assumed: a copy is only ever used behind a fingerprint of every byte of all three arrays, taken on the
+ * device in front of every multiply (asamd_csr_plan_csrmv_watched). */
+static int env_number(const char *name, int fallback) {
+  const char *v = getenv(name);
+  return v && *v ? atoi(v) : fallback;
+}
+
+static int stream_is_capturing(hipStream_t s) {
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(s, &st) != hipSuccess) {
+    (void)hipGetLastError();
+    return 1; /* unknown: do nothing that a capture forbids */
+  }
+  return st != hipStreamCaptureStatusNone;
+}
+
+/* lays out the watched copy if the analysis' model expects it to pay with the fingerprints' cost on top */
+static void promo_try(alphasparse_dcu_handle_t handle, asamd_record *r, const void *val) {
+  r->promo_state = 2; /* whatever happens below is not tried again for this record */
+  static const int kValSize[4] = {4, 8, 8, 16};
+  const double vs = (double)kValSize[r->dtype], nnz = (double)r->nnz;
+  /* the tiled copy is for large matrices whose x outgrows an L2 (the plan checks again) */
+  if (r->nnz < (1 << 22) || (double)r->n * vs < (double)(4 << 20)) return;
+  size_t free_b = 0, total_b = 0;
+  if (hipMemGetInfo(&free_b, &total_b) != hipSuccess) {
+    (void)hipGetLastError();
+    return;
+  }
+  if ((double)free_b < nnz * (3.0 * vs + 40.0)) return; /* copy, its layout's scratch, the product array */
+  asamd_csr_plan *p = NULL;
+  if (asamd_csr_plan_create_dtype(handle->stream, r->m, r->n, r->nnz, (const int32_t *)r->row_ptr,
+                                  (const int32_t *)r->col_ind, val, r->base, r->dtype, /*trusted=*/3, &p) != hipSuccess) {
+    (void)hipGetLastError();
+    return;
+  }
+  const asamd_csr_stats *st = asamd_csr_plan_stats(p);
+  /* three more passes: 4 bytes of row_ptr per row, 4 of col_ind and one value per entry, at 4.5 TB/s */
+  const double watch_ms = (nnz * (4.0 + vs) + 4.0 * (double)r->m) / 4.5e9;
+  int ok = st->algo == ASAMD_SPMV_TILED && st->tiled_built && st->tune_ms_base > 0.f &&
+           (double)st->tune_ms_tiled + watch_ms < 0.6 * (double)st->tune_ms_base;
+  hipEvent_t ev = NULL;
+  if (ok) ok = hipMalloc((void **)&r->d_watch, 2 * sizeof(uint64_t)) == hipSuccess;
+  if (ok) ok = hipHostMalloc((void **)&r->h_changed, sizeof(int32_t), hipHostMallocDefault) == hipSuccess;
+  if (ok) ok = hipEventCreateWithFlags(&ev, hipEventDisableTiming) == hipSuccess;
+  if (ok) {
+    r->promo_event = (void *)ev;
+    *r->h_changed = 0;
+    ok = asamd_handle_reserve(handle, asamd_csr_plan_watched_workspace_bytes(p)) == ALPHA_SPARSE_STATUS_SUCCESS;
+  }
+  if (ok)
+    ok = asamd_csr_plan_watch_begin(handle->stream, p, (const int32_t *)r->row_ptr, (const int32_t *)r->col_ind,
+                                    r->d_watch, handle->buffer, handle->buffer_size) == hipSuccess;
+  if (!ok) {
+    (void)hipGetLastError();
+    r->promo_plan = p;
+    promo_release(r);
+    return;
+  }
+  r->promo_plan = p;
+  r->promo_state = 1;
+  r->promo_misses = 0;
+}
+
+alphasparse_status_t asamd_lazy_multiply(alphasparse_dcu_handle_t handle, asamd_record *r, int32_t trans,
+                                         const void *alpha, const void *val, const void *row_ptr,
+                                         const void *col_ind, const void *x, const void *beta, void *y, int *done) {
+  *done = 0;
+  if (!r || r->kind != ASAMD_KEY_LAZY || r->promo_state == 2 || trans != 0) return ALPHA_SPARSE_STATUS_SUCCESS;
+  static int enabled = -1, after = 4;
+  if (enabled < 0) {
+    after = env_number("ALSPARSE_AMD_LAZY_AFTER", 4);
+    if (after < 1) after = 1;
+    enabled = env_number("ALSPARSE_AMD_LAZY_COPIES", 1) != 0 && asamd_env_algo() == ASAMD_SPMV_AUTO &&
+              !asamd_env_structure_only();
+  }
+  if (!enabled) return ALPHA_SPARSE_STATUS_SUCCESS;
+  (void)row_ptr; /* (the record was found by it) */
+  if (col_ind != r->col_ind || val != r->lazy_val) {
+    /* other arrays than last time: the count starts again, and a copy of the old ones goes */
+    r->col_ind = col_ind;
+    r->lazy_val = val;
+    r->lazy_calls = 1;
+    if (r->promo_state == 1) {
+      promo_release(r);
+      r->promo_state = 0;
+    }
+    return ALPHA_SPARSE_STATUS_SUCCESS;
+  }
+  ++r->lazy_calls;
+  const int capturing = stream_is_capturing(handle->stream);
+  if (r->promo_state == 0) {
+    if (r->lazy_calls < (uint32_t)after || capturing) return ALPHA_SPARSE_STATUS_SUCCESS;
+    promo_try(handle, r, val);
+    if (r->promo_state != 1) return ALPHA_SPARSE_STATUS_SUCCESS;
+  }
+  /* what the watched multiplies before this one found, if it has arrived (never waited for) */
+  if (capturing) {
+    /* (a capture forbids even asking) */
+  } else if (r->promo_pending && hipEventQuery((hipEvent_t)r->promo_event) == hipSuccess) {
+    r->promo_pending = 0;
+    r->promo_misses = *r->h_changed ? r->promo_misses + 1 : 0;
+    if (r->promo_misses >= 2) {
+      /* the arrays keep changing: the copy only costs */
+      promo_release(r);
+      r->promo_state = 2;
+      return ALPHA_SPARSE_STATUS_SUCCESS;
+    }
+  } else if (r->promo_pending) {
+    (void)hipGetLastError(); /* hipErrorNotReady is not an error */
+  }
+  const size_t need = asamd_csr_plan_watched_workspace_bytes(r->promo_plan);
+  if (handle->buffer_size < need) {
+    if (capturing || asamd_handle_reserve(handle, need) != ALPHA_SPARSE_STATUS_SUCCESS)
+      return ALPHA_SPARSE_STATUS_SUCCESS; /* the ordinary plan needs less */
+  }
+  const int32_t *changed = NULL;
+  ASAMD_HIP_STATUS(asamd_csr_plan_csrmv_watched(handle->stream, r->promo_plan, alpha, val, (const int32_t *)r->row_ptr,
+                                                (const int32_t *)col_ind, x, beta, y, r->d_watch, handle->buffer,
+                                                handle->buffer_size, &changed));
+  if (!capturing && !r->promo_pending && changed) {
+    if (hipMemcpyAsync(r->h_changed, changed, sizeof(int32_t), hipMemcpyDeviceToHost, handle->stream) == hipSuccess &&
+        hipEventRecord((hipEvent_t)r->promo_event, handle->stream) == hipSuccess)
+      r->promo_pending = 1;
+    else
+      (void)hipGetLastError();
+  }
+  *done = 1;
+  return ALPHA_SPARSE_STATUS_SUCCESS;
+}
+
+int asamd_registry_lazy_promoted(const void *handle, const void *row_ptr) {
+  int promoted = 0;
+  pthread_mutex_lock(&g_lock);
+  for (asamd_record *r = g_head[ASAMD_KEY_LAZY]; r; r = r->next)
+    if (r->key == row_ptr && r->owner == handle) promoted = r->promo_state == 1;
+  pthread_mutex_unlock(&g_lock);
+  return promoted;
 }
 
 /* every lazy record of a handle goes with the handle */

@@ -90,6 +90,9 @@ typedef struct {
 
 /* `width` in {2, 4, ..., 64} lanes sum a row (the reference's mapping, dcu_gemv_vector.h:14-57). */
 int asamd_spmv_vector(hipStream_t stream, const asamd_spmv_args *a, int32_t width);
+/* the same, launched whatever happens but returning at once unless the device word *run_if is non-zero
+ * (NULL: always runs): the stand-in for a kernel that a device-side guard may turn away */
+int asamd_spmv_vector_if(hipStream_t stream, const asamd_spmv_args *a, int32_t width, const int32_t *run_if);
 /* One lane per row, entries in storage order (src/plain/kernel/level2/mv/gemv/gemv_x_csr_plain.c:11-22). */
 int asamd_spmv_scalar(hipStream_t stream, const asamd_spmv_args *a);
 /* Every row has row_len entries (4, 8, ..., 256): no row_ptr traffic.  Real element types, row_ptr[0] ==
@@ -152,9 +155,11 @@ int asamd_tiled_build(hipStream_t stream, int32_t dtype, int32_t m, int32_t n, i
                       const int32_t *row_ptr, const int32_t *col_ind, const void *val, int32_t max_len,
                       int32_t entries_per_lane, asamd_tiled_layout *out);
 void asamd_tiled_free(asamd_tiled_layout *layout);
-/* y = alpha*A*x + beta*y from the layout (a->val, a->row_ptr, a->col_ind are not read) */
+/* y = alpha*A*x + beta*y from the layout (a->val, a->row_ptr, a->col_ind are not read).  skip: NULL, or a
+ * device word; when it is non-zero the kernels that write y return at once (a guard found that the layout no
+ * longer describes the caller's matrix, and asamd_spmv_vector_if on the same word computes y instead) */
 int asamd_spmv_tiled(hipStream_t stream, const asamd_spmv_args *a, const asamd_tiled_layout *layout,
-                     void *products, void *long_scratch);
+                     void *products, void *long_scratch, const int32_t *skip);
 
 /* Hot-column merge-path for power-law columns: the column stream rewritten as ranks of the popular
  * columns (pcol), whose x sits in LDS (the cols_lds most popular) or in a compact front (cols_front).
@@ -254,6 +259,9 @@ size_t asamd_value_guard_run(size_t nbytes);
 int asamd_value_guard(hipStream_t stream, const void *val, size_t nbytes, int32_t full, const uint64_t *stored,
                       void *ws);
 int asamd_value_guard_commit(hipStream_t stream, const void *ws, uint64_t *stored);
+/* *out = 1 if either of two guards' flags is set, else 0 (the guard works on any array of 4-byte words: the
+ * structure arrays of a matrix that nobody promised to leave alone are watched with it too) */
+int asamd_value_guard_any(hipStream_t stream, const void *ws_a, const void *ws_b, int32_t *out);
 /* out[q] = val[perm[q]] (conj != 0: conjugated) for q < nnz; gate: NULL, or a device flag (0 = do nothing) */
 int asamd_gather_values(hipStream_t stream, int32_t dtype, int32_t conj, int32_t nnz, const uint32_t *perm,
                         const void *val, void *out, const int32_t *gate);

@@ -80,7 +80,8 @@ typedef struct asamd_csr_plan asamd_csr_plan;
  * `algo_tuning` flag for exactly this, include/alphasparse/handle.h:120-123).  ALSPARSE_AMD_TUNE=model
  * decides from the statistics and fixed constants instead of timings, so that the same matrix always gets
  * the same family.  trusted == 2 builds every copy whatever the size and skips the timing (for tests of
- * those kernels); the kernel choice then stays the structural one. */
+ * those kernels); the kernel choice then stays the structural one.  trusted == 3: as 1, with the tiled copy
+ * as the only candidate (see asamd_csr_plan_csrmv_watched). */
 int asamd_csr_plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t nnz,
                           const int32_t *row_ptr, const int32_t *col_ind, const void *val,
                           int32_t base, int32_t val_size, int32_t trusted, asamd_csr_plan **plan);
@@ -125,6 +126,25 @@ int asamd_csr_plan_csrmv(hipStream_t stream, asamd_csr_plan *plan, int32_t op, c
                          const int32_t *row_ptr, const int32_t *col_ind, const void *x, const void *beta, void *y,
                          void *workspace, size_t workspace_bytes);
 
+/* A matrix that is WATCHED instead of promised fixed -- what a caller who never analyses gets once the same
+ * arrays have come back often enough.  The plan is one made with trusted == 3 (only the tiled copy is a
+ * candidate) whose analysis kept that copy.  Every watched multiply fingerprints EVERY byte of row_ptr, col_ind
+ * and val on the device, compares the first two with the words at watch[0..1] (set by asamd_csr_plan_watch_begin
+ * when the plan was made) and the third with the plan's own, gathers the copy's values again if they moved, and
+ * launches both the tiled kernels -- which return at once if the structure moved -- and a lane group per row on
+ * the caller's arrays -- which returns at once if it did not.  The result is that of the arrays as they are,
+ * whatever was done to them; nothing waits for the host.  *changed (if asked for) points at the device word
+ * that says which of the two ran (non-zero: the structure moved), inside the workspace.
+ * workspace: at least asamd_csr_plan_watched_workspace_bytes; hipErrorInvalidValue otherwise, or if the plan
+ * did not keep a tiled copy of exactly this val. */
+size_t asamd_csr_plan_watched_workspace_bytes(const asamd_csr_plan *plan);
+int asamd_csr_plan_watch_begin(hipStream_t stream, const asamd_csr_plan *plan, const int32_t *row_ptr,
+                               const int32_t *col_ind, uint64_t *watch, void *workspace, size_t workspace_bytes);
+int asamd_csr_plan_csrmv_watched(hipStream_t stream, asamd_csr_plan *plan, const void *alpha, const void *val,
+                                 const int32_t *row_ptr, const int32_t *col_ind, const void *x, const void *beta,
+                                 void *y, const uint64_t *watch, void *workspace, size_t workspace_bytes,
+                                 const int32_t **changed);
+
 /* Gathers every copy of the plan again from `val` (the array the copies were laid out from, or one
  * with the same structure) without looking whether anything changed: streaming kernels on `stream`
  * only, no sort, no allocation, no wait.  Not to be run while another stream multiplies with the plan. */
@@ -154,6 +174,9 @@ int asamd_csr_plan_transpose_arrays(const asamd_csr_plan *plan, int32_t conj, co
  * covers) that the library remembers at the moment: at most 64, the least recently used one makes room,
  * and a handle's own go with the handle.  For tests. */
 int asamd_registry_lazy_count(void);
+/* 1 if multiplies without analysis on `handle` with this device csr_row_ptr go through a watched tiled copy
+ * at the moment (the same arrays came back often enough and the copy is expected to pay).  For tests. */
+int asamd_registry_lazy_promoted(const void *handle, const void *row_ptr);
 
 /* Introspection for benchmarks and tests: statistics of the analysis that a multiply would use for
  * `key`, where key is the alphasparse_dcu_mat_info_t of an explicit analysis, or a device csr_row_ptr
