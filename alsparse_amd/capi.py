@@ -315,7 +315,7 @@ _COMMON = {
     "asamd_csr_plan_csrmv": [_P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, c_size_t],
     "asamd_handle_reserve": [_P, c_size_t],
     "asamd_csr_plan_watched_workspace_bytes": [_P],
-    "asamd_csr_plan_watch_begin": [_P, _P, _P, _P, _P, _P, c_size_t],
+    "asamd_csr_plan_watch_begin": [_P, _P, _P, _P, _P, _P, _P, c_size_t],
     "asamd_csr_plan_csrmv_watched": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_size_t, _P],
     # stateless launchers and layout builders (records are passed as opaque pointers here)
     "asamd_spmv_vector": [_P, POINTER(asamd_spmv_args), _I],

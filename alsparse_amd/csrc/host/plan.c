@@ -609,9 +609,9 @@ size_t asamd_csr_plan_watched_workspace_bytes(const asamd_csr_plan *p) {
   return asamd_csr_plan_workspace_bytes(p) + 3 * align256(ASAMD_GUARD_WS_BYTES) + WATCH_FLAG_BYTES;
 }
 
-int asamd_csr_plan_watch_begin(hipStream_t s, const asamd_csr_plan *p, const int32_t *rp, const int32_t *ci,
+int asamd_csr_plan_watch_begin(hipStream_t s, asamd_csr_plan *p, const int32_t *rp, const int32_t *ci, const void *val,
                                uint64_t *watch, void *workspace, size_t workspace_bytes) {
-  if (!p || !rp || !ci || !watch) return hipErrorInvalidValue;
+  if (!p || !rp || !ci || !val || !watch) return hipErrorInvalidValue;
   ws_cursor ws = ws_open(workspace, workspace_bytes);
   void *g = ws_take(&ws, ASAMD_GUARD_WS_BYTES);
   if (!g) return hipErrorInvalidValue;
@@ -620,6 +620,9 @@ int asamd_csr_plan_watch_begin(hipStream_t s, const asamd_csr_plan *p, const int
   if (e == hipSuccess) e = asamd_value_guard_commit(s, g, watch);
   if (e == hipSuccess) e = asamd_value_guard(s, ci, (size_t)st->nnz * 4, 1, NULL, g);
   if (e == hipSuccess) e = asamd_value_guard_commit(s, g, watch + 1);
+  /* the values' fingerprint of the plan, which may be a sampled one, becomes one of every byte as well */
+  if (e == hipSuccess) e = asamd_value_guard(s, val, (size_t)st->nnz * (size_t)p->val_size, 1, NULL, g);
+  if (e == hipSuccess) e = asamd_value_guard_commit(s, g, p->d_fp);
   return e;
 }
 

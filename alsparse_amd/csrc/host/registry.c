@@ -262,7 +262,7 @@ static void promo_try(alphasparse_dcu_handle_t handle, asamd_record *r, const vo
     ok = asamd_handle_reserve(handle, asamd_csr_plan_watched_workspace_bytes(p)) == ALPHA_SPARSE_STATUS_SUCCESS;
   }
   if (ok)
-    ok = asamd_csr_plan_watch_begin(handle->stream, p, (const int32_t *)r->row_ptr, (const int32_t *)r->col_ind,
+    ok = asamd_csr_plan_watch_begin(handle->stream, p, (const int32_t *)r->row_ptr, (const int32_t *)r->col_ind, val,
                                     r->d_watch, handle->buffer, handle->buffer_size) == hipSuccess;
   if (!ok) {
     (void)hipGetLastError();

@@ -927,7 +927,7 @@ def main():
         "cpu_baseline": main_res.get("cpu_baseline"),
         "vendor_baseline": main_res.get("vendor_baseline"),
     }
-    for k in ("analysis_bytes", "workspace_bytes", "value_check", "tune_mode", "locality_probe"):
+    for k in ("analysis_bytes", "workspace_bytes", "value_check", "tune_mode", "locality_probe", "calls_2_to_5_ms", "watched_copy"):
         if main_res.get(k) is not None:
             out["config"][k] = main_res[k]
     if ceilings:

@@ -138,8 +138,9 @@ int asamd_csr_plan_csrmv(hipStream_t stream, asamd_csr_plan *plan, int32_t op, c
  * workspace: at least asamd_csr_plan_watched_workspace_bytes; hipErrorInvalidValue otherwise, or if the plan
  * did not keep a tiled copy of exactly this val. */
 size_t asamd_csr_plan_watched_workspace_bytes(const asamd_csr_plan *plan);
-int asamd_csr_plan_watch_begin(hipStream_t stream, const asamd_csr_plan *plan, const int32_t *row_ptr,
-                               const int32_t *col_ind, uint64_t *watch, void *workspace, size_t workspace_bytes);
+int asamd_csr_plan_watch_begin(hipStream_t stream, asamd_csr_plan *plan, const int32_t *row_ptr,
+                               const int32_t *col_ind, const void *val, uint64_t *watch, void *workspace,
+                               size_t workspace_bytes);
 int asamd_csr_plan_csrmv_watched(hipStream_t stream, asamd_csr_plan *plan, const void *alpha, const void *val,
                                  const int32_t *row_ptr, const int32_t *col_ind, const void *x, const void *beta,
                                  void *y, const uint64_t *watch, void *workspace, size_t workspace_bytes,
