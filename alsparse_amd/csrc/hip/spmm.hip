@@ -768,10 +768,11 @@ __global__ __launch_bounds__(kSpmmBlock) void spmm_reuse_probe_kernel(int m, con
 // are being read and the row offsets of run i + 3.  A run whose entries or distinct columns exceed the staging
 // areas is multiplied straight from global memory, a wave per row.  Every sum is formed in CSR order: the same
 // bits every run.
-// Measured (27-point stencil 128 x 128 x 64, n = 64, fp32): 0.62 ms, against 0.52 ms for four rows of B per wave
-// instruction without LDS.  The L1 requests fall as intended, but a workgroup's five barriers and the hash's
-// atomics per run leave the three workgroups that fit a compute unit waiting 59% of their cycles; nothing is
-// saturated.  Not chosen by default.
+// Measured (27-point stencil 128 x 128 x 64, n = 64, fp32): 0.62 ms, against 0.51 ms for four rows of B per wave
+// instruction without LDS.  The L1 requests fall as intended (62 per row of A instead of 147), but the stages'
+// times add up instead of overlapping -- the sums alone take 0.28 ms: they read every entry's 256 bytes of B from
+// LDS, 7 GB in all, and the LDS data path is busy half of the kernel's clocks -- and hashing the next run two
+// iterations ahead, so that the rows of B travel for a whole iteration, changed nothing.  Not chosen by default.
 template <typename T>
 struct LdsSpmm {
   // rows of A per run, and rows of B that the tile holds (42 KiB; a 27-point stencil's 16 rows touch 9 x 18)
