@@ -28,9 +28,14 @@ template <typename T, int W>
 static void launch_vector(hipStream_t s, const asamd_spmv_args* a, const int32_t* run_if) {
   constexpr int rows_per_block = kRowsBlock / W;
   const unsigned grid = (unsigned)(((int64_t)a->m + rows_per_block - 1) / rows_per_block);
-  spmv_vector_kernel<T, W><<<grid, kRowsBlock, 0, s>>>(a->m, scalar_of<T>(a->alpha), (const T*)a->val, a->row_ptr,
-                                                       a->col_ind, (const T*)a->x, scalar_of<T>(a->beta), (T*)a->y,
-                                                       a->base, run_if);
+  if (run_if)
+    spmv_vector_standin_kernel<T, W><<<grid < 2048u ? grid : 2048u, kRowsBlock, 0, s>>>(
+        a->m, scalar_of<T>(a->alpha), (const T*)a->val, a->row_ptr, a->col_ind, (const T*)a->x, scalar_of<T>(a->beta),
+        (T*)a->y, a->base, grid, run_if);
+  else
+    spmv_vector_kernel<T, W><<<grid, kRowsBlock, 0, s>>>(a->m, scalar_of<T>(a->alpha), (const T*)a->val, a->row_ptr,
+                                                         a->col_ind, (const T*)a->x, scalar_of<T>(a->beta), (T*)a->y,
+                                                         a->base);
 }
 
 extern "C" int asamd_spmv_vector_if(hipStream_t s, const asamd_spmv_args* a, int32_t width, const int32_t* run_if) {

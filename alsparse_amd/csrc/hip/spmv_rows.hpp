@@ -24,14 +24,12 @@ namespace asamd {
 
 constexpr int kRowsBlock = 256;  // threads per workgroup of the row kernels
 
+// the rows of workgroup `bid`: W lanes per row
 template <typename T, int W>
-__global__ __launch_bounds__(kRowsBlock) void spmv_vector_kernel(
-    int m, T alpha, const T* __restrict__ val, const int* __restrict__ row_ptr,
-    const int* __restrict__ col_ind, const T* __restrict__ x, T beta, T* __restrict__ y, int base,
-    const int* __restrict__ run_if = nullptr) {
-  if (run_if && *run_if == 0) return;  // a stand-in that is only needed when another kernel was turned away
+__device__ __forceinline__ void spmv_vector_block(unsigned bid, int m, T alpha, const T* __restrict__ val,
+                                                  const int* __restrict__ row_ptr, const int* __restrict__ col_ind,
+                                                  const T* __restrict__ x, T beta, T* __restrict__ y, int base) {
   constexpr int kRowsPerBlock = kRowsBlock / W;
-  const unsigned bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
   const int lane = threadIdx.x % W;
   const int64_t row = (int64_t)bid * kRowsPerBlock + threadIdx.x / W;
   if (row >= m) return;  // whole lane groups leave together
@@ -72,6 +70,26 @@ __global__ __launch_bounds__(kRowsBlock) void spmv_vector_kernel(
   if (j < end) sum = fma_t(val[j], xb[col_ind[j]], sum);
   sum = group_sum<W>(sum);
   if (lane == 0) store_axpby(y, row, alpha, sum, beta);
+}
+
+template <typename T, int W>
+__global__ __launch_bounds__(kRowsBlock) void spmv_vector_kernel(
+    int m, T alpha, const T* __restrict__ val, const int* __restrict__ row_ptr,
+    const int* __restrict__ col_ind, const T* __restrict__ x, T beta, T* __restrict__ y, int base) {
+  spmv_vector_block<T, W>(xcd_contiguous_id(blockIdx.x, gridDim.x), m, alpha, val, row_ptr, col_ind, x, beta, y, base);
+}
+
+// The stand-in for a kernel that a device-side guard may turn away: launched every time, with a small grid
+// whose workgroups walk the row blocks in turn, so that the usual case -- *run_if == 0, nothing to do -- costs
+// a few hundred empty workgroups instead of one per row block.
+template <typename T, int W>
+__global__ __launch_bounds__(kRowsBlock) void spmv_vector_standin_kernel(
+    int m, T alpha, const T* __restrict__ val, const int* __restrict__ row_ptr,
+    const int* __restrict__ col_ind, const T* __restrict__ x, T beta, T* __restrict__ y, int base,
+    unsigned nblocks, const int* __restrict__ run_if) {
+  if (*run_if == 0) return;
+  for (unsigned b = blockIdx.x; b < nblocks; b += gridDim.x)
+    spmv_vector_block<T, W>(b, m, alpha, val, row_ptr, col_ind, x, beta, y, base);
 }
 
 template <typename T>
