@@ -36,16 +36,17 @@ def _promoted(lib, h, da):
     return lib.asamd_registry_lazy_promoted(h.h, da.row_ptr.c_ptr())
 
 
-def test_returning_matrix_goes_through_a_watched_copy_and_every_edit_shows(gpu):
+@pytest.mark.parametrize("base", [0, 1])
+def test_returning_matrix_goes_through_a_watched_copy_and_every_edit_shows(gpu, base):
     lib = capi.load()
-    a = wl.uniform_rows(1 << 21, 1 << 21, 16, np.float32)  # 8 MiB of x, scattered columns: the tiled copy's case
+    a = wl.uniform_rows(1 << 21, 1 << 21, 16, np.float32, base=base)  # 8 MiB of x, scattered columns: the tiled copy's case
     x, y0 = wl.uniform(a.cols, a.dtype, 3), wl.uniform(a.rows, a.dtype, 4)
     da = DeviceCsr(a)
     dx, dy = hiprt.DeviceArray.from_numpy(x), hiprt.DeviceArray.from_numpy(y0)
     h = capi.Handle()
-    descr = capi.make_descr()
+    descr = capi.make_descr(base=base)
     try:
-        announce("no analysis: the same arrays four times")
+        announce("no analysis: the same arrays four times, base", base)
         for call in range(1, 7):
             dy.copy_from(y0)
             _multiply(lib, h, descr, da, dx, dy, 1.5, 0.5)
