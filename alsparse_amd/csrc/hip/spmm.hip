@@ -257,12 +257,17 @@ __device__ __forceinline__ QuadChunk<T> quad_load_chunk(int64_t j0, int64_t end,
 // PERSISTENT waves, each walking the rows w, w + W, w + 2W, ... (W = waves of the grid) with the loads of three rows
 // in flight: the row offsets of the row after next, the entries of the next row, the rows of B of the current
 // one -- a wave that handles one row and exits waits for those three in turn.
-// What the kernel's time is (27-point stencil 128 x 128 x 64, n = 64, 0.51 ms): every row of A brings one row of B
-// that no cache holds yet (B has as many rows as A), so every row waits for memory at least once; a wave spends
-// 3 us per row all told, and a compute unit has as many rows in flight as it has waves -- 24 here, each holding
-// its row's 8 KB of B in registers.  Taking a third of the loads of B away, or a third of the ds_bpermutes, changed nothing; nor did row
-// offsets through vector loads, or one combined wait per row with the store of C delayed into the next row's
-// (0.52 / 0.57 ms); 7 or 8 waves per SIMD were had only with spills (0.76 ms).
+// What the kernel's time is (27-point stencil 128 x 128 x 64, n = 64, 0.51 ms): the path from the L1 to the
+// registers, not the waves' waiting for memory.  A row of A brings 8 KB of B through that path (eight wave-wide
+// 1 KB loads), and a load takes 24 clocks of its compute unit's time where the L1's 64 bytes per clock would
+// allow 16.  Two forms that took the waiting out -- the next rows' entries and offsets parked in LDS by
+// memory-to-LDS loads two rows ahead, and on top of that the rows of B of the next row of A requested before
+// the sums of the current one (two sets of registers, four waves per SIMD) -- took 0.52 and 0.51 ms: their
+// waves spend 60 % of their cycles waiting to ISSUE an instruction where this form's spend 75 % waiting for
+// loads to complete.  With every load of B turned away by the range check and no store of C all forms take
+// 0.31 ms: the LDS pipe (27 ds_bpermutes per row; 43 % of the wave cycles wait for it then).  Also without
+// effect: a third of the loads of B turned away; the store of C delayed into the next row (0.57 ms); 7 or 8
+// waves per SIMD, had only with spills (0.76 ms).
 template <typename T, bool NARROW>
 __global__ __launch_bounds__(kSpmmBlock) void spmm_rowmajor_quad_kernel(
     int m, int n, T alpha, const T* __restrict__ val, const int* __restrict__ row_ptr,
