@@ -279,6 +279,27 @@ __device__ __forceinline__ T segmented_scan(T v, bool head) {
   return v;
 }
 
+// v(l) + v(l ^ HALF) for HALF = 16 or 32, without the LDS crossbar that a shuffle goes through:
+// v_permlane16_swap / v_permlane32_swap exchange the odd 16-lane rows (the upper 32 lanes) of one register with
+// the even rows (the lower 32 lanes) of another, so two copies of v become "the even partner's" and "the odd
+// partner's" value in every lane.  (Two idle states in front: the hardware wants them between a write of the
+// registers and the swap, and the compiler does not look into the statement.)
+template <int HALF, typename T>
+__device__ __forceinline__ T sum_with_lane_xor(T v) {
+  static_assert(HALF == 16 || HALF == 32, "rows or halves");
+  static_assert(sizeof(T) % 4 == 0, "whole words");
+  struct Words { int w[sizeof(T) / 4]; };
+  Words a = __builtin_bit_cast(Words, v), b = a;
+#pragma unroll
+  for (int i = 0; i < (int)(sizeof(T) / 4); ++i) {
+    if constexpr (HALF == 16)
+      asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a.w[i]), "+v"(b.w[i]));
+    else
+      asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a.w[i]), "+v"(b.w[i]));
+  }
+  return __builtin_bit_cast(T, a) + __builtin_bit_cast(T, b);
+}
+
 template <int W, typename T>
 __device__ __forceinline__ T group_sum(T v) {
   static_assert(W >= 1 && W <= 64 && (W & (W - 1)) == 0, "group width");

@@ -366,9 +366,9 @@ __global__ __launch_bounds__(kSpmmBlock) void spmm_rowmajor_quad_kernel(
       }
     }
 #pragma unroll
-    for (int i = 0; i < E; ++i) acc[i] += bperm((lane ^ 16) * 4, acc[i]);
+    for (int i = 0; i < E; ++i) acc[i] = sum_with_lane_xor<16>(acc[i]);
 #pragma unroll
-    for (int i = 0; i < E; ++i) acc[i] += bperm((lane ^ 32) * 4, acc[i]);
+    for (int i = 0; i < E; ++i) acc[i] = sum_with_lane_xor<32>(acc[i]);
     if (g == 0 && owns) {
       T* crow = C + row * ldc + c0;
       Vec<T, E> out;
