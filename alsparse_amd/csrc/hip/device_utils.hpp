@@ -307,8 +307,8 @@ __device__ __forceinline__ T group_sum(T v) {
   if constexpr (W >= 4) v += dpp_mov<0x4E>(v);   // quad_perm [2,3,0,1]
   if constexpr (W >= 8) v += dpp_mov<0x141>(v);  // row_half_mirror: lane l <-> 7-l in each 8
   if constexpr (W >= 16) v += dpp_mov<0x140>(v); // row_mirror: lane l <-> 15-l in each 16
-  if constexpr (W >= 32) v += lane_xor(v, 16);
-  if constexpr (W >= 64) v += lane_xor(v, 32);
+  if constexpr (W >= 32) v = sum_with_lane_xor<16>(v);
+  if constexpr (W >= 64) v = sum_with_lane_xor<32>(v);
   return v;
 }
 
