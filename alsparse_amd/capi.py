@@ -330,6 +330,7 @@ _COMMON = {
     "asamd_tiled_fits": [_I, _I, _I, _I],
     "asamd_tiled_build": [_P, _I, _I, _I, _I, _I, _P, _P, _P, _I, _I, _P],
     "asamd_tiled_free": [_P],
+    "asamd_tiled_gather_values": [_P, _P, _P, _P],
     "asamd_spmv_tiled": [_P, POINTER(asamd_spmv_args), _P, _P, _P, _P],
     "asamd_hot_build": [_P, _I, _I, _I, _I, _I, _P, _P, _I, _I, _I, _P],
     "asamd_hot_free": [_P],

@@ -49,12 +49,11 @@ static hipError_t build_hot(hipStream_t stream, asamd_hot_layout* L, int m, int 
   const int64_t nb = ((int64_t)m + nnz_i + HK::Dims::items - 1) / HK::Dims::items;
   unsigned *d_cnt = nullptr, *d_key = nullptr, *d_key2 = nullptr, *d_idx = nullptr, *d_sorted = nullptr, *d_rank = nullptr;
   hipError_t e = hipMalloc(&d_cnt, (size_t)n * sizeof(unsigned));
-  if (e == hipSuccess) e = hipMalloc(&d_key, (size_t)n * sizeof(unsigned));
+  if (e == hipSuccess) e = hipMalloc(&d_key, (size_t)(n > 2 ? n : 2) * sizeof(unsigned));  // (also takes a 64-bit sum)
   if (e == hipSuccess) e = hipMalloc(&d_key2, (size_t)n * sizeof(unsigned));
   if (e == hipSuccess) e = hipMalloc(&d_idx, (size_t)n * sizeof(unsigned));
   if (e == hipSuccess) e = hipMalloc(&d_sorted, (size_t)n * sizeof(unsigned));
   if (e == hipSuccess) e = hipMemsetAsync(d_cnt, 0, (size_t)n * sizeof(unsigned), stream);
-  std::vector<unsigned> h_key((size_t)h1);
   // large matrices are counted through one chunk of entries in four (the ranking of the popular columns and the
   // share below are then estimates, good to a per cent or so)
   const int sample_shift = nnz_i >= (1 << 24) ? 2 : 0;
@@ -64,10 +63,15 @@ static hipError_t build_hot(hipStream_t stream, asamd_hot_layout* L, int m, int 
     e = hipGetLastError();
   }
   if (e == hipSuccess) e = sort_pairs_u32(stream, d_key, d_key2, d_idx, d_sorted, (size_t)n, 32);
-  if (e == hipSuccess) e = hipMemcpy(h_key.data(), d_key2, (size_t)h1 * sizeof(unsigned), hipMemcpyDeviceToHost);
+  unsigned long long h_head = 0;
   if (e == hipSuccess) {
-    double in_lds = 0.0;
-    for (int i = 0; i < h1; ++i) in_lds += (double)(~h_key[(size_t)i]) * (double)(1 << sample_shift);
+    // (d_key, the sort's input, is free again: its first words take the sum)
+    col_rank_head_sum_kernel<<<1, 256, 0, stream>>>(h1, d_key2, (unsigned long long*)d_key);
+    e = hipMemcpyAsync(&h_head, d_key, sizeof(h_head), hipMemcpyDeviceToHost, stream);
+  }
+  if (e == hipSuccess) e = hipStreamSynchronize(stream);
+  if (e == hipSuccess) {
+    const double in_lds = (double)h_head * (double)(1 << sample_shift);
     L->cols_lds = h1;
     L->cols_front = hc;
     L->share_lds = (float)(in_lds / (double)nnz);

@@ -46,6 +46,16 @@ static std::vector<int> cut_blocks(const int* off, int groups, int max_groups, i
   return start;
 }
 
+template <typename T>
+static void launch_gather_tiles(hipStream_t s, const asamd_tiled_layout* L, const void* val, const int32_t* gate) {
+  // eight tiles to a wave at a time, eight workgroups abreast (one per XCD), as many as the chip holds at once
+  const int64_t per_xcd = ((int64_t)(L->row_blocks + 7) / 8) * ((L->col_blocks + 7) / 8);
+  int64_t grid = (per_xcd + 3) / 4 * 8;
+  if (grid > 8 * 512) grid = 8 * 512;
+  gather_values_tiles_kernel<T, false><<<(unsigned)grid, 256, 0, s>>>(L->tperm, (const T*)val, (T*)L->tval, L->tile_ptr,
+                                                                     L->col_blocks, L->row_blocks, gate);
+}
+
 // Equal-entry column / row blocks, stable sort of the entries by (column block,
 // row block), then the arrays of both phases in that order and the tile tables.
 template <typename T>
@@ -65,6 +75,7 @@ static hipError_t build_tiled(hipStream_t stream, asamd_tiled_layout* L, const i
   LongTile* d_long_raw = nullptr;
   unsigned *d_key = nullptr, *d_key2 = nullptr, *d_idx = nullptr, *d_perm = nullptr;
   std::vector<int> h_off, cgb, rgb, cstart, rstart, h_colptr;
+  int* h_cnt = nullptr;  // pinned
   std::vector<TiledChunk> h_chunks;
   int cb = 0, rb = 0, count_stride = 1;
   int64_t tiles = 0;
@@ -78,12 +89,19 @@ static hipError_t build_tiled(hipStream_t stream, asamd_tiled_layout* L, const i
     while (((int64_t)nnz_i >> 23) >= (int64_t)2 * count_stride) count_stride *= 2;
     col_group_count_kernel<<<256 * 32, 256, 0, stream>>>(nnz_i, col_ind, base, count_stride, d_cnt);
     h_off.resize(cnt_n + 1);
-    e = hipMemcpyAsync(h_off.data() + 1, d_cnt, (size_t)col_groups * sizeof(int), hipMemcpyDeviceToHost, stream);
+    // The counts travel to pinned host memory through a kernel that writes there: a device-to-host copy of
+    // these 256 KB goes to the copy engine, and the first such copy after a pause took 6.4 ms here with the GPU
+    // idle (the 1 MB copy right behind it 0.2 ms).
+    e = hipHostMalloc((void**)&h_cnt, cnt_n * sizeof(int), hipHostMallocDefault);
+    if (e == hipSuccess) {
+      strided_gather_kernel<<<(unsigned)((col_groups + 255) / 256), 256, 0, stream>>>(col_groups, d_cnt, 1, h_cnt);
+      e = hipGetLastError();
+    }
   }
   if (e == hipSuccess) e = hipStreamSynchronize(stream);
   if (e == hipSuccess) {
     h_off[0] = 0;
-    for (int g = 0; g < col_groups; ++g) h_off[(size_t)g + 1] += h_off[(size_t)g];
+    for (int g = 0; g < col_groups; ++g) h_off[(size_t)g + 1] = h_off[(size_t)g] + h_cnt[(size_t)g];
     // Width of a column block: at most TileDims<T>::cols (the x slice of phase 1).  A row block cannot be
     // shorter than one group of 64 rows, whose tiles hold 64 * entries per row / column blocks entries on
     // average: where the rows are so long that this exceeds 64 the column blocks are made narrower
@@ -100,11 +118,12 @@ static hipError_t build_tiled(hipStream_t stream, asamd_tiled_layout* L, const i
                         (int64_t)h_off[(size_t)col_groups] / full + 1, cgb);  // h_off: sampled entries
     cb = (int)cstart.size() - 1;
     row_group_offsets_kernel<<<(row_groups + 1 + 255) / 256, 256, 0, stream>>>(m, row_ptr, row_groups, d_cnt);
-    e = hipMemcpyAsync(h_off.data(), d_cnt, ((size_t)row_groups + 1) * sizeof(int), hipMemcpyDeviceToHost, stream);
+    strided_gather_kernel<<<(unsigned)((row_groups + 1 + 255) / 256), 256, 0, stream>>>(row_groups + 1, d_cnt, 1, h_cnt);
+    e = hipGetLastError();
   }
   if (e == hipSuccess) e = hipStreamSynchronize(stream);
   if (e == hipSuccess) {
-    for (int g = 0; g <= row_groups; ++g) h_off[(size_t)g] -= base;
+    for (int g = 0; g <= row_groups; ++g) h_off[(size_t)g] = h_cnt[(size_t)g] - base;
     // Height of a row block: at most TileDims<T>::rows (the accumulators of a wave).  Phase 2 takes tiles
     // of up to 128 entries and longer ones go to the slow long-tile kernel: where the column blocks are
     // few (a narrow matrix) or the rows long, a full-height block would put more than that into most
@@ -208,7 +227,6 @@ static hipError_t build_tiled(hipStream_t stream, asamd_tiled_layout* L, const i
     if constexpr (kPayloadSort) {
       tile_unpack_kernel<<<256 * 32, 256, 0, stream>>>(nnz_i, (const unsigned long long*)d_perm, L->tperm,
                                                        L->tcol, L->trow);
-      gather_values_kernel<T, false><<<256 * 32, 256, 0, stream>>>(nnz_i, L->tperm, val, (T*)L->tval, nullptr);
     } else {
       tile_gather_kernel<T><<<256 * 32, 256, 0, stream>>>(nnz_i, d_perm, d_coo, col_ind, val, base, d_cgb, d_cbs,
                                                           d_rgb, L->row_block_start, (T*)L->tval,
@@ -218,6 +236,10 @@ static hipError_t build_tiled(hipStream_t stream, asamd_tiled_layout* L, const i
     }
     tile_bounds_kernel<<<(unsigned)((tiles + 1 + 255) / 256), 256, 0, stream>>>(nnz_i, d_key2, tiles,
                                                                                 d_tile_ptr);
+    if constexpr (kPayloadSort) {
+      L->tile_ptr = d_tile_ptr;  // stays with the layout: the values are gathered tile by tile, now and later
+      launch_gather_tiles<T>(stream, L, val, nullptr);
+    }
     // Entries in tiles of 65..128 entries: if they are few, phase 2 runs in its one-entry-per-lane form
     // (twice the tiles in flight) and leaves those tiles to phase 3.
     e = hipMemsetAsync(d_mid, 0, sizeof(unsigned long long), stream);
@@ -339,6 +361,8 @@ static hipError_t build_tiled(hipStream_t stream, asamd_tiled_layout* L, const i
   if (e == hipSuccess)
     e = hipFuncSetAttribute((const void*)tiled_reduce_kernel<T, 2>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, TileDims<T>::red_lds_bytes);
+  if (h_cnt) (void)hipHostFree(h_cnt);
+  if (L->tile_ptr == d_tile_ptr) d_tile_ptr = nullptr;
   for (void* d : {(void*)d_coo, (void*)d_key, (void*)d_key2, (void*)d_idx, (void*)d_perm, (void*)d_tile_ptr,
                   (void*)d_long_raw, (void*)d_long_count, (void*)d_mid, (void*)d_cnt, (void*)d_cgb, (void*)d_rgb, (void*)d_cbs})
     if (d) (void)hipFree(d);
@@ -352,6 +376,7 @@ static hipError_t build_tiled(hipStream_t stream, asamd_tiled_layout* L, const i
   L->n = n;
   L->nnz = nnz_i;
   const int64_t tables = (int64_t)tiles * (int64_t)sizeof(TileRange) + ((int64_t)rb + 1) * 4 +
+                         (L->tile_ptr ? ((int64_t)tiles + 1) * 4 : 0) +
                          (int64_t)L->n_chunks * (int64_t)sizeof(TiledChunk) +
                          (int64_t)L->n_long_chunks * (int64_t)sizeof(LongBlock) +
                          (int64_t)L->n_long_finish * (int64_t)sizeof(LongFinish);
@@ -388,7 +413,8 @@ extern "C" int asamd_tiled_build(hipStream_t stream, int32_t dtype, int32_t m, i
 
 extern "C" void asamd_tiled_free(asamd_tiled_layout* L) {
   if (!L) return;
-  free_all({L->tval, (void*)L->tperm, (void*)L->tcol, (void*)L->trow, (void*)L->row_block_start, L->ranges, L->chunks,
+  free_all({L->tval, (void*)L->tperm, (void*)L->tcol, (void*)L->trow, (void*)L->row_block_start, (void*)L->tile_ptr,
+            L->ranges, L->chunks,
             L->long_list, L->long_tiles, L->long_finish});
   *L = asamd_tiled_layout{};
 }
@@ -441,6 +467,19 @@ extern "C" int asamd_spmv_tiled(hipStream_t s, const asamd_spmv_args* a, const a
     if (L->n_long_finish > 0)
       tiled_long_finish_kernel<T><<<L->n_long_finish, 256, 0, s>>>((const LongFinish*)L->long_finish,
                                                                    (const T*)long_scratch, alpha, y, skip);
+    return hipGetLastError();
+  });
+}
+
+extern "C" int asamd_tiled_gather_values(hipStream_t s, const asamd_tiled_layout* L, const void* val,
+                                         const int32_t* gate) {
+  if (!L || !L->tval || !L->tperm || !val) return hipErrorInvalidValue;
+  if (L->nnz == 0) return hipSuccess;
+  if (!L->tile_ptr) return asamd_gather_values(s, L->dtype, 0, L->nnz, L->tperm, val, L->tval, gate);
+  return by_dtype(L->dtype, [&](auto* tag) -> int {
+    using T = std::remove_pointer_t<decltype(tag)>;
+    if ((uintptr_t)val % alignof(T)) return hipErrorInvalidValue;
+    launch_gather_tiles<T>(s, L, val, gate);
     return hipGetLastError();
   });
 }

@@ -331,6 +331,21 @@ static __global__ __launch_bounds__(256) void col_rank_keys_kernel(int n, const 
   key[c] = ~count[c];
   idx[c] = (unsigned)c;
 }
+// *total = the counts behind the first `first` sorted keys (one workgroup; the host wants this one number, and
+// a copy of the keys themselves goes to the copy engine, whose first copy after a pause takes milliseconds)
+static __global__ __launch_bounds__(256) void col_rank_head_sum_kernel(int first, const unsigned* __restrict__ key,
+                                                                unsigned long long* __restrict__ total) {
+  __shared__ unsigned long long part[256];
+  unsigned long long sum = 0;
+  for (int i = threadIdx.x; i < first; i += 256) sum += (unsigned long long)(~key[i]);
+  part[threadIdx.x] = sum;
+  __syncthreads();
+  for (int w = 128; w > 0; w >>= 1) {
+    if ((int)threadIdx.x < w) part[threadIdx.x] += part[threadIdx.x + w];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) *total = part[0];
+}
 // rank[sorted_col[i]] = i for i < hc (rank was filled with 0xFFFFFFFF)
 static __global__ __launch_bounds__(256) void col_rank_scatter_kernel(int hc, const unsigned* __restrict__ sorted_col,
                                                                unsigned* __restrict__ rank, int* __restrict__ hot_cols) {

@@ -479,7 +479,7 @@ static hipError_t refresh_main(hipStream_t s, asamd_csr_plan *p, const int32_t *
   const asamd_csr_stats *st = &p->st;
   hipError_t e = hipSuccess;
   if (st->tiled_built)
-    e = (hipError_t)asamd_gather_values(s, p->dtype, 0, st->nnz, p->tiled.tperm, val, p->tiled.tval, gate);
+    e = (hipError_t)asamd_tiled_gather_values(s, &p->tiled, val, gate);
   if (e == hipSuccess && st->ell_built)
     e = (hipError_t)asamd_csr2ell_gated(s, p->val_size, st->m, val, rp, ci, st->base, 0, st->ell_width, p->d_eval,
                                         p->d_ecol, gate);

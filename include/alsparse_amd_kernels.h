@@ -140,6 +140,7 @@ typedef struct {
   uint32_t *tperm;           /* nnz: CSR position of the entry in every slot                   */
   uint16_t *tcol, *trow;     /* nnz columns / rows local to their blocks                       */
   int32_t *row_block_start;  /* row_blocks + 1                                                 */
+  int32_t *tile_ptr;         /* col_blocks * row_blocks + 1: first slot of tile c * row_blocks + r */
   void *ranges, *chunks, *long_list, *long_tiles, *long_finish; /* tile tables and work lists  */
   int32_t dtype, m, n, nnz;
   int32_t col_blocks, row_blocks;
@@ -155,6 +156,11 @@ int asamd_tiled_build(hipStream_t stream, int32_t dtype, int32_t m, int32_t n, i
                       const int32_t *row_ptr, const int32_t *col_ind, const void *val, int32_t max_len,
                       int32_t entries_per_lane, asamd_tiled_layout *out);
 void asamd_tiled_free(asamd_tiled_layout *layout);
+/* layout->tval[q] = val[layout->tperm[q]] for every slot, the tiles taken row block by row block (each XCD its
+ * own row blocks), so that the stretch of val a row block's tiles pick their values from is fetched from memory
+ * once; gate as for asamd_gather_values */
+int asamd_tiled_gather_values(hipStream_t stream, const asamd_tiled_layout *layout, const void *val,
+                              const int32_t *gate);
 /* y = alpha*A*x + beta*y from the layout (a->val, a->row_ptr, a->col_ind are not read).  skip: NULL, or a
  * device word; when it is non-zero the kernels that write y return at once (a guard found that the layout no
  * longer describes the caller's matrix, and asamd_spmv_vector_if on the same word computes y instead) */
