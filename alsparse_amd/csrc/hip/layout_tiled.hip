@@ -76,6 +76,7 @@ static hipError_t build_tiled(hipStream_t stream, asamd_tiled_layout* L, const i
   unsigned *d_key = nullptr, *d_key2 = nullptr, *d_idx = nullptr, *d_perm = nullptr;
   std::vector<int> h_off, cgb, rgb, cstart, rstart, h_colptr;
   int* h_cnt = nullptr;  // pinned
+  char* d_arena = nullptr;
   std::vector<TiledChunk> h_chunks;
   int cb = 0, rb = 0, count_stride = 1;
   int64_t tiles = 0;
@@ -190,19 +191,35 @@ static hipError_t build_tiled(hipStream_t stream, asamd_tiled_layout* L, const i
     e = hipMemcpy(L->row_block_start, h_rbs.data(), ((size_t)rb + 1) * sizeof(int), hipMemcpyHostToDevice);
 
   // ---- 2. sort the entries by tile, gather the tile-ordered arrays ---------------
-  if (e == hipSuccess) e = hipMalloc(&d_coo, nnz * sizeof(int));
-  if (e == hipSuccess) e = hipMalloc(&d_key, nnz * sizeof(unsigned));
-  if (e == hipSuccess) e = hipMalloc(&d_key2, nnz * sizeof(unsigned));
   // 4-byte values: the local indices are sorted together with the keys (64-bit payloads that also carry
   // the entry's position); wider ones through a permutation alone
   constexpr bool kPayloadSort = sizeof(T) == 4;
   constexpr size_t kSortValBytes = kPayloadSort ? sizeof(unsigned long long) : sizeof(unsigned);
-  if (e == hipSuccess) e = hipMalloc(&d_idx, nnz * kSortValBytes);
-  if (e == hipSuccess) e = hipMalloc(&d_perm, nnz * kSortValBytes);
+  const size_t long_cap = nnz / kWave + 1;  // a long tile holds more than kWave entries, at the least
+  // (the pass's large temporaries in ONE allocation: an allocation of this size and its release cost 0.6 ms)
+  if (e == hipSuccess) {
+    const auto room = [](size_t bytes) { return (bytes + 255) / 256 * 256; };
+    const size_t perm_bytes = kPayloadSort ? room(nnz * kSortValBytes) : 0;  // else it stays with the layout
+    e = hipMalloc(&d_arena, 3 * room(nnz * sizeof(int)) + room(nnz * kSortValBytes) + perm_bytes +
+                                room(long_cap * sizeof(LongTile)));
+    if (e == hipSuccess) {
+      char* at = d_arena;
+      const auto take = [&](size_t bytes) {
+        char* p = at;
+        at += room(bytes);
+        return (void*)p;
+      };
+      d_coo = (int*)take(nnz * sizeof(int));
+      d_key = (unsigned*)take(nnz * sizeof(unsigned));
+      d_key2 = (unsigned*)take(nnz * sizeof(unsigned));
+      d_idx = (unsigned*)take(nnz * kSortValBytes);
+      if (kPayloadSort) d_perm = (unsigned*)take(nnz * kSortValBytes);
+      d_long_raw = (LongTile*)take(long_cap * sizeof(LongTile));
+    }
+  }
+  if (e == hipSuccess && !kPayloadSort) e = hipMalloc(&d_perm, nnz * kSortValBytes);
   if (e == hipSuccess) e = hipMalloc(&d_tile_ptr, (size_t)(tiles + 1) * sizeof(int));
   if (e == hipSuccess) e = hipMalloc(&L->ranges, (size_t)tiles * sizeof(TileRange));
-  const size_t long_cap = nnz / kWave + 1;  // a long tile holds more than kWave entries, at the least
-  if (e == hipSuccess) e = hipMalloc(&d_long_raw, long_cap * sizeof(LongTile));
   if (e == hipSuccess) e = hipMalloc(&d_long_count, sizeof(int));
   if (e == hipSuccess) e = hipMalloc(&d_mid, sizeof(unsigned long long));
   if (e == hipSuccess) e = hipMalloc(&L->tval, nnz * sizeof(T));
@@ -363,8 +380,9 @@ static hipError_t build_tiled(hipStream_t stream, asamd_tiled_layout* L, const i
                             hipFuncAttributeMaxDynamicSharedMemorySize, TileDims<T>::red_lds_bytes);
   if (h_cnt) (void)hipHostFree(h_cnt);
   if (L->tile_ptr == d_tile_ptr) d_tile_ptr = nullptr;
-  for (void* d : {(void*)d_coo, (void*)d_key, (void*)d_key2, (void*)d_idx, (void*)d_perm, (void*)d_tile_ptr,
-                  (void*)d_long_raw, (void*)d_long_count, (void*)d_mid, (void*)d_cnt, (void*)d_cgb, (void*)d_rgb, (void*)d_cbs})
+  if (kPayloadSort) d_perm = nullptr;  // part of the arena
+  for (void* d : {(void*)d_arena, (void*)d_perm, (void*)d_tile_ptr, (void*)d_long_count, (void*)d_mid, (void*)d_cnt,
+                  (void*)d_cgb, (void*)d_rgb, (void*)d_cbs})
     if (d) (void)hipFree(d);
   if (e != hipSuccess) {
     asamd_tiled_free(L);
