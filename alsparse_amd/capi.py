@@ -43,7 +43,7 @@ ALPHA_SPARSE_DATATYPE_FLOAT_COMPLEX, ALPHA_SPARSE_DATATYPE_DOUBLE_COMPLEX = 2, 3
 
 # kernel families of the thin kernel ABI (include/alsparse_amd_kernels.h)
 (ASAMD_SPMV_AUTO, ASAMD_SPMV_VECTOR, ASAMD_SPMV_ROWCONST, ASAMD_SPMV_MERGE, ASAMD_SPMV_SCALAR, ASAMD_SPMV_TILED,
- ASAMD_SPMV_STREAM, ASAMD_SPMV_ELL, ASAMD_SPMV_MERGE_HOT, ASAMD_SPMV_BINNED) = range(10)
+ ASAMD_SPMV_STREAM, ASAMD_SPMV_ELL, ASAMD_SPMV_MERGE_HOT, ASAMD_SPMV_BINNED, ASAMD_SPMV_XLDS) = range(11)
 ASAMD_HIST_BINS = 33
 
 
@@ -346,6 +346,8 @@ _COMMON = {
     "asamd_value_guard": [_P, _P, c_size_t, _I, _P, _P],
     "asamd_value_guard_commit": [_P, _P, _P],
     "asamd_gather_values": [_P, _I, _I, _I, _P, _P, _P, _P],
+    "asamd_spmv_xlds": [_P, _P, _I],
+    "asamd_spmv_xlds_fits": [_I, _I],
     "asamd_csr2ell_gated": [_P, _I, _I, _P, _P, _P, _I, _I, _I, _P, _P, _P],
     "asamd_csr_plan_build_transpose": [_P, _P, _P, _P, _P],
     "asamd_csr_plan_set_lazy_transpose": [_P, _I],
@@ -396,7 +398,8 @@ _RESTYPE = {"alpha_set_thread_num": None, "alpha_timing_wtime": c_double, "alpha
 ALGO_NAMES = {ASAMD_SPMV_AUTO: "auto", ASAMD_SPMV_VECTOR: "vector", ASAMD_SPMV_ROWCONST: "rowconst",
               ASAMD_SPMV_MERGE: "merge-path", ASAMD_SPMV_SCALAR: "scalar", ASAMD_SPMV_TILED: "tiled two-phase",
               ASAMD_SPMV_STREAM: "row-block stream", ASAMD_SPMV_ELL: "ell copy",
-              ASAMD_SPMV_MERGE_HOT: "merge-path, hot columns in LDS", ASAMD_SPMV_BINNED: "row-length bins"}
+              ASAMD_SPMV_MERGE_HOT: "merge-path, hot columns in LDS", ASAMD_SPMV_BINNED: "row-length bins",
+              ASAMD_SPMV_XLDS: "x in LDS"}
 
 _lib = None
 

@@ -1,0 +1,159 @@
+// CSR SpMV for matrices with so few columns that x fits the LDS of a compute unit (gfx950: 160 KB; wave64).
+//
+// The row kernels gather x from the caches: x[col] for 64 scattered columns is up to 64 cache-line requests per
+// instruction, and with an x of a hundred KB, far larger than the 32 KB L1, nearly every one goes on to the L2 --
+// a tall matrix (millions of rows, tens of thousands of columns, sixteen entries per row) then runs at a quarter
+// of the memory's speed while its streams would allow three times that.  Here every compute unit holds ONE
+// workgroup of 1 024 threads that copies x into LDS once and then walks its share of the rows, W lanes per row,
+// gathering from LDS; the CSR arrays are read in place, so nothing is kept between calls and a caller's new values
+// are seen by the next multiply.  The reference's kernel (src/kernel/dcu/level2/mv/csrmv/dcu_gemv_vector.h:14-57)
+// has the same row-to-lanes mapping and gathers from global memory.
+//
+// A lane group takes kXldsRows rows per trip (rows r, r + groups, r + 2 groups, ...: the groups of a wave sit on
+// adjacent rows, whose entries are adjacent in memory), all their first loads in flight together: with one
+// workgroup per compute unit the loads in flight per lane are what hides the memory's latency.  Rows of more
+// than kXldsWaveRow * W entries are left to the whole wave, one after the other, 64 lanes and four entries per
+// lane and trip.  Every row's sum is formed in an order that depends on W and the row alone.
+//
+// Measured (4 194 304 rows x 16 entries, fp32): 0.19 ms whatever the number of columns, where the row kernels take
+// 0.20 / 0.25 / 0.29 ms with 32 / 64 / 128 KB of x (fp64, 128 KB of x: 0.23 against 0.37 ms).  What it waits for is
+// the memory pipeline (three quarters of the L1s' busy cycles are stalls on pending lines): two workgroups per
+// compute unit where x leaves room changed nothing, nor did twelve rows per group and trip.  Two forms that
+// stream the matrix 16 bytes per lane through a staging area in LDS (a workgroup's, with two barriers per trip;
+// a wave's own, without) measured 0.25 and 0.21 ms and were dropped.
+#pragma once
+#include "device_utils.hpp"
+
+namespace asamd {
+
+constexpr int kXldsThreads = 1024;
+constexpr int kXldsRows = 8;      // rows per lane group and trip
+constexpr int kXldsWaveRow = 8;   // rows of more than this many entries per lane go to the wave
+
+// NT: the first entries of the rows are loaded non-temporally (rows of at most W entries on average: every line
+// of the streams is then wanted once; with longer rows the lines that the tails share with the next rows' heads
+// would be fetched twice -- 33 entries per row: 0.34 against 0.26 ms).
+template <typename T, int W, bool NT>
+__global__ __launch_bounds__(kXldsThreads) void spmv_xlds_kernel(int m, int n, T alpha, const T* __restrict__ val,
+                                                                 const int* __restrict__ row_ptr,
+                                                                 const int* __restrict__ col_ind,
+                                                                 const T* __restrict__ x, T beta, T* __restrict__ y,
+                                                                 int base) {
+  extern __shared__ __align__(16) unsigned char xlds_bytes[];
+  T* __restrict__ xs = reinterpret_cast<T*>(xlds_bytes);
+  constexpr int kGroups = kXldsThreads / W;
+  constexpr int K = kXldsRows;
+  const int lane = threadIdx.x % W;
+  const int group = threadIdx.x / W;
+  const int wave_lane = threadIdx.x % kWave;
+  const int64_t stride = (int64_t)gridDim.x * (kGroups * K);
+  int64_t row0 = (int64_t)blockIdx.x * (kGroups * K);
+  // the offsets of a trip's rows are requested one trip ahead (the first ones in front of the copy of x)
+  int start[K], end[K];
+  auto request_offsets = [&](int64_t first, int* lo, int* hi) __attribute__((always_inline)) {
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      // (rows past the last: the offset behind the last row, twice -- an empty row.  No load under a condition:
+      // with loads in branches the compiler does not know how many are pending, and waits for all of them
+      // wherever it waits for one.)
+      const int64_t r = first + (int64_t)k * kGroups + group;
+      lo[k] = row_ptr[r < m ? r : m];
+      hi[k] = row_ptr[r < m ? r + 1 : m];
+    }
+  };
+  request_offsets(row0, start, end);
+  // x into LDS: 16 bytes per lane and load where x allows, a trip's loads all requested before the first is stored
+  if ((reinterpret_cast<uintptr_t>(x) & 15u) == 0) {
+    typedef Int4 Wide;  // (16 bytes of x, whatever they hold)
+    constexpr int kPer = 16 / (int)sizeof(T);
+    const int wide_n = n / kPer;
+    constexpr int kAhead = 4;
+    int i = threadIdx.x;
+    for (; i + (kAhead - 1) * kXldsThreads < wide_n; i += kAhead * kXldsThreads) {
+      Wide w[kAhead];
+#pragma unroll
+      for (int u = 0; u < kAhead; ++u) w[u] = reinterpret_cast<const Wide*>(x)[i + u * kXldsThreads];
+#pragma unroll
+      for (int u = 0; u < kAhead; ++u) reinterpret_cast<Wide*>(xs)[i + u * kXldsThreads] = w[u];
+    }
+    for (; i < wide_n; i += kXldsThreads) reinterpret_cast<Wide*>(xs)[i] = reinterpret_cast<const Wide*>(x)[i];
+    for (int t = wide_n * kPer + threadIdx.x; t < n; t += kXldsThreads) xs[t] = x[t];
+  } else {
+    for (int i = threadIdx.x; i < n; i += kXldsThreads) xs[i] = x[i];
+  }
+  __syncthreads();
+  const T* __restrict__ xb = xs - base;  // (indexed with the caller's column numbers)
+  for (; row0 < m; row0 += stride) {
+    // (a wave's memory operations complete in the order of their issue as far as its wait counter goes: entries
+    // requested a trip ahead would be waited for with the first wait of this trip.  The offsets are waited for
+    // at the top of the next trip, where nothing else is pending.)
+    int next_start[K], next_end[K];
+    request_offsets(row0 + stride, next_start, next_end);
+    T sum[K];
+    // ---- first entry of every lane in all K rows, requested together ----
+    int c[K];
+    T v[K];
+    bool mine[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      start[k] -= base;
+      end[k] -= base;
+      const bool wave_row = end[k] - start[k] > kXldsWaveRow * W;
+      const int j = start[k] + lane;
+      mine[k] = j < end[k] && !wave_row;
+      // (entry 0 exists: the launcher turns empty matrices away)
+      c[k] = NT ? nt_load(col_ind + (mine[k] ? j : 0)) : col_ind[mine[k] ? j : 0];
+      v[k] = NT ? nt_load(val + (mine[k] ? j : 0)) : val[mine[k] ? j : 0];
+    }
+#pragma unroll
+    for (int k = 0; k < K; ++k) sum[k] = mine[k] ? v[k] * xb[c[k]] : T(0);
+    // ---- the rest of rows longer than W, up to kXldsWaveRow entries per lane ----
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      if (end[k] - start[k] > kXldsWaveRow * W) continue;
+      for (int j = start[k] + lane + W; j < end[k]; j += W) sum[k] = fma_t(val[j], xb[col_ind[j]], sum[k]);
+    }
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      sum[k] = group_sum<W>(sum[k]);
+      const int64_t r = row0 + (int64_t)k * kGroups + group;
+      if (lane == 0 && r < m && end[k] - start[k] <= kXldsWaveRow * W) store_axpby(y, r, alpha, sum[k], beta);
+    }
+    // ---- long rows: the wave takes them one at a time ----
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      unsigned long long todo = __ballot(lane == 0 && end[k] - start[k] > kXldsWaveRow * W);
+      while (todo) {
+        const int owner = __builtin_ctzll(todo);  // a group's first lane
+        todo &= todo - 1;
+        const int s = __builtin_amdgcn_readlane(start[k], owner), e = __builtin_amdgcn_readlane(end[k], owner);
+        T acc = T(0);
+        int j = s + wave_lane;
+        for (; j + 3 * kWave < e; j += 4 * kWave) {
+          T vv[4];
+          int cc[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            vv[u] = val[j + u * kWave];
+            cc[u] = col_ind[j + u * kWave];
+          }
+#pragma unroll
+          for (int u = 0; u < 4; ++u) acc = fma_t(vv[u], xb[cc[u]], acc);
+        }
+        for (; j < e; j += kWave) acc = fma_t(val[j], xb[col_ind[j]], acc);
+        acc = group_sum<kWave>(acc);
+        if (wave_lane == 0) {
+          const int64_t r = row0 + (int64_t)k * kGroups + (threadIdx.x / kWave) * (kWave / W) + owner / W;
+          store_axpby(y, r, alpha, acc, beta);
+        }
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      start[k] = next_start[k];
+      end[k] = next_end[k];
+    }
+  }
+}
+
+}  // namespace asamd

@@ -207,6 +207,7 @@ int asamd_env_algo(void) {
   if (!strcmp(e, "ell")) return ASAMD_SPMV_ELL;
   if (!strcmp(e, "hot")) return ASAMD_SPMV_MERGE_HOT;
   if (!strcmp(e, "binned")) return ASAMD_SPMV_BINNED;
+  if (!strcmp(e, "xlds")) return ASAMD_SPMV_XLDS;
   return ASAMD_SPMV_AUTO;
 }
 

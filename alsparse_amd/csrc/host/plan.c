@@ -22,6 +22,7 @@ struct asamd_csr_plan {
   asamd_csr_stats st;
   int auto_algo;           /* the analysis' choice */
   int struct_algo;         /* the choice from the row statistics alone (no copy involved) */
+  int plain_algo;          /* ... before x in LDS was considered */
   int auto_width;
   int dtype;               /* ASAMD_DTYPE_*: element type of the values */
   int val_size;            /* bytes per value */
@@ -113,6 +114,16 @@ static int stream_group(const asamd_csr_plan *p, int regular_only) {
 }
 static int stream_ok(const asamd_csr_plan *p) { return stream_group(p, 0) > 0; }
 
+/* x in LDS: for an x that the L1 (32 KB) does not hold and the LDS does, on matrices large enough for 256
+ * persistent workgroups.  4 M x 16 entries, fp32: rowconst 0.20 / 0.25 / 0.29 ms with 32 / 64 / 128 KB of x, this kernel
+ * 0.19 ms whatever x; fp64 with 128 KB of x 0.37 against 0.23 ms.  ALSPARSE_AMD_XLDS=0 leaves it out. */
+static int xlds_ok(const asamd_csr_plan *p) {
+  const asamd_csr_stats *st = &p->st;
+  const int64_t x_bytes = (int64_t)st->n * (int64_t)p->val_size;
+  return st->first_offset == 0 && st->m >= 1 && st->nnz >= (1 << 22) && x_bytes > (48 << 10) &&
+         asamd_spmv_xlds_fits(p->dtype, st->n) && env_int("ALSPARSE_AMD_XLDS", 1) > 0;
+}
+
 static void choose_algo(asamd_csr_plan *p) {
   asamd_csr_stats *st = &p->st;
   const double mean = st->m > 0 ? (double)st->nnz / st->m : 0.0;
@@ -138,6 +149,8 @@ static void choose_algo(asamd_csr_plan *p) {
   } else {
     p->auto_algo = ASAMD_SPMV_MERGE;
   }
+  p->plain_algo = p->auto_algo;
+  if (xlds_ok(p)) p->auto_algo = ASAMD_SPMV_XLDS;
   p->struct_algo = p->auto_algo;
   st->algo = p->auto_algo;
   st->vector_width = p->auto_width;
@@ -406,6 +419,9 @@ static int settle_algo(const asamd_csr_plan *p, int algo, const void *val, const
     else if (algo == ASAMD_SPMV_ELL && !st->ell_built) next = p->auto_algo == ASAMD_SPMV_ELL ? p->struct_algo : p->auto_algo;
     else if (algo == ASAMD_SPMV_MERGE_HOT && !st->hot_built) next = ASAMD_SPMV_MERGE;
     else if (algo == ASAMD_SPMV_BINNED && !st->binned_built) next = ASAMD_SPMV_MERGE;
+    else if (algo == ASAMD_SPMV_XLDS &&
+             (!asamd_spmv_xlds_fits(p->dtype, st->n) || st->first_offset != 0 || st->nnz < 1 || st->m < 1))
+      next = ASAMD_SPMV_VECTOR;
     else if (algo == ASAMD_SPMV_ROWCONST &&
              (!rowconst_ok(p) || (((uintptr_t)val | (uintptr_t)ci) & 15u) != 0)) /* 128-bit loads */
       next = ASAMD_SPMV_VECTOR;
@@ -436,6 +452,8 @@ static int run_algo(hipStream_t s, const asamd_csr_plan *p, int algo, const asam
       return asamd_spmv_stream(s, a, stream_group(p, 0), st->max_len, st->first_offset);
     case ASAMD_SPMV_SCALAR:
       return asamd_spmv_scalar(s, a);
+    case ASAMD_SPMV_XLDS:
+      return asamd_spmv_xlds(s, a, p->auto_width);
     case ASAMD_SPMV_BINNED: {
       void *partial = p->binned.chunks > 0 ? ws_take(&ws, (size_t)p->binned.chunks * vs) : NULL;
       if (p->binned.chunks > 0 && !partial) return -1;
@@ -902,6 +920,7 @@ static double model_ms(const asamd_csr_plan *p, int algo) {
     case ASAMD_SPMV_STREAM: rate = stream_group(p, 0) > 1 ? 5.2 : 6.6; break;
     case ASAMD_SPMV_VECTOR: rate = 2.4 * vector_utilisation(st, p->auto_width); break;
     case ASAMD_SPMV_MERGE: rate = 2.9; break;
+    case ASAMD_SPMV_XLDS: return nnz * (2.1 + 0.175 * vs) * 1e-9; /* measured: 2.8 ps per fp32 entry, 3.5 per fp64 */
     case ASAMD_SPMV_ELL: {
       const double ell_bytes = m * (double)st->max_len * (4.0 + vs) + (n + m) * vs;
       return hypot2(ell_bytes / 6.1e9, gather);
@@ -925,6 +944,14 @@ static hipError_t model_copies(hipStream_t stream, asamd_csr_plan *p, const int3
   asamd_csr_stats *st = &p->st;
   if (st->lines_per_entry_wave <= 0.f) return hipSuccess; /* not probed (a tiny matrix): the structural choice stays */
   double base = model_ms(p, p->auto_algo);
+  if (p->auto_algo == ASAMD_SPMV_XLDS) {
+    /* columns that neighbouring entries share are cheap to gather from the caches too */
+    const double plain = model_ms(p, p->plain_algo);
+    if (base > 0.95 * plain) {
+      p->auto_algo = p->struct_algo = p->plain_algo;
+      base = plain;
+    }
+  }
   if (structural_alternatives(p)) {
     const int alts[2] = {ASAMD_SPMV_MERGE, p->auto_algo == ASAMD_SPMV_STREAM ? ASAMD_SPMV_VECTOR : -1};
     for (int i = 0; i < 2; ++i) {
@@ -1112,7 +1139,8 @@ static hipError_t plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t 
       if (e == hipSuccess && tiled_ok) e = build_tiled(stream, p, row_ptr, col_ind, val);
       if (e == hipSuccess && ell_ok) e = build_ell(stream, p, row_ptr, col_ind, val);
       if (e == hipSuccess && hot_ok) e = build_hot(stream, p, row_ptr, col_ind, 1);
-    } else if (tiled_ok || ell_ok || hot_ok || binned_ok || structural_alternatives(p)) {
+    } else if (tiled_ok || ell_ok || hot_ok || binned_ok || structural_alternatives(p) ||
+               p->auto_algo == ASAMD_SPMV_XLDS) {
       e = st->tune_mode ? model_copies(stream, p, row_ptr, col_ind, val, tiled_ok, ell_ok, hot_ok, binned_ok)
                         : tune_copies(stream, p, row_ptr, col_ind, val, tiled_ok, ell_ok, hot_ok, binned_ok);
     }
@@ -1282,6 +1310,9 @@ int asamd_csr_plan_set_algo(asamd_csr_plan *p, int32_t algo) {
       break;
     case ASAMD_SPMV_MERGE:
       if (p->st.first_offset != 0) return hipErrorInvalidValue;
+      break;
+    case ASAMD_SPMV_XLDS:
+      if (!asamd_spmv_xlds_fits(p->dtype, p->st.n) || p->st.first_offset != 0) return hipErrorInvalidValue;
       break;
     case ASAMD_SPMV_VECTOR:
     case ASAMD_SPMV_SCALAR:

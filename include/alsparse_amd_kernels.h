@@ -42,9 +42,11 @@ enum asamd_spmv_algo {
   ASAMD_SPMV_MERGE_HOT = 8, /* merge-path whose persistent workgroups keep x of the most
                               popular columns in LDS (power-law graphs); the copy it
                               needs is structure only: values come from the caller  */
-  ASAMD_SPMV_BINNED = 9    /* one launch per row-length class (4, 16, 64 lanes per row;
+  ASAMD_SPMV_BINNED = 9,   /* one launch per row-length class (4, 16, 64 lanes per row;
                               the longest rows in chunks, a workgroup each): for very
                               uneven rows; keeps a list of row numbers, no values   */
+  ASAMD_SPMV_XLDS = 10     /* W lanes per row with x held in every compute unit's LDS:
+                              matrices of few columns (x <= 128 KB); keeps nothing  */
 };
 
 #define ASAMD_HIST_BINS 33
@@ -93,6 +95,11 @@ int asamd_spmv_vector(hipStream_t stream, const asamd_spmv_args *a, int32_t widt
 /* the same, launched whatever happens but returning at once unless the device word *run_if is non-zero
  * (NULL: always runs): the stand-in for a kernel that a device-side guard may turn away */
 int asamd_spmv_vector_if(hipStream_t stream, const asamd_spmv_args *a, int32_t width, const int32_t *run_if);
+/* x held in the LDS of every compute unit (one workgroup of 1 024 threads each), `width` lanes per row: for
+ * matrices whose x is at most ASAMD_XLDS_MAX_BYTES (asamd_spmv_xlds_fits); reads the CSR arrays in place. */
+#define ASAMD_XLDS_MAX_BYTES 131072
+int asamd_spmv_xlds_fits(int32_t dtype, int32_t n);
+int asamd_spmv_xlds(hipStream_t stream, const asamd_spmv_args *a, int32_t width);
 /* One lane per row, entries in storage order (src/plain/kernel/level2/mv/gemv/gemv_x_csr_plain.c:11-22). */
 int asamd_spmv_scalar(hipStream_t stream, const asamd_spmv_args *a);
 /* Every row has row_len entries (4, 8, ..., 256): no row_ptr traffic.  Real element types, row_ptr[0] ==

@@ -13,7 +13,8 @@ TOL = {np.dtype(np.float32): 1e-4, np.dtype(np.float64): 1e-12}
 
 ALGOS = {"auto": capi.ASAMD_SPMV_AUTO, "vector": capi.ASAMD_SPMV_VECTOR, "rowconst": capi.ASAMD_SPMV_ROWCONST,
          "merge": capi.ASAMD_SPMV_MERGE, "scalar": capi.ASAMD_SPMV_SCALAR, "tiled": capi.ASAMD_SPMV_TILED,
-         "stream": capi.ASAMD_SPMV_STREAM, "ell": capi.ASAMD_SPMV_ELL, "hot": capi.ASAMD_SPMV_MERGE_HOT, "binned": capi.ASAMD_SPMV_BINNED}
+         "stream": capi.ASAMD_SPMV_STREAM, "ell": capi.ASAMD_SPMV_ELL, "hot": capi.ASAMD_SPMV_MERGE_HOT, "binned": capi.ASAMD_SPMV_BINNED,
+         "xlds": capi.ASAMD_SPMV_XLDS}
 
 
 def announce(*what):
@@ -88,7 +89,7 @@ def run_plan_csrmv(da, algo, alpha, x, beta, y0, trusted=1):
     try:
         e = lib.asamd_csr_plan_set_algo(plan, ALGOS[algo])
         if e != 0:
-            assert algo in ("rowconst", "stream", "ell", "hot"), algo
+            assert algo in ("rowconst", "stream", "ell", "hot", "xlds"), algo
             return None  # this structure cannot run that family
         T = capi.scalar_type(a.dtype)
         dx = hiprt.DeviceArray.from_numpy(np.ascontiguousarray(x, dtype=a.dtype))

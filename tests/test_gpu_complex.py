@@ -117,7 +117,7 @@ def test_complex_csrmv_with_and_without_analysis(gpu, dtype, shape, op):
         da.free()
 
 
-@pytest.mark.parametrize("algo", ["vector", "merge", "scalar", "stream", "ell", "rowconst", "tiled", "hot", "binned"])
+@pytest.mark.parametrize("algo", ["vector", "merge", "scalar", "stream", "ell", "rowconst", "tiled", "hot", "binned", "xlds"])
 @pytest.mark.parametrize("dtype", CX, ids=IDS)
 def test_complex_kernel_families(gpu, dtype, algo):
     """The thin kernel ABI with a forced family; the constant-row-length family (128-bit quads of
@@ -135,7 +135,7 @@ def test_complex_kernel_families(gpu, dtype, algo):
                                                da.val.c_ptr(), a.base, capi.dtype_tag(dtype), 2, byref(plan)) == 0
         try:
             if lib.asamd_csr_plan_set_algo(plan, ALGOS[algo]) != 0:
-                assert algo in ("rowconst", "stream", "ell", "hot"), (algo, shape)
+                assert algo in ("rowconst", "stream", "ell", "hot", "xlds"), (algo, shape)
                 continue
             assert algo != "rowconst"
             ws = capi.Workspace(lib, plan)

@@ -95,6 +95,7 @@ def test_analysed_csrmv_replays_from_a_hip_graph(gpu, shape):
 
 CAPTURE_CASES = [(algo, "uniform") for algo in ("vector", "rowconst", "merge", "scalar", "tiled", "stream", "ell", "hot",
                                                 "binned")]
+CAPTURE_CASES += [("xlds", "narrow")]  # x must fit the LDS: 20 000 columns
 # heavy-tailed rows: the tiled copy's third phase, the bins' chunked long rows, merge blocks inside one row
 CAPTURE_CASES += [(algo, "powerlaw") for algo in ("merge", "tiled", "hot", "binned")]
 
@@ -103,7 +104,8 @@ CAPTURE_CASES += [(algo, "powerlaw") for algo in ("merge", "tiled", "hot", "binn
 def test_every_kernel_family_replays_from_a_hip_graph(gpu, algo, shape):
     """The thin kernel ABI with a forced family, recorded on a caller's stream."""
     lib, hip = capi.load(), hiprt.lib()
-    a = wl.uniform_rows(60000, 50000, 16, np.float32) if shape == "uniform" else wl.powerlaw_rmat(15, 200000, np.float32)
+    a = (wl.uniform_rows(60000, 50000, 16, np.float32) if shape == "uniform" else
+         wl.uniform_rows(60000, 20000, 16, np.float32) if shape == "narrow" else wl.powerlaw_rmat(15, 200000, np.float32))
     x, y0 = wl.uniform(a.cols, a.dtype, 5), wl.uniform(a.rows, a.dtype, 6)
     da = DeviceCsr(a)
     dx, dy = hiprt.DeviceArray.from_numpy(x), hiprt.DeviceArray.from_numpy(y0)

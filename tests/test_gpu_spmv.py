@@ -51,7 +51,7 @@ def test_every_kernel_family_matches_oracle(gpu, shape, dtype):
     x, y0 = _vectors(a)
     da = DeviceCsr(a)
     try:
-        for algo in ("vector", "merge", "scalar", "rowconst", "stream", "tiled", "ell", "hot", "binned", "auto"):
+        for algo in ("vector", "merge", "scalar", "rowconst", "stream", "tiled", "ell", "hot", "binned", "xlds", "auto"):
             for alpha, beta in ((1.0, 0.0), (2.0, 3.0), (-0.75, 1.0)):
                 announce("spmv", shape, np.dtype(dtype).name, algo, alpha, beta)
                 y = run_plan_csrmv(da, algo, alpha, x, beta, y0)
@@ -96,7 +96,7 @@ def test_random_structures_every_family(gpu, seed, dtype):
     x, y0 = _vectors(a)
     da = DeviceCsr(a, shift=shift)
     try:
-        for algo in ("vector", "merge", "scalar", "rowconst", "stream", "tiled", "ell", "binned", "auto"):
+        for algo in ("vector", "merge", "scalar", "rowconst", "stream", "tiled", "ell", "binned", "xlds", "auto"):
             alpha, beta = ((1.0, 0.0), (2.0, 3.0), (-0.75, 1.0))[int(rng.integers(0, 3))]
             announce("spmv random structure", seed, a.name, "base", a.base, "shift", shift, np.dtype(dtype).name, algo, alpha, beta)
             y = run_plan_csrmv(da, algo, alpha, x, beta, y0)
@@ -120,7 +120,7 @@ def test_streams_off_16_byte_alignment(gpu, dtype, shift):
         x, y0 = _vectors(a)
         da = DeviceCsr(a, shift=shift)
         try:
-            for algo in ("vector", "merge", "rowconst", "stream", "binned", "auto"):
+            for algo in ("vector", "merge", "rowconst", "stream", "binned", "xlds", "auto"):
                 announce("spmv shifted streams", a.name, np.dtype(dtype).name, algo, shift)
                 y = run_plan_csrmv(da, algo, 1.5, x, 0.25, y0)
                 if y is None:
@@ -140,7 +140,7 @@ def test_index_base_one(gpu, dtype):
         x, y0 = _vectors(a)
         da = DeviceCsr(a)
         try:
-            for algo in ("vector", "merge", "scalar", "stream", "tiled", "ell", "hot", "binned", "auto"):
+            for algo in ("vector", "merge", "scalar", "stream", "tiled", "ell", "hot", "binned", "xlds", "auto"):
                 announce("spmv base1", a.name, algo)
                 y = run_plan_csrmv(da, algo, 1.5, x, 0.25, y0)
                 if y is None:
@@ -160,7 +160,7 @@ def test_beta_zero_ignores_nan_in_y(gpu):
     y0 = np.full(a.rows, np.nan, dtype=np.float32)
     da = DeviceCsr(a)
     try:
-        for algo in ("vector", "merge", "scalar", "tiled", "hot", "binned"):
+        for algo in ("vector", "merge", "scalar", "tiled", "hot", "binned", "xlds"):
             announce("spmv beta0 nan", algo)
             y = run_plan_csrmv(da, algo, 1.0, x, 0.0, y0)
             assert np.isfinite(y).all()
@@ -197,7 +197,7 @@ def test_deterministic_across_runs(gpu):
     try:
         # the families that sum every row in a fixed order (no floating-point atomics)
         # (the tiled copy of this matrix has tiles too long for its second phase: the third phase runs)
-        for algo in ("merge", "hot", "binned", "vector", "tiled"):
+        for algo in ("merge", "hot", "binned", "vector", "tiled", "xlds"):
             announce("spmv determinism", algo)
             runs = [run_plan_csrmv(da, algo, 1.0, x, 0.5, y0) for _ in range(3)]
             assert np.array_equal(runs[0], runs[1]) and np.array_equal(runs[0], runs[2]), algo
@@ -356,7 +356,7 @@ def test_random_structures_every_family(gpu, seed):
     x, y0 = _vectors(a, seed)
     da = DeviceCsr(a)
     try:
-        for algo in ("vector", "merge", "scalar", "rowconst", "stream", "tiled", "ell", "hot", "binned", "auto"):
+        for algo in ("vector", "merge", "scalar", "rowconst", "stream", "tiled", "ell", "hot", "binned", "xlds", "auto"):
             for alpha, beta in ((1.5, 0.0), (-2.0, 0.5)):
                 announce("spmv random", seed, m, n, a.nnz, np.dtype(dtype).name, base, algo, alpha, beta)
                 y = run_plan_csrmv(da, algo, alpha, x, beta, y0)
@@ -386,7 +386,7 @@ def test_unsorted_and_duplicate_columns_and_non_finite_values(gpu, dtype):
     x, y0 = _vectors(a, 5)
     da = DeviceCsr(a)
     try:
-        for algo in ("vector", "merge", "scalar", "stream", "tiled", "ell", "hot", "binned", "auto"):
+        for algo in ("vector", "merge", "scalar", "stream", "tiled", "ell", "hot", "binned", "xlds", "auto"):
             announce("spmv unsorted", np.dtype(dtype).name, algo)
             y = run_plan_csrmv(da, algo, 1.5, x, 0.5, y0)
             if y is not None:
@@ -406,7 +406,7 @@ def test_unsorted_and_duplicate_columns_and_non_finite_values(gpu, dtype):
         ref = orc.csrmv_plain(b, 1.0, x2, 0.0, y0)
     db = DeviceCsr(b)
     try:
-        for algo in ("vector", "merge", "scalar", "tiled", "hot", "binned", "auto"):
+        for algo in ("vector", "merge", "scalar", "tiled", "hot", "binned", "xlds", "auto"):
             announce("spmv non-finite", np.dtype(dtype).name, algo)
             y = run_plan_csrmv(db, algo, 1.0, x2, 0.0, y0)
             assert np.array_equal(np.isnan(y), np.isnan(ref)), algo

@@ -1,0 +1,86 @@
+"""Matrices of few columns: x larger than the 32 KB L1 and small enough for a compute unit's LDS (128 KB at most).
+The library then multiplies with one persistent workgroup per compute unit that holds x in LDS and reads the CSR
+arrays in place -- with or without an analysis, since nothing is kept.  The reference has one kernel for every
+shape (src/kernel/dcu/level2/mv/csrmv/dcu_gemv_vector.h:14-57); results are compared with the CPU oracle."""
+from ctypes import byref, c_void_p
+
+import numpy as np
+import pytest
+
+from alsparse_amd import capi, hiprt, workloads as wl
+from helpers import DeviceCsr, announce, check_spmv, run_csrmv
+from helpers_shapes import csr_from_lengths
+
+pytestmark = pytest.mark.gpu
+
+
+def _plan_algo(lib, da, trusted=1):
+    a = da.a
+    plan = c_void_p()
+    assert lib.asamd_csr_plan_create(None, a.rows, a.cols, a.nnz, da.row_ptr.c_ptr(), da.col.c_ptr(), da.val.c_ptr(),
+                                     a.base, a.dtype.itemsize, trusted, byref(plan)) == 0
+    algo = lib.asamd_csr_plan_stats(plan).contents.algo
+    lib.asamd_csr_plan_destroy(plan)
+    return algo
+
+
+@pytest.mark.parametrize("dtype,cols", [(np.float32, 20000), (np.float32, 32768), (np.float64, 16384)],
+                         ids=["f32_20000", "f32_32768", "f64_16384"])
+def test_tall_matrix_is_multiplied_with_x_in_lds(gpu, dtype, cols, monkeypatch):
+    lib = capi.load()
+    a = wl.uniform_rows(300000, cols, 16, dtype)  # 4.8 M entries, scattered columns
+    x, y0 = wl.uniform(a.cols, a.dtype, 3), wl.uniform(a.rows, a.dtype, 4)
+    da = DeviceCsr(a)
+    try:
+        announce("x in LDS: the analysis' choice", np.dtype(dtype).name, cols)
+        assert _plan_algo(lib, da) == capi.ASAMD_SPMV_XLDS
+        monkeypatch.setenv("ALSPARSE_AMD_XLDS", "0")
+        assert _plan_algo(lib, da) != capi.ASAMD_SPMV_XLDS
+        monkeypatch.delenv("ALSPARSE_AMD_XLDS")
+        announce("x in LDS: multiply without analysis", np.dtype(dtype).name, cols)
+        for alpha, beta in ((1.0, 0.0), (-0.5, 2.0)):
+            y = run_csrmv(gpu, da, alpha, x, beta, y0)
+            check_spmv(a, alpha, x, beta, y0, y, "no analysis %s" % ((alpha, beta),))
+        assert lib.asamd_analysis_stats(da.row_ptr.c_ptr()).contents.algo == capi.ASAMD_SPMV_XLDS
+    finally:
+        da.free()
+
+
+def test_columns_that_neighbours_share_keep_the_plain_kernel(gpu):
+    """A band: the gathers of a wave fall into a few cache lines, and the row kernels are as fast from the caches."""
+    lib = capi.load()
+    m, n, per_row = 300000, 30000, 16
+    rows = np.repeat(np.arange(m, dtype=np.int64), per_row)
+    cols = (rows * n // m + np.tile(np.arange(per_row, dtype=np.int64), m)) % n
+    order = np.lexsort((cols, rows))
+    a = wl.Csr(m, n, np.arange(0, m * per_row + 1, per_row, dtype=np.int32), cols[order].astype(np.int32),
+               wl.uniform(m * per_row, np.float32, 9), 0, "band")
+    da = DeviceCsr(a)
+    try:
+        announce("x in LDS: a banded matrix keeps its row kernel")
+        assert _plan_algo(lib, da) != capi.ASAMD_SPMV_XLDS
+    finally:
+        da.free()
+
+
+def test_rows_of_every_length_and_both_bases(gpu):
+    """Rows for the lane groups, rows for the whole wave (more than eight entries per lane), empty rows, a last
+    trip that ends inside the matrix, index base one; the family forced on a matrix below its size threshold."""
+    from helpers import run_plan_csrmv
+    rng = np.random.default_rng(77)
+    lengths = rng.integers(0, 40, size=9000)
+    lengths[rng.integers(0, 9000, size=60)] = rng.integers(129, 6000, size=60)
+    lengths[:17] = [0, 1, 127, 128, 129, 5999, 0, 0, 64, 65, 1023, 1024, 1025, 16, 17, 15, 6000]
+    for dtype in (np.float32, np.float64):
+        for base in (0, 1):
+            a = csr_from_lengths(list(lengths), 6000, dtype, seed=5 + base, base=base)
+            x, y0 = wl.uniform(a.cols, a.dtype, 3), wl.uniform(a.rows, a.dtype, 4)
+            da = DeviceCsr(a)
+            try:
+                for alpha, beta in ((1.0, 0.0), (2.0, -1.0)):
+                    announce("x in LDS: ragged rows", np.dtype(dtype).name, "base", base, alpha, beta)
+                    y = run_plan_csrmv(da, "xlds", alpha, x, beta, y0)
+                    assert y is not None
+                    check_spmv(a, alpha, x, beta, y0, y, "ragged base %d %s" % (base, (alpha, beta)))
+            finally:
+                da.free()
