@@ -97,12 +97,58 @@ static int launch_xlds(hipStream_t s, const asamd_spmv_args* a) {
   return (int64_t)a->nnz <= (int64_t)a->m * W ? launch_xlds_as<T, W, true>(s, a) : launch_xlds_as<T, W, false>(s, a);
 }
 
+// four entries per lane and load: W lanes take the first 4 W entries of a row
+template <typename T, int W, bool NT>
+static int launch_xlds4_as(hipStream_t s, const asamd_spmv_args* a) {
+  static const int cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    return n;
+  }();
+  const size_t lds = ((size_t)a->n * sizeof(T) + 15) / 16 * 16;
+  static size_t allowed = 0;  // (per instantiation)
+  if (lds > allowed) {
+    const hipError_t e = hipFuncSetAttribute((const void*)spmv_xlds4_kernel<T, W, NT>,
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, ASAMD_XLDS_MAX_BYTES);
+    if (e != hipSuccess) return e;
+    allowed = ASAMD_XLDS_MAX_BYTES;
+  }
+  constexpr int rows_per_trip = (kXldsThreads / W) * kXlds4Rows;
+  int64_t grid = ((int64_t)a->m + rows_per_trip - 1) / rows_per_trip;
+  if (grid > cus) grid = cus;
+  spmv_xlds4_kernel<T, W, NT><<<(unsigned)grid, kXldsThreads, lds, s>>>(
+      a->m, a->n, (int64_t)a->nnz, scalar_of<T>(a->alpha), (const T*)a->val, a->row_ptr, a->col_ind, (const T*)a->x,
+      scalar_of<T>(a->beta), (T*)a->y, a->base);
+  return hipGetLastError();
+}
+template <typename T, int W>
+static int launch_xlds4(hipStream_t s, const asamd_spmv_args* a) {
+  return (int64_t)a->nnz <= (int64_t)a->m * 4 * W ? launch_xlds4_as<T, W, true>(s, a) : launch_xlds4_as<T, W, false>(s, a);
+}
+
 extern "C" int asamd_spmv_xlds(hipStream_t s, const asamd_spmv_args* a, int32_t width) {
   if (!a) return hipErrorInvalidValue;
   if (!asamd_spmv_xlds_fits(a->dtype, a->n) || a->nnz < 1 || a->m < 1) return hipErrorInvalidValue;
   return by_dtype(a->dtype, [&](auto* tag) -> int {
     using T = std::remove_pointer_t<decltype(tag)>;
     if (!args_ok<T>(a)) return hipErrorInvalidValue;
+    if constexpr (kIsReal<T>) {
+      // rows of four entries or more on average, at least four entries in the arrays: 16-byte loads, `width` / 4 lanes
+      static const bool narrow_only = getenv("ALSPARSE_AMD_XLDS_WIDE") && atoi(getenv("ALSPARSE_AMD_XLDS_WIDE")) == 0;
+      if (!narrow_only && a->nnz >= 4 && (int64_t)a->nnz >= 4 * (int64_t)a->m) {
+        switch (width) {
+          case 2:
+          case 4: return launch_xlds4<T, 1>(s, a);
+          case 8: return launch_xlds4<T, 2>(s, a);
+          case 16: return launch_xlds4<T, 4>(s, a);
+          case 32: return launch_xlds4<T, 8>(s, a);
+          case 64: return launch_xlds4<T, 16>(s, a);
+          default: return hipErrorInvalidValue;
+        }
+      }
+    }
     switch (width) {
       case 2: return launch_xlds<T, 2>(s, a);
       case 4: return launch_xlds<T, 4>(s, a);

@@ -15,12 +15,14 @@
 // than kXldsWaveRow * W entries are left to the whole wave, one after the other, 64 lanes and four entries per
 // lane and trip.  Every row's sum is formed in an order that depends on W and the row alone.
 //
-// Measured (4 194 304 rows x 16 entries, fp32): 0.19 ms whatever the number of columns, where the row kernels take
-// 0.20 / 0.25 / 0.29 ms with 32 / 64 / 128 KB of x (fp64, 128 KB of x: 0.23 against 0.37 ms).  What it waits for is
-// the memory pipeline (three quarters of the L1s' busy cycles are stalls on pending lines): two workgroups per
-// compute unit where x leaves room changed nothing, nor did twelve rows per group and trip.  Two forms that
-// stream the matrix 16 bytes per lane through a staging area in LDS (a workgroup's, with two barriers per trip;
-// a wave's own, without) measured 0.25 and 0.21 ms and were dropped.
+// Measured (4 194 304 rows x 16 entries, fp32): this kernel, one entry per lane and load, 0.19 ms whatever the
+// number of columns; the form below with four entries per lane and load 0.127 ms; the row kernels 0.105 / 0.125 /
+// 0.20 / 0.25 / 0.29 ms with 4 / 16 / 32 / 64 / 128 KB of x.  What this one waits for is the memory pipeline (three
+// quarters of the L1s' busy cycles are stalls on pending lines) -- two workgroups per compute unit where x leaves
+// room changed nothing, nor did twelve rows per group and trip; fewer, wider requests did.  Two forms that stream
+// the matrix 16 bytes per lane through a staging area in LDS (a workgroup's, with two barriers per trip; a wave's
+// own, without) measured 0.25 and 0.21 ms and were dropped.  This form stays for complex values and for rows of
+// fewer than four entries on average.
 #pragma once
 #include "device_utils.hpp"
 
@@ -141,6 +143,169 @@ __global__ __launch_bounds__(kXldsThreads) void spmv_xlds_kernel(int m, int n, T
           for (int u = 0; u < 4; ++u) acc = fma_t(vv[u], xb[cc[u]], acc);
         }
         for (; j < e; j += kWave) acc = fma_t(val[j], xb[col_ind[j]], acc);
+        acc = group_sum<kWave>(acc);
+        if (wave_lane == 0) {
+          const int64_t r = row0 + (int64_t)k * kGroups + (threadIdx.x / kWave) * (kWave / W) + owner / W;
+          store_axpby(y, r, alpha, acc, beta);
+        }
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      start[k] = next_start[k];
+      end[k] = next_end[k];
+    }
+  }
+}
+
+// ---- four consecutive entries per lane and load (real element types) ----------------------------------------
+// The same walk with 16 bytes of indices and 16 (32) bytes of values per lane and load: W lanes cover the first 4 W
+// entries of a row, and a wave instruction fetches what sixteen of the loads above fetch one by one.  (Global
+// loads of 16 bytes need no more than 4-byte alignment on this hardware, so rows may start anywhere.)  A piece
+// that would reach past the arrays' end -- the last rows' lanes only -- is read as the arrays' last four entries
+// and shifted into place; no load sits under a condition.  limit: entries in the arrays, at least 4.
+constexpr int kXlds4Rows = 4;  // rows per lane group and trip
+
+template <typename T>
+struct XldsPiece {
+  int c[4];
+  T v[4];
+};
+typedef int XldsInt4 __attribute__((ext_vector_type(4), aligned(4)));
+template <typename T>
+struct XldsVal4 {
+  typedef T type __attribute__((ext_vector_type(4), aligned(4)));
+};
+
+template <typename T, bool NT>
+__device__ __forceinline__ XldsPiece<T> xlds_load_piece(const T* __restrict__ val, const int* __restrict__ col_ind,
+                                                        int64_t j, int64_t limit) {
+  // j > limit - 4: the window [limit - 4, limit) instead, its entries moved down by j - (limit - 4)
+  const int64_t at = j + 4 <= limit ? j : limit - 4;
+  const int shift = (int)(j - at);
+  typedef typename XldsVal4<T>::type V4;
+  const XldsInt4 c = NT ? __builtin_nontemporal_load(reinterpret_cast<const XldsInt4*>(col_ind + at))
+                        : *reinterpret_cast<const XldsInt4*>(col_ind + at);
+  const V4 v = NT ? __builtin_nontemporal_load(reinterpret_cast<const V4*>(val + at))
+                  : *reinterpret_cast<const V4*>(val + at);
+  XldsPiece<T> p;
+  if (shift == 0) {  // (all lanes but the matrix' last few)
+    p.c[0] = c.x, p.c[1] = c.y, p.c[2] = c.z, p.c[3] = c.w;
+    p.v[0] = v.x, p.v[1] = v.y, p.v[2] = v.z, p.v[3] = v.w;
+  } else {
+    const int cc[4] = {c.x, c.y, c.z, c.w};
+    const T vv[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      p.c[i] = cc[0];
+      p.v[i] = T(0);
+#pragma unroll
+      for (int q = 1; q < 4; ++q)
+        if (shift + i == q) p.c[i] = cc[q], p.v[i] = vv[q];  // (entries past the arrays' end: never summed)
+    }
+  }
+  return p;
+}
+
+template <typename T, int W, bool NT>
+__global__ __launch_bounds__(kXldsThreads) void spmv_xlds4_kernel(int m, int n, int64_t limit, T alpha,
+                                                                  const T* __restrict__ val,
+                                                                  const int* __restrict__ row_ptr,
+                                                                  const int* __restrict__ col_ind,
+                                                                  const T* __restrict__ x, T beta, T* __restrict__ y,
+                                                                  int base) {
+  extern __shared__ __align__(16) unsigned char xlds_bytes[];
+  T* __restrict__ xs = reinterpret_cast<T*>(xlds_bytes);
+  constexpr int kGroups = kXldsThreads / W;
+  constexpr int K = kXlds4Rows;
+  constexpr int kWaveLen = kXldsWaveRow * 4 * W;  // longer rows go to the whole wave
+  const int lane = threadIdx.x % W;
+  const int group = threadIdx.x / W;
+  const int wave_lane = threadIdx.x % kWave;
+  const int64_t stride = (int64_t)gridDim.x * (kGroups * K);
+  int64_t row0 = (int64_t)blockIdx.x * (kGroups * K);
+  int start[K], end[K];
+  auto request_offsets = [&](int64_t first, int* lo, int* hi) __attribute__((always_inline)) {
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      const int64_t r = first + (int64_t)k * kGroups + group;
+      lo[k] = row_ptr[r < m ? r : m];
+      hi[k] = row_ptr[r < m ? r + 1 : m];
+    }
+  };
+  request_offsets(row0, start, end);
+  if ((reinterpret_cast<uintptr_t>(x) & 15u) == 0) {
+    constexpr int kPer = 16 / (int)sizeof(T);
+    const int wide_n = n / kPer;
+    constexpr int kAhead = 4;
+    int i = threadIdx.x;
+    for (; i + (kAhead - 1) * kXldsThreads < wide_n; i += kAhead * kXldsThreads) {
+      Int4 w[kAhead];
+#pragma unroll
+      for (int u = 0; u < kAhead; ++u) w[u] = reinterpret_cast<const Int4*>(x)[i + u * kXldsThreads];
+#pragma unroll
+      for (int u = 0; u < kAhead; ++u) reinterpret_cast<Int4*>(xs)[i + u * kXldsThreads] = w[u];
+    }
+    for (; i < wide_n; i += kXldsThreads) reinterpret_cast<Int4*>(xs)[i] = reinterpret_cast<const Int4*>(x)[i];
+    for (int t = wide_n * kPer + threadIdx.x; t < n; t += kXldsThreads) xs[t] = x[t];
+  } else {
+    for (int i = threadIdx.x; i < n; i += kXldsThreads) xs[i] = x[i];
+  }
+  __syncthreads();
+  const T* __restrict__ xb = xs - base;
+  // the lane's (up to four) entries from position j of a row that ends at e, times x, added up
+  auto piece_sum = [&](const XldsPiece<T>& p, int j, int e, T sum) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const bool mine = j + i < e;
+      const T xv = xb[mine ? p.c[i] : base];
+      sum = mine ? fma_t(p.v[i], xv, sum) : sum;
+    }
+    return sum;
+  };
+  for (; row0 < m; row0 += stride) {
+    int next_start[K], next_end[K];
+    request_offsets(row0 + stride, next_start, next_end);
+    XldsPiece<T> p[K];
+    T sum[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      start[k] -= base;
+      end[k] -= base;
+      const int j = start[k] + 4 * lane;
+      // (a lane with nothing to do, or a row for the wave: the matrix' first piece, never summed)
+      const bool mine = j < end[k] && end[k] - start[k] <= kWaveLen;
+      p[k] = xlds_load_piece<T, NT>(val, col_ind, mine ? (int64_t)j : 0, limit);
+    }
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      const bool group_row = end[k] - start[k] <= kWaveLen;
+      sum[k] = piece_sum(p[k], start[k] + 4 * lane, group_row ? end[k] : start[k], T(0));
+    }
+    // ---- the rest of rows longer than 4 W, up to kXldsWaveRow pieces per lane ----
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      if (end[k] - start[k] > kWaveLen) continue;
+      for (int j = start[k] + 4 * lane + 4 * W; j < end[k]; j += 4 * W)
+        sum[k] = piece_sum(xlds_load_piece<T, false>(val, col_ind, j, limit), j, end[k], sum[k]);
+    }
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      sum[k] = group_sum<W>(sum[k]);
+      const int64_t r = row0 + (int64_t)k * kGroups + group;
+      if (lane == 0 && r < m && end[k] - start[k] <= kWaveLen) store_axpby(y, r, alpha, sum[k], beta);
+    }
+    // ---- long rows: the wave takes them one at a time ----
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      unsigned long long todo = __ballot(lane == 0 && end[k] - start[k] > kWaveLen);
+      while (todo) {
+        const int owner = __builtin_ctzll(todo);  // a group's first lane
+        todo &= todo - 1;
+        const int s = __builtin_amdgcn_readlane(start[k], owner), e = __builtin_amdgcn_readlane(end[k], owner);
+        T acc = T(0);
+        for (int j = s + 4 * wave_lane; j < e; j += 4 * kWave)
+          acc = piece_sum(xlds_load_piece<T, false>(val, col_ind, j, limit), j, e, acc);
         acc = group_sum<kWave>(acc);
         if (wave_lane == 0) {
           const int64_t r = row0 + (int64_t)k * kGroups + (threadIdx.x / kWave) * (kWave / W) + owner / W;

@@ -114,13 +114,13 @@ static int stream_group(const asamd_csr_plan *p, int regular_only) {
 }
 static int stream_ok(const asamd_csr_plan *p) { return stream_group(p, 0) > 0; }
 
-/* x in LDS: for an x that the L1 (32 KB) does not hold and the LDS does, on matrices large enough for 256
- * persistent workgroups.  4 M x 16 entries, fp32: rowconst 0.20 / 0.25 / 0.29 ms with 32 / 64 / 128 KB of x, this kernel
- * 0.19 ms whatever x; fp64 with 128 KB of x 0.37 against 0.23 ms.  ALSPARSE_AMD_XLDS=0 leaves it out. */
+/* x in LDS: for an x that crowds the L1 (32 KB) and fits the LDS, on matrices large enough for 256 persistent
+ * workgroups.  4 M x 16 entries, fp32: rowconst 0.105 / 0.125 / 0.20 / 0.25 / 0.29 ms with 4 / 16 / 32 / 64 / 128 KB of x,
+ * this kernel 0.127 ms whatever x; fp64 with 128 KB of x 0.37 against 0.18 ms.  ALSPARSE_AMD_XLDS=0 leaves it out. */
 static int xlds_ok(const asamd_csr_plan *p) {
   const asamd_csr_stats *st = &p->st;
   const int64_t x_bytes = (int64_t)st->n * (int64_t)p->val_size;
-  return st->first_offset == 0 && st->m >= 1 && st->nnz >= (1 << 22) && x_bytes > (48 << 10) &&
+  return st->first_offset == 0 && st->m >= 1 && st->nnz >= (1 << 22) && x_bytes > (20 << 10) &&
          asamd_spmv_xlds_fits(p->dtype, st->n) && env_int("ALSPARSE_AMD_XLDS", 1) > 0;
 }
 
@@ -920,7 +920,7 @@ static double model_ms(const asamd_csr_plan *p, int algo) {
     case ASAMD_SPMV_STREAM: rate = stream_group(p, 0) > 1 ? 5.2 : 6.6; break;
     case ASAMD_SPMV_VECTOR: rate = 2.4 * vector_utilisation(st, p->auto_width); break;
     case ASAMD_SPMV_MERGE: rate = 2.9; break;
-    case ASAMD_SPMV_XLDS: return nnz * (2.1 + 0.175 * vs) * 1e-9; /* measured: 2.8 ps per fp32 entry, 3.5 per fp64 */
+    case ASAMD_SPMV_XLDS: return nnz * (1.15 + 0.1875 * vs) * 1e-9; /* measured: 1.9 ps per fp32 entry, 2.65 per fp64 */
     case ASAMD_SPMV_ELL: {
       const double ell_bytes = m * (double)st->max_len * (4.0 + vs) + (n + m) * vs;
       return hypot2(ell_bytes / 6.1e9, gather);
