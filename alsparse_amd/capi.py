@@ -135,13 +135,19 @@ class asamd_csr_stats(Structure):
                 ("binned_built", c_int32), ("bin_rows", c_int32 * 4), ("tune_ms_binned", c_float),
                 ("tile_long_blocks", c_int32), ("value_check", c_int32), ("tune_mode", c_int32),
                 ("device_bytes", c_int64), ("workspace_bytes", c_int64),
-                ("lines_per_entry_wave", c_float), ("lines_per_entry_segment", c_float)]
+                ("lines_per_entry_wave", c_float), ("lines_per_entry_segment", c_float),
+                ("xlds_slices", c_int32)]
 
 
 class asamd_spmv_args(Structure):  # include/alsparse_amd_kernels.h
     _fields_ = [("dtype", c_int32), ("m", c_int32), ("n", c_int32), ("nnz", c_int32), ("base", c_int32),
                 ("alpha", c_void_p), ("beta", c_void_p), ("val", c_void_p), ("row_ptr", c_void_p),
                 ("col_ind", c_void_p), ("x", c_void_p), ("y", c_void_p)]
+
+
+class asamd_xlds_layout(Structure):  # include/alsparse_amd_kernels.h
+    _fields_ = [("seg", c_void_p), ("slices", c_int32), ("slice_cols", c_int32), ("m", c_int32),
+                ("device_bytes", ctypes.c_int64)]
 
 
 class asamd_dense_strides(Structure):
@@ -348,6 +354,9 @@ _COMMON = {
     "asamd_gather_values": [_P, _I, _I, _I, _P, _P, _P, _P],
     "asamd_spmv_xlds": [_P, _P, _I],
     "asamd_spmv_xlds_fits": [_I, _I],
+    "asamd_xlds_build": [_P, _I, _I, _I, _I, _I, _P, _P, _P],
+    "asamd_xlds_free": [_P],
+    "asamd_spmv_xlds_sliced": [_P, POINTER(asamd_spmv_args), _I, _P, _P],
     "asamd_csr2ell_gated": [_P, _I, _I, _P, _P, _P, _I, _I, _I, _P, _P, _P],
     "asamd_csr_plan_build_transpose": [_P, _P, _P, _P, _P],
     "asamd_csr_plan_set_lazy_transpose": [_P, _I],
@@ -390,7 +399,7 @@ _RESTYPE = {"alpha_set_thread_num": None, "alpha_timing_wtime": c_double, "alpha
             "args_help": None, "args_get_if_check": c_bool, "args_get_data_file": ctypes.c_char_p,
             "args_get_data_fileA": ctypes.c_char_p, "args_get_data_fileB": ctypes.c_char_p,
             "alpha_args_get_matrix_descrA": alpha_matrix_descr, "alpha_args_get_matrix_descrB": alpha_matrix_descr,
-            "get_time_us": c_double, "asamd_csrmm_workspace_bytes": c_size_t, "asamd_csr2coo_workspace_bytes": c_size_t, "asamd_csr_plan_workspace_bytes": c_size_t, "asamd_csr_plan_watched_workspace_bytes": c_size_t, "asamd_value_guard_run": c_size_t, "asamd_tiled_free": None, "asamd_hot_free": None, "asamd_binned_free": None, "asamd_transpose_free": None, "asamd_csr_plan_stats": POINTER(asamd_csr_stats),
+            "get_time_us": c_double, "asamd_csrmm_workspace_bytes": c_size_t, "asamd_csr2coo_workspace_bytes": c_size_t, "asamd_csr_plan_workspace_bytes": c_size_t, "asamd_csr_plan_watched_workspace_bytes": c_size_t, "asamd_value_guard_run": c_size_t, "asamd_tiled_free": None, "asamd_xlds_free": None, "asamd_hot_free": None, "asamd_binned_free": None, "asamd_transpose_free": None, "asamd_csr_plan_stats": POINTER(asamd_csr_stats),
             "asamd_csr_plan_transpose_stats": POINTER(asamd_csr_stats),
             "asamd_analysis_transpose_stats": POINTER(asamd_csr_stats),
             "asamd_analysis_stats": POINTER(asamd_csr_stats)}

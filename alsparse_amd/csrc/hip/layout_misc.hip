@@ -13,6 +13,7 @@
 #include "spmv_hot.hpp"
 #include "spmv_tiled.hpp"  // tile_bounds_kernel
 #include "spmv_trans.hpp"
+#include "spmv_xlds.hpp"
 #include "tile_sort.hpp"
 
 using namespace asamd;
@@ -170,6 +171,56 @@ extern "C" int asamd_spmv_hot(hipStream_t s, const asamd_spmv_args* a, const asa
   if (a->dtype == ASAMD_DTYPE_FLOAT_COMPLEX)
     return spmv_hot_impl<Cx<float>>(s, a, L, front, carry_row, carry_val, head_val);
   return hipErrorInvalidValue;
+}
+
+// ---- column slices for the kernel that holds x in LDS ----------------------------------------------
+// As few slices as hold x in ASAMD_XLDS_MAX_BYTES each, of equal width (a multiple of 64 columns).
+extern "C" int asamd_xlds_build(hipStream_t stream, int32_t dtype, int32_t m, int32_t n, int32_t nnz, int32_t base,
+                                const int32_t* row_ptr, const int32_t* col_ind, asamd_xlds_layout* L) {
+  if (!L) return hipErrorInvalidValue;
+  *L = asamd_xlds_layout{};
+  const int vs = dtype_size(dtype);
+  if (!row_ptr || !col_ind || m < 1 || n < 1 || nnz < 1 || vs <= 0) return hipErrorInvalidValue;
+  const int64_t fill = (int64_t)ASAMD_XLDS_MAX_BYTES / vs;  // columns per LDS fill
+  const int64_t slices = ((int64_t)n + fill - 1) / fill;
+  if (slices < 2 || slices > 64 || (slices + 1) * (int64_t)m >= (int64_t)INT32_MAX) return hipSuccess;  // no layout
+  int64_t width = ((int64_t)n + slices - 1) / slices;
+  width = (width + 63) / 64 * 64;
+  if (width > fill) width = fill;
+  int* d_flag = nullptr;
+  int h_flag = 0;
+  hipError_t e = hipMalloc(&d_flag, sizeof(int));
+  if (e == hipSuccess) e = hipMemsetAsync(d_flag, 0, sizeof(int), stream);
+  if (e == hipSuccess) {
+    xlds_rows_ascend_kernel<<<(unsigned)(((int64_t)m + 3) / 4), 256, 0, stream>>>(m, row_ptr, col_ind, base, d_flag);
+    e = hipMemcpyAsync(&h_flag, d_flag, sizeof(int), hipMemcpyDeviceToHost, stream);
+  }
+  if (e == hipSuccess) e = hipStreamSynchronize(stream);
+  if (e == hipSuccess && h_flag == 0) {
+    const int64_t count = (slices + 1) * (int64_t)m;
+    e = hipMalloc(&L->seg, (size_t)count * sizeof(int));
+    if (e == hipSuccess) {
+      xlds_slice_offsets_kernel<<<(unsigned)((count + 255) / 256), 256, 0, stream>>>(m, (int)slices, (int)width, row_ptr,
+                                                                                    col_ind, base, L->seg);
+      e = hipGetLastError();
+    }
+    if (e == hipSuccess) e = hipStreamSynchronize(stream);
+    if (e == hipSuccess) {
+      L->slices = (int32_t)slices;
+      L->slice_cols = (int32_t)width;
+      L->m = m;
+      L->device_bytes = count * (int64_t)sizeof(int);
+    }
+  }
+  if (d_flag) (void)hipFree(d_flag);
+  if (e != hipSuccess) asamd_xlds_free(L);
+  return e;
+}
+
+extern "C" void asamd_xlds_free(asamd_xlds_layout* L) {
+  if (!L) return;
+  if (L->seg) (void)hipFree(L->seg);
+  *L = asamd_xlds_layout{};
 }
 
 // ---- row-length bins -----------------------------------------------------------------------------

@@ -97,9 +97,10 @@ static int launch_xlds(hipStream_t s, const asamd_spmv_args* a) {
   return (int64_t)a->nnz <= (int64_t)a->m * W ? launch_xlds_as<T, W, true>(s, a) : launch_xlds_as<T, W, false>(s, a);
 }
 
-// four entries per lane and load: W lanes take the first 4 W entries of a row
+// four entries per lane and load: W lanes take the first 4 W entries of a row.  L: column slices (their sums go to
+// `partials`, slices * m elements, and are added up by a second kernel), or null.
 template <typename T, int W, bool NT>
-static int launch_xlds4_as(hipStream_t s, const asamd_spmv_args* a) {
+static int launch_xlds4_as(hipStream_t s, const asamd_spmv_args* a, const asamd_xlds_layout* L, void* partials) {
   static const int cus = [] {
     int dev = 0, n = 0;
     if (hipGetDevice(&dev) != hipSuccess ||
@@ -107,7 +108,8 @@ static int launch_xlds4_as(hipStream_t s, const asamd_spmv_args* a) {
       n = 256;
     return n;
   }();
-  const size_t lds = ((size_t)a->n * sizeof(T) + 15) / 16 * 16;
+  const int slices = L ? L->slices : 1, slice_cols = L ? L->slice_cols : a->n;
+  const size_t lds = ((size_t)slice_cols * sizeof(T) + 15) / 16 * 16;
   static size_t allowed = 0;  // (per instantiation)
   if (lds > allowed) {
     const hipError_t e = hipFuncSetAttribute((const void*)spmv_xlds4_kernel<T, W, NT>,
@@ -117,15 +119,28 @@ static int launch_xlds4_as(hipStream_t s, const asamd_spmv_args* a) {
   }
   constexpr int rows_per_trip = (kXldsThreads / W) * kXlds4Rows;
   int64_t grid = ((int64_t)a->m + rows_per_trip - 1) / rows_per_trip;
-  if (grid > cus) grid = cus;
-  spmv_xlds4_kernel<T, W, NT><<<(unsigned)grid, kXldsThreads, lds, s>>>(
-      a->m, a->n, (int64_t)a->nnz, scalar_of<T>(a->alpha), (const T*)a->val, a->row_ptr, a->col_ind, (const T*)a->x,
-      scalar_of<T>(a->beta), (T*)a->y, a->base);
+  const int64_t per_slice = cus / slices > 0 ? cus / slices : 1;  // the workgroups share the compute units
+  if (grid > per_slice) grid = per_slice;
+  if (!L) {
+    spmv_xlds4_kernel<T, W, NT><<<(unsigned)grid, kXldsThreads, lds, s>>>(
+        a->m, a->n, a->n, (int64_t)a->nnz, scalar_of<T>(a->alpha), (const T*)a->val, a->row_ptr, a->row_ptr + 1, 0,
+        a->col_ind, (const T*)a->x, scalar_of<T>(a->beta), (T*)a->y, 0, a->base);
+    return hipGetLastError();
+  }
+  spmv_xlds4_kernel<T, W, NT><<<dim3((unsigned)grid, (unsigned)slices), kXldsThreads, lds, s>>>(
+      a->m, a->n, slice_cols, (int64_t)a->nnz, T(1), (const T*)a->val, L->seg, L->seg + a->m, (int64_t)a->m, a->col_ind,
+      (const T*)a->x, T(0), (T*)partials, (int64_t)a->m, a->base);
+  xlds_slices_sum_kernel<T><<<(unsigned)(((int64_t)a->m + 255) / 256), 256, 0, s>>>(
+      a->m, slices, scalar_of<T>(a->alpha), (const T*)partials, scalar_of<T>(a->beta), (T*)a->y);
   return hipGetLastError();
 }
+// (non-temporal first loads where the pieces of the rows hold at most 4 W entries on average)
 template <typename T, int W>
-static int launch_xlds4(hipStream_t s, const asamd_spmv_args* a) {
-  return (int64_t)a->nnz <= (int64_t)a->m * 4 * W ? launch_xlds4_as<T, W, true>(s, a) : launch_xlds4_as<T, W, false>(s, a);
+static int launch_xlds4(hipStream_t s, const asamd_spmv_args* a, const asamd_xlds_layout* L = nullptr,
+                        void* partials = nullptr) {
+  const int64_t pieces = (int64_t)a->m * (L ? L->slices : 1);
+  return (int64_t)a->nnz <= pieces * 4 * W ? launch_xlds4_as<T, W, true>(s, a, L, partials)
+                                           : launch_xlds4_as<T, W, false>(s, a, L, partials);
 }
 
 extern "C" int asamd_spmv_xlds(hipStream_t s, const asamd_spmv_args* a, int32_t width) {
@@ -157,6 +172,33 @@ extern "C" int asamd_spmv_xlds(hipStream_t s, const asamd_spmv_args* a, int32_t 
       case 32: return launch_xlds<T, 32>(s, a);
       case 64: return launch_xlds<T, 64>(s, a);
       default: return hipErrorInvalidValue;
+    }
+  });
+}
+
+// `width`: lanes per piece of a row if every lane took ONE entry (2 .. 64, from the pieces' mean length)
+extern "C" int asamd_spmv_xlds_sliced(hipStream_t s, const asamd_spmv_args* a, int32_t width, const asamd_xlds_layout* L,
+                                      void* partials) {
+  if (!a || !L || !L->seg || !partials || L->slices < 2 || L->m != a->m || a->nnz < 4 || a->m < 1)
+    return hipErrorInvalidValue;
+  if ((int64_t)L->slice_cols * dtype_size(a->dtype) > (int64_t)ASAMD_XLDS_MAX_BYTES ||
+      (int64_t)L->slices * L->slice_cols < (int64_t)a->n)
+    return hipErrorInvalidValue;
+  return by_dtype(a->dtype, [&](auto* tag) -> int {
+    using T = std::remove_pointer_t<decltype(tag)>;
+    if constexpr (!kIsReal<T>) {
+      return hipErrorInvalidValue;
+    } else {
+      if (!args_ok<T>(a) || (uintptr_t)partials % alignof(T)) return hipErrorInvalidValue;
+      switch (width) {
+        case 2:
+        case 4: return launch_xlds4<T, 1>(s, a, L, partials);
+        case 8: return launch_xlds4<T, 2>(s, a, L, partials);
+        case 16: return launch_xlds4<T, 4>(s, a, L, partials);
+        case 32: return launch_xlds4<T, 8>(s, a, L, partials);
+        case 64: return launch_xlds4<T, 16>(s, a, L, partials);
+        default: return hipErrorInvalidValue;
+      }
     }
   });
 }

@@ -207,15 +207,30 @@ __device__ __forceinline__ XldsPiece<T> xlds_load_piece(const T* __restrict__ va
   return p;
 }
 
+//
+// Column slices (gridDim.y > 1): for an x of several LDS fills the matrix is cut into slices of slice_cols columns,
+// workgroup row blockIdx.y taking slice blockIdx.y.  With ascending columns inside the rows a row's entries of one
+// slice are a contiguous piece of the CSR arrays, so all a slice needs is where its piece of every row begins and
+// ends: row_lo / row_hi then point at a table of slices + 1 rows of m offsets (offsets_per_slice = m apart; in
+// row_ptr's convention, base included), and the kernel writes the slice's sums (alpha = 1, beta = 0) to
+// y + blockIdx.y * y_per_slice for a second kernel to add up.  One slice: row_lo = row_ptr, row_hi = row_ptr + 1.
 template <typename T, int W, bool NT>
-__global__ __launch_bounds__(kXldsThreads) void spmv_xlds4_kernel(int m, int n, int64_t limit, T alpha,
-                                                                  const T* __restrict__ val,
-                                                                  const int* __restrict__ row_ptr,
+__global__ __launch_bounds__(kXldsThreads) void spmv_xlds4_kernel(int m, int n_total, int slice_cols, int64_t limit,
+                                                                  T alpha, const T* __restrict__ val,
+                                                                  const int* __restrict__ row_lo,
+                                                                  const int* __restrict__ row_hi,
+                                                                  int64_t offsets_per_slice,
                                                                   const int* __restrict__ col_ind,
                                                                   const T* __restrict__ x, T beta, T* __restrict__ y,
-                                                                  int base) {
+                                                                  int64_t y_per_slice, int base) {
   extern __shared__ __align__(16) unsigned char xlds_bytes[];
   T* __restrict__ xs = reinterpret_cast<T*>(xlds_bytes);
+  const int col0 = (int)blockIdx.y * slice_cols;  // the slice's first column
+  const int n = n_total - col0 < slice_cols ? n_total - col0 : slice_cols;
+  row_lo += (int64_t)blockIdx.y * offsets_per_slice;
+  row_hi += (int64_t)blockIdx.y * offsets_per_slice;
+  x += col0;
+  y += (int64_t)blockIdx.y * y_per_slice;
   constexpr int kGroups = kXldsThreads / W;
   constexpr int K = kXlds4Rows;
   constexpr int kWaveLen = kXldsWaveRow * 4 * W;  // longer rows go to the whole wave
@@ -228,9 +243,11 @@ __global__ __launch_bounds__(kXldsThreads) void spmv_xlds4_kernel(int m, int n, 
   auto request_offsets = [&](int64_t first, int* lo, int* hi) __attribute__((always_inline)) {
 #pragma unroll
     for (int k = 0; k < K; ++k) {
+      // (rows past the last: the last row's end, twice -- an empty row)
       const int64_t r = first + (int64_t)k * kGroups + group;
-      lo[k] = row_ptr[r < m ? r : m];
-      hi[k] = row_ptr[r < m ? r + 1 : m];
+      hi[k] = row_hi[r < m ? r : m - 1];
+      lo[k] = row_lo[r < m ? r : m - 1];
+      lo[k] = r < m ? lo[k] : hi[k];
     }
   };
   request_offsets(row0, start, end);
@@ -252,13 +269,14 @@ __global__ __launch_bounds__(kXldsThreads) void spmv_xlds4_kernel(int m, int n, 
     for (int i = threadIdx.x; i < n; i += kXldsThreads) xs[i] = x[i];
   }
   __syncthreads();
-  const T* __restrict__ xb = xs - base;
+  const int first_col = base + col0;
+  const T* __restrict__ xb = xs - first_col;  // (indexed with the caller's column numbers)
   // the lane's (up to four) entries from position j of a row that ends at e, times x, added up
   auto piece_sum = [&](const XldsPiece<T>& p, int j, int e, T sum) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const bool mine = j + i < e;
-      const T xv = xb[mine ? p.c[i] : base];
+      const T xv = xb[mine ? p.c[i] : first_col];
       sum = mine ? fma_t(p.v[i], xv, sum) : sum;
     }
     return sum;
@@ -319,6 +337,50 @@ __global__ __launch_bounds__(kXldsThreads) void spmv_xlds4_kernel(int m, int n, 
       end[k] = next_end[k];
     }
   }
+}
+
+// ---- column slices: the table of offsets, and the sum of the slices' results ------------------------------------
+// seg[s * m + r], s = 0 .. slices: where row r's entries of slice s begin (in row_ptr's convention, base included);
+// needs ascending columns inside every row
+static __global__ __launch_bounds__(256) void xlds_slice_offsets_kernel(int m, int slices, int slice_cols,
+                                                                        const int* __restrict__ row_ptr,
+                                                                        const int* __restrict__ col_ind, int base,
+                                                                        int* __restrict__ seg) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= ((int64_t)slices + 1) * m) return;
+  const int s = (int)(i / m), r = (int)(i % m);
+  int lo = row_ptr[r] - base, hi = row_ptr[r + 1] - base;
+  if (s == slices) lo = hi;
+  if (s > 0 && s < slices) {
+    const int64_t target = (int64_t)base + (int64_t)s * slice_cols;  // the slice's first column
+    while (lo < hi) {
+      const int mid = lo + (hi - lo) / 2;
+      if ((int64_t)col_ind[mid] < target) lo = mid + 1;
+      else hi = mid;
+    }
+  }
+  seg[i] = lo + base;
+}
+// *unsorted |= 1 if the columns of some row do not ascend; a wave per row
+static __global__ __launch_bounds__(256) void xlds_rows_ascend_kernel(int m, const int* __restrict__ row_ptr,
+                                                                      const int* __restrict__ col_ind, int base,
+                                                                      int* __restrict__ unsorted) {
+  const int64_t r = (int64_t)blockIdx.x * (256 / kWave) + threadIdx.x / kWave;
+  if (r >= m) return;
+  const int end = row_ptr[r + 1] - base;
+  bool bad = false;
+  for (int j = row_ptr[r] - base + (int)(threadIdx.x % kWave); j + 1 < end; j += kWave) bad |= col_ind[j] > col_ind[j + 1];
+  if (__ballot(bad) != 0 && threadIdx.x % kWave == 0) atomicOr(unsorted, 1);
+}
+// y = alpha * (the slices' sums, added in the order of the slices) + beta * y
+template <typename T>
+__global__ __launch_bounds__(256) void xlds_slices_sum_kernel(int m, int slices, T alpha, const T* __restrict__ part,
+                                                              T beta, T* __restrict__ y) {
+  const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (r >= m) return;
+  T sum = part[r];
+  for (int s = 1; s < slices; ++s) sum += part[(int64_t)s * m + r];
+  store_axpby(y, r, alpha, sum, beta);
 }
 
 }  // namespace asamd

@@ -31,6 +31,7 @@ struct asamd_csr_plan {
   asamd_tiled_layout tiled;
   asamd_hot_layout hot;
   asamd_binned_layout binned;
+  asamd_xlds_layout xlds;  /* column slices for the kernel that holds x in LDS (an x of several LDS fills) */
   void *d_eval;            /* ELL copy: ell_width * m values, column-major */
   int32_t *d_ecol;         /* ... and zero-based columns */
   const void *copy_val_src; /* the value array that the tiled / ELL copy was taken from */
@@ -122,6 +123,25 @@ static int xlds_ok(const asamd_csr_plan *p) {
   const int64_t x_bytes = (int64_t)st->n * (int64_t)p->val_size;
   return st->first_offset == 0 && st->m >= 1 && st->nnz >= (1 << 22) && x_bytes > (20 << 10) &&
          asamd_spmv_xlds_fits(p->dtype, st->n) && env_int("ALSPARSE_AMD_XLDS", 1) > 0;
+}
+
+/* ... and slice by slice for an x of several LDS fills, where the rows are long enough for their pieces: a slice's
+ * piece of a row should hold sixteen entries or more on average (262 144 x 262 144 x 400, fp32, 8 slices: merge-path
+ * 0.51 ms, this 0.23 ms; 1 M x 131 072 x 128, 4 slices: 0.41 ms).  Needs ascending columns inside the rows (the
+ * builder looks) and a structure that is promised fixed. */
+static int xlds_slices_for(const asamd_csr_plan *p) {
+  const int64_t x_bytes = (int64_t)p->st.n * (int64_t)p->val_size;
+  return (int)((x_bytes + ASAMD_XLDS_MAX_BYTES - 1) / ASAMD_XLDS_MAX_BYTES);
+}
+static int xlds_sliced_ok(const asamd_csr_plan *p, int force) {
+  const asamd_csr_stats *st = &p->st;
+  if (!st->trusted || st->first_offset != 0 || st->m < 1 || st->nnz < 4) return 0;
+  if (p->dtype != ASAMD_DTYPE_FLOAT && p->dtype != ASAMD_DTYPE_DOUBLE) return 0;
+  const int slices = xlds_slices_for(p);
+  if (slices < 2 || slices > 64 || ((int64_t)slices + 1) * st->m >= (int64_t)INT32_MAX) return 0;
+  if (force) return 1;
+  return st->nnz >= (1 << 22) && (double)st->nnz >= 16.0 * (double)slices * (double)st->m &&
+         env_int("ALSPARSE_AMD_XLDS", 1) > 0;
 }
 
 static void choose_algo(asamd_csr_plan *p) {
@@ -328,6 +348,8 @@ static size_t algo_scratch(const asamd_csr_plan *p, int algo) {
              2 * align256((size_t)p->hot.blocks * vs);
     case ASAMD_SPMV_BINNED:
       return st->binned_built ? align256((size_t)p->binned.chunks * vs) : 0;
+    case ASAMD_SPMV_XLDS:
+      return p->xlds.seg ? align256((size_t)p->xlds.slices * (size_t)st->m * vs) : 0;
     default:
       return 0;
   }
@@ -338,7 +360,7 @@ static int has_value_copy(const asamd_csr_plan *p) { return p->st.tiled_built ||
 size_t asamd_csr_plan_workspace_bytes(const asamd_csr_plan *p) {
   if (!p) return 0;
   size_t need = 0;
-  for (int a = ASAMD_SPMV_VECTOR; a <= ASAMD_SPMV_BINNED; ++a) {
+  for (int a = ASAMD_SPMV_VECTOR; a <= ASAMD_SPMV_XLDS; ++a) {
     if (a == ASAMD_SPMV_MERGE && p->st.first_offset != 0) continue;
     const size_t s = algo_scratch(p, a);
     if (s > need) need = s;
@@ -356,7 +378,7 @@ static void account(asamd_csr_plan *p) {
   asamd_csr_stats *st = &p->st;
   int64_t b = SETUP_BYTES + 3 * 8;
   if (p->d_block_row) b += ((int64_t)st->merge_blocks + 1) * 4;
-  b += p->tiled.device_bytes + p->hot.device_bytes + p->binned.device_bytes;
+  b += p->tiled.device_bytes + p->hot.device_bytes + p->binned.device_bytes + p->xlds.device_bytes;
   if (st->ell_built) b += (int64_t)st->m * st->ell_width * ((int64_t)p->val_size + 4);
   for (int w = 0; w < 2; ++w)
     if (p->tr[w].plan) b += p->tr[w].t.device_bytes + p->tr[w].plan->st.device_bytes;
@@ -419,7 +441,7 @@ static int settle_algo(const asamd_csr_plan *p, int algo, const void *val, const
     else if (algo == ASAMD_SPMV_ELL && !st->ell_built) next = p->auto_algo == ASAMD_SPMV_ELL ? p->struct_algo : p->auto_algo;
     else if (algo == ASAMD_SPMV_MERGE_HOT && !st->hot_built) next = ASAMD_SPMV_MERGE;
     else if (algo == ASAMD_SPMV_BINNED && !st->binned_built) next = ASAMD_SPMV_MERGE;
-    else if (algo == ASAMD_SPMV_XLDS &&
+    else if (algo == ASAMD_SPMV_XLDS && !p->xlds.seg &&
              (!asamd_spmv_xlds_fits(p->dtype, st->n) || st->first_offset != 0 || st->nnz < 1 || st->m < 1))
       next = ASAMD_SPMV_VECTOR;
     else if (algo == ASAMD_SPMV_ROWCONST &&
@@ -453,6 +475,12 @@ static int run_algo(hipStream_t s, const asamd_csr_plan *p, int algo, const asam
     case ASAMD_SPMV_SCALAR:
       return asamd_spmv_scalar(s, a);
     case ASAMD_SPMV_XLDS:
+      if (p->xlds.seg) {
+        void *partials = ws_take(&ws, (size_t)p->xlds.slices * (size_t)st->m * vs);
+        if (!partials) return -1;
+        const double piece = (double)st->nnz / ((double)st->m * (double)p->xlds.slices);
+        return asamd_spmv_xlds_sliced(s, a, width_for_mean(piece), &p->xlds, partials);
+      }
       return asamd_spmv_xlds(s, a, p->auto_width);
     case ASAMD_SPMV_BINNED: {
       void *partial = p->binned.chunks > 0 ? ws_take(&ws, (size_t)p->binned.chunks * vs) : NULL;
@@ -920,7 +948,14 @@ static double model_ms(const asamd_csr_plan *p, int algo) {
     case ASAMD_SPMV_STREAM: rate = stream_group(p, 0) > 1 ? 5.2 : 6.6; break;
     case ASAMD_SPMV_VECTOR: rate = 2.4 * vector_utilisation(st, p->auto_width); break;
     case ASAMD_SPMV_MERGE: rate = 2.9; break;
-    case ASAMD_SPMV_XLDS: return nnz * (1.15 + 0.1875 * vs) * 1e-9; /* measured: 1.9 ps per fp32 entry, 2.65 per fp64 */
+    case ASAMD_SPMV_XLDS: {
+      /* measured: 1.9 ps per fp32 entry, 2.65 per fp64; in slices the pieces of the rows start anywhere in their
+       * cache lines (pieces of 50 / 36 / 32 entries: 1.14 / 1.57 / 1.6 times that) and the slices' sums travel */
+      const double one = nnz * (1.15 + 0.1875 * vs) * 1e-9;
+      const int slices = p->xlds.seg ? p->xlds.slices : (asamd_spmv_xlds_fits(p->dtype, st->n) ? 1 : xlds_slices_for(p));
+      if (slices < 2) return one;
+      return one * (1.0 + 22.0 * (double)slices / mean) + (double)slices * m * 3.0 * vs / 4.0e9;
+    }
     case ASAMD_SPMV_ELL: {
       const double ell_bytes = m * (double)st->max_len * (4.0 + vs) + (n + m) * vs;
       return hypot2(ell_bytes / 6.1e9, gather);
@@ -944,7 +979,7 @@ static hipError_t model_copies(hipStream_t stream, asamd_csr_plan *p, const int3
   asamd_csr_stats *st = &p->st;
   if (st->lines_per_entry_wave <= 0.f) return hipSuccess; /* not probed (a tiny matrix): the structural choice stays */
   double base = model_ms(p, p->auto_algo);
-  if (p->auto_algo == ASAMD_SPMV_XLDS) {
+  if (p->auto_algo == ASAMD_SPMV_XLDS && !p->xlds.seg) {
     /* columns that neighbouring entries share are cheap to gather from the caches too */
     const double plain = model_ms(p, p->plain_algo);
     if (base > 0.95 * plain) {
@@ -1125,6 +1160,28 @@ static hipError_t plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t 
     st->lines_per_entry_wave = probe[0];
     st->lines_per_entry_segment = probe[1];
   }
+  if (col_ind && nnz > 0 && trusted != 3 && xlds_sliced_ok(p, trusted == 2)) {
+    /* x in LDS slice by slice, if the model expects it to beat the structural choice by a fifth (no probe: no
+     * estimate of that choice, and no slices) */
+    const int wanted = trusted == 2 || (st->lines_per_entry_wave > 0.f &&
+                                        model_ms(p, ASAMD_SPMV_XLDS) < 0.9 * model_ms(p, p->auto_algo));
+    if (wanted) {
+      e = (hipError_t)asamd_xlds_build(stream, p->dtype, m, n, nnz, base, row_ptr, col_ind, &p->xlds);
+      if (e == hipErrorOutOfMemory) {
+        (void)hipGetLastError();
+        e = hipSuccess;
+      }
+      if (e != hipSuccess) {
+        asamd_csr_plan_destroy(p);
+        return e;
+      }
+      st->xlds_slices = p->xlds.seg ? p->xlds.slices : 0;
+      if (p->xlds.seg && trusted != 2) {
+        p->auto_algo = p->struct_algo = ASAMD_SPMV_XLDS;
+        st->algo = p->auto_algo;
+      }
+    }
+  }
   if (col_ind && val && nnz > 0) {
     /* trusted == 2: build every copy whatever the size and skip the timing
      * (lets small matrices exercise those kernels) */
@@ -1194,6 +1251,7 @@ void asamd_csr_plan_destroy(asamd_csr_plan *p) {
   free_ell(p);
   free_hot(p);
   free_binned(p);
+  asamd_xlds_free(&p->xlds);
   free_transpose(p, 0);
   free_transpose(p, 1);
   free(p);
@@ -1312,7 +1370,8 @@ int asamd_csr_plan_set_algo(asamd_csr_plan *p, int32_t algo) {
       if (p->st.first_offset != 0) return hipErrorInvalidValue;
       break;
     case ASAMD_SPMV_XLDS:
-      if (!asamd_spmv_xlds_fits(p->dtype, p->st.n) || p->st.first_offset != 0) return hipErrorInvalidValue;
+      if (!p->xlds.seg && (!asamd_spmv_xlds_fits(p->dtype, p->st.n) || p->st.first_offset != 0))
+        return hipErrorInvalidValue;
       break;
     case ASAMD_SPMV_VECTOR:
     case ASAMD_SPMV_SCALAR:

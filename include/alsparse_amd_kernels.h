@@ -100,6 +100,22 @@ int asamd_spmv_vector_if(hipStream_t stream, const asamd_spmv_args *a, int32_t w
 #define ASAMD_XLDS_MAX_BYTES 131072
 int asamd_spmv_xlds_fits(int32_t dtype, int32_t n);
 int asamd_spmv_xlds(hipStream_t stream, const asamd_spmv_args *a, int32_t width);
+/* The same for an x of several LDS fills (real element types): the matrix in `slices` slices of slice_cols columns,
+ * a row of workgroups each.  With ascending columns inside the rows a row's entries of one slice are a contiguous
+ * piece of the caller's arrays, so the layout is a table of offsets only -- seg[s * m + r], s = 0 .. slices: where
+ * row r's piece of slice s begins (base included) -- and the values are read in place.  asamd_xlds_build leaves
+ * the record EMPTY (seg NULL, not an error) if some row's columns do not ascend.  Per-call scratch: slices * m
+ * elements of `partials`; `width` as for asamd_spmv_vector, from the pieces' mean length. */
+typedef struct {
+  int32_t *seg;  /* (slices + 1) * m offsets; NULL: no layout */
+  int32_t slices, slice_cols, m;
+  int64_t device_bytes;
+} asamd_xlds_layout;
+int asamd_xlds_build(hipStream_t stream, int32_t dtype, int32_t m, int32_t n, int32_t nnz, int32_t base,
+                     const int32_t *row_ptr, const int32_t *col_ind, asamd_xlds_layout *out);
+void asamd_xlds_free(asamd_xlds_layout *layout);
+int asamd_spmv_xlds_sliced(hipStream_t stream, const asamd_spmv_args *a, int32_t width, const asamd_xlds_layout *layout,
+                           void *partials);
 /* One lane per row, entries in storage order (src/plain/kernel/level2/mv/gemv/gemv_x_csr_plain.c:11-22). */
 int asamd_spmv_scalar(hipStream_t stream, const asamd_spmv_args *a);
 /* Every row has row_len entries (4, 8, ..., 256): no row_ptr traffic.  Real element types, row_ptr[0] ==

@@ -66,6 +66,7 @@ typedef struct {
   float lines_per_entry_wave;    /* locality probe (asamd_csr_locality_probe): distinct 128-byte lines of x
                                     per entry among 64 consecutive entries, or 0 if not probed          */
   float lines_per_entry_segment; /* ... and within runs of 32 768 consecutive entries                     */
+  int32_t xlds_slices;   /* column slices of the kernel that holds x in LDS (a table of offsets exists), or 0   */
 } asamd_csr_stats;
 
 typedef struct asamd_csr_plan asamd_csr_plan;

@@ -81,7 +81,7 @@ def run_plan_csrmv(da, algo, alpha, x, beta, y0, trusted=1):
     lib = capi.load()
     from ctypes import c_void_p
     plan = c_void_p()
-    if algo in ("tiled", "ell", "hot", "binned"):
+    if algo in ("tiled", "ell", "hot", "binned", "xlds"):
         trusted = 2  # build the copies whatever the size
     e = lib.asamd_csr_plan_create(None, a.rows, a.cols, a.nnz, da.row_ptr.c_ptr(), da.col.c_ptr(), da.val.c_ptr(),
                                   a.base, a.dtype.itemsize, trusted, byref(plan))

@@ -84,3 +84,63 @@ def test_rows_of_every_length_and_both_bases(gpu):
                     check_spmv(a, alpha, x, beta, y0, y, "ragged base %d %s" % (base, (alpha, beta)))
             finally:
                 da.free()
+
+
+SLICED = {
+    # 3 slices of fp32 columns, pieces of 100 entries
+    "f32_70000": lambda: wl.uniform_rows(16384, 70000, 300, np.float32),
+    # 5 slices of fp64 columns, index base one
+    "f64_80000_base1": lambda: wl.uniform_rows(20000, 80000, 250, np.float64, base=1),
+}
+
+
+@pytest.mark.parametrize("shape", sorted(SLICED))
+def test_long_rows_over_several_lds_fills_of_x_go_slice_by_slice(gpu, shape, monkeypatch):
+    """x of 280 / 640 KB under rows of hundreds of entries: the analysis lays out a table of offsets (where every
+    row's piece of every column slice begins) and the multiply runs a row of workgroups per slice; the values stay
+    in the caller's array, so new values need no second analysis."""
+    lib = capi.load()
+    a = SLICED[shape]()
+    x, y0 = wl.uniform(a.cols, a.dtype, 3), wl.uniform(a.rows, a.dtype, 4)
+    da = DeviceCsr(a)
+    info = capi.alphasparse_dcu_mat_info_t()
+    assert lib.alphasparse_dcu_create_mat_info(byref(info)) == 0
+    descr = capi.make_descr(base=a.base)
+    p = capi.prefix(a.dtype)
+    try:
+        announce("x in LDS, sliced: analysis", shape)
+        assert getattr(lib, "alphasparse_dcu_%s_csrmv_analysis" % p)(
+            gpu.h, 0, a.rows, a.cols, a.nnz, byref(descr), da.val.c_ptr(), da.row_ptr.c_ptr(), da.col.c_ptr(), info) == 0
+        st = lib.asamd_analysis_stats(info).contents
+        assert st.algo == capi.ASAMD_SPMV_XLDS and st.xlds_slices >= 2, (st.algo, st.xlds_slices)
+        for alpha, beta in ((1.0, 0.0), (-0.5, 2.0)):
+            announce("x in LDS, sliced: multiply", shape, alpha, beta)
+            y = run_csrmv(gpu, da, alpha, x, beta, y0, info=info)
+            check_spmv(a, alpha, x, beta, y0, y, "%s %s" % (shape, (alpha, beta)))
+        announce("x in LDS, sliced: new values in place", shape)
+        b = wl.Csr(a.rows, a.cols, a.row_ptr, a.col_ind, wl.uniform(a.nnz, a.dtype, 21), a.base, a.name)
+        da.val.copy_from(b.values)
+        y = run_csrmv(gpu, da, 2.0, x, 0.0, y0, info=info)
+        check_spmv(b, 2.0, x, 0.0, y0, y, "%s new values" % shape)
+        monkeypatch.setenv("ALSPARSE_AMD_XLDS", "0")
+        assert _plan_algo(lib, da) != capi.ASAMD_SPMV_XLDS
+    finally:
+        lib.alphasparse_dcu_destroy_mat_info(info)
+        da.free()
+
+
+def test_rows_whose_columns_do_not_ascend_get_no_slices(gpu):
+    lib = capi.load()
+    a = wl.uniform_rows(16384, 70000, 300, np.float32)
+    cols = a.col_ind.copy()
+    cols[5:7] = cols[5:7][::-1]  # one pair out of order in row 0
+    b = wl.Csr(a.rows, a.cols, a.row_ptr, cols, a.values, a.base, "unsorted")
+    da = DeviceCsr(b)
+    try:
+        announce("x in LDS, sliced: unsorted columns")
+        assert _plan_algo(lib, da) != capi.ASAMD_SPMV_XLDS
+        x, y0 = wl.uniform(b.cols, b.dtype, 3), wl.uniform(b.rows, b.dtype, 4)
+        y = run_csrmv(gpu, da, 1.0, x, 0.0, y0)
+        check_spmv(b, 1.0, x, 0.0, y0, y, "unsorted")
+    finally:
+        da.free()
