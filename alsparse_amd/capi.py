@@ -333,6 +333,8 @@ _COMMON = {
     "asamd_merge_partition": [_P, _I, _I, _P, _I, _I, _I, _P],
     "asamd_spmv_merge": [_P, POINTER(asamd_spmv_args), _I, _P, _P, _P, _P],
     "asamd_spmv_trans_scatter": [_P, POINTER(asamd_spmv_args), _I, _I],
+    "asamd_spmv_trans_ylds_bytes": [_I, _I, _I],
+    "asamd_spmv_trans_ylds": [_P, POINTER(asamd_spmv_args), _I, _I, _P],
     "asamd_tiled_fits": [_I, _I, _I, _I],
     "asamd_tiled_build": [_P, _I, _I, _I, _I, _I, _P, _P, _P, _I, _I, _P],
     "asamd_tiled_free": [_P],
@@ -399,7 +401,7 @@ _RESTYPE = {"alpha_set_thread_num": None, "alpha_timing_wtime": c_double, "alpha
             "args_help": None, "args_get_if_check": c_bool, "args_get_data_file": ctypes.c_char_p,
             "args_get_data_fileA": ctypes.c_char_p, "args_get_data_fileB": ctypes.c_char_p,
             "alpha_args_get_matrix_descrA": alpha_matrix_descr, "alpha_args_get_matrix_descrB": alpha_matrix_descr,
-            "get_time_us": c_double, "asamd_csrmm_workspace_bytes": c_size_t, "asamd_csr2coo_workspace_bytes": c_size_t, "asamd_csr_plan_workspace_bytes": c_size_t, "asamd_csr_plan_watched_workspace_bytes": c_size_t, "asamd_value_guard_run": c_size_t, "asamd_tiled_free": None, "asamd_xlds_free": None, "asamd_hot_free": None, "asamd_binned_free": None, "asamd_transpose_free": None, "asamd_csr_plan_stats": POINTER(asamd_csr_stats),
+            "get_time_us": c_double, "asamd_csrmm_workspace_bytes": c_size_t, "asamd_csr2coo_workspace_bytes": c_size_t, "asamd_csr_plan_workspace_bytes": c_size_t, "asamd_spmv_trans_ylds_bytes": c_size_t, "asamd_csr_plan_watched_workspace_bytes": c_size_t, "asamd_value_guard_run": c_size_t, "asamd_tiled_free": None, "asamd_xlds_free": None, "asamd_hot_free": None, "asamd_binned_free": None, "asamd_transpose_free": None, "asamd_csr_plan_stats": POINTER(asamd_csr_stats),
             "asamd_csr_plan_transpose_stats": POINTER(asamd_csr_stats),
             "asamd_analysis_transpose_stats": POINTER(asamd_csr_stats),
             "asamd_analysis_stats": POINTER(asamd_csr_stats)}

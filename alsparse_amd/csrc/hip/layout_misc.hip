@@ -183,7 +183,7 @@ extern "C" int asamd_xlds_build(hipStream_t stream, int32_t dtype, int32_t m, in
   if (!row_ptr || !col_ind || m < 1 || n < 1 || nnz < 1 || vs <= 0) return hipErrorInvalidValue;
   const int64_t fill = (int64_t)ASAMD_XLDS_MAX_BYTES / vs;  // columns per LDS fill
   const int64_t slices = ((int64_t)n + fill - 1) / fill;
-  if (slices < 2 || slices > 64 || (slices + 1) * (int64_t)m >= (int64_t)INT32_MAX) return hipSuccess;  // no layout
+  if (slices < 2 || slices > 1024 || (slices + 1) * (int64_t)m >= (int64_t)INT32_MAX) return hipSuccess;  // no layout
   int64_t width = ((int64_t)n + slices - 1) / slices;
   width = (width + 63) / 64 * 64;
   if (width > fill) width = fill;

@@ -367,6 +367,72 @@ extern "C" int asamd_spmv_merge(hipStream_t s, const asamd_spmv_args* a, int32_t
   });
 }
 
+// ---- transposed product with y in LDS --------------------------------------------------------------
+static int xlds_compute_units() {
+  static const int cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    return n;
+  }();
+  return cus;
+}
+// workgroups of the launch: as many as compute units, fewer for few rows (lanes per row do not matter: the least)
+static int64_t trans_ylds_groups(int32_t m) {
+  const int64_t rows_per_trip = (int64_t)(kXldsThreads / kWave) * kXldsRows;
+  int64_t grid = ((int64_t)m + rows_per_trip - 1) / rows_per_trip;
+  return grid > xlds_compute_units() ? xlds_compute_units() : (grid < 1 ? 1 : grid);
+}
+extern "C" size_t asamd_spmv_trans_ylds_bytes(int32_t dtype, int32_t m, int32_t n) {
+  if (m < 1 || !asamd_spmv_xlds_fits(dtype, n)) return 0;
+  return (size_t)trans_ylds_groups(m) * (size_t)n * (size_t)dtype_size(dtype);
+}
+
+template <typename T, int W, bool CONJ>
+static int launch_trans_ylds(hipStream_t s, const asamd_spmv_args* a, void* partials) {
+  const size_t lds = ((size_t)a->n * sizeof(T) + 15) / 16 * 16;
+  static size_t allowed = 0;  // (per instantiation)
+  if (lds > allowed) {
+    const hipError_t e = hipFuncSetAttribute((const void*)spmv_trans_ylds_kernel<T, W, CONJ>,
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, ASAMD_XLDS_MAX_BYTES);
+    if (e != hipSuccess) return e;
+    allowed = ASAMD_XLDS_MAX_BYTES;
+  }
+  const int64_t grid = trans_ylds_groups(a->m);
+  spmv_trans_ylds_kernel<T, W, CONJ><<<(unsigned)grid, kXldsThreads, lds, s>>>(
+      a->m, a->n, scalar_of<T>(a->alpha), (const T*)a->val, a->row_ptr, a->col_ind, (const T*)a->x, (T*)partials, a->base);
+  trans_partials_sum_kernel<T><<<(unsigned)(((int64_t)a->n + 255) / 256), 256, 0, s>>>(
+      a->n, (int)grid, (const T*)partials, scalar_of<T>(a->beta), (T*)a->y);
+  return hipGetLastError();
+}
+template <typename T, bool CONJ>
+static int trans_ylds(hipStream_t s, const asamd_spmv_args* a, int width, void* partials) {
+  switch (width) {
+    case 1:
+    case 2: return launch_trans_ylds<T, 2, CONJ>(s, a, partials);
+    case 4: return launch_trans_ylds<T, 4, CONJ>(s, a, partials);
+    case 8: return launch_trans_ylds<T, 8, CONJ>(s, a, partials);
+    case 16: return launch_trans_ylds<T, 16, CONJ>(s, a, partials);
+    case 32: return launch_trans_ylds<T, 32, CONJ>(s, a, partials);
+    case 64: return launch_trans_ylds<T, 64, CONJ>(s, a, partials);
+    default: return hipErrorInvalidValue;
+  }
+}
+// partials: asamd_spmv_trans_ylds_bytes(dtype, m, n) bytes of per-call scratch
+extern "C" int asamd_spmv_trans_ylds(hipStream_t s, const asamd_spmv_args* a, int32_t width, int32_t conj, void* partials) {
+  if (!a || !partials) return hipErrorInvalidValue;
+  if (asamd_spmv_trans_ylds_bytes(a->dtype, a->m, a->n) == 0 || a->nnz < 1) return hipErrorInvalidValue;
+  return by_dtype(a->dtype, [&](auto* tag) -> int {
+    using T = std::remove_pointer_t<decltype(tag)>;
+    if (!args_ok<T>(a) || (conj && kIsReal<T>) || (uintptr_t)partials % alignof(T)) return hipErrorInvalidValue;
+    if constexpr (!kIsReal<T>) {
+      if (conj) return trans_ylds<T, true>(s, a, width, partials);
+    }
+    return trans_ylds<T, false>(s, a, width, partials);
+  });
+}
+
 // ---- transposed product as an atomic scatter ------------------------------------------------------
 template <typename T, int W, bool CONJ>
 static void launch_trans_scatter(hipStream_t s, const asamd_spmv_args* a) {

@@ -138,7 +138,7 @@ static int xlds_sliced_ok(const asamd_csr_plan *p, int force) {
   if (!st->trusted || st->first_offset != 0 || st->m < 1 || st->nnz < 4) return 0;
   if (p->dtype != ASAMD_DTYPE_FLOAT && p->dtype != ASAMD_DTYPE_DOUBLE) return 0;
   const int slices = xlds_slices_for(p);
-  if (slices < 2 || slices > 64 || ((int64_t)slices + 1) * st->m >= (int64_t)INT32_MAX) return 0;
+  if (slices < 2 || slices > 1024 || ((int64_t)slices + 1) * st->m >= (int64_t)INT32_MAX) return 0;
   if (force) return 1;
   return st->nnz >= (1 << 22) && (double)st->nnz >= 16.0 * (double)slices * (double)st->m &&
          env_int("ALSPARSE_AMD_XLDS", 1) > 0;
@@ -357,6 +357,13 @@ static size_t algo_scratch(const asamd_csr_plan *p, int algo) {
 
 static int has_value_copy(const asamd_csr_plan *p) { return p->st.tiled_built || p->st.ell_built; }
 
+/* per-call scratch of the transposed multiply that keeps y in LDS, or 0 where the atomic scatter runs */
+static size_t trans_ylds_scratch(const asamd_csr_plan *p) {
+  const asamd_csr_stats *st = &p->st;
+  if (st->nnz < (1 << 20) || st->first_offset != 0 || env_int("ALSPARSE_AMD_XLDS", 1) <= 0) return 0;
+  return asamd_spmv_trans_ylds_bytes(p->dtype, st->m, st->n);
+}
+
 size_t asamd_csr_plan_workspace_bytes(const asamd_csr_plan *p) {
   if (!p) return 0;
   size_t need = 0;
@@ -366,6 +373,10 @@ size_t asamd_csr_plan_workspace_bytes(const asamd_csr_plan *p) {
     if (s > need) need = s;
   }
   if (has_value_copy(p)) need += align256(ASAMD_GUARD_WS_BYTES);
+  {
+    const size_t s = align256(ASAMD_GUARD_WS_BYTES) + align256(trans_ylds_scratch(p));
+    if (trans_ylds_scratch(p) && s > need) need = s;
+  }
   for (int w = 0; w < 2; ++w)
     if (p->tr[w].plan) {
       const size_t s = align256(ASAMD_GUARD_WS_BYTES) + asamd_csr_plan_workspace_bytes(p->tr[w].plan);
@@ -643,6 +654,12 @@ int asamd_csr_plan_csrmv(hipStream_t s, asamd_csr_plan *p, int32_t op, const voi
       fill_args(&at, t->plan, alpha, t->t.val, t->t.row_ptr, t->t.col_ind, x, beta, y);
       return csrmv_inner(s, t->plan, &at, ws, 0);
     }
+  }
+  /* y in LDS where it fits and the matrix is large enough for a workgroup per compute unit to pay */
+  const size_t ylds = trans_ylds_scratch(p);
+  if (ylds) {
+    void *partials = ws_take(&ws, ylds);
+    if (partials) return asamd_spmv_trans_ylds(s, &a, p->auto_width, which == 1, partials);
   }
   return asamd_spmv_trans_scatter(s, &a, p->auto_width, which == 1);
 }

@@ -238,7 +238,7 @@ def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False, vendor=Fa
     if stats.algo == capi.ASAMD_SPMV_VECTOR:
         algo += "(W=%d)" % stats.vector_width
     if transpose and not analysed:
-        algo = "scatter with atomics (no copy of the transpose)"
+        algo = "scatter with atomics (no copy of the transpose; in LDS where y fits it)"
     watched = bool(not analysed and not transpose and lib.asamd_registry_lazy_promoted(h.h, d_rp.c_ptr()))
     if watched:
         algo = "tiled two-phase behind fingerprints of row_ptr, col_ind and csr_val (laid out by the 4th call)"

@@ -146,6 +146,11 @@ int asamd_spmv_merge(hipStream_t stream, const asamd_spmv_args *a, int32_t ipt, 
  * src/kernel/dcu/level2/mv/csrmv/dcu_gemv_x_csr_trans.cpp:11-68 and dcu_gemv_c_csr_conj.cpp:22-75.
  * x has m elements.  conj != 0: complex types only. */
 int asamd_spmv_trans_scatter(hipStream_t stream, const asamd_spmv_args *a, int32_t width, int32_t conj);
+/* The same for a matrix of so few columns that y (n elements) fits a compute unit's LDS (asamd_spmv_xlds_fits):
+ * every workgroup adds up its rows' contributions in LDS and the workgroups' sums are added in order.  partials:
+ * asamd_spmv_trans_ylds_bytes(dtype, m, n) bytes of per-call scratch (0: the matrix does not suit). */
+size_t asamd_spmv_trans_ylds_bytes(int32_t dtype, int32_t m, int32_t n);
+int asamd_spmv_trans_ylds(hipStream_t stream, const asamd_spmv_args *a, int32_t width, int32_t conj, void *partials);
 
 /* ---- re-ordered copies of a CSR matrix ("layouts") and the kernels that multiply with them ------
  * A layout is a plain record of device pointers and counts, filled by its *_build call (which

@@ -32,6 +32,8 @@ SHAPES = {
     "long_and_empty": lambda rd: csr_from_lengths([0] * 300 + [9000] + [0] * 200 + [2, 4097, 4095, 0, 0, 1, 63, 64, 65],
                                                   20000, rd),
     "base_one": lambda rd: wl.uniform_rows(3000, 2500, 7, rd, base=1),
+    # 2^20 entries or more and few columns: x in LDS; without analysis the transposed operations add up in LDS
+    "tall": lambda rd: wl.uniform_rows(70000, 8000, 16, rd, base=1),
     "tiny": lambda rd: csr_from_lengths([2, 0, 1], 5, rd),
     # rows of similar lengths: the staged row-block kernel with several lanes per row
     "stencil27": lambda rd: wl.stencil3d(14, 11, 9, rd),

@@ -222,3 +222,30 @@ def test_transposed_full_size_configuration_3(gpu):
     finally:
         lib.alphasparse_dcu_destroy_mat_info(info)
         da.free()
+
+
+TALL = {
+    # >= 2^20 entries and a y (n elements) that fits a compute unit's LDS: the unanalysed transposed multiply adds
+    # up in LDS, a workgroup per compute unit, instead of scattering with global atomics
+    "uniform16_f32": lambda: wl.uniform_rows(100000, 20000, 16, np.float32),
+    "uniform40_f64_base1": lambda: wl.uniform_rows(40000, 15000, 40, np.float64, base=1),
+    "ragged_f32": lambda: csr_from_lengths(list((np.arange(60000) * 7) % 45), 30000, np.float32, seed=3),
+}
+
+
+@pytest.mark.parametrize("shape", sorted(TALL))
+def test_transposed_csrmv_without_analysis_on_tall_matrices(gpu, shape, monkeypatch):
+    a = TALL[shape]()
+    assert a.nnz >= 1 << 20
+    x, y0 = wl.uniform(a.rows, a.dtype, 3), wl.uniform(a.cols, a.dtype, 4)
+    da = DeviceCsr(a)
+    try:
+        for alpha, beta in ((1.0, 0.0), (-0.5, 2.0), (2.0, 1.0)):
+            announce("transposed csrmv, y in LDS", shape, alpha, beta)
+            y = run_csrmv_trans(gpu, da, alpha, x, beta, y0)
+            check_trans(a, alpha, x, beta, y0, y, "%s y in LDS %s" % (shape, (alpha, beta)))
+        monkeypatch.setenv("ALSPARSE_AMD_XLDS", "0")  # the scatter with global atomics, same inputs
+        y = run_csrmv_trans(gpu, da, 1.0, x, 0.0, y0)
+        check_trans(a, 1.0, x, 0.0, y0, y, "%s global atomics" % shape)
+    finally:
+        da.free()
