@@ -144,3 +144,37 @@ def test_rows_whose_columns_do_not_ascend_get_no_slices(gpu):
         check_spmv(b, 1.0, x, 0.0, y0, y, "unsorted")
     finally:
         da.free()
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_random_structures_slice_by_slice(gpu, seed):
+    """Seeded random structures over 2 .. 7 column slices: empty rows, rows that miss whole slices, rows of thousands
+    of entries, both index bases, both real types, val / col_ind off their 16-byte alignment."""
+    from helpers import run_plan_csrmv
+    rng = np.random.default_rng(4200 + seed)
+    dtype = (np.float32, np.float64)[seed % 2]
+    fill = 131072 // np.dtype(dtype).itemsize
+    cols = int(rng.integers(fill + 1, 7 * fill))
+    m = int(rng.integers(1, 4000))
+    law = seed % 3
+    if law == 0:
+        lengths = rng.integers(0, 200, size=m)
+    elif law == 1:
+        lengths = rng.geometric(1.0 / 40.0, size=m) - 1
+    else:
+        lengths = rng.integers(0, 12, size=m)
+        lengths[rng.integers(0, m, size=max(1, m // 100))] = rng.integers(1000, 9000)
+    base = int(rng.integers(0, 2))
+    a = csr_from_lengths(list(np.minimum(lengths, cols)), cols, dtype, seed=int(rng.integers(1, 1 << 30)), base=base)
+    if a.nnz < 4:
+        pytest.skip("drew a matrix of fewer than four entries")
+    x, y0 = wl.uniform(a.cols, a.dtype, 3, seed), wl.uniform(a.rows, a.dtype, 4, seed)
+    da = DeviceCsr(a, shift=int(rng.integers(0, 4)))
+    try:
+        for alpha, beta in ((1.0, 0.0), (2.0, 3.0)):
+            announce("x in LDS, sliced: random structure", seed, np.dtype(dtype).name, "cols", cols, "base", base, alpha, beta)
+            y = run_plan_csrmv(da, "xlds", alpha, x, beta, y0)
+            assert y is not None, "no slice table for a matrix with ascending columns"
+            check_spmv(a, alpha, x, beta, y0, y, "seed %d %s" % (seed, (alpha, beta)))
+    finally:
+        da.free()
