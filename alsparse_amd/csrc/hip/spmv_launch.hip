@@ -5,6 +5,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include "alsparse_amd_kernels.h"
 #include "launch_utils.hpp"
 #include "spmv_merge.hpp"
@@ -62,12 +64,7 @@ extern "C" int asamd_spmv_vector(hipStream_t s, const asamd_spmv_args* a, int32_
 }
 
 // ---- x in LDS ---------------------------------------------------------------------------------------
-extern "C" int asamd_spmv_xlds_fits(int32_t dtype, int32_t n) {
-  return n >= 1 && (int64_t)n * (int64_t)dtype_size(dtype) <= (int64_t)ASAMD_XLDS_MAX_BYTES;
-}
-
-template <typename T, int W, bool NT>
-static int launch_xlds_as(hipStream_t s, const asamd_spmv_args* a) {
+static int xlds_compute_units() {
   static const int cus = [] {
     int dev = 0, n = 0;
     if (hipGetDevice(&dev) != hipSuccess ||
@@ -75,14 +72,28 @@ static int launch_xlds_as(hipStream_t s, const asamd_spmv_args* a) {
       n = 256;
     return n;
   }();
+  return cus;
+}
+// A kernel may use more than 64 KB of dynamic LDS only after it has been told so, on every device it runs on:
+// `done` (one word per kernel: a static of the launcher's instantiation) remembers the devices.
+static hipError_t allow_full_lds(const void* kernel, std::atomic<uint64_t>& done) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return hipGetLastError();
+  if (dev >= 0 && dev < 64 && ((done.load(std::memory_order_relaxed) >> dev) & 1u)) return hipSuccess;
+  const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, ASAMD_XLDS_MAX_BYTES);
+  if (e == hipSuccess && dev >= 0 && dev < 64) done.fetch_or((uint64_t)1 << dev, std::memory_order_relaxed);
+  return e;
+}
+extern "C" int asamd_spmv_xlds_fits(int32_t dtype, int32_t n) {
+  return n >= 1 && (int64_t)n * (int64_t)dtype_size(dtype) <= (int64_t)ASAMD_XLDS_MAX_BYTES;
+}
+
+template <typename T, int W, bool NT>
+static int launch_xlds_as(hipStream_t s, const asamd_spmv_args* a) {
+  const int cus = xlds_compute_units();
   const size_t lds = ((size_t)a->n * sizeof(T) + 15) / 16 * 16;
-  static size_t allowed = 0;  // (per instantiation)
-  if (lds > allowed) {
-    const hipError_t e = hipFuncSetAttribute((const void*)spmv_xlds_kernel<T, W, NT>,
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, ASAMD_XLDS_MAX_BYTES);
-    if (e != hipSuccess) return e;
-    allowed = ASAMD_XLDS_MAX_BYTES;
-  }
+  static std::atomic<uint64_t> allowed{0};
+  if (const hipError_t e = allow_full_lds((const void*)spmv_xlds_kernel<T, W, NT>, allowed); e != hipSuccess) return e;
   constexpr int rows_per_trip = (kXldsThreads / W) * kXldsRows;
   int64_t grid = ((int64_t)a->m + rows_per_trip - 1) / rows_per_trip;
   if (grid > cus) grid = cus;
@@ -101,22 +112,11 @@ static int launch_xlds(hipStream_t s, const asamd_spmv_args* a) {
 // `partials`, slices * m elements, and are added up by a second kernel), or null.
 template <typename T, int W, bool NT>
 static int launch_xlds4_as(hipStream_t s, const asamd_spmv_args* a, const asamd_xlds_layout* L, void* partials) {
-  static const int cus = [] {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-      n = 256;
-    return n;
-  }();
+  const int cus = xlds_compute_units();
   const int slices = L ? L->slices : 1, slice_cols = L ? L->slice_cols : a->n;
   const size_t lds = ((size_t)slice_cols * sizeof(T) + 15) / 16 * 16;
-  static size_t allowed = 0;  // (per instantiation)
-  if (lds > allowed) {
-    const hipError_t e = hipFuncSetAttribute((const void*)spmv_xlds4_kernel<T, W, NT>,
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, ASAMD_XLDS_MAX_BYTES);
-    if (e != hipSuccess) return e;
-    allowed = ASAMD_XLDS_MAX_BYTES;
-  }
+  static std::atomic<uint64_t> allowed{0};
+  if (const hipError_t e = allow_full_lds((const void*)spmv_xlds4_kernel<T, W, NT>, allowed); e != hipSuccess) return e;
   constexpr int rows_per_trip = (kXldsThreads / W) * kXlds4Rows;
   int64_t grid = ((int64_t)a->m + rows_per_trip - 1) / rows_per_trip;
   const int64_t per_slice = cus / slices > 0 ? cus / slices : 1;  // the workgroups share the compute units
@@ -368,16 +368,6 @@ extern "C" int asamd_spmv_merge(hipStream_t s, const asamd_spmv_args* a, int32_t
 }
 
 // ---- transposed product with y in LDS --------------------------------------------------------------
-static int xlds_compute_units() {
-  static const int cus = [] {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-      n = 256;
-    return n;
-  }();
-  return cus;
-}
 // workgroups of the launch: as many as compute units, fewer for few rows (lanes per row do not matter: the least)
 static int64_t trans_ylds_groups(int32_t m) {
   const int64_t rows_per_trip = (int64_t)(kXldsThreads / kWave) * kXldsRows;
@@ -392,13 +382,9 @@ extern "C" size_t asamd_spmv_trans_ylds_bytes(int32_t dtype, int32_t m, int32_t 
 template <typename T, int W, bool CONJ>
 static int launch_trans_ylds(hipStream_t s, const asamd_spmv_args* a, void* partials) {
   const size_t lds = ((size_t)a->n * sizeof(T) + 15) / 16 * 16;
-  static size_t allowed = 0;  // (per instantiation)
-  if (lds > allowed) {
-    const hipError_t e = hipFuncSetAttribute((const void*)spmv_trans_ylds_kernel<T, W, CONJ>,
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, ASAMD_XLDS_MAX_BYTES);
-    if (e != hipSuccess) return e;
-    allowed = ASAMD_XLDS_MAX_BYTES;
-  }
+  static std::atomic<uint64_t> allowed{0};
+  if (const hipError_t e = allow_full_lds((const void*)spmv_trans_ylds_kernel<T, W, CONJ>, allowed); e != hipSuccess)
+    return e;
   const int64_t grid = trans_ylds_groups(a->m);
   spmv_trans_ylds_kernel<T, W, CONJ><<<(unsigned)grid, kXldsThreads, lds, s>>>(
       a->m, a->n, scalar_of<T>(a->alpha), (const T*)a->val, a->row_ptr, a->col_ind, (const T*)a->x, (T*)partials, a->base);
