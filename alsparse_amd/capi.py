@@ -147,7 +147,8 @@ class asamd_spmv_args(Structure):  # include/alsparse_amd_kernels.h
 
 class asamd_xlds_layout(Structure):  # include/alsparse_amd_kernels.h
     _fields_ = [("seg", c_void_p), ("slices", c_int32), ("slice_cols", c_int32), ("m", c_int32),
-                ("device_bytes", ctypes.c_int64)]
+                ("device_bytes", ctypes.c_int64), ("off", c_void_p), ("val", c_void_p), ("col", c_void_p),
+                ("dtype", c_int32), ("nnz", c_int32), ("base", c_int32)]
 
 
 class asamd_dense_strides(Structure):
@@ -356,7 +357,8 @@ _COMMON = {
     "asamd_gather_values": [_P, _I, _I, _I, _P, _P, _P, _P],
     "asamd_spmv_xlds": [_P, _P, _I],
     "asamd_spmv_xlds_fits": [_I, _I],
-    "asamd_xlds_build": [_P, _I, _I, _I, _I, _I, _P, _P, _P],
+    "asamd_xlds_build": [_P, _I, _I, _I, _I, _I, _P, _P, _P, _P],
+    "asamd_xlds_refresh_values": [_P, _P, _P, _P],
     "asamd_xlds_free": [_P],
     "asamd_spmv_xlds_sliced": [_P, POINTER(asamd_spmv_args), _I, _P, _P],
     "asamd_csr2ell_gated": [_P, _I, _I, _P, _P, _P, _I, _I, _I, _P, _P, _P],

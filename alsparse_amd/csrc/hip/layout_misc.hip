@@ -174,13 +174,31 @@ extern "C" int asamd_spmv_hot(hipStream_t s, const asamd_spmv_args* a, const asa
 }
 
 // ---- column slices for the kernel that holds x in LDS ----------------------------------------------
+template <typename T>
+static hipError_t xlds_copy_pieces(hipStream_t stream, const asamd_xlds_layout* L, const void* val, const int32_t* col_ind,
+                                   const int32_t* gate) {
+  const int64_t pieces = (int64_t)L->slices * L->m;
+  int64_t grid = (pieces + 31) / 32;
+  if (grid > (1 << 20)) grid = 1 << 20;
+  xlds_copy_pieces_kernel<T><<<(unsigned)grid, 256, 0, stream>>>(pieces, L->m, L->slice_cols, L->base, L->seg, L->off,
+                                                                (const T*)val, col_ind, (T*)L->val, L->col, gate);
+  return hipGetLastError();
+}
+static hipError_t xlds_copy_pieces_dtype(hipStream_t stream, const asamd_xlds_layout* L, const void* val,
+                                         const int32_t* col_ind, const int32_t* gate) {
+  if (L->dtype == ASAMD_DTYPE_FLOAT) return xlds_copy_pieces<float>(stream, L, val, col_ind, gate);
+  if (L->dtype == ASAMD_DTYPE_DOUBLE) return xlds_copy_pieces<double>(stream, L, val, col_ind, gate);
+  return hipErrorInvalidValue;
+}
+
 // As few slices as hold x in ASAMD_XLDS_MAX_BYTES each, of equal width (a multiple of 64 columns).
 extern "C" int asamd_xlds_build(hipStream_t stream, int32_t dtype, int32_t m, int32_t n, int32_t nnz, int32_t base,
-                                const int32_t* row_ptr, const int32_t* col_ind, asamd_xlds_layout* L) {
+                                const int32_t* row_ptr, const int32_t* col_ind, const void* val, asamd_xlds_layout* L) {
   if (!L) return hipErrorInvalidValue;
   *L = asamd_xlds_layout{};
   const int vs = dtype_size(dtype);
   if (!row_ptr || !col_ind || m < 1 || n < 1 || nnz < 1 || vs <= 0) return hipErrorInvalidValue;
+  if (val && dtype != ASAMD_DTYPE_FLOAT && dtype != ASAMD_DTYPE_DOUBLE) return hipErrorInvalidValue;
   const int64_t fill = (int64_t)ASAMD_XLDS_MAX_BYTES / vs;  // columns per LDS fill
   const int64_t slices = ((int64_t)n + fill - 1) / fill;
   if (slices < 2 || slices > 1024 || (slices + 1) * (int64_t)m >= (int64_t)INT32_MAX) return hipSuccess;  // no layout
@@ -209,7 +227,36 @@ extern "C" int asamd_xlds_build(hipStream_t stream, int32_t dtype, int32_t m, in
       L->slices = (int32_t)slices;
       L->slice_cols = (int32_t)width;
       L->m = m;
+      L->dtype = dtype;
+      L->nnz = nnz;
+      L->base = base;
       L->device_bytes = count * (int64_t)sizeof(int);
+    }
+    if (e == hipSuccess && val) {
+      // the copy: offsets (a running sum of the pieces' lengths, slice by slice), then the entries; four entries
+      // of padding so that a 16-byte load of the last piece stays inside
+      const int64_t pieces = slices * (int64_t)m;
+      const size_t off_bytes = ((size_t)pieces + 1) * sizeof(int), val_bytes = ((size_t)nnz + 4) * (size_t)vs,
+                   col_bytes = ((size_t)nnz + 4) * sizeof(uint16_t);
+      hipError_t c = hipMalloc(&L->off, off_bytes);
+      if (c == hipSuccess) c = hipMalloc(&L->val, val_bytes);
+      if (c == hipSuccess) c = hipMalloc(&L->col, col_bytes);
+      if (c == hipSuccess) c = hipMemsetAsync((char*)L->val + (size_t)nnz * vs, 0, 4 * (size_t)vs, stream);
+      if (c == hipSuccess) c = hipMemsetAsync(L->col + nnz, 0, 4 * sizeof(uint16_t), stream);
+      if (c == hipSuccess) c = scan_piece_lengths(stream, L->seg, m, pieces, L->off);
+      if (c == hipSuccess) c = xlds_copy_pieces_dtype(stream, L, val, col_ind, nullptr);
+      if (c == hipSuccess) c = hipStreamSynchronize(stream);
+      if (c == hipSuccess) {
+        L->device_bytes += (int64_t)(off_bytes + val_bytes + col_bytes);
+      } else {
+        // (no room for the copy, say: the table of offsets alone still serves)
+        if (c == hipErrorOutOfMemory) (void)hipGetLastError();
+        if (L->off) (void)hipFree(L->off);
+        if (L->val) (void)hipFree(L->val);
+        if (L->col) (void)hipFree(L->col);
+        L->off = nullptr, L->val = nullptr, L->col = nullptr;
+        if (c != hipErrorOutOfMemory) e = c;
+      }
     }
   }
   if (d_flag) (void)hipFree(d_flag);
@@ -217,9 +264,18 @@ extern "C" int asamd_xlds_build(hipStream_t stream, int32_t dtype, int32_t m, in
   return e;
 }
 
+extern "C" int asamd_xlds_refresh_values(hipStream_t stream, const asamd_xlds_layout* L, const void* val,
+                                         const int32_t* gate) {
+  if (!L || !L->seg || !L->off || !L->val || !val) return hipErrorInvalidValue;
+  return xlds_copy_pieces_dtype(stream, L, val, nullptr, gate);
+}
+
 extern "C" void asamd_xlds_free(asamd_xlds_layout* L) {
   if (!L) return;
   if (L->seg) (void)hipFree(L->seg);
+  if (L->off) (void)hipFree(L->off);
+  if (L->val) (void)hipFree(L->val);
+  if (L->col) (void)hipFree(L->col);
   *L = asamd_xlds_layout{};
 }
 

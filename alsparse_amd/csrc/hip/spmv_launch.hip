@@ -127,9 +127,20 @@ static int launch_xlds4_as(hipStream_t s, const asamd_spmv_args* a, const asamd_
         a->col_ind, (const T*)a->x, scalar_of<T>(a->beta), (T*)a->y, 0, a->base);
     return hipGetLastError();
   }
-  spmv_xlds4_kernel<T, W, NT><<<dim3((unsigned)grid, (unsigned)slices), kXldsThreads, lds, s>>>(
-      a->m, a->n, slice_cols, (int64_t)a->nnz, T(1), (const T*)a->val, L->seg, L->seg + a->m, (int64_t)a->m, a->col_ind,
-      (const T*)a->x, T(0), (T*)partials, (int64_t)a->m, a->base);
+  if (L->val) {
+    // the copy, slice by slice: a CSR matrix per slice, base 0, 16-bit columns
+    static std::atomic<uint64_t> allowed_copy{0};
+    if (const hipError_t e = allow_full_lds((const void*)spmv_xlds4_kernel<T, W, NT, unsigned short>, allowed_copy);
+        e != hipSuccess)
+      return e;
+    spmv_xlds4_kernel<T, W, NT, unsigned short><<<dim3((unsigned)grid, (unsigned)slices), kXldsThreads, lds, s>>>(
+        a->m, a->n, slice_cols, (int64_t)a->nnz + 4, T(1), (const T*)L->val, L->off, L->off + 1, (int64_t)a->m, L->col,
+        (const T*)a->x, T(0), (T*)partials, (int64_t)a->m, 0);
+  } else {
+    spmv_xlds4_kernel<T, W, NT><<<dim3((unsigned)grid, (unsigned)slices), kXldsThreads, lds, s>>>(
+        a->m, a->n, slice_cols, (int64_t)a->nnz, T(1), (const T*)a->val, L->seg, L->seg + a->m, (int64_t)a->m,
+        a->col_ind, (const T*)a->x, T(0), (T*)partials, (int64_t)a->m, a->base);
+  }
   xlds_slices_sum_kernel<T><<<(unsigned)(((int64_t)a->m + 255) / 256), 256, 0, s>>>(
       a->m, slices, scalar_of<T>(a->alpha), (const T*)partials, scalar_of<T>(a->beta), (T*)a->y);
   return hipGetLastError();
@@ -139,6 +150,9 @@ template <typename T, int W>
 static int launch_xlds4(hipStream_t s, const asamd_spmv_args* a, const asamd_xlds_layout* L = nullptr,
                         void* partials = nullptr) {
   const int64_t pieces = (int64_t)a->m * (L ? L->slices : 1);
+  // (the pieces of a copy are neighbours in memory and of many lengths: what one piece's load leaves of a cache line,
+  // the next piece or the piece's own second load takes from the caches)
+  if (L && L->val) return launch_xlds4_as<T, W, false>(s, a, L, partials);
   return (int64_t)a->nnz <= pieces * 4 * W ? launch_xlds4_as<T, W, true>(s, a, L, partials)
                                            : launch_xlds4_as<T, W, false>(s, a, L, partials);
 }
@@ -183,6 +197,8 @@ extern "C" int asamd_spmv_xlds_sliced(hipStream_t s, const asamd_spmv_args* a, i
     return hipErrorInvalidValue;
   if ((int64_t)L->slice_cols * dtype_size(a->dtype) > (int64_t)ASAMD_XLDS_MAX_BYTES ||
       (int64_t)L->slices * L->slice_cols < (int64_t)a->n)
+    return hipErrorInvalidValue;
+  if (L->val && (!L->off || !L->col || L->dtype != a->dtype || L->nnz != a->nnz || L->slice_cols > 65536))
     return hipErrorInvalidValue;
   return by_dtype(a->dtype, [&](auto* tag) -> int {
     using T = std::remove_pointer_t<decltype(tag)>;

@@ -177,15 +177,27 @@ struct XldsVal4 {
   typedef T type __attribute__((ext_vector_type(4), aligned(4)));
 };
 
-template <typename T, bool NT>
-__device__ __forceinline__ XldsPiece<T> xlds_load_piece(const T* __restrict__ val, const int* __restrict__ col_ind,
+typedef unsigned short XldsShort4 __attribute__((ext_vector_type(4), aligned(2)));
+template <typename C>
+struct XldsCol4 {
+  typedef XldsInt4 type;
+};
+template <>
+struct XldsCol4<unsigned short> {
+  typedef XldsShort4 type;
+};
+
+// C: int (the caller's column numbers) or unsigned short (columns counted from their slice's first, in a copy)
+template <typename T, bool NT, typename C = int>
+__device__ __forceinline__ XldsPiece<T> xlds_load_piece(const T* __restrict__ val, const C* __restrict__ col_ind,
                                                         int64_t j, int64_t limit) {
   // j > limit - 4: the window [limit - 4, limit) instead, its entries moved down by j - (limit - 4)
   const int64_t at = j + 4 <= limit ? j : limit - 4;
   const int shift = (int)(j - at);
   typedef typename XldsVal4<T>::type V4;
-  const XldsInt4 c = NT ? __builtin_nontemporal_load(reinterpret_cast<const XldsInt4*>(col_ind + at))
-                        : *reinterpret_cast<const XldsInt4*>(col_ind + at);
+  typedef typename XldsCol4<C>::type C4;
+  const C4 c = NT ? __builtin_nontemporal_load(reinterpret_cast<const C4*>(col_ind + at))
+                  : *reinterpret_cast<const C4*>(col_ind + at);
   const V4 v = NT ? __builtin_nontemporal_load(reinterpret_cast<const V4*>(val + at))
                   : *reinterpret_cast<const V4*>(val + at);
   XldsPiece<T> p;
@@ -193,7 +205,7 @@ __device__ __forceinline__ XldsPiece<T> xlds_load_piece(const T* __restrict__ va
     p.c[0] = c.x, p.c[1] = c.y, p.c[2] = c.z, p.c[3] = c.w;
     p.v[0] = v.x, p.v[1] = v.y, p.v[2] = v.z, p.v[3] = v.w;
   } else {
-    const int cc[4] = {c.x, c.y, c.z, c.w};
+    const int cc[4] = {(int)c.x, (int)c.y, (int)c.z, (int)c.w};
     const T vv[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -214,13 +226,17 @@ __device__ __forceinline__ XldsPiece<T> xlds_load_piece(const T* __restrict__ va
 // ends: row_lo / row_hi then point at a table of slices + 1 rows of m offsets (offsets_per_slice = m apart; in
 // row_ptr's convention, base included), and the kernel writes the slice's sums (alpha = 1, beta = 0) to
 // y + blockIdx.y * y_per_slice for a second kernel to add up.  One slice: row_lo = row_ptr, row_hi = row_ptr + 1.
-template <typename T, int W, bool NT>
+//
+// A copy of the entries slice by slice (C = unsigned short): every slice is a CSR matrix of its own in val / col_ind,
+// columns counted from the slice's first one; row_lo points at slices * m + 1 offsets into the copy (base 0,
+// offsets_per_slice = m, row_hi = row_lo + 1) and the pieces of consecutive rows are consecutive in memory.
+template <typename T, int W, bool NT, typename C = int>
 __global__ __launch_bounds__(kXldsThreads) void spmv_xlds4_kernel(int m, int n_total, int slice_cols, int64_t limit,
                                                                   T alpha, const T* __restrict__ val,
                                                                   const int* __restrict__ row_lo,
                                                                   const int* __restrict__ row_hi,
                                                                   int64_t offsets_per_slice,
-                                                                  const int* __restrict__ col_ind,
+                                                                  const C* __restrict__ col_ind,
                                                                   const T* __restrict__ x, T beta, T* __restrict__ y,
                                                                   int64_t y_per_slice, int base) {
   extern __shared__ __align__(16) unsigned char xlds_bytes[];
@@ -269,8 +285,8 @@ __global__ __launch_bounds__(kXldsThreads) void spmv_xlds4_kernel(int m, int n_t
     for (int i = threadIdx.x; i < n; i += kXldsThreads) xs[i] = x[i];
   }
   __syncthreads();
-  const int first_col = base + col0;
-  const T* __restrict__ xb = xs - first_col;  // (indexed with the caller's column numbers)
+  const int first_col = sizeof(C) == 2 ? 0 : base + col0;
+  const T* __restrict__ xb = xs - first_col;  // (indexed with the column numbers as the arrays hold them)
   // the lane's (up to four) entries from position j of a row that ends at e, times x, added up
   auto piece_sum = [&](const XldsPiece<T>& p, int j, int e, T sum) __attribute__((always_inline)) {
 #pragma unroll
@@ -293,7 +309,7 @@ __global__ __launch_bounds__(kXldsThreads) void spmv_xlds4_kernel(int m, int n_t
       const int j = start[k] + 4 * lane;
       // (a lane with nothing to do, or a row for the wave: the matrix' first piece, never summed)
       const bool mine = j < end[k] && end[k] - start[k] <= kWaveLen;
-      p[k] = xlds_load_piece<T, NT>(val, col_ind, mine ? (int64_t)j : 0, limit);
+      p[k] = xlds_load_piece<T, NT, C>(val, col_ind, mine ? (int64_t)j : 0, limit);
     }
 #pragma unroll
     for (int k = 0; k < K; ++k) {
@@ -305,7 +321,7 @@ __global__ __launch_bounds__(kXldsThreads) void spmv_xlds4_kernel(int m, int n_t
     for (int k = 0; k < K; ++k) {
       if (end[k] - start[k] > kWaveLen) continue;
       for (int j = start[k] + 4 * lane + 4 * W; j < end[k]; j += 4 * W)
-        sum[k] = piece_sum(xlds_load_piece<T, false>(val, col_ind, j, limit), j, end[k], sum[k]);
+        sum[k] = piece_sum(xlds_load_piece<T, false, C>(val, col_ind, j, limit), j, end[k], sum[k]);
     }
 #pragma unroll
     for (int k = 0; k < K; ++k) {
@@ -323,7 +339,7 @@ __global__ __launch_bounds__(kXldsThreads) void spmv_xlds4_kernel(int m, int n_t
         const int s = __builtin_amdgcn_readlane(start[k], owner), e = __builtin_amdgcn_readlane(end[k], owner);
         T acc = T(0);
         for (int j = s + 4 * wave_lane; j < e; j += 4 * kWave)
-          acc = piece_sum(xlds_load_piece<T, false>(val, col_ind, j, limit), j, e, acc);
+          acc = piece_sum(xlds_load_piece<T, false, C>(val, col_ind, j, limit), j, e, acc);
         acc = group_sum<kWave>(acc);
         if (wave_lane == 0) {
           const int64_t r = row0 + (int64_t)k * kGroups + (threadIdx.x / kWave) * (kWave / W) + owner / W;
@@ -455,6 +471,27 @@ static __global__ __launch_bounds__(256) void xlds_rows_ascend_kernel(int m, con
   bool bad = false;
   for (int j = row_ptr[r] - base + (int)(threadIdx.x % kWave); j + 1 < end; j += kWave) bad |= col_ind[j] > col_ind[j + 1];
   if (__ballot(bad) != 0 && threadIdx.x % kWave == 0) atomicOr(unsorted, 1);
+}
+// The entries slice by slice: piece i = s * m + r (slice s of row r) goes from [seg[i], seg[i + m]) of the caller's
+// arrays to off[i] .. of the copy, eight lanes per piece; col_ind == nullptr: the values only.  gate: nullptr, or a
+// word that is 0 when there is nothing to do.
+template <typename T>
+__global__ __launch_bounds__(256) void xlds_copy_pieces_kernel(int64_t pieces, int m, int slice_cols, int base,
+                                                               const int* __restrict__ seg, const int* __restrict__ off,
+                                                               const T* __restrict__ val, const int* __restrict__ col_ind,
+                                                               T* __restrict__ cval, unsigned short* __restrict__ ccol,
+                                                               const int* __restrict__ gate) {
+  if (gate && *gate == 0) return;
+  constexpr int kLanes = 8;
+  const int lane = threadIdx.x % kLanes;
+  for (int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) / kLanes; i < pieces; i += (int64_t)gridDim.x * (256 / kLanes)) {
+    const int from = seg[i] - base, len = seg[i + m] - base - from, to = off[i];
+    const int first_col = base + (int)(i / m) * slice_cols;
+    for (int k = lane; k < len; k += kLanes) {
+      cval[to + k] = val[from + k];
+      if (col_ind) ccol[to + k] = (unsigned short)(col_ind[from + k] - first_col);
+    }
+  }
 }
 // y = alpha * (the slices' sums, added in the order of the slices) + beta * y
 template <typename T>

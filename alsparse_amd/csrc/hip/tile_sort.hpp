@@ -10,4 +10,6 @@ hipError_t sort_pairs_u32(hipStream_t stream, unsigned* keys_in, unsigned* keys_
 // the same with 64-bit values (an entry's value and local indices travel with its key)
 hipError_t sort_pairs_u32_u64(hipStream_t stream, unsigned* keys_in, unsigned* keys_out, unsigned long long* vals_in,
                               unsigned long long* vals_out, size_t n, unsigned end_bit);
+// off[i] = seg[0 + m] - seg[0] + ... + seg[i - 1 + m] - seg[i - 1] for i = 0 .. pieces; waits for the stream
+hipError_t scan_piece_lengths(hipStream_t stream, const int* seg, int m, long long pieces, int* off);
 }

@@ -32,6 +32,7 @@ struct asamd_csr_plan {
   asamd_hot_layout hot;
   asamd_binned_layout binned;
   asamd_xlds_layout xlds;  /* column slices for the kernel that holds x in LDS (an x of several LDS fills) */
+  int xlds_copy_wanted;    /* the slices are to come with a copy of the entries (known before they are laid out) */
   void *d_eval;            /* ELL copy: ell_width * m values, column-major */
   int32_t *d_ecol;         /* ... and zero-based columns */
   const void *copy_val_src; /* the value array that the tiled / ELL copy was taken from */
@@ -133,14 +134,17 @@ static int xlds_slices_for(const asamd_csr_plan *p) {
   const int64_t x_bytes = (int64_t)p->st.n * (int64_t)p->val_size;
   return (int)((x_bytes + ASAMD_XLDS_MAX_BYTES - 1) / ASAMD_XLDS_MAX_BYTES);
 }
-static int xlds_sliced_ok(const asamd_csr_plan *p, int force) {
+/* With a copy of the entries slice by slice the pieces of consecutive rows are neighbours in memory and a piece of
+ * six entries is long enough (ALSPARSE_AMD_XLDS_COPY=0: never a copy). */
+#define ALGO_XLDS_IN_PLACE 64 /* internal: the slices over the caller's arrays although the plan holds a copy */
+static int xlds_sliced_ok(const asamd_csr_plan *p, int force, int copy) {
   const asamd_csr_stats *st = &p->st;
   if (!st->trusted || st->first_offset != 0 || st->m < 1 || st->nnz < 4) return 0;
   if (p->dtype != ASAMD_DTYPE_FLOAT && p->dtype != ASAMD_DTYPE_DOUBLE) return 0;
   const int slices = xlds_slices_for(p);
   if (slices < 2 || slices > 1024 || ((int64_t)slices + 1) * st->m >= (int64_t)INT32_MAX) return 0;
   if (force) return 1;
-  return st->nnz >= (1 << 22) && (double)st->nnz >= 16.0 * (double)slices * (double)st->m &&
+  return st->nnz >= (1 << 22) && (double)st->nnz >= (copy ? 6.0 : 16.0) * (double)slices * (double)st->m &&
          env_int("ALSPARSE_AMD_XLDS", 1) > 0;
 }
 
@@ -355,7 +359,13 @@ static size_t algo_scratch(const asamd_csr_plan *p, int algo) {
   }
 }
 
-static int has_value_copy(const asamd_csr_plan *p) { return p->st.tiled_built || p->st.ell_built; }
+static int has_value_copy(const asamd_csr_plan *p) {
+  return p->st.tiled_built || p->st.ell_built || p->xlds.val != NULL;
+}
+/* the families whose kernels read values that the plan keeps */
+static int holds_values(const asamd_csr_plan *p, int algo) {
+  return algo == ASAMD_SPMV_TILED || algo == ASAMD_SPMV_ELL || (algo == ASAMD_SPMV_XLDS && p->xlds.val != NULL);
+}
 
 /* per-call scratch of the transposed multiply that keeps y in LDS, or 0 where the atomic scatter runs */
 static size_t trans_ylds_scratch(const asamd_csr_plan *p) {
@@ -485,12 +495,22 @@ static int run_algo(hipStream_t s, const asamd_csr_plan *p, int algo, const asam
       return asamd_spmv_stream(s, a, stream_group(p, 0), st->max_len, st->first_offset);
     case ASAMD_SPMV_SCALAR:
       return asamd_spmv_scalar(s, a);
+    case ALGO_XLDS_IN_PLACE:
     case ASAMD_SPMV_XLDS:
       if (p->xlds.seg) {
         void *partials = ws_take(&ws, (size_t)p->xlds.slices * (size_t)st->m * vs);
         if (!partials) return -1;
         const double piece = (double)st->nnz / ((double)st->m * (double)p->xlds.slices);
-        return asamd_spmv_xlds_sliced(s, a, width_for_mean(piece), &p->xlds, partials);
+        asamd_xlds_layout view = p->xlds;
+        if (algo == ALGO_XLDS_IN_PLACE) view.val = NULL;
+        if (view.val) {
+          /* the copy's pieces: two loads for a piece of mean length beat one load with half of its lanes idle
+           * (pieces of 8 / 12 / 32 / 37 / 50 entries: 8 / 8 / 16 / 32 / 32 entries per load measured best) */
+          int width = 8;
+          while (width < 64 && 2 * width <= 0.9 * piece) width *= 2;
+          return asamd_spmv_xlds_sliced(s, a, width, &view, partials);
+        }
+        return asamd_spmv_xlds_sliced(s, a, width_for_mean(piece), &view, partials);
       }
       return asamd_spmv_xlds(s, a, p->auto_width);
     case ASAMD_SPMV_BINNED: {
@@ -530,7 +550,7 @@ static int run_algo(hipStream_t s, const asamd_csr_plan *p, int algo, const asam
   }
 }
 
-/* Gathers the plan's tiled / ELL copy again from val; gate: NULL, or the value guard's flag. */
+/* Gathers the plan's tiled / ELL / slice-by-slice copy again from val; gate: NULL, or the value guard's flag. */
 static hipError_t refresh_main(hipStream_t s, asamd_csr_plan *p, const int32_t *rp, const int32_t *ci, const void *val,
                                const int32_t *gate) {
   const asamd_csr_stats *st = &p->st;
@@ -540,6 +560,7 @@ static hipError_t refresh_main(hipStream_t s, asamd_csr_plan *p, const int32_t *
   if (e == hipSuccess && st->ell_built)
     e = (hipError_t)asamd_csr2ell_gated(s, p->val_size, st->m, val, rp, ci, st->base, 0, st->ell_width, p->d_eval,
                                         p->d_ecol, gate);
+  if (e == hipSuccess && p->xlds.val) e = (hipError_t)asamd_xlds_refresh_values(s, &p->xlds, val, gate);
   return e;
 }
 
@@ -554,19 +575,20 @@ static hipError_t refresh_trans(hipStream_t s, asamd_csr_plan *p, int which, con
 static int csrmv_inner(hipStream_t s, asamd_csr_plan *p, const asamd_spmv_args *a, ws_cursor ws, int guard) {
   const asamd_csr_stats *st = &p->st;
   int algo = st->algo;
-  /* The tiled and ELL copies hold the values of the array they were built from.  A multiply that brings
-   * another value array (same structure, new numbers) must not see the old ones: it runs the kernel that
-   * the row statistics alone would pick. */
-  if ((algo == ASAMD_SPMV_TILED || algo == ASAMD_SPMV_ELL) && p->copy_val_src && a->val != p->copy_val_src)
-    algo = p->struct_algo;
+  /* The tiled, ELL and slice-by-slice copies hold the values of the array they were built from.  A multiply that
+   * brings another value array (same structure, new numbers) must not see the old ones: it runs the kernel that
+   * the row statistics alone would pick (the column slices: over the caller's arrays). */
+  if (holds_values(p, algo) && p->copy_val_src && a->val != p->copy_val_src)
+    algo = algo == ASAMD_SPMV_XLDS ? ALGO_XLDS_IN_PLACE : p->struct_algo;
   algo = settle_algo(p, algo, a->val, a->col_ind);
-  if ((algo == ASAMD_SPMV_TILED || algo == ASAMD_SPMV_ELL) && guard && st->value_check) {
+  if (holds_values(p, algo) && guard && st->value_check) {
     /* Values changed IN PLACE under the copy: fingerprint, compare, gather again if need be, and only
      * then record the new fingerprint -- a multiply on another stream that reads the recorded word
      * either finds the old one (and gathers the same values again itself) or finds the copy done. */
     void *g = ws_take(&ws, ASAMD_GUARD_WS_BYTES);
     if (!g) {
-      algo = settle_algo(p, p->struct_algo, a->val, a->col_ind); /* no room to check the copy: do not use it */
+      /* no room to check the copy: do not use it */
+      algo = algo == ASAMD_SPMV_XLDS ? ALGO_XLDS_IN_PLACE : settle_algo(p, p->struct_algo, a->val, a->col_ind);
     } else {
       int e = asamd_value_guard(s, a->val, (size_t)st->nnz * (size_t)p->val_size, st->value_check == 2, p->d_fp, g);
       if (e == hipSuccess) e = (int)refresh_main(s, p, a->row_ptr, a->col_ind, a->val, ASAMD_GUARD_FLAG(g));
@@ -971,7 +993,13 @@ static double model_ms(const asamd_csr_plan *p, int algo) {
       const double one = nnz * (1.15 + 0.1875 * vs) * 1e-9;
       const int slices = p->xlds.seg ? p->xlds.slices : (asamd_spmv_xlds_fits(p->dtype, st->n) ? 1 : xlds_slices_for(p));
       if (slices < 2) return one;
-      return one * (1.0 + 22.0 * (double)slices / mean) + (double)slices * m * 3.0 * vs / 4.0e9;
+      const double sums = (double)slices * m * 3.0 * vs / 4.0e9;
+      if (p->xlds.seg ? p->xlds.val != NULL : p->xlds_copy_wanted) {
+        /* the copy (16-bit columns, neighbouring pieces), measured with pieces of 50 / 32 / 12.5 / 8 entries, fp32:
+         * 1.98 / 2.09 / 2.69 / 3.34 ps per entry, the slices' sums included; 37 entries, fp64: 3.03 */
+        return 0.92 * one + (double)slices * m * 13.0e-9;
+      }
+      return one * (1.0 + 22.0 * (double)slices / mean) + sums;
     }
     case ASAMD_SPMV_ELL: {
       const double ell_bytes = m * (double)st->max_len * (4.0 + vs) + (n + m) * vs;
@@ -1177,13 +1205,15 @@ static hipError_t plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t 
     st->lines_per_entry_wave = probe[0];
     st->lines_per_entry_segment = probe[1];
   }
-  if (col_ind && nnz > 0 && trusted != 3 && xlds_sliced_ok(p, trusted == 2)) {
+  p->xlds_copy_wanted = val != NULL && env_int("ALSPARSE_AMD_XLDS_COPY", 1) > 0;
+  if (col_ind && nnz > 0 && trusted != 3 && xlds_sliced_ok(p, trusted == 2, p->xlds_copy_wanted)) {
     /* x in LDS slice by slice, if the model expects it to beat the structural choice by a fifth (no probe: no
      * estimate of that choice, and no slices) */
     const int wanted = trusted == 2 || (st->lines_per_entry_wave > 0.f &&
                                         model_ms(p, ASAMD_SPMV_XLDS) < 0.9 * model_ms(p, p->auto_algo));
     if (wanted) {
-      e = (hipError_t)asamd_xlds_build(stream, p->dtype, m, n, nnz, base, row_ptr, col_ind, &p->xlds);
+      e = (hipError_t)asamd_xlds_build(stream, p->dtype, m, n, nnz, base, row_ptr, col_ind,
+                                       p->xlds_copy_wanted ? val : NULL, &p->xlds);
       if (e == hipErrorOutOfMemory) {
         (void)hipGetLastError();
         e = hipSuccess;
@@ -1191,6 +1221,12 @@ static hipError_t plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t 
       if (e != hipSuccess) {
         asamd_csr_plan_destroy(p);
         return e;
+      }
+      if (p->xlds.seg && !p->xlds.val && p->xlds_copy_wanted && trusted != 2) {
+        /* no room for the copy: the table alone, if it still pays */
+        p->xlds_copy_wanted = 0;
+        if (!xlds_sliced_ok(p, 0, 0) || !(model_ms(p, ASAMD_SPMV_XLDS) < 0.9 * model_ms(p, p->auto_algo)))
+          asamd_xlds_free(&p->xlds);
       }
       st->xlds_slices = p->xlds.seg ? p->xlds.slices : 0;
       if (p->xlds.seg && trusted != 2) {

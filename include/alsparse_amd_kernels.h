@@ -105,14 +105,25 @@ int asamd_spmv_xlds(hipStream_t stream, const asamd_spmv_args *a, int32_t width)
  * piece of the caller's arrays, so the layout is a table of offsets only -- seg[s * m + r], s = 0 .. slices: where
  * row r's piece of slice s begins (base included) -- and the values are read in place.  asamd_xlds_build leaves
  * the record EMPTY (seg NULL, not an error) if some row's columns do not ascend.  Per-call scratch: slices * m
- * elements of `partials`; `width` as for asamd_spmv_vector, from the pieces' mean length. */
+ * elements of `partials`; `width` as for asamd_spmv_vector, from the pieces' mean length.
+ * With `val` given, asamd_xlds_build also COPIES the entries slice by slice (every slice a CSR matrix of its own:
+ * the pieces of consecutive rows consecutive in memory, 16-bit columns counted from the slice's first one, off[s * m
+ * + r] the piece's place in the copy), which the multiply then reads instead of the caller's arrays; short pieces
+ * scattered over the caller's arrays cost whole cache lines each.  asamd_xlds_refresh_values copies the values again
+ * (gate: NULL, or a device word that is 0 when there is nothing to do). */
 typedef struct {
   int32_t *seg;  /* (slices + 1) * m offsets; NULL: no layout */
   int32_t slices, slice_cols, m;
   int64_t device_bytes;
+  int32_t *off;  /* slices * m + 1 offsets into the copy; NULL: no copy */
+  void *val;     /* nnz (+ 4 of padding) values, slice by slice */
+  uint16_t *col; /* their columns, counted from the slice's first */
+  int32_t dtype, nnz, base;
 } asamd_xlds_layout;
 int asamd_xlds_build(hipStream_t stream, int32_t dtype, int32_t m, int32_t n, int32_t nnz, int32_t base,
-                     const int32_t *row_ptr, const int32_t *col_ind, asamd_xlds_layout *out);
+                     const int32_t *row_ptr, const int32_t *col_ind, const void *val, asamd_xlds_layout *out);
+int asamd_xlds_refresh_values(hipStream_t stream, const asamd_xlds_layout *layout, const void *val,
+                              const int32_t *gate);
 void asamd_xlds_free(asamd_xlds_layout *layout);
 int asamd_spmv_xlds_sliced(hipStream_t stream, const asamd_spmv_args *a, int32_t width, const asamd_xlds_layout *layout,
                            void *partials);

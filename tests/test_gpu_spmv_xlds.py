@@ -94,11 +94,15 @@ SLICED = {
 }
 
 
+@pytest.mark.parametrize("copy", ["copy", "in_place"])
 @pytest.mark.parametrize("shape", sorted(SLICED))
-def test_long_rows_over_several_lds_fills_of_x_go_slice_by_slice(gpu, shape, monkeypatch):
+def test_long_rows_over_several_lds_fills_of_x_go_slice_by_slice(gpu, shape, copy, monkeypatch):
     """x of 280 / 640 KB under rows of hundreds of entries: the analysis lays out a table of offsets (where every
-    row's piece of every column slice begins) and the multiply runs a row of workgroups per slice; the values stay
-    in the caller's array, so new values need no second analysis."""
+    row's piece of every column slice begins) and the multiply runs a row of workgroups per slice -- over a copy of
+    the entries slice by slice, which the value guard brings up to date when the caller's values change in place,
+    or (ALSPARSE_AMD_XLDS_COPY=0) over the caller's arrays."""
+    if copy == "in_place":
+        monkeypatch.setenv("ALSPARSE_AMD_XLDS_COPY", "0")
     lib = capi.load()
     a = SLICED[shape]()
     x, y0 = wl.uniform(a.cols, a.dtype, 3), wl.uniform(a.rows, a.dtype, 4)
@@ -113,8 +117,13 @@ def test_long_rows_over_several_lds_fills_of_x_go_slice_by_slice(gpu, shape, mon
             gpu.h, 0, a.rows, a.cols, a.nnz, byref(descr), da.val.c_ptr(), da.row_ptr.c_ptr(), da.col.c_ptr(), info) == 0
         st = lib.asamd_analysis_stats(info).contents
         assert st.algo == capi.ASAMD_SPMV_XLDS and st.xlds_slices >= 2, (st.algo, st.xlds_slices)
+        table = (st.xlds_slices + 1) * a.rows * 4
+        if copy == "copy":
+            assert st.device_bytes > table + a.nnz * (a.dtype.itemsize + 2), "no copy of the entries was laid out"
+        else:
+            assert st.device_bytes < table + a.nnz, "a copy was laid out against ALSPARSE_AMD_XLDS_COPY=0"
         for alpha, beta in ((1.0, 0.0), (-0.5, 2.0)):
-            announce("x in LDS, sliced: multiply", shape, alpha, beta)
+            announce("x in LDS, sliced: multiply", shape, copy, alpha, beta)
             y = run_csrmv(gpu, da, alpha, x, beta, y0, info=info)
             check_spmv(a, alpha, x, beta, y0, y, "%s %s" % (shape, (alpha, beta)))
         announce("x in LDS, sliced: new values in place", shape)
@@ -146,11 +155,15 @@ def test_rows_whose_columns_do_not_ascend_get_no_slices(gpu):
         da.free()
 
 
+@pytest.mark.parametrize("copy", ["copy", "in_place"])
 @pytest.mark.parametrize("seed", range(10))
-def test_random_structures_slice_by_slice(gpu, seed):
+def test_random_structures_slice_by_slice(gpu, seed, copy, monkeypatch):
     """Seeded random structures over 2 .. 7 column slices: empty rows, rows that miss whole slices, rows of thousands
-    of entries, both index bases, both real types, val / col_ind off their 16-byte alignment."""
+    of entries, both index bases, both real types, val / col_ind off their 16-byte alignment; over the copy of the
+    entries slice by slice and over the caller's arrays."""
     from helpers import run_plan_csrmv
+    if copy == "in_place":
+        monkeypatch.setenv("ALSPARSE_AMD_XLDS_COPY", "0")
     rng = np.random.default_rng(4200 + seed)
     dtype = (np.float32, np.float64)[seed % 2]
     fill = 131072 // np.dtype(dtype).itemsize
@@ -172,9 +185,57 @@ def test_random_structures_slice_by_slice(gpu, seed):
     da = DeviceCsr(a, shift=int(rng.integers(0, 4)))
     try:
         for alpha, beta in ((1.0, 0.0), (2.0, 3.0)):
-            announce("x in LDS, sliced: random structure", seed, np.dtype(dtype).name, "cols", cols, "base", base, alpha, beta)
+            announce("x in LDS, sliced: random structure", seed, copy, np.dtype(dtype).name, "cols", cols, "base", base,
+                     alpha, beta)
             y = run_plan_csrmv(da, "xlds", alpha, x, beta, y0)
             assert y is not None, "no slice table for a matrix with ascending columns"
             check_spmv(a, alpha, x, beta, y0, y, "seed %d %s" % (seed, (alpha, beta)))
     finally:
+        da.free()
+
+
+def test_the_copy_follows_the_values(gpu):
+    """The slice-by-slice copy holds values: a multiply with ANOTHER value array (same structure) must not see them
+    (it runs over that array through the table of offsets), asamd_csr_plan_refresh_values re-bases the copy on the
+    new array, and pieces of every length -- none, one entry, more than a lane group's loads -- come out right."""
+    lib = capi.load()
+    rng = np.random.default_rng(99)
+    m, cols = 3000, 100000  # four fp32 slices
+    lengths = rng.integers(0, 60, size=m)
+    lengths[:8] = [0, 1, 2, 3, 4, 5, 20000, 9000]
+    a = csr_from_lengths(list(lengths), cols, np.float32, seed=8, base=1)
+    x, y0 = wl.uniform(a.cols, a.dtype, 3), wl.uniform(a.rows, a.dtype, 4)
+    da = DeviceCsr(a)
+    other = wl.uniform(a.nnz, a.dtype, 31)
+    b = wl.Csr(a.rows, a.cols, a.row_ptr, a.col_ind, other, a.base, "other values")
+    d_other = hiprt.DeviceArray.from_numpy(other)
+    plan = c_void_p()
+    assert lib.asamd_csr_plan_create(None, a.rows, a.cols, a.nnz, da.row_ptr.c_ptr(), da.col.c_ptr(), da.val.c_ptr(),
+                                     a.base, a.dtype.itemsize, 2, byref(plan)) == 0
+    T = capi.scalar_type(a.dtype)
+    dx, dy = hiprt.DeviceArray.from_numpy(x), hiprt.DeviceArray.from_numpy(y0)
+    try:
+        assert lib.asamd_csr_plan_set_algo(plan, capi.ASAMD_SPMV_XLDS) == 0
+        assert lib.asamd_csr_plan_stats(plan).contents.device_bytes > a.nnz * 6, "no copy of the entries"
+        ws = capi.Workspace(lib, plan)
+
+        def multiply(val, want, what):
+            announce("x in LDS, sliced copy:", what)
+            dy.copy_from(y0)
+            assert capi.plan_csrmv(lib, None, plan, 0, T(1.5), val.c_ptr(), da.row_ptr.c_ptr(), da.col.c_ptr(),
+                                   dx.c_ptr(), T(0.5), dy.c_ptr(), ws) == 0
+            hiprt.synchronize()
+            check_spmv(want, 1.5, x, 0.5, y0, dy.to_numpy(), what)
+
+        multiply(da.val, a, "the array the copy was taken from")
+        multiply(d_other, b, "another value array")
+        multiply(da.val, a, "the first array again")
+        assert lib.asamd_csr_plan_refresh_values(None, plan, da.row_ptr.c_ptr(), da.col.c_ptr(), d_other.c_ptr()) == 0
+        multiply(d_other, b, "the copy re-based on the other array")
+        multiply(da.val, a, "the first array, now the foreign one")
+        ws.buf.free()
+    finally:
+        lib.asamd_csr_plan_destroy(plan)
+        for d in (dx, dy, d_other):
+            d.free()
         da.free()
