@@ -1012,7 +1012,13 @@ static double model_ms(const asamd_csr_plan *p, int algo) {
       /* 4-byte values: twice the CSR bytes at 5.6 TB/s; wider ones move 3 values + 4 index bytes per entry
        * through both phases and their second phase (shorter row blocks) reaches 4.6 TB/s */
       const double stream = vs >= 8.0 ? (nnz * (3.0 * vs + 4.0) + (n + m) * vs) / 4.6e9 : 2.0 * bytes / 5.6e9;
-      return (0.045 + stream) * skew;
+      /* rows that all hold 64 entries and more make short row blocks (a tile holds 128 entries at most) and ran 1.37-1.64 times
+       * the estimate that fits rows of 16 (1 M x 1 M x 64: 0.346 ms, 2 M x 2 M x 64: 0.657, 1 M x 1 M x 128: 0.607) */
+      const double usual = mean < 4.0 * (st->min_len + 1.0) ? mean : 4.0 * (st->min_len + 1.0); /* (not a few long rows) */
+      double long_rows = 1.0 + 0.45 * (usual - 16.0) / 48.0;
+      if (long_rows < 1.0) long_rows = 1.0;
+      if (long_rows > 1.45) long_rows = 1.45;
+      return (0.045 + stream) * skew * long_rows;
     }
     default: break;
   }
@@ -1265,6 +1271,12 @@ static hipError_t plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t 
         p->auto_algo = p->struct_algo;
       st->algo = p->auto_algo;
       e = hipSuccess;
+    }
+    if (e == hipSuccess && !force && p->xlds.seg && p->auto_algo != ASAMD_SPMV_XLDS) {
+      /* another copy won against the column slices: their table and copy are not kept beside it */
+      asamd_xlds_free(&p->xlds);
+      st->xlds_slices = 0;
+      if (p->struct_algo == ASAMD_SPMV_XLDS) p->struct_algo = p->plain_algo;
     }
     if (e == hipSuccess && has_value_copy(p)) {
       p->copy_val_src = val;
