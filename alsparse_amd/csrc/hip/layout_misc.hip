@@ -178,8 +178,9 @@ template <typename T>
 static hipError_t xlds_copy_pieces(hipStream_t stream, const asamd_xlds_layout* L, const void* val, const int32_t* col_ind,
                                    const int32_t* gate) {
   const int64_t pieces = (int64_t)L->slices * L->m;
+  // (a refresh behind the value guard is launched with every multiply and mostly returns at once: few workgroups)
   int64_t grid = (pieces + 31) / 32;
-  if (grid > (1 << 20)) grid = 1 << 20;
+  if (grid > 4096) grid = 4096;
   xlds_copy_pieces_kernel<T><<<(unsigned)grid, 256, 0, stream>>>(pieces, L->m, L->slice_cols, L->base, L->seg, L->off,
                                                                 (const T*)val, col_ind, (T*)L->val, L->col, gate);
   return hipGetLastError();

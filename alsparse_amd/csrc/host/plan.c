@@ -135,7 +135,7 @@ static int xlds_slices_for(const asamd_csr_plan *p) {
   return (int)((x_bytes + ASAMD_XLDS_MAX_BYTES - 1) / ASAMD_XLDS_MAX_BYTES);
 }
 /* With a copy of the entries slice by slice the pieces of consecutive rows are neighbours in memory and a piece of
- * six entries is long enough (ALSPARSE_AMD_XLDS_COPY=0: never a copy). */
+ * three entries is long enough for the estimate to decide (ALSPARSE_AMD_XLDS_COPY=0: never a copy). */
 #define ALGO_XLDS_IN_PLACE 64 /* internal: the slices over the caller's arrays although the plan holds a copy */
 static int xlds_sliced_ok(const asamd_csr_plan *p, int force, int copy) {
   const asamd_csr_stats *st = &p->st;
@@ -144,7 +144,7 @@ static int xlds_sliced_ok(const asamd_csr_plan *p, int force, int copy) {
   const int slices = xlds_slices_for(p);
   if (slices < 2 || slices > 1024 || ((int64_t)slices + 1) * st->m >= (int64_t)INT32_MAX) return 0;
   if (force) return 1;
-  return st->nnz >= (1 << 22) && (double)st->nnz >= (copy ? 6.0 : 16.0) * (double)slices * (double)st->m &&
+  return st->nnz >= (1 << 22) && (double)st->nnz >= (copy ? 3.0 : 16.0) * (double)slices * (double)st->m &&
          env_int("ALSPARSE_AMD_XLDS", 1) > 0;
 }
 
@@ -996,8 +996,8 @@ static double model_ms(const asamd_csr_plan *p, int algo) {
       const double sums = (double)slices * m * 3.0 * vs / 4.0e9;
       if (p->xlds.seg ? p->xlds.val != NULL : p->xlds_copy_wanted) {
         /* the copy (16-bit columns, neighbouring pieces), measured with pieces of 50 / 32 / 12.5 / 8 entries, fp32:
-         * 1.98 / 2.09 / 2.69 / 3.34 ps per entry, the slices' sums included; 37 entries, fp64: 3.03 */
-        return 0.92 * one + (double)slices * m * 13.0e-9;
+         * 1.91 / 1.92 / 2.20 / 2.54 ps per entry, the slices' sums included; 37 entries, fp64: 2.82 */
+        return 0.94 * one + (double)slices * m * 6.0e-9;
       }
       return one * (1.0 + 22.0 * (double)slices / mean) + sums;
     }
