@@ -357,6 +357,10 @@ _COMMON = {
     "asamd_gather_values": [_P, _I, _I, _I, _P, _P, _P, _P],
     "asamd_spmv_xlds": [_P, _P, _I],
     "asamd_spmv_xlds_fits": [_I, _I],
+    "asamd_narrow_columns": [_P, _I, _I, _P, _P],
+    "asamd_narrow_rel_columns": [_P, _I, _I, _I, _I, _P, _P, _P, _P],
+    "asamd_spmv_stream_rel16": [_P, POINTER(asamd_spmv_args), _I, _I, _P],
+    "asamd_spmv_xlds_narrow": [_P, POINTER(asamd_spmv_args), _I, _P],
     "asamd_xlds_build": [_P, _I, _I, _I, _I, _I, _P, _P, _P, _P],
     "asamd_xlds_refresh_values": [_P, _P, _P, _P],
     "asamd_xlds_free": [_P],

@@ -111,6 +111,27 @@ static int launch_xlds(hipStream_t s, const asamd_spmv_args* a) {
 // four entries per lane and load: W lanes take the first 4 W entries of a row.  L: column slices (their sums go to
 // `partials`, slices * m elements, and are added up by a second kernel), or null.
 template <typename T, int W, bool NT>
+static int launch_xlds4_narrow_as(hipStream_t s, const asamd_spmv_args* a, const uint16_t* col16) {
+  const size_t lds = ((size_t)a->n * sizeof(T) + 15) / 16 * 16;
+  static std::atomic<uint64_t> allowed{0};
+  if (const hipError_t e = allow_full_lds((const void*)spmv_xlds4_kernel<T, W, NT, unsigned short>, allowed);
+      e != hipSuccess)
+    return e;
+  constexpr int rows_per_trip = (kXldsThreads / W) * kXlds4Rows;
+  int64_t grid = ((int64_t)a->m + rows_per_trip - 1) / rows_per_trip;
+  if (grid > xlds_compute_units()) grid = xlds_compute_units();
+  spmv_xlds4_kernel<T, W, NT, unsigned short><<<(unsigned)grid, kXldsThreads, lds, s>>>(
+      a->m, a->n, a->n, (int64_t)a->nnz, scalar_of<T>(a->alpha), (const T*)a->val, a->row_ptr, a->row_ptr + 1, 0, col16,
+      (const T*)a->x, scalar_of<T>(a->beta), (T*)a->y, 0, a->base);
+  return hipGetLastError();
+}
+template <typename T, int W>
+static int launch_xlds4_narrow(hipStream_t s, const asamd_spmv_args* a, const uint16_t* col16) {
+  return (int64_t)a->nnz <= (int64_t)a->m * 4 * W ? launch_xlds4_narrow_as<T, W, true>(s, a, col16)
+                                                  : launch_xlds4_narrow_as<T, W, false>(s, a, col16);
+}
+
+template <typename T, int W, bool NT>
 static int launch_xlds4_as(hipStream_t s, const asamd_spmv_args* a, const asamd_xlds_layout* L, void* partials) {
   const int cus = xlds_compute_units();
   const int slices = L ? L->slices : 1, slice_cols = L ? L->slice_cols : a->n;
@@ -186,6 +207,38 @@ extern "C" int asamd_spmv_xlds(hipStream_t s, const asamd_spmv_args* a, int32_t 
       case 32: return launch_xlds<T, 32>(s, a);
       case 64: return launch_xlds<T, 64>(s, a);
       default: return hipErrorInvalidValue;
+    }
+  });
+}
+
+extern "C" int asamd_narrow_columns(hipStream_t s, int32_t nnz, int32_t base, const int32_t* col_ind, uint16_t* col16) {
+  if (!col_ind || !col16 || nnz < 1) return hipErrorInvalidValue;
+  int64_t grid = ((int64_t)nnz + 4 + 256 * 8 - 1) / (256 * 8);
+  if (grid > 8192) grid = 8192;
+  narrow_columns_kernel<<<(unsigned)grid, 256, 0, s>>>((int64_t)nnz, base, col_ind, col16);
+  return hipGetLastError();
+}
+
+extern "C" int asamd_spmv_xlds_narrow(hipStream_t s, const asamd_spmv_args* a, int32_t width, const uint16_t* col16) {
+  if (!a || !col16) return hipErrorInvalidValue;
+  if (!asamd_spmv_xlds_fits(a->dtype, a->n) || a->n > 65536 || a->nnz < 4 || a->m < 1 ||
+      (int64_t)a->nnz < 4 * (int64_t)a->m)
+    return hipErrorInvalidValue;
+  return by_dtype(a->dtype, [&](auto* tag) -> int {
+    using T = std::remove_pointer_t<decltype(tag)>;
+    if constexpr (!kIsReal<T>) {
+      return hipErrorInvalidValue;
+    } else {
+      if (!args_ok<T>(a)) return hipErrorInvalidValue;
+      switch (width) {
+        case 2:
+        case 4: return launch_xlds4_narrow<T, 1>(s, a, col16);
+        case 8: return launch_xlds4_narrow<T, 2>(s, a, col16);
+        case 16: return launch_xlds4_narrow<T, 4>(s, a, col16);
+        case 32: return launch_xlds4_narrow<T, 8>(s, a, col16);
+        case 64: return launch_xlds4_narrow<T, 16>(s, a, col16);
+        default: return hipErrorInvalidValue;
+      }
     }
   });
 }
@@ -323,6 +376,57 @@ extern "C" int asamd_spmv_stream(hipStream_t s, const asamd_spmv_args* a, int32_
 #undef ASAMD_STREAM_LAUNCH
     return hipGetLastError();
   });
+}
+
+// The same with 16-bit column distances (real element types, val 16-byte aligned, row_ptr[0] == base; `g` must be the
+// group the distances were made for).
+extern "C" int asamd_narrow_rel_columns(hipStream_t s, int32_t m, int32_t nnz, int32_t base, int32_t g,
+                                        const int32_t* row_ptr, const int32_t* col_ind, int16_t* rel16, int32_t* too_far) {
+  if (!row_ptr || !col_ind || !rel16 || !too_far || m < 1 || nnz < 1) return hipErrorInvalidValue;
+  if (g < 1 || g > kStreamMaxGroup || (g & (g - 1)) != 0) return hipErrorInvalidValue;
+  narrow_rel_columns_kernel<<<(unsigned)(((int64_t)(m > 4 ? m : 4) + 255) / 256), 256, 0, s>>>(
+      m, (int64_t)nnz, base, kStreamRows / g, row_ptr, col_ind, rel16, too_far);
+  return hipGetLastError();
+}
+
+template <typename T>
+static int stream_rel16_impl(hipStream_t s, const asamd_spmv_args* a, int g, int max_len, const int16_t* rel16) {
+  if (!args_ok<T>(a)) return hipErrorInvalidValue;
+  constexpr int kCap = 64 / (int)sizeof(T);
+  if (g < 1 || g > kStreamMaxGroup || (g & (g - 1)) != 0) return hipErrorInvalidValue;
+  if ((((uintptr_t)a->val) & 15u) != 0 || (((uintptr_t)rel16) & 7u) != 0) return hipErrorInvalidValue;
+  const unsigned grid = (unsigned)(((int64_t)a->m * g + kStreamRows - 1) / kStreamRows);
+  const T alpha = scalar_of<T>(a->alpha), beta = scalar_of<T>(a->beta);
+  // measured on the 27-point stencil, 160^3 points, with neither / the values / the distances / both non-temporal:
+  // fp32 0.192 / 0.177 / 0.194 / 0.186 ms, fp64 0.273 / 0.299 / 0.273 / 0.298
+  static const int forced = getenv("ALSPARSE_AMD_STREAM_POLICY") ? atoi(getenv("ALSPARSE_AMD_STREAM_POLICY")) : -1;
+  const int policy = forced >= 0 ? (forced & (kStreamNtValues | kStreamNtIndices)) : (sizeof(T) == 4 ? kStreamNtValues : 0);
+#define ASAMD_STREAM_REL16(CAP, G)                                                                                   \
+  spmv_stream_wide_kernel<T, CAP, G, true><<<grid, kStreamRows, 0, s>>>(a->m, alpha, (const T*)a->val, a->row_ptr,   \
+                                                                        a->col_ind, (const T*)a->x, beta, (T*)a->y,  \
+                                                                        a->base, (int64_t)a->nnz, policy, rel16)
+  if (g == 1) {
+    if (max_len <= 4) ASAMD_STREAM_REL16(4, 1);
+    else if (max_len <= 8 || kCap < 16) ASAMD_STREAM_REL16(8, 1);
+    else ASAMD_STREAM_REL16(kCap, 1);
+  } else if (g == 2) {
+    ASAMD_STREAM_REL16(kCap, 2);
+  } else if (g == 4) {
+    ASAMD_STREAM_REL16(kCap, 4);
+  } else if (g == 8) {
+    ASAMD_STREAM_REL16(kCap, 8);
+  } else {
+    ASAMD_STREAM_REL16(kCap, 16);
+  }
+#undef ASAMD_STREAM_REL16
+  return hipGetLastError();
+}
+extern "C" int asamd_spmv_stream_rel16(hipStream_t s, const asamd_spmv_args* a, int32_t g, int32_t max_len,
+                                       const int16_t* rel16) {
+  if (!a || !rel16) return hipErrorInvalidValue;
+  if (a->dtype == ASAMD_DTYPE_FLOAT) return stream_rel16_impl<float>(s, a, g, max_len, rel16);
+  if (a->dtype == ASAMD_DTYPE_DOUBLE) return stream_rel16_impl<double>(s, a, g, max_len, rel16);
+  return hipErrorInvalidValue;
 }
 
 // ---- merge-path ------------------------------------------------------------------------------------

@@ -493,6 +493,12 @@ __global__ __launch_bounds__(256) void xlds_copy_pieces_kernel(int64_t pieces, i
     }
   }
 }
+// col16[i] = col_ind[i] - base for i < nnz, 0 for the four elements behind them
+static __global__ __launch_bounds__(256) void narrow_columns_kernel(int64_t nnz, int base, const int* __restrict__ col_ind,
+                                                                    unsigned short* __restrict__ col16) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nnz + 4; i += (int64_t)gridDim.x * 256)
+    col16[i] = i < nnz ? (unsigned short)(col_ind[i] - base) : (unsigned short)0;
+}
 // y = alpha * (the slices' sums, added in the order of the slices) + beta * y
 template <typename T>
 __global__ __launch_bounds__(256) void xlds_slices_sum_kernel(int m, int slices, T alpha, const T* __restrict__ part,

@@ -33,6 +33,10 @@ struct asamd_csr_plan {
   asamd_binned_layout binned;
   asamd_xlds_layout xlds;  /* column slices for the kernel that holds x in LDS (an x of several LDS fills) */
   int xlds_copy_wanted;    /* the slices are to come with a copy of the entries (known before they are laid out) */
+  uint16_t *d_col16;       /* x in LDS, one slice: the column numbers as 16-bit words (structure promised fixed) */
+  int16_t *d_rel16;        /* staged row blocks: the columns as 16-bit distances from the workgroup's first row */
+  int rel16_group;         /* the lanes per row they were made for */
+  int watched;             /* laid out for asamd_csr_plan_csrmv_watched: its fingerprints are the caller's account */
   void *d_eval;            /* ELL copy: ell_width * m values, column-major */
   int32_t *d_ecol;         /* ... and zero-based columns */
   const void *copy_val_src; /* the value array that the tiled / ELL copy was taken from */
@@ -399,6 +403,8 @@ static void account(asamd_csr_plan *p) {
   asamd_csr_stats *st = &p->st;
   int64_t b = SETUP_BYTES + 3 * 8;
   if (p->d_block_row) b += ((int64_t)st->merge_blocks + 1) * 4;
+  if (p->d_col16) b += ((int64_t)st->nnz + 4) * 2;
+  if (p->d_rel16) b += ((int64_t)st->nnz + 4) * 2;
   b += p->tiled.device_bytes + p->hot.device_bytes + p->binned.device_bytes + p->xlds.device_bytes;
   if (st->ell_built) b += (int64_t)st->m * st->ell_width * ((int64_t)p->val_size + 4);
   for (int w = 0; w < 2; ++w)
@@ -492,6 +498,8 @@ static int run_algo(hipStream_t s, const asamd_csr_plan *p, int algo, const asam
     case ASAMD_SPMV_ROWCONST:
       return asamd_spmv_rowconst(s, a, st->const_len);
     case ASAMD_SPMV_STREAM:
+      if (p->d_rel16 && p->rel16_group == stream_group(p, 0) && ((uintptr_t)a->val & 15u) == 0)
+        return asamd_spmv_stream_rel16(s, a, p->rel16_group, st->max_len, p->d_rel16);
       return asamd_spmv_stream(s, a, stream_group(p, 0), st->max_len, st->first_offset);
     case ASAMD_SPMV_SCALAR:
       return asamd_spmv_scalar(s, a);
@@ -512,6 +520,7 @@ static int run_algo(hipStream_t s, const asamd_csr_plan *p, int algo, const asam
         }
         return asamd_spmv_xlds_sliced(s, a, width_for_mean(piece), &view, partials);
       }
+      if (p->d_col16) return asamd_spmv_xlds_narrow(s, a, p->auto_width, p->d_col16);
       return asamd_spmv_xlds(s, a, p->auto_width);
     case ASAMD_SPMV_BINNED: {
       void *partial = p->binned.chunks > 0 ? ws_take(&ws, (size_t)p->binned.chunks * vs) : NULL;
@@ -984,7 +993,12 @@ static double model_ms(const asamd_csr_plan *p, int algo) {
   double rate = 2.9; /* TB/s */
   switch (algo) {
     case ASAMD_SPMV_ROWCONST: rate = 6.0; break;
-    case ASAMD_SPMV_STREAM: rate = stream_group(p, 0) > 1 ? 5.2 : 6.6; break;
+    case ASAMD_SPMV_STREAM:
+      rate = stream_group(p, 0) > 1 ? 5.2 : 6.6;
+      /* 16-bit distances for columns: half of the bytes they save shows (27-point stencil, 160^3 points: 0.204 ->
+       * 0.181 ms with 4-byte values, 0.300 -> 0.274 with 8-byte ones) */
+      if (p->d_rel16) return hypot2((bytes - 1.0 * nnz) / (rate * 1e9), gather);
+      break;
     case ASAMD_SPMV_VECTOR: rate = 2.4 * vector_utilisation(st, p->auto_width); break;
     case ASAMD_SPMV_MERGE: rate = 2.9; break;
     case ASAMD_SPMV_XLDS: {
@@ -1052,8 +1066,11 @@ static hipError_t model_copies(hipStream_t stream, asamd_csr_plan *p, const int3
   st->algo = p->auto_algo;
   st->tune_ms_base = (float)base;
   /* the copies in the order of their estimates; each is laid out only if it is the best one left */
-  const double est_tiled = tiled_ok ? model_ms(p, ASAMD_SPMV_TILED) : 0.0;
-  const double est_ell = ell_ok ? model_ms(p, ASAMD_SPMV_ELL) : 0.0;
+  /* a copy that holds values is multiplied behind the value guard: four small launches, 22-30 us (27-point stencil
+   * on 128 x 128 x 64 points: the ELL kernel 0.041 ms, the guarded multiply 0.057, the staged row blocks 0.046) */
+  const double guard_ms = st->value_check && !p->watched ? 0.022 : 0.0;
+  const double est_tiled = tiled_ok ? model_ms(p, ASAMD_SPMV_TILED) + guard_ms : 0.0;
+  const double est_ell = ell_ok ? model_ms(p, ASAMD_SPMV_ELL) + guard_ms : 0.0;
   st->tune_ms_tiled = (float)est_tiled;
   st->tune_ms_ell = (float)est_ell;
   /* The per-class launches read short rows in pieces of a few bytes; they win where the long rows hold nearly
@@ -1163,6 +1180,7 @@ static hipError_t plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t 
   st->tune_mode = env_tune_model();
   p->dtype = dtype;
   p->val_size = val_size;
+  p->watched = trusted == 3;
 
   hipError_t e = hipMalloc(&p->d_setup, SETUP_BYTES);
   if (e == hipSuccess) e = hipMalloc((void **)&p->d_fp, 3 * sizeof(uint64_t));
@@ -1241,6 +1259,34 @@ static hipError_t plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t 
       }
     }
   }
+  if (col_ind && st->trusted && trusted != 3 && (p->auto_algo == ASAMD_SPMV_STREAM || (trusted == 2 && stream_ok(p))) &&
+      (p->dtype == ASAMD_DTYPE_FLOAT || p->dtype == ASAMD_DTYPE_DOUBLE) && nnz >= 1 && st->first_offset == 0 &&
+      (trusted == 2 || (double)nnz * (4.0 + val_size) + ((double)m + n) * val_size > 400.0e6) &&
+      env_int("ALSPARSE_AMD_STREAM_NARROW", 1) > 0) {
+    /* staged row blocks and a structure that stays: where every entry lies within 32 767 columns of its workgroup's
+     * first row (a discretisation, a band) the kernel reads 16-bit distances instead of the column numbers.  Pays
+     * on matrices well beyond the memory-side cache (256 MB): 27-point stencil on 160^3 points 0.204 -> 0.177 ms,
+     * nothing on the 5-point Laplacian on 2048^2 (336 MB). */
+    int32_t *too_far = (int32_t *)p->d_setup;
+    int32_t h_far = 1;
+    p->rel16_group = stream_group(p, 0);
+    e = hipMalloc((void **)&p->d_rel16, ((size_t)nnz + 4) * sizeof(int16_t));
+    if (e == hipSuccess) e = hipMemsetAsync(too_far, 0, sizeof(int32_t), stream);
+    if (e == hipSuccess)
+      e = (hipError_t)asamd_narrow_rel_columns(stream, m, nnz, base, p->rel16_group, row_ptr, col_ind, p->d_rel16, too_far);
+    if (e == hipSuccess) e = hipMemcpyAsync(&h_far, too_far, sizeof(int32_t), hipMemcpyDeviceToHost, stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(stream);
+    if (e == hipErrorOutOfMemory) (void)hipGetLastError();
+    if (e == hipErrorOutOfMemory || (e == hipSuccess && h_far != 0)) {
+      if (p->d_rel16) (void)hipFree(p->d_rel16);
+      p->d_rel16 = NULL;
+      e = hipSuccess;
+    }
+    if (e != hipSuccess) {
+      asamd_csr_plan_destroy(p);
+      return e;
+    }
+  }
   if (col_ind && val && nnz > 0) {
     /* trusted == 2: build every copy whatever the size and skip the timing
      * (lets small matrices exercise those kernels) */
@@ -1288,6 +1334,29 @@ static hipError_t plan_create(hipStream_t stream, int32_t m, int32_t n, int32_t 
       return e;
     }
   }
+  if (col_ind && st->trusted && trusted != 3 && (p->auto_algo == ASAMD_SPMV_XLDS || trusted == 2) && !p->xlds.seg &&
+      n <= 65536 &&
+      (p->dtype == ASAMD_DTYPE_FLOAT || p->dtype == ASAMD_DTYPE_DOUBLE) && nnz >= 4 && (int64_t)nnz >= 4 * (int64_t)m &&
+      asamd_spmv_xlds_fits(p->dtype, n) && st->first_offset == 0 && env_int("ALSPARSE_AMD_XLDS_NARROW", 1) > 0) {
+    /* x in LDS and a structure that stays: the kernel reads 16-bit column numbers (a quarter of an fp32 entry's
+     * bytes less; 4 M x 32 768 x 16: 0.123 -> 0.109 ms, 262 144 x 30 000 x 400: 0.153 -> 0.137).  No room for them: the caller's columns serve. */
+    e = hipMalloc((void **)&p->d_col16, ((size_t)nnz + 4) * sizeof(uint16_t));
+    if (e == hipSuccess) e = (hipError_t)asamd_narrow_columns(stream, nnz, base, col_ind, p->d_col16);
+    if (e == hipSuccess) e = hipStreamSynchronize(stream);
+    if (e == hipErrorOutOfMemory) {
+      (void)hipGetLastError();
+      p->d_col16 = NULL;
+      e = hipSuccess;
+    }
+    if (e != hipSuccess) {
+      asamd_csr_plan_destroy(p);
+      return e;
+    }
+  }
+  if (p->d_rel16 && p->auto_algo != ASAMD_SPMV_STREAM && trusted != 2) {
+    (void)hipFree(p->d_rel16); /* another family was kept */
+    p->d_rel16 = NULL;
+  }
   account(p);
   *out = p;
   return hipSuccess;
@@ -1310,6 +1379,8 @@ int asamd_csr_plan_create_dtype(hipStream_t stream, int32_t m, int32_t n, int32_
 void asamd_csr_plan_destroy(asamd_csr_plan *p) {
   if (!p) return;
   if (p->d_block_row) (void)hipFree(p->d_block_row);
+  if (p->d_col16) (void)hipFree(p->d_col16);
+  if (p->d_rel16) (void)hipFree(p->d_rel16);
   if (p->d_setup) (void)hipFree(p->d_setup);
   if (p->d_fp) (void)hipFree(p->d_fp);
   free_tiled(p);

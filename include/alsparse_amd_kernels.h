@@ -100,6 +100,11 @@ int asamd_spmv_vector_if(hipStream_t stream, const asamd_spmv_args *a, int32_t w
 #define ASAMD_XLDS_MAX_BYTES 131072
 int asamd_spmv_xlds_fits(int32_t dtype, int32_t n);
 int asamd_spmv_xlds(hipStream_t stream, const asamd_spmv_args *a, int32_t width);
+/* The same with the column numbers read from a 16-bit copy (zero-based, nnz + 4 elements, made once by
+ * asamd_narrow_columns for a structure that stays): 6 instead of 8 bytes per fp32 entry.  Real element types, at least
+ * four entries per row on average, n <= 65536; a->col_ind is not read. */
+int asamd_narrow_columns(hipStream_t stream, int32_t nnz, int32_t base, const int32_t *col_ind, uint16_t *col16);
+int asamd_spmv_xlds_narrow(hipStream_t stream, const asamd_spmv_args *a, int32_t width, const uint16_t *col16);
 /* The same for an x of several LDS fills (real element types): the matrix in `slices` slices of slice_cols columns,
  * a row of workgroups each.  With ascending columns inside the rows a row's entries of one slice are a contiguous
  * piece of the caller's arrays, so the layout is a table of offsets only -- seg[s * m + r], s = 0 .. slices: where
@@ -137,6 +142,15 @@ int asamd_spmv_rowconst(hipStream_t stream, const asamd_spmv_args *a, int32_t ro
  * rows hold more entries than its staging area takes them from global memory, so a max_len that has
  * gone stale costs speed, not correctness.  first_offset = row_ptr[0] - base. */
 #define ASAMD_STREAM_MAX_GROUP 16
+/* The same with the column numbers read as 16-bit signed distances from the first row of the entry's workgroup
+ * (rel16: nnz + 4 elements, made once by asamd_narrow_rel_columns for a structure that stays and for THIS `group`;
+ * *too_far, a device word the caller has cleared, is set if some entry lies further than 32 767 columns from that
+ * row, and rel16 is then unusable): 10 instead of 12 bytes per fp64 entry.  Real element types, val 16-byte aligned,
+ * row_ptr[0] == base. */
+int asamd_narrow_rel_columns(hipStream_t stream, int32_t m, int32_t nnz, int32_t base, int32_t group,
+                             const int32_t *row_ptr, const int32_t *col_ind, int16_t *rel16, int32_t *too_far);
+int asamd_spmv_stream_rel16(hipStream_t stream, const asamd_spmv_args *a, int32_t group, int32_t max_len,
+                            const int16_t *rel16);
 int asamd_spmv_stream(hipStream_t stream, const asamd_spmv_args *a, int32_t group, int32_t max_len,
                       int32_t first_offset);
 

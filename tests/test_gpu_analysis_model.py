@@ -22,8 +22,8 @@ SHAPES = {
     "powerlaw_4M": (lambda: wl.powerlaw_rmat(22, 200000, np.float32), capi.ASAMD_SPMV_MERGE),
     # configuration 4 itself (32 MiB of x) -> merge-path with the popular columns' x in LDS
     "powerlaw_8M": (lambda: wl.powerlaw_rmat(23, 200000, np.float32), capi.ASAMD_SPMV_MERGE_HOT),
-    # 27-point stencil, fp64: rows of 8..27 entries -> the ELL copy
-    "stencil27_128": (lambda: wl.stencil3d(128, 128, 128, np.float64), capi.ASAMD_SPMV_ELL),
+    # 27-point stencil, fp64: rows of 8..27 entries -> the staged row blocks (with 16-bit column distances: 0.68 GB)
+    "stencil27_128": (lambda: wl.stencil3d(128, 128, 128, np.float64), capi.ASAMD_SPMV_STREAM),
 }
 
 
@@ -65,8 +65,9 @@ def test_model_and_timing_choose_the_same_family(gpu, shape):
         assert model[0]["algo"] == want, (shape, capi.ALGO_NAMES[model[0]["algo"]], model[0])
         # (a timing run may also keep the hot-column kernel at half of configuration 4's size, where it is 3 %
         # ahead of merge-path: the model lays it out only where the gain is beyond doubt)
-        # and the staged row-block kernel on the stencil, where the ELL copy wins by 8 % and must win by 5 %)
-        near_ties = {"powerlaw_4M": capi.ASAMD_SPMV_MERGE_HOT, "stencil27_128": capi.ASAMD_SPMV_STREAM}
+        # and the ELL copy on the stencil, whose kernel is a few per cent ahead of the staged row blocks when timed
+        # by itself: the model also counts the value guard's launches in front of a copy that holds values)
+        near_ties = {"powerlaw_4M": capi.ASAMD_SPMV_MERGE_HOT, "stencil27_128": capi.ASAMD_SPMV_ELL}
         timed_ok = {want, near_ties[shape]} if shape in near_ties else {want}
         assert timed["algo"] in timed_ok, (shape, capi.ALGO_NAMES[timed["algo"]], timed)
         # the model's decision and every number behind it are the same on every analysis

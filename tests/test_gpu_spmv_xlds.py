@@ -239,3 +239,45 @@ def test_the_copy_follows_the_values(gpu):
         for d in (dx, dy, d_other):
             d.free()
         da.free()
+
+
+@pytest.mark.parametrize("dtype,cols,base", [(np.float32, 32768, 0), (np.float32, 21001, 1), (np.float64, 16384, 1)],
+                         ids=["f32_32768", "f32_21001_base1", "f64_16384_base1"])
+def test_analysed_tall_matrix_reads_sixteen_bit_columns(gpu, dtype, cols, base, monkeypatch):
+    """With an analysis (a structure that stays) the kernel that holds x in LDS reads the column numbers from a 16-bit
+    copy made once; the values stay in the caller's array, so new values in place need nothing."""
+    lib = capi.load()
+    a = wl.uniform_rows(300000, cols, 16, dtype, base=base)
+    x, y0 = wl.uniform(a.cols, a.dtype, 3), wl.uniform(a.rows, a.dtype, 4)
+    da = DeviceCsr(a)
+    descr = capi.make_descr(base=a.base)
+    p = capi.prefix(a.dtype)
+
+    def analysed():
+        info = capi.alphasparse_dcu_mat_info_t()
+        assert lib.alphasparse_dcu_create_mat_info(byref(info)) == 0
+        assert getattr(lib, "alphasparse_dcu_%s_csrmv_analysis" % p)(
+            gpu.h, 0, a.rows, a.cols, a.nnz, byref(descr), da.val.c_ptr(), da.row_ptr.c_ptr(), da.col.c_ptr(), info) == 0
+        return info
+
+    try:
+        announce("x in LDS, 16-bit columns: analysis", np.dtype(dtype).name, cols)
+        info = analysed()
+        st = lib.asamd_analysis_stats(info).contents
+        assert st.algo == capi.ASAMD_SPMV_XLDS and st.xlds_slices == 0
+        assert st.device_bytes >= 2 * a.nnz, "no 16-bit copy of the columns"
+        for alpha, beta in ((1.0, 0.0), (-0.5, 2.0)):
+            announce("x in LDS, 16-bit columns: multiply", alpha, beta)
+            check_spmv(a, alpha, x, beta, y0, run_csrmv(gpu, da, alpha, x, beta, y0, info=info), "narrow %s" % ((alpha, beta),))
+        b = wl.Csr(a.rows, a.cols, a.row_ptr, a.col_ind, wl.uniform(a.nnz, a.dtype, 21), a.base, a.name)
+        da.val.copy_from(b.values)
+        check_spmv(b, 2.0, x, 0.0, y0, run_csrmv(gpu, da, 2.0, x, 0.0, y0, info=info), "narrow, new values in place")
+        lib.alphasparse_dcu_destroy_mat_info(info)
+        monkeypatch.setenv("ALSPARSE_AMD_XLDS_NARROW", "0")
+        info = analysed()
+        st = lib.asamd_analysis_stats(info).contents
+        assert st.algo == capi.ASAMD_SPMV_XLDS and st.device_bytes < 2 * a.nnz
+        check_spmv(b, 1.0, x, 0.0, y0, run_csrmv(gpu, da, 1.0, x, 0.0, y0, info=info), "32-bit columns")
+    finally:
+        lib.alphasparse_dcu_destroy_mat_info(info)
+        da.free()
