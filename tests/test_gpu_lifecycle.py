@@ -1,5 +1,5 @@
 """Device memory over a plan's life: whatever a plan lays out (tiled copy, hot-column table, ELL copy, binned rows,
-column-slice offsets, the transposed copy) goes back to the device when the plan is destroyed, and a second analysis
+column-slice offsets and copy, 16-bit column numbers and distances, the transposed copy) goes back to the device when the plan is destroyed, and a second analysis
 of the same arrays replaces the first one's memory instead of adding to it.  The reference frees its analysis in
 alphasparse_dcu_csrmv_clear (src/util_cpp/alphasparse_dcu_x_csrmv_analysis.cpp:393-414)."""
 from ctypes import byref, c_void_p
@@ -49,7 +49,7 @@ def _cycle(lib, da, algo, x, y0, check):
     assert lib.asamd_csr_plan_create(None, a.rows, a.cols, a.nnz, da.row_ptr.c_ptr(), da.col.c_ptr(), da.val.c_ptr(),
                                      a.base, a.dtype.itemsize, 2, byref(plan)) == 0
     try:
-        if lib.asamd_csr_plan_set_algo(plan, ALGOS[algo]) != 0:
+        if lib.asamd_csr_plan_set_algo(plan, ALGOS[algo.split("_")[0]]) != 0:
             return False
         T = capi.scalar_type(a.dtype)
         dx, dy = hiprt.DeviceArray.from_numpy(x), hiprt.DeviceArray.from_numpy(y0)
@@ -76,6 +76,8 @@ CASES = [
     ("binned", lambda: wl.uniform_rows(1 << 20, 1 << 20, 8, np.float32)),
     ("xlds", lambda: wl.uniform_rows(1 << 18, 1 << 17, 64, np.float32)),  # four column slices
     ("merge", lambda: wl.uniform_rows(1 << 20, 1 << 20, 16, np.float32)),
+    ("xlds_one_slice", lambda: wl.uniform_rows(1 << 20, 1 << 15, 16, np.float32)),  # 16-bit column numbers
+    ("stream", lambda: wl.stencil3d(96, 96, 96, np.float32)),  # 16-bit column distances
 ]
 
 
