@@ -249,3 +249,37 @@ def test_transposed_csrmv_without_analysis_on_tall_matrices(gpu, shape, monkeypa
         check_trans(a, 1.0, x, 0.0, y0, y, "%s global atomics" % shape)
     finally:
         da.free()
+
+
+def test_analysed_tall_transpose_runs_slice_by_slice_and_follows_the_values(gpu):
+    """4 M entries in 300 000 rows of 20 000 columns: the analysed transposed multiply runs on a CSR copy of the
+    transpose (20 000 rows of 240 entries, an x of 300 000 elements: ten LDS fills), which the analysis of that copy
+    multiplies slice by slice over its own copy of the entries.  New values written into the caller's array travel
+    through both copies before the next multiply."""
+    lib = capi.load()
+    a = wl.uniform_rows(300000, 20000, 16, np.float32)
+    x, y0 = wl.uniform(a.rows, a.dtype, 3), wl.uniform(a.cols, a.dtype, 4)
+    da = DeviceCsr(a)
+    info = capi.alphasparse_dcu_mat_info_t()
+    assert lib.alphasparse_dcu_create_mat_info(byref(info)) == 0
+    descr = capi.make_descr(base=a.base)
+    try:
+        announce("tall transpose: analysis")
+        assert lib.alphasparse_dcu_s_csrmv_analysis(gpu.h, TRANS, a.rows, a.cols, a.nnz, byref(descr), da.val.c_ptr(),
+                                                    da.row_ptr.c_ptr(), da.col.c_ptr(), info) == 0
+        st = lib.asamd_analysis_stats(info).contents
+        assert st.transpose_built == 1
+        tst = lib.asamd_analysis_transpose_stats(info).contents
+        assert tst.algo == capi.ASAMD_SPMV_XLDS and tst.xlds_slices == 10, (tst.algo, tst.xlds_slices)
+        assert tst.device_bytes > a.nnz * 6, "the transpose's analysis kept no copy slice by slice"
+        for alpha, beta in ((1.0, 0.0), (2.0, 3.0)):
+            announce("tall transpose: multiply", alpha, beta)
+            check_trans(a, alpha, x, beta, y0, run_csrmv_trans(gpu, da, alpha, x, beta, y0, info), "tall analysed")
+        for seed in (41, 42):
+            announce("tall transpose: new values in place", seed)
+            b = wl.Csr(a.rows, a.cols, a.row_ptr, a.col_ind, wl.uniform(a.nnz, a.dtype, seed), a.base, "new values")
+            da.val.copy_from(b.values)
+            check_trans(b, 1.5, x, 0.5, y0, run_csrmv_trans(gpu, da, 1.5, x, 0.5, y0, info), "tall, new values %d" % seed)
+    finally:
+        lib.alphasparse_dcu_destroy_mat_info(info)
+        da.free()
