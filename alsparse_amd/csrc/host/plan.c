@@ -123,10 +123,24 @@ static int stream_ok(const asamd_csr_plan *p) { return stream_group(p, 0) > 0; }
 /* x in LDS: for an x that crowds the L1 (32 KB) and fits the LDS, on matrices large enough for 256 persistent
  * workgroups.  4 M x 16 entries, fp32: rowconst 0.105 / 0.125 / 0.20 / 0.25 / 0.29 ms with 4 / 16 / 32 / 64 / 128 KB of x,
  * this kernel 0.127 ms whatever x; fp64 with 128 KB of x 0.37 against 0.18 ms.  ALSPARSE_AMD_XLDS=0 leaves it out. */
+/* The kernels that hold x in LDS give every row the lanes that fit the MEAN row, and a lane group walks a longer row
+ * load by load while the wave's other groups wait: where rows of more than four times the mean hold more than a
+ * tenth of the entries they lose to merge-path (rows of 4 and, every eighth, 256 entries, 4 M x 16 384: 0.84 against
+ * 0.56 ms; rows of 2 and, every sixteenth, 2 000, in 32 slices: 1.49 against 0.65 for the tiled pair).  A few long
+ * rows among regular ones go to whole waves and do not matter. */
+static int xlds_rows_regular(const asamd_csr_stats *st) {
+  if (st->m < 1 || st->nnz < 1) return 0;
+  const double mean = (double)st->nnz / (double)st->m;
+  double far = 0.0;
+  for (int b = 2; b < ASAMD_HIST_BINS; ++b) /* bin b: rows of 2^(b-1) .. 2^b - 1 entries */
+    if ((double)((int64_t)1 << (b - 1)) >= 4.0 * mean) far += (double)st->hist[b] * 0.75 * (double)((int64_t)1 << b);
+  return far <= 0.1 * (double)st->nnz;
+}
+
 static int xlds_ok(const asamd_csr_plan *p) {
   const asamd_csr_stats *st = &p->st;
   const int64_t x_bytes = (int64_t)st->n * (int64_t)p->val_size;
-  return st->first_offset == 0 && st->m >= 1 && st->nnz >= (1 << 22) && x_bytes > (20 << 10) &&
+  return st->first_offset == 0 && st->m >= 1 && st->nnz >= (1 << 22) && x_bytes > (20 << 10) && xlds_rows_regular(st) &&
          asamd_spmv_xlds_fits(p->dtype, st->n) && env_int("ALSPARSE_AMD_XLDS", 1) > 0;
 }
 
@@ -148,7 +162,8 @@ static int xlds_sliced_ok(const asamd_csr_plan *p, int force, int copy) {
   const int slices = xlds_slices_for(p);
   if (slices < 2 || slices > 1024 || ((int64_t)slices + 1) * st->m >= (int64_t)INT32_MAX) return 0;
   if (force) return 1;
-  return st->nnz >= (1 << 22) && (double)st->nnz >= (copy ? 3.0 : 16.0) * (double)slices * (double)st->m &&
+  return st->nnz >= (1 << 22) && xlds_rows_regular(st) &&
+         (double)st->nnz >= (copy ? 3.0 : 16.0) * (double)slices * (double)st->m &&
          env_int("ALSPARSE_AMD_XLDS", 1) > 0;
 }
 

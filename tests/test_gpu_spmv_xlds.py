@@ -281,3 +281,21 @@ def test_analysed_tall_matrix_reads_sixteen_bit_columns(gpu, dtype, cols, base, 
     finally:
         lib.alphasparse_dcu_destroy_mat_info(info)
         da.free()
+
+
+def test_rows_far_longer_than_the_mean_keep_the_balanced_kernels(gpu):
+    """Rows of 4 entries and, every eighth, 256 (nine tenths of the entries in rows of seven times the mean): the
+    kernel that holds x in LDS would walk the long rows load by load; the library keeps merge-path.  A milder mix
+    (12 and 24 entries) still takes it."""
+    lib = capi.load()
+    for short, long_, every, takes_xlds in ((4, 256, 8, False), (12, 24, 2, True)):
+        a = wl.bimodal_rows(300000, 16384, short, long_, every, np.float32)
+        assert a.nnz >= 1 << 22
+        da = DeviceCsr(a)
+        try:
+            announce("x in LDS: row-length mix", short, long_, every)
+            assert (_plan_algo(lib, da) == capi.ASAMD_SPMV_XLDS) == takes_xlds, (short, long_, every)
+            x, y0 = wl.uniform(a.cols, a.dtype, 3), wl.uniform(a.rows, a.dtype, 4)
+            check_spmv(a, 1.0, x, 0.0, y0, run_csrmv(gpu, da, 1.0, x, 0.0, y0), "mix %d/%d" % (short, long_))
+        finally:
+            da.free()
