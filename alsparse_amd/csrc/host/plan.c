@@ -137,11 +137,15 @@ static int xlds_rows_regular(const asamd_csr_stats *st) {
   return far <= 0.1 * (double)st->nnz;
 }
 
+/* an x that crowds the L1 and fits a compute unit's LDS */
+static int xlds_sized_x(const asamd_csr_plan *p) {
+  const int64_t x_bytes = (int64_t)p->st.n * (int64_t)p->val_size;
+  return x_bytes > (20 << 10) && asamd_spmv_xlds_fits(p->dtype, p->st.n);
+}
 static int xlds_ok(const asamd_csr_plan *p) {
   const asamd_csr_stats *st = &p->st;
-  const int64_t x_bytes = (int64_t)st->n * (int64_t)p->val_size;
-  return st->first_offset == 0 && st->m >= 1 && st->nnz >= (1 << 22) && x_bytes > (20 << 10) && xlds_rows_regular(st) &&
-         asamd_spmv_xlds_fits(p->dtype, st->n) && env_int("ALSPARSE_AMD_XLDS", 1) > 0;
+  return st->first_offset == 0 && st->m >= 1 && st->nnz >= (1 << 22) && xlds_sized_x(p) && xlds_rows_regular(st) &&
+         env_int("ALSPARSE_AMD_XLDS", 1) > 0;
 }
 
 /* ... and slice by slice for an x of several LDS fills, where the rows are long enough for their pieces: a slice's
@@ -228,6 +232,9 @@ static int hot_eligible(const asamd_csr_plan *p, int force) {
   /* An x that the L2 of one XCD holds is gathered fast enough as it is, and counting and ranking the columns
    * costs some twenty-five multiplies: large matrices only.  ALSPARSE_AMD_TUNE_HOT=0 leaves the copy out. */
   if (env_int("ALSPARSE_AMD_TUNE_HOT", 1) <= 0) return 0;
+  /* ... and matrices of few columns whose row lengths keep them from the kernel that holds x in LDS: the table then
+   * holds all of x, or most of it (see model_copies) */
+  if (xlds_sized_x(p) && st->nnz >= (1 << 22) && !xlds_rows_regular(st)) return 1;
   return (int64_t)st->n * (int64_t)p->val_size >= ((int64_t)8 << 20) && st->nnz >= (1 << 22);
 }
 
@@ -1107,6 +1114,11 @@ static hipError_t model_copies(hipStream_t stream, asamd_csr_plan *p, const int3
     const double stream_ms = (nnz * (4.0 + vs) + ((double)st->m + 1.0) * 4.0 + ((double)st->n + (double)st->m) * vs) / 2.9e9;
     const double gather_ms = nnz * (double)st->lines_per_entry_wave * gather_ps((double)st->lines_per_entry_segment) * 1e-9;
     want_hot = gather_ms >= 0.5 * stream_ms && st->lines_per_entry_segment >= 0.42f;
+    /* Few columns under rows of very different lengths: x is too large for the L1 and the kernel that holds it in
+     * LDS walks long rows load by load; merge-path with its table holding all of x (or the better part) balances
+     * them.  Rows of 4 and, every eighth, 256 entries, 4 M x 16 384: 0.57 -> 0.43 ms; 1 and, every 64th, 4 000,
+     * 2 M x 16 384: 0.39 -> 0.25. */
+    if (xlds_sized_x(p) && st->nnz >= (1 << 22) && !xlds_rows_regular(st)) want_hot = 1;
   }
   const char *ev = getenv("ALSPARSE_AMD_TUNE_PICK");
   int forced = -1;

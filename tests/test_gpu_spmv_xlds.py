@@ -285,8 +285,8 @@ def test_analysed_tall_matrix_reads_sixteen_bit_columns(gpu, dtype, cols, base, 
 
 def test_rows_far_longer_than_the_mean_keep_the_balanced_kernels(gpu):
     """Rows of 4 entries and, every eighth, 256 (nine tenths of the entries in rows of seven times the mean): the
-    kernel that holds x in LDS would walk the long rows load by load; the library keeps merge-path.  A milder mix
-    (12 and 24 entries) still takes it."""
+    kernel that holds x in LDS would walk the long rows load by load; the library keeps merge-path, with all of x in
+    that kernel's LDS table once analysed.  A milder mix (12 and 24 entries) still takes the x-in-LDS kernel."""
     lib = capi.load()
     for short, long_, every, takes_xlds in ((4, 256, 8, False), (12, 24, 2, True)):
         a = wl.bimodal_rows(300000, 16384, short, long_, every, np.float32)
@@ -294,8 +294,23 @@ def test_rows_far_longer_than_the_mean_keep_the_balanced_kernels(gpu):
         da = DeviceCsr(a)
         try:
             announce("x in LDS: row-length mix", short, long_, every)
-            assert (_plan_algo(lib, da) == capi.ASAMD_SPMV_XLDS) == takes_xlds, (short, long_, every)
+            algo = _plan_algo(lib, da)
+            assert (algo == capi.ASAMD_SPMV_XLDS) == takes_xlds, (short, long_, every)
             x, y0 = wl.uniform(a.cols, a.dtype, 3), wl.uniform(a.rows, a.dtype, 4)
             check_spmv(a, 1.0, x, 0.0, y0, run_csrmv(gpu, da, 1.0, x, 0.0, y0), "mix %d/%d" % (short, long_))
+            if not takes_xlds:
+                # an analysis balances the rows with merge-path and keeps all of x in that kernel's LDS table
+                assert algo == capi.ASAMD_SPMV_MERGE_HOT, capi.ALGO_NAMES[algo]
+                info = capi.alphasparse_dcu_mat_info_t()
+                assert lib.alphasparse_dcu_create_mat_info(byref(info)) == 0
+                descr = capi.make_descr(base=a.base)
+                try:
+                    assert lib.alphasparse_dcu_s_csrmv_analysis(gpu.h, 0, a.rows, a.cols, a.nnz, byref(descr),
+                                                                da.val.c_ptr(), da.row_ptr.c_ptr(), da.col.c_ptr(),
+                                                                info) == 0
+                    assert lib.asamd_analysis_stats(info).contents.algo == capi.ASAMD_SPMV_MERGE_HOT
+                    check_spmv(a, -0.5, x, 2.0, y0, run_csrmv(gpu, da, -0.5, x, 2.0, y0, info=info), "mix, analysed")
+                finally:
+                    lib.alphasparse_dcu_destroy_mat_info(info)
         finally:
             da.free()
