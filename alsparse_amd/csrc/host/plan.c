@@ -1033,7 +1033,9 @@ static double model_ms(const asamd_csr_plan *p, int algo) {
       if (p->xlds.seg ? p->xlds.val != NULL : p->xlds_copy_wanted) {
         /* the copy (16-bit columns, neighbouring pieces), measured with pieces of 50 / 32 / 12.5 / 8 entries, fp32:
          * 1.91 / 1.92 / 2.20 / 2.54 ps per entry, the slices' sums included; 37 entries, fp64: 2.82 */
-        return 0.94 * one + (double)slices * m * 6.0e-9;
+        /* (65 536 x 65 536 x 64, 4 M entries: 0.029 ms, of which the value guard's launches, the slices' sums and 256
+         * workgroups' fills of LDS are 0.02) */
+        return 0.02 + 0.94 * one + (double)slices * m * 6.0e-9;
       }
       return one * (1.0 + 22.0 * (double)slices / mean) + sums;
     }
