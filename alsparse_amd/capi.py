@@ -361,6 +361,7 @@ _COMMON = {
     "asamd_narrow_rel_columns": [_P, _I, _I, _I, _I, _P, _P, _P, _P],
     "asamd_spmv_stream_rel16": [_P, POINTER(asamd_spmv_args), _I, _I, _P],
     "asamd_spmv_xlds_narrow": [_P, POINTER(asamd_spmv_args), _I, _P],
+    "asamd_xlds_slices": [_I, _I],
     "asamd_xlds_build": [_P, _I, _I, _I, _I, _I, _P, _P, _P, _P],
     "asamd_xlds_refresh_values": [_P, _P, _P, _P],
     "asamd_xlds_free": [_P],

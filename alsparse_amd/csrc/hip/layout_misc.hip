@@ -192,7 +192,20 @@ static hipError_t xlds_copy_pieces_dtype(hipStream_t stream, const asamd_xlds_la
   return hipErrorInvalidValue;
 }
 
-// As few slices as hold x in ASAMD_XLDS_MAX_BYTES each, of equal width (a multiple of 64 columns).
+// As few slices as hold x in ASAMD_XLDS_MAX_BYTES each -- or up to a quarter more if that count divides the 256
+// compute units evenly: every slice then gets the same number of workgroups (7 slices of 36 workgroups leave four
+// compute units idle and measured 0.217 ms on 262 144 x 262 144 x 400 where 8 slices of 32 take 0.200).
+extern "C" int32_t asamd_xlds_slices(int32_t dtype, int32_t n) {
+  const int vs = dtype_size(dtype);
+  if (vs <= 0 || n < 1) return 0;
+  const int64_t fill = (int64_t)ASAMD_XLDS_MAX_BYTES / vs;  // columns per LDS fill
+  const int64_t need = ((int64_t)n + fill - 1) / fill;
+  for (int64_t s = need; s * 4 <= need * 5 && s <= 256; ++s)
+    if (256 % s == 0) return (int32_t)s;
+  return need > INT32_MAX ? INT32_MAX : (int32_t)need;
+}
+
+// Slices of equal width (a multiple of 64 columns).
 extern "C" int asamd_xlds_build(hipStream_t stream, int32_t dtype, int32_t m, int32_t n, int32_t nnz, int32_t base,
                                 const int32_t* row_ptr, const int32_t* col_ind, const void* val, asamd_xlds_layout* L) {
   if (!L) return hipErrorInvalidValue;
@@ -201,7 +214,7 @@ extern "C" int asamd_xlds_build(hipStream_t stream, int32_t dtype, int32_t m, in
   if (!row_ptr || !col_ind || m < 1 || n < 1 || nnz < 1 || vs <= 0) return hipErrorInvalidValue;
   if (val && dtype != ASAMD_DTYPE_FLOAT && dtype != ASAMD_DTYPE_DOUBLE) return hipErrorInvalidValue;
   const int64_t fill = (int64_t)ASAMD_XLDS_MAX_BYTES / vs;  // columns per LDS fill
-  const int64_t slices = ((int64_t)n + fill - 1) / fill;
+  const int64_t slices = asamd_xlds_slices(dtype, n);
   if (slices < 2 || slices > 1024 || (slices + 1) * (int64_t)m >= (int64_t)INT32_MAX) return hipSuccess;  // no layout
   int64_t width = ((int64_t)n + slices - 1) / slices;
   width = (width + 63) / 64 * 64;

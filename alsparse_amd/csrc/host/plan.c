@@ -152,10 +152,7 @@ static int xlds_ok(const asamd_csr_plan *p) {
  * piece of a row should hold sixteen entries or more on average (262 144 x 262 144 x 400, fp32, 8 slices: merge-path
  * 0.51 ms, this 0.23 ms; 1 M x 131 072 x 128, 4 slices: 0.41 ms).  Needs ascending columns inside the rows (the
  * builder looks) and a structure that is promised fixed. */
-static int xlds_slices_for(const asamd_csr_plan *p) {
-  const int64_t x_bytes = (int64_t)p->st.n * (int64_t)p->val_size;
-  return (int)((x_bytes + ASAMD_XLDS_MAX_BYTES - 1) / ASAMD_XLDS_MAX_BYTES);
-}
+static int xlds_slices_for(const asamd_csr_plan *p) { return asamd_xlds_slices(p->dtype, p->st.n); }
 /* With a copy of the entries slice by slice the pieces of consecutive rows are neighbours in memory and a piece of
  * three entries is long enough for the estimate to decide (ALSPARSE_AMD_XLDS_COPY=0: never a copy). */
 #define ALGO_XLDS_IN_PLACE 64 /* internal: the slices over the caller's arrays although the plan holds a copy */

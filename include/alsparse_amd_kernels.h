@@ -46,7 +46,7 @@ enum asamd_spmv_algo {
                               the longest rows in chunks, a workgroup each): for very
                               uneven rows; keeps a list of row numbers, no values   */
   ASAMD_SPMV_XLDS = 10     /* W lanes per row with x held in every compute unit's LDS:
-                              matrices of few columns (x <= 128 KB); keeps nothing  */
+                              matrices of few columns (x <= 160 KB); keeps nothing  */
 };
 
 #define ASAMD_HIST_BINS 33
@@ -97,7 +97,7 @@ int asamd_spmv_vector(hipStream_t stream, const asamd_spmv_args *a, int32_t widt
 int asamd_spmv_vector_if(hipStream_t stream, const asamd_spmv_args *a, int32_t width, const int32_t *run_if);
 /* x held in the LDS of every compute unit (one workgroup of 1 024 threads each), `width` lanes per row: for
  * matrices whose x is at most ASAMD_XLDS_MAX_BYTES (asamd_spmv_xlds_fits); reads the CSR arrays in place. */
-#define ASAMD_XLDS_MAX_BYTES 131072
+#define ASAMD_XLDS_MAX_BYTES 163840 /* the LDS of a compute unit */
 int asamd_spmv_xlds_fits(int32_t dtype, int32_t n);
 int asamd_spmv_xlds(hipStream_t stream, const asamd_spmv_args *a, int32_t width);
 /* The same with the column numbers read from a 16-bit copy (zero-based, nnz + 4 elements, made once by
@@ -125,6 +125,7 @@ typedef struct {
   uint16_t *col; /* their columns, counted from the slice's first */
   int32_t dtype, nnz, base;
 } asamd_xlds_layout;
+int32_t asamd_xlds_slices(int32_t dtype, int32_t n); /* the slices asamd_xlds_build would cut n columns into */
 int asamd_xlds_build(hipStream_t stream, int32_t dtype, int32_t m, int32_t n, int32_t nnz, int32_t base,
                      const int32_t *row_ptr, const int32_t *col_ind, const void *val, asamd_xlds_layout *out);
 int asamd_xlds_refresh_values(hipStream_t stream, const asamd_xlds_layout *layout, const void *val,

@@ -74,7 +74,7 @@ CASES = [
     ("hot", lambda: wl.uniform_rows(1 << 20, 1 << 20, 16, np.float32)),
     ("ell", lambda: wl.uniform_rows(1 << 20, 1 << 20, 8, np.float64)),
     ("binned", lambda: wl.uniform_rows(1 << 20, 1 << 20, 8, np.float32)),
-    ("xlds", lambda: wl.uniform_rows(1 << 18, 1 << 17, 64, np.float32)),  # four column slices
+    ("xlds", lambda: wl.uniform_rows(1 << 18, 1 << 17, 64, np.float32)),  # four column slices (512 KB of x)
     ("merge", lambda: wl.uniform_rows(1 << 20, 1 << 20, 16, np.float32)),
     ("xlds_one_slice", lambda: wl.uniform_rows(1 << 20, 1 << 15, 16, np.float32)),  # 16-bit column numbers
     ("stream", lambda: wl.stencil3d(96, 96, 96, np.float32)),  # 16-bit column distances

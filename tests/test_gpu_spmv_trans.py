@@ -252,12 +252,12 @@ def test_transposed_csrmv_without_analysis_on_tall_matrices(gpu, shape, monkeypa
 
 
 def test_analysed_tall_transpose_runs_slice_by_slice_and_follows_the_values(gpu):
-    """4 M entries in 300 000 rows of 20 000 columns: the analysed transposed multiply runs on a CSR copy of the
-    transpose (20 000 rows of 240 entries, an x of 300 000 elements: ten LDS fills), which the analysis of that copy
+    """19 M entries in 1 200 000 rows of 20 000 columns: the analysed transposed multiply runs on a CSR copy of the
+    transpose (20 000 rows of 960 entries, an x of 1 200 000 elements: thirty LDS fills, cut into 32 slices), which the analysis of that copy
     multiplies slice by slice over its own copy of the entries.  New values written into the caller's array travel
     through both copies before the next multiply."""
     lib = capi.load()
-    a = wl.uniform_rows(300000, 20000, 16, np.float32)
+    a = wl.uniform_rows(1200000, 20000, 16, np.float32)
     x, y0 = wl.uniform(a.rows, a.dtype, 3), wl.uniform(a.cols, a.dtype, 4)
     da = DeviceCsr(a)
     info = capi.alphasparse_dcu_mat_info_t()
@@ -270,7 +270,7 @@ def test_analysed_tall_transpose_runs_slice_by_slice_and_follows_the_values(gpu)
         st = lib.asamd_analysis_stats(info).contents
         assert st.transpose_built == 1
         tst = lib.asamd_analysis_transpose_stats(info).contents
-        assert tst.algo == capi.ASAMD_SPMV_XLDS and tst.xlds_slices == 10, (tst.algo, tst.xlds_slices)
+        assert tst.algo == capi.ASAMD_SPMV_XLDS and tst.xlds_slices == 32, (tst.algo, tst.xlds_slices)
         assert tst.device_bytes > a.nnz * 6, "the transpose's analysis kept no copy slice by slice"
         for alpha, beta in ((1.0, 0.0), (2.0, 3.0)):
             announce("tall transpose: multiply", alpha, beta)

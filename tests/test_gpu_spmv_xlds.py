@@ -1,4 +1,4 @@
-"""Matrices of few columns: x larger than the 32 KB L1 and small enough for a compute unit's LDS (128 KB at most).
+"""Matrices of few columns: x larger than the 32 KB L1 and small enough for a compute unit's LDS (160 KB at most).
 The library then multiplies with one persistent workgroup per compute unit that holds x in LDS and reads the CSR
 arrays in place -- with or without an analysis, since nothing is kept.  The reference has one kernel for every
 shape (src/kernel/dcu/level2/mv/csrmv/dcu_gemv_vector.h:14-57); results are compared with the CPU oracle."""
@@ -87,17 +87,18 @@ def test_rows_of_every_length_and_both_bases(gpu):
 
 
 SLICED = {
-    # 3 slices of fp32 columns, pieces of 100 entries
-    "f32_70000": lambda: wl.uniform_rows(16384, 70000, 300, np.float32),
-    # 5 slices of fp64 columns, index base one
-    "f64_80000_base1": lambda: wl.uniform_rows(20000, 80000, 250, np.float64, base=1),
+    # 2 slices of fp32 columns, pieces of 150 entries; 20 M entries (the slices carry a fixed cost of some 20 us per
+    # multiply: smaller matrices keep merge-path)
+    "f32_70000": lambda: wl.uniform_rows(65536, 70000, 300, np.float32),
+    # 4 slices of fp64 columns, index base one
+    "f64_80000_base1": lambda: wl.uniform_rows(100000, 80000, 250, np.float64, base=1),
 }
 
 
 @pytest.mark.parametrize("copy", ["copy", "in_place"])
 @pytest.mark.parametrize("shape", sorted(SLICED))
 def test_long_rows_over_several_lds_fills_of_x_go_slice_by_slice(gpu, shape, copy, monkeypatch):
-    """x of 280 / 640 KB under rows of hundreds of entries: the analysis lays out a table of offsets (where every
+    """x of 280 / 640 KB (two / four LDS fills) under rows of hundreds of entries: the analysis lays out a table of offsets (where every
     row's piece of every column slice begins) and the multiply runs a row of workgroups per slice -- over a copy of
     the entries slice by slice, which the value guard brings up to date when the caller's values change in place,
     or (ALSPARSE_AMD_XLDS_COPY=0) over the caller's arrays."""
@@ -140,7 +141,13 @@ def test_long_rows_over_several_lds_fills_of_x_go_slice_by_slice(gpu, shape, cop
 
 def test_rows_whose_columns_do_not_ascend_get_no_slices(gpu):
     lib = capi.load()
-    a = wl.uniform_rows(16384, 70000, 300, np.float32)
+    a = wl.uniform_rows(65536, 70000, 300, np.float32)
+    da = DeviceCsr(a)
+    try:
+        announce("x in LDS, sliced: the same matrix with ascending columns")
+        assert _plan_algo(lib, da) == capi.ASAMD_SPMV_XLDS
+    finally:
+        da.free()
     cols = a.col_ind.copy()
     cols[5:7] = cols[5:7][::-1]  # one pair out of order in row 0
     b = wl.Csr(a.rows, a.cols, a.row_ptr, cols, a.values, a.base, "unsorted")
@@ -166,7 +173,7 @@ def test_random_structures_slice_by_slice(gpu, seed, copy, monkeypatch):
         monkeypatch.setenv("ALSPARSE_AMD_XLDS_COPY", "0")
     rng = np.random.default_rng(4200 + seed)
     dtype = (np.float32, np.float64)[seed % 2]
-    fill = 131072 // np.dtype(dtype).itemsize
+    fill = 163840 // np.dtype(dtype).itemsize
     cols = int(rng.integers(fill + 1, 7 * fill))
     m = int(rng.integers(1, 4000))
     law = seed % 3
@@ -200,7 +207,7 @@ def test_the_copy_follows_the_values(gpu):
     new array, and pieces of every length -- none, one entry, more than a lane group's loads -- come out right."""
     lib = capi.load()
     rng = np.random.default_rng(99)
-    m, cols = 3000, 100000  # four fp32 slices
+    m, cols = 3000, 100000  # three fp32 slices
     lengths = rng.integers(0, 60, size=m)
     lengths[:8] = [0, 1, 2, 3, 4, 5, 20000, 9000]
     a = csr_from_lengths(list(lengths), cols, np.float32, seed=8, base=1)
