@@ -931,9 +931,14 @@ static hipError_t tune_copies(hipStream_t stream, asamd_csr_plan *p, const int32
   st->tune_ms_hot = t.best[CAND_HOT];
   /* a copy has to win by a margin to be worth its memory; among the winners the fastest is kept */
   const float margin[CAND_COUNT] = {1.f, 0.9f, 0.95f, 0.95f, 0.95f};
+  /* (the timing runs launch the kernels alone: a copy that holds values is multiplied behind the value guard's four
+   * small launches later on, and is compared with them counted) */
+  float cost[CAND_COUNT];
+  for (int c = 0; c < CAND_COUNT; ++c)
+    cost[c] = t.best[c] + (t.best[c] > 0.f && (c == CAND_TILED || c == CAND_ELL) && st->value_check && !p->watched ? 0.022f : 0.f);
   int pick = 0;
   for (int c = 1; c < CAND_COUNT; ++c)
-    if (t.best[c] > 0.f && t.best[c] < margin[c] * t.best[CAND_BASE] && (pick == 0 || t.best[c] < t.best[pick])) pick = c;
+    if (cost[c] > 0.f && cost[c] < margin[c] * cost[CAND_BASE] && (pick == 0 || cost[c] < cost[pick])) pick = c;
   /* ALSPARSE_AMD_TUNE_PICK = base | tiled | ell | hot | binned overrides the timing's verdict among the
    * candidates that were built (for profiling a kernel that lost) */
   const char *ev = getenv("ALSPARSE_AMD_TUNE_PICK");
@@ -1038,7 +1043,10 @@ static double model_ms(const asamd_csr_plan *p, int algo) {
     }
     case ASAMD_SPMV_ELL: {
       const double ell_bytes = m * (double)st->max_len * (4.0 + vs) + (n + m) * vs;
-      return hypot2(ell_bytes / 6.1e9, gather);
+      /* with 8-byte values the ELL kernel (two rows per lane) gathers scattered columns faster than the row kernels:
+       * 1 M x 1 M x 16 / x 32, fp64: 0.143 / 0.261 ms against rowconst's 0.186 / 0.355; fp32: 0.100 / 0.196 against
+       * 0.095 / 0.196 */
+      return hypot2(ell_bytes / 6.1e9, vs >= 8.0 ? 0.72 * gather : gather);
     }
     case ASAMD_SPMV_TILED: {
       double skew = 1.0 + 0.5 * ((double)st->max_len / mean - 1.0) / 8.0;
