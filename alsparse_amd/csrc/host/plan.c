@@ -1043,9 +1043,10 @@ static double model_ms(const asamd_csr_plan *p, int algo) {
     }
     case ASAMD_SPMV_ELL: {
       const double ell_bytes = m * (double)st->max_len * (4.0 + vs) + (n + m) * vs;
-      /* with 8-byte values the ELL kernel (two rows per lane) gathers scattered columns faster than the row kernels:
-       * 1 M x 1 M x 16 / x 32, fp64: 0.143 / 0.261 ms against rowconst's 0.186 / 0.355; fp32: 0.100 / 0.196 against
-       * 0.095 / 0.196 */
+      /* The lanes of one ELL gather hold the SAME position of 64 neighbouring rows; with ascending columns those
+       * fall into a narrower window of x than the positions of one row, which pays once x outgrows an XCD's L2:
+       * 1 M x 1 M x 16 / x 32, fp64 (8 MB of x): 0.143 / 0.261 ms against rowconst's 0.186 / 0.355 (more rows in
+       * flight per lane group do not help rowconst: 0.357); fp32 (4 MB): 0.100 / 0.196 against 0.095 / 0.196 */
       return hypot2(ell_bytes / 6.1e9, vs >= 8.0 ? 0.72 * gather : gather);
     }
     case ASAMD_SPMV_TILED: {
