@@ -232,8 +232,13 @@ extern "C" int asamd_xlds_build(hipStream_t stream, int32_t dtype, int32_t m, in
     const int64_t count = (slices + 1) * (int64_t)m;
     e = hipMalloc(&L->seg, (size_t)count * sizeof(int));
     if (e == hipSuccess) {
-      xlds_slice_offsets_kernel<<<(unsigned)((count + 255) / 256), 256, 0, stream>>>(m, (int)slices, (int)width, row_ptr,
-                                                                                    col_ind, base, L->seg);
+      // rows long enough to keep a wave's lanes busy are walked once; short rows are searched, a lane per row and slice
+      if ((int64_t)nnz >= 16 * (int64_t)m)
+        xlds_slice_offsets_walk_kernel<<<(unsigned)(((int64_t)m + 3) / 4), 256, 0, stream>>>(m, (int)slices, (int)width,
+                                                                                            row_ptr, col_ind, base, L->seg);
+      else
+        xlds_slice_offsets_kernel<<<(unsigned)((count + 255) / 256), 256, 0, stream>>>(m, (int)slices, (int)width,
+                                                                                      row_ptr, col_ind, base, L->seg);
       e = hipGetLastError();
     }
     if (e == hipSuccess) e = hipStreamSynchronize(stream);

@@ -461,6 +461,31 @@ static __global__ __launch_bounds__(256) void xlds_slice_offsets_kernel(int m, i
   }
   seg[i] = lo + base;
 }
+// The same table from one walk over every row (a wave per row): entry k begins the slices behind its predecessor's
+// up to its own, the row's first entry those up to its own, the row's end those behind its last entry.  One pass over
+// col_ind instead of a binary search per row and slice (32 slices x 1 M rows: 2.5 ms of searches).
+static __global__ __launch_bounds__(256) void xlds_slice_offsets_walk_kernel(int m, int slices, int slice_cols,
+                                                                             const int* __restrict__ row_ptr,
+                                                                             const int* __restrict__ col_ind, int base,
+                                                                             int* __restrict__ seg) {
+  const int64_t r = (int64_t)blockIdx.x * (256 / kWave) + threadIdx.x / kWave;
+  if (r >= m) return;
+  const int lane = threadIdx.x % kWave;
+  const int lo = row_ptr[r] - base, hi = row_ptr[r + 1] - base;
+  // (column numbers outside the matrix land in the first or the last slice: nothing is written outside the table)
+  auto slice_of = [&](int k) {
+    const int s = (col_ind[k] - base) / slice_cols;
+    return s < 0 ? 0 : (s >= slices ? slices - 1 : s);
+  };
+  for (int k = lo + lane; k < hi; k += kWave) {
+    const int s = slice_of(k), before = k == lo ? -1 : slice_of(k - 1);
+    for (int t = before + 1; t <= s; ++t) seg[(int64_t)t * m + r] = k + base;
+  }
+  if (lane == 0) {
+    const int last = hi > lo ? slice_of(hi - 1) : -1;
+    for (int t = last + 1; t <= slices; ++t) seg[(int64_t)t * m + r] = hi + base;
+  }
+}
 // *unsorted |= 1 if the columns of some row do not ascend; a wave per row
 static __global__ __launch_bounds__(256) void xlds_rows_ascend_kernel(int m, const int* __restrict__ row_ptr,
                                                                       const int* __restrict__ col_ind, int base,
