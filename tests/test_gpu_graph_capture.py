@@ -95,7 +95,8 @@ def test_analysed_csrmv_replays_from_a_hip_graph(gpu, shape):
 
 CAPTURE_CASES = [(algo, "uniform") for algo in ("vector", "rowconst", "merge", "scalar", "tiled", "stream", "ell", "hot",
                                                 "binned")]
-CAPTURE_CASES += [("xlds", "narrow")]  # x must fit the LDS: 20 000 columns
+CAPTURE_CASES += [("xlds", "narrow")]  # x fits the LDS: 20 000 columns, read as 16-bit numbers
+CAPTURE_CASES += [("xlds", "uniform")]  # 50 000 columns: two slices over a copy of the entries, behind the value guard
 # heavy-tailed rows: the tiled copy's third phase, the bins' chunked long rows, merge blocks inside one row
 CAPTURE_CASES += [(algo, "powerlaw") for algo in ("merge", "tiled", "hot", "binned")]
 
