@@ -397,10 +397,16 @@ static int stream_rel16_impl(hipStream_t s, const asamd_spmv_args* a, int g, int
   if ((((uintptr_t)a->val) & 15u) != 0 || (((uintptr_t)rel16) & 7u) != 0) return hipErrorInvalidValue;
   const unsigned grid = (unsigned)(((int64_t)a->m * g + kStreamRows - 1) / kStreamRows);
   const T alpha = scalar_of<T>(a->alpha), beta = scalar_of<T>(a->beta);
-  // measured on the 27-point stencil, 160^3 points, with neither / the values / the distances / both non-temporal:
-  // fp32 0.192 / 0.177 / 0.194 / 0.186 ms, fp64 0.273 / 0.299 / 0.273 / 0.298
+  // Measured with neither / the values / the distances / both non-temporal, ms per multiply:
+  //   27-point stencil 160^3      fp32 0.192 / 0.176 / 0.191 / 0.186      fp64 0.276 / 0.299 / 0.276 / 0.299
+  //   5-point Laplacian 4096^2    fp32 0.199 / 0.188 / 0.197 / 0.170      fp64 0.274 / 0.295 / 0.275 / 0.280
+  // 4-byte values always bypass the caches; the distances too unless they fit the memory-side cache beside what is
+  // not a matrix stream (49 MB of row offsets, x and y on the stencil, 201 MB on the Laplacian); 8-byte values: nothing.
   static const int forced = getenv("ALSPARSE_AMD_STREAM_POLICY") ? atoi(getenv("ALSPARSE_AMD_STREAM_POLICY")) : -1;
-  const int policy = forced >= 0 ? (forced & (kStreamNtValues | kStreamNtIndices)) : (sizeof(T) == 4 ? kStreamNtValues : 0);
+  const double rest = ((double)a->m + 1.0) * 4.0 + ((double)a->m + (double)a->n) * (double)sizeof(T);
+  int policy = 0;
+  if (sizeof(T) == 4) policy = kStreamNtValues | (rest + 2.0 * (double)a->nnz > 300.0e6 ? kStreamNtIndices : 0);
+  if (forced >= 0) policy = forced & (kStreamNtValues | kStreamNtIndices);
 #define ASAMD_STREAM_REL16(CAP, G)                                                                                   \
   spmv_stream_wide_kernel<T, CAP, G, true><<<grid, kStreamRows, 0, s>>>(a->m, alpha, (const T*)a->val, a->row_ptr,   \
                                                                         a->col_ind, (const T*)a->x, beta, (T*)a->y,  \

@@ -251,9 +251,8 @@ __global__ __launch_bounds__(kStreamRows) void spmv_stream_wide_kernel(
           const StreamShort4* from = reinterpret_cast<const StreamShort4*>(rel16 + a0 + k);
           if (policy & kStreamNtIndices) {
             // (An address the compiler cannot tell from the other branch's: it would merge the two loads into a plain
-            // one.  The launcher sets this bit only when ALSPARSE_AMD_STREAM_POLICY asks for it -- the small stream is
-            // best left to the caches -- but with one merged load the compiler's schedule of the piece's loads is the
-            // slower one: 27-point stencil on 160^3 points, fp64, 0.295 against 0.273 ms.)
+            // one, and with one merged load its schedule of the piece's loads is the slower one even where this
+            // branch is not taken: 27-point stencil on 160^3 points, fp64, 0.295 against 0.273 ms.)
             asm volatile("" : "+v"(from));
             d = nt_load_object(from);
           } else {

@@ -162,6 +162,12 @@ def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False, vendor=Fa
         x, y0, alpha, beta = wl.uniform(a.cols, udt, 3), wl.uniform(a.rows, udt, 4), 1.0, 0.5
         workload_name = "27-point stencil: CSR SpMV %s, %d x %d x %d grid (%d rows, %d nnz), alpha=1 beta=0.5" % (
             np.dtype(udt).name, gx, gy, gz, a.rows, a.nnz)
+    elif isinstance(cfg, tuple) and cfg[0] == "laplace2d":  # ("laplace2d", nx, ny, dtype)
+        _, gx, gy, udt = cfg
+        a = wl.laplace2d(gx, gy, udt)
+        x, y0, alpha, beta = wl.uniform(a.cols, udt, 3), wl.uniform(a.rows, udt, 4), 1.0, 0.5
+        workload_name = "5-point Laplacian: CSR SpMV %s, %d x %d grid (%d rows, %d nnz), alpha=1 beta=0.5" % (
+            np.dtype(udt).name, gx, gy, a.rows, a.nnz)
     elif isinstance(cfg, tuple):  # ("uniform", rows, cols, entries per row, dtype): not a benchmark configuration
         _, um, un, uk, udt = cfg
         a = wl.uniform_rows(um, un, uk, udt)
@@ -792,6 +798,8 @@ def main():
                          "and the others SHORT (the workload of the row-length bins)")
     ap.add_argument("--stencil3d", nargs=3, type=int, metavar=("NX", "NY", "NZ"),
                     help="instead of a configuration: the 27-point stencil on an NX x NY x NZ grid (8 to 27 entries per row)")
+    ap.add_argument("--laplace2d", nargs=2, type=int, metavar=("NX", "NY"),
+                    help="not a benchmark configuration: the 5-point Laplacian of configuration 2 on an NX x NY grid (fp32; --fp64)")
     ap.add_argument("--dense-cols", type=int, default=None, metavar="N",
                     help="with --config 5: N dense columns instead of 64 (with --stencil3d too: the stencil as the sparse matrix)")
     ap.add_argument("--fp64", action="store_true", help="with --uniform / --bimodal / --stencil3d: fp64 values")
@@ -866,11 +874,13 @@ def main():
             cfg = ("bimodal",) + tuple(args.bimodal) + (np.float64 if args.fp64 else np.float32,)
         if args.stencil3d:
             cfg = ("stencil3d",) + tuple(args.stencil3d) + (np.float64 if args.fp64 else np.float32,)
+        if args.laplace2d:
+            cfg = ("laplace2d",) + tuple(args.laplace2d) + (np.float64 if args.fp64 else np.float32,)
         main_res = run_spmv(cfg, args.steps, args.warmup, not args.no_cpu_baseline, check, args.transpose,
                             not args.no_vendor_baseline, args.cx, args.conjugate)
     others = {}
     ceilings = None
-    plain_default = (args.config == 3 and not (args.all or args.only or args.uniform or args.bimodal or args.stencil3d or args.no_analysis or args.transpose or args.cx or
+    plain_default = (args.config == 3 and not (args.all or args.only or args.uniform or args.bimodal or args.stencil3d or args.laplace2d or args.no_analysis or args.transpose or args.cx or
                                                args.conversions or args.col_major) and args.format == "csr")
     if plain_default:
         # what this GPU sustains with plain kernels, measured in this very run: the figures below are read against it

@@ -456,7 +456,7 @@ def test_copy_is_not_used_for_another_value_array(gpu, algo):
 def test_analysis_choices(gpu, tune, monkeypatch):
     """What the analysis decides and what it skips: a banded matrix runs the staged row-block kernel on the
     caller's arrays, or the ELL copy if that is at least 5 % faster by the analysis' model (or, with
-    ALSPARSE_AMD_TUNE=timed, by its timing run: the two are within a few per cent of each other), and never
+    ALSPARSE_AMD_TUNE=timed, by its timing run), the value guard's launches in front of the copy counted, and never
     lays out the tiled copy (slower than either); a matrix small enough to be launch-bound takes the
     single-kernel path however skewed its rows are."""
     monkeypatch.setenv("ALSPARSE_AMD_TUNE", tune)
@@ -476,7 +476,10 @@ def test_analysis_choices(gpu, tune, monkeypatch):
         assert st.tune_ms_ell > 0 and st.tune_ms_base > 0
         # timed: the tiled copy was not even tried; model: its estimate is there, and slower
         assert st.tune_ms_tiled == 0 if tune == "timed" else st.tune_ms_tiled > st.tune_ms_base
-        assert (st.algo == capi.ASAMD_SPMV_ELL) == (st.tune_ms_ell < 0.95 * st.tune_ms_base)
+        # (the model's estimate of a copy that holds values counts the value guard's launches, 0.022 ms; the timing
+        # run times the kernels alone and adds them before it compares)
+        ell_cost = st.tune_ms_ell + (0.022 if tune == "timed" else 0.0)
+        assert (st.algo == capi.ASAMD_SPMV_ELL) == (ell_cost < 0.95 * st.tune_ms_base), (st.tune_ms_ell, st.tune_ms_base)
         check_spmv(a, alpha, x, beta, y0, run_csrmv(gpu, da, alpha, x, beta, y0, info), "config 2 analysed")
     finally:
         lib.alphasparse_dcu_destroy_mat_info(info)
