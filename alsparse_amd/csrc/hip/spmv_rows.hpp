@@ -296,7 +296,10 @@ __global__ __launch_bounds__(kStreamRows) void spmv_stream_wide_kernel(
   T sum = T(0);
   for (int k = my_begin + lane; k < my_end; k += G) sum += s_prod[k];
   if constexpr (G > 1) sum = group_sum<G>(sum);
-  if (lane == 0) store_axpby(y, row, alpha, sum, beta);
+  if (lane == 0) {
+    if (policy & kStreamNtY) store_axpby_nt(y, row, alpha, sum, beta);
+    else store_axpby(y, row, alpha, sum, beta);
+  }
 }
 
 // rel16[k] = col_ind[k] - base - (first row of the workgroup that takes entry k's row), 0 for the four elements behind
