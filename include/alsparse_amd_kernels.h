@@ -102,7 +102,8 @@ int asamd_spmv_xlds_fits(int32_t dtype, int32_t n);
 int asamd_spmv_xlds(hipStream_t stream, const asamd_spmv_args *a, int32_t width);
 /* The same with the column numbers read from a 16-bit copy (zero-based, nnz + 4 elements, made once by
  * asamd_narrow_columns for a structure that stays): 6 instead of 8 bytes per fp32 entry.  Real element types, at least
- * four entries per row on average, n <= 65536; a->col_ind is not read. */
+ * four entries per row on average, n <= 65536; a->col_ind is not read.  (No counterpart in the reference, whose one
+ * kernel reads the caller's 32-bit columns: src/kernel/dcu/level2/mv/csrmv/dcu_gemv_vector.h:14-57.) */
 int asamd_narrow_columns(hipStream_t stream, int32_t nnz, int32_t base, const int32_t *col_ind, uint16_t *col16);
 int asamd_spmv_xlds_narrow(hipStream_t stream, const asamd_spmv_args *a, int32_t width, const uint16_t *col16);
 /* The same for an x of several LDS fills (real element types): the matrix in `slices` slices of slice_cols columns,
@@ -115,7 +116,8 @@ int asamd_spmv_xlds_narrow(hipStream_t stream, const asamd_spmv_args *a, int32_t
  * the pieces of consecutive rows consecutive in memory, 16-bit columns counted from the slice's first one, off[s * m
  * + r] the piece's place in the copy), which the multiply then reads instead of the caller's arrays; short pieces
  * scattered over the caller's arrays cost whole cache lines each.  asamd_xlds_refresh_values copies the values again
- * (gate: NULL, or a device word that is 0 when there is nothing to do). */
+ * (gate: NULL, or a device word that is 0 when there is nothing to do).  (No counterpart in the reference, which keeps
+ * no copy of a matrix: src/util_cpp/alphasparse_dcu_x_csrmv_analysis.cpp:269-391 records row blocks only.) */
 typedef struct {
   int32_t *seg;  /* (slices + 1) * m offsets; NULL: no layout */
   int32_t slices, slice_cols, m;
@@ -147,7 +149,7 @@ int asamd_spmv_rowconst(hipStream_t stream, const asamd_spmv_args *a, int32_t ro
  * (rel16: nnz + 4 elements, made once by asamd_narrow_rel_columns for a structure that stays and for THIS `group`;
  * *too_far, a device word the caller has cleared, is set if some entry lies further than 32 767 columns from that
  * row, and rel16 is then unusable): 10 instead of 12 bytes per fp64 entry.  Real element types, val 16-byte aligned,
- * row_ptr[0] == base. */
+ * row_ptr[0] == base.  (No counterpart in the reference: dcu_gemv_vector.h:14-57 reads 32-bit columns.) */
 int asamd_narrow_rel_columns(hipStream_t stream, int32_t m, int32_t nnz, int32_t base, int32_t group,
                              const int32_t *row_ptr, const int32_t *col_ind, int16_t *rel16, int32_t *too_far);
 int asamd_spmv_stream_rel16(hipStream_t stream, const asamd_spmv_args *a, int32_t group, int32_t max_len,
