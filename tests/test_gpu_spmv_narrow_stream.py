@@ -142,3 +142,27 @@ def test_analysed_stencil_beyond_the_cache_reads_distances(gpu, monkeypatch):
         if info is not None:
             lib.alphasparse_dcu_destroy_mat_info(info)
         da.free()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
+def test_large_laplacian_takes_the_non_temporal_forms(gpu, dtype):
+    """5-point Laplacian on 4096 x 4096 points (84 M entries): large enough for the cache policies that small
+    matrices never see -- 4-byte values and their distances past the caches, 8-byte values with y past the caches."""
+    lib = capi.load()
+    a = wl.laplace2d(4096, 4096, dtype)
+    x, y0 = wl.uniform(a.cols, a.dtype, 3), wl.uniform(a.rows, a.dtype, 4)
+    da = DeviceCsr(a)
+    descr = capi.make_descr(base=a.base)
+    info = capi.alphasparse_dcu_mat_info_t()
+    assert lib.alphasparse_dcu_create_mat_info(byref(info)) == 0
+    try:
+        announce("stream, 16-bit distances: large Laplacian", np.dtype(dtype).name)
+        assert getattr(lib, "alphasparse_dcu_%s_csrmv_analysis" % capi.prefix(a.dtype))(
+            gpu.h, 0, a.rows, a.cols, a.nnz, byref(descr), da.val.c_ptr(), da.row_ptr.c_ptr(), da.col.c_ptr(), info) == 0
+        st = lib.asamd_analysis_stats(info).contents
+        assert st.algo == capi.ASAMD_SPMV_STREAM and st.device_bytes >= 2 * a.nnz, (st.algo, st.device_bytes)
+        for alpha, beta in ((1.0, 0.0), (1.5, 0.5)):
+            check_spmv(a, alpha, x, beta, y0, run_csrmv(gpu, da, alpha, x, beta, y0, info=info), "laplace %s" % ((alpha, beta),))
+    finally:
+        lib.alphasparse_dcu_destroy_mat_info(info)
+        da.free()
