@@ -239,13 +239,15 @@ def test_small_workspace_still_multiplies_correctly(gpu):
         da.free()
 
 
-@pytest.mark.parametrize("shape", ["powerlaw", "tiled"])
+@pytest.mark.parametrize("shape", ["powerlaw", "tiled", "slices"])
 def test_one_analysis_from_two_handles_at_once(gpu, shape):
     """Two handles, each with a stream of its own, multiply with ONE info concurrently: every scratch word of a
     multiply lives in its handle's buffer, so each result equals the serial one bit for bit."""
     lib, hip = capi.load(), hiprt.lib()
     if shape == "powerlaw":
         a = wl.powerlaw_rmat(20, 1 << 20, np.float32)        # merge-path: carries and head sums per call
+    elif shape == "slices":
+        a = wl.uniform_rows(1 << 18, 1 << 17, 64, np.float32)  # x in LDS slice by slice: the slices' sums per call
     else:
         a = wl.uniform_rows(1 << 21, 1 << 21, 16, np.float32)  # tiled: the product array per call
     da = DeviceCsr(a)
@@ -267,7 +269,8 @@ def test_one_analysis_from_two_handles_at_once(gpu, shape):
         assert lib.alphasparse_dcu_s_csrmv_analysis(handles[0].h, 0, a.rows, a.cols, a.nnz, byref(descr), da.val.c_ptr(),
                                                     da.row_ptr.c_ptr(), da.col.c_ptr(), info) == 0
         st = lib.asamd_analysis_stats(info).contents
-        assert st.algo == (capi.ASAMD_SPMV_MERGE if shape == "powerlaw" else capi.ASAMD_SPMV_TILED), st.algo
+        want = {"powerlaw": capi.ASAMD_SPMV_MERGE, "slices": capi.ASAMD_SPMV_XLDS, "tiled": capi.ASAMD_SPMV_TILED}[shape]
+        assert st.algo == want and (shape != "slices" or st.xlds_slices >= 2), (st.algo, st.xlds_slices)
 
         def multiply(i, reps):
             for _ in range(reps):
