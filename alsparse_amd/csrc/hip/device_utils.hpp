@@ -346,7 +346,6 @@ struct alignas(16) Double2 { double x, y; };
 // non-temporal what would push the rest out of it (stream_policy in the plan).
 constexpr int kStreamNtValues = 1;
 constexpr int kStreamNtIndices = 2;
-constexpr int kStreamNtY = 4;  // (the staged row-block kernel: y read and written past the caches)
 
 // four consecutive values: 128-bit pieces for the real types, one load per value otherwise
 template <typename T>

@@ -384,8 +384,9 @@ extern "C" int asamd_narrow_rel_columns(hipStream_t s, int32_t m, int32_t nnz, i
                                         const int32_t* row_ptr, const int32_t* col_ind, int16_t* rel16, int32_t* too_far) {
   if (!row_ptr || !col_ind || !rel16 || !too_far || m < 1 || nnz < 1) return hipErrorInvalidValue;
   if (g < 1 || g > kStreamMaxGroup || (g & (g - 1)) != 0) return hipErrorInvalidValue;
-  narrow_rel_columns_kernel<<<(unsigned)(((int64_t)(m > 4 ? m : 4) + 255) / 256), 256, 0, s>>>(
-      m, (int64_t)nnz, base, kStreamRows / g, row_ptr, col_ind, rel16, too_far);
+  const int rows_per_group = kStreamRows / g;
+  narrow_rel_columns_kernel<<<(unsigned)(((int64_t)m + rows_per_group - 1) / rows_per_group), 256, 0, s>>>(
+      m, (int64_t)nnz, base, rows_per_group, row_ptr, col_ind, rel16, too_far);
   return hipGetLastError();
 }
 
@@ -401,15 +402,14 @@ static int stream_rel16_impl(hipStream_t s, const asamd_spmv_args* a, int g, int
   //   27-point stencil 160^3      fp32 0.192 / 0.176 / 0.191 / 0.186      fp64 0.276 / 0.299 / 0.276 / 0.299
   //   5-point Laplacian 4096^2    fp32 0.199 / 0.188 / 0.197 / 0.170      fp64 0.274 / 0.295 / 0.275 / 0.280
   // 4-byte values always bypass the caches; the distances too unless they fit the memory-side cache beside what is
-  // not a matrix stream (49 MB of row offsets, x and y on the stencil, 201 MB on the Laplacian); 8-byte values: nothing
-  // but y where those other arrays outgrow the cache by themselves (the fp64 Laplacian, 336 MB: 0.272 -> 0.266 ms;
-  // the fp32 one loses: 0.171 -> 0.181).
+  // not a matrix stream (49 MB of row offsets, x and y on the stencil, 201 MB on the Laplacian); 8-byte values: nothing.
+  // (y past the caches as well gained 2 % on the fp64 Laplacian and lost 6 % on the fp32 one, and the branch in the
+  // kernel's last lines cost the 27-point stencil, fp64, about 3 % whether taken or not: left out.)
   static const int forced = getenv("ALSPARSE_AMD_STREAM_POLICY") ? atoi(getenv("ALSPARSE_AMD_STREAM_POLICY")) : -1;
   const double rest = ((double)a->m + 1.0) * 4.0 + ((double)a->m + (double)a->n) * (double)sizeof(T);
   int policy = 0;
   if (sizeof(T) == 4) policy = kStreamNtValues | (rest + 2.0 * (double)a->nnz > 300.0e6 ? kStreamNtIndices : 0);
-  else if (rest > 256.0e6) policy = kStreamNtY;
-  if (forced >= 0) policy = forced & (kStreamNtValues | kStreamNtIndices | kStreamNtY);
+  if (forced >= 0) policy = forced & (kStreamNtValues | kStreamNtIndices);
 #define ASAMD_STREAM_REL16(CAP, G)                                                                                   \
   spmv_stream_wide_kernel<T, CAP, G, true><<<grid, kStreamRows, 0, s>>>(a->m, alpha, (const T*)a->val, a->row_ptr,   \
                                                                         a->col_ind, (const T*)a->x, beta, (T*)a->y,  \
