@@ -142,10 +142,16 @@ static int xlds_sized_x(const asamd_csr_plan *p) {
   const int64_t x_bytes = (int64_t)p->st.n * (int64_t)p->val_size;
   return x_bytes > (20 << 10) && asamd_spmv_xlds_fits(p->dtype, p->st.n);
 }
+/* ... and enough rows of moderate length: a lane group takes four rows per trip and rows beyond 512 entries go to
+ * single waves, so 2 048 rows of 2 048 entries keep 8 of the 256 workgroups busy (0.067 ms against merge-path's
+ * 0.018; 8 192 x 1 024: 0.053 against 0.035; 32 768 x 256: 0.016 against rowconst's 0.033). */
+static int xlds_rows_enough(const asamd_csr_stats *st, int slices) {
+  return (int64_t)st->m * slices >= 32768 && (double)st->nnz <= 512.0 * (double)slices * (double)st->m;
+}
 static int xlds_ok(const asamd_csr_plan *p) {
   const asamd_csr_stats *st = &p->st;
   return st->first_offset == 0 && st->m >= 1 && st->nnz >= (1 << 22) && xlds_sized_x(p) && xlds_rows_regular(st) &&
-         env_int("ALSPARSE_AMD_XLDS", 1) > 0;
+         xlds_rows_enough(st, 1) && env_int("ALSPARSE_AMD_XLDS", 1) > 0;
 }
 
 /* ... and slice by slice for an x of several LDS fills, where the rows are long enough for their pieces: a slice's
@@ -163,7 +169,7 @@ static int xlds_sliced_ok(const asamd_csr_plan *p, int force, int copy) {
   const int slices = xlds_slices_for(p);
   if (slices < 2 || slices > 1024 || ((int64_t)slices + 1) * st->m >= (int64_t)INT32_MAX) return 0;
   if (force) return 1;
-  return st->nnz >= (1 << 22) && xlds_rows_regular(st) &&
+  return st->nnz >= (1 << 22) && xlds_rows_regular(st) && xlds_rows_enough(st, slices) &&
          (double)st->nnz >= (copy ? 3.0 : 16.0) * (double)slices * (double)st->m &&
          env_int("ALSPARSE_AMD_XLDS", 1) > 0;
 }

@@ -321,3 +321,21 @@ def test_rows_far_longer_than_the_mean_keep_the_balanced_kernels(gpu):
                     lib.alphasparse_dcu_destroy_mat_info(info)
         finally:
             da.free()
+
+
+def test_few_very_long_rows_keep_the_balanced_kernels(gpu):
+    """2 048 rows of 2 048 entries under 16 384 columns: the kernel that holds x in LDS gives a lane group four rows per
+    trip and rows beyond 512 entries to single waves, so eight of its 256 workgroups would work; the library keeps
+    merge-path.  32 768 rows of 256 entries take it."""
+    lib = capi.load()
+    for rows, cols, per_row, takes_xlds in ((2048, 16384, 2048, False), (32768, 32768, 256, True)):
+        a = wl.uniform_rows(rows, cols, per_row, np.float32)
+        assert a.nnz >= 1 << 22
+        da = DeviceCsr(a)
+        try:
+            announce("x in LDS: rows", rows, "of", per_row)
+            assert (_plan_algo(lib, da) == capi.ASAMD_SPMV_XLDS) == takes_xlds, (rows, per_row)
+            x, y0 = wl.uniform(a.cols, a.dtype, 3), wl.uniform(a.rows, a.dtype, 4)
+            check_spmv(a, 1.0, x, 0.5, y0, run_csrmv(gpu, da, 1.0, x, 0.5, y0), "%d rows of %d" % (rows, per_row))
+        finally:
+            da.free()
