@@ -137,10 +137,11 @@ static int xlds_rows_regular(const asamd_csr_stats *st) {
   return far <= 0.1 * (double)st->nnz;
 }
 
-/* an x that crowds the L1 and fits a compute unit's LDS */
+/* an x that crowds the L1 and fits a compute unit's LDS (4 M x 5 000 x 16, fp32, 20 KB of x: 0.108 ms against
+ * rowconst's 0.138; with 16 KB the two are level) */
 static int xlds_sized_x(const asamd_csr_plan *p) {
   const int64_t x_bytes = (int64_t)p->st.n * (int64_t)p->val_size;
-  return x_bytes > (20 << 10) && asamd_spmv_xlds_fits(p->dtype, p->st.n);
+  return x_bytes >= (18 << 10) && asamd_spmv_xlds_fits(p->dtype, p->st.n);
 }
 /* ... and enough rows of moderate length: a lane group takes four rows per trip and rows beyond 512 entries go to
  * single waves, so 2 048 rows of 2 048 entries keep 8 of the 256 workgroups busy (0.067 ms against merge-path's
@@ -148,10 +149,16 @@ static int xlds_sized_x(const asamd_csr_plan *p) {
 static int xlds_rows_enough(const asamd_csr_stats *st, int slices) {
   return (int64_t)st->m * slices >= 32768 && (double)st->nnz <= 512.0 * (double)slices * (double)st->m;
 }
+/* Rows of fewer than four entries on average run the form with one entry per lane and two lanes per row, which pays
+ * where all rows are equally long (8 M rows of 2 entries: 0.056 ms against the staged row blocks' 0.074; of 3: 0.073
+ * against 0.102) and not otherwise (rows of 1 and 3 in turn: 0.091 against 0.073; one entry per row: 0.109 against 0.096). */
+static int xlds_rows_not_too_short(const asamd_csr_stats *st) {
+  return (int64_t)st->nnz >= 4 * (int64_t)st->m || st->const_len >= 2;
+}
 static int xlds_ok(const asamd_csr_plan *p) {
   const asamd_csr_stats *st = &p->st;
   return st->first_offset == 0 && st->m >= 1 && st->nnz >= (1 << 22) && xlds_sized_x(p) && xlds_rows_regular(st) &&
-         xlds_rows_enough(st, 1) && env_int("ALSPARSE_AMD_XLDS", 1) > 0;
+         xlds_rows_enough(st, 1) && xlds_rows_not_too_short(st) && env_int("ALSPARSE_AMD_XLDS", 1) > 0;
 }
 
 /* ... and slice by slice for an x of several LDS fills, where the rows are long enough for their pieces: a slice's
