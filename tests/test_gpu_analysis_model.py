@@ -16,6 +16,9 @@ pytestmark = pytest.mark.gpu
 SHAPES = {
     # configuration 2 itself: 5-point Laplacian, fp64 -> the staged row-block kernel on the caller's arrays
     "laplace_c2": (lambda: wl.laplace2d(2048, 2048, np.float64), capi.ASAMD_SPMV_STREAM),
+    # the same structure with complex128 values: the staged kernel moves 16-byte values at two thirds of its rate
+    # with 8-byte ones, the ELL copy does not (0.145 against 0.110 ms, the value guard's launches included)
+    "laplace_c2_complex": (lambda: wl.complexify(wl.laplace2d(2048, 2048, np.float64), np.complex128), capi.ASAMD_SPMV_ELL),
     # configuration 3's kind at an eighth of its size: scattered columns over 8 MiB of x -> the tiled copy
     "uniform_2M_16": (lambda: wl.uniform_rows(1 << 21, 1 << 21, 16, np.float32), capi.ASAMD_SPMV_TILED),
     # configuration 4's kind at half its size: power-law rows, R-MAT columns, 16 MiB of x -> merge-path
@@ -34,8 +37,8 @@ def _analyse(lib, da, mode):
     if mode:
         os.environ["ALSPARSE_AMD_TUNE"] = mode
     try:
-        assert lib.asamd_csr_plan_create(None, a.rows, a.cols, a.nnz, da.row_ptr.c_ptr(), da.col.c_ptr(), da.val.c_ptr(),
-                                         a.base, a.dtype.itemsize, 1, byref(plan)) == 0
+        assert lib.asamd_csr_plan_create_dtype(None, a.rows, a.cols, a.nnz, da.row_ptr.c_ptr(), da.col.c_ptr(),
+                                               da.val.c_ptr(), a.base, capi.dtype_tag(a.dtype), 1, byref(plan)) == 0
     finally:
         if old is None:
             os.environ.pop("ALSPARSE_AMD_TUNE", None)
@@ -76,7 +79,10 @@ def test_model_and_timing_choose_the_same_family(gpu, shape):
         # its estimate of the kept family is within a third of what the timing run measured
         key = {capi.ASAMD_SPMV_TILED: "tune_ms_tiled", capi.ASAMD_SPMV_ELL: "tune_ms_ell"}.get(want, "tune_ms_base")
         if timed[key] > 0:  # (a copy that the timing run did not lay out has no measurement)
-            assert 0.66 * timed[key] <= model[0][key] <= 1.5 * timed[key], (key, model[0][key], timed[key])
+            # (the model's figure for a copy that holds values counts the value guard's launches, 0.022 ms; the timing
+            # run launches the kernel alone)
+            est = model[0][key] - (0.022 if key != "tune_ms_base" else 0.0)
+            assert 0.66 * timed[key] <= est <= 1.5 * timed[key], (key, model[0][key], timed[key])
     finally:
         da.free()
 
