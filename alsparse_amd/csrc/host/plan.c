@@ -1032,7 +1032,8 @@ static double model_ms(const asamd_csr_plan *p, int algo) {
     case ASAMD_SPMV_ROWCONST: rate = 6.0; break;
     case ASAMD_SPMV_STREAM:
       rate = stream_group(p, 0) > 1 ? 5.2 : 6.6;
-      /* 16-byte values, one lane per row: 5-point Laplacian of 4 M rows, complex128 (570 MB), 0.139 ms */
+      /* 16-byte values (four per lane, so two lanes per row of five): 5-point Laplacian of 4 M rows, complex128
+       * (570 MB), 0.139 ms */
       if (vs >= 16.0 && rate > 4.2) rate = 4.2;
       /* 16-bit distances for columns: half of the bytes they save shows (27-point stencil, 160^3 points: 0.204 ->
        * 0.181 ms with 4-byte values, 0.300 -> 0.274 with 8-byte ones) */
