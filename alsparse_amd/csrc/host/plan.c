@@ -1063,7 +1063,11 @@ static double model_ms(const asamd_csr_plan *p, int algo) {
        * fall into a narrower window of x than the positions of one row, which pays once x outgrows an XCD's L2:
        * 1 M x 1 M x 16 / x 32, fp64 (8 MB of x): 0.143 / 0.261 ms against rowconst's 0.186 / 0.355 (more rows in
        * flight per lane group do not help rowconst: 0.357); fp32 (4 MB): 0.100 / 0.196 against 0.095 / 0.196 */
-      return hypot2(ell_bytes / 6.1e9, vs >= 8.0 ? 0.72 * gather : gather);
+      /* (rows of 16 and more; with few entries per row one position's columns spread as far as a row's: 2 M x 2 M x 4,
+       * fp64, 0.130 ms against rowconst's 0.128; 1 M x 1 M x 8: 0.086 against 0.096) */
+      double narrow = 1.0;
+      if (vs >= 8.0 && mean > 8.0) narrow = mean >= 16.0 ? 0.72 : 1.0 - 0.28 * (mean - 8.0) / 8.0;
+      return hypot2(ell_bytes / 6.1e9, narrow * gather);
     }
     case ASAMD_SPMV_TILED: {
       double skew = 1.0 + 0.5 * ((double)st->max_len / mean - 1.0) / 8.0;
@@ -1080,7 +1084,20 @@ static double model_ms(const asamd_csr_plan *p, int algo) {
       double long_rows = 1.0 + most * (usual - 16.0) / 48.0;
       if (long_rows < 1.0) long_rows = 1.0;
       if (long_rows > 1.0 + most) long_rows = 1.0 + most;
-      return (0.045 + stream) * skew * long_rows;
+      /* 8-byte values in short rows on matrices of up to 16 M entries ran below the estimate that fits rows of 16
+       * (2 M x 2 M x 4: 0.073 against 0.095 ms, 4 M x 4 M x 4: 0.125 / 0.162, 1 M x 1 M x 8: 0.079 / 0.088); with
+       * 32 M entries and more they do not (8 M x 8 M x 4: 0.301 / 0.278) */
+      if (vs >= 8.0 && usual < 16.0 && nnz < 33.5e6) {
+        double cut = 0.22 * (16.0 - usual) / 12.0;
+        if (cut > 0.22) cut = 0.22;
+        const double fade = nnz <= 16.8e6 ? 1.0 : (33.5e6 - nnz) / 16.7e6;
+        long_rows = 1.0 - cut * fade;
+      }
+      /* the fixed part: 0.045 ms from about 200 MB of CSR bytes on; a matrix of a few tens of MB has fewer tiles than
+       * the two phases keep in flight and runs them in less (4 M x 4 M x 2, 118 MB: 0.057 ms measured, 2 M x 2 M x 8,
+       * 158 MB: 0.089) */
+      const double fixed = 0.015 + 0.03 * (bytes < 200.0e6 ? bytes / 200.0e6 : 1.0);
+      return (fixed + stream) * skew * long_rows;
     }
     default: break;
   }
