@@ -985,7 +985,7 @@ static hipError_t tune_copies(hipStream_t stream, asamd_csr_plan *p, const int32
  *     T ps   3.6   4.7    5.6    5.9    10.5   10.5   13.5    17.8   19      beyond an XCD's L2 wait 3 x longer)
  *     TB/s   constant row length 6.0, staged row block 6.6 (one lane per row) / 5.2 (several), lane group per
  *            row 2.4 x the share of its lanes that hold an entry, merge-path 2.9, ELL copy 6.1 (of its padded
- *            streams); tiled pair: 0.045 ms + 2 x bytes / 5.6 TB/s (8-byte values and wider: their 28 / 52 bytes per
+ *            streams); tiled pair: 0.015 .. 0.045 ms (small matrices less) + 2 x bytes / 5.6 TB/s (8-byte values and wider: their 28 / 52 bytes per
  *            entry at 4.6 TB/s), x 1 .. 1.5 with the spread of the row lengths, x 2.5 for heavy-tailed rows.
  * The estimates are within about 10 % of the timings on the shapes they were read from (5-point and 27-point
  * stencils, uniform rows over 0.25 - 64 MiB of x, two row lengths, power-law rows and columns, fp32 / fp64). */
@@ -1084,10 +1084,11 @@ static double model_ms(const asamd_csr_plan *p, int algo) {
       double long_rows = 1.0 + most * (usual - 16.0) / 48.0;
       if (long_rows < 1.0) long_rows = 1.0;
       if (long_rows > 1.0 + most) long_rows = 1.0 + most;
-      /* 8-byte values in short rows on matrices of up to 16 M entries ran below the estimate that fits rows of 16
-       * (2 M x 2 M x 4: 0.073 against 0.095 ms, 4 M x 4 M x 4: 0.125 / 0.162, 1 M x 1 M x 8: 0.079 / 0.088); with
-       * 32 M entries and more they do not (8 M x 8 M x 4: 0.301 / 0.278) */
-      if (vs >= 8.0 && usual < 16.0 && nnz < 33.5e6) {
+      /* short rows on matrices of up to 16 M entries ran below the estimate that fits rows of 16 (8-byte values,
+       * 2 M x 2 M x 4: 0.073 against 0.095 ms, 4 M x 4 M x 4: 0.125 / 0.162, 1 M x 1 M x 8: 0.079 / 0.088; 4-byte ones,
+       * 2 M x 2 M x 4: 0.050 / 0.062, 4 M x 4 M x 2: 0.056 / 0.075, 2 M x 2 M x 8: 0.089 / 0.100); with 32 M entries and
+       * more they do not (8 M x 8 M x 4, 8-byte values: 0.301 / 0.278) */
+      if (usual < 16.0 && nnz < 33.5e6) {
         double cut = 0.22 * (16.0 - usual) / 12.0;
         if (cut > 0.22) cut = 0.22;
         const double fade = nnz <= 16.8e6 ? 1.0 : (33.5e6 - nnz) / 16.7e6;
