@@ -330,6 +330,8 @@ def run_spmv(cfg, steps, warmup, cpu_baseline, check, transpose=False, vendor=Fa
         assert st == 0, "repeated analysis status %d" % st
     hiprt.synchronize()
     reanalysis_ms = (time.perf_counter() - t0) * 1e3 if analysed else None
+    if analysed:  # the repeated analysis replaced the record that `stats` looked into
+        stats = (lib.asamd_analysis_transpose_stats(info) if transpose else lib.asamd_analysis_stats(info)).contents
     for k, v in env_old.items():
         if v is None:
             os.environ.pop(k, None)
